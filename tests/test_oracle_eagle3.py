@@ -1,0 +1,157 @@
+"""The oracle's EAGLE3 forward against the HF library blocks it restates, and
+its alignment invariants."""
+
+import pytest
+import torch
+
+from oracle import eagle3 as E
+from oracle import masks as M
+from oracle.attention import dense_attention
+
+
+def _tiny_shape(**kw):
+    base = dict(hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+                intermediate_size=128, vocab_size=128, draft_vocab_size=48, rms_norm_eps=1e-6,
+                rope_theta=10000.0)
+    base.update(kw)
+    return E.DraftShape(**base)
+
+
+def _batch(shape, t, seed=0, docs=None):
+    g = torch.Generator().manual_seed(seed)
+    hs = torch.randn(1, t, shape.num_aux * shape.hidden_size, generator=g)
+    ids = torch.randint(0, shape.vocab_size, (1, t), generator=g)
+    vl = torch.randn(1, t, shape.hidden_size, generator=g)
+    mask = (torch.rand(1, t, generator=g) < 0.7).float()
+    if docs is None:
+        doc = torch.zeros(1, t, dtype=torch.long)
+        pos = 1 + torch.arange(t).unsqueeze(0)
+    else:
+        doc = torch.full((1, t), -1, dtype=torch.long)
+        pos = torch.zeros(1, t, dtype=torch.long)
+        o = 0
+        for i, n in enumerate(docs):
+            doc[0, o:o + n] = i
+            pos[0, o:o + n] = 1 + torch.arange(n)
+            o += n
+        mask[0, o:] = 0
+    return hs, ids, doc, mask, pos, vl
+
+
+def test_dense_attention_equals_sdpa_library_routine():
+    g = torch.Generator().manual_seed(0)
+    t = 24
+    q = torch.randn(1, 4, t, 16, generator=g)
+    k = torch.randn(1, 2, 3 * t, 16, generator=g)
+    v = torch.randn(1, 2, 3 * t, 16, generator=g)
+    doc = torch.tensor([0] * 10 + [1] * 9 + [-1] * 5)
+    mask = M.ttt_mask_dense(doc, t, 2, sliding_window=6)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q, k.repeat_interleave(2, 1), v.repeat_interleave(2, 1), attn_mask=mask[None, None],
+        scale=0.25).transpose(1, 2)
+    assert torch.allclose(dense_attention(q, k, v, mask, 0.25), ref, atol=1e-5)
+
+
+def test_first_layer_equals_hf_llama_blocks():
+    from transformers import DynamicCache, LlamaConfig
+    from transformers.models.llama.modeling_llama import (
+        LlamaAttention, LlamaMLP, LlamaRMSNorm, LlamaRotaryEmbedding)
+
+    shape = _tiny_shape(norm_before_residual=True)
+    w = E.random_weights(shape, seed=1)
+    for k_ in list(w):
+        if k_.endswith("norm.weight") or "layernorm" in k_:
+            w[k_] = 1 + 0.1 * torch.randn_like(w[k_])
+    cfg = LlamaConfig(hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+                      intermediate_size=128, vocab_size=128, rms_norm_eps=1e-6,
+                      rope_parameters={"rope_type": "default", "rope_theta": 10000.0},
+                      num_hidden_layers=1, attention_bias=False)
+    cfg._attn_implementation = "eager"
+    attn = LlamaAttention(cfg, 0)
+    attn.q_proj = torch.nn.Linear(128, 64, bias=False)
+    attn.k_proj = torch.nn.Linear(128, 32, bias=False)
+    attn.v_proj = torch.nn.Linear(128, 32, bias=False)
+    p = "layers.0."
+    for n in "qkvo":
+        getattr(attn, n + "_proj").weight.data.copy_(w[p + f"self_attn.{n}_proj.weight"])
+    mlp = LlamaMLP(cfg)
+    for n in ("gate", "up", "down"):
+        getattr(mlp, n + "_proj").weight.data.copy_(w[p + f"mlp.{n}_proj.weight"])
+    norms = {}
+    for n in ("input_layernorm", "hidden_norm", "post_attention_layernorm"):
+        norms[n] = LlamaRMSNorm(64, eps=1e-6)
+        norms[n].weight.data.copy_(w[p + n + ".weight"])
+    rot_cfg = LlamaConfig(**{**cfg.to_dict(), "hidden_size": 128})
+    rot = LlamaRotaryEmbedding(rot_cfg)
+
+    t = 20
+    g = torch.Generator().manual_seed(5)
+    doc = torch.tensor([0] * 8 + [1] * 9 + [-1] * 3)
+    pos = torch.cat([1 + torch.arange(8), 1 + torch.arange(9), torch.zeros(3, dtype=torch.long)]).unsqueeze(0)
+    cache_hf, cache_or = DynamicCache(), {}
+    with torch.no_grad():
+        for step in range(3):
+            x = torch.randn(1, t, 128, generator=g)
+            mask = M.ttt_mask_dense(doc, t, step)
+            fmask = torch.zeros(1, 1, t, (step + 1) * t).masked_fill(~mask[None, None], float("-inf"))
+            cos, sin = rot(x, pos + step)
+            e, h = x.split(64, -1)
+            e, h = norms["input_layernorm"](e), norms["hidden_norm"](h)
+            a, _ = attn(hidden_states=torch.cat([e, h], -1), attention_mask=fmask,
+                        position_embeddings=(cos, sin), past_key_values=cache_hf,
+                        cache_position=torch.arange(step * t, (step + 1) * t))
+            y = h + a
+            ref = y + mlp(norms["post_attention_layernorm"](y))
+            c2, s2 = E.rope_tables(pos + step, 16, 10000.0, torch.float32)
+            assert torch.allclose(c2, cos, atol=1e-6) and torch.allclose(s2, sin, atol=1e-6)
+            got = E.first_layer(x, w, shape, c2, s2, cache_or, mask)
+            assert torch.allclose(got, ref, atol=2e-5), (step, (got - ref).abs().max())
+
+
+@pytest.mark.parametrize("attn", ["dense", "sdpa"])
+def test_forward_runs_and_backends_agree(attn):
+    shape = _tiny_shape(norm_output=True, norm_before_fc=True, norm_before_residual=True,
+                        sliding_window=8, sliding_layers=(0,), num_hidden_layers=2)
+    w = E.random_weights(shape, seed=0)
+    hs, ids, doc, mask, pos, vl = _batch(shape, 32, docs=[12, 15])
+    toks, loss, m = E.eagle3_forward(w, shape, hs, ids, doc, mask, pos, vl, ttt_steps=3,
+                                     ttt_step_loss_decay=0.9, attn=attn)
+    toks2, loss2, m2 = E.eagle3_forward(w, shape, hs, ids, doc, mask, pos, vl, ttt_steps=3,
+                                        ttt_step_loss_decay=0.9, attn="dense")
+    assert torch.isfinite(loss) and len(toks) == 3 and toks[0].shape == (1, 32)
+    # whole-model loss agreement across attention backends, the reference's own
+    # tolerance (tests/integration/models/test_model_forward.py:360-366)
+    assert torch.allclose(loss, loss2, atol=1e-3, rtol=1e-3)
+    for k in ("loss_0_sum", "full_acc_2_total", "cond_acc_1_total", "loss_sum", "loss_total"):
+        assert k in m
+    assert m["loss_sum"].item() == pytest.approx(sum(m[f"loss_{k}_sum"].item() for k in range(3)), rel=1e-6)
+
+
+def test_documents_are_independent_and_padding_is_inert():
+    """Packing invariant: the loss of a packed row equals what each document
+    contributes alone (the mask is block diagonal by document)."""
+    shape = _tiny_shape()
+    w = E.random_weights(shape, seed=2)
+    hs, ids, doc, mask, pos, vl = _batch(shape, 24, docs=[10, 9])
+    _, _, _, logits = E.eagle3_forward(w, shape, hs, ids, doc, mask, pos, vl, ttt_steps=2,
+                                       return_logits=True)
+    # document 1 alone (rows 10..18)
+    sl = slice(10, 19)
+    _, _, _, lg1 = E.eagle3_forward(w, shape, hs[:, sl], ids[:, sl], torch.zeros(1, 9, dtype=torch.long),
+                                    mask[:, sl], pos[:, sl], vl[:, sl], ttt_steps=2, return_logits=True)
+    # step 0 is identical row by row; step 1 is too except the last row of the
+    # document, whose teacher-forced input id comes from the neighbour in the packed row
+    assert torch.allclose(logits[0][:, sl], lg1[0], atol=1e-5)
+    assert torch.allclose(logits[1][:, 10:18], lg1[1][:, :8], atol=1e-5)
+
+
+def test_teacher_forcing_shift():
+    """Step k consumes input_ids shifted left by k (zero padded) and positions + k."""
+    shape = _tiny_shape()
+    w = E.random_weights(shape, seed=3)
+    hs, ids, doc, mask, pos, vl = _batch(shape, 16)
+    toks, loss, m = E.eagle3_forward(w, shape, hs, ids, doc, mask, pos, vl, ttt_steps=2)
+    ids2 = ids.clone(); ids2[0, 0] = (ids2[0, 0] + 1) % shape.vocab_size
+    toks2, loss2, _ = E.eagle3_forward(w, shape, hs, ids2, doc, mask, pos, vl, ttt_steps=2)
+    # token 0 is only ever used as the step-0 input of row 0
+    assert not torch.equal(toks[0], toks2[0]) or loss.item() != loss2.item()

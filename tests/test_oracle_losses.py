@@ -1,0 +1,178 @@
+"""Oracle losses: the identities the reference's tests assert
+(tests/unit/models/test_metrics.py), library routines, closed-form gradients."""
+
+import math
+from functools import partial
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import losses as L
+
+
+def _pair(seed=0, shape=(1, 4, 50), scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale, torch.randn(*shape, generator=g) * scale
+
+
+def test_kl_matches_library_kl_div():
+    a, b = _pair(1, (1, 6, 33), 3.0)
+    ref = F.kl_div(F.log_softmax(a, -1), F.softmax(b, -1), reduction="none").sum(-1)
+    assert torch.allclose(L.kl_div(a, b), ref, atol=1e-6)
+
+
+def test_ce_matches_library_cross_entropy_first_index_ties():
+    a, b = _pair(2, (1, 5, 17))
+    b[0, 0, 3] = b[0, 0, 9] = 50.0  # tie -> first index
+    ref = F.cross_entropy(a.reshape(-1, 17), b.argmax(-1).reshape(-1), reduction="none")
+    assert torch.allclose(L.ce(a, b).reshape(-1), ref, atol=1e-6)
+    assert int(b.argmax(-1)[0, 0]) == 3
+
+
+@pytest.mark.parametrize("fn", [L.kl_div, L.rkl, L.jsd])
+def test_identical_zero_random_nonnegative(fn):
+    x = torch.randn(1, 4, 8)
+    assert fn(x, x).sum().item() == pytest.approx(0.0, abs=1e-4)
+    a, b = _pair(0, (1, 4, 8))
+    assert (fn(a, b) >= -1e-6).all()
+
+
+def test_rkl_is_kl_swapped():
+    a, b = _pair(0, (1, 4, 8))
+    assert torch.allclose(L.rkl(a, b), L.kl_div(b, a), atol=1e-6)
+
+
+def test_jsd_symmetric_bounded_manual():
+    a, b = _pair(0, (1, 4, 50))
+    assert torch.allclose(L.jsd(a, b), L.jsd(b, a), atol=1e-6)
+    p = torch.full((1, 1, 4), -100.0); p[0, 0, 0] = 100.0
+    q = torch.full((1, 1, 4), -100.0); q[0, 0, 1] = 100.0
+    assert L.jsd(p, q).max().item() == pytest.approx(math.log(2), abs=1e-3)
+    pp, qq = torch.softmax(b, -1), torch.softmax(a, -1)
+    m = 0.5 * (pp + qq)
+    manual = 0.5 * ((pp * (pp / m).log()).sum(-1) + (qq * (qq / m).log()).sum(-1))
+    assert torch.allclose(L.jsd(a, b), manual, atol=1e-5)
+
+
+def test_tv_is_half_l1_in_unit_range():
+    a, b = _pair(0, (1, 4, 50))
+    l1 = 0.5 * (torch.softmax(a, -1) - torch.softmax(b, -1)).abs().sum(-1)
+    out = L.tv(a, b)
+    assert torch.allclose(out, l1, atol=1e-6)
+    assert (out >= 0).all() and (out <= 1).all()
+    assert torch.allclose(L.tv(a, a), torch.zeros(1, 4), atol=1e-6)
+
+
+def test_nla_forms():
+    a, b = _pair(0, (1, 4, 50))
+    assert torch.allclose(L.nla(a, a), torch.zeros(1, 4), atol=1e-5)
+    assert torch.allclose(L.nla(a, b), -torch.log((1 - L.tv(a, b)).clamp_min(1e-5)), atol=1e-6)
+    t = torch.full((1, 1, 50), -30.0); t[0, 0, 7] = 30.0
+    x = torch.randn(1, 1, 50)
+    assert torch.allclose(L.nla(x, t), L.ce(x, t), atol=1e-3)
+    d = torch.full((1, 1, 50), -30.0); d[0, 0, 0] = 30.0
+    t2 = torch.full((1, 1, 50), -30.0); t2[0, 0, 1] = 30.0
+    v = L.nla(d, t2)
+    assert torch.isfinite(v).all() and v.item() == pytest.approx(-math.log(1e-5), rel=1e-3)
+
+
+def test_lk_hybrid_limits_and_detached_weight():
+    a, b = _pair(0, (1, 4, 50))
+    assert torch.allclose(L.lk_hybrid(a, b, eta=0.0), L.kl_div(a, b), atol=1e-6)
+    assert torch.allclose(L.lk_hybrid(a, b, eta=1e6), L.tv(a, b), atol=1e-5)
+    x = torch.randn(1, 3, 40, requires_grad=True)
+    t = torch.randn(1, 3, 40)
+    g_impl = torch.autograd.grad(L.lk_hybrid(x, t, 3.0).sum(), x)[0]
+
+    def manual(detach):
+        dp, tp = torch.softmax(x, -1), torch.softmax(t, -1)
+        ov = torch.minimum(dp, tp).sum(-1)
+        lam = torch.exp(-3.0 * (ov.detach() if detach else ov))
+        return (lam * L.kl_div(x, t) + (1 - lam) * (1 - ov)).sum()
+
+    g_det = torch.autograd.grad(manual(True), x, retain_graph=True)[0]
+    g_no = torch.autograd.grad(manual(False), x)[0]
+    assert torch.allclose(g_impl, g_det, atol=1e-5)
+    assert not torch.allclose(g_det, g_no, atol=1e-4)
+
+
+@pytest.mark.parametrize("name", ["kl_div", "rkl", "jsd", "ce", "tv"])
+def test_closed_form_gradient_equals_autograd(name):
+    a, b = _pair(5, (1, 6, 64), 2.0)
+    a = a.double().requires_grad_(True)
+    out = L.LOSS_FNS[name](a, b.double())
+    # the oracle computes in fp32; compare with autograd through the same fp32 graph
+    g = torch.autograd.grad(out.sum(), a)[0].float()
+    closed = L.row_loss_grad(name, a.detach().float(), b)
+    assert torch.allclose(closed, g, atol=2e-6), (closed - g).abs().max()
+
+
+def test_saturated_rows_stay_finite():
+    # the +-30 point-mass regime of tests/unit/models/test_fused_losses.py:71-79
+    g = torch.Generator().manual_seed(0)
+    a = torch.randn(1, 8, 512, generator=g) * 3
+    b = torch.randn(1, 8, 512, generator=g) * 3
+    a[0, -2:] = -30.0; b[0, -2:] = -30.0
+    a[0, -2:, 0] = 30.0; b[0, -2, 0] = 30.0; b[0, -1, 7] = 30.0
+    for name, fn in L.LOSS_FNS.items():
+        assert torch.isfinite(fn(a, b)).all(), name
+    assert L.kl_div(a, b)[0, -2].item() == pytest.approx(0.0, abs=1e-5)
+    assert L.kl_div(a, b)[0, -1].item() == pytest.approx(60.0, rel=1e-4)
+
+
+def test_decay_scales_loss_and_masked_mean():
+    g = torch.Generator().manual_seed(42)
+    a = torch.randn(1, 16, 8, generator=g); b = torch.randn(1, 16, 8, generator=g)
+    m = torch.ones(1, 16)
+    d = partial(L.exp_loss_decay, gamma=0.5)
+    l0 = L.loss_function(a, b, m, torch.zeros(1, 16, dtype=torch.long), L.kl_div, d)
+    l2 = L.loss_function(a, b, m, torch.full((1, 16), 2), L.kl_div, d)
+    assert torch.isclose(l2, l0 * 0.25, rtol=1e-4)
+    assert L.loss_function(a, b, torch.zeros(1, 16), torch.zeros(1, 16), L.kl_div).item() == pytest.approx(0, abs=1e-4)
+    mm = torch.tensor([[1, 0, 1, 1, 0, 1.0]])
+    r = L.loss_function(a[:, :6], b[:, :6], mm, torch.zeros(1, 6), L.kl_div)
+    assert torch.isclose(r, (L.kl_div(a[:, :6], b[:, :6]) * mm).sum() / (mm.sum() + 1e-5))
+
+
+def test_decay_known_values():
+    pos = torch.arange(4, dtype=torch.float)
+    d = L.dflash_loss_decay(pos, gamma=4.0)
+    assert d[0].item() == 0.0 and d[1].item() == pytest.approx(1.0)
+    assert d[2].item() == pytest.approx(math.exp(-0.25)) and d[3].item() == pytest.approx(math.exp(-0.5))
+    s = L.dflash_loss_decay(pos, gamma=4.0, sample_from_anchor=True)
+    assert s[0].item() == pytest.approx(1.0) and s[2].item() == pytest.approx(math.exp(-0.5))
+    assert L.exp_loss_decay(torch.tensor(2.0), gamma=0.5).item() == pytest.approx(0.25)
+    assert L.exp_loss_decay(torch.tensor(0.0), gamma=0.5).item() == pytest.approx(1.0)
+
+
+def test_dpace_hand_computed_two_blocks():
+    # block 0: CE = [0, ln2, ln4], mask [1,1,1], alpha=.5 -> s = [1,.75,.625]
+    # prefix = [1,.75,.46875]; w = [2.21875, 1.21875, .46875]
+    # block 1: mask [0,1,1], CE = [9, 0, ln2] -> s = [1,1,.75]; prefix*m = [0,1,.75]; w=[0,1.75,.75]
+    ce = torch.tensor([[0.0, math.log(2), math.log(4), 9.0, 0.0, math.log(2)]])
+    m = torch.tensor([[1, 1, 1, 0, 1, 1.0]])
+    w = L.dpace_loss_decay(None, m, 3, 0.5, ce)
+    assert torch.allclose(w, torch.tensor([[2.21875, 1.21875, 0.46875, 0.0, 1.75, 0.75]]), atol=1e-6)
+
+
+def test_bf16_inputs_fp32_math_gradient_within_2_percent_of_fp64():
+    # the regime of tests/unit/models/test_metrics.py:388-439
+    g = torch.Generator().manual_seed(0)
+    t = (torch.randn(1, 8, 4096, generator=g) * 2).bfloat16()
+    x = (t.float() + torch.randn(1, 8, 4096, generator=g) * 0.1).bfloat16()
+    for name in ["kl_div", "rkl", "jsd", "tv"]:
+        xd = x.double().requires_grad_(True)
+        pd, qd = torch.softmax(t.double(), -1), torch.softmax(xd, -1)
+        if name == "kl_div":
+            ref = (pd * (pd.log() - qd.log())).sum()
+        elif name == "rkl":
+            ref = (qd * (qd.log() - pd.log())).sum()
+        elif name == "jsd":
+            md = 0.5 * (pd + qd)
+            ref = 0.5 * ((pd * (pd / md).log()).sum() + (qd * (qd / md).log()).sum())
+        else:
+            ref = (1 - torch.minimum(pd, qd).sum(-1)).sum()
+        exact = torch.autograd.grad(ref, xd)[0]
+        got = L.row_loss_grad(name, x, t).double()
+        assert ((got - exact).norm() / exact.norm()).item() < 0.02, name

@@ -1,0 +1,137 @@
+"""Oracle acceptance counts / step alignment / vocabulary tables."""
+
+import pytest
+import torch
+
+from oracle import losses as L
+from oracle import metrics as MT
+from oracle import vocab as V
+
+
+def test_prev_correct_chain_golden():
+    # tests/unit/models/test_metrics.py:326-370
+    prev = torch.ones(1, 4, dtype=torch.bool)
+    fc, ft, cc, ct = MT.accuracy_single_step(
+        torch.tensor([[1, 2, 3, 0]]), torch.tensor([[1, 2, 3, 4]]), None, prev)
+    assert (fc.item(), ft.item(), cc.item(), ct.item()) == (3, 4, 3, 4)
+    assert prev.tolist() == [[True, True, True, False]]
+    fc, ft, cc, ct = MT.accuracy_single_step(
+        torch.tensor([[1, 2, 0, 4]]), torch.tensor([[1, 2, 5, 4]]), None, prev)
+    assert prev.tolist() == [[True, True, False, False]]
+    assert (fc.item(), ft.item(), cc.item(), ct.item()) == (2, 4, 2, 3)
+
+
+def test_accuracy_single_step_with_mask_and_float_prev():
+    prev = torch.tensor([[1.0, 1.0, 0.0, 1.0, 1.0]])
+    mask = torch.tensor([[1.0, 0.0, 1.0, 1.0, 1.0]])
+    pred = torch.tensor([[5, 5, 5, 5, 1]])
+    tgt = torch.tensor([[5, 5, 5, 2, 1]])
+    fc, ft, cc, ct = MT.accuracy_single_step(pred, tgt, mask, prev)
+    # cond_total counted before the update over ALL rows of the view; counted rows: mask
+    assert ct.item() == 4 and ft.item() == 4
+    assert prev.tolist() == [[1.0, 1.0, 0.0, 0.0, 1.0]] and prev.dtype == torch.float32
+    assert fc.item() == 2 and cc.item() == 2  # rows 0 and 4 (row 1 is unmasked)
+
+
+def _ids_to_logits(ids, v):
+    out = torch.zeros(*ids.shape, v)
+    out.scatter_(-1, ids.unsqueeze(-1), 100.0)
+    return out
+
+
+def test_multi_step_per_position_counts_golden():
+    # tests/unit/models/test_dflash_metrics.py:90-132
+    logits = torch.tensor([[[0, 0, 1.0], [0, 1.0, 0], [1.0, 0, 0], [0, 1.0, 0]]])
+    tg = _ids_to_logits(torch.tensor([[2, 1, 0, 0]]), 3)
+    pos = torch.arange(4).unsqueeze(0) % 2
+    c, t = MT.accuracy_multi_step(logits.argmax(-1), tg.argmax(-1), torch.ones(1, 4), pos, 2)
+    assert c.tolist() == [2.0, 1.0] and t.tolist() == [2.0, 2.0]
+    tg = _ids_to_logits(torch.tensor([[2, 0, 0, 1]]), 3)
+    c, t = MT.accuracy_multi_step(logits.argmax(-1), tg.argmax(-1),
+                                  torch.tensor([[1, 0, 1, 1]]), pos, 2)
+    assert c.tolist() == [2.0, 1.0] and t.tolist() == [2.0, 1.0]
+    c, t = MT.accuracy_multi_step(logits.argmax(-1), tg.argmax(-1),
+                                  torch.zeros(1, 4), pos, 2)
+    assert c.sum().item() == 0 and t.sum().item() == 0
+
+
+def test_align_for_step_views():
+    t, v = 7, 5
+    logits = torch.arange(t * v, dtype=torch.float).reshape(1, t, v)
+    targets = -logits
+    mask = torch.arange(t).reshape(1, t)
+    prev = torch.ones(1, t)
+    for k in range(3):
+        a, b, m, p = MT.align_for_step(logits, targets, mask, prev, k)
+        assert a.shape[1] == b.shape[1] == m.shape[1] == p.shape[1] == t - k
+        assert torch.equal(a[0, 0], logits[0, 0]) and torch.equal(b[0, 0], targets[0, k])
+        assert m[0, 0].item() == k
+        p.zero_()  # a view: writes through
+        assert prev[0, : t - k].sum().item() == 0
+        prev.fill_(1)
+
+
+def test_eagle3_compute_metrics_brute_force_chain():
+    g = torch.Generator().manual_seed(3)
+    t, v, steps = 12, 6, 3
+    targets = torch.randn(1, t, v, generator=g)
+    mask = (torch.rand(1, t, generator=g) < 0.7).float()
+    prev = mask.clone()
+    ref_prev = mask[0].bool().tolist()
+    total = 0.0
+    for k in range(steps):
+        logits = torch.randn(1, t, v, generator=g)
+        # make many rows agree with the (shifted) target argmax
+        for i in range(0, t - k, 2):
+            logits[0, i, targets[0, i + k].argmax()] += 10
+        loss, m = MT.eagle3_compute_metrics(logits, targets, mask, prev, k, 0.8)
+        # brute force
+        cond_total = sum(ref_prev[: t - k])
+        corr = 0
+        num = 0.0
+        for i in range(t - k):
+            match = int(logits[0, i].argmax()) == int(targets[0, i + k].argmax())
+            ref_prev[i] = ref_prev[i] and match
+            if mask[0, i + k] > 0:
+                corr += int(ref_prev[i])
+                num += L.kl_div(logits[:, i:i + 1], targets[:, i + k:i + k + 1]).item()
+        den = mask[0, k:].sum().item() + 1e-5
+        assert m[f"cond_acc_{k}_total"].item() == cond_total
+        assert m[f"full_acc_{k}_sum"].item() == corr == m[f"cond_acc_{k}_sum"].item()
+        assert m[f"full_acc_{k}_total"].item() == mask[0, k:].sum().item()
+        assert loss.item() == pytest.approx(0.8 ** k * num / den, rel=1e-5)
+        assert prev[0].bool().tolist() == ref_prev
+        total += loss.item()
+
+
+def test_dflash_compute_metrics_keys_and_eal():
+    g = torch.Generator().manual_seed(1)
+    bs, a, v = 4, 3, 7
+    logits = torch.randn(1, a * bs, v, generator=g)
+    targets = torch.randn(1, a * bs, v, generator=g)
+    mask = torch.ones(1, a * bs); mask[:, ::bs] = 0
+    loss, m = MT.dflash_compute_metrics(logits, targets, mask, bs, gamma=4.0)
+    pos = (torch.arange(a * bs) % bs).float()
+    w = L.dflash_loss_decay(pos, 4.0)
+    expect = (L.kl_div(logits, targets)[0] * mask[0] * w).sum() / (mask.sum() + 1e-5)
+    assert loss.item() == pytest.approx(expect.item(), rel=1e-6)
+    acc = [m[f"position_{s}_acc_sum"] / m[f"position_{s}_acc_total"].clamp(min=1) for s in range(1, bs)]
+    eal = acc[0] + acc[0] * acc[1] + acc[0] * acc[1] * acc[2]
+    assert m["eal_sum"].item() == pytest.approx(eal.item(), abs=1e-6)
+    assert "position_0_acc_sum" not in m
+    assert m["full_acc_total"].item() == a * (bs - 1)
+
+
+def test_vocab_tables_closed_form_and_gather_identity():
+    g = torch.Generator().manual_seed(0)
+    vt, vd, h = 97, 31, 8
+    sel = torch.randperm(vt, generator=g)[:vd]
+    d2t, t2d = V.build_vocab_mappings(sel.tolist(), vt)
+    assert torch.equal(torch.nonzero(t2d).reshape(-1), torch.arange(vd) + d2t)
+    assert (d2t[1:] >= d2t[:-1]).all() and int(t2d.sum()) == vd
+    V.validate_vocab_mappings(t2d, d2t, vd, vt)
+    with pytest.raises(ValueError):
+        V.validate_vocab_mappings(t2d, d2t, vd + 1, vt)
+    w = torch.randn(vt, h, generator=g, dtype=torch.double)
+    x = torch.randn(5, h, generator=g, dtype=torch.double)
+    assert torch.allclose(V.gather_targets(x @ w.T, d2t), x @ w[t2d].T, atol=1e-12)
