@@ -1,0 +1,128 @@
+/*
+ * C-ABI of libspx_hip.so -- the MI355X (gfx950) kernels behind the draft-model
+ * training hot path of vllm-project/speculators.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its comment says "host";
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     every entry point only enqueues work on that stream and returns;
+ *   - the caller owns every buffer, workspaces included; entry points allocate
+ *     nothing;
+ *   - the return value is 0 on success, 1 for a rejected argument, 2 for a HIP
+ *     launch error; spx_last_error() holds the message (thread-local);
+ *   - `dtype` codes: 0 = bf16, 1 = f32.  Mask element codes (`*_kind`):
+ *     0 = 1-byte (bool / uint8), 1 = int32, 2 = int64, 3 = f32, 4 = bf16.
+ *   - reference citations are relative to src/speculators/ of the reference.
+ */
+#ifndef SPX_H
+#define SPX_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SPX_DTYPE_BF16 0
+#define SPX_DTYPE_F32 1
+
+#define SPX_KIND_U8 0
+#define SPX_KIND_I32 1
+#define SPX_KIND_I64 2
+#define SPX_KIND_F32 3
+#define SPX_KIND_BF16 4
+
+/* loss selector; the same five reductions as the `OP` constexpr of
+ * losses/fused.py:38-46 */
+#define SPX_LOSS_KL 0
+#define SPX_LOSS_RKL 1
+#define SPX_LOSS_JSD 2
+#define SPX_LOSS_CE 3
+#define SPX_LOSS_TV 4
+
+int spx_version(void);
+const char* spx_last_error(void); /* host string, valid until the next failing call on this thread */
+
+/* ---------------------------------------------------------------- vocabulary
+ * out[r, i] = full[r, i + d2t[i]]  (bit-exact copy of bf16 / f32 elements).
+ * Replaces the t2d row-slice of the verifier head, model.py:161-169, with a
+ * gather of full-vocabulary verifier logits through the d2t offset table of
+ * train/vocab_mapping.py:86-96.  Indices outside [0, vt) are rejected on the
+ * device by writing -inf (they cannot occur for a table built by the
+ * reference). */
+int spx_vocab_gather(const void* full, int64_t ld_full, const int64_t* d2t,
+                     void* out, int64_t ld_out, int64_t rows, int64_t vd,
+                     int64_t vt, int dtype, void* stream);
+
+/* ---------------------------------------------------------------- fused loss
+ * One streaming pass per row over a draft row and a target row:
+ *   loss[r]       row loss selected by `op` (fp32)
+ *   lse_draft[r]  log-sum-exp of the draft row,  lse_target[r] of the target row
+ *   extra[r]      kl/rkl: the row loss; jsd: KL(q||m); tv: sum of q where q<=p;
+ *                 ce: unused (the label is argmax_target[r])
+ *   argmax_draft[r], argmax_target[r]  first-index argmax (torch.argmax rule)
+ * Replaces loss_forward_kernel (losses/fused.py:91-175) and the two
+ * torch.argmax calls of compute_metrics (models/eagle3/metrics.py:100-101,
+ * models/dflash/metrics.py:77-78).  Row r of `logits` is paired with row r of
+ * `targets`; the TTT shift of align_for_step (models/eagle3/metrics.py:16-48)
+ * is a pointer offset made by the caller.  ld_* are row strides in elements.
+ * The argmax outputs may be NULL. */
+int spx_fused_vocab_loss_fwd(int op, const void* logits, int64_t ld_logits,
+                             const void* targets, int64_t ld_targets,
+                             int64_t rows, int64_t vocab, int dtype,
+                             float* loss, float* lse_draft, float* lse_target,
+                             float* extra, int32_t* argmax_draft,
+                             int32_t* argmax_target, void* stream);
+
+/* grad_logits[r, :] = g_r * dL_r/dlogits, g_r = row_grad[r] * (*scale)
+ * (scale may be NULL = 1).  Rows with g_r == 0 are written as exact zeros
+ * without reading the inputs.  Closed forms of losses/fused.py:11-18; replaces
+ * loss_backward_kernel (losses/fused.py:177-235).  grad dtype = `dtype`. */
+int spx_fused_vocab_loss_bwd(int op, const void* logits, int64_t ld_logits,
+                             const void* targets, int64_t ld_targets,
+                             int64_t rows, int64_t vocab, int dtype,
+                             const float* lse_draft, const float* lse_target,
+                             const float* extra, const int32_t* argmax_target,
+                             const float* row_grad, const float* scale,
+                             void* grad_logits, int64_t ld_grad, void* stream);
+
+/* Masked mean and acceptance chain of one TTT step over `rows` aligned rows:
+ *   out[0] = weight * sum_r loss[r] * m_r / (sum_r m_r + 1e-5)
+ *            (loss_function, losses/utils.py:269-304, with the exp_loss_decay
+ *            weight gamma**step, losses/utils.py:51-61, passed as `weight`)
+ *   out[1] = full_correct = out[3] = cond_correct
+ *            = #{r : m_r != 0 and prev_r and pred_r == tgt_r}
+ *   out[2] = full_total = #{r : m_r != 0}
+ *   out[4] = cond_total = #{r : prev_r}  counted BEFORE the update
+ *   out[5] = sum_r m_r
+ *   prev_correct[r] <- prev_correct[r] and (pred_r == tgt_r), in place
+ *   row_weight[r]   = weight * m_r / (sum m + 1e-5)   (d out[0] / d loss[r])
+ * Replaces the reduction of loss_function and compute_accuracy_single_step
+ * (models/metrics.py:6-36) as called from compute_metrics
+ * (models/eagle3/metrics.py:86-117).  `mask` / `prev_correct` may be NULL
+ * (all ones / not tracked: then cond_total = rows).  Counts are exact
+ * integers stored as fp32 (rows < 2^24).  Deterministic. */
+int spx_ttt_step_reduce(const float* loss, const int32_t* argmax_draft,
+                        const int32_t* argmax_target, const void* mask,
+                        int mask_kind, void* prev_correct, int prev_kind,
+                        int64_t rows, float weight, float* out,
+                        float* row_weight, void* stream);
+
+/* Weighted masked mean and per-slot acceptance counts of a DFlash block batch:
+ *   out[0] = sum_r loss[r] m_r w_r / (sum m + 1e-5),  out[1] = sum m
+ *   correct[s], total[s]  (s < block_size): matches / rows with m_r != 0 at
+ *   slot s = r % block_size   (compute_accuracy_multi_step, models/metrics.py:39-69)
+ *   row_weight[r] = m_r w_r / (sum m + 1e-5)
+ * `pos_weight` (fp32 [rows]) is the per-row weight: dflash_loss_decay
+ * (losses/utils.py:17-48) or the D-PACE weight (losses/utils.py:64-112);
+ * NULL = 1.  Replaces the reduction part of models/dflash/metrics.py:20-108. */
+int spx_block_reduce(const float* loss, const int32_t* argmax_draft,
+                     const int32_t* argmax_target, const void* mask,
+                     int mask_kind, const float* pos_weight, int64_t rows,
+                     int32_t block_size, float* out, float* correct,
+                     float* total, float* row_weight, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPX_H */

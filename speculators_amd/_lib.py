@@ -1,0 +1,98 @@
+"""ctypes binding of ``libspx_hip.so``.
+
+There is no CPU or PyTorch fallback: if the library is not built, or a call is
+made with tensors that are not on a HIP device, the call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libspx_hip.so")
+
+_P, _I64, _I, _F = c_void_p, c_int64, c_int, c_float
+
+# name -> argument types (all return int); mirrors include/spx.h
+SIGNATURES: dict[str, list] = {
+    "spx_vocab_gather": [_P, _I64, _P, _P, _I64, _I64, _I64, _I64, _I, _P],
+    "spx_fused_vocab_loss_fwd": [_I, _P, _I64, _P, _I64, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P],
+    "spx_fused_vocab_loss_bwd": [_I, _P, _I64, _P, _I64, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P,
+                                 _I64, _P],
+    "spx_ttt_step_reduce": [_P, _P, _P, _P, _I, _P, _I, _I64, _F, _P, _P, _P],
+    "spx_block_reduce": [_P, _P, _P, _P, _I, _P, _I64, c_int32, _P, _P, _P, _P, _P],
+}
+
+_lib = None
+
+
+class SpxError(RuntimeError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise SpxError(
+            f"{LIB_PATH} is missing: build it with `make -C speculators_amd/csrc` "
+            "(or __graft_entry__.build()); there is no fallback path"
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.spx_version.restype = c_int
+    lib.spx_version.argtypes = []
+    lib.spx_last_error.restype = c_char_p
+    lib.spx_last_error.argtypes = []
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = c_int
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def call(name: str, *args) -> None:
+    lib = load()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise SpxError(f"{name} failed ({rc}): {lib.spx_last_error().decode()}")
+
+
+def ptr(t: torch.Tensor | None):
+    """Device pointer of a tensor (None -> NULL).  Refuses host tensors."""
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise SpxError("libspx_hip works on HIP device tensors only (got a CPU tensor)")
+    return t.data_ptr()
+
+
+def stream_ptr(device=None):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+DTYPE_CODE = {torch.bfloat16: 0, torch.float32: 1}
+KIND_CODE = {
+    torch.bool: 0, torch.uint8: 0, torch.int8: 0, torch.int32: 1, torch.int64: 2,
+    torch.float32: 3, torch.bfloat16: 4,
+}
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    try:
+        return DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise SpxError(f"unsupported dtype {t.dtype}: bf16 and f32 only") from None
+
+
+def kind_code(t: torch.Tensor) -> int:
+    try:
+        return KIND_CODE[t.dtype]
+    except KeyError:
+        raise SpxError(f"unsupported mask dtype {t.dtype}") from None

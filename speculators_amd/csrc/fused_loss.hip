@@ -1,0 +1,612 @@
+// Fused vocabulary loss for gfx950: one workgroup streams one (draft row,
+// target row) pair with 16-byte loads, keeps online soft-max statistics of
+// both rows, the first-index arg-max of both rows and the loss reduction in
+// registers, and never materialises probabilities.  HBM-bound: algorithmic
+// traffic is 2 rows read (forward) and 2 rows read + 1 row written (backward).
+//
+// All exponentials run in the base-2 domain (v_exp_f32 is 2^x): logits are
+// pre-scaled by log2(e), statistics are converted back at the end.
+
+#include "spx_common.h"
+#include "../../include/spx.h"
+
+namespace spx {
+
+constexpr int kLossThreads = 256;
+constexpr int kLossWaves = kLossThreads / 64;
+
+// ---- 8-element chunk loads -------------------------------------------------
+// VEC: the row base is 16-byte aligned and the chunk is complete.
+template <typename T>
+__device__ __forceinline__ void load8_vec(const T* p, float v[8]);
+
+template <>
+__device__ __forceinline__ void load8_vec<uint16_t>(const uint16_t* p, float v[8]) {
+  u32x4 raw = *reinterpret_cast<const u32x4*>(p);
+  v[0] = bf16_lo(raw.x); v[1] = bf16_hi(raw.x);
+  v[2] = bf16_lo(raw.y); v[3] = bf16_hi(raw.y);
+  v[4] = bf16_lo(raw.z); v[5] = bf16_hi(raw.z);
+  v[6] = bf16_lo(raw.w); v[7] = bf16_hi(raw.w);
+}
+template <>
+__device__ __forceinline__ void load8_vec<float>(const float* p, float v[8]) {
+  f32x4 a = *reinterpret_cast<const f32x4*>(p);
+  f32x4 b = *reinterpret_cast<const f32x4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+  v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+__device__ __forceinline__ float load1(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+__device__ __forceinline__ float load1(const float* p) { return *p; }
+
+template <typename T>
+__device__ __forceinline__ void load8_guard(const T* p, int64_t base, int64_t n, float v[8]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = (base + i < n) ? load1(p + base + i) : kNegBig;
+}
+
+template <typename T, bool VEC>
+__device__ __forceinline__ void load8(const T* row, int64_t base, int64_t n, float v[8]) {
+  if (VEC && base + 8 <= n) load8_vec<T>(row + base, v);
+  else load8_guard<T>(row, base, n, v);
+}
+
+template <typename T>
+__device__ __forceinline__ void store8_vec(T* p, const float v[8]);
+template <>
+__device__ __forceinline__ void store8_vec<uint16_t>(uint16_t* p, const float v[8]) {
+  u32x4 raw;
+  raw.x = pack_bf16x2(v[0], v[1]); raw.y = pack_bf16x2(v[2], v[3]);
+  raw.z = pack_bf16x2(v[4], v[5]); raw.w = pack_bf16x2(v[6], v[7]);
+  *reinterpret_cast<u32x4*>(p) = raw;
+}
+template <>
+__device__ __forceinline__ void store8_vec<float>(float* p, const float v[8]) {
+  f32x4 a = {v[0], v[1], v[2], v[3]}, b = {v[4], v[5], v[6], v[7]};
+  *reinterpret_cast<f32x4*>(p) = a;
+  *reinterpret_cast<f32x4*>(p + 4) = b;
+}
+__device__ __forceinline__ void store1(uint16_t* p, float v) { *p = (uint16_t)f32_to_bf16_bits(v); }
+__device__ __forceinline__ void store1(float* p, float v) { *p = v; }
+
+template <typename T, bool VEC>
+__device__ __forceinline__ void store8(T* row, int64_t base, int64_t n, const float v[8]) {
+  if (VEC && base + 8 <= n) store8_vec<T>(row + base, v);
+  else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (base + i < n) store1(row + base + i, v[i]);
+  }
+}
+
+// ---- running statistics ----------------------------------------------------
+struct RowStats {
+  float md, zd;        // draft: running max (base-2 scaled) and sum of 2^(x' - md)
+  float mt, zt, at;    // target: same, and sum of 2^(y' - mt) * (y - x)
+  float bd; int id;    // draft arg-max value / first index
+  float bt; int it; float xt;  // target arg-max value / first index / draft logit there
+};
+
+__device__ __forceinline__ void merge(RowStats& a, const RowStats& b) {
+  float m = fmaxf(a.md, b.md);
+  a.zd = a.zd * fast_exp2(a.md - m) + b.zd * fast_exp2(b.md - m);
+  a.md = m;
+  m = fmaxf(a.mt, b.mt);
+  float ra = fast_exp2(a.mt - m), rb = fast_exp2(b.mt - m);
+  a.zt = a.zt * ra + b.zt * rb;
+  a.at = a.at * ra + b.at * rb;
+  a.mt = m;
+  if (b.bd > a.bd || (b.bd == a.bd && b.id < a.id)) { a.bd = b.bd; a.id = b.id; }
+  if (b.bt > a.bt || (b.bt == a.bt && b.it < a.it)) { a.bt = b.bt; a.it = b.it; a.xt = b.xt; }
+}
+
+__device__ __forceinline__ RowStats shuffle_xor(const RowStats& s, int m) {
+  RowStats o;
+  o.md = __shfl_xor(s.md, m, 64); o.zd = __shfl_xor(s.zd, m, 64);
+  o.mt = __shfl_xor(s.mt, m, 64); o.zt = __shfl_xor(s.zt, m, 64);
+  o.at = __shfl_xor(s.at, m, 64);
+  o.bd = __shfl_xor(s.bd, m, 64); o.id = __shfl_xor(s.id, m, 64);
+  o.bt = __shfl_xor(s.bt, m, 64); o.it = __shfl_xor(s.it, m, 64);
+  o.xt = __shfl_xor(s.xt, m, 64);
+  return o;
+}
+
+__device__ __forceinline__ float block_sum(float v, float* lds) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int w = 0; w < kLossWaves; ++w) t += lds[w];
+  return t;
+}
+
+// log((2^a' + 2^b')/2) in natural units from natural-log inputs
+__device__ __forceinline__ float log_mix(float la, float lb) {
+  float mx = fmaxf(la, lb);
+  float s = fast_exp2((la - mx) * kLog2e) + fast_exp2((lb - mx) * kLog2e);
+  return mx + fast_log2(s) * kLn2 - kLn2;
+}
+
+// ---- forward ---------------------------------------------------------------
+template <typename T, int OP, bool VEC>
+__global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
+    const T* __restrict__ logits, int64_t ld_logits, const T* __restrict__ targets,
+    int64_t ld_targets, int64_t vocab, float* __restrict__ loss, float* __restrict__ lse_draft,
+    float* __restrict__ lse_target, float* __restrict__ extra, int32_t* __restrict__ argmax_draft,
+    int32_t* __restrict__ argmax_target) {
+  const int64_t r = blockIdx.x;
+  const T* xrow = logits + r * ld_logits;
+  const T* yrow = targets + r * ld_targets;
+  const int tid = threadIdx.x;
+  const int64_t nchunks = (vocab + 7) >> 3;
+
+  RowStats s;
+  s.md = kNegBig; s.zd = 0.f; s.mt = kNegBig; s.zt = 0.f; s.at = 0.f;
+  s.bd = -INFINITY; s.id = 0x7fffffff; s.bt = -INFINITY; s.it = 0x7fffffff; s.xt = 0.f;
+
+  for (int64_t c = tid; c < nchunks; c += kLossThreads) {
+    const int64_t base = c << 3;
+    float x[8], y[8];
+    load8<T, VEC>(xrow, base, vocab, x);
+    load8<T, VEC>(yrow, base, vocab, y);
+    float cx = x[0], cy = y[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) { cx = fmaxf(cx, x[i]); cy = fmaxf(cy, y[i]); }
+    if (cx > s.bd) {  // strict: an earlier chunk of this thread keeps a tie
+      int k = 7;
+#pragma unroll
+      for (int i = 6; i >= 0; --i) k = (x[i] == cx) ? i : k;
+      s.bd = cx; s.id = (int)base + k;
+    }
+    if (cy > s.bt) {
+      int k = 7;
+      float xv = x[7];
+#pragma unroll
+      for (int i = 6; i >= 0; --i) {
+        const bool hit = y[i] == cy;
+        k = hit ? i : k;
+        xv = hit ? x[i] : xv;
+      }
+      s.bt = cy; s.it = (int)base + k; s.xt = xv;
+    }
+    {
+      float mn = fmaxf(s.md, cx * kLog2e);
+      float z = s.zd * fast_exp2(s.md - mn);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) z += fast_exp2(fmaf(x[i], kLog2e, -mn));
+      s.zd = z; s.md = mn;
+    }
+    if (OP != SPX_LOSS_CE) {
+      float mn = fmaxf(s.mt, cy * kLog2e);
+      float rs = fast_exp2(s.mt - mn);
+      float z = s.zt * rs, a = s.at * rs;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float e = fast_exp2(fmaf(y[i], kLog2e, -mn));
+        z += e;
+        a = fmaf(e, y[i] - x[i], a);
+      }
+      s.zt = z; s.at = a; s.mt = mn;
+    }
+  }
+
+  // tail padding must never win an arg-max: padded values are kNegBig, and
+  // a padded index only enters when cx == kNegBig > -inf on an all-padding
+  // chunk, which cannot exist (every chunk holds at least one real element).
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) merge(s, shuffle_xor(s, m));
+
+  __shared__ RowStats part[kLossWaves];
+  __shared__ float red[kLossWaves];
+  if ((tid & 63) == 0) part[tid >> 6] = s;
+  __syncthreads();
+  s = part[0];
+#pragma unroll
+  for (int w = 1; w < kLossWaves; ++w) merge(s, part[w]);
+
+  const float lse_d = (s.md + fast_log2(s.zd)) * kLn2;
+  const float lse_t = (OP != SPX_LOSS_CE) ? (s.mt + fast_log2(s.zt)) * kLn2 : 0.f;
+
+  float row_loss = 0.f, row_extra = 0.f;
+  if (OP == SPX_LOSS_KL) {
+    row_loss = s.at / s.zt - lse_t + lse_d;
+    row_extra = row_loss;
+  } else if (OP == SPX_LOSS_CE) {
+    row_loss = lse_d - s.xt;
+  } else {
+    // second streaming pass (the row pair is L2 resident by now)
+    float acc = 0.f, ext = 0.f;
+    for (int64_t c = tid; c < nchunks; c += kLossThreads) {
+      const int64_t base = c << 3;
+      float x[8], y[8];
+      load8<T, VEC>(xrow, base, vocab, x);
+      load8<T, VEC>(yrow, base, vocab, y);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float ldp = x[i] - lse_d, ltp = y[i] - lse_t;
+        float dp = fast_exp2(ldp * kLog2e), tp = fast_exp2(ltp * kLog2e);
+        if (OP == SPX_LOSS_RKL) {
+          acc = fmaf(dp, ldp - ltp, acc);
+        } else if (OP == SPX_LOSS_JSD) {
+          float lm = log_mix(ldp, ltp);
+          acc = fmaf(dp, ldp - lm, acc);
+          ext = fmaf(tp, ltp - lm, ext);
+        } else {  // TV
+          acc += fminf(dp, tp);
+          ext += (dp <= tp) ? dp : 0.f;
+        }
+      }
+    }
+    acc = block_sum(acc, red);
+    if (OP != SPX_LOSS_RKL) ext = block_sum(ext, red);
+    if (OP == SPX_LOSS_RKL) { row_loss = acc; row_extra = acc; }
+    else if (OP == SPX_LOSS_JSD) { row_loss = 0.5f * (acc + ext); row_extra = acc; }
+    else { row_loss = 1.f - acc; row_extra = ext; }
+  }
+  if (tid == 0) {
+    loss[r] = row_loss;
+    lse_draft[r] = lse_d;
+    lse_target[r] = lse_t;
+    extra[r] = row_extra;
+    if (argmax_draft) argmax_draft[r] = s.id;
+    if (argmax_target) argmax_target[r] = s.it;
+  }
+}
+
+// ---- backward --------------------------------------------------------------
+template <typename T, int OP, bool VEC>
+__global__ __launch_bounds__(kLossThreads) void loss_bwd_kernel(
+    const T* __restrict__ logits, int64_t ld_logits, const T* __restrict__ targets,
+    int64_t ld_targets, int64_t vocab, const float* __restrict__ lse_draft,
+    const float* __restrict__ lse_target, const float* __restrict__ extra,
+    const int32_t* __restrict__ argmax_target, const float* __restrict__ row_grad,
+    const float* __restrict__ scale, T* __restrict__ grad, int64_t ld_grad) {
+  const int64_t r = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int64_t nchunks = (vocab + 7) >> 3;
+  T* grow = grad + r * ld_grad;
+  float g = row_grad[r];
+  if (scale) g *= *scale;
+  if (g == 0.f) {
+    const float z[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int64_t c = tid; c < nchunks; c += kLossThreads) store8<T, VEC>(grow, c << 3, vocab, z);
+    return;
+  }
+  const T* xrow = logits + r * ld_logits;
+  const T* yrow = (OP != SPX_LOSS_CE) ? targets + r * ld_targets : nullptr;
+  const float lse_d = lse_draft[r];
+  const float lse_t = (OP != SPX_LOSS_CE) ? lse_target[r] : 0.f;
+  const float ex = (OP == SPX_LOSS_RKL || OP == SPX_LOSS_JSD || OP == SPX_LOSS_TV) ? extra[r] : 0.f;
+  const int label = (OP == SPX_LOSS_CE) ? argmax_target[r] : -1;
+  const float cd = -lse_d * kLog2e, ct = -lse_t * kLog2e;
+
+  for (int64_t c = tid; c < nchunks; c += kLossThreads) {
+    const int64_t base = c << 3;
+    float x[8], y[8], o[8];
+    load8<T, VEC>(xrow, base, vocab, x);
+    if (OP != SPX_LOSS_CE) load8<T, VEC>(yrow, base, vocab, y);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (OP == SPX_LOSS_CE) {
+        float dp = fast_exp2(fmaf(x[i], kLog2e, cd));
+        o[i] = g * (dp - (((int)base + i) == label ? 1.f : 0.f));
+      } else if (OP == SPX_LOSS_KL) {
+        float dp = fast_exp2(fmaf(x[i], kLog2e, cd));
+        float tp = fast_exp2(fmaf(y[i], kLog2e, ct));
+        o[i] = g * (dp - tp);
+      } else {
+        // same expressions as the forward's second pass, so that the
+        // q <= p comparison of tv resolves identically in both directions
+        float ldp = x[i] - lse_d, ltp = y[i] - lse_t;
+        float dp = fast_exp2(ldp * kLog2e), tp = fast_exp2(ltp * kLog2e);
+        if (OP == SPX_LOSS_RKL) o[i] = g * dp * (ldp - ltp - ex);
+        else if (OP == SPX_LOSS_JSD) o[i] = g * 0.5f * dp * (ldp - log_mix(ldp, ltp) - ex);
+        else o[i] = -g * dp * ((dp <= tp ? 1.f : 0.f) - ex);
+      }
+    }
+    store8<T, VEC>(grow, base, vocab, o);
+  }
+}
+
+// ---- gather through the d2t offset table -------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void vocab_gather_kernel(
+    const T* __restrict__ full, int64_t ld_full, const int64_t* __restrict__ d2t,
+    T* __restrict__ out, int64_t ld_out, int64_t vd, int64_t vt, T neg_inf_bits) {
+  const int64_t r = blockIdx.y;
+  const T* src = full + r * ld_full;
+  T* dst = out + r * ld_out;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < vd; i += (int64_t)gridDim.x * 256) {
+    int64_t j = i + d2t[i];
+    dst[i] = (j >= 0 && j < vt) ? src[j] : neg_inf_bits;
+  }
+}
+
+// ---- mask element access ---------------------------------------------------
+__device__ __forceinline__ float mask_value(const void* p, int kind, int64_t i) {
+  switch (kind) {
+    case SPX_KIND_U8: return (float)reinterpret_cast<const uint8_t*>(p)[i];
+    case SPX_KIND_I32: return (float)reinterpret_cast<const int32_t*>(p)[i];
+    case SPX_KIND_I64: return (float)reinterpret_cast<const int64_t*>(p)[i];
+    case SPX_KIND_F32: return reinterpret_cast<const float*>(p)[i];
+    default: return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+  }
+}
+__device__ __forceinline__ void store_flag(void* p, int kind, int64_t i, bool v) {
+  switch (kind) {
+    case SPX_KIND_U8: reinterpret_cast<uint8_t*>(p)[i] = v ? 1 : 0; break;
+    case SPX_KIND_I32: reinterpret_cast<int32_t*>(p)[i] = v ? 1 : 0; break;
+    case SPX_KIND_I64: reinterpret_cast<int64_t*>(p)[i] = v ? 1 : 0; break;
+    case SPX_KIND_F32: reinterpret_cast<float*>(p)[i] = v ? 1.f : 0.f; break;
+    default: reinterpret_cast<uint16_t*>(p)[i] = v ? 0x3f80 : 0; break;
+  }
+}
+
+constexpr int kReduceThreads = 1024;
+
+__device__ __forceinline__ float block_sum_f(float v, float* lds) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int w = 0; w < kReduceThreads / 64; ++w) t += lds[w];
+  return t;
+}
+__device__ __forceinline__ int block_sum_i(int v, int* lds) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  int t = 0;
+  for (int w = 0; w < kReduceThreads / 64; ++w) t += lds[w];
+  return t;
+}
+
+__global__ __launch_bounds__(kReduceThreads) void ttt_step_reduce_kernel(
+    const float* __restrict__ loss, const int32_t* __restrict__ pred,
+    const int32_t* __restrict__ tgt, const void* __restrict__ mask, int mask_kind,
+    void* prev, int prev_kind, int64_t rows, float weight, float* __restrict__ out,
+    float* __restrict__ row_weight) {
+  __shared__ float fl[kReduceThreads / 64];
+  __shared__ int il[kReduceThreads / 64];
+  float lsum = 0.f, msum = 0.f;
+  int full_total = 0, correct = 0, cond_total = 0;
+  for (int64_t r = threadIdx.x; r < rows; r += kReduceThreads) {
+    float m = mask ? mask_value(mask, mask_kind, r) : 1.f;
+    bool was = prev ? (mask_value(prev, prev_kind, r) != 0.f) : true;
+    bool hit = pred[r] == tgt[r];
+    bool now = was && hit;
+    cond_total += was ? 1 : 0;
+    if (prev) store_flag(prev, prev_kind, r, now);
+    if (m != 0.f) { full_total += 1; correct += now ? 1 : 0; }
+    lsum = fmaf(loss[r], m, lsum);
+    msum += m;
+  }
+  lsum = block_sum_f(lsum, fl);
+  msum = block_sum_f(msum, fl);
+  full_total = block_sum_i(full_total, il);
+  correct = block_sum_i(correct, il);
+  cond_total = block_sum_i(cond_total, il);
+  const float inv = weight / (msum + 1e-5f);
+  if (threadIdx.x == 0) {
+    out[0] = lsum * inv;
+    out[1] = (float)correct;
+    out[2] = (float)full_total;
+    out[3] = (float)correct;
+    out[4] = prev ? (float)cond_total : (float)rows;
+    out[5] = msum;
+  }
+  if (row_weight) {
+    for (int64_t r = threadIdx.x; r < rows; r += kReduceThreads) {
+      float m = mask ? mask_value(mask, mask_kind, r) : 1.f;
+      row_weight[r] = m * inv;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kReduceThreads) void block_reduce_kernel(
+    const float* __restrict__ loss, const int32_t* __restrict__ pred,
+    const int32_t* __restrict__ tgt, const void* __restrict__ mask, int mask_kind,
+    const float* __restrict__ pos_weight, int64_t rows, int block_size, float* __restrict__ out,
+    float* __restrict__ correct, float* __restrict__ total, float* __restrict__ row_weight) {
+  __shared__ float fl[kReduceThreads / 64];
+  extern __shared__ int slots[];  // [2 * block_size]
+  for (int i = threadIdx.x; i < 2 * block_size; i += kReduceThreads) slots[i] = 0;
+  __syncthreads();
+  float lsum = 0.f, msum = 0.f;
+  for (int64_t r = threadIdx.x; r < rows; r += kReduceThreads) {
+    float m = mask ? mask_value(mask, mask_kind, r) : 1.f;
+    float w = pos_weight ? pos_weight[r] : 1.f;
+    if (m != 0.f) {
+      int s = (int)(r % block_size);
+      atomicAdd(&slots[block_size + s], 1);
+      if (pred[r] == tgt[r]) atomicAdd(&slots[s], 1);
+    }
+    lsum = fmaf(loss[r] * m, w, lsum);
+    msum += m;
+  }
+  lsum = block_sum_f(lsum, fl);
+  msum = block_sum_f(msum, fl);
+  const float inv = 1.f / (msum + 1e-5f);
+  if (threadIdx.x == 0) { out[0] = lsum * inv; out[1] = msum; }
+  __syncthreads();
+  for (int i = threadIdx.x; i < block_size; i += kReduceThreads) {
+    correct[i] = (float)slots[i];
+    total[i] = (float)slots[block_size + i];
+  }
+  if (row_weight) {
+    for (int64_t r = threadIdx.x; r < rows; r += kReduceThreads) {
+      float m = mask ? mask_value(mask, mask_kind, r) : 1.f;
+      float w = pos_weight ? pos_weight[r] : 1.f;
+      row_weight[r] = m * w * inv;
+    }
+  }
+}
+
+// ---- dispatch ----------------------------------------------------------------
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <typename T, bool VEC>
+static void launch_fwd(int op, const T* lg, int64_t ldl, const T* tg, int64_t ldt, int64_t rows,
+                       int64_t vocab, float* loss, float* lsd, float* lst, float* ex, int32_t* ad,
+                       int32_t* at, hipStream_t st) {
+  dim3 grid((unsigned)rows), block(kLossThreads);
+#define SPX_FWD(OPV)                                                                         \
+  case OPV:                                                                                  \
+    hipLaunchKernelGGL((loss_fwd_kernel<T, OPV, VEC>), grid, block, 0, st, lg, ldl, tg, ldt, \
+                       vocab, loss, lsd, lst, ex, ad, at);                                   \
+    break;
+  switch (op) {
+    SPX_FWD(SPX_LOSS_KL) SPX_FWD(SPX_LOSS_RKL) SPX_FWD(SPX_LOSS_JSD) SPX_FWD(SPX_LOSS_CE)
+    SPX_FWD(SPX_LOSS_TV)
+  }
+#undef SPX_FWD
+}
+
+template <typename T, bool VEC>
+static void launch_bwd(int op, const T* lg, int64_t ldl, const T* tg, int64_t ldt, int64_t rows,
+                       int64_t vocab, const float* lsd, const float* lst, const float* ex,
+                       const int32_t* at, const float* rg, const float* sc, T* grad, int64_t ldg,
+                       hipStream_t st) {
+  dim3 grid((unsigned)rows), block(kLossThreads);
+#define SPX_BWD(OPV)                                                                         \
+  case OPV:                                                                                  \
+    hipLaunchKernelGGL((loss_bwd_kernel<T, OPV, VEC>), grid, block, 0, st, lg, ldl, tg, ldt, \
+                       vocab, lsd, lst, ex, at, rg, sc, grad, ldg);                          \
+    break;
+  switch (op) {
+    SPX_BWD(SPX_LOSS_KL) SPX_BWD(SPX_LOSS_RKL) SPX_BWD(SPX_LOSS_JSD) SPX_BWD(SPX_LOSS_CE)
+    SPX_BWD(SPX_LOSS_TV)
+  }
+#undef SPX_BWD
+}
+
+}  // namespace spx
+
+using namespace spx;
+
+extern "C" int spx_fused_vocab_loss_fwd(int op, const void* logits, int64_t ld_logits,
+                                        const void* targets, int64_t ld_targets, int64_t rows,
+                                        int64_t vocab, int dtype, float* loss, float* lse_draft,
+                                        float* lse_target, float* extra, int32_t* argmax_draft,
+                                        int32_t* argmax_target, void* stream) {
+  SPX_REQUIRE(op >= SPX_LOSS_KL && op <= SPX_LOSS_TV, "unknown loss op");
+  SPX_REQUIRE(dtype == SPX_DTYPE_BF16 || dtype == SPX_DTYPE_F32, "dtype must be bf16 or f32");
+  SPX_REQUIRE(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "rows >= 0 and 0 < vocab < 2^31");
+  SPX_REQUIRE(ld_logits >= vocab && ld_targets >= vocab, "row stride smaller than vocab");
+  SPX_REQUIRE(rows < (1ll << 31), "too many rows");
+  if (rows == 0) return SPX_OK;
+  SPX_REQUIRE(logits && targets && loss && lse_draft && lse_target && extra, "null buffer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int64_t per16 = dtype == SPX_DTYPE_BF16 ? 8 : 4;
+  const bool vec = aligned16(logits) && aligned16(targets) && ld_logits % per16 == 0 &&
+                   ld_targets % per16 == 0;
+  if (dtype == SPX_DTYPE_BF16) {
+    auto lg = reinterpret_cast<const uint16_t*>(logits);
+    auto tg = reinterpret_cast<const uint16_t*>(targets);
+    if (vec) launch_fwd<uint16_t, true>(op, lg, ld_logits, tg, ld_targets, rows, vocab, loss, lse_draft, lse_target, extra, argmax_draft, argmax_target, st);
+    else launch_fwd<uint16_t, false>(op, lg, ld_logits, tg, ld_targets, rows, vocab, loss, lse_draft, lse_target, extra, argmax_draft, argmax_target, st);
+  } else {
+    auto lg = reinterpret_cast<const float*>(logits);
+    auto tg = reinterpret_cast<const float*>(targets);
+    if (vec) launch_fwd<float, true>(op, lg, ld_logits, tg, ld_targets, rows, vocab, loss, lse_draft, lse_target, extra, argmax_draft, argmax_target, st);
+    else launch_fwd<float, false>(op, lg, ld_logits, tg, ld_targets, rows, vocab, loss, lse_draft, lse_target, extra, argmax_draft, argmax_target, st);
+  }
+  return check_launch(__func__);
+}
+
+extern "C" int spx_fused_vocab_loss_bwd(int op, const void* logits, int64_t ld_logits,
+                                        const void* targets, int64_t ld_targets, int64_t rows,
+                                        int64_t vocab, int dtype, const float* lse_draft,
+                                        const float* lse_target, const float* extra,
+                                        const int32_t* argmax_target, const float* row_grad,
+                                        const float* scale, void* grad_logits, int64_t ld_grad,
+                                        void* stream) {
+  SPX_REQUIRE(op >= SPX_LOSS_KL && op <= SPX_LOSS_TV, "unknown loss op");
+  SPX_REQUIRE(dtype == SPX_DTYPE_BF16 || dtype == SPX_DTYPE_F32, "dtype must be bf16 or f32");
+  SPX_REQUIRE(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "rows >= 0 and 0 < vocab < 2^31");
+  SPX_REQUIRE(ld_logits >= vocab && ld_grad >= vocab, "row stride smaller than vocab");
+  SPX_REQUIRE(rows < (1ll << 31), "too many rows");
+  if (rows == 0) return SPX_OK;
+  SPX_REQUIRE(logits && grad_logits && lse_draft && row_grad, "null buffer");
+  if (op == SPX_LOSS_CE) SPX_REQUIRE(argmax_target, "ce needs argmax_target");
+  else SPX_REQUIRE(targets && lse_target && ld_targets >= vocab, "targets / lse_target missing");
+  if (op == SPX_LOSS_RKL || op == SPX_LOSS_JSD || op == SPX_LOSS_TV) SPX_REQUIRE(extra, "extra missing");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int64_t per16 = dtype == SPX_DTYPE_BF16 ? 8 : 4;
+  const bool vec = aligned16(logits) && (op == SPX_LOSS_CE || (aligned16(targets) && ld_targets % per16 == 0)) &&
+                   aligned16(grad_logits) && ld_logits % per16 == 0 && ld_grad % per16 == 0;
+  if (dtype == SPX_DTYPE_BF16) {
+    auto lg = reinterpret_cast<const uint16_t*>(logits);
+    auto tg = reinterpret_cast<const uint16_t*>(targets);
+    auto gr = reinterpret_cast<uint16_t*>(grad_logits);
+    if (vec) launch_bwd<uint16_t, true>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, st);
+    else launch_bwd<uint16_t, false>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, st);
+  } else {
+    auto lg = reinterpret_cast<const float*>(logits);
+    auto tg = reinterpret_cast<const float*>(targets);
+    auto gr = reinterpret_cast<float*>(grad_logits);
+    if (vec) launch_bwd<float, true>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, st);
+    else launch_bwd<float, false>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, st);
+  }
+  return check_launch(__func__);
+}
+
+extern "C" int spx_vocab_gather(const void* full, int64_t ld_full, const int64_t* d2t, void* out,
+                                int64_t ld_out, int64_t rows, int64_t vd, int64_t vt, int dtype,
+                                void* stream) {
+  SPX_REQUIRE(dtype == SPX_DTYPE_BF16 || dtype == SPX_DTYPE_F32, "dtype must be bf16 or f32");
+  SPX_REQUIRE(rows >= 0 && vd > 0 && vt > 0, "rows >= 0, vd > 0, vt > 0");
+  SPX_REQUIRE(ld_full >= vt && ld_out >= vd, "row stride smaller than the row");
+  SPX_REQUIRE(rows < 65536, "at most 65535 rows per call");
+  if (rows == 0) return SPX_OK;
+  SPX_REQUIRE(full && d2t && out, "null buffer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  unsigned gx = (unsigned)((vd + 256 * 4 - 1) / (256 * 4));
+  dim3 grid(gx, (unsigned)rows), block(256);
+  if (dtype == SPX_DTYPE_BF16)
+    hipLaunchKernelGGL(vocab_gather_kernel<uint16_t>, grid, block, 0, st,
+                       reinterpret_cast<const uint16_t*>(full), ld_full, d2t,
+                       reinterpret_cast<uint16_t*>(out), ld_out, vd, vt, (uint16_t)0xff80);
+  else
+    hipLaunchKernelGGL(vocab_gather_kernel<float>, grid, block, 0, st,
+                       reinterpret_cast<const float*>(full), ld_full, d2t,
+                       reinterpret_cast<float*>(out), ld_out, vd, vt, -INFINITY);
+  return check_launch(__func__);
+}
+
+static bool kind_ok(int k) { return k >= SPX_KIND_U8 && k <= SPX_KIND_BF16; }
+
+extern "C" int spx_ttt_step_reduce(const float* loss, const int32_t* argmax_draft,
+                                   const int32_t* argmax_target, const void* mask, int mask_kind,
+                                   void* prev_correct, int prev_kind, int64_t rows, float weight,
+                                   float* out, float* row_weight, void* stream) {
+  SPX_REQUIRE(rows >= 0 && rows < (1ll << 24), "0 <= rows < 2^24");
+  SPX_REQUIRE(loss && argmax_draft && argmax_target && out, "null buffer");
+  SPX_REQUIRE(!mask || kind_ok(mask_kind), "unknown mask element kind");
+  SPX_REQUIRE(!prev_correct || kind_ok(prev_kind), "unknown prev_correct element kind");
+  hipLaunchKernelGGL(ttt_step_reduce_kernel, dim3(1), dim3(kReduceThreads), 0,
+                     reinterpret_cast<hipStream_t>(stream), loss, argmax_draft, argmax_target, mask,
+                     mask_kind, prev_correct, prev_kind, rows, weight, out, row_weight);
+  return check_launch(__func__);
+}
+
+extern "C" int spx_block_reduce(const float* loss, const int32_t* argmax_draft,
+                                const int32_t* argmax_target, const void* mask, int mask_kind,
+                                const float* pos_weight, int64_t rows, int32_t block_size,
+                                float* out, float* correct, float* total, float* row_weight,
+                                void* stream) {
+  SPX_REQUIRE(rows >= 0 && rows < (1ll << 24), "0 <= rows < 2^24");
+  SPX_REQUIRE(block_size > 0 && block_size <= 4096, "0 < block_size <= 4096");
+  SPX_REQUIRE(loss && argmax_draft && argmax_target && out && correct && total, "null buffer");
+  SPX_REQUIRE(!mask || kind_ok(mask_kind), "unknown mask element kind");
+  hipLaunchKernelGGL(block_reduce_kernel, dim3(1), dim3(kReduceThreads),
+                     2 * block_size * sizeof(int), reinterpret_cast<hipStream_t>(stream), loss,
+                     argmax_draft, argmax_target, mask, mask_kind, pos_weight, rows, block_size, out,
+                     correct, total, row_weight);
+  return check_launch(__func__);
+}

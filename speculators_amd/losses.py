@@ -1,0 +1,198 @@
+"""Loss-function registry backed by the HIP fused vocabulary loss.
+
+Mirror of the reference's loss plug-in (``speculators/losses/utils.py``): a
+``LossConfig`` is ``{name: (fn(logits, targets) -> [B, T] float32, weight)}``
+(losses/utils.py:12-14) and ``resolve_loss_config(spec, implementation)``
+(losses/utils.py:184-230) turns ``"kl_div"`` or a JSON dict of weights into
+one.  The implementation name registered here is ``"hip"``; its functions are
+differentiable with respect to ``logits`` only, like the reference's fused
+losses (losses/fused.py:238-291).
+"""
+
+from __future__ import annotations
+
+import json
+from collections.abc import Callable
+
+import torch
+
+from . import _lib
+
+LossConfig = dict[str, tuple[Callable[[torch.Tensor, torch.Tensor], torch.Tensor], float]]
+
+OP_KL, OP_RKL, OP_JSD, OP_CE, OP_TV = 0, 1, 2, 3, 4
+_NLA_EPS = 1e-5  # losses/fused.py:294
+
+
+def _rows_2d(t: torch.Tensor) -> torch.Tensor:
+    """[B, T, V] -> [B*T, V] view with unit inner stride (copies only if the
+    vocabulary axis itself is strided or the rows are not equally spaced)."""
+    v = t.shape[-1]
+    if t.stride(-1) != 1:
+        t = t.contiguous()
+    try:
+        return t.view(-1, v)
+    except RuntimeError:
+        return t.reshape(-1, v)
+
+
+def fused_loss_forward(op: int, logits: torch.Tensor, targets: torch.Tensor):
+    """Run the forward kernel.  Returns (loss [R] f32, lse_d, lse_t, extra,
+    argmax_draft [R] i32, argmax_target [R] i32, logits2d, targets2d)."""
+    if logits.shape != targets.shape:
+        raise ValueError(f"logits {tuple(logits.shape)} and targets {tuple(targets.shape)} differ")
+    if logits.dtype != targets.dtype:
+        targets = targets.to(logits.dtype)
+    x, y = _rows_2d(logits), _rows_2d(targets)
+    rows, vocab = x.shape
+    dev = x.device
+    stats = torch.empty(4, rows, device=dev, dtype=torch.float32)
+    arg = torch.empty(2, rows, device=dev, dtype=torch.int32)
+    _lib.call(
+        "spx_fused_vocab_loss_fwd", op, _lib.ptr(x), x.stride(0), _lib.ptr(y), y.stride(0),
+        rows, vocab, _lib.dtype_code(x), _lib.ptr(stats[0]), _lib.ptr(stats[1]),
+        _lib.ptr(stats[2]), _lib.ptr(stats[3]), _lib.ptr(arg[0]), _lib.ptr(arg[1]),
+        _lib.stream_ptr(dev),
+    )
+    return stats[0], stats[1], stats[2], stats[3], arg[0], arg[1], x, y
+
+
+class _FusedLoss(torch.autograd.Function):
+    """``(logits, targets, op) -> (row_loss [B, T] f32, argmax_draft, argmax_target)``;
+    the autograd counterpart of ``_FusedLoss`` in losses/fused.py:238-291.  Targets
+    get no gradient."""
+
+    @staticmethod
+    def forward(ctx, logits, targets, op):
+        loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, logits, targets)
+        ctx.save_for_backward(x, None if op == OP_CE else y, lse_d, lse_t, extra, am_t)
+        ctx.op = op
+        ctx.shape = logits.shape
+        lead = logits.shape[:-1]
+        am_d, am_t = am_d.view(lead), am_t.view(lead)
+        ctx.mark_non_differentiable(am_d, am_t)
+        return loss.view(lead), am_d, am_t
+
+    @staticmethod
+    def backward(ctx, grad_rows, _gd, _gt):
+        x, y, lse_d, lse_t, extra, am_t = ctx.saved_tensors
+        rows, vocab = x.shape
+        g = grad_rows.reshape(-1).to(torch.float32).contiguous()
+        grad = torch.empty(rows, vocab, device=x.device, dtype=x.dtype)
+        _lib.call(
+            "spx_fused_vocab_loss_bwd", ctx.op, _lib.ptr(x), x.stride(0), _lib.ptr(y),
+            y.stride(0) if y is not None else 0, rows, vocab, _lib.dtype_code(x),
+            _lib.ptr(lse_d), _lib.ptr(lse_t), _lib.ptr(extra), _lib.ptr(am_t), _lib.ptr(g), None,
+            _lib.ptr(grad), grad.stride(0), _lib.stream_ptr(x.device),
+        )
+        return grad.view(ctx.shape), None, None
+
+
+def fused_rows(op: int, logits, targets):
+    """(row_loss, argmax_draft, argmax_target) of one primitive reduction."""
+    return _FusedLoss.apply(logits, targets, op)
+
+
+def kl_div_loss(logits, targets):
+    return fused_rows(OP_KL, logits, targets)[0]
+
+
+def reverse_kl_div_loss(logits, targets):
+    return fused_rows(OP_RKL, logits, targets)[0]
+
+
+def js_div_loss(logits, targets):
+    return fused_rows(OP_JSD, logits, targets)[0]
+
+
+def ce_loss(logits, targets):
+    return fused_rows(OP_CE, logits, targets)[0]
+
+
+def tv_loss(logits, targets):
+    return fused_rows(OP_TV, logits, targets)[0]
+
+
+def neg_log_acceptance_loss(logits, targets):
+    """-log(max(1 - tv, 1e-5)) composed on the [B, T] tv rows (losses/fused.py:322-324)."""
+    return -torch.log((1.0 - tv_loss(logits, targets)).clamp_min(_NLA_EPS))
+
+
+def lk_hybrid_loss(logits, targets, eta: float = 3.0):
+    """lam*kl + (1-lam)*tv with lam = exp(-eta*stopgrad(1-tv)) (losses/fused.py:327-334)."""
+    kl = kl_div_loss(logits, targets)
+    tv = tv_loss(logits, targets)
+    lam = torch.exp(-eta * (1.0 - tv).detach())
+    return lam * kl + (1.0 - lam) * tv
+
+
+_HIP_LOSS_FN_MAP: dict[str, Callable] = {
+    "kl_div": kl_div_loss,
+    "rkl": reverse_kl_div_loss,
+    "jsd": js_div_loss,
+    "ce": ce_loss,
+    "tv": tv_loss,
+    "nla": neg_log_acceptance_loss,
+    "lk_hybrid": lk_hybrid_loss,
+}
+
+# which primitive kernel reduction also yields the arg-maxes for a named loss
+PRIMITIVE_OP = {"kl_div": OP_KL, "rkl": OP_RKL, "jsd": OP_JSD, "ce": OP_CE, "tv": OP_TV}
+
+_LOSS_FN_MAPS = {"hip": _HIP_LOSS_FN_MAP}
+
+
+def resolve_loss_config(spec: str, implementation: str = "hip") -> LossConfig:
+    """``"kl_div"`` or ``'{"ce": 0.1, "tv": 0.9}'`` -> ``{name: (fn, weight)}`` with the
+    error behaviour of losses/utils.py:184-230."""
+    try:
+        table = _LOSS_FN_MAPS[implementation]
+    except KeyError:
+        raise ValueError(
+            f"Unknown loss implementation '{implementation}'. Choose from: {sorted(_LOSS_FN_MAPS)}"
+        ) from None
+    if spec in table:
+        return {spec: (table[spec], 1.0)}
+    try:
+        parsed = json.loads(spec)
+    except json.JSONDecodeError:
+        raise ValueError(
+            f"Unknown loss function '{spec}'. Pass a known name ({sorted(table)}) or a JSON dict, "
+            'e.g. \'{"ce": 0.1, "tv": 0.9}\'.'
+        ) from None
+    if not isinstance(parsed, dict) or not parsed:
+        raise ValueError(
+            "Loss config must be a non-empty JSON dict mapping loss names to weights, "
+            f'e.g. \'{{"ce": 0.1, "tv": 0.9}}\'. Got: {spec}'
+        )
+    out: LossConfig = {}
+    for name, weight in parsed.items():
+        if name not in table:
+            raise ValueError(
+                f"Unknown loss function '{name}' in loss config. Choose from: {sorted(table)}"
+            )
+        if isinstance(weight, bool) or not isinstance(weight, (int, float)):
+            raise ValueError(
+                f"Loss weight for '{name}' must be a number, got {type(weight).__name__}"
+            )
+        out[name] = (table[name], float(weight))
+    return out
+
+
+def vocab_gather(full_logits: torch.Tensor, d2t: torch.Tensor) -> torch.Tensor:
+    """``full_logits[..., i + d2t[i]]`` on the device: verifier logits over the target
+    vocabulary restricted to the draft vocabulary (the gather form of the t2d row-slice,
+    model.py:161-169, with the offset table of train/vocab_mapping.py:86-96)."""
+    x = _rows_2d(full_logits)
+    rows, vt = x.shape
+    vd = d2t.numel()
+    d2t = d2t.to(device=x.device, dtype=torch.int64).contiguous()
+    out = torch.empty(rows, vd, device=x.device, dtype=x.dtype)
+    done = 0
+    while done < rows:  # the gather grid carries rows in its y dimension
+        n = min(rows - done, 65535)
+        xs, os_ = x[done:done + n], out[done:done + n]
+        _lib.call("spx_vocab_gather", _lib.ptr(xs), x.stride(0), _lib.ptr(d2t), _lib.ptr(os_),
+                  out.stride(0), n, vd, vt, _lib.dtype_code(x), _lib.stream_ptr(x.device))
+        done += n
+    return out.view(*full_logits.shape[:-1], vd)

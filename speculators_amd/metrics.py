@@ -1,0 +1,238 @@
+"""Per-step loss and acceptance metrics on the device.
+
+Drop-in replacements, with identical metric keys and the identical in-place
+mutation of ``prev_correct``, for
+  * ``compute_metrics`` of EAGLE3 (models/eagle3/metrics.py:51-119) and
+  * ``compute_metrics`` of DFlash (models/dflash/metrics.py:20-108).
+The row losses and both arg-maxes come out of one pass of the fused loss
+kernel; the masked mean, the acceptance chain and the counts are one more
+single-workgroup kernel.  Nothing of size ``[T, V]`` is ever created here.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from . import _lib
+from . import losses as L
+
+
+def _as_mask(t: torch.Tensor) -> torch.Tensor:
+    """1-D unit-stride view of a ``[1, n]`` mask (its dtype is kept)."""
+    t = t.reshape(-1)
+    return t if t.stride(0) == 1 else t.contiguous()
+
+
+class _StepReduce(torch.autograd.Function):
+    """(row_loss [n] f32) -> weighted masked mean (0-d); also fills ``out`` (6 floats)
+    and updates ``prev_correct`` in place.  d/d row_loss = row_weight."""
+
+    @staticmethod
+    def forward(ctx, row_loss, am_d, am_t, mask, prev, weight, out):
+        n = row_loss.numel()
+        row_loss = row_loss.reshape(-1).contiguous()
+        row_weight = torch.empty(n, device=row_loss.device, dtype=torch.float32)
+        _lib.call(
+            "spx_ttt_step_reduce", _lib.ptr(row_loss), _lib.ptr(am_d), _lib.ptr(am_t),
+            _lib.ptr(mask), _lib.kind_code(mask) if mask is not None else 0,
+            _lib.ptr(prev), _lib.kind_code(prev) if prev is not None else 0,
+            n, float(weight), _lib.ptr(out), _lib.ptr(row_weight),
+            _lib.stream_ptr(row_loss.device),
+        )
+        ctx.save_for_backward(row_weight)
+        ctx.shape = row_loss.shape
+        return out[0].clone()
+
+    @staticmethod
+    def backward(ctx, g):
+        (row_weight,) = ctx.saved_tensors
+        return (row_weight * g).view(ctx.shape), None, None, None, None, None, None
+
+
+def _step_views(logits, targets, loss_mask, prev_correct, ttt_step):
+    """align_for_step (models/eagle3/metrics.py:16-48): views only."""
+    n = logits.shape[1] - ttt_step
+    return (
+        logits[:, :n],
+        targets[:, ttt_step:],
+        None if loss_mask is None else loss_mask[:, ttt_step:],
+        None if prev_correct is None else prev_correct[:, :n],
+    )
+
+
+def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
+                    ttt_step_loss_decay: float, loss_config: L.LossConfig | None = None):
+    """EAGLE3 per-step loss + metrics; same contract as models/eagle3/metrics.py:51-119.
+
+    ``prev_correct`` (any mask dtype) is updated in place.  Returns
+    ``(loss 0-d, metrics dict of 0-d tensors)``.
+    """
+    if logits.shape[0] != 1:
+        raise ValueError("the packed batch layout has batch size 1 (train/data.py:306-393)")
+    if loss_config is None:
+        loss_config = {"kl_div": (L.kl_div_loss, 1.0)}
+    s_logits, s_targets, s_mask, s_prev = _step_views(
+        logits, targets, loss_mask, prev_correct, ttt_step)
+    dev = logits.device
+    # gamma ** step evaluated in fp32 like exp_loss_decay on a float tensor
+    # (losses/utils.py:51-61)
+    weight = float(np.float32(ttt_step_loss_decay) ** np.float32(ttt_step))
+
+    mask1 = None if s_mask is None else _as_mask(s_mask)
+    prev1 = None
+    if s_prev is not None:
+        prev1 = s_prev.reshape(-1)
+        if prev1.stride(0) != 1:
+            raise ValueError("prev_correct must be contiguous (it is updated in place)")
+
+    total = None
+    terms = {}
+    multi = len(loss_config) > 1
+    first_out = None
+    for ti, (name, (fn, w)) in enumerate(loss_config.items()):
+        out = torch.empty(6, device=dev, dtype=torch.float32)
+        op = L.PRIMITIVE_OP.get(name)
+        if fn is L._HIP_LOSS_FN_MAP.get(name) and op is not None:
+            rows, am_d, am_t = L.fused_rows(op, s_logits, s_targets)
+        else:
+            rows = fn(s_logits, s_targets)
+            _, am_d, am_t = L.fused_rows(L.OP_CE, s_logits.detach(), s_targets)
+        # only the first term advances the acceptance chain
+        term = _StepReduce.apply(rows.reshape(-1), am_d.reshape(-1), am_t.reshape(-1), mask1,
+                                 prev1 if ti == 0 else None, weight, out)
+        if ti == 0:
+            first_out = out
+        if multi:
+            terms[f"{name}_loss"] = term.detach()
+        total = w * term if total is None else total + w * term
+
+    one = torch.ones((), device=dev)
+    m = {f"loss_{ttt_step}_sum": total.detach().clone(), f"loss_{ttt_step}_total": one}
+    for tname, tval in terms.items():
+        m[f"{tname}_{ttt_step}_sum"] = tval
+        m[f"{tname}_{ttt_step}_total"] = one.clone()
+    m[f"full_acc_{ttt_step}_sum"] = first_out[1]
+    m[f"full_acc_{ttt_step}_total"] = first_out[2]
+    m[f"cond_acc_{ttt_step}_sum"] = first_out[3]
+    m[f"cond_acc_{ttt_step}_total"] = first_out[4]
+    return total, m
+
+
+def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
+    """First-index arg-max over the last axis as int64, through the loss kernel's
+    arg-max path (pairs every row with itself)."""
+    x = L._rows_2d(logits)
+    rows, vocab = x.shape
+    dev = x.device
+    scratch = torch.empty(4, max(rows, 1), device=dev, dtype=torch.float32)
+    out = torch.empty(max(rows, 1), device=dev, dtype=torch.int32)
+    if rows:
+        _lib.call(
+            "spx_fused_vocab_loss_fwd", L.OP_CE, _lib.ptr(x), x.stride(0), _lib.ptr(x),
+            x.stride(0), rows, vocab, _lib.dtype_code(x), _lib.ptr(scratch[0]),
+            _lib.ptr(scratch[1]), _lib.ptr(scratch[2]), _lib.ptr(scratch[3]), _lib.ptr(out),
+            None, _lib.stream_ptr(dev),
+        )
+    return out[:rows].to(torch.int64).view(logits.shape[:-1])
+
+
+class _BlockReduce(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, row_loss, am_d, am_t, mask, pos_weight, block_size, out, correct, total):
+        n = row_loss.numel()
+        row_loss = row_loss.reshape(-1).contiguous()
+        row_weight = torch.empty(n, device=row_loss.device, dtype=torch.float32)
+        _lib.call(
+            "spx_block_reduce", _lib.ptr(row_loss), _lib.ptr(am_d), _lib.ptr(am_t), _lib.ptr(mask),
+            _lib.kind_code(mask), _lib.ptr(pos_weight), n, int(block_size), _lib.ptr(out),
+            _lib.ptr(correct), _lib.ptr(total), _lib.ptr(row_weight),
+            _lib.stream_ptr(row_loss.device),
+        )
+        ctx.save_for_backward(row_weight)
+        ctx.shape = row_loss.shape
+        return out[0].clone()
+
+    @staticmethod
+    def backward(ctx, g):
+        (row_weight,) = ctx.saved_tensors
+        return (row_weight * g).view(ctx.shape), None, None, None, None, None, None, None, None
+
+
+def dflash_loss_decay(pos_idx: torch.Tensor, gamma: float, sample_from_anchor: bool = False):
+    """Per-slot weight of losses/utils.py:17-48 (a [block_size]-periodic vector)."""
+    pos = pos_idx.to(torch.float32)
+    if sample_from_anchor:
+        return torch.exp(-pos / gamma)
+    w = torch.exp(-(pos - 1.0).clamp_min(0.0) / gamma)
+    return torch.where(pos == 0, torch.zeros_like(w), w)
+
+
+def dpace_loss_decay(row_ce: torch.Tensor, loss_mask: torch.Tensor, block_size: int,
+                     dpace_alpha: float) -> torch.Tensor:
+    """D-PACE weight from masked CE row losses (losses/utils.py:64-112); no gradient."""
+    with torch.no_grad():
+        n = row_ce.numel()
+        if n % block_size != 0:
+            raise ValueError(f"q.shape[1] ({n}) must be divisible by block_size ({block_size})")
+        conf = torch.exp(-row_ce.float()).reshape(n // block_size, block_size)
+        m = loss_mask.reshape(n // block_size, block_size).to(conf.dtype)
+        s = torch.where(m > 0, (1.0 - dpace_alpha) * conf + dpace_alpha, torch.ones_like(conf))
+        prefix = torch.cumprod(s, dim=-1) * m
+        suffix = torch.flip(torch.cumsum(torch.flip(prefix, dims=[-1]), dim=-1), dims=[-1])
+        return (suffix * m).reshape(-1)
+
+
+def dflash_compute_metrics(logits, targets, loss_mask, block_size: int = 1, gamma: float = 4.0,
+                           loss_config: L.LossConfig | None = None,
+                           per_position_loss_weight: str = "fixed-exp-decay",
+                           dpace_alpha: float = 0.5, sample_from_anchor: bool = False):
+    """DFlash loss + per-slot accuracy + EAL; contract of models/dflash/metrics.py:20-108."""
+    if loss_config is None:
+        loss_config = {"kl_div": (L.kl_div_loss, 1.0)}
+    dev = logits.device
+    n = logits.shape[1]
+    mask1 = _as_mask(loss_mask)
+    pos = torch.arange(n, device=dev) % block_size
+    total_loss = None
+    terms = {}
+    multi = len(loss_config) > 1
+    correct = total = None
+    for ti, (name, (fn, w)) in enumerate(loss_config.items()):
+        op = L.PRIMITIVE_OP.get(name)
+        if fn is L._HIP_LOSS_FN_MAP.get(name) and op is not None:
+            rows, am_d, am_t = L.fused_rows(op, logits, targets)
+        else:
+            rows = fn(logits, targets)
+            _, am_d, am_t = L.fused_rows(L.OP_CE, logits.detach(), targets)
+        if per_position_loss_weight == "dpace":
+            masked = rows.detach().reshape(-1) * mask1.to(torch.float32)
+            pw = dpace_loss_decay(masked, mask1, block_size, dpace_alpha)
+        else:
+            pw = dflash_loss_decay(pos, gamma, sample_from_anchor)
+        out = torch.empty(2, device=dev, dtype=torch.float32)
+        c = torch.empty(block_size, device=dev, dtype=torch.float32)
+        t = torch.empty(block_size, device=dev, dtype=torch.float32)
+        term = _BlockReduce.apply(rows.reshape(-1), am_d.reshape(-1), am_t.reshape(-1), mask1,
+                                  pw.contiguous(), block_size, out, c, t)
+        if ti == 0:
+            correct, total = c, t
+        if multi:
+            terms[f"{name}_loss"] = term.detach()
+        total_loss = w * term if total_loss is None else total_loss + w * term
+
+    one = torch.ones((), device=dev)
+    m = {"loss_sum": total_loss.detach().clone(), "loss_total": one}
+    for tname, tval in terms.items():
+        m[f"{tname}_sum"] = tval
+        m[f"{tname}_total"] = one.clone()
+    first = 0 if sample_from_anchor else 1
+    m["full_acc_sum"] = correct[first:].sum()
+    m["full_acc_total"] = total[first:].sum()
+    acc = correct[first:] / total[first:].clamp(min=1.0)
+    m["eal_sum"] = torch.cumprod(acc, dim=0).sum() if acc.numel() else torch.zeros((), device=dev)
+    m["eal_total"] = one.clone()
+    for s in range(first, block_size):
+        m[f"position_{s}_acc_sum"] = correct[s]
+        m[f"position_{s}_acc_total"] = total[s]
+    return total_loss, m

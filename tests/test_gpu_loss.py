@@ -1,0 +1,209 @@
+"""HIP fused vocabulary loss against the CPU oracle (through the C ABI)."""
+
+import pytest
+import torch
+
+from oracle import losses as OL
+from oracle import metrics as OM
+from oracle import vocab as OV
+
+pytestmark = pytest.mark.gpu
+
+LOSS_TOL = dict(atol=1e-4, rtol=1e-3)  # tests/unit/models/test_fused_losses.py:35
+GRAD_TOL = dict(atol=1e-3, rtol=1e-2)  # tests/unit/models/test_fused_losses.py:36
+NAMES = ["kl_div", "rkl", "jsd", "ce", "tv", "nla", "lk_hybrid"]
+
+
+def _check(name, logits, targets, loss_tol=LOSS_TOL, grad_tol=GRAD_TOL):
+    from speculators_amd import losses as L
+
+    fn = L.resolve_loss_config(name)[name][0]
+    lg = logits.cuda().detach().clone().requires_grad_(True)
+    out = fn(lg, targets.cuda())
+    assert out.dtype == torch.float32 and out.shape == logits.shape[:-1]
+    lo = logits.float().detach().clone().requires_grad_(True)
+    ref = OL.LOSS_FNS[name](lo, targets.float())
+    torch.testing.assert_close(out.cpu(), ref.detach(), **loss_tol)
+    g = torch.Generator().manual_seed(9)
+    go = torch.randn(ref.shape, generator=g)
+    go[:, ::3] = 0.0  # rows that take the zero-gradient early-out
+    (ref * go).sum().backward()
+    (out * go.cuda()).sum().backward()
+    got = lg.grad.float().cpu()
+    torch.testing.assert_close(got, lo.grad, **grad_tol)
+    assert (got[:, ::3] == 0).all()
+
+
+@pytest.mark.parametrize("name", NAMES)
+def test_fp32_with_saturated_rows(name):
+    # the regime of tests/unit/models/test_fused_losses.py:71-79
+    g = torch.Generator().manual_seed(0)
+    a = torch.randn(1, 32, 512, generator=g) * 3
+    b = torch.randn(1, 32, 512, generator=g) * 3
+    a[0, -2:] = -30.0; b[0, -2:] = -30.0
+    a[0, -2:, 0] = 30.0; b[0, -2, 0] = 30.0; b[0, -1, 7] = 30.0
+    _check(name, a, b)
+
+
+@pytest.mark.parametrize("name", NAMES)
+def test_bf16(name):
+    g = torch.Generator().manual_seed(1)
+    a = (torch.randn(1, 64, 512, generator=g) * 3).bfloat16()
+    b = (torch.randn(1, 64, 512, generator=g) * 3).bfloat16()
+    # the oracle computes in fp32 from the same bf16 inputs; the gradient is rounded to bf16
+    _check(name, a, b, grad_tol=dict(atol=1e-3, rtol=1e-2))
+
+
+@pytest.mark.parametrize("name", NAMES)
+def test_wide_vocab_151936(name):
+    g = torch.Generator().manual_seed(2)
+    a = torch.randn(1, 3, 151936, generator=g) * 3
+    b = torch.randn(1, 3, 151936, generator=g) * 3
+    _check(name, a, b)
+
+
+@pytest.mark.parametrize("vocab", [1, 7, 8, 9, 250, 32000 + 3])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ragged_vocab_and_unaligned_rows(vocab, dtype):
+    from speculators_amd import losses as L
+
+    g = torch.Generator().manual_seed(vocab)
+    a = (torch.randn(1, 5, vocab, generator=g) * 2).to(dtype)
+    b = (torch.randn(1, 5, vocab, generator=g) * 2).to(dtype)
+    rows, am_d, am_t = L.fused_rows(L.OP_KL, a.cuda(), b.cuda())
+    torch.testing.assert_close(rows.cpu(), OL.kl_div(a, b), **LOSS_TOL)
+    assert torch.equal(am_d.cpu().long(), a.float().argmax(-1))
+    assert torch.equal(am_t.cpu().long(), b.float().argmax(-1))
+
+
+def test_argmax_first_index_on_ties_bit_exact():
+    from speculators_amd import losses as L
+    from speculators_amd.metrics import argmax_rows
+
+    g = torch.Generator().manual_seed(3)
+    # coarse bf16 values: many exact ties per row
+    a = (torch.randint(-4, 5, (1, 257, 32000), generator=g).float() * 0.5).bfloat16()
+    b = (torch.randint(-4, 5, (1, 257, 32000), generator=g).float() * 0.5).bfloat16()
+    _, am_d, am_t = L.fused_rows(L.OP_KL, a.cuda(), b.cuda())
+    assert torch.equal(am_d.cpu().long(), a.float().argmax(-1))
+    assert torch.equal(am_t.cpu().long(), b.float().argmax(-1))
+    assert torch.equal(argmax_rows(a.cuda()).cpu(), a.float().argmax(-1))
+    # a late unique maximum and an early one
+    a[0, 0, :] = 0; a[0, 0, 31999] = 1
+    a[0, 1, :] = 0; a[0, 1, 0] = 1
+    assert argmax_rows(a.cuda())[0, :2].tolist() == [31999, 0]
+
+
+def test_vocab_gather_bit_exact():
+    from speculators_amd import losses as L
+
+    g = torch.Generator().manual_seed(4)
+    vt, vd = 128256, 32000
+    sel = torch.randperm(vt, generator=g)[:vd]
+    d2t, t2d = OV.build_vocab_mappings(sel.tolist(), vt)
+    full = (torch.randn(1, 9, vt, generator=g) * 2).bfloat16()
+    got = L.vocab_gather(full.cuda(), d2t.cuda()).cpu()
+    assert torch.equal(got, OV.gather_targets(full, d2t))
+    assert torch.equal(got, full[..., t2d])
+    full32 = torch.randn(3, vt, generator=g)
+    assert torch.equal(L.vocab_gather(full32.cuda(), d2t.cuda()).cpu(), full32[..., t2d])
+
+
+@pytest.mark.parametrize("mask_dtype", [torch.float32, torch.bool, torch.int64, torch.bfloat16])
+def test_eagle3_compute_metrics_chain_matches_oracle(mask_dtype):
+    from speculators_amd import losses as L
+    from speculators_amd.metrics import compute_metrics
+
+    g = torch.Generator().manual_seed(5)
+    t, v, steps = 300, 1000, 4
+    targets = (torch.randn(1, t, v, generator=g) * 2).bfloat16()
+    mask = (torch.rand(1, t, generator=g) < 0.7).to(mask_dtype)
+    prev_ref = mask.clone()
+    prev_gpu = mask.clone().cuda()
+    for k in range(steps):
+        logits = (torch.randn(1, t, v, generator=g) * 2).bfloat16()
+        for i in range(0, t - k, 2):  # make half the rows agree with the shifted target
+            logits[0, i, targets[0, i + k].float().argmax()] = 20.0
+        lg = logits.cuda().requires_grad_(True)
+        loss, m = compute_metrics(lg, targets.cuda(), mask.cuda(), prev_gpu, k, 0.8,
+                                  L.resolve_loss_config("kl_div"))
+        lo = logits.float().requires_grad_(True)
+        rloss, rm = OM.eagle3_compute_metrics(lo, targets.float(), mask, prev_ref, k, 0.8)
+        assert loss.item() == pytest.approx(rloss.item(), rel=1e-3)
+        for key in rm:
+            if "acc" in key:  # integer counts: bit exact
+                assert m[key].item() == rm[key].item(), key
+            else:
+                assert m[key].item() == pytest.approx(rm[key].item(), rel=1e-3), key
+        assert set(m) == set(rm)
+        assert torch.equal(prev_gpu.cpu(), prev_ref) and prev_gpu.dtype == mask_dtype
+        loss.backward(); rloss.backward()
+        torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, atol=1e-5, rtol=2e-2)
+
+
+def test_compound_loss_config_and_no_mask():
+    from speculators_amd import losses as L
+    from speculators_amd.metrics import compute_metrics
+
+    g = torch.Generator().manual_seed(6)
+    logits = torch.randn(1, 40, 333, generator=g)
+    targets = torch.randn(1, 40, 333, generator=g)
+    cfg = L.resolve_loss_config('{"ce": 0.25, "tv": 0.75}')
+    loss, m = compute_metrics(logits.cuda(), targets.cuda(), None, None, 2, 0.5, cfg)
+    rloss, rm = OM.eagle3_compute_metrics(logits, targets, None, None, 2, 0.5,
+                                          OL.resolve_loss_config({"ce": 0.25, "tv": 0.75}))
+    assert set(m) == set(rm)
+    for key in rm:
+        assert m[key].item() == pytest.approx(rm[key].item(), rel=1e-3, abs=1e-6), key
+
+
+@pytest.mark.parametrize("weighting", ["fixed-exp-decay", "dpace"])
+def test_dflash_compute_metrics_matches_oracle(weighting):
+    from speculators_amd import losses as L
+    from speculators_amd.metrics import dflash_compute_metrics
+
+    g = torch.Generator().manual_seed(7)
+    bs, a, v = 8, 37, 2000
+    logits = (torch.randn(1, a * bs, v, generator=g) * 2).bfloat16()
+    targets = (torch.randn(1, a * bs, v, generator=g) * 2).bfloat16()
+    for i in range(0, a * bs, 3):
+        logits[0, i, targets[0, i].float().argmax()] = 20.0
+    mask = (torch.rand(1, a * bs, generator=g) < 0.8).float()
+    mask[:, ::bs] = 0
+    name = "ce" if weighting == "dpace" else "kl_div"
+    lg = logits.cuda().requires_grad_(True)
+    loss, m = dflash_compute_metrics(lg, targets.cuda(), mask.cuda(), bs, 4.0,
+                                     L.resolve_loss_config(name), weighting, 0.5)
+    lo = logits.float().requires_grad_(True)
+    rloss, rm = OM.dflash_compute_metrics(lo, targets.float(), mask, bs, 4.0,
+                                          OL.resolve_loss_config(name), weighting, 0.5)
+    assert set(m) == set(rm)
+    for key in rm:
+        if "acc" in key:
+            assert m[key].item() == rm[key].item(), key
+        else:
+            assert m[key].item() == pytest.approx(rm[key].item(), rel=1e-3, abs=1e-6), key
+    loss.backward(); rloss.backward()
+    torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, atol=1e-5, rtol=2e-2)
+
+
+def test_full_size_rows_properties():
+    """Config[1] row shape (32000-wide bf16): properties that need no oracle at size --
+    KL(x, x) == 0, loss >= 0, gradient rows sum to ~0, determinism."""
+    from speculators_amd import losses as L
+
+    g = torch.Generator(device="cuda").manual_seed(8)
+    x = (torch.randn(1, 4096, 32000, device="cuda", generator=g) * 2).bfloat16().requires_grad_(True)
+    y = (torch.randn(1, 4096, 32000, device="cuda", generator=g) * 2).bfloat16()
+    same = L.kl_div_loss(x.detach(), x.detach())
+    assert same.abs().max().item() < 1e-4
+    rows, am_d, _ = L.fused_rows(L.OP_KL, x, y)
+    rows2, am_d2, _ = L.fused_rows(L.OP_KL, x, y)
+    assert torch.equal(rows, rows2) and torch.equal(am_d, am_d2)
+    assert (rows >= 0).all()
+    rows.sum().backward()
+    assert x.grad.float().sum(-1).abs().max().item() < 2e-2
+    # a 64-row sample against the oracle
+    idx = torch.arange(0, 4096, 64)
+    ref = OL.kl_div(x.detach()[:, idx].cpu(), y[:, idx].cpu())
+    torch.testing.assert_close(rows[:, idx].detach().cpu(), ref, **LOSS_TOL)
