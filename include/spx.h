@@ -122,6 +122,38 @@ int spx_block_reduce(const float* loss, const int32_t* argmax_draft,
                      int32_t block_size, float* out, float* correct,
                      float* total, float* row_weight, void* stream);
 
+/* ---------------------------------------------------------------- TTT attention
+ * row_lo[i] = lowest context key visible to query i: the interval form
+ * row_lo[i] <= c <= i of the step-0 part of create_combined_mask_mod
+ * (models/eagle3/attention.py:11-34) for run-contiguous document ids (what
+ * CollateFn emits, train/data.py:323-393): start of i's document, raised to
+ * i - W + 1 under a sliding window W (sliding_window <= 0: none), and i itself
+ * for padding rows (document id -1).  Replaces the dense [T, T] mask that
+ * create_block_mask materialises (models/eagle3/core.py:149-162). */
+int spx_ttt_row_lo(const void* document_ids, int doc_kind, int64_t T,
+                   int64_t sliding_window, int32_t* row_lo, void* stream);
+
+/* bytes of caller-owned scratch the attention entry points need */
+int64_t spx_ttt_attn_workspace_bytes(int64_t T, int32_t Hq, int32_t Hkv,
+                                     int32_t D, int32_t backward);
+
+/* out[i, h, :] = softmax_c(scaling * q[h, i] . k[h / (Hq/Hkv), c]) v[..]  over the
+ * keys of TTT step `ttt_step` (0-based): context keys row_lo[i] <= c <= i of
+ * the first T rows of k/v, plus the rows j*T + i for j = 1..ttt_step (the
+ * diagonals that extend_mask_for_draft_tokens appends,
+ * models/eagle3/attention.py:37-132).  Replaces flex_attention_forward
+ * (models/attention.py:20-66) for the EAGLE3 mask.
+ *   q   bf16 [Hq, T, D]  (head stride q_head_stride elements, rows contiguous)
+ *   k,v bf16 [Hkv, (ttt_step+1)*T, D]  (the cache layout of DynamicCache)
+ *   out bf16 [T, Hq, D];  lse f32 [Hq, T]: log2-domain row log-sum-exp, opaque,
+ *   consumed by spx_ttt_attn_bwd.   D in {64, 128}. */
+int spx_ttt_attn_fwd(const void* q, int64_t q_head_stride, const void* k,
+                     int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                     const int32_t* row_lo, int64_t T, int32_t ttt_step,
+                     int32_t Hq, int32_t Hkv, int32_t D, float scaling,
+                     void* out, float* lse, void* workspace,
+                     int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

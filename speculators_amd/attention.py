@@ -1,0 +1,148 @@
+"""Attention plug-in: the HIP TTT / anchored-block attention behind the
+reference's attention-function interface.
+
+The reference selects an attention function by name from an
+``AttentionInterface`` registry (models/attention.py:107-108) and calls it as
+``fn(module, q[B,Hq,Q,D], k[B,Hkv,KV,D], v, attention_mask, scaling=..., **kw)
+-> (out[B,Q,Hq,D], None)`` (models/attention.py:20-66).  ``attention_mask`` is
+whatever the model's mask builder returned; for the HIP kernels it is a small
+descriptor (``TTTMask``) instead of a BlockMask or a dense tensor, and the
+model's "extend the mask for the next TTT step" operation just bumps a counter.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+
+ATTN_IMPL_TTT = "ttt_hip"
+
+_lib.SIGNATURES.update({
+    "spx_ttt_row_lo": [_lib._P, _lib._I, _lib._I64, _lib._I64, _lib._P, _lib._P],
+    "spx_ttt_attn_fwd": [_lib._P, _lib._I64, _lib._P, _lib._I64, _lib._P, _lib._I64, _lib._P,
+                         _lib._I64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                         _lib._F, _lib._P, _lib._P, _lib._P, _lib._I64, _lib._P],
+})
+
+
+def _workspace_bytes(t, hq, hkv, d, backward):
+    lib = _lib.load()
+    fn = lib.spx_ttt_attn_workspace_bytes
+    fn.restype = ctypes.c_int64
+    fn.argtypes = [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
+    return int(fn(t, hq, hkv, d, int(backward)))
+
+
+@dataclass
+class TTTMask:
+    """Descriptor of the EAGLE3 mask of one layer: ``row_lo`` (int32 ``[T]``, lowest
+    visible context key per query), the sequence length and the current TTT step.
+    Stands where the reference passes a BlockMask / dense mask
+    (models/eagle3/core.py:149-162, 341-356)."""
+
+    row_lo: torch.Tensor
+    total_seq_len: int
+    ttt_step: int = 0
+    sliding_window: int | None = None
+
+    def extended(self) -> "TTTMask":
+        """The mask of the next TTT step (one more diagonal of keys); the
+        counterpart of extend_mask_for_draft_tokens (models/eagle3/attention.py:37-132)."""
+        return TTTMask(self.row_lo, self.total_seq_len, self.ttt_step + 1, self.sliding_window)
+
+
+def create_ttt_mask(document_ids: torch.Tensor, total_seq_len: int,
+                    sliding_window: int | None = None) -> TTTMask:
+    """Build the step-0 descriptor from ``document_ids`` (``[T]`` or ``[1, T]``, -1 =
+    padding); the counterpart of ``_build_attn_mask`` (models/eagle3/core.py:149-162).
+    ``document_ids`` must be run-contiguous, as the packing collate produces them."""
+    doc = document_ids.reshape(-1)
+    if doc.numel() != total_seq_len:
+        raise ValueError(f"document_ids has {doc.numel()} entries, expected {total_seq_len}")
+    if doc.dtype not in (torch.int32, torch.int64):
+        doc = doc.to(torch.int64)
+    doc = doc.contiguous()
+    row_lo = torch.empty(total_seq_len, device=doc.device, dtype=torch.int32)
+    _lib.call("spx_ttt_row_lo", _lib.ptr(doc), _lib.kind_code(doc), total_seq_len,
+              int(sliding_window) if sliding_window else 0, _lib.ptr(row_lo),
+              _lib.stream_ptr(doc.device))
+    return TTTMask(row_lo, total_seq_len, 0, sliding_window)
+
+
+def _check_qkv(q, k, v, mask: TTTMask):
+    if q.dim() != 4 or q.shape[0] != 1:
+        raise ValueError("the packed batch layout has batch size 1: q must be [1, Hq, T, D]")
+    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
+        raise _lib.SpxError("the HIP attention kernels take bf16 q/k/v")
+    _, hq, t, d = q.shape
+    hkv, kv_len = k.shape[1], k.shape[2]
+    if t != mask.total_seq_len or kv_len != (mask.ttt_step + 1) * t or v.shape != k.shape:
+        raise ValueError(
+            f"q {tuple(q.shape)} / k {tuple(k.shape)} do not match TTT step {mask.ttt_step} "
+            f"of a length-{mask.total_seq_len} sequence")
+    return hq, hkv, t, d
+
+
+class _TTTAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, mask: TTTMask, scaling: float):
+        hq, hkv, t, d = _check_qkv(q, k, v, mask)
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        dev = q.device
+        out = torch.empty(1, t, hq, d, device=dev, dtype=torch.bfloat16)
+        lse = torch.empty(hq, t, device=dev, dtype=torch.float32)
+        ws = torch.empty(_workspace_bytes(t, hq, hkv, d, False), device=dev, dtype=torch.uint8)
+        _lib.call("spx_ttt_attn_fwd", _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1),
+                  _lib.ptr(v), v.stride(1), _lib.ptr(mask.row_lo), t, mask.ttt_step, hq, hkv, d,
+                  float(scaling), _lib.ptr(out), _lib.ptr(lse), _lib.ptr(ws), ws.numel(),
+                  _lib.stream_ptr(dev))
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.mask, ctx.scaling = mask, float(scaling)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        raise NotImplementedError
+
+
+def ttt_attention(q, k, v, mask: TTTMask, scaling: float | None = None) -> torch.Tensor:
+    """``[1, Hq, T, D]`` x ``[1, Hkv, (step+1)*T, D]`` -> ``[1, T, Hq, D]`` (bf16)."""
+    if scaling is None:
+        scaling = q.shape[-1] ** -0.5
+    return _TTTAttention.apply(q, k, v, mask, scaling)
+
+
+def ttt_hip_attention_forward(module, query, key, value, attention_mask, scaling=None, **_kwargs):
+    """The attention-function signature of the reference registry
+    (models/attention.py:20-66); ``attention_mask`` must be a ``TTTMask``."""
+    if not isinstance(attention_mask, TTTMask):
+        raise TypeError(
+            f"attention impl '{ATTN_IMPL_TTT}' needs a TTTMask descriptor as attention_mask, "
+            f"got {type(attention_mask).__name__}")
+    return ttt_attention(query, key, value, attention_mask, scaling), None
+
+
+class AttentionRegistry(dict):
+    """Name -> attention function; the local mirror of the reference's
+    ``ALL_ATTENTION_FUNCTIONS`` (models/attention.py:107-108)."""
+
+    def register(self, name, fn):
+        self[name] = fn
+
+
+ALL_ATTENTION_FUNCTIONS = AttentionRegistry()
+ALL_ATTENTION_FUNCTIONS.register(ATTN_IMPL_TTT, ttt_hip_attention_forward)
+
+
+def register_with_transformers() -> None:
+    """Also register the HIP attention functions in HF's global ``AttentionInterface`` so a
+    ``LlamaAttention`` / ``Qwen3Attention`` whose config says
+    ``_attn_implementation = "ttt_hip"`` dispatches to them."""
+    from transformers.modeling_utils import AttentionInterface
+
+    for name, fn in ALL_ATTENTION_FUNCTIONS.items():
+        AttentionInterface.register(name, fn)
