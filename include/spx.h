@@ -154,6 +154,21 @@ int spx_ttt_attn_fwd(const void* q, int64_t q_head_stride, const void* k,
                      void* out, float* lse, void* workspace,
                      int64_t workspace_bytes, void* stream);
 
+/* Gradients of spx_ttt_attn_fwd.  dout bf16 [T, Hq, D] (the layout of `out`),
+ * lse as written by the forward.  dq bf16 [Hq, T, D]; dk, dv bf16
+ * [Hkv, (ttt_step+1)*T, D]: every row is written (context rows by the tiled
+ * kernels, the diagonal rows j*T + i by a per-position kernel; no atomics, so
+ * the result is deterministic).  Replaces the autograd of flex_attention at
+ * the call site models/attention.py:55-63. */
+int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
+                     int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                     const void* out, const void* dout, const float* lse,
+                     const int32_t* row_lo, int64_t T, int32_t ttt_step,
+                     int32_t Hq, int32_t Hkv, int32_t D, float scaling, void* dq,
+                     int64_t dq_head_stride, void* dk, int64_t dk_head_stride,
+                     void* dv, int64_t dv_head_stride, void* workspace,
+                     int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

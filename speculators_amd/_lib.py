@@ -17,15 +17,24 @@ LIB_PATH = os.path.join(_HERE, "libspx_hip.so")
 
 _P, _I64, _I, _F = c_void_p, c_int64, c_int, c_float
 
-# name -> argument types (all return int); mirrors include/spx.h
+_I32 = c_int32
+
+# name -> argument types (return type int unless listed in RESTYPES); mirrors include/spx.h
 SIGNATURES: dict[str, list] = {
     "spx_vocab_gather": [_P, _I64, _P, _P, _I64, _I64, _I64, _I64, _I, _P],
     "spx_fused_vocab_loss_fwd": [_I, _P, _I64, _P, _I64, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P],
     "spx_fused_vocab_loss_bwd": [_I, _P, _I64, _P, _I64, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P,
                                  _I64, _P],
     "spx_ttt_step_reduce": [_P, _P, _P, _P, _I, _P, _I, _I64, _F, _P, _P, _P],
-    "spx_block_reduce": [_P, _P, _P, _P, _I, _P, _I64, c_int32, _P, _P, _P, _P, _P],
+    "spx_block_reduce": [_P, _P, _P, _P, _I, _P, _I64, _I32, _P, _P, _P, _P, _P],
+    "spx_ttt_row_lo": [_P, _I, _I64, _I64, _P, _P],
+    "spx_ttt_attn_workspace_bytes": [_I64, _I32, _I32, _I32, _I32],
+    "spx_ttt_attn_fwd": [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I32, _I32, _I32, _I32, _F, _P, _P,
+                         _P, _I64, _P],
+    "spx_ttt_attn_bwd": [_P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32,
+                         _F, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P],
 }
+RESTYPES = {"spx_ttt_attn_workspace_bytes": c_int64}
 
 _lib = None
 
@@ -51,7 +60,7 @@ def load() -> ctypes.CDLL:
     lib.spx_last_error.argtypes = []
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)
-        fn.restype = c_int
+        fn.restype = RESTYPES.get(name, c_int)
         fn.argtypes = argtypes
     _lib = lib
     return lib

@@ -12,7 +12,6 @@ model's "extend the mask for the next TTT step" operation just bumps a counter.
 
 from __future__ import annotations
 
-import ctypes
 from dataclasses import dataclass
 
 import torch
@@ -21,20 +20,9 @@ from . import _lib
 
 ATTN_IMPL_TTT = "ttt_hip"
 
-_lib.SIGNATURES.update({
-    "spx_ttt_row_lo": [_lib._P, _lib._I, _lib._I64, _lib._I64, _lib._P, _lib._P],
-    "spx_ttt_attn_fwd": [_lib._P, _lib._I64, _lib._P, _lib._I64, _lib._P, _lib._I64, _lib._P,
-                         _lib._I64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
-                         _lib._F, _lib._P, _lib._P, _lib._P, _lib._I64, _lib._P],
-})
-
 
 def _workspace_bytes(t, hq, hkv, d, backward):
-    lib = _lib.load()
-    fn = lib.spx_ttt_attn_workspace_bytes
-    fn.restype = ctypes.c_int64
-    fn.argtypes = [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
-    return int(fn(t, hq, hkv, d, int(backward)))
+    return int(_lib.load().spx_ttt_attn_workspace_bytes(t, hq, hkv, d, int(backward)))
 
 
 @dataclass
@@ -106,7 +94,22 @@ class _TTTAttention(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout):
-        raise NotImplementedError
+        q, k, v, out, lse = ctx.saved_tensors
+        mask = ctx.mask
+        _, hq, t, d = q.shape
+        hkv = k.shape[1]
+        dev = q.device
+        dout = dout.to(torch.bfloat16).contiguous()
+        dq = torch.empty_like(q)
+        dk = torch.empty_like(k)
+        dv = torch.empty_like(v)
+        ws = torch.empty(_workspace_bytes(t, hq, hkv, d, True), device=dev, dtype=torch.uint8)
+        _lib.call("spx_ttt_attn_bwd", _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1),
+                  _lib.ptr(v), v.stride(1), _lib.ptr(out), _lib.ptr(dout), _lib.ptr(lse),
+                  _lib.ptr(mask.row_lo), t, mask.ttt_step, hq, hkv, d, ctx.scaling,
+                  _lib.ptr(dq), dq.stride(1), _lib.ptr(dk), dk.stride(1), _lib.ptr(dv),
+                  dv.stride(1), _lib.ptr(ws), ws.numel(), _lib.stream_ptr(dev))
+        return dq, dk, dv, None, None
 
 
 def ttt_attention(q, k, v, mask: TTTMask, scaling: float | None = None) -> torch.Tensor:

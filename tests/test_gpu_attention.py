@@ -58,3 +58,32 @@ def test_forward_matches_dense_oracle(t, hq, hkv, d, docs, window, steps):
         err = (out.float().cpu() - ref).abs().max().item()
         assert err <= 2e-2 * ref.abs().max().item(), (step, err)
         mask = mask.extended()
+
+
+@pytest.mark.parametrize("t,hq,hkv,d,docs,window,steps", CASES)
+def test_backward_matches_dense_oracle_autograd(t, hq, hkv, d, docs, window, steps):
+    from speculators_amd.attention import create_ttt_mask, ttt_attention
+
+    g = torch.Generator().manual_seed(7 * t + d)
+    doc = torch.zeros(t, dtype=torch.long) if docs is None else _docs(t, docs)
+    step = steps - 1
+    mask = create_ttt_mask(doc.cuda(), t, window)
+    for _ in range(step):
+        mask = mask.extended()
+    q = torch.randn(1, hq, t, d, generator=g).bfloat16()
+    k = torch.randn(1, hkv, steps * t, d, generator=g).bfloat16()
+    v = torch.randn(1, hkv, steps * t, d, generator=g).bfloat16()
+    go = torch.randn(1, t, hq, d, generator=g).bfloat16()
+    qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    out = ttt_attention(qg, kg, vg, mask, d ** -0.5)
+    out.backward(go.cuda())
+    qr, kr, vr = (x.float().requires_grad_(True) for x in (q, k, v))
+    ref = dense_attention(qr, kr, vr, OM.ttt_mask_dense(doc, t, step, window), d ** -0.5)
+    ref.backward(go.float())
+    for name, got, want in (("dq", qg.grad, qr.grad), ("dk", kg.grad, kr.grad), ("dv", vg.grad, vr.grad)):
+        err = (got.float().cpu() - want).abs().max().item()
+        assert err <= 2e-2 * want.abs().max().item(), (name, err, want.abs().max().item())
+    # the diagonal rows of dk/dv are exactly the per-position gradients: check them apart
+    if step > 0:
+        err = (kg.grad.float().cpu()[:, :, t:] - kr.grad[:, :, t:]).abs().max().item()
+        assert err <= 2e-2 * kr.grad[:, :, t:].abs().max().item()
