@@ -169,6 +169,17 @@ int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
                      void* dv, int64_t dv_head_stride, void* workspace,
                      int64_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------- GEMM
+ * c[M, N] = a[M, K] * b[N, K]^T, bf16 inputs, fp32 accumulation, bf16 output:
+ * the product of torch.nn.Linear (no bias).  Replaces the fc Linear
+ * (models/eagle3/core.py:76,244), the lm_head and verifier_lm_head Linears
+ * (model.py:66-69; call sites models/eagle3/core.py:251-253,302-306) and, with
+ * b = the transposed weight, the input-gradient product of their backward.
+ * lda/ldb/ldc are row strides in elements; K, lda, ldb multiples of 8. */
+int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb,
+                     void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                     void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -34,6 +34,7 @@ SIGNATURES: dict[str, list] = {
     "spx_ttt_attn_bwd": [_P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32,
                          _F, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P],
 }
+SIGNATURES["spx_gemm_bf16_nt"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P]
 RESTYPES = {"spx_ttt_attn_workspace_bytes": c_int64}
 
 _lib = None

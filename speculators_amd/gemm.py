@@ -1,0 +1,62 @@
+"""bf16 Linear products on the MFMA GEMM kernel.
+
+``linear(x, weight)`` is ``torch.nn.functional.linear`` without bias
+(``x @ weight.T``) for bf16 tensors.  The backward computes the input gradient
+with the same NT kernel against a transposed copy of the weight
+(``weight_t``, ``[K, N]`` contiguous) -- kept by the caller for frozen weights
+such as ``lm_head`` (model.py:70-71) so it is made once -- and leaves the
+weight gradient (a TN product) to the rocBLAS/hipBLASLt matmul of PyTorch.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``a[M, K] @ b[N, K].T -> [M, N]`` (bf16, fp32 accumulation)."""
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
+        raise _lib.SpxError("gemm_nt takes bf16 operands")
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise ValueError(f"shape mismatch: a {tuple(a.shape)} b {tuple(b.shape)}")
+    if a.stride(1) != 1:
+        a = a.contiguous()
+    if b.stride(1) != 1:
+        b = b.contiguous()
+    m, k = a.shape
+    n = b.shape[0]
+    if out is None:
+        out = torch.empty(m, n, device=a.device, dtype=torch.bfloat16)
+    _lib.call("spx_gemm_bf16_nt", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
+              _lib.ptr(out), out.stride(0), m, n, k, _lib.stream_ptr(a.device))
+    return out
+
+
+class _Linear(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, weight_t):
+        x2 = x.reshape(-1, x.shape[-1])
+        y = gemm_nt(x2, weight)
+        ctx.save_for_backward(x2, weight, weight_t)
+        ctx.x_shape = x.shape
+        return y.view(*x.shape[:-1], weight.shape[0])
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, weight, weight_t = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.shape[-1]).to(torch.bfloat16)
+        dx = dw = None
+        if ctx.needs_input_grad[0]:
+            wt = weight_t if weight_t is not None else weight.t().contiguous()
+            dx = gemm_nt(dy2, wt).view(ctx.x_shape)
+        if ctx.needs_input_grad[1]:
+            dw = torch.matmul(dy2.t(), x2)
+        return dx, dw, None
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor | None = None):
+    """``x[..., K] @ weight[N, K].T`` on the HIP GEMM; ``weight_t`` optionally holds
+    ``weight.T`` contiguous for the backward."""
+    return _Linear.apply(x, weight, weight_t)
