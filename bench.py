@@ -1,0 +1,287 @@
+#!/usr/bin/env python
+"""Headline benchmark: EAGLE3 draft train tokens/s (forward + backward) at the
+Llama-3.1-8B shape, seq 4096, TTT 7, bf16, on one MI355X.
+
+A "step" is one forward + backward of the draft over one packed synthetic row
+(inputs already resident in HBM).  Prints ONE JSON line.  Besides the whole-job
+throughput it times every hand-written kernel at its real shape with HIP
+events on the launch stream and reports the fraction of the roofline that
+bounds it, and times the CPU oracle (the restatement of the reference path) on
+a bounded sample of the same workload on the host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+CONFIG1 = dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+               intermediate_size=14336, vocab_size=128256, draft_vocab_size=32000,
+               rope_theta=500000.0, rms_norm_eps=1e-5)
+SEQ_LEN, TTT_STEPS = 4096, 7
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
+    ap.add_argument("--ttt-steps", type=int, default=TTT_STEPS)
+    ap.add_argument("--targets", choices=["hidden", "logits"], default="hidden",
+                    help="hidden: verifier_last_hidden_states through the frozen verifier head "
+                         "(the reference's forward contract); logits: full-vocab verifier "
+                         "logits gathered through d2t")
+    ap.add_argument("--cpu-baseline", choices=["sample", "off"], default="sample")
+    ap.add_argument("--cpu-seq-len", type=int, default=256)
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline timing")
+    return ap.parse_args()
+
+
+def make_inputs(torch, cfg, t, device, with_logits):
+    g = torch.Generator(device=device).manual_seed(0)
+    h, vt, vd = cfg["hidden_size"], cfg["vocab_size"], cfg["draft_vocab_size"]
+    batch = {
+        "hidden_states": (torch.randn(1, t, 3 * h, device=device, generator=g) * 4).bfloat16(),
+        "input_ids": torch.randint(0, vt, (1, t), device=device, generator=g),
+        "document_ids": torch.zeros(1, t, dtype=torch.long, device=device),
+        "loss_mask": (torch.rand(1, t, device=device, generator=g) < 0.7).float(),
+        "position_ids": 1 + torch.arange(t, device=device).unsqueeze(0),
+    }
+    sel = torch.randperm(vt, device=device, generator=g)[:vd].sort().values
+    d2t = sel - torch.arange(vd, device=device)
+    t2d = torch.zeros(vt, dtype=torch.bool, device=device)
+    t2d[sel] = True
+    if with_logits:
+        batch["verifier_logits"] = (torch.randn(1, t, vt, device=device, generator=g) * 2).bfloat16()
+    else:
+        batch["verifier_last_hidden_states"] = torch.randn(1, t, h, device=device, generator=g).bfloat16()
+    return batch, d2t, t2d
+
+
+def make_model(torch, cfg, device, d2t, t2d):
+    from speculators_amd.eagle3 import Eagle3Config, Eagle3DraftModel
+
+    model = Eagle3DraftModel(Eagle3Config(**cfg))
+    g = torch.Generator(device=device).manual_seed(1)
+    model = model.to(torch.bfloat16).to(device)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith("norm.weight") or "layernorm" in name:
+                p.fill_(1.0)
+            else:
+                p.copy_((torch.randn(p.shape, device=device, generator=g) * 0.02).to(p.dtype))
+    model.load_vocab_mappings(t2d, d2t)
+    return model
+
+
+def time_events(torch, fn, iters, warmup=2):
+    for _ in range(warmup):
+        fn()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters  # ms per launch
+
+
+def kernel_rooflines(torch, cfg, t, k_steps, device):
+    """Per-kernel average launch time (HIP events on the launch stream) against the
+    algorithmic flops / bytes of that launch."""
+    from speculators_amd import _lib
+    from speculators_amd import attention as A
+    from speculators_amd import losses as L
+    from speculators_amd.gemm import gemm_nt
+
+    h, vd = cfg["hidden_size"], cfg["draft_vocab_size"]
+    hq, hkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    g = torch.Generator(device=device).manual_seed(2)
+    out = []
+
+    def mfma(name, flops, ms, launches):
+        tf = flops / (ms * 1e-3) / 1e12
+        out.append({"kernel": name, "bound": "mfma", "achieved": round(tf, 1),
+                    "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4),
+                    "traffic": None, "ms_per_launch": round(ms, 4), "launches_per_step": launches})
+
+    def hbm(name, nbytes, ms, launches):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        out.append({"kernel": name, "bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+                    "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None,
+                    "ms_per_launch": round(ms, 4), "launches_per_step": launches})
+
+    # lm_head GEMM (forward shape; the input-gradient product has the same flops)
+    x = torch.randn(t, h, device=device, generator=g).bfloat16()
+    w = (torch.randn(vd, h, device=device, generator=g) * 0.02).bfloat16()
+    y = torch.empty(t, vd, device=device, dtype=torch.bfloat16)
+    ms = time_events(torch, lambda: gemm_nt(x, w, y), 20)
+    mfma("gemm_bf16_nt_kernel[lm_head fwd T x H x Vd]", 2.0 * t * h * vd, ms, k_steps + 1)
+    wt = w.t().contiguous()
+    dx = torch.empty(t, h, device=device, dtype=torch.bfloat16)
+    ms = time_events(torch, lambda: gemm_nt(y, wt, dx), 20)
+    mfma("gemm_bf16_nt_kernel[lm_head dX T x Vd x H]", 2.0 * t * h * vd, ms, k_steps)
+    del wt, dx
+
+    # fused loss forward / backward over T rows (step 0 shape)
+    tg = (torch.randn(t, vd, device=device, generator=g) * 2).bfloat16()
+    lg = (torch.randn(t, vd, device=device, generator=g) * 2).bfloat16()
+    stats = torch.empty(4, t, device=device)
+    arg = torch.empty(2, t, device=device, dtype=torch.int32)
+    st = _lib.stream_ptr(device)
+
+    def loss_fwd():
+        _lib.call("spx_fused_vocab_loss_fwd", L.OP_KL, _lib.ptr(lg), vd, _lib.ptr(tg), vd, t, vd, 0,
+                  _lib.ptr(stats[0]), _lib.ptr(stats[1]), _lib.ptr(stats[2]), _lib.ptr(stats[3]),
+                  _lib.ptr(arg[0]), _lib.ptr(arg[1]), st)
+
+    ms = time_events(torch, loss_fwd, 20)
+    hbm("loss_fwd_kernel[KL, T rows x Vd]", 2.0 * t * vd * 2, ms, k_steps)
+    rg = torch.full((t,), 1.0 / t, device=device)
+    grad = torch.empty(t, vd, device=device, dtype=torch.bfloat16)
+
+    def loss_bwd():
+        _lib.call("spx_fused_vocab_loss_bwd", L.OP_KL, _lib.ptr(lg), vd, _lib.ptr(tg), vd, t, vd, 0,
+                  _lib.ptr(stats[1]), _lib.ptr(stats[2]), _lib.ptr(stats[3]), _lib.ptr(arg[1]),
+                  _lib.ptr(rg), None, _lib.ptr(grad), vd, st)
+
+    ms = time_events(torch, loss_bwd, 20)
+    hbm("loss_bwd_kernel[KL, T rows x Vd]", 3.0 * t * vd * 2, ms, k_steps)
+    del tg, lg, grad, y
+
+    # TTT attention at the last step (k = K-1 diagonals): forward and backward
+    step = k_steps - 1
+    mask = A.create_ttt_mask(torch.zeros(t, dtype=torch.long, device=device), t, None)
+    for _ in range(step):
+        mask = mask.extended()
+    q = torch.randn(1, hq, t, d, device=device, generator=g).bfloat16().requires_grad_(True)
+    kk = torch.randn(1, hkv, (step + 1) * t, d, device=device, generator=g).bfloat16().requires_grad_(True)
+    vv = torch.randn(1, hkv, (step + 1) * t, d, device=device, generator=g).bfloat16().requires_grad_(True)
+    pairs = t * (t + 1) / 2 + step * t
+    ms_f = time_events(torch, lambda: A.ttt_attention(q.detach(), kk.detach(), vv.detach(), mask), 10)
+    mfma(f"ttt_attn_fwd_kernel[step {step}]", 4.0 * pairs * d * hq, ms_f, 1)
+    o = A.ttt_attention(q, kk, vv, mask)
+    go = torch.randn_like(o)
+
+    def attn_bwd():
+        torch.autograd.grad(o, (q, kk, vv), go, retain_graph=True)
+
+    ms_b = time_events(torch, attn_bwd, 10)
+    mfma(f"ttt_attn_bwd[dq+dkv+diag kernels, step {step}]", 10.0 * pairs * d * hq, ms_b, 1)
+    return out
+
+
+def cpu_baseline(cfg, t, k_steps):
+    """The oracle (CPU restatement of the reference eager path) timed on the host cores:
+    one forward + backward at the config[1] shape on a shortened sequence."""
+    import torch
+
+    from oracle import eagle3 as OE
+
+    cores = os.cpu_count() or 1
+    threads = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(threads)
+    shape = OE.DraftShape(**cfg)
+    w = OE.random_weights(shape, seed=0)
+    for name, p in w.items():
+        if name not in ("embed_tokens.weight", "lm_head.weight", "verifier_lm_head.weight",
+                        "verifier_norm.weight"):
+            p.requires_grad_(True)
+    g = torch.Generator().manual_seed(0)
+    hs = torch.randn(1, t, 3 * shape.hidden_size, generator=g) * 4
+    ids = torch.randint(0, shape.vocab_size, (1, t), generator=g)
+    vl = torch.randn(1, t, shape.hidden_size, generator=g)
+    mask = (torch.rand(1, t, generator=g) < 0.7).float()
+    doc = torch.zeros(1, t, dtype=torch.long)
+    t0 = time.perf_counter()
+    _, loss, _ = OE.eagle3_forward(w, shape, hs, ids, doc, mask, None, vl, ttt_steps=k_steps, attn="sdpa")
+    loss.backward()
+    dt = time.perf_counter() - t0
+    return {"value": round(t / dt, 2), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"config[1] shape (Llama-3.1-8B draft, TTT {k_steps}, fp32 oracle), sequence "
+                      f"shortened to {t} tokens, 1 forward+backward, no warm-up, {dt:.1f} s",
+            "loss": round(float(loss), 6)}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (no collectives are built); got --gpus {args.gpus}",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from speculators_amd import _lib
+
+    _lib.load()  # fail loudly if the HIP library is not built
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    t, k_steps = args.seq_len, args.ttt_steps
+    batch, d2t, t2d = make_inputs(torch, CONFIG1, t, device, args.targets == "logits")
+    model = make_model(torch, CONFIG1, device, d2t, t2d)
+    loss_cfg = None  # kl_div, the reference default
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        _, loss, _ = model(**batch, ttt_steps=k_steps, ttt_step_loss_decay=1.0, loss_config=loss_cfg)
+        loss.backward()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    tokens = int((batch["document_ids"] != -1).sum().item())
+    value = tokens / (ms_per_step * 1e-3)
+
+    kernels = [] if args.no_kernels else kernel_rooflines(torch, CONFIG1, t, k_steps, device)
+    dominant = None
+    if kernels:
+        dominant = max(kernels, key=lambda r: r["ms_per_launch"] * r["launches_per_step"])
+    cpu = None
+    if args.cpu_baseline != "off":
+        del model
+        torch.cuda.empty_cache()
+        cpu = cpu_baseline(CONFIG1, args.cpu_seq_len, k_steps)
+
+    line = {
+        "metric": "draft train tokens/sec (fwd+bwd) @Llama-3.1-8B EAGLE3 TTT7",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[1]: EAGLE3 draft, Llama-3.1-8B shape, one draft layer, "
+                               f"batch 1, seq {t}, TTT {k_steps}, vocab 128256 -> draft 32000, "
+                               "kl_div loss, bf16 weights and activations, full attention, "
+                               f"targets from {'verifier hidden states through the frozen verifier head' if args.targets == 'hidden' else 'full-vocab verifier logits gathered through d2t'}",
+                   "seq_len": t, "ttt_steps": k_steps, "tokens_per_step": tokens,
+                   "final_loss": round(float(loss), 6)},
+        "roofline": ({k: dominant[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
+                     | {"kernel": dominant["kernel"]}) if dominant else None,
+        "kernels": kernels,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

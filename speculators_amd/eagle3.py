@@ -1,0 +1,316 @@
+"""EAGLE3 draft model: host side of the HIP training hot path.
+
+Keeps the reference model's call contract
+(``Eagle3DraftModel.forward``, models/eagle3/core.py:192-365):
+
+    forward(hidden_states, input_ids, document_ids, loss_mask, position_ids,
+            verifier_last_hidden_states, ttt_steps, ttt_step_loss_decay,
+            loss_config) -> (draft_tokens, loss, metrics)
+
+and its state-dict names (models/eagle3/core.py:31-42), so a checkpoint of the
+reference loads with ``load_state_dict``.  The attention of every TTT step
+runs on the HIP TTT kernel, fc / lm_head / verifier head on the MFMA GEMM, the
+per-step loss, arg-maxes and acceptance counts on the fused vocabulary loss.
+The decoder-internal projections use PyTorch's (hipBLASLt) matmul.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import attention as A
+from . import gemm
+from . import losses as L
+from . import metrics as MT
+
+
+@dataclass
+class Eagle3Config:
+    """Shape and switches of the draft (the subset of Eagle3SpeculatorConfig +
+    transformer_layer_config the forward reads; models/eagle3/config.py)."""
+
+    hidden_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    intermediate_size: int
+    vocab_size: int  # verifier vocabulary
+    draft_vocab_size: int
+    num_aux: int = 3
+    num_hidden_layers: int = 1
+    rms_norm_eps: float = 1e-5
+    rope_theta: float = 500000.0
+    norm_before_residual: bool = False
+    norm_before_fc: bool = False
+    fc_norm: bool = False
+    norm_output: bool = False
+    qk_norm: bool = False
+    sliding_window: int | None = None
+    sliding_layers: tuple = field(default_factory=tuple)
+    attn_implementation: str = A.ATTN_IMPL_TTT
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim: int, eps: float):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim))
+        self.eps = eps
+
+    def forward(self, x):
+        xf = x.float()
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)
+        return self.weight.to(x.dtype) * xf.to(x.dtype)
+
+
+def _rotate_half(x):
+    h = x.shape[-1] // 2
+    return torch.cat([-x[..., h:], x[..., :h]], dim=-1)
+
+
+def _rope_tables(position_ids, head_dim, theta, dtype):
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32,
+                                        device=position_ids.device) / head_dim))
+    ang = position_ids.reshape(1, -1, 1).float() * inv.reshape(1, 1, -1)
+    ang = torch.cat([ang, ang], dim=-1)
+    return ang.cos().to(dtype), ang.sin().to(dtype)
+
+
+class Attention(nn.Module):
+    def __init__(self, cfg: Eagle3Config, in_features: int):
+        super().__init__()
+        hq, hkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+        self.hq, self.hkv, self.d = hq, hkv, d
+        self.q_proj = nn.Linear(in_features, hq * d, bias=False)
+        self.k_proj = nn.Linear(in_features, hkv * d, bias=False)
+        self.v_proj = nn.Linear(in_features, hkv * d, bias=False)
+        self.o_proj = nn.Linear(hq * d, cfg.hidden_size, bias=False)
+        if cfg.qk_norm:
+            self.q_norm = RMSNorm(d, cfg.rms_norm_eps)
+            self.k_norm = RMSNorm(d, cfg.rms_norm_eps)
+        self.qk_norm = cfg.qk_norm
+        self.scaling = d ** -0.5
+        self.attn_fn = A.ALL_ATTENTION_FUNCTIONS[cfg.attn_implementation]
+
+    def forward(self, x, cos, sin, cache: dict, mask):
+        t = x.shape[1]
+        q = self.q_proj(x).view(1, t, self.hq, self.d)
+        k = self.k_proj(x).view(1, t, self.hkv, self.d)
+        v = self.v_proj(x).view(1, t, self.hkv, self.d)
+        if self.qk_norm:
+            q, k = self.q_norm(q), self.k_norm(k)
+        q, k, v = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
+        c, s = cos.unsqueeze(1), sin.unsqueeze(1)
+        q = q * c + _rotate_half(q) * s
+        k = k * c + _rotate_half(k) * s
+        # the K/V cache grows by T keys per TTT step (DynamicCache.update in the reference)
+        cache["k"] = k if "k" not in cache else torch.cat([cache["k"], k], dim=2)
+        cache["v"] = v if "v" not in cache else torch.cat([cache["v"], v], dim=2)
+        out, _ = self.attn_fn(self, q, cache["k"], cache["v"], mask, scaling=self.scaling)
+        return self.o_proj(out.reshape(1, t, self.hq * self.d))
+
+
+class MLP(nn.Module):
+    def __init__(self, cfg: Eagle3Config):
+        super().__init__()
+        self.gate_proj = nn.Linear(cfg.hidden_size, cfg.intermediate_size, bias=False)
+        self.up_proj = nn.Linear(cfg.hidden_size, cfg.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(cfg.intermediate_size, cfg.hidden_size, bias=False)
+
+    def forward(self, x):
+        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+class DecoderLayer(nn.Module):
+    """Layer 0 carries the EAGLE3 first-layer changes
+    (models/eagle3/model_definitions.py:14-110): q/k/v read ``cat([embeds, hidden])``
+    (2H wide), embeds and hidden are normalised separately, the residual is the
+    (optionally normalised) hidden half."""
+
+    def __init__(self, cfg: Eagle3Config, layer_idx: int):
+        super().__init__()
+        self.first = layer_idx == 0
+        self.cfg = cfg
+        self.self_attn = Attention(cfg, (2 if self.first else 1) * cfg.hidden_size)
+        self.mlp = MLP(cfg)
+        self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+        self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+        if self.first:
+            self.hidden_norm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+
+    def forward(self, x, cos, sin, cache, mask):
+        if self.first:
+            h = self.cfg.hidden_size
+            embeds, hidden = x[..., :h], x[..., h:]
+            residual = hidden
+            embeds = self.input_layernorm(embeds)
+            hidden = self.hidden_norm(hidden)
+            if self.cfg.norm_before_residual:
+                residual = hidden
+            a = self.self_attn(torch.cat([embeds, hidden], dim=-1), cos, sin, cache, mask)
+        else:
+            residual = x
+            a = self.self_attn(self.input_layernorm(x), cos, sin, cache, mask)
+        y = residual + a
+        return y + self.mlp(self.post_attention_layernorm(y))
+
+
+class Eagle3DraftModel(nn.Module):
+    def __init__(self, config: Eagle3Config):
+        super().__init__()
+        self.config = config
+        h = config.hidden_size
+        self.hidden_size = h
+        self.draft_vocab_size = config.draft_vocab_size
+        self.verifier_vocab_size = config.vocab_size
+        self.use_draft_vocab = config.draft_vocab_size != config.vocab_size
+        if self.use_draft_vocab:
+            self.register_buffer("t2d", torch.zeros(config.vocab_size, dtype=torch.bool))
+            self.register_buffer("d2t", torch.zeros(config.draft_vocab_size, dtype=torch.long))
+        else:
+            self.t2d = self.d2t = None
+        self.embed_tokens = nn.Embedding(config.vocab_size, h)
+        self.lm_head = nn.Linear(h, config.draft_vocab_size, bias=False)
+        self.verifier_lm_head = nn.Linear(h, config.draft_vocab_size, bias=False)
+        self.fc = nn.Linear(config.num_aux * h, h, bias=False)
+        self.layers = nn.ModuleList(DecoderLayer(config, i) for i in range(config.num_hidden_layers))
+        self.norm = RMSNorm(h, config.rms_norm_eps)
+        self.verifier_norm = RMSNorm(h, config.rms_norm_eps)
+        self.input_norm = RMSNorm(config.num_aux * h, config.rms_norm_eps) if config.norm_before_fc else None
+        self.fc_norm = (nn.ModuleList(RMSNorm(h, config.rms_norm_eps) for _ in range(config.num_aux))
+                        if config.fc_norm else None)
+        # frozen, as in model.py:63-71 and models/eagle3/core.py:68,120
+        for p in (self.embed_tokens.weight, self.lm_head.weight, self.verifier_lm_head.weight,
+                  self.verifier_norm.weight):
+            p.requires_grad_(False)
+        self.uses_sliding_window_attn = bool(config.sliding_layers)
+        self.uses_full_attn = config.num_hidden_layers > len(config.sliding_layers)
+        self._frozen_t: dict = {}
+
+    # ------------------------------------------------------------------ helpers
+    def load_vocab_mappings(self, t2d, d2t):
+        """Validation rules of model.py:81-121."""
+        if t2d is None and d2t is None:
+            return
+        if t2d is None or d2t is None:
+            raise ValueError("Both t2d and d2t must be provided together, or both must be None.")
+        if not self.use_draft_vocab:
+            return
+        if t2d.shape[0] != self.verifier_vocab_size:
+            raise ValueError(f"t2d.shape[0] ({t2d.shape[0]}) must match verifier_vocab_size "
+                             f"({self.verifier_vocab_size}).")
+        if int(t2d.sum(dtype=torch.long).item()) != self.draft_vocab_size:
+            raise ValueError(f"t2d has {int(t2d.sum(dtype=torch.long).item())} non-zero values, "
+                             f"expected {self.draft_vocab_size}.")
+        if d2t.shape[0] != self.draft_vocab_size:
+            raise ValueError(f"d2t.shape[0] ({d2t.shape[0]}) must match draft_vocab_size "
+                             f"({self.draft_vocab_size}).")
+        self.t2d.copy_(t2d.to(self.t2d.device))
+        self.d2t.copy_(d2t.to(self.d2t.device))
+
+    def _transposed_frozen(self, weight: torch.Tensor) -> torch.Tensor:
+        """``weight.T`` contiguous, cached: frozen weights never change between steps."""
+        key = (weight.data_ptr(), weight._version, weight.dtype)
+        hit = self._frozen_t.get(id(weight))
+        if hit is None or hit[0] != key:
+            hit = (key, weight.detach().t().contiguous())
+            self._frozen_t[id(weight)] = hit
+        return hit[1]
+
+    def _linear(self, x, weight, frozen: bool = False):
+        if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
+            wt = self._transposed_frozen(weight) if frozen and x.requires_grad else None
+            return gemm.linear(x, weight, wt)
+        raise RuntimeError("the HIP draft path runs in bf16: cast the model and its inputs to bfloat16")
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, hidden_states, input_ids, document_ids, loss_mask=None, position_ids=None,
+                verifier_last_hidden_states=None, ttt_steps: int = 3,
+                ttt_step_loss_decay: float = 1.0, loss_config: L.LossConfig | None = None,
+                verifier_logits=None, **_kwargs):
+        """See the module docstring.  ``verifier_logits`` (``[1, T, Vt]`` over the target
+        vocabulary) is an alternative to ``verifier_last_hidden_states``: the targets are
+        then the d2t gather of those logits instead of the row-sliced verifier head."""
+        cfg = self.config
+        device = hidden_states.device
+        t = hidden_states.shape[1]
+        if position_ids is None:
+            position_ids = 1 + torch.arange(t, dtype=torch.long, device=device).unsqueeze(0)
+        doc = document_ids.reshape(-1).to(device)
+        full_mask = A.create_ttt_mask(doc, t, None) if self.uses_full_attn else None
+        sw_mask = (A.create_ttt_mask(doc, t, cfg.sliding_window)
+                   if self.uses_sliding_window_attn else None)
+
+        x = hidden_states
+        if self.input_norm is not None:
+            x = self.input_norm(x)
+        if self.fc_norm is not None:
+            chunks = x.chunk(len(self.fc_norm), dim=-1)
+            x = torch.cat([n(c) for n, c in zip(self.fc_norm, chunks, strict=True)], dim=-1)
+        hidden = self._linear(x, self.fc.weight)
+
+        original_ids = input_ids.detach().clone()
+        return_loss = verifier_last_hidden_states is not None or verifier_logits is not None
+        if return_loss:
+            with torch.no_grad():
+                if verifier_logits is not None:
+                    targets = (L.vocab_gather(verifier_logits, self.d2t) if self.use_draft_vocab
+                               else verifier_logits)
+                else:
+                    targets = self._linear(self.verifier_norm(verifier_last_hidden_states),
+                                           self.verifier_lm_head.weight)
+            loss = torch.zeros((), device=device)
+            prev_correct = (loss_mask.clone() if loss_mask is not None
+                            else torch.ones(1, t, device=device, dtype=torch.bool))
+            metrics: dict = {}
+
+        caches = [dict() for _ in self.layers]
+        draft_tokens = []
+        for step in range(ttt_steps):
+            with torch.no_grad():
+                embeds = F.embedding(input_ids, self.embed_tokens.weight)
+            cos, sin = _rope_tables(position_ids, cfg.head_dim, cfg.rope_theta, hidden.dtype)
+            y = torch.cat([embeds.to(hidden.dtype), hidden], dim=-1)
+            for li, layer in enumerate(self.layers):
+                mask = sw_mask if li in cfg.sliding_layers else full_mask
+                y = layer(y, cos, sin, caches[li], mask)
+            if cfg.norm_output:
+                hidden = self.norm(y)
+                logits = self._linear(hidden, self.lm_head.weight, frozen=True)
+            else:
+                hidden = y
+                logits = self._linear(self.norm(y), self.lm_head.weight, frozen=True)
+
+            if return_loss:
+                s_loss, s_metrics = MT.compute_metrics(
+                    logits, targets, loss_mask, prev_correct, step, ttt_step_loss_decay,
+                    loss_config=loss_config)
+                loss = loss + s_loss
+                metrics.update(s_metrics)
+            draft_tokens.append(MT.argmax_rows(logits.detach()))
+
+            input_ids = torch.cat(
+                [original_ids[:, 1 + step:], original_ids.new_zeros(1, 1 + step)], dim=-1)
+            if full_mask is not None:
+                full_mask = full_mask.extended()
+            if sw_mask is not None:
+                sw_mask = sw_mask.extended()
+            position_ids = position_ids + 1
+
+        if not return_loss:
+            return draft_tokens
+        metrics["loss_sum"] = loss.detach().clone()
+        metrics["loss_total"] = torch.ones((), device=device)
+        return draft_tokens, loss, metrics
+
+    @staticmethod
+    def get_trainer_kwargs(**kwargs):
+        """(train_call_kwargs, val_call_kwargs) like models/eagle3/core.py:428-451."""
+        loss_config = L.resolve_loss_config(kwargs["loss_fn"], kwargs.get("loss_implementation", "hip"))
+        shared = {"ttt_steps": kwargs["ttt_steps"],
+                  "ttt_step_loss_decay": kwargs["ttt_step_loss_decay"],
+                  "loss_config": loss_config}
+        return dict(shared), dict(shared)

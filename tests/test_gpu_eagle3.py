@@ -1,0 +1,140 @@
+"""Whole EAGLE3 draft forward + backward on the HIP path against the CPU oracle."""
+
+import pytest
+import torch
+
+from oracle import eagle3 as OE
+from oracle import losses as OL
+
+pytestmark = pytest.mark.gpu
+
+
+def _shape(**kw):
+    base = dict(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=64,
+                intermediate_size=512, vocab_size=2000, draft_vocab_size=704, rms_norm_eps=1e-5,
+                rope_theta=10000.0)
+    base.update(kw)
+    return OE.DraftShape(**base)
+
+
+def _batch(shape, t, seed, docs):
+    g = torch.Generator().manual_seed(seed)
+    hs = torch.randn(1, t, shape.num_aux * shape.hidden_size, generator=g)
+    ids = torch.randint(0, shape.vocab_size, (1, t), generator=g)
+    vl = torch.randn(1, t, shape.hidden_size, generator=g)
+    mask = (torch.rand(1, t, generator=g) < 0.7).float()
+    doc = torch.full((1, t), -1, dtype=torch.long)
+    pos = torch.zeros(1, t, dtype=torch.long)
+    o = 0
+    for i, n in enumerate(docs):
+        doc[0, o:o + n] = i
+        pos[0, o:o + n] = 1 + torch.arange(n)
+        o += n
+    mask[0, o:] = 0
+    return hs, ids, doc, mask, pos, vl
+
+
+def _make(shape, w):
+    from speculators_amd.eagle3 import Eagle3Config, Eagle3DraftModel
+
+    cfg = Eagle3Config(**{k: getattr(shape, k) for k in (
+        "hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim", "intermediate_size",
+        "vocab_size", "draft_vocab_size", "num_aux", "num_hidden_layers", "rms_norm_eps", "rope_theta",
+        "norm_before_residual", "norm_before_fc", "fc_norm", "norm_output", "qk_norm",
+        "sliding_window", "sliding_layers")})
+    model = Eagle3DraftModel(cfg)
+    missing, unexpected = model.load_state_dict(w, strict=False)
+    assert not unexpected and set(missing) <= {"t2d", "d2t"}, (missing, unexpected)
+    return model.to(torch.bfloat16).cuda()
+
+
+VARIANTS = [
+    dict(),
+    dict(norm_before_residual=True, norm_output=True, norm_before_fc=True),
+    dict(num_hidden_layers=2, sliding_window=48, sliding_layers=(0,), qk_norm=True),
+]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_forward_backward_matches_oracle(variant):
+    shape = _shape(**variant)
+    w32 = OE.random_weights(shape, seed=1, std=0.05)
+    g = torch.Generator().manual_seed(11)
+    for k_ in w32:  # non-trivial norm gains
+        if k_.endswith("norm.weight") or "layernorm" in k_:
+            w32[k_] = 1 + 0.1 * torch.randn(w32[k_].shape, generator=g)
+    w = {k_: v.bfloat16() for k_, v in w32.items()}  # both sides start from the same bf16 values
+    t, steps = 320, 3
+    hs, ids, doc, mask, pos, vl = _batch(shape, t, 2, [120, 170])
+    hs, vl = hs.bfloat16(), vl.bfloat16()
+
+    model = _make(shape, w)
+    toks, loss, m = model(hs.cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.cuda(),
+                          ttt_steps=steps, ttt_step_loss_decay=0.9)
+    loss.backward()
+
+    wf = {k_: v.float().requires_grad_(v.dtype.is_floating_point) for k_, v in w.items()}
+    rt, rloss, rm, rlogits = OE.eagle3_forward(
+        wf, shape, hs.float(), ids, doc, mask, pos, vl.float(), ttt_steps=steps,
+        ttt_step_loss_decay=0.9, return_logits=True)
+    rloss.backward()
+
+    rel = abs(loss.item() - rloss.item()) / abs(rloss.item())
+    print("loss", loss.item(), rloss.item(), rel)
+    assert rel < 5e-3  # bf16 activations against an fp32 oracle
+    assert set(m) == set(rm)
+    for key in rm:
+        if key.endswith("_total"):
+            assert m[key].item() == rm[key].item(), key  # mask / row counts: exact
+    for name, p in model.named_parameters():
+        if not p.requires_grad:
+            assert p.grad is None
+            continue
+        want = wf[name].grad
+        err = (p.grad.float().cpu() - want).abs().max().item()
+        assert err <= 3e-2 * want.abs().max().item() + 1e-6, (name, err, want.abs().max().item())
+    assert len(toks) == steps and toks[0].shape == (1, t) and toks[0].dtype == torch.int64
+    # draft tokens are an arg-max of bf16 logits: compare where the oracle's top-2 margin is clear
+    for k in range(steps):
+        top2 = rlogits[k].topk(2, dim=-1).values
+        clear = (top2[..., 0] - top2[..., 1]) > 0.05 * top2[..., 0].abs().clamp_min(1.0)
+        assert torch.equal(toks[k].cpu()[clear], rt[k][clear])
+
+
+def test_verifier_logits_entry_point_equals_row_sliced_head():
+    """targets from a d2t gather of full-vocab verifier logits == the row-sliced verifier head."""
+    from oracle import vocab as OV
+
+    shape = _shape()
+    w = {k_: v.bfloat16() for k_, v in OE.random_weights(shape, seed=3, std=0.05).items()}
+    g = torch.Generator().manual_seed(5)
+    sel = torch.randperm(shape.vocab_size, generator=g)[: shape.draft_vocab_size]
+    d2t, t2d = OV.build_vocab_mappings(sel.tolist(), shape.vocab_size)
+    full_head = (torch.randn(shape.vocab_size, shape.hidden_size, generator=g) * 0.05).bfloat16()
+    w["verifier_lm_head.weight"] = full_head[t2d]
+    model = _make(shape, w)
+    model.load_vocab_mappings(t2d, d2t)
+    t = 128
+    hs, ids, doc, mask, pos, vl = _batch(shape, t, 6, [128])
+    hs, vl = hs.bfloat16().cuda(), vl.bfloat16().cuda()
+    args = (hs, ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda())
+    _, loss_a, m_a = model(*args, verifier_last_hidden_states=vl, ttt_steps=2)
+    with torch.no_grad():
+        full_logits = torch.nn.functional.linear(model.verifier_norm(vl), full_head.cuda())
+    _, loss_b, m_b = model(*args, verifier_logits=full_logits, ttt_steps=2)
+    assert loss_a.item() == pytest.approx(loss_b.item(), rel=2e-3)
+    for key in m_a:
+        if "acc" in key and key.endswith("_total"):
+            assert m_a[key].item() == m_b[key].item()
+
+
+def test_requires_bf16_and_hip_tensors():
+    from speculators_amd._lib import SpxError
+
+    shape = _shape()
+    w = OE.random_weights(shape, seed=3)
+    from speculators_amd.eagle3 import Eagle3Config, Eagle3DraftModel
+    model = _make(shape, {k_: v.bfloat16() for k_, v in w.items()})
+    hs, ids, doc, mask, pos, vl = _batch(shape, 128, 6, [128])
+    with pytest.raises(RuntimeError):
+        model(hs.cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.cuda(), ttt_steps=1)
