@@ -169,6 +169,54 @@ int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
                      void* dv, int64_t dv_head_stride, void* workspace,
                      int64_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------- DFlash attention
+ * Per-row key intervals of the anchored-block mask, create_anchor_block_mask_mod
+ * (models/dflash/attention.py:7-100), for run-contiguous document ids.  Row
+ * r = j*block_size + s belongs to anchor j (position a_j):
+ *   context keys  ctx_lo[r] <= c < ctx_hi[r]:  ctx_hi = a_j, ctx_lo = start of
+ *     a_j's document, raised to a_j - W under a sliding window W (<= 0: none);
+ *     empty when a_j sits on a padding position;
+ *   block keys (rows T + c of k/v)  blk_lo[r] <= c < blk_hi[r]:  the rows of the
+ *     query's own block, all of them, or only c <= r when causal_block != 0
+ *     (a sliding-window layer without sliding_window_non_causal).
+ * run_start_scratch: int32 [T] scratch.  Replaces the compiled create_block_mask
+ * of models/dflash/core.py:273-328. */
+int spx_dflash_row_ranges(const void* document_ids, int doc_kind, int64_t T,
+                          const void* anchors, int anchor_kind, int64_t n_anchors,
+                          int32_t block_size, int64_t sliding_window,
+                          int32_t causal_block, int32_t* ctx_lo, int32_t* ctx_hi,
+                          int32_t* blk_lo, int32_t* blk_hi,
+                          int32_t* run_start_scratch, void* stream);
+
+int64_t spx_dflash_attn_workspace_bytes(int64_t T, int64_t NQ, int32_t Hq,
+                                        int32_t Hkv, int32_t D, int32_t backward);
+
+/* Anchored-block attention: q bf16 [Hq, NQ, D] (NQ = n_anchors * block_size mask
+ * tokens), k/v bf16 [Hkv, T + NQ, D] = context keys followed by the mask-token
+ * keys (the concatenation Qwen3DFlashAttention builds,
+ * models/dflash/model_definitions.py:97-155); out bf16 [NQ, Hq, D]; lse f32
+ * [Hq, NQ] (opaque).  Replaces flex_attention_forward (models/attention.py:20-66)
+ * for the DFlash mask. */
+int spx_dflash_attn_fwd(const void* q, int64_t q_head_stride, const void* k,
+                        int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                        const int32_t* ctx_lo, const int32_t* ctx_hi,
+                        const int32_t* blk_lo, const int32_t* blk_hi, int64_t T,
+                        int64_t NQ, int32_t Hq, int32_t Hkv, int32_t D,
+                        float scaling, void* out, float* lse, void* workspace,
+                        int64_t workspace_bytes, void* stream);
+
+/* Gradients of spx_dflash_attn_fwd: dq [Hq, NQ, D], dk / dv [Hkv, T + NQ, D],
+ * every row written, deterministic. */
+int spx_dflash_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
+                        int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                        const void* out, const void* dout, const float* lse,
+                        const int32_t* ctx_lo, const int32_t* ctx_hi,
+                        const int32_t* blk_lo, const int32_t* blk_hi, int64_t T,
+                        int64_t NQ, int32_t Hq, int32_t Hkv, int32_t D,
+                        float scaling, void* dq, int64_t dq_head_stride, void* dk,
+                        int64_t dk_head_stride, void* dv, int64_t dv_head_stride,
+                        void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------- GEMM
  * c[M, N] = a[M, K] * b[N, K]^T, bf16 inputs, fp32 accumulation, bf16 output:
  * the product of torch.nn.Linear (no bias).  Replaces the fc Linear

@@ -13,7 +13,7 @@ from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libspx_hip.so")
+LIB_PATH = os.environ.get("SPX_LIB_PATH") or os.path.join(_HERE, "libspx_hip.so")
 
 _P, _I64, _I, _F = c_void_p, c_int64, c_int, c_float
 
@@ -34,8 +34,15 @@ SIGNATURES: dict[str, list] = {
     "spx_ttt_attn_bwd": [_P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32,
                          _F, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P],
 }
+SIGNATURES["spx_dflash_row_ranges"] = [_P, _I, _I64, _P, _I, _I64, _I32, _I64, _I32, _P, _P, _P, _P, _P, _P]
+SIGNATURES["spx_dflash_attn_workspace_bytes"] = [_I64, _I64, _I32, _I32, _I32, _I32]
+SIGNATURES["spx_dflash_attn_fwd"] = [_P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _P, _I64, _I64, _I32,
+                                     _I32, _I32, _F, _P, _P, _P, _I64, _P]
+SIGNATURES["spx_dflash_attn_bwd"] = [_P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I64,
+                                     _I64, _I32, _I32, _I32, _F, _P, _I64, _P, _I64, _P, _I64, _P,
+                                     _I64, _P]
 SIGNATURES["spx_gemm_bf16_nt"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P]
-RESTYPES = {"spx_ttt_attn_workspace_bytes": c_int64}
+RESTYPES = {"spx_ttt_attn_workspace_bytes": c_int64, "spx_dflash_attn_workspace_bytes": c_int64}
 
 _lib = None
 

@@ -1,0 +1,1302 @@
+// Draft-model attention for gfx950: EAGLE3 test-time-training (TTT) attention
+// and DFlash anchored-block attention, forward and backward, from one family
+// of interval-masked flash-attention kernels.
+//
+// Every query row r sees up to two key INTERVALS of the K/V rows, plus (TTT
+// only) a few single keys:
+//   * context keys      a1[r] <= c < b1[r]          (rows [0, T) of K/V)
+//   * block keys    T + a2[r] <= c < T + b2[r]      (rows [T, T+NQ): DFlash's own
+//                                                    mask-token block)
+//   * TTT diagonal keys: rows j*T + r, j = 1..n_extra -- ONE key per earlier
+//     step, handled as n_extra dot products per row instead of 128x128 tiles.
+// TTT:    a1 = row_lo (document start / window / the row itself for padding),
+//         b1 = r + 1, no block interval.
+// DFlash: a1 = max(doc start, anchor - W), b1 = anchor, a2/b2 = the query's own
+//         block (all of it, or up to the query under a causal window layer).
+// Key tiles that no row of a workgroup can see are skipped analytically; no
+// dense mask or BlockMask exists anywhere.
+
+#include "attn_common.h"
+#include "../../include/spx.h"
+
+namespace spx {
+
+struct AttnParams {
+  const uint16_t* Q; int64_t q_hs;   // [Hq][NQ][D]
+  const uint16_t* K; int64_t k_hs;   // [Hkv][>= NKV (+ n_extra*T)][D]
+  const uint16_t* V; int64_t v_hs;
+  const int32_t* a1; const int32_t* b1;  // b1 == nullptr: b1[r] = r + 1
+  const int32_t* a2; const int32_t* b2;  // nullptr: no block interval
+  int NQ, T, NKV, NKVp;  // NKVp: row length of the transposed operands (multiple of 128)
+  int n_extra, Hq, Hkv;
+  float scale_log2e, scaling;
+};
+
+// ---------------------------------------------------------------- mask descriptors
+template <typename I>
+__global__ __launch_bounds__(1024) void ttt_row_lo_kernel(const I* __restrict__ doc, int64_t T,
+                                                          int64_t window, int32_t* __restrict__ lo) {
+  __shared__ int seg_max[1024];
+  const int t = threadIdx.x;
+  const int64_t len = (T + 1023) / 1024;
+  const int64_t b = t * len, e = (b + len < T) ? b + len : T;
+  int run = -1;
+  for (int64_t i = b; i < e; ++i)
+    if (i == 0 || doc[i] != doc[i - 1]) run = (int)i;
+  seg_max[t] = run;
+  __syncthreads();
+  int carry = -1;
+  for (int s = 0; s < t; ++s) carry = max(carry, seg_max[s]);
+  run = carry;
+  for (int64_t i = b; i < e; ++i) {
+    if (i == 0 || doc[i] != doc[i - 1]) run = (int)i;
+    int v = run;
+    if (doc[i] == (I)-1) v = (int)i;
+    else if (window > 0 && i - window + 1 > v) v = (int)(i - window + 1);
+    lo[i] = v;
+  }
+}
+
+// start of the run of equal document ids that contains position i
+template <typename I>
+__global__ __launch_bounds__(1024) void doc_run_start_kernel(const I* __restrict__ doc, int64_t T,
+                                                             int32_t* __restrict__ start) {
+  __shared__ int seg_max[1024];
+  const int t = threadIdx.x;
+  const int64_t len = (T + 1023) / 1024;
+  const int64_t b = t * len, e = (b + len < T) ? b + len : T;
+  int run = -1;
+  for (int64_t i = b; i < e; ++i)
+    if (i == 0 || doc[i] != doc[i - 1]) run = (int)i;
+  seg_max[t] = run;
+  __syncthreads();
+  int carry = -1;
+  for (int s = 0; s < t; ++s) carry = max(carry, seg_max[s]);
+  run = carry;
+  for (int64_t i = b; i < e; ++i) {
+    if (i == 0 || doc[i] != doc[i - 1]) run = (int)i;
+    start[i] = run;
+  }
+}
+
+template <typename I, typename J>
+__global__ __launch_bounds__(256) void dflash_ranges_kernel(
+    const I* __restrict__ doc, const int32_t* __restrict__ run_start, const J* __restrict__ anchors,
+    int64_t n_anchors, int block_size, int64_t window, int causal_block, int64_t T,
+    int32_t* __restrict__ a1, int32_t* __restrict__ b1, int32_t* __restrict__ a2,
+    int32_t* __restrict__ b2) {
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= n_anchors * block_size) return;
+  const int64_t j = r / block_size;
+  int64_t a = (int64_t)anchors[j];
+  a = a < 0 ? 0 : (a >= T ? T - 1 : a);
+  int lo = 0, hi = 0;
+  if (doc[a] != (I)-1) {
+    lo = run_start[a];
+    if (window > 0 && a - window > lo) lo = (int)(a - window);
+    hi = (int)a;
+    if (hi < lo) hi = lo;
+  }
+  a1[r] = lo;
+  b1[r] = hi;
+  a2[r] = (int)(j * block_size);
+  b2[r] = causal_block ? (int)(r + 1) : (int)((j + 1) * block_size);
+}
+
+// ---------------------------------------------------------------- transpose
+// dst[h][c][r] = src[h][r][c] for r < rows, c < cols; dst row stride ld_dst >= rows,
+// columns rows..ld_dst-1 of dst are zero filled.  64x64 tiles through LDS.
+__global__ __launch_bounds__(256) void transpose_bf16_kernel(
+    const uint16_t* __restrict__ src, int64_t src_hs, int64_t src_ld, int rows, int cols,
+    uint16_t* __restrict__ dst, int64_t dst_hs, int64_t ld_dst) {
+  __shared__ uint16_t tile[64][66];
+  const int h = blockIdx.z;
+  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  const uint16_t* s = src + (int64_t)h * src_hs;
+  uint16_t* d = dst + (int64_t)h * dst_hs;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int rr = ty; rr < 64; rr += 4) {
+    int r = r0 + rr, c = c0 + tx;
+    tile[rr][tx] = (r < rows && c < cols) ? s[(int64_t)r * src_ld + c] : (uint16_t)0;
+  }
+  __syncthreads();
+  for (int cc = ty; cc < 64; cc += 4) {
+    int c = c0 + cc, r = r0 + tx;
+    if (c < cols && r < ld_dst) d[(int64_t)c * ld_dst + r] = tile[tx][cc];
+  }
+}
+
+// per-lane intervals of the NSB query rows a lane owns, and their wave / block extents
+template <int NSB>
+struct RowBounds {
+  int a1[NSB], b1[NSB], a2[NSB], b2[NSB];
+  int w_a1min, w_a1max, w_b1min, w_b1max;
+  int w_a2min, w_a2max, w_b2min, w_b2max;
+  int blk_a1, blk_b1, blk_a2, blk_b2;
+};
+
+__device__ __forceinline__ int wave_min_i(int v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v = min(v, __shfl_xor(v, m, 64));
+  return v;
+}
+__device__ __forceinline__ int wave_max_i(int v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v = max(v, __shfl_xor(v, m, 64));
+  return v;
+}
+
+template <int NSB, int NW>
+__device__ __forceinline__ void load_bounds(const AttnParams& p, const int (&ic)[NSB], int wave,
+                                            int lane, int* red /* [4 * NW] LDS */, RowBounds<NSB>& rb) {
+  int a1mn = 0x7fffffff, a1mx = 0, b1mn = 0x7fffffff, b1mx = 0;
+  int a2mn = 0x7fffffff, a2mx = 0, b2mn = 0x7fffffff, b2mx = 0;
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) {
+    rb.a1[sb] = p.a1[ic[sb]];
+    rb.b1[sb] = p.b1 ? p.b1[ic[sb]] : ic[sb] + 1;
+    if (p.a2) {
+      rb.a2[sb] = p.T + p.a2[ic[sb]];
+      rb.b2[sb] = p.T + p.b2[ic[sb]];
+    } else {
+      rb.a2[sb] = 0; rb.b2[sb] = 0;
+    }
+    a1mn = min(a1mn, rb.a1[sb]); a1mx = max(a1mx, rb.a1[sb]);
+    b1mn = min(b1mn, rb.b1[sb]); b1mx = max(b1mx, rb.b1[sb]);
+    a2mn = min(a2mn, rb.a2[sb]); a2mx = max(a2mx, rb.a2[sb]);
+    b2mn = min(b2mn, rb.b2[sb]); b2mx = max(b2mx, rb.b2[sb]);
+  }
+  rb.w_a1min = wave_min_i(a1mn); rb.w_a1max = wave_max_i(a1mx);
+  rb.w_b1min = wave_min_i(b1mn); rb.w_b1max = wave_max_i(b1mx);
+  rb.w_a2min = wave_min_i(a2mn); rb.w_a2max = wave_max_i(a2mx);
+  rb.w_b2min = wave_min_i(b2mn); rb.w_b2max = wave_max_i(b2mx);
+  if (lane == 0) {
+    red[wave * 4 + 0] = rb.w_a1min; red[wave * 4 + 1] = rb.w_b1max;
+    red[wave * 4 + 2] = rb.w_a2min; red[wave * 4 + 3] = rb.w_b2max;
+  }
+  __syncthreads();
+  rb.blk_a1 = red[0]; rb.blk_b1 = red[1]; rb.blk_a2 = red[2]; rb.blk_b2 = red[3];
+#pragma unroll
+  for (int w = 1; w < NW; ++w) {
+    rb.blk_a1 = min(rb.blk_a1, red[w * 4 + 0]); rb.blk_b1 = max(rb.blk_b1, red[w * 4 + 1]);
+    rb.blk_a2 = min(rb.blk_a2, red[w * 4 + 2]); rb.blk_b2 = max(rb.blk_b2, red[w * 4 + 3]);
+  }
+}
+
+// ---------------------------------------------------------------- forward
+// One workgroup = 4 waves = 4 * 32 * NSB query rows of one head.  With NSB = 2 a
+// wave owns two 32-row sub-blocks, so every K / V^T fragment read from LDS
+// feeds two MFMAs (LDS bandwidth, not the matrix core, bounds NSB = 1).
+template <int D, int NSB, int NW, bool PF>
+__global__ __launch_bounds__(64 * NW) void attn_fwd_kernel(AttnParams p,
+                                                                const uint16_t* __restrict__ Vt,
+                                                                uint16_t* __restrict__ O,
+                                                                float* __restrict__ LSE) {
+  constexpr int KS = D + kKPad;
+  constexpr int VS = kBN + kVPad;
+  constexpr int NKK = D / 16;
+  constexpr int NDB = D / 32;
+  constexpr int NT = 64 * NW;
+  constexpr int CPT = (kBN * D / 8) / NT;
+  constexpr int BMW = 32 * NSB;
+  constexpr int BM = NW * BMW;
+
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[kBN * KS];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[D * VS];
+  __shared__ int red[4 * NW];
+
+  const int group = p.Hq / p.Hkv;
+  const int L = blockIdx.x;
+  const int kvh = L % p.Hkv;
+  const int rest = L / p.Hkv;
+  const int h = kvh * group + rest % group;
+  const int n_qb = (p.NQ + BM - 1) / BM;
+  const int qb = n_qb - 1 - rest / group;  // late (heavy, under a causal mask) blocks first
+  const int m0 = qb * BM;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 5, col = lane & 31;
+  int i[NSB], ic[NSB];
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) {
+    i[sb] = m0 + wave * BMW + sb * 32 + col;
+    ic[sb] = i[sb] < p.NQ ? i[sb] : p.NQ - 1;
+  }
+  RowBounds<NSB> rb;
+  load_bounds<NSB, NW>(p, ic, wave, lane, red, rb);
+
+  bf16x8 qf[NSB][NKK];
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) {
+    const uint16_t* qrow = p.Q + (int64_t)h * p.q_hs + (int64_t)ic[sb] * D + g * 8;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk)
+      qf[sb][kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(qrow + kk * 16));
+  }
+  f32x16 acc[NSB][NDB];
+  float m_run[NSB], l_run[NSB];
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) {
+    m_run[sb] = kNegBig; l_run[sb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[sb][db][r] = 0.f;
+  }
+
+  const uint16_t* Kh = p.K + (int64_t)kvh * p.k_hs;
+  const uint16_t* Vth = Vt + (int64_t)kvh * D * p.NKVp;
+  const int last_row = p.NKV - 1;
+
+  u32x4 kreg[CPT], vreg[CPT];
+  auto fetch = [&](int n0) {
+#pragma unroll
+    for (int n = 0; n < CPT; ++n) {
+      const int c = tid + NT * n;
+      const int krow = c / (D / 8), kcol = (c % (D / 8)) * 8;
+      const int kr = min(n0 + krow, last_row);
+      kreg[n] = *reinterpret_cast<const u32x4*>(Kh + (int64_t)kr * D + kcol);
+      const int vd = c >> 3, vcol = (c & 7) * 8;
+      vreg[n] = *reinterpret_cast<const u32x4*>(Vth + (int64_t)vd * p.NKVp + n0 + vcol);
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int n = 0; n < CPT; ++n) {
+      const int c = tid + NT * n;
+      const int krow = c / (D / 8), kcol = (c % (D / 8)) * 8;
+      *reinterpret_cast<u32x4*>(&Ks[krow * KS + kcol]) = kreg[n];
+      const int vd = c >> 3, vcol = (c & 7) * 8;
+      u32x2 a = {vreg[n].x, vreg[n].y}, b = {vreg[n].z, vreg[n].w};
+      *reinterpret_cast<u32x2*>(&Vs[vd * VS + vcol]) = a;
+      *reinterpret_cast<u32x2*>(&Vs[vd * VS + vcol + 4]) = b;
+    }
+  };
+
+  auto direct = [&](int n0) {  // global -> LDS without holding the tile in registers
+#pragma unroll
+    for (int n = 0; n < CPT; ++n) {
+      const int c = tid + NT * n;
+      const int krow = c / (D / 8), kcol = (c % (D / 8)) * 8;
+      const int kr = min(n0 + krow, last_row);
+      *reinterpret_cast<u32x4*>(&Ks[krow * KS + kcol]) =
+          *reinterpret_cast<const u32x4*>(Kh + (int64_t)kr * D + kcol);
+      const int vd = c >> 3, vcol = (c & 7) * 8;
+      const u32x4 t = *reinterpret_cast<const u32x4*>(Vth + (int64_t)vd * p.NKVp + n0 + vcol);
+      u32x2 a = {t.x, t.y}, b = {t.z, t.w};
+      *reinterpret_cast<u32x2*>(&Vs[vd * VS + vcol]) = a;
+      *reinterpret_cast<u32x2*>(&Vs[vd * VS + vcol + 4]) = b;
+    }
+  };
+
+  // one pass over the key tiles of one interval class
+  auto run_pass = [&](const int (&aa)[NSB], const int (&bb)[NSB], int w_amin, int w_amax,
+                      int w_bmin, int w_bmax, int blk_a, int blk_b) {
+    if (blk_b <= blk_a) return;
+    const int n_begin = (blk_a / kBN) * kBN;
+    if (PF) fetch(n_begin);
+    for (int n0 = n_begin; n0 < blk_b; n0 += kBN) {
+      __syncthreads();
+      if (PF) stash(); else direct(n0);
+      __syncthreads();
+      if (PF && n0 + kBN < blk_b) fetch(n0 + kBN);
+      if (n0 >= w_bmax || n0 + kBN <= w_amin) continue;  // nothing visible for this wave
+
+      f32x16 st[NSB][2];
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) st[sb][kb][r] = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const uint16_t* krow = &Ks[(kb * 32 + col) * KS + g * 8];
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk) {
+          const bf16x8 ka = as_bf16x8(*reinterpret_cast<const u32x4*>(krow + kk * 16));
+#pragma unroll
+          for (int sb = 0; sb < NSB; ++sb) st[sb][kb] = mfma32(ka, qf[sb][kk], st[sb][kb]);
+        }
+      }
+      const bool need_mask = (n0 < w_amax) || (n0 + kBN > w_bmin);
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            float s = st[sb][kb][r] * p.scale_log2e;
+            if (need_mask) {
+              const int c = n0 + kb * 32 + acc_row(r, g);
+              if (c < aa[sb] || c >= bb[sb]) s = -INFINITY;
+            }
+            st[sb][kb][r] = s;
+            mx = fmaxf(mx, s);
+          }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run[sb], mx);
+        const float alpha = fast_exp2(m_run[sb] - m_new);
+        float rs = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float pv = fast_exp2(st[sb][kb][r] - m_new);
+            st[sb][kb][r] = pv;
+            rs += pv;
+          }
+        rs += __shfl_xor(rs, 32, 64);
+        l_run[sb] = l_run[sb] * alpha + rs;
+        m_run[sb] = m_new;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[sb][db][r] *= alpha;
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        bf16x8 pb[NSB];
+#pragma unroll
+        for (int sb = 0; sb < NSB; ++sb) pb[sb] = pack8(st[sb][s >> 1], (s & 1) * 8);
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          const uint16_t* vrow = &Vs[(db * 32 + col) * VS + s * 16 + 4 * g];
+          const bf16x8 va = join_bf16x4(*reinterpret_cast<const u32x2*>(vrow),
+                                        *reinterpret_cast<const u32x2*>(vrow + 8));
+#pragma unroll
+          for (int sb = 0; sb < NSB; ++sb) acc[sb][db] = mfma32(va, pb[sb], acc[sb][db]);
+        }
+      }
+    }
+  };
+
+  run_pass(rb.a1, rb.b1, rb.w_a1min, rb.w_a1max, rb.w_b1min, rb.w_b1max, rb.blk_a1, rb.blk_b1);
+  if (p.a2)
+    run_pass(rb.a2, rb.b2, rb.w_a2min, rb.w_a2max, rb.w_b2min, rb.w_b2max, rb.blk_a2, rb.blk_b2);
+
+  // TTT diagonal keys (j, r), j = 1..n_extra: one dot product each
+  for (int j = 1; j <= p.n_extra; ++j) {
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb) {
+      const uint16_t* kj = p.K + (int64_t)kvh * p.k_hs + ((int64_t)j * p.T + ic[sb]) * D + g * 8;
+      float dot = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+        float kv[8];
+        unpack8(*reinterpret_cast<const u32x4*>(kj + kk * 16), kv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dot = fmaf((float)qf[sb][kk][e], kv[e], dot);
+      }
+      dot += __shfl_xor(dot, 32, 64);
+      const float s = dot * p.scale_log2e;
+      const float m_new = fmaxf(m_run[sb], s);
+      const float alpha = fast_exp2(m_run[sb] - m_new);
+      const float pv = fast_exp2(s - m_new);
+      l_run[sb] = l_run[sb] * alpha + pv;
+      m_run[sb] = m_new;
+      const uint16_t* vj = p.V + (int64_t)kvh * p.v_hs + ((int64_t)j * p.T + ic[sb]) * D + 4 * g;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          float vv[4];
+          unpack4(*reinterpret_cast<const u32x2*>(vj + db * 32 + 8 * r4), vv);
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            acc[sb][db][r4 * 4 + t] = fmaf(pv, vv[t], acc[sb][db][r4 * 4 + t] * alpha);
+        }
+    }
+  }
+
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) {
+    if (i[sb] >= p.NQ) continue;
+    const float inv = l_run[sb] > 0.f ? 1.f / l_run[sb] : 0.f;
+    uint16_t* orow = O + ((int64_t)i[sb] * p.Hq + h) * D + 4 * g;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        u32x2 w;
+        w.x = pack_bf16x2(acc[sb][db][r4 * 4 + 0] * inv, acc[sb][db][r4 * 4 + 1] * inv);
+        w.y = pack_bf16x2(acc[sb][db][r4 * 4 + 2] * inv, acc[sb][db][r4 * 4 + 3] * inv);
+        *reinterpret_cast<u32x2*>(orow + db * 32 + 8 * r4) = w;
+      }
+    // a row that sees no key at all (cannot happen for the two masks built here) gets lse = 0
+    if (g == 0) LSE[(int64_t)h * p.NQ + i[sb]] = l_run[sb] > 0.f ? m_run[sb] + fast_log2(l_run[sb]) : 0.f;
+  }
+}
+
+// ---------------------------------------------------------------- backward
+// delta[h, i] = sum_d dO[i, h, d] * O[i, h, d]
+template <int D>
+__global__ __launch_bounds__(256) void attn_delta_kernel(const uint16_t* __restrict__ O,
+                                                         const uint16_t* __restrict__ dO, int NQ,
+                                                         int Hq, float* __restrict__ delta) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // = i * Hq + h
+  if (row >= (int64_t)NQ * Hq) return;
+  const int lane = threadIdx.x & 63;
+  float acc = 0.f;
+  for (int d = lane * 2; d < D; d += 128) {
+    uint32_t a = *reinterpret_cast<const uint32_t*>(O + row * D + d);
+    uint32_t b = *reinterpret_cast<const uint32_t*>(dO + row * D + d);
+    acc = fmaf(bf16_lo(a), bf16_lo(b), acc);
+    acc = fmaf(bf16_hi(a), bf16_hi(b), acc);
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) delta[(row % Hq) * (int64_t)NQ + row / Hq] = acc;
+}
+
+// dQ: same tiling as the forward.
+//   P^T = exp2(S'^T - lse), dP^T = V dO^T, dS^T = P^T (dP^T - delta), dQ^T += K^T dS^T
+template <int D, int NSB, int NW, bool PF>
+__global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(
+    AttnParams p, const uint16_t* __restrict__ dO, const uint16_t* __restrict__ Kt,
+    const float* __restrict__ LSE, const float* __restrict__ Delta, uint16_t* __restrict__ dQ,
+    int64_t dq_hs) {
+  constexpr int KS = D + kKPad;
+  constexpr int VS = kBN + kVPad;
+  constexpr int NKK = D / 16;
+  constexpr int NDB = D / 32;
+  constexpr int NT = 64 * NW;
+  constexpr int CPT = (kBN * D / 8) / NT;
+  constexpr int BMW = 32 * NSB;
+  constexpr int BM = NW * BMW;
+
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[kBN * KS];
+  __shared__ __attribute__((aligned(16))) uint16_t Vn[kBN * KS];
+  __shared__ __attribute__((aligned(16))) uint16_t Kts[D * VS];
+  __shared__ int red[4 * NW];
+
+  const int group = p.Hq / p.Hkv;
+  const int L = blockIdx.x;
+  const int kvh = L % p.Hkv;
+  const int rest = L / p.Hkv;
+  const int h = kvh * group + rest % group;
+  const int n_qb = (p.NQ + BM - 1) / BM;
+  const int qb = n_qb - 1 - rest / group;
+  const int m0 = qb * BM;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 5, col = lane & 31;
+  int i[NSB], ic[NSB];
+  float lse_i[NSB], delta_i[NSB];
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) {
+    i[sb] = m0 + wave * BMW + sb * 32 + col;
+    ic[sb] = i[sb] < p.NQ ? i[sb] : p.NQ - 1;
+    lse_i[sb] = LSE[(int64_t)h * p.NQ + ic[sb]];
+    delta_i[sb] = Delta[(int64_t)h * p.NQ + ic[sb]];
+  }
+  RowBounds<NSB> rb;
+  load_bounds<NSB, NW>(p, ic, wave, lane, red, rb);
+
+  bf16x8 qf[NSB][NKK], dof[NSB][NKK];
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) {
+    const uint16_t* qrow = p.Q + (int64_t)h * p.q_hs + (int64_t)ic[sb] * D + g * 8;
+    const uint16_t* drow = dO + ((int64_t)ic[sb] * p.Hq + h) * D + g * 8;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      qf[sb][kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(qrow + kk * 16));
+      dof[sb][kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(drow + kk * 16));
+    }
+  }
+  f32x16 acc[NSB][NDB];
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[sb][db][r] = 0.f;
+
+  const uint16_t* Kh = p.K + (int64_t)kvh * p.k_hs;
+  const uint16_t* Vh = p.V + (int64_t)kvh * p.v_hs;
+  const uint16_t* Kth = Kt + (int64_t)kvh * D * p.NKVp;
+  const int last_row = p.NKV - 1;
+
+  u32x4 kreg[CPT], vreg[CPT], treg[CPT];
+  auto fetch = [&](int n0) {
+#pragma unroll
+    for (int n = 0; n < CPT; ++n) {
+      const int c = tid + NT * n;
+      const int krow = c / (D / 8), kcol = (c % (D / 8)) * 8;
+      const int kr = min(n0 + krow, last_row);
+      kreg[n] = *reinterpret_cast<const u32x4*>(Kh + (int64_t)kr * D + kcol);
+      vreg[n] = *reinterpret_cast<const u32x4*>(Vh + (int64_t)kr * D + kcol);
+      const int vd = c >> 3, vcol = (c & 7) * 8;
+      treg[n] = *reinterpret_cast<const u32x4*>(Kth + (int64_t)vd * p.NKVp + n0 + vcol);
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int n = 0; n < CPT; ++n) {
+      const int c = tid + NT * n;
+      const int krow = c / (D / 8), kcol = (c % (D / 8)) * 8;
+      *reinterpret_cast<u32x4*>(&Ks[krow * KS + kcol]) = kreg[n];
+      *reinterpret_cast<u32x4*>(&Vn[krow * KS + kcol]) = vreg[n];
+      const int vd = c >> 3, vcol = (c & 7) * 8;
+      u32x2 a = {treg[n].x, treg[n].y}, b = {treg[n].z, treg[n].w};
+      *reinterpret_cast<u32x2*>(&Kts[vd * VS + vcol]) = a;
+      *reinterpret_cast<u32x2*>(&Kts[vd * VS + vcol + 4]) = b;
+    }
+  };
+
+  auto direct = [&](int n0) {
+#pragma unroll
+    for (int n = 0; n < CPT; ++n) {
+      const int c = tid + NT * n;
+      const int krow = c / (D / 8), kcol = (c % (D / 8)) * 8;
+      const int kr = min(n0 + krow, last_row);
+      *reinterpret_cast<u32x4*>(&Ks[krow * KS + kcol]) =
+          *reinterpret_cast<const u32x4*>(Kh + (int64_t)kr * D + kcol);
+      *reinterpret_cast<u32x4*>(&Vn[krow * KS + kcol]) =
+          *reinterpret_cast<const u32x4*>(Vh + (int64_t)kr * D + kcol);
+      const int vd = c >> 3, vcol = (c & 7) * 8;
+      const u32x4 t = *reinterpret_cast<const u32x4*>(Kth + (int64_t)vd * p.NKVp + n0 + vcol);
+      u32x2 a = {t.x, t.y}, b = {t.z, t.w};
+      *reinterpret_cast<u32x2*>(&Kts[vd * VS + vcol]) = a;
+      *reinterpret_cast<u32x2*>(&Kts[vd * VS + vcol + 4]) = b;
+    }
+  };
+
+  auto run_pass = [&](const int (&aa)[NSB], const int (&bb)[NSB], int w_amin, int w_bmax,
+                      int blk_a, int blk_b) {
+    if (blk_b <= blk_a) return;
+    const int n_begin = (blk_a / kBN) * kBN;
+    if (PF) fetch(n_begin);
+    for (int n0 = n_begin; n0 < blk_b; n0 += kBN) {
+      __syncthreads();
+      if (PF) stash(); else direct(n0);
+      __syncthreads();
+      if (PF && n0 + kBN < blk_b) fetch(n0 + kBN);
+      if (n0 >= w_bmax || n0 + kBN <= w_amin) continue;
+
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb) {
+        f32x16 st[2], dp[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) { st[kb][r] = 0.f; dp[kb][r] = 0.f; }
+          const uint16_t* krow = &Ks[(kb * 32 + col) * KS + g * 8];
+          const uint16_t* vrow = &Vn[(kb * 32 + col) * KS + g * 8];
+#pragma unroll
+          for (int kk = 0; kk < NKK; ++kk) {
+            st[kb] = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(krow + kk * 16)), qf[sb][kk], st[kb]);
+            dp[kb] = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(vrow + kk * 16)), dof[sb][kk], dp[kb]);
+          }
+        }
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int c = n0 + kb * 32 + acc_row(r, g);
+            float pv = fast_exp2(fmaf(st[kb][r], p.scale_log2e, -lse_i[sb]));
+            if (c < aa[sb] || c >= bb[sb]) pv = 0.f;
+            dp[kb][r] = pv * (dp[kb][r] - delta_i[sb]);
+          }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const bf16x8 db8 = pack8(dp[s >> 1], (s & 1) * 8);
+#pragma unroll
+          for (int db = 0; db < NDB; ++db) {
+            const uint16_t* trow = &Kts[(db * 32 + col) * VS + s * 16 + 4 * g];
+            const bf16x8 ka = join_bf16x4(*reinterpret_cast<const u32x2*>(trow),
+                                          *reinterpret_cast<const u32x2*>(trow + 8));
+            acc[sb][db] = mfma32(ka, db8, acc[sb][db]);
+          }
+        }
+      }
+    }
+  };
+
+  run_pass(rb.a1, rb.b1, rb.w_a1min, rb.w_b1max, rb.blk_a1, rb.blk_b1);
+  if (p.a2) run_pass(rb.a2, rb.b2, rb.w_a2min, rb.w_b2max, rb.blk_a2, rb.blk_b2);
+
+  for (int j = 1; j <= p.n_extra; ++j) {
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb) {
+      const uint16_t* kj = p.K + (int64_t)kvh * p.k_hs + ((int64_t)j * p.T + ic[sb]) * D;
+      const uint16_t* vj = p.V + (int64_t)kvh * p.v_hs + ((int64_t)j * p.T + ic[sb]) * D;
+      float dot = 0.f, dpv = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+        float kv[8], vv[8];
+        unpack8(*reinterpret_cast<const u32x4*>(kj + g * 8 + kk * 16), kv);
+        unpack8(*reinterpret_cast<const u32x4*>(vj + g * 8 + kk * 16), vv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          dot = fmaf((float)qf[sb][kk][e], kv[e], dot);
+          dpv = fmaf((float)dof[sb][kk][e], vv[e], dpv);
+        }
+      }
+      dot += __shfl_xor(dot, 32, 64);
+      dpv += __shfl_xor(dpv, 32, 64);
+      const float pv = fast_exp2(fmaf(dot, p.scale_log2e, -lse_i[sb]));
+      const float ds = pv * (dpv - delta_i[sb]);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          float kk4[4];
+          unpack4(*reinterpret_cast<const u32x2*>(kj + 4 * g + db * 32 + 8 * r4), kk4);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) acc[sb][db][r4 * 4 + t] = fmaf(ds, kk4[t], acc[sb][db][r4 * 4 + t]);
+        }
+    }
+  }
+
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) {
+    if (i[sb] >= p.NQ) continue;
+    uint16_t* orow = dQ + (int64_t)h * dq_hs + (int64_t)i[sb] * D + 4 * g;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        u32x2 w;
+        w.x = pack_bf16x2(acc[sb][db][r4 * 4 + 0] * p.scaling, acc[sb][db][r4 * 4 + 1] * p.scaling);
+        w.y = pack_bf16x2(acc[sb][db][r4 * 4 + 2] * p.scaling, acc[sb][db][r4 * 4 + 3] * p.scaling);
+        *reinterpret_cast<u32x2*>(orow + db * 32 + 8 * r4) = w;
+      }
+  }
+}
+
+// per 64-row query tile: min a / max b of both interval classes (for the dK/dV tile loop)
+__global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int32_t* __restrict__ tb) {
+  const int tile = blockIdx.x;
+  const int r = tile * 64 + threadIdx.x;
+  const bool ok = r < p.NQ;
+  int a1 = ok ? p.a1[r] : 0x7fffffff;
+  int b1 = ok ? (p.b1 ? p.b1[r] : r + 1) : 0;
+  int a2 = (ok && p.a2) ? p.T + p.a2[r] : 0x7fffffff;
+  int b2 = (ok && p.a2) ? p.T + p.b2[r] : 0;
+  a1 = wave_min_i(a1); b1 = wave_max_i(b1); a2 = wave_min_i(a2); b2 = wave_max_i(b2);
+  if (threadIdx.x == 0) {
+    tb[tile * 4 + 0] = a1; tb[tile * 4 + 1] = b1; tb[tile * 4 + 2] = a2; tb[tile * 4 + 3] = b2;
+  }
+}
+
+// dK / dV of the tiled keys: one workgroup = 128 keys x ONE query head (a wave owns 32
+// keys: lane column = key), looping over the 64-row query tiles that can see the block.
+// Scores are produced in the S = Q K^T orientation so that a lane holds one KEY:
+//   dV^T += dO^T P,   dK^T += Q^T dS,   dS = P (dO V^T - delta)
+// The per-head results go to fp32 partial buffers that attn_dkv_reduce_kernel sums over
+// the heads of a group (fixed order: deterministic, no atomics).
+template <int D, int NW, bool PF>
+__global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_kernel(
+    AttnParams p, const uint16_t* __restrict__ dO, const uint16_t* __restrict__ Qt,
+    const uint16_t* __restrict__ dOt, int NQp, const float* __restrict__ LSE,
+    const float* __restrict__ Delta, const int32_t* __restrict__ tile_bounds,
+    float* __restrict__ dKp, float* __restrict__ dVp) {
+  constexpr int QS = D + kKPad;
+  constexpr int TS = 64 + kVPad;
+  constexpr int NKK = D / 16;
+  constexpr int NDB = D / 32;
+  constexpr int NT = 64 * NW;
+  constexpr int KB = 32 * NW;  // keys per workgroup
+  constexpr int CPT = (64 * D / 8) / NT;
+
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  uint16_t* Qs = smem;                 // [64][QS]
+  uint16_t* dOs = Qs + 64 * QS;        // [64][QS]
+  uint16_t* Qts = dOs + 64 * QS;       // [D][TS]
+  uint16_t* dOts = Qts + D * TS;       // [D][TS]
+  float* lse_s = reinterpret_cast<float*>(dOts + D * TS);  // [64]
+  float* delta_s = lse_s + 64;                               // [64]
+  int* a1_s = reinterpret_cast<int*>(delta_s + 64);          // [64] each
+  int* b1_s = a1_s + 64;
+  int* a2_s = b1_s + 64;
+  int* b2_s = a2_s + 64;
+
+  // heavy key blocks first: under a causal mask the EARLY key blocks are seen by most rows
+  const int h = blockIdx.x % p.Hq;
+  const int kb_idx = blockIdx.x / p.Hq;
+  const int kvh = h / (p.Hq / p.Hkv);
+  const int n0 = kb_idx * KB;
+  const int key_last = min(n0 + KB - 1, p.NKV - 1);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 5, col = lane & 31;
+  const int cw = n0 + wave * 32;
+  const int c = cw + col;
+  const int cc = c < p.NKV ? c : p.NKV - 1;
+
+  bf16x8 kf[NKK], vf[NKK];
+  {
+    const uint16_t* krow = p.K + (int64_t)kvh * p.k_hs + (int64_t)cc * D + g * 8;
+    const uint16_t* vrow = p.V + (int64_t)kvh * p.v_hs + (int64_t)cc * D + g * 8;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      kf[kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(krow + kk * 16));
+      vf[kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(vrow + kk * 16));
+    }
+  }
+  f32x16 acc_dk[NDB], acc_dv[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { acc_dk[db][r] = 0.f; acc_dv[db][r] = 0.f; }
+
+  const uint16_t* Qh = p.Q + (int64_t)h * p.q_hs;
+  const uint16_t* Qth = Qt + (int64_t)h * D * NQp;
+  const uint16_t* dOth = dOt + (int64_t)h * D * NQp;
+  const int n_qt = (p.NQ + 63) / 64;
+
+  u32x4 qreg[CPT], dreg[CPT], qtreg[CPT], dtreg[CPT];
+  float lse_r = 0.f, delta_r = 0.f;
+  int a1_r = 0, b1_r = 0, a2_r = 0, b2_r = 0;
+  auto visible = [&](int qt) {
+    const int ta1 = tile_bounds[qt * 4 + 0], tb1 = tile_bounds[qt * 4 + 1];
+    const int ta2 = tile_bounds[qt * 4 + 2], tb2 = tile_bounds[qt * 4 + 3];
+    return (ta1 <= key_last && tb1 > n0) || (ta2 <= key_last && tb2 > n0);
+  };
+  auto fetch = [&](int mq) {
+#pragma unroll
+    for (int n = 0; n < CPT; ++n) {
+      const int ch = tid + NT * n;
+      const int qr = ch / (D / 8), qc = (ch % (D / 8)) * 8;
+      const int ir = min(mq + qr, p.NQ - 1);
+      qreg[n] = *reinterpret_cast<const u32x4*>(Qh + (int64_t)ir * D + qc);
+      dreg[n] = *reinterpret_cast<const u32x4*>(dO + ((int64_t)ir * p.Hq + h) * D + qc);
+      const int td = ch >> 3, tc = (ch & 7) * 8;
+      qtreg[n] = *reinterpret_cast<const u32x4*>(Qth + (int64_t)td * NQp + mq + tc);
+      dtreg[n] = *reinterpret_cast<const u32x4*>(dOth + (int64_t)td * NQp + mq + tc);
+    }
+    if (tid < 64) {
+      const int ir = mq + tid;
+      const bool ok = ir < p.NQ;
+      lse_r = ok ? LSE[(int64_t)h * p.NQ + ir] : 0.f;
+      delta_r = ok ? Delta[(int64_t)h * p.NQ + ir] : 0.f;
+      a1_r = ok ? p.a1[ir] : 0x7fffffff;
+      b1_r = ok ? (p.b1 ? p.b1[ir] : ir + 1) : 0;
+      a2_r = (ok && p.a2) ? p.T + p.a2[ir] : 0x7fffffff;
+      b2_r = (ok && p.a2) ? p.T + p.b2[ir] : 0;
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int n = 0; n < CPT; ++n) {
+      const int ch = tid + NT * n;
+      const int qr = ch / (D / 8), qc = (ch % (D / 8)) * 8;
+      *reinterpret_cast<u32x4*>(&Qs[qr * QS + qc]) = qreg[n];
+      *reinterpret_cast<u32x4*>(&dOs[qr * QS + qc]) = dreg[n];
+      const int td = ch >> 3, tc = (ch & 7) * 8;
+      u32x2 a0 = {qtreg[n].x, qtreg[n].y}, a1v = {qtreg[n].z, qtreg[n].w};
+      u32x2 b0 = {dtreg[n].x, dtreg[n].y}, b1v = {dtreg[n].z, dtreg[n].w};
+      *reinterpret_cast<u32x2*>(&Qts[td * TS + tc]) = a0;
+      *reinterpret_cast<u32x2*>(&Qts[td * TS + tc + 4]) = a1v;
+      *reinterpret_cast<u32x2*>(&dOts[td * TS + tc]) = b0;
+      *reinterpret_cast<u32x2*>(&dOts[td * TS + tc + 4]) = b1v;
+    }
+    if (tid < 64) {
+      lse_s[tid] = lse_r; delta_s[tid] = delta_r;
+      a1_s[tid] = a1_r; b1_s[tid] = b1_r; a2_s[tid] = a2_r; b2_s[tid] = b2_r;
+    }
+  };
+
+  auto direct = [&](int mq) {
+#pragma unroll
+    for (int n = 0; n < CPT; ++n) {
+      const int ch = tid + NT * n;
+      const int qr = ch / (D / 8), qc = (ch % (D / 8)) * 8;
+      const int ir = min(mq + qr, p.NQ - 1);
+      *reinterpret_cast<u32x4*>(&Qs[qr * QS + qc]) =
+          *reinterpret_cast<const u32x4*>(Qh + (int64_t)ir * D + qc);
+      *reinterpret_cast<u32x4*>(&dOs[qr * QS + qc]) =
+          *reinterpret_cast<const u32x4*>(dO + ((int64_t)ir * p.Hq + h) * D + qc);
+      const int td = ch >> 3, tc = (ch & 7) * 8;
+      const u32x4 a = *reinterpret_cast<const u32x4*>(Qth + (int64_t)td * NQp + mq + tc);
+      const u32x4 b = *reinterpret_cast<const u32x4*>(dOth + (int64_t)td * NQp + mq + tc);
+      u32x2 a0 = {a.x, a.y}, a1v = {a.z, a.w}, b0 = {b.x, b.y}, b1v = {b.z, b.w};
+      *reinterpret_cast<u32x2*>(&Qts[td * TS + tc]) = a0;
+      *reinterpret_cast<u32x2*>(&Qts[td * TS + tc + 4]) = a1v;
+      *reinterpret_cast<u32x2*>(&dOts[td * TS + tc]) = b0;
+      *reinterpret_cast<u32x2*>(&dOts[td * TS + tc + 4]) = b1v;
+    }
+    if (tid < 64) {
+      const int ir = mq + tid;
+      const bool ok = ir < p.NQ;
+      lse_s[tid] = ok ? LSE[(int64_t)h * p.NQ + ir] : 0.f;
+      delta_s[tid] = ok ? Delta[(int64_t)h * p.NQ + ir] : 0.f;
+      a1_s[tid] = ok ? p.a1[ir] : 0x7fffffff;
+      b1_s[tid] = ok ? (p.b1 ? p.b1[ir] : ir + 1) : 0;
+      a2_s[tid] = (ok && p.a2) ? p.T + p.a2[ir] : 0x7fffffff;
+      b2_s[tid] = (ok && p.a2) ? p.T + p.b2[ir] : 0;
+    }
+  };
+
+  int qt = 0;
+  while (qt < n_qt && !visible(qt)) ++qt;
+  if (PF && qt < n_qt) fetch(qt * 64);
+  while (qt < n_qt) {
+    int nxt = qt + 1;
+    while (nxt < n_qt && !visible(nxt)) ++nxt;
+    __syncthreads();
+    if (PF) stash(); else direct(qt * 64);
+    __syncthreads();
+    if (PF && nxt < n_qt) fetch(nxt * 64);
+    qt = nxt;
+
+    // the two 32-row halves of the query tile one after the other (keeps 32 score
+    // registers live instead of 64)
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      f32x16 st, dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { st[r] = 0.f; dp[r] = 0.f; }
+      const uint16_t* qrow = &Qs[(qb * 32 + col) * QS + g * 8];
+      const uint16_t* drow = &dOs[(qb * 32 + col) * QS + g * 8];
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+        st = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(qrow + kk * 16)), kf[kk], st);
+        dp = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(drow + kk * 16)), vf[kk], dp);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int qi = qb * 32 + acc_row(r, g);
+        const bool ok = ((c >= a1_s[qi] && c < b1_s[qi]) || (c >= a2_s[qi] && c < b2_s[qi])) &&
+                        (c < p.NKV);
+        const float pv = ok ? fast_exp2(fmaf(st[r], p.scale_log2e, -lse_s[qi])) : 0.f;
+        st[r] = pv;
+        dp[r] = pv * (dp[r] - delta_s[qi]);
+      }
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const int s = qb * 2 + s2;
+        const bf16x8 pb = pack8(st, s2 * 8);
+        const bf16x8 sb = pack8(dp, s2 * 8);
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          const uint16_t* arow = &dOts[(db * 32 + col) * TS + s * 16 + 4 * g];
+          const uint16_t* brow = &Qts[(db * 32 + col) * TS + s * 16 + 4 * g];
+          acc_dv[db] = mfma32(join_bf16x4(*reinterpret_cast<const u32x2*>(arow),
+                                          *reinterpret_cast<const u32x2*>(arow + 8)), pb, acc_dv[db]);
+          acc_dk[db] = mfma32(join_bf16x4(*reinterpret_cast<const u32x2*>(brow),
+                                          *reinterpret_cast<const u32x2*>(brow + 8)), sb, acc_dk[db]);
+        }
+      }
+    }
+  }
+
+  if (c < p.NKV) {
+    float* krow = dKp + ((int64_t)h * p.NKV + c) * D + 4 * g;
+    float* vrow = dVp + ((int64_t)h * p.NKV + c) * D + 4 * g;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        f32x4 wk = {acc_dk[db][r4 * 4 + 0], acc_dk[db][r4 * 4 + 1], acc_dk[db][r4 * 4 + 2], acc_dk[db][r4 * 4 + 3]};
+        f32x4 wv = {acc_dv[db][r4 * 4 + 0], acc_dv[db][r4 * 4 + 1], acc_dv[db][r4 * 4 + 2], acc_dv[db][r4 * 4 + 3]};
+        *reinterpret_cast<f32x4*>(krow + db * 32 + 8 * r4) = wk;
+        *reinterpret_cast<f32x4*>(vrow + db * 32 + 8 * r4) = wv;
+      }
+  }
+}
+
+// dK[kvh, c, :] = scaling * sum_{h in group} dKp[h, c, :],  dV likewise (no scaling); bf16 out
+__global__ __launch_bounds__(256) void attn_dkv_reduce_kernel(
+    const float* __restrict__ dKp, const float* __restrict__ dVp, int NKV, int D, int Hq, int Hkv,
+    float scaling, uint16_t* __restrict__ dK, int64_t dk_hs, uint16_t* __restrict__ dV, int64_t dv_hs) {
+  const int64_t per_head = (int64_t)NKV * D / 4;  // float4 items
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= per_head * Hkv) return;
+  const int kvh = (int)(idx / per_head);
+  const int64_t off = (idx % per_head) * 4;
+  const int group = Hq / Hkv;
+  f32x4 sk = {0, 0, 0, 0}, sv = {0, 0, 0, 0};
+  for (int hh = 0; hh < group; ++hh) {
+    const int64_t base = ((int64_t)(kvh * group + hh) * NKV) * D + off;
+    sk += *reinterpret_cast<const f32x4*>(dKp + base);
+    sv += *reinterpret_cast<const f32x4*>(dVp + base);
+  }
+  u32x2 wk, wv;
+  wk.x = pack_bf16x2(sk.x * scaling, sk.y * scaling); wk.y = pack_bf16x2(sk.z * scaling, sk.w * scaling);
+  wv.x = pack_bf16x2(sv.x, sv.y); wv.y = pack_bf16x2(sv.z, sv.w);
+  *reinterpret_cast<u32x2*>(dK + (int64_t)kvh * dk_hs + off) = wk;
+  *reinterpret_cast<u32x2*>(dV + (int64_t)kvh * dv_hs + off) = wv;
+}
+
+// dK / dV of the TTT diagonal keys (j, i), j >= 1: one wave per (position, K/V head);
+// each such key is seen by exactly the `group` query heads at its own position.
+template <int D>
+__global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
+    const uint16_t* __restrict__ Q, int64_t q_hs, const uint16_t* __restrict__ K, int64_t k_hs,
+    const uint16_t* __restrict__ V, int64_t v_hs, const uint16_t* __restrict__ dO,
+    const float* __restrict__ LSE, const float* __restrict__ Delta, int T, int n_extra, int Hq,
+    int Hkv, float scale_log2e, float scaling, uint16_t* __restrict__ dK, int64_t dk_hs,
+    uint16_t* __restrict__ dV, int64_t dv_hs) {
+  constexpr int EPL = D / 64;
+  const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // = i * Hkv + kvh
+  if (item >= (int64_t)T * Hkv) return;
+  const int lane = threadIdx.x & 63;
+  const int i = (int)(item / Hkv), kvh = (int)(item % Hkv);
+  const int group = Hq / Hkv;
+  const int d0 = lane * EPL;
+  for (int j = 1; j <= n_extra; ++j) {
+    const int64_t krow = (int64_t)kvh * k_hs + ((int64_t)j * T + i) * D + d0;
+    const int64_t vrow = (int64_t)kvh * v_hs + ((int64_t)j * T + i) * D + d0;
+    float kv[EPL], vv[EPL], gk[EPL], gv[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      kv[e] = bf16_bits_to_f32(K[krow + e]);
+      vv[e] = bf16_bits_to_f32(V[vrow + e]);
+      gk[e] = 0.f; gv[e] = 0.f;
+    }
+    for (int hh = 0; hh < group; ++hh) {
+      const int h = kvh * group + hh;
+      float qv[EPL], dv[EPL];
+      float dot = 0.f, dpv = 0.f;
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        qv[e] = bf16_bits_to_f32(Q[(int64_t)h * q_hs + (int64_t)i * D + d0 + e]);
+        dv[e] = bf16_bits_to_f32(dO[((int64_t)i * Hq + h) * D + d0 + e]);
+        dot = fmaf(qv[e], kv[e], dot);
+        dpv = fmaf(dv[e], vv[e], dpv);
+      }
+      dot = wave_sum(dot);
+      dpv = wave_sum(dpv);
+      const float pv = fast_exp2(fmaf(dot, scale_log2e, -LSE[(int64_t)h * T + i]));
+      const float ds = pv * (dpv - Delta[(int64_t)h * T + i]) * scaling;
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        gv[e] = fmaf(pv, dv[e], gv[e]);
+        gk[e] = fmaf(ds, qv[e], gk[e]);
+      }
+    }
+    const int64_t gko = (int64_t)kvh * dk_hs + ((int64_t)j * T + i) * D + d0;
+    const int64_t gvo = (int64_t)kvh * dv_hs + ((int64_t)j * T + i) * D + d0;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      dK[gko + e] = (uint16_t)f32_to_bf16_bits(gk[e]);
+      dV[gvo + e] = (uint16_t)f32_to_bf16_bits(gv[e]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------- launchers
+static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
+
+#ifndef SPX_FWD_CFG
+#define SPX_FWD_CFG 2, 2, false
+#endif
+#ifndef SPX_DQ_CFG
+#define SPX_DQ_CFG 1, 4, true
+#endif
+#ifndef SPX_DKV_CFG
+#define SPX_DKV_CFG 2, false
+#endif
+// (sub-blocks per wave, waves per workgroup, register prefetch) of the forward / dQ kernels,
+// (waves per workgroup, register prefetch) of the dK/dV kernel
+constexpr int cfg_nsb(int nsb, int, bool) { return nsb; }
+constexpr int cfg_nw(int, int nw, bool) { return nw; }
+constexpr int cfg_nw(int nw, bool) { return nw; }
+constexpr int kFwdNSB = cfg_nsb(SPX_FWD_CFG), kFwdNW = cfg_nw(SPX_FWD_CFG);
+constexpr int kDqNSB = cfg_nsb(SPX_DQ_CFG), kDqNW = cfg_nw(SPX_DQ_CFG);
+constexpr int kDkvNW = cfg_nw(SPX_DKV_CFG);
+
+static int64_t fwd_workspace_bytes(int64_t NKV, int Hkv, int D) {
+  return round_up((int64_t)Hkv * D * round_up(NKV, 128) * 2, 256);
+}
+static int64_t bwd_workspace_bytes(int64_t NQ, int64_t NKV, int Hq, int Hkv, int D) {
+  const int64_t NKVp = round_up(NKV, 128), NQp = round_up(NQ, 128);
+  int64_t b = (int64_t)Hkv * D * NKVp * 2;          // K^T
+  b += 2 * (int64_t)Hq * D * NQp * 2;                // Q^T, dO^T
+  b = round_up(b, 256) + round_up((int64_t)Hq * NQ * 4, 256);       // delta
+  b += round_up(((NQ + 63) / 64) * 16, 256);                        // tile bounds
+  b += 2 * round_up((int64_t)Hq * NKV * D * 4, 256);                // fp32 per-head dK, dV
+  return b;
+}
+
+template <int D>
+static int launch_fwd(AttnParams p, void* workspace, uint16_t* O, float* lse, hipStream_t st,
+                      const char* fn) {
+  uint16_t* vt = reinterpret_cast<uint16_t*>(workspace);
+  dim3 tgrid((unsigned)(p.NKVp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hkv);
+  hipLaunchKernelGGL(transpose_bf16_kernel, tgrid, dim3(256), 0, st, p.V, p.v_hs, (int64_t)D, p.NKV, D,
+                     vt, (int64_t)D * p.NKVp, (int64_t)p.NKVp);
+  constexpr int BM = 32 * kFwdNSB * kFwdNW;
+  const int n_qb = (p.NQ + BM - 1) / BM;
+  hipLaunchKernelGGL((attn_fwd_kernel<D, SPX_FWD_CFG>), dim3((unsigned)(n_qb * p.Hq)),
+                     dim3(64 * kFwdNW), 0, st, p, vt, O, lse);
+  return check_launch(fn);
+}
+
+template <int D>
+static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, const float* lse,
+                      uint16_t* dQp, int64_t dq_hs, uint16_t* dKp, int64_t dk_hs, uint16_t* dVp,
+                      int64_t dv_hs, void* workspace, hipStream_t st, const char* fn) {
+  const int NQp = (int)round_up(p.NQ, 128);
+  char* w = reinterpret_cast<char*>(workspace);
+  uint16_t* kt = reinterpret_cast<uint16_t*>(w);
+  uint16_t* qt = kt + (int64_t)p.Hkv * D * p.NKVp;
+  uint16_t* dot = qt + (int64_t)p.Hq * D * NQp;
+  w += round_up(((int64_t)p.Hkv * D * p.NKVp + 2 * (int64_t)p.Hq * D * NQp) * 2, 256);
+  float* delta = reinterpret_cast<float*>(w);
+  w += round_up((int64_t)p.Hq * p.NQ * 4, 256);
+  int32_t* tb = reinterpret_cast<int32_t*>(w);
+  w += round_up(((p.NQ + 63) / 64) * 16, 256);
+  float* dkp = reinterpret_cast<float*>(w);
+  w += round_up((int64_t)p.Hq * p.NKV * D * 4, 256);
+  float* dvp = reinterpret_cast<float*>(w);
+
+  dim3 tgrid((unsigned)(p.NKVp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hkv);
+  hipLaunchKernelGGL(transpose_bf16_kernel, tgrid, dim3(256), 0, st, p.K, p.k_hs, (int64_t)D, p.NKV, D,
+                     kt, (int64_t)D * p.NKVp, (int64_t)p.NKVp);
+  dim3 qgrid((unsigned)(NQp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hq);
+  hipLaunchKernelGGL(transpose_bf16_kernel, qgrid, dim3(256), 0, st, p.Q, p.q_hs, (int64_t)D, p.NQ, D,
+                     qt, (int64_t)D * NQp, (int64_t)NQp);
+  hipLaunchKernelGGL(transpose_bf16_kernel, qgrid, dim3(256), 0, st, dOp, (int64_t)D,
+                     (int64_t)p.Hq * D, p.NQ, D, dot, (int64_t)D * NQp, (int64_t)NQp);
+  hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)(((int64_t)p.NQ * p.Hq + 3) / 4)), dim3(256),
+                     0, st, Op, dOp, p.NQ, p.Hq, delta);
+  hipLaunchKernelGGL(attn_tile_bounds_kernel, dim3((unsigned)((p.NQ + 63) / 64)), dim3(64), 0, st, p, tb);
+
+  constexpr int BM = 32 * kDqNSB * kDqNW;
+  const int n_qb = (p.NQ + BM - 1) / BM;
+  hipLaunchKernelGGL((attn_bwd_dq_kernel<D, SPX_DQ_CFG>), dim3((unsigned)(n_qb * p.Hq)),
+                     dim3(64 * kDqNW), 0, st, p, dOp, kt, lse, delta, dQp, dq_hs);
+
+  const size_t smem = (size_t)(2 * 64 * (D + kKPad) + 2 * D * (64 + kVPad)) * 2 + 64 * 4 * 6;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, SPX_DKV_CFG>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) {
+      last_error() = std::string(fn) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
+      return SPX_ERR_HIP;
+    }
+    attr_set = true;
+  }
+  const int n_kb = (p.NKV + 32 * kDkvNW - 1) / (32 * kDkvNW);
+  hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, SPX_DKV_CFG>), dim3((unsigned)(n_kb * p.Hq)), dim3(64 * kDkvNW), smem, st,
+                     p, dOp, qt, dot, NQp, lse, delta, tb, dkp, dvp);
+  const int64_t items = (int64_t)p.NKV * D / 4 * p.Hkv;
+  hipLaunchKernelGGL(attn_dkv_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, dkp,
+                     dvp, p.NKV, D, p.Hq, p.Hkv, p.scaling, dKp, dk_hs, dVp, dv_hs);
+  if (p.n_extra > 0)
+    hipLaunchKernelGGL(ttt_attn_bwd_diag_kernel<D>, dim3((unsigned)(((int64_t)p.T * p.Hkv + 3) / 4)),
+                       dim3(256), 0, st, p.Q, p.q_hs, p.K, p.k_hs, p.V, p.v_hs, dOp, lse, delta, p.T,
+                       p.n_extra, p.Hq, p.Hkv, p.scale_log2e, p.scaling, dKp, dk_hs, dVp, dv_hs);
+  return check_launch(fn);
+}
+
+static int shape_checks(const char* fn, int64_t NQ, int64_t NKV, int32_t Hq, int32_t Hkv, int32_t D) {
+  if (!(NQ > 0 && NQ < (1ll << 24) && NKV > 0 && NKV < (1ll << 26))) return fail_arg(fn, "sequence length out of range");
+  if (!(Hkv > 0 && Hq > 0 && Hq % Hkv == 0)) return fail_arg(fn, "Hq must be a multiple of Hkv");
+  if (!(D == 64 || D == 128)) return fail_arg(fn, "head_dim must be 64 or 128");
+  return SPX_OK;
+}
+
+static bool all_aligned16(std::initializer_list<const void*> ps) {
+  for (const void* q : ps)
+    if (reinterpret_cast<uintptr_t>(q) & 15) return false;
+  return true;
+}
+
+}  // namespace spx
+
+using namespace spx;
+
+// ================================================================ TTT entry points
+extern "C" int spx_ttt_row_lo(const void* document_ids, int doc_kind, int64_t T,
+                              int64_t sliding_window, int32_t* row_lo, void* stream) {
+  SPX_REQUIRE(doc_kind == SPX_KIND_I32 || doc_kind == SPX_KIND_I64, "document_ids must be int32 or int64");
+  SPX_REQUIRE(T > 0 && T < (1ll << 30), "0 < T < 2^30");
+  SPX_REQUIRE(document_ids && row_lo, "null buffer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (doc_kind == SPX_KIND_I32)
+    hipLaunchKernelGGL(ttt_row_lo_kernel<int32_t>, dim3(1), dim3(1024), 0, st,
+                       reinterpret_cast<const int32_t*>(document_ids), T, sliding_window, row_lo);
+  else
+    hipLaunchKernelGGL(ttt_row_lo_kernel<int64_t>, dim3(1), dim3(1024), 0, st,
+                       reinterpret_cast<const int64_t*>(document_ids), T, sliding_window, row_lo);
+  return check_launch(__func__);
+}
+
+extern "C" int64_t spx_ttt_attn_workspace_bytes(int64_t T, int32_t Hq, int32_t Hkv, int32_t D,
+                                                int32_t backward) {
+  return backward ? bwd_workspace_bytes(T, T, Hq, Hkv, D) : fwd_workspace_bytes(T, Hkv, D);
+}
+
+static AttnParams ttt_params(const void* q, int64_t q_hs, const void* k, int64_t k_hs, const void* v,
+                             int64_t v_hs, const int32_t* row_lo, int64_t T, int32_t ttt_step,
+                             int32_t Hq, int32_t Hkv, float scaling) {
+  AttnParams p;
+  p.Q = reinterpret_cast<const uint16_t*>(q); p.q_hs = q_hs;
+  p.K = reinterpret_cast<const uint16_t*>(k); p.k_hs = k_hs;
+  p.V = reinterpret_cast<const uint16_t*>(v); p.v_hs = v_hs;
+  p.a1 = row_lo; p.b1 = nullptr; p.a2 = nullptr; p.b2 = nullptr;
+  p.NQ = (int)T; p.T = (int)T; p.NKV = (int)T; p.NKVp = (int)round_up(T, 128);
+  p.n_extra = ttt_step; p.Hq = Hq; p.Hkv = Hkv;
+  p.scaling = scaling; p.scale_log2e = scaling * kLog2e;
+  return p;
+}
+
+extern "C" int spx_ttt_attn_fwd(const void* q, int64_t q_head_stride, const void* k,
+                                int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                                const int32_t* row_lo, int64_t T, int32_t ttt_step, int32_t Hq,
+                                int32_t Hkv, int32_t D, float scaling, void* out, float* lse,
+                                void* workspace, int64_t workspace_bytes, void* stream) {
+  if (int rc = shape_checks(__func__, T, T, Hq, Hkv, D)) return rc;
+  SPX_REQUIRE(ttt_step >= 0 && ttt_step < 64, "0 <= ttt_step < 64");
+  SPX_REQUIRE(q && k && v && row_lo && out && lse && workspace, "null buffer");
+  SPX_REQUIRE(q_head_stride >= T * D, "q head stride smaller than T*D");
+  SPX_REQUIRE(k_head_stride >= (int64_t)(ttt_step + 1) * T * D &&
+              v_head_stride >= (int64_t)(ttt_step + 1) * T * D,
+              "k/v head stride smaller than (ttt_step+1)*T*D");
+  SPX_REQUIRE(q_head_stride % 8 == 0 && k_head_stride % 8 == 0 && v_head_stride % 8 == 0,
+              "head strides must be multiples of 8 elements");
+  SPX_REQUIRE(workspace_bytes >= fwd_workspace_bytes(T, Hkv, D), "workspace too small");
+  SPX_REQUIRE(all_aligned16({q, k, v, out, workspace}), "buffers must be 16-byte aligned");
+  AttnParams p = ttt_params(q, q_head_stride, k, k_head_stride, v, v_head_stride, row_lo, T, ttt_step,
+                            Hq, Hkv, scaling);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (D == 128) return launch_fwd<128>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
+  return launch_fwd<64>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
+}
+
+extern "C" int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
+                                int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                                const void* out, const void* dout, const float* lse,
+                                const int32_t* row_lo, int64_t T, int32_t ttt_step, int32_t Hq,
+                                int32_t Hkv, int32_t D, float scaling, void* dq,
+                                int64_t dq_head_stride, void* dk, int64_t dk_head_stride, void* dv,
+                                int64_t dv_head_stride, void* workspace, int64_t workspace_bytes,
+                                void* stream) {
+  if (int rc = shape_checks(__func__, T, T, Hq, Hkv, D)) return rc;
+  SPX_REQUIRE(ttt_step >= 0 && ttt_step < 64, "0 <= ttt_step < 64");
+  SPX_REQUIRE(q && k && v && out && dout && lse && row_lo && dq && dk && dv && workspace, "null buffer");
+  const int64_t kv_rows = (int64_t)(ttt_step + 1) * T * D;
+  SPX_REQUIRE(q_head_stride >= T * D && dq_head_stride >= T * D, "q / dq head stride smaller than T*D");
+  SPX_REQUIRE(k_head_stride >= kv_rows && v_head_stride >= kv_rows && dk_head_stride >= kv_rows &&
+              dv_head_stride >= kv_rows, "k/v/dk/dv head stride smaller than (ttt_step+1)*T*D");
+  SPX_REQUIRE((q_head_stride | k_head_stride | v_head_stride | dq_head_stride | dk_head_stride |
+               dv_head_stride) % 8 == 0, "head strides must be multiples of 8 elements");
+  SPX_REQUIRE(workspace_bytes >= bwd_workspace_bytes(T, T, Hq, Hkv, D), "workspace too small");
+  SPX_REQUIRE(all_aligned16({q, k, v, out, dout, dq, dk, dv, workspace}), "buffers must be 16-byte aligned");
+  AttnParams p = ttt_params(q, q_head_stride, k, k_head_stride, v, v_head_stride, row_lo, T, ttt_step,
+                            Hq, Hkv, scaling);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  auto Op = reinterpret_cast<const uint16_t*>(out);
+  auto dOp = reinterpret_cast<const uint16_t*>(dout);
+  auto dQp = reinterpret_cast<uint16_t*>(dq);
+  auto dKp = reinterpret_cast<uint16_t*>(dk);
+  auto dVp = reinterpret_cast<uint16_t*>(dv);
+  if (D == 128)
+    return launch_bwd<128>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp,
+                           dv_head_stride, workspace, st, __func__);
+  return launch_bwd<64>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp, dv_head_stride,
+                        workspace, st, __func__);
+}
+
+// ================================================================ DFlash entry points
+extern "C" int spx_dflash_row_ranges(const void* document_ids, int doc_kind, int64_t T,
+                                     const void* anchors, int anchor_kind, int64_t n_anchors,
+                                     int32_t block_size, int64_t sliding_window, int32_t causal_block,
+                                     int32_t* ctx_lo, int32_t* ctx_hi, int32_t* blk_lo, int32_t* blk_hi,
+                                     int32_t* run_start_scratch, void* stream) {
+  SPX_REQUIRE(doc_kind == SPX_KIND_I32 || doc_kind == SPX_KIND_I64, "document_ids must be int32 or int64");
+  SPX_REQUIRE(anchor_kind == SPX_KIND_I32 || anchor_kind == SPX_KIND_I64, "anchors must be int32 or int64");
+  SPX_REQUIRE(T > 0 && T < (1ll << 30) && n_anchors > 0 && block_size > 0, "bad sizes");
+  SPX_REQUIRE(n_anchors * block_size < (1ll << 24), "too many block rows");
+  SPX_REQUIRE(document_ids && anchors && ctx_lo && ctx_hi && blk_lo && blk_hi && run_start_scratch, "null buffer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const unsigned grid = (unsigned)((n_anchors * block_size + 255) / 256);
+#define SPX_RANGES(I, J)                                                                          \
+  do {                                                                                            \
+    hipLaunchKernelGGL(doc_run_start_kernel<I>, dim3(1), dim3(1024), 0, st,                       \
+                       reinterpret_cast<const I*>(document_ids), T, run_start_scratch);           \
+    hipLaunchKernelGGL((dflash_ranges_kernel<I, J>), dim3(grid), dim3(256), 0, st,                \
+                       reinterpret_cast<const I*>(document_ids), run_start_scratch,               \
+                       reinterpret_cast<const J*>(anchors), n_anchors, (int)block_size,           \
+                       sliding_window, (int)causal_block, T, ctx_lo, ctx_hi, blk_lo, blk_hi);     \
+  } while (0)
+  if (doc_kind == SPX_KIND_I32 && anchor_kind == SPX_KIND_I32) SPX_RANGES(int32_t, int32_t);
+  else if (doc_kind == SPX_KIND_I32) SPX_RANGES(int32_t, int64_t);
+  else if (anchor_kind == SPX_KIND_I32) SPX_RANGES(int64_t, int32_t);
+  else SPX_RANGES(int64_t, int64_t);
+#undef SPX_RANGES
+  return check_launch(__func__);
+}
+
+extern "C" int64_t spx_dflash_attn_workspace_bytes(int64_t T, int64_t NQ, int32_t Hq, int32_t Hkv,
+                                                   int32_t D, int32_t backward) {
+  return backward ? bwd_workspace_bytes(NQ, T + NQ, Hq, Hkv, D) : fwd_workspace_bytes(T + NQ, Hkv, D);
+}
+
+static AttnParams dflash_params(const void* q, int64_t q_hs, const void* k, int64_t k_hs, const void* v,
+                                int64_t v_hs, const int32_t* a1, const int32_t* b1, const int32_t* a2,
+                                const int32_t* b2, int64_t T, int64_t NQ, int32_t Hq, int32_t Hkv,
+                                float scaling) {
+  AttnParams p;
+  p.Q = reinterpret_cast<const uint16_t*>(q); p.q_hs = q_hs;
+  p.K = reinterpret_cast<const uint16_t*>(k); p.k_hs = k_hs;
+  p.V = reinterpret_cast<const uint16_t*>(v); p.v_hs = v_hs;
+  p.a1 = a1; p.b1 = b1; p.a2 = a2; p.b2 = b2;
+  p.NQ = (int)NQ; p.T = (int)T; p.NKV = (int)(T + NQ); p.NKVp = (int)round_up(T + NQ, 128);
+  p.n_extra = 0; p.Hq = Hq; p.Hkv = Hkv;
+  p.scaling = scaling; p.scale_log2e = scaling * kLog2e;
+  return p;
+}
+
+extern "C" int spx_dflash_attn_fwd(const void* q, int64_t q_head_stride, const void* k,
+                                   int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                                   const int32_t* ctx_lo, const int32_t* ctx_hi, const int32_t* blk_lo,
+                                   const int32_t* blk_hi, int64_t T, int64_t NQ, int32_t Hq, int32_t Hkv,
+                                   int32_t D, float scaling, void* out, float* lse, void* workspace,
+                                   int64_t workspace_bytes, void* stream) {
+  if (int rc = shape_checks(__func__, NQ, T + NQ, Hq, Hkv, D)) return rc;
+  SPX_REQUIRE(T > 0, "T must be positive");
+  SPX_REQUIRE(q && k && v && ctx_lo && ctx_hi && blk_lo && blk_hi && out && lse && workspace, "null buffer");
+  SPX_REQUIRE(q_head_stride >= NQ * D, "q head stride smaller than NQ*D");
+  SPX_REQUIRE(k_head_stride >= (T + NQ) * D && v_head_stride >= (T + NQ) * D,
+              "k/v head stride smaller than (T+NQ)*D");
+  SPX_REQUIRE(q_head_stride % 8 == 0 && k_head_stride % 8 == 0 && v_head_stride % 8 == 0,
+              "head strides must be multiples of 8 elements");
+  SPX_REQUIRE(workspace_bytes >= fwd_workspace_bytes(T + NQ, Hkv, D), "workspace too small");
+  SPX_REQUIRE(all_aligned16({q, k, v, out, workspace}), "buffers must be 16-byte aligned");
+  AttnParams p = dflash_params(q, q_head_stride, k, k_head_stride, v, v_head_stride, ctx_lo, ctx_hi,
+                               blk_lo, blk_hi, T, NQ, Hq, Hkv, scaling);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (D == 128) return launch_fwd<128>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
+  return launch_fwd<64>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
+}
+
+extern "C" int spx_dflash_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
+                                   int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                                   const void* out, const void* dout, const float* lse,
+                                   const int32_t* ctx_lo, const int32_t* ctx_hi, const int32_t* blk_lo,
+                                   const int32_t* blk_hi, int64_t T, int64_t NQ, int32_t Hq, int32_t Hkv,
+                                   int32_t D, float scaling, void* dq, int64_t dq_head_stride, void* dk,
+                                   int64_t dk_head_stride, void* dv, int64_t dv_head_stride,
+                                   void* workspace, int64_t workspace_bytes, void* stream) {
+  if (int rc = shape_checks(__func__, NQ, T + NQ, Hq, Hkv, D)) return rc;
+  SPX_REQUIRE(T > 0, "T must be positive");
+  SPX_REQUIRE(q && k && v && out && dout && lse && ctx_lo && ctx_hi && blk_lo && blk_hi && dq && dk &&
+              dv && workspace, "null buffer");
+  SPX_REQUIRE(q_head_stride >= NQ * D && dq_head_stride >= NQ * D, "q / dq head stride smaller than NQ*D");
+  const int64_t kv_rows = (T + NQ) * D;
+  SPX_REQUIRE(k_head_stride >= kv_rows && v_head_stride >= kv_rows && dk_head_stride >= kv_rows &&
+              dv_head_stride >= kv_rows, "k/v/dk/dv head stride smaller than (T+NQ)*D");
+  SPX_REQUIRE((q_head_stride | k_head_stride | v_head_stride | dq_head_stride | dk_head_stride |
+               dv_head_stride) % 8 == 0, "head strides must be multiples of 8 elements");
+  SPX_REQUIRE(workspace_bytes >= bwd_workspace_bytes(NQ, T + NQ, Hq, Hkv, D), "workspace too small");
+  SPX_REQUIRE(all_aligned16({q, k, v, out, dout, dq, dk, dv, workspace}), "buffers must be 16-byte aligned");
+  AttnParams p = dflash_params(q, q_head_stride, k, k_head_stride, v, v_head_stride, ctx_lo, ctx_hi,
+                               blk_lo, blk_hi, T, NQ, Hq, Hkv, scaling);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  auto Op = reinterpret_cast<const uint16_t*>(out);
+  auto dOp = reinterpret_cast<const uint16_t*>(dout);
+  auto dQp = reinterpret_cast<uint16_t*>(dq);
+  auto dKp = reinterpret_cast<uint16_t*>(dk);
+  auto dVp = reinterpret_cast<uint16_t*>(dv);
+  if (D == 128)
+    return launch_bwd<128>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp,
+                           dv_head_stride, workspace, st, __func__);
+  return launch_bwd<64>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp, dv_head_stride,
+                        workspace, st, __func__);
+}
