@@ -665,18 +665,21 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(
   }
 }
 
-// per 64-row query tile: min a / max b of both interval classes (for the dK/dV tile loop)
+// per 64-row query tile: min / max of the interval ends of both classes (for the dK/dV
+// tile loop): [a1min, a1max, b1min, b1max, a2min, a2max, b2min, b2max]
 __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int32_t* __restrict__ tb) {
   const int tile = blockIdx.x;
   const int r = tile * 64 + threadIdx.x;
   const bool ok = r < p.NQ;
-  int a1 = ok ? p.a1[r] : 0x7fffffff;
-  int b1 = ok ? (p.b1 ? p.b1[r] : r + 1) : 0;
-  int a2 = (ok && p.a2) ? p.T + p.a2[r] : 0x7fffffff;
-  int b2 = (ok && p.a2) ? p.T + p.b2[r] : 0;
-  a1 = wave_min_i(a1); b1 = wave_max_i(b1); a2 = wave_min_i(a2); b2 = wave_max_i(b2);
+  const int a1 = ok ? p.a1[r] : 0x7fffffff;
+  const int b1 = ok ? (p.b1 ? p.b1[r] : r + 1) : 0;
+  const int a2 = (ok && p.a2) ? p.T + p.a2[r] : 0x7fffffff;
+  const int b2 = (ok && p.a2) ? p.T + p.b2[r] : 0;
+  const int v[8] = {wave_min_i(a1), wave_max_i(a1), wave_min_i(b1), wave_max_i(b1),
+                    wave_min_i(a2), wave_max_i(a2), wave_min_i(b2), wave_max_i(b2)};
   if (threadIdx.x == 0) {
-    tb[tile * 4 + 0] = a1; tb[tile * 4 + 1] = b1; tb[tile * 4 + 2] = a2; tb[tile * 4 + 3] = b2;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) tb[tile * 8 + k] = v[k];
   }
 }
 
@@ -750,9 +753,14 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_kernel(
   float lse_r = 0.f, delta_r = 0.f;
   int a1_r = 0, b1_r = 0, a2_r = 0, b2_r = 0;
   auto visible = [&](int qt) {
-    const int ta1 = tile_bounds[qt * 4 + 0], tb1 = tile_bounds[qt * 4 + 1];
-    const int ta2 = tile_bounds[qt * 4 + 2], tb2 = tile_bounds[qt * 4 + 3];
+    const int ta1 = tile_bounds[qt * 8 + 0], tb1 = tile_bounds[qt * 8 + 3];
+    const int ta2 = tile_bounds[qt * 8 + 4], tb2 = tile_bounds[qt * 8 + 7];
     return (ta1 <= key_last && tb1 > n0) || (ta2 <= key_last && tb2 > n0);
+  };
+  // every row of the tile sees every key of this block: no per-element interval test
+  auto fully_visible = [&](int qt) {
+    return (tile_bounds[qt * 8 + 1] <= n0 && tile_bounds[qt * 8 + 2] >= n0 + KB) ||
+           (tile_bounds[qt * 8 + 5] <= n0 && tile_bounds[qt * 8 + 6] >= n0 + KB);
   };
   auto fetch = [&](int mq) {
 #pragma unroll
@@ -835,6 +843,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_kernel(
   while (qt < n_qt) {
     int nxt = qt + 1;
     while (nxt < n_qt && !visible(nxt)) ++nxt;
+    const bool full = fully_visible(qt);
     __syncthreads();
     if (PF) stash(); else direct(qt * 64);
     __syncthreads();
@@ -856,13 +865,30 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_kernel(
         dp = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(drow + kk * 16)), vf[kk], dp);
       }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int qi = qb * 32 + acc_row(r, g);
-        const bool ok = ((c >= a1_s[qi] && c < b1_s[qi]) || (c >= a2_s[qi] && c < b2_s[qi])) &&
-                        (c < p.NKV);
-        const float pv = ok ? fast_exp2(fmaf(st[r], p.scale_log2e, -lse_s[qi])) : 0.f;
-        st[r] = pv;
-        dp[r] = pv * (dp[r] - delta_s[qi]);
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int q0 = qb * 32 + 8 * r4 + 4 * g;  // 4 consecutive query rows: one 16-byte LDS read each
+        const f32x4 ls = *reinterpret_cast<const f32x4*>(&lse_s[q0]);
+        const f32x4 dl = *reinterpret_cast<const f32x4*>(&delta_s[q0]);
+        float pv[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) pv[t] = fast_exp2(fmaf(st[r4 * 4 + t], p.scale_log2e, -ls[t]));
+        if (!full) {
+          typedef __attribute__((ext_vector_type(4))) int i32x4;
+          const i32x4 a1v = *reinterpret_cast<const i32x4*>(&a1_s[q0]);
+          const i32x4 b1v = *reinterpret_cast<const i32x4*>(&b1_s[q0]);
+          const i32x4 a2v = *reinterpret_cast<const i32x4*>(&a2_s[q0]);
+          const i32x4 b2v = *reinterpret_cast<const i32x4*>(&b2_s[q0]);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const bool ok = ((c >= a1v[t] && c < b1v[t]) || (c >= a2v[t] && c < b2v[t])) && (c < p.NKV);
+            pv[t] = ok ? pv[t] : 0.f;
+          }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          st[r4 * 4 + t] = pv[t];
+          dp[r4 * 4 + t] = pv[t] * (dp[r4 * 4 + t] - dl[t]);
+        }
       }
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
@@ -981,13 +1007,13 @@ __global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
 static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 
 #ifndef SPX_FWD_CFG
-#define SPX_FWD_CFG 2, 2, false
+#define SPX_FWD_CFG 1, 4, true
 #endif
 #ifndef SPX_DQ_CFG
 #define SPX_DQ_CFG 1, 4, true
 #endif
 #ifndef SPX_DKV_CFG
-#define SPX_DKV_CFG 2, false
+#define SPX_DKV_CFG 4, true
 #endif
 // (sub-blocks per wave, waves per workgroup, register prefetch) of the forward / dQ kernels,
 // (waves per workgroup, register prefetch) of the dK/dV kernel
@@ -1006,7 +1032,7 @@ static int64_t bwd_workspace_bytes(int64_t NQ, int64_t NKV, int Hq, int Hkv, int
   int64_t b = (int64_t)Hkv * D * NKVp * 2;          // K^T
   b += 2 * (int64_t)Hq * D * NQp * 2;                // Q^T, dO^T
   b = round_up(b, 256) + round_up((int64_t)Hq * NQ * 4, 256);       // delta
-  b += round_up(((NQ + 63) / 64) * 16, 256);                        // tile bounds
+  b += round_up(((NQ + 63) / 64) * 32, 256);                        // tile bounds
   b += 2 * round_up((int64_t)Hq * NKV * D * 4, 256);                // fp32 per-head dK, dV
   return b;
 }
@@ -1038,7 +1064,7 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   float* delta = reinterpret_cast<float*>(w);
   w += round_up((int64_t)p.Hq * p.NQ * 4, 256);
   int32_t* tb = reinterpret_cast<int32_t*>(w);
-  w += round_up(((p.NQ + 63) / 64) * 16, 256);
+  w += round_up(((p.NQ + 63) / 64) * 32, 256);
   float* dkp = reinterpret_cast<float*>(w);
   w += round_up((int64_t)p.Hq * p.NKV * D * 4, 256);
   float* dvp = reinterpret_cast<float*>(w);
