@@ -19,6 +19,7 @@ import torch
 from . import _lib
 
 ATTN_IMPL_TTT = "ttt_hip"
+ATTN_IMPL_DFLASH = "dflash_hip"
 
 
 def _workspace_bytes(t, hq, hkv, d, backward):
@@ -129,6 +130,120 @@ def ttt_hip_attention_forward(module, query, key, value, attention_mask, scaling
     return ttt_attention(query, key, value, attention_mask, scaling), None
 
 
+# ---------------------------------------------------------------------- DFlash
+@dataclass
+class DFlashMask:
+    """Descriptor of the anchored-block mask of one layer: per query row the visible
+    interval of context keys ``[ctx_lo, ctx_hi)`` and of its own block's keys
+    ``[blk_lo, blk_hi)`` (all int32 ``[A * block_size]``).  Stands where the reference
+    passes the BlockMask built from create_anchor_block_mask_mod
+    (models/dflash/attention.py:7-100, models/dflash/core.py:273-328)."""
+
+    ctx_lo: torch.Tensor
+    ctx_hi: torch.Tensor
+    blk_lo: torch.Tensor
+    blk_hi: torch.Tensor
+    total_seq_len: int
+    q_len: int
+
+
+def create_dflash_mask(document_ids: torch.Tensor, total_seq_len: int,
+                       anchor_positions: torch.Tensor, block_size: int,
+                       sliding_window: int | None = None,
+                       sliding_window_non_causal: bool = False) -> DFlashMask:
+    """Counterpart of ``_create_attention_mask`` (models/dflash/core.py:273-297): block
+    keys are non-causal for full-attention layers and for ``sliding_window_non_causal``,
+    causal otherwise.  ``document_ids`` must be run-contiguous."""
+    doc = document_ids.reshape(-1)
+    if doc.numel() != total_seq_len:
+        raise ValueError(f"document_ids has {doc.numel()} entries, expected {total_seq_len}")
+    if anchor_positions.dim() != 1:
+        raise ValueError(f"anchor_positions must be 1D, got shape {tuple(anchor_positions.shape)}")
+    if doc.dtype not in (torch.int32, torch.int64):
+        doc = doc.to(torch.int64)
+    doc = doc.contiguous()
+    anchors = anchor_positions.to(device=doc.device)
+    if anchors.dtype not in (torch.int32, torch.int64):
+        anchors = anchors.to(torch.int64)
+    anchors = anchors.contiguous()
+    n_q = anchors.numel() * block_size
+    dev = doc.device
+    bounds = torch.empty(4, n_q, device=dev, dtype=torch.int32)
+    scratch = torch.empty(total_seq_len, device=dev, dtype=torch.int32)
+    causal_block = sliding_window is not None and not sliding_window_non_causal
+    _lib.call("spx_dflash_row_ranges", _lib.ptr(doc), _lib.kind_code(doc), total_seq_len,
+              _lib.ptr(anchors), _lib.kind_code(anchors), anchors.numel(), int(block_size),
+              int(sliding_window) if sliding_window else 0, int(causal_block),
+              _lib.ptr(bounds[0]), _lib.ptr(bounds[1]), _lib.ptr(bounds[2]), _lib.ptr(bounds[3]),
+              _lib.ptr(scratch), _lib.stream_ptr(dev))
+    return DFlashMask(bounds[0], bounds[1], bounds[2], bounds[3], total_seq_len, n_q)
+
+
+class _DFlashAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, mask: DFlashMask, scaling: float):
+        if q.dim() != 4 or q.shape[0] != 1:
+            raise ValueError("the packed batch layout has batch size 1: q must be [1, Hq, NQ, D]")
+        if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
+            raise _lib.SpxError("the HIP attention kernels take bf16 q/k/v")
+        _, hq, nq, d = q.shape
+        hkv = k.shape[1]
+        t = mask.total_seq_len
+        if nq != mask.q_len or k.shape[2] != t + nq or v.shape != k.shape:
+            raise ValueError(f"q {tuple(q.shape)} / k {tuple(k.shape)} do not match the mask "
+                             f"(T {t}, {mask.q_len} block rows)")
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        dev = q.device
+        out = torch.empty(1, nq, hq, d, device=dev, dtype=torch.bfloat16)
+        lse = torch.empty(hq, nq, device=dev, dtype=torch.float32)
+        nbytes = int(_lib.load().spx_dflash_attn_workspace_bytes(t, nq, hq, hkv, d, 0))
+        ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+        _lib.call("spx_dflash_attn_fwd", _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1),
+                  _lib.ptr(v), v.stride(1), _lib.ptr(mask.ctx_lo), _lib.ptr(mask.ctx_hi),
+                  _lib.ptr(mask.blk_lo), _lib.ptr(mask.blk_hi), t, nq, hq, hkv, d, float(scaling),
+                  _lib.ptr(out), _lib.ptr(lse), _lib.ptr(ws), ws.numel(), _lib.stream_ptr(dev))
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.mask, ctx.scaling = mask, float(scaling)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse = ctx.saved_tensors
+        mask = ctx.mask
+        _, hq, nq, d = q.shape
+        hkv = k.shape[1]
+        t = mask.total_seq_len
+        dev = q.device
+        dout = dout.to(torch.bfloat16).contiguous()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        nbytes = int(_lib.load().spx_dflash_attn_workspace_bytes(t, nq, hq, hkv, d, 1))
+        ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+        _lib.call("spx_dflash_attn_bwd", _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1),
+                  _lib.ptr(v), v.stride(1), _lib.ptr(out), _lib.ptr(dout), _lib.ptr(lse),
+                  _lib.ptr(mask.ctx_lo), _lib.ptr(mask.ctx_hi), _lib.ptr(mask.blk_lo),
+                  _lib.ptr(mask.blk_hi), t, nq, hq, hkv, d, ctx.scaling, _lib.ptr(dq), dq.stride(1),
+                  _lib.ptr(dk), dk.stride(1), _lib.ptr(dv), dv.stride(1), _lib.ptr(ws), ws.numel(),
+                  _lib.stream_ptr(dev))
+        return dq, dk, dv, None, None
+
+
+def dflash_attention(q, k, v, mask: DFlashMask, scaling: float | None = None) -> torch.Tensor:
+    """``[1, Hq, NQ, D]`` x ``[1, Hkv, T + NQ, D]`` -> ``[1, NQ, Hq, D]`` (bf16)."""
+    if scaling is None:
+        scaling = q.shape[-1] ** -0.5
+    return _DFlashAttention.apply(q, k, v, mask, scaling)
+
+
+def dflash_hip_attention_forward(module, query, key, value, attention_mask, scaling=None, **_kwargs):
+    """Attention-function signature of the reference registry (models/attention.py:20-66,
+    called from models/dflash/model_definitions.py:134-152); the mask is a ``DFlashMask``."""
+    if not isinstance(attention_mask, DFlashMask):
+        raise TypeError(
+            f"attention impl '{ATTN_IMPL_DFLASH}' needs a DFlashMask descriptor as attention_mask, "
+            f"got {type(attention_mask).__name__}")
+    return dflash_attention(query, key, value, attention_mask, scaling), None
+
+
 class AttentionRegistry(dict):
     """Name -> attention function; the local mirror of the reference's
     ``ALL_ATTENTION_FUNCTIONS`` (models/attention.py:107-108)."""
@@ -139,6 +254,7 @@ class AttentionRegistry(dict):
 
 ALL_ATTENTION_FUNCTIONS = AttentionRegistry()
 ALL_ATTENTION_FUNCTIONS.register(ATTN_IMPL_TTT, ttt_hip_attention_forward)
+ALL_ATTENTION_FUNCTIONS.register(ATTN_IMPL_DFLASH, dflash_hip_attention_forward)
 
 
 def register_with_transformers() -> None:

@@ -1,0 +1,236 @@
+"""DFlash draft model: host side of the HIP anchored-block training path.
+
+Keeps the call contract of ``DFlashDraftModel.forward``
+(models/dflash/core.py:441-478):
+
+    forward(hidden_states, input_ids, loss_mask, verifier_last_hidden_states,
+            document_ids, position_ids, loss_config, gamma, max_anchors,
+            per_position_loss_weight, dpace_alpha) -> (None, loss, metrics)
+
+and the reference's state-dict names (models/dflash/core.py:36-120).  The
+anchored-block attention of every layer runs on the HIP interval-masked
+kernel, fc / lm_head / verifier head on the MFMA GEMM, loss and per-slot
+acceptance counts on the fused vocabulary loss kernel.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import attention as A
+from . import gemm
+from . import losses as L
+from . import metrics as MT
+from .eagle3 import MLP, RMSNorm, _rope_tables, _rotate_half
+
+
+@dataclass
+class DFlashConfig:
+    hidden_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    intermediate_size: int
+    vocab_size: int
+    draft_vocab_size: int
+    num_aux: int = 5
+    num_hidden_layers: int = 5
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 1000000.0
+    block_size: int = 8
+    mask_token_id: int | None = None
+    sliding_window: int | None = None
+    sliding_layers: tuple = field(default_factory=tuple)
+    sliding_window_non_causal: bool = False
+    sample_from_anchor: bool = False
+    attn_implementation: str = A.ATTN_IMPL_DFLASH
+
+
+def get_base_indices_for_anchored_blocks(anchor_positions: torch.Tensor, block_size: int):
+    """[a, a+1, ..., a+bs-1] per anchor, flattened (models/dflash/utils.py:6-18)."""
+    a = anchor_positions.to(dtype=torch.long).view(-1)
+    off = torch.arange(block_size, device=a.device, dtype=torch.long)
+    return (a[:, None] + off[None, :]).reshape(-1)
+
+
+def select_anchors(loss_mask: torch.Tensor, num_anchors: int, block_size: int):
+    """Random anchors among the positions with loss_mask set, excluding the last
+    ``block_size`` positions; sorted; padded with position 0 / invalid
+    (models/dflash/utils.py:21-67)."""
+    if loss_mask.ndim != 2:
+        raise ValueError(f"Expected [B, T], got {loss_mask.shape}")
+    if block_size <= 0:
+        raise ValueError(f"Expected block size > 0, got {block_size}")
+    valid = loss_mask.bool().clone()
+    valid[:, -block_size:] = False
+    idx = torch.nonzero(valid.squeeze(0), as_tuple=False).squeeze(-1)
+    dev = loss_mask.device
+    anchors = torch.zeros(num_anchors, dtype=torch.long, device=dev)
+    ok = torch.zeros(num_anchors, dtype=torch.bool, device=dev)
+    k = min(num_anchors, idx.numel())
+    perm = torch.randperm(idx.numel(), device=dev)
+    anchors[:k] = torch.sort(idx[perm[:k]]).values
+    ok[:k] = True
+    return anchors, ok
+
+
+class DFlashAttention(nn.Module):
+    """q from the mask tokens; k/v from ``cat([context, mask tokens])``; per-head q/k
+    RMSNorm; RoPE with the last q_len positions for q
+    (models/dflash/model_definitions.py:47-155)."""
+
+    def __init__(self, cfg: DFlashConfig):
+        super().__init__()
+        hq, hkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+        self.hq, self.hkv, self.d = hq, hkv, d
+        self.q_proj = nn.Linear(cfg.hidden_size, hq * d, bias=False)
+        self.k_proj = nn.Linear(cfg.hidden_size, hkv * d, bias=False)
+        self.v_proj = nn.Linear(cfg.hidden_size, hkv * d, bias=False)
+        self.o_proj = nn.Linear(hq * d, cfg.hidden_size, bias=False)
+        self.q_norm = RMSNorm(d, cfg.rms_norm_eps)
+        self.k_norm = RMSNorm(d, cfg.rms_norm_eps)
+        self.scaling = d ** -0.5
+        self.attn_fn = A.ALL_ATTENTION_FUNCTIONS[cfg.attn_implementation]
+
+    def forward(self, x, ctx, cos, sin, mask):
+        ql, tl = x.shape[1], ctx.shape[1]
+        q = self.q_norm(self.q_proj(x).view(1, ql, self.hq, self.d)).transpose(1, 2)
+        k = torch.cat([self.k_proj(ctx), self.k_proj(x)], dim=1).view(1, tl + ql, self.hkv, self.d)
+        v = torch.cat([self.v_proj(ctx), self.v_proj(x)], dim=1).view(1, tl + ql, self.hkv, self.d)
+        k = self.k_norm(k).transpose(1, 2)
+        v = v.transpose(1, 2)
+        c, s = cos.unsqueeze(1), sin.unsqueeze(1)
+        q = q * c[..., -ql:, :] + _rotate_half(q) * s[..., -ql:, :]
+        k = k * c + _rotate_half(k) * s
+        out, _ = self.attn_fn(self, q, k, v, mask, scaling=self.scaling)
+        return self.o_proj(out.reshape(1, ql, self.hq * self.d))
+
+
+class DFlashDecoderLayer(nn.Module):
+    def __init__(self, cfg: DFlashConfig):
+        super().__init__()
+        self.self_attn = DFlashAttention(cfg)
+        mlp_cfg = type("C", (), {"hidden_size": cfg.hidden_size,
+                                 "intermediate_size": cfg.intermediate_size})
+        self.mlp = MLP(mlp_cfg)
+        self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+        self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+
+    def forward(self, x, ctx, cos, sin, mask):
+        y = x + self.self_attn(self.input_layernorm(x), ctx, cos, sin, mask)
+        return y + self.mlp(self.post_attention_layernorm(y))
+
+
+class DFlashDraftModel(nn.Module):
+    def __init__(self, config: DFlashConfig):
+        super().__init__()
+        self.config = config
+        h = config.hidden_size
+        self.block_size = config.block_size
+        self.draft_vocab_size = config.draft_vocab_size
+        self.verifier_vocab_size = config.vocab_size
+        self.use_draft_vocab = config.draft_vocab_size != config.vocab_size
+        if self.use_draft_vocab:
+            self.register_buffer("t2d", torch.zeros(config.vocab_size, dtype=torch.bool))
+            self.register_buffer("d2t", torch.zeros(config.draft_vocab_size, dtype=torch.long))
+        else:
+            self.t2d = self.d2t = None
+        self.embed_tokens = nn.Embedding(config.vocab_size, h)
+        self.lm_head = nn.Linear(h, config.draft_vocab_size, bias=False)
+        self.verifier_lm_head = nn.Linear(h, config.draft_vocab_size, bias=False)
+        self.fc = nn.Linear(config.num_aux * h, h, bias=False)
+        self.hidden_norm = RMSNorm(h, config.rms_norm_eps)
+        self.layers = nn.ModuleList(DFlashDecoderLayer(config) for _ in range(config.num_hidden_layers))
+        self.norm = RMSNorm(h, config.rms_norm_eps)
+        self.verifier_norm = RMSNorm(h, config.rms_norm_eps)
+        for p in (self.embed_tokens.weight, self.lm_head.weight, self.verifier_lm_head.weight,
+                  self.verifier_norm.weight):
+            p.requires_grad_(False)
+        self.uses_sliding_window_attn = bool(config.sliding_layers)
+        self.uses_full_attn = config.num_hidden_layers > len(config.sliding_layers)
+        self._frozen_t: dict = {}
+
+    @property
+    def mask_token_id(self) -> int:
+        if self.config.mask_token_id is None:
+            raise ValueError(
+                "mask_token_id is not set on the config. Pass --mask-token-id during training or "
+                "ensure the config was saved with mask_token_id set.")
+        return self.config.mask_token_id
+
+    def _linear(self, x, weight, frozen=False):
+        if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+            raise RuntimeError("the HIP draft path runs in bf16: cast the model and its inputs to bfloat16")
+        wt = None
+        if frozen and x.requires_grad:
+            key = (weight.data_ptr(), weight._version)
+            hit = self._frozen_t.get(id(weight))
+            if hit is None or hit[0] != key:
+                hit = (key, weight.detach().t().contiguous())
+                self._frozen_t[id(weight)] = hit
+            wt = hit[1]
+        return gemm.linear(x, weight, wt)
+
+    def forward(self, hidden_states, input_ids, loss_mask, verifier_last_hidden_states,
+                document_ids, position_ids=None, loss_config: L.LossConfig | None = None,
+                gamma: float = 4.0, max_anchors: int = 512,
+                per_position_loss_weight: str = "fixed-exp-decay", dpace_alpha: float = 0.5,
+                anchors=None, **_kwargs):
+        """``anchors=(positions, valid)`` overrides the random anchor selection."""
+        cfg = self.config
+        device = hidden_states.device
+        t = hidden_states.shape[1]
+        bs = self.block_size
+        if position_ids is None:
+            position_ids = torch.arange(t, dtype=torch.long, device=device).unsqueeze(0)
+        if anchors is None:
+            anchors = select_anchors(loss_mask, max_anchors, bs)
+        anchor_pos, anchor_valid = anchors
+        doc = document_ids.reshape(-1).to(device)
+        full_mask = (A.create_dflash_mask(doc, t, anchor_pos, bs, None)
+                     if self.uses_full_attn else None)
+        sw_mask = (A.create_dflash_mask(doc, t, anchor_pos, bs, cfg.sliding_window,
+                                        cfg.sliding_window_non_causal)
+                   if self.uses_sliding_window_attn else None)
+        n_q = anchor_pos.numel() * bs
+        ids = torch.full((1, n_q), self.mask_token_id, dtype=torch.long, device=device)
+        ids[:, ::bs] = input_ids[:, anchor_pos]
+        with torch.no_grad():
+            noise = F.embedding(ids, self.embed_tokens.weight).to(hidden_states.dtype)
+        ctx = self.hidden_norm(self._linear(hidden_states, self.fc.weight))
+        block_pos = get_base_indices_for_anchored_blocks(position_ids[0, anchor_pos], bs)
+        all_pos = torch.cat([position_ids, block_pos.unsqueeze(0)], dim=1)
+        cos, sin = _rope_tables(all_pos, cfg.head_dim, cfg.rope_theta, hidden_states.dtype)
+        block_idx = get_base_indices_for_anchored_blocks(anchor_pos, bs)
+        with torch.no_grad():
+            idx = block_idx if cfg.sample_from_anchor else (block_idx - 1) % t
+            targets = self._linear(self.verifier_norm(verifier_last_hidden_states[:, idx]),
+                                   self.verifier_lm_head.weight)
+        for li, layer in enumerate(self.layers):
+            noise = layer(noise, ctx, cos, sin, sw_mask if li in cfg.sliding_layers else full_mask)
+        logits = self._linear(self.norm(noise), self.lm_head.weight, frozen=True)
+        aligned = loss_mask.clone()[:, block_idx]
+        aligned = aligned * anchor_valid.repeat_interleave(bs).unsqueeze(0).to(aligned.dtype)
+        if not cfg.sample_from_anchor:
+            aligned[:, ::bs] = 0
+        loss, metrics = MT.dflash_compute_metrics(
+            logits, targets, aligned, bs, gamma=gamma, loss_config=loss_config,
+            per_position_loss_weight=per_position_loss_weight, dpace_alpha=dpace_alpha,
+            sample_from_anchor=cfg.sample_from_anchor)
+        return None, loss, metrics
+
+    @staticmethod
+    def get_trainer_kwargs(**kwargs):
+        """(train_call_kwargs, val_call_kwargs) like models/dflash/core.py:234-262."""
+        shared = {
+            "loss_config": L.resolve_loss_config(kwargs["loss_fn"], kwargs.get("loss_implementation", "hip")),
+            "gamma": kwargs.get("dflash_decay_gamma", 4.0),
+            "max_anchors": kwargs.get("max_anchors", 512),
+            "per_position_loss_weight": kwargs.get("per_position_loss_weight", "fixed-exp-decay"),
+            "dpace_alpha": kwargs.get("dpace_alpha", 0.5),
+        }
+        return dict(shared), dict(shared)

@@ -81,18 +81,26 @@ def test_forward_backward_matches_oracle(variant):
 
     rel = abs(loss.item() - rloss.item()) / abs(rloss.item())
     print("loss", loss.item(), rloss.item(), rel)
-    assert rel < 5e-3  # bf16 activations against an fp32 oracle
+    assert rel < 1e-3  # bf16 activations against an fp32 oracle
     assert set(m) == set(rm)
     for key in rm:
         if key.endswith("_total"):
             assert m[key].item() == rm[key].item(), key  # mask / row counts: exact
+    # the same oracle in bf16 on the CPU gives the rounding noise floor of this model
+    wb = {k_: v.clone().requires_grad_(v.dtype.is_floating_point) for k_, v in w.items()}
+    _, bloss, _ = OE.eagle3_forward(wb, shape, hs, ids, doc, mask, pos, vl, ttt_steps=steps,
+                                    ttt_step_loss_decay=0.9)
+    bloss.backward()
     for name, p in model.named_parameters():
         if not p.requires_grad:
             assert p.grad is None
             continue
         want = wf[name].grad
+        scale = want.abs().max().item()
         err = (p.grad.float().cpu() - want).abs().max().item()
-        assert err <= 3e-2 * want.abs().max().item() + 1e-6, (name, err, want.abs().max().item())
+        floor = (wb[name].grad.float() - want).abs().max().item()
+        # 2e-2 relative max-norm, or twice the error a bf16 PyTorch run of the oracle makes
+        assert err <= max(2e-2 * scale, 2 * floor) + 1e-6, (name, err, floor, scale)
     assert len(toks) == steps and toks[0].shape == (1, t) and toks[0].dtype == torch.int64
     # draft tokens are an arg-max of bf16 logits: compare where the oracle's top-2 margin is clear
     for k in range(steps):
