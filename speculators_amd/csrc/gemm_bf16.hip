@@ -1,25 +1,36 @@
 // C[M, N] = A[M, K] * B[N, K]^T  (the nn.Linear product), bf16 in, fp32
 // accumulate, bf16 out, for gfx950.
 //
-// One workgroup of 4 waves owns a 256 x 256 tile of C and walks K in steps of
-// 64; each wave owns a 128 x 128 quadrant as 4 x 4 accumulators of
-// v_mfma_f32_32x32x16_bf16 (256 accumulator registers per lane).  A and B
-// tiles are staged global -> registers -> LDS with the next tile's global
+// One workgroup of 8 waves (4 along M x 2 along N) owns a 256 x 256 tile of C
+// and walks K in steps of 64; each wave owns a 64 x 128 patch as 2 x 4
+// accumulators of v_mfma_f32_32x32x16_bf16, two waves per SIMD so one wave's
+// LDS reads overlap the other's MFMAs.  A and B tiles are staged global ->
+// registers -> LDS through two LDS stages (the next tile is written while the
+// current one is read: one barrier per K step) with the next tile's global
 // loads in flight during the current tile's MFMAs.  LDS rows are padded by 16
-// bytes so the 16-byte operand reads of 16 consecutive lanes hit 16 distinct
-// bank groups.  Workgroup ids are remapped so that each XCD (ids are dealt
-// round-robin over the 8 XCDs) works on a compact band of tiles and shares
-// its A / B panels in that XCD's L2.
+// bytes so the 16-byte operand reads of consecutive lanes hit distinct bank
+// groups (measured: zero bank conflicts).  Workgroup ids are remapped so that
+// each XCD (ids are dealt round-robin over the 8 XCDs) works on a compact
+// band of tiles and shares its A / B panels in that XCD's L2.
 
 #include "spx_common.h"
 #include "../../include/spx.h"
 
 namespace spx {
 
-constexpr int kGemmThreads = 256;
+#ifndef SPX_GEMM_WM
+#define SPX_GEMM_WM 4
+#endif
+#ifndef SPX_GEMM_WN
+#define SPX_GEMM_WN 2
+#endif
+constexpr int kWM = SPX_GEMM_WM, kWN = SPX_GEMM_WN;  // waves along M / N of the tile
+constexpr int kGemmThreads = 64 * kWM * kWN;
 constexpr int kTM = 256, kTN = 256, kTK = 64;
+constexpr int kMI = kTM / kWM / 32, kNI = kTN / kWN / 32;  // 32x32 accumulators per wave
 constexpr int kLdsStride = kTK + 8;  // elements
-constexpr int kGemmSmem = (kTM + kTN) * kLdsStride * 2;
+constexpr int kStageElems = (kTM + kTN) * kLdsStride;
+constexpr int kGemmSmem = 2 * kStageElems * 2;  // two stages
 
 __device__ __forceinline__ bf16x8 lds_frag(const uint16_t* p) {
   union { u32x4 u; bf16x8 b; } c;
@@ -31,8 +42,6 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_nt_kernel(
     const uint16_t* __restrict__ A, int64_t lda, const uint16_t* __restrict__ B, int64_t ldb,
     uint16_t* __restrict__ C, int64_t ldc, int M, int N, int K, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-  uint16_t* As = smem;
-  uint16_t* Bs = smem + kTM * kLdsStride;
 
   // workgroup id -> tile: XCD-contiguous bands, then groups of 8 tile rows
   const int n_wg = tiles_m * tiles_n;
@@ -55,66 +64,85 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_nt_kernel(
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 5, col = lane & 31;
-  const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
+  const int wm = (wave / kWN) * (kTM / kWM), wn = (wave % kWN) * (kTN / kWN);
 
-  // global -> register staging: 8 chunks of 16 bytes per operand per thread
+  // global -> register staging: 16-byte chunks, 8 per row of the 64-wide K tile
+  constexpr int kRowsPerPass = kGemmThreads / 8;
+  constexpr int kPasses = kTM / kRowsPerPass;
   const int lrow = tid >> 3, lcol = (tid & 7) * 8;
-  u32x4 areg[8], breg[8];
+  u32x4 areg[kPasses], breg[kPasses];
+  // row pointers are fixed for the whole K walk (rows past the edge are clamped: their
+  // products land in accumulators that are never stored)
+  const uint16_t* aptr[kPasses];
+  const uint16_t* bptr[kPasses];
+#pragma unroll
+  for (int n = 0; n < kPasses; ++n) {
+    const int r = lrow + kRowsPerPass * n;
+    aptr[n] = A + (int64_t)min(m0 + r, M - 1) * lda + lcol;
+    bptr[n] = B + (int64_t)min(n0 + r, N - 1) * ldb + lcol;
+  }
   auto fetch = [&](int k0) {
     const bool kin = k0 + lcol < K;
+    const u32x4 z = {0, 0, 0, 0};
 #pragma unroll
-    for (int n = 0; n < 8; ++n) {
-      const int r = lrow + 32 * n;
-      const int am = min(m0 + r, M - 1), bn = min(n0 + r, N - 1);
-      const u32x4 z = {0, 0, 0, 0};
-      areg[n] = kin ? *reinterpret_cast<const u32x4*>(A + (int64_t)am * lda + k0 + lcol) : z;
-      breg[n] = kin ? *reinterpret_cast<const u32x4*>(B + (int64_t)bn * ldb + k0 + lcol) : z;
+    for (int n = 0; n < kPasses; ++n) {
+      areg[n] = kin ? *reinterpret_cast<const u32x4*>(aptr[n] + k0) : z;
+      breg[n] = kin ? *reinterpret_cast<const u32x4*>(bptr[n] + k0) : z;
     }
   };
-  auto stash = [&]() {
+  auto stash = [&](int stage) {
+    uint16_t* As = smem + stage * kStageElems;
+    uint16_t* Bs = As + kTM * kLdsStride;
 #pragma unroll
-    for (int n = 0; n < 8; ++n) {
-      const int r = lrow + 32 * n;
+    for (int n = 0; n < kPasses; ++n) {
+      const int r = lrow + kRowsPerPass * n;
       *reinterpret_cast<u32x4*>(&As[r * kLdsStride + lcol]) = areg[n];
       *reinterpret_cast<u32x4*>(&Bs[r * kLdsStride + lcol]) = breg[n];
     }
   };
 
-  f32x16 acc[4][4];
+  f32x16 acc[kMI][kNI];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < kMI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < kNI; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+  // two LDS stages: the next tile is written while the current one is read, one
+  // barrier per K step
   fetch(0);
+  stash(0);
+  __syncthreads();
+  int stage = 0;
   for (int k0 = 0; k0 < K; k0 += kTK) {
-    __syncthreads();
-    stash();
-    __syncthreads();
-    if (k0 + kTK < K) fetch(k0 + kTK);
+    const bool more = k0 + kTK < K;
+    if (more) fetch(k0 + kTK);
+    const uint16_t* As = smem + stage * kStageElems;
+    const uint16_t* Bs = As + kTM * kLdsStride;
 #pragma unroll
     for (int kk = 0; kk < kTK / 16; ++kk) {
-      bf16x8 af[4], bf[4];
+      bf16x8 af[kMI], bf[kNI];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        af[i] = lds_frag(&As[(wm + i * 32 + col) * kLdsStride + kk * 16 + g * 8]);
-        bf[i] = lds_frag(&Bs[(wn + i * 32 + col) * kLdsStride + kk * 16 + g * 8]);
-      }
+      for (int i = 0; i < kMI; ++i) af[i] = lds_frag(&As[(wm + i * 32 + col) * kLdsStride + kk * 16 + g * 8]);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int j = 0; j < kNI; ++j) bf[j] = lds_frag(&Bs[(wn + j * 32 + col) * kLdsStride + kk * 16 + g * 8]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+      for (int i = 0; i < kMI; ++i)
+#pragma unroll
+        for (int j = 0; j < kNI; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
     }
+    if (more) stash(stage ^ 1);
+    __syncthreads();
+    stage ^= 1;
   }
 
   // accumulator (i, j): lane column = n, register r = row 8*(r/4) + 4*g + r%4
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < kMI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kNI; ++j) {
       const int n = n0 + wn + j * 32 + col;
       if (n >= N) continue;
 #pragma unroll
