@@ -217,6 +217,42 @@ int spx_dflash_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
                         int64_t dk_head_stride, void* dv, int64_t dv_head_stride,
                         void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------- layer glue
+ * RMSNorm with the rounding points of the HF blocks the reference builds on
+ * (LlamaRMSNorm / Qwen3RMSNorm as used in models/eagle3/model_definitions.py:70-85,
+ * models/eagle3/core.py:236-253,302-306, models/dflash/model_definitions.py:97-155):
+ * y = weight * bf16(x * rsqrt(mean(x^2) + eps)), bf16 in/out, rstd f32 [rows]
+ * saved for the backward (may be NULL). */
+int spx_rmsnorm_fwd(const void* x, int64_t ld_x, const void* weight, void* y,
+                    int64_t ld_y, float* rstd, int64_t rows, int64_t H, float eps,
+                    void* stream);
+/* number of partial-sum slots the backward needs: dw_scratch holds slots * H floats */
+int64_t spx_rmsnorm_bwd_slots(int64_t rows, int64_t H);
+/* dx and (optionally, dweight != NULL) dweight = sum_rows dy * xhat, reduced in a
+ * fixed order (deterministic). */
+int spx_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weight, const void* dy,
+                    int64_t ld_dy, const float* rstd, void* dx, int64_t ld_dx,
+                    void* dweight, float* dw_scratch, int64_t rows, int64_t H,
+                    void* stream);
+
+/* Rotary embedding fused with the head-major relayout that precedes attention
+ * (apply_rotary_pos_emb + the view/transpose of LlamaAttention.forward; for
+ * DFlash models/dflash/model_definitions.py:29-45):
+ *   inverse == 0: out[h, t, :] = rope(x[t, h*D : (h+1)*D], position_ids[t] + position_offset)
+ *   inverse != 0: out[t, h*D : (h+1)*D] = rope^T(x[h, t, :], ...)   (its backward)
+ * rotate == 0 only relayouts (V).  inv_freq: f32 [D/2].  Half-split rotation,
+ * cos/sin evaluated in fp32 and rounded to bf16 like the HF rotary module. */
+int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* position_ids,
+                      const float* inv_freq, void* out, int64_t ld_out, int64_t T,
+                      int32_t heads, int32_t D, int32_t rotate, int32_t inverse,
+                      int64_t position_offset, void* stream);
+
+/* out = bf16(silu(gate)) * up  (LlamaMLP / Qwen3MLP act_fn(gate_proj(x)) * up_proj(x)),
+ * n elements, bf16; and its backward. */
+int spx_swiglu_fwd(const void* gate, const void* up, void* out, int64_t n, void* stream);
+int spx_swiglu_bwd(const void* gate, const void* up, const void* dout, void* dgate,
+                   void* dup, int64_t n, void* stream);
+
 /* ---------------------------------------------------------------- GEMM
  * c[M, N] = a[M, K] * b[N, K]^T, bf16 inputs, fp32 accumulation, bf16 output:
  * the product of torch.nn.Linear (no bias).  Replaces the fc Linear

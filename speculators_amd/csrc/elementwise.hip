@@ -1,0 +1,356 @@
+// HBM-bound glue of the draft decoder layer for gfx950: RMSNorm, rotary
+// embedding fused with the [T, heads*D] -> [heads, T, D] relayout, and the
+// SwiGLU gate.  bf16 in / out, fp32 inside, 16-byte accesses.  Rounding points
+// follow the HF blocks the reference is built from (LlamaRMSNorm,
+// apply_rotary_pos_emb, LlamaMLP): every bf16 tensor op of the eager path is
+// one rounding here.
+
+#include "spx_common.h"
+#include "../../include/spx.h"
+
+namespace spx {
+
+__device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+__device__ __forceinline__ void unpack8f(u32x4 raw, float v[8]) {
+  v[0] = bf16_lo(raw.x); v[1] = bf16_hi(raw.x);
+  v[2] = bf16_lo(raw.y); v[3] = bf16_hi(raw.y);
+  v[4] = bf16_lo(raw.z); v[5] = bf16_hi(raw.z);
+  v[6] = bf16_lo(raw.w); v[7] = bf16_hi(raw.w);
+}
+__device__ __forceinline__ u32x4 pack8f(const float v[8]) {
+  u32x4 r;
+  r.x = pack_bf16x2(v[0], v[1]); r.y = pack_bf16x2(v[2], v[3]);
+  r.z = pack_bf16x2(v[4], v[5]); r.w = pack_bf16x2(v[6], v[7]);
+  return r;
+}
+
+__device__ __forceinline__ float block_sum_256(float v, float* lds) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return lds[0] + lds[1] + lds[2] + lds[3];
+}
+
+// ---------------------------------------------------------------- RMSNorm
+// y = w * bf16(x * rsqrt(mean(x^2) + eps));  one workgroup per row (H >= 512) or one
+// wave per row (small H, e.g. per-head q/k norm).  MAXC = 16-byte chunks a lane keeps.
+template <int MAXC, bool WAVE_ROWS>
+__global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(
+    const uint16_t* __restrict__ x, int64_t ld_x, const uint16_t* __restrict__ w,
+    uint16_t* __restrict__ y, int64_t ld_y, float* __restrict__ rstd, int64_t rows, int H,
+    float eps) {
+  __shared__ float red[4];
+  const int nthr = WAVE_ROWS ? 64 : 256;
+  const int t = WAVE_ROWS ? (threadIdx.x & 63) : threadIdx.x;
+  const int64_t row = WAVE_ROWS ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
+  if (WAVE_ROWS && row >= rows) return;
+  const int nch = H / 8;
+  float v[MAXC][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int ch = t + c * nthr;
+    if (ch < nch) {
+      unpack8f(*reinterpret_cast<const u32x4*>(x + row * ld_x + ch * 8), v[c]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss = fmaf(v[c][e], v[c][e], ss);
+    }
+  }
+  ss = WAVE_ROWS ? wave_sum(ss) : block_sum_256(ss, red);
+  const float r = rsqrtf(ss / (float)H + eps);
+  if (t == 0 && rstd) rstd[row] = r;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int ch = t + c * nthr;
+    if (ch < nch) {
+      float wv[8], o[8];
+      unpack8f(*reinterpret_cast<const u32x4*>(w + ch * 8), wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = wv[e] * round_bf16(v[c][e] * r);
+      *reinterpret_cast<u32x4*>(y + row * ld_y + ch * 8) = pack8f(o);
+    }
+  }
+}
+
+// dx = rstd * (g - xhat * mean(g * xhat)), g = dy * w, xhat = x * rstd;
+// dw partial sums: block b accumulates the rows b, b + gridDim.x, ... per column.
+template <int MAXC, bool WAVE_ROWS>
+__global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(
+    const uint16_t* __restrict__ x, int64_t ld_x, const uint16_t* __restrict__ w,
+    const uint16_t* __restrict__ dy, int64_t ld_dy, const float* __restrict__ rstd,
+    uint16_t* __restrict__ dx, int64_t ld_dx, float* __restrict__ dw_part, int64_t rows, int H) {
+  __shared__ float red[4];
+  const int nthr = WAVE_ROWS ? 64 : 256;
+  const int t = WAVE_ROWS ? (threadIdx.x & 63) : threadIdx.x;
+  const int wave = threadIdx.x >> 6;
+  const int nch = H / 8;
+  float wv[MAXC][8], dwacc[MAXC][8];
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int ch = t + c * nthr;
+    if (ch < nch) unpack8f(*reinterpret_cast<const u32x4*>(w + ch * 8), wv[c]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dwacc[c][e] = 0.f;
+  }
+  const int64_t first = WAVE_ROWS ? (int64_t)blockIdx.x * 4 + wave : blockIdx.x;
+  const int64_t stride = WAVE_ROWS ? (int64_t)gridDim.x * 4 : gridDim.x;
+  for (int64_t row = first; row < rows; row += stride) {
+    const float r = rstd[row];
+    float xh[MAXC][8], g[MAXC][8];
+    float dot = 0.f;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+      const int ch = t + c * nthr;
+      if (ch < nch) {
+        float xv[8], dv[8];
+        unpack8f(*reinterpret_cast<const u32x4*>(x + row * ld_x + ch * 8), xv);
+        unpack8f(*reinterpret_cast<const u32x4*>(dy + row * ld_dy + ch * 8), dv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          xh[c][e] = xv[e] * r;
+          g[c][e] = dv[e] * wv[c][e];
+          dot = fmaf(g[c][e], xh[c][e], dot);
+          dwacc[c][e] = fmaf(dv[e], xh[c][e], dwacc[c][e]);
+        }
+      }
+    }
+    dot = WAVE_ROWS ? wave_sum(dot) : block_sum_256(dot, red);
+    const float mean = dot / (float)H;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+      const int ch = t + c * nthr;
+      if (ch < nch) {
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = r * (g[c][e] - xh[c][e] * mean);
+        *reinterpret_cast<u32x4*>(dx + row * ld_dx + ch * 8) = pack8f(o);
+      }
+    }
+  }
+  if (dw_part) {
+    const int64_t slot = WAVE_ROWS ? (int64_t)blockIdx.x * 4 + wave : blockIdx.x;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+      const int ch = t + c * nthr;
+      if (ch < nch) {
+        float* o = dw_part + slot * H + ch * 8;
+        f32x4 a = {dwacc[c][0], dwacc[c][1], dwacc[c][2], dwacc[c][3]};
+        f32x4 b = {dwacc[c][4], dwacc[c][5], dwacc[c][6], dwacc[c][7]};
+        *reinterpret_cast<f32x4*>(o) = a;
+        *reinterpret_cast<f32x4*>(o + 4) = b;
+      }
+    }
+  }
+}
+
+// dw[c] = sum_s dw_part[s, c]  (fixed order: deterministic), bf16 out
+__global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ part, int64_t slots,
+                                                     int H, uint16_t* __restrict__ out) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= H) return;
+  float s = 0.f;
+  for (int64_t i = 0; i < slots; ++i) s += part[i * H + c];
+  out[c] = (uint16_t)f32_to_bf16_bits(s);
+}
+
+// ---------------------------------------------------------------- RoPE + relayout
+// forward:  out[h, t, :] = rope(x[t, h, :], pos[t])      x: [T, heads*D] (row stride ld_x)
+// inverse:  out[t, h, :] = rope^T(x[h, t, :], pos[t])    (the backward of the above)
+// rotate == 0: relayout only (used for V).  cos / sin are evaluated in fp32 from
+// pos * inv_freq and rounded to bf16, as the HF rotary module does.
+template <bool INVERSE>
+__global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ x, int64_t ld_x,
+                                                   const int64_t* __restrict__ pos,
+                                                   const float* __restrict__ inv_freq,
+                                                   uint16_t* __restrict__ out, int64_t ld_out, int T,
+                                                   int heads, int D, int rotate, int64_t pos_offset) {
+  // one thread: 8 consecutive d of the first half and the matching 8 of the second half
+  const int per_row = D / 16;
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t total = (int64_t)T * heads * per_row;
+  if (item >= total) return;
+  const int d0 = (int)(item % per_row) * 8;
+  const int h = (int)((item / per_row) % heads);
+  const int t = (int)(item / ((int64_t)per_row * heads));
+  const int half = D / 2;
+  const uint16_t* src = INVERSE ? x + ((int64_t)h * T + t) * D : x + (int64_t)t * ld_x + h * D;
+  uint16_t* dst = INVERSE ? out + (int64_t)t * ld_out + h * D : out + ((int64_t)h * T + t) * D;
+  float a[8], b[8], oa[8], ob[8];
+  unpack8f(*reinterpret_cast<const u32x4*>(src + d0), a);
+  unpack8f(*reinterpret_cast<const u32x4*>(src + half + d0), b);
+  if (rotate) {
+    const float p = (float)(pos[t] + pos_offset);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float ang = p * inv_freq[d0 + e];
+      const float c = round_bf16(cosf(ang));
+      float s = round_bf16(sinf(ang));
+      if (INVERSE) s = -s;
+      // x*cos + rotate_half(x)*sin with each bf16 op rounded
+      oa[e] = round_bf16(a[e] * c) + round_bf16(-b[e] * s);
+      ob[e] = round_bf16(b[e] * c) + round_bf16(a[e] * s);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { oa[e] = a[e]; ob[e] = b[e]; }
+  }
+  *reinterpret_cast<u32x4*>(dst + d0) = pack8f(oa);
+  *reinterpret_cast<u32x4*>(dst + half + d0) = pack8f(ob);
+}
+
+// ---------------------------------------------------------------- SwiGLU
+__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint16_t* __restrict__ g,
+                                                         const uint16_t* __restrict__ u,
+                                                         uint16_t* __restrict__ out, int64_t n8) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+    float gv[8], uv[8], o[8];
+    unpack8f(*reinterpret_cast<const u32x4*>(g + i * 8), gv);
+    unpack8f(*reinterpret_cast<const u32x4*>(u + i * 8), uv);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float sg = 1.f / (1.f + __expf(-gv[e]));
+      o[e] = round_bf16(gv[e] * sg) * uv[e];
+    }
+    *reinterpret_cast<u32x4*>(out + i * 8) = pack8f(o);
+  }
+}
+
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* __restrict__ g,
+                                                         const uint16_t* __restrict__ u,
+                                                         const uint16_t* __restrict__ dout,
+                                                         uint16_t* __restrict__ dg,
+                                                         uint16_t* __restrict__ du, int64_t n8) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+    float gv[8], uv[8], dv[8], og[8], ou[8];
+    unpack8f(*reinterpret_cast<const u32x4*>(g + i * 8), gv);
+    unpack8f(*reinterpret_cast<const u32x4*>(u + i * 8), uv);
+    unpack8f(*reinterpret_cast<const u32x4*>(dout + i * 8), dv);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float sg = 1.f / (1.f + __expf(-gv[e]));
+      const float act = gv[e] * sg;
+      ou[e] = dv[e] * act;
+      og[e] = dv[e] * uv[e] * (sg * (1.f + gv[e] * (1.f - sg)));
+    }
+    *reinterpret_cast<u32x4*>(dg + i * 8) = pack8f(og);
+    *reinterpret_cast<u32x4*>(du + i * 8) = pack8f(ou);
+  }
+}
+
+static bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace spx
+
+using namespace spx;
+
+extern "C" int64_t spx_rmsnorm_bwd_slots(int64_t rows, int64_t H) {
+  if (H <= 512) return 4 * (rows < 4096 ? (rows + 3) / 4 : 1024);
+  return rows < 1024 ? rows : 1024;
+}
+
+extern "C" int spx_rmsnorm_fwd(const void* x, int64_t ld_x, const void* weight, void* y, int64_t ld_y,
+                               float* rstd, int64_t rows, int64_t H, float eps, void* stream) {
+  SPX_REQUIRE(rows >= 0 && H > 0, "bad sizes");
+  SPX_REQUIRE(H % 8 == 0 && ld_x % 8 == 0 && ld_y % 8 == 0, "H and the row strides must be multiples of 8");
+  SPX_REQUIRE(H <= 16384, "H must be at most 16384");
+  SPX_REQUIRE(rows < (1ll << 31), "too many rows");
+  if (rows == 0) return SPX_OK;
+  SPX_REQUIRE(x && weight && y, "null buffer");
+  SPX_REQUIRE(al16(x) && al16(weight) && al16(y), "buffers must be 16-byte aligned");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  auto xp = reinterpret_cast<const uint16_t*>(x);
+  auto wp = reinterpret_cast<const uint16_t*>(weight);
+  auto yp = reinterpret_cast<uint16_t*>(y);
+  if (H <= 512)
+    hipLaunchKernelGGL((rmsnorm_fwd_kernel<1, true>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, xp,
+                       ld_x, wp, yp, ld_y, rstd, rows, (int)H, eps);
+  else if (H <= 4096)
+    hipLaunchKernelGGL((rmsnorm_fwd_kernel<2, false>), dim3((unsigned)rows), dim3(256), 0, st, xp, ld_x, wp,
+                       yp, ld_y, rstd, rows, (int)H, eps);
+  else
+    hipLaunchKernelGGL((rmsnorm_fwd_kernel<8, false>), dim3((unsigned)rows), dim3(256), 0, st, xp, ld_x, wp,
+                       yp, ld_y, rstd, rows, (int)H, eps);
+  return check_launch(__func__);
+}
+
+extern "C" int spx_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weight, const void* dy,
+                               int64_t ld_dy, const float* rstd, void* dx, int64_t ld_dx, void* dweight,
+                               float* dw_scratch, int64_t rows, int64_t H, void* stream) {
+  SPX_REQUIRE(rows > 0 && H > 0, "bad sizes");
+  SPX_REQUIRE(H % 8 == 0 && ld_x % 8 == 0 && ld_dy % 8 == 0 && ld_dx % 8 == 0,
+              "H and the row strides must be multiples of 8");
+  SPX_REQUIRE(H <= 16384, "H must be at most 16384");
+  SPX_REQUIRE(x && weight && dy && rstd && dx, "null buffer");
+  SPX_REQUIRE(!dweight || dw_scratch, "dweight needs dw_scratch (spx_rmsnorm_bwd_slots(rows, H) * H floats)");
+  SPX_REQUIRE(al16(x) && al16(weight) && al16(dy) && al16(dx) && al16(dw_scratch), "buffers must be 16-byte aligned");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  auto xp = reinterpret_cast<const uint16_t*>(x);
+  auto wp = reinterpret_cast<const uint16_t*>(weight);
+  auto dyp = reinterpret_cast<const uint16_t*>(dy);
+  auto dxp = reinterpret_cast<uint16_t*>(dx);
+  float* part = dweight ? dw_scratch : nullptr;
+  const int64_t slots = spx_rmsnorm_bwd_slots(rows, H);
+  if (H <= 512)
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<1, true>), dim3((unsigned)(slots / 4)), dim3(256), 0, st, xp, ld_x,
+                       wp, dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H);
+  else if (H <= 4096)
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<2, false>), dim3((unsigned)slots), dim3(256), 0, st, xp, ld_x, wp,
+                       dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H);
+  else
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<8, false>), dim3((unsigned)slots), dim3(256), 0, st, xp, ld_x, wp,
+                       dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H);
+  if (dweight)
+    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((H + 255) / 256)), dim3(256), 0, st, part, slots, (int)H,
+                       reinterpret_cast<uint16_t*>(dweight));
+  return check_launch(__func__);
+}
+
+extern "C" int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* position_ids,
+                                 const float* inv_freq, void* out, int64_t ld_out, int64_t T,
+                                 int32_t heads, int32_t D, int32_t rotate, int32_t inverse,
+                                 int64_t position_offset, void* stream) {
+  SPX_REQUIRE(T > 0 && heads > 0 && D > 0 && D % 16 == 0, "T, heads > 0 and D a multiple of 16");
+  SPX_REQUIRE(x && out && (!rotate || (position_ids && inv_freq)), "null buffer");
+  SPX_REQUIRE(al16(x) && al16(out), "buffers must be 16-byte aligned");
+  if (inverse) SPX_REQUIRE(ld_out % 8 == 0 && ld_out >= (int64_t)heads * D, "bad output row stride");
+  else SPX_REQUIRE(ld_x % 8 == 0 && ld_x >= (int64_t)heads * D, "bad input row stride");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int64_t total = T * heads * (D / 16);
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  auto xp = reinterpret_cast<const uint16_t*>(x);
+  auto op = reinterpret_cast<uint16_t*>(out);
+  if (inverse)
+    hipLaunchKernelGGL(rope_kernel<true>, dim3(grid), dim3(256), 0, st, xp, ld_x, position_ids, inv_freq, op,
+                       ld_out, (int)T, (int)heads, (int)D, (int)rotate, position_offset);
+  else
+    hipLaunchKernelGGL(rope_kernel<false>, dim3(grid), dim3(256), 0, st, xp, ld_x, position_ids, inv_freq, op,
+                       ld_out, (int)T, (int)heads, (int)D, (int)rotate, position_offset);
+  return check_launch(__func__);
+}
+
+extern "C" int spx_swiglu_fwd(const void* gate, const void* up, void* out, int64_t n, void* stream) {
+  SPX_REQUIRE(n > 0 && n % 8 == 0, "n must be a positive multiple of 8");
+  SPX_REQUIRE(gate && up && out && al16(gate) && al16(up) && al16(out), "null or unaligned buffer");
+  const int64_t n8 = n / 8;
+  const unsigned grid = (unsigned)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536);
+  hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(grid), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     reinterpret_cast<const uint16_t*>(gate), reinterpret_cast<const uint16_t*>(up),
+                     reinterpret_cast<uint16_t*>(out), n8);
+  return check_launch(__func__);
+}
+
+extern "C" int spx_swiglu_bwd(const void* gate, const void* up, const void* dout, void* dgate, void* dup,
+                              int64_t n, void* stream) {
+  SPX_REQUIRE(n > 0 && n % 8 == 0, "n must be a positive multiple of 8");
+  SPX_REQUIRE(gate && up && dout && dgate && dup, "null buffer");
+  SPX_REQUIRE(al16(gate) && al16(up) && al16(dout) && al16(dgate) && al16(dup), "buffers must be 16-byte aligned");
+  const int64_t n8 = n / 8;
+  const unsigned grid = (unsigned)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536);
+  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(grid), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     reinterpret_cast<const uint16_t*>(gate), reinterpret_cast<const uint16_t*>(up),
+                     reinterpret_cast<const uint16_t*>(dout), reinterpret_cast<uint16_t*>(dgate),
+                     reinterpret_cast<uint16_t*>(dup), n8);
+  return check_launch(__func__);
+}

@@ -22,10 +22,11 @@ import torch.nn.functional as F
 from torch import nn
 
 from . import attention as A
+from . import fused_ops as FO
 from . import gemm
 from . import losses as L
 from . import metrics as MT
-from .eagle3 import MLP, RMSNorm, _rope_tables, _rotate_half
+from .eagle3 import MLP, RMSNorm
 
 
 @dataclass
@@ -96,16 +97,15 @@ class DFlashAttention(nn.Module):
         self.scaling = d ** -0.5
         self.attn_fn = A.ALL_ATTENTION_FUNCTIONS[cfg.attn_implementation]
 
-    def forward(self, x, ctx, cos, sin, mask):
+    def forward(self, x, ctx, q_pos, kv_pos, inv_freq, mask):
         ql, tl = x.shape[1], ctx.shape[1]
-        q = self.q_norm(self.q_proj(x).view(1, ql, self.hq, self.d)).transpose(1, 2)
-        k = torch.cat([self.k_proj(ctx), self.k_proj(x)], dim=1).view(1, tl + ql, self.hkv, self.d)
-        v = torch.cat([self.v_proj(ctx), self.v_proj(x)], dim=1).view(1, tl + ql, self.hkv, self.d)
-        k = self.k_norm(k).transpose(1, 2)
-        v = v.transpose(1, 2)
-        c, s = cos.unsqueeze(1), sin.unsqueeze(1)
-        q = q * c[..., -ql:, :] + _rotate_half(q) * s[..., -ql:, :]
-        k = k * c + _rotate_half(k) * s
+        q = self.q_norm(self.q_proj(x).view(1, ql, self.hq, self.d)).view(1, ql, self.hq * self.d)
+        k = torch.cat([self.k_proj(ctx), self.k_proj(x)], dim=1)
+        v = torch.cat([self.v_proj(ctx), self.v_proj(x)], dim=1)
+        k = self.k_norm(k.view(1, tl + ql, self.hkv, self.d)).view(1, tl + ql, self.hkv * self.d)
+        q = FO.rope_relayout(q, q_pos, inv_freq, self.hq, True, 0)
+        k = FO.rope_relayout(k, kv_pos, inv_freq, self.hkv, True, 0)
+        v = FO.rope_relayout(v, kv_pos, inv_freq, self.hkv, False, 0)
         out, _ = self.attn_fn(self, q, k, v, mask, scaling=self.scaling)
         return self.o_proj(out.reshape(1, ql, self.hq * self.d))
 
@@ -120,8 +120,8 @@ class DFlashDecoderLayer(nn.Module):
         self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
         self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
 
-    def forward(self, x, ctx, cos, sin, mask):
-        y = x + self.self_attn(self.input_layernorm(x), ctx, cos, sin, mask)
+    def forward(self, x, ctx, q_pos, kv_pos, inv_freq, mask):
+        y = x + self.self_attn(self.input_layernorm(x), ctx, q_pos, kv_pos, inv_freq, mask)
         return y + self.mlp(self.post_attention_layernorm(y))
 
 
@@ -203,15 +203,17 @@ class DFlashDraftModel(nn.Module):
             noise = F.embedding(ids, self.embed_tokens.weight).to(hidden_states.dtype)
         ctx = self.hidden_norm(self._linear(hidden_states, self.fc.weight))
         block_pos = get_base_indices_for_anchored_blocks(position_ids[0, anchor_pos], bs)
-        all_pos = torch.cat([position_ids, block_pos.unsqueeze(0)], dim=1)
-        cos, sin = _rope_tables(all_pos, cfg.head_dim, cfg.rope_theta, hidden_states.dtype)
+        kv_pos = torch.cat([position_ids.reshape(-1), block_pos]).to(torch.int64).contiguous()
+        q_pos = block_pos.to(torch.int64).contiguous()
+        inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device)
         block_idx = get_base_indices_for_anchored_blocks(anchor_pos, bs)
         with torch.no_grad():
             idx = block_idx if cfg.sample_from_anchor else (block_idx - 1) % t
             targets = self._linear(self.verifier_norm(verifier_last_hidden_states[:, idx]),
                                    self.verifier_lm_head.weight)
         for li, layer in enumerate(self.layers):
-            noise = layer(noise, ctx, cos, sin, sw_mask if li in cfg.sliding_layers else full_mask)
+            noise = layer(noise, ctx, q_pos, kv_pos, inv_freq,
+                          sw_mask if li in cfg.sliding_layers else full_mask)
         logits = self._linear(self.norm(noise), self.lm_head.weight, frozen=True)
         aligned = loss_mask.clone()[:, block_idx]
         aligned = aligned * anchor_valid.repeat_interleave(bs).unsqueeze(0).to(aligned.dtype)

@@ -23,6 +23,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from . import attention as A
+from . import fused_ops as FO
 from . import gemm
 from . import losses as L
 from . import metrics as MT
@@ -61,22 +62,7 @@ class RMSNorm(nn.Module):
         self.eps = eps
 
     def forward(self, x):
-        xf = x.float()
-        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)
-        return self.weight.to(x.dtype) * xf.to(x.dtype)
-
-
-def _rotate_half(x):
-    h = x.shape[-1] // 2
-    return torch.cat([-x[..., h:], x[..., :h]], dim=-1)
-
-
-def _rope_tables(position_ids, head_dim, theta, dtype):
-    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32,
-                                        device=position_ids.device) / head_dim))
-    ang = position_ids.reshape(1, -1, 1).float() * inv.reshape(1, 1, -1)
-    ang = torch.cat([ang, ang], dim=-1)
-    return ang.cos().to(dtype), ang.sin().to(dtype)
+        return FO.rms_norm(x, self.weight, self.eps)
 
 
 class Attention(nn.Module):
@@ -95,17 +81,16 @@ class Attention(nn.Module):
         self.scaling = d ** -0.5
         self.attn_fn = A.ALL_ATTENTION_FUNCTIONS[cfg.attn_implementation]
 
-    def forward(self, x, cos, sin, cache: dict, mask):
+    def forward(self, x, position_ids, pos_offset, inv_freq, cache: dict, mask):
         t = x.shape[1]
-        q = self.q_proj(x).view(1, t, self.hq, self.d)
-        k = self.k_proj(x).view(1, t, self.hkv, self.d)
-        v = self.v_proj(x).view(1, t, self.hkv, self.d)
+        q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
         if self.qk_norm:
-            q, k = self.q_norm(q), self.k_norm(k)
-        q, k, v = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
-        c, s = cos.unsqueeze(1), sin.unsqueeze(1)
-        q = q * c + _rotate_half(q) * s
-        k = k * c + _rotate_half(k) * s
+            q = self.q_norm(q.view(1, t, self.hq, self.d)).view(1, t, self.hq * self.d)
+            k = self.k_norm(k.view(1, t, self.hkv, self.d)).view(1, t, self.hkv * self.d)
+        # rotary embedding + [T, heads*D] -> [heads, T, D] in one pass each
+        q = FO.rope_relayout(q, position_ids, inv_freq, self.hq, True, pos_offset)
+        k = FO.rope_relayout(k, position_ids, inv_freq, self.hkv, True, pos_offset)
+        v = FO.rope_relayout(v, position_ids, inv_freq, self.hkv, False, 0)
         # the K/V cache grows by T keys per TTT step (DynamicCache.update in the reference)
         cache["k"] = k if "k" not in cache else torch.cat([cache["k"], k], dim=2)
         cache["v"] = v if "v" not in cache else torch.cat([cache["v"], v], dim=2)
@@ -121,7 +106,7 @@ class MLP(nn.Module):
         self.down_proj = nn.Linear(cfg.intermediate_size, cfg.hidden_size, bias=False)
 
     def forward(self, x):
-        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+        return self.down_proj(FO.swiglu(self.gate_proj(x), self.up_proj(x)))
 
 
 class DecoderLayer(nn.Module):
@@ -141,7 +126,7 @@ class DecoderLayer(nn.Module):
         if self.first:
             self.hidden_norm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
 
-    def forward(self, x, cos, sin, cache, mask):
+    def forward(self, x, position_ids, pos_offset, inv_freq, cache, mask):
         if self.first:
             h = self.cfg.hidden_size
             embeds, hidden = x[..., :h], x[..., h:]
@@ -150,10 +135,11 @@ class DecoderLayer(nn.Module):
             hidden = self.hidden_norm(hidden)
             if self.cfg.norm_before_residual:
                 residual = hidden
-            a = self.self_attn(torch.cat([embeds, hidden], dim=-1), cos, sin, cache, mask)
+            a = self.self_attn(torch.cat([embeds, hidden], dim=-1), position_ids, pos_offset, inv_freq,
+                               cache, mask)
         else:
             residual = x
-            a = self.self_attn(self.input_layernorm(x), cos, sin, cache, mask)
+            a = self.self_attn(self.input_layernorm(x), position_ids, pos_offset, inv_freq, cache, mask)
         y = residual + a
         return y + self.mlp(self.post_attention_layernorm(y))
 
@@ -268,15 +254,16 @@ class Eagle3DraftModel(nn.Module):
             metrics: dict = {}
 
         caches = [dict() for _ in self.layers]
+        inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device)
+        position_ids = position_ids.reshape(-1).to(torch.int64).contiguous()
         draft_tokens = []
         for step in range(ttt_steps):
             with torch.no_grad():
                 embeds = F.embedding(input_ids, self.embed_tokens.weight)
-            cos, sin = _rope_tables(position_ids, cfg.head_dim, cfg.rope_theta, hidden.dtype)
             y = torch.cat([embeds.to(hidden.dtype), hidden], dim=-1)
             for li, layer in enumerate(self.layers):
                 mask = sw_mask if li in cfg.sliding_layers else full_mask
-                y = layer(y, cos, sin, caches[li], mask)
+                y = layer(y, position_ids, step, inv_freq, caches[li], mask)
             if cfg.norm_output:
                 hidden = self.norm(y)
                 logits = self._linear(hidden, self.lm_head.weight, frozen=True)
@@ -298,7 +285,6 @@ class Eagle3DraftModel(nn.Module):
                 full_mask = full_mask.extended()
             if sw_mask is not None:
                 sw_mask = sw_mask.extended()
-            position_ids = position_ids + 1
 
         if not return_loss:
             return draft_tokens

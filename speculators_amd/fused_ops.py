@@ -1,0 +1,125 @@
+"""Autograd wrappers of the HBM-bound layer glue kernels: RMSNorm, rotary embedding
+fused with the head-major relayout, SwiGLU.  bf16 HIP tensors only."""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+def _need_bf16(*ts):
+    for t in ts:
+        if t.dtype != torch.bfloat16:
+            raise _lib.SpxError("the HIP layer kernels take bf16 tensors: cast the model and its "
+                                "inputs to bfloat16")
+
+
+class _RMSNorm(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, eps):
+        _need_bf16(x, weight)
+        h = x.shape[-1]
+        x2 = x.reshape(-1, h)
+        if x2.stride(1) != 1:
+            x2 = x2.contiguous()
+        rows = x2.shape[0]
+        y = torch.empty(rows, h, device=x.device, dtype=torch.bfloat16)
+        rstd = torch.empty(rows, device=x.device, dtype=torch.float32)
+        w = weight.contiguous()
+        _lib.call("spx_rmsnorm_fwd", _lib.ptr(x2), x2.stride(0), _lib.ptr(w), _lib.ptr(y), h,
+                  _lib.ptr(rstd), rows, h, float(eps), _lib.stream_ptr(x.device))
+        ctx.save_for_backward(x2, w, rstd)
+        ctx.shape = x.shape
+        return y.view(x.shape)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, w, rstd = ctx.saved_tensors
+        rows, h = x2.shape
+        dy2 = dy.reshape(rows, h).to(torch.bfloat16)
+        if dy2.stride(1) != 1:
+            dy2 = dy2.contiguous()
+        dx = torch.empty(rows, h, device=x2.device, dtype=torch.bfloat16)
+        dw = scratch = None
+        if ctx.needs_input_grad[1]:
+            slots = int(_lib.load().spx_rmsnorm_bwd_slots(rows, h))
+            scratch = torch.empty(slots * h, device=x2.device, dtype=torch.float32)
+            dw = torch.empty(h, device=x2.device, dtype=torch.bfloat16)
+        _lib.call("spx_rmsnorm_bwd", _lib.ptr(x2), x2.stride(0), _lib.ptr(w), _lib.ptr(dy2),
+                  dy2.stride(0), _lib.ptr(rstd), _lib.ptr(dx), h, _lib.ptr(dw), _lib.ptr(scratch),
+                  rows, h, _lib.stream_ptr(x2.device))
+        return dx.view(ctx.shape), dw, None
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    return _RMSNorm.apply(x, weight, eps)
+
+
+class _RopeRelayout(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, position_ids, inv_freq, heads, rotate, offset):
+        _need_bf16(x)
+        t = x.shape[-2]
+        d = x.shape[-1] // heads
+        x2 = x.reshape(t, heads * d)
+        if x2.stride(1) != 1:
+            x2 = x2.contiguous()
+        out = torch.empty(1, heads, t, d, device=x.device, dtype=torch.bfloat16)
+        _lib.call("spx_rope_relayout", _lib.ptr(x2), x2.stride(0), _lib.ptr(position_ids),
+                  _lib.ptr(inv_freq), _lib.ptr(out), 0, t, heads, d, int(rotate), 0, int(offset),
+                  _lib.stream_ptr(x.device))
+        ctx.save_for_backward(position_ids, inv_freq)
+        ctx.meta = (x.shape, heads, d, t, rotate, offset)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        position_ids, inv_freq = ctx.saved_tensors
+        shape, heads, d, t, rotate, offset = ctx.meta
+        dout = dout.to(torch.bfloat16).contiguous()
+        dx = torch.empty(t, heads * d, device=dout.device, dtype=torch.bfloat16)
+        _lib.call("spx_rope_relayout", _lib.ptr(dout), 0, _lib.ptr(position_ids), _lib.ptr(inv_freq),
+                  _lib.ptr(dx), heads * d, t, heads, d, int(rotate), 1, int(offset),
+                  _lib.stream_ptr(dout.device))
+        return dx.view(shape), None, None, None, None, None
+
+
+def rope_relayout(x, position_ids, inv_freq, heads: int, rotate: bool = True, offset: int = 0):
+    """``[1, T, heads*D]`` -> ``[1, heads, T, D]`` with (``rotate``) the rotary embedding of
+    position ``position_ids[t] + offset`` applied; ``position_ids`` int64 ``[T]``."""
+    pos = position_ids.reshape(-1)
+    if pos.dtype != torch.int64:
+        pos = pos.to(torch.int64)
+    return _RopeRelayout.apply(x, pos.contiguous(), inv_freq, heads, rotate, offset)
+
+
+def rope_inv_freq(head_dim: int, theta: float, device) -> torch.Tensor:
+    """fp32 inverse frequencies, evaluated like the HF default rotary initialisation."""
+    return (1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))).to(device)
+
+
+class _SwiGLU(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, gate, up):
+        _need_bf16(gate, up)
+        gate, up = gate.contiguous(), up.contiguous()
+        out = torch.empty_like(gate)
+        _lib.call("spx_swiglu_fwd", _lib.ptr(gate), _lib.ptr(up), _lib.ptr(out), gate.numel(),
+                  _lib.stream_ptr(gate.device))
+        ctx.save_for_backward(gate, up)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        gate, up = ctx.saved_tensors
+        dout = dout.to(torch.bfloat16).contiguous()
+        dg, du = torch.empty_like(gate), torch.empty_like(up)
+        _lib.call("spx_swiglu_bwd", _lib.ptr(gate), _lib.ptr(up), _lib.ptr(dout), _lib.ptr(dg),
+                  _lib.ptr(du), gate.numel(), _lib.stream_ptr(gate.device))
+        return dg, du
+
+
+def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` (bf16)."""
+    return _SwiGLU.apply(gate, up)
