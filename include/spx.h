@@ -259,7 +259,8 @@ int spx_swiglu_bwd(const void* gate, const void* up, const void* dout, void* dga
  * (models/eagle3/core.py:76,244), the lm_head and verifier_lm_head Linears
  * (model.py:66-69; call sites models/eagle3/core.py:251-253,302-306) and, with
  * b = the transposed weight, the input-gradient product of their backward.
- * lda/ldb/ldc are row strides in elements; K, lda, ldb multiples of 8. */
+ * lda/ldb/ldc are row strides in elements; K, lda, ldb multiples of 8; each
+ * operand spans less than 2 GiB. */
 int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb,
                      void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
                      void* stream);

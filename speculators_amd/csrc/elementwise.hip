@@ -145,14 +145,21 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(
   }
 }
 
-// dw[c] = sum_s dw_part[s, c]  (fixed order: deterministic), bf16 out
+// dw[c] = sum_s dw_part[s, c]  (fixed order: deterministic), bf16 out.  One workgroup
+// sums 64 columns: wave w adds the slots w, w+4, ..., then the four partial sums are
+// combined through LDS.
 __global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ part, int64_t slots,
                                                      int H, uint16_t* __restrict__ out) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= H) return;
+  __shared__ float red[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
   float s = 0.f;
-  for (int64_t i = 0; i < slots; ++i) s += part[i * H + c];
-  out[c] = (uint16_t)f32_to_bf16_bits(s);
+  if (c < H)
+    for (int64_t i = wave; i < slots; i += 4) s += part[i * H + c];
+  red[wave][lane] = s;
+  __syncthreads();
+  if (wave == 0 && c < H)
+    out[c] = (uint16_t)f32_to_bf16_bits((red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]));
 }
 
 // ---------------------------------------------------------------- RoPE + relayout
@@ -246,8 +253,8 @@ static bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) =
 using namespace spx;
 
 extern "C" int64_t spx_rmsnorm_bwd_slots(int64_t rows, int64_t H) {
-  if (H <= 512) return 4 * (rows < 4096 ? (rows + 3) / 4 : 1024);
-  return rows < 1024 ? rows : 1024;
+  if (H <= 512) return 4 * (rows < 1024 ? (rows + 3) / 4 : 256);
+  return rows < 256 ? rows : 256;
 }
 
 extern "C" int spx_rmsnorm_fwd(const void* x, int64_t ld_x, const void* weight, void* y, int64_t ld_y,
@@ -302,7 +309,7 @@ extern "C" int spx_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weight, 
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<8, false>), dim3((unsigned)slots), dim3(256), 0, st, xp, ld_x, wp,
                        dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H);
   if (dweight)
-    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((H + 255) / 256)), dim3(256), 0, st, part, slots, (int)H,
+    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((H + 63) / 64)), dim3(256), 0, st, part, slots, (int)H,
                        reinterpret_cast<uint16_t*>(dweight));
   return check_launch(__func__);
 }

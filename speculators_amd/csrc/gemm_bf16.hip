@@ -5,13 +5,16 @@
 // and walks K in steps of 64; each wave owns a 64 x 128 patch as 2 x 4
 // accumulators of v_mfma_f32_32x32x16_bf16, two waves per SIMD so one wave's
 // LDS reads overlap the other's MFMAs.  A and B tiles are staged global ->
-// registers -> LDS through two LDS stages (the next tile is written while the
+// registers -> LDS (buffer loads: rows past the edge read as zero, no per-lane
+// predicates) through two LDS stages (the next tile is written while the
 // current one is read: one barrier per K step) with the next tile's global
 // loads in flight during the current tile's MFMAs.  LDS rows are padded by 16
 // bytes so the 16-byte operand reads of consecutive lanes hit distinct bank
 // groups (measured: zero bank conflicts).  Workgroup ids are remapped so that
 // each XCD (ids are dealt round-robin over the 8 XCDs) works on a compact
 // band of tiles and shares its A / B panels in that XCD's L2.
+
+#include <type_traits>
 
 #include "spx_common.h"
 #include "../../include/spx.h"
@@ -24,7 +27,11 @@ namespace spx {
 #ifndef SPX_GEMM_WN
 #define SPX_GEMM_WN 2
 #endif
+#ifndef SPX_GEMM_PGR
+#define SPX_GEMM_PGR 1
+#endif
 constexpr int kWM = SPX_GEMM_WM, kWN = SPX_GEMM_WN;  // waves along M / N of the tile
+constexpr int kPGR = SPX_GEMM_PGR;  // K tiles whose global loads are in flight ahead of the MFMAs
 constexpr int kGemmThreads = 64 * kWM * kWN;
 constexpr int kTM = 256, kTN = 256, kTK = 64;
 constexpr int kMI = kTM / kWM / 32, kNI = kTN / kWN / 32;  // 32x32 accumulators per wave
@@ -70,37 +77,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_nt_kernel(
   constexpr int kRowsPerPass = kGemmThreads / 8;
   constexpr int kPasses = kTM / kRowsPerPass;
   const int lrow = tid >> 3, lcol = (tid & 7) * 8;
-  u32x4 areg[kPasses], breg[kPasses];
-  // row pointers are fixed for the whole K walk (rows past the edge are clamped: their
-  // products land in accumulators that are never stored)
-  const uint16_t* aptr[kPasses];
-  const uint16_t* bptr[kPasses];
-#pragma unroll
-  for (int n = 0; n < kPasses; ++n) {
-    const int r = lrow + kRowsPerPass * n;
-    aptr[n] = A + (int64_t)min(m0 + r, M - 1) * lda + lcol;
-    bptr[n] = B + (int64_t)min(n0 + r, N - 1) * ldb + lcol;
-  }
-  auto fetch = [&](int k0) {
-    const bool kin = k0 + lcol < K;
-    const u32x4 z = {0, 0, 0, 0};
-#pragma unroll
-    for (int n = 0; n < kPasses; ++n) {
-      areg[n] = kin ? *reinterpret_cast<const u32x4*>(aptr[n] + k0) : z;
-      breg[n] = kin ? *reinterpret_cast<const u32x4*>(bptr[n] + k0) : z;
-    }
-  };
-  auto stash = [&](int stage) {
-    uint16_t* As = smem + stage * kStageElems;
-    uint16_t* Bs = As + kTM * kLdsStride;
-#pragma unroll
-    for (int n = 0; n < kPasses; ++n) {
-      const int r = lrow + kRowsPerPass * n;
-      *reinterpret_cast<u32x4*>(&As[r * kLdsStride + lcol]) = areg[n];
-      *reinterpret_cast<u32x4*>(&Bs[r * kLdsStride + lcol]) = breg[n];
-    }
-  };
-
+  u32x4 areg[kPGR][kPasses], breg[kPGR][kPasses];
   f32x16 acc[kMI][kNI];
 #pragma unroll
   for (int i = 0; i < kMI; ++i)
@@ -109,18 +86,52 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_nt_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // two LDS stages: the next tile is written while the current one is read, one
-  // barrier per K step
-  fetch(0);
-  stash(0);
-  __syncthreads();
-  int stage = 0;
-  for (int k0 = 0; k0 < K; k0 += kTK) {
-    const bool more = k0 + kTK < K;
-    if (more) fetch(k0 + kTK);
+  // buffer loads: one resource per operand, a fixed 32-bit byte offset per staged row and
+  // the K position in the scalar offset.  Rows past the matrix edge fall outside the
+  // resource and read as zero, so no clamping or per-lane predicate is needed.
+  const __amdgpu_buffer_rsrc_t ares = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(A), 0, (int)((((int64_t)M - 1) * lda + K) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t bres = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(B), 0, (int)((((int64_t)N - 1) * ldb + K) * 2), 0x00020000);
+  int aoff[kPasses], boff[kPasses];
+#pragma unroll
+  for (int n = 0; n < kPasses; ++n) {
+    const int r = lrow + kRowsPerPass * n;
+    // a row index past the edge is moved far outside the resource (the plain product
+    // row * ld could wrap around 2^32 for huge strides)
+    aoff[n] = (m0 + r < M) ? (int)((((int64_t)(m0 + r)) * lda + lcol) * 2) : 0x7ffffff0;
+    boff[n] = (n0 + r < N) ? (int)((((int64_t)(n0 + r)) * ldb + lcol) * 2) : 0x7ffffff0;
+  }
+  const bool ktail = (K % kTK) != 0;
+#define SPX_FETCH(k0v, S)                                                              \
+  do {                                                                                 \
+    const int k0_ = (k0v);                                                             \
+    _Pragma("unroll") for (int n = 0; n < kPasses; ++n) {                              \
+      areg[S][n] = __builtin_amdgcn_raw_buffer_load_b128(ares, aoff[n], k0_ * 2, 0);   \
+      breg[S][n] = __builtin_amdgcn_raw_buffer_load_b128(bres, boff[n], k0_ * 2, 0);   \
+    }                                                                                  \
+    if (ktail && k0_ + lcol >= K) {                                                    \
+      const u32x4 z = {0, 0, 0, 0};                                                    \
+      _Pragma("unroll") for (int n = 0; n < kPasses; ++n) { areg[S][n] = z; breg[S][n] = z; } \
+    }                                                                                  \
+  } while (0)
+#define SPX_STASH(stagev, S)                                                           \
+  do {                                                                                 \
+    uint16_t* As_ = smem + (stagev) * kStageElems;                                     \
+    uint16_t* Bs_ = As_ + kTM * kLdsStride;                                            \
+    _Pragma("unroll") for (int n = 0; n < kPasses; ++n) {                              \
+      const int r = lrow + kRowsPerPass * n;                                           \
+      *reinterpret_cast<u32x4*>(&As_[r * kLdsStride + lcol]) = areg[S][n];             \
+      *reinterpret_cast<u32x4*>(&Bs_[r * kLdsStride + lcol]) = breg[S][n];             \
+    }                                                                                  \
+  } while (0)
+  auto compute = [&](int stage) {
     const uint16_t* As = smem + stage * kStageElems;
     const uint16_t* Bs = As + kTM * kLdsStride;
-#pragma unroll
+#ifndef SPX_GEMM_KKUNROLL
+#define SPX_GEMM_KKUNROLL 4
+#endif
+#pragma unroll SPX_GEMM_KKUNROLL
     for (int kk = 0; kk < kTK / 16; ++kk) {
       bf16x8 af[kMI], bf[kNI];
 #pragma unroll
@@ -133,10 +144,49 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_nt_kernel(
         for (int j = 0; j < kNI; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
     }
-    if (more) stash(stage ^ 1);
+  };
+  constexpr int S1 = kPGR - 1;
+  // two LDS stages: the next tile is written while the current one is read, one
+  // barrier per K step.  kPGR = 2 keeps the global loads of TWO tiles in flight (in two
+  // register sets) so that a tile's load latency is covered by two K steps of MFMAs.
+  if (kPGR == 1) {
+    SPX_FETCH(0, 0);
+    SPX_STASH(0, 0);
     __syncthreads();
-    stage ^= 1;
+    int stage = 0;
+    for (int k0 = 0; k0 < K; k0 += kTK) {
+      const bool more = k0 + kTK < K;
+      if (more) SPX_FETCH(k0 + kTK, 0);
+      compute(stage);
+      if (more) SPX_STASH(stage ^ 1, 0);
+      __syncthreads();
+      stage ^= 1;
+    }
+  } else {
+    SPX_FETCH(0, 0);
+    if (kTK < K) SPX_FETCH(kTK, S1);
+    SPX_STASH(0, 0);
+    __syncthreads();
+    int stage = 0;
+    for (int k0 = 0; k0 < K; k0 += kTK) {
+      // tile k0 sits in LDS stage `stage`; the register set of the other parity holds
+      // tile k0 + 1, this parity's set is free for tile k0 + 2
+      const bool more1 = k0 + kTK < K, more2 = k0 + 2 * kTK < K;
+      if (more2) {
+        if (stage == 0) SPX_FETCH(k0 + 2 * kTK, 0);
+        else SPX_FETCH(k0 + 2 * kTK, S1);
+      }
+      compute(stage);
+      if (more1) {
+        if (stage == 0) SPX_STASH(1, S1);
+        else SPX_STASH(0, 0);
+      }
+      __syncthreads();
+      stage ^= 1;
+    }
   }
+#undef SPX_FETCH
+#undef SPX_STASH
 
   // accumulator (i, j): lane column = n, register r = row 8*(r/4) + 4*g + r%4
 #pragma unroll
@@ -165,6 +215,8 @@ extern "C" int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64
   SPX_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0, "K, lda, ldb must be multiples of 8");
   SPX_REQUIRE(lda >= K && ldb >= K && ldc >= N, "leading dimension too small");
   SPX_REQUIRE(((uintptr_t)a | (uintptr_t)b) % 16 == 0, "a and b must be 16-byte aligned");
+  SPX_REQUIRE(((M - 1) * lda + K) * 2 < 0x7ffffff0ll && ((N - 1) * ldb + K) * 2 < 0x7ffffff0ll,
+              "each operand must span less than 2 GiB (32-bit buffer offsets)");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   static bool attr_set = false;
   if (!attr_set) {
