@@ -145,10 +145,18 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
     def loss_fwd():
         _lib.call("spx_fused_vocab_loss_fwd", L.OP_KL, _lib.ptr(lg), vd, _lib.ptr(tg), vd, t, vd, 0,
                   _lib.ptr(stats[0]), _lib.ptr(stats[1]), _lib.ptr(stats[2]), _lib.ptr(stats[3]),
-                  _lib.ptr(arg[0]), _lib.ptr(arg[1]), st)
+                  _lib.ptr(arg[0]), _lib.ptr(arg[1]), 0, st)
+
+    def loss_fwd_reuse():  # steps >= 1: the target rows' statistics come from step 0
+        _lib.call("spx_fused_vocab_loss_fwd", L.OP_KL, _lib.ptr(lg), vd, _lib.ptr(tg), vd, t, vd, 0,
+                  _lib.ptr(stats[0]), _lib.ptr(stats[1]), _lib.ptr(stats[2]), _lib.ptr(stats[3]),
+                  _lib.ptr(arg[0]), _lib.ptr(arg[1]), 1, st)
 
     ms = time_events(torch, loss_fwd, 20)
-    hbm("loss_fwd_kernel[KL, T rows x Vd]", 2.0 * t * vd * 2, ms, k_steps)
+    hbm("loss_fwd_kernel[KL, T rows x Vd, step 0]", 2.0 * t * vd * 2, ms, 1)
+    ms = time_events(torch, loss_fwd_reuse, 20)
+    hbm("loss_fwd_kernel[KL, T rows x Vd, steps >= 1 (target statistics reused)]", 2.0 * t * vd * 2,
+        ms, k_steps - 1)
     rg = torch.full((t,), 1.0 / t, device=device)
     grad = torch.empty(t, vd, device=device, dtype=torch.bfloat16)
 

@@ -66,13 +66,19 @@ int spx_vocab_gather(const void* full, int64_t ld_full, const int64_t* d2t,
  * models/dflash/metrics.py:77-78).  Row r of `logits` is paired with row r of
  * `targets`; the TTT shift of align_for_step (models/eagle3/metrics.py:16-48)
  * is a pointer offset made by the caller.  ld_* are row strides in elements.
- * The argmax outputs may be NULL. */
+ * The argmax outputs may be NULL.
+ * reuse_target_stats != 0 (kl and ce only; ignored for the others): lse_target
+ * and argmax_target are INPUTS holding the statistics of the same target rows
+ * from an earlier call -- the verifier row is the same at every TTT step, only
+ * shifted -- so the target max / sum / arg-max are not recomputed, and ce does
+ * not read the target rows at all. */
 int spx_fused_vocab_loss_fwd(int op, const void* logits, int64_t ld_logits,
                              const void* targets, int64_t ld_targets,
                              int64_t rows, int64_t vocab, int dtype,
                              float* loss, float* lse_draft, float* lse_target,
                              float* extra, int32_t* argmax_draft,
-                             int32_t* argmax_target, void* stream);
+                             int32_t* argmax_target, int reuse_target_stats,
+                             void* stream);
 
 /* grad_logits[r, :] = g_r * dL_r/dlogits, g_r = row_grad[r] * (*scale)
  * (scale may be NULL = 1).  Rows with g_r == 0 are written as exact zeros

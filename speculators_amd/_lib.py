@@ -22,7 +22,8 @@ _I32 = c_int32
 # name -> argument types (return type int unless listed in RESTYPES); mirrors include/spx.h
 SIGNATURES: dict[str, list] = {
     "spx_vocab_gather": [_P, _I64, _P, _P, _I64, _I64, _I64, _I64, _I, _P],
-    "spx_fused_vocab_loss_fwd": [_I, _P, _I64, _P, _I64, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P],
+    "spx_fused_vocab_loss_fwd": [_I, _P, _I64, _P, _I64, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _I,
+                                 _P],
     "spx_fused_vocab_loss_bwd": [_I, _P, _I64, _P, _I64, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P,
                                  _I64, _P],
     "spx_ttt_step_reduce": [_P, _P, _P, _P, _I, _P, _I, _I64, _F, _P, _P, _P],

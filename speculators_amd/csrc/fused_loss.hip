@@ -130,7 +130,10 @@ __device__ __forceinline__ float log_mix(float la, float lb) {
 }
 
 // ---- forward ---------------------------------------------------------------
-template <typename T, int OP, bool VEC>
+// KNOWN: lse_target / argmax_target are INPUTS (the target row's statistics from an
+// earlier pass over the same row); the target max / sum / arg-max tracking is skipped and
+// the cross-entropy reduction does not read the target row at all.
+template <typename T, int OP, bool VEC, bool KNOWN>
 __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
     const T* __restrict__ logits, int64_t ld_logits, const T* __restrict__ targets,
     int64_t ld_targets, int64_t vocab, float* __restrict__ loss, float* __restrict__ lse_draft,
@@ -142,6 +145,8 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
   const int tid = threadIdx.x;
   const int64_t nchunks = (vocab + 7) >> 3;
 
+  const float lt2_known = KNOWN ? lse_target[r] * kLog2e : 0.f;  // base-2 target lse
+  const bool read_y = !(KNOWN && OP == SPX_LOSS_CE);
   RowStats s;
   s.md = kNegBig; s.zd = 0.f; s.mt = kNegBig; s.zt = 0.f; s.at = 0.f;
   s.bd = -INFINITY; s.id = 0x7fffffff; s.bt = -INFINITY; s.it = 0x7fffffff; s.xt = 0.f;
@@ -150,17 +155,21 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
     const int64_t base = c << 3;
     float x[8], y[8];
     load8<T, VEC>(xrow, base, vocab, x);
-    load8<T, VEC>(yrow, base, vocab, y);
+    if (read_y) load8<T, VEC>(yrow, base, vocab, y);
     float cx = x[0], cy = y[0];
 #pragma unroll
-    for (int i = 1; i < 8; ++i) { cx = fmaxf(cx, x[i]); cy = fmaxf(cy, y[i]); }
+    for (int i = 1; i < 8; ++i) cx = fmaxf(cx, x[i]);
+    if (!KNOWN) {
+#pragma unroll
+      for (int i = 1; i < 8; ++i) cy = fmaxf(cy, y[i]);
+    }
     if (cx > s.bd) {  // strict: an earlier chunk of this thread keeps a tie
       int k = 7;
 #pragma unroll
       for (int i = 6; i >= 0; --i) k = (x[i] == cx) ? i : k;
       s.bd = cx; s.id = (int)base + k;
     }
-    if (cy > s.bt) {
+    if (!KNOWN && cy > s.bt) {
       int k = 7;
       float xv = x[7];
 #pragma unroll
@@ -172,13 +181,25 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
       s.bt = cy; s.it = (int)base + k; s.xt = xv;
     }
     {
-      float mn = fmaxf(s.md, cx * kLog2e);
-      float z = s.zd * fast_exp2(s.md - mn);
+      const float cxs = cx * kLog2e;
+      float mn = s.md, z = s.zd;
+      if (cxs > mn) {  // the running max moves rarely once a few chunks have been seen
+        z *= fast_exp2(mn - cxs);
+        mn = cxs;
+      }
 #pragma unroll
       for (int i = 0; i < 8; ++i) z += fast_exp2(fmaf(x[i], kLog2e, -mn));
       s.zd = z; s.md = mn;
     }
-    if (OP != SPX_LOSS_CE) {
+    if (KNOWN && OP != SPX_LOSS_CE) {
+      float a = s.at;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float pr = fast_exp2(fmaf(y[i], kLog2e, -lt2_known));  // the target probability
+        a = fmaf(pr, y[i] - x[i], a);
+      }
+      s.at = a;
+    } else if (OP != SPX_LOSS_CE) {
       float mn = fmaxf(s.mt, cy * kLog2e);
       float rs = fast_exp2(s.mt - mn);
       float z = s.zt * rs, a = s.at * rs;
@@ -207,11 +228,16 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
   for (int w = 1; w < kLossWaves; ++w) merge(s, part[w]);
 
   const float lse_d = (s.md + fast_log2(s.zd)) * kLn2;
-  const float lse_t = (OP != SPX_LOSS_CE) ? (s.mt + fast_log2(s.zt)) * kLn2 : 0.f;
+  const float lse_t = KNOWN ? lse_target[r]
+                            : ((OP != SPX_LOSS_CE) ? (s.mt + fast_log2(s.zt)) * kLn2 : 0.f);
+  if (KNOWN) {
+    s.it = argmax_target ? argmax_target[r] : 0;
+    if (OP == SPX_LOSS_CE) s.xt = load1(xrow + s.it);
+  }
 
   float row_loss = 0.f, row_extra = 0.f;
   if (OP == SPX_LOSS_KL) {
-    row_loss = s.at / s.zt - lse_t + lse_d;
+    row_loss = (KNOWN ? s.at : s.at / s.zt) - lse_t + lse_d;
     row_extra = row_loss;
   } else if (OP == SPX_LOSS_CE) {
     row_loss = lse_d - s.xt;
@@ -248,10 +274,12 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
   if (tid == 0) {
     loss[r] = row_loss;
     lse_draft[r] = lse_d;
-    lse_target[r] = lse_t;
     extra[r] = row_extra;
     if (argmax_draft) argmax_draft[r] = s.id;
-    if (argmax_target) argmax_target[r] = s.it;
+    if (!KNOWN) {
+      lse_target[r] = lse_t;
+      if (argmax_target) argmax_target[r] = s.it;
+    }
   }
 }
 
@@ -450,15 +478,15 @@ __global__ __launch_bounds__(kReduceThreads) void block_reduce_kernel(
 // ---- dispatch ----------------------------------------------------------------
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-template <typename T, bool VEC>
+template <typename T, bool VEC, bool KNOWN>
 static void launch_fwd(int op, const T* lg, int64_t ldl, const T* tg, int64_t ldt, int64_t rows,
                        int64_t vocab, float* loss, float* lsd, float* lst, float* ex, int32_t* ad,
                        int32_t* at, hipStream_t st) {
   dim3 grid((unsigned)rows), block(kLossThreads);
-#define SPX_FWD(OPV)                                                                         \
-  case OPV:                                                                                  \
-    hipLaunchKernelGGL((loss_fwd_kernel<T, OPV, VEC>), grid, block, 0, st, lg, ldl, tg, ldt, \
-                       vocab, loss, lsd, lst, ex, ad, at);                                   \
+#define SPX_FWD(OPV)                                                                                \
+  case OPV:                                                                                         \
+    hipLaunchKernelGGL((loss_fwd_kernel<T, OPV, VEC, KNOWN>), grid, block, 0, st, lg, ldl, tg, ldt, \
+                       vocab, loss, lsd, lst, ex, ad, at);                                          \
     break;
   switch (op) {
     SPX_FWD(SPX_LOSS_KL) SPX_FWD(SPX_LOSS_RKL) SPX_FWD(SPX_LOSS_JSD) SPX_FWD(SPX_LOSS_CE)
@@ -493,7 +521,8 @@ extern "C" int spx_fused_vocab_loss_fwd(int op, const void* logits, int64_t ld_l
                                         const void* targets, int64_t ld_targets, int64_t rows,
                                         int64_t vocab, int dtype, float* loss, float* lse_draft,
                                         float* lse_target, float* extra, int32_t* argmax_draft,
-                                        int32_t* argmax_target, void* stream) {
+                                        int32_t* argmax_target, int reuse_target_stats,
+                                        void* stream) {
   SPX_REQUIRE(op >= SPX_LOSS_KL && op <= SPX_LOSS_TV, "unknown loss op");
   SPX_REQUIRE(dtype == SPX_DTYPE_BF16 || dtype == SPX_DTYPE_F32, "dtype must be bf16 or f32");
   SPX_REQUIRE(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "rows >= 0 and 0 < vocab < 2^31");
@@ -501,21 +530,25 @@ extern "C" int spx_fused_vocab_loss_fwd(int op, const void* logits, int64_t ld_l
   SPX_REQUIRE(rows < (1ll << 31), "too many rows");
   if (rows == 0) return SPX_OK;
   SPX_REQUIRE(logits && targets && loss && lse_draft && lse_target && extra, "null buffer");
+  // the second-pass reductions (rkl, jsd, tv) recompute from both rows anyway
+  const bool known = reuse_target_stats && (op == SPX_LOSS_KL || op == SPX_LOSS_CE);
+  if (known && op == SPX_LOSS_CE) SPX_REQUIRE(argmax_target, "ce with reused statistics needs argmax_target");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const int64_t per16 = dtype == SPX_DTYPE_BF16 ? 8 : 4;
   const bool vec = aligned16(logits) && aligned16(targets) && ld_logits % per16 == 0 &&
                    ld_targets % per16 == 0;
+#define SPX_GO(TT, VV, KK)                                                                       \
+  launch_fwd<TT, VV, KK>(op, reinterpret_cast<const TT*>(logits), ld_logits,                     \
+                         reinterpret_cast<const TT*>(targets), ld_targets, rows, vocab, loss,    \
+                         lse_draft, lse_target, extra, argmax_draft, argmax_target, st)
   if (dtype == SPX_DTYPE_BF16) {
-    auto lg = reinterpret_cast<const uint16_t*>(logits);
-    auto tg = reinterpret_cast<const uint16_t*>(targets);
-    if (vec) launch_fwd<uint16_t, true>(op, lg, ld_logits, tg, ld_targets, rows, vocab, loss, lse_draft, lse_target, extra, argmax_draft, argmax_target, st);
-    else launch_fwd<uint16_t, false>(op, lg, ld_logits, tg, ld_targets, rows, vocab, loss, lse_draft, lse_target, extra, argmax_draft, argmax_target, st);
+    if (vec) { if (known) SPX_GO(uint16_t, true, true); else SPX_GO(uint16_t, true, false); }
+    else { if (known) SPX_GO(uint16_t, false, true); else SPX_GO(uint16_t, false, false); }
   } else {
-    auto lg = reinterpret_cast<const float*>(logits);
-    auto tg = reinterpret_cast<const float*>(targets);
-    if (vec) launch_fwd<float, true>(op, lg, ld_logits, tg, ld_targets, rows, vocab, loss, lse_draft, lse_target, extra, argmax_draft, argmax_target, st);
-    else launch_fwd<float, false>(op, lg, ld_logits, tg, ld_targets, rows, vocab, loss, lse_draft, lse_target, extra, argmax_draft, argmax_target, st);
+    if (vec) { if (known) SPX_GO(float, true, true); else SPX_GO(float, true, false); }
+    else { if (known) SPX_GO(float, false, true); else SPX_GO(float, false, false); }
   }
+#undef SPX_GO
   return check_launch(__func__);
 }
 

@@ -254,6 +254,7 @@ class Eagle3DraftModel(nn.Module):
             metrics: dict = {}
 
         caches = [dict() for _ in self.layers]
+        stats_cache: dict = {}
         inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device)
         position_ids = position_ids.reshape(-1).to(torch.int64).contiguous()
         draft_tokens = []
@@ -272,12 +273,19 @@ class Eagle3DraftModel(nn.Module):
                 logits = self._linear(self.norm(y), self.lm_head.weight, frozen=True)
 
             if return_loss:
-                s_loss, s_metrics = MT.compute_metrics(
+                s_loss, s_metrics, pred = MT.compute_metrics(
                     logits, targets, loss_mask, prev_correct, step, ttt_step_loss_decay,
-                    loss_config=loss_config)
+                    loss_config=loss_config, target_stats_cache=stats_cache, return_pred=True)
                 loss = loss + s_loss
                 metrics.update(s_metrics)
-            draft_tokens.append(MT.argmax_rows(logits.detach()))
+                # draft tokens: the loss kernel's arg-max for the aligned rows, plus the
+                # last `step` rows (which have no target) on their own
+                pred = pred.to(torch.int64)
+                if step:
+                    pred = torch.cat([pred, MT.argmax_rows(logits.detach()[0, t - step:])])
+                draft_tokens.append(pred.view(1, t))
+            else:
+                draft_tokens.append(MT.argmax_rows(logits.detach()))
 
             input_ids = torch.cat(
                 [original_ids[:, 1 + step:], original_ids.new_zeros(1, 1 + step)], dim=-1)

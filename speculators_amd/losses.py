@@ -36,9 +36,13 @@ def _rows_2d(t: torch.Tensor) -> torch.Tensor:
         return t.reshape(-1, v)
 
 
-def fused_loss_forward(op: int, logits: torch.Tensor, targets: torch.Tensor):
+def fused_loss_forward(op: int, logits: torch.Tensor, targets: torch.Tensor, target_stats=None):
     """Run the forward kernel.  Returns (loss [R] f32, lse_d, lse_t, extra,
-    argmax_draft [R] i32, argmax_target [R] i32, logits2d, targets2d)."""
+    argmax_draft [R] i32, argmax_target [R] i32, logits2d, targets2d).
+
+    ``target_stats = (lse_target [R] f32, argmax_target [R] i32)`` from an earlier call on
+    the same target rows lets kl / ce skip the target row statistics (ce then does not
+    read the targets at all)."""
     if logits.shape != targets.shape:
         raise ValueError(f"logits {tuple(logits.shape)} and targets {tuple(targets.shape)} differ")
     if logits.dtype != targets.dtype:
@@ -46,35 +50,43 @@ def fused_loss_forward(op: int, logits: torch.Tensor, targets: torch.Tensor):
     x, y = _rows_2d(logits), _rows_2d(targets)
     rows, vocab = x.shape
     dev = x.device
+    reuse = target_stats is not None and op in (OP_KL, OP_CE)
     stats = torch.empty(4, rows, device=dev, dtype=torch.float32)
     arg = torch.empty(2, rows, device=dev, dtype=torch.int32)
+    lse_t, am_t = stats[2], arg[1]
+    if reuse:
+        lse_t = target_stats[0].reshape(-1)
+        am_t = target_stats[1].reshape(-1)
+        if lse_t.numel() != rows or am_t.numel() != rows or lse_t.stride(0) != 1 or am_t.stride(0) != 1:
+            raise ValueError("target_stats must be contiguous [rows] tensors")
     _lib.call(
         "spx_fused_vocab_loss_fwd", op, _lib.ptr(x), x.stride(0), _lib.ptr(y), y.stride(0),
         rows, vocab, _lib.dtype_code(x), _lib.ptr(stats[0]), _lib.ptr(stats[1]),
-        _lib.ptr(stats[2]), _lib.ptr(stats[3]), _lib.ptr(arg[0]), _lib.ptr(arg[1]),
+        _lib.ptr(lse_t), _lib.ptr(stats[3]), _lib.ptr(arg[0]), _lib.ptr(am_t), int(reuse),
         _lib.stream_ptr(dev),
     )
-    return stats[0], stats[1], stats[2], stats[3], arg[0], arg[1], x, y
+    return stats[0], stats[1], lse_t, stats[3], arg[0], am_t, x, y
 
 
 class _FusedLoss(torch.autograd.Function):
-    """``(logits, targets, op) -> (row_loss [B, T] f32, argmax_draft, argmax_target)``;
-    the autograd counterpart of ``_FusedLoss`` in losses/fused.py:238-291.  Targets
-    get no gradient."""
+    """``(logits, targets, op[, lse_t, am_t]) -> (row_loss [B, T] f32, argmax_draft,
+    argmax_target, lse_target)``; the autograd counterpart of ``_FusedLoss`` in
+    losses/fused.py:238-291.  Targets get no gradient."""
 
     @staticmethod
-    def forward(ctx, logits, targets, op):
-        loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, logits, targets)
+    def forward(ctx, logits, targets, op, known_lse_t=None, known_am_t=None):
+        known = (known_lse_t, known_am_t) if known_lse_t is not None else None
+        loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, logits, targets, known)
         ctx.save_for_backward(x, None if op == OP_CE else y, lse_d, lse_t, extra, am_t)
         ctx.op = op
         ctx.shape = logits.shape
         lead = logits.shape[:-1]
-        am_d, am_t = am_d.view(lead), am_t.view(lead)
-        ctx.mark_non_differentiable(am_d, am_t)
-        return loss.view(lead), am_d, am_t
+        am_d, am_t, lse_t = am_d.view(lead), am_t.view(lead), lse_t.view(lead)
+        ctx.mark_non_differentiable(am_d, am_t, lse_t)
+        return loss.view(lead), am_d, am_t, lse_t
 
     @staticmethod
-    def backward(ctx, grad_rows, _gd, _gt):
+    def backward(ctx, grad_rows, _gd, _gt, _gl):
         x, y, lse_d, lse_t, extra, am_t = ctx.saved_tensors
         rows, vocab = x.shape
         g = grad_rows.reshape(-1).to(torch.float32).contiguous()
@@ -85,12 +97,14 @@ class _FusedLoss(torch.autograd.Function):
             _lib.ptr(lse_d), _lib.ptr(lse_t), _lib.ptr(extra), _lib.ptr(am_t), _lib.ptr(g), None,
             _lib.ptr(grad), grad.stride(0), _lib.stream_ptr(x.device),
         )
-        return grad.view(ctx.shape), None, None
+        return grad.view(ctx.shape), None, None, None, None
 
 
-def fused_rows(op: int, logits, targets):
-    """(row_loss, argmax_draft, argmax_target) of one primitive reduction."""
-    return _FusedLoss.apply(logits, targets, op)
+def fused_rows(op: int, logits, targets, target_stats=None):
+    """(row_loss, argmax_draft, argmax_target, lse_target) of one primitive reduction."""
+    if target_stats is None:
+        return _FusedLoss.apply(logits, targets, op)
+    return _FusedLoss.apply(logits, targets, op, target_stats[0], target_stats[1])
 
 
 def kl_div_loss(logits, targets):

@@ -62,11 +62,18 @@ def _step_views(logits, targets, loss_mask, prev_correct, ttt_step):
 
 
 def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
-                    ttt_step_loss_decay: float, loss_config: L.LossConfig | None = None):
+                    ttt_step_loss_decay: float, loss_config: L.LossConfig | None = None,
+                    target_stats_cache: dict | None = None, return_pred: bool = False):
     """EAGLE3 per-step loss + metrics; same contract as models/eagle3/metrics.py:51-119.
 
     ``prev_correct`` (any mask dtype) is updated in place.  Returns
     ``(loss 0-d, metrics dict of 0-d tensors)``.
+
+    Two optional extras beyond the reference contract: ``target_stats_cache`` (a dict the
+    caller keeps across the TTT steps of ONE forward) lets steps >= 1 reuse the verifier
+    rows' log-sum-exp / arg-max computed at step 0 (``targets`` is the same tensor at every
+    step, only shifted); ``return_pred=True`` also returns the draft arg-max of the aligned
+    rows (int32 ``[T - ttt_step]``).
     """
     if logits.shape[0] != 1:
         raise ValueError("the packed batch layout has batch size 1 (train/data.py:306-393)")
@@ -94,10 +101,23 @@ def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
         out = torch.empty(6, device=dev, dtype=torch.float32)
         op = L.PRIMITIVE_OP.get(name)
         if fn is L._HIP_LOSS_FN_MAP.get(name) and op is not None:
-            rows, am_d, am_t = L.fused_rows(op, s_logits, s_targets)
+            known = None
+            if target_stats_cache is not None and op in (L.OP_KL, L.OP_CE):
+                full = target_stats_cache.get("kl" if op == L.OP_KL else "ce")
+                if full is None and op == L.OP_CE:
+                    full = target_stats_cache.get("kl")  # the arg-max is all ce needs
+                if full is not None:
+                    known = (full[0][ttt_step:], full[1][ttt_step:])
+            rows, am_d, am_t, lse_t = L.fused_rows(op, s_logits, s_targets, known)
+            if (target_stats_cache is not None and known is None and ttt_step == 0
+                    and op in (L.OP_KL, L.OP_CE)):
+                target_stats_cache["kl" if op == L.OP_KL else "ce"] = (
+                    lse_t.reshape(-1), am_t.reshape(-1))
         else:
             rows = fn(s_logits, s_targets)
-            _, am_d, am_t = L.fused_rows(L.OP_CE, s_logits.detach(), s_targets)
+            _, am_d, am_t, _ = L.fused_rows(L.OP_CE, s_logits.detach(), s_targets)
+        if ti == 0:
+            pred = am_d.reshape(-1)
         # only the first term advances the acceptance chain
         term = _StepReduce.apply(rows.reshape(-1), am_d.reshape(-1), am_t.reshape(-1), mask1,
                                  prev1 if ti == 0 else None, weight, out)
@@ -116,6 +136,8 @@ def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
     m[f"full_acc_{ttt_step}_total"] = first_out[2]
     m[f"cond_acc_{ttt_step}_sum"] = first_out[3]
     m[f"cond_acc_{ttt_step}_total"] = first_out[4]
+    if return_pred:
+        return total, m, pred
     return total, m
 
 
@@ -132,7 +154,7 @@ def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
             "spx_fused_vocab_loss_fwd", L.OP_CE, _lib.ptr(x), x.stride(0), _lib.ptr(x),
             x.stride(0), rows, vocab, _lib.dtype_code(x), _lib.ptr(scratch[0]),
             _lib.ptr(scratch[1]), _lib.ptr(scratch[2]), _lib.ptr(scratch[3]), _lib.ptr(out),
-            None, _lib.stream_ptr(dev),
+            None, 0, _lib.stream_ptr(dev),
         )
     return out[:rows].to(torch.int64).view(logits.shape[:-1])
 
@@ -201,10 +223,10 @@ def dflash_compute_metrics(logits, targets, loss_mask, block_size: int = 1, gamm
     for ti, (name, (fn, w)) in enumerate(loss_config.items()):
         op = L.PRIMITIVE_OP.get(name)
         if fn is L._HIP_LOSS_FN_MAP.get(name) and op is not None:
-            rows, am_d, am_t = L.fused_rows(op, logits, targets)
+            rows, am_d, am_t, _ = L.fused_rows(op, logits, targets)
         else:
             rows = fn(logits, targets)
-            _, am_d, am_t = L.fused_rows(L.OP_CE, logits.detach(), targets)
+            _, am_d, am_t, _ = L.fused_rows(L.OP_CE, logits.detach(), targets)
         if per_position_loss_weight == "dpace":
             masked = rows.detach().reshape(-1) * mask1.to(torch.float32)
             pw = dpace_loss_decay(masked, mask1, block_size, dpace_alpha)

@@ -70,7 +70,7 @@ def test_ragged_vocab_and_unaligned_rows(vocab, dtype):
     g = torch.Generator().manual_seed(vocab)
     a = (torch.randn(1, 5, vocab, generator=g) * 2).to(dtype)
     b = (torch.randn(1, 5, vocab, generator=g) * 2).to(dtype)
-    rows, am_d, am_t = L.fused_rows(L.OP_KL, a.cuda(), b.cuda())
+    rows, am_d, am_t, _ = L.fused_rows(L.OP_KL, a.cuda(), b.cuda())
     torch.testing.assert_close(rows.cpu(), OL.kl_div(a, b), **LOSS_TOL)
     assert torch.equal(am_d.cpu().long(), a.float().argmax(-1))
     assert torch.equal(am_t.cpu().long(), b.float().argmax(-1))
@@ -84,7 +84,7 @@ def test_argmax_first_index_on_ties_bit_exact():
     # coarse bf16 values: many exact ties per row
     a = (torch.randint(-4, 5, (1, 257, 32000), generator=g).float() * 0.5).bfloat16()
     b = (torch.randint(-4, 5, (1, 257, 32000), generator=g).float() * 0.5).bfloat16()
-    _, am_d, am_t = L.fused_rows(L.OP_KL, a.cuda(), b.cuda())
+    _, am_d, am_t, _ = L.fused_rows(L.OP_KL, a.cuda(), b.cuda())
     assert torch.equal(am_d.cpu().long(), a.float().argmax(-1))
     assert torch.equal(am_t.cpu().long(), b.float().argmax(-1))
     assert torch.equal(argmax_rows(a.cuda()).cpu(), a.float().argmax(-1))
@@ -197,8 +197,8 @@ def test_full_size_rows_properties():
     y = (torch.randn(1, 4096, 32000, device="cuda", generator=g) * 2).bfloat16()
     same = L.kl_div_loss(x.detach(), x.detach())
     assert same.abs().max().item() < 1e-4
-    rows, am_d, _ = L.fused_rows(L.OP_KL, x, y)
-    rows2, am_d2, _ = L.fused_rows(L.OP_KL, x, y)
+    rows, am_d, _, _ = L.fused_rows(L.OP_KL, x, y)
+    rows2, am_d2, _, _ = L.fused_rows(L.OP_KL, x, y)
     assert torch.equal(rows, rows2) and torch.equal(am_d, am_d2)
     assert (rows >= 0).all()
     rows.sum().backward()
@@ -207,3 +207,27 @@ def test_full_size_rows_properties():
     idx = torch.arange(0, 4096, 64)
     ref = OL.kl_div(x.detach()[:, idx].cpu(), y[:, idx].cpu())
     torch.testing.assert_close(rows[:, idx].detach().cpu(), ref, **LOSS_TOL)
+
+
+@pytest.mark.parametrize("op_name", ["kl_div", "ce"])
+def test_reused_target_statistics_give_the_same_rows(op_name):
+    """Steps >= 1 reuse the verifier rows' lse / arg-max from step 0: same loss, arg-maxes
+    and gradient as recomputing them."""
+    from speculators_amd import losses as L
+
+    op = L.PRIMITIVE_OP[op_name]
+    g = torch.Generator().manual_seed(11)
+    t, v, k = 200, 4000, 3
+    logits = (torch.randn(1, t, v, generator=g) * 2).bfloat16().cuda()
+    targets = (torch.randn(1, t, v, generator=g) * 2).bfloat16().cuda()
+    _, _, am_full, lse_full = L.fused_rows(op, logits, targets)
+    a = logits[:, : t - k].detach().clone().requires_grad_(True)
+    b = logits[:, : t - k].detach().clone().requires_grad_(True)
+    fresh, pd_f, pt_f, _ = L.fused_rows(op, a, targets[:, k:])
+    known = (lse_full.reshape(-1)[k:], am_full.reshape(-1)[k:])
+    reused, pd_r, pt_r, _ = L.fused_rows(op, b, targets[:, k:], known)
+    assert torch.equal(pd_f, pd_r) and torch.equal(pt_f, pt_r)
+    torch.testing.assert_close(reused, fresh, atol=2e-6, rtol=1e-5)
+    go = torch.randn_like(fresh)
+    (fresh * go).sum().backward(); (reused * go).sum().backward()
+    torch.testing.assert_close(b.grad.float(), a.grad.float(), atol=1e-6, rtol=1e-3)

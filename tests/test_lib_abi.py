@@ -38,10 +38,10 @@ def test_argument_errors_do_not_need_a_gpu():
 
     lib = _lib.load()
     rc = lib.spx_fused_vocab_loss_fwd(99, None, 0, None, 0, 1, 8, 0, None, None, None, None, None,
-                                      None, None)
+                                      None, 0, None)
     assert rc == 1 and b"unknown loss op" in lib.spx_last_error()
     rc = lib.spx_fused_vocab_loss_fwd(0, None, 4, None, 4, 1, 8, 0, None, None, None, None, None,
-                                      None, None)
+                                      None, 0, None)
     assert rc == 1 and b"stride" in lib.spx_last_error()
 
 
