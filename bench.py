@@ -25,6 +25,21 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
+# HBM traffic per launch (bytes) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the
+# default shapes and scaled by what the same counters read for a plain copy of known size
+# (FETCH_SIZE under-reads by 1.9998x on this hardware, WRITE_SIZE reads 1.0x); the summary of
+# those runs is profiles/kernels_config1_hbm_traffic_pmc.txt.  Only valid for the default
+# --seq-len / --ttt-steps; other shapes report null.
+KIB = 1024
+MEASURED_TRAFFIC = {
+    "gemm_fwd": int((1.9998 * 873383 + 264118) * KIB),
+    "gemm_dx": int((1.9998 * 768994 + 43293) * KIB),
+    "loss_fwd": int((1.9998 * 256049 + 768) * KIB),
+    "loss_fwd_reuse": int((1.9998 * 256165 + 512) * KIB),
+    "loss_bwd": int((1.9998 * 256418 + 256000) * KIB),
+    "attn_fwd": int((1.9998 * 85247 + 33280) * KIB),
+}
+
 CONFIG1 = dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
                intermediate_size=14336, vocab_size=128256, draft_vocab_size=32000,
                rope_theta=500000.0, rms_norm_eps=1e-5)
@@ -45,6 +60,8 @@ def parse_args():
     ap.add_argument("--cpu-baseline", choices=["sample", "off"], default="sample")
     ap.add_argument("--cpu-seq-len", type=int, default=256)
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline timing")
+    ap.add_argument("--only-kernels", action="store_true",
+                    help="run only the per-kernel timing loops (for rocprofv3 counter runs)")
     return ap.parse_args()
 
 
@@ -111,28 +128,43 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
     g = torch.Generator(device=device).manual_seed(2)
     out = []
 
-    def mfma(name, flops, ms, launches):
+    default_shape = (t == SEQ_LEN and k_steps == TTT_STEPS)
+
+    def traffic_of(key):
+        return MEASURED_TRAFFIC.get(key) if (default_shape and key) else None
+
+    def mfma(name, flops, ms, launches, key=None):
         tf = flops / (ms * 1e-3) / 1e12
         out.append({"kernel": name, "bound": "mfma", "achieved": round(tf, 1),
                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4),
-                    "traffic": None, "ms_per_launch": round(ms, 4), "launches_per_step": launches})
+                    "traffic": traffic_of(key), "algorithmic_flops": flops,
+                    "ms_per_launch": round(ms, 4), "launches_per_step": launches})
 
-    def hbm(name, nbytes, ms, launches):
+    def hbm(name, nbytes, ms, launches, key=None):
         gbs = nbytes / (ms * 1e-3) / 1e9
         out.append({"kernel": name, "bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
-                    "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None,
+                    "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": traffic_of(key),
+                    "algorithmic_bytes": nbytes,
                     "ms_per_launch": round(ms, 4), "launches_per_step": launches})
+
+    # a plain copy of known size (T x Vd bf16 read + written once): the yardstick the
+    # FETCH_SIZE / WRITE_SIZE counters of the other kernels are scaled by
+    src = torch.randn(t, vd, device=device, generator=g).bfloat16()
+    dst = torch.empty_like(src)
+    ms = time_events(torch, lambda: dst.copy_(src), 20)
+    hbm("reference copy[T x Vd bf16, torch copy_]", 2.0 * t * vd * 2, ms, 0)
+    del src, dst
 
     # lm_head GEMM (forward shape; the input-gradient product has the same flops)
     x = torch.randn(t, h, device=device, generator=g).bfloat16()
     w = (torch.randn(vd, h, device=device, generator=g) * 0.02).bfloat16()
     y = torch.empty(t, vd, device=device, dtype=torch.bfloat16)
     ms = time_events(torch, lambda: gemm_nt(x, w, y), 20)
-    mfma("gemm_bf16_nt_kernel[lm_head fwd T x H x Vd]", 2.0 * t * h * vd, ms, k_steps + 1)
+    mfma("gemm_bf16_nt_kernel[lm_head fwd T x H x Vd]", 2.0 * t * h * vd, ms, k_steps + 1, "gemm_fwd")
     wt = w.t().contiguous()
     dx = torch.empty(t, h, device=device, dtype=torch.bfloat16)
     ms = time_events(torch, lambda: gemm_nt(y, wt, dx), 20)
-    mfma("gemm_bf16_nt_kernel[lm_head dX T x Vd x H]", 2.0 * t * h * vd, ms, k_steps)
+    mfma("gemm_bf16_nt_kernel[lm_head dX T x Vd x H]", 2.0 * t * h * vd, ms, k_steps, "gemm_dx")
     del wt, dx
 
     # fused loss forward / backward over T rows (step 0 shape)
@@ -153,10 +185,10 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
                   _lib.ptr(arg[0]), _lib.ptr(arg[1]), 1, st)
 
     ms = time_events(torch, loss_fwd, 20)
-    hbm("loss_fwd_kernel[KL, T rows x Vd, step 0]", 2.0 * t * vd * 2, ms, 1)
+    hbm("loss_fwd_kernel[KL, T rows x Vd, step 0]", 2.0 * t * vd * 2, ms, 1, "loss_fwd")
     ms = time_events(torch, loss_fwd_reuse, 20)
     hbm("loss_fwd_kernel[KL, T rows x Vd, steps >= 1 (target statistics reused)]", 2.0 * t * vd * 2,
-        ms, k_steps - 1)
+        ms, k_steps - 1, "loss_fwd_reuse")
     rg = torch.full((t,), 1.0 / t, device=device)
     grad = torch.empty(t, vd, device=device, dtype=torch.bfloat16)
 
@@ -166,7 +198,7 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
                   _lib.ptr(rg), None, _lib.ptr(grad), vd, st)
 
     ms = time_events(torch, loss_bwd, 20)
-    hbm("loss_bwd_kernel[KL, T rows x Vd]", 3.0 * t * vd * 2, ms, k_steps)
+    hbm("loss_bwd_kernel[KL, T rows x Vd]", 3.0 * t * vd * 2, ms, k_steps, "loss_bwd")
     del tg, lg, grad, y
 
     # TTT attention at the last step (k = K-1 diagonals): forward and backward
@@ -179,7 +211,7 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
     vv = torch.randn(1, hkv, (step + 1) * t, d, device=device, generator=g).bfloat16().requires_grad_(True)
     pairs = t * (t + 1) / 2 + step * t
     ms_f = time_events(torch, lambda: A.ttt_attention(q.detach(), kk.detach(), vv.detach(), mask), 10)
-    mfma(f"ttt_attn_fwd_kernel[step {step}]", 4.0 * pairs * d * hq, ms_f, 1)
+    mfma(f"attn_fwd_kernel[TTT step {step}]", 4.0 * pairs * d * hq, ms_f, 1, "attn_fwd")
     o = A.ttt_attention(q, kk, vv, mask)
     go = torch.randn_like(o)
 
@@ -187,7 +219,7 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
         torch.autograd.grad(o, (q, kk, vv), go, retain_graph=True)
 
     ms_b = time_events(torch, attn_bwd, 10)
-    mfma(f"ttt_attn_bwd[dq+dkv+diag kernels, step {step}]", 10.0 * pairs * d * hq, ms_b, 1)
+    mfma(f"attn_bwd[dq + dkv + diag kernels, TTT step {step}]", 10.0 * pairs * d * hq, ms_b, 1)
     return out
 
 
@@ -240,6 +272,9 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     t, k_steps = args.seq_len, args.ttt_steps
+    if args.only_kernels:
+        print(json.dumps({"kernels": kernel_rooflines(torch, CONFIG1, t, k_steps, device)}))
+        return
     batch, d2t, t2d = make_inputs(torch, CONFIG1, t, device, args.targets == "logits")
     model = make_model(torch, CONFIG1, device, d2t, t2d)
     loss_cfg = None  # kl_div, the reference default
@@ -266,6 +301,8 @@ def main():
     dominant = None
     if kernels:
         dominant = max(kernels, key=lambda r: r["ms_per_launch"] * r["launches_per_step"])
+        kernels = [k for k in kernels if k["launches_per_step"] > 0] + \
+                  [k for k in kernels if k["launches_per_step"] == 0]
     cpu = None
     if args.cpu_baseline != "off":
         del model

@@ -20,9 +20,28 @@ constexpr int kLossWaves = kLossThreads / 64;
 template <typename T>
 __device__ __forceinline__ void load8_vec(const T* p, float v[8]);
 
+// streaming accesses bypass the cache hierarchy's allocate-on-access policy: every row is
+// read (and every gradient row written) exactly once per launch
+#ifndef SPX_LOSS_NT
+#define SPX_LOSS_NT 1
+#endif
+__device__ __forceinline__ u32x4 ld16(const void* p) {
+#if SPX_LOSS_NT
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+#else
+  return *reinterpret_cast<const u32x4*>(p);
+#endif
+}
+__device__ __forceinline__ void st16(void* p, u32x4 v) {
+#if SPX_LOSS_NT
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+#else
+  *reinterpret_cast<u32x4*>(p) = v;
+#endif
+}
 template <>
 __device__ __forceinline__ void load8_vec<uint16_t>(const uint16_t* p, float v[8]) {
-  u32x4 raw = *reinterpret_cast<const u32x4*>(p);
+  u32x4 raw = ld16(p);
   v[0] = bf16_lo(raw.x); v[1] = bf16_hi(raw.x);
   v[2] = bf16_lo(raw.y); v[3] = bf16_hi(raw.y);
   v[4] = bf16_lo(raw.z); v[5] = bf16_hi(raw.z);
@@ -58,7 +77,7 @@ __device__ __forceinline__ void store8_vec<uint16_t>(uint16_t* p, const float v[
   u32x4 raw;
   raw.x = pack_bf16x2(v[0], v[1]); raw.y = pack_bf16x2(v[2], v[3]);
   raw.z = pack_bf16x2(v[4], v[5]); raw.w = pack_bf16x2(v[6], v[7]);
-  *reinterpret_cast<u32x4*>(p) = raw;
+  st16(p, raw);
 }
 template <>
 __device__ __forceinline__ void store8_vec<float>(float* p, const float v[8]) {
@@ -310,11 +329,28 @@ __global__ __launch_bounds__(kLossThreads) void loss_bwd_kernel(
   const int label = (OP == SPX_LOSS_CE) ? argmax_target[r] : -1;
   const float cd = -lse_d * kLog2e, ct = -lse_t * kLog2e;
 
-  for (int64_t c = tid; c < nchunks; c += kLossThreads) {
+#ifndef SPX_LOSS_BWD_UNROLL
+#define SPX_LOSS_BWD_UNROLL 1
+#endif
+  constexpr int UNR = SPX_LOSS_BWD_UNROLL;
+  for (int64_t c0 = tid; c0 < nchunks; c0 += kLossThreads * UNR) {
+    float xs[UNR][8], ys[UNR][8];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int64_t c = c0 + (int64_t)u * kLossThreads;
+      if (c < nchunks) {
+        load8<T, VEC>(xrow, c << 3, vocab, xs[u]);
+        if (OP != SPX_LOSS_CE) load8<T, VEC>(yrow, c << 3, vocab, ys[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+    const int64_t c = c0 + (int64_t)u * kLossThreads;
+    if (c >= nchunks) break;
     const int64_t base = c << 3;
-    float x[8], y[8], o[8];
-    load8<T, VEC>(xrow, base, vocab, x);
-    if (OP != SPX_LOSS_CE) load8<T, VEC>(yrow, base, vocab, y);
+    float o[8];
+    float* x = xs[u];
+    float* y = ys[u];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       if (OP == SPX_LOSS_CE) {
@@ -335,6 +371,7 @@ __global__ __launch_bounds__(kLossThreads) void loss_bwd_kernel(
       }
     }
     store8<T, VEC>(grow, base, vocab, o);
+    }
   }
 }
 
