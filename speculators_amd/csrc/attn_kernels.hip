@@ -322,38 +322,42 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_kernel(AttnParams p,
       const bool need_mask = (n0 < w_amax) || (n0 + kBN > w_bmin);
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb) {
+        // running max on the raw scores; the soft-max scale is folded into the exp2 argument
         float mx = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            float s = st[sb][kb][r] * p.scale_log2e;
+            float sv = st[sb][kb][r];
             if (need_mask) {
               const int c = n0 + kb * 32 + acc_row(r, g);
-              if (c < aa[sb] || c >= bb[sb]) s = -INFINITY;
+              if (c < aa[sb] || c >= bb[sb]) sv = -INFINITY;
+              st[sb][kb][r] = sv;
             }
-            st[sb][kb][r] = s;
-            mx = fmaxf(mx, s);
+            mx = fmaxf(mx, sv);
           }
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run[sb], mx);
+        const float m_new = fmaxf(m_run[sb], mx * p.scale_log2e);
         const float alpha = fast_exp2(m_run[sb] - m_new);
         float rs = 0.f;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float pv = fast_exp2(st[sb][kb][r] - m_new);
+            const float pv = fast_exp2(fmaf(st[sb][kb][r], p.scale_log2e, -m_new));
             st[sb][kb][r] = pv;
             rs += pv;
           }
         rs += __shfl_xor(rs, 32, 64);
         l_run[sb] = l_run[sb] * alpha + rs;
+        // the accumulator only needs rescaling when some row's max moved
+        if (__any(m_new != m_run[sb])) {
+#pragma unroll
+          for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[sb][db][r] *= alpha;
+        }
         m_run[sb] = m_new;
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[sb][db][r] *= alpha;
       }
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
@@ -562,8 +566,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(
     }
   };
 
-  auto run_pass = [&](const int (&aa)[NSB], const int (&bb)[NSB], int w_amin, int w_bmax,
-                      int blk_a, int blk_b) {
+  auto run_pass = [&](const int (&aa)[NSB], const int (&bb)[NSB], int w_amin, int w_amax,
+                      int w_bmin, int w_bmax, int blk_a, int blk_b) {
     if (blk_b <= blk_a) return;
     const int n_begin = (blk_a / kBN) * kBN;
     if (PF) fetch(n_begin);
@@ -589,13 +593,16 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(
             dp[kb] = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(vrow + kk * 16)), dof[sb][kk], dp[kb]);
           }
         }
+        const bool need_mask = (n0 < w_amax) || (n0 + kBN > w_bmin);
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const int c = n0 + kb * 32 + acc_row(r, g);
             float pv = fast_exp2(fmaf(st[kb][r], p.scale_log2e, -lse_i[sb]));
-            if (c < aa[sb] || c >= bb[sb]) pv = 0.f;
+            if (need_mask) {
+              const int c = n0 + kb * 32 + acc_row(r, g);
+              if (c < aa[sb] || c >= bb[sb]) pv = 0.f;
+            }
             dp[kb][r] = pv * (dp[kb][r] - delta_i[sb]);
           }
 #pragma unroll
@@ -613,8 +620,9 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(
     }
   };
 
-  run_pass(rb.a1, rb.b1, rb.w_a1min, rb.w_b1max, rb.blk_a1, rb.blk_b1);
-  if (p.a2) run_pass(rb.a2, rb.b2, rb.w_a2min, rb.w_b2max, rb.blk_a2, rb.blk_b2);
+  run_pass(rb.a1, rb.b1, rb.w_a1min, rb.w_a1max, rb.w_b1min, rb.w_b1max, rb.blk_a1, rb.blk_b1);
+  if (p.a2)
+    run_pass(rb.a2, rb.b2, rb.w_a2min, rb.w_a2max, rb.w_b2min, rb.w_b2max, rb.blk_a2, rb.blk_b2);
 
   for (int j = 1; j <= p.n_extra; ++j) {
 #pragma unroll

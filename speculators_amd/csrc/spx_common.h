@@ -46,8 +46,15 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   u += 0x7fffu + ((u >> 16) & 1u);
   return u >> 16;
 }
+// two fp32 -> packed bf16 pair with the gfx950 conversion instruction
+// (v_cvt_pk_bf16_f32, round-to-nearest-even)
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+  union { bf16x2_t b; uint32_t u; } c;
+  f32x2_t v = {lo, hi};
+  c.b = __builtin_convertvector(v, bf16x2_t);
+  return c.u;
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

@@ -99,15 +99,18 @@ class DFlashAttention(nn.Module):
 
     def forward(self, x, ctx, q_pos, kv_pos, inv_freq, mask):
         ql, tl = x.shape[1], ctx.shape[1]
-        q = self.q_norm(self.q_proj(x).view(1, ql, self.hq, self.d)).view(1, ql, self.hq * self.d)
-        k = torch.cat([self.k_proj(ctx), self.k_proj(x)], dim=1)
-        v = torch.cat([self.v_proj(ctx), self.v_proj(x)], dim=1)
+        lin = gemm.linear_accumulate
+        q = self.q_norm(lin(x, self.q_proj.weight).view(1, ql, self.hq, self.d)).view(1, ql, self.hq * self.d)
+        # one projection of cat([context, mask tokens]) instead of two per weight
+        both = torch.cat([ctx, x], dim=1)
+        k = lin(both, self.k_proj.weight)
+        v = lin(both, self.v_proj.weight)
         k = self.k_norm(k.view(1, tl + ql, self.hkv, self.d)).view(1, tl + ql, self.hkv * self.d)
         q = FO.rope_relayout(q, q_pos, inv_freq, self.hq, True, 0)
         k = FO.rope_relayout(k, kv_pos, inv_freq, self.hkv, True, 0)
         v = FO.rope_relayout(v, kv_pos, inv_freq, self.hkv, False, 0)
         out, _ = self.attn_fn(self, q, k, v, mask, scaling=self.scaling)
-        return self.o_proj(out.reshape(1, ql, self.hq * self.d))
+        return gemm.linear_accumulate(out.reshape(1, ql, self.hq * self.d), self.o_proj.weight)
 
 
 class DFlashDecoderLayer(nn.Module):

@@ -83,7 +83,10 @@ class Attention(nn.Module):
 
     def forward(self, x, position_ids, pos_offset, inv_freq, cache: dict, mask):
         t = x.shape[1]
-        q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+        lin = gemm.linear_accumulate
+        q = lin(x, self.q_proj.weight)
+        k = lin(x, self.k_proj.weight)
+        v = lin(x, self.v_proj.weight)
         if self.qk_norm:
             q = self.q_norm(q.view(1, t, self.hq, self.d)).view(1, t, self.hq * self.d)
             k = self.k_norm(k.view(1, t, self.hkv, self.d)).view(1, t, self.hkv * self.d)
@@ -95,7 +98,7 @@ class Attention(nn.Module):
         cache["k"] = k if "k" not in cache else torch.cat([cache["k"], k], dim=2)
         cache["v"] = v if "v" not in cache else torch.cat([cache["v"], v], dim=2)
         out, _ = self.attn_fn(self, q, cache["k"], cache["v"], mask, scaling=self.scaling)
-        return self.o_proj(out.reshape(1, t, self.hq * self.d))
+        return gemm.linear_accumulate(out.reshape(1, t, self.hq * self.d), self.o_proj.weight)
 
 
 class MLP(nn.Module):
@@ -106,7 +109,9 @@ class MLP(nn.Module):
         self.down_proj = nn.Linear(cfg.intermediate_size, cfg.hidden_size, bias=False)
 
     def forward(self, x):
-        return self.down_proj(FO.swiglu(self.gate_proj(x), self.up_proj(x)))
+        lin = gemm.linear_accumulate
+        return lin(FO.swiglu(lin(x, self.gate_proj.weight), lin(x, self.up_proj.weight)),
+                   self.down_proj.weight)
 
 
 class DecoderLayer(nn.Module):

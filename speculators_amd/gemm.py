@@ -10,6 +10,8 @@ weight gradient (a TN product) to the rocBLAS/hipBLASLt matmul of PyTorch.
 
 from __future__ import annotations
 
+import os
+
 import torch
 
 from . import _lib
@@ -60,3 +62,43 @@ def linear(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor | None 
     """``x[..., K] @ weight[N, K].T`` on the HIP GEMM; ``weight_t`` optionally holds
     ``weight.T`` contiguous for the backward."""
     return _Linear.apply(x, weight, weight_t)
+
+
+FUSE_WGRAD_ACCUMULATION = os.environ.get("SPX_FUSE_WGRAD", "1") != "0"
+
+
+class _LinearAccumulate(torch.autograd.Function):
+    """``x @ weight.T`` on PyTorch's (hipBLASLt) matmul whose backward ADDS the weight
+    gradient into ``weight.grad`` inside the GEMM (beta = 1) instead of returning a fresh
+    tensor for autograd to add.  A weight that is applied once per TTT step otherwise costs
+    one full read-modify-write pass over a weight-sized tensor per step after the first."""
+
+    @staticmethod
+    def forward(ctx, x, weight):
+        ctx.save_for_backward(x, weight)
+        return torch.nn.functional.linear(x, weight)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight = ctx.saved_tensors
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dx = torch.matmul(dy, weight)
+        if weight.requires_grad:
+            dy2 = dy.reshape(-1, dy.shape[-1])
+            x2 = x.reshape(-1, x.shape[-1])
+            if weight.grad is None:
+                weight.grad = torch.matmul(dy2.t(), x2)
+            else:
+                torch.addmm(weight.grad, dy2.t(), x2, out=weight.grad)
+        return dx, None
+
+
+def linear_accumulate(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """See ``_LinearAccumulate``.  The weight gradient lands in ``weight.grad`` during
+    ``backward()`` (it is not visible to ``torch.autograd.grad``)."""
+    if not FUSE_WGRAD_ACCUMULATION or not torch.is_grad_enabled() or not (
+            x.requires_grad or weight.requires_grad):
+        return torch.nn.functional.linear(x, weight)
+    # autograd must see a differentiable input even when only the weight needs a gradient
+    return _LinearAccumulate.apply(x, weight)
