@@ -48,6 +48,19 @@ __device__ __forceinline__ bf16x8 pack8(const f32x16& a, int base) {
   return c.b;
 }
 
+// dot product of two 8-element bf16 fragments, accumulated in fp32 with the packed
+// bf16 dot instruction (v_dot2c_f32_bf16): no conversion of the operands to fp32
+__device__ __forceinline__ float dot8_bf16(bf16x8 a, u32x4 b, float acc) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+  union { bf16x8 v; bf16x2_t p[4]; } ua;
+  union { u32x4 v; bf16x2_t p[4]; } ub;
+  ua.v = a;
+  ub.v = b;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_fdot2_f32_bf16(ua.p[i], ub.p[i], acc, false);
+  return acc;
+}
+
 __device__ __forceinline__ void unpack8(u32x4 raw, float v[8]) {
   v[0] = bf16_lo(raw.x); v[1] = bf16_hi(raw.x);
   v[2] = bf16_lo(raw.y); v[3] = bf16_hi(raw.y);

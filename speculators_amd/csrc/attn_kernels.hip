@@ -187,8 +187,17 @@ __device__ __forceinline__ void load_bounds(const AttnParams& p, const int (&ic)
 // One workgroup = 4 waves = 4 * 32 * NSB query rows of one head.  With NSB = 2 a
 // wave owns two 32-row sub-blocks, so every K / V^T fragment read from LDS
 // feeds two MFMAs (LDS bandwidth, not the matrix core, bounds NSB = 1).
+#ifndef SPX_FWD_MINB
+#define SPX_FWD_MINB 2
+#endif
+#ifndef SPX_DQ_MINB
+#define SPX_DQ_MINB 2
+#endif
+#ifndef SPX_DKV_MINB
+#define SPX_DKV_MINB 1
+#endif
 template <int D, int NSB, int NW, bool PF>
-__global__ __launch_bounds__(64 * NW) void attn_fwd_kernel(AttnParams p,
+__global__ __launch_bounds__(64 * NW, SPX_FWD_MINB) void attn_fwd_kernel(AttnParams p,
                                                                 const uint16_t* __restrict__ Vt,
                                                                 uint16_t* __restrict__ O,
                                                                 float* __restrict__ LSE) {
@@ -387,12 +396,8 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_kernel(AttnParams p,
       const uint16_t* kj = p.K + (int64_t)kvh * p.k_hs + ((int64_t)j * p.T + ic[sb]) * D + g * 8;
       float dot = 0.f;
 #pragma unroll
-      for (int kk = 0; kk < NKK; ++kk) {
-        float kv[8];
-        unpack8(*reinterpret_cast<const u32x4*>(kj + kk * 16), kv);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) dot = fmaf((float)qf[sb][kk][e], kv[e], dot);
-      }
+      for (int kk = 0; kk < NKK; ++kk)
+        dot = dot8_bf16(qf[sb][kk], *reinterpret_cast<const u32x4*>(kj + kk * 16), dot);
       dot += __shfl_xor(dot, 32, 64);
       const float s = dot * p.scale_log2e;
       const float m_new = fmaxf(m_run[sb], s);
@@ -456,7 +461,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const uint16_t* __restr
 // dQ: same tiling as the forward.
 //   P^T = exp2(S'^T - lse), dP^T = V dO^T, dS^T = P^T (dP^T - delta), dQ^T += K^T dS^T
 template <int D, int NSB, int NW, bool PF>
-__global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(
+__global__ __launch_bounds__(64 * NW, SPX_DQ_MINB) void attn_bwd_dq_kernel(
     AttnParams p, const uint16_t* __restrict__ dO, const uint16_t* __restrict__ Kt,
     const float* __restrict__ LSE, const float* __restrict__ Delta, uint16_t* __restrict__ dQ,
     int64_t dq_hs) {
@@ -578,42 +583,49 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(
       if (PF && n0 + kBN < blk_b) fetch(n0 + kBN);
       if (n0 >= w_bmax || n0 + kBN <= w_amin) continue;
 
+      const bool need_mask = (n0 < w_amax) || (n0 + kBN > w_bmin);
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb) {
-        f32x16 st[2], dp[2];
+        // the two 32-key halves of the tile one after the other: 32 score registers live
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
+          f32x16 st, dp;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) { st[kb][r] = 0.f; dp[kb][r] = 0.f; }
+          for (int r = 0; r < 16; ++r) { st[r] = 0.f; dp[r] = 0.f; }
           const uint16_t* krow = &Ks[(kb * 32 + col) * KS + g * 8];
           const uint16_t* vrow = &Vn[(kb * 32 + col) * KS + g * 8];
+#ifndef SPX_DQ_KKU
+#define SPX_DQ_KKU 8
+#endif
 #pragma unroll
-          for (int kk = 0; kk < NKK; ++kk) {
-            st[kb] = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(krow + kk * 16)), qf[sb][kk], st[kb]);
-            dp[kb] = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(vrow + kk * 16)), dof[sb][kk], dp[kb]);
+          for (int kk0 = 0; kk0 < NKK; kk0 += SPX_DQ_KKU) {
+#pragma unroll
+            for (int kk = kk0; kk < kk0 + SPX_DQ_KKU && kk < NKK; ++kk) {
+              st = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(krow + kk * 16)), qf[sb][kk], st);
+              dp = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(vrow + kk * 16)), dof[sb][kk], dp);
+            }
+            if (SPX_DQ_KKU < NKK) __builtin_amdgcn_sched_barrier(0);
           }
-        }
-        const bool need_mask = (n0 < w_amax) || (n0 + kBN > w_bmin);
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            float pv = fast_exp2(fmaf(st[kb][r], p.scale_log2e, -lse_i[sb]));
+            float pv = fast_exp2(fmaf(st[r], p.scale_log2e, -lse_i[sb]));
             if (need_mask) {
               const int c = n0 + kb * 32 + acc_row(r, g);
               if (c < aa[sb] || c >= bb[sb]) pv = 0.f;
             }
-            dp[kb][r] = pv * (dp[kb][r] - delta_i[sb]);
+            dp[r] = pv * (dp[r] - delta_i[sb]);
           }
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          const bf16x8 db8 = pack8(dp[s >> 1], (s & 1) * 8);
+          for (int s2 = 0; s2 < 2; ++s2) {
+            const int s = kb * 2 + s2;
+            const bf16x8 db8 = pack8(dp, s2 * 8);
 #pragma unroll
-          for (int db = 0; db < NDB; ++db) {
-            const uint16_t* trow = &Kts[(db * 32 + col) * VS + s * 16 + 4 * g];
-            const bf16x8 ka = join_bf16x4(*reinterpret_cast<const u32x2*>(trow),
-                                          *reinterpret_cast<const u32x2*>(trow + 8));
-            acc[sb][db] = mfma32(ka, db8, acc[sb][db]);
+            for (int db = 0; db < NDB; ++db) {
+              const uint16_t* trow = &Kts[(db * 32 + col) * VS + s * 16 + 4 * g];
+              const bf16x8 ka = join_bf16x4(*reinterpret_cast<const u32x2*>(trow),
+                                            *reinterpret_cast<const u32x2*>(trow + 8));
+              acc[sb][db] = mfma32(ka, db8, acc[sb][db]);
+            }
           }
         }
       }
@@ -632,14 +644,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(
       float dot = 0.f, dpv = 0.f;
 #pragma unroll
       for (int kk = 0; kk < NKK; ++kk) {
-        float kv[8], vv[8];
-        unpack8(*reinterpret_cast<const u32x4*>(kj + g * 8 + kk * 16), kv);
-        unpack8(*reinterpret_cast<const u32x4*>(vj + g * 8 + kk * 16), vv);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          dot = fmaf((float)qf[sb][kk][e], kv[e], dot);
-          dpv = fmaf((float)dof[sb][kk][e], vv[e], dpv);
-        }
+        dot = dot8_bf16(qf[sb][kk], *reinterpret_cast<const u32x4*>(kj + g * 8 + kk * 16), dot);
+        dpv = dot8_bf16(dof[sb][kk], *reinterpret_cast<const u32x4*>(vj + g * 8 + kk * 16), dpv);
       }
       dot += __shfl_xor(dot, 32, 64);
       dpv += __shfl_xor(dpv, 32, 64);
@@ -698,7 +704,7 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
 // The per-head results go to fp32 partial buffers that attn_dkv_reduce_kernel sums over
 // the heads of a group (fixed order: deterministic, no atomics).
 template <int D, int NW, bool PF>
-__global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_kernel(
+__global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     AttnParams p, const uint16_t* __restrict__ dO, const uint16_t* __restrict__ Qt,
     const uint16_t* __restrict__ dOt, int NQp, const float* __restrict__ LSE,
     const float* __restrict__ Delta, const int32_t* __restrict__ tile_bounds,
@@ -1018,7 +1024,7 @@ static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 #define SPX_FWD_CFG 1, 4, true
 #endif
 #ifndef SPX_DQ_CFG
-#define SPX_DQ_CFG 1, 4, true
+#define SPX_DQ_CFG 1, 4, false
 #endif
 #ifndef SPX_DKV_CFG
 #define SPX_DKV_CFG 4, true
