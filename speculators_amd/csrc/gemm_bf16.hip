@@ -1,18 +1,28 @@
 // C[M, N] = A[M, K] * B[N, K]^T  (the nn.Linear product), bf16 in, fp32
 // accumulate, bf16 out, for gfx950.
 //
-// One workgroup of 8 waves (4 along M x 2 along N) owns a 256 x 256 tile of C
-// and walks K in steps of 64; each wave owns a 64 x 128 patch as 2 x 4
-// accumulators of v_mfma_f32_32x32x16_bf16, two waves per SIMD so one wave's
-// LDS reads overlap the other's MFMAs.  A and B tiles are staged global ->
-// registers -> LDS (buffer loads: rows past the edge read as zero, no per-lane
-// predicates) through two LDS stages (the next tile is written while the
-// current one is read: one barrier per K step) with the next tile's global
-// loads in flight during the current tile's MFMAs.  LDS rows are padded by 16
-// bytes so the 16-byte operand reads of consecutive lanes hit distinct bank
-// groups (measured: zero bank conflicts).  Workgroup ids are remapped so that
-// each XCD (ids are dealt round-robin over the 8 XCDs) works on a compact
-// band of tiles and shares its A / B panels in that XCD's L2.
+// One workgroup of 4 waves owns a 256 x 256 tile of C (each wave a 128 x 128
+// patch = 4 x 4 accumulators of v_mfma_f32_32x32x16_bf16, one wave per SIMD)
+// and walks K in slabs of 64.
+//
+// Global -> LDS directly (buffer_load ... lds): no staging registers and no
+// LDS store instructions.  A wave-load fills 8 rows x 128 B of LDS linearly
+// (lane i -> byte 16 i), so every fetch is a whole 128-byte line; the
+// bank-conflict-free layout comes from WHICH 16-byte K chunk a lane fetches:
+// chunk c of row r sits in slot c ^ f(r), f(r) = (r & 7) ^ ((r >> 3) & 1).
+// Two slab buffers: the loads of slab s+1 are in flight while slab s is
+// multiplied.  They are issued one at a time between the MFMAs (a burst would
+// stall the wave at issue until the memory pipeline has room), and so are the
+// LDS reads: operand fragments are double buffered in registers, the reads of
+// K step kk+1 run under the MFMAs of step kk, and the last step of a slab is
+// multiplied after the barrier that opens the next slab, so no LDS latency is
+// exposed and there is one barrier per slab.
+//
+// The accumulators are kept transposed (lane = row of C, registers = 4
+// consecutive columns); v_permlane32_swap pairs them into 8 consecutive
+// columns for 16-byte stores.  Workgroup ids are remapped so that each XCD
+// (ids are dealt round-robin over the 8 XCDs) works on a compact band of
+// tiles and shares its A / B panels in that XCD's L2.
 
 #include <type_traits>
 
@@ -22,35 +32,80 @@
 namespace spx {
 
 #ifndef SPX_GEMM_WM
-#define SPX_GEMM_WM 4
+#define SPX_GEMM_WM 2
 #endif
 #ifndef SPX_GEMM_WN
 #define SPX_GEMM_WN 2
 #endif
-#ifndef SPX_GEMM_PGR
-#define SPX_GEMM_PGR 1
+#ifndef SPX_GEMM_MINW
+#define SPX_GEMM_MINW 1
+#endif
+#ifndef SPX_GEMM_GROUP_M
+#define SPX_GEMM_GROUP_M 8
 #endif
 constexpr int kWM = SPX_GEMM_WM, kWN = SPX_GEMM_WN;  // waves along M / N of the tile
-constexpr int kPGR = SPX_GEMM_PGR;  // K tiles whose global loads are in flight ahead of the MFMAs
-constexpr int kGemmThreads = 64 * kWM * kWN;
+constexpr int kNW = kWM * kWN;
+constexpr int kGemmThreads = 64 * kNW;
 constexpr int kTM = 256, kTN = 256, kTK = 64;
 constexpr int kMI = kTM / kWM / 32, kNI = kTN / kWN / 32;  // 32x32 accumulators per wave
-constexpr int kLdsStride = kTK + 8;  // elements
-constexpr int kStageElems = (kTM + kTN) * kLdsStride;
-constexpr int kGemmSmem = 2 * kStageElems * 2;  // two stages
+constexpr int kRowBytes = kTK * 2;                          // 128
+constexpr int kABytes = kTM * kRowBytes;                    // one slab of A: 32 KB
+constexpr int kBBytes = kTN * kRowBytes;
+constexpr int kBBase = 2 * kABytes;
+constexpr int kGemmSmem = 2 * (kABytes + kBBytes);  // 128 KB
+constexpr int kLA = kTM / 8 / kNW;                  // wave-loads of A per wave per slab
+constexpr int kLB = kTN / 8 / kNW;
+constexpr int kL = kLA + kLB;
+constexpr int kOob = 0x7ffffff0;
+static_assert(kABytes == 32768 && kBBytes == 32768, "the buffer toggle flips bit 15");
+static_assert(kLA % 4 == 0 && kLB % 4 == 0, "loads are grouped in fours (immediate offsets)");
 
-__device__ __forceinline__ bf16x8 lds_frag(const uint16_t* p) {
+// 64 lanes x 16 bytes, global -> LDS at M0 + IMM + 16 * lane; the global address is
+// base + voff + soff + IMM.  Lanes whose voff + IMM lies outside the resource write
+// zeros.  M0 is an input operand: the compiler writes it only when the value changes.
+// The s_nop covers the M0-write -> LDS-DMA wait state for the first load of a group.
+template <int IMM>
+__device__ __forceinline__ void load_to_lds16(u32x4 rsrc, uint32_t lds_addr, int voff, int soff) {
+  if (IMM == 0)
+    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "{m0}"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory");
+  else
+    asm volatile("buffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds"
+                 :
+                 : "{m0}"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM)
+                 : "memory");
+}
+
+__device__ __forceinline__ bf16x8 as_frag(u32x4 v) {
   union { u32x4 u; bf16x8 b; } c;
-  c.u = *reinterpret_cast<const u32x4*>(p);
+  c.u = v;
   return c.b;
 }
 
-__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_nt_kernel(
+__device__ __forceinline__ u32x4 make_rsrc(const void* p, uint32_t bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(p);
+  u32x4 r;
+  r.x = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  r.y = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+  r.z = __builtin_amdgcn_readfirstlane(bytes);
+  r.w = 0x00020000u;
+  return r;
+}
+
+// kImm: consecutive loads of a group of four share one M0 value and differ in the
+// instruction's immediate offset (which moves the LDS and the global address alike, so
+// the per-lane global offset is stored minus that immediate).  Needs every row offset to
+// be at least the immediate: lda, ldb >= 64.  Without it every load sets M0 itself.
+template <bool kImm>
+__global__ __launch_bounds__(kGemmThreads, SPX_GEMM_MINW)
+__attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf16_nt_kernel(
     const uint16_t* __restrict__ A, int64_t lda, const uint16_t* __restrict__ B, int64_t ldb,
     uint16_t* __restrict__ C, int64_t ldc, int M, int N, int K, int tiles_m, int tiles_n) {
-  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
-  // workgroup id -> tile: XCD-contiguous bands, then groups of 8 tile rows
+  // workgroup id -> tile: XCD-contiguous bands, then groups of GROUP_M tile rows
   const int n_wg = tiles_m * tiles_n;
   int pid = blockIdx.x;
   {
@@ -60,7 +115,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_nt_kernel(
     // only remap when the grid divides evenly, otherwise keep the identity
     if (n_wg % 8 == 0) pid = cand;
   }
-  constexpr int GROUP_M = 8;
+  constexpr int GROUP_M = SPX_GEMM_GROUP_M;
   const int in_group = GROUP_M * tiles_n;
   const int group_id = pid / in_group;
   const int first_m = group_id * GROUP_M;
@@ -69,138 +124,189 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_nt_kernel(
   const int tile_n = (pid % in_group) / group_sz;
   const int m0 = tile_m * kTM, n0 = tile_n * kTN;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5, col = lane & 31;
   const int wm = (wave / kWN) * (kTM / kWM), wn = (wave % kWN) * (kTN / kWN);
 
-  // global -> register staging: 16-byte chunks, 8 per row of the 64-wide K tile
-  constexpr int kRowsPerPass = kGemmThreads / 8;
-  constexpr int kPasses = kTM / kRowsPerPass;
-  const int lrow = tid >> 3, lcol = (tid & 7) * 8;
-  u32x4 areg[kPGR][kPasses], breg[kPGR][kPasses];
-  f32x16 acc[kMI][kNI];
+  // acc[j][i]: registers = 32 columns of C at wn + 32 j, lane = row of C at wm + 32 i
+  f32x16 acc[kNI][kMI];
 #pragma unroll
-  for (int i = 0; i < kMI; ++i)
+  for (int j = 0; j < kNI; ++j)
+#pragma unroll
+    for (int i = 0; i < kMI; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[j][i][r] = 0.f;
+
+  // One buffer resource per operand; the K position goes into the scalar offset.  Rows
+  // past the matrix edge get an offset outside the resource and read as zero, so no
+  // clamping or per-lane predicate is needed.
+  const u32x4 ares = make_rsrc(A, (uint32_t)((((int64_t)M - 1) * lda + K) * 2));
+  const u32x4 bres = make_rsrc(B, (uint32_t)((((int64_t)N - 1) * ldb + K) * 2));
+
+  // global side: wave-load j of this wave covers tile rows wave*8*kLA + 8 j + lane/8; the
+  // lane's LDS slot is lane % 8, so it fetches chunk slot ^ f(row)
+  const int lrow = lane >> 3;
+  int gchunk[2];
+  gchunk[0] = (lane & 7) ^ (lrow & 7);      // rows 0..7 of a 16-row group
+  gchunk[1] = (lane & 7) ^ (lrow & 7) ^ 1;  // rows 8..15
+  int aoff[kLA], boff[kLB];
+#pragma unroll
+  for (int j = 0; j < kLA; ++j) {
+    const int r = wave * (8 * kLA) + j * 8 + lrow;
+    const int imm = kImm ? (j & 3) * 8 * kRowBytes : 0;
+    aoff[j] = (m0 + r < M) ? (int)((((int64_t)(m0 + r)) * lda + gchunk[j & 1] * 8) * 2) - imm : kOob;
+  }
+#pragma unroll
+  for (int j = 0; j < kLB; ++j) {
+    const int r = wave * (8 * kLB) + j * 8 + lrow;
+    const int imm = kImm ? (j & 3) * 8 * kRowBytes : 0;
+    boff[j] = (n0 + r < N) ? (int)((((int64_t)(n0 + r)) * ldb + gchunk[j & 1] * 8) * 2) - imm : kOob;
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+  const uint32_t lds_a = lds0 + wave * (8 * kLA) * kRowBytes;
+  const uint32_t lds_b = lds0 + kBBase + wave * (8 * kLB) * kRowBytes;
+
+  uint32_t bufoff = 0;  // slab buffer the next loads go to
+  int ld_k0 = 0;        // first K column of the slab being loaded
+  // load l (A loads first, then B) of the slab at ld_k0; full: the slab lies inside K
+  auto issue_one = [&](int l, bool full) __attribute__((always_inline)) {
+    const bool isa = l < kLA;
+    const int j = isa ? l : l - kLA;
+    int voff = isa ? aoff[j] : boff[j];
+    if (!full) voff = (ld_k0 + gchunk[j & 1] * 8 < K) ? voff : kOob;
+    const u32x4 res = isa ? ares : bres;
+    const uint32_t base = (isa ? lds_a : lds_b) + bufoff;
+    if (kImm) {
+      const uint32_t grp = base + (j & ~3) * 8 * kRowBytes;
+      switch (j & 3) {
+        case 0: load_to_lds16<0>(res, grp, voff, ld_k0 * 2); break;
+        case 1: load_to_lds16<8 * kRowBytes>(res, grp, voff, ld_k0 * 2); break;
+        case 2: load_to_lds16<16 * kRowBytes>(res, grp, voff, ld_k0 * 2); break;
+        default: load_to_lds16<24 * kRowBytes>(res, grp, voff, ld_k0 * 2); break;
+      }
+    } else {
+      load_to_lds16<0>(res, base + j * 8 * kRowBytes, voff, ld_k0 * 2);
+    }
+  };
+  auto next_slab = [&]() __attribute__((always_inline)) { bufoff ^= kABytes; ld_k0 += kTK; };
+
+  // read side: row = lane % 32 of a 32-row block, K chunk 2 kk + g in slot chunk ^ f(row)
+  const int fr = (col & 7) ^ ((col >> 3) & 1);
+  const int off0 = col * kRowBytes + ((g ^ fr) * 16);
+  uint32_t a_rd[4], b_rd[4];  // per K step of 16; bit 15 selects the slab buffer
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    a_rd[kk] = wm * kRowBytes + (off0 ^ (kk * 32));
+    b_rd[kk] = kBBase + wn * kRowBytes + (off0 ^ (kk * 32));
+  }
+
+  bf16x8 fa[2][kMI], fb[2][kNI];
+  // operand fragment f (A fragments first, then B) of K step kk into register set `set`
+  auto read_one = [&](int set, int kk, int f) __attribute__((always_inline)) {
+    if (f < kMI)
+      fa[set][f] = as_frag(*reinterpret_cast<const u32x4*>(smem + a_rd[kk] + f * 32 * kRowBytes));
+    else
+      fb[set][f - kMI] = as_frag(*reinterpret_cast<const u32x4*>(smem + b_rd[kk] + (f - kMI) * 32 * kRowBytes));
+  };
+  // One K step: the kNI x kMI MFMAs on register set `set`; between them, one at a time,
+  // the LDS reads that fill the other set with K step rk and the global loads
+  // [l0, l0 + nl).  Reads go first: their data is needed at the next step.
+  auto step = [&](int set, int rk, int l0, int nl, bool full) __attribute__((always_inline)) {
+    constexpr int kN = kNI * kMI, kF = kMI + kNI;
+    int reads = 0, loads = 0;
 #pragma unroll
     for (int j = 0; j < kNI; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  // buffer loads: one resource per operand, a fixed 32-bit byte offset per staged row and
-  // the K position in the scalar offset.  Rows past the matrix edge fall outside the
-  // resource and read as zero, so no clamping or per-lane predicate is needed.
-  const __amdgpu_buffer_rsrc_t ares = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(A), 0, (int)((((int64_t)M - 1) * lda + K) * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t bres = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(B), 0, (int)((((int64_t)N - 1) * ldb + K) * 2), 0x00020000);
-  int aoff[kPasses], boff[kPasses];
-#pragma unroll
-  for (int n = 0; n < kPasses; ++n) {
-    const int r = lrow + kRowsPerPass * n;
-    // a row index past the edge is moved far outside the resource (the plain product
-    // row * ld could wrap around 2^32 for huge strides)
-    aoff[n] = (m0 + r < M) ? (int)((((int64_t)(m0 + r)) * lda + lcol) * 2) : 0x7ffffff0;
-    boff[n] = (n0 + r < N) ? (int)((((int64_t)(n0 + r)) * ldb + lcol) * 2) : 0x7ffffff0;
-  }
-  const bool ktail = (K % kTK) != 0;
-#define SPX_FETCH(k0v, S)                                                              \
-  do {                                                                                 \
-    const int k0_ = (k0v);                                                             \
-    _Pragma("unroll") for (int n = 0; n < kPasses; ++n) {                              \
-      areg[S][n] = __builtin_amdgcn_raw_buffer_load_b128(ares, aoff[n], k0_ * 2, 0);   \
-      breg[S][n] = __builtin_amdgcn_raw_buffer_load_b128(bres, boff[n], k0_ * 2, 0);   \
-    }                                                                                  \
-    if (ktail && k0_ + lcol >= K) {                                                    \
-      const u32x4 z = {0, 0, 0, 0};                                                    \
-      _Pragma("unroll") for (int n = 0; n < kPasses; ++n) { areg[S][n] = z; breg[S][n] = z; } \
-    }                                                                                  \
-  } while (0)
-#define SPX_STASH(stagev, S)                                                           \
-  do {                                                                                 \
-    uint16_t* As_ = smem + (stagev) * kStageElems;                                     \
-    uint16_t* Bs_ = As_ + kTM * kLdsStride;                                            \
-    _Pragma("unroll") for (int n = 0; n < kPasses; ++n) {                              \
-      const int r = lrow + kRowsPerPass * n;                                           \
-      *reinterpret_cast<u32x4*>(&As_[r * kLdsStride + lcol]) = areg[S][n];             \
-      *reinterpret_cast<u32x4*>(&Bs_[r * kLdsStride + lcol]) = breg[S][n];             \
-    }                                                                                  \
-  } while (0)
-  auto compute = [&](int stage) {
-    const uint16_t* As = smem + stage * kStageElems;
-    const uint16_t* Bs = As + kTM * kLdsStride;
-#ifndef SPX_GEMM_KKUNROLL
-#define SPX_GEMM_KKUNROLL 4
-#endif
-#pragma unroll SPX_GEMM_KKUNROLL
-    for (int kk = 0; kk < kTK / 16; ++kk) {
-      bf16x8 af[kMI], bf[kNI];
-#pragma unroll
-      for (int i = 0; i < kMI; ++i) af[i] = lds_frag(&As[(wm + i * 32 + col) * kLdsStride + kk * 16 + g * 8]);
-#pragma unroll
-      for (int j = 0; j < kNI; ++j) bf[j] = lds_frag(&Bs[(wn + j * 32 + col) * kLdsStride + kk * 16 + g * 8]);
-#pragma unroll
-      for (int i = 0; i < kMI; ++i)
-#pragma unroll
-        for (int j = 0; j < kNI; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
-    }
+      for (int i = 0; i < kMI; ++i) {
+        acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[set][j], fa[set][i], acc[j][i], 0, 0, 0);
+        const int idx = j * kMI + i;
+        __builtin_amdgcn_sched_barrier(0);
+        if (reads < kF) {
+          read_one(set ^ 1, rk, reads++);
+          if (kF > kN && reads < kF) read_one(set ^ 1, rk, reads++);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (nl > 0 && (nl >= kN || idx % (kN / nl) == kN / nl - 1) && loads < nl) {
+          issue_one(l0 + loads++, full);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
   };
-  constexpr int S1 = kPGR - 1;
-  // two LDS stages: the next tile is written while the current one is read, one
-  // barrier per K step.  kPGR = 2 keeps the global loads of TWO tiles in flight (in two
-  // register sets) so that a tile's load latency is covered by two K steps of MFMAs.
-  if (kPGR == 1) {
-    SPX_FETCH(0, 0);
-    SPX_STASH(0, 0);
-    __syncthreads();
-    int stage = 0;
-    for (int k0 = 0; k0 < K; k0 += kTK) {
-      const bool more = k0 + kTK < K;
-      if (more) SPX_FETCH(k0 + kTK, 0);
-      compute(stage);
-      if (more) SPX_STASH(stage ^ 1, 0);
-      __syncthreads();
-      stage ^= 1;
-    }
-  } else {
-    SPX_FETCH(0, 0);
-    if (kTK < K) SPX_FETCH(kTK, S1);
-    SPX_STASH(0, 0);
-    __syncthreads();
-    int stage = 0;
-    for (int k0 = 0; k0 < K; k0 += kTK) {
-      // tile k0 sits in LDS stage `stage`; the register set of the other parity holds
-      // tile k0 + 1, this parity's set is free for tile k0 + 2
-      const bool more1 = k0 + kTK < K, more2 = k0 + 2 * kTK < K;
-      if (more2) {
-        if (stage == 0) SPX_FETCH(k0 + 2 * kTK, 0);
-        else SPX_FETCH(k0 + 2 * kTK, S1);
-      }
-      compute(stage);
-      if (more1) {
-        if (stage == 0) SPX_STASH(1, S1);
-        else SPX_STASH(0, 0);
-      }
-      __syncthreads();
-      stage ^= 1;
-    }
-  }
-#undef SPX_FETCH
-#undef SPX_STASH
 
-  // accumulator (i, j): lane column = n, register r = row 8*(r/4) + 4*g + r%4
+  // the loads of a slab are spread over the step after the barrier (kLdT of them) and
+  // step 0 of the next slab (the rest); steps 1 and 2 give them time to land
+  constexpr int kLdT = kL / 2, kLd0 = kL - kLdT;
+  // one slab: on entry set 0 holds (or is receiving) K step 0 of slab s and the first
+  // kLdT loads of slab s+1 are issued
+  auto slab = [&](bool full) __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    step(0, 1, kLdT, kLd0, full);
+    next_slab();
+    step(1, 2, 0, 0, full);
+    step(0, 3, 0, 0, full);
+    // every read of this slab's buffer has returned once set 1 is complete; then the
+    // barrier says: slab s+1 has landed for everybody, this buffer is free
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int i = 0; i < kMI; ++i)
+    for (int kk = 0; kk < 4; ++kk) { a_rd[kk] ^= kABytes; b_rd[kk] ^= kBBytes; }
+    // K step 3 of slab s, under it the reads of step 0 of slab s+1 and the first loads
+    // of slab s+2
+    step(1, 0, 0, kLdT, full);
+  };
+
+  const int nslab = (K + kTK - 1) / kTK;
+#pragma unroll
+  for (int l = 0; l < kL; ++l) issue_one(l, false);
+  next_slab();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  // past the last slab every lane is out of range: zeros go into the free buffer
+#pragma unroll
+  for (int l = 0; l < kLdT; ++l) issue_one(l, false);
+#pragma unroll
+  for (int f = 0; f < kMI + kNI; ++f) read_one(0, 0, f);
+  // slab s issues loads of slabs s+1 and s+2: no K-edge predicate while (s+3)*64 <= K
+  const int nfull = max(K / kTK - 2, 0);
+  int s = 0;
+  for (; s < nfull; ++s) slab(true);
+  for (; s < nslab; ++s) slab(false);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  // epilogue: a lane holds row m of C and, per accumulator, columns 8 q + 4 g + {0..3}
+  // (q = 0..3).  Swapping the q-odd words of the lower half-wave with the q-even words of
+  // the upper half-wave leaves every lane with 8 consecutive columns: 16-byte stores.
+  const bool fast = (ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0) && (n0 + kTN <= N);
+#pragma unroll
+  for (int i = 0; i < kMI; ++i) {
+    const int m = m0 + wm + i * 32 + col;
 #pragma unroll
     for (int j = 0; j < kNI; ++j) {
-      const int n = n0 + wn + j * 32 + col;
-      if (n >= N) continue;
+      const f32x16& a = acc[j][i];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
-        if (m < M) C[(int64_t)m * ldc + n] = (uint16_t)f32_to_bf16_bits(acc[i][j][r]);
+      for (int h = 0; h < 2; ++h) {  // q pair (2h, 2h+1)
+        const uint32_t e0 = pack_bf16x2(a[8 * h + 0], a[8 * h + 1]), e1 = pack_bf16x2(a[8 * h + 2], a[8 * h + 3]);
+        const uint32_t o0 = pack_bf16x2(a[8 * h + 4], a[8 * h + 5]), o1 = pack_bf16x2(a[8 * h + 6], a[8 * h + 7]);
+        // lanes 32..63 of the first operand <-> lanes 0..31 of the second
+        const auto s0 = __builtin_amdgcn_permlane32_swap(e0, o0, false, false);
+        const auto s1 = __builtin_amdgcn_permlane32_swap(e1, o1, false, false);
+        // lower half: (own q-even, partner's q-even) = columns 16 h + 0..7;
+        // upper half: (partner's q-odd, own q-odd) = columns 16 h + 8..15
+        u32x4 v;
+        v.x = s0[0]; v.y = s1[0]; v.z = s0[1]; v.w = s1[1];
+        const int n = n0 + wn + j * 32 + 16 * h + 8 * g;
+        if (fast) {
+          if (m < M) *reinterpret_cast<u32x4*>(&C[(int64_t)m * ldc + n]) = v;
+        } else if (m < M) {
+          const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n + e < N) C[(int64_t)m * ldc + n + e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+        }
       }
     }
+  }
 }
 
 }  // namespace spx
@@ -218,21 +324,28 @@ extern "C" int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64
   SPX_REQUIRE(((M - 1) * lda + K) * 2 < 0x7ffffff0ll && ((N - 1) * ldb + K) * 2 < 0x7ffffff0ll,
               "each operand must span less than 2 GiB (32-bit buffer offsets)");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_bf16_nt_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kGemmSmem);
+  const bool imm = lda >= kTK && ldb >= kTK;
+  static bool attr_set[2] = {false, false};
+  const void* fn = imm ? reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<true>)
+                       : reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<false>);
+  if (!attr_set[imm]) {
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kGemmSmem);
     if (e != hipSuccess) {
       last_error() = std::string("spx_gemm_bf16_nt: hipFuncSetAttribute: ") + hipGetErrorString(e);
       return SPX_ERR_HIP;
     }
-    attr_set = true;
+    attr_set[imm] = true;
   }
   const int tiles_m = (int)((M + kTM - 1) / kTM), tiles_n = (int)((N + kTN - 1) / kTN);
   SPX_REQUIRE((int64_t)tiles_m * tiles_n < (1ll << 31), "too many tiles");
-  hipLaunchKernelGGL(gemm_bf16_nt_kernel, dim3((unsigned)(tiles_m * tiles_n)), dim3(kGemmThreads),
-                     kGemmSmem, st, reinterpret_cast<const uint16_t*>(a), lda,
-                     reinterpret_cast<const uint16_t*>(b), ldb, reinterpret_cast<uint16_t*>(c), ldc,
-                     (int)M, (int)N, (int)K, tiles_m, tiles_n);
+  const dim3 grid((unsigned)(tiles_m * tiles_n)), block(kGemmThreads);
+  if (imm)
+    hipLaunchKernelGGL(gemm_bf16_nt_kernel<true>, grid, block, kGemmSmem, st,
+                       reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,
+                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n);
+  else
+    hipLaunchKernelGGL(gemm_bf16_nt_kernel<false>, grid, block, kGemmSmem, st,
+                       reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,
+                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n);
   return check_launch(__func__);
 }
