@@ -92,6 +92,26 @@ int spx_fused_vocab_loss_bwd(int op, const void* logits, int64_t ld_logits,
                              const float* row_grad, const float* scale,
                              void* grad_logits, int64_t ld_grad, void* stream);
 
+/* Cross-entropy of full-vocabulary logits against integer labels, the loss of
+ * the multi-token-prediction path: loss[r] = logsumexp(logits[r, :]) -
+ * logits[r, labels[r]], 0 where labels[r] == ignore_index (such rows are not
+ * read unless argmax is requested); lse[r] is kept for the backward; argmax
+ * (may be NULL) = first index of the row maximum.  A label outside [0, vocab)
+ * other than ignore_index gives NaN.  fp32 statistics whatever `dtype` is.
+ * Replaces F.cross_entropy(logits.permute(0, 2, 1), targets, ignore_index=-100,
+ * reduction="none") of models/mtp/core.py:204-216. */
+int spx_label_ce_fwd(const void* logits, int64_t ld_logits, const int64_t* labels,
+                     int64_t rows, int64_t vocab, int dtype, int64_t ignore_index,
+                     float* loss, float* lse, int32_t* argmax, void* stream);
+
+/* dlogits[r, j] = grad_rows[r] * (softmax(logits[r, :])[j] - [j == labels[r]]);
+ * rows with grad_rows[r] == 0 or an ignored label are exact zeros and are not
+ * read.  The autograd backward of the call above (models/mtp/core.py:204-218). */
+int spx_label_ce_bwd(const void* logits, int64_t ld_logits, const int64_t* labels,
+                     const float* lse, const float* grad_rows, int64_t rows,
+                     int64_t vocab, int dtype, int64_t ignore_index, void* dlogits,
+                     int64_t ld_out, void* stream);
+
 /* Masked mean and acceptance chain of one TTT step over `rows` aligned rows:
  *   out[0] = weight * sum_r loss[r] * m_r / (sum_r m_r + 1e-5)
  *            (loss_function, losses/utils.py:269-304, with the exp_loss_decay
@@ -152,7 +172,7 @@ int64_t spx_ttt_attn_workspace_bytes(int64_t T, int32_t Hq, int32_t Hkv,
  *   q   bf16 [Hq, T, D]  (head stride q_head_stride elements, rows contiguous)
  *   k,v bf16 [Hkv, (ttt_step+1)*T, D]  (the cache layout of DynamicCache)
  *   out bf16 [T, Hq, D];  lse f32 [Hq, T]: log2-domain row log-sum-exp, opaque,
- *   consumed by spx_ttt_attn_bwd.   D in {64, 128}. */
+ *   consumed by spx_ttt_attn_bwd.   D in {64, 128, 256}. */
 int spx_ttt_attn_fwd(const void* q, int64_t q_head_stride, const void* k,
                      int64_t k_head_stride, const void* v, int64_t v_head_stride,
                      const int32_t* row_lo, int64_t T, int32_t ttt_step,

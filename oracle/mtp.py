@@ -1,0 +1,178 @@
+"""CPU restatement of the MTP (multi-token prediction) training forward.
+
+TEST INFRASTRUCTURE ONLY: nothing under ``speculators_amd`` may import this.
+
+Follows, in plain PyTorch on the CPU:
+  * ``compute_step_weights``            models/mtp/core.py:29-38
+  * ``MTPDraftModel.forward``           models/mtp/core.py:114-231
+  * ``MTPLayerMixin.forward``           models/mtp/model_definitions.py:95-116
+  * the Qwen3 decoder layer it wraps    transformers ``modeling_qwen3.py``
+    (pre-norm attention with per-head q/k RMSNorm, SwiGLU MLP)
+  * the packed-sequence causal mask     transformers ``masking_utils.py``
+    ``find_packed_sequence_indices`` (called through ``create_causal_mask`` with
+    ``attention_mask=None`` at models/mtp/core.py:180-186)
+
+Pinned by: the block-diagonal causal matrix of
+tests/unit/models/test_mtp_attention.py:17-55 (documents [1, 3, 2]), the loss
+properties of tests/unit/models/test_mtp_model.py (all-zero mask -> exactly 0,
+zero step weight -> that step's loss 0, short sequences give fewer steps), the
+closed form of the step weights, ``F.cross_entropy`` (a library routine) for the
+loss, and agreement of the dense attention with ``F.scaled_dot_product_attention``.
+Whole-model values on random weights have no golden vector in the reference.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+from .attention import dense_attention
+from .eagle3 import DraftShape, apply_rope, rms_norm, rope_tables, swiglu_mlp
+
+IGNORE_INDEX = -100
+
+
+def compute_step_weights(beta: float = 0.6, num_steps: int = 3) -> list[float]:
+    """alpha_k = beta^k / sum_j beta^j, k = 0..K-1 (models/mtp/core.py:29-38)."""
+    raw = [beta**k for k in range(num_steps)]
+    total = sum(raw)
+    return [r / total for r in raw]
+
+
+def packed_sequence_ids(position_ids: torch.Tensor) -> torch.Tensor:
+    """``[B, L]`` positions -> ``[B, L]`` sequence index inside each row: a new sequence
+    starts wherever the position does not grow by exactly one."""
+    first = position_ids[:, :1] - 1
+    diff = torch.diff(position_ids, prepend=first, dim=-1)
+    return (diff != 1).cumsum(-1)
+
+
+def packed_causal_mask(position_ids: torch.Tensor) -> torch.Tensor:
+    """Dense bool ``[B, L, L]``: query i sees key j iff j <= i and both lie in the same
+    packed sequence of the row."""
+    seq = packed_sequence_ids(position_ids)
+    n = position_ids.shape[1]
+    idx = torch.arange(n)
+    causal = idx[:, None] >= idx[None, :]
+    return causal[None] & (seq[:, :, None] == seq[:, None, :])
+
+
+def _qwen3_layer(x, w, p, shape: DraftShape, cos, sin, mask, attn):
+    """One row ``[1, L, H]`` through the Qwen3 decoder layer."""
+    n = x.shape[1]
+    hq, hkv, d = shape.num_attention_heads, shape.num_key_value_heads, shape.head_dim
+    a = p + "self_attn."
+    y = rms_norm(x, w[p + "input_layernorm.weight"], shape.rms_norm_eps)
+    q = rms_norm(F.linear(y, w[a + "q_proj.weight"]).view(1, n, hq, d), w[a + "q_norm.weight"],
+                 shape.rms_norm_eps).transpose(1, 2)
+    k = rms_norm(F.linear(y, w[a + "k_proj.weight"]).view(1, n, hkv, d), w[a + "k_norm.weight"],
+                 shape.rms_norm_eps).transpose(1, 2)
+    v = F.linear(y, w[a + "v_proj.weight"]).view(1, n, hkv, d).transpose(1, 2)
+    q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+    if attn == "sdpa":
+        g = hq // hkv
+        o = F.scaled_dot_product_attention(q, k.repeat_interleave(g, 1), v.repeat_interleave(g, 1),
+                                           attn_mask=mask[None, None], scale=d**-0.5)
+        o = o.transpose(1, 2).contiguous()
+    else:
+        o = dense_attention(q, k, v, mask, d**-0.5)
+    x = x + F.linear(o.reshape(1, n, hq * d), w[a + "o_proj.weight"])
+    z = rms_norm(x, w[p + "post_attention_layernorm.weight"], shape.rms_norm_eps)
+    return x + swiglu_mlp(z, w, p + "mlp.")
+
+
+def mtp_layer(hidden, embeds, w, shape: DraftShape, cos, sin, mask, attn="dense"):
+    """models/mtp/model_definitions.py:95-116 on one row."""
+    p = "mtp_layers.0."
+    hn = rms_norm(hidden, w[p + "hidden_layernorm.weight"], shape.rms_norm_eps)
+    en = rms_norm(embeds, w[p + "token_layernorm.weight"], shape.rms_norm_eps)
+    proj = F.linear(torch.cat([en, hn], dim=-1), w[p + "input_proj.weight"])
+    out = _qwen3_layer(proj, w, p, shape, cos, sin, mask, attn)
+    return rms_norm(out, w[p + "final_layernorm.weight"], shape.rms_norm_eps)
+
+
+def mtp_forward(w, shape: DraftShape, input_ids, hidden_states, position_ids=None, loss_mask=None,
+                step_weights=None, num_steps: int = 3, attn: str = "dense"):
+    """``(logits_list, loss, metrics)`` of models/mtp/core.py:114-231."""
+    input_ids = input_ids.long()
+    b, n = input_ids.shape
+    if step_weights is not None and len(step_weights) != num_steps:
+        raise ValueError(f"step_weights has {len(step_weights)} entries but num_speculative_steps="
+                         f"{num_steps}; expected exactly {num_steps} weights.")
+    if position_ids is None:
+        position_ids = torch.arange(n).unsqueeze(0).expand(b, -1)
+    logits_list = []
+    total = torch.tensor(0.0)
+    metrics = {}
+    steps = min(num_steps, max(0, n - 2))
+    valid = n - steps - 1
+    if valid <= 0 or steps == 0:
+        metrics["loss_sum"] = total.clone()
+        metrics["loss_total"] = torch.tensor(1.0)
+        return logits_list, total, metrics
+    pos = position_ids[:, :valid]
+    masks = packed_causal_mask(pos)
+    current = hidden_states
+    for step in range(steps):
+        hid = current[:, :valid]
+        emb = F.embedding(input_ids[:, step + 1:step + 1 + valid], w["embed_tokens.weight"])
+        rows = []
+        for r in range(b):
+            cos, sin = rope_tables(pos[r], shape.head_dim, shape.rope_theta, hid.dtype)
+            rows.append(mtp_layer(hid[r:r + 1], emb[r:r + 1].to(hid.dtype), w, shape, cos, sin,
+                                  masks[r], attn))
+        out = torch.cat(rows, dim=0)
+        logits = F.linear(out, w["lm_head.weight"])
+        logits_list.append(logits)
+        tgt = input_ids[:, step + 2:step + 2 + valid]
+        if loss_mask is not None:
+            tgt = tgt.clone()
+            tgt[loss_mask[:, step + 2:step + 2 + valid] == 0] = IGNORE_INDEX
+        weight = step_weights[step] if step_weights is not None else 1.0
+        unreduced = F.cross_entropy(logits.permute(0, 2, 1).float(), tgt, ignore_index=IGNORE_INDEX,
+                                    reduction="none")
+        count = (tgt != IGNORE_INDEX).sum()
+        step_loss = weight * unreduced.sum() / count.clamp(min=1)
+        total = total + step_loss
+        metrics[f"loss_step_{step}"] = step_loss.detach().clone()
+        current = out
+    metrics["loss_sum"] = total.detach().clone()
+    metrics["loss_total"] = torch.tensor(1.0)
+    return logits_list, total, metrics
+
+
+def random_weights(shape: DraftShape, seed: int = 0, dtype=torch.float32, std: float = 0.02):
+    """Seeded weights keyed by the MTP state-dict names (models/mtp/core.py:41-96,
+    models/mtp/model_definitions.py:85-93).  Norm weights are 1 + noise so that a missing
+    or swapped norm shows."""
+    g = torch.Generator().manual_seed(seed)
+    h, hq, hkv, d = (shape.hidden_size, shape.num_attention_heads,
+                     shape.num_key_value_heads, shape.head_dim)
+    f = shape.intermediate_size
+
+    def rnd(*s):
+        return (torch.randn(*s, generator=g) * std).to(dtype)
+
+    def nrm(k):
+        return (1.0 + 0.1 * torch.randn(k, generator=g)).to(dtype)
+
+    p = "mtp_layers.0."
+    return {
+        "embed_tokens.weight": (torch.randn(shape.vocab_size, h, generator=g)).to(dtype),
+        "lm_head.weight": rnd(shape.vocab_size, h),
+        p + "hidden_layernorm.weight": nrm(h),
+        p + "token_layernorm.weight": nrm(h),
+        p + "input_proj.weight": rnd(h, 2 * h),
+        p + "final_layernorm.weight": nrm(h),
+        p + "input_layernorm.weight": nrm(h),
+        p + "post_attention_layernorm.weight": nrm(h),
+        p + "self_attn.q_proj.weight": rnd(hq * d, h),
+        p + "self_attn.k_proj.weight": rnd(hkv * d, h),
+        p + "self_attn.v_proj.weight": rnd(hkv * d, h),
+        p + "self_attn.o_proj.weight": rnd(h, hq * d),
+        p + "self_attn.q_norm.weight": nrm(d),
+        p + "self_attn.k_norm.weight": nrm(d),
+        p + "mlp.gate_proj.weight": rnd(f, h),
+        p + "mlp.up_proj.weight": rnd(f, h),
+        p + "mlp.down_proj.weight": rnd(h, f),
+    }

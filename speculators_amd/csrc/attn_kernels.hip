@@ -197,7 +197,7 @@ __device__ __forceinline__ void load_bounds(const AttnParams& p, const int (&ic)
 #define SPX_DKV_MINB 1
 #endif
 template <int D, int NSB, int NW, bool PF>
-__global__ __launch_bounds__(64 * NW, SPX_FWD_MINB) void attn_fwd_kernel(AttnParams p,
+__global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_kernel(AttnParams p,
                                                                 const uint16_t* __restrict__ Vt,
                                                                 uint16_t* __restrict__ O,
                                                                 float* __restrict__ LSE) {
@@ -461,7 +461,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const uint16_t* __restr
 // dQ: same tiling as the forward.
 //   P^T = exp2(S'^T - lse), dP^T = V dO^T, dS^T = P^T (dP^T - delta), dQ^T += K^T dS^T
 template <int D, int NSB, int NW, bool PF>
-__global__ __launch_bounds__(64 * NW, SPX_DQ_MINB) void attn_bwd_dq_kernel(
+__global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_dq_kernel(
     AttnParams p, const uint16_t* __restrict__ dO, const uint16_t* __restrict__ Kt,
     const float* __restrict__ LSE, const float* __restrict__ Delta, uint16_t* __restrict__ dQ,
     int64_t dq_hs) {
@@ -1127,7 +1127,7 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
 static int shape_checks(const char* fn, int64_t NQ, int64_t NKV, int32_t Hq, int32_t Hkv, int32_t D) {
   if (!(NQ > 0 && NQ < (1ll << 24) && NKV > 0 && NKV < (1ll << 26))) return fail_arg(fn, "sequence length out of range");
   if (!(Hkv > 0 && Hq > 0 && Hq % Hkv == 0)) return fail_arg(fn, "Hq must be a multiple of Hkv");
-  if (!(D == 64 || D == 128)) return fail_arg(fn, "head_dim must be 64 or 128");
+  if (!(D == 64 || D == 128 || D == 256)) return fail_arg(fn, "head_dim must be 64, 128 or 256");
   return SPX_OK;
 }
 
@@ -1195,6 +1195,7 @@ extern "C" int spx_ttt_attn_fwd(const void* q, int64_t q_head_stride, const void
   AttnParams p = ttt_params(q, q_head_stride, k, k_head_stride, v, v_head_stride, row_lo, T, ttt_step,
                             Hq, Hkv, scaling);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (D == 256) return launch_fwd<256>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
   if (D == 128) return launch_fwd<128>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
   return launch_fwd<64>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
 }
@@ -1226,6 +1227,9 @@ extern "C" int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void
   auto dQp = reinterpret_cast<uint16_t*>(dq);
   auto dKp = reinterpret_cast<uint16_t*>(dk);
   auto dVp = reinterpret_cast<uint16_t*>(dv);
+  if (D == 256)
+    return launch_bwd<256>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp, dv_head_stride,
+                           workspace, st, __func__);
   if (D == 128)
     return launch_bwd<128>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp,
                            dv_head_stride, workspace, st, __func__);
@@ -1302,6 +1306,7 @@ extern "C" int spx_dflash_attn_fwd(const void* q, int64_t q_head_stride, const v
   AttnParams p = dflash_params(q, q_head_stride, k, k_head_stride, v, v_head_stride, ctx_lo, ctx_hi,
                                blk_lo, blk_hi, T, NQ, Hq, Hkv, scaling);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (D == 256) return launch_fwd<256>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
   if (D == 128) return launch_fwd<128>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
   return launch_fwd<64>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
 }
@@ -1334,6 +1339,9 @@ extern "C" int spx_dflash_attn_bwd(const void* q, int64_t q_head_stride, const v
   auto dQp = reinterpret_cast<uint16_t*>(dq);
   auto dKp = reinterpret_cast<uint16_t*>(dk);
   auto dVp = reinterpret_cast<uint16_t*>(dv);
+  if (D == 256)
+    return launch_bwd<256>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp, dv_head_stride,
+                           workspace, st, __func__);
   if (D == 128)
     return launch_bwd<128>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp,
                            dv_head_stride, workspace, st, __func__);

@@ -16,6 +16,8 @@ import torch
 
 from . import _lib
 
+_MAX_SPAN = 0x7ffffff0 - 64  # bytes one GEMM operand may span
+
 
 def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """``a[M, K] @ b[N, K].T -> [M, N]`` (bf16, fp32 accumulation)."""
@@ -31,8 +33,18 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -
     n = b.shape[0]
     if out is None:
         out = torch.empty(m, n, device=a.device, dtype=torch.bfloat16)
-    _lib.call("spx_gemm_bf16_nt", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
-              _lib.ptr(out), out.stride(0), m, n, k, _lib.stream_ptr(a.device))
+    # the kernel addresses each operand with 32-bit byte offsets: an operand that spans
+    # 2 GiB or more is fed in row bands (full-vocabulary logits gradients are that large)
+    rows_a = max(_MAX_SPAN // (2 * a.stride(0)), 1) if m > 1 else 1
+    rows_b = max(_MAX_SPAN // (2 * b.stride(0)), 1) if n > 1 else 1
+    st = _lib.stream_ptr(a.device)
+    for m0 in range(0, m, max(rows_a, 1)):
+        am = a[m0:m0 + rows_a]
+        for n0 in range(0, n, max(rows_b, 1)):
+            bn = b[n0:n0 + rows_b]
+            o = out[m0:m0 + rows_a, n0:n0 + rows_b]
+            _lib.call("spx_gemm_bf16_nt", _lib.ptr(am), am.stride(0), _lib.ptr(bn), bn.stride(0),
+                      _lib.ptr(o), o.stride(0), am.shape[0], bn.shape[0], k, st)
     return out
 
 

@@ -193,6 +193,49 @@ def resolve_loss_config(spec: str, implementation: str = "hip") -> LossConfig:
     return out
 
 
+class _LabelCE(torch.autograd.Function):
+    """Per-row cross-entropy of ``logits [R, V]`` against integer ``labels [R]`` with an
+    ignore index, on the HIP label-CE kernels (one read of the logits in the forward, one
+    read + one write in the backward)."""
+
+    @staticmethod
+    def forward(ctx, logits2d, labels, ignore_index):
+        rows, vocab = logits2d.shape
+        dev = logits2d.device
+        out = torch.empty(2, rows, device=dev, dtype=torch.float32)
+        _lib.call("spx_label_ce_fwd", _lib.ptr(logits2d), logits2d.stride(0), _lib.ptr(labels), rows,
+                  vocab, _lib.dtype_code(logits2d), int(ignore_index), _lib.ptr(out[0]),
+                  _lib.ptr(out[1]), None, _lib.stream_ptr(dev))
+        ctx.save_for_backward(logits2d, labels, out[1])
+        ctx.ignore_index = int(ignore_index)
+        return out[0]
+
+    @staticmethod
+    def backward(ctx, grad_rows):
+        logits2d, labels, lse = ctx.saved_tensors
+        rows, vocab = logits2d.shape
+        g = grad_rows.to(torch.float32).contiguous()
+        dlogits = torch.empty(rows, vocab, device=logits2d.device, dtype=logits2d.dtype)
+        _lib.call("spx_label_ce_bwd", _lib.ptr(logits2d), logits2d.stride(0), _lib.ptr(labels),
+                  _lib.ptr(lse), _lib.ptr(g), rows, vocab, _lib.dtype_code(logits2d),
+                  ctx.ignore_index, _lib.ptr(dlogits), dlogits.stride(0),
+                  _lib.stream_ptr(logits2d.device))
+        return dlogits, None, None
+
+
+def label_cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int = -100):
+    """``F.cross_entropy(logits.permute(0, 2, 1), labels, ignore_index=..., reduction="none")``
+    (models/mtp/core.py:204-216) for ``logits [..., V]`` (bf16 or fp32) and integer ``labels
+    [...]``: returns float32 losses of the shape of ``labels``, 0 at ignored positions."""
+    if logits.shape[:-1] != labels.shape:
+        raise ValueError(f"logits {tuple(logits.shape)} and labels {tuple(labels.shape)} do not match")
+    if logits.dtype not in (torch.bfloat16, torch.float32):
+        raise _lib.SpxError("label_cross_entropy takes bf16 or fp32 logits")
+    x = _rows_2d(logits)
+    lab = labels.reshape(-1).to(torch.int64).contiguous()
+    return _LabelCE.apply(x, lab, ignore_index).view(labels.shape)
+
+
 def vocab_gather(full_logits: torch.Tensor, d2t: torch.Tensor) -> torch.Tensor:
     """``full_logits[..., i + d2t[i]]`` on the device: verifier logits over the target
     vocabulary restricted to the draft vocabulary (the gather form of the t2d row-slice,

@@ -1,0 +1,194 @@
+"""MTP (multi-token prediction) draft model: host side of the HIP training path.
+
+Keeps the call contract of ``MTPDraftModel.forward`` (models/mtp/core.py:114-231):
+
+    forward(input_ids, hidden_states, attention_mask=None, position_ids=None,
+            loss_mask=None, step_weights=None) -> (logits_list, loss, metrics)
+
+with the reference's metric keys (``loss_step_{k}``, ``loss_sum``, ``loss_total``) and
+state-dict names (``mtp_layers.0.*``, ``embed_tokens``, ``lm_head``).  The layer is
+the Qwen3 flavour of ``MTPLayerMixin`` (models/mtp/model_definitions.py:78-151):
+two RMSNorms, ``input_proj (2H -> H)``, a Qwen3 decoder layer with per-head q/k
+RMSNorm, a final RMSNorm.  Attention runs on the HIP interval-masked kernel (causal
+inside each packed sequence, sequences found from the position restarts as
+``create_causal_mask`` does at models/mtp/core.py:180-186), ``lm_head`` on the MFMA
+GEMM, the loss on the label cross-entropy kernel.
+
+A batch ``[B, L]`` is laid out as one packed row ``[1, B*L]`` whose sequences never
+cross a batch row: every op other than attention is row-wise, and attention sees
+the same keys.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import attention as A
+from . import fused_ops as FO
+from . import gemm
+from . import losses as L
+from .eagle3 import MLP, Attention, RMSNorm
+
+IGNORE_INDEX = -100
+
+
+def compute_step_weights(beta: float = 0.6, num_steps: int = 3) -> list[float]:
+    """Normalised exponential-decay step weights (models/mtp/core.py:29-38)."""
+    raw = [beta**k for k in range(num_steps)]
+    total = sum(raw)
+    return [w / total for w in raw]
+
+
+@dataclass
+class MTPConfig:
+    hidden_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    intermediate_size: int
+    vocab_size: int
+    num_speculative_steps: int = 3
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 1000000.0
+    model_type: str = "qwen3"
+    attn_implementation: str = A.ATTN_IMPL_TTT
+    qk_norm: bool = True  # Qwen3 attention
+
+
+class MTPLayer(nn.Module):
+    """``Qwen3MTPLayer`` (models/mtp/model_definitions.py:78-151)."""
+
+    def __init__(self, cfg: MTPConfig):
+        super().__init__()
+        h, eps = cfg.hidden_size, cfg.rms_norm_eps
+        self.hidden_layernorm = RMSNorm(h, eps)
+        self.token_layernorm = RMSNorm(h, eps)
+        self.input_proj = nn.Linear(2 * h, h, bias=False)
+        self.final_layernorm = RMSNorm(h, eps)
+        self.input_layernorm = RMSNorm(h, eps)
+        self.post_attention_layernorm = RMSNorm(h, eps)
+        self.self_attn = Attention(cfg, h)
+        self.mlp = MLP(cfg)
+
+    def forward(self, hidden, embeds, position_ids, inv_freq, mask):
+        x = gemm.linear_accumulate(
+            torch.cat([self.token_layernorm(embeds), self.hidden_layernorm(hidden)], dim=-1),
+            self.input_proj.weight)
+        x = x + self.self_attn(self.input_layernorm(x), position_ids, 0, inv_freq, {}, mask)
+        x = x + self.mlp(self.post_attention_layernorm(x))
+        return self.final_layernorm(x)
+
+
+class MTPDraftModel(nn.Module):
+    def __init__(self, config: MTPConfig):
+        super().__init__()
+        if config.model_type != "qwen3":
+            raise ValueError(f"Unsupported MTP model type '{config.model_type}'. Supported types: ['qwen3']")
+        self.config = config
+        self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size)
+        self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
+        self.mtp_layers = nn.ModuleList([MTPLayer(config)])
+        # the verifier's embedding and head are frozen (model.py:70-71)
+        self.embed_tokens.weight.requires_grad_(False)
+        self.lm_head.weight.requires_grad_(False)
+        self._frozen_t: dict = {}
+
+    @property
+    def layers(self) -> nn.ModuleList:
+        return self.mtp_layers
+
+    def _lm_head(self, x):
+        w = self.lm_head.weight
+        wt = None
+        if x.requires_grad:
+            key = (w.data_ptr(), w._version)
+            hit = self._frozen_t.get("lm_head")
+            if hit is None or hit[0] != key:
+                hit = (key, w.detach().t().contiguous())
+                self._frozen_t["lm_head"] = hit
+            wt = hit[1]
+        return gemm.linear(x, w, wt)
+
+    def forward(self, input_ids, hidden_states, attention_mask=None, position_ids=None,
+                loss_mask=None, step_weights=None, return_dict: bool = True, **_kwargs):
+        cfg = self.config
+        if attention_mask is not None:
+            raise NotImplementedError(
+                "the HIP MTP path takes packed rows without padding masks (attention_mask=None, "
+                "as the training collate produces them)")
+        if hidden_states.dtype != torch.bfloat16:
+            raise RuntimeError("the HIP draft path runs in bf16: cast the model and its inputs to bfloat16")
+        input_ids = input_ids.long()
+        device = input_ids.device
+        b, n = input_ids.shape
+        num_steps = cfg.num_speculative_steps
+        if step_weights is not None and len(step_weights) != num_steps:
+            raise ValueError(
+                f"step_weights has {len(step_weights)} entries but num_speculative_steps={num_steps}; "
+                f"expected exactly {num_steps} weights.")
+        if position_ids is None:
+            position_ids = torch.arange(n, device=device).unsqueeze(0).expand(b, -1)
+
+        all_logits: list[torch.Tensor] = []
+        total_loss = torch.tensor(0.0, device=device)
+        metrics: dict = {}
+        steps = min(num_steps, max(0, n - 2))
+        valid = n - steps - 1
+        if valid <= 0 or steps == 0:
+            metrics["loss_sum"] = total_loss.detach().clone()
+            metrics["loss_total"] = torch.tensor(1.0, device=device)
+            return all_logits, total_loss, metrics
+
+        pos = position_ids[:, :valid].to(torch.int64)
+        # sequence index inside each row (a new sequence wherever the position does not grow
+        # by one), made unique across rows: the packed row [1, B * valid] never mixes rows
+        diff = torch.diff(pos, prepend=pos[:, :1] - 1, dim=-1)
+        seq = (diff != 1).cumsum(-1) + torch.arange(b, device=device).unsqueeze(1) * (valid + 1)
+        mask = A.create_ttt_mask(seq.reshape(-1), b * valid, None)
+        flat_pos = pos.reshape(-1).contiguous()
+        inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device)
+        layer = self.mtp_layers[0]
+
+        current = hidden_states
+        for step in range(steps):
+            hid = current[:, :valid].reshape(1, b * valid, cfg.hidden_size)
+            with torch.no_grad():
+                emb = F.embedding(input_ids[:, step + 1:step + 1 + valid], self.embed_tokens.weight)
+                emb = emb.to(hidden_states.dtype).reshape(1, b * valid, cfg.hidden_size)
+            out = layer(hid, emb, flat_pos, inv_freq, mask)
+            logits = self._lm_head(out).view(b, valid, cfg.vocab_size)
+            all_logits.append(logits)
+
+            targets = input_ids[:, step + 2:step + 2 + valid]
+            if loss_mask is not None:
+                targets = targets.clone()
+                targets[loss_mask[:, step + 2:step + 2 + valid] == 0] = IGNORE_INDEX
+            weight = step_weights[step] if step_weights is not None else 1.0
+            unreduced = L.label_cross_entropy(logits, targets, IGNORE_INDEX)
+            valid_count = (targets != IGNORE_INDEX).sum()
+            step_loss = weight * unreduced.sum() / valid_count.clamp(min=1)
+            total_loss = total_loss + step_loss
+            metrics[f"loss_step_{step}"] = step_loss.detach().clone()
+            current = out.view(b, valid, cfg.hidden_size)
+
+        metrics["loss_sum"] = total_loss.detach().clone()
+        metrics["loss_total"] = torch.tensor(1.0, device=device)
+        return all_logits, total_loss, metrics
+
+    @staticmethod
+    def get_trainer_kwargs(**kwargs):
+        """(train_call_kwargs, val_call_kwargs): ``step_weights`` as given, else computed from
+        ``step_weight_beta`` and ``num_speculative_steps`` (models/mtp/core.py:280-304)."""
+        step_weights = kwargs.get("step_weights")
+        if step_weights is None:
+            if "num_speculative_steps" not in kwargs:
+                raise ValueError("num_speculative_steps must be set from the model config "
+                                 "before calling get_trainer_kwargs")
+            step_weights = compute_step_weights(beta=kwargs.get("step_weight_beta", 0.6),
+                                                num_steps=kwargs["num_speculative_steps"])
+        train_kwargs = {"step_weights": step_weights}
+        return train_kwargs, train_kwargs.copy()

@@ -1,0 +1,210 @@
+"""HIP MTP path (label cross-entropy kernel, head_dim-256 attention, whole model) against
+the CPU oracle, through the C ABI."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import masks as OMK
+from oracle import mtp as OM
+from oracle.attention import dense_attention
+from oracle.eagle3 import DraftShape
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("rows,vocab,dtype", [(37, 1000, torch.float32), (64, 50257, torch.bfloat16),
+                                              (16, 151936, torch.bfloat16), (5, 7, torch.float32)])
+def test_label_ce_matches_torch_cross_entropy(rows, vocab, dtype):
+    from speculators_amd.losses import label_cross_entropy
+
+    g = torch.Generator().manual_seed(rows + vocab)
+    x = (torch.randn(rows, vocab, generator=g) * 3).to(dtype)
+    lab = torch.randint(0, vocab, (rows,), generator=g)
+    lab[::5] = -100
+    go = torch.randn(rows, generator=g)
+    go[1::7] = 0
+    xg = x.cuda().requires_grad_(True)
+    loss = label_cross_entropy(xg, lab.cuda())
+    loss.backward(go.cuda())
+    xr = x.float().requires_grad_(True)
+    ref = F.cross_entropy(xr, lab, ignore_index=-100, reduction="none")
+    ref.backward(go)
+    assert loss.dtype == torch.float32 and loss.shape == (rows,)
+    torch.testing.assert_close(loss.cpu(), ref, rtol=1e-5, atol=2e-5)
+    assert (loss.cpu()[lab == -100] == 0).all()
+    tol = 1e-6 if dtype == torch.float32 else 4e-3  # bf16 gradient rounding: 2^-8 relative
+    err = (xg.grad.float().cpu() - xr.grad).abs().max().item()
+    assert err <= tol * xr.grad.abs().max().item() + 1e-9, err
+    # ignored rows and rows without upstream gradient are exact zeros
+    dead = (lab == -100) | (go == 0)
+    assert (xg.grad.cpu()[dead] == 0).all()
+
+
+def test_label_ce_strided_rows_and_argmax_first_index():
+    from speculators_amd import _lib
+
+    g = torch.Generator().manual_seed(1)
+    full = torch.randn(9, 300, generator=g).bfloat16()
+    full[2, 17] = full[2, 250] = 9.0   # tie: the first index wins
+    full[4, :] = 1.0                   # all equal
+    x = full.cuda()[:, 3:203]          # unaligned, strided rows
+    lab = torch.randint(0, 200, (9,), generator=g).cuda()
+    out = torch.empty(2, 9, device="cuda")
+    am = torch.empty(9, dtype=torch.int32, device="cuda")
+    _lib.call("spx_label_ce_fwd", _lib.ptr(x), x.stride(0), _lib.ptr(lab), 9, 200, 0, -100,
+              _lib.ptr(out[0]), _lib.ptr(out[1]), _lib.ptr(am), _lib.stream_ptr(x.device))
+    xs = full[:, 3:203].float()
+    assert torch.equal(am.cpu().long(), xs.argmax(-1))
+    assert am[2].item() == 14 and am[4].item() == 0
+    torch.testing.assert_close(out[1].cpu(), torch.logsumexp(xs, -1), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(out[0].cpu(), F.cross_entropy(xs, lab.cpu(), reduction="none"),
+                               rtol=1e-5, atol=2e-5)
+
+
+def test_label_ce_bad_label_is_nan_and_errors():
+    from speculators_amd import _lib
+    from speculators_amd.losses import label_cross_entropy
+
+    x = torch.randn(3, 40).cuda()
+    lab = torch.tensor([1, 40, -5]).cuda()
+    out = label_cross_entropy(x, lab)
+    assert torch.isfinite(out[0]) and torch.isnan(out[1]) and torch.isnan(out[2])
+    with pytest.raises(ValueError):
+        label_cross_entropy(x, lab[:2])
+    with pytest.raises(_lib.SpxError):
+        label_cross_entropy(x.half(), lab)
+
+
+def test_gemm_row_bands_equal_single_call(monkeypatch):
+    from speculators_amd import gemm
+
+    g = torch.Generator().manual_seed(0)
+    a = torch.randn(700, 256, generator=g).bfloat16().cuda()
+    b = torch.randn(520, 256, generator=g).bfloat16().cuda()
+    want = gemm.gemm_nt(a, b)
+    monkeypatch.setattr(gemm, "_MAX_SPAN", 256 * 2 * 300)  # bands of 300 rows
+    got = gemm.gemm_nt(a, b)
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("t,hq,hkv,docs", [(192, 2, 1, [192]), (300, 4, 2, [100, 130, 70])])
+def test_attention_head_dim_256(t, hq, hkv, docs):
+    from speculators_amd.attention import create_ttt_mask, ttt_attention
+
+    d = 256
+    g = torch.Generator().manual_seed(t)
+    doc = torch.cat([torch.full((n,), i) for i, n in enumerate(docs)])
+    mask = create_ttt_mask(doc.cuda(), t, None)
+    q = torch.randn(1, hq, t, d, generator=g).bfloat16()
+    k = torch.randn(1, hkv, t, d, generator=g).bfloat16()
+    v = torch.randn(1, hkv, t, d, generator=g).bfloat16()
+    go = torch.randn(1, t, hq, d, generator=g).bfloat16()
+    qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    out = ttt_attention(qg, kg, vg, mask, d ** -0.5)
+    out.backward(go.cuda())
+    qr, kr, vr = (x.float().requires_grad_(True) for x in (q, k, v))
+    ref = dense_attention(qr, kr, vr, OMK.ttt_mask_dense(doc, t, 0, None), d ** -0.5)
+    ref.backward(go.float())
+    err = (out.float().cpu() - ref).abs().max().item()
+    assert err <= 2e-2 * ref.abs().max().item(), err
+    for name, got, want in (("dq", qg.grad, qr.grad), ("dk", kg.grad, kr.grad), ("dv", vg.grad, vr.grad)):
+        err = (got.float().cpu() - want).abs().max().item()
+        assert err <= 2e-2 * want.abs().max().item(), (name, err, want.abs().max().item())
+
+
+def _shape(**kw):
+    base = dict(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=64,
+                intermediate_size=512, vocab_size=1000, draft_vocab_size=1000, rms_norm_eps=1e-6,
+                rope_theta=10000.0, qk_norm=True)
+    base.update(kw)
+    return DraftShape(**base)
+
+
+def _make(shape, w, steps):
+    from speculators_amd.mtp import MTPConfig, MTPDraftModel
+
+    cfg = MTPConfig(hidden_size=shape.hidden_size, num_attention_heads=shape.num_attention_heads,
+                    num_key_value_heads=shape.num_key_value_heads, head_dim=shape.head_dim,
+                    intermediate_size=shape.intermediate_size, vocab_size=shape.vocab_size,
+                    num_speculative_steps=steps, rms_norm_eps=shape.rms_norm_eps,
+                    rope_theta=shape.rope_theta)
+    model = MTPDraftModel(cfg)
+    missing, unexpected = model.load_state_dict(w, strict=True)
+    return model.to(torch.bfloat16).cuda()
+
+
+@pytest.mark.parametrize("variant", [dict(), dict(head_dim=128, num_attention_heads=2, num_key_value_heads=1),
+                                     dict(head_dim=256, num_attention_heads=2, num_key_value_heads=1)])
+def test_model_forward_backward_matches_oracle(variant):
+    shape = _shape(**variant)
+    steps = 3
+    w32 = OM.random_weights(shape, seed=2, std=0.05)
+    w = {k: v.bfloat16() for k, v in w32.items()}
+    g = torch.Generator().manual_seed(5)
+    b, n = 2, 200
+    ids = torch.randint(0, shape.vocab_size, (b, n), generator=g)
+    hs = torch.randn(b, n, shape.hidden_size, generator=g).bfloat16()
+    pos = torch.stack([torch.cat([torch.arange(70), torch.arange(90), torch.arange(40)]),
+                       torch.arange(n)])
+    lm = (torch.rand(b, n, generator=g) < 0.7).float()
+    sw = OM.compute_step_weights(0.6, steps)
+
+    model = _make(shape, w, steps)
+    logits, loss, m = model(ids.cuda(), hs.cuda(), position_ids=pos.cuda(), loss_mask=lm.cuda(),
+                            step_weights=sw)
+    loss.backward()
+
+    wf = {k: v.float().requires_grad_(True) for k, v in w.items()}
+    rl, rloss, rm = OM.mtp_forward(wf, shape, ids, hs.float(), position_ids=pos, loss_mask=lm,
+                                   step_weights=sw, num_steps=steps)
+    rloss.backward()
+    rel = abs(loss.item() - rloss.item()) / abs(rloss.item())
+    print("loss", loss.item(), rloss.item(), rel)
+    assert rel < 1e-3
+    assert set(m) == set(rm)
+    for k in range(steps):
+        assert logits[k].shape == rl[k].shape == (b, n - steps - 1, shape.vocab_size)
+        err = (logits[k].float().cpu() - rl[k]).abs().max().item()
+        assert err <= 2e-2 * rl[k].abs().max().item(), (k, err)
+        assert abs(m[f"loss_step_{k}"].item() - rm[f"loss_step_{k}"].item()) <= 1e-3 * rm[f"loss_step_{k}"].item()
+    # the same oracle in bf16 on the CPU gives the rounding noise floor of this model
+    wb = {k: v.clone().requires_grad_(True) for k, v in w.items()}
+    _, bloss, _ = OM.mtp_forward(wb, shape, ids, hs, position_ids=pos, loss_mask=lm, step_weights=sw,
+                                 num_steps=steps)
+    bloss.backward()
+    for name, p in model.named_parameters():
+        if not p.requires_grad:
+            assert p.grad is None
+            continue
+        want = wf[name].grad
+        scale = want.abs().max().item()
+        err = (p.grad.float().cpu() - want).abs().max().item()
+        floor = (wb[name].grad.float() - want).abs().max().item()
+        assert err <= max(2e-2 * scale, 2 * floor) + 1e-6, (name, err, floor, scale)
+
+
+def test_model_properties_of_the_reference_tests():
+    # tests/unit/models/test_mtp_model.py on the HIP path
+    shape = _shape()
+    w = {k: v.bfloat16() for k, v in OM.random_weights(shape, seed=3, std=0.05).items()}
+    model = _make(shape, w, 3)
+    g = torch.Generator().manual_seed(9)
+    ids = torch.randint(0, shape.vocab_size, (1, 40), generator=g).cuda()
+    hs = torch.randn(1, 40, shape.hidden_size, generator=g).bfloat16().cuda()
+    with torch.no_grad():
+        logits, loss, m = model(ids, hs)
+        assert len(logits) == 3 and logits[0].shape == (1, 36, shape.vocab_size)
+        assert set(m) == {"loss_step_0", "loss_step_1", "loss_step_2", "loss_sum", "loss_total"}
+        _, l0, _ = model(ids, hs, loss_mask=torch.zeros(1, 40, device="cuda"))
+        assert l0.item() == 0.0
+        _, _, mz = model(ids, hs, step_weights=[1.0, 0.0, 0.0])
+        assert mz["loss_step_0"] > 0 and mz["loss_step_1"] == 0.0 and mz["loss_step_2"] == 0.0
+        short, _, _ = model(ids[:, :3], hs[:, :3])
+        assert len(short) == 1
+        with pytest.raises(ValueError, match="expected exactly 3 weights"):
+            model(ids, hs, step_weights=[1.0])
+        with pytest.raises(NotImplementedError):
+            model(ids, hs, attention_mask=torch.ones(1, 40, device="cuda"))
+        with pytest.raises(RuntimeError, match="bf16"):
+            model(ids, hs.float())
