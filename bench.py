@@ -49,6 +49,8 @@ SEQ_LEN, TTT_STEPS = 4096, 7
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--workload", choices=["eagle3", "mtp"], default="eagle3",
+                    help="eagle3 = configs[1], the headline; mtp = configs[4] (MTP head, full-vocab CE)")
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
@@ -255,12 +257,178 @@ def cpu_baseline(cfg, t, k_steps):
             "loss": round(float(loss), 6)}
 
 
+# configs[4]: MTP head finetune, Qwen3-Next-like shape.  The FFN width is not stated there;
+# 3 x hidden is assumed.  The layer built is the Qwen3 flavour of the MTP layer.
+CONFIG4 = dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=2, head_dim=256,
+               intermediate_size=6144, vocab_size=151936, rms_norm_eps=1e-6, rope_theta=1000000.0)
+MTP_SEQ_LEN, MTP_BATCH, MTP_STEPS = 16384, 2, 3
+
+
+def run_mtp(args):
+    """configs[4]: MTP forward + backward, tokens/s over all B x T positions, and the roofline of
+    the label cross-entropy kernels, the full-vocabulary lm_head GEMMs and the attention."""
+    import torch
+
+    from speculators_amd import _lib, gemm
+    from speculators_amd.attention import create_ttt_mask, ttt_attention
+    from speculators_amd.losses import label_cross_entropy
+    from speculators_amd.mtp import MTPConfig, MTPDraftModel, compute_step_weights
+
+    _lib.load()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    n = args.seq_len if args.seq_len != SEQ_LEN else MTP_SEQ_LEN
+    b, k_steps = MTP_BATCH, MTP_STEPS
+    cfg = MTPConfig(num_speculative_steps=k_steps, **CONFIG4)
+    torch.manual_seed(0)
+    model = MTPDraftModel(cfg)
+    with torch.no_grad():
+        for name, p_ in model.named_parameters():
+            if name.endswith("norm.weight"):
+                p_.fill_(1.0)
+            else:
+                p_.normal_(0.0, 0.02)
+    model = model.to(torch.bfloat16).to(device)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    ids = torch.randint(0, cfg.vocab_size, (b, n), generator=g).to(device)
+    hs = torch.randn(b, n, cfg.hidden_size, generator=g).bfloat16().to(device)
+    lm = (torch.rand(b, n, generator=g) < 0.7).float().to(device)
+    pos = torch.arange(n, device=device).unsqueeze(0).expand(b, -1).contiguous()
+    sw = compute_step_weights(0.6, k_steps)
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        _, loss, _ = model(ids, hs, position_ids=pos, loss_mask=lm, step_weights=sw)
+        loss.backward()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    tokens = b * n
+    final_loss = float(loss)
+    del loss
+    model.zero_grad(set_to_none=True)
+    torch.cuda.empty_cache()
+
+    rows, v, h = b * (n - k_steps - 1), cfg.vocab_size, cfg.hidden_size
+    kernels = []
+
+    def rec(name, bound, work, ms, launches):
+        peak = PEAK_BF16_TFLOPS if bound == "mfma" else PEAK_HBM_GBS
+        ach = work / (ms * 1e-3) / (1e12 if bound == "mfma" else 1e9)
+        kernels.append({"kernel": name, "bound": bound, "achieved": round(ach, 1), "peak": peak,
+                        "unit": "TFLOP/s" if bound == "mfma" else "GB/s", "frac": round(ach / peak, 4),
+                        "traffic": None, "ms_per_launch": round(ms, 4), "launches_per_step": launches,
+                        ("algorithmic_flops" if bound == "mfma" else "algorithmic_bytes"): float(work)})
+
+    x = torch.randn(rows, h, device=device).bfloat16()
+    w = model.lm_head.weight
+    logits = gemm.gemm_nt(x, w)
+    rec("gemm_bf16_nt_kernel[lm_head fwd rows x H x V]", "mfma", 2.0 * rows * h * v,
+        time_events(torch, lambda: gemm.gemm_nt(x, w, out=logits), 5), k_steps)
+    lab = torch.randint(0, v, (rows,), device=device)
+    lab[torch.rand(rows, device=device) > 0.7] = -100
+    live = int((lab != -100).sum())
+    lg = logits.detach().requires_grad_(True)
+    out = label_cross_entropy(lg, lab)
+    rec("label_ce_fwd_kernel[rows x V, 70% live rows]", "hbm", live * v * 2.0,
+        time_events(torch, lambda: label_cross_entropy(logits, lab), 5), k_steps)
+    go = torch.ones_like(out)
+
+    def ce_bwd():
+        lg.grad = None
+        out.backward(go, retain_graph=True)
+
+    # live rows: one read + one write; dead rows: one write of zeros
+    rec("label_ce_bwd_kernel[rows x V, 70% live rows]", "hbm", (2 * live + (rows - live)) * v * 2.0,
+        time_events(torch, ce_bwd, 5), k_steps)
+    dl = lg.grad
+    del lg, out
+    wt = w.detach().t().contiguous()
+    rec("gemm_bf16_nt_kernel[lm_head dX rows x V x H, in row bands below 2 GiB]", "mfma",
+        2.0 * rows * h * v, time_events(torch, lambda: gemm.gemm_nt(dl, wt), 3), k_steps)
+    del dl, logits, wt
+    torch.cuda.empty_cache()
+    hq, hkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    t_row = n - k_steps - 1
+    doc = torch.arange(b, device=device).repeat_interleave(t_row)
+    mask = create_ttt_mask(doc, b * t_row, None)
+    q = torch.randn(1, hq, b * t_row, d, device=device).bfloat16().requires_grad_(True)
+    kk = torch.randn(1, hkv, b * t_row, d, device=device).bfloat16().requires_grad_(True)
+    vv = torch.randn(1, hkv, b * t_row, d, device=device).bfloat16().requires_grad_(True)
+    pairs = b * t_row * (t_row + 1) / 2
+    rec("attn_fwd_kernel[head_dim 256, causal per row]", "mfma", 4.0 * pairs * d * hq,
+        time_events(torch, lambda: ttt_attention(q.detach(), kk.detach(), vv.detach(), mask, d ** -0.5), 3),
+        k_steps)
+    o = ttt_attention(q, kk, vv, mask, d ** -0.5)
+    gd = torch.randn_like(o)
+
+    def attn_bwd():
+        q.grad = kk.grad = vv.grad = None
+        o.backward(gd, retain_graph=True)
+
+    rec("attn_bwd[head_dim 256, causal per row]", "mfma", 10.0 * pairs * d * hq,
+        time_events(torch, attn_bwd, 3), k_steps)
+    dominant = max(kernels, key=lambda r: r["ms_per_launch"] * r["launches_per_step"])
+
+    cpu = None
+    if args.cpu_baseline != "off":
+        from oracle import mtp as OM
+        from oracle.eagle3 import DraftShape
+
+        shape = DraftShape(draft_vocab_size=CONFIG4["vocab_size"], qk_norm=True, **CONFIG4)
+        tn = args.cpu_seq_len
+        torch.set_num_threads(os.cpu_count() or 1)
+        wts = {k_: v_.requires_grad_(k_ not in ("embed_tokens.weight", "lm_head.weight"))
+               for k_, v_ in OM.random_weights(shape, 0).items()}
+        cg = torch.Generator().manual_seed(0)
+        cids = torch.randint(0, shape.vocab_size, (b, tn), generator=cg)
+        chs = torch.randn(b, tn, shape.hidden_size, generator=cg)
+
+        def cpu_step():
+            for v_ in wts.values():
+                v_.grad = None
+            _, l_, _ = OM.mtp_forward(wts, shape, cids, chs, step_weights=sw, num_steps=k_steps, attn="sdpa")
+            l_.backward()
+
+        cpu_step()
+        c0 = time.perf_counter()
+        cpu_step()
+        cdt = time.perf_counter() - c0
+        cpu = {"value": round(b * tn / cdt, 2), "unit": "tokens/s", "cores": torch.get_num_threads(),
+               "kind": "port", "sample": f"oracle MTP forward+backward, configs[4] shape at batch {b} x seq {tn}, "
+                                         "fp32, 1 warm-up + 1 timed iteration"}
+    print(json.dumps({
+        "metric": "MTP train tokens/sec (fwd+bwd) @Qwen3-Next-like MTP head, full-vocab CE",
+        "value": round(tokens / (ms_per_step * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"configs[4]: MTP head, one Qwen3 decoder layer, hidden 2048, 16 q / 2 kv heads, "
+                               f"head_dim 256, FFN 6144 (assumed), vocab 151936, batch {b}, seq {n}, "
+                               f"{k_steps} prediction steps, label cross-entropy, loss_mask Bernoulli(0.7)",
+                   "seq_len": n, "batch": b, "steps": k_steps, "tokens_per_step": tokens,
+                   "final_loss": round(final_loss, 6)},
+        "roofline": {k_: dominant[k_] for k_ in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
+                    | {"kernel": dominant["kernel"]},
+        "kernels": kernels, "cpu_baseline": cpu}))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on ONE GPU (no collectives are built); got --gpus {args.gpus}",
               file=sys.stderr)
         sys.exit(2)
+    if args.workload == "mtp":
+        run_mtp(args)
+        return
     import torch
 
     from speculators_amd import _lib

@@ -19,7 +19,7 @@ constexpr int kAttnThreads = 256;
 constexpr int kBM = 128;  // query rows per workgroup
 constexpr int kBN = 64;   // keys per tile
 constexpr int kKPad = 8;  // K tile row stride = D + 8 elements  (272 B at D=128)
-constexpr int kVPad = 4;  // V^T tile row stride = 64 + 4 elements (136 B)
+constexpr int kVPad = 8;  // V^T tile row stride = 64 + 8 elements (144 B: 16-byte aligned rows)
 
 __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);

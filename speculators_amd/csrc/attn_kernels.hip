@@ -104,8 +104,11 @@ __global__ __launch_bounds__(256) void dflash_ranges_kernel(
 }
 
 // ---------------------------------------------------------------- transpose
-// dst[h][c][r] = src[h][r][c] for r < rows, c < cols; dst row stride ld_dst >= rows,
-// columns rows..ld_dst-1 of dst are zero filled.  64x64 tiles through LDS.
+// dst[h][c][perm(r)] = src[h][r][c] for r < rows, c < cols; dst row stride ld_dst >= rows
+// (a multiple of 16), the columns of r in rows..ld_dst-1 are zero filled.  perm swaps bits
+// 2 and 3 of r: inside every group of 16 the order is 0-3, 8-11, 4-7, 12-15, which puts
+// the 8 rows a lane half needs as MFMA k-slots (4 g + 0..3 and 8 + 4 g + 0..3) side by
+// side, so that operand is ONE 16-byte LDS read.  64x64 tiles through LDS.
 __global__ __launch_bounds__(256) void transpose_bf16_kernel(
     const uint16_t* __restrict__ src, int64_t src_hs, int64_t src_ld, int rows, int cols,
     uint16_t* __restrict__ dst, int64_t dst_hs, int64_t ld_dst) {
@@ -122,7 +125,8 @@ __global__ __launch_bounds__(256) void transpose_bf16_kernel(
   __syncthreads();
   for (int cc = ty; cc < 64; cc += 4) {
     int c = c0 + cc, r = r0 + tx;
-    if (c < cols && r < ld_dst) d[(int64_t)c * ld_dst + r] = tile[tx][cc];
+    const int rp = (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);
+    if (c < cols && r < ld_dst) d[(int64_t)c * ld_dst + rp] = tile[tx][cc];
   }
 }
 
@@ -166,10 +170,13 @@ __device__ __forceinline__ void load_bounds(const AttnParams& p, const int (&ic)
     a2mn = min(a2mn, rb.a2[sb]); a2mx = max(a2mx, rb.a2[sb]);
     b2mn = min(b2mn, rb.b2[sb]); b2mx = max(b2mx, rb.b2[sb]);
   }
-  rb.w_a1min = wave_min_i(a1mn); rb.w_a1max = wave_max_i(a1mx);
-  rb.w_b1min = wave_min_i(b1mn); rb.w_b1max = wave_max_i(b1mx);
-  rb.w_a2min = wave_min_i(a2mn); rb.w_a2max = wave_max_i(a2mx);
-  rb.w_b2min = wave_min_i(b2mn); rb.w_b2max = wave_max_i(b2mx);
+  // wave-uniform values are moved to scalar registers: the tests on them then compile to
+  // scalar branches (a masked and an unmasked tile path) instead of per-lane selects
+  auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+  rb.w_a1min = uni(wave_min_i(a1mn)); rb.w_a1max = uni(wave_max_i(a1mx));
+  rb.w_b1min = uni(wave_min_i(b1mn)); rb.w_b1max = uni(wave_max_i(b1mx));
+  rb.w_a2min = uni(wave_min_i(a2mn)); rb.w_a2max = uni(wave_max_i(a2mx));
+  rb.w_b2min = uni(wave_min_i(b2mn)); rb.w_b2max = uni(wave_max_i(b2mx));
   if (lane == 0) {
     red[wave * 4 + 0] = rb.w_a1min; red[wave * 4 + 1] = rb.w_b1max;
     red[wave * 4 + 2] = rb.w_a2min; red[wave * 4 + 3] = rb.w_b2max;
@@ -181,6 +188,8 @@ __device__ __forceinline__ void load_bounds(const AttnParams& p, const int (&ic)
     rb.blk_a1 = min(rb.blk_a1, red[w * 4 + 0]); rb.blk_b1 = max(rb.blk_b1, red[w * 4 + 1]);
     rb.blk_a2 = min(rb.blk_a2, red[w * 4 + 2]); rb.blk_b2 = max(rb.blk_b2, red[w * 4 + 3]);
   }
+  rb.blk_a1 = uni(rb.blk_a1); rb.blk_b1 = uni(rb.blk_b1);
+  rb.blk_a2 = uni(rb.blk_a2); rb.blk_b2 = uni(rb.blk_b2);
 }
 
 // ---------------------------------------------------------------- forward
@@ -276,9 +285,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
       const int krow = c / (D / 8), kcol = (c % (D / 8)) * 8;
       *reinterpret_cast<u32x4*>(&Ks[krow * KS + kcol]) = kreg[n];
       const int vd = c >> 3, vcol = (c & 7) * 8;
-      u32x2 a = {vreg[n].x, vreg[n].y}, b = {vreg[n].z, vreg[n].w};
-      *reinterpret_cast<u32x2*>(&Vs[vd * VS + vcol]) = a;
-      *reinterpret_cast<u32x2*>(&Vs[vd * VS + vcol + 4]) = b;
+      *reinterpret_cast<u32x4*>(&Vs[vd * VS + vcol]) = vreg[n];
     }
   };
 
@@ -292,9 +299,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
           *reinterpret_cast<const u32x4*>(Kh + (int64_t)kr * D + kcol);
       const int vd = c >> 3, vcol = (c & 7) * 8;
       const u32x4 t = *reinterpret_cast<const u32x4*>(Vth + (int64_t)vd * p.NKVp + n0 + vcol);
-      u32x2 a = {t.x, t.y}, b = {t.z, t.w};
-      *reinterpret_cast<u32x2*>(&Vs[vd * VS + vcol]) = a;
-      *reinterpret_cast<u32x2*>(&Vs[vd * VS + vcol + 4]) = b;
+      *reinterpret_cast<u32x4*>(&Vs[vd * VS + vcol]) = t;
     }
   };
 
@@ -318,33 +323,54 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) st[sb][kb][r] = 0.f;
+      // K fragments go through a ring of four registers: the read of fragment f + 4 is
+      // issued right after the MFMA of fragment f, so no MFMA waits for LDS; the two
+      // 32-key halves alternate so that consecutive MFMAs use different accumulators
+      {
+        constexpr int NF = 2 * NKK;
+        bf16x8 kfr[4];
+        auto kread = [&](int f) {
+          kfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+              &Ks[((f & 1) * 32 + col) * KS + g * 8 + (f >> 1) * 16]));
+        };
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const uint16_t* krow = &Ks[(kb * 32 + col) * KS + g * 8];
+        for (int f = 0; f < 4; ++f) kread(f);
 #pragma unroll
-        for (int kk = 0; kk < NKK; ++kk) {
-          const bf16x8 ka = as_bf16x8(*reinterpret_cast<const u32x4*>(krow + kk * 16));
+        for (int f = 0; f < NF; ++f) {
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int sb = 0; sb < NSB; ++sb) st[sb][kb] = mfma32(ka, qf[sb][kk], st[sb][kb]);
+          for (int sb = 0; sb < NSB; ++sb)
+            st[sb][f & 1] = mfma32(kfr[f & 3], qf[sb][f >> 1], st[sb][f & 1]);
+          __builtin_amdgcn_sched_barrier(0);
+          if (f + 4 < NF) kread(f + 4);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
       const bool need_mask = (n0 < w_amax) || (n0 + kBN > w_bmin);
+      int m_lo[NSB], m_hi[NSB];
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb) { m_lo[sb] = aa[sb] - n0 - 4 * g; m_hi[sb] = bb[sb] - n0 - 4 * g; }
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb) {
         // running max on the raw scores; the soft-max scale is folded into the exp2 argument
+        if (need_mask) {
+          // a real (scalar) branch: the asm statement keeps the compiler from turning the
+          // masking into selects that every tile would pay for
+          asm volatile("; masked tile");
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              // key index = n0 + 4 g + (compile-time part): compare the constant part
+              const int cr = kb * 32 + 8 * (r >> 2) + (r & 3);
+              if (cr < m_lo[sb] || cr >= m_hi[sb]) st[sb][kb][r] = -INFINITY;
+            }
+        }
         float mx = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            float sv = st[sb][kb][r];
-            if (need_mask) {
-              const int c = n0 + kb * 32 + acc_row(r, g);
-              if (c < aa[sb] || c >= bb[sb]) sv = -INFINITY;
-              st[sb][kb][r] = sv;
-            }
-            mx = fmaxf(mx, sv);
-          }
+          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[sb][kb][r]);
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m_run[sb], mx * p.scale_log2e);
         const float alpha = fast_exp2(m_run[sb] - m_new);
@@ -368,19 +394,31 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         }
         m_run[sb] = m_new;
       }
+      {
+        // V^T fragments through the same kind of ring; fragment f = (16-key step s, D block db)
+        constexpr int NF = 4 * NDB;
+        bf16x8 vfr[4];
+        auto vread = [&](int f) {
+          vfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+              &Vs[((f % NDB) * 32 + col) * VS + (f / NDB) * 16 + 8 * g]));
+        };
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
+        for (int f = 0; f < 4; ++f) vread(f);
         bf16x8 pb[NSB];
 #pragma unroll
-        for (int sb = 0; sb < NSB; ++sb) pb[sb] = pack8(st[sb][s >> 1], (s & 1) * 8);
+        for (int f = 0; f < NF; ++f) {
+          const int s = f / NDB, db = f % NDB;
+          if (db == 0) {
 #pragma unroll
-        for (int db = 0; db < NDB; ++db) {
-          const uint16_t* vrow = &Vs[(db * 32 + col) * VS + s * 16 + 4 * g];
-          const bf16x8 va = join_bf16x4(*reinterpret_cast<const u32x2*>(vrow),
-                                        *reinterpret_cast<const u32x2*>(vrow + 8));
+            for (int sb = 0; sb < NSB; ++sb) pb[sb] = pack8(st[sb][s >> 1], (s & 1) * 8);
+          }
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int sb = 0; sb < NSB; ++sb) acc[sb][db] = mfma32(va, pb[sb], acc[sb][db]);
+          for (int sb = 0; sb < NSB; ++sb) acc[sb][db] = mfma32(vfr[f & 3], pb[sb], acc[sb][db]);
+          __builtin_amdgcn_sched_barrier(0);
+          if (f + 4 < NF) vread(f + 4);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
@@ -547,9 +585,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
       *reinterpret_cast<u32x4*>(&Ks[krow * KS + kcol]) = kreg[n];
       *reinterpret_cast<u32x4*>(&Vn[krow * KS + kcol]) = vreg[n];
       const int vd = c >> 3, vcol = (c & 7) * 8;
-      u32x2 a = {treg[n].x, treg[n].y}, b = {treg[n].z, treg[n].w};
-      *reinterpret_cast<u32x2*>(&Kts[vd * VS + vcol]) = a;
-      *reinterpret_cast<u32x2*>(&Kts[vd * VS + vcol + 4]) = b;
+      *reinterpret_cast<u32x4*>(&Kts[vd * VS + vcol]) = treg[n];
     }
   };
 
@@ -565,9 +601,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
           *reinterpret_cast<const u32x4*>(Vh + (int64_t)kr * D + kcol);
       const int vd = c >> 3, vcol = (c & 7) * 8;
       const u32x4 t = *reinterpret_cast<const u32x4*>(Kth + (int64_t)vd * p.NKVp + n0 + vcol);
-      u32x2 a = {t.x, t.y}, b = {t.z, t.w};
-      *reinterpret_cast<u32x2*>(&Kts[vd * VS + vcol]) = a;
-      *reinterpret_cast<u32x2*>(&Kts[vd * VS + vcol + 4]) = b;
+      *reinterpret_cast<u32x4*>(&Kts[vd * VS + vcol]) = t;
     }
   };
 
@@ -621,9 +655,8 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
             const bf16x8 db8 = pack8(dp, s2 * 8);
 #pragma unroll
             for (int db = 0; db < NDB; ++db) {
-              const uint16_t* trow = &Kts[(db * 32 + col) * VS + s * 16 + 4 * g];
-              const bf16x8 ka = join_bf16x4(*reinterpret_cast<const u32x2*>(trow),
-                                            *reinterpret_cast<const u32x2*>(trow + 8));
+              const bf16x8 ka = as_bf16x8(
+                  *reinterpret_cast<const u32x4*>(&Kts[(db * 32 + col) * VS + s * 16 + 8 * g]));
               acc[sb][db] = mfma32(ka, db8, acc[sb][db]);
             }
           }
@@ -703,7 +736,10 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
 //   dV^T += dO^T P,   dK^T += Q^T dS,   dS = P (dO V^T - delta)
 // The per-head results go to fp32 partial buffers that attn_dkv_reduce_kernel sums over
 // the heads of a group (fixed order: deterministic, no atomics).
-template <int D, int NW, bool PF>
+// PASS 0 computes dK and dV together; PASS 1 only dV, PASS 2 only dK (head_dim 256: the two
+// accumulator sets and both operand fragments do not fit the register file together, so
+// the kernel is launched once per pass and the scores are recomputed).
+template <int D, int NW, bool PF, int PASS>
 __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     AttnParams p, const uint16_t* __restrict__ dO, const uint16_t* __restrict__ Qt,
     const uint16_t* __restrict__ dOt, int NQp, const float* __restrict__ LSE,
@@ -742,21 +778,28 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
   const int c = cw + col;
   const int cc = c < p.NKV ? c : p.NKV - 1;
 
-  bf16x8 kf[NKK], vf[NKK];
+  constexpr bool kDoV = PASS != 2, kDoK = PASS != 1;
+  constexpr int NVF = kDoK ? NKK : 1;                    // V fragments feed dP, a dK-only term
+  constexpr int NAK = kDoK ? NDB : 1, NAV = kDoV ? NDB : 1;
+  bf16x8 kf[NKK], vf[NVF];
   {
     const uint16_t* krow = p.K + (int64_t)kvh * p.k_hs + (int64_t)cc * D + g * 8;
     const uint16_t* vrow = p.V + (int64_t)kvh * p.v_hs + (int64_t)cc * D + g * 8;
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) {
       kf[kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(krow + kk * 16));
-      vf[kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(vrow + kk * 16));
+      if (kDoK) vf[kk % NVF] = as_bf16x8(*reinterpret_cast<const u32x4*>(vrow + kk * 16));
     }
   }
-  f32x16 acc_dk[NDB], acc_dv[NDB];
+  f32x16 acc_dk[NAK], acc_dv[NAV];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db)
+  for (int db = 0; db < NAK; ++db)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { acc_dk[db][r] = 0.f; acc_dv[db][r] = 0.f; }
+    for (int r = 0; r < 16; ++r) acc_dk[db][r] = 0.f;
+#pragma unroll
+  for (int db = 0; db < NAV; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc_dv[db][r] = 0.f;
 
   const uint16_t* Qh = p.Q + (int64_t)h * p.q_hs;
   const uint16_t* Qth = Qt + (int64_t)h * D * NQp;
@@ -807,12 +850,8 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       *reinterpret_cast<u32x4*>(&Qs[qr * QS + qc]) = qreg[n];
       *reinterpret_cast<u32x4*>(&dOs[qr * QS + qc]) = dreg[n];
       const int td = ch >> 3, tc = (ch & 7) * 8;
-      u32x2 a0 = {qtreg[n].x, qtreg[n].y}, a1v = {qtreg[n].z, qtreg[n].w};
-      u32x2 b0 = {dtreg[n].x, dtreg[n].y}, b1v = {dtreg[n].z, dtreg[n].w};
-      *reinterpret_cast<u32x2*>(&Qts[td * TS + tc]) = a0;
-      *reinterpret_cast<u32x2*>(&Qts[td * TS + tc + 4]) = a1v;
-      *reinterpret_cast<u32x2*>(&dOts[td * TS + tc]) = b0;
-      *reinterpret_cast<u32x2*>(&dOts[td * TS + tc + 4]) = b1v;
+      *reinterpret_cast<u32x4*>(&Qts[td * TS + tc]) = qtreg[n];
+      *reinterpret_cast<u32x4*>(&dOts[td * TS + tc]) = dtreg[n];
     }
     if (tid < 64) {
       lse_s[tid] = lse_r; delta_s[tid] = delta_r;
@@ -833,11 +872,8 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       const int td = ch >> 3, tc = (ch & 7) * 8;
       const u32x4 a = *reinterpret_cast<const u32x4*>(Qth + (int64_t)td * NQp + mq + tc);
       const u32x4 b = *reinterpret_cast<const u32x4*>(dOth + (int64_t)td * NQp + mq + tc);
-      u32x2 a0 = {a.x, a.y}, a1v = {a.z, a.w}, b0 = {b.x, b.y}, b1v = {b.z, b.w};
-      *reinterpret_cast<u32x2*>(&Qts[td * TS + tc]) = a0;
-      *reinterpret_cast<u32x2*>(&Qts[td * TS + tc + 4]) = a1v;
-      *reinterpret_cast<u32x2*>(&dOts[td * TS + tc]) = b0;
-      *reinterpret_cast<u32x2*>(&dOts[td * TS + tc + 4]) = b1v;
+      *reinterpret_cast<u32x4*>(&Qts[td * TS + tc]) = a;
+      *reinterpret_cast<u32x4*>(&dOts[td * TS + tc]) = b;
     }
     if (tid < 64) {
       const int ir = mq + tid;
@@ -876,7 +912,7 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
 #pragma unroll
       for (int kk = 0; kk < NKK; ++kk) {
         st = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(qrow + kk * 16)), kf[kk], st);
-        dp = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(drow + kk * 16)), vf[kk], dp);
+        if (kDoK) dp = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(drow + kk * 16)), vf[kk % NVF], dp);
       }
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
@@ -911,12 +947,13 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         const bf16x8 sb = pack8(dp, s2 * 8);
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-          const uint16_t* arow = &dOts[(db * 32 + col) * TS + s * 16 + 4 * g];
-          const uint16_t* brow = &Qts[(db * 32 + col) * TS + s * 16 + 4 * g];
-          acc_dv[db] = mfma32(join_bf16x4(*reinterpret_cast<const u32x2*>(arow),
-                                          *reinterpret_cast<const u32x2*>(arow + 8)), pb, acc_dv[db]);
-          acc_dk[db] = mfma32(join_bf16x4(*reinterpret_cast<const u32x2*>(brow),
-                                          *reinterpret_cast<const u32x2*>(brow + 8)), sb, acc_dk[db]);
+          const int off = (db * 32 + col) * TS + s * 16 + 8 * g;
+          if (kDoV)
+            acc_dv[db % NAV] = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(&dOts[off])), pb,
+                                      acc_dv[db % NAV]);
+          if (kDoK)
+            acc_dk[db % NAK] = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(&Qts[off])), sb,
+                                      acc_dk[db % NAK]);
         }
       }
     }
@@ -929,10 +966,16 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
-        f32x4 wk = {acc_dk[db][r4 * 4 + 0], acc_dk[db][r4 * 4 + 1], acc_dk[db][r4 * 4 + 2], acc_dk[db][r4 * 4 + 3]};
-        f32x4 wv = {acc_dv[db][r4 * 4 + 0], acc_dv[db][r4 * 4 + 1], acc_dv[db][r4 * 4 + 2], acc_dv[db][r4 * 4 + 3]};
-        *reinterpret_cast<f32x4*>(krow + db * 32 + 8 * r4) = wk;
-        *reinterpret_cast<f32x4*>(vrow + db * 32 + 8 * r4) = wv;
+        if (kDoK) {
+          const f32x16& a = acc_dk[db % NAK];
+          f32x4 wk = {a[r4 * 4 + 0], a[r4 * 4 + 1], a[r4 * 4 + 2], a[r4 * 4 + 3]};
+          *reinterpret_cast<f32x4*>(krow + db * 32 + 8 * r4) = wk;
+        }
+        if (kDoV) {
+          const f32x16& a = acc_dv[db % NAV];
+          f32x4 wv = {a[r4 * 4 + 0], a[r4 * 4 + 1], a[r4 * 4 + 2], a[r4 * 4 + 3]};
+          *reinterpret_cast<f32x4*>(vrow + db * 32 + 8 * r4) = wv;
+        }
       }
   }
 }
@@ -1060,8 +1103,12 @@ static int launch_fwd(AttnParams p, void* workspace, uint16_t* O, float* lse, hi
                      vt, (int64_t)D * p.NKVp, (int64_t)p.NKVp);
   constexpr int BM = 32 * kFwdNSB * kFwdNW;
   const int n_qb = (p.NQ + BM - 1) / BM;
-  hipLaunchKernelGGL((attn_fwd_kernel<D, SPX_FWD_CFG>), dim3((unsigned)(n_qb * p.Hq)),
-                     dim3(64 * kFwdNW), 0, st, p, vt, O, lse);
+  if constexpr (D > 128)  // no register prefetch: the tile would not fit beside the accumulators
+    hipLaunchKernelGGL((attn_fwd_kernel<D, kFwdNSB, kFwdNW, false>), dim3((unsigned)(n_qb * p.Hq)),
+                       dim3(64 * kFwdNW), 0, st, p, vt, O, lse);
+  else
+    hipLaunchKernelGGL((attn_fwd_kernel<D, SPX_FWD_CFG>), dim3((unsigned)(n_qb * p.Hq)),
+                       dim3(64 * kFwdNW), 0, st, p, vt, O, lse);
   return check_launch(fn);
 }
 
@@ -1101,19 +1148,34 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
                      dim3(64 * kDqNW), 0, st, p, dOp, kt, lse, delta, dQp, dq_hs);
 
   const size_t smem = (size_t)(2 * 64 * (D + kKPad) + 2 * D * (64 + kVPad)) * 2 + 64 * 4 * 6;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, SPX_DKV_CFG>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) {
-      last_error() = std::string(fn) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
-      return SPX_ERR_HIP;
-    }
-    attr_set = true;
-  }
   const int n_kb = (p.NKV + 32 * kDkvNW - 1) / (32 * kDkvNW);
-  hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, SPX_DKV_CFG>), dim3((unsigned)(n_kb * p.Hq)), dim3(64 * kDkvNW), smem, st,
-                     p, dOp, qt, dot, NQp, lse, delta, tb, dkp, dvp);
+  const dim3 kgrid((unsigned)(n_kb * p.Hq)), kblock(64 * kDkvNW);
+  auto set_smem = [&](const void* f) {
+    hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) last_error() = std::string(fn) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
+    return e == hipSuccess;
+  };
+  static bool attr_set = false;
+  if constexpr (D > 128) {
+    // one launch per gradient, no register prefetch
+    if (!attr_set) {
+      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, false, 1>)) ||
+          !set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, false, 2>)))
+        return SPX_ERR_HIP;
+      attr_set = true;
+    }
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, false, 1>), kgrid, kblock, smem, st, p, dOp, qt, dot,
+                       NQp, lse, delta, tb, dkp, dvp);
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, false, 2>), kgrid, kblock, smem, st, p, dOp, qt, dot,
+                       NQp, lse, delta, tb, dkp, dvp);
+  } else {
+    if (!attr_set) {
+      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, SPX_DKV_CFG, 0>))) return SPX_ERR_HIP;
+      attr_set = true;
+    }
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, SPX_DKV_CFG, 0>), kgrid, kblock, smem, st, p, dOp, qt, dot,
+                       NQp, lse, delta, tb, dkp, dvp);
+  }
   const int64_t items = (int64_t)p.NKV * D / 4 * p.Hkv;
   hipLaunchKernelGGL(attn_dkv_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, dkp,
                      dvp, p.NKV, D, p.Hq, p.Hkv, p.scaling, dKp, dk_hs, dVp, dv_hs);
