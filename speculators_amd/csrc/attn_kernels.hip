@@ -626,39 +626,62 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
           f32x16 st, dp;
 #pragma unroll
           for (int r = 0; r < 16; ++r) { st[r] = 0.f; dp[r] = 0.f; }
-          const uint16_t* krow = &Ks[(kb * 32 + col) * KS + g * 8];
-          const uint16_t* vrow = &Vn[(kb * 32 + col) * KS + g * 8];
-#ifndef SPX_DQ_KKU
-#define SPX_DQ_KKU 8
-#endif
+          // K and V fragments alternate through a ring of four registers (fragment 2 kk is
+          // K, 2 kk + 1 is V): the read of fragment f + 4 follows the MFMA of fragment f
+          {
+            constexpr int NF = 2 * NKK;
+            bf16x8 fr[4];
+            auto fread = [&](int f) {
+              const uint16_t* base = (f & 1) ? Vn : Ks;
+              fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                  &base[(kb * 32 + col) * KS + g * 8 + (f >> 1) * 16]));
+            };
 #pragma unroll
-          for (int kk0 = 0; kk0 < NKK; kk0 += SPX_DQ_KKU) {
+            for (int f = 0; f < 4; ++f) fread(f);
 #pragma unroll
-            for (int kk = kk0; kk < kk0 + SPX_DQ_KKU && kk < NKK; ++kk) {
-              st = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(krow + kk * 16)), qf[sb][kk], st);
-              dp = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(vrow + kk * 16)), dof[sb][kk], dp);
+            for (int f = 0; f < NF; ++f) {
+              __builtin_amdgcn_sched_barrier(0);
+              if (f & 1) dp = mfma32(fr[f & 3], dof[sb][f >> 1], dp);
+              else st = mfma32(fr[f & 3], qf[sb][f >> 1], st);
+              __builtin_amdgcn_sched_barrier(0);
+              if (f + 4 < NF) fread(f + 4);
             }
-            if (SPX_DQ_KKU < NKK) __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_sched_barrier(0);
           }
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            float pv = fast_exp2(fmaf(st[r], p.scale_log2e, -lse_i[sb]));
-            if (need_mask) {
-              const int c = n0 + kb * 32 + acc_row(r, g);
-              if (c < aa[sb] || c >= bb[sb]) pv = 0.f;
+          for (int r = 0; r < 16; ++r) st[r] = fast_exp2(fmaf(st[r], p.scale_log2e, -lse_i[sb]));
+          if (need_mask) {
+            // a real (scalar) branch, see the forward kernel
+            asm volatile("; masked tile");
+            const int lo = aa[sb] - n0 - 4 * g, hi = bb[sb] - n0 - 4 * g;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int cr = kb * 32 + 8 * (r >> 2) + (r & 3);
+              if (cr < lo || cr >= hi) st[r] = 0.f;
             }
-            dp[r] = pv * (dp[r] - delta_i[sb]);
           }
 #pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2) {
-            const int s = kb * 2 + s2;
-            const bf16x8 db8 = pack8(dp, s2 * 8);
+          for (int r = 0; r < 16; ++r) dp[r] = st[r] * (dp[r] - delta_i[sb]);
+          {
+            // K^T fragments through the same kind of ring; fragment f = (16-key step s2, D block db)
+            constexpr int NF = 2 * NDB;
+            bf16x8 fr[4];
+            auto fread = [&](int f) {
+              fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                  &Kts[((f % NDB) * 32 + col) * VS + (kb * 2 + f / NDB) * 16 + 8 * g]));
+            };
 #pragma unroll
-            for (int db = 0; db < NDB; ++db) {
-              const bf16x8 ka = as_bf16x8(
-                  *reinterpret_cast<const u32x4*>(&Kts[(db * 32 + col) * VS + s * 16 + 8 * g]));
-              acc[sb][db] = mfma32(ka, db8, acc[sb][db]);
+            for (int f = 0; f < 4 && f < NF; ++f) fread(f);
+            bf16x8 db8 = pack8(dp, 0);
+#pragma unroll
+            for (int f = 0; f < NF; ++f) {
+              if (f == NDB) db8 = pack8(dp, 8);
+              __builtin_amdgcn_sched_barrier(0);
+              acc[sb][f % NDB] = mfma32(fr[f & 3], db8, acc[sb][f % NDB]);
+              __builtin_amdgcn_sched_barrier(0);
+              if (f + 4 < NF) fread(f + 4);
             }
+            __builtin_amdgcn_sched_barrier(0);
           }
         }
       }
@@ -907,23 +930,43 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       f32x16 st, dp;
 #pragma unroll
       for (int r = 0; r < 16; ++r) { st[r] = 0.f; dp[r] = 0.f; }
-      const uint16_t* qrow = &Qs[(qb * 32 + col) * QS + g * 8];
-      const uint16_t* drow = &dOs[(qb * 32 + col) * QS + g * 8];
+      {
+        // Q (and, for dK, dO) row fragments through a ring of four registers: the read of
+        // fragment f + 4 follows the MFMA of fragment f, so no MFMA waits for LDS
+        constexpr int PER = kDoK ? 2 : 1;  // fragments per K step: Q [, dO]
+        constexpr int NF = PER * NKK;
+        bf16x8 fr[4];
+        auto fread = [&](int f) {
+          const uint16_t* base = (PER == 2 && (f & 1)) ? dOs : Qs;
+          fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+              &base[(qb * 32 + col) * QS + g * 8 + (f / PER) * 16]));
+        };
 #pragma unroll
-      for (int kk = 0; kk < NKK; ++kk) {
-        st = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(qrow + kk * 16)), kf[kk], st);
-        if (kDoK) dp = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(drow + kk * 16)), vf[kk % NVF], dp);
+        for (int f = 0; f < 4; ++f) fread(f);
+#pragma unroll
+        for (int f = 0; f < NF; ++f) {
+          __builtin_amdgcn_sched_barrier(0);
+          if (PER == 2 && (f & 1)) dp = mfma32(fr[f & 3], vf[(f / PER) % NVF], dp);
+          else st = mfma32(fr[f & 3], kf[f / PER], st);
+          __builtin_amdgcn_sched_barrier(0);
+          if (f + 4 < NF) fread(f + 4);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         const int q0 = qb * 32 + 8 * r4 + 4 * g;  // 4 consecutive query rows: one 16-byte LDS read each
         const f32x4 ls = *reinterpret_cast<const f32x4*>(&lse_s[q0]);
-        const f32x4 dl = *reinterpret_cast<const f32x4*>(&delta_s[q0]);
-        float pv[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) pv[t] = fast_exp2(fmaf(st[r4 * 4 + t], p.scale_log2e, -ls[t]));
-        if (!full) {
-          typedef __attribute__((ext_vector_type(4))) int i32x4;
+        for (int t = 0; t < 4; ++t) st[r4 * 4 + t] = fast_exp2(fmaf(st[r4 * 4 + t], p.scale_log2e, -ls[t]));
+      }
+      if (!full) {
+        // a real (scalar) branch: only tiles that straddle an interval edge pay for the mask
+        asm volatile("; masked tile");
+        typedef __attribute__((ext_vector_type(4))) int i32x4;
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const int q0 = qb * 32 + 8 * r4 + 4 * g;
           const i32x4 a1v = *reinterpret_cast<const i32x4*>(&a1_s[q0]);
           const i32x4 b1v = *reinterpret_cast<const i32x4*>(&b1_s[q0]);
           const i32x4 a2v = *reinterpret_cast<const i32x4*>(&a2_s[q0]);
@@ -931,30 +974,47 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
             const bool ok = ((c >= a1v[t] && c < b1v[t]) || (c >= a2v[t] && c < b2v[t])) && (c < p.NKV);
-            pv[t] = ok ? pv[t] : 0.f;
+            if (!ok) st[r4 * 4 + t] = 0.f;
           }
         }
+      }
+      if (kDoK) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          st[r4 * 4 + t] = pv[t];
-          dp[r4 * 4 + t] = pv[t] * (dp[r4 * 4 + t] - dl[t]);
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const f32x4 dl = *reinterpret_cast<const f32x4*>(&delta_s[qb * 32 + 8 * r4 + 4 * g]);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) dp[r4 * 4 + t] = st[r4 * 4 + t] * (dp[r4 * 4 + t] - dl[t]);
         }
       }
+      {
+        // dO^T / Q^T fragments through the same kind of ring; per (16-row step s2, D block db):
+        // dO^T [, Q^T]
+        constexpr int PER = (kDoV ? 1 : 0) + (kDoK ? 1 : 0);
+        constexpr int NF = PER * 2 * NDB;
+        bf16x8 fr[4];
+        auto fread = [&](int f) {
+          const int e = f / PER, s2 = e / NDB, db = e % NDB;
+          const bool is_q = kDoK && (!kDoV || (f % PER) == 1);
+          const uint16_t* base = is_q ? Qts : dOts;
+          fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+              &base[(db * 32 + col) * TS + (qb * 2 + s2) * 16 + 8 * g]));
+        };
 #pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        const int s = qb * 2 + s2;
-        const bf16x8 pb = pack8(st, s2 * 8);
-        const bf16x8 sb = pack8(dp, s2 * 8);
+        for (int f = 0; f < 4; ++f) fread(f);
+        bf16x8 pb = pack8(st, 0), sb8 = pack8(dp, 0);
 #pragma unroll
-        for (int db = 0; db < NDB; ++db) {
-          const int off = (db * 32 + col) * TS + s * 16 + 8 * g;
-          if (kDoV)
-            acc_dv[db % NAV] = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(&dOts[off])), pb,
-                                      acc_dv[db % NAV]);
-          if (kDoK)
-            acc_dk[db % NAK] = mfma32(as_bf16x8(*reinterpret_cast<const u32x4*>(&Qts[off])), sb,
-                                      acc_dk[db % NAK]);
+        for (int f = 0; f < NF; ++f) {
+          const int e = f / PER, s2 = e / NDB, db = e % NDB;
+          const bool is_q = kDoK && (!kDoV || (f % PER) == 1);
+          if (f == PER * NDB) { pb = pack8(st, 8); sb8 = pack8(dp, 8); }
+          __builtin_amdgcn_sched_barrier(0);
+          if (is_q) acc_dk[db % NAK] = mfma32(fr[f & 3], sb8, acc_dk[db % NAK]);
+          else acc_dv[db % NAV] = mfma32(fr[f & 3], pb, acc_dv[db % NAV]);
+          __builtin_amdgcn_sched_barrier(0);
+          if (f + 4 < NF) fread(f + 4);
+          (void)s2;
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   }
