@@ -74,13 +74,17 @@ class _FusedLoss(torch.autograd.Function):
     losses/fused.py:238-291.  Targets get no gradient."""
 
     @staticmethod
-    def forward(ctx, logits, targets, op, known_lse_t=None, known_am_t=None):
+    def forward(ctx, logits, targets, op, known_lse_t=None, known_am_t=None, n_rows=None):
         known = (known_lse_t, known_am_t) if known_lse_t is not None else None
-        loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, logits, targets, known)
+        # n_rows: only the first n_rows rows of ``logits`` (a [1, T, V] tensor) take part, the
+        # rest get a zero gradient.  Doing the cut here instead of slicing outside keeps
+        # autograd from materialising a zero-padded copy of the whole gradient.
+        ctx.full_shape = logits.shape
+        used = logits if n_rows is None else logits[:, :n_rows]
+        loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, used, targets, known)
         ctx.save_for_backward(x, None if op == OP_CE else y, lse_d, lse_t, extra, am_t)
         ctx.op = op
-        ctx.shape = logits.shape
-        lead = logits.shape[:-1]
+        lead = used.shape[:-1]
         am_d, am_t, lse_t = am_d.view(lead), am_t.view(lead), lse_t.view(lead)
         ctx.mark_non_differentiable(am_d, am_t, lse_t)
         return loss.view(lead), am_d, am_t, lse_t
@@ -89,22 +93,29 @@ class _FusedLoss(torch.autograd.Function):
     def backward(ctx, grad_rows, _gd, _gt, _gl):
         x, y, lse_d, lse_t, extra, am_t = ctx.saved_tensors
         rows, vocab = x.shape
+        full_rows = 1
+        for d in ctx.full_shape[:-1]:
+            full_rows *= d
         g = grad_rows.reshape(-1).to(torch.float32).contiguous()
-        grad = torch.empty(rows, vocab, device=x.device, dtype=x.dtype)
+        grad = torch.empty(full_rows, vocab, device=x.device, dtype=x.dtype)
         _lib.call(
             "spx_fused_vocab_loss_bwd", ctx.op, _lib.ptr(x), x.stride(0), _lib.ptr(y),
             y.stride(0) if y is not None else 0, rows, vocab, _lib.dtype_code(x),
             _lib.ptr(lse_d), _lib.ptr(lse_t), _lib.ptr(extra), _lib.ptr(am_t), _lib.ptr(g), None,
             _lib.ptr(grad), grad.stride(0), _lib.stream_ptr(x.device),
         )
-        return grad.view(ctx.shape), None, None, None, None
+        if full_rows > rows:
+            grad[rows:].zero_()
+        return grad.view(ctx.full_shape), None, None, None, None, None
 
 
-def fused_rows(op: int, logits, targets, target_stats=None):
-    """(row_loss, argmax_draft, argmax_target, lse_target) of one primitive reduction."""
+def fused_rows(op: int, logits, targets, target_stats=None, n_rows=None):
+    """(row_loss, argmax_draft, argmax_target, lse_target) of one primitive reduction;
+    ``n_rows`` restricts ``logits [1, T, V]`` to its first ``n_rows`` rows (``targets`` already
+    has that many) without slicing it under autograd."""
     if target_stats is None:
-        return _FusedLoss.apply(logits, targets, op)
-    return _FusedLoss.apply(logits, targets, op, target_stats[0], target_stats[1])
+        return _FusedLoss.apply(logits, targets, op, None, None, n_rows)
+    return _FusedLoss.apply(logits, targets, op, target_stats[0], target_stats[1], n_rows)
 
 
 def kl_div_loss(logits, targets):

@@ -108,7 +108,9 @@ def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
                     full = target_stats_cache.get("kl")  # the arg-max is all ce needs
                 if full is not None:
                     known = (full[0][ttt_step:], full[1][ttt_step:])
-            rows, am_d, am_t, lse_t = L.fused_rows(op, s_logits, s_targets, known)
+            # the full logits go in with a row count: see _FusedLoss.forward
+            rows, am_d, am_t, lse_t = L.fused_rows(op, logits, s_targets, known,
+                                                   n_rows=s_logits.shape[1])
             if (target_stats_cache is not None and known is None and ttt_step == 0
                     and op in (L.OP_KL, L.OP_CE)):
                 target_stats_cache["kl" if op == L.OP_KL else "ce"] = (
