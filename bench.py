@@ -124,6 +124,7 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
     from speculators_amd import attention as A
     from speculators_amd import losses as L
     from speculators_amd.gemm import gemm_nt
+    from speculators_amd.data import plan_rows
 
     h, vd = cfg["hidden_size"], cfg["draft_vocab_size"]
     hq, hkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
@@ -202,6 +203,31 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
     ms = time_events(torch, loss_bwd, 20)
     hbm("loss_bwd_kernel[KL, T rows x Vd]", 3.0 * t * vd * 2, ms, k_steps, "loss_bwd")
     del tg, lg, grad, y
+
+    # batch producer: 8 documents of (T + 8) / 8 rows, 3 auxiliary layers + the last one, bf16 ->
+    # the packed [1, T, ...] row (outside the timed step: it runs on a side stream ahead of it)
+    n_docs = 8
+    rows = t + n_docs
+    hs = torch.randn(rows, 4, h, device=device, generator=g).bfloat16()
+    ids = torch.randint(0, 1000, (rows,), device=device, generator=g)
+    lm = torch.ones(rows, device=device, dtype=torch.int64)
+    lens = [rows // n_docs] * n_docs
+    src_s, out_s = plan_rows(lens, t, 1)
+    plan = torch.tensor([src_s, out_s], device=device, dtype=torch.int64)
+    p_aux = torch.empty(t, 3 * h, device=device, dtype=torch.bfloat16)
+    p_last = torch.empty(t, h, device=device, dtype=torch.bfloat16)
+    p_i64 = torch.empty(4, t, device=device, dtype=torch.int64)
+
+    def pack():
+        _lib.call("spx_pack_batch", _lib.ptr(hs), _lib.dtype_code(hs), rows, 3, h, _lib.ptr(ids),
+                  _lib.ptr(lm), 8, None, _lib.ptr(plan[0]), _lib.ptr(plan[1]), n_docs, t, 1,
+                  _lib.ptr(p_aux), _lib.ptr(p_last), _lib.ptr(p_i64[0]), _lib.ptr(p_i64[1]),
+                  _lib.ptr(p_i64[2]), _lib.ptr(p_i64[3]), st)
+
+    ms = time_events(torch, pack, 20)
+    hbm("pack_batch_kernel[8 documents -> T x (3H + H) bf16, ids, mask, positions, document ids]",
+        2.0 * t * 4 * h * 2 + t * 7 * 8, ms, 0)
+    del hs, p_aux, p_last
 
     # TTT attention at the last step (k = K-1 diagonals): forward and backward
     step = k_steps - 1

@@ -112,6 +112,32 @@ int spx_label_ce_bwd(const void* logits, int64_t ld_logits, const int64_t* label
                      int64_t vocab, int dtype, int64_t ignore_index, void* dlogits,
                      int64_t ld_out, void* stream);
 
+/* Batch layout producer: packs `n_docs` samples, staged back to back in the layout
+ * of the hidden-state files (`src_hs [n_src_rows, layers + 1, hidden]`, bf16 or fp32,
+ * with `src_ids [n_src_rows]` int64 and `src_mask [n_src_rows]` of `mask_elem`-byte
+ * elements), into the one-row batch the draft models consume.  Output row r of
+ * document d (the last d with out_start[d] <= r < out_start[n_docs]), offset
+ * o = r - out_start[d]:
+ *   out_aux [r, :]  = bf16(src_hs[src_start[d] + o, 0:layers, :])        (may be NULL)
+ *   out_last[r, :]  = bf16(src_hs[src_start[d] + o + shift, layers, :])  (may be NULL)
+ *   out_ids / out_mask [r] = src_ids / src_mask [src_start[d] + o + shift]
+ *   out_pos [r] = src_pos ? src_pos[src_start[d] + o + shift] : o + shift
+ *   out_doc [r] = d
+ * rows r >= out_start[n_docs] are padding: zeros, out_doc = -1.  `src_start` and
+ * `out_start` are device int64 arrays of n_docs + 1 entries (out_start[0] = 0,
+ * non-decreasing, out_start[n_docs] <= max_len); a row whose source index falls outside
+ * [0, n_src_rows) is written as padding, never read.  shift = 1 gives the EAGLE3
+ * alignment (x[i+1], g[i], y[i+1], mask[i+1]), shift = 0 the DFlash / MTP one.
+ * Replaces, on the device, CollateFn.__call__ (train/data.py:323-393) composed with
+ * shift_batch (models/eagle3/data.py:8-44) or shift_batch_mtp (models/mtp/data.py:6-18)
+ * and the layer split of ArrowDataset._get_raw_data (train/data.py:293-303). */
+int spx_pack_batch(const void* src_hs, int src_dtype, int64_t n_src_rows, int64_t layers,
+                   int64_t hidden, const int64_t* src_ids, const void* src_mask, int mask_elem,
+                   const int64_t* src_pos, const int64_t* src_start, const int64_t* out_start,
+                   int64_t n_docs, int64_t max_len, int shift, void* out_aux, void* out_last,
+                   int64_t* out_ids, void* out_mask, int64_t* out_pos, int64_t* out_doc,
+                   void* stream);
+
 /* Masked mean and acceptance chain of one TTT step over `rows` aligned rows:
  *   out[0] = weight * sum_r loss[r] * m_r / (sum_r m_r + 1e-5)
  *            (loss_function, losses/utils.py:269-304, with the exp_loss_decay
