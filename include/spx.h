@@ -280,12 +280,27 @@ int spx_rmsnorm_fwd(const void* x, int64_t ld_x, const void* weight, void* y,
                     void* stream);
 /* number of partial-sum slots the backward needs: dw_scratch holds slots * H floats */
 int64_t spx_rmsnorm_bwd_slots(int64_t rows, int64_t H);
-/* dx and (optionally, dweight != NULL) dweight = sum_rows dy * xhat, reduced in a
- * fixed order (deterministic). */
+/* dx (may be NULL when only dweight is wanted) and (optionally, dweight != NULL)
+ * dweight = sum_rows dy * xhat, reduced in a fixed order (deterministic). */
 int spx_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weight, const void* dy,
                     int64_t ld_dy, const float* rstd, void* dx, int64_t ld_dx,
                     void* dweight, float* dw_scratch, int64_t rows, int64_t H,
                     void* stream);
+/* The residual add in front of a norm fused into it: sum = bf16(a + b) (written, it is
+ * the residual stream) and y = rmsnorm(sum).  Replaces `hidden_states = residual +
+ * hidden_states` followed by the next RMSNorm in the decoder layer
+ * (models/eagle3/model_definitions.py:96-110 and the HF LlamaDecoderLayer it patches;
+ * models/eagle3/core.py:302-306 for the final norm). */
+int spx_add_rmsnorm_fwd(const void* a, int64_t ld_a, const void* b, int64_t ld_b, void* sum,
+                        int64_t ld_sum, const void* weight, void* y, int64_t ld_y,
+                        float* rstd, int64_t rows, int64_t H, float eps, void* stream);
+/* Its backward: dx = dres + rmsnorm_bwd(dy) in one rounding, where dres (may be NULL)
+ * is the gradient reaching `sum` along the residual stream; x is the saved `sum`.
+ * dx is the gradient of both a and b. */
+int spx_add_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weight, const void* dy,
+                        int64_t ld_dy, const void* dres, int64_t ld_dres, const float* rstd,
+                        void* dx, int64_t ld_dx, void* dweight, float* dw_scratch,
+                        int64_t rows, int64_t H, void* stream);
 
 /* Rotary embedding fused with the head-major relayout that precedes attention
  * (apply_rotary_pos_emb + the view/transpose of LlamaAttention.forward; for

@@ -36,11 +36,14 @@ __device__ __forceinline__ float block_sum_256(float v, float* lds) {
 // ---------------------------------------------------------------- RMSNorm
 // y = w * bf16(x * rsqrt(mean(x^2) + eps));  one workgroup per row (H >= 512) or one
 // wave per row (small H, e.g. per-head q/k norm).  MAXC = 16-byte chunks a lane keeps.
-template <int MAXC, bool WAVE_ROWS>
+// RES: x is the sum of two tensors, x = bf16(x + res) (one rounding, as a bf16 tensor add),
+// which is also written to `sum` for the residual stream.
+template <int MAXC, bool WAVE_ROWS, bool RES = false>
 __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(
     const uint16_t* __restrict__ x, int64_t ld_x, const uint16_t* __restrict__ w,
     uint16_t* __restrict__ y, int64_t ld_y, float* __restrict__ rstd, int64_t rows, int H,
-    float eps) {
+    float eps, const uint16_t* __restrict__ res = nullptr, int64_t ld_res = 0,
+    uint16_t* __restrict__ sum = nullptr, int64_t ld_sum = 0) {
   __shared__ float red[4];
   const int nthr = WAVE_ROWS ? 64 : 256;
   const int t = WAVE_ROWS ? (threadIdx.x & 63) : threadIdx.x;
@@ -54,6 +57,15 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(
     const int ch = t + c * nthr;
     if (ch < nch) {
       unpack8f(*reinterpret_cast<const u32x4*>(x + row * ld_x + ch * 8), v[c]);
+      if (RES) {
+        float b[8];
+        unpack8f(*reinterpret_cast<const u32x4*>(res + row * ld_res + ch * 8), b);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[c][e] += b[e];
+        const u32x4 packed = pack8f(v[c]);
+        *reinterpret_cast<u32x4*>(sum + row * ld_sum + ch * 8) = packed;
+        unpack8f(packed, v[c]);
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) ss = fmaf(v[c][e], v[c][e], ss);
     }
@@ -76,11 +88,14 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(
 
 // dx = rstd * (g - xhat * mean(g * xhat)), g = dy * w, xhat = x * rstd;
 // dw partial sums: block b accumulates the rows b, b + gridDim.x, ... per column.
+// dres (may be null): gradient that reaches x along the residual stream, added before the
+// one rounding of dx.  dx may be null (only dw wanted).
 template <int MAXC, bool WAVE_ROWS>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(
     const uint16_t* __restrict__ x, int64_t ld_x, const uint16_t* __restrict__ w,
     const uint16_t* __restrict__ dy, int64_t ld_dy, const float* __restrict__ rstd,
-    uint16_t* __restrict__ dx, int64_t ld_dx, float* __restrict__ dw_part, int64_t rows, int H) {
+    uint16_t* __restrict__ dx, int64_t ld_dx, float* __restrict__ dw_part, int64_t rows, int H,
+    const uint16_t* __restrict__ dres = nullptr, int64_t ld_dres = 0) {
   __shared__ float red[4];
   const int nthr = WAVE_ROWS ? 64 : 256;
   const int t = WAVE_ROWS ? (threadIdx.x & 63) : threadIdx.x;
@@ -116,6 +131,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(
         }
       }
     }
+    if (dx == nullptr) continue;  // uniform: only the weight gradient is wanted
     dot = WAVE_ROWS ? wave_sum(dot) : block_sum_256(dot, red);
     const float mean = dot / (float)H;
 #pragma unroll
@@ -125,6 +141,12 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(
         float o[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = r * (g[c][e] - xh[c][e] * mean);
+        if (dres) {
+          float dr[8];
+          unpack8f(*reinterpret_cast<const u32x4*>(dres + row * ld_dres + ch * 8), dr);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) o[e] += dr[e];
+        }
         *reinterpret_cast<u32x4*>(dx + row * ld_dx + ch * 8) = pack8f(o);
       }
     }
@@ -146,20 +168,28 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(
 }
 
 // dw[c] = sum_s dw_part[s, c]  (fixed order: deterministic), bf16 out.  One workgroup
-// sums 64 columns: wave w adds the slots w, w+4, ..., then the four partial sums are
-// combined through LDS.
+// sums 32 columns (one 128-byte line per slot row): lane = (slot row j of 32, 4 columns),
+// thread j adds the slots j, j + 32, ..., then the 32 partial sums are combined through LDS
+// in a fixed order.
 __global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ part, int64_t slots,
                                                      int H, uint16_t* __restrict__ out) {
-  __shared__ float red[4][64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int c = blockIdx.x * 64 + lane;
-  float s = 0.f;
+  __shared__ float red[32][33];
+  const int q = threadIdx.x & 7, j = threadIdx.x >> 3;
+  const int c = blockIdx.x * 32 + q * 4;
+  f32x4 s = {0.f, 0.f, 0.f, 0.f};
   if (c < H)
-    for (int64_t i = wave; i < slots; i += 4) s += part[i * H + c];
-  red[wave][lane] = s;
+    for (int64_t i = j; i < slots; i += 32) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(part + i * H + c);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+  red[j][q * 4 + 0] = s.x; red[j][q * 4 + 1] = s.y; red[j][q * 4 + 2] = s.z; red[j][q * 4 + 3] = s.w;
   __syncthreads();
-  if (wave == 0 && c < H)
-    out[c] = (uint16_t)f32_to_bf16_bits((red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]));
+  if (threadIdx.x < 32 && blockIdx.x * 32 + threadIdx.x < H) {
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < 32; ++k) t += red[k][threadIdx.x];
+    out[blockIdx.x * 32 + threadIdx.x] = (uint16_t)f32_to_bf16_bits(t);
+  }
 }
 
 // ---------------------------------------------------------------- RoPE + relayout
@@ -254,64 +284,108 @@ using namespace spx;
 
 extern "C" int64_t spx_rmsnorm_bwd_slots(int64_t rows, int64_t H) {
   if (H <= 512) return 4 * (rows < 1024 ? (rows + 3) / 4 : 256);
-  return rows < 256 ? rows : 256;
+  return rows < 1024 ? rows : 1024;  // four workgroups per compute unit
+}
+
+static int rmsnorm_fwd_launch(const char* fn, const void* x, int64_t ld_x, const void* res, int64_t ld_res,
+                              void* sum, int64_t ld_sum, const void* weight, void* y, int64_t ld_y,
+                              float* rstd, int64_t rows, int64_t H, float eps, void* stream) {
+  if (!(rows >= 0 && H > 0)) return fail_arg(fn, "bad sizes");
+  if (!(H % 8 == 0 && ld_x % 8 == 0 && ld_y % 8 == 0 && ld_res % 8 == 0 && ld_sum % 8 == 0))
+    return fail_arg(fn, "H and the row strides must be multiples of 8");
+  if (H > 16384) return fail_arg(fn, "H must be at most 16384");
+  if (rows >= (1ll << 31)) return fail_arg(fn, "too many rows");
+  if (rows == 0) return SPX_OK;
+  if (!(x && weight && y)) return fail_arg(fn, "null buffer");
+  if (!(al16(x) && al16(weight) && al16(y) && al16(res) && al16(sum)))
+    return fail_arg(fn, "buffers must be 16-byte aligned");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  auto xp = reinterpret_cast<const uint16_t*>(x);
+  auto rp = reinterpret_cast<const uint16_t*>(res);
+  auto sp = reinterpret_cast<uint16_t*>(sum);
+  auto wp = reinterpret_cast<const uint16_t*>(weight);
+  auto yp = reinterpret_cast<uint16_t*>(y);
+#define SPX_LAUNCH(MAXC, WR, GRID)                                                                  \
+  do {                                                                                              \
+    if (res)                                                                                        \
+      hipLaunchKernelGGL((rmsnorm_fwd_kernel<MAXC, WR, true>), dim3((unsigned)(GRID)), dim3(256), 0, st, \
+                         xp, ld_x, wp, yp, ld_y, rstd, rows, (int)H, eps, rp, ld_res, sp, ld_sum);  \
+    else                                                                                            \
+      hipLaunchKernelGGL((rmsnorm_fwd_kernel<MAXC, WR, false>), dim3((unsigned)(GRID)), dim3(256), 0, st, \
+                         xp, ld_x, wp, yp, ld_y, rstd, rows, (int)H, eps, nullptr, 0, nullptr, 0);  \
+  } while (0)
+  if (H <= 512) SPX_LAUNCH(1, true, (rows + 3) / 4);
+  else if (H <= 4096) SPX_LAUNCH(2, false, rows);
+  else SPX_LAUNCH(8, false, rows);
+#undef SPX_LAUNCH
+  return check_launch(fn);
 }
 
 extern "C" int spx_rmsnorm_fwd(const void* x, int64_t ld_x, const void* weight, void* y, int64_t ld_y,
                                float* rstd, int64_t rows, int64_t H, float eps, void* stream) {
-  SPX_REQUIRE(rows >= 0 && H > 0, "bad sizes");
-  SPX_REQUIRE(H % 8 == 0 && ld_x % 8 == 0 && ld_y % 8 == 0, "H and the row strides must be multiples of 8");
-  SPX_REQUIRE(H <= 16384, "H must be at most 16384");
-  SPX_REQUIRE(rows < (1ll << 31), "too many rows");
-  if (rows == 0) return SPX_OK;
-  SPX_REQUIRE(x && weight && y, "null buffer");
-  SPX_REQUIRE(al16(x) && al16(weight) && al16(y), "buffers must be 16-byte aligned");
-  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  auto xp = reinterpret_cast<const uint16_t*>(x);
-  auto wp = reinterpret_cast<const uint16_t*>(weight);
-  auto yp = reinterpret_cast<uint16_t*>(y);
-  if (H <= 512)
-    hipLaunchKernelGGL((rmsnorm_fwd_kernel<1, true>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, xp,
-                       ld_x, wp, yp, ld_y, rstd, rows, (int)H, eps);
-  else if (H <= 4096)
-    hipLaunchKernelGGL((rmsnorm_fwd_kernel<2, false>), dim3((unsigned)rows), dim3(256), 0, st, xp, ld_x, wp,
-                       yp, ld_y, rstd, rows, (int)H, eps);
-  else
-    hipLaunchKernelGGL((rmsnorm_fwd_kernel<8, false>), dim3((unsigned)rows), dim3(256), 0, st, xp, ld_x, wp,
-                       yp, ld_y, rstd, rows, (int)H, eps);
-  return check_launch(__func__);
+  return rmsnorm_fwd_launch(__func__, x, ld_x, nullptr, 0, nullptr, 0, weight, y, ld_y, rstd, rows, H, eps,
+                            stream);
 }
 
-extern "C" int spx_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weight, const void* dy,
-                               int64_t ld_dy, const float* rstd, void* dx, int64_t ld_dx, void* dweight,
-                               float* dw_scratch, int64_t rows, int64_t H, void* stream) {
-  SPX_REQUIRE(rows > 0 && H > 0, "bad sizes");
-  SPX_REQUIRE(H % 8 == 0 && ld_x % 8 == 0 && ld_dy % 8 == 0 && ld_dx % 8 == 0,
-              "H and the row strides must be multiples of 8");
-  SPX_REQUIRE(H <= 16384, "H must be at most 16384");
-  SPX_REQUIRE(x && weight && dy && rstd && dx, "null buffer");
-  SPX_REQUIRE(!dweight || dw_scratch, "dweight needs dw_scratch (spx_rmsnorm_bwd_slots(rows, H) * H floats)");
-  SPX_REQUIRE(al16(x) && al16(weight) && al16(dy) && al16(dx) && al16(dw_scratch), "buffers must be 16-byte aligned");
+extern "C" int spx_add_rmsnorm_fwd(const void* a, int64_t ld_a, const void* b, int64_t ld_b, void* sum,
+                                   int64_t ld_sum, const void* weight, void* y, int64_t ld_y, float* rstd,
+                                   int64_t rows, int64_t H, float eps, void* stream) {
+  SPX_REQUIRE(rows == 0 || (b && sum), "null buffer");
+  return rmsnorm_fwd_launch(__func__, a, ld_a, b, ld_b, sum, ld_sum, weight, y, ld_y, rstd, rows, H, eps,
+                            stream);
+}
+
+static int rmsnorm_bwd_launch(const char* fn, const void* x, int64_t ld_x, const void* weight, const void* dy,
+                              int64_t ld_dy, const void* dres, int64_t ld_dres, const float* rstd, void* dx,
+                              int64_t ld_dx, void* dweight, float* dw_scratch, int64_t rows, int64_t H,
+                              void* stream) {
+  if (!(rows > 0 && H > 0)) return fail_arg(fn, "bad sizes");
+  if (!(H % 8 == 0 && ld_x % 8 == 0 && ld_dy % 8 == 0 && ld_dx % 8 == 0 && ld_dres % 8 == 0))
+    return fail_arg(fn, "H and the row strides must be multiples of 8");
+  if (H > 16384) return fail_arg(fn, "H must be at most 16384");
+  if (!(x && weight && dy && rstd)) return fail_arg(fn, "null buffer");
+  if (!(dx || dweight)) return fail_arg(fn, "neither dx nor dweight requested");
+  if (dres && !dx) return fail_arg(fn, "a residual gradient needs dx");
+  if (dweight && !dw_scratch)
+    return fail_arg(fn, "dweight needs dw_scratch (spx_rmsnorm_bwd_slots(rows, H) * H floats)");
+  if (!(al16(x) && al16(weight) && al16(dy) && al16(dx) && al16(dw_scratch) && al16(dres)))
+    return fail_arg(fn, "buffers must be 16-byte aligned");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   auto xp = reinterpret_cast<const uint16_t*>(x);
   auto wp = reinterpret_cast<const uint16_t*>(weight);
   auto dyp = reinterpret_cast<const uint16_t*>(dy);
+  auto drp = reinterpret_cast<const uint16_t*>(dres);
   auto dxp = reinterpret_cast<uint16_t*>(dx);
   float* part = dweight ? dw_scratch : nullptr;
   const int64_t slots = spx_rmsnorm_bwd_slots(rows, H);
   if (H <= 512)
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<1, true>), dim3((unsigned)(slots / 4)), dim3(256), 0, st, xp, ld_x,
-                       wp, dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H);
+                       wp, dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H, drp, ld_dres);
   else if (H <= 4096)
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<2, false>), dim3((unsigned)slots), dim3(256), 0, st, xp, ld_x, wp,
-                       dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H);
+                       dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H, drp, ld_dres);
   else
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<8, false>), dim3((unsigned)slots), dim3(256), 0, st, xp, ld_x, wp,
-                       dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H);
+                       dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H, drp, ld_dres);
   if (dweight)
-    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((H + 63) / 64)), dim3(256), 0, st, part, slots, (int)H,
+    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((H + 31) / 32)), dim3(256), 0, st, part, slots, (int)H,
                        reinterpret_cast<uint16_t*>(dweight));
-  return check_launch(__func__);
+  return check_launch(fn);
+}
+
+extern "C" int spx_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weight, const void* dy,
+                               int64_t ld_dy, const float* rstd, void* dx, int64_t ld_dx, void* dweight,
+                               float* dw_scratch, int64_t rows, int64_t H, void* stream) {
+  return rmsnorm_bwd_launch(__func__, x, ld_x, weight, dy, ld_dy, nullptr, 0, rstd, dx, ld_dx, dweight,
+                            dw_scratch, rows, H, stream);
+}
+
+extern "C" int spx_add_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weight, const void* dy,
+                                   int64_t ld_dy, const void* dres, int64_t ld_dres, const float* rstd,
+                                   void* dx, int64_t ld_dx, void* dweight, float* dw_scratch, int64_t rows,
+                                   int64_t H, void* stream) {
+  return rmsnorm_bwd_launch(__func__, x, ld_x, weight, dy, ld_dy, dres, ld_dres, rstd, dx, ld_dx, dweight,
+                            dw_scratch, rows, H, stream);
 }
 
 extern "C" int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* position_ids,

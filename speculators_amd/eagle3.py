@@ -17,6 +17,7 @@ The decoder-internal projections use PyTorch's (hipBLASLt) matmul.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from typing import NamedTuple
 
 import torch
 import torch.nn.functional as F
@@ -80,20 +81,30 @@ class Attention(nn.Module):
         self.qk_norm = cfg.qk_norm
         self.scaling = d ** -0.5
         self.attn_fn = A.ALL_ATTENTION_FUNCTIONS[cfg.attn_implementation]
+        self._merged_qkv = gemm._MergedQKV()
 
     def forward(self, x, position_ids, pos_offset, inv_freq, cache: dict, mask):
         t = x.shape[1]
         lin = gemm.linear_accumulate
-        q = lin(x, self.q_proj.weight)
-        k = lin(x, self.k_proj.weight)
-        v = lin(x, self.v_proj.weight)
-        if self.qk_norm:
-            q = self.q_norm(q.view(1, t, self.hq, self.d)).view(1, t, self.hq * self.d)
-            k = self.k_norm(k.view(1, t, self.hkv, self.d)).view(1, t, self.hkv * self.d)
-        # rotary embedding + [T, heads*D] -> [heads, T, D] in one pass each
-        q = FO.rope_relayout(q, position_ids, inv_freq, self.hq, True, pos_offset)
-        k = FO.rope_relayout(k, position_ids, inv_freq, self.hkv, True, pos_offset)
-        v = FO.rope_relayout(v, position_ids, inv_freq, self.hkv, False, 0)
+        if not self.qk_norm and gemm.FUSE_WGRAD_ACCUMULATION and torch.is_grad_enabled():
+            # one GEMM for q, k and v; rotary embedding + [T, heads*D] -> [heads, T, D] fused behind it
+            pos = position_ids.reshape(-1)
+            if pos.dtype != torch.int64:
+                pos = pos.to(torch.int64)
+            q, k, v = gemm.qkv_rope(x, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight,
+                                    pos.contiguous(), inv_freq, self.hq, self.hkv, self.d, pos_offset,
+                                    self._merged_qkv)
+        else:
+            q = lin(x, self.q_proj.weight)
+            k = lin(x, self.k_proj.weight)
+            v = lin(x, self.v_proj.weight)
+            if self.qk_norm:
+                q = self.q_norm(q.view(1, t, self.hq, self.d)).view(1, t, self.hq * self.d)
+                k = self.k_norm(k.view(1, t, self.hkv, self.d)).view(1, t, self.hkv * self.d)
+            # rotary embedding + [T, heads*D] -> [heads, T, D] in one pass each
+            q = FO.rope_relayout(q, position_ids, inv_freq, self.hq, True, pos_offset)
+            k = FO.rope_relayout(k, position_ids, inv_freq, self.hkv, True, pos_offset)
+            v = FO.rope_relayout(v, position_ids, inv_freq, self.hkv, False, 0)
         # the K/V cache grows by T keys per TTT step (DynamicCache.update in the reference)
         cache["k"] = k if "k" not in cache else torch.cat([cache["k"], k], dim=2)
         cache["v"] = v if "v" not in cache else torch.cat([cache["v"], v], dim=2)
@@ -114,6 +125,13 @@ class MLP(nn.Module):
                    self.down_proj.weight)
 
 
+class _Prenormed(NamedTuple):
+    """A hidden state together with the next layer's input norm of it."""
+
+    value: torch.Tensor
+    normed: torch.Tensor
+
+
 class DecoderLayer(nn.Module):
     """Layer 0 carries the EAGLE3 first-layer changes
     (models/eagle3/model_definitions.py:14-110): q/k/v read ``cat([embeds, hidden])``
@@ -131,22 +149,37 @@ class DecoderLayer(nn.Module):
         if self.first:
             self.hidden_norm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
 
-    def forward(self, x, position_ids, pos_offset, inv_freq, cache, mask):
+    def forward(self, x, position_ids, pos_offset, inv_freq, cache, mask, next_norm=None):
+        """``x``: the hidden state, or for the first layer the pair ``(embeds, hidden)`` (their
+        concatenation is what the reference passes).  With ``next_norm`` (the RMSNorm that
+        consumes this layer's output) the result is ``(out, next_norm(out))``: the last
+        residual add is fused into that norm."""
         if self.first:
-            h = self.cfg.hidden_size
-            embeds, hidden = x[..., :h], x[..., h:]
-            residual = hidden
-            embeds = self.input_layernorm(embeds)
-            hidden = self.hidden_norm(hidden)
+            embeds, hidden = x
+            eps = self.cfg.rms_norm_eps
             if self.cfg.norm_before_residual:
+                embeds = self.input_layernorm(embeds)
+                hidden = self.hidden_norm(hidden)
                 residual = hidden
-            a = self.self_attn(torch.cat([embeds, hidden], dim=-1), position_ids, pos_offset, inv_freq,
-                               cache, mask)
+                xin = torch.cat([embeds, hidden], dim=-1)
+            else:
+                residual = hidden
+                # both norms write straight into the halves of the 2H-wide projection input
+                xin = FO.pair_norm_cat(embeds, hidden, self.input_layernorm.weight,
+                                       self.hidden_norm.weight, eps)
+            a = self.self_attn(xin, position_ids, pos_offset, inv_freq, cache, mask)
         else:
-            residual = x
-            a = self.self_attn(self.input_layernorm(x), position_ids, pos_offset, inv_freq, cache, mask)
-        y = residual + a
-        return y + self.mlp(self.post_attention_layernorm(y))
+            if isinstance(x, _Prenormed):  # the previous layer already applied this layer's input norm
+                residual, xn = x
+            else:
+                residual, xn = x, self.input_layernorm(x)
+            a = self.self_attn(xn, position_ids, pos_offset, inv_freq, cache, mask)
+        post = self.post_attention_layernorm
+        y, z = FO.add_rms_norm(residual, a, post.weight, post.eps)
+        m = self.mlp(z)
+        if next_norm is None:
+            return y + m
+        return FO.add_rms_norm(y, m, next_norm.weight, next_norm.eps)
 
 
 class Eagle3DraftModel(nn.Module):
@@ -266,16 +299,19 @@ class Eagle3DraftModel(nn.Module):
         for step in range(ttt_steps):
             with torch.no_grad():
                 embeds = F.embedding(input_ids, self.embed_tokens.weight)
-            y = torch.cat([embeds.to(hidden.dtype), hidden], dim=-1)
+            y = (embeds.to(hidden.dtype), hidden)
+            normed = None
+            last = len(self.layers) - 1
             for li, layer in enumerate(self.layers):
                 mask = sw_mask if li in cfg.sliding_layers else full_mask
-                y = layer(y, position_ids, step, inv_freq, caches[li], mask)
-            if cfg.norm_output:
-                hidden = self.norm(y)
-                logits = self._linear(hidden, self.lm_head.weight, frozen=True)
-            else:
-                hidden = y
-                logits = self._linear(self.norm(y), self.lm_head.weight, frozen=True)
+                # the norm that reads this layer's output: the next layer's input norm, or the
+                # final norm -- the layer fuses its last residual add into it
+                nxt = self.norm if li == last else self.layers[li + 1].input_layernorm
+                y, normed = layer(y, position_ids, step, inv_freq, caches[li], mask, next_norm=nxt)
+                if li != last:
+                    y = _Prenormed(y, normed)
+            hidden = normed if cfg.norm_output else y
+            logits = self._linear(normed, self.lm_head.weight, frozen=True)
 
             if return_loss:
                 s_loss, s_metrics, pred = MT.compute_metrics(

@@ -43,9 +43,7 @@ class _RMSNorm(torch.autograd.Function):
         dx = torch.empty(rows, h, device=x2.device, dtype=torch.bfloat16)
         dw = scratch = None
         if ctx.needs_input_grad[1]:
-            slots = int(_lib.load().spx_rmsnorm_bwd_slots(rows, h))
-            scratch = torch.empty(slots * h, device=x2.device, dtype=torch.float32)
-            dw = torch.empty(h, device=x2.device, dtype=torch.bfloat16)
+            scratch, dw = _dw_buffers(rows, h, x2.device)
         _lib.call("spx_rmsnorm_bwd", _lib.ptr(x2), x2.stride(0), _lib.ptr(w), _lib.ptr(dy2),
                   dy2.stride(0), _lib.ptr(rstd), _lib.ptr(dx), h, _lib.ptr(dw), _lib.ptr(scratch),
                   rows, h, _lib.stream_ptr(x2.device))
@@ -54,6 +52,125 @@ class _RMSNorm(torch.autograd.Function):
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return _RMSNorm.apply(x, weight, eps)
+
+
+def _dw_buffers(rows: int, h: int, device):
+    slots = int(_lib.load().spx_rmsnorm_bwd_slots(rows, h))
+    return (torch.empty(slots * h, device=device, dtype=torch.float32),
+            torch.empty(h, device=device, dtype=torch.bfloat16))
+
+
+class _AddRMSNorm(torch.autograd.Function):
+    """``s = a + b; y = rms_norm(s)`` in one pass; returns ``(s, y)``.  The backward folds the
+    gradient that reaches ``s`` along the residual stream into the norm's input gradient."""
+
+    @staticmethod
+    def forward(ctx, a, b, weight, eps):
+        _need_bf16(a, b, weight)
+        h = a.shape[-1]
+        a2, b2 = a.reshape(-1, h), b.reshape(-1, h)
+        if a2.stride(1) != 1:
+            a2 = a2.contiguous()
+        if b2.stride(1) != 1:
+            b2 = b2.contiguous()
+        rows = a2.shape[0]
+        s = torch.empty(rows, h, device=a.device, dtype=torch.bfloat16)
+        y = torch.empty(rows, h, device=a.device, dtype=torch.bfloat16)
+        rstd = torch.empty(rows, device=a.device, dtype=torch.float32)
+        w = weight.contiguous()
+        _lib.call("spx_add_rmsnorm_fwd", _lib.ptr(a2), a2.stride(0), _lib.ptr(b2), b2.stride(0),
+                  _lib.ptr(s), h, _lib.ptr(w), _lib.ptr(y), h, _lib.ptr(rstd), rows, h, float(eps),
+                  _lib.stream_ptr(a.device))
+        ctx.save_for_backward(s, w, rstd)
+        ctx.shape = a.shape
+        ctx.set_materialize_grads(False)  # an unused output arrives as None, not as zeros
+        return s.view(a.shape), y.view(a.shape)
+
+    @staticmethod
+    def backward(ctx, ds, dy):
+        s, w, rstd = ctx.saved_tensors
+        rows, h = s.shape
+        if dy is None:  # the normalised output was not used
+            return ds, ds, None, None
+        dy2 = dy.reshape(rows, h).to(torch.bfloat16)
+        if dy2.stride(1) != 1:
+            dy2 = dy2.contiguous()
+        ds2 = None
+        if ds is not None:
+            ds2 = ds.reshape(rows, h).to(torch.bfloat16)
+            if ds2.stride(1) != 1:
+                ds2 = ds2.contiguous()
+        dx = torch.empty(rows, h, device=s.device, dtype=torch.bfloat16)
+        scratch = dw = None
+        if ctx.needs_input_grad[2]:
+            scratch, dw = _dw_buffers(rows, h, s.device)
+        _lib.call("spx_add_rmsnorm_bwd", _lib.ptr(s), h, _lib.ptr(w), _lib.ptr(dy2), dy2.stride(0),
+                  _lib.ptr(ds2), ds2.stride(0) if ds2 is not None else 0, _lib.ptr(rstd), _lib.ptr(dx),
+                  h, _lib.ptr(dw), _lib.ptr(scratch), rows, h, _lib.stream_ptr(s.device))
+        dx = dx.view(ctx.shape)
+        return dx, dx, dw, None
+
+
+def add_rms_norm(a: torch.Tensor, b: torch.Tensor, weight: torch.Tensor, eps: float):
+    """``(a + b, rms_norm(a + b))``: the residual add in front of a norm, fused into it."""
+    return _AddRMSNorm.apply(a, b, weight, eps)
+
+
+class _PairNormCat(torch.autograd.Function):
+    """``cat([rms_norm(a, wa), rms_norm(b, wb)], -1)`` written straight into the halves of one
+    ``[rows, 2H]`` buffer (the input of the first EAGLE3 layer's q/k/v projections,
+    models/eagle3/model_definitions.py:70-94)."""
+
+    @staticmethod
+    def forward(ctx, a, b, wa, wb, eps):
+        _need_bf16(a, b, wa, wb)
+        h = a.shape[-1]
+        a2, b2 = a.reshape(-1, h), b.reshape(-1, h)
+        if a2.stride(1) != 1:
+            a2 = a2.contiguous()
+        if b2.stride(1) != 1:
+            b2 = b2.contiguous()
+        rows = a2.shape[0]
+        out = torch.empty(rows, 2 * h, device=a.device, dtype=torch.bfloat16)
+        rstd = torch.empty(2, rows, device=a.device, dtype=torch.float32)
+        wa, wb = wa.contiguous(), wb.contiguous()
+        st = _lib.stream_ptr(a.device)
+        _lib.call("spx_rmsnorm_fwd", _lib.ptr(a2), a2.stride(0), _lib.ptr(wa), _lib.ptr(out), 2 * h,
+                  _lib.ptr(rstd[0]), rows, h, float(eps), st)
+        _lib.call("spx_rmsnorm_fwd", _lib.ptr(b2), b2.stride(0), _lib.ptr(wb), _lib.ptr(out[:, h:]), 2 * h,
+                  _lib.ptr(rstd[1]), rows, h, float(eps), st)
+        ctx.save_for_backward(a2, b2, wa, wb, rstd)
+        ctx.shapes = (a.shape, b.shape)
+        return out.view(*a.shape[:-1], 2 * h)
+
+    @staticmethod
+    def backward(ctx, dy):
+        a2, b2, wa, wb, rstd = ctx.saved_tensors
+        rows, h = a2.shape
+        dy2 = dy.reshape(rows, 2 * h).to(torch.bfloat16)
+        if dy2.stride(1) != 1:
+            dy2 = dy2.contiguous()
+        st = _lib.stream_ptr(a2.device)
+        grads = []
+        for i, (x, w) in enumerate(((a2, wa), (b2, wb))):
+            need_dx, need_dw = ctx.needs_input_grad[i], ctx.needs_input_grad[2 + i]
+            dx = dw = scratch = None
+            if need_dx:
+                dx = torch.empty(rows, h, device=x.device, dtype=torch.bfloat16)
+            if need_dw:
+                scratch, dw = _dw_buffers(rows, h, x.device)
+            if need_dx or need_dw:
+                half = dy2[:, i * h:]
+                _lib.call("spx_rmsnorm_bwd", _lib.ptr(x), x.stride(0), _lib.ptr(w), _lib.ptr(half),
+                          dy2.stride(0), _lib.ptr(rstd[i]), _lib.ptr(dx), h, _lib.ptr(dw),
+                          _lib.ptr(scratch), rows, h, st)
+            grads.append((dx.view(ctx.shapes[i]) if dx is not None else None, dw))
+        return grads[0][0], grads[1][0], grads[0][1], grads[1][1], None
+
+
+def pair_norm_cat(a, b, weight_a, weight_b, eps: float) -> torch.Tensor:
+    """See ``_PairNormCat``."""
+    return _PairNormCat.apply(a, b, weight_a, weight_b, eps)
 
 
 class _RopeRelayout(torch.autograd.Function):

@@ -114,3 +114,107 @@ def linear_accumulate(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         return torch.nn.functional.linear(x, weight)
     # autograd must see a differentiable input even when only the weight needs a gradient
     return _LinearAccumulate.apply(x, weight)
+
+
+class _MergedQKV:
+    """Per-module state of the merged q/k/v projection: the concatenated weight of the current
+    weight versions, and the merged gradient buffer the three ``.grad`` tensors are views of."""
+
+    def __init__(self):
+        self.key = None
+        self.weight = None
+        self.grad = None
+
+    def merged_weight(self, ws):
+        key = tuple((w.data_ptr(), w._version) for w in ws)
+        if key != self.key:
+            self.weight = torch.cat([w.detach() for w in ws], dim=0)
+            self.key = key
+        return self.weight
+
+    def accumulate(self, ws, dy2, x2):
+        """``grad(w_i) += dy2[:, rows_i].T @ x2`` for the three weights with one GEMM.  While the
+        three ``.grad`` are the views this object handed out, the GEMM adds into their shared buffer
+        (beta = 1); otherwise (gradients that came from elsewhere) it falls back to one add each."""
+        sizes = [w.shape[0] for w in ws]
+        views = None
+        if self.grad is not None:
+            views = self.grad.split(sizes, dim=0)
+            if not all(w.grad is not None and w.grad.data_ptr() == v.data_ptr()
+                       and w.grad.shape == v.shape for w, v in zip(ws, views, strict=True)):
+                views = None
+        if views is not None:
+            torch.addmm(self.grad, dy2.t(), x2, out=self.grad)
+            return
+        fresh = torch.matmul(dy2.t(), x2)
+        parts = fresh.split(sizes, dim=0)
+        if all(w.grad is None for w in ws):
+            self.grad = fresh
+            for w, v in zip(ws, parts, strict=True):
+                w.grad = v
+        else:
+            self.grad = None
+            for w, v in zip(ws, parts, strict=True):
+                if w.requires_grad:
+                    w.grad = v.clone() if w.grad is None else w.grad.add_(v)
+
+
+class _QKVRope(torch.autograd.Function):
+    """q/k/v projections of one input as ONE GEMM against the concatenated weight, followed by
+    the rotary embedding + head-major relayout of each part.  The backward undoes the relayout
+    into the three column blocks of one ``[T, Nq + 2 Nkv]`` buffer, so the input gradient is one
+    GEMM (no per-projection partial results to add up) and the weight gradient one GEMM that
+    accumulates across TTT steps."""
+
+    @staticmethod
+    def forward(ctx, x, wq, wk, wv, position_ids, inv_freq, hq, hkv, d, offset, state):
+        t = x.shape[-2]
+        x2 = x.reshape(t, x.shape[-1])
+        wcat = state.merged_weight((wq, wk, wv))
+        qkv = torch.nn.functional.linear(x2, wcat)
+        n = qkv.shape[1]
+        st = _lib.stream_ptr(x.device)
+        outs, col = [], 0
+        for heads, rotate in ((hq, 1), (hkv, 1), (hkv, 0)):
+            out = torch.empty(1, heads, t, d, device=x.device, dtype=torch.bfloat16)
+            part = qkv[:, col:]
+            _lib.call("spx_rope_relayout", _lib.ptr(part), n, _lib.ptr(position_ids), _lib.ptr(inv_freq),
+                      _lib.ptr(out), 0, t, heads, d, rotate, 0, int(offset), st)
+            outs.append(out)
+            col += heads * d
+        ctx.save_for_backward(x2, wq, wk, wv, position_ids, inv_freq)
+        ctx.meta = (x.shape, hq, hkv, d, offset, n, state, wcat)
+        ctx.set_materialize_grads(False)
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, dq, dk, dv):
+        x2, wq, wk, wv, position_ids, inv_freq = ctx.saved_tensors
+        shape, hq, hkv, d, offset, n, state, wcat = ctx.meta
+        t = x2.shape[0]
+        st = _lib.stream_ptr(x2.device)
+        dqkv = torch.empty(t, n, device=x2.device, dtype=torch.bfloat16)
+        col = 0
+        for g, heads, rotate in ((dq, hq, 1), (dk, hkv, 1), (dv, hkv, 0)):
+            part = dqkv[:, col:]
+            if g is None:
+                dqkv[:, col:col + heads * d].zero_()
+            else:
+                g = g.to(torch.bfloat16).contiguous()
+                _lib.call("spx_rope_relayout", _lib.ptr(g), 0, _lib.ptr(position_ids), _lib.ptr(inv_freq),
+                          _lib.ptr(part), n, t, heads, d, rotate, 1, int(offset), st)
+            col += heads * d
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dx = torch.matmul(dqkv, wcat).view(shape)
+        if any(w.requires_grad for w in (wq, wk, wv)):
+            state.accumulate((wq, wk, wv), dqkv, x2)
+        return (dx,) + (None,) * 10
+
+
+def qkv_rope(x, wq, wk, wv, position_ids, inv_freq, hq: int, hkv: int, d: int, offset: int,
+             state: _MergedQKV):
+    """``(q [1,Hq,T,D], k [1,Hkv,T,D], v [1,Hkv,T,D])`` with the rotary embedding at
+    ``position_ids + offset`` applied to q and k.  Weight gradients land in ``.grad`` during
+    ``backward()`` (like ``linear_accumulate``)."""
+    return _QKVRope.apply(x, wq, wk, wv, position_ids, inv_freq, hq, hkv, d, offset, state)

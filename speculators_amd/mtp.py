@@ -75,12 +75,17 @@ class MTPLayer(nn.Module):
         self.mlp = MLP(cfg)
 
     def forward(self, hidden, embeds, position_ids, inv_freq, mask):
+        # both norms write into the halves of the 2H-wide projection input; each residual add is
+        # fused into the norm that follows it
         x = gemm.linear_accumulate(
-            torch.cat([self.token_layernorm(embeds), self.hidden_layernorm(hidden)], dim=-1),
+            FO.pair_norm_cat(embeds, hidden, self.token_layernorm.weight, self.hidden_layernorm.weight,
+                             self.token_layernorm.eps),
             self.input_proj.weight)
-        x = x + self.self_attn(self.input_layernorm(x), position_ids, 0, inv_freq, {}, mask)
-        x = x + self.mlp(self.post_attention_layernorm(x))
-        return self.final_layernorm(x)
+        a = self.self_attn(self.input_layernorm(x), position_ids, 0, inv_freq, {}, mask)
+        post, final = self.post_attention_layernorm, self.final_layernorm
+        y, z = FO.add_rms_norm(x, a, post.weight, post.eps)
+        _, out = FO.add_rms_norm(y, self.mlp(z), final.weight, final.eps)
+        return out
 
 
 class MTPDraftModel(nn.Module):

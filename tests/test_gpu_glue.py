@@ -77,3 +77,106 @@ def test_swiglu_forward_backward():
     yr = torch.nn.functional.silu(ar) * br
     yr.backward(go.float())
     _close(y, yr.detach()); _close(ag.grad, ar.grad); _close(bg.grad, br.grad)
+
+
+@pytest.mark.parametrize("rows,h", [(300, 4096), (1500, 2048), (40, 256), (33, 8192)])
+def test_add_rms_norm_matches_the_two_ops(rows, h):
+    """``(a + b, rms_norm(a + b))`` fused, against the bf16 add followed by the norm."""
+    from speculators_amd.fused_ops import add_rms_norm
+
+    g = torch.Generator().manual_seed(rows + h)
+    a = (torch.randn(1, rows, h, generator=g) * 2).bfloat16()
+    b = (torch.randn(1, rows, h, generator=g) * 2).bfloat16()
+    w = (1 + 0.2 * torch.randn(h, generator=g)).bfloat16()
+    gs = torch.randn(1, rows, h, generator=g).bfloat16()
+    gy = torch.randn(1, rows, h, generator=g).bfloat16()
+    ag, bg, wg = (t.cuda().requires_grad_(True) for t in (a, b, w))
+    s, y = add_rms_norm(ag, bg, wg, 1e-5)
+    torch.autograd.backward((s, y), (gs.cuda(), gy.cuda()))
+    assert torch.equal(s.cpu(), a + b)  # one bf16 rounding, like the tensor add
+    ref_bf16 = OE.rms_norm(a + b, w, 1e-5)
+    assert (y.cpu() != ref_bf16).float().mean().item() < 2e-3
+    ar, br, wr = (t.float().requires_grad_(True) for t in (a, b, w))
+    sr = (ar + br).bfloat16().float()  # the norm sees the rounded sum
+    sr = ar + br + (sr - (ar + br)).detach()
+    yr = OE.rms_norm(sr, wr, 1e-5)
+    torch.autograd.backward((sr, yr), (gs.float(), gy.float()))
+    _close(y, yr.detach()); _close(ag.grad, ar.grad); _close(bg.grad, br.grad); _close(wg.grad, wr.grad)
+    assert torch.equal(ag.grad, bg.grad)
+    # only one of the two outputs used
+    ag.grad = bg.grad = wg.grad = None
+    s, y = add_rms_norm(ag, bg, wg, 1e-5)
+    s.backward(gs.cuda())
+    assert torch.equal(ag.grad.cpu(), gs) and wg.grad is None
+    ag.grad = bg.grad = None
+    s, y = add_rms_norm(ag, bg, wg, 1e-5)
+    y.backward(gy.cuda())
+    ar.grad = br.grad = wr.grad = None
+    OE.rms_norm(ar + br, wr, 1e-5).backward(gy.float())
+    _close(ag.grad, ar.grad); _close(wg.grad, wr.grad)
+
+
+@pytest.mark.parametrize("rows,h,embeds_grad", [(300, 4096, False), (129, 512, True), (64, 2048, False)])
+def test_pair_norm_cat_matches_cat_of_norms(rows, h, embeds_grad):
+    from speculators_amd.fused_ops import pair_norm_cat, rms_norm
+
+    g = torch.Generator().manual_seed(rows + h)
+    a = (torch.randn(1, rows, h, generator=g) * 2).bfloat16().cuda().requires_grad_(embeds_grad)
+    b = (torch.randn(1, rows, h, generator=g) * 3).bfloat16().cuda().requires_grad_(True)
+    wa = (1 + 0.2 * torch.randn(h, generator=g)).bfloat16().cuda().requires_grad_(True)
+    wb = (1 + 0.2 * torch.randn(h, generator=g)).bfloat16().cuda().requires_grad_(True)
+    go = torch.randn(1, rows, 2 * h, generator=g).bfloat16().cuda()
+    out = pair_norm_cat(a, b, wa, wb, 1e-5)
+    out.backward(go)
+    got = [t.grad for t in (a, b, wa, wb)]
+    for t in (a, b, wa, wb):
+        t.grad = None
+    ref = torch.cat([rms_norm(a, wa, 1e-5), rms_norm(b, wb, 1e-5)], dim=-1)
+    ref.backward(go)
+    assert torch.equal(out, ref)  # the same kernel, written in place
+    for gt, t in zip(got, (a, b, wa, wb), strict=True):
+        if t.grad is None:
+            assert gt is None
+        else:
+            assert torch.equal(gt, t.grad)
+
+
+@pytest.mark.parametrize("t,h_in,hq,hkv,d", [(300, 1024, 8, 2, 128), (129, 512, 4, 4, 64)])
+def test_qkv_rope_matches_separate_projections(t, h_in, hq, hkv, d):
+    """One merged q/k/v GEMM + fused relayouts == three projections + three relayouts, and the
+    weight gradients accumulate over calls like ``linear_accumulate``."""
+    from speculators_amd import gemm
+    from speculators_amd.fused_ops import rope_inv_freq, rope_relayout
+
+    g = torch.Generator().manual_seed(t)
+    x = torch.randn(1, t, h_in, generator=g).bfloat16().cuda().requires_grad_(True)
+    ws = [(torch.randn(n, h_in, generator=g) * 0.05).bfloat16().cuda().requires_grad_(True)
+          for n in (hq * d, hkv * d, hkv * d)]
+    pos = torch.randint(0, 4000, (t,), generator=g).cuda()
+    inv = rope_inv_freq(d, 500000.0, "cuda")
+    gos = [torch.randn(1, n, t, d, generator=g).bfloat16().cuda() for n in (hq, hkv, hkv)]
+    state = gemm._MergedQKV()
+    for rep in range(2):  # the second call accumulates into the same merged gradient buffer
+        outs = gemm.qkv_rope(x, *ws, pos, inv, hq, hkv, d, 3, state)
+        torch.autograd.backward(outs, gos)
+    got_x = x.grad.clone()
+    got_w = [w.grad.clone() for w in ws]
+    assert ws[0].grad.data_ptr() == state.grad.data_ptr()
+    x.grad = None
+    for w in ws:
+        w.grad = None
+    ref = []
+    for w, heads, rot in zip(ws, (hq, hkv, hkv), (True, True, False), strict=True):
+        ref.append(rope_relayout(torch.nn.functional.linear(x, w), pos, inv, heads, rot, 3 if rot else 0))
+    for o, r in zip(outs, ref, strict=True):
+        _close(o, r.detach().cpu(), rel=1e-2)
+    torch.autograd.backward(ref, gos)
+    _close(got_x, 2 * x.grad.cpu())
+    for gw, w in zip(got_w, ws, strict=True):
+        _close(gw, 2 * w.grad.cpu())
+    # gradients that did not come from the merged buffer are added to, not replaced
+    for w in ws:
+        w.grad = torch.ones_like(w)
+    torch.autograd.backward(gemm.qkv_rope(x, *ws, pos, inv, hq, hkv, d, 3, state), gos)
+    for gw, w in zip(got_w, ws, strict=True):
+        _close(w.grad - 1, 0.5 * gw.cpu())
