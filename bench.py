@@ -42,7 +42,10 @@ MEASURED_TRAFFIC = {
 
 CONFIG1 = dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
                intermediate_size=14336, vocab_size=128256, draft_vocab_size=32000,
-               rope_theta=500000.0, rms_norm_eps=1e-5)
+               rope_theta=500000.0, rms_norm_eps=1e-5,
+               # the rotary frequency scaling Llama-3.1 ships with (the draft layer inherits it)
+               rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                             "high_freq_factor": 4.0, "original_max_position_embeddings": 8192})
 SEQ_LEN, TTT_STEPS = 4096, 7
 
 

@@ -112,7 +112,7 @@ def dflash_forward(w, shape: DraftShape, hidden_states, input_ids, loss_mask,
                    shape.rms_norm_eps)
     block_pos = base_indices_for_anchored_blocks(position_ids[0, anchor_pos], block_size)
     all_pos = torch.cat([position_ids, block_pos.unsqueeze(0)], dim=1)
-    cos, sin = rope_tables(all_pos, shape.head_dim, shape.rope_theta, dtype)
+    cos, sin = rope_tables(all_pos, shape.head_dim, shape.rope_theta, dtype, shape.rope_scaling)
     block_idx = base_indices_for_anchored_blocks(anchor_pos, block_size)
     with torch.no_grad():
         targets = dflash_targets(w, shape, verifier_last_hidden_states, block_idx,

@@ -21,6 +21,8 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+import math
+
 import torch
 import torch.nn.functional as F
 
@@ -49,6 +51,7 @@ class DraftShape:
     qk_norm: bool = False  # Qwen3-style per-head RMSNorm of q and k
     sliding_window: int | None = None
     sliding_layers: tuple = field(default_factory=tuple)  # indices of windowed layers
+    rope_scaling: dict | None = None  # HF rope parameters: {"rope_type": "llama3" | "linear", ...}
 
 
 def rms_norm(x, weight, eps):
@@ -58,9 +61,37 @@ def rms_norm(x, weight, eps):
     return weight * xf.to(x.dtype)
 
 
-def rope_tables(position_ids, head_dim, theta, dtype):
+def rope_inv_freq(head_dim, theta, scaling=None):
+    """fp32 inverse frequencies of the rotary embedding.  ``scaling`` follows the HF rope
+    parameters the draft inherits from its verifier (models/eagle3/core.py:105-112 keeps them
+    in the layer config; Llama-3.1 ships ``rope_type = "llama3"``):
+      linear: every frequency divided by ``factor``;
+      llama3: wavelengths above ``L / low_freq_factor`` (L = original_max_position_embeddings)
+              are divided by ``factor``, those below ``L / high_freq_factor`` kept, and the band
+              between is blended linearly in ``L / wavelength``.
+    Pinned against ``transformers.modeling_rope_utils.ROPE_INIT_FUNCTIONS``."""
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
+    kind = (scaling or {}).get("rope_type", (scaling or {}).get("type", "default"))
+    if kind == "default":
+        return inv
+    factor = float(scaling["factor"])
+    if kind == "linear":
+        return inv / factor
+    if kind != "llama3":
+        raise NotImplementedError(f"rope_type '{kind}'")
+    lo, hi = float(scaling["low_freq_factor"]), float(scaling["high_freq_factor"])
+    ctx = float(scaling["original_max_position_embeddings"])
+    wavelen = 2 * math.pi / inv
+    out = torch.where(wavelen > ctx / lo, inv / factor, inv)
+    blend = (ctx / wavelen - lo) / (hi - lo)
+    mid = (1 - blend) * out / factor + blend * out
+    band = ~(wavelen < ctx / hi) & ~(wavelen > ctx / lo)
+    return torch.where(band, mid, out)
+
+
+def rope_tables(position_ids, head_dim, theta, dtype, scaling=None):
     """cos/sin ``[1, T, D]``: fp32 outer product, duplicated halves, cast."""
-    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    inv = rope_inv_freq(head_dim, theta, scaling)
     ang = position_ids.reshape(1, -1, 1).float() * inv.reshape(1, 1, -1)
     ang = torch.cat([ang, ang], dim=-1)
     return ang.cos().to(dtype), ang.sin().to(dtype)
@@ -177,7 +208,7 @@ def eagle3_forward(w, shape: DraftShape, hidden_states, input_ids, document_ids,
     for step in range(ttt_steps):
         with torch.no_grad():
             embeds = F.embedding(input_ids, w["embed_tokens.weight"])
-        cos, sin = rope_tables(position_ids, shape.head_dim, shape.rope_theta, dtype)
+        cos, sin = rope_tables(position_ids, shape.head_dim, shape.rope_theta, dtype, shape.rope_scaling)
         y = first_layer(torch.cat([embeds, hidden], -1), w, shape, cos, sin,
                         caches[0], mask_for(0, step), attn)
         for li in range(1, shape.num_hidden_layers):

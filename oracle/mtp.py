@@ -118,7 +118,8 @@ def mtp_forward(w, shape: DraftShape, input_ids, hidden_states, position_ids=Non
         emb = F.embedding(input_ids[:, step + 1:step + 1 + valid], w["embed_tokens.weight"])
         rows = []
         for r in range(b):
-            cos, sin = rope_tables(pos[r], shape.head_dim, shape.rope_theta, hid.dtype)
+            cos, sin = rope_tables(pos[r], shape.head_dim, shape.rope_theta, hid.dtype,
+                                       shape.rope_scaling)
             rows.append(mtp_layer(hid[r:r + 1], emb[r:r + 1].to(hid.dtype), w, shape, cos, sin,
                                   masks[r], attn))
         out = torch.cat(rows, dim=0)

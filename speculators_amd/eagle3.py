@@ -46,6 +46,7 @@ class Eagle3Config:
     num_hidden_layers: int = 1
     rms_norm_eps: float = 1e-5
     rope_theta: float = 500000.0
+    rope_scaling: dict | None = None  # HF rope parameters (rope_type default / linear / llama3)
     norm_before_residual: bool = False
     norm_before_fc: bool = False
     fc_norm: bool = False
@@ -293,7 +294,7 @@ class Eagle3DraftModel(nn.Module):
 
         caches = [dict() for _ in self.layers]
         stats_cache: dict = {}
-        inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device)
+        inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device, cfg.rope_scaling)
         position_ids = position_ids.reshape(-1).to(torch.int64).contiguous()
         draft_tokens = []
         for step in range(ttt_steps):

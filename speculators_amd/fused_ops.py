@@ -3,6 +3,8 @@ fused with the head-major relayout, SwiGLU.  bf16 HIP tensors only."""
 
 from __future__ import annotations
 
+import math
+
 import torch
 
 from . import _lib
@@ -211,9 +213,31 @@ def rope_relayout(x, position_ids, inv_freq, heads: int, rotate: bool = True, of
     return _RopeRelayout.apply(x, pos.contiguous(), inv_freq, heads, rotate, offset)
 
 
-def rope_inv_freq(head_dim: int, theta: float, device) -> torch.Tensor:
-    """fp32 inverse frequencies, evaluated like the HF default rotary initialisation."""
-    return (1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))).to(device)
+def rope_inv_freq(head_dim: int, theta: float, device, scaling: dict | None = None) -> torch.Tensor:
+    """fp32 inverse frequencies, evaluated like the HF rotary initialisation the draft layer
+    inherits from its verifier config: ``scaling`` is the HF rope-parameter dict
+    (``rope_type`` "default", "linear" or "llama3"; Llama-3.1 verifiers use "llama3")."""
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    kind = "default"
+    if scaling:
+        kind = scaling.get("rope_type", scaling.get("type", "default"))
+    if kind == "linear":
+        inv = inv / float(scaling["factor"])
+    elif kind == "llama3":
+        factor = float(scaling["factor"])
+        low, high = float(scaling["low_freq_factor"]), float(scaling["high_freq_factor"])
+        old_len = float(scaling["original_max_position_embeddings"])
+        wavelen = 2 * math.pi / inv
+        # long wavelengths are stretched by `factor`, short ones kept, the band between blended
+        scaled = torch.where(wavelen > old_len / low, inv / factor, inv)
+        smooth = (old_len / wavelen - low) / (high - low)
+        blended = (1 - smooth) * scaled / factor + smooth * scaled
+        medium = (wavelen >= old_len / high) & (wavelen <= old_len / low)
+        inv = torch.where(medium, blended, scaled)
+    elif kind != "default":
+        raise NotImplementedError(
+            f"rope_type '{kind}' is not built on the HIP path (default, linear and llama3 are)")
+    return inv.to(device)
 
 
 class _SwiGLU(torch.autograd.Function):

@@ -54,6 +54,7 @@ class MTPConfig:
     num_speculative_steps: int = 3
     rms_norm_eps: float = 1e-6
     rope_theta: float = 1000000.0
+    rope_scaling: dict | None = None  # HF rope parameters (rope_type default / linear / llama3)
     model_type: str = "qwen3"
     attn_implementation: str = A.ATTN_IMPL_TTT
     qk_norm: bool = True  # Qwen3 attention
@@ -155,7 +156,7 @@ class MTPDraftModel(nn.Module):
         seq = (diff != 1).cumsum(-1) + torch.arange(b, device=device).unsqueeze(1) * (valid + 1)
         mask = A.create_ttt_mask(seq.reshape(-1), b * valid, None)
         flat_pos = pos.reshape(-1).contiguous()
-        inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device)
+        inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device, cfg.rope_scaling)
         layer = self.mtp_layers[0]
 
         current = hidden_states

@@ -41,7 +41,7 @@ def _make(shape, w):
         "hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim", "intermediate_size",
         "vocab_size", "draft_vocab_size", "num_aux", "num_hidden_layers", "rms_norm_eps", "rope_theta",
         "norm_before_residual", "norm_before_fc", "fc_norm", "norm_output", "qk_norm",
-        "sliding_window", "sliding_layers")})
+        "sliding_window", "sliding_layers", "rope_scaling")})
     model = Eagle3DraftModel(cfg)
     missing, unexpected = model.load_state_dict(w, strict=False)
     assert not unexpected and set(missing) <= {"t2d", "d2t"}, (missing, unexpected)
@@ -52,6 +52,10 @@ VARIANTS = [
     dict(),
     dict(norm_before_residual=True, norm_output=True, norm_before_fc=True),
     dict(num_hidden_layers=2, sliding_window=48, sliding_layers=(0,), qk_norm=True),
+    # Llama-3.1 style frequency scaling, with a short original context so that it matters here
+    dict(num_hidden_layers=2, rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                                            "high_freq_factor": 4.0,
+                                            "original_max_position_embeddings": 64}),
 ]
 
 

@@ -155,3 +155,49 @@ def test_teacher_forcing_shift():
     toks2, loss2, _ = E.eagle3_forward(w, shape, hs, ids2, doc, mask, pos, vl, ttt_steps=2)
     # token 0 is only ever used as the step-0 input of row 0
     assert not torch.equal(toks[0], toks2[0]) or loss.item() != loss2.item()
+
+
+# ---------------------------------------------------------------- rope frequency scaling
+_LLAMA31 = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+            "original_max_position_embeddings": 8192}
+
+
+@pytest.mark.parametrize("scaling", [None, {"rope_type": "linear", "factor": 4.0}, _LLAMA31,
+                                     dict(_LLAMA31, factor=32.0, original_max_position_embeddings=64)])
+@pytest.mark.parametrize("head_dim,theta", [(128, 500000.0), (64, 10000.0)])
+def test_rope_inv_freq_matches_transformers(scaling, head_dim, theta):
+    """The oracle's inverse frequencies == the HF rotary initialisation (library routine), and
+    the product's host-side evaluation == the oracle's, bit for bit."""
+    from transformers import LlamaConfig
+    from transformers.modeling_rope_utils import ROPE_INIT_FUNCTIONS
+
+    from speculators_amd.fused_ops import rope_inv_freq
+
+    got = E.rope_inv_freq(head_dim, theta, scaling)
+    params = {"rope_type": "default", "rope_theta": theta}
+    params.update(scaling or {})
+    cfg = LlamaConfig(hidden_size=head_dim * 4, num_attention_heads=4, head_dim=head_dim,
+                      rope_parameters=params, max_position_embeddings=131072)
+    kind = params["rope_type"]
+    if kind == "default":
+        from transformers.models.llama.modeling_llama import LlamaRotaryEmbedding
+
+        want = LlamaRotaryEmbedding(cfg).inv_freq
+        factor = 1.0
+    else:
+        want, factor = ROPE_INIT_FUNCTIONS[kind](cfg, "cpu")
+    assert factor == 1.0
+    assert torch.equal(got, want)
+    assert torch.equal(rope_inv_freq(head_dim, theta, "cpu", scaling), got)
+    if kind == "llama3":  # the scaling does something: low frequencies shrink by `factor`
+        base = E.rope_inv_freq(head_dim, theta, None)
+        assert torch.equal(got[0], base[0]) and torch.isclose(got[-1], base[-1] / scaling["factor"])
+
+
+def test_rope_scaling_rejects_unknown_types():
+    from speculators_amd.fused_ops import rope_inv_freq
+
+    with pytest.raises(NotImplementedError):
+        rope_inv_freq(64, 10000.0, "cpu", {"rope_type": "yarn", "factor": 2.0})
+    with pytest.raises(NotImplementedError):
+        E.rope_inv_freq(64, 10000.0, {"rope_type": "yarn", "factor": 2.0})
