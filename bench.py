@@ -47,13 +47,17 @@ CONFIG1 = dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, 
                rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
                              "high_freq_factor": 4.0, "original_max_position_embeddings": 8192})
 SEQ_LEN, TTT_STEPS = 4096, 7
+# configs[3]: the Llama-3.1-70B shape (seq 8192, TTT 5), same code path as configs[1]
+CONFIG3 = dict(CONFIG1, hidden_size=8192, num_attention_heads=64, intermediate_size=28672)
+SEQ_LEN3, TTT_STEPS3 = 8192, 5
 
 
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", choices=["eagle3", "mtp"], default="eagle3",
-                    help="eagle3 = configs[1], the headline; mtp = configs[4] (MTP head, full-vocab CE)")
+    ap.add_argument("--workload", choices=["eagle3", "eagle3-70b", "mtp", "dflash"], default="eagle3",
+                    help="eagle3 = configs[1], the headline; eagle3-70b = configs[3]; mtp = configs[4] (MTP "
+                         "head, full-vocab CE); dflash = configs[2] (anchored blocks, 5 layers)")
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
@@ -449,6 +453,116 @@ def run_mtp(args):
         "kernels": kernels, "cpu_baseline": cpu}))
 
 
+# configs[2]: DFlash on a Qwen3-8B shaped verifier.  5 draft layers (the reference default for
+# dflash), every layer windowed; 512 anchors on a uniform non-overlapping grid.
+CONFIG2 = dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+               intermediate_size=12288, vocab_size=151936, draft_vocab_size=32000, num_aux=5,
+               num_hidden_layers=5, rms_norm_eps=1e-6, rope_theta=1000000.0, block_size=16,
+               mask_token_id=151935, sliding_window=2048, sliding_layers=(0, 1, 2, 3, 4))
+DFLASH_SEQ_LEN, DFLASH_ANCHORS = 8192, 512
+
+
+def run_dflash(args):
+    """configs[2]: DFlash forward + backward, tokens/s over the T context positions, and the
+    roofline of the anchored-block attention."""
+    import torch
+
+    from speculators_amd import _lib
+    from speculators_amd import attention as A
+    from speculators_amd.dflash import DFlashConfig, DFlashDraftModel
+    from speculators_amd.losses import resolve_loss_config
+
+    _lib.load()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    t = args.seq_len if args.seq_len != SEQ_LEN else DFLASH_SEQ_LEN
+    cfg = DFlashConfig(**CONFIG2)
+    bs, n_anchor = cfg.block_size, DFLASH_ANCHORS
+    torch.manual_seed(0)
+    model = DFlashDraftModel(cfg)
+    with torch.no_grad():
+        for name, p_ in model.named_parameters():
+            if name.endswith("norm.weight") or "layernorm" in name:
+                p_.fill_(1.0)
+            else:
+                p_.normal_(0.0, 0.02)
+    g = torch.Generator().manual_seed(0)
+    sel = torch.randperm(cfg.vocab_size, generator=g)[:cfg.draft_vocab_size].sort().values
+    t2d = torch.zeros(cfg.vocab_size, dtype=torch.bool)
+    t2d[sel] = True
+    model.t2d.copy_(t2d)
+    model.d2t.copy_(sel - torch.arange(cfg.draft_vocab_size))
+    model = model.to(torch.bfloat16).to(device)
+    hs = (torch.randn(1, t, cfg.num_aux * cfg.hidden_size, generator=g) * 4).bfloat16().to(device)
+    vl = torch.randn(1, t, cfg.hidden_size, generator=g).bfloat16().to(device)
+    ids = torch.randint(0, cfg.vocab_size, (1, t), generator=g).to(device)
+    lm = (torch.rand(1, t, generator=g) < 0.7).float().to(device)
+    doc = torch.zeros(1, t, dtype=torch.long, device=device)
+    stride = (t - bs) // n_anchor
+    anchor_pos = (torch.arange(n_anchor) * stride + 1).to(device)
+    anchors = (anchor_pos, torch.ones(n_anchor, dtype=torch.bool, device=device))
+    loss_config = resolve_loss_config("kl_div", "hip")
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        _, loss, _ = model(hs, ids, lm, vl, doc, loss_config=loss_config, anchors=anchors)
+        loss.backward()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    final_loss = float(loss.detach())
+    del loss
+    model.zero_grad(set_to_none=True)
+
+    kernels = []
+    hq, hkv, d, w = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.sliding_window
+    n_q = n_anchor * bs
+    # live (query, key) pairs: the context window in front of the anchor + the causal part of the block
+    pairs = float((torch.clamp(anchor_pos.cpu(), max=w) * bs).sum() + n_anchor * bs * (bs + 1) // 2)
+    mask = A.create_dflash_mask(doc.reshape(-1), t, anchor_pos, bs, w, False)
+    gq = torch.Generator(device=device).manual_seed(1)
+    q = torch.randn(1, hq, n_q, d, device=device, generator=gq).bfloat16().requires_grad_(True)
+    kk = torch.randn(1, hkv, t + n_q, d, device=device, generator=gq).bfloat16().requires_grad_(True)
+    vv = torch.randn(1, hkv, t + n_q, d, device=device, generator=gq).bfloat16().requires_grad_(True)
+
+    def rec(name, flops, ms, launches):
+        tf = flops / (ms * 1e-3) / 1e12
+        kernels.append({"kernel": name, "bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS,
+                        "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                        "algorithmic_flops": flops, "ms_per_launch": round(ms, 4),
+                        "launches_per_step": launches})
+
+    ms_f = time_events(torch, lambda: A.dflash_attention(q.detach(), kk.detach(), vv.detach(), mask), 10)
+    rec(f"attn_fwd_kernel[DFlash, {n_anchor} anchors x block {bs}, window {w}]", 4.0 * pairs * d * hq, ms_f,
+        cfg.num_hidden_layers)
+    o = A.dflash_attention(q, kk, vv, mask)
+    go = torch.randn_like(o)
+    ms_b = time_events(torch, lambda: torch.autograd.grad(o, (q, kk, vv), go, retain_graph=True), 10)
+    rec(f"attn_bwd[DFlash, {n_anchor} anchors x block {bs}, window {w}]", 10.0 * pairs * d * hq, ms_b,
+        cfg.num_hidden_layers)
+    dominant = max(kernels, key=lambda r: r["ms_per_launch"] * r["launches_per_step"])
+    print(json.dumps({
+        "metric": "draft train tokens/sec (fwd+bwd) @Qwen3-8B DFlash", "value": round(t / (ms_per_step * 1e-3), 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"configs[2]: DFlash draft, Qwen3-8B shape, {cfg.num_hidden_layers} layers, seq {t}, "
+                               f"{n_anchor} anchors x block {bs} (queries {n_q}, keys {t + n_q}), window {w} on "
+                               "every layer, 5 auxiliary layers, vocab 151936 -> draft 32000, kl_div loss",
+                   "seq_len": t, "anchors": n_anchor, "block_size": bs, "tokens_per_step": t,
+                   "final_loss": round(final_loss, 6)},
+        "roofline": {k_: dominant[k_] for k_ in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
+                    | {"kernel": dominant["kernel"]},
+        "kernels": kernels, "cpu_baseline": None}))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -457,6 +571,9 @@ def main():
         sys.exit(2)
     if args.workload == "mtp":
         run_mtp(args)
+        return
+    if args.workload == "dflash":
+        run_dflash(args)
         return
     import torch
 
@@ -469,6 +586,11 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     t, k_steps = args.seq_len, args.ttt_steps
+    big = args.workload == "eagle3-70b"
+    CONFIG1 = CONFIG3 if big else globals()["CONFIG1"]  # noqa: N806 - the config of this run
+    if big:
+        t = SEQ_LEN3 if t == SEQ_LEN else t
+        k_steps = TTT_STEPS3 if k_steps == TTT_STEPS else k_steps
     if args.only_kernels:
         print(json.dumps({"kernels": kernel_rooflines(torch, CONFIG1, t, k_steps, device)}))
         return
@@ -507,11 +629,14 @@ def main():
         cpu = cpu_baseline(CONFIG1, args.cpu_seq_len, k_steps)
 
     line = {
-        "metric": "draft train tokens/sec (fwd+bwd) @Llama-3.1-8B EAGLE3 TTT7",
+        "metric": ("draft train tokens/sec (fwd+bwd) @Llama-3.1-70B EAGLE3 TTT5" if big else
+                   "draft train tokens/sec (fwd+bwd) @Llama-3.1-8B EAGLE3 TTT7"),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "configs[1]: EAGLE3 draft, Llama-3.1-8B shape, one draft layer, "
+        "config": {"workload": ("configs[3]: EAGLE3 draft, Llama-3.1-70B shape, one draft layer, " if big else
+                                "configs[1]: EAGLE3 draft, Llama-3.1-8B shape, one draft layer, ")
+                               +
                                f"batch 1, seq {t}, TTT {k_steps}, vocab 128256 -> draft 32000, "
                                "kl_div loss, bf16 weights and activations, full attention, "
                                f"targets from {'verifier hidden states through the frozen verifier head' if args.targets == 'hidden' else 'full-vocab verifier logits gathered through d2t'}",

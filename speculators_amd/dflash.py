@@ -125,8 +125,10 @@ class DFlashDecoderLayer(nn.Module):
         self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
 
     def forward(self, x, ctx, q_pos, kv_pos, inv_freq, mask):
-        y = x + self.self_attn(self.input_layernorm(x), ctx, q_pos, kv_pos, inv_freq, mask)
-        return y + self.mlp(self.post_attention_layernorm(y))
+        a = self.self_attn(self.input_layernorm(x), ctx, q_pos, kv_pos, inv_freq, mask)
+        post = self.post_attention_layernorm
+        y, z = FO.add_rms_norm(x, a, post.weight, post.eps)  # residual add fused into the norm
+        return y + self.mlp(z)
 
 
 class DFlashDraftModel(nn.Module):
