@@ -762,6 +762,12 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
 // PASS 0 computes dK and dV together; PASS 1 only dV, PASS 2 only dK (head_dim 256: the two
 // accumulator sets and both operand fragments do not fit the register file together, so
 // the kernel is launched once per pass and the scores are recomputed).
+#ifndef SPX_DKV256_PF1
+#define SPX_DKV256_PF1 true
+#endif
+#ifndef SPX_DKV256_PF2
+#define SPX_DKV256_PF2 true
+#endif
 template <int D, int NW, bool PF, int PASS>
 __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     AttnParams p, const uint16_t* __restrict__ dO, const uint16_t* __restrict__ Qt,
@@ -849,10 +855,10 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       const int qr = ch / (D / 8), qc = (ch % (D / 8)) * 8;
       const int ir = min(mq + qr, p.NQ - 1);
       qreg[n] = *reinterpret_cast<const u32x4*>(Qh + (int64_t)ir * D + qc);
-      dreg[n] = *reinterpret_cast<const u32x4*>(dO + ((int64_t)ir * p.Hq + h) * D + qc);
+      if (kDoK) dreg[n] = *reinterpret_cast<const u32x4*>(dO + ((int64_t)ir * p.Hq + h) * D + qc);
       const int td = ch >> 3, tc = (ch & 7) * 8;
-      qtreg[n] = *reinterpret_cast<const u32x4*>(Qth + (int64_t)td * NQp + mq + tc);
-      dtreg[n] = *reinterpret_cast<const u32x4*>(dOth + (int64_t)td * NQp + mq + tc);
+      if (kDoK) qtreg[n] = *reinterpret_cast<const u32x4*>(Qth + (int64_t)td * NQp + mq + tc);
+      if (kDoV) dtreg[n] = *reinterpret_cast<const u32x4*>(dOth + (int64_t)td * NQp + mq + tc);
     }
     if (tid < 64) {
       const int ir = mq + tid;
@@ -871,10 +877,10 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       const int ch = tid + NT * n;
       const int qr = ch / (D / 8), qc = (ch % (D / 8)) * 8;
       *reinterpret_cast<u32x4*>(&Qs[qr * QS + qc]) = qreg[n];
-      *reinterpret_cast<u32x4*>(&dOs[qr * QS + qc]) = dreg[n];
+      if (kDoK) *reinterpret_cast<u32x4*>(&dOs[qr * QS + qc]) = dreg[n];
       const int td = ch >> 3, tc = (ch & 7) * 8;
-      *reinterpret_cast<u32x4*>(&Qts[td * TS + tc]) = qtreg[n];
-      *reinterpret_cast<u32x4*>(&dOts[td * TS + tc]) = dtreg[n];
+      if (kDoK) *reinterpret_cast<u32x4*>(&Qts[td * TS + tc]) = qtreg[n];
+      if (kDoV) *reinterpret_cast<u32x4*>(&dOts[td * TS + tc]) = dtreg[n];
     }
     if (tid < 64) {
       lse_s[tid] = lse_r; delta_s[tid] = delta_r;
@@ -888,15 +894,20 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       const int ch = tid + NT * n;
       const int qr = ch / (D / 8), qc = (ch % (D / 8)) * 8;
       const int ir = min(mq + qr, p.NQ - 1);
+      // only the tiles this pass multiplies with: Q always (scores), dO and Q^T for dK,
+      // dO^T for dV
       *reinterpret_cast<u32x4*>(&Qs[qr * QS + qc]) =
           *reinterpret_cast<const u32x4*>(Qh + (int64_t)ir * D + qc);
-      *reinterpret_cast<u32x4*>(&dOs[qr * QS + qc]) =
-          *reinterpret_cast<const u32x4*>(dO + ((int64_t)ir * p.Hq + h) * D + qc);
+      if (kDoK)
+        *reinterpret_cast<u32x4*>(&dOs[qr * QS + qc]) =
+            *reinterpret_cast<const u32x4*>(dO + ((int64_t)ir * p.Hq + h) * D + qc);
       const int td = ch >> 3, tc = (ch & 7) * 8;
-      const u32x4 a = *reinterpret_cast<const u32x4*>(Qth + (int64_t)td * NQp + mq + tc);
-      const u32x4 b = *reinterpret_cast<const u32x4*>(dOth + (int64_t)td * NQp + mq + tc);
-      *reinterpret_cast<u32x4*>(&Qts[td * TS + tc]) = a;
-      *reinterpret_cast<u32x4*>(&dOts[td * TS + tc]) = b;
+      if (kDoK)
+        *reinterpret_cast<u32x4*>(&Qts[td * TS + tc]) =
+            *reinterpret_cast<const u32x4*>(Qth + (int64_t)td * NQp + mq + tc);
+      if (kDoV)
+        *reinterpret_cast<u32x4*>(&dOts[td * TS + tc]) =
+            *reinterpret_cast<const u32x4*>(dOth + (int64_t)td * NQp + mq + tc);
     }
     if (tid < 64) {
       const int ir = mq + tid;
@@ -1129,6 +1140,14 @@ static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 #ifndef SPX_DQ_CFG
 #define SPX_DQ_CFG 1, 4, false
 #endif
+// head_dim 256: the next tile is prefetched into registers as well; the few registers that
+// spill cost far less than exposing the global-load latency with one workgroup per CU
+#ifndef SPX_FWD256_PF
+#define SPX_FWD256_PF true
+#endif
+#ifndef SPX_DQ256_PF
+#define SPX_DQ256_PF true
+#endif
 #ifndef SPX_DKV_CFG
 #define SPX_DKV_CFG 4, true
 #endif
@@ -1163,8 +1182,8 @@ static int launch_fwd(AttnParams p, void* workspace, uint16_t* O, float* lse, hi
                      vt, (int64_t)D * p.NKVp, (int64_t)p.NKVp);
   constexpr int BM = 32 * kFwdNSB * kFwdNW;
   const int n_qb = (p.NQ + BM - 1) / BM;
-  if constexpr (D > 128)  // no register prefetch: the tile would not fit beside the accumulators
-    hipLaunchKernelGGL((attn_fwd_kernel<D, kFwdNSB, kFwdNW, false>), dim3((unsigned)(n_qb * p.Hq)),
+  if constexpr (D > 128)
+    hipLaunchKernelGGL((attn_fwd_kernel<D, kFwdNSB, kFwdNW, SPX_FWD256_PF>), dim3((unsigned)(n_qb * p.Hq)),
                        dim3(64 * kFwdNW), 0, st, p, vt, O, lse);
   else
     hipLaunchKernelGGL((attn_fwd_kernel<D, SPX_FWD_CFG>), dim3((unsigned)(n_qb * p.Hq)),
@@ -1204,8 +1223,12 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
 
   constexpr int BM = 32 * kDqNSB * kDqNW;
   const int n_qb = (p.NQ + BM - 1) / BM;
-  hipLaunchKernelGGL((attn_bwd_dq_kernel<D, SPX_DQ_CFG>), dim3((unsigned)(n_qb * p.Hq)),
-                     dim3(64 * kDqNW), 0, st, p, dOp, kt, lse, delta, dQp, dq_hs);
+  if constexpr (D > 128)
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<D, kDqNSB, kDqNW, SPX_DQ256_PF>), dim3((unsigned)(n_qb * p.Hq)),
+                       dim3(64 * kDqNW), 0, st, p, dOp, kt, lse, delta, dQp, dq_hs);
+  else
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<D, SPX_DQ_CFG>), dim3((unsigned)(n_qb * p.Hq)),
+                       dim3(64 * kDqNW), 0, st, p, dOp, kt, lse, delta, dQp, dq_hs);
 
   const size_t smem = (size_t)(2 * 64 * (D + kKPad) + 2 * D * (64 + kVPad)) * 2 + 64 * 4 * 6;
   const int n_kb = (p.NKV + 32 * kDkvNW - 1) / (32 * kDkvNW);
@@ -1217,17 +1240,17 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   };
   static bool attr_set = false;
   if constexpr (D > 128) {
-    // one launch per gradient, no register prefetch
+    // one launch per gradient (each loads only the tiles it multiplies with)
     if (!attr_set) {
-      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, false, 1>)) ||
-          !set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, false, 2>)))
+      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, SPX_DKV256_PF1, 1>)) ||
+          !set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, SPX_DKV256_PF2, 2>)))
         return SPX_ERR_HIP;
       attr_set = true;
     }
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, false, 1>), kgrid, kblock, smem, st, p, dOp, qt, dot,
-                       NQp, lse, delta, tb, dkp, dvp);
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, false, 2>), kgrid, kblock, smem, st, p, dOp, qt, dot,
-                       NQp, lse, delta, tb, dkp, dvp);
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, SPX_DKV256_PF1, 1>), kgrid, kblock, smem, st, p, dOp, qt,
+                       dot, NQp, lse, delta, tb, dkp, dvp);
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, SPX_DKV256_PF2, 2>), kgrid, kblock, smem, st, p, dOp, qt,
+                       dot, NQp, lse, delta, tb, dkp, dvp);
   } else {
     if (!attr_set) {
       if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, SPX_DKV_CFG, 0>))) return SPX_ERR_HIP;
