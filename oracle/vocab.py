@@ -38,3 +38,19 @@ def gather_targets(full_logits: torch.Tensor, d2t: torch.Tensor) -> torch.Tensor
     (model.py:161-169)."""
     idx = torch.arange(d2t.numel(), dtype=torch.long) + d2t.long()
     return full_logits.index_select(-1, idx)
+
+
+def build_vocab_mappings_from_distribution(token_freq: dict, draft_vocab_size: int, target_vocab_size: int):
+    """train/vocab_mapping.py:64-96 in full: rank ids by (count descending, id ascending), keep
+    the first ``draft_vocab_size``; if fewer were seen, walk ids 0, 1, 2, ... below
+    ``draft_vocab_size`` and add the ones not yet chosen."""
+    ranked = sorted(token_freq.items(), key=lambda kv: (-kv[1], kv[0]))
+    chosen = [tid for tid, _ in ranked[:draft_vocab_size]]
+    have = set(chosen)
+    tid = 0
+    while len(chosen) < draft_vocab_size and tid < draft_vocab_size:
+        if tid not in have:
+            chosen.append(tid)
+            have.add(tid)
+        tid += 1
+    return build_vocab_mappings(chosen, target_vocab_size)

@@ -135,3 +135,45 @@ def test_vocab_tables_closed_form_and_gather_identity():
     w = torch.randn(vt, h, generator=g, dtype=torch.double)
     x = torch.randn(5, h, generator=g, dtype=torch.double)
     assert torch.allclose(V.gather_targets(x @ w.T, d2t), x @ w[t2d].T, atol=1e-12)
+
+
+# ---------------------------------------------------------------- draft vocabulary selection
+def test_vocab_selection_hand_worked():
+    """train/vocab_mapping.py:64-96 on a case small enough to do by hand: counts
+    {7: 5, 2: 5, 9: 1, 4: 3}, draft size 3 of 12 -> ids ranked (2, 7, 4, 9): ties on the count
+    go to the smaller id; chosen {2, 4, 7} -> offsets [2, 3, 5]."""
+    d2t, t2d = V.build_vocab_mappings_from_distribution({7: 5, 2: 5, 9: 1, 4: 3}, 3, 12)
+    assert d2t.tolist() == [2, 3, 5]
+    assert torch.nonzero(t2d).reshape(-1).tolist() == [2, 4, 7]
+    # fewer ids seen than the draft size: the smallest unused ids below the draft size fill up
+    d2t, t2d = V.build_vocab_mappings_from_distribution({9: 4, 1: 2}, 4, 12)
+    assert torch.nonzero(t2d).reshape(-1).tolist() == [0, 1, 2, 9]
+    assert d2t.tolist() == [0, 0, 0, 6]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_vocab_selection_product_matches_oracle(seed):
+    from speculators_amd.vocab import build_vocab_mappings_from_distribution, count_token_frequencies
+
+    g = torch.Generator().manual_seed(seed)
+    vt = 97
+    vd = [5, 40, 96, 97, 1, 60][seed]
+    samples = []
+    for _ in range(4):
+        n = int(torch.randint(1, 60, (1,), generator=g))
+        hi = [vt, 30, vt, vt, 8, 20][seed]  # some seeds see fewer ids than the draft size
+        samples.append({"input_ids": torch.randint(0, hi, (n,), generator=g),
+                        "loss_mask": torch.randint(0, 2, (n,), generator=g)})
+    counts = count_token_frequencies(samples, vt)
+    freq = {}
+    for s in samples:  # the dict the reference stores: counts of the masked tokens
+        for tid, m in zip(s["input_ids"].tolist(), s["loss_mask"].tolist(), strict=True):
+            if m:
+                freq[tid] = freq.get(tid, 0) + 1
+    assert {i: int(c) for i, c in enumerate(counts.tolist()) if c} == freq
+    want = V.build_vocab_mappings_from_distribution(freq, vd, vt)
+    for src in (freq, counts):
+        d2t, t2d = build_vocab_mappings_from_distribution(src, vd, vt)
+        assert torch.equal(d2t, want[0]) and torch.equal(t2d, want[1])
+        V.validate_vocab_mappings(t2d, d2t, vd, vt)
+        assert torch.equal(torch.nonzero(t2d).reshape(-1), torch.arange(vd) + d2t)
