@@ -59,7 +59,7 @@ def parse_args():
                     help="eagle3 = configs[1], the headline; eagle3-70b = configs[3]; mtp = configs[4] (MTP "
                          "head, full-vocab CE); dflash = configs[2] (anchored blocks, 5 layers)")
     ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
     ap.add_argument("--ttt-steps", type=int, default=TTT_STEPS)
     ap.add_argument("--targets", choices=["hidden", "logits"], default="hidden",
@@ -109,6 +109,25 @@ def make_model(torch, cfg, device, d2t, t2d):
                 p.copy_((torch.randn(p.shape, device=device, generator=g) * 0.02).to(p.dtype))
     model.load_vocab_mappings(t2d, d2t)
     return model
+
+
+class quiet_gc:
+    """The timed region runs without the cyclic garbage collector: one of its full passes in
+    the middle of a forward (tens of milliseconds of host time) drains the GPU's launch queue and
+    shows up as one slow step."""
+
+    def __enter__(self):
+        import gc
+
+        gc.collect()
+        self.was = gc.isenabled()
+        gc.disable()
+
+    def __exit__(self, *exc):
+        import gc
+
+        if self.was:
+            gc.enable()
 
 
 def time_events(torch, fn, iters, warmup=2):
@@ -337,11 +356,12 @@ def run_mtp(args):
 
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        loss = step()
-    torch.cuda.synchronize()
+    with quiet_gc():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            loss = step()
+        torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
     tokens = b * n
     final_loss = float(loss)
@@ -511,11 +531,12 @@ def run_dflash(args):
 
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        loss = step()
-    torch.cuda.synchronize()
+    with quiet_gc():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            loss = step()
+        torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
     final_loss = float(loss.detach())
     del loss
@@ -606,11 +627,12 @@ def main():
 
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        loss = step()
-    torch.cuda.synchronize()
+    with quiet_gc():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            loss = step()
+        torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
     tokens = int((batch["document_ids"] != -1).sum().item())
