@@ -283,7 +283,7 @@ static bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) =
 using namespace spx;
 
 extern "C" int64_t spx_rmsnorm_bwd_slots(int64_t rows, int64_t H) {
-  if (H <= 512) return 4 * (rows < 1024 ? (rows + 3) / 4 : 256);
+  if (H <= 512) return 4 * (rows < 8192 ? (rows + 3) / 4 : 2048);  // one wave per slot, 8 workgroups per CU
   return rows < 1024 ? rows : 1024;  // four workgroups per compute unit
 }
 
