@@ -55,6 +55,7 @@ class Eagle3Config:
     sliding_window: int | None = None
     sliding_layers: tuple = field(default_factory=tuple)
     attn_implementation: str = A.ATTN_IMPL_TTT
+    embed_requires_grad: bool = False  # requires_grad of embed_tokens.weight (models/eagle3/core.py:68)
 
 
 class RMSNorm(nn.Module):
@@ -211,6 +212,7 @@ class Eagle3DraftModel(nn.Module):
         for p in (self.embed_tokens.weight, self.lm_head.weight, self.verifier_lm_head.weight,
                   self.verifier_norm.weight):
             p.requires_grad_(False)
+        self.embed_tokens.weight.requires_grad_(config.embed_requires_grad)
         self.uses_sliding_window_attn = bool(config.sliding_layers)
         self.uses_full_attn = config.num_hidden_layers > len(config.sliding_layers)
         self._frozen_t: dict = {}
@@ -298,6 +300,8 @@ class Eagle3DraftModel(nn.Module):
         position_ids = position_ids.reshape(-1).to(torch.int64).contiguous()
         draft_tokens = []
         for step in range(ttt_steps):
+            # looked up without a graph whatever embed_requires_grad says, as the reference does
+            # (models/eagle3/core.py:270-271): the flag only marks the parameter as trainable
             with torch.no_grad():
                 embeds = F.embedding(input_ids, self.embed_tokens.weight)
             y = (embeds.to(hidden.dtype), hidden)
