@@ -87,3 +87,93 @@ def test_backward_matches_dense_oracle_autograd(t, hq, hkv, d, docs, window, ste
     if step > 0:
         err = (kg.grad.float().cpu()[:, :, t:] - kr.grad[:, :, t:]).abs().max().item()
         assert err <= 2e-2 * kr.grad[:, :, t:].abs().max().item()
+
+
+def _check_sampled_rows(q, k, v, out, go, rows, heads, visible, scale):
+    """Forward output and dQ of single (row, head) pairs against the explicit fp32 soft-max over
+    the keys ``visible(row)`` marks: both depend on that row only."""
+    hq, hkv = q.shape[1], k.shape[1]
+    for i, h in zip(rows, heads, strict=True):
+        kvh = h // (hq // hkv)
+        vis = visible(i).cuda()
+        qi = q.detach()[0, h, i].float().cpu().requires_grad_(True)
+        ks, vs = k.detach()[0, kvh, vis].float().cpu(), v.detach()[0, kvh, vis].float().cpu()
+        p = torch.softmax((ks @ qi) * scale, dim=0)
+        want = p @ vs
+        (want * go[0, i, h].float().cpu()).sum().backward()
+        got = out.detach()[0, i, h].float().cpu()
+        assert (got - want.detach()).abs().max() <= 2e-2 * want.detach().abs().max() + 1e-3, (i, h)
+        dq = q.grad[0, h, i].float().cpu()
+        assert (dq - qi.grad).abs().max() <= 3e-2 * qi.grad.abs().max() + 1e-3, (i, h)
+
+
+def _check_dv_checksum(v, go, hq):
+    """Rows of P sum to one, so per K/V head: sum over keys of dV == sum over its query heads
+    and rows of dO."""
+    hkv, d, t = v.shape[1], v.shape[3], go.shape[1]
+    want = go[0].float().view(t, hkv, hq // hkv, d).sum(dim=(0, 2)).cpu()
+    got = v.grad[0].float().sum(dim=1).cpu()
+    err = (got - want).abs().max().item()
+    assert err <= 2e-2 * want.abs().max().item() + 0.5, err
+
+
+def test_full_size_sampled_rows_and_checksums():
+    """The headline shape (T 4096, 32 q / 8 kv heads, head_dim 128, last TTT step of 7, three
+    packed documents and a padded tail), checked through what does not need a dense T x 7T oracle:
+    sampled query rows (forward and dQ) and the column-sum identity of dV."""
+    from speculators_amd import attention as A
+
+    t, hq, hkv, d, step = 4096, 32, 8, 128, 6
+    g = torch.Generator().manual_seed(7)
+    doc = torch.full((t,), -1, dtype=torch.long)
+    doc[:1500], doc[1500:1501], doc[1501:4000] = 0, 1, 2  # a one-token document in the middle
+    q = torch.randn(1, hq, t, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    k = torch.randn(1, hkv, (step + 1) * t, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    v = torch.randn(1, hkv, (step + 1) * t, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    go = torch.randn(1, t, hq, d, generator=g).bfloat16().cuda()
+    mask = A.create_ttt_mask(doc.cuda(), t, None)
+    for _ in range(step):
+        mask = mask.extended()
+    out = A.ttt_attention(q, k, v, mask)
+    out.backward(go)
+    assert torch.isfinite(out).all() and torch.isfinite(q.grad).all() and torch.isfinite(k.grad).all()
+
+    rows = torch.cat([torch.tensor([0, 1, 1499, 1500, 1501, 3999, 4000, 4095]),
+                      torch.randint(0, t, (56,), generator=g)]).tolist()
+    heads = torch.randint(0, hq, (len(rows),), generator=g).tolist()
+    kv_idx = torch.arange((step + 1) * t)
+
+    def visible(i):
+        vis = (kv_idx % t) == i  # one key of every step at the row's own position
+        if doc[i] != -1:
+            vis = vis | ((kv_idx <= i) & (kv_idx < t) & (doc[kv_idx % t] == doc[i]))
+        return vis
+
+    _check_sampled_rows(q, k, v, out, go, rows, heads, visible, d ** -0.5)
+    _check_dv_checksum(v, go, hq)
+    # a key of a later step is seen by exactly one row: its gradient is that row's, never zero
+    assert (k.grad[0, :, t:2 * t].float().abs().sum(dim=-1) > 0).all()
+
+
+def test_full_size_head_dim_256_sampled_rows():
+    """The MTP shape (two packed sequences of 16380, 16 q / 2 kv heads, head_dim 256, causal
+    inside each sequence): sampled rows and the dV checksum."""
+    from speculators_amd import attention as A
+
+    n, b, hq, hkv, d = 16380, 2, 16, 2, 256
+    t = n * b
+    g = torch.Generator().manual_seed(9)
+    seq = torch.arange(b).repeat_interleave(n)
+    q = torch.randn(1, hq, t, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    k = torch.randn(1, hkv, t, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    v = torch.randn(1, hkv, t, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    go = torch.randn(1, t, hq, d, generator=g).bfloat16().cuda()
+    out = A.ttt_attention(q, k, v, A.create_ttt_mask(seq.cuda(), t, None), d ** -0.5)
+    out.backward(go)
+    rows = torch.cat([torch.tensor([0, 1, n - 1, n, n + 1, t - 1]),
+                      torch.randint(0, t, (26,), generator=g)]).tolist()
+    heads = torch.randint(0, hq, (len(rows),), generator=g).tolist()
+    kv_idx = torch.arange(t)
+    _check_sampled_rows(q, k, v, out, go, rows, heads,
+                        lambda i: (kv_idx <= i) & (seq == seq[i]), d ** -0.5)
+    _check_dv_checksum(v, go, hq)

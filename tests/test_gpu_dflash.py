@@ -141,3 +141,38 @@ def test_model_forward_backward_matches_oracle(weighting, sliding):
         floor = (wb[name].grad.float() - want).abs().max().item()
         # 2e-2 relative max-norm, or twice the error a bf16 PyTorch run of the oracle makes
         assert err <= max(2e-2 * scale, 2 * floor) + 1e-6, (name, err, floor, scale)
+
+
+def test_full_size_sampled_rows():
+    """configs[2] shape (seq 8192, 512 anchors x block 16 -> 8192 queries, 16384 keys, window
+    2048, 32 q / 8 kv heads, head_dim 128): sampled rows (forward and dQ) against the explicit
+    fp32 soft-max over the keys the mask rule of models/dflash/attention.py:7-100 lets each row
+    see, and the dV column-sum identity."""
+    from speculators_amd import attention as A
+    from tests.test_gpu_attention import _check_dv_checksum, _check_sampled_rows
+
+    t, bs, n_anchor, w, hq, hkv, d = 8192, 16, 512, 2048, 32, 8, 128
+    g = torch.Generator().manual_seed(13)
+    doc = torch.zeros(t, dtype=torch.long)
+    doc[5000:] = 1
+    anchors = (torch.arange(n_anchor) * ((t - bs) // n_anchor) + 1)
+    n_q = n_anchor * bs
+    q = torch.randn(1, hq, n_q, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    k = torch.randn(1, hkv, t + n_q, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    v = torch.randn(1, hkv, t + n_q, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    go = torch.randn(1, n_q, hq, d, generator=g).bfloat16().cuda()
+    mask = A.create_dflash_mask(doc.cuda(), t, anchors.cuda(), bs, w, False)
+    out = A.dflash_attention(q, k, v, mask)
+    out.backward(go)
+    rows = torch.cat([torch.tensor([0, 15, 16, n_q - 1]), torch.randint(0, n_q, (28,), generator=g)]).tolist()
+    heads = torch.randint(0, hq, (len(rows),), generator=g).tolist()
+    kv_idx = torch.arange(t + n_q)
+
+    def visible(i):
+        blk, a = i // bs, int(anchors[i // bs])
+        ctx = (kv_idx < t) & (kv_idx < a) & (kv_idx >= a - w) & (doc[kv_idx.clamp(max=t - 1)] == doc[a])
+        own = (kv_idx >= t) & ((kv_idx - t) // bs == blk) & (kv_idx - t <= i)  # windowed layer: causal block
+        return ctx | own
+
+    _check_sampled_rows(q, k, v, out, go, rows, heads, visible, d ** -0.5)
+    _check_dv_checksum(v, go, hq)
