@@ -139,6 +139,20 @@ struct RowBounds {
   int blk_a1, blk_b1, blk_a2, blk_b2;
 };
 
+// value of the partner lane (lane ^ 32) combined with the own one, through v_permlane32_swap
+// (a VALU move) instead of an LDS permute: swapping (x, x) leaves the lower half of the wave's
+// values in every lane of the first result and the upper half in the second
+__device__ __forceinline__ float half_swap_max(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto s = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(s[0]), __uint_as_float(s[1]));
+}
+__device__ __forceinline__ float half_swap_sum(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto s = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(s[0]) + __uint_as_float(s[1]);
+}
+
 __device__ __forceinline__ int wave_min_i(int v) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) v = min(v, __shfl_xor(v, m, 64));
@@ -371,7 +385,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[sb][kb][r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = half_swap_max(mx);
         const float m_new = fmaxf(m_run[sb], mx * p.scale_log2e);
         const float alpha = fast_exp2(m_run[sb] - m_new);
         float rs = 0.f;
@@ -383,7 +397,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
             st[sb][kb][r] = pv;
             rs += pv;
           }
-        rs += __shfl_xor(rs, 32, 64);
+        rs = half_swap_sum(rs);
         l_run[sb] = l_run[sb] * alpha + rs;
         // the accumulator only needs rescaling when some row's max moved
         if (__any(m_new != m_run[sb])) {
@@ -436,7 +450,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
 #pragma unroll
       for (int kk = 0; kk < NKK; ++kk)
         dot = dot8_bf16(qf[sb][kk], *reinterpret_cast<const u32x4*>(kj + kk * 16), dot);
-      dot += __shfl_xor(dot, 32, 64);
+      dot = half_swap_sum(dot);
       const float s = dot * p.scale_log2e;
       const float m_new = fmaxf(m_run[sb], s);
       const float alpha = fast_exp2(m_run[sb] - m_new);
@@ -478,22 +492,70 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
 
 // ---------------------------------------------------------------- backward
 // delta[h, i] = sum_d dO[i, h, d] * O[i, h, d]
+// sum over each row of sixteen lanes, left in every lane of the row
+__device__ __forceinline__ float row16_sum(float v) {
+  // quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror: afterwards every lane
+  // of a 16-lane row holds the sum over the row
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true));
+  return v;
+}
+
+// EPL (4, 8 or 16) consecutive bf16 of one lane in 8- or 16-byte accesses
+template <int EPL>
+__device__ __forceinline__ void ld_bf16s(const uint16_t* p, float (&v)[EPL]) {
+  if constexpr (EPL == 4) {
+    const u32x2 u = *reinterpret_cast<const u32x2*>(p);
+    v[0] = bf16_lo(u.x); v[1] = bf16_hi(u.x); v[2] = bf16_lo(u.y); v[3] = bf16_hi(u.y);
+  } else {
+    static_assert(EPL % 8 == 0, "4, 8 or 16 elements per lane");
+#pragma unroll
+    for (int c = 0; c < EPL / 8; ++c) {
+      const u32x4 u = *reinterpret_cast<const u32x4*>(p + 8 * c);
+      v[8 * c + 0] = bf16_lo(u.x); v[8 * c + 1] = bf16_hi(u.x);
+      v[8 * c + 2] = bf16_lo(u.y); v[8 * c + 3] = bf16_hi(u.y);
+      v[8 * c + 4] = bf16_lo(u.z); v[8 * c + 5] = bf16_hi(u.z);
+      v[8 * c + 6] = bf16_lo(u.w); v[8 * c + 7] = bf16_hi(u.w);
+    }
+  }
+}
+template <int EPL>
+__device__ __forceinline__ void st_bf16s(uint16_t* p, const float (&v)[EPL]) {
+  if constexpr (EPL == 4) {
+    u32x2 u;
+    u.x = pack_bf16x2(v[0], v[1]); u.y = pack_bf16x2(v[2], v[3]);
+    *reinterpret_cast<u32x2*>(p) = u;
+  } else {
+#pragma unroll
+    for (int c = 0; c < EPL / 8; ++c) {
+      u32x4 u;
+      u.x = pack_bf16x2(v[8 * c + 0], v[8 * c + 1]); u.y = pack_bf16x2(v[8 * c + 2], v[8 * c + 3]);
+      u.z = pack_bf16x2(v[8 * c + 4], v[8 * c + 5]); u.w = pack_bf16x2(v[8 * c + 6], v[8 * c + 7]);
+      *reinterpret_cast<u32x4*>(p + 8 * c) = u;
+    }
+  }
+}
+
 template <int D>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const uint16_t* __restrict__ O,
                                                          const uint16_t* __restrict__ dO, int NQ,
                                                          int Hq, float* __restrict__ delta) {
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // = i * Hq + h
-  if (row >= (int64_t)NQ * Hq) return;
-  const int lane = threadIdx.x & 63;
+  // sixteen lanes per (row, head): D / 16 consecutive elements each, summed with DPP moves
+  constexpr int EPL = D / 16;
+  const int64_t n_rows = (int64_t)NQ * Hq;
+  const int64_t raw = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 4 + ((threadIdx.x & 63) >> 4);
+  const int64_t row = raw < n_rows ? raw : n_rows - 1;  // = i * Hq + h
+  const int d0 = (threadIdx.x & 15) * EPL;
+  float a[EPL], b[EPL];
+  ld_bf16s<EPL>(O + row * D + d0, a);
+  ld_bf16s<EPL>(dO + row * D + d0, b);
   float acc = 0.f;
-  for (int d = lane * 2; d < D; d += 128) {
-    uint32_t a = *reinterpret_cast<const uint32_t*>(O + row * D + d);
-    uint32_t b = *reinterpret_cast<const uint32_t*>(dO + row * D + d);
-    acc = fmaf(bf16_lo(a), bf16_lo(b), acc);
-    acc = fmaf(bf16_hi(a), bf16_hi(b), acc);
-  }
-  acc = wave_sum(acc);
-  if (lane == 0) delta[(row % Hq) * (int64_t)NQ + row / Hq] = acc;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) acc = fmaf(a[e], b[e], acc);
+  acc = row16_sum(acc);
+  if ((threadIdx.x & 15) == 0 && raw < n_rows) delta[(row % Hq) * (int64_t)NQ + row / Hq] = acc;
 }
 
 // dQ: same tiling as the forward.
@@ -703,8 +765,8 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
         dot = dot8_bf16(qf[sb][kk], *reinterpret_cast<const u32x4*>(kj + g * 8 + kk * 16), dot);
         dpv = dot8_bf16(dof[sb][kk], *reinterpret_cast<const u32x4*>(vj + g * 8 + kk * 16), dpv);
       }
-      dot += __shfl_xor(dot, 32, 64);
-      dpv += __shfl_xor(dpv, 32, 64);
+      dot = half_swap_sum(dot);
+      dpv = half_swap_sum(dpv);
       const float pv = fast_exp2(fmaf(dot, p.scale_log2e, -lse_i[sb]));
       const float ds = pv * (dpv - delta_i[sb]);
 #pragma unroll
@@ -1074,59 +1136,94 @@ __global__ __launch_bounds__(256) void attn_dkv_reduce_kernel(
   *reinterpret_cast<u32x2*>(dV + (int64_t)kvh * dv_hs + off) = wv;
 }
 
-// dK / dV of the TTT diagonal keys (j, i), j >= 1: one wave per (position, K/V head);
-// each such key is seen by exactly the `group` query heads at its own position.
+// dK / dV of the TTT diagonal keys (j, i), j >= 1: sixteen lanes per (position, K/V head)
+// item, four items per wave; each such key is seen by exactly the `group` query heads at its
+// own position.  A lane holds D / 16 consecutive elements (one or two 16-byte accesses); the dot
+// products are summed over the sixteen lanes with DPP moves (no LDS traffic).
 template <int D>
 __global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
     const uint16_t* __restrict__ Q, int64_t q_hs, const uint16_t* __restrict__ K, int64_t k_hs,
     const uint16_t* __restrict__ V, int64_t v_hs, const uint16_t* __restrict__ dO,
     const float* __restrict__ LSE, const float* __restrict__ Delta, int T, int n_extra, int Hq,
-    int Hkv, float scale_log2e, float scaling, uint16_t* __restrict__ dK, int64_t dk_hs,
-    uint16_t* __restrict__ dV, int64_t dv_hs) {
-  constexpr int EPL = D / 64;
-  const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // = i * Hkv + kvh
-  if (item >= (int64_t)T * Hkv) return;
-  const int lane = threadIdx.x & 63;
-  const int i = (int)(item / Hkv), kvh = (int)(item % Hkv);
+    int Hkv, float scale_log2e, float scaling, uint16_t* dK, int64_t dk_hs, uint16_t* dV,
+    int64_t dv_hs) {
+  constexpr int EPL = D / 16;
+  constexpr int MAXG = 4;  // query heads per K/V head kept in registers at a time
+  // item = kvh * T + i: neighbouring 16-lane rows take neighbouring positions of one K/V head, so
+  // their key / value / gradient rows are contiguous in memory.  The tail clamps (no early
+  // return: the DPP sums need whole rows of lanes)
+  const int64_t n_items = (int64_t)T * Hkv;
+  const int64_t raw = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 4 + ((threadIdx.x & 63) >> 4);
+  const bool live = raw < n_items;
+  const int64_t item = live ? raw : n_items - 1;
+  const int kvh = (int)(item / T), i = (int)(item % T);
   const int group = Hq / Hkv;
-  const int d0 = lane * EPL;
-  for (int j = 1; j <= n_extra; ++j) {
-    const int64_t krow = (int64_t)kvh * k_hs + ((int64_t)j * T + i) * D + d0;
-    const int64_t vrow = (int64_t)kvh * v_hs + ((int64_t)j * T + i) * D + d0;
-    float kv[EPL], vv[EPL], gk[EPL], gv[EPL];
+  const int d0 = (threadIdx.x & 15) * EPL;
+  for (int h0 = 0; h0 < group; h0 += MAXG) {
+    // the row's query and output-gradient vectors of up to MAXG heads are read once and reused
+    // for every diagonal key (they do not depend on j)
+    const int ng = min(group - h0, MAXG);
+    float qv[MAXG][EPL], dv[MAXG][EPL], lse_h[MAXG], delta_h[MAXG];
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) {
-      kv[e] = bf16_bits_to_f32(K[krow + e]);
-      vv[e] = bf16_bits_to_f32(V[vrow + e]);
-      gk[e] = 0.f; gv[e] = 0.f;
+    for (int hh = 0; hh < MAXG; ++hh) {
+      const int h = kvh * group + h0 + (hh < ng ? hh : 0);
+      ld_bf16s<EPL>(Q + (int64_t)h * q_hs + (int64_t)i * D + d0, qv[hh]);
+      ld_bf16s<EPL>(dO + ((int64_t)i * Hq + h) * D + d0, dv[hh]);
+      lse_h[hh] = LSE[(int64_t)h * T + i];
+      delta_h[hh] = Delta[(int64_t)h * T + i];
     }
-    for (int hh = 0; hh < group; ++hh) {
-      const int h = kvh * group + hh;
-      float qv[EPL], dv[EPL];
-      float dot = 0.f, dpv = 0.f;
+    // the key / value rows of diagonal j + 1 are requested before diagonal j is worked on: the
+    // loop is a chain of dependent global loads otherwise
+    float kn[EPL], vn[EPL];
+    {
+      const int64_t r1 = ((int64_t)T + i) * D + d0;
+      ld_bf16s<EPL>(K + (int64_t)kvh * k_hs + r1, kn);
+      ld_bf16s<EPL>(V + (int64_t)kvh * v_hs + r1, vn);
+    }
+    for (int j = 1; j <= n_extra; ++j) {
+      const int64_t gko = (int64_t)kvh * dk_hs + ((int64_t)j * T + i) * D + d0;
+      const int64_t gvo = (int64_t)kvh * dv_hs + ((int64_t)j * T + i) * D + d0;
+      float kv[EPL], vv[EPL], gk[EPL], gv[EPL];
 #pragma unroll
       for (int e = 0; e < EPL; ++e) {
-        qv[e] = bf16_bits_to_f32(Q[(int64_t)h * q_hs + (int64_t)i * D + d0 + e]);
-        dv[e] = bf16_bits_to_f32(dO[((int64_t)i * Hq + h) * D + d0 + e]);
-        dot = fmaf(qv[e], kv[e], dot);
-        dpv = fmaf(dv[e], vv[e], dpv);
+        kv[e] = kn[e];
+        vv[e] = vn[e];
+        gk[e] = 0.f;
+        gv[e] = 0.f;
       }
-      dot = wave_sum(dot);
-      dpv = wave_sum(dpv);
-      const float pv = fast_exp2(fmaf(dot, scale_log2e, -LSE[(int64_t)h * T + i]));
-      const float ds = pv * (dpv - Delta[(int64_t)h * T + i]) * scaling;
-#pragma unroll
-      for (int e = 0; e < EPL; ++e) {
-        gv[e] = fmaf(pv, dv[e], gv[e]);
-        gk[e] = fmaf(ds, qv[e], gk[e]);
+      if (h0) {  // groups wider than MAXG accumulate over several passes
+        ld_bf16s<EPL>(dK + gko, gk);
+        ld_bf16s<EPL>(dV + gvo, gv);
       }
-    }
-    const int64_t gko = (int64_t)kvh * dk_hs + ((int64_t)j * T + i) * D + d0;
-    const int64_t gvo = (int64_t)kvh * dv_hs + ((int64_t)j * T + i) * D + d0;
+      if (j < n_extra) {
+        const int64_t rn = ((int64_t)(j + 1) * T + i) * D + d0;
+        ld_bf16s<EPL>(K + (int64_t)kvh * k_hs + rn, kn);
+        ld_bf16s<EPL>(V + (int64_t)kvh * v_hs + rn, vn);
+      }
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) {
-      dK[gko + e] = (uint16_t)f32_to_bf16_bits(gk[e]);
-      dV[gvo + e] = (uint16_t)f32_to_bf16_bits(gv[e]);
+      for (int hh = 0; hh < MAXG; ++hh) {
+        if (hh < ng) {
+          float dot = 0.f, dpv = 0.f;
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) {
+            dot = fmaf(qv[hh][e], kv[e], dot);
+            dpv = fmaf(dv[hh][e], vv[e], dpv);
+          }
+          dot = row16_sum(dot);
+          dpv = row16_sum(dpv);
+          const float pv = fast_exp2(fmaf(dot, scale_log2e, -lse_h[hh]));
+          const float ds = pv * (dpv - delta_h[hh]) * scaling;
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) {
+            gv[e] = fmaf(pv, dv[hh][e], gv[e]);
+            gk[e] = fmaf(ds, qv[hh][e], gk[e]);
+          }
+        }
+      }
+      if (live) {
+        st_bf16s<EPL>(dK + gko, gk);
+        st_bf16s<EPL>(dV + gvo, gv);
+      }
     }
   }
 }
@@ -1217,7 +1314,7 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
                      qt, (int64_t)D * NQp, (int64_t)NQp);
   hipLaunchKernelGGL(transpose_bf16_kernel, qgrid, dim3(256), 0, st, dOp, (int64_t)D,
                      (int64_t)p.Hq * D, p.NQ, D, dot, (int64_t)D * NQp, (int64_t)NQp);
-  hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)(((int64_t)p.NQ * p.Hq + 3) / 4)), dim3(256),
+  hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)(((int64_t)p.NQ * p.Hq + 15) / 16)), dim3(256),
                      0, st, Op, dOp, p.NQ, p.Hq, delta);
   hipLaunchKernelGGL(attn_tile_bounds_kernel, dim3((unsigned)((p.NQ + 63) / 64)), dim3(64), 0, st, p, tb);
 
@@ -1263,7 +1360,7 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   hipLaunchKernelGGL(attn_dkv_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, dkp,
                      dvp, p.NKV, D, p.Hq, p.Hkv, p.scaling, dKp, dk_hs, dVp, dv_hs);
   if (p.n_extra > 0)
-    hipLaunchKernelGGL(ttt_attn_bwd_diag_kernel<D>, dim3((unsigned)(((int64_t)p.T * p.Hkv + 3) / 4)),
+    hipLaunchKernelGGL(ttt_attn_bwd_diag_kernel<D>, dim3((unsigned)(((int64_t)p.T * p.Hkv + 15) / 16)),
                        dim3(256), 0, st, p.Q, p.q_hs, p.K, p.k_hs, p.V, p.v_hs, dOp, lse, delta, p.T,
                        p.n_extra, p.Hq, p.Hkv, p.scale_log2e, p.scaling, dKp, dk_hs, dVp, dv_hs);
   return check_launch(fn);
