@@ -124,11 +124,19 @@ class DFlashDecoderLayer(nn.Module):
         self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
         self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
 
-    def forward(self, x, ctx, q_pos, kv_pos, inv_freq, mask):
-        a = self.self_attn(self.input_layernorm(x), ctx, q_pos, kv_pos, inv_freq, mask)
+    def forward(self, x, ctx, q_pos, kv_pos, inv_freq, mask, x_normed=None, next_norm=None):
+        """``x_normed``: ``input_layernorm(x)`` when the previous layer already produced it;
+        ``next_norm``: the RMSNorm that reads this layer's output -- the result is then
+        ``(out, next_norm(out))`` with the last residual add fused into that norm."""
+        if x_normed is None:
+            x_normed = self.input_layernorm(x)
+        a = self.self_attn(x_normed, ctx, q_pos, kv_pos, inv_freq, mask)
         post = self.post_attention_layernorm
         y, z = FO.add_rms_norm(x, a, post.weight, post.eps)  # residual add fused into the norm
-        return y + self.mlp(z)
+        m = self.mlp(z)
+        if next_norm is None:
+            return y + m
+        return FO.add_rms_norm(y, m, next_norm.weight, next_norm.eps)
 
 
 class DFlashDraftModel(nn.Module):
@@ -217,10 +225,15 @@ class DFlashDraftModel(nn.Module):
             idx = block_idx if cfg.sample_from_anchor else (block_idx - 1) % t
             targets = self._linear(self.verifier_norm(verifier_last_hidden_states[:, idx]),
                                    self.verifier_lm_head.weight)
+        normed = None
+        last = len(self.layers) - 1
         for li, layer in enumerate(self.layers):
-            noise = layer(noise, ctx, q_pos, kv_pos, inv_freq,
-                          sw_mask if li in cfg.sliding_layers else full_mask)
-        logits = self._linear(self.norm(noise), self.lm_head.weight, frozen=True)
+            # the norm that reads this layer's output: the next layer's input norm or the final one
+            nxt = self.norm if li == last else self.layers[li + 1].input_layernorm
+            noise, normed = layer(noise, ctx, q_pos, kv_pos, inv_freq,
+                                  sw_mask if li in cfg.sliding_layers else full_mask,
+                                  x_normed=normed, next_norm=nxt)
+        logits = self._linear(normed, self.lm_head.weight, frozen=True)
         aligned = loss_mask.clone()[:, block_idx]
         aligned = aligned * anchor_valid.repeat_interleave(bs).unsqueeze(0).to(aligned.dtype)
         if not cfg.sample_from_anchor:
