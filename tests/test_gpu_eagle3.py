@@ -154,3 +154,46 @@ def test_requires_bf16_and_hip_tensors():
     hs, ids, doc, mask, pos, vl = _batch(shape, 128, 6, [128])
     with pytest.raises(RuntimeError):
         model(hs.cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.cuda(), ttt_steps=1)
+
+
+def test_gradient_accumulation_semantics_across_iterations():
+    """The weight gradients are written into ``.grad`` by the GEMMs themselves (merged q/k/v
+    buffer, beta = 1 accumulation over TTT steps): a second backward without ``zero_grad`` must
+    add to them, ``zero_grad(set_to_none=False)`` must be honoured, and a fresh run must give the
+    first run's bits again (every kernel reduces in a fixed order)."""
+    shape = _shape(num_hidden_layers=2)
+    w = {k_: v.bfloat16() for k_, v in OE.random_weights(shape, seed=4, std=0.05).items()}
+    model = _make(shape, w)
+    hs, ids, doc, mask, pos, vl = _batch(shape, 192, 9, [100, 80])
+    args = (hs.bfloat16().cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.bfloat16().cuda())
+
+    def run():
+        _, loss, _ = model(*args, ttt_steps=3, ttt_step_loss_decay=0.9)
+        loss.backward()
+        return loss.item()
+
+    params = {n: p for n, p in model.named_parameters() if p.requires_grad}
+    l1 = run()
+    g1 = {n: p.grad.clone() for n, p in params.items()}
+    assert all(torch.isfinite(g).all() for g in g1.values())
+    l2 = run()  # accumulates
+    assert l2 == l1
+    for n, p in params.items():
+        want = 2 * g1[n].float()
+        err = (p.grad.float() - want).abs().max().item()
+        assert err <= 2 ** -7 * want.abs().max().item() + 1e-8, (n, err)  # one more bf16 rounding
+    model.zero_grad(set_to_none=False)
+    assert all(not p.grad.any() for p in params.values())
+    run()
+    for n, p in params.items():
+        assert torch.equal(p.grad, g1[n]), n
+    model.zero_grad(set_to_none=True)
+    run()
+    for n, p in params.items():
+        assert torch.equal(p.grad, g1[n]), n
+    # a plain optimizer step works on the (view) gradients and changes the next loss
+    opt = torch.optim.SGD(params.values(), lr=0.05)
+    opt.step()
+    model.zero_grad(set_to_none=True)
+    l3 = run()
+    assert l3 < l1
