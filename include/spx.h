@@ -315,7 +315,14 @@ int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* position_ids,
                       int64_t position_offset, void* stream);
 
 /* out = bf16(silu(gate)) * up  (LlamaMLP / Qwen3MLP act_fn(gate_proj(x)) * up_proj(x)),
- * n elements, bf16; and its backward. */
+ * bf16; and its backward.  rows x F elements per tensor, each with its own row stride, so
+ * that gate and up can be the two column halves of one merged gate/up projection. */
+int spx_swiglu_rows_fwd(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                        void* out, int64_t ld_out, int64_t rows, int64_t F, void* stream);
+int spx_swiglu_rows_bwd(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                        const void* dout, int64_t ld_dout, void* dgate, int64_t ld_dgate,
+                        void* dup, int64_t ld_dup, int64_t rows, int64_t F, void* stream);
+/* the same on contiguous tensors of n elements */
 int spx_swiglu_fwd(const void* gate, const void* up, void* out, int64_t n, void* stream);
 int spx_swiglu_bwd(const void* gate, const void* up, const void* dout, void* dgate,
                    void* dup, int64_t n, void* stream);

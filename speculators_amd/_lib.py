@@ -48,6 +48,8 @@ SIGNATURES["spx_rmsnorm_bwd"] = [_P, _I64, _P, _P, _I64, _P, _P, _I64, _P, _P, _
 SIGNATURES["spx_add_rmsnorm_fwd"] = [_P, _I64, _P, _I64, _P, _I64, _P, _P, _I64, _P, _I64, _I64, _F, _P]
 SIGNATURES["spx_add_rmsnorm_bwd"] = [_P, _I64, _P, _P, _I64, _P, _I64, _P, _P, _I64, _P, _P, _I64, _I64, _P]
 SIGNATURES["spx_rope_relayout"] = [_P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _I64, _P]
+SIGNATURES["spx_swiglu_rows_fwd"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _P]
+SIGNATURES["spx_swiglu_rows_bwd"] = [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _P]
 SIGNATURES["spx_swiglu_fwd"] = [_P, _P, _P, _I64, _P]
 SIGNATURES["spx_swiglu_bwd"] = [_P, _P, _P, _P, _P, _I64, _P]
 SIGNATURES["spx_label_ce_fwd"] = [_P, _I64, _P, _I64, _I64, _I, _I64, _P, _P, _P, _P]

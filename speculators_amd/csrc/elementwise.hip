@@ -238,32 +238,40 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
 }
 
 // ---------------------------------------------------------------- SwiGLU
-__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint16_t* __restrict__ g,
-                                                         const uint16_t* __restrict__ u,
-                                                         uint16_t* __restrict__ out, int64_t n8) {
+// rows x F elements per tensor, every tensor with its own row stride (so gate and up may be the
+// two column halves of one merged projection output); chunk = 8 consecutive elements of a row
+__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint16_t* __restrict__ g, int64_t ld_g,
+                                                         const uint16_t* __restrict__ u, int64_t ld_u,
+                                                         uint16_t* __restrict__ out, int64_t ld_o,
+                                                         int64_t rows, int64_t f8) {
+  const int64_t n8 = rows * f8;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / f8, c = (i - r * f8) * 8;
     float gv[8], uv[8], o[8];
-    unpack8f(*reinterpret_cast<const u32x4*>(g + i * 8), gv);
-    unpack8f(*reinterpret_cast<const u32x4*>(u + i * 8), uv);
+    unpack8f(*reinterpret_cast<const u32x4*>(g + r * ld_g + c), gv);
+    unpack8f(*reinterpret_cast<const u32x4*>(u + r * ld_u + c), uv);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float sg = 1.f / (1.f + __expf(-gv[e]));
       o[e] = round_bf16(gv[e] * sg) * uv[e];
     }
-    *reinterpret_cast<u32x4*>(out + i * 8) = pack8f(o);
+    *reinterpret_cast<u32x4*>(out + r * ld_o + c) = pack8f(o);
   }
 }
 
-__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* __restrict__ g,
-                                                         const uint16_t* __restrict__ u,
-                                                         const uint16_t* __restrict__ dout,
-                                                         uint16_t* __restrict__ dg,
-                                                         uint16_t* __restrict__ du, int64_t n8) {
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* __restrict__ g, int64_t ld_g,
+                                                         const uint16_t* __restrict__ u, int64_t ld_u,
+                                                         const uint16_t* __restrict__ dout, int64_t ld_d,
+                                                         uint16_t* __restrict__ dg, int64_t ld_dg,
+                                                         uint16_t* __restrict__ du, int64_t ld_du,
+                                                         int64_t rows, int64_t f8) {
+  const int64_t n8 = rows * f8;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / f8, c = (i - r * f8) * 8;
     float gv[8], uv[8], dv[8], og[8], ou[8];
-    unpack8f(*reinterpret_cast<const u32x4*>(g + i * 8), gv);
-    unpack8f(*reinterpret_cast<const u32x4*>(u + i * 8), uv);
-    unpack8f(*reinterpret_cast<const u32x4*>(dout + i * 8), dv);
+    unpack8f(*reinterpret_cast<const u32x4*>(g + r * ld_g + c), gv);
+    unpack8f(*reinterpret_cast<const u32x4*>(u + r * ld_u + c), uv);
+    unpack8f(*reinterpret_cast<const u32x4*>(dout + r * ld_d + c), dv);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float sg = 1.f / (1.f + __expf(-gv[e]));
@@ -271,8 +279,8 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* __restr
       ou[e] = dv[e] * act;
       og[e] = dv[e] * uv[e] * (sg * (1.f + gv[e] * (1.f - sg)));
     }
-    *reinterpret_cast<u32x4*>(dg + i * 8) = pack8f(og);
-    *reinterpret_cast<u32x4*>(du + i * 8) = pack8f(ou);
+    *reinterpret_cast<u32x4*>(dg + r * ld_dg + c) = pack8f(og);
+    *reinterpret_cast<u32x4*>(du + r * ld_du + c) = pack8f(ou);
   }
 }
 
@@ -411,27 +419,47 @@ extern "C" int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* pos
   return check_launch(__func__);
 }
 
-extern "C" int spx_swiglu_fwd(const void* gate, const void* up, void* out, int64_t n, void* stream) {
-  SPX_REQUIRE(n > 0 && n % 8 == 0, "n must be a positive multiple of 8");
+static unsigned swiglu_grid(int64_t n8) {
+  return (unsigned)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536);
+}
+
+extern "C" int spx_swiglu_rows_fwd(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                                   void* out, int64_t ld_out, int64_t rows, int64_t F, void* stream) {
+  SPX_REQUIRE(rows > 0 && F > 0 && F % 8 == 0, "rows > 0 and F a positive multiple of 8");
+  SPX_REQUIRE(ld_gate >= F && ld_up >= F && ld_out >= F && ld_gate % 8 == 0 && ld_up % 8 == 0 && ld_out % 8 == 0,
+              "row strides must be multiples of 8 and at least F");
   SPX_REQUIRE(gate && up && out && al16(gate) && al16(up) && al16(out), "null or unaligned buffer");
-  const int64_t n8 = n / 8;
-  const unsigned grid = (unsigned)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536);
-  hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(grid), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
-                     reinterpret_cast<const uint16_t*>(gate), reinterpret_cast<const uint16_t*>(up),
-                     reinterpret_cast<uint16_t*>(out), n8);
+  const int64_t f8 = F / 8;
+  hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(swiglu_grid(rows * f8)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const uint16_t*>(gate), ld_gate,
+                     reinterpret_cast<const uint16_t*>(up), ld_up, reinterpret_cast<uint16_t*>(out), ld_out,
+                     rows, f8);
   return check_launch(__func__);
+}
+
+extern "C" int spx_swiglu_rows_bwd(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                                   const void* dout, int64_t ld_dout, void* dgate, int64_t ld_dgate,
+                                   void* dup, int64_t ld_dup, int64_t rows, int64_t F, void* stream) {
+  SPX_REQUIRE(rows > 0 && F > 0 && F % 8 == 0, "rows > 0 and F a positive multiple of 8");
+  SPX_REQUIRE(ld_gate >= F && ld_up >= F && ld_dout >= F && ld_dgate >= F && ld_dup >= F &&
+                  ld_gate % 8 == 0 && ld_up % 8 == 0 && ld_dout % 8 == 0 && ld_dgate % 8 == 0 && ld_dup % 8 == 0,
+              "row strides must be multiples of 8 and at least F");
+  SPX_REQUIRE(gate && up && dout && dgate && dup, "null buffer");
+  SPX_REQUIRE(al16(gate) && al16(up) && al16(dout) && al16(dgate) && al16(dup), "buffers must be 16-byte aligned");
+  const int64_t f8 = F / 8;
+  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(swiglu_grid(rows * f8)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const uint16_t*>(gate), ld_gate,
+                     reinterpret_cast<const uint16_t*>(up), ld_up, reinterpret_cast<const uint16_t*>(dout), ld_dout,
+                     reinterpret_cast<uint16_t*>(dgate), ld_dgate, reinterpret_cast<uint16_t*>(dup), ld_dup, rows,
+                     f8);
+  return check_launch(__func__);
+}
+
+extern "C" int spx_swiglu_fwd(const void* gate, const void* up, void* out, int64_t n, void* stream) {
+  return spx_swiglu_rows_fwd(gate, n, up, n, out, n, 1, n, stream);
 }
 
 extern "C" int spx_swiglu_bwd(const void* gate, const void* up, const void* dout, void* dgate, void* dup,
                               int64_t n, void* stream) {
-  SPX_REQUIRE(n > 0 && n % 8 == 0, "n must be a positive multiple of 8");
-  SPX_REQUIRE(gate && up && dout && dgate && dup, "null buffer");
-  SPX_REQUIRE(al16(gate) && al16(up) && al16(dout) && al16(dgate) && al16(dup), "buffers must be 16-byte aligned");
-  const int64_t n8 = n / 8;
-  const unsigned grid = (unsigned)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536);
-  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(grid), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
-                     reinterpret_cast<const uint16_t*>(gate), reinterpret_cast<const uint16_t*>(up),
-                     reinterpret_cast<const uint16_t*>(dout), reinterpret_cast<uint16_t*>(dgate),
-                     reinterpret_cast<uint16_t*>(dup), n8);
-  return check_launch(__func__);
+  return spx_swiglu_rows_bwd(gate, n, up, n, dout, n, dgate, n, dup, n, 1, n, stream);
 }

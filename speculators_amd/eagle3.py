@@ -120,11 +120,16 @@ class MLP(nn.Module):
         self.gate_proj = nn.Linear(cfg.hidden_size, cfg.intermediate_size, bias=False)
         self.up_proj = nn.Linear(cfg.hidden_size, cfg.intermediate_size, bias=False)
         self.down_proj = nn.Linear(cfg.intermediate_size, cfg.hidden_size, bias=False)
+        self._merged_gate_up = gemm._MergedWeights()
 
     def forward(self, x):
         lin = gemm.linear_accumulate
-        return lin(FO.swiglu(lin(x, self.gate_proj.weight), lin(x, self.up_proj.weight)),
-                   self.down_proj.weight)
+        if gemm.FUSE_WGRAD_ACCUMULATION and torch.is_grad_enabled() and x.dtype == torch.bfloat16:
+            # gate and up as one GEMM, SwiGLU on the two halves of its output
+            act = gemm.gate_up_swiglu(x, self.gate_proj.weight, self.up_proj.weight, self._merged_gate_up)
+        else:
+            act = FO.swiglu(lin(x, self.gate_proj.weight), lin(x, self.up_proj.weight))
+        return lin(act, self.down_proj.weight)
 
 
 class _Prenormed(NamedTuple):

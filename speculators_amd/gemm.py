@@ -116,9 +116,9 @@ def linear_accumulate(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return _LinearAccumulate.apply(x, weight)
 
 
-class _MergedQKV:
-    """Per-module state of the merged q/k/v projection: the concatenated weight of the current
-    weight versions, and the merged gradient buffer the three ``.grad`` tensors are views of."""
+class _MergedWeights:
+    """Per-module state of a merged projection (q/k/v, or gate/up): the concatenated weight of the
+    current weight versions, and the merged gradient buffer the ``.grad`` tensors are views of."""
 
     def __init__(self):
         self.key = None
@@ -133,8 +133,8 @@ class _MergedQKV:
         return self.weight
 
     def accumulate(self, ws, dy2, x2):
-        """``grad(w_i) += dy2[:, rows_i].T @ x2`` for the three weights with one GEMM.  While the
-        three ``.grad`` are the views this object handed out, the GEMM adds into their shared buffer
+        """``grad(w_i) += dy2[:, rows_i].T @ x2`` for all the weights with one GEMM.  While their
+        ``.grad`` are the views this object handed out, the GEMM adds into the shared buffer
         (beta = 1); otherwise (gradients that came from elsewhere) it falls back to one add each."""
         sizes = [w.shape[0] for w in ws]
         views = None
@@ -213,8 +213,58 @@ class _QKVRope(torch.autograd.Function):
 
 
 def qkv_rope(x, wq, wk, wv, position_ids, inv_freq, hq: int, hkv: int, d: int, offset: int,
-             state: _MergedQKV):
+             state: _MergedWeights):
     """``(q [1,Hq,T,D], k [1,Hkv,T,D], v [1,Hkv,T,D])`` with the rotary embedding at
     ``position_ids + offset`` applied to q and k.  Weight gradients land in ``.grad`` during
     ``backward()`` (like ``linear_accumulate``)."""
     return _QKVRope.apply(x, wq, wk, wv, position_ids, inv_freq, hq, hkv, d, offset, state)
+
+
+_MergedQKV = _MergedWeights
+
+
+class _GateUpSwiGLU(torch.autograd.Function):
+    """``silu(x @ Wg.T) * (x @ Wu.T)`` with the two projections as ONE GEMM against the
+    concatenated weight; the SwiGLU kernels read (and, in the backward, write) the two column
+    halves of the merged ``[T, 2F]`` buffer in place, so the input gradient is one GEMM and the
+    weight gradient one GEMM that accumulates across TTT steps."""
+
+    @staticmethod
+    def forward(ctx, x, wg, wu, state):
+        if x.dtype != torch.bfloat16:
+            raise _lib.SpxError("the HIP layer kernels take bf16 tensors")
+        x2 = x.reshape(-1, x.shape[-1])
+        f = wg.shape[0]
+        wcat = state.merged_weight((wg, wu))
+        gu = torch.nn.functional.linear(x2, wcat)  # [T, 2F]
+        rows = x2.shape[0]
+        out = torch.empty(rows, f, device=x.device, dtype=torch.bfloat16)
+        _lib.call("spx_swiglu_rows_fwd", _lib.ptr(gu), 2 * f, _lib.ptr(gu[:, f:]), 2 * f, _lib.ptr(out), f,
+                  rows, f, _lib.stream_ptr(x.device))
+        ctx.save_for_backward(x2, gu, wg, wu)
+        ctx.meta = (x.shape, f, state, wcat)
+        return out.view(*x.shape[:-1], f)
+
+    @staticmethod
+    def backward(ctx, dout):
+        x2, gu, wg, wu = ctx.saved_tensors
+        shape, f, state, wcat = ctx.meta
+        rows = x2.shape[0]
+        d2 = dout.reshape(rows, f).to(torch.bfloat16)
+        if d2.stride(1) != 1 or d2.stride(0) % 8:
+            d2 = d2.contiguous()
+        dgu = torch.empty(rows, 2 * f, device=x2.device, dtype=torch.bfloat16)
+        _lib.call("spx_swiglu_rows_bwd", _lib.ptr(gu), 2 * f, _lib.ptr(gu[:, f:]), 2 * f, _lib.ptr(d2),
+                  d2.stride(0), _lib.ptr(dgu), 2 * f, _lib.ptr(dgu[:, f:]), 2 * f, rows, f,
+                  _lib.stream_ptr(x2.device))
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dx = torch.matmul(dgu, wcat).view(shape)
+        if wg.requires_grad or wu.requires_grad:
+            state.accumulate((wg, wu), dgu, x2)
+        return dx, None, None, None
+
+
+def gate_up_swiglu(x, w_gate, w_up, state: _MergedWeights):
+    """See ``_GateUpSwiGLU``.  Weight gradients land in ``.grad`` during ``backward()``."""
+    return _GateUpSwiGLU.apply(x, w_gate, w_up, state)

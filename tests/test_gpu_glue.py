@@ -180,3 +180,27 @@ def test_qkv_rope_matches_separate_projections(t, h_in, hq, hkv, d):
     torch.autograd.backward(gemm.qkv_rope(x, *ws, pos, inv, hq, hkv, d, 3, state), gos)
     for gw, w in zip(got_w, ws, strict=True):
         _close(w.grad - 1, 0.5 * gw.cpu())
+
+
+@pytest.mark.parametrize("t,h,f", [(300, 512, 1024), (129, 256, 640)])
+def test_gate_up_swiglu_matches_separate_projections(t, h, f):
+    """One merged gate/up GEMM + SwiGLU on its two halves == two projections + SwiGLU."""
+    from speculators_amd import gemm
+    from speculators_amd.fused_ops import swiglu
+
+    g = torch.Generator().manual_seed(t + f)
+    x = torch.randn(1, t, h, generator=g).bfloat16().cuda().requires_grad_(True)
+    wg = (torch.randn(f, h, generator=g) * 0.05).bfloat16().cuda().requires_grad_(True)
+    wu = (torch.randn(f, h, generator=g) * 0.05).bfloat16().cuda().requires_grad_(True)
+    go = torch.randn(1, t, f, generator=g).bfloat16().cuda()
+    state = gemm._MergedWeights()
+    out = gemm.gate_up_swiglu(x, wg, wu, state)
+    out.backward(go)
+    got = [x.grad.clone(), wg.grad.clone(), wu.grad.clone()]
+    assert wg.grad.data_ptr() == state.grad.data_ptr()
+    x.grad = wg.grad = wu.grad = None
+    ref = swiglu(torch.nn.functional.linear(x, wg), torch.nn.functional.linear(x, wu))
+    ref.backward(go)
+    _close(out, ref.detach().cpu(), rel=1e-2)
+    for a, b in zip(got, (x.grad, wg.grad, wu.grad), strict=True):
+        _close(a, b.cpu())
