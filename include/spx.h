@@ -308,7 +308,10 @@ int spx_add_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weight, const v
  *   inverse == 0: out[h, t, :] = rope(x[t, h*D : (h+1)*D], position_ids[t] + position_offset)
  *   inverse != 0: out[t, h*D : (h+1)*D] = rope^T(x[h, t, :], ...)   (its backward)
  * rotate == 0 only relayouts (V).  inv_freq: f32 [D/2].  Half-split rotation,
- * cos/sin evaluated in fp32 and rounded to bf16 like the HF rotary module. */
+ * cos/sin evaluated in fp32 and rounded to bf16 like the HF rotary module.
+ * The stride argument of the head-major side (ld_out when inverse == 0, ld_x otherwise) is
+ * its HEAD stride in elements, 0 meaning T * D: the head-major tensor may be a window of a
+ * longer K/V cache [heads, steps * T, D] (DynamicCache.update without the copy). */
 int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* position_ids,
                       const float* inv_freq, void* out, int64_t ld_out, int64_t T,
                       int32_t heads, int32_t D, int32_t rotate, int32_t inverse,

@@ -113,6 +113,86 @@ class _TTTAttention(torch.autograd.Function):
         return dq, dk, dv, None, None
 
 
+class TTTKVCache:
+    """K / V of all TTT steps of one layer in ONE preallocated buffer ``[1, Hkv, steps * T, D]``
+    (step j's keys are rows ``j*T .. j*T+T-1``: the layout ``DynamicCache.update`` builds by
+    concatenation, models/eagle3/core.py:283-300, without the growing copies).  ``window(j)``
+    is where step j's projection writes; the kernels read rows ``[0, (j+1) * T)``."""
+
+    def __init__(self, hkv: int, t: int, d: int, steps: int, device):
+        self.t, self.steps = t, steps
+        self.k = torch.empty(1, hkv, steps * t, d, device=device, dtype=torch.bfloat16)
+        self.v = torch.empty(1, hkv, steps * t, d, device=device, dtype=torch.bfloat16)
+        self.k_parts: list = []
+        self.v_parts: list = []
+
+    def window(self, j: int):
+        lo = j * self.t
+        return self.k[:, :, lo:lo + self.t], self.v[:, :, lo:lo + self.t]
+
+
+class _TTTAttentionCached(torch.autograd.Function):
+    """TTT attention over a ``TTTKVCache``: the per-step key / value tensors (windows of the
+    cache, already written) are the differentiable inputs, the kernels read the cache in place and
+    the backward hands every step the matching window of the full dK / dV."""
+
+    @staticmethod
+    def forward(ctx, q, mask: TTTMask, scaling: float, cache: TTTKVCache, n_parts: int, *parts):
+        t = cache.t
+        k = cache.k[:, :, :n_parts * t]
+        v = cache.v[:, :, :n_parts * t]
+        hq, hkv, t, d = _check_qkv(q, k, v, mask)
+        q = q.contiguous()
+        dev = q.device
+        out = torch.empty(1, t, hq, d, device=dev, dtype=torch.bfloat16)
+        lse = torch.empty(hq, t, device=dev, dtype=torch.float32)
+        ws = torch.empty(_workspace_bytes(t, hq, hkv, d, False), device=dev, dtype=torch.uint8)
+        _lib.call("spx_ttt_attn_fwd", _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1),
+                  _lib.ptr(v), v.stride(1), _lib.ptr(mask.row_lo), t, mask.ttt_step, hq, hkv, d,
+                  float(scaling), _lib.ptr(out), _lib.ptr(lse), _lib.ptr(ws), ws.numel(),
+                  _lib.stream_ptr(dev))
+        ctx.save_for_backward(q, out, lse)
+        ctx.kv = (k, v)  # windows of the cache: later steps only write rows beyond them
+        ctx.mask, ctx.scaling, ctx.n_parts = mask, float(scaling), n_parts
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, out, lse = ctx.saved_tensors
+        k, v = ctx.kv
+        mask, n = ctx.mask, ctx.n_parts
+        _, hq, t, d = q.shape
+        hkv = k.shape[1]
+        dev = q.device
+        dout = dout.to(torch.bfloat16).contiguous()
+        dq = torch.empty_like(q)
+        dk = torch.empty(1, hkv, n * t, d, device=dev, dtype=torch.bfloat16)
+        dv = torch.empty(1, hkv, n * t, d, device=dev, dtype=torch.bfloat16)
+        ws = torch.empty(_workspace_bytes(t, hq, hkv, d, True), device=dev, dtype=torch.uint8)
+        _lib.call("spx_ttt_attn_bwd", _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1),
+                  _lib.ptr(v), v.stride(1), _lib.ptr(out), _lib.ptr(dout), _lib.ptr(lse),
+                  _lib.ptr(mask.row_lo), t, mask.ttt_step, hq, hkv, d, ctx.scaling,
+                  _lib.ptr(dq), dq.stride(1), _lib.ptr(dk), dk.stride(1), _lib.ptr(dv),
+                  dv.stride(1), _lib.ptr(ws), ws.numel(), _lib.stream_ptr(dev))
+        dks = [dk[:, :, i * t:(i + 1) * t] for i in range(n)]
+        dvs = [dv[:, :, i * t:(i + 1) * t] for i in range(n)]
+        return (dq, None, None, None, None, *dks, *dvs)
+
+
+def ttt_attention_cached(q, k_new, v_new, cache: TTTKVCache, mask: TTTMask,
+                         scaling: float | None = None) -> torch.Tensor:
+    """TTT attention of the step whose keys / values ``k_new`` / ``v_new`` (the windows
+    ``cache.window(step)``, already written) were just appended; ``[1, T, Hq, D]`` (bf16)."""
+    if scaling is None:
+        scaling = q.shape[-1] ** -0.5
+    cache.k_parts.append(k_new)
+    cache.v_parts.append(v_new)
+    n = len(cache.k_parts)
+    if n != mask.ttt_step + 1:
+        raise ValueError(f"the cache holds {n} steps but the mask is at TTT step {mask.ttt_step}")
+    return _TTTAttentionCached.apply(q, mask, scaling, cache, n, *cache.k_parts, *cache.v_parts)
+
+
 def ttt_attention(q, k, v, mask: TTTMask, scaling: float | None = None) -> torch.Tensor:
     """``[1, Hq, T, D]`` x ``[1, Hkv, (step+1)*T, D]`` -> ``[1, T, Hq, D]`` (bf16)."""
     if scaling is None:

@@ -212,8 +212,11 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
   const int h = (int)((item / per_row) % heads);
   const int t = (int)(item / ((int64_t)per_row * heads));
   const int half = D / 2;
-  const uint16_t* src = INVERSE ? x + ((int64_t)h * T + t) * D : x + (int64_t)t * ld_x + h * D;
-  uint16_t* dst = INVERSE ? out + (int64_t)t * ld_out + h * D : out + ((int64_t)h * T + t) * D;
+  // the head-major side is [heads][T][D] with a head stride of its own (0 = T * D, contiguous):
+  // it may be a window of a longer key / value cache
+  const int64_t hs = INVERSE ? (ld_x ? ld_x : (int64_t)T * D) : (ld_out ? ld_out : (int64_t)T * D);
+  const uint16_t* src = INVERSE ? x + (int64_t)h * hs + (int64_t)t * D : x + (int64_t)t * ld_x + h * D;
+  uint16_t* dst = INVERSE ? out + (int64_t)t * ld_out + h * D : out + (int64_t)h * hs + (int64_t)t * D;
   float a[8], b[8], oa[8], ob[8];
   unpack8f(*reinterpret_cast<const u32x4*>(src + d0), a);
   unpack8f(*reinterpret_cast<const u32x4*>(src + half + d0), b);
@@ -403,8 +406,13 @@ extern "C" int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* pos
   SPX_REQUIRE(T > 0 && heads > 0 && D > 0 && D % 16 == 0, "T, heads > 0 and D a multiple of 16");
   SPX_REQUIRE(x && out && (!rotate || (position_ids && inv_freq)), "null buffer");
   SPX_REQUIRE(al16(x) && al16(out), "buffers must be 16-byte aligned");
-  if (inverse) SPX_REQUIRE(ld_out % 8 == 0 && ld_out >= (int64_t)heads * D, "bad output row stride");
-  else SPX_REQUIRE(ld_x % 8 == 0 && ld_x >= (int64_t)heads * D, "bad input row stride");
+  if (inverse) {
+    SPX_REQUIRE(ld_out % 8 == 0 && ld_out >= (int64_t)heads * D, "bad output row stride");
+    SPX_REQUIRE(ld_x == 0 || (ld_x % 8 == 0 && ld_x >= T * D), "bad head stride of the head-major input");
+  } else {
+    SPX_REQUIRE(ld_x % 8 == 0 && ld_x >= (int64_t)heads * D, "bad input row stride");
+    SPX_REQUIRE(ld_out == 0 || (ld_out % 8 == 0 && ld_out >= T * D), "bad head stride of the head-major output");
+  }
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const int64_t total = T * heads * (D / 16);
   const unsigned grid = (unsigned)((total + 255) / 256);

@@ -93,9 +93,17 @@ class Attention(nn.Module):
             pos = position_ids.reshape(-1)
             if pos.dtype != torch.int64:
                 pos = pos.to(torch.int64)
+            kvc = cache.get("kv")
+            if kvc is None and cache.get("steps") and self.attn_fn is A.ttt_hip_attention_forward:
+                # all TTT steps' keys / values of this layer in one buffer, written in place
+                kvc = cache["kv"] = A.TTTKVCache(self.hkv, t, self.d, cache["steps"], x.device)
             q, k, v = gemm.qkv_rope(x, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight,
                                     pos.contiguous(), inv_freq, self.hq, self.hkv, self.d, pos_offset,
-                                    self._merged_qkv)
+                                    self._merged_qkv,
+                                    kv_out=None if kvc is None else kvc.window(pos_offset))
+            if kvc is not None:
+                out = A.ttt_attention_cached(q, k, v, kvc, mask, self.scaling)
+                return gemm.linear_accumulate(out.reshape(1, t, self.hq * self.d), self.o_proj.weight)
         else:
             q = lin(x, self.q_proj.weight)
             k = lin(x, self.k_proj.weight)
@@ -299,7 +307,7 @@ class Eagle3DraftModel(nn.Module):
                             else torch.ones(1, t, device=device, dtype=torch.bool))
             metrics: dict = {}
 
-        caches = [dict() for _ in self.layers]
+        caches = [{"steps": ttt_steps} for _ in self.layers]
         stats_cache: dict = {}
         inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device, cfg.rope_scaling)
         position_ids = position_ids.reshape(-1).to(torch.int64).contiguous()

@@ -167,7 +167,7 @@ class _QKVRope(torch.autograd.Function):
     accumulates across TTT steps."""
 
     @staticmethod
-    def forward(ctx, x, wq, wk, wv, position_ids, inv_freq, hq, hkv, d, offset, state):
+    def forward(ctx, x, wq, wk, wv, position_ids, inv_freq, hq, hkv, d, offset, state, kv_out=None):
         t = x.shape[-2]
         x2 = x.reshape(t, x.shape[-1])
         wcat = state.merged_weight((wq, wk, wv))
@@ -175,11 +175,17 @@ class _QKVRope(torch.autograd.Function):
         n = qkv.shape[1]
         st = _lib.stream_ptr(x.device)
         outs, col = [], 0
-        for heads, rotate in ((hq, 1), (hkv, 1), (hkv, 0)):
-            out = torch.empty(1, heads, t, d, device=x.device, dtype=torch.bfloat16)
+        for idx, (heads, rotate) in enumerate(((hq, 1), (hkv, 1), (hkv, 0))):
+            if idx and kv_out is not None:
+                # a [1, Hkv, T, D] window of the preallocated K / V cache: written in place
+                out = kv_out[idx - 1]
+                head_stride = out.stride(1)
+            else:
+                out = torch.empty(1, heads, t, d, device=x.device, dtype=torch.bfloat16)
+                head_stride = 0
             part = qkv[:, col:]
             _lib.call("spx_rope_relayout", _lib.ptr(part), n, _lib.ptr(position_ids), _lib.ptr(inv_freq),
-                      _lib.ptr(out), 0, t, heads, d, rotate, 0, int(offset), st)
+                      _lib.ptr(out), head_stride, t, heads, d, rotate, 0, int(offset), st)
             outs.append(out)
             col += heads * d
         ctx.save_for_backward(x2, wq, wk, wv, position_ids, inv_freq)
@@ -200,24 +206,29 @@ class _QKVRope(torch.autograd.Function):
             if g is None:
                 dqkv[:, col:col + heads * d].zero_()
             else:
-                g = g.to(torch.bfloat16).contiguous()
-                _lib.call("spx_rope_relayout", _lib.ptr(g), 0, _lib.ptr(position_ids), _lib.ptr(inv_freq),
-                          _lib.ptr(part), n, t, heads, d, rotate, 1, int(offset), st)
+                g = g.to(torch.bfloat16)
+                # a window of a longer gradient tensor is read in place through its head stride
+                if not (g.stride(3) == 1 and g.stride(2) == d and g.stride(1) % 8 == 0
+                        and g.stride(1) >= t * d and g.data_ptr() % 16 == 0):
+                    g = g.contiguous()
+                _lib.call("spx_rope_relayout", _lib.ptr(g), g.stride(1), _lib.ptr(position_ids),
+                          _lib.ptr(inv_freq), _lib.ptr(part), n, t, heads, d, rotate, 1, int(offset), st)
             col += heads * d
         dx = None
         if ctx.needs_input_grad[0]:
             dx = torch.matmul(dqkv, wcat).view(shape)
         if any(w.requires_grad for w in (wq, wk, wv)):
             state.accumulate((wq, wk, wv), dqkv, x2)
-        return (dx,) + (None,) * 10
+        return (dx,) + (None,) * 11
 
 
 def qkv_rope(x, wq, wk, wv, position_ids, inv_freq, hq: int, hkv: int, d: int, offset: int,
-             state: _MergedWeights):
+             state: _MergedWeights, kv_out=None):
     """``(q [1,Hq,T,D], k [1,Hkv,T,D], v [1,Hkv,T,D])`` with the rotary embedding at
     ``position_ids + offset`` applied to q and k.  Weight gradients land in ``.grad`` during
-    ``backward()`` (like ``linear_accumulate``)."""
-    return _QKVRope.apply(x, wq, wk, wv, position_ids, inv_freq, hq, hkv, d, offset, state)
+    ``backward()`` (like ``linear_accumulate``).  ``kv_out = (k_window, v_window)``: write k and v
+    straight into these ``[1, Hkv, T, D]`` windows of a K / V cache and return them."""
+    return _QKVRope.apply(x, wq, wk, wv, position_ids, inv_freq, hq, hkv, d, offset, state, kv_out)
 
 
 _MergedQKV = _MergedWeights
