@@ -67,7 +67,7 @@ def parse_args():
                          "(the reference's forward contract); logits: full-vocab verifier "
                          "logits gathered through d2t")
     ap.add_argument("--cpu-baseline", choices=["sample", "off"], default="sample")
-    ap.add_argument("--cpu-seq-len", type=int, default=512)
+    ap.add_argument("--cpu-seq-len", type=int, default=1024)
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline timing")
     ap.add_argument("--only-kernels", action="store_true",
                     help="run only the per-kernel timing loops (for rocprofv3 counter runs)")
