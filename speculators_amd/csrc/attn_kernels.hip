@@ -210,6 +210,18 @@ __device__ __forceinline__ void load_bounds(const AttnParams& p, const int (&ic)
 // One workgroup = 4 waves = 4 * 32 * NSB query rows of one head.  With NSB = 2 a
 // wave owns two 32-row sub-blocks, so every K / V^T fragment read from LDS
 // feeds two MFMAs (LDS bandwidth, not the matrix core, bounds NSB = 1).
+// wave priority around the MFMA clusters: with two waves on a SIMD the arbiter then prefers the
+// wave that is in its matrix phase and fills the gaps with the other wave's vector work
+#ifndef SPX_PRIO
+#define SPX_PRIO 1
+#endif
+#if SPX_PRIO
+#define SPX_PRIO_MFMA() __builtin_amdgcn_s_setprio(3)
+#define SPX_PRIO_VALU() __builtin_amdgcn_s_setprio(0)
+#else
+#define SPX_PRIO_MFMA()
+#define SPX_PRIO_VALU()
+#endif
 #ifndef SPX_FWD_MINB
 #define SPX_FWD_MINB 2
 #endif
@@ -337,6 +349,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) st[sb][kb][r] = 0.f;
+      SPX_PRIO_MFMA();
       // K fragments go through a ring of four registers: the read of fragment f + 4 is
       // issued right after the MFMA of fragment f, so no MFMA waits for LDS; the two
       // 32-key halves alternate so that consecutive MFMAs use different accumulators
@@ -360,6 +373,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         }
         __builtin_amdgcn_sched_barrier(0);
       }
+      SPX_PRIO_VALU();
       const bool need_mask = (n0 < w_amax) || (n0 + kBN > w_bmin);
       int m_lo[NSB], m_hi[NSB];
 #pragma unroll
@@ -408,6 +422,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         }
         m_run[sb] = m_new;
       }
+      SPX_PRIO_MFMA();
       {
         // V^T fragments through the same kind of ring; fragment f = (16-key step s, D block db)
         constexpr int NF = 4 * NDB;
@@ -434,6 +449,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         }
         __builtin_amdgcn_sched_barrier(0);
       }
+      SPX_PRIO_VALU();
     }
   };
 
@@ -690,6 +706,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
           for (int r = 0; r < 16; ++r) { st[r] = 0.f; dp[r] = 0.f; }
           // K and V fragments alternate through a ring of four registers (fragment 2 kk is
           // K, 2 kk + 1 is V): the read of fragment f + 4 follows the MFMA of fragment f
+          SPX_PRIO_MFMA();
           {
             constexpr int NF = 2 * NKK;
             bf16x8 fr[4];
@@ -710,6 +727,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
             }
             __builtin_amdgcn_sched_barrier(0);
           }
+          SPX_PRIO_VALU();
 #pragma unroll
           for (int r = 0; r < 16; ++r) st[r] = fast_exp2(fmaf(st[r], p.scale_log2e, -lse_i[sb]));
           if (need_mask) {
@@ -724,6 +742,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
           }
 #pragma unroll
           for (int r = 0; r < 16; ++r) dp[r] = st[r] * (dp[r] - delta_i[sb]);
+          SPX_PRIO_MFMA();
           {
             // K^T fragments through the same kind of ring; fragment f = (16-key step s2, D block db)
             constexpr int NF = 2 * NDB;
@@ -745,6 +764,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
             }
             __builtin_amdgcn_sched_barrier(0);
           }
+          SPX_PRIO_VALU();
         }
       }
     }
