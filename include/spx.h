@@ -342,6 +342,18 @@ int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb,
                      void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
                      void* stream);
 
+/* c[M, N] (+)= a[T, M]^T * b[T, N], bf16 inputs, fp32 accumulation, bf16 output:
+ * the weight-gradient product of the backward of torch.nn.Linear (dW = dY^T X)
+ * for every Linear of the draft layers (models/eagle3/core.py:76,244 and the
+ * q/k/v/o/gate/up/down projections of the decoder layer, model_definitions.py).
+ * accumulate != 0 adds the product to what c holds (one rounding to bf16 of
+ * old + product): the weights are applied once per TTT step and their gradients
+ * sum over the steps (models/eagle3/core.py:289-345).  M, N, lda, ldb multiples
+ * of 8; a and b 16-byte aligned; each operand spans less than 2 GiB. */
+int spx_gemm_bf16_tn(const void* a, int64_t lda, const void* b, int64_t ldb,
+                     void* c, int64_t ldc, int64_t M, int64_t N, int64_t T,
+                     int accumulate, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

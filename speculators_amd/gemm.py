@@ -48,6 +48,37 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -
     return out
 
 
+def gemm_tn(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
+            accumulate: bool = False) -> torch.Tensor:
+    """``a[T, M].T @ b[T, N] -> [M, N]`` (bf16, fp32 accumulation): the weight gradient
+    ``dY.T @ X`` of a Linear.  ``accumulate`` adds the product to ``out``."""
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
+        raise _lib.SpxError("gemm_tn takes bf16 operands")
+    if a.dim() != 2 or b.dim() != 2 or a.shape[0] != b.shape[0]:
+        raise ValueError(f"shape mismatch: a {tuple(a.shape)} b {tuple(b.shape)}")
+    if a.stride(1) != 1:
+        a = a.contiguous()
+    if b.stride(1) != 1:
+        b = b.contiguous()
+    t, m = a.shape
+    n = b.shape[1]
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate needs the tensor to add to")
+        out = torch.empty(m, n, device=a.device, dtype=torch.bfloat16)
+    elif out.shape != (m, n) or out.dtype != torch.bfloat16 or out.stride(1) != 1:
+        raise ValueError(f"out must be a bf16 [{m}, {n}] tensor with unit column stride")
+    # 32-bit byte offsets inside the kernel: a contraction that spans 2 GiB or more of an
+    # operand is fed in bands of rows, every band after the first added to the result
+    rows = max(_MAX_SPAN // (2 * max(a.stride(0), b.stride(0))) - 256, 1)
+    st = _lib.stream_ptr(a.device)
+    for t0 in range(0, t, rows):
+        at, bt = a[t0:t0 + rows], b[t0:t0 + rows]
+        _lib.call("spx_gemm_bf16_tn", _lib.ptr(at), at.stride(0), _lib.ptr(bt), bt.stride(0),
+                  _lib.ptr(out), out.stride(0), m, n, at.shape[0], int(accumulate or t0 > 0), st)
+    return out
+
+
 class _Linear(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, weight_t):

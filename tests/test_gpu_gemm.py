@@ -75,3 +75,73 @@ def test_full_size_lm_head_shape_sampled_and_linear():
     assert (c_sum[rows].float() - want_s).abs().max() <= 2 ** -8 * want_s.abs().max() + 1e-3
     # identical inputs give identical bits (fixed reduction order)
     assert torch.equal(c, gemm_nt(a, b))
+
+
+@pytest.mark.parametrize("t,m,n", [(64, 256, 256), (72, 8, 8), (1, 16, 24), (200, 264, 520),
+                                   (129, 40, 1000), (4096, 512, 256), (257, 776, 392)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_gemm_tn_matches_fp32_reference(t, m, n, accumulate):
+    """The weight-gradient product dY^T X, plain and added to what the output holds: tile
+    edges in all three dimensions, a contraction shorter than one slab, odd slab counts."""
+    from speculators_amd.gemm import gemm_tn
+
+    g = torch.Generator().manual_seed(t + m + n)
+    a = torch.randn(t, m, generator=g).bfloat16()
+    b = torch.randn(t, n, generator=g).bfloat16()
+    ref = a.float().T @ b.float()
+    if accumulate:
+        c0 = (torch.randn(m, n, generator=g) * 30).bfloat16()
+        ref = ref + c0.float()
+        got = gemm_tn(a.cuda(), b.cuda(), c0.cuda(), accumulate=True).float().cpu()
+    else:
+        got = gemm_tn(a.cuda(), b.cuda()).float().cpu()
+    # one rounding to bf16 of the fp32 result
+    assert (got - ref).abs().max() <= 2 ** -8 * ref.abs().max() + 1e-3
+
+
+def test_gemm_tn_strided_operands_and_output():
+    from speculators_amd.gemm import gemm_tn
+
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(300, 272, generator=g).bfloat16().cuda()[:, :264]
+    b = torch.randn(300, 144, generator=g).bfloat16().cuda()[:, 8:144]
+    out_full = torch.full((264, 200), 7.0, dtype=torch.bfloat16, device="cuda")
+    out = out_full[:, 32:168]
+    gemm_tn(a, b, out)
+    ref = a.float().T @ b.float()
+    assert (out.float() - ref).abs().max() <= 2 ** -8 * ref.abs().max() + 1e-3
+    # nothing outside the view was touched
+    assert (out_full[:, :32] == 7).all() and (out_full[:, 168:] == 7).all()
+
+
+def test_gemm_tn_matches_library_on_a_layer_shape():
+    """The o_proj weight gradient of the 8B draft layer (T = 4096, 4096 x 4096): sampled rows
+    against fp32, repeatability, and accumulation over two calls against one fp32 sum."""
+    from speculators_amd.gemm import gemm_tn
+
+    g = torch.Generator(device="cuda").manual_seed(11)
+    dy = torch.randn(4096, 4096, device="cuda", generator=g).bfloat16()
+    x = torch.randn(4096, 4096, device="cuda", generator=g).bfloat16()
+    c = gemm_tn(dy, x)
+    rows = torch.tensor([0, 255, 256, 1000, 4095], device="cuda")
+    want = dy[:, rows].float().t() @ x.float()
+    assert (c[rows].float() - want).abs().max() <= 2 ** -8 * want.abs().max() + 1e-3
+    assert torch.equal(c, gemm_tn(dy, x))
+    acc = c.clone()
+    gemm_tn(dy, x, acc, accumulate=True)
+    want2 = c[rows].float() + want
+    assert (acc[rows].float() - want2).abs().max() <= 2 ** -8 * want2.abs().max() + 1e-3
+
+
+def test_gemm_tn_rejects_bad_arguments():
+    from speculators_amd import _lib
+    from speculators_amd.gemm import gemm_tn
+
+    a = torch.zeros(16, 12, dtype=torch.bfloat16, device="cuda")  # M not a multiple of 8
+    b = torch.zeros(16, 8, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_lib.SpxError):
+        gemm_tn(a, b)
+    with pytest.raises(ValueError):
+        gemm_tn(b, torch.zeros(8, 8, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        gemm_tn(b, b, accumulate=True)
