@@ -231,13 +231,27 @@ __device__ __forceinline__ void load_bounds(const AttnParams& p, const int (&ic)
 #ifndef SPX_DKV_MINB
 #define SPX_DKV_MINB 1
 #endif
-template <int D, int NSB, int NW, bool PF>
+// How the forward kernel brings a key tile into LDS: through registers at the point of use (0),
+// through registers one tile ahead (1), or with global -> LDS loads into the other of two tile
+// buffers (2).  A 16-byte LDS write from registers holds the LDS pipe twice as long as a 16-byte
+// read, and these kernels keep that pipe busy all the time: mode 2 takes the writes off it.
+template <int D, int NW, int PF>
+struct FwdSmem {
+  static constexpr int KS = D + kKPad, VS = kBN + kVPad;
+  static constexpr int kTileK = kBN * D * 2, kTileV = D * kBN * 2;  // mode 2: unpadded, swizzled
+  static constexpr int kBuf = kTileK + kTileV;
+  static constexpr int kTiles = PF == 2 ? 2 * kBuf : (kBN * KS + D * VS) * 2;
+  static constexpr int kBytes = kTiles + 4 * NW * (int)sizeof(int);
+};
+
+template <int D, int NSB, int NW, int PF>
 __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_kernel(AttnParams p,
                                                                 const uint16_t* __restrict__ Vt,
                                                                 uint16_t* __restrict__ O,
                                                                 float* __restrict__ LSE) {
-  constexpr int KS = D + kKPad;
-  constexpr int VS = kBN + kVPad;
+  using SM = FwdSmem<D, NW, PF>;
+  constexpr int KS = SM::KS;
+  constexpr int VS = SM::VS;
   constexpr int NKK = D / 16;
   constexpr int NDB = D / 32;
   constexpr int NT = 64 * NW;
@@ -245,9 +259,10 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
   constexpr int BMW = 32 * NSB;
   constexpr int BM = NW * BMW;
 
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[kBN * KS];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[D * VS];
-  __shared__ int red[4 * NW];
+  extern __shared__ __attribute__((aligned(16))) uint8_t fwd_smem[];
+  uint16_t* const Ks = reinterpret_cast<uint16_t*>(fwd_smem);
+  uint16_t* const Vs = Ks + kBN * KS;
+  int* const red = reinterpret_cast<int*>(fwd_smem + SM::kTiles);
 
   const int group = p.Hq / p.Hkv;
   const int L = blockIdx.x;
@@ -329,17 +344,74 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
     }
   };
 
+  // ---- mode 2: tiles as 1 KB wave loads global -> LDS.  K tile: rows of D * 2 bytes, V^T tile: rows
+  // of 128 bytes; the 16-byte chunk c of row r lives in slot c ^ swz(r), which makes the fragment
+  // reads (32 lanes = 32 rows, one logical chunk) conflict free without padding.
+  constexpr int RBK = D * 2, CKK = RBK / 16;             // bytes and chunks per K row
+  constexpr int LPK = (kBN * RBK / 1024) / NW;           // wave loads per wave: K tile
+  constexpr int LPV = (D * 128 / 1024) / NW;             // V^T tile
+  auto swz_k = [](int r) { return CKK == 8 ? (r >> 1) & 7 : r & 15; };
+  auto swz_v = [](int r) { return (r >> 1) & 7; };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)fwd_smem;
+  u32x4 kres, vres;
+  int k_row[PF == 2 ? LPK : 1], k_col[PF == 2 ? LPK : 1], v_off[PF == 2 ? LPV : 1];
+  if constexpr (PF == 2) {
+    kres = make_rsrc(Kh, (uint32_t)((int64_t)p.NKV * RBK));
+    vres = make_rsrc(Vth, (uint32_t)((int64_t)D * p.NKVp * 2));
+#pragma unroll
+    for (int j = 0; j < LPK; ++j) {
+      const int r = (wave * LPK + j) * (1024 / RBK) + lane / CKK;
+      k_row[j] = r;
+      k_col[j] = ((lane % CKK) ^ swz_k(r)) * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < LPV; ++j) {
+      const int r = (wave * LPV + j) * 8 + lane / 8;
+      v_off[j] = r * p.NKVp * 2 + ((lane & 7) ^ swz_v(r)) * 16;
+    }
+  }
+  auto issue = [&](int n0, int buf) __attribute__((always_inline)) {
+    if constexpr (PF == 2) {
+      const uint32_t kb = lds0 + buf * SM::kBuf + wave * LPK * 1024;
+#pragma unroll
+      for (int j = 0; j < LPK; ++j)
+        load_to_lds16<0>(kres, kb + j * 1024, min(n0 + k_row[j], last_row) * RBK + k_col[j], 0);
+      const uint32_t vb = lds0 + buf * SM::kBuf + SM::kTileK + wave * LPV * 1024;
+#pragma unroll
+      for (int j = 0; j < LPV; ++j) load_to_lds16<0>(vres, vb + j * 1024, v_off[j], n0 * 2);
+    }
+  };
+  // fragment reads of mode 2: byte offsets of this lane's row and chunk (step 0) inside a tile
+  const int rdk = col * RBK + ((g ^ swz_k(col)) * 16);
+  const int rdv = col * 128 + ((g ^ swz_v(col)) * 16);
+
   // one pass over the key tiles of one interval class
   auto run_pass = [&](const int (&aa)[NSB], const int (&bb)[NSB], int w_amin, int w_amax,
                       int w_bmin, int w_bmax, int blk_a, int blk_b) {
     if (blk_b <= blk_a) return;
     const int n_begin = (blk_a / kBN) * kBN;
-    if (PF) fetch(n_begin);
+    if (PF == 1) fetch(n_begin);
+    int buf = 0;
+    if constexpr (PF == 2) {
+      __syncthreads();  // a previous pass may still be reading either buffer
+      issue(n_begin, 0);
+    }
     for (int n0 = n_begin; n0 < blk_b; n0 += kBN) {
-      __syncthreads();
-      if (PF) stash(); else direct(n0);
-      __syncthreads();
-      if (PF && n0 + kBN < blk_b) fetch(n0 + kBN);
+      if constexpr (PF == 2) {
+        // this wave's loads of tile n0 have landed; after the barrier everybody's have, and nobody
+        // reads the other buffer any more: the next tile goes there
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (n0 + kBN < blk_b) issue(n0 + kBN, buf ^ 1);
+      } else {
+        __syncthreads();
+        if (PF) stash(); else direct(n0);
+        __syncthreads();
+        if (PF && n0 + kBN < blk_b) fetch(n0 + kBN);
+      }
+      const uint8_t* const tk = fwd_smem + buf * SM::kBuf;
+      const uint8_t* const tv = tk + SM::kTileK;
+      buf ^= 1;
       if (n0 >= w_bmax || n0 + kBN <= w_amin) continue;  // nothing visible for this wave
 
       f32x16 st[NSB][2];
@@ -357,8 +429,12 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         constexpr int NF = 2 * NKK;
         bf16x8 kfr[4];
         auto kread = [&](int f) {
-          kfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-              &Ks[((f & 1) * 32 + col) * KS + g * 8 + (f >> 1) * 16]));
+          if constexpr (PF == 2)
+            kfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                tk + (f & 1) * 32 * RBK + (rdk ^ ((f >> 1) * 32))));
+          else
+            kfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                &Ks[((f & 1) * 32 + col) * KS + g * 8 + (f >> 1) * 16]));
         };
 #pragma unroll
         for (int f = 0; f < 4; ++f) kread(f);
@@ -428,8 +504,12 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         constexpr int NF = 4 * NDB;
         bf16x8 vfr[4];
         auto vread = [&](int f) {
-          vfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-              &Vs[((f % NDB) * 32 + col) * VS + (f / NDB) * 16 + 8 * g]));
+          if constexpr (PF == 2)
+            vfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                tv + (f % NDB) * 32 * 128 + (rdv ^ ((f / NDB) * 32))));
+          else
+            vfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                &Vs[((f % NDB) * 32 + col) * VS + (f / NDB) * 16 + 8 * g]));
         };
 #pragma unroll
         for (int f = 0; f < 4; ++f) vread(f);
@@ -845,12 +925,29 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
 // accumulator sets and both operand fragments do not fit the register file together, so
 // the kernel is launched once per pass and the scores are recomputed).
 #ifndef SPX_DKV256_PF1
-#define SPX_DKV256_PF1 true
+#define SPX_DKV256_PF1 2
 #endif
 #ifndef SPX_DKV256_PF2
-#define SPX_DKV256_PF2 true
+#define SPX_DKV256_PF2 1
 #endif
-template <int D, int NW, bool PF, int PASS>
+// PF: how the query tiles reach LDS (see FwdSmem): 0 at the point of use, 1 through registers one
+// tile ahead, 2 global -> LDS into the other of two buffers.  A buffer holds the tiles the pass
+// multiplies with: Q always, dO and Q^T for dK, dO^T for dV (at head_dim 256 two buffers of the dK
+// pass's three tiles do not fit the 160 KB of LDS: that pass stays on mode 1).
+template <int D, int PASS>
+struct DkvSmem {
+  static constexpr bool kDoV = PASS != 2, kDoK = PASS != 1;
+  static constexpr int kTileR = 64 * D * 2, kTileT = D * 128;  // Q / dO and Q^T / dO^T tiles, unpadded
+  static constexpr int kOffdO = kTileR;
+  static constexpr int kOffQt = (kDoK ? 2 : 1) * kTileR;
+  static constexpr int kOffdOt = kOffQt + (kDoK ? kTileT : 0);
+  static constexpr int kBuf = kOffdOt + (kDoV ? kTileT : 0);
+  static constexpr int kSmall = 6 * 64 * 4;                     // lse, delta, a1, b1, a2, b2 of 64 rows
+  static constexpr int kBytesDma = 2 * kBuf + 2 * kSmall;
+  static constexpr int kBytes = (2 * 64 * (D + kKPad) + 2 * D * (64 + kVPad)) * 2 + kSmall;
+};
+
+template <int D, int NW, int PF, int PASS>
 __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     AttnParams p, const uint16_t* __restrict__ dO, const uint16_t* __restrict__ Qt,
     const uint16_t* __restrict__ dOt, int NQp, const float* __restrict__ LSE,
@@ -869,7 +966,10 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
   uint16_t* dOs = Qs + 64 * QS;        // [64][QS]
   uint16_t* Qts = dOs + 64 * QS;       // [D][TS]
   uint16_t* dOts = Qts + D * TS;       // [D][TS]
-  float* lse_s = reinterpret_cast<float*>(dOts + D * TS);  // [64]
+  using SM = DkvSmem<D, PASS>;
+  static_assert(PF != 2 || SM::kBytesDma <= 160 * 1024, "two buffers of this pass's tiles do not fit in LDS");
+  uint8_t* const sm8 = reinterpret_cast<uint8_t*>(smem);
+  float* lse_s = reinterpret_cast<float*>(PF == 2 ? sm8 + 2 * SM::kBuf : sm8 + (2 * 64 * QS + 2 * D * TS) * 2);  // [64]
   float* delta_s = lse_s + 64;                               // [64]
   int* a1_s = reinterpret_cast<int*>(delta_s + 64);          // [64] each
   int* b1_s = a1_s + 64;
@@ -930,6 +1030,27 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     return (tile_bounds[qt * 8 + 1] <= n0 && tile_bounds[qt * 8 + 2] >= n0 + KB) ||
            (tile_bounds[qt * 8 + 5] <= n0 && tile_bounds[qt * 8 + 6] >= n0 + KB);
   };
+  // the per-row scalars of a query tile: wave 0 loads them into registers ...
+  auto small_fetch = [&](int mq) {
+    if (tid < 64) {
+      const int ir = mq + tid;
+      const bool ok = ir < p.NQ;
+      lse_r = ok ? LSE[(int64_t)h * p.NQ + ir] : 0.f;
+      delta_r = ok ? Delta[(int64_t)h * p.NQ + ir] : 0.f;
+      a1_r = ok ? p.a1[ir] : 0x7fffffff;
+      b1_r = ok ? (p.b1 ? p.b1[ir] : ir + 1) : 0;
+      a2_r = (ok && p.a2) ? p.T + p.a2[ir] : 0x7fffffff;
+      b2_r = (ok && p.a2) ? p.T + p.b2[ir] : 0;
+    }
+  };
+  // ... and writes them to LDS (set `b` of the six arrays: only the two-buffer mode has a second one)
+  auto small_stash = [&](int b) {
+    if (tid < 64) {
+      const int o = b * (SM::kSmall / 4);
+      lse_s[o + tid] = lse_r; delta_s[o + tid] = delta_r;
+      a1_s[o + tid] = a1_r; b1_s[o + tid] = b1_r; a2_s[o + tid] = a2_r; b2_s[o + tid] = b2_r;
+    }
+  };
   auto fetch = [&](int mq) {
 #pragma unroll
     for (int n = 0; n < CPT; ++n) {
@@ -942,16 +1063,7 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       if (kDoK) qtreg[n] = *reinterpret_cast<const u32x4*>(Qth + (int64_t)td * NQp + mq + tc);
       if (kDoV) dtreg[n] = *reinterpret_cast<const u32x4*>(dOth + (int64_t)td * NQp + mq + tc);
     }
-    if (tid < 64) {
-      const int ir = mq + tid;
-      const bool ok = ir < p.NQ;
-      lse_r = ok ? LSE[(int64_t)h * p.NQ + ir] : 0.f;
-      delta_r = ok ? Delta[(int64_t)h * p.NQ + ir] : 0.f;
-      a1_r = ok ? p.a1[ir] : 0x7fffffff;
-      b1_r = ok ? (p.b1 ? p.b1[ir] : ir + 1) : 0;
-      a2_r = (ok && p.a2) ? p.T + p.a2[ir] : 0x7fffffff;
-      b2_r = (ok && p.a2) ? p.T + p.b2[ir] : 0;
-    }
+    small_fetch(mq);
   };
   auto stash = [&]() {
 #pragma unroll
@@ -964,10 +1076,7 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       if (kDoK) *reinterpret_cast<u32x4*>(&Qts[td * TS + tc]) = qtreg[n];
       if (kDoV) *reinterpret_cast<u32x4*>(&dOts[td * TS + tc]) = dtreg[n];
     }
-    if (tid < 64) {
-      lse_s[tid] = lse_r; delta_s[tid] = delta_r;
-      a1_s[tid] = a1_r; b1_s[tid] = b1_r; a2_s[tid] = a2_r; b2_s[tid] = b2_r;
-    }
+    small_stash(0);
   };
 
   auto direct = [&](int mq) {
@@ -1003,17 +1112,89 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     }
   };
 
+  // ---- two-buffer mode: the four tiles as 1 KB wave loads global -> LDS; chunk c of row r lives in
+  // slot c ^ swz(r) (conflict-free fragment reads without padding)
+  constexpr int RBQ = D * 2, CKQ = RBQ / 16;
+  constexpr int LPR = (64 * RBQ / 1024) / NW, LPT = (D * 128 / 1024) / NW;  // wave loads per wave and tile
+  auto swz_r = [](int r) { return CKQ == 8 ? (r >> 1) & 7 : r & 15; };
+  auto swz_t = [](int r) { return (r >> 1) & 7; };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)sm8;
+  u32x4 qres, dres, qtres, dtres;
+  int r_row[PF == 2 ? LPR : 1], r_col[PF == 2 ? LPR : 1], t_off[PF == 2 ? LPT : 1];
+  if constexpr (PF == 2) {
+    qres = make_rsrc(Qh, (uint32_t)((int64_t)p.NQ * RBQ));
+    dres = make_rsrc(dO + (int64_t)h * D, (uint32_t)((((int64_t)p.NQ - 1) * p.Hq * D + D) * 2));
+    qtres = make_rsrc(Qth, (uint32_t)((int64_t)D * NQp * 2));
+    dtres = make_rsrc(dOth, (uint32_t)((int64_t)D * NQp * 2));
+#pragma unroll
+    for (int j = 0; j < LPR; ++j) {
+      const int r = (wave * LPR + j) * (1024 / RBQ) + lane / CKQ;
+      r_row[j] = r;
+      r_col[j] = ((lane % CKQ) ^ swz_r(r)) * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < LPT; ++j) {
+      const int r = (wave * LPT + j) * 8 + lane / 8;
+      t_off[j] = r * NQp * 2 + ((lane & 7) ^ swz_t(r)) * 16;
+    }
+  }
+  auto issue = [&](int mq, int b) __attribute__((always_inline)) {
+    if constexpr (PF == 2) {
+      const uint32_t rb = lds0 + b * SM::kBuf + wave * LPR * 1024;
+#pragma unroll
+      for (int j = 0; j < LPR; ++j) {
+        const int ir = min(mq + r_row[j], p.NQ - 1);
+        load_to_lds16<0>(qres, rb + j * 1024, ir * RBQ + r_col[j], 0);
+        if (kDoK) load_to_lds16<0>(dres, rb + SM::kOffdO + j * 1024, ir * (p.Hq * RBQ) + r_col[j], 0);
+      }
+      const uint32_t tb2 = lds0 + b * SM::kBuf + wave * LPT * 1024;
+#pragma unroll
+      for (int j = 0; j < LPT; ++j) {
+        if (kDoK) load_to_lds16<0>(qtres, tb2 + SM::kOffQt + j * 1024, t_off[j], mq * 2);
+        if (kDoV) load_to_lds16<0>(dtres, tb2 + SM::kOffdOt + j * 1024, t_off[j], mq * 2);
+      }
+    }
+  };
+  const int rdr = col * RBQ + ((g ^ swz_r(col)) * 16);
+  const int rdt = col * 128 + ((g ^ swz_t(col)) * 16);
+  const float* const lse_s0 = lse_s;
+  const uint8_t* tile = sm8;
+  int buf = 0;
+
   int qt = 0;
   while (qt < n_qt && !visible(qt)) ++qt;
-  if (PF && qt < n_qt) fetch(qt * 64);
+  if (PF == 1 && qt < n_qt) fetch(qt * 64);
+  if (PF == 2 && qt < n_qt) {
+    issue(qt * 64, 0);
+    small_fetch(qt * 64);
+    small_stash(0);
+  }
   while (qt < n_qt) {
     int nxt = qt + 1;
     while (nxt < n_qt && !visible(nxt)) ++nxt;
     const bool full = fully_visible(qt);
-    __syncthreads();
-    if (PF) stash(); else direct(qt * 64);
-    __syncthreads();
-    if (PF && nxt < n_qt) fetch(nxt * 64);
+    if constexpr (PF == 2) {
+      // this wave's loads of the tile have landed; behind the barrier everybody's have, the per-row
+      // scalars written at the end of the last iteration are visible, and the other buffer is free
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (nxt < n_qt) {
+        issue(nxt * 64, buf ^ 1);
+        small_fetch(nxt * 64);
+      }
+      tile = sm8 + buf * SM::kBuf;
+      const int o = buf * (SM::kSmall / 4);
+      lse_s = const_cast<float*>(lse_s0) + o;
+      delta_s = lse_s + 64;
+      a1_s = reinterpret_cast<int*>(delta_s + 64);
+      b1_s = a1_s + 64; a2_s = b1_s + 64; b2_s = a2_s + 64;
+    } else {
+      __syncthreads();
+      if (PF) stash(); else direct(qt * 64);
+      __syncthreads();
+      if (PF && nxt < n_qt) fetch(nxt * 64);
+    }
+    const bool have_next = nxt < n_qt;
     qt = nxt;
 
     // the two 32-row halves of the query tile one after the other (keeps 32 score
@@ -1030,9 +1211,15 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         constexpr int NF = PER * NKK;
         bf16x8 fr[4];
         auto fread = [&](int f) {
-          const uint16_t* base = (PER == 2 && (f & 1)) ? dOs : Qs;
-          fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-              &base[(qb * 32 + col) * QS + g * 8 + (f / PER) * 16]));
+          if constexpr (PF == 2) {
+            const uint8_t* base = tile + ((PER == 2 && (f & 1)) ? SM::kOffdO : 0);
+            fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                base + qb * 32 * RBQ + (rdr ^ ((f / PER) * 32))));
+          } else {
+            const uint16_t* base = (PER == 2 && (f & 1)) ? dOs : Qs;
+            fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                &base[(qb * 32 + col) * QS + g * 8 + (f / PER) * 16]));
+          }
         };
 #pragma unroll
         for (int f = 0; f < 4; ++f) fread(f);
@@ -1088,9 +1275,15 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         auto fread = [&](int f) {
           const int e = f / PER, s2 = e / NDB, db = e % NDB;
           const bool is_q = kDoK && (!kDoV || (f % PER) == 1);
-          const uint16_t* base = is_q ? Qts : dOts;
-          fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-              &base[(db * 32 + col) * TS + (qb * 2 + s2) * 16 + 8 * g]));
+          if constexpr (PF == 2) {
+            const uint8_t* base = tile + (is_q ? SM::kOffQt : SM::kOffdOt);
+            fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                base + db * 32 * 128 + (rdt ^ ((qb * 2 + s2) * 32))));
+          } else {
+            const uint16_t* base = is_q ? Qts : dOts;
+            fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                &base[(db * 32 + col) * TS + (qb * 2 + s2) * 16 + 8 * g]));
+          }
         };
 #pragma unroll
         for (int f = 0; f < 4; ++f) fread(f);
@@ -1110,6 +1303,16 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    if constexpr (PF == 2) {
+      // the per-row scalars of the next tile go into the other set: nobody reads it before the barrier
+      if (have_next) {
+        lse_s = const_cast<float*>(lse_s0); delta_s = lse_s + 64;
+        a1_s = reinterpret_cast<int*>(delta_s + 64); b1_s = a1_s + 64; a2_s = b1_s + 64; b2_s = a2_s + 64;
+        small_stash(buf ^ 1);
+      }
+      buf ^= 1;
+    }
+    (void)have_next;
   }
 
   if (c < p.NKV) {
@@ -1252,7 +1455,7 @@ __global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
 static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 
 #ifndef SPX_FWD_CFG
-#define SPX_FWD_CFG 1, 4, true
+#define SPX_FWD_CFG 1, 4, 2
 #endif
 #ifndef SPX_DQ_CFG
 #define SPX_DQ_CFG 1, 4, false
@@ -1260,22 +1463,24 @@ static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 // head_dim 256: the next tile is prefetched into registers as well; the few registers that
 // spill cost far less than exposing the global-load latency with one workgroup per CU
 #ifndef SPX_FWD256_PF
-#define SPX_FWD256_PF true
+#define SPX_FWD256_PF 2
 #endif
 #ifndef SPX_DQ256_PF
 #define SPX_DQ256_PF true
 #endif
 #ifndef SPX_DKV_CFG
-#define SPX_DKV_CFG 4, true
+#define SPX_DKV_CFG 4, 2
 #endif
 // (sub-blocks per wave, waves per workgroup, register prefetch) of the forward / dQ kernels,
 // (waves per workgroup, register prefetch) of the dK/dV kernel
-constexpr int cfg_nsb(int nsb, int, bool) { return nsb; }
-constexpr int cfg_nw(int, int nw, bool) { return nw; }
-constexpr int cfg_nw(int nw, bool) { return nw; }
-constexpr int kFwdNSB = cfg_nsb(SPX_FWD_CFG), kFwdNW = cfg_nw(SPX_FWD_CFG);
+constexpr int cfg_nsb(int nsb, int, int) { return nsb; }
+constexpr int cfg_nw(int, int nw, int) { return nw; }
+constexpr int cfg_pf(int, int, int pf) { return pf; }
+constexpr int cfg_nw(int nw, int) { return nw; }
+constexpr int cfg_pf(int, int pf) { return pf; }
+constexpr int kFwdNSB = cfg_nsb(SPX_FWD_CFG), kFwdNW = cfg_nw(SPX_FWD_CFG), kFwdPF = cfg_pf(SPX_FWD_CFG);
 constexpr int kDqNSB = cfg_nsb(SPX_DQ_CFG), kDqNW = cfg_nw(SPX_DQ_CFG);
-constexpr int kDkvNW = cfg_nw(SPX_DKV_CFG);
+constexpr int kDkvNW = cfg_nw(SPX_DKV_CFG), kDkvPF = cfg_pf(SPX_DKV_CFG);
 
 static int64_t fwd_workspace_bytes(int64_t NKV, int Hkv, int D) {
   return round_up((int64_t)Hkv * D * round_up(NKV, 128) * 2, 256);
@@ -1299,12 +1504,24 @@ static int launch_fwd(AttnParams p, void* workspace, uint16_t* O, float* lse, hi
                      vt, (int64_t)D * p.NKVp, (int64_t)p.NKVp);
   constexpr int BM = 32 * kFwdNSB * kFwdNW;
   const int n_qb = (p.NQ + BM - 1) / BM;
-  if constexpr (D > 128)
-    hipLaunchKernelGGL((attn_fwd_kernel<D, kFwdNSB, kFwdNW, SPX_FWD256_PF>), dim3((unsigned)(n_qb * p.Hq)),
-                       dim3(64 * kFwdNW), 0, st, p, vt, O, lse);
-  else
-    hipLaunchKernelGGL((attn_fwd_kernel<D, SPX_FWD_CFG>), dim3((unsigned)(n_qb * p.Hq)),
-                       dim3(64 * kFwdNW), 0, st, p, vt, O, lse);
+  constexpr int PF = D > 128 ? (int)SPX_FWD256_PF : kFwdPF;
+  constexpr int smem = FwdSmem<D, kFwdNW, PF>::kBytes;
+  if (PF == 2 && ((int64_t)p.NKV * D * 2 >= (1ll << 31) || (int64_t)D * p.NKVp * 2 >= (1ll << 31))) {
+    last_error() = std::string(fn) + ": keys of one head must span less than 2 GiB";
+    return SPX_ERR_ARG;
+  }
+  static bool attr_set = false;  // one flag per head_dim instantiation
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, kFwdNSB, kFwdNW, PF>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) {
+      last_error() = std::string(fn) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
+      return SPX_ERR_HIP;
+    }
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((attn_fwd_kernel<D, kFwdNSB, kFwdNW, PF>), dim3((unsigned)(n_qb * p.Hq)),
+                     dim3(64 * kFwdNW), smem, st, p, vt, O, lse);
   return check_launch(fn);
 }
 
@@ -1347,10 +1564,15 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
     hipLaunchKernelGGL((attn_bwd_dq_kernel<D, SPX_DQ_CFG>), dim3((unsigned)(n_qb * p.Hq)),
                        dim3(64 * kDqNW), 0, st, p, dOp, kt, lse, delta, dQp, dq_hs);
 
-  const size_t smem = (size_t)(2 * 64 * (D + kKPad) + 2 * D * (64 + kVPad)) * 2 + 64 * 4 * 6;
+  constexpr int kPF = D > 128 ? 1 : kDkvPF;
+  constexpr int kPF1 = SPX_DKV256_PF1, kPF2 = SPX_DKV256_PF2;
+  if ((kPF == 2 || (D > 128 && (kPF1 == 2 || kPF2 == 2))) && (int64_t)p.NQ * p.Hq * D * 2 >= (1ll << 31)) {
+    last_error() = std::string(fn) + ": queries must span less than 2 GiB";
+    return SPX_ERR_ARG;
+  }
   const int n_kb = (p.NKV + 32 * kDkvNW - 1) / (32 * kDkvNW);
   const dim3 kgrid((unsigned)(n_kb * p.Hq)), kblock(64 * kDkvNW);
-  auto set_smem = [&](const void* f) {
+  auto set_smem = [&](const void* f, size_t smem) {
     hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) last_error() = std::string(fn) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
     return e == hipSuccess;
@@ -1358,22 +1580,25 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   static bool attr_set = false;
   if constexpr (D > 128) {
     // one launch per gradient (each loads only the tiles it multiplies with)
+    constexpr size_t smem1 = kPF1 == 2 ? DkvSmem<D, 1>::kBytesDma : DkvSmem<D, 1>::kBytes;
+    constexpr size_t smem2 = kPF2 == 2 ? DkvSmem<D, 2>::kBytesDma : DkvSmem<D, 2>::kBytes;
     if (!attr_set) {
-      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, SPX_DKV256_PF1, 1>)) ||
-          !set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, SPX_DKV256_PF2, 2>)))
+      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF1, 1>), smem1) ||
+          !set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF2, 2>), smem2))
         return SPX_ERR_HIP;
       attr_set = true;
     }
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, SPX_DKV256_PF1, 1>), kgrid, kblock, smem, st, p, dOp, qt,
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF1, 1>), kgrid, kblock, smem1, st, p, dOp, qt,
                        dot, NQp, lse, delta, tb, dkp, dvp);
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, SPX_DKV256_PF2, 2>), kgrid, kblock, smem, st, p, dOp, qt,
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF2, 2>), kgrid, kblock, smem2, st, p, dOp, qt,
                        dot, NQp, lse, delta, tb, dkp, dvp);
   } else {
+    constexpr size_t smem = kPF == 2 ? DkvSmem<D, 0>::kBytesDma : DkvSmem<D, 0>::kBytes;
     if (!attr_set) {
-      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, SPX_DKV_CFG, 0>))) return SPX_ERR_HIP;
+      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF, 0>), smem)) return SPX_ERR_HIP;
       attr_set = true;
     }
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, SPX_DKV_CFG, 0>), kgrid, kblock, smem, st, p, dOp, qt, dot,
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF, 0>), kgrid, kblock, smem, st, p, dOp, qt, dot,
                        NQp, lse, delta, tb, dkp, dvp);
   }
   const int64_t items = (int64_t)p.NKV * D / 4 * p.Hkv;

@@ -60,39 +60,12 @@ constexpr int kOob = 0x7ffffff0;
 static_assert(kABytes == 32768 && kBBytes == 32768, "the buffer toggle flips bit 15");
 static_assert(kLA % 4 == 0 && kLB % 4 == 0, "loads are grouped in fours (immediate offsets)");
 
-// 64 lanes x 16 bytes, global -> LDS at M0 + IMM + 16 * lane; the global address is
-// base + voff + soff + IMM.  Lanes whose voff + IMM lies outside the resource write
-// zeros.  M0 is an input operand: the compiler writes it only when the value changes.
-// The s_nop covers the M0-write -> LDS-DMA wait state for the first load of a group.
-template <int IMM>
-__device__ __forceinline__ void load_to_lds16(u32x4 rsrc, uint32_t lds_addr, int voff, int soff) {
-  if (IMM == 0)
-    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :
-                 : "{m0}"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
-                 : "memory");
-  else
-    asm volatile("buffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds"
-                 :
-                 : "{m0}"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM)
-                 : "memory");
-}
-
 __device__ __forceinline__ bf16x8 as_frag(u32x4 v) {
   union { u32x4 u; bf16x8 b; } c;
   c.u = v;
   return c.b;
 }
 
-__device__ __forceinline__ u32x4 make_rsrc(const void* p, uint32_t bytes) {
-  const uint64_t a = reinterpret_cast<uint64_t>(p);
-  u32x4 r;
-  r.x = __builtin_amdgcn_readfirstlane((uint32_t)a);
-  r.y = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
-  r.z = __builtin_amdgcn_readfirstlane(bytes);
-  r.w = 0x00020000u;
-  return r;
-}
 
 // kImm: consecutive loads of a group of four share one M0 value and differ in the
 // instruction's immediate offset (which moves the LDS and the global address alike, so
