@@ -924,6 +924,9 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
 // PASS 0 computes dK and dV together; PASS 1 only dV, PASS 2 only dK (head_dim 256: the two
 // accumulator sets and both operand fragments do not fit the register file together, so
 // the kernel is launched once per pass and the scores are recomputed).
+#ifndef SPX_DKV_XCD
+#define SPX_DKV_XCD 1
+#endif
 #ifndef SPX_DKV256_PF1
 #define SPX_DKV256_PF1 2
 #endif
@@ -976,9 +979,19 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
   int* a2_s = b1_s + 64;
   int* b2_s = a2_s + 64;
 
-  // heavy key blocks first: under a causal mask the EARLY key blocks are seen by most rows
-  const int h = blockIdx.x % p.Hq;
-  const int kb_idx = blockIdx.x / p.Hq;
+  // Workgroups go to the eight XCDs round robin.  The query-side tiles a workgroup streams belong to
+  // its query head, so the workgroups that share an XCD (and its L2) at a time get the SAME head and
+  // consecutive key blocks: neighbours in that order read the same tile two steps apart.
+  // Heavy key blocks first: under a causal mask the EARLY key blocks are seen by most rows.
+  int h, kb_idx;
+  if (SPX_DKV_XCD && p.Hq % 8 == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, n_kb = gridDim.x / p.Hq;
+    h = xcd + 8 * (slot / n_kb);
+    kb_idx = slot % n_kb;
+  } else {
+    h = blockIdx.x % p.Hq;
+    kb_idx = blockIdx.x / p.Hq;
+  }
   const int kvh = h / (p.Hq / p.Hkv);
   const int n0 = kb_idx * KB;
   const int key_last = min(n0 + KB - 1, p.NKV - 1);
@@ -1161,24 +1174,27 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
   const uint8_t* tile = sm8;
   int buf = 0;
 
-  int qt = 0;
-  while (qt < n_qt && !visible(qt)) ++qt;
-  if (PF == 1 && qt < n_qt) fetch(qt * 64);
-  if (PF == 2 && qt < n_qt) {
-    issue(qt * 64, 0);
-    small_fetch(qt * 64);
+  // (walking the tiles from the last one down, so that every workgroup of a head reads the same tile at
+  // the same time, was slower: 256 workgroups then hit the same few memory channels at once)
+  int qi = 0;
+  while (qi < n_qt && !visible(qi)) ++qi;
+  if (PF == 1 && qi < n_qt) fetch(qi * 64);
+  if (PF == 2 && qi < n_qt) {
+    issue(qi * 64, 0);
+    small_fetch(qi * 64);
     small_stash(0);
   }
-  while (qt < n_qt) {
-    int nxt = qt + 1;
-    while (nxt < n_qt && !visible(nxt)) ++nxt;
+  while (qi < n_qt) {
+    int nxi = qi + 1;
+    while (nxi < n_qt && !visible(nxi)) ++nxi;
+    const int qt = qi, nxt = nxi;
     const bool full = fully_visible(qt);
     if constexpr (PF == 2) {
       // this wave's loads of the tile have landed; behind the barrier everybody's have, the per-row
       // scalars written at the end of the last iteration are visible, and the other buffer is free
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      if (nxt < n_qt) {
+      if (nxi < n_qt) {
         issue(nxt * 64, buf ^ 1);
         small_fetch(nxt * 64);
       }
@@ -1192,10 +1208,10 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       __syncthreads();
       if (PF) stash(); else direct(qt * 64);
       __syncthreads();
-      if (PF && nxt < n_qt) fetch(nxt * 64);
+      if (PF && nxi < n_qt) fetch(nxt * 64);
     }
-    const bool have_next = nxt < n_qt;
-    qt = nxt;
+    const bool have_next = nxi < n_qt;
+    qi = nxi;
 
     // the two 32-row halves of the query tile one after the other (keeps 32 score
     // registers live instead of 64)
