@@ -82,11 +82,44 @@ def test_backward_matches_dense_oracle_autograd(t, hq, hkv, d, docs, window, ste
     ref.backward(go.float())
     for name, got, want in (("dq", qg.grad, qr.grad), ("dk", kg.grad, kr.grad), ("dv", vg.grad, vr.grad)):
         err = (got.float().cpu() - want).abs().max().item()
-        assert err <= 2e-2 * want.abs().max().item(), (name, err, want.abs().max().item())
+        # the absolute floor covers gradients that are exactly zero in exact arithmetic (a query that
+        # sees a single key has dq = 0; the kernel leaves rounding noise of the order of 1e-7 there)
+        assert err <= 2e-2 * want.abs().max().item() + 1e-5, (name, err, want.abs().max().item())
     # the diagonal rows of dk/dv are exactly the per-position gradients: check them apart
     if step > 0:
         err = (kg.grad.float().cpu()[:, :, t:] - kr.grad[:, :, t:]).abs().max().item()
-        assert err <= 2e-2 * kr.grad[:, :, t:].abs().max().item()
+        assert err <= 2e-2 * kr.grad[:, :, t:].abs().max().item() + 1e-5
+
+
+def _random_cases(n, seed):
+    """Seeded shapes that land on every edge of the tiling: sequences shorter than one key tile,
+    one row past a tile, ragged document packs with and without padding, windows shorter and
+    longer than a tile, all three head sizes, several query heads per key head."""
+    import random
+
+    rnd = random.Random(seed)
+    cases = []
+    for _ in range(n):
+        d = rnd.choice([64, 128, 128, 256])
+        t = rnd.choice([1, 2, 31, 33, 63, 64, 65, 127, 129, 191, 257, rnd.randint(3, 400)])
+        hkv = rnd.choice([1, 2])
+        hq = hkv * rnd.choice([1, 2, 4])
+        docs = None
+        if t >= 4 and rnd.random() < 0.6:
+            cuts = sorted(rnd.sample(range(1, t), min(rnd.randint(1, 4), t - 1)))
+            lengths = [b - a for a, b in zip([0] + cuts, cuts + [t])]
+            if rnd.random() < 0.5:
+                lengths = lengths[:-1]  # the tail becomes padding
+            docs = lengths
+        window = rnd.choice([None, None, 1, 5, 64, 100])
+        cases.append((t, hq, hkv, d, docs, window, rnd.randint(1, 3)))
+    return cases
+
+
+@pytest.mark.parametrize("t,hq,hkv,d,docs,window,steps", _random_cases(24, 20240611))
+def test_random_shapes_forward_and_backward(t, hq, hkv, d, docs, window, steps):
+    test_forward_matches_dense_oracle(t, hq, hkv, d, docs, window, steps)
+    test_backward_matches_dense_oracle_autograd(t, hq, hkv, d, docs, window, steps)
 
 
 def _check_sampled_rows(q, k, v, out, go, rows, heads, visible, scale):

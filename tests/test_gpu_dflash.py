@@ -70,7 +70,42 @@ def test_forward_backward_match_dense_oracle(t, hq, hkv, d, docs, anchors, bs, w
     assert err <= 2e-2 * ref.abs().max().item(), err
     for name, got, want in (("dq", qg.grad, qr.grad), ("dk", kg.grad, kr.grad), ("dv", vg.grad, vr.grad)):
         e = (got.float().cpu() - want).abs().max().item()
-        assert e <= 2e-2 * want.abs().max().item(), (name, e, want.abs().max().item())
+        assert e <= 2e-2 * want.abs().max().item() + 1e-5, (name, e, want.abs().max().item())
+
+
+def _random_cases(n, seed):
+    """Seeded anchored-block cases on the edges of the tiling: contexts shorter than one key tile or
+    one row past it, block sizes 1 .. 16, a single anchor, padded anchor lists, windows shorter than a
+    block, all three head sizes."""
+    import random
+
+    rnd = random.Random(seed)
+    cases = []
+    while len(cases) < n:
+        d = rnd.choice([64, 128, 128, 256])
+        bs = rnd.choice([1, 2, 5, 8, 16])
+        t = rnd.choice([33, 64, 65, 130, 257, rnd.randint(bs + 2, 300)])
+        if t <= bs + 1:
+            continue
+        hkv = rnd.choice([1, 2])
+        hq = hkv * rnd.choice([1, 2, 4])
+        cuts = sorted(rnd.sample(range(1, t), min(rnd.randint(0, 3), t - 1)))
+        lengths = [b - a for a, b in zip([0] + cuts, cuts + [t])]
+        if len(lengths) > 1 and rnd.random() < 0.4:
+            lengths = lengths[:-1]  # the tail becomes padding
+        live = min(sum(lengths), t - bs)
+        anchors = sorted(rnd.sample(range(live), min(rnd.randint(1, 12), live)))
+        if rnd.random() < 0.3:
+            anchors += [0] * rnd.randint(1, 3)  # padded anchor slots
+        window = rnd.choice([None, None, 1, 5, 64])
+        cases.append((t, hq, hkv, d, lengths, anchors, bs, window, window is not None and rnd.random() < 0.5))
+    return cases
+
+
+@pytest.mark.parametrize("t,hq,hkv,d,docs,anchors,bs,window,ncf", _random_cases(20, 977))
+def test_random_shapes(t, hq, hkv, d, docs, anchors, bs, window, ncf):
+    test_row_ranges_bit_exact(t, hq, hkv, d, docs, anchors, bs, window, ncf)
+    test_forward_backward_match_dense_oracle(t, hq, hkv, d, docs, anchors, bs, window, ncf)
 
 
 @pytest.mark.parametrize("weighting,sliding", [("fixed-exp-decay", False), ("dpace", True)])
