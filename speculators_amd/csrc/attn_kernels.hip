@@ -222,6 +222,9 @@ __device__ __forceinline__ void load_bounds(const AttnParams& p, const int (&ic)
 #define SPX_PRIO_MFMA()
 #define SPX_PRIO_VALU()
 #endif
+#ifndef SPX_DKV_REMAT
+#define SPX_DKV_REMAT 1
+#endif
 #ifndef SPX_FWD_MINB
 #define SPX_FWD_MINB 2
 #endif
@@ -724,9 +727,13 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
 
   u32x4 kreg[CPT], vreg[CPT], treg[CPT];
   auto fetch = [&](int n0) {
+    // offsets recomputed per tile on purpose (see the dK/dV kernel): kept live through the loop they spill
+    // at head_dim 256, and a spill reload waits for the prefetch issued here
+    int tid_v = tid;
+    if (SPX_DKV_REMAT) asm volatile("" : "+v"(tid_v));
 #pragma unroll
     for (int n = 0; n < CPT; ++n) {
-      const int c = tid + NT * n;
+      const int c = tid_v + NT * n;
       const int krow = c / (D / 8), kcol = (c % (D / 8)) * 8;
       const int kr = min(n0 + krow, last_row);
       kreg[n] = *reinterpret_cast<const u32x4*>(Kh + (int64_t)kr * D + kcol);
@@ -1065,9 +1072,14 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     }
   };
   auto fetch = [&](int mq) {
+    // The per-load row / column offsets are recomputed here on purpose.  Hoisted out of the tile loop they
+    // stay live through it, and at head_dim 256 that is what spills; a spill reload inside the loop waits
+    // for every older vector-memory operation, i.e. for the prefetch this function has just issued.
+    int tid_v = tid;
+    if (SPX_DKV_REMAT) asm volatile("" : "+v"(tid_v));
 #pragma unroll
     for (int n = 0; n < CPT; ++n) {
-      const int ch = tid + NT * n;
+      const int ch = tid_v + NT * n;
       const int qr = ch / (D / 8), qc = (ch % (D / 8)) * 8;
       const int ir = min(mq + qr, p.NQ - 1);
       qreg[n] = *reinterpret_cast<const u32x4*>(Qh + (int64_t)ir * D + qc);
