@@ -443,7 +443,7 @@ def run_mtp(args):
     dl = lg.grad
     del lg, out
     wt = w.detach().t().contiguous()
-    rec("gemm_bf16_nt_kernel[lm_head dX rows x V x H, in row bands below 2 GiB]", "mfma",
+    rec("gemm_bf16_nt_kernel[lm_head dX rows x V x H, all rows]", "mfma",
         2.0 * rows * h * v, time_events(torch, lambda: gemm.gemm_nt(dl, wt), 3), k_steps)
     del dl, logits, wt
     torch.cuda.empty_cache()

@@ -112,6 +112,18 @@ int spx_label_ce_bwd(const void* logits, int64_t ld_logits, const int64_t* label
                      int64_t vocab, int dtype, int64_t ignore_index, void* dlogits,
                      int64_t ld_out, void* stream);
 
+/* The same gradient with the live rows packed to the front: row r is written to
+ * row row_map[r] of dlogits, rows with row_map[r] < 0 are not written at all
+ * (their gradient is zero: ignored label or grad_rows[r] == 0; the caller builds
+ * the map as a running count of the live rows).  Feeds spx_gemm_bf16_nt_rows, which
+ * then skips the dead rows of the lm_head input-gradient product.  No counterpart
+ * in the reference, where that product runs over all rows. */
+int spx_label_ce_bwd_packed(const void* logits, int64_t ld_logits, const int64_t* labels,
+                            const float* lse, const float* grad_rows, int64_t rows,
+                            int64_t vocab, int dtype, int64_t ignore_index,
+                            const int32_t* row_map, void* dlogits, int64_t ld_out,
+                            void* stream);
+
 /* Batch layout producer: packs `n_docs` samples, staged back to back in the layout
  * of the hidden-state files (`src_hs [n_src_rows, layers + 1, hidden]`, bf16 or fp32,
  * with `src_ids [n_src_rows]` int64 and `src_mask [n_src_rows]` of `mask_elem`-byte
@@ -336,11 +348,20 @@ int spx_swiglu_bwd(const void* gate, const void* up, const void* dout, void* dga
  * (models/eagle3/core.py:76,244), the lm_head and verifier_lm_head Linears
  * (model.py:66-69; call sites models/eagle3/core.py:251-253,302-306) and, with
  * b = the transposed weight, the input-gradient product of their backward.
- * lda/ldb/ldc are row strides in elements; K, lda, ldb multiples of 8; each
- * operand spans less than 2 GiB. */
+ * lda/ldb/ldc are row strides in elements; K, lda, ldb multiples of 8; 256 rows
+ * of an operand span less than 2 GiB (the operands themselves may be larger). */
 int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb,
                      void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
                      void* stream);
+
+/* The same product with the number of rows of a (and c) that count read from device
+ * memory at run time: rows >= min(M, *m_live) are neither read nor written.  For an
+ * operand whose producer packs its live rows to the front (spx_label_ce_bwd_packed:
+ * positions with an ignored label have a zero gradient row, models/mtp/core.py:204-216)
+ * without the host learning how many there are.  No counterpart in the reference. */
+int spx_gemm_bf16_nt_rows(const void* a, int64_t lda, const void* b, int64_t ldb,
+                          void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                          const int32_t* m_live, void* stream);
 
 /* c[M, N] (+)= a[T, M]^T * b[T, N], bf16 inputs, fp32 accumulation, bf16 output:
  * the weight-gradient product of the backward of torch.nn.Linear (dW = dY^T X)

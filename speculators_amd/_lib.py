@@ -54,9 +54,11 @@ SIGNATURES["spx_swiglu_fwd"] = [_P, _P, _P, _I64, _P]
 SIGNATURES["spx_swiglu_bwd"] = [_P, _P, _P, _P, _P, _I64, _P]
 SIGNATURES["spx_label_ce_fwd"] = [_P, _I64, _P, _I64, _I64, _I, _I64, _P, _P, _P, _P]
 SIGNATURES["spx_label_ce_bwd"] = [_P, _I64, _P, _P, _P, _I64, _I64, _I, _I64, _P, _I64, _P]
+SIGNATURES["spx_label_ce_bwd_packed"] = [_P, _I64, _P, _P, _P, _I64, _I64, _I, _I64, _P, _P, _I64, _P]
 SIGNATURES["spx_pack_batch"] = [_P, _I, _I64, _I64, _I64, _P, _P, _I, _P, _P, _P, _I64, _I64, _I,
                                 _P, _P, _P, _P, _P, _P, _P]
 SIGNATURES["spx_gemm_bf16_nt"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P]
+SIGNATURES["spx_gemm_bf16_nt_rows"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P, _P]
 SIGNATURES["spx_gemm_bf16_tn"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I, _P]
 RESTYPES = {"spx_ttt_attn_workspace_bytes": c_int64, "spx_dflash_attn_workspace_bytes": c_int64,
             "spx_rmsnorm_bwd_slots": c_int64}

@@ -75,18 +75,26 @@ template <bool kImm>
 __global__ __launch_bounds__(kGemmThreads, SPX_GEMM_MINW)
 __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf16_nt_kernel(
     const uint16_t* __restrict__ A, int64_t lda, const uint16_t* __restrict__ B, int64_t ldb,
-    uint16_t* __restrict__ C, int64_t ldc, int M, int N, int K, int tiles_m, int tiles_n) {
+    uint16_t* __restrict__ C, int64_t ldc, int M, int N, int K, int tiles_m, int tiles_n,
+    const int32_t* __restrict__ m_live) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  // the row count may live on the device (rows packed to the front by the producer of A): the tile
+  // grid shrinks to the rows that count and the workgroups beyond it leave at once
+  if (m_live) {
+    M = min(M, max(*m_live, 0));
+    tiles_m = (M + kTM - 1) / kTM;
+  }
 
-  // workgroup id -> tile: XCD-contiguous bands, then groups of GROUP_M tile rows
+  // workgroup id -> tile: XCD-contiguous bands, then groups of GROUP_M tile rows.  Workgroups go to
+  // the eight XCDs round robin: XCD x gets the ids x, x + 8, ...; they are renumbered so that each XCD
+  // works on one contiguous band of tiles (any grid size: the first n % 8 XCDs get one more)
   const int n_wg = tiles_m * tiles_n;
-  int pid = blockIdx.x;
+  if ((int)blockIdx.x >= n_wg) return;
+  int pid;
   {
-    const int per_xcd = (n_wg + 7) / 8;
-    const int xcd = pid % 8, local = pid / 8;
-    const int cand = xcd * per_xcd + local;
-    // only remap when the grid divides evenly, otherwise keep the identity
-    if (n_wg % 8 == 0) pid = cand;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int base = n_wg >> 3, rem = n_wg & 7;
+    pid = xcd * base + min(xcd, rem) + local;
   }
   constexpr int GROUP_M = SPX_GEMM_GROUP_M;
   const int in_group = GROUP_M * tiles_n;
@@ -114,8 +122,9 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   // One buffer resource per operand; the K position goes into the scalar offset.  Rows
   // past the matrix edge get an offset outside the resource and read as zero, so no
   // clamping or per-lane predicate is needed.
-  const u32x4 ares = make_rsrc(A, (uint32_t)((((int64_t)M - 1) * lda + K) * 2));
-  const u32x4 bres = make_rsrc(B, (uint32_t)((((int64_t)N - 1) * ldb + K) * 2));
+  // (the resources start at the tile's first row: offsets stay below 256 rows whatever the operand's size)
+  const u32x4 ares = make_rsrc(A + (int64_t)m0 * lda, (uint32_t)((((int64_t)min(M - m0, kTM) - 1) * lda + K) * 2));
+  const u32x4 bres = make_rsrc(B + (int64_t)n0 * ldb, (uint32_t)((((int64_t)min(N - n0, kTN) - 1) * ldb + K) * 2));
 
   // global side: wave-load j of this wave covers tile rows wave*8*kLA + 8 j + lane/8; the
   // lane's LDS slot is lane % 8, so it fetches chunk slot ^ f(row)
@@ -128,13 +137,13 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   for (int j = 0; j < kLA; ++j) {
     const int r = wave * (8 * kLA) + j * 8 + lrow;
     const int imm = kImm ? (j & 3) * 8 * kRowBytes : 0;
-    aoff[j] = (m0 + r < M) ? (int)((((int64_t)(m0 + r)) * lda + gchunk[j & 1] * 8) * 2) - imm : kOob;
+    aoff[j] = (m0 + r < M) ? (int)(((int64_t)r * lda + gchunk[j & 1] * 8) * 2) - imm : kOob;
   }
 #pragma unroll
   for (int j = 0; j < kLB; ++j) {
     const int r = wave * (8 * kLB) + j * 8 + lrow;
     const int imm = kImm ? (j & 3) * 8 * kRowBytes : 0;
-    boff[j] = (n0 + r < N) ? (int)((((int64_t)(n0 + r)) * ldb + gchunk[j & 1] * 8) * 2) - imm : kOob;
+    boff[j] = (n0 + r < N) ? (int)(((int64_t)r * ldb + gchunk[j & 1] * 8) * 2) - imm : kOob;
   }
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
   const uint32_t lds_a = lds0 + wave * (8 * kLA) * kRowBytes;
@@ -286,16 +295,17 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
 
 using namespace spx;
 
-extern "C" int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
-                                int64_t ldc, int64_t M, int64_t N, int64_t K, void* stream) {
-  SPX_REQUIRE(M > 0 && N > 0 && K > 0, "M, N, K must be positive");
-  SPX_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "dimension too large");
-  SPX_REQUIRE(a && b && c, "null buffer");
-  SPX_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0, "K, lda, ldb must be multiples of 8");
-  SPX_REQUIRE(lda >= K && ldb >= K && ldc >= N, "leading dimension too small");
-  SPX_REQUIRE(((uintptr_t)a | (uintptr_t)b) % 16 == 0, "a and b must be 16-byte aligned");
-  SPX_REQUIRE(((M - 1) * lda + K) * 2 < 0x7ffffff0ll && ((N - 1) * ldb + K) * 2 < 0x7ffffff0ll,
-              "each operand must span less than 2 GiB (32-bit buffer offsets)");
+#define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fname, what); } while (0)
+static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                        int64_t ldc, int64_t M, int64_t N, int64_t K, const int32_t* m_live, void* stream) {
+  SPX_REQ_FN(M > 0 && N > 0 && K > 0, "M, N, K must be positive");
+  SPX_REQ_FN(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "dimension too large");
+  SPX_REQ_FN(a && b && c, "null buffer");
+  SPX_REQ_FN(K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0, "K, lda, ldb must be multiples of 8");
+  SPX_REQ_FN(lda >= K && ldb >= K && ldc >= N, "leading dimension too small");
+  SPX_REQ_FN(((uintptr_t)a | (uintptr_t)b) % 16 == 0, "a and b must be 16-byte aligned");
+  SPX_REQ_FN((kTM * lda + K) * 2 < 0x7ffffff0ll && (kTN * ldb + K) * 2 < 0x7ffffff0ll,
+             "256 rows of an operand must span less than 2 GiB (32-bit offsets inside a tile)");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool imm = lda >= kTK && ldb >= kTK;
   static bool attr_set[2] = {false, false};
@@ -304,21 +314,37 @@ extern "C" int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64
   if (!attr_set[imm]) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kGemmSmem);
     if (e != hipSuccess) {
-      last_error() = std::string("spx_gemm_bf16_nt: hipFuncSetAttribute: ") + hipGetErrorString(e);
+      last_error() = std::string(fname) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
       return SPX_ERR_HIP;
     }
     attr_set[imm] = true;
   }
   const int tiles_m = (int)((M + kTM - 1) / kTM), tiles_n = (int)((N + kTN - 1) / kTN);
-  SPX_REQUIRE((int64_t)tiles_m * tiles_n < (1ll << 31), "too many tiles");
+  SPX_REQ_FN((int64_t)tiles_m * tiles_n < (1ll << 31), "too many tiles");
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(kGemmThreads);
   if (imm)
     hipLaunchKernelGGL(gemm_bf16_nt_kernel<true>, grid, block, kGemmSmem, st,
                        reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,
-                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n);
+                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live);
   else
     hipLaunchKernelGGL(gemm_bf16_nt_kernel<false>, grid, block, kGemmSmem, st,
                        reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,
-                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n);
-  return check_launch(__func__);
+                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live);
+  return check_launch(fname);
+}
+#undef SPX_REQ_FN
+
+extern "C" int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                                int64_t ldc, int64_t M, int64_t N, int64_t K, void* stream) {
+  return gemm_nt_impl(__func__, a, lda, b, ldb, c, ldc, M, N, K, nullptr, stream);
+}
+
+extern "C" int spx_gemm_bf16_nt_rows(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                                     int64_t ldc, int64_t M, int64_t N, int64_t K,
+                                     const int32_t* m_live, void* stream) {
+  if (!m_live) {
+    last_error() = std::string(__func__) + ": null row count";
+    return SPX_ERR_ARG;
+  }
+  return gemm_nt_impl(__func__, a, lda, b, ldb, c, ldc, M, N, K, m_live, stream);
 }

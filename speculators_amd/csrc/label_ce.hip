@@ -90,17 +90,24 @@ __global__ __launch_bounds__(kLossThreads) void label_ce_fwd_kernel(
 }
 
 // dlogits[r, j] = g[r] * (softmax(x[r])[j] - [j == label[r]]); rows with g == 0 or an ignored
-// label are written as zeros without reading the logits.
+// label are written as zeros without reading the logits.  With a row map the gradient of row r
+// goes to row row_map[r] of the output and rows mapped to -1 are not written at all (the live
+// rows packed to the front: the product that consumes them skips the dead ones).
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kLossThreads) void label_ce_bwd_kernel(
     const T* __restrict__ logits, int64_t ld, const int64_t* __restrict__ labels,
     const float* __restrict__ lse, const float* __restrict__ grad_rows, int64_t vocab,
-    int64_t ignore_index, T* __restrict__ dlogits, int64_t ld_out) {
+    int64_t ignore_index, T* __restrict__ dlogits, int64_t ld_out, const int32_t* __restrict__ row_map) {
   const int64_t r = blockIdx.x;
   const int64_t label = labels[r];
   const float g = grad_rows[r];
   const T* row = logits + r * ld;
-  T* out = dlogits + r * ld_out;
+  int64_t dst = r;
+  if (row_map) {
+    dst = row_map[r];
+    if (dst < 0) return;
+  }
+  T* out = dlogits + dst * ld_out;
   const int tid = threadIdx.x;
   const int64_t nchunks = (vocab + 7) >> 3;
   if (g == 0.f || label == ignore_index) {
@@ -155,13 +162,13 @@ extern "C" int spx_label_ce_fwd(const void* logits, int64_t ld_logits, const int
   return check_launch(__func__);
 }
 
-extern "C" int spx_label_ce_bwd(const void* logits, int64_t ld_logits, const int64_t* labels,
-                                const float* lse, const float* grad_rows, int64_t rows,
-                                int64_t vocab, int dtype, int64_t ignore_index, void* dlogits,
-                                int64_t ld_out, void* stream) {
-  if (int rc = label_ce_checks(__func__, logits, ld_logits, labels, rows, vocab, dtype)) return rc;
-  SPX_REQUIRE(lse && grad_rows && dlogits, "null buffer");
-  SPX_REQUIRE(ld_out >= vocab, "leading dimension of the gradient smaller than vocab");
+static int label_ce_bwd_impl(const char* fn, const void* logits, int64_t ld_logits, const int64_t* labels,
+                             const float* lse, const float* grad_rows, int64_t rows, int64_t vocab,
+                             int dtype, int64_t ignore_index, void* dlogits, int64_t ld_out,
+                             const int32_t* row_map, void* stream) {
+  if (int rc = label_ce_checks(fn, logits, ld_logits, labels, rows, vocab, dtype)) return rc;
+  if (!(lse && grad_rows && dlogits)) return fail_arg(fn, "null buffer");
+  if (ld_out < vocab) return fail_arg(fn, "leading dimension of the gradient smaller than vocab");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const int esz = dtype == SPX_DTYPE_BF16 ? 2 : 4;
   const bool vec = ptr_aligned16(logits) && ptr_aligned16(dlogits) && (ld_logits * esz) % 16 == 0 &&
@@ -170,9 +177,27 @@ extern "C" int spx_label_ce_bwd(const void* logits, int64_t ld_logits, const int
 #define SPX_LAUNCH(T, V)                                                                       \
   hipLaunchKernelGGL((label_ce_bwd_kernel<T, V>), grid, block, 0, st,                          \
                      reinterpret_cast<const T*>(logits), ld_logits, labels, lse, grad_rows, vocab, \
-                     ignore_index, reinterpret_cast<T*>(dlogits), ld_out)
+                     ignore_index, reinterpret_cast<T*>(dlogits), ld_out, row_map)
   if (dtype == SPX_DTYPE_BF16) { if (vec) SPX_LAUNCH(uint16_t, true); else SPX_LAUNCH(uint16_t, false); }
   else { if (vec) SPX_LAUNCH(float, true); else SPX_LAUNCH(float, false); }
 #undef SPX_LAUNCH
-  return check_launch(__func__);
+  return check_launch(fn);
+}
+
+extern "C" int spx_label_ce_bwd(const void* logits, int64_t ld_logits, const int64_t* labels,
+                                const float* lse, const float* grad_rows, int64_t rows,
+                                int64_t vocab, int dtype, int64_t ignore_index, void* dlogits,
+                                int64_t ld_out, void* stream) {
+  return label_ce_bwd_impl(__func__, logits, ld_logits, labels, lse, grad_rows, rows, vocab, dtype,
+                           ignore_index, dlogits, ld_out, nullptr, stream);
+}
+
+extern "C" int spx_label_ce_bwd_packed(const void* logits, int64_t ld_logits, const int64_t* labels,
+                                       const float* lse, const float* grad_rows, int64_t rows,
+                                       int64_t vocab, int dtype, int64_t ignore_index,
+                                       const int32_t* row_map, void* dlogits, int64_t ld_out,
+                                       void* stream) {
+  if (!row_map) return fail_arg(__func__, "null row map");
+  return label_ce_bwd_impl(__func__, logits, ld_logits, labels, lse, grad_rows, rows, vocab, dtype,
+                           ignore_index, dlogits, ld_out, row_map, stream);
 }

@@ -19,8 +19,13 @@ from . import _lib
 _MAX_SPAN = 0x7ffffff0 - 64  # bytes one GEMM operand may span
 
 
-def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """``a[M, K] @ b[N, K].T -> [M, N]`` (bf16, fp32 accumulation)."""
+def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
+            m_live: torch.Tensor | None = None) -> torch.Tensor:
+    """``a[M, K] @ b[N, K].T -> [M, N]`` (bf16, fp32 accumulation).
+
+    ``m_live`` (a one-element int32 device tensor) says how many leading rows of ``a`` count:
+    the rows from there on are neither read nor written, and the host never learns the
+    number (no synchronisation)."""
     if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
         raise _lib.SpxError("gemm_nt takes bf16 operands")
     if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
@@ -33,18 +38,16 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -
     n = b.shape[0]
     if out is None:
         out = torch.empty(m, n, device=a.device, dtype=torch.bfloat16)
-    # the kernel addresses each operand with 32-bit byte offsets: an operand that spans
-    # 2 GiB or more is fed in row bands (full-vocabulary logits gradients are that large)
-    rows_a = max(_MAX_SPAN // (2 * a.stride(0)), 1) if m > 1 else 1
-    rows_b = max(_MAX_SPAN // (2 * b.stride(0)), 1) if n > 1 else 1
+    # (operands of any size go in one launch: the kernel's 32-bit offsets are relative to a tile)
     st = _lib.stream_ptr(a.device)
-    for m0 in range(0, m, max(rows_a, 1)):
-        am = a[m0:m0 + rows_a]
-        for n0 in range(0, n, max(rows_b, 1)):
-            bn = b[n0:n0 + rows_b]
-            o = out[m0:m0 + rows_a, n0:n0 + rows_b]
-            _lib.call("spx_gemm_bf16_nt", _lib.ptr(am), am.stride(0), _lib.ptr(bn), bn.stride(0),
-                      _lib.ptr(o), o.stride(0), am.shape[0], bn.shape[0], k, st)
+    if m_live is None:
+        _lib.call("spx_gemm_bf16_nt", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
+                  _lib.ptr(out), out.stride(0), m, n, k, st)
+    else:
+        if m_live.dtype != torch.int32 or m_live.numel() != 1 or m_live.device != a.device:
+            raise ValueError("m_live must be a one-element int32 tensor on the operands' device")
+        _lib.call("spx_gemm_bf16_nt_rows", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
+                  _lib.ptr(out), out.stride(0), m, n, k, _lib.ptr(m_live), st)
     return out
 
 

@@ -247,6 +247,76 @@ def label_cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index
     return _LabelCE.apply(x, lab, ignore_index).view(labels.shape)
 
 
+class _HeadLabelCE(torch.autograd.Function):
+    """A frozen output head and the label cross-entropy behind it as ONE autograd node:
+    ``(x [R, H], weight [V, H], weight_t [H, V], labels [R]) -> (row loss [R] f32, logits [R, V])``.
+
+    What the single node buys is the backward: a position with an ignored label (or a zero
+    incoming gradient) has an all-zero logits-gradient row, so the loss backward packs the live
+    rows to the front (``spx_label_ce_bwd_packed``) and the input-gradient product runs over
+    those rows only (``spx_gemm_bf16_nt_rows``, row count read on the device, no host
+    synchronisation); the dead rows of ``dx`` are exact zeros, as they are when the product
+    runs over all rows.  The logits come back for the caller's metrics / return value but carry
+    no gradient of their own."""
+
+    @staticmethod
+    def forward(ctx, x2, weight, weight_t, labels, ignore_index):
+        from .gemm import gemm_nt
+
+        logits = gemm_nt(x2, weight)
+        rows, vocab = logits.shape
+        out = torch.empty(2, rows, device=logits.device, dtype=torch.float32)
+        _lib.call("spx_label_ce_fwd", _lib.ptr(logits), logits.stride(0), _lib.ptr(labels), rows,
+                  vocab, _lib.dtype_code(logits), int(ignore_index), _lib.ptr(out[0]),
+                  _lib.ptr(out[1]), None, _lib.stream_ptr(logits.device))
+        ctx.save_for_backward(logits, labels, out[1], weight_t)
+        ctx.ignore_index = int(ignore_index)
+        ctx.mark_non_differentiable(logits)
+        return out[0], logits
+
+    @staticmethod
+    def backward(ctx, grad_rows, _grad_logits):
+        from .gemm import gemm_nt
+
+        logits, labels, lse, weight_t = ctx.saved_tensors
+        rows, vocab = logits.shape
+        g = grad_rows.to(torch.float32).contiguous()
+        live = (labels != ctx.ignore_index) & (g != 0)
+        count = torch.cumsum(live, 0, dtype=torch.int32)
+        row_map = torch.where(live, count - 1, torch.full_like(count, -1))
+        packed = torch.empty(rows, vocab, device=logits.device, dtype=logits.dtype)
+        _lib.call("spx_label_ce_bwd_packed", _lib.ptr(logits), logits.stride(0), _lib.ptr(labels),
+                  _lib.ptr(lse), _lib.ptr(g), rows, vocab, _lib.dtype_code(logits), ctx.ignore_index,
+                  _lib.ptr(row_map), _lib.ptr(packed), packed.stride(0),
+                  _lib.stream_ptr(logits.device))
+        dx_packed = gemm_nt(packed, weight_t, m_live=count[-1:])
+        # back to one row per position: live rows from their packed slot, the others zero (the rows
+        # of dx_packed past the count were never written)
+        dx = dx_packed.index_select(0, row_map.clamp(min=0))
+        dx.masked_fill_(~live.unsqueeze(1), 0)
+        return dx, None, None, None, None
+
+
+def head_label_cross_entropy(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor,
+                             labels: torch.Tensor, ignore_index: int = -100):
+    """``logits = x @ weight.T`` and ``F.cross_entropy(logits, labels, ignore_index=...,
+    reduction="none")`` (models/mtp/core.py:190-216) for a FROZEN ``weight [V, H]`` whose
+    transpose ``weight_t [H, V]`` the caller keeps: returns ``(loss [...] f32, logits [..., V])``.
+    Gradient flows to ``x`` through the loss only; the returned logits are detached."""
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or weight_t.dtype != torch.bfloat16:
+        raise _lib.SpxError("head_label_cross_entropy takes bf16 operands")
+    if weight.requires_grad:
+        raise ValueError("head_label_cross_entropy is for a frozen head (no weight gradient is produced)")
+    if x.shape[:-1] != labels.shape:
+        raise ValueError(f"x {tuple(x.shape)} and labels {tuple(labels.shape)} do not match")
+    if weight_t.shape != (weight.shape[1], weight.shape[0]) or not weight_t.is_contiguous():
+        raise ValueError("weight_t must be the contiguous transpose of weight")
+    x2 = x.reshape(-1, x.shape[-1])
+    lab = labels.reshape(-1).to(torch.int64).contiguous()
+    loss, logits = _HeadLabelCE.apply(x2, weight, weight_t, lab, ignore_index)
+    return loss.view(labels.shape), logits.view(*labels.shape, weight.shape[0])
+
+
 def vocab_gather(full_logits: torch.Tensor, d2t: torch.Tensor) -> torch.Tensor:
     """``full_logits[..., i + d2t[i]]`` on the device: verifier logits over the target
     vocabulary restricted to the draft vocabulary (the gather form of the t2d row-slice,

@@ -102,22 +102,27 @@ class MTPDraftModel(nn.Module):
         self.embed_tokens.weight.requires_grad_(False)
         self.lm_head.weight.requires_grad_(False)
         self._frozen_t: dict = {}
+        # lm_head and the loss as one autograd node while the head is frozen (False: two nodes, logits
+        # returned with their own gradient path as in the reference)
+        self.fuse_head_loss = True
 
     @property
     def layers(self) -> nn.ModuleList:
         return self.mtp_layers
 
+    def _lm_head_t(self):
+        """``lm_head.weight.T`` contiguous, cached until the weight changes."""
+        w = self.lm_head.weight
+        key = (w.data_ptr(), w._version)
+        hit = self._frozen_t.get("lm_head")
+        if hit is None or hit[0] != key:
+            hit = (key, w.detach().t().contiguous())
+            self._frozen_t["lm_head"] = hit
+        return hit[1]
+
     def _lm_head(self, x):
         w = self.lm_head.weight
-        wt = None
-        if x.requires_grad:
-            key = (w.data_ptr(), w._version)
-            hit = self._frozen_t.get("lm_head")
-            if hit is None or hit[0] != key:
-                hit = (key, w.detach().t().contiguous())
-                self._frozen_t["lm_head"] = hit
-            wt = hit[1]
-        return gemm.linear(x, w, wt)
+        return gemm.linear(x, w, self._lm_head_t() if x.requires_grad else None)
 
     def forward(self, input_ids, hidden_states, attention_mask=None, position_ids=None,
                 loss_mask=None, step_weights=None, return_dict: bool = True, **_kwargs):
@@ -166,15 +171,21 @@ class MTPDraftModel(nn.Module):
                 emb = F.embedding(input_ids[:, step + 1:step + 1 + valid], self.embed_tokens.weight)
                 emb = emb.to(hidden_states.dtype).reshape(1, b * valid, cfg.hidden_size)
             out = layer(hid, emb, flat_pos, inv_freq, mask)
-            logits = self._lm_head(out).view(b, valid, cfg.vocab_size)
-            all_logits.append(logits)
-
             targets = input_ids[:, step + 2:step + 2 + valid]
             if loss_mask is not None:
                 targets = targets.clone()
                 targets[loss_mask[:, step + 2:step + 2 + valid] == 0] = IGNORE_INDEX
             weight = step_weights[step] if step_weights is not None else 1.0
-            unreduced = L.label_cross_entropy(logits, targets, IGNORE_INDEX)
+            if self.fuse_head_loss and out.requires_grad and not self.lm_head.weight.requires_grad:
+                # head + loss as one autograd node: the backward skips the ignored positions in the
+                # input-gradient product of the head (the returned logits carry no gradient)
+                unreduced, logits = L.head_label_cross_entropy(
+                    out.view(b, valid, cfg.hidden_size), self.lm_head.weight, self._lm_head_t(),
+                    targets, IGNORE_INDEX)
+            else:
+                logits = self._lm_head(out).view(b, valid, cfg.vocab_size)
+                unreduced = L.label_cross_entropy(logits, targets, IGNORE_INDEX)
+            all_logits.append(logits)
             valid_count = (targets != IGNORE_INDEX).sum()
             step_loss = weight * unreduced.sum() / valid_count.clamp(min=1)
             total_loss = total_loss + step_loss

@@ -145,3 +145,23 @@ def test_gemm_tn_rejects_bad_arguments():
         gemm_tn(b, torch.zeros(8, 8, dtype=torch.bfloat16, device="cuda"))
     with pytest.raises(ValueError):
         gemm_tn(b, b, accumulate=True)
+
+
+@pytest.mark.parametrize("m,live", [(600, 0), (600, 1), (600, 256), (600, 257), (600, 599), (600, 600), (600, 900)])
+def test_gemm_nt_with_a_row_count_on_the_device(m, live):
+    """Rows from the device-side count on are neither read (they hold NaN here) nor written
+    (the output keeps its fill value); the rows before it equal the plain product bit for bit."""
+    from speculators_amd.gemm import gemm_nt
+
+    g = torch.Generator().manual_seed(live)
+    a = torch.randn(m, 136, generator=g).bfloat16().cuda()
+    b = torch.randn(300, 136, generator=g).bfloat16().cuda()
+    want = gemm_nt(a, b)
+    n_live = min(live, m)
+    a_dirty = a.clone()
+    a_dirty[n_live:] = float("nan")
+    out = torch.full((m, 300), 7.0, dtype=torch.bfloat16, device="cuda")
+    count = torch.tensor([live], dtype=torch.int32, device="cuda")
+    gemm_nt(a_dirty, b, out, m_live=count)
+    assert torch.equal(out[:n_live], want[:n_live])
+    assert (out[n_live:] == 7).all()

@@ -76,16 +76,25 @@ def test_label_ce_bad_label_is_nan_and_errors():
         label_cross_entropy(x.half(), lab)
 
 
-def test_gemm_row_bands_equal_single_call(monkeypatch):
+def test_gemm_operand_above_2_gib_in_one_launch():
+    """A logits-gradient-sized first operand (2.2 GB) goes through ONE launch: the kernel's 32-bit
+    offsets are relative to the tile.  Rows on both sides of the 2 GiB line against an fp32
+    product of the same rows."""
     from speculators_amd import gemm
 
-    g = torch.Generator().manual_seed(0)
-    a = torch.randn(700, 256, generator=g).bfloat16().cuda()
-    b = torch.randn(520, 256, generator=g).bfloat16().cuda()
-    want = gemm.gemm_nt(a, b)
-    monkeypatch.setattr(gemm, "_MAX_SPAN", 256 * 2 * 300)  # bands of 300 rows
+    g = torch.Generator(device="cuda").manual_seed(0)
+    m, k, n = 8200, 131080, 264
+    a = torch.randn(m, k, device="cuda", generator=g).bfloat16()
+    b = (torch.randn(n, k, device="cuda", generator=g) * 0.05).bfloat16()
+    assert a.numel() * 2 > 2 ** 31
     got = gemm.gemm_nt(a, b)
-    assert torch.equal(got, want)
+    rows = torch.tensor([0, 255, 256, 8190, 8191, 8192, 8193, m - 1], device="cuda")
+    want = a[rows].float() @ b.float().t()
+    assert (got[rows].float() - want).abs().max() <= 2 ** -8 * want.abs().max() + 1e-3
+    count = torch.tensor([8195], dtype=torch.int32, device="cuda")
+    out = torch.full((m, n), 3.0, dtype=torch.bfloat16, device="cuda")
+    gemm.gemm_nt(a, b, out, m_live=count)
+    assert torch.equal(out[:8195], got[:8195]) and (out[8195:] == 3).all()
 
 
 @pytest.mark.parametrize("t,hq,hkv,docs", [(192, 2, 1, [192]), (300, 4, 2, [100, 130, 70])])
@@ -208,3 +217,84 @@ def test_model_properties_of_the_reference_tests():
             model(ids, hs, attention_mask=torch.ones(1, 40, device="cuda"))
         with pytest.raises(RuntimeError, match="bf16"):
             model(ids, hs.float())
+
+
+def test_head_and_loss_as_one_node_equals_the_two_node_path():
+    """Frozen head + label cross-entropy as one autograd node (packed loss backward, row-counted
+    input-gradient product) against linear + label_cross_entropy: same losses, same logits, and
+    the same input gradient bit for bit -- zero rows included."""
+    from speculators_amd import gemm
+    from speculators_amd import losses as L
+
+    g = torch.Generator().manual_seed(3)
+    rows, h, v = 700, 128, 1000
+    x = torch.randn(2, rows // 2, h, generator=g).bfloat16().cuda()
+    w = (torch.randn(v, h, generator=g) * 0.05).bfloat16().cuda()
+    wt = w.t().contiguous()
+    labels = torch.randint(0, v, (2, rows // 2), generator=g)
+    labels[torch.rand(2, rows // 2, generator=g) < 0.35] = -100
+    labels[0, :5] = -100           # a dead run at the very start
+    labels = labels.cuda()
+    gw = torch.rand(2, rows // 2, generator=g).cuda()
+    gw[1, 7] = 0.0                  # a live label with a zero incoming gradient
+
+    x1 = x.clone().requires_grad_(True)
+    loss1, logits1 = L.head_label_cross_entropy(x1, w, wt, labels)
+    (loss1 * gw).sum().backward()
+    x2 = x.clone().requires_grad_(True)
+    logits2 = gemm.linear(x2, w, wt)
+    loss2 = L.label_cross_entropy(logits2, labels)
+    (loss2 * gw).sum().backward()
+    assert torch.equal(loss1, loss2) and torch.equal(logits1, logits2.detach())
+    assert not logits1.requires_grad
+    assert torch.equal(x1.grad, x2.grad)
+    dead = (labels == -100) | (gw == 0)
+    assert (x1.grad[dead] == 0).all() and (x1.grad[~dead] != 0).any()
+
+
+@pytest.mark.parametrize("frac", [0.0, 1.0])
+def test_head_and_loss_node_with_no_or_all_rows_live(frac):
+    from speculators_amd import losses as L
+
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(1, 300, 64, generator=g).bfloat16().cuda().requires_grad_(True)
+    w = (torch.randn(520, 64, generator=g) * 0.05).bfloat16().cuda()
+    labels = torch.randint(0, 520, (1, 300), generator=g).cuda()
+    if frac == 0.0:
+        labels[:] = -100
+    loss, _ = L.head_label_cross_entropy(x, w, w.t().contiguous(), labels)
+    loss.sum().backward()
+    ref = x.detach().clone().requires_grad_(True)
+    L.label_cross_entropy((ref.float() @ w.float().t()).bfloat16(), labels)  # shape / dtype check only
+    if frac == 0.0:
+        assert (x.grad == 0).all() and (loss == 0).all()
+    else:
+        assert torch.isfinite(x.grad.float()).all() and (x.grad != 0).any()
+
+
+def test_model_with_and_without_the_fused_head_node_agree():
+    """The MTP model's loss, logits and parameter gradients do not depend on whether the head and
+    the loss are one autograd node or two (bit for bit: the packed product computes the same
+    dot products in the same order)."""
+    shape = _shape()
+    steps = 2
+    w = {k: v.bfloat16() for k, v in OM.random_weights(shape, seed=4, std=0.05).items()}
+    g = torch.Generator().manual_seed(9)
+    b, n = 2, 150
+    ids = torch.randint(0, shape.vocab_size, (b, n), generator=g).cuda()
+    hs = torch.randn(b, n, shape.hidden_size, generator=g).bfloat16().cuda()
+    lm = (torch.rand(b, n, generator=g) < 0.6).float().cuda()
+    got = []
+    for fuse in (True, False):
+        model = _make(shape, w, steps)
+        model.fuse_head_loss = fuse
+        logits, loss, _ = model(ids, hs, loss_mask=lm)
+        loss.backward()
+        got.append((loss.detach(), [x.detach() for x in logits],
+                    {k: p.grad.clone() for k, p in model.named_parameters() if p.grad is not None}))
+    assert torch.equal(got[0][0], got[1][0])
+    for x, y in zip(got[0][1], got[1][1]):
+        assert torch.equal(x, y)
+    assert got[0][2].keys() == got[1][2].keys() and len(got[0][2]) > 0
+    for k in got[0][2]:
+        assert torch.equal(got[0][2][k], got[1][2][k]), k
