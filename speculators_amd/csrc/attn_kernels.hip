@@ -934,6 +934,9 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
 #ifndef SPX_DKV_XCD
 #define SPX_DKV_XCD 1
 #endif
+#ifndef SPX_DKV256_ONEPASS
+#define SPX_DKV256_ONEPASS 1
+#endif
 #ifndef SPX_DKV256_PF1
 #define SPX_DKV256_PF1 2
 #endif
@@ -941,13 +944,14 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
 #define SPX_DKV256_PF2 1
 #endif
 // PF: how the query tiles reach LDS (see FwdSmem): 0 at the point of use, 1 through registers one
-// tile ahead, 2 global -> LDS into the other of two buffers.  A buffer holds the tiles the pass
-// multiplies with: Q always, dO and Q^T for dK, dO^T for dV (at head_dim 256 two buffers of the dK
-// pass's three tiles do not fit the 160 KB of LDS: that pass stays on mode 1).
-template <int D, int PASS>
+// tile ahead, 2 global -> LDS into the other of two buffers, 3 the same with tiles of 32 instead of 64
+// query rows.  A buffer holds the tiles the pass multiplies with: Q always, dO and Q^T for dK, dO^T for
+// dV.  At head_dim 256 two buffers of 64-row tiles fit the 160 KB of LDS only for the dV pass; with
+// 32-row tiles all four fit, the register staging is gone and dK and dV come out of ONE pass.
+template <int D, int PASS, int QT = 64>
 struct DkvSmem {
   static constexpr bool kDoV = PASS != 2, kDoK = PASS != 1;
-  static constexpr int kTileR = 64 * D * 2, kTileT = D * 128;  // Q / dO and Q^T / dO^T tiles, unpadded
+  static constexpr int kTileR = QT * D * 2, kTileT = D * QT * 2;  // Q / dO and Q^T / dO^T tiles, unpadded
   static constexpr int kOffdO = kTileR;
   static constexpr int kOffQt = (kDoK ? 2 : 1) * kTileR;
   static constexpr int kOffdOt = kOffQt + (kDoK ? kTileT : 0);
@@ -976,10 +980,13 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
   uint16_t* dOs = Qs + 64 * QS;        // [64][QS]
   uint16_t* Qts = dOs + 64 * QS;       // [D][TS]
   uint16_t* dOts = Qts + D * TS;       // [D][TS]
-  using SM = DkvSmem<D, PASS>;
-  static_assert(PF != 2 || SM::kBytesDma <= 160 * 1024, "two buffers of this pass's tiles do not fit in LDS");
+  constexpr bool kDma = PF >= 2;
+  constexpr int QT = PF == 3 ? 32 : 64;          // query rows per LDS tile
+  constexpr int NQB = QT / 32, NSUB = 64 / QT;   // 32-row halves per tile, tiles per 64-row step
+  using SM = DkvSmem<D, PASS, QT>;
+  static_assert(!kDma || SM::kBytesDma <= 160 * 1024, "two buffers of this pass's tiles do not fit in LDS");
   uint8_t* const sm8 = reinterpret_cast<uint8_t*>(smem);
-  float* lse_s = reinterpret_cast<float*>(PF == 2 ? sm8 + 2 * SM::kBuf : sm8 + (2 * 64 * QS + 2 * D * TS) * 2);  // [64]
+  float* lse_s = reinterpret_cast<float*>(kDma ? sm8 + 2 * SM::kBuf : sm8 + (2 * 64 * QS + 2 * D * TS) * 2);  // [64]
   float* delta_s = lse_s + 64;                               // [64]
   int* a1_s = reinterpret_cast<int*>(delta_s + 64);          // [64] each
   int* b1_s = a1_s + 64;
@@ -1137,16 +1144,17 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     }
   };
 
-  // ---- two-buffer mode: the four tiles as 1 KB wave loads global -> LDS; chunk c of row r lives in
+  // ---- two-buffer modes: the tiles as 1 KB wave loads global -> LDS; chunk c of row r lives in
   // slot c ^ swz(r) (conflict-free fragment reads without padding)
-  constexpr int RBQ = D * 2, CKQ = RBQ / 16;
-  constexpr int LPR = (64 * RBQ / 1024) / NW, LPT = (D * 128 / 1024) / NW;  // wave loads per wave and tile
+  constexpr int RBQ = D * 2, CKQ = RBQ / 16;   // bytes / 16-byte chunks per row of Q and dO
+  constexpr int RBT = QT * 2, CKT = RBT / 16;  // ... of Q^T and dO^T
+  constexpr int LPR = (QT * RBQ / 1024) / NW, LPT = (D * RBT / 1024) / NW;  // wave loads per wave and tile
   auto swz_r = [](int r) { return CKQ == 8 ? (r >> 1) & 7 : r & 15; };
-  auto swz_t = [](int r) { return (r >> 1) & 7; };
+  auto swz_t = [](int r) { return CKT == 8 ? (r >> 1) & 7 : (r >> 2) & 3; };
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)sm8;
   u32x4 qres, dres, qtres, dtres;
-  int r_row[PF == 2 ? LPR : 1], r_col[PF == 2 ? LPR : 1], t_off[PF == 2 ? LPT : 1];
-  if constexpr (PF == 2) {
+  int r_row[kDma ? LPR : 1], r_col[kDma ? LPR : 1], t_off[kDma ? LPT : 1];
+  if constexpr (kDma) {
     qres = make_rsrc(Qh, (uint32_t)((int64_t)p.NQ * RBQ));
     dres = make_rsrc(dO + (int64_t)h * D, (uint32_t)((((int64_t)p.NQ - 1) * p.Hq * D + D) * 2));
     qtres = make_rsrc(Qth, (uint32_t)((int64_t)D * NQp * 2));
@@ -1159,12 +1167,12 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     }
 #pragma unroll
     for (int j = 0; j < LPT; ++j) {
-      const int r = (wave * LPT + j) * 8 + lane / 8;
-      t_off[j] = r * NQp * 2 + ((lane & 7) ^ swz_t(r)) * 16;
+      const int r = (wave * LPT + j) * (1024 / RBT) + lane / CKT;
+      t_off[j] = r * NQp * 2 + ((lane % CKT) ^ swz_t(r)) * 16;
     }
   }
   auto issue = [&](int mq, int b) __attribute__((always_inline)) {
-    if constexpr (PF == 2) {
+    if constexpr (kDma) {
       const uint32_t rb = lds0 + b * SM::kBuf + wave * LPR * 1024;
 #pragma unroll
       for (int j = 0; j < LPR; ++j) {
@@ -1181,37 +1189,43 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     }
   };
   const int rdr = col * RBQ + ((g ^ swz_r(col)) * 16);
-  const int rdt = col * 128 + ((g ^ swz_t(col)) * 16);
+  const int rdt = col * RBT + ((g ^ swz_t(col)) * 16);
   const float* const lse_s0 = lse_s;
   const uint8_t* tile = sm8;
   int buf = 0;
 
   // (walking the tiles from the last one down, so that every workgroup of a head reads the same tile at
   // the same time, was slower: 256 workgroups then hit the same few memory channels at once)
-  int qi = 0;
+  int qi = 0, sub = 0, sbuf = 0;  // 64-row step, tile inside it, set of per-row scalars in use
   while (qi < n_qt && !visible(qi)) ++qi;
   if (PF == 1 && qi < n_qt) fetch(qi * 64);
-  if (PF == 2 && qi < n_qt) {
+  if (kDma && qi < n_qt) {
     issue(qi * 64, 0);
     small_fetch(qi * 64);
     small_stash(0);
   }
   while (qi < n_qt) {
-    int nxi = qi + 1;
-    while (nxi < n_qt && !visible(nxi)) ++nxi;
+    // what comes next: the other tile of this 64-row step, or the first tile of the next visible step
+    int nxi = qi, nsub = sub + 1;
+    if (nsub == NSUB) {
+      nsub = 0;
+      ++nxi;
+      while (nxi < n_qt && !visible(nxi)) ++nxi;
+    }
     const int qt = qi, nxt = nxi;
     const bool full = fully_visible(qt);
-    if constexpr (PF == 2) {
+    const bool have_next = nxi < n_qt;
+    if constexpr (kDma) {
       // this wave's loads of the tile have landed; behind the barrier everybody's have, the per-row
       // scalars written at the end of the last iteration are visible, and the other buffer is free
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      if (nxi < n_qt) {
-        issue(nxt * 64, buf ^ 1);
-        small_fetch(nxt * 64);
+      if (have_next) {
+        issue(nxt * 64 + nsub * QT, buf ^ 1);
+        if (nsub == 0) small_fetch(nxt * 64);
       }
       tile = sm8 + buf * SM::kBuf;
-      const int o = buf * (SM::kSmall / 4);
+      const int o = sbuf * (SM::kSmall / 4);
       lse_s = const_cast<float*>(lse_s0) + o;
       delta_s = lse_s + 64;
       a1_s = reinterpret_cast<int*>(delta_s + 64);
@@ -1220,15 +1234,17 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       __syncthreads();
       if (PF) stash(); else direct(qt * 64);
       __syncthreads();
-      if (PF && nxi < n_qt) fetch(nxt * 64);
+      if (PF && have_next) fetch(nxt * 64);
     }
-    const bool have_next = nxi < n_qt;
+    const int sub_now = sub;
     qi = nxi;
+    sub = nsub;
 
     // the two 32-row halves of the query tile one after the other (keeps 32 score
     // registers live instead of 64)
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
+    for (int qbl = 0; qbl < NQB; ++qbl) {
+      const int qb = sub_now * NQB + qbl;  // 32-row half inside the 64-row step (per-row scalars); qbl: inside the LDS tile
       f32x16 st, dp;
 #pragma unroll
       for (int r = 0; r < 16; ++r) { st[r] = 0.f; dp[r] = 0.f; }
@@ -1239,10 +1255,10 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         constexpr int NF = PER * NKK;
         bf16x8 fr[4];
         auto fread = [&](int f) {
-          if constexpr (PF == 2) {
+          if constexpr (kDma) {
             const uint8_t* base = tile + ((PER == 2 && (f & 1)) ? SM::kOffdO : 0);
             fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-                base + qb * 32 * RBQ + (rdr ^ ((f / PER) * 32))));
+                base + qbl * 32 * RBQ + (rdr ^ ((f / PER) * 32))));
           } else {
             const uint16_t* base = (PER == 2 && (f & 1)) ? dOs : Qs;
             fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
@@ -1303,10 +1319,10 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         auto fread = [&](int f) {
           const int e = f / PER, s2 = e / NDB, db = e % NDB;
           const bool is_q = kDoK && (!kDoV || (f % PER) == 1);
-          if constexpr (PF == 2) {
+          if constexpr (kDma) {
             const uint8_t* base = tile + (is_q ? SM::kOffQt : SM::kOffdOt);
             fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-                base + db * 32 * 128 + (rdt ^ ((qb * 2 + s2) * 32))));
+                base + db * 32 * RBT + (rdt ^ ((qbl * 2 + s2) * 32))));
           } else {
             const uint16_t* base = is_q ? Qts : dOts;
             fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
@@ -1331,16 +1347,19 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    if constexpr (PF == 2) {
-      // the per-row scalars of the next tile go into the other set: nobody reads it before the barrier
-      if (have_next) {
-        lse_s = const_cast<float*>(lse_s0); delta_s = lse_s + 64;
-        a1_s = reinterpret_cast<int*>(delta_s + 64); b1_s = a1_s + 64; a2_s = b1_s + 64; b2_s = a2_s + 64;
-        small_stash(buf ^ 1);
+    if constexpr (kDma) {
+      // the per-row scalars of the next 64-row step go into the other set: nobody reads it before the
+      // barrier
+      if (nsub == 0) {
+        if (have_next) {
+          lse_s = const_cast<float*>(lse_s0); delta_s = lse_s + 64;
+          a1_s = reinterpret_cast<int*>(delta_s + 64); b1_s = a1_s + 64; a2_s = b1_s + 64; b2_s = a2_s + 64;
+          small_stash(sbuf ^ 1);
+        }
+        sbuf ^= 1;
       }
       buf ^= 1;
     }
-    (void)have_next;
   }
 
   if (c < p.NKV) {
@@ -1594,7 +1613,7 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
 
   constexpr int kPF = D > 128 ? 1 : kDkvPF;
   constexpr int kPF1 = SPX_DKV256_PF1, kPF2 = SPX_DKV256_PF2;
-  if ((kPF == 2 || (D > 128 && (kPF1 == 2 || kPF2 == 2))) && (int64_t)p.NQ * p.Hq * D * 2 >= (1ll << 31)) {
+  if ((kPF == 2 || D > 128) && (int64_t)p.NQ * p.Hq * D * 2 >= (1ll << 31)) {
     last_error() = std::string(fn) + ": queries must span less than 2 GiB";
     return SPX_ERR_ARG;
   }
@@ -1606,7 +1625,16 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
     return e == hipSuccess;
   };
   static bool attr_set = false;
-  if constexpr (D > 128) {
+  if constexpr (D > 128 && SPX_DKV256_ONEPASS) {
+    // dK and dV in one pass over 32-row tiles (two buffers of four 16 KB tiles)
+    constexpr size_t smem = DkvSmem<D, 0, 32>::kBytesDma;
+    if (!attr_set) {
+      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, 3, 0>), smem)) return SPX_ERR_HIP;
+      attr_set = true;
+    }
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, 3, 0>), kgrid, kblock, smem, st, p, dOp, qt, dot,
+                       NQp, lse, delta, tb, dkp, dvp);
+  } else if constexpr (D > 128) {
     // one launch per gradient (each loads only the tiles it multiplies with)
     constexpr size_t smem1 = kPF1 == 2 ? DkvSmem<D, 1>::kBytesDma : DkvSmem<D, 1>::kBytes;
     constexpr size_t smem2 = kPF2 == 2 ? DkvSmem<D, 2>::kBytesDma : DkvSmem<D, 2>::kBytes;
