@@ -158,12 +158,12 @@ class GemmProbe:
         self.orig = self.gemm.gemm_nt
         ev = self.torch.cuda.Event
 
-        def probed(a, b, out=None):
+        def probed(a, b, out=None, **kw):
             if (tuple(a.shape), tuple(b.shape)) != self.shape:
-                return self.orig(a, b, out)
+                return self.orig(a, b, out, **kw)
             e0, e1 = ev(enable_timing=True), ev(enable_timing=True)
             e0.record()
-            r = self.orig(a, b, out)
+            r = self.orig(a, b, out, **kw)
             e1.record()
             self.pairs.append((e0, e1))
             return r

@@ -92,6 +92,20 @@ int spx_fused_vocab_loss_bwd(int op, const void* logits, int64_t ld_logits,
                              const float* row_grad, const float* scale,
                              void* grad_logits, int64_t ld_grad, void* stream);
 
+/* The same gradient with the live rows packed to the front: row r goes to row
+ * row_map[r] of grad_logits, rows with row_map[r] < 0 (zero gradient: masked out
+ * of the loss, losses/utils.py:233-304) are not written.  Feeds
+ * spx_gemm_bf16_nt_rows, which skips them in the lm_head input-gradient product.
+ * No counterpart in the reference, where that product runs over all rows. */
+int spx_fused_vocab_loss_bwd_packed(int op, const void* logits, int64_t ld_logits,
+                                    const void* targets, int64_t ld_targets,
+                                    int64_t rows, int64_t vocab, int dtype,
+                                    const float* lse_draft, const float* lse_target,
+                                    const float* extra, const int32_t* argmax_target,
+                                    const float* row_grad, const float* scale,
+                                    const int32_t* row_map, void* grad_logits,
+                                    int64_t ld_grad, void* stream);
+
 /* Cross-entropy of full-vocabulary logits against integer labels, the loss of
  * the multi-token-prediction path: loss[r] = logsumexp(logits[r, :]) -
  * logits[r, labels[r]], 0 where labels[r] == ignore_index (such rows are not
@@ -362,6 +376,18 @@ int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb,
 int spx_gemm_bf16_nt_rows(const void* a, int64_t lda, const void* b, int64_t ldb,
                           void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
                           const int32_t* m_live, void* stream);
+
+/* The two ends of a packed-rows product (spx_*_bwd_packed -> spx_gemm_bf16_nt_rows).
+ * spx_pack_row_map: row_map[r] = number of live rows before r if row r is live
+ * (row_grad[r] != 0 and, when labels is not NULL, labels[r] != ignore_index), else -1;
+ * *count = number of live rows (device memory: the host never reads it).
+ * spx_unpack_rows (bf16): out[r, :] = packed[row_map[r], :] for live rows, zeros for
+ * the others and for rows <= r < total_rows.  No counterpart in the reference. */
+int spx_pack_row_map(const float* row_grad, const int64_t* labels, int64_t ignore_index,
+                     int64_t rows, int32_t* row_map, int32_t* count, void* stream);
+int spx_unpack_rows(const void* packed, int64_t ld_packed, const int32_t* row_map,
+                    int64_t rows, int64_t total_rows, int64_t cols, void* out,
+                    int64_t ld_out, void* stream);
 
 /* c[M, N] (+)= a[T, M]^T * b[T, N], bf16 inputs, fp32 accumulation, bf16 output:
  * the weight-gradient product of the backward of torch.nn.Linear (dW = dY^T X)

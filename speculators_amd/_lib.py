@@ -26,6 +26,8 @@ SIGNATURES: dict[str, list] = {
                                  _P],
     "spx_fused_vocab_loss_bwd": [_I, _P, _I64, _P, _I64, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P,
                                  _I64, _P],
+    "spx_fused_vocab_loss_bwd_packed": [_I, _P, _I64, _P, _I64, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P,
+                                        _P, _I64, _P],
     "spx_ttt_step_reduce": [_P, _P, _P, _P, _I, _P, _I, _I64, _F, _P, _P, _P],
     "spx_block_reduce": [_P, _P, _P, _P, _I, _P, _I64, _I32, _P, _P, _P, _P, _P],
     "spx_ttt_row_lo": [_P, _I, _I64, _I64, _P, _P],
@@ -58,6 +60,8 @@ SIGNATURES["spx_label_ce_bwd_packed"] = [_P, _I64, _P, _P, _P, _I64, _I64, _I, _
 SIGNATURES["spx_pack_batch"] = [_P, _I, _I64, _I64, _I64, _P, _P, _I, _P, _P, _P, _I64, _I64, _I,
                                 _P, _P, _P, _P, _P, _P, _P]
 SIGNATURES["spx_gemm_bf16_nt"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P]
+SIGNATURES["spx_pack_row_map"] = [_P, _P, _I64, _I64, _P, _P, _P]
+SIGNATURES["spx_unpack_rows"] = [_P, _I64, _P, _I64, _I64, _I64, _P, _I64, _P]
 SIGNATURES["spx_gemm_bf16_nt_rows"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P, _P]
 SIGNATURES["spx_gemm_bf16_tn"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I, _P]
 RESTYPES = {"spx_ttt_attn_workspace_bytes": c_int64, "spx_dflash_attn_workspace_bytes": c_int64,

@@ -289,9 +289,82 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* __restr
 
 static bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// ---- packed rows: map of the live rows, and back to one row per position
+// row_map[r] = number of live rows before r if row r is live (row_grad[r] != 0 and, with labels,
+// labels[r] != ignore_index), else -1; *count = number of live rows.  One workgroup, rows in order.
+__global__ __launch_bounds__(1024) void pack_row_map_kernel(const float* __restrict__ row_grad,
+                                                            const int64_t* __restrict__ labels,
+                                                            int64_t ignore_index, int rows,
+                                                            int32_t* __restrict__ row_map,
+                                                            int32_t* __restrict__ count) {
+  __shared__ int wave_tot[16];
+  __shared__ int base_s;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) base_s = 0;
+  __syncthreads();
+  for (int r0 = 0; r0 < rows; r0 += 1024) {
+    const int r = r0 + tid;
+    const bool live = r < rows && row_grad[r] != 0.f && (!labels || labels[r] != ignore_index);
+    const unsigned long long m = __ballot(live);
+    const int before = __popcll(m & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_tot[wave] = __popcll(m);
+    __syncthreads();
+    int off = base_s;
+    for (int w = 0; w < wave; ++w) off += wave_tot[w];
+    if (r < rows) row_map[r] = live ? off + before : -1;
+    __syncthreads();
+    if (tid == 0) {
+      int t = 0;
+      for (int w = 0; w < 16; ++w) t += wave_tot[w];
+      base_s += t;
+    }
+    __syncthreads();
+  }
+  if (tid == 0) *count = base_s;
+}
+
+// out[r, :] = row_map[r] >= 0 ? packed[row_map[r], :] : 0 for r < rows, 0 for rows <= r < total_rows
+__global__ __launch_bounds__(256) void unpack_rows_kernel(const uint16_t* __restrict__ packed, int64_t ld,
+                                                          const int32_t* __restrict__ row_map, int rows,
+                                                          int cols8, uint16_t* __restrict__ out,
+                                                          int64_t ld_out) {
+  const int r = blockIdx.x;
+  const int src = r < rows ? row_map[r] : -1;
+  u32x4* o = reinterpret_cast<u32x4*>(out + (int64_t)r * ld_out);
+  if (src < 0) {
+    const u32x4 z = {0, 0, 0, 0};
+    for (int c = threadIdx.x; c < cols8; c += 256) o[c] = z;
+    return;
+  }
+  const u32x4* in = reinterpret_cast<const u32x4*>(packed + (int64_t)src * ld);
+  for (int c = threadIdx.x; c < cols8; c += 256) o[c] = in[c];
+}
+
 }  // namespace spx
 
 using namespace spx;
+
+extern "C" int spx_pack_row_map(const float* row_grad, const int64_t* labels, int64_t ignore_index,
+                                int64_t rows, int32_t* row_map, int32_t* count, void* stream) {
+  SPX_REQUIRE(rows > 0 && rows < (1ll << 31), "rows out of range");
+  SPX_REQUIRE(row_grad && row_map && count, "null buffer");
+  hipLaunchKernelGGL(pack_row_map_kernel, dim3(1), dim3(1024), 0, reinterpret_cast<hipStream_t>(stream), row_grad,
+                     labels, ignore_index, (int)rows, row_map, count);
+  return check_launch(__func__);
+}
+
+extern "C" int spx_unpack_rows(const void* packed, int64_t ld_packed, const int32_t* row_map, int64_t rows,
+                               int64_t total_rows, int64_t cols, void* out, int64_t ld_out, void* stream) {
+  SPX_REQUIRE(rows > 0 && total_rows >= rows && total_rows < (1ll << 31), "rows out of range");
+  SPX_REQUIRE(cols > 0 && cols % 8 == 0 && ld_packed % 8 == 0 && ld_out % 8 == 0 && ld_packed >= cols && ld_out >= cols,
+              "cols and the row strides must be multiples of 8 (bf16), strides at least cols");
+  SPX_REQUIRE(packed && row_map && out, "null buffer");
+  SPX_REQUIRE(al16(packed) && al16(out), "buffers must be 16-byte aligned");
+  hipLaunchKernelGGL(unpack_rows_kernel, dim3((unsigned)total_rows), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const uint16_t*>(packed), ld_packed,
+                     row_map, (int)rows, (int)(cols / 8), reinterpret_cast<uint16_t*>(out), ld_out);
+  return check_launch(__func__);
+}
 
 extern "C" int64_t spx_rmsnorm_bwd_slots(int64_t rows, int64_t H) {
   if (H <= 512) return 4 * (rows < 8192 ? (rows + 3) / 4 : 2048);  // one wave per slot, 8 workgroups per CU

@@ -223,11 +223,19 @@ __global__ __launch_bounds__(kLossThreads) void loss_bwd_kernel(
     int64_t ld_targets, int64_t vocab, const float* __restrict__ lse_draft,
     const float* __restrict__ lse_target, const float* __restrict__ extra,
     const int32_t* __restrict__ argmax_target, const float* __restrict__ row_grad,
-    const float* __restrict__ scale, T* __restrict__ grad, int64_t ld_grad) {
+    const float* __restrict__ scale, T* __restrict__ grad, int64_t ld_grad,
+    const int32_t* __restrict__ row_map) {
   const int64_t r = blockIdx.x;
   const int tid = threadIdx.x;
   const int64_t nchunks = (vocab + 7) >> 3;
-  T* grow = grad + r * ld_grad;
+  // with a row map the gradient of row r goes to row row_map[r] and rows mapped to -1 (zero gradient)
+  // are not written: the live rows packed to the front
+  int64_t dst = r;
+  if (row_map) {
+    dst = row_map[r];
+    if (dst < 0) return;
+  }
+  T* grow = grad + dst * ld_grad;
   float g = row_grad[r];
   if (scale) g *= *scale;
   if (g == 0.f) {
@@ -450,12 +458,12 @@ template <typename T, bool VEC>
 static void launch_bwd(int op, const T* lg, int64_t ldl, const T* tg, int64_t ldt, int64_t rows,
                        int64_t vocab, const float* lsd, const float* lst, const float* ex,
                        const int32_t* at, const float* rg, const float* sc, T* grad, int64_t ldg,
-                       hipStream_t st) {
+                       const int32_t* row_map, hipStream_t st) {
   dim3 grid((unsigned)rows), block(kLossThreads);
 #define SPX_BWD(OPV)                                                                         \
   case OPV:                                                                                  \
     hipLaunchKernelGGL((loss_bwd_kernel<T, OPV, VEC>), grid, block, 0, st, lg, ldl, tg, ldt, \
-                       vocab, lsd, lst, ex, at, rg, sc, grad, ldg);                          \
+                       vocab, lsd, lst, ex, at, rg, sc, grad, ldg, row_map);                 \
     break;
   switch (op) {
     SPX_BWD(SPX_LOSS_KL) SPX_BWD(SPX_LOSS_RKL) SPX_BWD(SPX_LOSS_JSD) SPX_BWD(SPX_LOSS_CE)
@@ -503,23 +511,24 @@ extern "C" int spx_fused_vocab_loss_fwd(int op, const void* logits, int64_t ld_l
   return check_launch(__func__);
 }
 
-extern "C" int spx_fused_vocab_loss_bwd(int op, const void* logits, int64_t ld_logits,
-                                        const void* targets, int64_t ld_targets, int64_t rows,
-                                        int64_t vocab, int dtype, const float* lse_draft,
-                                        const float* lse_target, const float* extra,
-                                        const int32_t* argmax_target, const float* row_grad,
-                                        const float* scale, void* grad_logits, int64_t ld_grad,
-                                        void* stream) {
-  SPX_REQUIRE(op >= SPX_LOSS_KL && op <= SPX_LOSS_TV, "unknown loss op");
-  SPX_REQUIRE(dtype == SPX_DTYPE_BF16 || dtype == SPX_DTYPE_F32, "dtype must be bf16 or f32");
-  SPX_REQUIRE(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "rows >= 0 and 0 < vocab < 2^31");
-  SPX_REQUIRE(ld_logits >= vocab && ld_grad >= vocab, "row stride smaller than vocab");
-  SPX_REQUIRE(rows < (1ll << 31), "too many rows");
+#define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fname, what); } while (0)
+static int loss_bwd_impl(const char* fname, int op, const void* logits, int64_t ld_logits,
+                         const void* targets, int64_t ld_targets, int64_t rows,
+                         int64_t vocab, int dtype, const float* lse_draft,
+                         const float* lse_target, const float* extra,
+                         const int32_t* argmax_target, const float* row_grad,
+                         const float* scale, void* grad_logits, int64_t ld_grad,
+                         const int32_t* row_map, void* stream) {
+  SPX_REQ_FN(op >= SPX_LOSS_KL && op <= SPX_LOSS_TV, "unknown loss op");
+  SPX_REQ_FN(dtype == SPX_DTYPE_BF16 || dtype == SPX_DTYPE_F32, "dtype must be bf16 or f32");
+  SPX_REQ_FN(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "rows >= 0 and 0 < vocab < 2^31");
+  SPX_REQ_FN(ld_logits >= vocab && ld_grad >= vocab, "row stride smaller than vocab");
+  SPX_REQ_FN(rows < (1ll << 31), "too many rows");
   if (rows == 0) return SPX_OK;
-  SPX_REQUIRE(logits && grad_logits && lse_draft && row_grad, "null buffer");
-  if (op == SPX_LOSS_CE) SPX_REQUIRE(argmax_target, "ce needs argmax_target");
-  else SPX_REQUIRE(targets && lse_target && ld_targets >= vocab, "targets / lse_target missing");
-  if (op == SPX_LOSS_RKL || op == SPX_LOSS_JSD || op == SPX_LOSS_TV) SPX_REQUIRE(extra, "extra missing");
+  SPX_REQ_FN(logits && grad_logits && lse_draft && row_grad, "null buffer");
+  if (op == SPX_LOSS_CE) SPX_REQ_FN(argmax_target, "ce needs argmax_target");
+  else SPX_REQ_FN(targets && lse_target && ld_targets >= vocab, "targets / lse_target missing");
+  if (op == SPX_LOSS_RKL || op == SPX_LOSS_JSD || op == SPX_LOSS_TV) SPX_REQ_FN(extra, "extra missing");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const int64_t per16 = dtype == SPX_DTYPE_BF16 ? 8 : 4;
   const bool vec = aligned16(logits) && (op == SPX_LOSS_CE || (aligned16(targets) && ld_targets % per16 == 0)) &&
@@ -528,16 +537,40 @@ extern "C" int spx_fused_vocab_loss_bwd(int op, const void* logits, int64_t ld_l
     auto lg = reinterpret_cast<const uint16_t*>(logits);
     auto tg = reinterpret_cast<const uint16_t*>(targets);
     auto gr = reinterpret_cast<uint16_t*>(grad_logits);
-    if (vec) launch_bwd<uint16_t, true>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, st);
-    else launch_bwd<uint16_t, false>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, st);
+    if (vec) launch_bwd<uint16_t, true>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, row_map, st);
+    else launch_bwd<uint16_t, false>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, row_map, st);
   } else {
     auto lg = reinterpret_cast<const float*>(logits);
     auto tg = reinterpret_cast<const float*>(targets);
     auto gr = reinterpret_cast<float*>(grad_logits);
-    if (vec) launch_bwd<float, true>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, st);
-    else launch_bwd<float, false>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, st);
+    if (vec) launch_bwd<float, true>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, row_map, st);
+    else launch_bwd<float, false>(op, lg, ld_logits, tg, ld_targets, rows, vocab, lse_draft, lse_target, extra, argmax_target, row_grad, scale, gr, ld_grad, row_map, st);
   }
-  return check_launch(__func__);
+  return check_launch(fname);
+}
+#undef SPX_REQ_FN
+
+extern "C" int spx_fused_vocab_loss_bwd(int op, const void* logits, int64_t ld_logits,
+                                        const void* targets, int64_t ld_targets, int64_t rows,
+                                        int64_t vocab, int dtype, const float* lse_draft,
+                                        const float* lse_target, const float* extra,
+                                        const int32_t* argmax_target, const float* row_grad,
+                                        const float* scale, void* grad_logits, int64_t ld_grad,
+                                        void* stream) {
+  return loss_bwd_impl(__func__, op, logits, ld_logits, targets, ld_targets, rows, vocab, dtype, lse_draft,
+                       lse_target, extra, argmax_target, row_grad, scale, grad_logits, ld_grad, nullptr, stream);
+}
+
+extern "C" int spx_fused_vocab_loss_bwd_packed(int op, const void* logits, int64_t ld_logits,
+                                               const void* targets, int64_t ld_targets, int64_t rows,
+                                               int64_t vocab, int dtype, const float* lse_draft,
+                                               const float* lse_target, const float* extra,
+                                               const int32_t* argmax_target, const float* row_grad,
+                                               const float* scale, const int32_t* row_map,
+                                               void* grad_logits, int64_t ld_grad, void* stream) {
+  if (!row_map) return spx::fail_arg(__func__, "null row map");
+  return loss_bwd_impl(__func__, op, logits, ld_logits, targets, ld_targets, rows, vocab, dtype, lse_draft,
+                       lse_target, extra, argmax_target, row_grad, scale, grad_logits, ld_grad, row_map, stream);
 }
 
 extern "C" int spx_vocab_gather(const void* full, int64_t ld_full, const int64_t* d2t, void* out,

@@ -229,6 +229,9 @@ class Eagle3DraftModel(nn.Module):
         self.uses_sliding_window_attn = bool(config.sliding_layers)
         self.uses_full_attn = config.num_hidden_layers > len(config.sliding_layers)
         self._frozen_t: dict = {}
+        # lm_head and the loss as one autograd node while the head is frozen and the loss is a single
+        # fused reduction (False: always two nodes)
+        self.fuse_head_loss = True
 
     # ------------------------------------------------------------------ helpers
     def load_vocab_mappings(self, t2d, d2t):
@@ -329,12 +332,21 @@ class Eagle3DraftModel(nn.Module):
                 if li != last:
                     y = _Prenormed(y, normed)
             hidden = normed if cfg.norm_output else y
-            logits = self._linear(normed, self.lm_head.weight, frozen=True)
+            fuse = (return_loss and self.fuse_head_loss and normed.requires_grad
+                    and not self.lm_head.weight.requires_grad and normed.dtype == torch.bfloat16
+                    and self.lm_head.weight.dtype == torch.bfloat16)
+            if not fuse:
+                logits = self._linear(normed, self.lm_head.weight, frozen=True)
 
             if return_loss:
+                # head + loss as one autograd node while the head is frozen (see metrics.Head)
+                lg = MT.Head(normed, self.lm_head.weight,
+                             self._transposed_frozen(self.lm_head.weight)) if fuse else logits
                 s_loss, s_metrics, pred = MT.compute_metrics(
-                    logits, targets, loss_mask, prev_correct, step, ttt_step_loss_decay,
+                    lg, targets, loss_mask, prev_correct, step, ttt_step_loss_decay,
                     loss_config=loss_config, target_stats_cache=stats_cache, return_pred=True)
+                if fuse:
+                    logits = lg.logits
                 loss = loss + s_loss
                 metrics.update(s_metrics)
                 # draft tokens: the loss kernel's arg-max for the aligned rows, plus the

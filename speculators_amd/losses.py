@@ -109,6 +109,91 @@ class _FusedLoss(torch.autograd.Function):
         return grad.view(ctx.full_shape), None, None, None, None, None
 
 
+def _packed_row_map(row_grad: torch.Tensor, labels: torch.Tensor | None = None, ignore_index: int = -100):
+    """(row map int32 [rows], live-row count int32 [1]): a row is live when its incoming gradient is
+    non-zero (and its label is not the ignored one); live row r goes to slot ``#live rows before
+    r``, the others to -1.  One small kernel; the count stays on the device."""
+    rows = row_grad.numel()
+    out = torch.empty(rows + 1, device=row_grad.device, dtype=torch.int32)
+    _lib.call("spx_pack_row_map", _lib.ptr(row_grad), _lib.ptr(labels), int(ignore_index), rows,
+              _lib.ptr(out), _lib.ptr(out[rows:]), _lib.stream_ptr(row_grad.device))
+    return out[:rows], out[rows:]
+
+
+def _unpack_rows(packed: torch.Tensor, row_map: torch.Tensor, total_rows: int):
+    """One row per position again: live rows from their packed slot, the others (and the rows past
+    the map, up to ``total_rows``) zero.  Slots past the count are never read."""
+    out = torch.empty(total_rows, packed.shape[1], device=packed.device, dtype=packed.dtype)
+    _lib.call("spx_unpack_rows", _lib.ptr(packed), packed.stride(0), _lib.ptr(row_map), row_map.numel(),
+              total_rows, packed.shape[1], _lib.ptr(out), out.stride(0), _lib.stream_ptr(packed.device))
+    return out
+
+
+class _HeadFusedLoss(torch.autograd.Function):
+    """A frozen ``lm_head`` and the fused vocabulary loss behind it as ONE autograd node:
+    ``(x [T, H], weight [Vd, H], weight_t [H, Vd], targets [n_rows, Vd], op, ...) ->
+    (row loss [n_rows], argmax_draft, argmax_target, lse_target, logits [T, Vd])``.
+
+    Rows the loss mask removes (and the rows past ``n_rows``) have an all-zero logits gradient.
+    With both steps in one node the backward packs the live rows to the front
+    (``spx_fused_vocab_loss_bwd_packed``) and the input-gradient product of the head runs over
+    them only (``spx_gemm_bf16_nt_rows``, count read on the device); dead rows of the result are
+    exact zeros, as they are when the product runs over all rows.  The logits come back for the
+    metrics and the draft tokens and carry no gradient of their own."""
+
+    @staticmethod
+    def forward(ctx, x2, weight, weight_t, targets, op, known_lse_t, known_am_t, n_rows):
+        from .gemm import gemm_nt
+
+        logits = gemm_nt(x2, weight)
+        known = (known_lse_t, known_am_t) if known_lse_t is not None else None
+        loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, logits[:n_rows], targets, known)
+        ctx.save_for_backward(x, None if op == OP_CE else y, lse_d, lse_t, extra, am_t, weight_t)
+        ctx.op, ctx.total_rows = op, logits.shape[0]
+        ctx.mark_non_differentiable(am_d, am_t, lse_t, logits)
+        return loss, am_d, am_t, lse_t, logits
+
+    @staticmethod
+    def backward(ctx, grad_rows, _gd, _gt, _gl, _glogits):
+        from .gemm import gemm_nt
+
+        x, y, lse_d, lse_t, extra, am_t, weight_t = ctx.saved_tensors
+        rows, vocab = x.shape
+        g = grad_rows.reshape(-1).to(torch.float32).contiguous()
+        row_map, count = _packed_row_map(g)
+        packed = torch.empty(rows, vocab, device=x.device, dtype=x.dtype)
+        _lib.call(
+            "spx_fused_vocab_loss_bwd_packed", ctx.op, _lib.ptr(x), x.stride(0), _lib.ptr(y),
+            y.stride(0) if y is not None else 0, rows, vocab, _lib.dtype_code(x),
+            _lib.ptr(lse_d), _lib.ptr(lse_t), _lib.ptr(extra), _lib.ptr(am_t), _lib.ptr(g), None,
+            _lib.ptr(row_map), _lib.ptr(packed), packed.stride(0), _lib.stream_ptr(x.device),
+        )
+        dx_packed = gemm_nt(packed, weight_t, m_live=count)
+        return (_unpack_rows(dx_packed, row_map, ctx.total_rows), None, None, None, None, None,
+                None, None)
+
+
+def head_fused_rows(op: int, x, weight, weight_t, targets, target_stats=None, n_rows=None):
+    """``fused_rows`` with the frozen head in front: ``x [1, T, H]`` instead of logits.  Returns
+    ``(row_loss [1, n_rows], argmax_draft, argmax_target, lse_target, logits [1, T, Vd])``."""
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise _lib.SpxError("head_fused_rows takes bf16 operands")
+    if weight.requires_grad:
+        raise ValueError("head_fused_rows is for a frozen head (no weight gradient is produced)")
+    if x.dim() != 3 or x.shape[0] != 1:
+        raise ValueError("x must be [1, T, H] (the packed batch layout)")
+    t = x.shape[1]
+    n = t if n_rows is None else int(n_rows)
+    y = _rows_2d(targets)
+    if y.shape[0] != n:
+        raise ValueError(f"targets have {y.shape[0]} rows, expected {n}")
+    ks = (None, None) if target_stats is None else (target_stats[0], target_stats[1])
+    loss, am_d, am_t, lse_t, logits = _HeadFusedLoss.apply(x[0], weight, weight_t, y, op, ks[0], ks[1], n)
+    lead = (1, n)
+    return (loss.view(lead), am_d.view(lead), am_t.view(lead), lse_t.view(lead),
+            logits.view(1, t, weight.shape[0]))
+
+
 def fused_rows(op: int, logits, targets, target_stats=None, n_rows=None):
     """(row_loss, argmax_draft, argmax_target, lse_target) of one primitive reduction;
     ``n_rows`` restricts ``logits [1, T, V]`` to its first ``n_rows`` rows (``targets`` already
@@ -281,20 +366,14 @@ class _HeadLabelCE(torch.autograd.Function):
         logits, labels, lse, weight_t = ctx.saved_tensors
         rows, vocab = logits.shape
         g = grad_rows.to(torch.float32).contiguous()
-        live = (labels != ctx.ignore_index) & (g != 0)
-        count = torch.cumsum(live, 0, dtype=torch.int32)
-        row_map = torch.where(live, count - 1, torch.full_like(count, -1))
+        row_map, count = _packed_row_map(g, labels, ctx.ignore_index)
         packed = torch.empty(rows, vocab, device=logits.device, dtype=logits.dtype)
         _lib.call("spx_label_ce_bwd_packed", _lib.ptr(logits), logits.stride(0), _lib.ptr(labels),
                   _lib.ptr(lse), _lib.ptr(g), rows, vocab, _lib.dtype_code(logits), ctx.ignore_index,
                   _lib.ptr(row_map), _lib.ptr(packed), packed.stride(0),
                   _lib.stream_ptr(logits.device))
-        dx_packed = gemm_nt(packed, weight_t, m_live=count[-1:])
-        # back to one row per position: live rows from their packed slot, the others zero (the rows
-        # of dx_packed past the count were never written)
-        dx = dx_packed.index_select(0, row_map.clamp(min=0))
-        dx.masked_fill_(~live.unsqueeze(1), 0)
-        return dx, None, None, None, None
+        dx_packed = gemm_nt(packed, weight_t, m_live=count)
+        return _unpack_rows(dx_packed, row_map, rows), None, None, None, None
 
 
 def head_label_cross_entropy(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor,

@@ -61,6 +61,25 @@ def _step_views(logits, targets, loss_mask, prev_correct, ttt_step):
     )
 
 
+class Head:
+    """The frozen ``lm_head`` applied lazily: ``compute_metrics`` takes this in place of the logits
+    and, when the loss is a single fused HIP reduction, runs head and loss as ONE autograd node (the
+    backward then skips the rows the loss mask removes in the head's input-gradient product,
+    ``losses.head_fused_rows``); otherwise the logits are made the ordinary way.  Either way
+    ``.logits`` holds them afterwards (``[1, T, Vd]``)."""
+
+    def __init__(self, x, weight, weight_t):
+        self.x, self.weight, self.weight_t = x, weight, weight_t
+        self.logits = None
+
+    def materialize(self):
+        from . import gemm
+
+        if self.logits is None:
+            self.logits = gemm.linear(self.x, self.weight, self.weight_t)
+        return self.logits
+
+
 def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
                     ttt_step_loss_decay: float, loss_config: L.LossConfig | None = None,
                     target_stats_cache: dict | None = None, return_pred: bool = False):
@@ -75,10 +94,22 @@ def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
     step, only shifted); ``return_pred=True`` also returns the draft arg-max of the aligned
     rows (int32 ``[T - ttt_step]``).
     """
-    if logits.shape[0] != 1:
-        raise ValueError("the packed batch layout has batch size 1 (train/data.py:306-393)")
     if loss_config is None:
         loss_config = {"kl_div": (L.kl_div_loss, 1.0)}
+    head = None
+    if isinstance(logits, Head):
+        # one node for head + loss only when the whole loss is one fused reduction
+        (name0, (fn0, _w0)), = list(loss_config.items())[:1]
+        single = (len(loss_config) == 1 and name0 in L.PRIMITIVE_OP and fn0 is L._HIP_LOSS_FN_MAP.get(name0)
+                  and logits.x.requires_grad and not logits.weight.requires_grad
+                  and logits.weight_t is not None)
+        if single:
+            head = logits
+            logits = torch.empty(1, head.x.shape[1], 0, device=head.x.device)  # shape carrier only
+        else:
+            logits = logits.materialize()
+    if logits.shape[0] != 1:
+        raise ValueError("the packed batch layout has batch size 1 (train/data.py:306-393)")
     s_logits, s_targets, s_mask, s_prev = _step_views(
         logits, targets, loss_mask, prev_correct, ttt_step)
     dev = logits.device
@@ -109,8 +140,12 @@ def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
                 if full is not None:
                     known = (full[0][ttt_step:], full[1][ttt_step:])
             # the full logits go in with a row count: see _FusedLoss.forward
-            rows, am_d, am_t, lse_t = L.fused_rows(op, logits, s_targets, known,
-                                                   n_rows=s_logits.shape[1])
+            if head is not None:
+                rows, am_d, am_t, lse_t, head.logits = L.head_fused_rows(
+                    op, head.x, head.weight, head.weight_t, s_targets, known, n_rows=s_logits.shape[1])
+            else:
+                rows, am_d, am_t, lse_t = L.fused_rows(op, logits, s_targets, known,
+                                                       n_rows=s_logits.shape[1])
             if (target_stats_cache is not None and known is None and ttt_step == 0
                     and op in (L.OP_KL, L.OP_CE)):
                 target_stats_cache["kl" if op == L.OP_KL else "ce"] = (

@@ -197,3 +197,56 @@ def test_gradient_accumulation_semantics_across_iterations():
     model.zero_grad(set_to_none=True)
     l3 = run()
     assert l3 < l1
+
+
+@pytest.mark.parametrize("loss_fn", ["kl_div", "ce", "tv"])
+def test_head_and_loss_as_one_node_changes_nothing(loss_fn):
+    """lm_head + fused loss as one autograd node (packed loss backward, row-counted head product)
+    against the two-node form: loss, metrics, draft tokens and every parameter gradient bit for bit."""
+    from speculators_amd import losses as L
+
+    shape = _shape(num_hidden_layers=2)
+    w = {k: v.bfloat16() for k, v in OE.random_weights(shape, seed=1, std=0.05).items()}
+    t = 300
+    hs, ids, doc, mask, pos, vl = _batch(shape, t, 3, [120, 140])
+    mask[0, :7] = 0  # a dead run at the start
+    got = []
+    for fuse in (True, False):
+        model = _make(shape, w)
+        model.fuse_head_loss = fuse
+        toks, loss, metrics = model(
+            hs.bfloat16().cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.bfloat16().cuda(),
+            ttt_steps=3, ttt_step_loss_decay=0.8, loss_config=L.resolve_loss_config(loss_fn))
+        loss.backward()
+        got.append((loss.detach(), [x.clone() for x in toks], {k: v.clone() for k, v in metrics.items()},
+                    {k: p.grad.clone() for k, p in model.named_parameters() if p.grad is not None}))
+    assert torch.equal(got[0][0], got[1][0])
+    for a, b in zip(got[0][1], got[1][1]):
+        assert torch.equal(a, b)
+    assert got[0][2].keys() == got[1][2].keys()
+    for k in got[0][2]:
+        assert torch.equal(got[0][2][k], got[1][2][k]), k
+    assert got[0][3].keys() == got[1][3].keys() and len(got[0][3]) > 5
+    for k in got[0][3]:
+        assert torch.equal(got[0][3][k], got[1][3][k]), k
+
+
+def test_head_node_falls_back_for_compound_losses():
+    """A weighted sum of losses keeps the two-node form (the logits feed several reductions)."""
+    from speculators_amd import losses as L
+
+    shape = _shape()
+    w = {k: v.bfloat16() for k, v in OE.random_weights(shape, seed=2, std=0.05).items()}
+    hs, ids, doc, mask, pos, vl = _batch(shape, 200, 4, [200])
+    got = []
+    for fuse in (True, False):
+        model = _make(shape, w)
+        model.fuse_head_loss = fuse
+        _, loss, _ = model(hs.bfloat16().cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(),
+                           vl.bfloat16().cuda(), ttt_steps=2,
+                           loss_config=L.resolve_loss_config('{"ce": 0.3, "tv": 0.7}'))
+        loss.backward()
+        got.append((loss.detach(), {k: p.grad.clone() for k, p in model.named_parameters() if p.grad is not None}))
+    assert torch.equal(got[0][0], got[1][0])
+    for k in got[0][1]:
+        assert torch.equal(got[0][1][k], got[1][1][k]), k

@@ -204,3 +204,36 @@ def test_gate_up_swiglu_matches_separate_projections(t, h, f):
     _close(out, ref.detach().cpu(), rel=1e-2)
     for a, b in zip(got, (x.grad, wg.grad, wu.grad), strict=True):
         _close(a, b.cpu())
+
+
+@pytest.mark.parametrize("rows", [1, 63, 64, 1024, 1025, 5000])
+@pytest.mark.parametrize("with_labels", [False, True])
+def test_pack_row_map_and_unpack_rows(rows, with_labels):
+    """Row map of the live rows (bit-exact against a running count) and the way back from packed rows."""
+    from speculators_amd import _lib
+
+    g = torch.Generator().manual_seed(rows)
+    grad = torch.rand(rows, generator=g)
+    grad[torch.rand(rows, generator=g) < 0.3] = 0.0
+    labels = torch.randint(0, 50, (rows,), generator=g)
+    labels[torch.rand(rows, generator=g) < 0.2] = -100
+    live = grad != 0
+    if with_labels:
+        live &= labels != -100
+    want = torch.where(live, torch.cumsum(live, 0) - 1, torch.full((rows,), -1)).to(torch.int32)
+
+    gd, ld = grad.cuda(), labels.cuda()
+    out = torch.empty(rows + 1, dtype=torch.int32, device="cuda")
+    _lib.call("spx_pack_row_map", _lib.ptr(gd), _lib.ptr(ld) if with_labels else None, -100, rows,
+              _lib.ptr(out), _lib.ptr(out[rows:]), _lib.stream_ptr(gd.device))
+    assert torch.equal(out[:rows].cpu(), want) and int(out[rows]) == int(live.sum())
+
+    cols, total = 72, rows + 3
+    packed = torch.randn(rows, cols, generator=g).bfloat16().cuda()
+    packed[int(live.sum()):] = float("nan")  # slots past the count must never be read
+    back = torch.full((total, 80), 5.0, dtype=torch.bfloat16, device="cuda")
+    _lib.call("spx_unpack_rows", _lib.ptr(packed), packed.stride(0), _lib.ptr(out), rows, total, cols,
+              _lib.ptr(back), back.stride(0), _lib.stream_ptr(gd.device))
+    ref = torch.zeros(total, cols, dtype=torch.bfloat16)
+    ref[:rows][live] = packed.cpu()[want[live].long()]
+    assert torch.equal(back[:, :cols].cpu(), ref) and (back[:, cols:] == 5).all()
