@@ -167,6 +167,9 @@ class DFlashDraftModel(nn.Module):
         self.uses_sliding_window_attn = bool(config.sliding_layers)
         self.uses_full_attn = config.num_hidden_layers > len(config.sliding_layers)
         self._frozen_t: dict = {}
+        # lm_head and the loss as one autograd node while the head is frozen and the loss is a single
+        # fused reduction (False: always two nodes)
+        self.fuse_head_loss = True
 
     @property
     def mask_token_id(self) -> int:
@@ -176,17 +179,19 @@ class DFlashDraftModel(nn.Module):
                 "ensure the config was saved with mask_token_id set.")
         return self.config.mask_token_id
 
+    def _transposed_frozen(self, weight):
+        """``weight.T`` contiguous, cached: frozen weights never change between steps."""
+        key = (weight.data_ptr(), weight._version)
+        hit = self._frozen_t.get(id(weight))
+        if hit is None or hit[0] != key:
+            hit = (key, weight.detach().t().contiguous())
+            self._frozen_t[id(weight)] = hit
+        return hit[1]
+
     def _linear(self, x, weight, frozen=False):
         if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
             raise RuntimeError("the HIP draft path runs in bf16: cast the model and its inputs to bfloat16")
-        wt = None
-        if frozen and x.requires_grad:
-            key = (weight.data_ptr(), weight._version)
-            hit = self._frozen_t.get(id(weight))
-            if hit is None or hit[0] != key:
-                hit = (key, weight.detach().t().contiguous())
-                self._frozen_t[id(weight)] = hit
-            wt = hit[1]
+        wt = self._transposed_frozen(weight) if frozen and x.requires_grad else None
         return gemm.linear(x, weight, wt)
 
     def forward(self, hidden_states, input_ids, loss_mask, verifier_last_hidden_states,
@@ -233,7 +238,12 @@ class DFlashDraftModel(nn.Module):
             noise, normed = layer(noise, ctx, q_pos, kv_pos, inv_freq,
                                   sw_mask if li in cfg.sliding_layers else full_mask,
                                   x_normed=normed, next_norm=nxt)
-        logits = self._linear(normed, self.lm_head.weight, frozen=True)
+        if (self.fuse_head_loss and normed.requires_grad and not self.lm_head.weight.requires_grad
+                and normed.dtype == torch.bfloat16 and self.lm_head.weight.dtype == torch.bfloat16):
+            # head + loss as one autograd node while the head is frozen (see metrics.Head)
+            logits = MT.Head(normed, self.lm_head.weight, self._transposed_frozen(self.lm_head.weight))
+        else:
+            logits = self._linear(normed, self.lm_head.weight, frozen=True)
         aligned = loss_mask.clone()[:, block_idx]
         aligned = aligned * anchor_valid.repeat_interleave(bs).unsqueeze(0).to(aligned.dtype)
         if not cfg.sample_from_anchor:

@@ -246,9 +246,20 @@ def dflash_compute_metrics(logits, targets, loss_mask, block_size: int = 1, gamm
                            loss_config: L.LossConfig | None = None,
                            per_position_loss_weight: str = "fixed-exp-decay",
                            dpace_alpha: float = 0.5, sample_from_anchor: bool = False):
-    """DFlash loss + per-slot accuracy + EAL; contract of models/dflash/metrics.py:20-108."""
+    """DFlash loss + per-slot accuracy + EAL; contract of models/dflash/metrics.py:20-108.
+    ``logits`` may be a ``Head`` (see ``compute_metrics``)."""
     if loss_config is None:
         loss_config = {"kl_div": (L.kl_div_loss, 1.0)}
+    head = None
+    if isinstance(logits, Head):
+        (name0, (fn0, _w0)), = list(loss_config.items())[:1]
+        if (len(loss_config) == 1 and name0 in L.PRIMITIVE_OP and fn0 is L._HIP_LOSS_FN_MAP.get(name0)
+                and logits.x.requires_grad and not logits.weight.requires_grad
+                and logits.weight_t is not None):
+            head = logits
+            logits = torch.empty(1, head.x.shape[1], 0, device=head.x.device)  # shape carrier only
+        else:
+            logits = logits.materialize()
     dev = logits.device
     n = logits.shape[1]
     mask1 = _as_mask(loss_mask)
@@ -259,7 +270,10 @@ def dflash_compute_metrics(logits, targets, loss_mask, block_size: int = 1, gamm
     correct = total = None
     for ti, (name, (fn, w)) in enumerate(loss_config.items()):
         op = L.PRIMITIVE_OP.get(name)
-        if fn is L._HIP_LOSS_FN_MAP.get(name) and op is not None:
+        if head is not None:
+            rows, am_d, am_t, _, head.logits = L.head_fused_rows(
+                op, head.x, head.weight, head.weight_t, targets)
+        elif fn is L._HIP_LOSS_FN_MAP.get(name) and op is not None:
             rows, am_d, am_t, _ = L.fused_rows(op, logits, targets)
         else:
             rows = fn(logits, targets)

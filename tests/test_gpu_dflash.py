@@ -211,3 +211,45 @@ def test_full_size_sampled_rows():
 
     _check_sampled_rows(q, k, v, out, go, rows, heads, visible, d ** -0.5)
     _check_dv_checksum(v, go, hq)
+
+
+@pytest.mark.parametrize("weighting,loss_name", [("fixed-exp-decay", "kl_div"), ("dpace", "ce")])
+def test_head_and_loss_as_one_node_changes_nothing(weighting, loss_name):
+    """lm_head + fused loss as one autograd node against the two-node form: loss, metrics and every
+    parameter gradient bit for bit."""
+    from speculators_amd import losses as L
+    from speculators_amd.dflash import DFlashConfig, DFlashDraftModel
+
+    kw = dict(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=64,
+              intermediate_size=512, vocab_size=2000, draft_vocab_size=704, num_aux=2,
+              num_hidden_layers=2, rms_norm_eps=1e-6, rope_theta=10000.0)
+    shape = DraftShape(qk_norm=True, **kw)
+    w = {k_: v.bfloat16() for k_, v in OD.random_weights(shape, seed=6, std=0.05).items()}
+    g = torch.Generator().manual_seed(13)
+    t, bs = 256, 8
+    hs = torch.randn(1, t, 2 * 256, generator=g).bfloat16()
+    ids = torch.randint(0, 2000, (1, t), generator=g)
+    vl = torch.randn(1, t, 256, generator=g).bfloat16()
+    mask = (torch.rand(1, t, generator=g) < 0.6).float()
+    doc = _docs(t, [100, 156]).unsqueeze(0)
+    pos = torch.cat([torch.arange(100), torch.arange(156)]).unsqueeze(0)
+    anchors = OD.select_anchors(mask, 20, bs, g)
+    got = []
+    for fuse in (True, False):
+        model = DFlashDraftModel(DFlashConfig(block_size=bs, mask_token_id=7, **kw))
+        model.load_state_dict(w, strict=False)
+        model = model.to(torch.bfloat16).cuda()
+        model.fuse_head_loss = fuse
+        _, loss, m = model(hs.cuda(), ids.cuda(), mask.cuda(), vl.cuda(), doc.cuda(), pos.cuda(),
+                           loss_config=L.resolve_loss_config(loss_name), gamma=4.0,
+                           per_position_loss_weight=weighting, dpace_alpha=0.5,
+                           anchors=(anchors[0].cuda(), anchors[1].cuda()))
+        loss.backward()
+        got.append((loss.detach(), {k_: v.clone() for k_, v in m.items()},
+                    {k_: p.grad.clone() for k_, p in model.named_parameters() if p.grad is not None}))
+    assert torch.equal(got[0][0], got[1][0])
+    for k_ in got[0][1]:
+        assert torch.equal(got[0][1][k_], got[1][1][k_]), k_
+    assert got[0][2].keys() == got[1][2].keys() and len(got[0][2]) > 5
+    for k_ in got[0][2]:
+        assert torch.equal(got[0][2][k_], got[1][2][k_]), k_
