@@ -16,7 +16,7 @@ import torch
 
 from . import _lib
 
-_MAX_SPAN = 0x7ffffff0 - 64  # bytes one GEMM operand may span
+_MAX_SPAN = 0x7ffffff0 - 64  # bytes an operand of the weight-gradient product (gemm_tn) may span per call
 
 
 def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
