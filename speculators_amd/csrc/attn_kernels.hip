@@ -1153,38 +1153,34 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
   auto swz_t = [](int r) { return CKT == 8 ? (r >> 1) & 7 : (r >> 2) & 3; };
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)sm8;
   u32x4 qres, dres, qtres, dtres;
-  int r_row[kDma ? LPR : 1], r_col[kDma ? LPR : 1], t_off[kDma ? LPT : 1];
   if constexpr (kDma) {
     qres = make_rsrc(Qh, (uint32_t)((int64_t)p.NQ * RBQ));
     dres = make_rsrc(dO + (int64_t)h * D, (uint32_t)((((int64_t)p.NQ - 1) * p.Hq * D + D) * 2));
     qtres = make_rsrc(Qth, (uint32_t)((int64_t)D * NQp * 2));
     dtres = make_rsrc(dOth, (uint32_t)((int64_t)D * NQp * 2));
-#pragma unroll
-    for (int j = 0; j < LPR; ++j) {
-      const int r = (wave * LPR + j) * (1024 / RBQ) + lane / CKQ;
-      r_row[j] = r;
-      r_col[j] = ((lane % CKQ) ^ swz_r(r)) * 16;
-    }
-#pragma unroll
-    for (int j = 0; j < LPT; ++j) {
-      const int r = (wave * LPT + j) * (1024 / RBT) + lane / CKT;
-      t_off[j] = r * NQp * 2 + ((lane % CKT) ^ swz_t(r)) * 16;
-    }
   }
   auto issue = [&](int mq, int b) __attribute__((always_inline)) {
     if constexpr (kDma) {
+      // per-load offsets recomputed here on purpose: hoisted out of the tile loop they cost registers that
+      // the two-workgroups-per-CU build does not have
+      int lane_v = lane;
+      if (SPX_DKV_REMAT) asm volatile("" : "+v"(lane_v));
       const uint32_t rb = lds0 + b * SM::kBuf + wave * LPR * 1024;
 #pragma unroll
       for (int j = 0; j < LPR; ++j) {
-        const int ir = min(mq + r_row[j], p.NQ - 1);
-        load_to_lds16<0>(qres, rb + j * 1024, ir * RBQ + r_col[j], 0);
-        if (kDoK) load_to_lds16<0>(dres, rb + SM::kOffdO + j * 1024, ir * (p.Hq * RBQ) + r_col[j], 0);
+        const int r = (wave * LPR + j) * (1024 / RBQ) + lane_v / CKQ;
+        const int cofs = ((lane_v % CKQ) ^ swz_r(r)) * 16;
+        const int ir = min(mq + r, p.NQ - 1);
+        load_to_lds16<0>(qres, rb + j * 1024, ir * RBQ + cofs, 0);
+        if (kDoK) load_to_lds16<0>(dres, rb + SM::kOffdO + j * 1024, ir * (p.Hq * RBQ) + cofs, 0);
       }
       const uint32_t tb2 = lds0 + b * SM::kBuf + wave * LPT * 1024;
 #pragma unroll
       for (int j = 0; j < LPT; ++j) {
-        if (kDoK) load_to_lds16<0>(qtres, tb2 + SM::kOffQt + j * 1024, t_off[j], mq * 2);
-        if (kDoV) load_to_lds16<0>(dtres, tb2 + SM::kOffdOt + j * 1024, t_off[j], mq * 2);
+        const int r = (wave * LPT + j) * (1024 / RBT) + lane_v / CKT;
+        const int tofs = r * NQp * 2 + ((lane_v % CKT) ^ swz_t(r)) * 16;
+        if (kDoK) load_to_lds16<0>(qtres, tb2 + SM::kOffQt + j * 1024, tofs, mq * 2);
+        if (kDoV) load_to_lds16<0>(dtres, tb2 + SM::kOffdOt + j * 1024, tofs, mq * 2);
       }
     }
   };
