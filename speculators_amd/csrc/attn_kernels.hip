@@ -108,25 +108,41 @@ __global__ __launch_bounds__(256) void dflash_ranges_kernel(
 // (a multiple of 16), the columns of r in rows..ld_dst-1 are zero filled.  perm swaps bits
 // 2 and 3 of r: inside every group of 16 the order is 0-3, 8-11, 4-7, 12-15, which puts
 // the 8 rows a lane half needs as MFMA k-slots (4 g + 0..3 and 8 + 4 g + 0..3) side by
-// side, so that operand is ONE 16-byte LDS read.  64x64 tiles through LDS.
-__global__ __launch_bounds__(256) void transpose_bf16_kernel(
+// side, so that operand is ONE 16-byte LDS read.
+// One wave per 64 x 64 tile, no LDS: a lane loads an 8 (r) x 8 (c) block with eight 16-byte row loads
+// (eight lanes read a whole 128-byte line), transposes it in registers (v_perm_b32) and writes, for each
+// of its 8 columns, the two 4-row halves of the block to their permuted places (8 bytes each; the eight
+// lanes that share a column fill its 128-byte line in two store instructions).  cols a multiple of 8.
+__global__ __launch_bounds__(64) void transpose_bf16_kernel(
     const uint16_t* __restrict__ src, int64_t src_hs, int64_t src_ld, int rows, int cols,
     uint16_t* __restrict__ dst, int64_t dst_hs, int64_t ld_dst) {
-  __shared__ uint16_t tile[64][66];
   const int h = blockIdx.z;
-  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
-  const uint16_t* s = src + (int64_t)h * src_hs;
-  uint16_t* d = dst + (int64_t)h * dst_hs;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-  for (int rr = ty; rr < 64; rr += 4) {
-    int r = r0 + rr, c = c0 + tx;
-    tile[rr][tx] = (r < rows && c < cols) ? s[(int64_t)r * src_ld + c] : (uint16_t)0;
+  const int lane = threadIdx.x;
+  const int rb = lane >> 3, cb = lane & 7;
+  const int r0 = blockIdx.x * 64 + rb * 8, c0 = blockIdx.y * 64 + cb * 8;
+  if (c0 >= cols) return;
+  const uint16_t* s = src + (int64_t)h * src_hs + c0;
+  u32x4 in[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const u32x4 z = {0, 0, 0, 0};
+    in[j] = (r0 + j < rows) ? *reinterpret_cast<const u32x4*>(s + (int64_t)(r0 + j) * src_ld) : z;
   }
-  __syncthreads();
-  for (int cc = ty; cc < 64; cc += 4) {
-    int c = c0 + cc, r = r0 + tx;
-    const int rp = (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);
-    if (c < cols && r < ld_dst) d[(int64_t)c * ld_dst + rp] = tile[tx][cc];
+  // where the block's two halves go: r0 % 16 == 0 -> r0 and r0 + 8, r0 % 16 == 8 -> r0 - 4 and r0 + 4
+  const int p_lo = (r0 & 8) ? r0 - 4 : r0, p_hi = (r0 & 8) ? r0 + 4 : r0 + 8;
+  uint16_t* d = dst + (int64_t)h * dst_hs + (int64_t)c0 * ld_dst;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    // column c0 + i of the block: element e = in[e] element i
+    const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
+    const int w = i >> 1;
+    u32x2 lo, hi;
+    lo.x = __builtin_amdgcn_perm(in[1][w], in[0][w], sel);
+    lo.y = __builtin_amdgcn_perm(in[3][w], in[2][w], sel);
+    hi.x = __builtin_amdgcn_perm(in[5][w], in[4][w], sel);
+    hi.y = __builtin_amdgcn_perm(in[7][w], in[6][w], sel);
+    *reinterpret_cast<u32x2*>(d + (int64_t)i * ld_dst + p_lo) = lo;
+    *reinterpret_cast<u32x2*>(d + (int64_t)i * ld_dst + p_hi) = hi;
   }
 }
 
@@ -1543,7 +1559,7 @@ static int launch_fwd(AttnParams p, void* workspace, uint16_t* O, float* lse, hi
                       const char* fn) {
   uint16_t* vt = reinterpret_cast<uint16_t*>(workspace);
   dim3 tgrid((unsigned)(p.NKVp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hkv);
-  hipLaunchKernelGGL(transpose_bf16_kernel, tgrid, dim3(256), 0, st, p.V, p.v_hs, (int64_t)D, p.NKV, D,
+  hipLaunchKernelGGL(transpose_bf16_kernel, tgrid, dim3(64), 0, st, p.V, p.v_hs, (int64_t)D, p.NKV, D,
                      vt, (int64_t)D * p.NKVp, (int64_t)p.NKVp);
   constexpr int BM = 32 * kFwdNSB * kFwdNW;
   const int n_qb = (p.NQ + BM - 1) / BM;
@@ -1587,12 +1603,12 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   float* dvp = reinterpret_cast<float*>(w);
 
   dim3 tgrid((unsigned)(p.NKVp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hkv);
-  hipLaunchKernelGGL(transpose_bf16_kernel, tgrid, dim3(256), 0, st, p.K, p.k_hs, (int64_t)D, p.NKV, D,
+  hipLaunchKernelGGL(transpose_bf16_kernel, tgrid, dim3(64), 0, st, p.K, p.k_hs, (int64_t)D, p.NKV, D,
                      kt, (int64_t)D * p.NKVp, (int64_t)p.NKVp);
   dim3 qgrid((unsigned)(NQp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hq);
-  hipLaunchKernelGGL(transpose_bf16_kernel, qgrid, dim3(256), 0, st, p.Q, p.q_hs, (int64_t)D, p.NQ, D,
+  hipLaunchKernelGGL(transpose_bf16_kernel, qgrid, dim3(64), 0, st, p.Q, p.q_hs, (int64_t)D, p.NQ, D,
                      qt, (int64_t)D * NQp, (int64_t)NQp);
-  hipLaunchKernelGGL(transpose_bf16_kernel, qgrid, dim3(256), 0, st, dOp, (int64_t)D,
+  hipLaunchKernelGGL(transpose_bf16_kernel, qgrid, dim3(64), 0, st, dOp, (int64_t)D,
                      (int64_t)p.Hq * D, p.NQ, D, dot, (int64_t)D * NQp, (int64_t)NQp);
   hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)(((int64_t)p.NQ * p.Hq + 15) / 16)), dim3(256),
                      0, st, Op, dOp, p.NQ, p.Hq, delta);
