@@ -675,13 +675,29 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const uint16_t* __restr
 
 // dQ: same tiling as the forward.
 //   P^T = exp2(S'^T - lse), dP^T = V dO^T, dS^T = P^T (dP^T - delta), dQ^T += K^T dS^T
-template <int D, int NSB, int NW, bool PF>
+// PF: how a key tile reaches LDS: 0 through registers at the point of use, 1 through registers one tile
+// ahead, 3 global -> LDS directly into the other of two buffers, with tiles of 32 instead of 64 keys so
+// that two buffers of the three tiles (K, V, K^T) fit beside a second workgroup (see FwdSmem).
+template <int D, int NW, int PF>
+struct DqSmem {
+  static constexpr int TB = PF == 3 ? 32 : kBN;                      // keys per tile
+  static constexpr int KS = D + kKPad, VS = kBN + kVPad;
+  static constexpr int kTileK = TB * D * 2, kTileT = D * TB * 2;     // mode 3: unpadded, swizzled
+  static constexpr int kBuf = 2 * kTileK + kTileT;
+  static constexpr int kTiles = PF == 3 ? 2 * kBuf : (2 * kBN * KS + D * VS) * 2;
+  static constexpr int kBytes = kTiles + 4 * NW * (int)sizeof(int);
+};
+
+template <int D, int NSB, int NW, int PF>
 __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_dq_kernel(
     AttnParams p, const uint16_t* __restrict__ dO, const uint16_t* __restrict__ Kt,
     const float* __restrict__ LSE, const float* __restrict__ Delta, uint16_t* __restrict__ dQ,
     int64_t dq_hs) {
-  constexpr int KS = D + kKPad;
-  constexpr int VS = kBN + kVPad;
+  using SM = DqSmem<D, NW, PF>;
+  constexpr bool kDma = PF == 3;
+  constexpr int TB = SM::TB;
+  constexpr int KS = SM::KS;
+  constexpr int VS = SM::VS;
   constexpr int NKK = D / 16;
   constexpr int NDB = D / 32;
   constexpr int NT = 64 * NW;
@@ -689,10 +705,11 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
   constexpr int BMW = 32 * NSB;
   constexpr int BM = NW * BMW;
 
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[kBN * KS];
-  __shared__ __attribute__((aligned(16))) uint16_t Vn[kBN * KS];
-  __shared__ __attribute__((aligned(16))) uint16_t Kts[D * VS];
-  __shared__ int red[4 * NW];
+  extern __shared__ __attribute__((aligned(16))) uint8_t dq_smem[];
+  uint16_t* const Ks = reinterpret_cast<uint16_t*>(dq_smem);
+  uint16_t* const Vn = Ks + kBN * KS;
+  uint16_t* const Kts = Vn + kBN * KS;
+  int* const red = reinterpret_cast<int*>(dq_smem + SM::kTiles);
 
   const int group = p.Hq / p.Hkv;
   const int L = blockIdx.x;
@@ -786,24 +803,74 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
     }
   };
 
+  // ---- mode 3: the three tiles as 1 KB wave loads global -> LDS (chunk c of row r in slot c ^ swz(r))
+  constexpr int RBK = D * 2, CKK = RBK / 16;   // bytes / 16-byte chunks per row of K and V
+  constexpr int RBT = TB * 2, CKT = RBT / 16;  // ... of K^T
+  constexpr int LPK = (TB * RBK / 1024) / NW, LPT = (D * RBT / 1024) / NW;
+  auto swz_k = [](int r) { return CKK == 8 ? (r >> 1) & 7 : r & 15; };
+  auto swz_t = [](int r) { return CKT == 8 ? (r >> 1) & 7 : (r >> 2) & 3; };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)dq_smem;
+  u32x4 kres, vres, tres;
+  if constexpr (kDma) {
+    static_assert(!kDma || (LPK >= 1 && LPT >= 1), "a tile is at least one 1 KB load per wave");
+    kres = make_rsrc(Kh, (uint32_t)((int64_t)p.NKV * RBK));
+    vres = make_rsrc(Vh, (uint32_t)((int64_t)p.NKV * RBK));
+    tres = make_rsrc(Kth, (uint32_t)((int64_t)D * p.NKVp * 2));
+  }
+  auto issue = [&](int n0, int b) __attribute__((always_inline)) {
+    if constexpr (kDma) {
+      int lane_v = lane;
+      if (SPX_DKV_REMAT) asm volatile("" : "+v"(lane_v));  // offsets recomputed per tile, not kept live
+      const uint32_t kb0 = lds0 + b * SM::kBuf + wave * LPK * 1024;
+#pragma unroll
+      for (int j = 0; j < LPK; ++j) {
+        const int r = (wave * LPK + j) * (1024 / RBK) + lane_v / CKK;
+        const int off = min(n0 + r, last_row) * RBK + ((lane_v % CKK) ^ swz_k(r)) * 16;
+        load_to_lds16<0>(kres, kb0 + j * 1024, off, 0);
+        load_to_lds16<0>(vres, kb0 + SM::kTileK + j * 1024, off, 0);
+      }
+      const uint32_t tb0 = lds0 + b * SM::kBuf + 2 * SM::kTileK + wave * LPT * 1024;
+#pragma unroll
+      for (int j = 0; j < LPT; ++j) {
+        const int r = (wave * LPT + j) * (1024 / RBT) + lane_v / CKT;
+        load_to_lds16<0>(tres, tb0 + j * 1024, r * p.NKVp * 2 + ((lane_v % CKT) ^ swz_t(r)) * 16, n0 * 2);
+      }
+    }
+  };
+  const int rdk = col * RBK + ((g ^ swz_k(col)) * 16);
+  const int rdt = col * RBT + ((g ^ swz_t(col)) * 16);
+
   auto run_pass = [&](const int (&aa)[NSB], const int (&bb)[NSB], int w_amin, int w_amax,
                       int w_bmin, int w_bmax, int blk_a, int blk_b) {
     if (blk_b <= blk_a) return;
-    const int n_begin = (blk_a / kBN) * kBN;
-    if (PF) fetch(n_begin);
-    for (int n0 = n_begin; n0 < blk_b; n0 += kBN) {
-      __syncthreads();
-      if (PF) stash(); else direct(n0);
-      __syncthreads();
-      if (PF && n0 + kBN < blk_b) fetch(n0 + kBN);
-      if (n0 >= w_bmax || n0 + kBN <= w_amin) continue;
+    const int n_begin = (blk_a / TB) * TB;
+    if (PF == 1) fetch(n_begin);
+    int buf = 0;
+    if constexpr (kDma) {
+      __syncthreads();  // a previous pass may still be reading either buffer
+      issue(n_begin, 0);
+    }
+    for (int n0 = n_begin; n0 < blk_b; n0 += TB) {
+      if constexpr (kDma) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (n0 + TB < blk_b) issue(n0 + TB, buf ^ 1);
+      } else {
+        __syncthreads();
+        if (PF) stash(); else direct(n0);
+        __syncthreads();
+        if (PF && n0 + kBN < blk_b) fetch(n0 + kBN);
+      }
+      const uint8_t* const tile = dq_smem + buf * SM::kBuf;
+      buf ^= 1;
+      if (n0 >= w_bmax || n0 + TB <= w_amin) continue;
 
-      const bool need_mask = (n0 < w_amax) || (n0 + kBN > w_bmin);
+      const bool need_mask = (n0 < w_amax) || (n0 + TB > w_bmin);
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb) {
-        // the two 32-key halves of the tile one after the other: 32 score registers live
+        // the 32-key halves of the tile one after the other: 32 score registers live
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int kb = 0; kb < TB / 32; ++kb) {
           f32x16 st, dp;
 #pragma unroll
           for (int r = 0; r < 16; ++r) { st[r] = 0.f; dp[r] = 0.f; }
@@ -814,9 +881,14 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
             constexpr int NF = 2 * NKK;
             bf16x8 fr[4];
             auto fread = [&](int f) {
-              const uint16_t* base = (f & 1) ? Vn : Ks;
-              fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-                  &base[(kb * 32 + col) * KS + g * 8 + (f >> 1) * 16]));
+              if constexpr (kDma) {
+                fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                    tile + ((f & 1) ? SM::kTileK : 0) + kb * 32 * RBK + (rdk ^ ((f >> 1) * 32))));
+              } else {
+                const uint16_t* base = (f & 1) ? Vn : Ks;
+                fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                    &base[(kb * 32 + col) * KS + g * 8 + (f >> 1) * 16]));
+              }
             };
 #pragma unroll
             for (int f = 0; f < 4; ++f) fread(f);
@@ -851,8 +923,12 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
             constexpr int NF = 2 * NDB;
             bf16x8 fr[4];
             auto fread = [&](int f) {
-              fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-                  &Kts[((f % NDB) * 32 + col) * VS + (kb * 2 + f / NDB) * 16 + 8 * g]));
+              if constexpr (kDma)
+                fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                    tile + 2 * SM::kTileK + (f % NDB) * 32 * RBT + (rdt ^ ((kb * 2 + f / NDB) * 32))));
+              else
+                fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                    &Kts[((f % NDB) * 32 + col) * VS + (kb * 2 + f / NDB) * 16 + 8 * g]));
             };
 #pragma unroll
             for (int f = 0; f < 4 && f < NF; ++f) fread(f);
@@ -1517,7 +1593,7 @@ static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 #define SPX_FWD_CFG 1, 4, 2
 #endif
 #ifndef SPX_DQ_CFG
-#define SPX_DQ_CFG 1, 4, false
+#define SPX_DQ_CFG 1, 4, 3
 #endif
 // head_dim 256: the next tile is prefetched into registers as well; the few registers that
 // spill cost far less than exposing the global-load latency with one workgroup per CU
@@ -1525,7 +1601,7 @@ static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 #define SPX_FWD256_PF 2
 #endif
 #ifndef SPX_DQ256_PF
-#define SPX_DQ256_PF true
+#define SPX_DQ256_PF 3
 #endif
 #ifndef SPX_DKV_CFG
 #define SPX_DKV_CFG 4, 2
@@ -1538,7 +1614,7 @@ constexpr int cfg_pf(int, int, int pf) { return pf; }
 constexpr int cfg_nw(int nw, int) { return nw; }
 constexpr int cfg_pf(int, int pf) { return pf; }
 constexpr int kFwdNSB = cfg_nsb(SPX_FWD_CFG), kFwdNW = cfg_nw(SPX_FWD_CFG), kFwdPF = cfg_pf(SPX_FWD_CFG);
-constexpr int kDqNSB = cfg_nsb(SPX_DQ_CFG), kDqNW = cfg_nw(SPX_DQ_CFG);
+constexpr int kDqNSB = cfg_nsb(SPX_DQ_CFG), kDqNW = cfg_nw(SPX_DQ_CFG), kDqPF = cfg_pf(SPX_DQ_CFG);
 constexpr int kDkvNW = cfg_nw(SPX_DKV_CFG), kDkvPF = cfg_pf(SPX_DKV_CFG);
 
 static int64_t fwd_workspace_bytes(int64_t NKV, int Hkv, int D) {
@@ -1616,12 +1692,27 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
 
   constexpr int BM = 32 * kDqNSB * kDqNW;
   const int n_qb = (p.NQ + BM - 1) / BM;
-  if constexpr (D > 128)
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<D, kDqNSB, kDqNW, SPX_DQ256_PF>), dim3((unsigned)(n_qb * p.Hq)),
-                       dim3(64 * kDqNW), 0, st, p, dOp, kt, lse, delta, dQp, dq_hs);
-  else
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<D, SPX_DQ_CFG>), dim3((unsigned)(n_qb * p.Hq)),
-                       dim3(64 * kDqNW), 0, st, p, dOp, kt, lse, delta, dQp, dq_hs);
+  {
+    constexpr int kDqPFd = D > 128 ? (int)SPX_DQ256_PF : kDqPF;
+    constexpr int dq_smem = DqSmem<D, kDqNW, kDqPFd>::kBytes;
+    if (kDqPFd == 3 && ((int64_t)p.NKV * D * 2 >= (1ll << 31) || (int64_t)D * p.NKVp * 2 >= (1ll << 31))) {
+      last_error() = std::string(fn) + ": keys of one head must span less than 2 GiB";
+      return SPX_ERR_ARG;
+    }
+    static bool dq_attr_set = false;  // one flag per head_dim instantiation
+    if (!dq_attr_set) {
+      hipError_t e = hipFuncSetAttribute(
+          reinterpret_cast<const void*>(&attn_bwd_dq_kernel<D, kDqNSB, kDqNW, kDqPFd>),
+          hipFuncAttributeMaxDynamicSharedMemorySize, dq_smem);
+      if (e != hipSuccess) {
+        last_error() = std::string(fn) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
+        return SPX_ERR_HIP;
+      }
+      dq_attr_set = true;
+    }
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<D, kDqNSB, kDqNW, kDqPFd>), dim3((unsigned)(n_qb * p.Hq)),
+                       dim3(64 * kDqNW), dq_smem, st, p, dOp, kt, lse, delta, dQp, dq_hs);
+  }
 
   constexpr int kPF = D > 128 ? 1 : kDkvPF;
   constexpr int kPF1 = SPX_DKV256_PF1, kPF2 = SPX_DKV256_PF2;
