@@ -32,12 +32,12 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # --seq-len / --ttt-steps; other shapes report null.
 KIB = 1024
 MEASURED_TRAFFIC = {
-    "gemm_fwd": int((1.9998 * 922144 + 256584) * KIB),
-    "gemm_dx": int((1.9998 * 768453 + 32834) * KIB),
+    "gemm_fwd": int((1.9998 * 954294 + 256566) * KIB),
+    "gemm_dx": int((1.9998 * 768419 + 32833) * KIB),
     "loss_fwd": int((1.9998 * 256051 + 768) * KIB),
     "loss_fwd_reuse": int((1.9998 * 256166 + 512) * KIB),
     "loss_bwd": int((1.9998 * 256416 + 256000) * KIB),
-    "attn_fwd": int((1.9998 * 78191 + 33280) * KIB),
+    "attn_fwd": int((1.9998 * 78162 + 33280) * KIB),
 }
 
 CONFIG1 = dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
