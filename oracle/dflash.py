@@ -8,8 +8,13 @@ the anchor helpers of models/dflash/utils.py:6-67.
 Pinned by: index-helper known answers and the sortedness of sampled anchors
 (tests/unit/models/test_dflash_utils.py:12-59), the targets alignment rule
 ``targets == roll(full_logits, 1)[:, idx]``
-(tests/unit/models/test_dflash_targets.py:37-63), the mask brute force, and
-dense attention == SDPA.  ``select_anchors`` consumes torch's RNG stream the way
+(tests/unit/models/test_dflash_targets.py:37-63), the mask brute force,
+dense attention == SDPA; the layer against the HF Qwen3 library blocks wired like
+``Qwen3DFlashAttention`` / ``Qwen3DFlashDecoderLayer`` (two layers, one windowed, causal and
+non-causal blocks, packed documents, a padded anchor, non-trivial norm gains), against HF
+``Qwen3DecoderLayer`` itself where no context key is visible, the whole forward against
+the same blocks composed as ``_backbone_forward``, and the aligned loss mask by a
+hand-worked literal.  ``select_anchors`` consumes torch's RNG stream the way
 the reference does (one ``randperm`` over the valid positions), so the same
 seed selects the same anchors.
 """

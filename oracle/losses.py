@@ -146,7 +146,8 @@ def dflash_loss_decay(pos_idx, gamma: float, sample_from_anchor: bool = False, *
 
 def dpace_loss_decay(pos_idx, loss_mask, block_size: int, dpace_alpha: float,
                      elementwise_loss, **_):
-    """D-PACE weight (losses/utils.py:64-112; parity unpinned).  Per block:
+    """D-PACE weight (losses/utils.py:64-112; the reference holds no test of it: pinned by a
+    per-element float64 double loop over random masks and a hand-worked example).  Per block:
     c = exp(-CE), s = (1-a)c + a (1 where the mask is 0), prefix = cumprod(s),
     w_i = m_i * sum_{j>=i} prefix_j m_j.  No gradient flows through it."""
     with torch.no_grad():

@@ -176,3 +176,39 @@ def test_bf16_inputs_fp32_math_gradient_within_2_percent_of_fp64():
         exact = torch.autograd.grad(ref, xd)[0]
         got = L.row_loss_grad(name, x, t).double()
         assert ((got - exact).norm() / exact.norm()).item() < 0.02, name
+
+
+def test_dpace_equals_per_block_double_loop_on_random_masks():
+    """losses/utils.py:64-112 spelled out per element in float64: within a block,
+    w_i = m_i * sum_{j >= i} m_j * prod_{l <= j} s_l,  s_l = (1 - a) exp(-CE_l) + a where the
+    mask is set and 1 elsewhere.  Random masks (also all-zero and all-one blocks), several block
+    sizes and smoothing constants."""
+    g = torch.Generator().manual_seed(0)
+    for bs, blocks, alpha in [(1, 5, 0.5), (4, 7, 0.5), (16, 9, 0.1), (5, 6, 0.0), (8, 4, 1.0)]:
+        n = bs * blocks
+        ce = torch.rand(1, n, generator=g) * 6
+        m = (torch.rand(1, n, generator=g) < 0.6).float()
+        m[0, :bs] = 0
+        if blocks > 1:
+            m[0, bs:2 * bs] = 1
+        got = L.dpace_loss_decay(None, m, bs, alpha, ce)
+        want = torch.zeros(n, dtype=torch.float64)
+        for b in range(blocks):
+            for i in range(bs):
+                if m[0, b * bs + i] == 0:
+                    continue
+                acc = 0.0
+                for j in range(i, bs):
+                    if m[0, b * bs + j] == 0:
+                        continue
+                    prod = 1.0
+                    for l in range(j + 1):
+                        if m[0, b * bs + l] != 0:
+                            prod *= (1 - alpha) * math.exp(-ce[0, b * bs + l].item()) + alpha
+                    acc += prod
+                want[b * bs + i] = acc
+        assert got.shape == (1, n)
+        assert torch.allclose(got[0].double(), want, rtol=1e-5, atol=1e-7), (bs, alpha)
+    # no gradient reaches the row losses through the weight
+    ce = torch.rand(1, 8, generator=g, requires_grad=True)
+    assert not L.dpace_loss_decay(None, torch.ones(1, 8), 4, 0.5, ce).requires_grad
