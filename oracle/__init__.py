@@ -12,8 +12,6 @@ pinned (reference golden vectors, closed forms, brute force) is listed in the
 docstring of the module that holds it; functions without such a pin say
 "parity unpinned".
 
-Parity unpinned:
-  * ``losses.dpace_loss_decay`` -- the reference holds no test for it; it is
-    restated from the formula and checked against a hand-computed two-block
-    example only.
+Parity unpinned: none.  (``losses.dpace_loss_decay`` has no test in the reference; it is
+pinned by what its formula fixes: a per-element float64 double loop over random masks.)
 """

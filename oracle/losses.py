@@ -13,7 +13,7 @@ RKL(a,b)=KL(b,a), JSD symmetric / <= log 2 / manual formula, TV = L1/2 in
 LK-hybrid eta=0 -> KL and eta->inf -> TV with a detached blend weight, the
 masked-mean and gamma**step rules; by the library routines
 ``F.kl_div`` / ``F.cross_entropy``; and by autograd == closed-form gradient.
-``dpace_loss_decay``: parity unpinned (no reference test), see package header.
+``dpace_loss_decay`` (no reference test): per-element float64 double loop over random masks.
 """
 
 from __future__ import annotations
