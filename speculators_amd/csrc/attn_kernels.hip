@@ -1645,16 +1645,10 @@ static int launch_fwd(AttnParams p, void* workspace, uint16_t* O, float* lse, hi
     last_error() = std::string(fn) + ": keys of one head must span less than 2 GiB";
     return SPX_ERR_ARG;
   }
-  static bool attr_set = false;  // one flag per head_dim instantiation
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, kFwdNSB, kFwdNW, PF>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) {
-      last_error() = std::string(fn) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
-      return SPX_ERR_HIP;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_set;  // per head_dim instantiation, one bit per device
+  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_fwd_kernel<D, kFwdNSB, kFwdNW, PF>),
+                                  smem, lds_set, fn))
+    return rc;
   hipLaunchKernelGGL((attn_fwd_kernel<D, kFwdNSB, kFwdNW, PF>), dim3((unsigned)(n_qb * p.Hq)),
                      dim3(64 * kFwdNW), smem, st, p, vt, O, lse);
   return check_launch(fn);
@@ -1699,17 +1693,11 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
       last_error() = std::string(fn) + ": keys of one head must span less than 2 GiB";
       return SPX_ERR_ARG;
     }
-    static bool dq_attr_set = false;  // one flag per head_dim instantiation
-    if (!dq_attr_set) {
-      hipError_t e = hipFuncSetAttribute(
-          reinterpret_cast<const void*>(&attn_bwd_dq_kernel<D, kDqNSB, kDqNW, kDqPFd>),
-          hipFuncAttributeMaxDynamicSharedMemorySize, dq_smem);
-      if (e != hipSuccess) {
-        last_error() = std::string(fn) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
-        return SPX_ERR_HIP;
-      }
-      dq_attr_set = true;
-    }
+    static std::atomic<uint64_t> dq_lds_set;  // per head_dim instantiation, one bit per device
+    if (int rc = ensure_dynamic_lds(
+            reinterpret_cast<const void*>(&attn_bwd_dq_kernel<D, kDqNSB, kDqNW, kDqPFd>), dq_smem,
+            dq_lds_set, fn))
+      return rc;
     hipLaunchKernelGGL((attn_bwd_dq_kernel<D, kDqNSB, kDqNW, kDqPFd>), dim3((unsigned)(n_qb * p.Hq)),
                        dim3(64 * kDqNW), dq_smem, st, p, dOp, kt, lse, delta, dQp, dq_hs);
   }
@@ -1722,41 +1710,34 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   }
   const int n_kb = (p.NKV + 32 * kDkvNW - 1) / (32 * kDkvNW);
   const dim3 kgrid((unsigned)(n_kb * p.Hq)), kblock(64 * kDkvNW);
-  auto set_smem = [&](const void* f, size_t smem) {
-    hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) last_error() = std::string(fn) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
-    return e == hipSuccess;
-  };
-  static bool attr_set = false;
+  static std::atomic<uint64_t> dkv_lds_set[2];  // per head_dim instantiation, one bit per device
   if constexpr (D > 128 && SPX_DKV256_ONEPASS) {
     // dK and dV in one pass over 32-row tiles (two buffers of four 16 KB tiles)
     constexpr size_t smem = DkvSmem<D, 0, 32>::kBytesDma;
-    if (!attr_set) {
-      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, 3, 0>), smem)) return SPX_ERR_HIP;
-      attr_set = true;
-    }
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, 3, 0>),
+                                    (int)smem, dkv_lds_set[0], fn))
+      return rc;
     hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, 3, 0>), kgrid, kblock, smem, st, p, dOp, qt, dot,
                        NQp, lse, delta, tb, dkp, dvp);
   } else if constexpr (D > 128) {
     // one launch per gradient (each loads only the tiles it multiplies with)
     constexpr size_t smem1 = kPF1 == 2 ? DkvSmem<D, 1>::kBytesDma : DkvSmem<D, 1>::kBytes;
     constexpr size_t smem2 = kPF2 == 2 ? DkvSmem<D, 2>::kBytesDma : DkvSmem<D, 2>::kBytes;
-    if (!attr_set) {
-      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF1, 1>), smem1) ||
-          !set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF2, 2>), smem2))
-        return SPX_ERR_HIP;
-      attr_set = true;
-    }
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF1, 1>),
+                                    (int)smem1, dkv_lds_set[0], fn))
+      return rc;
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF2, 2>),
+                                    (int)smem2, dkv_lds_set[1], fn))
+      return rc;
     hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF1, 1>), kgrid, kblock, smem1, st, p, dOp, qt,
                        dot, NQp, lse, delta, tb, dkp, dvp);
     hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF2, 2>), kgrid, kblock, smem2, st, p, dOp, qt,
                        dot, NQp, lse, delta, tb, dkp, dvp);
   } else {
     constexpr size_t smem = kPF == 2 ? DkvSmem<D, 0>::kBytesDma : DkvSmem<D, 0>::kBytes;
-    if (!attr_set) {
-      if (!set_smem(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF, 0>), smem)) return SPX_ERR_HIP;
-      attr_set = true;
-    }
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF, 0>),
+                                    (int)smem, dkv_lds_set[0], fn))
+      return rc;
     hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF, 0>), kgrid, kblock, smem, st, p, dOp, qt, dot,
                        NQp, lse, delta, tb, dkp, dvp);
   }

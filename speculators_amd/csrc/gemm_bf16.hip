@@ -308,17 +308,10 @@ static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const voi
              "256 rows of an operand must span less than 2 GiB (32-bit offsets inside a tile)");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool imm = lda >= kTK && ldb >= kTK;
-  static bool attr_set[2] = {false, false};
+  static std::atomic<uint64_t> lds_set[2];  // per kernel instantiation, one bit per device
   const void* fn = imm ? reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<true>)
                        : reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<false>);
-  if (!attr_set[imm]) {
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kGemmSmem);
-    if (e != hipSuccess) {
-      last_error() = std::string(fname) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
-      return SPX_ERR_HIP;
-    }
-    attr_set[imm] = true;
-  }
+  if (int rc = ensure_dynamic_lds(fn, kGemmSmem, lds_set[imm], fname)) return rc;
   const int tiles_m = (int)((M + kTM - 1) / kTM), tiles_n = (int)((N + kTN - 1) / kTN);
   SPX_REQ_FN((int64_t)tiles_m * tiles_n < (1ll << 31), "too many tiles");
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(kGemmThreads);

@@ -288,17 +288,10 @@ extern "C" int spx_gemm_bf16_tn(const void* a, int64_t lda, const void* b, int64
   SPX_REQUIRE(((T + 4 * tn::kTK) * lda) * 2 < 0x7ffffff0ll && ((T + 4 * tn::kTK) * ldb) * 2 < 0x7ffffff0ll,
               "each operand must span less than 2 GiB (32-bit buffer offsets)");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  static bool attr_set[2] = {false, false};
+  static std::atomic<uint64_t> lds_set[2];  // per kernel instantiation, one bit per device
   const void* fn = accumulate ? reinterpret_cast<const void*>(&tn::gemm_bf16_tn_kernel<true>)
                               : reinterpret_cast<const void*>(&tn::gemm_bf16_tn_kernel<false>);
-  if (!attr_set[accumulate ? 1 : 0]) {
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, tn::kSmem);
-    if (e != hipSuccess) {
-      last_error() = std::string(__func__) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
-      return SPX_ERR_HIP;
-    }
-    attr_set[accumulate ? 1 : 0] = true;
-  }
+  if (int rc = ensure_dynamic_lds(fn, tn::kSmem, lds_set[accumulate ? 1 : 0], __func__)) return rc;
   const int tiles_m = (int)((M + tn::kTM - 1) / tn::kTM), tiles_n = (int)((N + tn::kTN - 1) / tn::kTN);
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(tn::kThreads);
   auto ap = reinterpret_cast<const uint16_t*>(a);

@@ -21,6 +21,24 @@ int check_launch(const char* fn) {
   return SPX_ERR_HIP;
 }
 
+int ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done, const char* fn) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    last_error() = std::string(fn) + ": hipGetDevice: " + hipGetErrorString(e);
+    return SPX_ERR_HIP;
+  }
+  const uint64_t bit = (dev >= 0 && dev < 64) ? (1ull << dev) : 0;
+  if (bit && (done.load(std::memory_order_acquire) & bit)) return SPX_OK;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) {
+    last_error() = std::string(fn) + ": hipFuncSetAttribute: " + hipGetErrorString(e);
+    return SPX_ERR_HIP;
+  }
+  if (bit) done.fetch_or(bit, std::memory_order_release);
+  return SPX_OK;
+}
+
 }  // namespace spx
 
 extern "C" int spx_version(void) { return 100; }

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <string>
 
 #define SPX_OK 0
@@ -16,6 +17,11 @@ namespace spx {
 std::string& last_error();
 int fail_arg(const char* fn, const char* what);
 int check_launch(const char* fn);
+// Raises a kernel's dynamic-LDS limit to `bytes`, once per device: `done` (one object per kernel
+// instantiation) holds one bit per device ordinal on which the limit has been raised.  The
+// attribute is idempotent, so two threads that race here at worst both set it; devices with an
+// ordinal of 64 or more set it on every call.
+int ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done, const char* fn);
 
 #define SPX_REQUIRE(cond, what) \
   do {                          \
