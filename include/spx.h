@@ -232,6 +232,24 @@ int spx_ttt_attn_fwd(const void* q, int64_t q_head_stride, const void* k,
                      void* out, float* lse, void* workspace,
                      int64_t workspace_bytes, void* stream);
 
+/* spx_ttt_attn_fwd without a workspace argument, for callers that cannot allocate one:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference.  The forward's only scratch, the key-contiguous copy
+ * V^T [Hkv, D, round_up(T, 128)] bf16, lives in a static device array of
+ * spx_ttt_attn_fwd_static_max_bytes() = 16 MiB inside the library (each GPU the library runs
+ * on holds it until the process ends); shapes with Hkv * D * round_up(T, 128) * 2 bytes above
+ * that are rejected with status 1 (use spx_ttt_attn_fwd).  Neither this call nor anything it
+ * launches allocates or frees memory.  Results are bit-identical to spx_ttt_attn_fwd.  All calls
+ * on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two
+ * host threads) race on it; calls ordered on one stream do not.  Nothing has to be cleared
+ * between calls: each call rewrites every byte of the array it later reads. */
+int64_t spx_ttt_attn_fwd_static_max_bytes(void);
+int spx_ttt_attn_fwd_static(const void* q, int64_t q_head_stride, const void* k,
+                            int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                            const int32_t* row_lo, int64_t T, int32_t ttt_step,
+                            int32_t Hq, int32_t Hkv, int32_t D, float scaling,
+                            void* out, float* lse, void* stream);
+
 /* Gradients of spx_ttt_attn_fwd.  dout bf16 [T, Hq, D] (the layout of `out`),
  * lse as written by the forward.  dq bf16 [Hq, T, D]; dk, dv bf16
  * [Hkv, (ttt_step+1)*T, D]: every row is written (context rows by the tiled

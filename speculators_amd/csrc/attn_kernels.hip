@@ -1864,6 +1864,57 @@ extern "C" int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void
                         workspace, st, __func__);
 }
 
+// ---------------------------------------------------------------- allocation-free variant
+// The forward's only scratch is the key-contiguous copy V^T [Hkv, D, round_up(T, 128)].  Here it
+// lives in a file-scope device array instead of a caller-owned workspace.  Every GPU holds its
+// own copy of the array at its own address: the address is looked up once per device with that
+// device current and kept; host code never uses the array's name as a pointer.
+constexpr int64_t kStaticScratchBytes = 16ll << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+static int static_scratch(void** out, const char* fn) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    last_error() = std::string(fn) + ": hipGetDevice: " + hipGetErrorString(e);
+    return SPX_ERR_HIP;
+  }
+  if (dev < 0 || dev >= kMaxDevices) return fail_arg(fn, "device ordinal out of range");
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      last_error() = std::string(fn) + ": hipGetSymbolAddress: " + hipGetErrorString(e);
+      return SPX_ERR_HIP;
+    }
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // same value from every thread
+  }
+  *out = ptr;
+  return SPX_OK;
+}
+
+extern "C" int64_t spx_ttt_attn_fwd_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int spx_ttt_attn_fwd_static(const void* q, int64_t q_head_stride, const void* k,
+                                       int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                                       const int32_t* row_lo, int64_t T, int32_t ttt_step,
+                                       int32_t Hq, int32_t Hkv, int32_t D, float scaling, void* out,
+                                       float* lse, void* stream) {
+  if (int rc = shape_checks(__func__, T, T, Hq, Hkv, D)) return rc;
+  if (fwd_workspace_bytes(T, Hkv, D) > kStaticScratchBytes)
+    return fail_arg(__func__, "Hkv * D * round_up(T, 128) * 2 bytes exceed the 16 MiB static scratch; "
+                              "use spx_ttt_attn_fwd with a caller-owned workspace");
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws, __func__)) return rc;
+  // every byte of V^T the kernel reads is rewritten by this call's transpose (padding columns
+  // included), so nothing of an earlier call has to be cleared
+  return spx_ttt_attn_fwd(q, q_head_stride, k, k_head_stride, v, v_head_stride, row_lo, T, ttt_step, Hq,
+                          Hkv, D, scaling, out, lse, ws, kStaticScratchBytes, stream);
+}
+
 // ================================================================ DFlash entry points
 extern "C" int spx_dflash_row_ranges(const void* document_ids, int doc_kind, int64_t T,
                                      const void* anchors, int anchor_kind, int64_t n_anchors,
