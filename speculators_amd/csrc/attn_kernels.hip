@@ -1497,8 +1497,12 @@ __global__ __launch_bounds__(256) void attn_dkv_reduce_kernel(
 // dK / dV of the TTT diagonal keys (j, i), j >= 1: sixteen lanes per (position, K/V head)
 // item, four items per wave; each such key is seen by exactly the `group` query heads at its
 // own position.  A lane holds D / 16 consecutive elements (one or two 16-byte accesses); the dot
-// products are summed over the sixteen lanes with DPP moves (no LDS traffic).
-template <int D>
+// products are summed over the sixteen lanes with DPP moves (no LDS traffic).  The sums over the
+// heads of a group stay in fp32 registers until the one store (one rounding to bf16).
+// MAXG = query heads per K/V head whose rows are kept in registers: a group of at most MAXG heads
+// reads its query / output-gradient rows once for all diagonals; a wider group walks its heads in
+// passes of MAXG inside every diagonal (rows re-read per diagonal, from L2).
+template <int D, int MAXG>
 __global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
     const uint16_t* __restrict__ Q, int64_t q_hs, const uint16_t* __restrict__ K, int64_t k_hs,
     const uint16_t* __restrict__ V, int64_t v_hs, const uint16_t* __restrict__ dO,
@@ -1506,7 +1510,6 @@ __global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
     int Hkv, float scale_log2e, float scaling, uint16_t* dK, int64_t dk_hs, uint16_t* dV,
     int64_t dv_hs) {
   constexpr int EPL = D / 16;
-  constexpr int MAXG = 4;  // query heads per K/V head kept in registers at a time
   // item = kvh * T + i: neighbouring 16-lane rows take neighbouring positions of one K/V head, so
   // their key / value / gradient rows are contiguous in memory.  The tail clamps (no early
   // return: the DPP sums need whole rows of lanes)
@@ -1517,11 +1520,10 @@ __global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
   const int kvh = (int)(item / T), i = (int)(item % T);
   const int group = Hq / Hkv;
   const int d0 = (threadIdx.x & 15) * EPL;
-  for (int h0 = 0; h0 < group; h0 += MAXG) {
-    // the row's query and output-gradient vectors of up to MAXG heads are read once and reused
-    // for every diagonal key (they do not depend on j)
-    const int ng = min(group - h0, MAXG);
-    float qv[MAXG][EPL], dv[MAXG][EPL], lse_h[MAXG], delta_h[MAXG];
+  const bool one_pass = group <= MAXG;
+
+  float qv[MAXG][EPL], dv[MAXG][EPL], lse_h[MAXG], delta_h[MAXG];
+  auto load_heads = [&](int h0, int ng) {
 #pragma unroll
     for (int hh = 0; hh < MAXG; ++hh) {
       const int h = kvh * group + h0 + (hh < ng ? hh : 0);
@@ -1530,34 +1532,35 @@ __global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
       lse_h[hh] = LSE[(int64_t)h * T + i];
       delta_h[hh] = Delta[(int64_t)h * T + i];
     }
-    // the key / value rows of diagonal j + 1 are requested before diagonal j is worked on: the
-    // loop is a chain of dependent global loads otherwise
-    float kn[EPL], vn[EPL];
-    {
-      const int64_t r1 = ((int64_t)T + i) * D + d0;
-      ld_bf16s<EPL>(K + (int64_t)kvh * k_hs + r1, kn);
-      ld_bf16s<EPL>(V + (int64_t)kvh * v_hs + r1, vn);
-    }
-    for (int j = 1; j <= n_extra; ++j) {
-      const int64_t gko = (int64_t)kvh * dk_hs + ((int64_t)j * T + i) * D + d0;
-      const int64_t gvo = (int64_t)kvh * dv_hs + ((int64_t)j * T + i) * D + d0;
-      float kv[EPL], vv[EPL], gk[EPL], gv[EPL];
+  };
+  if (one_pass) load_heads(0, group);
+  // the key / value rows of diagonal j + 1 are requested before diagonal j is worked on: the
+  // loop is a chain of dependent global loads otherwise
+  float kn[EPL], vn[EPL];
+  {
+    const int64_t r1 = ((int64_t)T + i) * D + d0;
+    ld_bf16s<EPL>(K + (int64_t)kvh * k_hs + r1, kn);
+    ld_bf16s<EPL>(V + (int64_t)kvh * v_hs + r1, vn);
+  }
+  for (int j = 1; j <= n_extra; ++j) {
+    const int64_t gko = (int64_t)kvh * dk_hs + ((int64_t)j * T + i) * D + d0;
+    const int64_t gvo = (int64_t)kvh * dv_hs + ((int64_t)j * T + i) * D + d0;
+    float kv[EPL], vv[EPL], gk[EPL], gv[EPL];
 #pragma unroll
-      for (int e = 0; e < EPL; ++e) {
-        kv[e] = kn[e];
-        vv[e] = vn[e];
-        gk[e] = 0.f;
-        gv[e] = 0.f;
-      }
-      if (h0) {  // groups wider than MAXG accumulate over several passes
-        ld_bf16s<EPL>(dK + gko, gk);
-        ld_bf16s<EPL>(dV + gvo, gv);
-      }
-      if (j < n_extra) {
-        const int64_t rn = ((int64_t)(j + 1) * T + i) * D + d0;
-        ld_bf16s<EPL>(K + (int64_t)kvh * k_hs + rn, kn);
-        ld_bf16s<EPL>(V + (int64_t)kvh * v_hs + rn, vn);
-      }
+    for (int e = 0; e < EPL; ++e) {
+      kv[e] = kn[e];
+      vv[e] = vn[e];
+      gk[e] = 0.f;
+      gv[e] = 0.f;
+    }
+    if (j < n_extra) {
+      const int64_t rn = ((int64_t)(j + 1) * T + i) * D + d0;
+      ld_bf16s<EPL>(K + (int64_t)kvh * k_hs + rn, kn);
+      ld_bf16s<EPL>(V + (int64_t)kvh * v_hs + rn, vn);
+    }
+    for (int h0 = 0; h0 < group; h0 += MAXG) {
+      const int ng = min(group - h0, MAXG);
+      if (!one_pass) load_heads(h0, ng);
 #pragma unroll
       for (int hh = 0; hh < MAXG; ++hh) {
         if (hh < ng) {
@@ -1578,10 +1581,10 @@ __global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
           }
         }
       }
-      if (live) {
-        st_bf16s<EPL>(dK + gko, gk);
-        st_bf16s<EPL>(dV + gvo, gv);
-      }
+    }
+    if (live) {
+      st_bf16s<EPL>(dK + gko, gk);
+      st_bf16s<EPL>(dV + gvo, gv);
     }
   }
 }
@@ -1744,10 +1747,18 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   const int64_t items = (int64_t)p.NKV * D / 4 * p.Hkv;
   hipLaunchKernelGGL(attn_dkv_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, dkp,
                      dvp, p.NKV, D, p.Hq, p.Hkv, p.scaling, dKp, dk_hs, dVp, dv_hs);
-  if (p.n_extra > 0)
-    hipLaunchKernelGGL(ttt_attn_bwd_diag_kernel<D>, dim3((unsigned)(((int64_t)p.T * p.Hkv + 15) / 16)),
-                       dim3(256), 0, st, p.Q, p.q_hs, p.K, p.k_hs, p.V, p.v_hs, dOp, lse, delta, p.T,
-                       p.n_extra, p.Hq, p.Hkv, p.scale_log2e, p.scaling, dKp, dk_hs, dVp, dv_hs);
+  if (p.n_extra > 0) {
+    const dim3 dgrid((unsigned)(((int64_t)p.T * p.Hkv + 15) / 16));
+    // eight heads per K/V head in registers where they fit (head_dim <= 128), else four
+    if (D <= 128 && p.Hq / p.Hkv > 4)
+      hipLaunchKernelGGL((ttt_attn_bwd_diag_kernel<D, (D <= 128 ? 8 : 4)>), dgrid, dim3(256), 0, st, p.Q,
+                         p.q_hs, p.K, p.k_hs, p.V, p.v_hs, dOp, lse, delta, p.T, p.n_extra, p.Hq, p.Hkv,
+                         p.scale_log2e, p.scaling, dKp, dk_hs, dVp, dv_hs);
+    else
+      hipLaunchKernelGGL((ttt_attn_bwd_diag_kernel<D, 4>), dgrid, dim3(256), 0, st, p.Q, p.q_hs, p.K,
+                         p.k_hs, p.V, p.v_hs, dOp, lse, delta, p.T, p.n_extra, p.Hq, p.Hkv,
+                         p.scale_log2e, p.scaling, dKp, dk_hs, dVp, dv_hs);
+  }
   return check_launch(fn);
 }
 

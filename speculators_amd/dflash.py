@@ -27,6 +27,7 @@ from . import gemm
 from . import losses as L
 from . import metrics as MT
 from .eagle3 import MLP, RMSNorm
+from .weights import WeightStager, compute_input
 
 
 @dataclass
@@ -85,44 +86,43 @@ class DFlashAttention(nn.Module):
     RMSNorm; RoPE with the last q_len positions for q
     (models/dflash/model_definitions.py:47-155)."""
 
-    def __init__(self, cfg: DFlashConfig):
+    def __init__(self, cfg: DFlashConfig, stager: WeightStager):
         super().__init__()
         hq, hkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
         self.hq, self.hkv, self.d = hq, hkv, d
+        self._stager = stager
         self.q_proj = nn.Linear(cfg.hidden_size, hq * d, bias=False)
         self.k_proj = nn.Linear(cfg.hidden_size, hkv * d, bias=False)
         self.v_proj = nn.Linear(cfg.hidden_size, hkv * d, bias=False)
         self.o_proj = nn.Linear(hq * d, cfg.hidden_size, bias=False)
-        self.q_norm = RMSNorm(d, cfg.rms_norm_eps)
-        self.k_norm = RMSNorm(d, cfg.rms_norm_eps)
+        self.q_norm = RMSNorm(d, cfg.rms_norm_eps, stager)
+        self.k_norm = RMSNorm(d, cfg.rms_norm_eps, stager)
         self.scaling = d ** -0.5
         self.attn_fn = A.ALL_ATTENTION_FUNCTIONS[cfg.attn_implementation]
 
     def forward(self, x, ctx, q_pos, kv_pos, inv_freq, mask):
         ql, tl = x.shape[1], ctx.shape[1]
-        lin = gemm.linear_accumulate
-        q = self.q_norm(lin(x, self.q_proj.weight).view(1, ql, self.hq, self.d)).view(1, ql, self.hq * self.d)
+        lin, W = gemm.linear_staged, self._stager.get
+        q = self.q_norm(lin(x, W(self.q_proj.weight)).view(1, ql, self.hq, self.d)).view(1, ql, self.hq * self.d)
         # one projection of cat([context, mask tokens]) instead of two per weight
         both = torch.cat([ctx, x], dim=1)
-        k = lin(both, self.k_proj.weight)
-        v = lin(both, self.v_proj.weight)
+        k = lin(both, W(self.k_proj.weight))
+        v = lin(both, W(self.v_proj.weight))
         k = self.k_norm(k.view(1, tl + ql, self.hkv, self.d)).view(1, tl + ql, self.hkv * self.d)
         q = FO.rope_relayout(q, q_pos, inv_freq, self.hq, True, 0)
         k = FO.rope_relayout(k, kv_pos, inv_freq, self.hkv, True, 0)
         v = FO.rope_relayout(v, kv_pos, inv_freq, self.hkv, False, 0)
         out, _ = self.attn_fn(self, q, k, v, mask, scaling=self.scaling)
-        return gemm.linear_accumulate(out.reshape(1, ql, self.hq * self.d), self.o_proj.weight)
+        return lin(out.reshape(1, ql, self.hq * self.d), W(self.o_proj.weight))
 
 
 class DFlashDecoderLayer(nn.Module):
-    def __init__(self, cfg: DFlashConfig):
+    def __init__(self, cfg: DFlashConfig, stager: WeightStager):
         super().__init__()
-        self.self_attn = DFlashAttention(cfg)
-        mlp_cfg = type("C", (), {"hidden_size": cfg.hidden_size,
-                                 "intermediate_size": cfg.intermediate_size})
-        self.mlp = MLP(mlp_cfg)
-        self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
-        self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+        self.self_attn = DFlashAttention(cfg, stager)
+        self.mlp = MLP(cfg, stager)
+        self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps, stager)
+        self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps, stager)
 
     def forward(self, x, ctx, q_pos, kv_pos, inv_freq, mask, x_normed=None, next_norm=None):
         """``x_normed``: ``input_layernorm(x)`` when the previous layer already produced it;
@@ -132,11 +132,11 @@ class DFlashDecoderLayer(nn.Module):
             x_normed = self.input_layernorm(x)
         a = self.self_attn(x_normed, ctx, q_pos, kv_pos, inv_freq, mask)
         post = self.post_attention_layernorm
-        y, z = FO.add_rms_norm(x, a, post.weight, post.eps)  # residual add fused into the norm
+        y, z = FO.add_rms_norm(x, a, post.gain, post.eps)  # residual add fused into the norm
         m = self.mlp(z)
         if next_norm is None:
             return y + m
-        return FO.add_rms_norm(y, m, next_norm.weight, next_norm.eps)
+        return FO.add_rms_norm(y, m, next_norm.gain, next_norm.eps)
 
 
 class DFlashDraftModel(nn.Module):
@@ -145,6 +145,7 @@ class DFlashDraftModel(nn.Module):
         self.config = config
         h = config.hidden_size
         self.block_size = config.block_size
+        self._stager = st = WeightStager()
         self.draft_vocab_size = config.draft_vocab_size
         self.verifier_vocab_size = config.vocab_size
         self.use_draft_vocab = config.draft_vocab_size != config.vocab_size
@@ -157,16 +158,15 @@ class DFlashDraftModel(nn.Module):
         self.lm_head = nn.Linear(h, config.draft_vocab_size, bias=False)
         self.verifier_lm_head = nn.Linear(h, config.draft_vocab_size, bias=False)
         self.fc = nn.Linear(config.num_aux * h, h, bias=False)
-        self.hidden_norm = RMSNorm(h, config.rms_norm_eps)
-        self.layers = nn.ModuleList(DFlashDecoderLayer(config) for _ in range(config.num_hidden_layers))
-        self.norm = RMSNorm(h, config.rms_norm_eps)
-        self.verifier_norm = RMSNorm(h, config.rms_norm_eps)
+        self.hidden_norm = RMSNorm(h, config.rms_norm_eps, st)
+        self.layers = nn.ModuleList(DFlashDecoderLayer(config, st) for _ in range(config.num_hidden_layers))
+        self.norm = RMSNorm(h, config.rms_norm_eps, st)
+        self.verifier_norm = RMSNorm(h, config.rms_norm_eps, st)
         for p in (self.embed_tokens.weight, self.lm_head.weight, self.verifier_lm_head.weight,
                   self.verifier_norm.weight):
             p.requires_grad_(False)
         self.uses_sliding_window_attn = bool(config.sliding_layers)
         self.uses_full_attn = config.num_hidden_layers > len(config.sliding_layers)
-        self._frozen_t: dict = {}
         # lm_head and the loss as one autograd node while the head is frozen and the loss is a single
         # fused reduction (False: always two nodes)
         self.fuse_head_loss = True
@@ -179,20 +179,24 @@ class DFlashDraftModel(nn.Module):
                 "ensure the config was saved with mask_token_id set.")
         return self.config.mask_token_id
 
-    def _transposed_frozen(self, weight):
-        """``weight.T`` contiguous, cached: frozen weights never change between steps."""
-        key = (weight.data_ptr(), weight._version)
-        hit = self._frozen_t.get(id(weight))
-        if hit is None or hit[0] != key:
-            hit = (key, weight.detach().t().contiguous())
-            self._frozen_t[id(weight)] = hit
-        return hit[1]
+    def invalidate_weight_caches(self):
+        """Drop the kept bf16 / transposed copies of the frozen weights.  They are keyed on the
+        parameter's address and version counter, which a write through ``param.data`` does not
+        change: call this after such a write.  ``train()`` / ``eval()`` and ``load_state_dict``
+        call it."""
+        self._stager.invalidate()
 
-    def _linear(self, x, weight, frozen=False):
-        if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
-            raise RuntimeError("the HIP draft path runs in bf16: cast the model and its inputs to bfloat16")
-        wt = self._transposed_frozen(weight) if frozen and x.requires_grad else None
-        return gemm.linear(x, weight, wt)
+    def train(self, mode: bool = True):
+        self._stager.invalidate()
+        return super().train(mode)
+
+    def load_state_dict(self, *args, **kwargs):
+        self._stager.invalidate()
+        return super().load_state_dict(*args, **kwargs)
+
+    def _linear(self, x, weight):
+        """``x @ weight.T`` on the MFMA kernel of this library (fc, lm_head, verifier head)."""
+        return gemm.linear_staged(x, self._stager.get(weight), hip=True)
 
     def forward(self, hidden_states, input_ids, loss_mask, verifier_last_hidden_states,
                 document_ids, position_ids=None, loss_config: L.LossConfig | None = None,
@@ -204,6 +208,9 @@ class DFlashDraftModel(nn.Module):
         device = hidden_states.device
         t = hidden_states.shape[1]
         bs = self.block_size
+        self._stager.begin()
+        hidden_states = compute_input(hidden_states)
+        verifier_last_hidden_states = compute_input(verifier_last_hidden_states)
         if position_ids is None:
             position_ids = torch.arange(t, dtype=torch.long, device=device).unsqueeze(0)
         if anchors is None:
@@ -238,12 +245,12 @@ class DFlashDraftModel(nn.Module):
             noise, normed = layer(noise, ctx, q_pos, kv_pos, inv_freq,
                                   sw_mask if li in cfg.sliding_layers else full_mask,
                                   x_normed=normed, next_norm=nxt)
-        if (self.fuse_head_loss and normed.requires_grad and not self.lm_head.weight.requires_grad
-                and normed.dtype == torch.bfloat16 and self.lm_head.weight.dtype == torch.bfloat16):
+        head = self._stager.get(self.lm_head.weight)
+        if self.fuse_head_loss and normed.requires_grad and not head.trainable:
             # head + loss as one autograd node while the head is frozen (see metrics.Head)
-            logits = MT.Head(normed, self.lm_head.weight, self._transposed_frozen(self.lm_head.weight))
+            logits = MT.Head(normed, head.w, head.wt)
         else:
-            logits = self._linear(normed, self.lm_head.weight, frozen=True)
+            logits = gemm.linear_staged(normed, head, hip=True)
         aligned = loss_mask.clone()[:, block_idx]
         aligned = aligned * anchor_valid.repeat_interleave(bs).unsqueeze(0).to(aligned.dtype)
         if not cfg.sample_from_anchor:

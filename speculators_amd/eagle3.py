@@ -28,6 +28,7 @@ from . import fused_ops as FO
 from . import gemm
 from . import losses as L
 from . import metrics as MT
+from .weights import WeightStager, compute_input
 
 
 @dataclass
@@ -59,17 +60,25 @@ class Eagle3Config:
 
 
 class RMSNorm(nn.Module):
-    def __init__(self, dim: int, eps: float):
+    """``stager``: the model's ``WeightStager`` (the gain is then read through it: bf16 compute copy
+    of an fp32 master gain); None for a stand-alone norm on bf16 tensors."""
+
+    def __init__(self, dim: int, eps: float, stager: WeightStager | None = None):
         super().__init__()
         self.weight = nn.Parameter(torch.ones(dim))
         self.eps = eps
+        self._stager = stager
+
+    @property
+    def gain(self) -> torch.Tensor:
+        return self.weight if self._stager is None else self._stager.gain(self.weight)
 
     def forward(self, x):
-        return FO.rms_norm(x, self.weight, self.eps)
+        return FO.rms_norm(x, self.gain, self.eps)
 
 
 class Attention(nn.Module):
-    def __init__(self, cfg: Eagle3Config, in_features: int):
+    def __init__(self, cfg: Eagle3Config, in_features: int, stager: WeightStager):
         super().__init__()
         hq, hkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
         self.hq, self.hkv, self.d = hq, hkv, d
@@ -78,17 +87,17 @@ class Attention(nn.Module):
         self.v_proj = nn.Linear(in_features, hkv * d, bias=False)
         self.o_proj = nn.Linear(hq * d, cfg.hidden_size, bias=False)
         if cfg.qk_norm:
-            self.q_norm = RMSNorm(d, cfg.rms_norm_eps)
-            self.k_norm = RMSNorm(d, cfg.rms_norm_eps)
+            self.q_norm = RMSNorm(d, cfg.rms_norm_eps, stager)
+            self.k_norm = RMSNorm(d, cfg.rms_norm_eps, stager)
         self.qk_norm = cfg.qk_norm
         self.scaling = d ** -0.5
         self.attn_fn = A.ALL_ATTENTION_FUNCTIONS[cfg.attn_implementation]
-        self._merged_qkv = gemm._MergedQKV()
+        self._stager = stager
 
     def forward(self, x, position_ids, pos_offset, inv_freq, cache: dict, mask):
         t = x.shape[1]
-        lin = gemm.linear_accumulate
-        if not self.qk_norm and gemm.FUSE_WGRAD_ACCUMULATION and torch.is_grad_enabled():
+        W = self._stager.get
+        if not self.qk_norm:
             # one GEMM for q, k and v; rotary embedding + [T, heads*D] -> [heads, T, D] fused behind it
             pos = position_ids.reshape(-1)
             if pos.dtype != torch.int64:
@@ -97,20 +106,18 @@ class Attention(nn.Module):
             if kvc is None and cache.get("steps") and self.attn_fn is A.ttt_hip_attention_forward:
                 # all TTT steps' keys / values of this layer in one buffer, written in place
                 kvc = cache["kv"] = A.TTTKVCache(self.hkv, t, self.d, cache["steps"], x.device)
-            q, k, v = gemm.qkv_rope(x, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight,
+            q, k, v = gemm.qkv_rope(x, W(self.q_proj.weight, self.k_proj.weight, self.v_proj.weight),
                                     pos.contiguous(), inv_freq, self.hq, self.hkv, self.d, pos_offset,
-                                    self._merged_qkv,
                                     kv_out=None if kvc is None else kvc.window(pos_offset))
             if kvc is not None:
                 out = A.ttt_attention_cached(q, k, v, kvc, mask, self.scaling)
-                return gemm.linear_accumulate(out.reshape(1, t, self.hq * self.d), self.o_proj.weight)
+                return gemm.linear_staged(out.reshape(1, t, self.hq * self.d), W(self.o_proj.weight))
         else:
-            q = lin(x, self.q_proj.weight)
-            k = lin(x, self.k_proj.weight)
-            v = lin(x, self.v_proj.weight)
-            if self.qk_norm:
-                q = self.q_norm(q.view(1, t, self.hq, self.d)).view(1, t, self.hq * self.d)
-                k = self.k_norm(k.view(1, t, self.hkv, self.d)).view(1, t, self.hkv * self.d)
+            q = gemm.linear_staged(x, W(self.q_proj.weight))
+            k = gemm.linear_staged(x, W(self.k_proj.weight))
+            v = gemm.linear_staged(x, W(self.v_proj.weight))
+            q = self.q_norm(q.view(1, t, self.hq, self.d)).view(1, t, self.hq * self.d)
+            k = self.k_norm(k.view(1, t, self.hkv, self.d)).view(1, t, self.hkv * self.d)
             # rotary embedding + [T, heads*D] -> [heads, T, D] in one pass each
             q = FO.rope_relayout(q, position_ids, inv_freq, self.hq, True, pos_offset)
             k = FO.rope_relayout(k, position_ids, inv_freq, self.hkv, True, pos_offset)
@@ -119,25 +126,22 @@ class Attention(nn.Module):
         cache["k"] = k if "k" not in cache else torch.cat([cache["k"], k], dim=2)
         cache["v"] = v if "v" not in cache else torch.cat([cache["v"], v], dim=2)
         out, _ = self.attn_fn(self, q, cache["k"], cache["v"], mask, scaling=self.scaling)
-        return gemm.linear_accumulate(out.reshape(1, t, self.hq * self.d), self.o_proj.weight)
+        return gemm.linear_staged(out.reshape(1, t, self.hq * self.d), W(self.o_proj.weight))
 
 
 class MLP(nn.Module):
-    def __init__(self, cfg: Eagle3Config):
+    def __init__(self, cfg, stager: WeightStager):
         super().__init__()
         self.gate_proj = nn.Linear(cfg.hidden_size, cfg.intermediate_size, bias=False)
         self.up_proj = nn.Linear(cfg.hidden_size, cfg.intermediate_size, bias=False)
         self.down_proj = nn.Linear(cfg.intermediate_size, cfg.hidden_size, bias=False)
-        self._merged_gate_up = gemm._MergedWeights()
+        self._stager = stager
 
     def forward(self, x):
-        lin = gemm.linear_accumulate
-        if gemm.FUSE_WGRAD_ACCUMULATION and torch.is_grad_enabled() and x.dtype == torch.bfloat16:
-            # gate and up as one GEMM, SwiGLU on the two halves of its output
-            act = gemm.gate_up_swiglu(x, self.gate_proj.weight, self.up_proj.weight, self._merged_gate_up)
-        else:
-            act = FO.swiglu(lin(x, self.gate_proj.weight), lin(x, self.up_proj.weight))
-        return lin(act, self.down_proj.weight)
+        W = self._stager.get
+        # gate and up as one GEMM, SwiGLU on the two halves of its output
+        act = gemm.gate_up_swiglu(x, W(self.gate_proj.weight, self.up_proj.weight))
+        return gemm.linear_staged(act, W(self.down_proj.weight))
 
 
 class _Prenormed(NamedTuple):
@@ -153,16 +157,16 @@ class DecoderLayer(nn.Module):
     (2H wide), embeds and hidden are normalised separately, the residual is the
     (optionally normalised) hidden half."""
 
-    def __init__(self, cfg: Eagle3Config, layer_idx: int):
+    def __init__(self, cfg: Eagle3Config, layer_idx: int, stager: WeightStager):
         super().__init__()
         self.first = layer_idx == 0
         self.cfg = cfg
-        self.self_attn = Attention(cfg, (2 if self.first else 1) * cfg.hidden_size)
-        self.mlp = MLP(cfg)
-        self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
-        self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+        self.self_attn = Attention(cfg, (2 if self.first else 1) * cfg.hidden_size, stager)
+        self.mlp = MLP(cfg, stager)
+        self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps, stager)
+        self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps, stager)
         if self.first:
-            self.hidden_norm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+            self.hidden_norm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps, stager)
 
     def forward(self, x, position_ids, pos_offset, inv_freq, cache, mask, next_norm=None):
         """``x``: the hidden state, or for the first layer the pair ``(embeds, hidden)`` (their
@@ -180,8 +184,8 @@ class DecoderLayer(nn.Module):
             else:
                 residual = hidden
                 # both norms write straight into the halves of the 2H-wide projection input
-                xin = FO.pair_norm_cat(embeds, hidden, self.input_layernorm.weight,
-                                       self.hidden_norm.weight, eps)
+                xin = FO.pair_norm_cat(embeds, hidden, self.input_layernorm.gain,
+                                       self.hidden_norm.gain, eps)
             a = self.self_attn(xin, position_ids, pos_offset, inv_freq, cache, mask)
         else:
             if isinstance(x, _Prenormed):  # the previous layer already applied this layer's input norm
@@ -190,11 +194,11 @@ class DecoderLayer(nn.Module):
                 residual, xn = x, self.input_layernorm(x)
             a = self.self_attn(xn, position_ids, pos_offset, inv_freq, cache, mask)
         post = self.post_attention_layernorm
-        y, z = FO.add_rms_norm(residual, a, post.weight, post.eps)
+        y, z = FO.add_rms_norm(residual, a, post.gain, post.eps)
         m = self.mlp(z)
         if next_norm is None:
             return y + m
-        return FO.add_rms_norm(y, m, next_norm.weight, next_norm.eps)
+        return FO.add_rms_norm(y, m, next_norm.gain, next_norm.eps)
 
 
 class Eagle3DraftModel(nn.Module):
@@ -203,6 +207,7 @@ class Eagle3DraftModel(nn.Module):
         self.config = config
         h = config.hidden_size
         self.hidden_size = h
+        self._stager = st = WeightStager()
         self.draft_vocab_size = config.draft_vocab_size
         self.verifier_vocab_size = config.vocab_size
         self.use_draft_vocab = config.draft_vocab_size != config.vocab_size
@@ -215,11 +220,12 @@ class Eagle3DraftModel(nn.Module):
         self.lm_head = nn.Linear(h, config.draft_vocab_size, bias=False)
         self.verifier_lm_head = nn.Linear(h, config.draft_vocab_size, bias=False)
         self.fc = nn.Linear(config.num_aux * h, h, bias=False)
-        self.layers = nn.ModuleList(DecoderLayer(config, i) for i in range(config.num_hidden_layers))
-        self.norm = RMSNorm(h, config.rms_norm_eps)
-        self.verifier_norm = RMSNorm(h, config.rms_norm_eps)
-        self.input_norm = RMSNorm(config.num_aux * h, config.rms_norm_eps) if config.norm_before_fc else None
-        self.fc_norm = (nn.ModuleList(RMSNorm(h, config.rms_norm_eps) for _ in range(config.num_aux))
+        self.layers = nn.ModuleList(DecoderLayer(config, i, st) for i in range(config.num_hidden_layers))
+        self.norm = RMSNorm(h, config.rms_norm_eps, st)
+        self.verifier_norm = RMSNorm(h, config.rms_norm_eps, st)
+        self.input_norm = (RMSNorm(config.num_aux * h, config.rms_norm_eps, st)
+                           if config.norm_before_fc else None)
+        self.fc_norm = (nn.ModuleList(RMSNorm(h, config.rms_norm_eps, st) for _ in range(config.num_aux))
                         if config.fc_norm else None)
         # frozen, as in model.py:63-71 and models/eagle3/core.py:68,120
         for p in (self.embed_tokens.weight, self.lm_head.weight, self.verifier_lm_head.weight,
@@ -228,7 +234,6 @@ class Eagle3DraftModel(nn.Module):
         self.embed_tokens.weight.requires_grad_(config.embed_requires_grad)
         self.uses_sliding_window_attn = bool(config.sliding_layers)
         self.uses_full_attn = config.num_hidden_layers > len(config.sliding_layers)
-        self._frozen_t: dict = {}
         # lm_head and the loss as one autograd node while the head is frozen and the loss is a single
         # fused reduction (False: always two nodes)
         self.fuse_head_loss = True
@@ -254,20 +259,24 @@ class Eagle3DraftModel(nn.Module):
         self.t2d.copy_(t2d.to(self.t2d.device))
         self.d2t.copy_(d2t.to(self.d2t.device))
 
-    def _transposed_frozen(self, weight: torch.Tensor) -> torch.Tensor:
-        """``weight.T`` contiguous, cached: frozen weights never change between steps."""
-        key = (weight.data_ptr(), weight._version, weight.dtype)
-        hit = self._frozen_t.get(id(weight))
-        if hit is None or hit[0] != key:
-            hit = (key, weight.detach().t().contiguous())
-            self._frozen_t[id(weight)] = hit
-        return hit[1]
+    def invalidate_weight_caches(self):
+        """Drop the kept bf16 / transposed copies of the frozen weights (``lm_head``,
+        ``verifier_lm_head``, ``verifier_norm``).  They are keyed on the parameter's address and
+        version counter, which a write through ``param.data`` does not change: call this after
+        such a write.  ``train()`` / ``eval()`` and ``load_state_dict`` call it."""
+        self._stager.invalidate()
 
-    def _linear(self, x, weight, frozen: bool = False):
-        if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
-            wt = self._transposed_frozen(weight) if frozen and x.requires_grad else None
-            return gemm.linear(x, weight, wt)
-        raise RuntimeError("the HIP draft path runs in bf16: cast the model and its inputs to bfloat16")
+    def train(self, mode: bool = True):
+        self._stager.invalidate()
+        return super().train(mode)
+
+    def load_state_dict(self, *args, **kwargs):
+        self._stager.invalidate()
+        return super().load_state_dict(*args, **kwargs)
+
+    def _linear(self, x, weight):
+        """``x @ weight.T`` on the MFMA kernel of this library (fc, lm_head, verifier head)."""
+        return gemm.linear_staged(x, self._stager.get(weight), hip=True)
 
     # ------------------------------------------------------------------ forward
     def forward(self, hidden_states, input_ids, document_ids, loss_mask=None, position_ids=None,
@@ -280,6 +289,10 @@ class Eagle3DraftModel(nn.Module):
         cfg = self.config
         device = hidden_states.device
         t = hidden_states.shape[1]
+        self._stager.begin()
+        hidden_states = compute_input(hidden_states)
+        if verifier_last_hidden_states is not None:
+            verifier_last_hidden_states = compute_input(verifier_last_hidden_states)
         if position_ids is None:
             position_ids = 1 + torch.arange(t, dtype=torch.long, device=device).unsqueeze(0)
         doc = document_ids.reshape(-1).to(device)
@@ -332,16 +345,15 @@ class Eagle3DraftModel(nn.Module):
                 if li != last:
                     y = _Prenormed(y, normed)
             hidden = normed if cfg.norm_output else y
+            head = self._stager.get(self.lm_head.weight)
             fuse = (return_loss and self.fuse_head_loss and normed.requires_grad
-                    and not self.lm_head.weight.requires_grad and normed.dtype == torch.bfloat16
-                    and self.lm_head.weight.dtype == torch.bfloat16)
+                    and not head.trainable)
             if not fuse:
-                logits = self._linear(normed, self.lm_head.weight, frozen=True)
+                logits = gemm.linear_staged(normed, head, hip=True)
 
             if return_loss:
                 # head + loss as one autograd node while the head is frozen (see metrics.Head)
-                lg = MT.Head(normed, self.lm_head.weight,
-                             self._transposed_frozen(self.lm_head.weight)) if fuse else logits
+                lg = MT.Head(normed, head.w, head.wt) if fuse else logits
                 s_loss, s_metrics, pred = MT.compute_metrics(
                     lg, targets, loss_mask, prev_correct, step, ttt_step_loss_decay,
                     loss_config=loss_config, target_stats_cache=stats_cache, return_pred=True)

@@ -6,11 +6,10 @@ with the same NT kernel against a transposed copy of the weight
 (``weight_t``, ``[K, N]`` contiguous) -- kept by the caller for frozen weights
 such as ``lm_head`` (model.py:70-71) so it is made once -- and leaves the
 weight gradient (a TN product) to the rocBLAS/hipBLASLt matmul of PyTorch.
+The models call the ``*_staged`` forms below with the compute weights of ``weights.WeightStager``.
 """
 
 from __future__ import annotations
-
-import os
 
 import torch
 
@@ -110,101 +109,58 @@ def linear(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor | None 
     return _Linear.apply(x, weight, weight_t)
 
 
-FUSE_WGRAD_ACCUMULATION = os.environ.get("SPX_FUSE_WGRAD", "1") != "0"
-
-
-class _LinearAccumulate(torch.autograd.Function):
-    """``x @ weight.T`` on PyTorch's (hipBLASLt) matmul whose backward ADDS the weight
-    gradient into ``weight.grad`` inside the GEMM (beta = 1) instead of returning a fresh
-    tensor for autograd to add.  A weight that is applied once per TTT step otherwise costs
-    one full read-modify-write pass over a weight-sized tensor per step after the first."""
+class _StagedLinear(torch.autograd.Function):
+    """``x @ w.T`` against a staged weight (``weights.Staged``): on the MFMA kernel of this library
+    (``hip``) or on PyTorch's hipBLASLt matmul.  The weight gradient is added into the staged
+    weight's fp32 accumulator inside the GEMM; the first such product of a backward returns the
+    accumulator to autograd, the others nothing (see ``weights``)."""
 
     @staticmethod
-    def forward(ctx, x, weight):
-        ctx.save_for_backward(x, weight)
-        return torch.nn.functional.linear(x, weight)
+    def forward(ctx, x, _token, staged, hip: bool):
+        if x.dtype != torch.bfloat16:
+            raise _lib.SpxError("the HIP layer kernels take bf16 tensors")
+        w = staged.w
+        x2 = x.reshape(-1, x.shape[-1])
+        y = gemm_nt(x2, w) if hip else torch.nn.functional.linear(x2, w)
+        ctx.save_for_backward(x2, w)
+        ctx.staged, ctx.hip, ctx.x_shape = staged, hip, x.shape
+        return y.view(*x.shape[:-1], w.shape[0])
 
     @staticmethod
     def backward(ctx, dy):
-        x, weight = ctx.saved_tensors
-        dx = None
+        x2, w = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.shape[-1]).to(torch.bfloat16)
+        dx = dw = None
         if ctx.needs_input_grad[0]:
-            dx = torch.matmul(dy, weight)
-        if weight.requires_grad:
-            dy2 = dy.reshape(-1, dy.shape[-1])
-            x2 = x.reshape(-1, x.shape[-1])
-            if weight.grad is None:
-                weight.grad = torch.matmul(dy2.t(), x2)
-            else:
-                torch.addmm(weight.grad, dy2.t(), x2, out=weight.grad)
-        return dx, None
+            dx = (gemm_nt(dy2, ctx.staged.wt) if ctx.hip else torch.matmul(dy2, w)).view(ctx.x_shape)
+        if ctx.needs_input_grad[1]:
+            dw = ctx.staged.add_wgrad(dy2, x2)
+        return dx, dw, None, None
 
 
-def linear_accumulate(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """See ``_LinearAccumulate``.  The weight gradient lands in ``weight.grad`` during
-    ``backward()`` (it is not visible to ``torch.autograd.grad``)."""
-    if not FUSE_WGRAD_ACCUMULATION or not torch.is_grad_enabled() or not (
-            x.requires_grad or weight.requires_grad):
-        return torch.nn.functional.linear(x, weight)
-    # autograd must see a differentiable input even when only the weight needs a gradient
-    return _LinearAccumulate.apply(x, weight)
-
-
-class _MergedWeights:
-    """Per-module state of a merged projection (q/k/v, or gate/up): the concatenated weight of the
-    current weight versions, and the merged gradient buffer the ``.grad`` tensors are views of."""
-
-    def __init__(self):
-        self.key = None
-        self.weight = None
-        self.grad = None
-
-    def merged_weight(self, ws):
-        key = tuple((w.data_ptr(), w._version) for w in ws)
-        if key != self.key:
-            self.weight = torch.cat([w.detach() for w in ws], dim=0)
-            self.key = key
-        return self.weight
-
-    def accumulate(self, ws, dy2, x2):
-        """``grad(w_i) += dy2[:, rows_i].T @ x2`` for all the weights with one GEMM.  While their
-        ``.grad`` are the views this object handed out, the GEMM adds into the shared buffer
-        (beta = 1); otherwise (gradients that came from elsewhere) it falls back to one add each."""
-        sizes = [w.shape[0] for w in ws]
-        views = None
-        if self.grad is not None:
-            views = self.grad.split(sizes, dim=0)
-            if not all(w.grad is not None and w.grad.data_ptr() == v.data_ptr()
-                       and w.grad.shape == v.shape for w, v in zip(ws, views, strict=True)):
-                views = None
-        if views is not None:
-            torch.addmm(self.grad, dy2.t(), x2, out=self.grad)
-            return
-        fresh = torch.matmul(dy2.t(), x2)
-        parts = fresh.split(sizes, dim=0)
-        if all(w.grad is None for w in ws):
-            self.grad = fresh
-            for w, v in zip(ws, parts, strict=True):
-                w.grad = v
-        else:
-            self.grad = None
-            for w, v in zip(ws, parts, strict=True):
-                if w.requires_grad:
-                    w.grad = v.clone() if w.grad is None else w.grad.add_(v)
+def linear_staged(x: torch.Tensor, staged, hip: bool = False) -> torch.Tensor:
+    """``x[..., K] @ staged.w[N, K].T``; see ``_StagedLinear``."""
+    if not torch.is_grad_enabled() or not (x.requires_grad or staged.trainable):
+        x2 = x.reshape(-1, x.shape[-1])
+        y = gemm_nt(x2, staged.w) if hip else torch.nn.functional.linear(x2, staged.w)
+        return y.view(*x.shape[:-1], staged.w.shape[0])
+    return _StagedLinear.apply(x, staged.token, staged, hip)
 
 
 class _QKVRope(torch.autograd.Function):
-    """q/k/v projections of one input as ONE GEMM against the concatenated weight, followed by
-    the rotary embedding + head-major relayout of each part.  The backward undoes the relayout
-    into the three column blocks of one ``[T, Nq + 2 Nkv]`` buffer, so the input gradient is one
-    GEMM (no per-projection partial results to add up) and the weight gradient one GEMM that
-    accumulates across TTT steps."""
+    """q/k/v projections of one input as ONE GEMM against the staged concatenation of the three
+    weights, followed by the rotary embedding + head-major relayout of each part.  The backward
+    undoes the relayout into the three column blocks of one ``[T, Nq + 2 Nkv]`` buffer, so the
+    input gradient is one GEMM (no per-projection partial results to add up) and the weight
+    gradient one GEMM that accumulates across TTT steps in fp32."""
 
     @staticmethod
-    def forward(ctx, x, wq, wk, wv, position_ids, inv_freq, hq, hkv, d, offset, state, kv_out=None):
+    def forward(ctx, x, _token, staged, position_ids, inv_freq, hq, hkv, d, offset, kv_out=None):
+        if x.dtype != torch.bfloat16:
+            raise _lib.SpxError("the HIP layer kernels take bf16 tensors")
+        wcat = staged.w
         t = x.shape[-2]
         x2 = x.reshape(t, x.shape[-1])
-        wcat = state.merged_weight((wq, wk, wv))
         qkv = torch.nn.functional.linear(x2, wcat)
         n = qkv.shape[1]
         st = _lib.stream_ptr(x.device)
@@ -222,15 +178,15 @@ class _QKVRope(torch.autograd.Function):
                       _lib.ptr(out), head_stride, t, heads, d, rotate, 0, int(offset), st)
             outs.append(out)
             col += heads * d
-        ctx.save_for_backward(x2, wq, wk, wv, position_ids, inv_freq)
-        ctx.meta = (x.shape, hq, hkv, d, offset, n, state, wcat)
+        ctx.save_for_backward(x2, wcat, position_ids, inv_freq)
+        ctx.meta = (x.shape, hq, hkv, d, offset, n, staged)
         ctx.set_materialize_grads(False)
         return tuple(outs)
 
     @staticmethod
     def backward(ctx, dq, dk, dv):
-        x2, wq, wk, wv, position_ids, inv_freq = ctx.saved_tensors
-        shape, hq, hkv, d, offset, n, state, wcat = ctx.meta
+        x2, wcat, position_ids, inv_freq = ctx.saved_tensors
+        shape, hq, hkv, d, offset, n, staged = ctx.meta
         t = x2.shape[0]
         st = _lib.stream_ptr(x2.device)
         dqkv = torch.empty(t, n, device=x2.device, dtype=torch.bfloat16)
@@ -248,52 +204,48 @@ class _QKVRope(torch.autograd.Function):
                 _lib.call("spx_rope_relayout", _lib.ptr(g), g.stride(1), _lib.ptr(position_ids),
                           _lib.ptr(inv_freq), _lib.ptr(part), n, t, heads, d, rotate, 1, int(offset), st)
             col += heads * d
-        dx = None
+        dx = dw = None
         if ctx.needs_input_grad[0]:
             dx = torch.matmul(dqkv, wcat).view(shape)
-        if any(w.requires_grad for w in (wq, wk, wv)):
-            state.accumulate((wq, wk, wv), dqkv, x2)
-        return (dx,) + (None,) * 11
+        if ctx.needs_input_grad[1]:
+            dw = staged.add_wgrad(dqkv, x2)
+        return (dx, dw) + (None,) * 8
 
 
-def qkv_rope(x, wq, wk, wv, position_ids, inv_freq, hq: int, hkv: int, d: int, offset: int,
-             state: _MergedWeights, kv_out=None):
+def qkv_rope(x, staged, position_ids, inv_freq, hq: int, hkv: int, d: int, offset: int, kv_out=None):
     """``(q [1,Hq,T,D], k [1,Hkv,T,D], v [1,Hkv,T,D])`` with the rotary embedding at
-    ``position_ids + offset`` applied to q and k.  Weight gradients land in ``.grad`` during
-    ``backward()`` (like ``linear_accumulate``).  ``kv_out = (k_window, v_window)``: write k and v
-    straight into these ``[1, Hkv, T, D]`` windows of a K / V cache and return them."""
-    return _QKVRope.apply(x, wq, wk, wv, position_ids, inv_freq, hq, hkv, d, offset, state, kv_out)
-
-
-_MergedQKV = _MergedWeights
+    ``position_ids + offset`` applied to q and k; ``staged`` holds the row-wise concatenation of
+    the q, k and v weights.  ``kv_out = (k_window, v_window)``: write k and v straight into these
+    ``[1, Hkv, T, D]`` windows of a K / V cache and return them."""
+    return _QKVRope.apply(x, staged.token, staged, position_ids, inv_freq, hq, hkv, d, offset, kv_out)
 
 
 class _GateUpSwiGLU(torch.autograd.Function):
-    """``silu(x @ Wg.T) * (x @ Wu.T)`` with the two projections as ONE GEMM against the
-    concatenated weight; the SwiGLU kernels read (and, in the backward, write) the two column
-    halves of the merged ``[T, 2F]`` buffer in place, so the input gradient is one GEMM and the
-    weight gradient one GEMM that accumulates across TTT steps."""
+    """``silu(x @ Wg.T) * (x @ Wu.T)`` with the two projections as ONE GEMM against the staged
+    concatenation of the two weights; the SwiGLU kernels read (and, in the backward, write) the two
+    column halves of the merged ``[T, 2F]`` buffer in place, so the input gradient is one GEMM and
+    the weight gradient one GEMM that accumulates across TTT steps in fp32."""
 
     @staticmethod
-    def forward(ctx, x, wg, wu, state):
+    def forward(ctx, x, _token, staged):
         if x.dtype != torch.bfloat16:
             raise _lib.SpxError("the HIP layer kernels take bf16 tensors")
+        wcat = staged.w
         x2 = x.reshape(-1, x.shape[-1])
-        f = wg.shape[0]
-        wcat = state.merged_weight((wg, wu))
+        f = wcat.shape[0] // 2
         gu = torch.nn.functional.linear(x2, wcat)  # [T, 2F]
         rows = x2.shape[0]
         out = torch.empty(rows, f, device=x.device, dtype=torch.bfloat16)
         _lib.call("spx_swiglu_rows_fwd", _lib.ptr(gu), 2 * f, _lib.ptr(gu[:, f:]), 2 * f, _lib.ptr(out), f,
                   rows, f, _lib.stream_ptr(x.device))
-        ctx.save_for_backward(x2, gu, wg, wu)
-        ctx.meta = (x.shape, f, state, wcat)
+        ctx.save_for_backward(x2, gu, wcat)
+        ctx.meta = (x.shape, f, staged)
         return out.view(*x.shape[:-1], f)
 
     @staticmethod
     def backward(ctx, dout):
-        x2, gu, wg, wu = ctx.saved_tensors
-        shape, f, state, wcat = ctx.meta
+        x2, gu, wcat = ctx.saved_tensors
+        shape, f, staged = ctx.meta
         rows = x2.shape[0]
         d2 = dout.reshape(rows, f).to(torch.bfloat16)
         if d2.stride(1) != 1 or d2.stride(0) % 8:
@@ -302,14 +254,15 @@ class _GateUpSwiGLU(torch.autograd.Function):
         _lib.call("spx_swiglu_rows_bwd", _lib.ptr(gu), 2 * f, _lib.ptr(gu[:, f:]), 2 * f, _lib.ptr(d2),
                   d2.stride(0), _lib.ptr(dgu), 2 * f, _lib.ptr(dgu[:, f:]), 2 * f, rows, f,
                   _lib.stream_ptr(x2.device))
-        dx = None
+        dx = dw = None
         if ctx.needs_input_grad[0]:
             dx = torch.matmul(dgu, wcat).view(shape)
-        if wg.requires_grad or wu.requires_grad:
-            state.accumulate((wg, wu), dgu, x2)
-        return dx, None, None, None
+        if ctx.needs_input_grad[1]:
+            dw = staged.add_wgrad(dgu, x2)
+        return dx, dw, None
 
 
-def gate_up_swiglu(x, w_gate, w_up, state: _MergedWeights):
-    """See ``_GateUpSwiGLU``.  Weight gradients land in ``.grad`` during ``backward()``."""
-    return _GateUpSwiGLU.apply(x, w_gate, w_up, state)
+def gate_up_swiglu(x, staged):
+    """See ``_GateUpSwiGLU``; ``staged`` holds the row-wise concatenation of the gate and up
+    weights."""
+    return _GateUpSwiGLU.apply(x, staged.token, staged)

@@ -32,6 +32,7 @@ from . import fused_ops as FO
 from . import gemm
 from . import losses as L
 from .eagle3 import MLP, Attention, RMSNorm
+from .weights import WeightStager, compute_input
 
 IGNORE_INDEX = -100
 
@@ -63,29 +64,30 @@ class MTPConfig:
 class MTPLayer(nn.Module):
     """``Qwen3MTPLayer`` (models/mtp/model_definitions.py:78-151)."""
 
-    def __init__(self, cfg: MTPConfig):
+    def __init__(self, cfg: MTPConfig, stager: WeightStager):
         super().__init__()
         h, eps = cfg.hidden_size, cfg.rms_norm_eps
-        self.hidden_layernorm = RMSNorm(h, eps)
-        self.token_layernorm = RMSNorm(h, eps)
+        self._stager = stager
+        self.hidden_layernorm = RMSNorm(h, eps, stager)
+        self.token_layernorm = RMSNorm(h, eps, stager)
         self.input_proj = nn.Linear(2 * h, h, bias=False)
-        self.final_layernorm = RMSNorm(h, eps)
-        self.input_layernorm = RMSNorm(h, eps)
-        self.post_attention_layernorm = RMSNorm(h, eps)
-        self.self_attn = Attention(cfg, h)
-        self.mlp = MLP(cfg)
+        self.final_layernorm = RMSNorm(h, eps, stager)
+        self.input_layernorm = RMSNorm(h, eps, stager)
+        self.post_attention_layernorm = RMSNorm(h, eps, stager)
+        self.self_attn = Attention(cfg, h, stager)
+        self.mlp = MLP(cfg, stager)
 
     def forward(self, hidden, embeds, position_ids, inv_freq, mask):
         # both norms write into the halves of the 2H-wide projection input; each residual add is
         # fused into the norm that follows it
-        x = gemm.linear_accumulate(
-            FO.pair_norm_cat(embeds, hidden, self.token_layernorm.weight, self.hidden_layernorm.weight,
+        x = gemm.linear_staged(
+            FO.pair_norm_cat(embeds, hidden, self.token_layernorm.gain, self.hidden_layernorm.gain,
                              self.token_layernorm.eps),
-            self.input_proj.weight)
+            self._stager.get(self.input_proj.weight))
         a = self.self_attn(self.input_layernorm(x), position_ids, 0, inv_freq, {}, mask)
         post, final = self.post_attention_layernorm, self.final_layernorm
-        y, z = FO.add_rms_norm(x, a, post.weight, post.eps)
-        _, out = FO.add_rms_norm(y, self.mlp(z), final.weight, final.eps)
+        y, z = FO.add_rms_norm(x, a, post.gain, post.eps)
+        _, out = FO.add_rms_norm(y, self.mlp(z), final.gain, final.eps)
         return out
 
 
@@ -95,13 +97,13 @@ class MTPDraftModel(nn.Module):
         if config.model_type != "qwen3":
             raise ValueError(f"Unsupported MTP model type '{config.model_type}'. Supported types: ['qwen3']")
         self.config = config
+        self._stager = WeightStager()
         self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size)
         self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
-        self.mtp_layers = nn.ModuleList([MTPLayer(config)])
+        self.mtp_layers = nn.ModuleList([MTPLayer(config, self._stager)])
         # the verifier's embedding and head are frozen (model.py:70-71)
         self.embed_tokens.weight.requires_grad_(False)
         self.lm_head.weight.requires_grad_(False)
-        self._frozen_t: dict = {}
         # lm_head and the loss as one autograd node while the head is frozen (False: two nodes, logits
         # returned with their own gradient path as in the reference)
         self.fuse_head_loss = True
@@ -110,19 +112,20 @@ class MTPDraftModel(nn.Module):
     def layers(self) -> nn.ModuleList:
         return self.mtp_layers
 
-    def _lm_head_t(self):
-        """``lm_head.weight.T`` contiguous, cached until the weight changes."""
-        w = self.lm_head.weight
-        key = (w.data_ptr(), w._version)
-        hit = self._frozen_t.get("lm_head")
-        if hit is None or hit[0] != key:
-            hit = (key, w.detach().t().contiguous())
-            self._frozen_t["lm_head"] = hit
-        return hit[1]
+    def invalidate_weight_caches(self):
+        """Drop the kept bf16 / transposed copies of the frozen weights.  They are keyed on the
+        parameter's address and version counter, which a write through ``param.data`` does not
+        change: call this after such a write.  ``train()`` / ``eval()`` and ``load_state_dict``
+        call it."""
+        self._stager.invalidate()
 
-    def _lm_head(self, x):
-        w = self.lm_head.weight
-        return gemm.linear(x, w, self._lm_head_t() if x.requires_grad else None)
+    def train(self, mode: bool = True):
+        self._stager.invalidate()
+        return super().train(mode)
+
+    def load_state_dict(self, *args, **kwargs):
+        self._stager.invalidate()
+        return super().load_state_dict(*args, **kwargs)
 
     def forward(self, input_ids, hidden_states, attention_mask=None, position_ids=None,
                 loss_mask=None, step_weights=None, return_dict: bool = True, **_kwargs):
@@ -131,8 +134,8 @@ class MTPDraftModel(nn.Module):
             raise NotImplementedError(
                 "the HIP MTP path takes packed rows without padding masks (attention_mask=None, "
                 "as the training collate produces them)")
-        if hidden_states.dtype != torch.bfloat16:
-            raise RuntimeError("the HIP draft path runs in bf16: cast the model and its inputs to bfloat16")
+        self._stager.begin()
+        hidden_states = compute_input(hidden_states)
         input_ids = input_ids.long()
         device = input_ids.device
         b, n = input_ids.shape
@@ -176,14 +179,14 @@ class MTPDraftModel(nn.Module):
                 targets = targets.clone()
                 targets[loss_mask[:, step + 2:step + 2 + valid] == 0] = IGNORE_INDEX
             weight = step_weights[step] if step_weights is not None else 1.0
-            if self.fuse_head_loss and out.requires_grad and not self.lm_head.weight.requires_grad:
+            head = self._stager.get(self.lm_head.weight)
+            if self.fuse_head_loss and out.requires_grad and not head.trainable:
                 # head + loss as one autograd node: the backward skips the ignored positions in the
                 # input-gradient product of the head (the returned logits carry no gradient)
                 unreduced, logits = L.head_label_cross_entropy(
-                    out.view(b, valid, cfg.hidden_size), self.lm_head.weight, self._lm_head_t(),
-                    targets, IGNORE_INDEX)
+                    out.view(b, valid, cfg.hidden_size), head.w, head.wt, targets, IGNORE_INDEX)
             else:
-                logits = self._lm_head(out).view(b, valid, cfg.vocab_size)
+                logits = gemm.linear_staged(out, head, hip=True).view(b, valid, cfg.vocab_size)
                 unreduced = L.label_cross_entropy(logits, targets, IGNORE_INDEX)
             all_logits.append(logits)
             valid_count = (targets != IGNORE_INDEX).sum()

@@ -25,6 +25,13 @@ CASES = [
     (320, 4, 1, 128, [100, 150, 50], None, 3),   # 20 padding rows, ragged T
     (512, 4, 4, 128, [200, 300], 64, 2),
     (200, 2, 2, 64, [77], 16, 4),                # T not a tile multiple, padding tail
+    # eight and more query heads per key head with diagonal keys (the 70B shape is 64 : 8):
+    # the diagonal-key backward keeps eight heads in registers, walks wider groups in passes
+    (256, 8, 1, 128, [100, 140], None, 3),
+    (192, 16, 2, 64, None, 32, 3),
+    (160, 16, 1, 64, [150], None, 2),            # group 16: two passes of eight heads
+    (130, 8, 1, 256, None, None, 3),             # head_dim 256: passes of four heads
+    (96, 12, 1, 128, None, None, 2),             # a group that is not a multiple of the pass
 ]
 
 
@@ -186,6 +193,59 @@ def test_full_size_sampled_rows_and_checksums():
     _check_dv_checksum(v, go, hq)
     # a key of a later step is seen by exactly one row: its gradient is that row's, never zero
     assert (k.grad[0, :, t:2 * t].float().abs().sum(dim=-1) > 0).all()
+
+
+def test_70b_shape_sampled_rows_and_checksums():
+    """The Llama-3.3-70B draft shape: 64 query heads on 8 key heads (group 8), T 8192, head_dim 128,
+    the last of 5 TTT steps; sampled rows (forward, dQ), the dV column-sum identity, and sampled
+    diagonal-key gradients against their closed form (a diagonal key is seen by the eight heads of
+    its group at its own position only)."""
+    from speculators_amd import attention as A
+
+    t, hq, hkv, d, step = 8192, 64, 8, 128, 4
+    g = torch.Generator().manual_seed(11)
+    doc = torch.full((t,), -1, dtype=torch.long)
+    doc[:3000], doc[3000:8000] = 0, 1
+    q = torch.randn(1, hq, t, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    k = torch.randn(1, hkv, (step + 1) * t, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    v = torch.randn(1, hkv, (step + 1) * t, d, generator=g).bfloat16().cuda().requires_grad_(True)
+    go = torch.randn(1, t, hq, d, generator=g).bfloat16().cuda()
+    mask = A.create_ttt_mask(doc.cuda(), t, None)
+    for _ in range(step):
+        mask = mask.extended()
+    out = A.ttt_attention(q, k, v, mask)
+    out.backward(go)
+    rows = torch.cat([torch.tensor([0, 2999, 3000, 7999, 8000, 8191]),
+                      torch.randint(0, t, (26,), generator=g)]).tolist()
+    heads = torch.randint(0, hq, (len(rows),), generator=g).tolist()
+    kv_idx = torch.arange((step + 1) * t)
+
+    def visible(i):
+        vis = (kv_idx % t) == i
+        if doc[i] != -1:
+            vis = vis | ((kv_idx <= i) & (kv_idx < t) & (doc[kv_idx % t] == doc[i]))
+        return vis
+
+    _check_sampled_rows(q, k, v, out, go, rows, heads, visible, d ** -0.5)
+    _check_dv_checksum(v, go, hq)
+    # dK / dV of the diagonal key (j, i) of K/V head c: sum over the 8 heads h of its group of
+    # p_h (dO_h . v - delta_h) scale q_h  and  p_h dO_h, with p_h from the explicit soft-max
+    scale, grp = d ** -0.5, hq // hkv
+    for i, c, j in [(5, 0, 1), (2999, 3, 4), (8100, 7, 2), (4096, 5, 3)]:
+        vis = visible(i).cuda()
+        want_k, want_v = torch.zeros(d), torch.zeros(d)
+        for h in range(c * grp, (c + 1) * grp):
+            qi = q.detach()[0, h, i].float().cpu()
+            ks, vs = k.detach()[0, c, vis].float().cpu(), v.detach()[0, c, vis].float().cpu()
+            p = torch.softmax((ks @ qi) * scale, dim=0)
+            do = go[0, i, h].float().cpu()
+            delta = (p @ vs) @ do
+            pos = int((torch.nonzero(vis.cpu()).reshape(-1) == j * t + i).nonzero())
+            want_k += p[pos] * (vs[pos] @ do - delta) * scale * qi
+            want_v += p[pos] * do
+        got_k, got_v = k.grad[0, c, j * t + i].float().cpu(), v.grad[0, c, j * t + i].float().cpu()
+        assert (got_k - want_k).abs().max() <= 2e-2 * want_k.abs().max() + 1e-4, (i, c, j)
+        assert (got_v - want_v).abs().max() <= 2e-2 * want_v.abs().max() + 1e-4, (i, c, j)
 
 
 def test_full_size_head_dim_256_sampled_rows():

@@ -34,7 +34,7 @@ def _batch(shape, t, seed, docs):
     return hs, ids, doc, mask, pos, vl
 
 
-def _make(shape, w, **extra):
+def _make(shape, w, param_dtype=torch.bfloat16, **extra):
     from speculators_amd.eagle3 import Eagle3Config, Eagle3DraftModel
 
     cfg = Eagle3Config(**extra, **{k: getattr(shape, k) for k in (
@@ -45,7 +45,7 @@ def _make(shape, w, **extra):
     model = Eagle3DraftModel(cfg)
     missing, unexpected = model.load_state_dict(w, strict=False)
     assert not unexpected and set(missing) <= {"t2d", "d2t"}, (missing, unexpected)
-    return model.to(torch.bfloat16).cuda()
+    return model.to(param_dtype).cuda()
 
 
 VARIANTS = [
@@ -115,6 +115,68 @@ def test_forward_backward_matches_oracle(variant):
         top2 = rlogits[k].topk(2, dim=-1).values
         clear = (top2[..., 0] - top2[..., 1]) > 0.05 * top2[..., 0].abs().clamp_min(1.0)
         assert torch.equal(toks[k].cpu()[clear], rt[k][clear])
+
+
+@pytest.mark.parametrize("variant", [VARIANTS[1], VARIANTS[2]])
+def test_fp32_master_weights_under_autocast_match_oracle(variant):
+    """The trainer's regime (train/trainer.py:459-465): fp32 master parameters, forward under
+    ``torch.autocast(bf16)``, fp32 gradients.  Against the fp32 oracle (loss 1e-3, gradients 2e-2
+    relative max-norm or twice the error of the same oracle under CPU autocast), and through
+    ``torch.autograd.grad`` as well as ``backward()``."""
+    shape = _shape(**variant)
+    w32 = OE.random_weights(shape, seed=1, std=0.05)
+    g = torch.Generator().manual_seed(11)
+    for k_ in w32:
+        if k_.endswith("norm.weight") or "layernorm" in k_:
+            w32[k_] = 1 + 0.1 * torch.randn(w32[k_].shape, generator=g)
+    t, steps = 320, 3
+    hs, ids, doc, mask, pos, vl = _batch(shape, t, 2, [120, 170])
+    hs, vl = hs.bfloat16(), vl.bfloat16()  # hidden states are stored in bf16 (train/data.py)
+
+    model = _make(shape, w32, param_dtype=torch.float32)
+    assert model.fc.weight.dtype == torch.float32
+    args = (hs.cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.cuda())
+    with pytest.raises(RuntimeError, match="autocast"):
+        model(*args, ttt_steps=1)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        toks, loss, m = model(*args, ttt_steps=steps, ttt_step_loss_decay=0.9)
+    assert loss.dtype == torch.float32
+    params = {n: p for n, p in model.named_parameters() if p.requires_grad}
+    via_grad = torch.autograd.grad(loss, list(params.values()), retain_graph=True)
+    loss.backward()
+    for (n, p), gg in zip(params.items(), via_grad, strict=True):
+        assert p.grad.dtype == torch.float32 and torch.equal(p.grad, gg), n
+
+    def oracle(autocast):
+        wf = {k_: v.clone().requires_grad_(v.dtype.is_floating_point) for k_, v in w32.items()}
+        with torch.autocast("cpu", dtype=torch.bfloat16, enabled=autocast):
+            _, rl, rm = OE.eagle3_forward(wf, shape, hs.float(), ids, doc, mask, pos, vl.float(),
+                                          ttt_steps=steps, ttt_step_loss_decay=0.9)
+        rl.backward()
+        return rl, rm, wf
+
+    rloss, rm, wf = oracle(False)
+    _, _, wa = oracle(True)
+    rel = abs(loss.item() - rloss.item()) / abs(rloss.item())
+    print("loss", loss.item(), rloss.item(), rel)
+    assert rel < 1e-3
+    for key in rm:
+        if key.endswith("_total"):
+            assert m[key].item() == rm[key].item(), key
+    for name, p in params.items():
+        want = wf[name].grad
+        err = (p.grad.cpu() - want).abs().max().item()
+        floor = (wa[name].grad - want).abs().max().item()
+        assert err <= max(2e-2 * want.abs().max().item(), 2 * floor) + 1e-6, (name, err, floor)
+    # validation: no graph, same loss
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        _, vloss, _ = model(*args, ttt_steps=steps, ttt_step_loss_decay=0.9)
+    assert vloss.item() == loss.item()
+    # an optimizer step on the fp32 masters is seen by the next forward (nothing stale is kept)
+    torch.optim.SGD(params.values(), lr=0.05).step()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        _, vloss2, _ = model(*args, ttt_steps=steps, ttt_step_loss_decay=0.9)
+    assert vloss2.item() < vloss.item()
 
 
 def test_verifier_logits_entry_point_equals_row_sliced_head():

@@ -141,44 +141,62 @@ def test_pair_norm_cat_matches_cat_of_norms(rows, h, embeds_grad):
             assert torch.equal(gt, t.grad)
 
 
+@pytest.mark.parametrize("master", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("t,h_in,hq,hkv,d", [(300, 1024, 8, 2, 128), (129, 512, 4, 4, 64)])
-def test_qkv_rope_matches_separate_projections(t, h_in, hq, hkv, d):
-    """One merged q/k/v GEMM + fused relayouts == three projections + three relayouts, and the
-    weight gradients accumulate over calls like ``linear_accumulate``."""
+def test_qkv_rope_matches_separate_projections(t, h_in, hq, hkv, d, master):
+    """One merged q/k/v GEMM + fused relayouts == three projections + three relayouts; two uses of
+    the staged weight in one graph (two TTT steps) sum their weight gradients in one fp32
+    accumulator that reaches the parameters through autograd, in the parameters' dtype: bf16
+    parameters, and fp32 master parameters under bf16 autocast."""
     from speculators_amd import gemm
     from speculators_amd.fused_ops import rope_inv_freq, rope_relayout
+    from speculators_amd.weights import WeightStager
 
     g = torch.Generator().manual_seed(t)
     x = torch.randn(1, t, h_in, generator=g).bfloat16().cuda().requires_grad_(True)
-    ws = [(torch.randn(n, h_in, generator=g) * 0.05).bfloat16().cuda().requires_grad_(True)
+    ws = [(torch.randn(n, h_in, generator=g) * 0.05).bfloat16().to(master).cuda().requires_grad_(True)
           for n in (hq * d, hkv * d, hkv * d)]
     pos = torch.randint(0, 4000, (t,), generator=g).cuda()
     inv = rope_inv_freq(d, 500000.0, "cuda")
     gos = [torch.randn(1, n, t, d, generator=g).bfloat16().cuda() for n in (hq, hkv, hkv)]
-    state = gemm._MergedQKV()
-    for rep in range(2):  # the second call accumulates into the same merged gradient buffer
-        outs = gemm.qkv_rope(x, *ws, pos, inv, hq, hkv, d, 3, state)
-        torch.autograd.backward(outs, gos)
-    got_x = x.grad.clone()
-    got_w = [w.grad.clone() for w in ws]
-    assert ws[0].grad.data_ptr() == state.grad.data_ptr()
+    stager = WeightStager()
+    seen = []
+    ws[1].register_hook(lambda gr: seen.append(gr.dtype))
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=master == torch.float32):
+        stager.begin()
+        st = stager.get(*ws)
+        assert st.w.dtype == torch.bfloat16 and st.w.shape == ((hq + 2 * hkv) * d, h_in)
+        outs = gemm.qkv_rope(x, st, pos, inv, hq, hkv, d, 3) + gemm.qkv_rope(x, st, pos, inv, hq, hkv, d, 3)
+    via_grad = torch.autograd.grad(outs, [x, *ws], gos + gos, retain_graph=True)
+    torch.autograd.backward(outs, gos + gos)  # a second pass over the retained graph starts afresh
+    assert seen == [master, master]
+    for got, t_ in zip(via_grad, [x, *ws], strict=True):
+        assert got.dtype == t_.dtype and torch.equal(got, t_.grad)
+    got_x, got_w = x.grad.clone(), [w.grad.clone() for w in ws]
     x.grad = None
     for w in ws:
         w.grad = None
     ref = []
     for w, heads, rot in zip(ws, (hq, hkv, hkv), (True, True, False), strict=True):
-        ref.append(rope_relayout(torch.nn.functional.linear(x, w), pos, inv, heads, rot, 3 if rot else 0))
-    for o, r in zip(outs, ref, strict=True):
+        ref.append(rope_relayout(torch.nn.functional.linear(x, w.bfloat16()), pos, inv, heads, rot,
+                                 3 if rot else 0))
+    for o, r in zip(outs[:3], ref, strict=True):
         _close(o, r.detach().cpu(), rel=1e-2)
     torch.autograd.backward(ref, gos)
     _close(got_x, 2 * x.grad.cpu())
     for gw, w in zip(got_w, ws, strict=True):
+        assert gw.dtype == master
         _close(gw, 2 * w.grad.cpu())
-    # gradients that did not come from the merged buffer are added to, not replaced
-    for w in ws:
+    # existing gradients are added to, not replaced; a frozen member of the group gets none
+    ws[2].requires_grad_(False)
+    ws[2].grad = None
+    for w in ws[:2]:
         w.grad = torch.ones_like(w)
-    torch.autograd.backward(gemm.qkv_rope(x, *ws, pos, inv, hq, hkv, d, 3, state), gos)
-    for gw, w in zip(got_w, ws, strict=True):
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=master == torch.float32):
+        stager.begin()
+        torch.autograd.backward(gemm.qkv_rope(x, stager.get(*ws), pos, inv, hq, hkv, d, 3), gos)
+    assert ws[2].grad is None
+    for gw, w in zip(got_w[:2], ws[:2], strict=True):
         _close(w.grad - 1, 0.5 * gw.cpu())
 
 
@@ -187,23 +205,50 @@ def test_gate_up_swiglu_matches_separate_projections(t, h, f):
     """One merged gate/up GEMM + SwiGLU on its two halves == two projections + SwiGLU."""
     from speculators_amd import gemm
     from speculators_amd.fused_ops import swiglu
+    from speculators_amd.weights import WeightStager
 
     g = torch.Generator().manual_seed(t + f)
     x = torch.randn(1, t, h, generator=g).bfloat16().cuda().requires_grad_(True)
     wg = (torch.randn(f, h, generator=g) * 0.05).bfloat16().cuda().requires_grad_(True)
     wu = (torch.randn(f, h, generator=g) * 0.05).bfloat16().cuda().requires_grad_(True)
     go = torch.randn(1, t, f, generator=g).bfloat16().cuda()
-    state = gemm._MergedWeights()
-    out = gemm.gate_up_swiglu(x, wg, wu, state)
+    stager = WeightStager()
+    stager.begin()
+    out = gemm.gate_up_swiglu(x, stager.get(wg, wu))
     out.backward(go)
     got = [x.grad.clone(), wg.grad.clone(), wu.grad.clone()]
-    assert wg.grad.data_ptr() == state.grad.data_ptr()
     x.grad = wg.grad = wu.grad = None
     ref = swiglu(torch.nn.functional.linear(x, wg), torch.nn.functional.linear(x, wu))
     ref.backward(go)
     _close(out, ref.detach().cpu(), rel=1e-2)
     for a, b in zip(got, (x.grad, wg.grad, wu.grad), strict=True):
         _close(a, b.cpu())
+
+
+def test_stager_refuses_fp32_outside_autocast_and_keeps_frozen_copies():
+    from speculators_amd.weights import WeightStager, compute_input
+
+    w = torch.randn(64, 32, device="cuda")
+    stager = WeightStager()
+    stager.begin()
+    with pytest.raises(RuntimeError, match="autocast"):
+        stager.get(w)
+    with pytest.raises(RuntimeError, match="autocast"):
+        compute_input(torch.randn(4, 4, device="cuda"))
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        a = stager.get(w)
+        assert a.w.dtype == torch.bfloat16 and torch.equal(a.w, w.bfloat16())
+        assert torch.equal(a.wt, w.bfloat16().t().contiguous())
+        stager.begin()
+        assert stager.get(w) is a and not a.trainable   # a frozen weight is cast once and kept
+        w.mul_(2)                            # an in-place change bumps the version counter
+        stager.begin()
+        b = stager.get(w)
+        assert b is not a and torch.equal(b.w, w.bfloat16())
+        w.data.add_(1)                       # a write through .data does not: invalidate() does
+        stager.invalidate()
+        assert torch.equal(stager.get(w).w, w.bfloat16())
+        assert compute_input(torch.ones(2, 2, device="cuda")).dtype == torch.bfloat16
 
 
 @pytest.mark.parametrize("rows", [1, 63, 64, 1024, 1025, 5000])
