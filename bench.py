@@ -25,20 +25,46 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-# HBM traffic per launch (bytes) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the
-# default shapes and scaled by what the same counters read for a plain copy of known size
-# (FETCH_SIZE under-reads by 1.9998x on this hardware, WRITE_SIZE reads 1.0x); the summary of
-# those runs is profiles/kernels_config1_hbm_traffic_pmc.txt.  Only valid for the default
-# --seq-len / --ttt-steps; other shapes report null.
-KIB = 1024
-MEASURED_TRAFFIC = {
-    "gemm_fwd": int((1.9998 * 954294 + 256566) * KIB),
-    "gemm_dx": int((1.9998 * 768419 + 32833) * KIB),
-    "loss_fwd": int((1.9998 * 256051 + 768) * KIB),
-    "loss_fwd_reuse": int((1.9998 * 256166 + 512) * KIB),
-    "loss_bwd": int((1.9998 * 256416 + 256000) * KIB),
-    "attn_fwd": int((1.9998 * 78162 + 33280) * KIB),
+# HBM traffic per launch (bytes): read at import from the committed rocprofv3 --pmc summary
+# (FETCH_SIZE / WRITE_SIZE in KiB per dispatch, one counter per run, at the default shapes), scaled
+# by what the same counters read for a plain copy of known size (the factor is stated in that
+# file).  Only valid for the default --seq-len / --ttt-steps; other shapes, and kernels the
+# summary does not list, report null.
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "kernels_config1_hbm_traffic_pmc.txt")
+# bench key -> (substring of the kernel name, launch grid in threads or None = any)
+TRAFFIC_ROWS = {
+    "gemm_fwd": ("gemm_bf16_nt_kernel", 512000),
+    "gemm_dx": ("gemm_bf16_nt_kernel", 65536),
+    "loss_fwd": ("loss_fwd_kernel<unsigned short, 0, true, false", None),
+    "loss_fwd_reuse": ("loss_fwd_kernel<unsigned short, 0, true, true", None),
+    "loss_bwd": ("loss_bwd_kernel<unsigned short, 0", None),
+    "attn_fwd": ("attn_fwd_kernel<128", None),
 }
+
+
+def load_measured_traffic(path=TRAFFIC_SUMMARY):
+    import re
+
+    try:
+        text = open(path).read()
+    except OSError:
+        return {}
+    m = re.search(r"FETCH_SIZE under-reads by\s+a factor ([0-9.]+)", text.replace("\n#", " "))
+    fetch_scale = float(m.group(1)) if m else 1.0
+    rows = []
+    for line in text.splitlines():
+        m = re.match(r"^(?!#)(.*?) grid=(\d+)\s+n=\s*\d+\s+FETCH_KiB avg\s+([0-9.]+)\s+WRITE_KiB avg\s+([0-9.]+)", line)
+        if m:
+            rows.append((m.group(1), int(m.group(2)), float(m.group(3)), float(m.group(4))))
+    out = {}
+    for key, (name, grid) in TRAFFIC_ROWS.items():
+        hit = [r for r in rows if name in r[0] and (grid is None or r[1] == grid)]
+        if len(hit) == 1:
+            out[key] = int((fetch_scale * hit[0][2] + hit[0][3]) * 1024)
+    return out
+
+
+MEASURED_TRAFFIC = load_measured_traffic()
 
 CONFIG1 = dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
                intermediate_size=14336, vocab_size=128256, draft_vocab_size=32000,
@@ -66,6 +92,10 @@ def parse_args():
                     help="hidden: verifier_last_hidden_states through the frozen verifier head "
                          "(the reference's forward contract); logits: full-vocab verifier "
                          "logits gathered through d2t")
+    ap.add_argument("--regime", choices=["autocast", "bf16"], default="autocast",
+                    help="autocast: fp32 master weights, forward under torch.autocast(bf16), fp32 "
+                         "gradients (the regime of the reference's Trainer, train/trainer.py:459-465); "
+                         "bf16: the whole model cast to bf16 (the reference's integration tests)")
     ap.add_argument("--cpu-baseline", choices=["sample", "off"], default="sample")
     ap.add_argument("--cpu-seq-len", type=int, default=1024)
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline timing")
@@ -95,18 +125,20 @@ def make_inputs(torch, cfg, t, device, with_logits):
     return batch, d2t, t2d
 
 
-def make_model(torch, cfg, device, d2t, t2d):
+def make_model(torch, cfg, device, d2t, t2d, param_dtype=None):
+    """Random-init draft of the given shape; the same bf16-representable values in either
+    parameter dtype, so the two regimes start from identical weights."""
     from speculators_amd.eagle3 import Eagle3Config, Eagle3DraftModel
 
     model = Eagle3DraftModel(Eagle3Config(**cfg))
     g = torch.Generator(device=device).manual_seed(1)
-    model = model.to(torch.bfloat16).to(device)
+    model = model.to(param_dtype or torch.bfloat16).to(device)
     with torch.no_grad():
         for name, p in model.named_parameters():
             if name.endswith("norm.weight") or "layernorm" in name:
                 p.fill_(1.0)
             else:
-                p.copy_((torch.randn(p.shape, device=device, generator=g) * 0.02).to(p.dtype))
+                p.copy_((torch.randn(p.shape, device=device, generator=g) * 0.02).bfloat16().to(p.dtype))
     model.load_vocab_mappings(t2d, d2t)
     return model
 
@@ -316,36 +348,109 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
     return out
 
 
-def cpu_baseline(cfg, t, k_steps):
-    """The oracle (CPU restatement of the reference eager path) timed on the host cores:
-    one forward + backward at the config[1] shape on a shortened sequence."""
-    import torch
+CONFIG0 = dict(hidden_size=2048, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+               intermediate_size=8192, vocab_size=128256, draft_vocab_size=32000,
+               rope_theta=500000.0, rms_norm_eps=1e-5)
+SEQ_LEN0, TTT_STEPS0 = 512, 3
 
+
+def _cpu_model_name():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _oracle_case(torch, cfg, t, scale):
+    """Seeded weights and one packed row of the given shape, on the host (fp32)."""
     from oracle import eagle3 as OE
 
+    shape = OE.DraftShape(**cfg)
+    w = OE.random_weights(shape, seed=0)
+    g = torch.Generator().manual_seed(0)
+    hs = (torch.randn(1, t, 3 * shape.hidden_size, generator=g) * scale).bfloat16().float()
+    ids = torch.randint(0, shape.vocab_size, (1, t), generator=g)
+    vl = torch.randn(1, t, shape.hidden_size, generator=g).bfloat16().float()
+    mask = (torch.rand(1, t, generator=g) < 0.7).float()
+    doc = torch.zeros(1, t, dtype=torch.long)
+    return shape, w, (hs, ids, doc, mask, None, vl)
+
+
+def _oracle_step(torch, shape, w, case, k_steps):
+    from oracle import eagle3 as OE
+
+    frozen = ("embed_tokens.weight", "lm_head.weight", "verifier_lm_head.weight", "verifier_norm.weight")
+    for name, p in w.items():
+        p.grad = None
+        p.requires_grad_(name not in frozen)
+    t0 = time.perf_counter()
+    _, loss, metrics = OE.eagle3_forward(w, shape, *case, ttt_steps=k_steps, attn="sdpa")
+    loss.backward()
+    return time.perf_counter() - t0, float(loss.detach()), metrics
+
+
+def _hip_same_case(torch, device, cfg, w, case, k_steps):
+    """The HIP model (fp32 master weights under bf16 autocast) on the oracle's weights and inputs."""
+    from speculators_amd.eagle3 import Eagle3Config, Eagle3DraftModel
+
+    model = Eagle3DraftModel(Eagle3Config(**cfg))
+    model.load_state_dict({k: v.detach() for k, v in w.items()}, strict=False)
+    model = model.to(device)
+    hs, ids, doc, mask, _pos, vl = case
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        _, loss, metrics = model(hs.bfloat16().to(device), ids.to(device), doc.to(device), mask.to(device),
+                                 None, vl.bfloat16().to(device), ttt_steps=k_steps)
+    loss.backward()
+    out = float(loss.detach()), {k: float(v) for k, v in metrics.items()}
+    del model
+    torch.cuda.empty_cache()
+    return out
+
+
+def cpu_baseline(torch, device, cfg, t, k_steps):
+    """The oracle (CPU restatement of the reference eager path, fp32) timed on the host cores:
+    configs[0] in full (1 warm-up + 3 timed forward + backward), and one forward + backward of
+    the headline shape on a shortened sequence.  Both cases also go through the HIP model with the
+    same weights and inputs: an in-run parity check (loss, exact mask counts)."""
     cores = os.cpu_count() or 1
     threads = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(threads)
-    shape = OE.DraftShape(**cfg)
-    w = OE.random_weights(shape, seed=0)
-    for name, p in w.items():
-        if name not in ("embed_tokens.weight", "lm_head.weight", "verifier_lm_head.weight",
-                        "verifier_norm.weight"):
-            p.requires_grad_(True)
-    g = torch.Generator().manual_seed(0)
-    hs = torch.randn(1, t, 3 * shape.hidden_size, generator=g) * 4
-    ids = torch.randint(0, shape.vocab_size, (1, t), generator=g)
-    vl = torch.randn(1, t, shape.hidden_size, generator=g)
-    mask = (torch.rand(1, t, generator=g) < 0.7).float()
-    doc = torch.zeros(1, t, dtype=torch.long)
-    t0 = time.perf_counter()
-    _, loss, _ = OE.eagle3_forward(w, shape, hs, ids, doc, mask, None, vl, ttt_steps=k_steps, attn="sdpa")
-    loss.backward()
-    dt = time.perf_counter() - t0
+
+    def parity(gpu, cpu_loss, cpu_metrics):
+        gl, gm = gpu
+        totals = [k for k in cpu_metrics if k.endswith("_total")]
+        return {"loss_gpu": round(gl, 6), "loss_cpu": round(cpu_loss, 6),
+                "rel": round(abs(gl - cpu_loss) / abs(cpu_loss), 7),
+                "counts_equal": all(gm[k] == float(cpu_metrics[k]) for k in totals)}
+
+    # configs[0]: the reference's own CPU-runnable case, in full
+    shape0, w0, case0 = _oracle_case(torch, CONFIG0, SEQ_LEN0, 1.0)
+    _oracle_step(torch, shape0, w0, case0, TTT_STEPS0)
+    times = []
+    for _ in range(3):
+        dt, loss0, m0 = _oracle_step(torch, shape0, w0, case0, TTT_STEPS0)
+        times.append(dt)
+    mean0 = sum(times) / len(times)
+    std0 = (sum((x - mean0) ** 2 for x in times) / len(times)) ** 0.5
+    cfg0 = {"workload": f"configs[0]: Llama-3.2-1B shape, seq {SEQ_LEN0}, TTT {TTT_STEPS0}, fp32, in full",
+            "value": round(SEQ_LEN0 / mean0, 2), "unit": "tokens/s",
+            "s_per_iteration": round(mean0, 3), "s_std": round(std0, 3), "iterations": "1 warm-up + 3 timed",
+            "parity": parity(_hip_same_case(torch, device, CONFIG0, w0, case0, TTT_STEPS0), loss0, m0)}
+    del w0, case0
+
+    # the headline shape on a shortened sequence
+    shape, w, case = _oracle_case(torch, cfg, t, 4.0)
+    dt, loss, m = _oracle_step(torch, shape, w, case, k_steps)
+    par = parity(_hip_same_case(torch, device, cfg, w, case, k_steps), loss, m)
     return {"value": round(t / dt, 2), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "cpu_model": _cpu_model_name(), "host_cpus": cores,
             "sample": f"config[1] shape (Llama-3.1-8B draft, TTT {k_steps}, fp32 oracle), sequence "
                       f"shortened to {t} tokens, 1 forward+backward, no warm-up, {dt:.1f} s",
-            "loss": round(float(loss), 6)}
+            "parity": par, "configs0": cfg0}
 
 
 # configs[4]: MTP head finetune, Qwen3-Next-like shape.  The FFN width is not stated there;
@@ -403,7 +508,7 @@ def run_mtp(args):
         torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
     tokens = b * n
-    final_loss = float(loss)
+    final_loss = float(loss.detach())
     del loss
     model.zero_grad(set_to_none=True)
     torch.cuda.empty_cache()
@@ -655,15 +760,36 @@ def main():
         print(json.dumps({"kernels": kernel_rooflines(torch, CONFIG1, t, k_steps, device)}))
         return
     batch, d2t, t2d = make_inputs(torch, CONFIG1, t, device, args.targets == "logits")
-    model = make_model(torch, CONFIG1, device, d2t, t2d)
     loss_cfg = None  # kl_div, the reference default
+    autocast = args.regime == "autocast"
 
-    def step():
-        model.zero_grad(set_to_none=True)
-        _, loss, _ = model(**batch, ttt_steps=k_steps, ttt_step_loss_decay=1.0, loss_config=loss_cfg)
-        loss.backward()
-        return loss
+    def build(auto):
+        mdl = make_model(torch, CONFIG1, device, d2t, t2d, torch.float32 if auto else torch.bfloat16)
 
+        def one_step():
+            mdl.zero_grad(set_to_none=True)
+            with torch.autocast("cuda", dtype=torch.bfloat16, enabled=auto):
+                _, loss_, _ = mdl(**batch, ttt_steps=k_steps, ttt_step_loss_decay=1.0, loss_config=loss_cfg)
+            loss_.backward()
+            return loss_
+        return mdl, one_step
+
+    # the other regime first, timed the same way (reported beside the headline, not as `value`)
+    model, step = build(not autocast)
+    for _ in range(args.warmup):
+        step()
+    with quiet_gc():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            loss = step()
+        torch.cuda.synchronize()
+    other_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    other_loss = float(loss.detach())
+    del model, step, loss
+    torch.cuda.empty_cache()
+
+    model, step = build(autocast)
     for _ in range(args.warmup):
         step()
     # the lm_head forward product (and the verifier head, the same shape) is timed where it runs:
@@ -700,7 +826,7 @@ def main():
     if args.cpu_baseline != "off":
         del model
         torch.cuda.empty_cache()
-        cpu = cpu_baseline(CONFIG1, args.cpu_seq_len, k_steps)
+        cpu = cpu_baseline(torch, device, CONFIG1, args.cpu_seq_len, k_steps)
 
     line = {
         "metric": ("draft train tokens/sec (fwd+bwd) @Llama-3.1-70B EAGLE3 TTT5" if big else
@@ -712,10 +838,17 @@ def main():
                                 "configs[1]: EAGLE3 draft, Llama-3.1-8B shape, one draft layer, ")
                                +
                                f"batch 1, seq {t}, TTT {k_steps}, vocab 128256 -> draft 32000, "
-                               "kl_div loss, bf16 weights and activations, full attention, "
+                               "kl_div loss, "
+                               + ("fp32 master weights under torch.autocast(bf16), fp32 gradients "
+                                  "(the reference Trainer's regime), " if autocast else
+                                  "bf16 weights and activations (whole model cast), ")
+                               + "full attention, "
                                f"targets from {'verifier hidden states through the frozen verifier head' if args.targets == 'hidden' else 'full-vocab verifier logits gathered through d2t'}",
                    "seq_len": t, "ttt_steps": k_steps, "tokens_per_step": tokens,
-                   "final_loss": round(float(loss), 6)},
+                   "regime": args.regime, "final_loss": round(float(loss.detach()), 6)},
+        "other_regime": {"regime": "bf16" if autocast else "autocast", "ms_per_step": round(other_ms, 3),
+                         "value": round(tokens / (other_ms * 1e-3), 1), "unit": "tokens/s",
+                         "final_loss": round(other_loss, 6)},
         "roofline": ({k: dominant[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
                      | {"kernel": dominant["kernel"]}) if dominant else None,
         "kernels": kernels,
