@@ -167,9 +167,13 @@ def later_layer(x, w, idx, shape, cos, sin, cache, mask, attn="dense"):
 def eagle3_forward(w, shape: DraftShape, hidden_states, input_ids, document_ids,
                    loss_mask=None, position_ids=None, verifier_last_hidden_states=None,
                    ttt_steps: int = 3, ttt_step_loss_decay: float = 1.0,
-                   loss_config=None, attn: str = "dense", return_logits: bool = False):
+                   loss_config=None, attn: str = "dense", return_logits: bool = False,
+                   verifier_logits=None, d2t=None):
     """-> (draft_tokens, loss, metrics[, logits per step]).
-    models/eagle3/core.py:192-365."""
+    models/eagle3/core.py:192-365.  ``verifier_logits`` (``[1, T, Vt]``, with the ``d2t`` offset
+    table) stands in for ``verifier_last_hidden_states``: the targets are then those logits at
+    the draft ids ``i + d2t[i]`` -- what the row-sliced verifier head computes, by the identity
+    ``(W h)[t2d] == W[t2d] h`` (model.py:161-169; pinned in tests/test_oracle_metrics.py)."""
     t = hidden_states.shape[1]
     dtype = hidden_states.dtype
     if position_ids is None:
@@ -190,14 +194,19 @@ def eagle3_forward(w, shape: DraftShape, hidden_states, input_ids, document_ids,
     hidden = F.linear(x, w["fc.weight"])
 
     original_ids = input_ids.detach().clone()
-    with_loss = verifier_last_hidden_states is not None
-    if with_loss:
+    with_loss = verifier_last_hidden_states is not None or verifier_logits is not None
+    if verifier_logits is not None:
+        from .vocab import gather_targets
+
+        targets = (gather_targets(verifier_logits, d2t) if d2t is not None else verifier_logits).detach()
+    elif with_loss:
         with torch.no_grad():
             targets = F.linear(
                 rms_norm(verifier_last_hidden_states, w["verifier_norm.weight"],
                          shape.rms_norm_eps),
                 w["verifier_lm_head.weight"],
             )
+    if with_loss:
         loss = torch.zeros(())
         prev_correct = (loss_mask.clone() if loss_mask is not None
                         else torch.ones(1, t, dtype=torch.bool))

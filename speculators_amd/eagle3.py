@@ -237,6 +237,10 @@ class Eagle3DraftModel(nn.Module):
         # lm_head and the loss as one autograd node while the head is frozen and the loss is a single
         # fused reduction (False: always two nodes)
         self.fuse_head_loss = True
+        # True: every forward leaves its per-step draft logits ([1, T, Vd], detached) in
+        # ``last_logits`` (for parity checks; the reference returns no logits either)
+        self.keep_logits = False
+        self.last_logits: list = []
 
     # ------------------------------------------------------------------ helpers
     def load_vocab_mappings(self, t2d, d2t):
@@ -328,6 +332,7 @@ class Eagle3DraftModel(nn.Module):
         inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device, cfg.rope_scaling)
         position_ids = position_ids.reshape(-1).to(torch.int64).contiguous()
         draft_tokens = []
+        self.last_logits = []
         for step in range(ttt_steps):
             # looked up without a graph whatever embed_requires_grad says, as the reference does
             # (models/eagle3/core.py:270-271): the flag only marks the parameter as trainable
@@ -370,6 +375,8 @@ class Eagle3DraftModel(nn.Module):
             else:
                 draft_tokens.append(MT.argmax_rows(logits.detach()))
 
+            if self.keep_logits:
+                self.last_logits.append(logits.detach())
             input_ids = torch.cat(
                 [original_ids[:, 1 + step:], original_ids.new_zeros(1, 1 + step)], dim=-1)
             if full_mask is not None:

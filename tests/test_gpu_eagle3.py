@@ -179,6 +179,66 @@ def test_fp32_master_weights_under_autocast_match_oracle(variant):
     assert vloss2.item() < vloss.item()
 
 
+@pytest.mark.parametrize("regime", ["bf16", "autocast"])
+def test_configs0_in_full_matches_oracle(regime):
+    """The reference's own CPU-runnable case at its real size: Llama-3.2-1B shape (hidden 2048,
+    32 q / 8 kv heads, head_dim 64, FFN 8192), target vocabulary 128 256 -> draft 32 000 through
+    a sorted random d2t subset, seq 512, 3 TTT steps, verifier logits ~ N(0, 2^2) over the target
+    vocabulary, hidden states ~ N(0, 1), loss_mask Bernoulli(0.7), seeded.  Whole model on the
+    HIP path against the fp32 oracle: loss 1e-3, per-step logits and every gradient 2e-2 relative
+    max-norm, mask / row counts exact, the gathered targets bit-exact."""
+    from oracle import vocab as OV
+    from speculators_amd import losses as L
+
+    shape = OE.DraftShape(hidden_size=2048, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+                          intermediate_size=8192, vocab_size=128256, draft_vocab_size=32000,
+                          rms_norm_eps=1e-5, rope_theta=500000.0)
+    t, steps = 512, 3
+    g = torch.Generator().manual_seed(0)
+    w32 = {k_: v.bfloat16().float() for k_, v in OE.random_weights(shape, seed=0).items()}
+    hs = torch.randn(1, t, 3 * shape.hidden_size, generator=g).bfloat16()
+    ids = torch.randint(0, shape.vocab_size, (1, t), generator=g)
+    vlogits = (torch.randn(1, t, shape.vocab_size, generator=g) * 2).bfloat16()
+    mask = (torch.rand(1, t, generator=g) < 0.7).float()
+    doc = torch.zeros(1, t, dtype=torch.long)
+    sel = torch.randperm(shape.vocab_size, generator=g)[: shape.draft_vocab_size]
+    d2t, t2d = OV.build_vocab_mappings(sel.tolist(), shape.vocab_size)
+
+    auto = regime == "autocast"
+    model = _make(shape, w32, param_dtype=torch.float32 if auto else torch.bfloat16)
+    model.load_vocab_mappings(t2d, d2t)
+    model.keep_logits = True
+    # index mapping: bit-exact against the oracle's gather
+    got_targets = L.vocab_gather(vlogits.cuda(), model.d2t)
+    assert torch.equal(got_targets.cpu(), OV.gather_targets(vlogits, d2t))
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=auto):
+        toks, loss, m = model(hs.cuda(), ids.cuda(), doc.cuda(), mask.cuda(), None,
+                              verifier_logits=vlogits.cuda(), ttt_steps=steps)
+    loss.backward()
+
+    wf = {k_: v.clone().requires_grad_(True) for k_, v in w32.items()}
+    rt, rloss, rm, rlogits = OE.eagle3_forward(wf, shape, hs.float(), ids, doc, mask, None,
+                                               ttt_steps=steps, verifier_logits=vlogits.float(), d2t=d2t,
+                                               return_logits=True, attn="sdpa")
+    rloss.backward()
+    rel = abs(loss.item() - rloss.item()) / abs(rloss.item())
+    print(regime, "loss", loss.item(), rloss.item(), rel)
+    assert rel < 1e-3
+    assert set(m) == set(rm)
+    for key in rm:
+        if key.endswith("_total"):
+            assert m[key].item() == rm[key].item(), key
+    for k_ in range(steps):
+        got, want = model.last_logits[k_].float().cpu(), rlogits[k_].detach()
+        assert (got - want).abs().max() <= 2e-2 * want.abs().max(), k_
+    for name, p in model.named_parameters():
+        if not p.requires_grad:
+            continue
+        want = wf[name].grad
+        err = (p.grad.float().cpu() - want).abs().max().item()
+        assert err <= 2e-2 * want.abs().max().item() + 1e-7, (name, err, want.abs().max().item())
+
+
 def test_verifier_logits_entry_point_equals_row_sliced_head():
     """targets from a d2t gather of full-vocab verifier logits == the row-sliced verifier head."""
     from oracle import vocab as OV

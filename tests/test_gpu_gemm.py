@@ -51,22 +51,23 @@ def test_linear_autograd_matches_fp32():
             assert err <= 2e-2 * want.abs().max().item()
 
 
-def test_full_size_lm_head_shape_sampled_and_linear():
-    """The lm_head shape (4096 x 4096 x 32000): sampled output rows against an fp32 product of
-    the same bf16 operands, and linearity in the first operand (bf16 rounding of each result
-    aside)."""
+@pytest.mark.parametrize("m,k", [(4096, 4096), (8192, 8192)])
+def test_full_size_lm_head_shape_sampled_and_linear(m, k):
+    """The lm_head shapes of the 8B draft (4096 x 4096 x 32000) and of the 70B draft
+    (8192 x 8192 x 32000): sampled output rows against an fp32 product of the same bf16 operands,
+    and linearity in the first operand (bf16 rounding of each result aside)."""
     from speculators_amd.gemm import gemm_nt
 
     g = torch.Generator(device="cuda").manual_seed(3)
-    a = torch.randn(4096, 4096, device="cuda", generator=g).bfloat16()
-    a2 = torch.randn(4096, 4096, device="cuda", generator=g).bfloat16()
-    b = (torch.randn(32000, 4096, device="cuda", generator=g) * 0.02).bfloat16()
+    a = torch.randn(m, k, device="cuda", generator=g).bfloat16()
+    a2 = torch.randn(m, k, device="cuda", generator=g).bfloat16()
+    b = (torch.randn(32000, k, device="cuda", generator=g) * 0.02).bfloat16()
     c = gemm_nt(a, b)
-    rows = torch.randint(0, 4096, (64,), device="cuda", generator=g)
+    rows = torch.randint(0, m, (64,), device="cuda", generator=g)
     want = a[rows].float() @ b.float().t()
     assert (c[rows].float() - want).abs().max() <= 2 ** -8 * want.abs().max() + 1e-3
     # every tile edge of the 256 x 256 tiling is exercised: first / last rows and columns
-    edge = torch.tensor([0, 255, 256, 4095], device="cuda")
+    edge = torch.tensor([0, 255, 256, m - 1], device="cuda")
     want_e = a[edge].float() @ b.float().t()
     assert (c[edge].float() - want_e).abs().max() <= 2 ** -8 * want_e.abs().max() + 1e-3
     s = (a.float() + a2.float()).bfloat16()  # exact sums are not representable: compare against fp32
