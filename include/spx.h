@@ -80,6 +80,36 @@ int spx_fused_vocab_loss_fwd(int op, const void* logits, int64_t ld_logits,
                              int32_t* argmax_target, int reuse_target_stats,
                              void* stream);
 
+/* The whole per-row work of one TTT step in ONE streaming pass: spx_fused_vocab_loss_fwd plus
+ *   - d2t != NULL: `targets` holds FULL-vocabulary verifier rows (vt columns, row stride
+ *     ld_targets) and target element i is read at column i + d2t[i] -- the d2t / t2d mapping
+ *     of model.py:161-169 and train/vocab_mapping.py:86-96 applied while streaming, no
+ *     [rows, vocab] copy of the targets is needed first.  `gathered` (may be NULL) receives
+ *     that draft-vocabulary row (bit-exact copy), for the later TTT steps and the backward,
+ *     which then stream vocab-wide rows.  Columns outside [0, vt) read as -inf.
+ *     reuse_target_stats must be 0 in this form.
+ *   - counts != NULL (int32[3], zeroed by the caller): the row's part of the acceptance chain
+ *     of compute_accuracy_single_step (models/metrics.py:6-36) as called from compute_metrics
+ *     (models/eagle3/metrics.py:100-117).  With m = mask[r] != 0 (NULL: 1), was =
+ *     prev_correct[r] != 0 (NULL: 1), now = was && argmax_draft[r] == argmax_target[r]:
+ *       counts[0] += m && now   (full_correct = cond_correct)
+ *       counts[1] += m          (full_total)
+ *       counts[2] += was        (cond_total, counted before the update)
+ *       prev_correct[r] = now   (in place, in prev_correct's own element type)
+ *     Integer atomics: the result does not depend on the order in which rows finish.
+ *     Needs both arg-max outputs.  spx_ttt_step_mean turns the counts and the row losses
+ *     into the step's scalars.
+ * Replaces, together, the t2d row slice (model.py:161-169), loss_forward_kernel
+ * (losses/fused.py:91-175), both torch.argmax calls and compute_accuracy_single_step. */
+int spx_vocab_loss_step_fwd(int op, const void* logits, int64_t ld_logits,
+                            const void* targets, int64_t ld_targets, const int64_t* d2t,
+                            int64_t vt, void* gathered, int64_t ld_gathered, int64_t rows,
+                            int64_t vocab, int dtype, float* loss, float* lse_draft,
+                            float* lse_target, float* extra, int32_t* argmax_draft,
+                            int32_t* argmax_target, int reuse_target_stats,
+                            const void* mask, int mask_kind, void* prev_correct,
+                            int prev_kind, int32_t* counts, void* stream);
+
 /* grad_logits[r, :] = g_r * dL_r/dlogits, g_r = row_grad[r] * (*scale)
  * (scale may be NULL = 1).  Rows with g_r == 0 are written as exact zeros
  * without reading the inputs.  Closed forms of losses/fused.py:11-18; replaces
@@ -185,6 +215,13 @@ int spx_ttt_step_reduce(const float* loss, const int32_t* argmax_draft,
                         int mask_kind, void* prev_correct, int prev_kind,
                         int64_t rows, float weight, float* out,
                         float* row_weight, void* stream);
+
+/* spx_ttt_step_reduce for a step whose acceptance chain was already done row by row by
+ * spx_vocab_loss_step_fwd: the masked mean and row_weight as there, out[1] = out[3] =
+ * counts[0], out[2] = counts[1], out[4] = counts[2], out[5] = sum of the mask. */
+int spx_ttt_step_mean(const float* loss, const void* mask, int mask_kind, int64_t rows,
+                      float weight, const int32_t* counts, float* out, float* row_weight,
+                      void* stream);
 
 /* Weighted masked mean and per-slot acceptance counts of a DFlash block batch:
  *   out[0] = sum_r loss[r] m_r w_r / (sum m + 1e-5),  out[1] = sum m

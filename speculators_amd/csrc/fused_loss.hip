@@ -62,19 +62,73 @@ __device__ __forceinline__ float log_mix(float la, float lb) {
   return mx + fast_log2(s) * kLn2 - kLn2;
 }
 
+// ---- mask element access ---------------------------------------------------
+__device__ __forceinline__ float mask_value(const void* p, int kind, int64_t i) {
+  switch (kind) {
+    case SPX_KIND_U8: return (float)reinterpret_cast<const uint8_t*>(p)[i];
+    case SPX_KIND_I32: return (float)reinterpret_cast<const int32_t*>(p)[i];
+    case SPX_KIND_I64: return (float)reinterpret_cast<const int64_t*>(p)[i];
+    case SPX_KIND_F32: return reinterpret_cast<const float*>(p)[i];
+    default: return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+  }
+}
+__device__ __forceinline__ void store_flag(void* p, int kind, int64_t i, bool v) {
+  switch (kind) {
+    case SPX_KIND_U8: reinterpret_cast<uint8_t*>(p)[i] = v ? 1 : 0; break;
+    case SPX_KIND_I32: reinterpret_cast<int32_t*>(p)[i] = v ? 1 : 0; break;
+    case SPX_KIND_I64: reinterpret_cast<int64_t*>(p)[i] = v ? 1 : 0; break;
+    case SPX_KIND_F32: reinterpret_cast<float*>(p)[i] = v ? 1.f : 0.f; break;
+    default: reinterpret_cast<uint16_t*>(p)[i] = v ? 0x3f80 : 0; break;
+  }
+}
+
+// ---- what one TTT step adds to the row pass --------------------------------------
+// d2t != nullptr: `targets` are full-vocabulary rows (vt wide) and target element i is read at
+// i + d2t[i] (model.py:161-169, train/vocab_mapping.py:86-96); `gathered` (may be nullptr) then
+// receives the draft-vocabulary row, for the later steps and the backward.
+// counts != nullptr: the row's part of the acceptance chain (models/metrics.py:6-36): with
+// m = mask[r] != 0, was = prev[r] != 0, hit = argmax_draft == argmax_target, now = was && hit:
+//   counts[0] += m && now,  counts[1] += m,  counts[2] += was,  prev[r] = now.
+// Integer atomics: the sums do not depend on the order of the rows.
+struct StepArgs {
+  const int64_t* d2t; int64_t vt;
+  void* gathered; int64_t ld_gathered;
+  const void* mask; int mask_kind;
+  void* prev; int prev_kind;
+  int32_t* counts;
+};
+
+// eight target elements through the offset table (ascending indices: neighbouring lanes read
+// neighbouring sectors of the full row)
+template <typename T>
+__device__ __forceinline__ void load8_gather(const T* full, const int64_t* __restrict__ d2t, int64_t base,
+                                             int64_t n, int64_t vt, float v[8]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float val = kNegBig;  // tail padding, like load8_guard
+    if (base + i < n) {
+      const int64_t j = base + i + d2t[base + i];
+      val = (j >= 0 && j < vt) ? load1(full + j) : -INFINITY;
+    }
+    v[i] = val;
+  }
+}
+
 // ---- forward ---------------------------------------------------------------
 // KNOWN: lse_target / argmax_target are INPUTS (the target row's statistics from an
 // earlier pass over the same row); the target max / sum / arg-max tracking is skipped and
 // the cross-entropy reduction does not read the target row at all.
-template <typename T, int OP, bool VEC, bool KNOWN>
+// GATHER: the target row is read through the d2t offset table (see StepArgs).
+template <typename T, int OP, bool VEC, bool KNOWN, bool GATHER>
 __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
     const T* __restrict__ logits, int64_t ld_logits, const T* __restrict__ targets,
     int64_t ld_targets, int64_t vocab, float* __restrict__ loss, float* __restrict__ lse_draft,
     float* __restrict__ lse_target, float* __restrict__ extra, int32_t* __restrict__ argmax_draft,
-    int32_t* __restrict__ argmax_target) {
+    int32_t* __restrict__ argmax_target, StepArgs sa) {
   const int64_t r = blockIdx.x;
   const T* xrow = logits + r * ld_logits;
   const T* yrow = targets + r * ld_targets;
+  T* grow = (GATHER && sa.gathered) ? reinterpret_cast<T*>(sa.gathered) + r * sa.ld_gathered : nullptr;
   const int tid = threadIdx.x;
   const int64_t nchunks = (vocab + 7) >> 3;
 
@@ -88,7 +142,12 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
     const int64_t base = c << 3;
     float x[8], y[8];
     load8<T, VEC>(xrow, base, vocab, x);
-    if (read_y) load8<T, VEC>(yrow, base, vocab, y);
+    if (GATHER) {
+      load8_gather<T>(yrow, sa.d2t, base, vocab, sa.vt, y);
+      if (grow) store8<T, VEC>(grow, base, vocab, y);
+    } else if (read_y) {
+      load8<T, VEC>(yrow, base, vocab, y);
+    }
     float cx = x[0], cy = y[0];
 #pragma unroll
     for (int i = 1; i < 8; ++i) cx = fmaxf(cx, x[i]);
@@ -181,7 +240,8 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
       const int64_t base = c << 3;
       float x[8], y[8];
       load8<T, VEC>(xrow, base, vocab, x);
-      load8<T, VEC>(yrow, base, vocab, y);
+      if (GATHER) load8_gather<T>(yrow, sa.d2t, base, vocab, sa.vt, y);
+      else load8<T, VEC>(yrow, base, vocab, y);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         float ldp = x[i] - lse_d, ltp = y[i] - lse_t;
@@ -212,6 +272,15 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
     if (!KNOWN) {
       lse_target[r] = lse_t;
       if (argmax_target) argmax_target[r] = s.it;
+    }
+    if (sa.counts) {
+      const bool m = sa.mask ? mask_value(sa.mask, sa.mask_kind, r) != 0.f : true;
+      const bool was = sa.prev ? mask_value(sa.prev, sa.prev_kind, r) != 0.f : true;
+      const bool now = was && (s.id == s.it);
+      if (m && now) atomicAdd(&sa.counts[0], 1);
+      if (m) atomicAdd(&sa.counts[1], 1);
+      if (was) atomicAdd(&sa.counts[2], 1);
+      if (sa.prev) store_flag(sa.prev, sa.prev_kind, r, now);
     }
   }
 }
@@ -311,26 +380,6 @@ __global__ __launch_bounds__(256) void vocab_gather_kernel(
   }
 }
 
-// ---- mask element access ---------------------------------------------------
-__device__ __forceinline__ float mask_value(const void* p, int kind, int64_t i) {
-  switch (kind) {
-    case SPX_KIND_U8: return (float)reinterpret_cast<const uint8_t*>(p)[i];
-    case SPX_KIND_I32: return (float)reinterpret_cast<const int32_t*>(p)[i];
-    case SPX_KIND_I64: return (float)reinterpret_cast<const int64_t*>(p)[i];
-    case SPX_KIND_F32: return reinterpret_cast<const float*>(p)[i];
-    default: return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
-  }
-}
-__device__ __forceinline__ void store_flag(void* p, int kind, int64_t i, bool v) {
-  switch (kind) {
-    case SPX_KIND_U8: reinterpret_cast<uint8_t*>(p)[i] = v ? 1 : 0; break;
-    case SPX_KIND_I32: reinterpret_cast<int32_t*>(p)[i] = v ? 1 : 0; break;
-    case SPX_KIND_I64: reinterpret_cast<int64_t*>(p)[i] = v ? 1 : 0; break;
-    case SPX_KIND_F32: reinterpret_cast<float*>(p)[i] = v ? 1.f : 0.f; break;
-    default: reinterpret_cast<uint16_t*>(p)[i] = v ? 0x3f80 : 0; break;
-  }
-}
-
 constexpr int kReduceThreads = 1024;
 
 __device__ __forceinline__ float block_sum_f(float v, float* lds) {
@@ -357,34 +406,42 @@ __global__ __launch_bounds__(kReduceThreads) void ttt_step_reduce_kernel(
     const float* __restrict__ loss, const int32_t* __restrict__ pred,
     const int32_t* __restrict__ tgt, const void* __restrict__ mask, int mask_kind,
     void* prev, int prev_kind, int64_t rows, float weight, float* __restrict__ out,
-    float* __restrict__ row_weight) {
+    float* __restrict__ row_weight, const int32_t* __restrict__ counts) {
   __shared__ float fl[kReduceThreads / 64];
   __shared__ int il[kReduceThreads / 64];
   float lsum = 0.f, msum = 0.f;
   int full_total = 0, correct = 0, cond_total = 0;
+  // counts != nullptr: the acceptance chain was done row by row in the loss pass (StepArgs);
+  // only the masked mean is left here and the counts are copied out
   for (int64_t r = threadIdx.x; r < rows; r += kReduceThreads) {
     float m = mask ? mask_value(mask, mask_kind, r) : 1.f;
-    bool was = prev ? (mask_value(prev, prev_kind, r) != 0.f) : true;
-    bool hit = pred[r] == tgt[r];
-    bool now = was && hit;
-    cond_total += was ? 1 : 0;
-    if (prev) store_flag(prev, prev_kind, r, now);
-    if (m != 0.f) { full_total += 1; correct += now ? 1 : 0; }
+    if (!counts) {
+      bool was = prev ? (mask_value(prev, prev_kind, r) != 0.f) : true;
+      bool hit = pred[r] == tgt[r];
+      bool now = was && hit;
+      cond_total += was ? 1 : 0;
+      if (prev) store_flag(prev, prev_kind, r, now);
+      if (m != 0.f) { full_total += 1; correct += now ? 1 : 0; }
+    }
     lsum = fmaf(loss[r], m, lsum);
     msum += m;
   }
   lsum = block_sum_f(lsum, fl);
   msum = block_sum_f(msum, fl);
-  full_total = block_sum_i(full_total, il);
-  correct = block_sum_i(correct, il);
-  cond_total = block_sum_i(cond_total, il);
+  if (!counts) {
+    full_total = block_sum_i(full_total, il);
+    correct = block_sum_i(correct, il);
+    cond_total = block_sum_i(cond_total, il);
+  } else {
+    correct = counts[0]; full_total = counts[1]; cond_total = counts[2];
+  }
   const float inv = weight / (msum + 1e-5f);
   if (threadIdx.x == 0) {
     out[0] = lsum * inv;
     out[1] = (float)correct;
     out[2] = (float)full_total;
     out[3] = (float)correct;
-    out[4] = prev ? (float)cond_total : (float)rows;
+    out[4] = (prev || counts) ? (float)cond_total : (float)rows;
     out[5] = msum;
   }
   if (row_weight) {
@@ -437,15 +494,15 @@ __global__ __launch_bounds__(kReduceThreads) void block_reduce_kernel(
 // ---- dispatch ----------------------------------------------------------------
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-template <typename T, bool VEC, bool KNOWN>
+template <typename T, bool VEC, bool KNOWN, bool GATHER>
 static void launch_fwd(int op, const T* lg, int64_t ldl, const T* tg, int64_t ldt, int64_t rows,
                        int64_t vocab, float* loss, float* lsd, float* lst, float* ex, int32_t* ad,
-                       int32_t* at, hipStream_t st) {
+                       int32_t* at, const StepArgs& sa, hipStream_t st) {
   dim3 grid((unsigned)rows), block(kLossThreads);
-#define SPX_FWD(OPV)                                                                                \
-  case OPV:                                                                                         \
-    hipLaunchKernelGGL((loss_fwd_kernel<T, OPV, VEC, KNOWN>), grid, block, 0, st, lg, ldl, tg, ldt, \
-                       vocab, loss, lsd, lst, ex, ad, at);                                          \
+#define SPX_FWD(OPV)                                                                                 \
+  case OPV:                                                                                          \
+    hipLaunchKernelGGL((loss_fwd_kernel<T, OPV, VEC, KNOWN, GATHER>), grid, block, 0, st, lg, ldl,   \
+                       tg, ldt, vocab, loss, lsd, lst, ex, ad, at, sa);                              \
     break;
   switch (op) {
     SPX_FWD(SPX_LOSS_KL) SPX_FWD(SPX_LOSS_RKL) SPX_FWD(SPX_LOSS_JSD) SPX_FWD(SPX_LOSS_CE)
@@ -476,42 +533,83 @@ static void launch_bwd(int op, const T* lg, int64_t ldl, const T* tg, int64_t ld
 
 using namespace spx;
 
+static bool kind_ok(int k) { return k >= SPX_KIND_U8 && k <= SPX_KIND_BF16; }
+
+#define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fname, what); } while (0)
+static int loss_fwd_impl(const char* fname, int op, const void* logits, int64_t ld_logits,
+                         const void* targets, int64_t ld_targets, int64_t rows, int64_t vocab,
+                         int dtype, float* loss, float* lse_draft, float* lse_target, float* extra,
+                         int32_t* argmax_draft, int32_t* argmax_target, int reuse_target_stats,
+                         const StepArgs& sa, void* stream) {
+  SPX_REQ_FN(op >= SPX_LOSS_KL && op <= SPX_LOSS_TV, "unknown loss op");
+  SPX_REQ_FN(dtype == SPX_DTYPE_BF16 || dtype == SPX_DTYPE_F32, "dtype must be bf16 or f32");
+  SPX_REQ_FN(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "rows >= 0 and 0 < vocab < 2^31");
+  const bool gather = sa.d2t != nullptr;
+  SPX_REQ_FN(ld_logits >= vocab && ld_targets >= (gather ? sa.vt : vocab), "row stride smaller than vocab");
+  SPX_REQ_FN(rows < (1ll << 31), "too many rows");
+  if (gather) {
+    SPX_REQ_FN(sa.vt > 0 && sa.vt < (1ll << 31), "0 < vt < 2^31");
+    SPX_REQ_FN(!reuse_target_stats, "the gather form computes the target statistics itself");
+    SPX_REQ_FN(!sa.gathered || sa.ld_gathered >= vocab, "gathered row stride smaller than vocab");
+  }
+  if (sa.counts) {
+    SPX_REQ_FN(argmax_draft && argmax_target, "the acceptance chain needs both arg-max outputs");
+    SPX_REQ_FN(!sa.mask || kind_ok(sa.mask_kind), "unknown mask element kind");
+    SPX_REQ_FN(!sa.prev || kind_ok(sa.prev_kind), "unknown prev_correct element kind");
+  }
+  if (rows == 0) return SPX_OK;
+  SPX_REQ_FN(logits && targets && loss && lse_draft && lse_target && extra, "null buffer");
+  // the second-pass reductions (rkl, jsd, tv) recompute from both rows anyway
+  const bool known = reuse_target_stats && (op == SPX_LOSS_KL || op == SPX_LOSS_CE);
+  if (known && op == SPX_LOSS_CE) SPX_REQ_FN(argmax_target, "ce with reused statistics needs argmax_target");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int64_t per16 = dtype == SPX_DTYPE_BF16 ? 8 : 4;
+  const bool vec = aligned16(logits) && ld_logits % per16 == 0 &&
+                   (gather ? (!sa.gathered || (aligned16(sa.gathered) && sa.ld_gathered % per16 == 0))
+                           : (aligned16(targets) && ld_targets % per16 == 0));
+#define SPX_GO(TT, VV, KK, GG)                                                                    \
+  launch_fwd<TT, VV, KK, GG>(op, reinterpret_cast<const TT*>(logits), ld_logits,                  \
+                             reinterpret_cast<const TT*>(targets), ld_targets, rows, vocab, loss, \
+                             lse_draft, lse_target, extra, argmax_draft, argmax_target, sa, st)
+#define SPX_GO_T(TT)                                                                   \
+  do {                                                                                 \
+    if (gather) { if (vec) SPX_GO(TT, true, false, true); else SPX_GO(TT, false, false, true); } \
+    else if (vec) { if (known) SPX_GO(TT, true, true, false); else SPX_GO(TT, true, false, false); } \
+    else { if (known) SPX_GO(TT, false, true, false); else SPX_GO(TT, false, false, false); } \
+  } while (0)
+  if (dtype == SPX_DTYPE_BF16) SPX_GO_T(uint16_t);
+  else SPX_GO_T(float);
+#undef SPX_GO_T
+#undef SPX_GO
+  return check_launch(fname);
+}
+
 extern "C" int spx_fused_vocab_loss_fwd(int op, const void* logits, int64_t ld_logits,
                                         const void* targets, int64_t ld_targets, int64_t rows,
                                         int64_t vocab, int dtype, float* loss, float* lse_draft,
                                         float* lse_target, float* extra, int32_t* argmax_draft,
                                         int32_t* argmax_target, int reuse_target_stats,
                                         void* stream) {
-  SPX_REQUIRE(op >= SPX_LOSS_KL && op <= SPX_LOSS_TV, "unknown loss op");
-  SPX_REQUIRE(dtype == SPX_DTYPE_BF16 || dtype == SPX_DTYPE_F32, "dtype must be bf16 or f32");
-  SPX_REQUIRE(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "rows >= 0 and 0 < vocab < 2^31");
-  SPX_REQUIRE(ld_logits >= vocab && ld_targets >= vocab, "row stride smaller than vocab");
-  SPX_REQUIRE(rows < (1ll << 31), "too many rows");
-  if (rows == 0) return SPX_OK;
-  SPX_REQUIRE(logits && targets && loss && lse_draft && lse_target && extra, "null buffer");
-  // the second-pass reductions (rkl, jsd, tv) recompute from both rows anyway
-  const bool known = reuse_target_stats && (op == SPX_LOSS_KL || op == SPX_LOSS_CE);
-  if (known && op == SPX_LOSS_CE) SPX_REQUIRE(argmax_target, "ce with reused statistics needs argmax_target");
-  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  const int64_t per16 = dtype == SPX_DTYPE_BF16 ? 8 : 4;
-  const bool vec = aligned16(logits) && aligned16(targets) && ld_logits % per16 == 0 &&
-                   ld_targets % per16 == 0;
-#define SPX_GO(TT, VV, KK)                                                                       \
-  launch_fwd<TT, VV, KK>(op, reinterpret_cast<const TT*>(logits), ld_logits,                     \
-                         reinterpret_cast<const TT*>(targets), ld_targets, rows, vocab, loss,    \
-                         lse_draft, lse_target, extra, argmax_draft, argmax_target, st)
-  if (dtype == SPX_DTYPE_BF16) {
-    if (vec) { if (known) SPX_GO(uint16_t, true, true); else SPX_GO(uint16_t, true, false); }
-    else { if (known) SPX_GO(uint16_t, false, true); else SPX_GO(uint16_t, false, false); }
-  } else {
-    if (vec) { if (known) SPX_GO(float, true, true); else SPX_GO(float, true, false); }
-    else { if (known) SPX_GO(float, false, true); else SPX_GO(float, false, false); }
-  }
-#undef SPX_GO
-  return check_launch(__func__);
+  const StepArgs none = {nullptr, 0, nullptr, 0, nullptr, 0, nullptr, 0, nullptr};
+  return loss_fwd_impl(__func__, op, logits, ld_logits, targets, ld_targets, rows, vocab, dtype, loss,
+                       lse_draft, lse_target, extra, argmax_draft, argmax_target, reuse_target_stats,
+                       none, stream);
 }
 
-#define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fname, what); } while (0)
+extern "C" int spx_vocab_loss_step_fwd(int op, const void* logits, int64_t ld_logits,
+                                       const void* targets, int64_t ld_targets, const int64_t* d2t,
+                                       int64_t vt, void* gathered, int64_t ld_gathered, int64_t rows,
+                                       int64_t vocab, int dtype, float* loss, float* lse_draft,
+                                       float* lse_target, float* extra, int32_t* argmax_draft,
+                                       int32_t* argmax_target, int reuse_target_stats,
+                                       const void* mask, int mask_kind, void* prev_correct,
+                                       int prev_kind, int32_t* counts, void* stream) {
+  const StepArgs sa = {d2t, vt, gathered, ld_gathered, mask, mask_kind, prev_correct, prev_kind, counts};
+  return loss_fwd_impl(__func__, op, logits, ld_logits, targets, ld_targets, rows, vocab, dtype, loss,
+                       lse_draft, lse_target, extra, argmax_draft, argmax_target, reuse_target_stats,
+                       sa, stream);
+}
+
 static int loss_bwd_impl(const char* fname, int op, const void* logits, int64_t ld_logits,
                          const void* targets, int64_t ld_targets, int64_t rows,
                          int64_t vocab, int dtype, const float* lse_draft,
@@ -596,8 +694,6 @@ extern "C" int spx_vocab_gather(const void* full, int64_t ld_full, const int64_t
   return check_launch(__func__);
 }
 
-static bool kind_ok(int k) { return k >= SPX_KIND_U8 && k <= SPX_KIND_BF16; }
-
 extern "C" int spx_ttt_step_reduce(const float* loss, const int32_t* argmax_draft,
                                    const int32_t* argmax_target, const void* mask, int mask_kind,
                                    void* prev_correct, int prev_kind, int64_t rows, float weight,
@@ -608,7 +704,19 @@ extern "C" int spx_ttt_step_reduce(const float* loss, const int32_t* argmax_draf
   SPX_REQUIRE(!prev_correct || kind_ok(prev_kind), "unknown prev_correct element kind");
   hipLaunchKernelGGL(ttt_step_reduce_kernel, dim3(1), dim3(kReduceThreads), 0,
                      reinterpret_cast<hipStream_t>(stream), loss, argmax_draft, argmax_target, mask,
-                     mask_kind, prev_correct, prev_kind, rows, weight, out, row_weight);
+                     mask_kind, prev_correct, prev_kind, rows, weight, out, row_weight, nullptr);
+  return check_launch(__func__);
+}
+
+extern "C" int spx_ttt_step_mean(const float* loss, const void* mask, int mask_kind, int64_t rows,
+                                 float weight, const int32_t* counts, float* out, float* row_weight,
+                                 void* stream) {
+  SPX_REQUIRE(rows >= 0 && rows < (1ll << 24), "0 <= rows < 2^24");
+  SPX_REQUIRE(loss && counts && out, "null buffer");
+  SPX_REQUIRE(!mask || kind_ok(mask_kind), "unknown mask element kind");
+  hipLaunchKernelGGL(ttt_step_reduce_kernel, dim3(1), dim3(kReduceThreads), 0,
+                     reinterpret_cast<hipStream_t>(stream), loss, nullptr, nullptr, mask, mask_kind,
+                     nullptr, 0, rows, weight, out, row_weight, counts);
   return check_launch(__func__);
 }
 

@@ -317,8 +317,9 @@ class Eagle3DraftModel(nn.Module):
         if return_loss:
             with torch.no_grad():
                 if verifier_logits is not None:
-                    targets = (L.vocab_gather(verifier_logits, self.d2t) if self.use_draft_vocab
-                               else verifier_logits)
+                    # gathered through d2t inside the first step's loss pass (metrics.TargetGather)
+                    targets = (MT.TargetGather(compute_input(verifier_logits), self.d2t)
+                               if self.use_draft_vocab else compute_input(verifier_logits))
                 else:
                     targets = self._linear(self.verifier_norm(verifier_last_hidden_states),
                                            self.verifier_lm_head.weight)

@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import json
 from collections.abc import Callable
+from dataclasses import dataclass
 
 import torch
 
@@ -36,20 +37,67 @@ def _rows_2d(t: torch.Tensor) -> torch.Tensor:
         return t.reshape(-1, v)
 
 
-def fused_loss_forward(op: int, logits: torch.Tensor, targets: torch.Tensor, target_stats=None):
+@dataclass
+class StepPass:
+    """What one TTT step adds to the row pass of the loss kernel (``spx_vocab_loss_step_fwd``).
+
+    ``d2t`` (int64 ``[Vd]``): the targets are FULL-vocabulary verifier rows and target element i
+    is read at column ``i + d2t[i]`` while streaming; the draft-vocabulary rows come back in
+    ``gathered`` (``[rows, Vd]``) for the later steps and the backward.
+    ``counts`` (int32 ``[3]``, zeroed): the acceptance chain is done row by row in the same pass
+    (``mask`` / ``prev`` are the step's 1-D views, ``prev`` is updated in place)."""
+
+    d2t: torch.Tensor | None = None
+    gathered: torch.Tensor | None = None
+    mask: torch.Tensor | None = None
+    prev: torch.Tensor | None = None
+    counts: torch.Tensor | None = None
+
+
+def fused_loss_forward(op: int, logits: torch.Tensor, targets: torch.Tensor, target_stats=None,
+                       step: StepPass | None = None):
     """Run the forward kernel.  Returns (loss [R] f32, lse_d, lse_t, extra,
     argmax_draft [R] i32, argmax_target [R] i32, logits2d, targets2d).
 
     ``target_stats = (lse_target [R] f32, argmax_target [R] i32)`` from an earlier call on
     the same target rows lets kl / ce skip the target row statistics (ce then does not
-    read the targets at all)."""
-    if logits.shape != targets.shape:
+    read the targets at all).  ``step``: see ``StepPass``; with ``step.d2t`` the returned
+    ``targets2d`` are the gathered draft-vocabulary rows."""
+    gather = step is not None and step.d2t is not None
+    if not gather and logits.shape != targets.shape:
         raise ValueError(f"logits {tuple(logits.shape)} and targets {tuple(targets.shape)} differ")
+    if gather and logits.shape[:-1] != targets.shape[:-1]:
+        raise ValueError(f"logits {tuple(logits.shape)} and full-vocabulary targets "
+                         f"{tuple(targets.shape)} differ in their rows")
     if logits.dtype != targets.dtype:
         targets = targets.to(logits.dtype)
     x, y = _rows_2d(logits), _rows_2d(targets)
     rows, vocab = x.shape
     dev = x.device
+    if step is not None:
+        if gather:
+            if target_stats is not None:
+                raise ValueError("the gather form computes the target statistics itself")
+            if step.d2t.dtype != torch.int64 or step.d2t.numel() != vocab or not step.d2t.is_contiguous():
+                raise ValueError("d2t must be a contiguous int64 [draft vocabulary] tensor")
+            step.gathered = torch.empty(rows, vocab, device=dev, dtype=x.dtype)
+        stats = torch.empty(4, rows, device=dev, dtype=torch.float32)
+        arg = torch.empty(2, rows, device=dev, dtype=torch.int32)
+        reuse = target_stats is not None and op in (OP_KL, OP_CE)
+        lse_t, am_t = stats[2], arg[1]
+        if reuse:
+            lse_t, am_t = target_stats[0].reshape(-1), target_stats[1].reshape(-1)
+        g = step.gathered
+        _lib.call(
+            "spx_vocab_loss_step_fwd", op, _lib.ptr(x), x.stride(0), _lib.ptr(y), y.stride(0),
+            _lib.ptr(step.d2t), y.shape[1] if gather else 0, _lib.ptr(g) if gather else None,
+            g.stride(0) if gather else 0, rows, vocab, _lib.dtype_code(x), _lib.ptr(stats[0]),
+            _lib.ptr(stats[1]), _lib.ptr(lse_t), _lib.ptr(stats[3]), _lib.ptr(arg[0]), _lib.ptr(am_t),
+            int(reuse), _lib.ptr(step.mask), _lib.kind_code(step.mask) if step.mask is not None else 0,
+            _lib.ptr(step.prev), _lib.kind_code(step.prev) if step.prev is not None else 0,
+            _lib.ptr(step.counts), _lib.stream_ptr(dev),
+        )
+        return stats[0], stats[1], lse_t, stats[3], arg[0], am_t, x, (g if gather else y)
     reuse = target_stats is not None and op in (OP_KL, OP_CE)
     stats = torch.empty(4, rows, device=dev, dtype=torch.float32)
     arg = torch.empty(2, rows, device=dev, dtype=torch.int32)
@@ -74,14 +122,14 @@ class _FusedLoss(torch.autograd.Function):
     losses/fused.py:238-291.  Targets get no gradient."""
 
     @staticmethod
-    def forward(ctx, logits, targets, op, known_lse_t=None, known_am_t=None, n_rows=None):
+    def forward(ctx, logits, targets, op, known_lse_t=None, known_am_t=None, n_rows=None, step=None):
         known = (known_lse_t, known_am_t) if known_lse_t is not None else None
         # n_rows: only the first n_rows rows of ``logits`` (a [1, T, V] tensor) take part, the
         # rest get a zero gradient.  Doing the cut here instead of slicing outside keeps
         # autograd from materialising a zero-padded copy of the whole gradient.
         ctx.full_shape = logits.shape
         used = logits if n_rows is None else logits[:, :n_rows]
-        loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, used, targets, known)
+        loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, used, targets, known, step)
         ctx.save_for_backward(x, None if op == OP_CE else y, lse_d, lse_t, extra, am_t)
         ctx.op = op
         lead = used.shape[:-1]
@@ -106,7 +154,7 @@ class _FusedLoss(torch.autograd.Function):
         )
         if full_rows > rows:
             grad[rows:].zero_()
-        return grad.view(ctx.full_shape), None, None, None, None, None
+        return grad.view(ctx.full_shape), None, None, None, None, None, None
 
 
 def _packed_row_map(row_grad: torch.Tensor, labels: torch.Tensor | None = None, ignore_index: int = -100):
@@ -142,12 +190,13 @@ class _HeadFusedLoss(torch.autograd.Function):
     metrics and the draft tokens and carry no gradient of their own."""
 
     @staticmethod
-    def forward(ctx, x2, weight, weight_t, targets, op, known_lse_t, known_am_t, n_rows):
+    def forward(ctx, x2, weight, weight_t, targets, op, known_lse_t, known_am_t, n_rows, step=None):
         from .gemm import gemm_nt
 
         logits = gemm_nt(x2, weight)
         known = (known_lse_t, known_am_t) if known_lse_t is not None else None
-        loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, logits[:n_rows], targets, known)
+        loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, logits[:n_rows], targets, known,
+                                                                         step)
         ctx.save_for_backward(x, None if op == OP_CE else y, lse_d, lse_t, extra, am_t, weight_t)
         ctx.op, ctx.total_rows = op, logits.shape[0]
         ctx.mark_non_differentiable(am_d, am_t, lse_t, logits)
@@ -170,10 +219,10 @@ class _HeadFusedLoss(torch.autograd.Function):
         )
         dx_packed = gemm_nt(packed, weight_t, m_live=count)
         return (_unpack_rows(dx_packed, row_map, ctx.total_rows), None, None, None, None, None,
-                None, None)
+                None, None, None)
 
 
-def head_fused_rows(op: int, x, weight, weight_t, targets, target_stats=None, n_rows=None):
+def head_fused_rows(op: int, x, weight, weight_t, targets, target_stats=None, n_rows=None, step=None):
     """``fused_rows`` with the frozen head in front: ``x [1, T, H]`` instead of logits.  Returns
     ``(row_loss [1, n_rows], argmax_draft, argmax_target, lse_target, logits [1, T, Vd])``."""
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
@@ -188,19 +237,20 @@ def head_fused_rows(op: int, x, weight, weight_t, targets, target_stats=None, n_
     if y.shape[0] != n:
         raise ValueError(f"targets have {y.shape[0]} rows, expected {n}")
     ks = (None, None) if target_stats is None else (target_stats[0], target_stats[1])
-    loss, am_d, am_t, lse_t, logits = _HeadFusedLoss.apply(x[0], weight, weight_t, y, op, ks[0], ks[1], n)
+    loss, am_d, am_t, lse_t, logits = _HeadFusedLoss.apply(x[0], weight, weight_t, y, op, ks[0], ks[1], n,
+                                                           step)
     lead = (1, n)
     return (loss.view(lead), am_d.view(lead), am_t.view(lead), lse_t.view(lead),
             logits.view(1, t, weight.shape[0]))
 
 
-def fused_rows(op: int, logits, targets, target_stats=None, n_rows=None):
+def fused_rows(op: int, logits, targets, target_stats=None, n_rows=None, step: StepPass | None = None):
     """(row_loss, argmax_draft, argmax_target, lse_target) of one primitive reduction;
     ``n_rows`` restricts ``logits [1, T, V]`` to its first ``n_rows`` rows (``targets`` already
-    has that many) without slicing it under autograd."""
+    has that many) without slicing it under autograd; ``step``: see ``StepPass``."""
     if target_stats is None:
-        return _FusedLoss.apply(logits, targets, op, None, None, n_rows)
-    return _FusedLoss.apply(logits, targets, op, target_stats[0], target_stats[1], n_rows)
+        return _FusedLoss.apply(logits, targets, op, None, None, n_rows, step)
+    return _FusedLoss.apply(logits, targets, op, target_stats[0], target_stats[1], n_rows, step)
 
 
 def kl_div_loss(logits, targets):

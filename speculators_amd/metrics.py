@@ -26,20 +26,29 @@ def _as_mask(t: torch.Tensor) -> torch.Tensor:
 
 class _StepReduce(torch.autograd.Function):
     """(row_loss [n] f32) -> weighted masked mean (0-d); also fills ``out`` (6 floats)
-    and updates ``prev_correct`` in place.  d/d row_loss = row_weight."""
+    and updates ``prev_correct`` in place.  d/d row_loss = row_weight.  With ``counts`` (int32
+    ``[3]``) the acceptance chain was already done by the loss pass (``losses.StepPass``): only
+    the mean is reduced here and the counts are copied into ``out``."""
 
     @staticmethod
-    def forward(ctx, row_loss, am_d, am_t, mask, prev, weight, out):
+    def forward(ctx, row_loss, am_d, am_t, mask, prev, weight, out, counts=None):
         n = row_loss.numel()
         row_loss = row_loss.reshape(-1).contiguous()
         row_weight = torch.empty(n, device=row_loss.device, dtype=torch.float32)
-        _lib.call(
-            "spx_ttt_step_reduce", _lib.ptr(row_loss), _lib.ptr(am_d), _lib.ptr(am_t),
-            _lib.ptr(mask), _lib.kind_code(mask) if mask is not None else 0,
-            _lib.ptr(prev), _lib.kind_code(prev) if prev is not None else 0,
-            n, float(weight), _lib.ptr(out), _lib.ptr(row_weight),
-            _lib.stream_ptr(row_loss.device),
-        )
+        if counts is not None:
+            _lib.call(
+                "spx_ttt_step_mean", _lib.ptr(row_loss), _lib.ptr(mask),
+                _lib.kind_code(mask) if mask is not None else 0, n, float(weight), _lib.ptr(counts),
+                _lib.ptr(out), _lib.ptr(row_weight), _lib.stream_ptr(row_loss.device),
+            )
+        else:
+            _lib.call(
+                "spx_ttt_step_reduce", _lib.ptr(row_loss), _lib.ptr(am_d), _lib.ptr(am_t),
+                _lib.ptr(mask), _lib.kind_code(mask) if mask is not None else 0,
+                _lib.ptr(prev), _lib.kind_code(prev) if prev is not None else 0,
+                n, float(weight), _lib.ptr(out), _lib.ptr(row_weight),
+                _lib.stream_ptr(row_loss.device),
+            )
         ctx.save_for_backward(row_weight)
         ctx.shape = row_loss.shape
         return out[0].clone()
@@ -47,7 +56,27 @@ class _StepReduce(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         (row_weight,) = ctx.saved_tensors
-        return (row_weight * g).view(ctx.shape), None, None, None, None, None, None
+        return (row_weight * g).view(ctx.shape), None, None, None, None, None, None, None
+
+
+class TargetGather:
+    """Full-vocabulary verifier logits (``[1, T, Vt]``) with the ``d2t`` offset table, standing
+    where ``compute_metrics`` takes the targets.  The first TTT step reads its target rows
+    THROUGH the table inside the loss pass (no gather kernel, no ``[T, Vd]`` copy made first) and
+    leaves the draft-vocabulary rows in ``compact`` (``[1, T, Vd]``), which the later steps and the
+    backward stream."""
+
+    def __init__(self, full_logits: torch.Tensor, d2t: torch.Tensor):
+        if full_logits.dim() != 3 or full_logits.shape[0] != 1:
+            raise ValueError("verifier logits must be [1, T, Vt] (the packed batch layout)")
+        self.full = full_logits
+        self.d2t = d2t.to(torch.int64).contiguous()
+        self.compact = None
+
+    def materialize(self) -> torch.Tensor:
+        if self.compact is None:
+            self.compact = L.vocab_gather(self.full, self.d2t)
+        return self.compact
 
 
 def _step_views(logits, targets, loss_mask, prev_correct, ttt_step):
@@ -110,6 +139,14 @@ def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
             logits = logits.materialize()
     if logits.shape[0] != 1:
         raise ValueError("the packed batch layout has batch size 1 (train/data.py:306-393)")
+    gather = None
+    if isinstance(targets, TargetGather):
+        name0, (fn0, _) = next(iter(loss_config.items()))
+        if (targets.compact is None and ttt_step == 0 and name0 in L.PRIMITIVE_OP
+                and fn0 is L._HIP_LOSS_FN_MAP.get(name0)):
+            gather, targets = targets, targets.full  # read through d2t inside the first loss pass
+        else:
+            targets = targets.materialize()
     s_logits, s_targets, s_mask, s_prev = _step_views(
         logits, targets, loss_mask, prev_correct, ttt_step)
     dev = logits.device
@@ -128,12 +165,22 @@ def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
     terms = {}
     multi = len(loss_config) > 1
     first_out = None
+    counts = None
     for ti, (name, (fn, w)) in enumerate(loss_config.items()):
         out = torch.empty(6, device=dev, dtype=torch.float32)
         op = L.PRIMITIVE_OP.get(name)
+        step = None
+        if ti == 0:
+            # the first term's row pass also gathers the targets (first step of a TargetGather)
+            # and advances the acceptance chain
+            counts = torch.zeros(3, device=dev, dtype=torch.int32)
+            step = L.StepPass(d2t=gather.d2t if gather is not None else None, mask=mask1, prev=prev1,
+                              counts=counts)
+        elif gather is not None:
+            s_targets = gather.compact
         if fn is L._HIP_LOSS_FN_MAP.get(name) and op is not None:
             known = None
-            if target_stats_cache is not None and op in (L.OP_KL, L.OP_CE):
+            if target_stats_cache is not None and op in (L.OP_KL, L.OP_CE) and gather is None:
                 full = target_stats_cache.get("kl" if op == L.OP_KL else "ce")
                 if full is None and op == L.OP_CE:
                     full = target_stats_cache.get("kl")  # the arg-max is all ce needs
@@ -142,22 +189,25 @@ def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
             # the full logits go in with a row count: see _FusedLoss.forward
             if head is not None:
                 rows, am_d, am_t, lse_t, head.logits = L.head_fused_rows(
-                    op, head.x, head.weight, head.weight_t, s_targets, known, n_rows=s_logits.shape[1])
+                    op, head.x, head.weight, head.weight_t, s_targets, known, n_rows=s_logits.shape[1],
+                    step=step)
             else:
                 rows, am_d, am_t, lse_t = L.fused_rows(op, logits, s_targets, known,
-                                                       n_rows=s_logits.shape[1])
+                                                       n_rows=s_logits.shape[1], step=step)
+            if step is not None and step.gathered is not None:
+                gather.compact = step.gathered.view(1, -1, step.gathered.shape[-1])
             if (target_stats_cache is not None and known is None and ttt_step == 0
                     and op in (L.OP_KL, L.OP_CE)):
                 target_stats_cache["kl" if op == L.OP_KL else "ce"] = (
                     lse_t.reshape(-1), am_t.reshape(-1))
         else:
             rows = fn(s_logits, s_targets)
-            _, am_d, am_t, _ = L.fused_rows(L.OP_CE, s_logits.detach(), s_targets)
+            _, am_d, am_t, _ = L.fused_rows(L.OP_CE, s_logits.detach(), s_targets, step=step)
         if ti == 0:
             pred = am_d.reshape(-1)
-        # only the first term advances the acceptance chain
+        # only the first term advances the acceptance chain (inside its row pass)
         term = _StepReduce.apply(rows.reshape(-1), am_d.reshape(-1), am_t.reshape(-1), mask1,
-                                 prev1 if ti == 0 else None, weight, out)
+                                 None, weight, out, counts if ti == 0 else None)
         if ti == 0:
             first_out = out
         if multi:

@@ -109,6 +109,87 @@ def test_vocab_gather_bit_exact():
     assert torch.equal(L.vocab_gather(full32.cuda(), d2t.cuda()).cpu(), full32[..., t2d])
 
 
+@pytest.mark.parametrize("op_name", ["kl_div", "rkl", "jsd", "ce", "tv"])
+@pytest.mark.parametrize("dtype,vt,vd", [(torch.bfloat16, 128256, 32000), (torch.float32, 1000, 333),
+                                         (torch.bfloat16, 5003, 1001)])
+def test_step_pass_gathers_and_counts_in_the_row_pass(op_name, dtype, vt, vd):
+    """The one-pass form (targets read through d2t, acceptance chain inside the row pass) against
+    the three-kernel form (gather, loss, chain reduce): gathered rows bit-exact against the
+    oracle's index mapping, row losses / statistics / arg-maxes bit-identical, counts and the
+    in-place ``prev_correct`` identical."""
+    from speculators_amd import _lib
+    from speculators_amd import losses as L
+
+    g = torch.Generator().manual_seed(vt + vd)
+    rows = 37
+    sel = torch.randperm(vt, generator=g)[:vd]
+    d2t, t2d = OV.build_vocab_mappings(sel.tolist(), vt)
+    full = (torch.randn(rows, vt, generator=g) * 2).to(dtype).cuda()
+    logits = (torch.randn(rows, vd, generator=g) * 2).to(dtype).cuda()
+    compact = L.vocab_gather(full, d2t.cuda())
+    assert torch.equal(compact.cpu(), OV.gather_targets(full.cpu(), d2t))
+    for i in range(0, rows, 3):  # a third of the rows agree with their target
+        logits[i, compact[i].float().argmax()] = 30.0
+    mask = (torch.rand(rows, generator=g) < 0.7).float().cuda()
+    prev0 = (torch.rand(rows, generator=g) < 0.8).cuda()
+    op = L.PRIMITIVE_OP[op_name]
+
+    ref = L.fused_loss_forward(op, logits, compact)
+    out = torch.empty(6, device="cuda")
+    prev_ref = prev0.clone()
+    _lib.call("spx_ttt_step_reduce", _lib.ptr(ref[0]), _lib.ptr(ref[4]), _lib.ptr(ref[5]), _lib.ptr(mask),
+              _lib.kind_code(mask), _lib.ptr(prev_ref), _lib.kind_code(prev_ref), rows, 0.7,
+              _lib.ptr(out), None, _lib.stream_ptr(mask.device))
+
+    prev_got = prev0.clone()
+    step = L.StepPass(d2t=d2t.cuda(), mask=mask, prev=prev_got,
+                      counts=torch.zeros(3, dtype=torch.int32, device="cuda"))
+    got = L.fused_loss_forward(op, logits, full, step=step)
+    assert torch.equal(step.gathered, compact)
+    for a, b in zip(got[:6], ref[:6], strict=True):
+        assert torch.equal(a, b)
+    assert torch.equal(prev_got, prev_ref)
+    assert step.counts.tolist() == [int(out[1]), int(out[2]), int(out[4])]
+    out2 = torch.empty(6, device="cuda")
+    _lib.call("spx_ttt_step_mean", _lib.ptr(got[0]), _lib.ptr(mask), _lib.kind_code(mask), rows, 0.7,
+              _lib.ptr(step.counts), _lib.ptr(out2), None, _lib.stream_ptr(mask.device))
+    assert torch.equal(out2, out)
+
+
+def test_compute_metrics_with_target_gather_equals_materialised_targets():
+    """compute_metrics over three TTT steps with the targets given as full-vocabulary logits +
+    d2t (first step reads through the table and leaves the draft-vocabulary rows behind) against
+    the same call on gathered targets: every metric, the loss and the gradients bit for bit."""
+    from speculators_amd import losses as L
+    from speculators_amd.metrics import TargetGather, compute_metrics
+
+    g = torch.Generator().manual_seed(8)
+    t, vt, vd, steps = 130, 4000, 1000, 3
+    sel = torch.randperm(vt, generator=g)[:vd]
+    d2t, _ = OV.build_vocab_mappings(sel.tolist(), vt)
+    full = (torch.randn(1, t, vt, generator=g) * 2).bfloat16().cuda()
+    mask = (torch.rand(1, t, generator=g) < 0.7).float().cuda()
+    logits = [(torch.randn(1, t, vd, generator=g) * 2).bfloat16().cuda() for _ in range(steps)]
+    runs = []
+    for form in ("gather", "materialised"):
+        tg = TargetGather(full, d2t.cuda()) if form == "gather" else L.vocab_gather(full, d2t.cuda())
+        prev, cache, res = mask.clone(), {}, []
+        for k in range(steps):
+            lg = logits[k].clone().requires_grad_(True)
+            loss, m = compute_metrics(lg, tg, mask, prev, k, 0.9, L.resolve_loss_config("kl_div"),
+                                      target_stats_cache=cache)
+            loss.backward()
+            res.append((loss.detach(), m, lg.grad, prev.clone()))
+        if form == "gather":
+            assert torch.equal(tg.compact, L.vocab_gather(full, d2t.cuda()))
+        runs.append(res)
+    for (la, ma, ga, pa), (lb, mb, gb, pb) in zip(*runs, strict=True):
+        assert torch.equal(la, lb) and torch.equal(ga, gb) and torch.equal(pa, pb)
+        assert ma.keys() == mb.keys()
+        for key in ma:
+            assert torch.equal(ma[key], mb[key]), key
+
+
 @pytest.mark.parametrize("mask_dtype", [torch.float32, torch.bool, torch.int64, torch.bfloat16])
 def test_eagle3_compute_metrics_chain_matches_oracle(mask_dtype):
     from speculators_amd import losses as L
