@@ -298,8 +298,49 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
                   _lib.ptr(rg), None, _lib.ptr(grad), vd, st)
 
     ms = time_events(torch, loss_bwd, 20)
-    hbm("loss_bwd_kernel[KL, T rows x Vd]", 3.0 * t * vd * 2, ms, k_steps, "loss_bwd")
-    del tg, lg, grad, y
+    hbm("loss_bwd_kernel[KL, T rows x Vd]", 3.0 * t * vd * 2, ms, 0, "loss_bwd")
+
+    # what the model launches while lm_head is frozen: the same gradient with the live rows (loss
+    # mask Bernoulli(0.7), as in the timed step) packed to the front; dead rows are neither read
+    # nor written
+    live_mask = torch.rand(t, device=device, generator=g) < 0.7
+    rg_live = torch.where(live_mask, rg, torch.zeros_like(rg))
+    row_map, _count = L._packed_row_map(rg_live)
+    n_live = int(live_mask.sum().item())
+
+    def loss_bwd_packed():
+        _lib.call("spx_fused_vocab_loss_bwd_packed", L.OP_KL, _lib.ptr(lg), vd, _lib.ptr(tg), vd, t, vd, 0,
+                  _lib.ptr(stats[1]), _lib.ptr(stats[2]), _lib.ptr(stats[3]), _lib.ptr(arg[1]),
+                  _lib.ptr(rg_live), None, _lib.ptr(row_map), _lib.ptr(grad), vd, st)
+
+    ms = time_events(torch, loss_bwd_packed, 20)
+    hbm(f"loss_bwd_kernel[KL, packed: {n_live} live of T rows x Vd]", 3.0 * n_live * vd * 2, ms, k_steps)
+
+    # the first step of the verifier-logits entry point: target rows read THROUGH d2t from the
+    # full-vocabulary logits, draft-vocabulary rows written out for the later steps, acceptance
+    # chain in the same pass.  Algorithmic bytes per row: the draft row, the 64-byte sectors of the
+    # full row that hold a selected id, the gathered row written.
+    vt = cfg["vocab_size"]
+    sel = torch.randperm(vt, device=device, generator=g)[:vd].sort().values
+    d2t = (sel - torch.arange(vd, device=device)).contiguous()
+    touched = int(torch.unique(sel // 32).numel()) * 64
+    full = (torch.randn(t, vt, device=device, generator=g) * 2).bfloat16()
+    gathered = torch.empty(t, vd, device=device, dtype=torch.bfloat16)
+    mask_f = live_mask.float()
+    prev = live_mask.clone()
+    counts = torch.zeros(3, device=device, dtype=torch.int32)
+
+    def loss_step_gather():
+        _lib.call("spx_vocab_loss_step_fwd", L.OP_KL, _lib.ptr(lg), vd, _lib.ptr(full), vt, _lib.ptr(d2t),
+                  vt, _lib.ptr(gathered), vd, t, vd, 0, _lib.ptr(stats[0]), _lib.ptr(stats[1]),
+                  _lib.ptr(stats[2]), _lib.ptr(stats[3]), _lib.ptr(arg[0]), _lib.ptr(arg[1]), 0,
+                  _lib.ptr(mask_f), _lib.kind_code(mask_f), _lib.ptr(prev), _lib.kind_code(prev),
+                  _lib.ptr(counts), st)
+
+    ms = time_events(torch, loss_step_gather, 20)
+    hbm("loss_fwd_kernel[KL + d2t gather from T x Vt + acceptance chain, step 0 of --targets logits]",
+        float(t) * (vd * 2 + touched + vd * 2), ms, 0)
+    del tg, lg, grad, y, full, gathered
 
     # batch producer: 8 documents of (T + 8) / 8 rows, 3 auxiliary layers + the last one, bf16 ->
     # the packed [1, T, ...] row (outside the timed step: it runs on a side stream ahead of it)

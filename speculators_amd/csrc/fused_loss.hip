@@ -138,16 +138,72 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
   s.md = kNegBig; s.zd = 0.f; s.mt = kNegBig; s.zt = 0.f; s.at = 0.f;
   s.bd = -INFINITY; s.id = 0x7fffffff; s.bt = -INFINITY; s.it = 0x7fffffff; s.xt = 0.f;
 
-  for (int64_t c = tid; c < nchunks; c += kLossThreads) {
+  // GATHER: the draft ids of one tile (256 chunks) map to an ascending span of the full row.
+  // The span is brought into LDS with coalesced 16-byte loads and the eight elements of a lane
+  // are picked from there; a span that does not fit (or rows without 16-byte alignment) and any
+  // id that falls outside the span (a table that is not ascending) read the row directly.
+  constexpr int kStageElems = GATHER ? 32768 / (int)sizeof(T) : 1;
+  __shared__ __attribute__((aligned(16))) T stage[kStageElems];
+  for (int64_t c0 = 0; c0 < nchunks; c0 += kLossThreads) {
+    const int64_t c = c0 + tid;
+    const bool active = c < nchunks;
     const int64_t base = c << 3;
     float x[8], y[8];
-    load8<T, VEC>(xrow, base, vocab, x);
     if (GATHER) {
-      load8_gather<T>(yrow, sa.d2t, base, vocab, sa.vt, y);
-      if (grow) store8<T, VEC>(grow, base, vocab, y);
-    } else if (read_y) {
-      load8<T, VEC>(yrow, base, vocab, y);
+      // this lane's draft row chunk and its eight target columns first: their latency runs
+      // under the staging of the span
+      int64_t jj[8];
+      if (active) {
+        load8<T, VEC>(xrow, base, vocab, x);
+        if (base + 8 <= vocab && ptr_aligned16(sa.d2t)) {
+          const u32x4* dp = reinterpret_cast<const u32x4*>(sa.d2t + base);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const u32x4 w = dp[q];
+            jj[2 * q] = base + 2 * q + (int64_t)(((uint64_t)w.y << 32) | w.x);
+            jj[2 * q + 1] = base + 2 * q + 1 + (int64_t)(((uint64_t)w.w << 32) | w.z);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) jj[i] = base + i < vocab ? base + i + sa.d2t[base + i] : -1;
+        }
+      }
+      const int64_t i0 = c0 << 3, i1 = min(vocab, (c0 + kLossThreads) << 3) - 1;
+      int64_t lo = i0 + sa.d2t[i0], hi = i1 + sa.d2t[i1] + 1;
+      lo = max((int64_t)0, min(lo, sa.vt)) & ~(int64_t)7;
+      hi = max(lo, min(hi, sa.vt));
+      constexpr int EPV = 16 / (int)sizeof(T);  // elements per 16-byte access
+      const bool staged = VEC && (hi - lo) <= kStageElems && ((ld_targets & 7) == 0) &&
+                          ptr_aligned16(targets);
+      if (staged) {
+        __syncthreads();  // the previous tile's picks are done
+        for (int64_t e = (int64_t)tid * EPV; lo + e < hi; e += kLossThreads * EPV) {
+          if (lo + e + EPV <= sa.vt)
+            *reinterpret_cast<u32x4*>(&stage[e]) = ld16(yrow + lo + e);
+          else
+            for (int q = 0; q < EPV; ++q)
+              if (lo + e + q < sa.vt) stage[e + q] = yrow[lo + e + q];
+        }
+        __syncthreads();
+      }
+      if (active) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float val = kNegBig;  // tail padding, like load8_guard
+          if (base + i < vocab) {
+            const int64_t j = jj[i];
+            if (staged && j >= lo && j < hi) val = load1(&stage[j - lo]);
+            else val = (j >= 0 && j < sa.vt) ? load1(yrow + j) : -INFINITY;
+          }
+          y[i] = val;
+        }
+        if (grow) store8<T, VEC>(grow, base, vocab, y);
+      }
+    } else if (active) {
+      load8<T, VEC>(xrow, base, vocab, x);
+      if (read_y) load8<T, VEC>(yrow, base, vocab, y);
     }
+    if (!active) continue;
     float cx = x[0], cy = y[0];
 #pragma unroll
     for (int i = 1; i < 8; ++i) cx = fmaxf(cx, x[i]);
