@@ -103,6 +103,20 @@ __global__ __launch_bounds__(256) void dflash_ranges_kernel(
   b2[r] = causal_block ? (int)(r + 1) : (int)((j + 1) * block_size);
 }
 
+// Eight bf16 values times a scalar, rounded back to bf16 (round to nearest even).  The queries
+// enter every score product as bf16(q * scale * log2 e): the forward, the dQ kernel (both scale
+// their register fragments with this function) and the dK/dV and diagonal-key kernels (which
+// read the copy the backward's prologue writes with it) must see the SAME rounded values, or the
+// probabilities the backward recomputes would not match the forward's log-sum-exp.
+__device__ __forceinline__ u32x4 scale_bf16x8(u32x4 raw, float c) {
+  u32x4 w;
+  w.x = pack_bf16x2(bf16_lo(raw.x) * c, bf16_hi(raw.x) * c);
+  w.y = pack_bf16x2(bf16_lo(raw.y) * c, bf16_hi(raw.y) * c);
+  w.z = pack_bf16x2(bf16_lo(raw.z) * c, bf16_hi(raw.z) * c);
+  w.w = pack_bf16x2(bf16_lo(raw.w) * c, bf16_hi(raw.w) * c);
+  return w;
+}
+
 // ---------------------------------------------------------------- transpose
 // dst[h][c][perm(r)] = src[h][r][c] for r < rows, c < cols; dst row stride ld_dst >= rows
 // (a multiple of 16), the columns of r in rows..ld_dst-1 are zero filled.  perm swaps bits
@@ -113,9 +127,13 @@ __global__ __launch_bounds__(256) void dflash_ranges_kernel(
 // (eight lanes read a whole 128-byte line), transposes it in registers (v_perm_b32) and writes, for each
 // of its 8 columns, the two 4-row halves of the block to their permuted places (8 bytes each; the eight
 // lanes that share a column fill its 128-byte line in two store instructions).  cols a multiple of 8.
+// SCALED: the elements are multiplied by `scale` first (scale_bf16x8) and the scaled rows are also
+// written row-major to `scaled` ([h][rows][cols], head stride rows * cols).
+template <bool SCALED>
 __global__ __launch_bounds__(64) void transpose_bf16_kernel(
     const uint16_t* __restrict__ src, int64_t src_hs, int64_t src_ld, int rows, int cols,
-    uint16_t* __restrict__ dst, int64_t dst_hs, int64_t ld_dst) {
+    uint16_t* __restrict__ dst, int64_t dst_hs, int64_t ld_dst, float scale,
+    uint16_t* __restrict__ scaled) {
   const int h = blockIdx.z;
   const int lane = threadIdx.x;
   const int rb = lane >> 3, cb = lane & 7;
@@ -127,6 +145,11 @@ __global__ __launch_bounds__(64) void transpose_bf16_kernel(
   for (int j = 0; j < 8; ++j) {
     const u32x4 z = {0, 0, 0, 0};
     in[j] = (r0 + j < rows) ? *reinterpret_cast<const u32x4*>(s + (int64_t)(r0 + j) * src_ld) : z;
+    if (SCALED) {
+      in[j] = scale_bf16x8(in[j], scale);
+      if (r0 + j < rows)
+        *reinterpret_cast<u32x4*>(scaled + ((int64_t)h * rows + r0 + j) * cols + c0) = in[j];
+    }
   }
   // where the block's two halves go: r0 % 16 == 0 -> r0 and r0 + 8, r0 % 16 == 8 -> r0 - 4 and r0 + 4
   const int p_lo = (r0 & 8) ? r0 - 4 : r0, p_hi = (r0 & 8) ? r0 + 4 : r0 + 8;
@@ -303,19 +326,34 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
   RowBounds<NSB> rb;
   load_bounds<NSB, NW>(p, ic, wave, lane, red, rb);
 
+  // The query fragments carry the soft-max scale and log2(e): the scores then come out of the
+  // MFMA in the base-2 exponent domain and need no multiply of their own.
   bf16x8 qf[NSB][NKK];
 #pragma unroll
   for (int sb = 0; sb < NSB; ++sb) {
     const uint16_t* qrow = p.Q + (int64_t)h * p.q_hs + (int64_t)ic[sb] * D + g * 8;
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk)
-      qf[sb][kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(qrow + kk * 16));
+      qf[sb][kk] = as_bf16x8(scale_bf16x8(*reinterpret_cast<const u32x4*>(qrow + kk * 16), p.scale_log2e));
   }
-  f32x16 acc[NSB][NDB];
-  float m_run[NSB], l_run[NSB];
+  // Soft-max bookkeeping per query (a lane owns one query; its partner lane ^ 32 the same one):
+  //   m_ref  the value subtracted from the scores before the exp2.  It is NOT the running maximum:
+  //          it only moves when a tile's largest score exceeds it by more than kRefSlack (or when
+  //          the row sees its first key), so most tiles skip the rescaling pass altogether.  A
+  //          common factor 2^k on a row's probabilities is exact in binary floating point and
+  //          cancels in O / l; the slack only has to keep 2^(s - m_ref) far from overflow.
+  //   nref   -m_ref in all sixteen accumulator slots: the C operand of the first score MFMA, so
+  //          the subtraction costs no instruction.
+  //   l_run  this LANE's part of the row sum (its 32 of a tile's 64 keys); the halves are added
+  //          once, after the last tile.
+  constexpr float kRefSlack = 12.f;
+  f32x16 acc[NSB][NDB], nref[NSB];
+  float m_ref[NSB], l_run[NSB];
 #pragma unroll
   for (int sb = 0; sb < NSB; ++sb) {
-    m_run[sb] = kNegBig; l_run[sb] = 0.f;
+    m_ref[sb] = -INFINITY; l_run[sb] = 0.f;  // -inf: the row has not seen a key yet
+#pragma unroll
+    for (int r = 0; r < 16; ++r) nref[sb][r] = 0.f;
 #pragma unroll
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
@@ -434,12 +472,6 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
       if (n0 >= w_bmax || n0 + kBN <= w_amin) continue;  // nothing visible for this wave
 
       f32x16 st[NSB][2];
-#pragma unroll
-      for (int sb = 0; sb < NSB; ++sb)
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) st[sb][kb][r] = 0.f;
       SPX_PRIO_MFMA();
       // K fragments go through a ring of four registers: the read of fragment f + 4 is
       // issued right after the MFMA of fragment f, so no MFMA waits for LDS; the two
@@ -462,7 +494,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int sb = 0; sb < NSB; ++sb)
-            st[sb][f & 1] = mfma32(kfr[f & 3], qf[sb][f >> 1], st[sb][f & 1]);
+            st[sb][f & 1] = mfma32(kfr[f & 3], qf[sb][f >> 1], f < 2 ? nref[sb] : st[sb][f & 1]);
           __builtin_amdgcn_sched_barrier(0);
           if (f + 4 < NF) kread(f + 4);
         }
@@ -489,33 +521,43 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
               if (cr < m_lo[sb] || cr >= m_hi[sb]) st[sb][kb][r] = -INFINITY;
             }
         }
-        float mx = -INFINITY;
+        // st holds s - m_ref.  Largest of the 32 scores of this lane (three-operand maxima)
+        float mx = fmaxf(st[sb][0][0], st[sb][1][0]);
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[sb][kb][r]);
+        for (int r = 1; r < 16; r += 2) {
+          mx = fmaxf(fmaxf(mx, st[sb][0][r]), st[sb][0][r + 1 < 16 ? r + 1 : r]);
+          mx = fmaxf(fmaxf(mx, st[sb][1][r]), st[sb][1][r + 1 < 16 ? r + 1 : r]);
+        }
         mx = half_swap_max(mx);
-        const float m_new = fmaxf(m_run[sb], mx * p.scale_log2e);
-        const float alpha = fast_exp2(m_run[sb] - m_new);
-        float rs = 0.f;
+        const bool unset = m_ref[sb] == -INFINITY;
+        const bool move = mx > -INFINITY && (unset || mx > kRefSlack);
+        if (__any(move)) {
+          // some row's reference moves: shift its scores, rescale its sum and its accumulator
+          asm volatile("; reference moves");
+          const float delta = move ? mx : 0.f;
+          const float alpha = (move && !unset) ? fast_exp2(-delta) : 1.f;  // unset rows hold zeros
+          m_ref[sb] = move ? (unset ? mx : m_ref[sb] + mx) : m_ref[sb];
+          const float nr = unset && !move ? 0.f : -m_ref[sb];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+          for (int r = 0; r < 16; ++r) nref[sb][r] = nr;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float pv = fast_exp2(fmaf(st[sb][kb][r], p.scale_log2e, -m_new));
-            st[sb][kb][r] = pv;
-            rs += pv;
-          }
-        rs = half_swap_sum(rs);
-        l_run[sb] = l_run[sb] * alpha + rs;
-        // the accumulator only needs rescaling when some row's max moved
-        if (__any(m_new != m_run[sb])) {
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) st[sb][kb][r] -= delta;
+          l_run[sb] *= alpha;
 #pragma unroll
           for (int db = 0; db < NDB; ++db)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[sb][db][r] *= alpha;
         }
-        m_run[sb] = m_new;
+        float rs0 = 0.f, rs1 = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float p0 = fast_exp2(st[sb][0][r]), p1 = fast_exp2(st[sb][1][r]);
+          st[sb][0][r] = p0; st[sb][1][r] = p1;
+          rs0 += p0; rs1 += p1;
+        }
+        l_run[sb] += rs0 + rs1;
       }
       SPX_PRIO_MFMA();
       {
@@ -556,6 +598,11 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
   if (p.a2)
     run_pass(rb.a2, rb.b2, rb.w_a2min, rb.w_a2max, rb.w_b2min, rb.w_b2max, rb.blk_a2, rb.blk_b2);
 
+  // from here on l_run is the whole row's sum in both lanes of a query
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) l_run[sb] = half_swap_sum(l_run[sb]);
+  float (&m_run)[NSB] = m_ref;
+
   // TTT diagonal keys (j, r), j = 1..n_extra: one dot product each
   for (int j = 1; j <= p.n_extra; ++j) {
 #pragma unroll
@@ -565,10 +612,9 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
 #pragma unroll
       for (int kk = 0; kk < NKK; ++kk)
         dot = dot8_bf16(qf[sb][kk], *reinterpret_cast<const u32x4*>(kj + kk * 16), dot);
-      dot = half_swap_sum(dot);
-      const float s = dot * p.scale_log2e;
+      const float s = half_swap_sum(dot);  // the query fragments carry the scale
       const float m_new = fmaxf(m_run[sb], s);
-      const float alpha = fast_exp2(m_run[sb] - m_new);
+      const float alpha = fast_exp2(m_run[sb] - m_new);  // a row without context keys: exp2(-inf) = 0
       const float pv = fast_exp2(s - m_new);
       l_run[sb] = l_run[sb] * alpha + pv;
       m_run[sb] = m_new;
@@ -734,16 +780,22 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
   RowBounds<NSB> rb;
   load_bounds<NSB, NW>(p, ic, wave, lane, red, rb);
 
+  // the query fragments carry scale * log2(e) (see scale_bf16x8); -lse and -delta of the lane's
+  // query sit in all sixteen slots of two blocks that the first MFMA of each product takes as its
+  // C operand, so s - lse and dP - delta come out of the matrix pipe
   bf16x8 qf[NSB][NKK], dof[NSB][NKK];
+  f32x16 nlse[NSB], ndel[NSB];
 #pragma unroll
   for (int sb = 0; sb < NSB; ++sb) {
     const uint16_t* qrow = p.Q + (int64_t)h * p.q_hs + (int64_t)ic[sb] * D + g * 8;
     const uint16_t* drow = dO + ((int64_t)ic[sb] * p.Hq + h) * D + g * 8;
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) {
-      qf[sb][kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(qrow + kk * 16));
+      qf[sb][kk] = as_bf16x8(scale_bf16x8(*reinterpret_cast<const u32x4*>(qrow + kk * 16), p.scale_log2e));
       dof[sb][kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(drow + kk * 16));
     }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { nlse[sb][r] = -lse_i[sb]; ndel[sb][r] = -delta_i[sb]; }
   }
   f32x16 acc[NSB][NDB];
 #pragma unroll
@@ -872,8 +924,6 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
 #pragma unroll
         for (int kb = 0; kb < TB / 32; ++kb) {
           f32x16 st, dp;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) { st[r] = 0.f; dp[r] = 0.f; }
           // K and V fragments alternate through a ring of four registers (fragment 2 kk is
           // K, 2 kk + 1 is V): the read of fragment f + 4 follows the MFMA of fragment f
           SPX_PRIO_MFMA();
@@ -895,8 +945,8 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
 #pragma unroll
             for (int f = 0; f < NF; ++f) {
               __builtin_amdgcn_sched_barrier(0);
-              if (f & 1) dp = mfma32(fr[f & 3], dof[sb][f >> 1], dp);
-              else st = mfma32(fr[f & 3], qf[sb][f >> 1], st);
+              if (f & 1) dp = mfma32(fr[f & 3], dof[sb][f >> 1], f == 1 ? ndel[sb] : dp);
+              else st = mfma32(fr[f & 3], qf[sb][f >> 1], f == 0 ? nlse[sb] : st);
               __builtin_amdgcn_sched_barrier(0);
               if (f + 4 < NF) fread(f + 4);
             }
@@ -904,7 +954,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
           }
           SPX_PRIO_VALU();
 #pragma unroll
-          for (int r = 0; r < 16; ++r) st[r] = fast_exp2(fmaf(st[r], p.scale_log2e, -lse_i[sb]));
+          for (int r = 0; r < 16; ++r) st[r] = fast_exp2(st[r]);
           if (need_mask) {
             // a real (scalar) branch, see the forward kernel
             asm volatile("; masked tile");
@@ -916,7 +966,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
             }
           }
 #pragma unroll
-          for (int r = 0; r < 16; ++r) dp[r] = st[r] * (dp[r] - delta_i[sb]);
+          for (int r = 0; r < 16; ++r) dp[r] *= st[r];
           SPX_PRIO_MFMA();
           {
             // K^T fragments through the same kind of ring; fragment f = (16-key step s2, D block db)
@@ -966,7 +1016,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
       }
       dot = half_swap_sum(dot);
       dpv = half_swap_sum(dpv);
-      const float pv = fast_exp2(fmaf(dot, p.scale_log2e, -lse_i[sb]));
+      const float pv = fast_exp2(dot - lse_i[sb]);  // the query fragments carry the scale
       const float ds = pv * (dpv - delta_i[sb]);
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
@@ -1154,8 +1204,8 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     if (tid < 64) {
       const int ir = mq + tid;
       const bool ok = ir < p.NQ;
-      lse_r = ok ? LSE[(int64_t)h * p.NQ + ir] : 0.f;
-      delta_r = ok ? Delta[(int64_t)h * p.NQ + ir] : 0.f;
+      lse_r = ok ? -LSE[(int64_t)h * p.NQ + ir] : 0.f;    // negated: they are MFMA C operands
+      delta_r = ok ? -Delta[(int64_t)h * p.NQ + ir] : 0.f;
       a1_r = ok ? p.a1[ir] : 0x7fffffff;
       b1_r = ok ? (p.b1 ? p.b1[ir] : ir + 1) : 0;
       a2_r = (ok && p.a2) ? p.T + p.a2[ir] : 0x7fffffff;
@@ -1227,8 +1277,8 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     if (tid < 64) {
       const int ir = mq + tid;
       const bool ok = ir < p.NQ;
-      lse_s[tid] = ok ? LSE[(int64_t)h * p.NQ + ir] : 0.f;
-      delta_s[tid] = ok ? Delta[(int64_t)h * p.NQ + ir] : 0.f;
+      lse_s[tid] = ok ? -LSE[(int64_t)h * p.NQ + ir] : 0.f;
+      delta_s[tid] = ok ? -Delta[(int64_t)h * p.NQ + ir] : 0.f;
       a1_s[tid] = ok ? p.a1[ir] : 0x7fffffff;
       b1_s[tid] = ok ? (p.b1 ? p.b1[ir] : ir + 1) : 0;
       a2_s[tid] = (ok && p.a2) ? p.T + p.a2[ir] : 0x7fffffff;
@@ -1333,9 +1383,25 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
 #pragma unroll
     for (int qbl = 0; qbl < NQB; ++qbl) {
       const int qb = sub_now * NQB + qbl;  // 32-row half inside the 64-row step (per-row scalars); qbl: inside the LDS tile
+      // the scores start from -lse of their query row and dO V^T from -delta (LDS holds both
+      // negated): s - lse and dP - delta come out of the matrix pipe.  The Q tile is the scaled
+      // copy (bf16(q * scale * log2 e)), so the scores are base-2 exponents already
       f32x16 st, dp;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { st[r] = 0.f; dp[r] = 0.f; }
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int q0 = qb * 32 + 8 * r4 + 4 * g;  // 4 consecutive query rows: one 16-byte LDS read each
+        const f32x4 ls = *reinterpret_cast<const f32x4*>(&lse_s[q0]);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) st[r4 * 4 + t] = ls[t];
+        if (kDoK) {
+          const f32x4 dl = *reinterpret_cast<const f32x4*>(&delta_s[q0]);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) dp[r4 * 4 + t] = dl[t];
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) dp[r4 * 4 + t] = 0.f;
+        }
+      }
       {
         // Q (and, for dK, dO) row fragments through a ring of four registers: the read of
         // fragment f + 4 follows the MFMA of fragment f, so no MFMA waits for LDS
@@ -1366,12 +1432,7 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        const int q0 = qb * 32 + 8 * r4 + 4 * g;  // 4 consecutive query rows: one 16-byte LDS read each
-        const f32x4 ls = *reinterpret_cast<const f32x4*>(&lse_s[q0]);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) st[r4 * 4 + t] = fast_exp2(fmaf(st[r4 * 4 + t], p.scale_log2e, -ls[t]));
-      }
+      for (int r = 0; r < 16; ++r) st[r] = fast_exp2(st[r]);
       if (!full) {
         // a real (scalar) branch: only tiles that straddle an interval edge pay for the mask
         asm volatile("; masked tile");
@@ -1392,11 +1453,7 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       }
       if (kDoK) {
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          const f32x4 dl = *reinterpret_cast<const f32x4*>(&delta_s[qb * 32 + 8 * r4 + 4 * g]);
-#pragma unroll
-          for (int t = 0; t < 4; ++t) dp[r4 * 4 + t] = st[r4 * 4 + t] * (dp[r4 * 4 + t] - dl[t]);
-        }
+        for (int r = 0; r < 16; ++r) dp[r] *= st[r];
       }
       {
         // dO^T / Q^T fragments through the same kind of ring; per (16-row step s2, D block db):
@@ -1626,10 +1683,11 @@ static int64_t fwd_workspace_bytes(int64_t NKV, int Hkv, int D) {
 static int64_t bwd_workspace_bytes(int64_t NQ, int64_t NKV, int Hq, int Hkv, int D) {
   const int64_t NKVp = round_up(NKV, 128), NQp = round_up(NQ, 128);
   int64_t b = (int64_t)Hkv * D * NKVp * 2;          // K^T
-  b += 2 * (int64_t)Hq * D * NQp * 2;                // Q^T, dO^T
+  b += 2 * (int64_t)Hq * D * NQp * 2;                // Q^T (scaled), dO^T
   b = round_up(b, 256) + round_up((int64_t)Hq * NQ * 4, 256);       // delta
   b += round_up(((NQ + 63) / 64) * 32, 256);                        // tile bounds
   b += 2 * round_up((int64_t)Hq * NKV * D * 4, 256);                // fp32 per-head dK, dV
+  b += round_up((int64_t)Hq * NQ * D * 2, 256);                     // Q scaled, row-major
   return b;
 }
 
@@ -1638,8 +1696,8 @@ static int launch_fwd(AttnParams p, void* workspace, uint16_t* O, float* lse, hi
                       const char* fn) {
   uint16_t* vt = reinterpret_cast<uint16_t*>(workspace);
   dim3 tgrid((unsigned)(p.NKVp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hkv);
-  hipLaunchKernelGGL(transpose_bf16_kernel, tgrid, dim3(64), 0, st, p.V, p.v_hs, (int64_t)D, p.NKV, D,
-                     vt, (int64_t)D * p.NKVp, (int64_t)p.NKVp);
+  hipLaunchKernelGGL(transpose_bf16_kernel<false>, tgrid, dim3(64), 0, st, p.V, p.v_hs, (int64_t)D, p.NKV, D,
+                     vt, (int64_t)D * p.NKVp, (int64_t)p.NKVp, 1.f, nullptr);
   constexpr int BM = 32 * kFwdNSB * kFwdNW;
   const int n_qb = (p.NQ + BM - 1) / BM;
   constexpr int PF = D > 128 ? (int)SPX_FWD256_PF : kFwdPF;
@@ -1674,15 +1732,23 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   float* dkp = reinterpret_cast<float*>(w);
   w += round_up((int64_t)p.Hq * p.NKV * D * 4, 256);
   float* dvp = reinterpret_cast<float*>(w);
+  w += round_up((int64_t)p.Hq * p.NKV * D * 4, 256);
+  uint16_t* qs = reinterpret_cast<uint16_t*>(w);  // bf16(q * scale * log2 e), [Hq][NQ][D]
 
   dim3 tgrid((unsigned)(p.NKVp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hkv);
-  hipLaunchKernelGGL(transpose_bf16_kernel, tgrid, dim3(64), 0, st, p.K, p.k_hs, (int64_t)D, p.NKV, D,
-                     kt, (int64_t)D * p.NKVp, (int64_t)p.NKVp);
+  hipLaunchKernelGGL(transpose_bf16_kernel<false>, tgrid, dim3(64), 0, st, p.K, p.k_hs, (int64_t)D, p.NKV, D,
+                     kt, (int64_t)D * p.NKVp, (int64_t)p.NKVp, 1.f, nullptr);
   dim3 qgrid((unsigned)(NQp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hq);
-  hipLaunchKernelGGL(transpose_bf16_kernel, qgrid, dim3(64), 0, st, p.Q, p.q_hs, (int64_t)D, p.NQ, D,
-                     qt, (int64_t)D * NQp, (int64_t)NQp);
-  hipLaunchKernelGGL(transpose_bf16_kernel, qgrid, dim3(64), 0, st, dOp, (int64_t)D,
-                     (int64_t)p.Hq * D, p.NQ, D, dot, (int64_t)D * NQp, (int64_t)NQp);
+  hipLaunchKernelGGL(transpose_bf16_kernel<true>, qgrid, dim3(64), 0, st, p.Q, p.q_hs, (int64_t)D, p.NQ, D,
+                     qt, (int64_t)D * NQp, (int64_t)NQp, p.scale_log2e, qs);
+  hipLaunchKernelGGL(transpose_bf16_kernel<false>, qgrid, dim3(64), 0, st, dOp, (int64_t)D,
+                     (int64_t)p.Hq * D, p.NQ, D, dot, (int64_t)D * NQp, (int64_t)NQp, 1.f, nullptr);
+  // the dK/dV and diagonal-key kernels read the scaled queries: their scores are q' . k with no
+  // factor of their own, and what they accumulate against q' carries scale * log2(e) once too
+  // often: dK = ln 2 * sum dS q'
+  AttnParams ps = p;
+  ps.Q = qs;
+  ps.q_hs = (int64_t)p.NQ * D;
   hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)(((int64_t)p.NQ * p.Hq + 15) / 16)), dim3(256),
                      0, st, Op, dOp, p.NQ, p.Hq, delta);
   hipLaunchKernelGGL(attn_tile_bounds_kernel, dim3((unsigned)((p.NQ + 63) / 64)), dim3(64), 0, st, p, tb);
@@ -1720,7 +1786,7 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, 3, 0>),
                                     (int)smem, dkv_lds_set[0], fn))
       return rc;
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, 3, 0>), kgrid, kblock, smem, st, p, dOp, qt, dot,
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, 3, 0>), kgrid, kblock, smem, st, ps, dOp, qt, dot,
                        NQp, lse, delta, tb, dkp, dvp);
   } else if constexpr (D > 128) {
     // one launch per gradient (each loads only the tiles it multiplies with)
@@ -1732,32 +1798,32 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF2, 2>),
                                     (int)smem2, dkv_lds_set[1], fn))
       return rc;
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF1, 1>), kgrid, kblock, smem1, st, p, dOp, qt,
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF1, 1>), kgrid, kblock, smem1, st, ps, dOp, qt,
                        dot, NQp, lse, delta, tb, dkp, dvp);
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF2, 2>), kgrid, kblock, smem2, st, p, dOp, qt,
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF2, 2>), kgrid, kblock, smem2, st, ps, dOp, qt,
                        dot, NQp, lse, delta, tb, dkp, dvp);
   } else {
     constexpr size_t smem = kPF == 2 ? DkvSmem<D, 0>::kBytesDma : DkvSmem<D, 0>::kBytes;
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF, 0>),
                                     (int)smem, dkv_lds_set[0], fn))
       return rc;
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF, 0>), kgrid, kblock, smem, st, p, dOp, qt, dot,
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF, 0>), kgrid, kblock, smem, st, ps, dOp, qt, dot,
                        NQp, lse, delta, tb, dkp, dvp);
   }
   const int64_t items = (int64_t)p.NKV * D / 4 * p.Hkv;
   hipLaunchKernelGGL(attn_dkv_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, dkp,
-                     dvp, p.NKV, D, p.Hq, p.Hkv, p.scaling, dKp, dk_hs, dVp, dv_hs);
+                     dvp, p.NKV, D, p.Hq, p.Hkv, kLn2, dKp, dk_hs, dVp, dv_hs);
   if (p.n_extra > 0) {
     const dim3 dgrid((unsigned)(((int64_t)p.T * p.Hkv + 15) / 16));
     // eight heads per K/V head in registers where they fit (head_dim <= 128), else four
     if (D <= 128 && p.Hq / p.Hkv > 4)
-      hipLaunchKernelGGL((ttt_attn_bwd_diag_kernel<D, (D <= 128 ? 8 : 4)>), dgrid, dim3(256), 0, st, p.Q,
-                         p.q_hs, p.K, p.k_hs, p.V, p.v_hs, dOp, lse, delta, p.T, p.n_extra, p.Hq, p.Hkv,
-                         p.scale_log2e, p.scaling, dKp, dk_hs, dVp, dv_hs);
+      hipLaunchKernelGGL((ttt_attn_bwd_diag_kernel<D, (D <= 128 ? 8 : 4)>), dgrid, dim3(256), 0, st, ps.Q,
+                         ps.q_hs, p.K, p.k_hs, p.V, p.v_hs, dOp, lse, delta, p.T, p.n_extra, p.Hq, p.Hkv,
+                         1.f, kLn2, dKp, dk_hs, dVp, dv_hs);
     else
-      hipLaunchKernelGGL((ttt_attn_bwd_diag_kernel<D, 4>), dgrid, dim3(256), 0, st, p.Q, p.q_hs, p.K,
+      hipLaunchKernelGGL((ttt_attn_bwd_diag_kernel<D, 4>), dgrid, dim3(256), 0, st, ps.Q, ps.q_hs, p.K,
                          p.k_hs, p.V, p.v_hs, dOp, lse, delta, p.T, p.n_extra, p.Hq, p.Hkv,
-                         p.scale_log2e, p.scaling, dKp, dk_hs, dVp, dv_hs);
+                         1.f, kLn2, dKp, dk_hs, dVp, dv_hs);
   }
   return check_launch(fn);
 }

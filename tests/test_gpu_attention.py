@@ -144,7 +144,12 @@ def _check_sampled_rows(q, k, v, out, go, rows, heads, visible, scale):
         got = out.detach()[0, i, h].float().cpu()
         assert (got - want.detach()).abs().max() <= 2e-2 * want.detach().abs().max() + 1e-3, (i, h)
         dq = q.grad[0, h, i].float().cpu()
-        assert (dq - qi.grad).abs().max() <= 3e-2 * qi.grad.abs().max() + 1e-3, (i, h)
+        # delta = dO . O is taken from the bf16-rounded output (as in every flash-attention backward):
+        # |d delta| <= 2^-9 sum_d |dO_d O_d|, and it reaches dQ through sum_j P_j k_j * scale.  That
+        # floor matters for rows with very few keys, where dP - delta nearly cancels
+        do = go[0, i, h].float().cpu()
+        floor = 2.0 ** -9 * float(do.abs() @ want.detach().abs()) * scale * float(ks.abs().max())
+        assert (dq - qi.grad).abs().max() <= 3e-2 * qi.grad.abs().max() + 1e-3 + floor, (i, h)
 
 
 def _check_dv_checksum(v, go, hq):
