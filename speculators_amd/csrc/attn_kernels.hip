@@ -245,6 +245,14 @@ __device__ __forceinline__ void load_bounds(const AttnParams& p, const int (&ic)
   rb.blk_a2 = uni(rb.blk_a2); rb.blk_b2 = uni(rb.blk_b2);
 }
 
+// Passes a score block through an empty volatile asm statement.  Placed inside the branch that
+// masks a tile it keeps the compiler from turning that branch into selects which every tile, masked
+// or not, would then execute (96 vector instructions per tile): volatile asm is never speculated.
+__device__ __forceinline__ void pin_block(f32x16& a) {
+  asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]));
+  asm volatile("" : "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
+}
+
 // ---------------------------------------------------------------- forward
 // One workgroup = 4 waves = 4 * 32 * NSB query rows of one head.  With NSB = 2 a
 // wave owns two 32-row sub-blocks, so every K / V^T fragment read from LDS
@@ -286,6 +294,11 @@ struct FwdSmem {
   static constexpr int kBytes = kTiles + 4 * NW * (int)sizeof(int);
 };
 
+// operand fragments in flight per product (registers: 4 per fragment): the LDS pipe delivers
+// well over 150 B/clk per CU, what a wave waits for is the latency of its own reads
+#ifndef SPX_FWD_RING
+#define SPX_FWD_RING 8
+#endif
 template <int D, int NSB, int NW, int PF>
 __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_kernel(AttnParams p,
                                                                 const uint16_t* __restrict__ Vt,
@@ -478,25 +491,26 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
       // 32-key halves alternate so that consecutive MFMAs use different accumulators
       {
         constexpr int NF = 2 * NKK;
-        bf16x8 kfr[4];
+        constexpr int RG = SPX_FWD_RING;
+        bf16x8 kfr[RG];
         auto kread = [&](int f) {
           if constexpr (PF == 2)
-            kfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+            kfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 tk + (f & 1) * 32 * RBK + (rdk ^ ((f >> 1) * 32))));
           else
-            kfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+            kfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 &Ks[((f & 1) * 32 + col) * KS + g * 8 + (f >> 1) * 16]));
         };
 #pragma unroll
-        for (int f = 0; f < 4; ++f) kread(f);
+        for (int f = 0; f < RG; ++f) kread(f);
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int sb = 0; sb < NSB; ++sb)
-            st[sb][f & 1] = mfma32(kfr[f & 3], qf[sb][f >> 1], f < 2 ? nref[sb] : st[sb][f & 1]);
+            st[sb][f & 1] = mfma32(kfr[f % RG], qf[sb][f >> 1], f < 2 ? nref[sb] : st[sb][f & 1]);
           __builtin_amdgcn_sched_barrier(0);
-          if (f + 4 < NF) kread(f + 4);
+          if (f + RG < NF) kread(f + RG);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -511,15 +525,17 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         if (need_mask) {
           // a real (scalar) branch: the asm statement keeps the compiler from turning the
           // masking into selects that every tile would pay for
-          asm volatile("; masked tile");
 #pragma unroll
-          for (int kb = 0; kb < 2; ++kb)
+          for (int kb = 0; kb < 2; ++kb) {
+            pin_block(st[sb][kb]);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
               // key index = n0 + 4 g + (compile-time part): compare the constant part
               const int cr = kb * 32 + 8 * (r >> 2) + (r & 3);
               if (cr < m_lo[sb] || cr >= m_hi[sb]) st[sb][kb][r] = -INFINITY;
             }
+            pin_block(st[sb][kb]);
+          }
         }
         // st holds s - m_ref.  Largest of the 32 scores of this lane (three-operand maxima)
         float mx = fmaxf(st[sb][0][0], st[sb][1][0]);
@@ -563,17 +579,18 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
       {
         // V^T fragments through the same kind of ring; fragment f = (16-key step s, D block db)
         constexpr int NF = 4 * NDB;
-        bf16x8 vfr[4];
+        constexpr int RG = SPX_FWD_RING;
+        bf16x8 vfr[RG];
         auto vread = [&](int f) {
           if constexpr (PF == 2)
-            vfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+            vfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 tv + (f % NDB) * 32 * 128 + (rdv ^ ((f / NDB) * 32))));
           else
-            vfr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+            vfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 &Vs[((f % NDB) * 32 + col) * VS + (f / NDB) * 16 + 8 * g]));
         };
 #pragma unroll
-        for (int f = 0; f < 4; ++f) vread(f);
+        for (int f = 0; f < RG; ++f) vread(f);
         bf16x8 pb[NSB];
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
@@ -584,9 +601,9 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
           }
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int sb = 0; sb < NSB; ++sb) acc[sb][db] = mfma32(vfr[f & 3], pb[sb], acc[sb][db]);
+          for (int sb = 0; sb < NSB; ++sb) acc[sb][db] = mfma32(vfr[f % RG], pb[sb], acc[sb][db]);
           __builtin_amdgcn_sched_barrier(0);
-          if (f + 4 < NF) vread(f + 4);
+          if (f + RG < NF) vread(f + RG);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -603,32 +620,71 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
   for (int sb = 0; sb < NSB; ++sb) l_run[sb] = half_swap_sum(l_run[sb]);
   float (&m_run)[NSB] = m_ref;
 
-  // TTT diagonal keys (j, r), j = 1..n_extra: one dot product each
-  for (int j = 1; j <= p.n_extra; ++j) {
+  // TTT diagonal keys (j, r), j = 1..n_extra: one dot product each.  The key / value rows of a
+  // wave's 32 queries are 32 CONSECUTIVE rows of step j: they come in as whole 1 KB wave loads
+  // global -> LDS (a lane reading its own row from global memory touches 32 lines per instruction)
+  // into this wave's quarter of the tile buffers, chunk c of row r in slot c ^ (r mod chunks), and
+  // each lane then picks its row's pieces from LDS.  The loads of step j + 1 are issued as soon
+  // as step j's rows have been read.
+  if (p.n_extra > 0) {
+    static_assert(NSB == 1, "one 32-row block per wave");
+    constexpr int XCK = RBK / 16;                  // 16-byte chunks per row
+    constexpr int XRL = 1024 / RBK;                // rows per 1 KB wave load
+    constexpr int XNL = 32 / XRL;                  // wave loads per 32 rows
+    static_assert(SM::kTiles / NW >= 2 * 32 * RBK, "a wave's share of the tile buffers holds K and V rows");
+    __syncthreads();  // every wave is done with the tile buffers
+    const uint32_t xk = lds0 + wave * (2 * 32 * RBK), xv = xk + 32 * RBK;
+    const int64_t kv_bytes = (int64_t)(p.n_extra + 1) * p.T * RBK;
+    const u32x4 xkres = make_rsrc(p.K + (int64_t)kvh * p.k_hs, (uint32_t)kv_bytes);
+    const u32x4 xvres = make_rsrc(p.V + (int64_t)kvh * p.v_hs, (uint32_t)kv_bytes);
+    int goff[XNL];
 #pragma unroll
-    for (int sb = 0; sb < NSB; ++sb) {
-      const uint16_t* kj = p.K + (int64_t)kvh * p.k_hs + ((int64_t)j * p.T + ic[sb]) * D + g * 8;
+    for (int n = 0; n < XNL; ++n) {
+      const int r = n * XRL + lane / XCK;
+      goff[n] = r * RBK + (((lane % XCK) ^ (r & (XCK - 1))) * 16);
+    }
+    const int row0 = __builtin_amdgcn_readfirstlane(m0 + wave * BMW);
+    auto issue_x = [&](const u32x4& res, uint32_t dst, int j) __attribute__((always_inline)) {
+      const int soff = __builtin_amdgcn_readfirstlane((j * p.T + row0) * RBK);
+#pragma unroll
+      for (int n = 0; n < XNL; ++n) load_to_lds16<0>(res, dst + n * 1024, goff[n], soff);
+    };
+    const uint8_t* const xkp = fwd_smem + wave * (2 * 32 * RBK);
+    const uint8_t* const xvp = xkp + 32 * RBK;
+    const int xrow = col * RBK, xsw = col & (XCK - 1);
+    issue_x(xkres, xk, 1);
+    issue_x(xvres, xv, 1);
+    for (int j = 1; j <= p.n_extra; ++j) {
+      // K rows of step j have landed (the V rows, issued after them, may still be in flight)
+      if constexpr (XNL == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      else if constexpr (XNL == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
       float dot = 0.f;
 #pragma unroll
       for (int kk = 0; kk < NKK; ++kk)
-        dot = dot8_bf16(qf[sb][kk], *reinterpret_cast<const u32x4*>(kj + kk * 16), dot);
-      const float s = half_swap_sum(dot);  // the query fragments carry the scale
-      const float m_new = fmaxf(m_run[sb], s);
-      const float alpha = fast_exp2(m_run[sb] - m_new);  // a row without context keys: exp2(-inf) = 0
-      const float pv = fast_exp2(s - m_new);
-      l_run[sb] = l_run[sb] * alpha + pv;
-      m_run[sb] = m_new;
-      const uint16_t* vj = p.V + (int64_t)kvh * p.v_hs + ((int64_t)j * p.T + ic[sb]) * D + 4 * g;
+        dot = dot8_bf16(qf[0][kk], *reinterpret_cast<const u32x4*>(xkp + xrow + (((2 * kk + g) ^ xsw) * 16)), dot);
+      const float sj = half_swap_sum(dot);  // the query fragments carry the scale
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // V rows landed, K rows read
+      if (j < p.n_extra) issue_x(xkres, xk, j + 1);
+      const float m_new = fmaxf(m_run[0], sj);
+      const float alpha = fast_exp2(m_run[0] - m_new);  // a row without context keys: exp2(-inf) = 0
+      const float pv = fast_exp2(sj - m_new);
+      l_run[0] = l_run[0] * alpha + pv;
+      m_run[0] = m_new;
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
           float vv[4];
-          unpack4(*reinterpret_cast<const u32x2*>(vj + db * 32 + 8 * r4), vv);
+          unpack4(*reinterpret_cast<const u32x2*>(xvp + xrow + (((db * 4 + r4) ^ xsw) * 16) + 8 * g), vv);
 #pragma unroll
           for (int t = 0; t < 4; ++t)
-            acc[sb][db][r4 * 4 + t] = fmaf(pv, vv[t], acc[sb][db][r4 * 4 + t] * alpha);
+            acc[0][db][r4 * 4 + t] = fmaf(pv, vv[t], acc[0][db][r4 * 4 + t] * alpha);
         }
+      if (j < p.n_extra) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // V rows read
+        issue_x(xvres, xv, j + 1);
+      }
     }
   }
 
@@ -957,13 +1013,14 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
           for (int r = 0; r < 16; ++r) st[r] = fast_exp2(st[r]);
           if (need_mask) {
             // a real (scalar) branch, see the forward kernel
-            asm volatile("; masked tile");
             const int lo = aa[sb] - n0 - 4 * g, hi = bb[sb] - n0 - 4 * g;
+            pin_block(st);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
               const int cr = kb * 32 + 8 * (r >> 2) + (r & 3);
               if (cr < lo || cr >= hi) st[r] = 0.f;
             }
+            pin_block(st);
           }
 #pragma unroll
           for (int r = 0; r < 16; ++r) dp[r] *= st[r];
@@ -1103,6 +1160,17 @@ struct DkvSmem {
   static constexpr int kBytes = (2 * 64 * (D + kKPad) + 2 * D * (64 + kVPad)) * 2 + kSmall;
 };
 
+// operand fragments in flight per product in the dK/dV kernel (one wave per SIMD: nothing else
+// hides the latency of its LDS reads)
+#ifndef SPX_DKV_RING
+#define SPX_DKV_RING 8
+#endif
+#ifndef SPX_DKV_PIPE
+#define SPX_DKV_PIPE 0
+#endif
+#ifndef SPX_DKV_PRING
+#define SPX_DKV_PRING 4
+#endif
 template <int D, int NW, int PF, int PASS>
 __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     AttnParams p, const uint16_t* __restrict__ dO, const uint16_t* __restrict__ Qt,
@@ -1359,7 +1427,9 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (have_next) {
+#ifndef SPX_EXP_NODMA
         issue(nxt * 64 + nsub * QT, buf ^ 1);
+#endif
         if (nsub == 0) small_fetch(nxt * 64);
       }
       tile = sm8 + buf * SM::kBuf;
@@ -1377,6 +1447,95 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     const int sub_now = sub;
     qi = nxi;
     sub = nsub;
+
+    // ---- fully visible 64-row tile, both gradients in one pass: the two 32-row halves are software
+    // pipelined inside the wave (one wave per SIMD: nothing else would overlap the two pipes).
+    //   A: scores / dP of half 0               (16 MFMAs)
+    //   B: scores / dP of half 1               (16 MFMAs)  with the exp2 / dS arithmetic of half 0 between them
+    //   C: dV / dK contributions of half 0     (16 MFMAs)  with the arithmetic of half 1 between them
+    //   D: dV / dK contributions of half 1     (16 MFMAs)
+    // The arithmetic of one accumulator slot (two register moves, exp2, multiply) is issued behind each
+    // MFMA of the neighbouring stage, so the matrix pipe never waits for the vector pipe.
+    if constexpr (SPX_DKV_PIPE && kDma && NQB == 2 && kDoK && kDoV) {
+      if (full) {
+        constexpr int RG = SPX_DKV_PRING;
+        f32x16 st2[2], dp2[2];
+        auto cinit = [&](int qbl) __attribute__((always_inline)) {
+          const int qb = sub_now * NQB + qbl;
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const int q0 = qb * 32 + 8 * r4 + 4 * g;
+            const f32x4 ls = *reinterpret_cast<const f32x4*>(&lse_s[q0]);
+            const f32x4 dl = *reinterpret_cast<const f32x4*>(&delta_s[q0]);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) { st2[qbl][r4 * 4 + t] = ls[t]; dp2[qbl][r4 * 4 + t] = dl[t]; }
+          }
+        };
+        // exp2 and dS of accumulator slot r of half q
+        auto arith = [&](int q, int r) __attribute__((always_inline)) {
+          const float pr = fast_exp2(st2[q][r]);
+          st2[q][r] = pr;
+          dp2[q][r] *= pr;
+        };
+        // scores and dP of half qbl; `hook(f)` is issued behind MFMA f
+        auto chain1 = [&](int qbl, auto&& hook) __attribute__((always_inline)) {
+          constexpr int NF = 2 * NKK;
+          bf16x8 fr[RG];
+          auto fread = [&](int f) {
+            const uint8_t* base = tile + ((f & 1) ? SM::kOffdO : 0);
+            fr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                base + qbl * 32 * RBQ + (rdr ^ ((f / 2) * 32))));
+          };
+#pragma unroll
+          for (int f = 0; f < RG && f < NF; ++f) fread(f);
+#pragma unroll
+          for (int f = 0; f < NF; ++f) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (f & 1) dp2[qbl] = mfma32(fr[f % RG], vf[(f / 2) % NVF], dp2[qbl]);
+            else st2[qbl] = mfma32(fr[f % RG], kf[f / 2], st2[qbl]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (f + RG < NF) fread(f + RG);
+            hook(f);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        // dV / dK contributions of half qbl from its packed P and dS
+        auto chain2 = [&](int qbl, const bf16x8 (&pb)[2], const bf16x8 (&sb)[2], auto&& hook)
+            __attribute__((always_inline)) {
+          constexpr int NF = 2 * 2 * NDB;
+          bf16x8 fr[RG];
+          auto fread = [&](int f) {
+            const int e = f / 2, s2 = e / NDB, db = e % NDB;
+            const uint8_t* base = tile + ((f & 1) ? SM::kOffQt : SM::kOffdOt);
+            fr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                base + db * 32 * RBT + (rdt ^ ((qbl * 2 + s2) * 32))));
+          };
+#pragma unroll
+          for (int f = 0; f < RG && f < NF; ++f) fread(f);
+#pragma unroll
+          for (int f = 0; f < NF; ++f) {
+            const int e = f / 2, s2 = e / NDB, db = e % NDB;
+            __builtin_amdgcn_sched_barrier(0);
+            if (f & 1) acc_dk[db % NAK] = mfma32(fr[f % RG], sb[s2], acc_dk[db % NAK]);
+            else acc_dv[db % NAV] = mfma32(fr[f % RG], pb[s2], acc_dv[db % NAV]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (f + RG < NF) fread(f + RG);
+            hook(f);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        auto nothing = [](int) {};
+        cinit(0);
+        cinit(1);
+        chain1(0, nothing);
+        chain1(1, [&](int f) { arith(0, f); });
+        bf16x8 pb0[2] = {pack8(st2[0], 0), pack8(st2[0], 8)}, sb0[2] = {pack8(dp2[0], 0), pack8(dp2[0], 8)};
+        chain2(0, pb0, sb0, [&](int f) { arith(1, f); });
+        bf16x8 pb1[2] = {pack8(st2[1], 0), pack8(st2[1], 8)}, sb1[2] = {pack8(dp2[1], 0), pack8(dp2[1], 8)};
+        chain2(1, pb1, sb1, nothing);
+        goto tile_done;
+      }
+    }
 
     // the two 32-row halves of the query tile one after the other (keeps 32 score
     // registers live instead of 64)
@@ -1407,27 +1566,28 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         // fragment f + 4 follows the MFMA of fragment f, so no MFMA waits for LDS
         constexpr int PER = kDoK ? 2 : 1;  // fragments per K step: Q [, dO]
         constexpr int NF = PER * NKK;
-        bf16x8 fr[4];
+        constexpr int RG = SPX_DKV_RING;
+        bf16x8 fr[RG];
         auto fread = [&](int f) {
           if constexpr (kDma) {
             const uint8_t* base = tile + ((PER == 2 && (f & 1)) ? SM::kOffdO : 0);
-            fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+            fr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 base + qbl * 32 * RBQ + (rdr ^ ((f / PER) * 32))));
           } else {
             const uint16_t* base = (PER == 2 && (f & 1)) ? dOs : Qs;
-            fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+            fr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 &base[(qb * 32 + col) * QS + g * 8 + (f / PER) * 16]));
           }
         };
 #pragma unroll
-        for (int f = 0; f < 4; ++f) fread(f);
+        for (int f = 0; f < RG && f < NF; ++f) fread(f);
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
           __builtin_amdgcn_sched_barrier(0);
-          if (PER == 2 && (f & 1)) dp = mfma32(fr[f & 3], vf[(f / PER) % NVF], dp);
-          else st = mfma32(fr[f & 3], kf[f / PER], st);
+          if (PER == 2 && (f & 1)) dp = mfma32(fr[f % RG], vf[(f / PER) % NVF], dp);
+          else st = mfma32(fr[f % RG], kf[f / PER], st);
           __builtin_amdgcn_sched_barrier(0);
-          if (f + 4 < NF) fread(f + 4);
+          if (f + RG < NF) fread(f + RG);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -1435,8 +1595,8 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       for (int r = 0; r < 16; ++r) st[r] = fast_exp2(st[r]);
       if (!full) {
         // a real (scalar) branch: only tiles that straddle an interval edge pay for the mask
-        asm volatile("; masked tile");
         typedef __attribute__((ext_vector_type(4))) int i32x4;
+        pin_block(st);
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
           const int q0 = qb * 32 + 8 * r4 + 4 * g;
@@ -1450,6 +1610,7 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
             if (!ok) st[r4 * 4 + t] = 0.f;
           }
         }
+        pin_block(st);
       }
       if (kDoK) {
 #pragma unroll
@@ -1460,22 +1621,23 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         // dO^T [, Q^T]
         constexpr int PER = (kDoV ? 1 : 0) + (kDoK ? 1 : 0);
         constexpr int NF = PER * 2 * NDB;
-        bf16x8 fr[4];
+        constexpr int RG = SPX_DKV_RING;
+        bf16x8 fr[RG];
         auto fread = [&](int f) {
           const int e = f / PER, s2 = e / NDB, db = e % NDB;
           const bool is_q = kDoK && (!kDoV || (f % PER) == 1);
           if constexpr (kDma) {
             const uint8_t* base = tile + (is_q ? SM::kOffQt : SM::kOffdOt);
-            fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+            fr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 base + db * 32 * RBT + (rdt ^ ((qbl * 2 + s2) * 32))));
           } else {
             const uint16_t* base = is_q ? Qts : dOts;
-            fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+            fr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 &base[(db * 32 + col) * TS + (qb * 2 + s2) * 16 + 8 * g]));
           }
         };
 #pragma unroll
-        for (int f = 0; f < 4; ++f) fread(f);
+        for (int f = 0; f < RG && f < NF; ++f) fread(f);
         bf16x8 pb = pack8(st, 0), sb8 = pack8(dp, 0);
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
@@ -1483,15 +1645,16 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
           const bool is_q = kDoK && (!kDoV || (f % PER) == 1);
           if (f == PER * NDB) { pb = pack8(st, 8); sb8 = pack8(dp, 8); }
           __builtin_amdgcn_sched_barrier(0);
-          if (is_q) acc_dk[db % NAK] = mfma32(fr[f & 3], sb8, acc_dk[db % NAK]);
-          else acc_dv[db % NAV] = mfma32(fr[f & 3], pb, acc_dv[db % NAV]);
+          if (is_q) acc_dk[db % NAK] = mfma32(fr[f % RG], sb8, acc_dk[db % NAK]);
+          else acc_dv[db % NAV] = mfma32(fr[f % RG], pb, acc_dv[db % NAV]);
           __builtin_amdgcn_sched_barrier(0);
-          if (f + 4 < NF) fread(f + 4);
+          if (f + RG < NF) fread(f + RG);
           (void)s2;
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+  tile_done:
     if constexpr (kDma) {
       // the per-row scalars of the next 64-row step go into the other set: nobody reads it before the
       // barrier
