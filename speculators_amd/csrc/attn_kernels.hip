@@ -786,7 +786,9 @@ struct DqSmem {
   static constexpr int KS = D + kKPad, VS = kBN + kVPad;
   static constexpr int kTileK = TB * D * 2, kTileT = D * TB * 2;     // mode 3: unpadded, swizzled
   static constexpr int kBuf = 2 * kTileK + kTileT;
-  static constexpr int kTiles = PF == 3 ? 2 * kBuf : (2 * kBN * KS + D * VS) * 2;
+  static constexpr int kDiag = NW * 2 * 32 * D * 2;  // K and V rows of 32 queries per wave (TTT diagonal keys)
+  static constexpr int kTiles0 = PF == 3 ? 2 * kBuf : (2 * kBN * KS + D * VS) * 2;
+  static constexpr int kTiles = kTiles0 > kDiag ? kTiles0 : kDiag;
   static constexpr int kBytes = kTiles + 4 * NW * (int)sizeof(int);
 };
 
@@ -1060,30 +1062,56 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
   if (p.a2)
     run_pass(rb.a2, rb.b2, rb.w_a2min, rb.w_a2max, rb.w_b2min, rb.w_b2max, rb.blk_a2, rb.blk_b2);
 
-  for (int j = 1; j <= p.n_extra; ++j) {
+  // TTT diagonal keys: the key / value rows of a wave's 32 queries come in as coalesced 1 KB wave
+  // loads global -> LDS into the wave's share of the tile buffers (see the forward kernel)
+  if (p.n_extra > 0) {
+    static_assert(NSB == 1, "one 32-row block per wave");
+    constexpr int XCK = RBK / 16, XRL = 1024 / RBK, XNL = 32 / XRL;
+    __syncthreads();  // every wave is done with the tile buffers
+    const uint32_t xk = lds0 + wave * (2 * 32 * RBK), xv = xk + 32 * RBK;
+    const int64_t kv_bytes = (int64_t)(p.n_extra + 1) * p.T * RBK;
+    const u32x4 xkres = make_rsrc(Kh, (uint32_t)kv_bytes);
+    const u32x4 xvres = make_rsrc(Vh, (uint32_t)kv_bytes);
+    int goff[XNL];
 #pragma unroll
-    for (int sb = 0; sb < NSB; ++sb) {
-      const uint16_t* kj = p.K + (int64_t)kvh * p.k_hs + ((int64_t)j * p.T + ic[sb]) * D;
-      const uint16_t* vj = p.V + (int64_t)kvh * p.v_hs + ((int64_t)j * p.T + ic[sb]) * D;
+    for (int n = 0; n < XNL; ++n) {
+      const int r = n * XRL + lane / XCK;
+      goff[n] = r * RBK + (((lane % XCK) ^ (r & (XCK - 1))) * 16);
+    }
+    const int row0 = __builtin_amdgcn_readfirstlane(m0 + wave * BMW);
+    auto issue_x = [&](const u32x4& res, uint32_t dst, int j) __attribute__((always_inline)) {
+      const int soff = __builtin_amdgcn_readfirstlane((j * p.T + row0) * RBK);
+#pragma unroll
+      for (int n = 0; n < XNL; ++n) load_to_lds16<0>(res, dst + n * 1024, goff[n], soff);
+    };
+    const uint8_t* const xkp = dq_smem + wave * (2 * 32 * RBK);
+    const uint8_t* const xvp = xkp + 32 * RBK;
+    const int xrow = col * RBK, xsw = col & (XCK - 1);
+    for (int j = 1; j <= p.n_extra; ++j) {
+      issue_x(xkres, xk, j);
+      issue_x(xvres, xv, j);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       float dot = 0.f, dpv = 0.f;
 #pragma unroll
       for (int kk = 0; kk < NKK; ++kk) {
-        dot = dot8_bf16(qf[sb][kk], *reinterpret_cast<const u32x4*>(kj + g * 8 + kk * 16), dot);
-        dpv = dot8_bf16(dof[sb][kk], *reinterpret_cast<const u32x4*>(vj + g * 8 + kk * 16), dpv);
+        const int o = xrow + (((2 * kk + g) ^ xsw) * 16);
+        dot = dot8_bf16(qf[0][kk], *reinterpret_cast<const u32x4*>(xkp + o), dot);
+        dpv = dot8_bf16(dof[0][kk], *reinterpret_cast<const u32x4*>(xvp + o), dpv);
       }
       dot = half_swap_sum(dot);
       dpv = half_swap_sum(dpv);
-      const float pv = fast_exp2(dot - lse_i[sb]);  // the query fragments carry the scale
-      const float ds = pv * (dpv - delta_i[sb]);
+      const float pv = fast_exp2(dot - lse_i[0]);  // the query fragments carry the scale
+      const float ds = pv * (dpv - delta_i[0]);
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
           float kk4[4];
-          unpack4(*reinterpret_cast<const u32x2*>(kj + 4 * g + db * 32 + 8 * r4), kk4);
+          unpack4(*reinterpret_cast<const u32x2*>(xkp + xrow + (((db * 4 + r4) ^ xsw) * 16) + 8 * g), kk4);
 #pragma unroll
-          for (int t = 0; t < 4; ++t) acc[sb][db][r4 * 4 + t] = fmaf(ds, kk4[t], acc[sb][db][r4 * 4 + t]);
+          for (int t = 0; t < 4; ++t) acc[0][db][r4 * 4 + t] = fmaf(ds, kk4[t], acc[0][db][r4 * 4 + t]);
         }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // rows read before the next step overwrites them
     }
   }
 
