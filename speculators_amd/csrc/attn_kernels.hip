@@ -151,6 +151,7 @@ __global__ __launch_bounds__(64) void transpose_bf16_kernel(
         *reinterpret_cast<u32x4*>(scaled + ((int64_t)h * rows + r0 + j) * cols + c0) = in[j];
     }
   }
+  if (SCALED && dst == nullptr) return;  // only the scaled row-major copy is wanted
   // where the block's two halves go: r0 % 16 == 0 -> r0 and r0 + 8, r0 % 16 == 8 -> r0 - 4 and r0 + 4
   const int p_lo = (r0 & 8) ? r0 - 4 : r0, p_hi = (r0 & 8) ? r0 + 4 : r0 + 8;
   uint16_t* d = dst + (int64_t)h * dst_hs + (int64_t)c0 * ld_dst;
@@ -755,10 +756,17 @@ __device__ __forceinline__ void st_bf16s(uint16_t* p, const float (&v)[EPL]) {
   }
 }
 
+__global__ __launch_bounds__(256) void fill_zero_kernel(float* __restrict__ x, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x[i] = 0.f;
+}
+
 template <int D>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const uint16_t* __restrict__ O,
                                                          const uint16_t* __restrict__ dO, int NQ,
-                                                         int Hq, float* __restrict__ delta) {
+                                                         int Hq, float* __restrict__ delta,
+                                                         const float* __restrict__ lse, int NQp,
+                                                         float* __restrict__ neg) {
   // sixteen lanes per (row, head): D / 16 consecutive elements each, summed with DPP moves
   constexpr int EPL = D / 16;
   const int64_t n_rows = (int64_t)NQ * Hq;
@@ -772,7 +780,14 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const uint16_t* __restr
 #pragma unroll
   for (int e = 0; e < EPL; ++e) acc = fmaf(a[e], b[e], acc);
   acc = row16_sum(acc);
-  if ((threadIdx.x & 15) == 0 && raw < n_rows) delta[(row % Hq) * (int64_t)NQ + row / Hq] = acc;
+  if ((threadIdx.x & 15) == 0 && raw < n_rows) {
+    const int64_t hh = row % Hq, i = row / Hq;
+    delta[hh * NQ + i] = acc;
+    // -lse and -delta in rows of NQp (the padding stays zero: see the launcher), the C operands of the
+    // wave-specialised dK/dV kernel's score products
+    neg[hh * NQp + i] = -lse[hh * NQ + i];
+    neg[((int64_t)Hq + hh) * NQp + i] = -acc;
+  }
 }
 
 // dQ: same tiling as the forward.
@@ -1133,7 +1148,10 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
 
 // per 64-row query tile: min / max of the interval ends of both classes (for the dK/dV
 // tile loop): [a1min, a1max, b1min, b1max, a2min, a2max, b2min, b2max]
-__global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int32_t* __restrict__ tb) {
+// rows[4][NQp] (NQp a multiple of 64): the interval ends of every row as the kernels compare them
+// (a1, b1, T + a2, T + b2; an empty interval where a class is absent or the row is padding)
+__global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int32_t* __restrict__ tb,
+                                                              int NQp, int32_t* __restrict__ rows) {
   const int tile = blockIdx.x;
   const int r = tile * 64 + threadIdx.x;
   const bool ok = r < p.NQ;
@@ -1141,9 +1159,12 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
   const int b1 = ok ? (p.b1 ? p.b1[r] : r + 1) : 0;
   const int a2 = (ok && p.a2) ? p.T + p.a2[r] : 0x7fffffff;
   const int b2 = (ok && p.a2) ? p.T + p.b2[r] : 0;
+  if (r < NQp) {
+    rows[r] = a1; rows[NQp + r] = b1; rows[2 * (int64_t)NQp + r] = a2; rows[3 * (int64_t)NQp + r] = b2;
+  }
   const int v[8] = {wave_min_i(a1), wave_max_i(a1), wave_min_i(b1), wave_max_i(b1),
                     wave_min_i(a2), wave_max_i(a2), wave_min_i(b2), wave_max_i(b2)};
-  if (threadIdx.x == 0) {
+  if (threadIdx.x == 0 && tile * 64 < p.NQ) {
 #pragma unroll
     for (int k = 0; k < 8; ++k) tb[tile * 8 + k] = v[k];
   }
@@ -1192,12 +1213,6 @@ struct DkvSmem {
 // hides the latency of its LDS reads)
 #ifndef SPX_DKV_RING
 #define SPX_DKV_RING 8
-#endif
-#ifndef SPX_DKV_PIPE
-#define SPX_DKV_PIPE 0
-#endif
-#ifndef SPX_DKV_PRING
-#define SPX_DKV_PRING 4
 #endif
 template <int D, int NW, int PF, int PASS>
 __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
@@ -1455,9 +1470,7 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (have_next) {
-#ifndef SPX_EXP_NODMA
         issue(nxt * 64 + nsub * QT, buf ^ 1);
-#endif
         if (nsub == 0) small_fetch(nxt * 64);
       }
       tile = sm8 + buf * SM::kBuf;
@@ -1475,95 +1488,6 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     const int sub_now = sub;
     qi = nxi;
     sub = nsub;
-
-    // ---- fully visible 64-row tile, both gradients in one pass: the two 32-row halves are software
-    // pipelined inside the wave (one wave per SIMD: nothing else would overlap the two pipes).
-    //   A: scores / dP of half 0               (16 MFMAs)
-    //   B: scores / dP of half 1               (16 MFMAs)  with the exp2 / dS arithmetic of half 0 between them
-    //   C: dV / dK contributions of half 0     (16 MFMAs)  with the arithmetic of half 1 between them
-    //   D: dV / dK contributions of half 1     (16 MFMAs)
-    // The arithmetic of one accumulator slot (two register moves, exp2, multiply) is issued behind each
-    // MFMA of the neighbouring stage, so the matrix pipe never waits for the vector pipe.
-    if constexpr (SPX_DKV_PIPE && kDma && NQB == 2 && kDoK && kDoV) {
-      if (full) {
-        constexpr int RG = SPX_DKV_PRING;
-        f32x16 st2[2], dp2[2];
-        auto cinit = [&](int qbl) __attribute__((always_inline)) {
-          const int qb = sub_now * NQB + qbl;
-#pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4) {
-            const int q0 = qb * 32 + 8 * r4 + 4 * g;
-            const f32x4 ls = *reinterpret_cast<const f32x4*>(&lse_s[q0]);
-            const f32x4 dl = *reinterpret_cast<const f32x4*>(&delta_s[q0]);
-#pragma unroll
-            for (int t = 0; t < 4; ++t) { st2[qbl][r4 * 4 + t] = ls[t]; dp2[qbl][r4 * 4 + t] = dl[t]; }
-          }
-        };
-        // exp2 and dS of accumulator slot r of half q
-        auto arith = [&](int q, int r) __attribute__((always_inline)) {
-          const float pr = fast_exp2(st2[q][r]);
-          st2[q][r] = pr;
-          dp2[q][r] *= pr;
-        };
-        // scores and dP of half qbl; `hook(f)` is issued behind MFMA f
-        auto chain1 = [&](int qbl, auto&& hook) __attribute__((always_inline)) {
-          constexpr int NF = 2 * NKK;
-          bf16x8 fr[RG];
-          auto fread = [&](int f) {
-            const uint8_t* base = tile + ((f & 1) ? SM::kOffdO : 0);
-            fr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-                base + qbl * 32 * RBQ + (rdr ^ ((f / 2) * 32))));
-          };
-#pragma unroll
-          for (int f = 0; f < RG && f < NF; ++f) fread(f);
-#pragma unroll
-          for (int f = 0; f < NF; ++f) {
-            __builtin_amdgcn_sched_barrier(0);
-            if (f & 1) dp2[qbl] = mfma32(fr[f % RG], vf[(f / 2) % NVF], dp2[qbl]);
-            else st2[qbl] = mfma32(fr[f % RG], kf[f / 2], st2[qbl]);
-            __builtin_amdgcn_sched_barrier(0);
-            if (f + RG < NF) fread(f + RG);
-            hook(f);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        };
-        // dV / dK contributions of half qbl from its packed P and dS
-        auto chain2 = [&](int qbl, const bf16x8 (&pb)[2], const bf16x8 (&sb)[2], auto&& hook)
-            __attribute__((always_inline)) {
-          constexpr int NF = 2 * 2 * NDB;
-          bf16x8 fr[RG];
-          auto fread = [&](int f) {
-            const int e = f / 2, s2 = e / NDB, db = e % NDB;
-            const uint8_t* base = tile + ((f & 1) ? SM::kOffQt : SM::kOffdOt);
-            fr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-                base + db * 32 * RBT + (rdt ^ ((qbl * 2 + s2) * 32))));
-          };
-#pragma unroll
-          for (int f = 0; f < RG && f < NF; ++f) fread(f);
-#pragma unroll
-          for (int f = 0; f < NF; ++f) {
-            const int e = f / 2, s2 = e / NDB, db = e % NDB;
-            __builtin_amdgcn_sched_barrier(0);
-            if (f & 1) acc_dk[db % NAK] = mfma32(fr[f % RG], sb[s2], acc_dk[db % NAK]);
-            else acc_dv[db % NAV] = mfma32(fr[f % RG], pb[s2], acc_dv[db % NAV]);
-            __builtin_amdgcn_sched_barrier(0);
-            if (f + RG < NF) fread(f + RG);
-            hook(f);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        };
-        auto nothing = [](int) {};
-        cinit(0);
-        cinit(1);
-        chain1(0, nothing);
-        chain1(1, [&](int f) { arith(0, f); });
-        bf16x8 pb0[2] = {pack8(st2[0], 0), pack8(st2[0], 8)}, sb0[2] = {pack8(dp2[0], 0), pack8(dp2[0], 8)};
-        chain2(0, pb0, sb0, [&](int f) { arith(1, f); });
-        bf16x8 pb1[2] = {pack8(st2[1], 0), pack8(st2[1], 8)}, sb1[2] = {pack8(dp2[1], 0), pack8(dp2[1], 8)};
-        chain2(1, pb1, sb1, nothing);
-        goto tile_done;
-      }
-    }
 
     // the two 32-row halves of the query tile one after the other (keeps 32 score
     // registers live instead of 64)
@@ -1682,7 +1606,6 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-  tile_done:
     if constexpr (kDma) {
       // the per-row scalars of the next 64-row step go into the other set: nobody reads it before the
       // barrier
@@ -1717,6 +1640,494 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         }
       }
   }
+}
+
+#ifndef SPX_DKV_WS
+#define SPX_DKV_WS 1
+#endif
+// ---------------------------------------------------------------- dK / dV, wave-specialised
+// The work of attn_bwd_dkv_kernel for head_dim <= 128 (both gradients in one pass), split over
+// TWO waves per SIMD that run different halves of it, so that each SIMD has a wave for the matrix
+// pipe while the other is in its vector phase, and every MFMA works on plain vector registers:
+//   producer wave i (waves 0-3): keeps K / V fragments of its 32 keys; per 32-row query tile
+//     S = Q' K^T - lse and dP = dO V^T - delta (16 MFMAs at head_dim 128), P = exp2(S), dS = P dP,
+//     both rounded to bf16 in the B-operand layout and handed over through a 4 KB LDS slot;
+//   consumer wave i (waves 4-7, same SIMD): keeps the dK / dV accumulators of those 32 keys
+//     (128 registers); per tile dV^T += dO^T P and dK^T += Q'^T dS (16 MFMAs) from the slot.
+// Both roles read the SAME row-major query tile (32 rows of Q' and of dO): the consumers take
+// their A operands (dO^T, Q'^T fragments) with transposing LDS reads (ds_read_b64_tr_b16), so no
+// transposed copy of the queries exists in memory.  Everything a step needs comes global -> LDS
+// directly, kAhead tiles ahead, into a ring of kStages buffers: the tile, and the per-row scalars
+// (-lse, -delta: the C operands of the score products; the mask interval ends).  In step b the
+// producers turn the scores of tile b (computed one step earlier) into P and dS first, while the
+// consumers' MFMAs of tile b - 1 run, and compute the scores of tile b + 1 after that.  One
+// workgroup barrier per step; slots are double buffered.
+template <int D>
+struct DkvWsSmem {
+  static constexpr int kStages = 6;
+  static constexpr int kAhead = 4;                     // tile b + kAhead is issued in step b
+  static constexpr int kTile = 2 * 32 * D * 2;         // Q', dO: 32 rows of D each
+  static constexpr int kSlot = 16 * 64 * 4;            // 16 registers of 64 lanes
+  static constexpr int kOffSlot = kStages * kTile;
+  static constexpr int kOffSmall = kOffSlot + 4 * 2 * kSlot;
+  static constexpr int kSmall = 6 * 32 * 4;            // -lse, -delta, a1, b1, a2, b2 of 32 rows
+  static constexpr int kSets = 8;                      // sets of per-row scalars (tile k: set k % 8)
+  static constexpr int kOffList = kOffSmall + kSets * kSmall + 256;  // (+ a spare area)
+  static constexpr int kListCap = 2048;                // visible 64-row tiles per key block, at most
+  static constexpr int kList = (kListCap + 1) * 4;     // ... their list, closed by an end mark
+  static constexpr int kBytes = kOffList + 2 * kList + 64;  // two key blocks; scratch of the list builder
+  static constexpr uint32_t kListEnd = 0x7fffffffu;
+  static_assert(kStages >= kAhead + 2, "a buffer is free two steps after its tile's scores");
+};
+
+// Values a non-inlined device function receives arrive in vector registers; these make them
+// wave-uniform (scalar registers) again, which addresses of the global -> LDS loads must be.
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+template <typename T>
+__device__ __forceinline__ T* uni(T* q) {
+  const uint64_t a = reinterpret_cast<uint64_t>(q);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return reinterpret_cast<T*>(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ int64_t uni(int64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+#ifdef SPX_WS_TIMING
+__device__ unsigned long long g_ws_dbg[128 * 16];
+extern "C" int spx_debug_ws_timing(unsigned long long* host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_ws_dbg), sizeof(g_ws_dbg));
+}
+#endif
+
+// Four 16-bit values per lane from LDS, transposed inside every group of 16 lanes: lane 4u + w of
+// a group receives, as element j, element w of the 8 bytes that lane 4j + u of the group points at.
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ i16x4 lds_read_tr16(const uint8_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) i16x4*)(uintptr_t)(uint32_t)(uintptr_t)(
+          (__attribute__((address_space(3))) const uint8_t*)p));
+}
+
+// One role of the kernel as a function of its own (not inlined): the register allocation of the
+// producers (K / V fragments, scores) and of the consumers (128 accumulator registers) then do not
+// add up.  Both roles walk the same sequence of steps and meet at the same barriers.
+template <int D, bool PRODUCER>
+__device__ __attribute__((noinline)) void dkv_ws_role(
+    const AttnParams& p_in, const uint16_t* dO_in, int NQp_in, const float* neg_in,
+    const int32_t* mrows_in, float* dKp_in, float* dVp_in) {
+  using SM = DkvWsSmem<D>;
+  extern __shared__ __attribute__((aligned(16))) uint8_t ws_smem[];
+  AttnParams p;
+  p.Q = uni(p_in.Q); p.q_hs = uni(p_in.q_hs);
+  p.K = uni(p_in.K); p.k_hs = uni(p_in.k_hs);
+  p.V = uni(p_in.V); p.v_hs = uni(p_in.v_hs);
+  p.a1 = nullptr; p.b1 = nullptr; p.a2 = nullptr; p.b2 = nullptr;
+  p.NQ = uni(p_in.NQ); p.T = uni(p_in.T); p.NKV = uni(p_in.NKV); p.NKVp = uni(p_in.NKVp);
+  p.n_extra = uni(p_in.n_extra); p.Hq = uni(p_in.Hq); p.Hkv = uni(p_in.Hkv);
+  p.scale_log2e = p_in.scale_log2e; p.scaling = p_in.scaling;
+  const uint16_t* __restrict__ dO = uni(dO_in);
+  const int NQp = uni(NQp_in);
+  const float* __restrict__ neg = uni(neg_in);        // -lse [Hq][NQp], -delta [Hq][NQp]
+  const int32_t* __restrict__ mrows = uni(mrows_in);  // interval ends of every row, [4][NQp]
+  float* __restrict__ dKp = uni(dKp_in);
+  float* __restrict__ dVp = uni(dVp_in);
+
+  constexpr bool producer = PRODUCER;
+  constexpr int NKK = D / 16, NDB = D / 32;
+  constexpr int KB = 128;                                 // keys per workgroup
+  constexpr int RBQ = D * 2, CKQ = RBQ / 16;              // bytes / 16-byte chunks per row of Q' and dO
+  constexpr int NLQ = 32 * RBQ / 1024;                    // 1 KB wave loads per 32-row operand
+  constexpr int LPW = 2 * NLQ / 8;                        // tile loads per wave
+  constexpr int kLoads = LPW + 1;                         // ... plus one of per-row scalars
+  constexpr int RG = 4;
+  constexpr int NS = SM::kStages, AH = SM::kAhead;
+  static_assert(LPW >= 1 && 2 * NLQ % 8 == 0, "every wave issues the same number of loads per tile");
+  // A workgroup takes key blocks i and n_kb - 1 - i of one head, one after the other: under a causal
+  // mask block i is seen by all later query tiles and its partner by correspondingly few, so every
+  // workgroup walks about the same number of tiles.
+  const int n_kb = (p.NKV + KB - 1) / KB, n_pair = (n_kb + 1) / 2;
+  int h, pair;
+  if (SPX_DKV_XCD && p.Hq % 8 == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    h = xcd + 8 * (slot / n_pair);
+    pair = slot % n_pair;
+  } else {
+    h = blockIdx.x % p.Hq;
+    pair = blockIdx.x / p.Hq;
+  }
+  const int kvh = h / (p.Hq / p.Hkv);
+  for (int part = 0; part < 2; ++part) {
+  const int kb_idx = part == 0 ? pair : n_kb - 1 - pair;
+  if (part == 1) {
+    if (kb_idx == pair) break;   // the middle block of an odd count has no partner
+    __syncthreads();             // everybody is done with the ring, the slots and the sets
+  }
+  const int n0 = kb_idx * KB;
+  const int key_last = min(n0 + KB - 1, p.NKV - 1);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6);
+  const int pw = wave & 3;                 // pair index: the 32 keys of this wave
+  const int g = lane >> 5, col = lane & 31;
+  const int c = n0 + pw * 32 + col;
+  const int cc = c < p.NKV ? c : p.NKV - 1;
+  const int n_qt = (p.NQ + 63) / 64;
+
+  // the steps: the two 32-row halves of every 64-row query tile that sees the block, in order.  The
+  // kernel has listed those tiles in LDS (bit 31: every key of the block is visible to all rows of the
+  // tile); step k is half k & 1 of list entry k / 2.
+  const uint32_t* const lst = reinterpret_cast<const uint32_t*>(ws_smem + SM::kOffList + part * SM::kList);
+  const int s_end = n_qt * 2;
+  auto step_of = [&](uint32_t e, int k_) { return (e & 0x7fffffffu) == SM::kListEnd ? s_end : (int)(e & 0x7fffffffu) * 2 + (k_ & 1); };
+  const int n_vis = uni(reinterpret_cast<const int*>(ws_smem + SM::kOffList + 2 * SM::kList)[8 + part]);
+  auto entry = [&](int k_) { return lst[min(k_ >> 1, n_vis)]; };
+
+  // position of 16-byte chunk c of row r inside its LDS row: c ^ swz_r(r).  Row-wise 16-byte reads of 32
+  // rows (the producers) and the transposing reads of 4 + 4 rows x 64 bytes (the consumers) both
+  // spread evenly over the banks.
+  auto swz_r = [](int r) {
+    return CKQ == 8 ? ((r & 4) | ((r >> 2) & 2) | ((r >> 1) & 1)) : ((r & 3) << 2) | ((r >> 2) & 3);
+  };
+  const uint32_t lds0 = (uint32_t)uni((int)(uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)ws_smem);
+  const u32x4 qres = make_rsrc(p.Q + (int64_t)h * p.q_hs, (uint32_t)((int64_t)p.NQ * RBQ));
+  const u32x4 dres = make_rsrc(dO + (int64_t)h * D, (uint32_t)((((int64_t)p.NQ - 1) * p.Hq * D + D) * 2));
+  // per-row scalars of a tile: -lse | -delta, a1 | b1, a2 | b2 (32 values each), one 256-byte load
+  // by each of waves 0-2 (the others repeat the first into a spare area so that all waves count alike)
+  const u32x4 nres = make_rsrc(neg + (int64_t)h * NQp, (uint32_t)((((int64_t)p.Hq + 1) * NQp) * 4));
+  const u32x4 mres = make_rsrc(mrows, (uint32_t)(4 * (int64_t)NQp * 4));
+  const bool sm_mask = wave == 1 || wave == 2;
+  const int sm_off = (lane & 31) * 4 + (lane >> 5) * (sm_mask ? NQp * 4 : p.Hq * NQp * 4) +
+                     (wave == 2 ? 2 * NQp * 4 : 0);
+  // this wave's loads of a tile: load li = wave + 8 j of the 2 * NLQ that make it (Q' first, then dO);
+  // rows past the last query read as zeros (and contribute nothing)
+  int ld_off[LPW], ld_mul[LPW], ld_dst[LPW];
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) {
+    const int li = wave + 8 * j;
+    const bool is_do = li >= NLQ;
+    const int l = is_do ? li - NLQ : li;
+    const int r = l * (1024 / RBQ) + lane / CKQ;
+    const int cofs = ((lane % CKQ) ^ swz_r(r)) * 16;
+    ld_mul[j] = is_do ? p.Hq * RBQ : RBQ;          // bytes per query row in global memory
+    ld_off[j] = r * ld_mul[j] + cofs;
+    ld_dst[j] = (is_do ? 32 * RBQ : 0) + l * 1024;
+  }
+  auto issue = [&](int s_, int buf, int set) __attribute__((always_inline)) {
+    const int mq = s_ * 32;
+#ifdef SPX_WS_NODMA
+    if (p.NQ > 0) return;
+#endif
+    const uint32_t rb = lds0 + buf * SM::kTile;
+#pragma unroll
+    for (int j = 0; j < LPW; ++j)
+      load_to_lds16<0>(wave + 8 * j >= NLQ ? dres : qres, rb + ld_dst[j], ld_off[j] + mq * ld_mul[j], 0);
+    const uint32_t sb = lds0 + SM::kOffSmall + (wave >= 3 ? SM::kSets * SM::kSmall : set * SM::kSmall + wave * 256);
+    load_to_lds4(sm_mask ? mres : nres, sb, sm_off + mq * 4, 0);
+  };
+  float* const small0 = reinterpret_cast<float*>(ws_smem + SM::kOffSmall);
+
+  // ---- role state
+  bf16x8 kf[producer ? NKK : 1], vf[producer ? NKK : 1];
+  f32x16 acc_dk[producer ? 1 : NDB], acc_dv[producer ? 1 : NDB];
+  if constexpr (producer) {
+    const uint16_t* krow = p.K + (int64_t)kvh * p.k_hs + (int64_t)cc * D + g * 8;
+    const uint16_t* vrow = p.V + (int64_t)kvh * p.v_hs + (int64_t)cc * D + g * 8;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      kf[kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(krow + kk * 16));
+      vf[kk] = as_bf16x8(*reinterpret_cast<const u32x4*>(vrow + kk * 16));
+    }
+  } else {
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { acc_dk[db][r] = 0.f; acc_dv[db][r] = 0.f; }
+  }
+  // producers: row `col`, 16-byte chunk 2 kk + g of Q' / dO
+  const int rdr = col * RBQ + ((g ^ swz_r(col)) * 16);
+  // consumers: lane s of 16-lane group G points at row 4 (G >> 1) + (s >> 2) (+ 8 for the second read) of
+  // a 16-row k step, bytes 8 (s & 3) of the 64-byte block 32 db + 16 (G & 1).  (The k index of the
+  // P / dS operand: element j of the lanes with g = lane / 32 is query row 4 g + j for j < 4 and
+  // 8 + 4 g + j - 4 after that, the accumulator layout of the score product.)
+  const int tG = lane >> 4, ts = lane & 15;
+  const int trow = 4 * (tG >> 1) + (ts >> 2);
+  const int tcl = 2 * (tG & 1) + ((ts & 3) >> 1);
+  const int rt0 = trow * RBQ + ((tcl ^ swz_r(trow)) * 16) + (ts & 1) * 8;
+  const int rt1 = (trow + 8) * RBQ + ((tcl ^ swz_r(trow + 8)) * 16) + (ts & 1) * 8;
+  uint8_t* const slot0 = ws_smem + SM::kOffSlot + pw * 2 * SM::kSlot;
+
+  // ---- the producers' two halves of a tile (kIdx: its index in the sequence of steps)
+  f32x16 st, dp;
+  auto score_mfma = [&](int buf, int set) __attribute__((always_inline)) {
+    const uint8_t* const tile = ws_smem + buf * SM::kTile;
+    const float* const lse_s = small0 + set * (SM::kSmall / 4);
+    const float* const delta_s = lse_s + 32;
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      const int q0 = 8 * r4 + 4 * g;  // 4 consecutive query rows: one 16-byte LDS read each
+      const f32x4 ls = *reinterpret_cast<const f32x4*>(&lse_s[q0]);
+      const f32x4 dl = *reinterpret_cast<const f32x4*>(&delta_s[q0]);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) { st[r4 * 4 + t] = ls[t]; dp[r4 * 4 + t] = dl[t]; }
+    }
+    SPX_PRIO_MFMA();
+    constexpr int NF = 2 * NKK;
+    bf16x8 fr[RG];
+    auto fread = [&](int f) {
+      fr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+          tile + ((f & 1) ? 32 * RBQ : 0) + (rdr ^ ((f / 2) * 32))));
+    };
+#pragma unroll
+    for (int f = 0; f < RG; ++f) fread(f);
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (f & 1) dp = mfma32(fr[f % RG], vf[producer ? f / 2 : 0], dp);
+      else st = mfma32(fr[f % RG], kf[producer ? f / 2 : 0], st);
+      __builtin_amdgcn_sched_barrier(0);
+      if (f + RG < NF) fread(f + RG);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    SPX_PRIO_VALU();
+  };
+  auto soft_valu = [&](int set, int par, bool full) __attribute__((always_inline)) {
+    const int* const a1_s = reinterpret_cast<const int*>(small0 + set * (SM::kSmall / 4) + 64);
+    const int* const b1_s = a1_s + 32; const int* const a2_s = b1_s + 32; const int* const b2_s = a2_s + 32;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st[r] = fast_exp2(st[r]);
+    if (!full) {
+      typedef __attribute__((ext_vector_type(4))) int i32x4;
+      pin_block(st);
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int q0 = 8 * r4 + 4 * g;
+        const i32x4 a1v = *reinterpret_cast<const i32x4*>(&a1_s[q0]);
+        const i32x4 b1v = *reinterpret_cast<const i32x4*>(&b1_s[q0]);
+        const i32x4 a2v = *reinterpret_cast<const i32x4*>(&a2_s[q0]);
+        const i32x4 b2v = *reinterpret_cast<const i32x4*>(&b2_s[q0]);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const bool ok = ((c >= a1v[t] && c < b1v[t]) || (c >= a2v[t] && c < b2v[t])) && (c < p.NKV);
+          if (!ok) st[r4 * 4 + t] = 0.f;
+        }
+      }
+      pin_block(st);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dp[r] *= st[r];
+    // hand P and dS over: four 16-byte stores per lane, slot row = register quad, column = lane
+    uint8_t* const slot = slot0 + par * SM::kSlot + lane * 16;
+    *reinterpret_cast<bf16x8*>(slot + 0 * 1024) = pack8(st, 0);
+    *reinterpret_cast<bf16x8*>(slot + 1 * 1024) = pack8(st, 8);
+    *reinterpret_cast<bf16x8*>(slot + 2 * 1024) = pack8(dp, 0);
+    *reinterpret_cast<bf16x8*>(slot + 3 * 1024) = pack8(dp, 8);
+  };
+  // ---- the consumers' half: dV^T += dO^T P, dK^T += Q'^T dS
+  auto consume = [&](int buf, int par) __attribute__((always_inline)) {
+    const uint8_t* const tile = ws_smem + buf * SM::kTile;
+    const uint8_t* const slot = slot0 + par * SM::kSlot + lane * 16;
+    bf16x8 pb[2], sb[2];
+    pb[0] = *reinterpret_cast<const bf16x8*>(slot + 0 * 1024);
+    pb[1] = *reinterpret_cast<const bf16x8*>(slot + 1 * 1024);
+    sb[0] = *reinterpret_cast<const bf16x8*>(slot + 2 * 1024);
+    sb[1] = *reinterpret_cast<const bf16x8*>(slot + 3 * 1024);
+    SPX_PRIO_MFMA();
+    constexpr int NF = 2 * 2 * NDB;
+    i16x4 lo[RG], hi[RG];
+    // fragment f: even = dO^T (for dV), odd = Q'^T (for dK); e = f / 2: k step s2 = e / NDB, row block db
+    auto fread = [&](int f) {
+      const int e = f / 2, s2 = e / NDB, db = e % NDB;
+      const uint8_t* const base = tile + ((f & 1) ? 0 : 32 * RBQ) + s2 * 16 * RBQ;
+#ifdef SPX_WS_SLOWT
+      // element-wise gather of the same fragment (checking aid)
+      i16x4 l4, h4;
+      for (int j = 0; j < 8; ++j) {
+        const int qr = s2 * 16 + (j < 4 ? 4 * g + j : 8 + 4 * g + j - 4), dd = db * 32 + col;
+        const int pos = ((dd >> 3) ^ swz_r(qr)) * 16 + (dd & 7) * 2;
+        const short v = *reinterpret_cast<const short*>(tile + ((f & 1) ? 0 : 32 * RBQ) + qr * RBQ + pos);
+        if (j < 4) l4[j] = v; else h4[j - 4] = v;
+      }
+      lo[f % RG] = l4; hi[f % RG] = h4;
+#else
+      lo[f % RG] = lds_read_tr16(base + (rt0 ^ (db * 64)));
+      hi[f % RG] = lds_read_tr16(base + (rt1 ^ (db * 64)));
+#endif
+    };
+    auto frag = [&](int f) {
+      const i16x8 v = __builtin_shufflevector(lo[f % RG], hi[f % RG], 0, 1, 2, 3, 4, 5, 6, 7);
+      return __builtin_bit_cast(bf16x8, v);
+    };
+#pragma unroll
+    for (int f = 0; f < RG; ++f) fread(f);
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+      const int e = f / 2, s2 = e / NDB, db = e % NDB;
+      __builtin_amdgcn_sched_barrier(0);
+      if (f & 1) acc_dk[producer ? 0 : db] = mfma32(frag(f), sb[s2], acc_dk[producer ? 0 : db]);   // Q'^T dS
+      else acc_dv[producer ? 0 : db] = mfma32(frag(f), pb[s2], acc_dv[producer ? 0 : db]);         // dO^T P
+      __builtin_amdgcn_sched_barrier(0);
+      if (f + RG < NF) fread(f + RG);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    SPX_PRIO_VALU();
+  };
+
+  // ---- prologue.  Tile k of the sequence of steps lives in ring buffer k % kStages, its per-row
+  // scalars in set k % kSets, its P / dS in slot k % 2.
+  int sq[AH + 1];               // sq[i]: the step (tile) of sequence index b + i
+  bool fq[AH + 1];              // ... whether every key of the block is visible to all of its rows
+#pragma unroll
+  for (int i = 0; i <= AH; ++i) {
+    const uint32_t e = (uint32_t)uni((int)entry(i));
+    sq[i] = step_of(e, i);
+    fq[i] = (e >> 31) != 0;
+  }
+  uint32_t pref = entry(AH + 1);   // fetched one step before it joins the queue
+  int sC = s_end;               // the consumers' tile: b - 1
+#pragma unroll
+  for (int i = 0; i < AH; ++i)
+    if (sq[i] < s_end) issue(sq[i], i, i);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if constexpr (producer) {
+    if (sq[0] < s_end) score_mfma(0, 0);
+  }
+  int rb = 0, kP = 0;           // ring buffer of tile b; b itself
+  auto wrap = [](int x) { return x >= NS ? x - NS : x; };
+  for (;; ++kP) {
+    const bool p_active = sq[0] < s_end, c_active = sC < s_end;
+    if (!p_active && !c_active) break;
+    // tile b + 1 has landed when at most the loads of tiles b + 2 .. b + kAhead - 1 are in flight
+    static_assert(AH == 4, "the wait below counts two tiles");
+#ifdef SPX_WS_TIMING
+    const bool dbg = blockIdx.x == 0 && lane == 0 && (wave & 3) == SPX_WS_TIMING && kP < 128;
+    unsigned long long* const dbg_row = g_ws_dbg + kP * 16 + (producer ? 0 : 8);
+    if (dbg) dbg_row[4] = __builtin_amdgcn_s_memtime();
+#endif
+    const int later = (sq[2] < s_end ? 1 : 0) + (sq[3] < s_end ? 1 : 0);
+#ifdef SPX_WS_WAITALL
+    if (later >= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else
+#endif
+    if (later == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoads) : "memory");
+    else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#ifdef SPX_WS_TIMING
+    if (dbg) dbg_row[5] = __builtin_amdgcn_s_memtime();
+#endif
+    __syncthreads();
+#ifdef SPX_WS_TIMING
+    if (dbg) dbg_row[0] = __builtin_amdgcn_s_memtime();
+#endif
+    // tile b + kAhead into the buffer tile b - 2 left behind
+    if (sq[AH] < s_end) issue(sq[AH], wrap(rb + AH), (kP + AH) & (SM::kSets - 1));
+#ifdef SPX_WS_TIMING
+    if (dbg) dbg_row[3] = __builtin_amdgcn_s_memtime();
+#endif
+    if constexpr (producer) {
+      if (p_active) {
+        soft_valu(kP & (SM::kSets - 1), kP & 1, fq[0]);
+#ifdef SPX_WS_TIMING
+        if (dbg) dbg_row[1] = __builtin_amdgcn_s_memtime();
+#endif
+        if (sq[1] < s_end) score_mfma(wrap(rb + 1), (kP + 1) & (SM::kSets - 1));
+#ifdef SPX_WS_TIMING
+        if (dbg) dbg_row[2] = __builtin_amdgcn_s_memtime();
+#endif
+      }
+    } else {
+      if (c_active) {
+        consume(wrap(rb + NS - 1), (kP - 1) & 1);
+#ifdef SPX_WS_TIMING
+        if (dbg) dbg_row[1] = __builtin_amdgcn_s_memtime();
+#endif
+      }
+    }
+    // next step
+    sC = sq[0];
+#pragma unroll
+    for (int i = 0; i < AH; ++i) { sq[i] = sq[i + 1]; fq[i] = fq[i + 1]; }
+    {
+      const uint32_t e = (uint32_t)uni((int)pref);
+      sq[AH] = step_of(e, kP + 1 + AH);
+      fq[AH] = (e >> 31) != 0;
+      pref = entry(kP + 2 + AH);
+    }
+    rb = wrap(rb + 1);
+  }
+
+  if constexpr (!producer) if (c < p.NKV) {
+    float* krow = dKp + ((int64_t)h * p.NKV + c) * D + 4 * g;
+    float* vrow = dVp + ((int64_t)h * p.NKV + c) * D + 4 * g;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const f32x4 wk = {acc_dk[db][r4 * 4 + 0], acc_dk[db][r4 * 4 + 1], acc_dk[db][r4 * 4 + 2], acc_dk[db][r4 * 4 + 3]};
+        const f32x4 wv = {acc_dv[db][r4 * 4 + 0], acc_dv[db][r4 * 4 + 1], acc_dv[db][r4 * 4 + 2], acc_dv[db][r4 * 4 + 3]};
+        *reinterpret_cast<f32x4*>(krow + db * 32 + 8 * r4) = wk;
+        *reinterpret_cast<f32x4*>(vrow + db * 32 + 8 * r4) = wv;
+      }
+  }
+  }  // part
+}
+
+template <int D>
+__global__ __launch_bounds__(512, 1) void attn_bwd_dkv_ws_kernel(
+    AttnParams p, const uint16_t* __restrict__ dO, int NQp, const float* __restrict__ neg,
+    const int32_t* __restrict__ mrows, const int32_t* __restrict__ tile_bounds,
+    float* __restrict__ dKp, float* __restrict__ dVp) {
+  using SM = DkvWsSmem<D>;
+  extern __shared__ __attribute__((aligned(16))) uint8_t ws_smem[];
+  // ---- the visible query tiles of both key blocks, in order, into LDS (all 512 threads)
+  {
+    constexpr int KB = 128;
+    const int n_kb = (p.NKV + KB - 1) / KB, n_pair = (n_kb + 1) / 2;
+    const int pair = (SPX_DKV_XCD && p.Hq % 8 == 0) ? (int)(blockIdx.x >> 3) % n_pair : (int)blockIdx.x / p.Hq;
+    const int n_qt = (p.NQ + 63) / 64;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int* const wtot = reinterpret_cast<int*>(ws_smem + SM::kOffList + 2 * SM::kList);
+    for (int part = 0; part < 2; ++part) {
+      const int kb_idx = part == 0 ? pair : n_kb - 1 - pair;
+      const int n0 = kb_idx * KB, key_last = min(n0 + KB - 1, p.NKV - 1);
+      uint32_t* const lst = reinterpret_cast<uint32_t*>(ws_smem + SM::kOffList + part * SM::kList);
+      int base = 0;
+      for (int q0 = 0; q0 < n_qt; q0 += 512) {
+        const int qt = q0 + tid;
+        bool vis = false, full = false;
+        if (qt < n_qt) {
+          const int32_t* tb = tile_bounds + qt * 8;
+          vis = (tb[0] <= key_last && tb[3] > n0) || (tb[4] <= key_last && tb[7] > n0);
+          full = (tb[1] <= n0 && tb[2] >= n0 + KB) || (tb[5] <= n0 && tb[6] >= n0 + KB);
+        }
+        const unsigned long long m = __ballot(vis);
+        const int before = __popcll(m & ((1ull << lane) - 1));
+        if (lane == 0) wtot[wave] = __popcll(m);
+        __syncthreads();
+        int off = base, all = 0;
+        for (int w = 0; w < 8; ++w) {
+          if (w < wave) off += wtot[w];
+          all += wtot[w];
+        }
+        if (vis) lst[off + before] = (uint32_t)qt | (full ? 0x80000000u : 0u);
+        base += all;
+        __syncthreads();
+      }
+      if (tid == 0) {
+        lst[base] = SM::kListEnd;
+        wtot[8 + part] = base;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x < 256)
+    dkv_ws_role<D, true>(p, dO, NQp, neg, mrows, dKp, dVp);
+  else
+    dkv_ws_role<D, false>(p, dO, NQp, neg, mrows, dKp, dVp);
 }
 
 // dK[kvh, c, :] = scaling * sum_{h in group} dKp[h, c, :],  dV likewise (no scaling); bf16 out
@@ -1879,6 +2290,8 @@ static int64_t bwd_workspace_bytes(int64_t NQ, int64_t NKV, int Hq, int Hkv, int
   b += round_up(((NQ + 63) / 64) * 32, 256);                        // tile bounds
   b += 2 * round_up((int64_t)Hq * NKV * D * 4, 256);                // fp32 per-head dK, dV
   b += round_up((int64_t)Hq * NQ * D * 2, 256);                     // Q scaled, row-major
+  b += round_up(2 * (int64_t)Hq * NQp * 4, 256);                    // -lse, -delta in padded rows
+  b += round_up(4 * NQp * 4, 256);                                  // interval ends of every row
   return b;
 }
 
@@ -1925,24 +2338,36 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   float* dvp = reinterpret_cast<float*>(w);
   w += round_up((int64_t)p.Hq * p.NKV * D * 4, 256);
   uint16_t* qs = reinterpret_cast<uint16_t*>(w);  // bf16(q * scale * log2 e), [Hq][NQ][D]
+  w += round_up((int64_t)p.Hq * p.NQ * D * 2, 256);
+  float* neg = reinterpret_cast<float*>(w);       // -lse [Hq][NQp], -delta [Hq][NQp]
+  w += round_up(2 * (int64_t)p.Hq * NQp * 4, 256);
+  int32_t* mrows = reinterpret_cast<int32_t*>(w); // [4][NQp]
 
   dim3 tgrid((unsigned)(p.NKVp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hkv);
   hipLaunchKernelGGL(transpose_bf16_kernel<false>, tgrid, dim3(64), 0, st, p.K, p.k_hs, (int64_t)D, p.NKV, D,
                      kt, (int64_t)D * p.NKVp, (int64_t)p.NKVp, 1.f, nullptr);
   dim3 qgrid((unsigned)(NQp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hq);
+  // (the wave-specialised dK/dV kernel transposes inside LDS and needs no Q^T / dO^T; it lists the query
+  // tiles that see a key block in LDS, which bounds their number)
+  const bool use_ws = D <= 128 && SPX_DKV_WS && (p.NQ + 63) / 64 <= DkvWsSmem<(D <= 128 ? D : 128)>::kListCap;
+  const bool kNeedT = !use_ws;
   hipLaunchKernelGGL(transpose_bf16_kernel<true>, qgrid, dim3(64), 0, st, p.Q, p.q_hs, (int64_t)D, p.NQ, D,
-                     qt, (int64_t)D * NQp, (int64_t)NQp, p.scale_log2e, qs);
-  hipLaunchKernelGGL(transpose_bf16_kernel<false>, qgrid, dim3(64), 0, st, dOp, (int64_t)D,
-                     (int64_t)p.Hq * D, p.NQ, D, dot, (int64_t)D * NQp, (int64_t)NQp, 1.f, nullptr);
+                     kNeedT ? qt : nullptr, (int64_t)D * NQp, (int64_t)NQp, p.scale_log2e, qs);
+  if (kNeedT)
+    hipLaunchKernelGGL(transpose_bf16_kernel<false>, qgrid, dim3(64), 0, st, dOp, (int64_t)D,
+                       (int64_t)p.Hq * D, p.NQ, D, dot, (int64_t)D * NQp, (int64_t)NQp, 1.f, nullptr);
   // the dK/dV and diagonal-key kernels read the scaled queries: their scores are q' . k with no
   // factor of their own, and what they accumulate against q' carries scale * log2(e) once too
   // often: dK = ln 2 * sum dS q'
   AttnParams ps = p;
   ps.Q = qs;
   ps.q_hs = (int64_t)p.NQ * D;
+  if (NQp != p.NQ)  // the padding of the negated rows reads as zero
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((2 * (int64_t)p.Hq * NQp + 255) / 256)), dim3(256), 0,
+                       st, neg, 2 * (int64_t)p.Hq * NQp);
   hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)(((int64_t)p.NQ * p.Hq + 15) / 16)), dim3(256),
-                     0, st, Op, dOp, p.NQ, p.Hq, delta);
-  hipLaunchKernelGGL(attn_tile_bounds_kernel, dim3((unsigned)((p.NQ + 63) / 64)), dim3(64), 0, st, p, tb);
+                     0, st, Op, dOp, p.NQ, p.Hq, delta, lse, NQp, neg);
+  hipLaunchKernelGGL(attn_tile_bounds_kernel, dim3((unsigned)(NQp / 64)), dim3(64), 0, st, p, tb, NQp, mrows);
 
   constexpr int BM = 32 * kDqNSB * kDqNW;
   const int n_qb = (p.NQ + BM - 1) / BM;
@@ -1971,7 +2396,18 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   const int n_kb = (p.NKV + 32 * kDkvNW - 1) / (32 * kDkvNW);
   const dim3 kgrid((unsigned)(n_kb * p.Hq)), kblock(64 * kDkvNW);
   static std::atomic<uint64_t> dkv_lds_set[2];  // per head_dim instantiation, one bit per device
-  if constexpr (D > 128 && SPX_DKV256_ONEPASS) {
+  if (use_ws) {
+   if constexpr (D <= 128 && SPX_DKV_WS) {
+    // producer / consumer waves, two per SIMD (see attn_bwd_dkv_ws_kernel)
+    constexpr int smem = DkvWsSmem<D>::kBytes;
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_ws_kernel<D>), smem,
+                                    dkv_lds_set[0], fn))
+      return rc;
+    const int n_pair_ws = ((p.NKV + 127) / 128 + 1) / 2;  // a workgroup takes two key blocks
+    hipLaunchKernelGGL((attn_bwd_dkv_ws_kernel<D>), dim3((unsigned)(n_pair_ws * p.Hq)), dim3(512), smem, st, ps,
+                       dOp, NQp, neg, mrows, tb, dkp, dvp);
+   }
+  } else if constexpr (D > 128 && SPX_DKV256_ONEPASS) {
     // dK and dV in one pass over 32-row tiles (two buffers of four 16 KB tiles)
     constexpr size_t smem = DkvSmem<D, 0, 32>::kBytesDma;
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, 3, 0>),

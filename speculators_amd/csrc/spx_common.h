@@ -88,6 +88,9 @@ __device__ __forceinline__ float wave_max(float v) {
 // The s_nop covers the M0-write -> LDS-DMA wait state for the first load of a group.
 template <int IMM>
 __device__ __forceinline__ void load_to_lds16(u32x4 rsrc, uint32_t lds_addr, int voff, int soff) {
+  // wave-uniform by contract; the reads cost nothing where the compiler already knows it
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+  soff = __builtin_amdgcn_readfirstlane(soff);
   if (IMM == 0)
     asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
@@ -98,6 +101,16 @@ __device__ __forceinline__ void load_to_lds16(u32x4 rsrc, uint32_t lds_addr, int
                  :
                  : "{m0}"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM)
                  : "memory");
+}
+
+// 64 lanes x 4 bytes, global -> LDS at M0 + 4 * lane (same addressing as load_to_lds16)
+__device__ __forceinline__ void load_to_lds4(u32x4 rsrc, uint32_t lds_addr, int voff, int soff) {
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+  soff = __builtin_amdgcn_readfirstlane(soff);
+  asm volatile("s_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :
+               : "{m0}"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory");
 }
 
 // buffer resource over `bytes` bytes at p (raw, no stride): offsets past the end read as zero
