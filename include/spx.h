@@ -456,6 +456,15 @@ int spx_gemm_bf16_tn(const void* a, int64_t lda, const void* b, int64_t ldb,
                      void* c, int64_t ldc, int64_t M, int64_t N, int64_t T,
                      int accumulate, void* stream);
 
+/* The same product with an fp32 result c[M, N] (ldc in floats): with accumulate != 0
+ * the weight gradient sums over the TTT steps in fp32 with no rounding between
+ * them, which is what autograd's accumulation into an fp32 master weight's .grad
+ * does in the reference's trainer (train/trainer.py:459-465 runs the model under
+ * bf16 autocast over fp32 parameters). */
+int spx_gemm_bf16_tn_f32(const void* a, int64_t lda, const void* b, int64_t ldb,
+                         void* c, int64_t ldc, int64_t M, int64_t N, int64_t T,
+                         int accumulate, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

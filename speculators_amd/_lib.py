@@ -70,6 +70,7 @@ SIGNATURES["spx_pack_row_map"] = [_P, _P, _I64, _I64, _P, _P, _P]
 SIGNATURES["spx_unpack_rows"] = [_P, _I64, _P, _I64, _I64, _I64, _P, _I64, _P]
 SIGNATURES["spx_gemm_bf16_nt_rows"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P, _P]
 SIGNATURES["spx_gemm_bf16_tn"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I, _P]
+SIGNATURES["spx_gemm_bf16_tn_f32"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I, _P]
 RESTYPES = {"spx_ttt_attn_workspace_bytes": c_int64, "spx_ttt_attn_fwd_static_max_bytes": c_int64, "spx_dflash_attn_workspace_bytes": c_int64,
             "spx_rmsnorm_bwd_slots": c_int64}
 

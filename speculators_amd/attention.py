@@ -137,14 +137,17 @@ class _TTTAttentionCached(torch.autograd.Function):
     the backward hands every step the matching window of the full dK / dV."""
 
     @staticmethod
-    def forward(ctx, q, mask: TTTMask, scaling: float, cache: TTTKVCache, n_parts: int, *parts):
+    def forward(ctx, q, mask: TTTMask, scaling: float, cache: TTTKVCache, n_parts: int, out, *parts):
         t = cache.t
         k = cache.k[:, :, :n_parts * t]
         v = cache.v[:, :, :n_parts * t]
         hq, hkv, t, d = _check_qkv(q, k, v, mask)
         q = q.contiguous()
         dev = q.device
-        out = torch.empty(1, t, hq, d, device=dev, dtype=torch.bfloat16)
+        if out is not None and out.numel() == t * hq * d and out.is_contiguous() and out.dtype == torch.bfloat16:
+            out = out.view(1, t, hq, d)
+        else:
+            out = torch.empty(1, t, hq, d, device=dev, dtype=torch.bfloat16)
         lse = torch.empty(hq, t, device=dev, dtype=torch.float32)
         ws = torch.empty(_workspace_bytes(t, hq, hkv, d, False), device=dev, dtype=torch.uint8)
         _lib.call("spx_ttt_attn_fwd", _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1),
@@ -176,13 +179,14 @@ class _TTTAttentionCached(torch.autograd.Function):
                   dv.stride(1), _lib.ptr(ws), ws.numel(), _lib.stream_ptr(dev))
         dks = [dk[:, :, i * t:(i + 1) * t] for i in range(n)]
         dvs = [dv[:, :, i * t:(i + 1) * t] for i in range(n)]
-        return (dq, None, None, None, None, *dks, *dvs)
+        return (dq, None, None, None, None, None, *dks, *dvs)
 
 
 def ttt_attention_cached(q, k_new, v_new, cache: TTTKVCache, mask: TTTMask,
-                         scaling: float | None = None) -> torch.Tensor:
+                         scaling: float | None = None, out=None) -> torch.Tensor:
     """TTT attention of the step whose keys / values ``k_new`` / ``v_new`` (the windows
-    ``cache.window(step)``, already written) were just appended; ``[1, T, Hq, D]`` (bf16)."""
+    ``cache.window(step)``, already written) were just appended; ``[1, T, Hq, D]`` (bf16),
+    written into ``out`` (a contiguous bf16 buffer of ``T * Hq * D`` elements) if given."""
     if scaling is None:
         scaling = q.shape[-1] ** -0.5
     cache.k_parts.append(k_new)
@@ -190,7 +194,7 @@ def ttt_attention_cached(q, k_new, v_new, cache: TTTKVCache, mask: TTTMask,
     n = len(cache.k_parts)
     if n != mask.ttt_step + 1:
         raise ValueError(f"the cache holds {n} steps but the mask is at TTT step {mask.ttt_step}")
-    return _TTTAttentionCached.apply(q, mask, scaling, cache, n, *cache.k_parts, *cache.v_parts)
+    return _TTTAttentionCached.apply(q, mask, scaling, cache, n, out, *cache.k_parts, *cache.v_parts)
 
 
 def ttt_attention(q, k, v, mask: TTTMask, scaling: float | None = None) -> torch.Tensor:

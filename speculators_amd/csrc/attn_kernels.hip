@@ -1742,11 +1742,11 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
   constexpr int KB = 128;                                 // keys per workgroup
   constexpr int RBQ = D * 2, CKQ = RBQ / 16;              // bytes / 16-byte chunks per row of Q' and dO
   constexpr int NLQ = 32 * RBQ / 1024;                    // 1 KB wave loads per 32-row operand
-  constexpr int LPW = 2 * NLQ / 8;                        // tile loads per wave
+  constexpr int LPW = 2 * NLQ / 4;                        // tile loads per consumer wave (they issue them all)
   constexpr int kLoads = LPW + 1;                         // ... plus one of per-row scalars
   constexpr int RG = 4;
   constexpr int NS = SM::kStages, AH = SM::kAhead;
-  static_assert(LPW >= 1 && 2 * NLQ % 8 == 0, "every wave issues the same number of loads per tile");
+  static_assert(LPW >= 1 && 2 * NLQ % 4 == 0, "every consumer wave issues the same number of loads per tile");
   // A workgroup takes key blocks i and n_kb - 1 - i of one head, one after the other: under a causal
   // mask block i is seen by all later query tiles and its partner by correspondingly few, so every
   // workgroup walks about the same number of tiles.
@@ -1796,18 +1796,19 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
   const u32x4 qres = make_rsrc(p.Q + (int64_t)h * p.q_hs, (uint32_t)((int64_t)p.NQ * RBQ));
   const u32x4 dres = make_rsrc(dO + (int64_t)h * D, (uint32_t)((((int64_t)p.NQ - 1) * p.Hq * D + D) * 2));
   // per-row scalars of a tile: -lse | -delta, a1 | b1, a2 | b2 (32 values each), one 256-byte load
-  // by each of waves 0-2 (the others repeat the first into a spare area so that all waves count alike)
+  // by each of consumer waves 0-2 (the fourth repeats the first into a spare area so that all count
+  // alike).  The consumers issue every load: they have time to spare, the producers do not.
   const u32x4 nres = make_rsrc(neg + (int64_t)h * NQp, (uint32_t)((((int64_t)p.Hq + 1) * NQp) * 4));
   const u32x4 mres = make_rsrc(mrows, (uint32_t)(4 * (int64_t)NQp * 4));
-  const bool sm_mask = wave == 1 || wave == 2;
+  const bool sm_mask = pw == 1 || pw == 2;
   const int sm_off = (lane & 31) * 4 + (lane >> 5) * (sm_mask ? NQp * 4 : p.Hq * NQp * 4) +
-                     (wave == 2 ? 2 * NQp * 4 : 0);
-  // this wave's loads of a tile: load li = wave + 8 j of the 2 * NLQ that make it (Q' first, then dO);
+                     (pw == 2 ? 2 * NQp * 4 : 0);
+  // this wave's loads of a tile: load li = pw + 4 j of the 2 * NLQ that make it (Q' first, then dO);
   // rows past the last query read as zeros (and contribute nothing)
   int ld_off[LPW], ld_mul[LPW], ld_dst[LPW];
 #pragma unroll
   for (int j = 0; j < LPW; ++j) {
-    const int li = wave + 8 * j;
+    const int li = pw + 4 * j;
     const bool is_do = li >= NLQ;
     const int l = is_do ? li - NLQ : li;
     const int r = l * (1024 / RBQ) + lane / CKQ;
@@ -1824,8 +1825,8 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
     const uint32_t rb = lds0 + buf * SM::kTile;
 #pragma unroll
     for (int j = 0; j < LPW; ++j)
-      load_to_lds16<0>(wave + 8 * j >= NLQ ? dres : qres, rb + ld_dst[j], ld_off[j] + mq * ld_mul[j], 0);
-    const uint32_t sb = lds0 + SM::kOffSmall + (wave >= 3 ? SM::kSets * SM::kSmall : set * SM::kSmall + wave * 256);
+      load_to_lds16<0>(pw + 4 * j >= NLQ ? dres : qres, rb + ld_dst[j], ld_off[j] + mq * ld_mul[j], 0);
+    const uint32_t sb = lds0 + SM::kOffSmall + (pw == 3 ? SM::kSets * SM::kSmall : set * SM::kSmall + pw * 256);
     load_to_lds4(sm_mask ? mres : nres, sb, sm_off + mq * 4, 0);
   };
   float* const small0 = reinterpret_cast<float*>(ws_smem + SM::kOffSmall);
@@ -1861,9 +1862,19 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
   uint8_t* const slot0 = ws_smem + SM::kOffSlot + pw * 2 * SM::kSlot;
 
   // ---- the producers' two halves of a tile (kIdx: its index in the sequence of steps)
-  f32x16 st, dp;
-  auto score_mfma = [&](int buf, int set) __attribute__((always_inline)) {
-    const uint8_t* const tile = ws_smem + buf * SM::kTile;
+  f32x16 st, dp;      // scores / dP of the tile in work
+  f32x16 stn, dpn;    // -lse, -delta of the next tile (the C operands of its first products)
+  constexpr int NFP = 2 * NKK;
+  bf16x8 pfr[RG];
+  const uint8_t* ptile = ws_smem;
+  auto pfread = [&](int f) __attribute__((always_inline)) {
+    pfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+        ptile + ((f & 1) ? 32 * RBQ : 0) + (rdr ^ ((f / 2) * 32))));
+  };
+  // first half: the LDS reads whose results the products start from (issued before the soft-max half
+  // of the previous tile, so that they are back when it ends)
+  auto score_begin = [&](int buf, int set) __attribute__((always_inline)) {
+    ptile = ws_smem + buf * SM::kTile;
     const float* const lse_s = small0 + set * (SM::kSmall / 4);
     const float* const delta_s = lse_s + 32;
 #pragma unroll
@@ -1872,24 +1883,21 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
       const f32x4 ls = *reinterpret_cast<const f32x4*>(&lse_s[q0]);
       const f32x4 dl = *reinterpret_cast<const f32x4*>(&delta_s[q0]);
 #pragma unroll
-      for (int t = 0; t < 4; ++t) { st[r4 * 4 + t] = ls[t]; dp[r4 * 4 + t] = dl[t]; }
+      for (int t = 0; t < 4; ++t) { stn[r4 * 4 + t] = ls[t]; dpn[r4 * 4 + t] = dl[t]; }
     }
+#pragma unroll
+    for (int f = 0; f < RG; ++f) pfread(f);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto score_finish = [&]() __attribute__((always_inline)) {
     SPX_PRIO_MFMA();
-    constexpr int NF = 2 * NKK;
-    bf16x8 fr[RG];
-    auto fread = [&](int f) {
-      fr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-          tile + ((f & 1) ? 32 * RBQ : 0) + (rdr ^ ((f / 2) * 32))));
-    };
 #pragma unroll
-    for (int f = 0; f < RG; ++f) fread(f);
-#pragma unroll
-    for (int f = 0; f < NF; ++f) {
+    for (int f = 0; f < NFP; ++f) {
       __builtin_amdgcn_sched_barrier(0);
-      if (f & 1) dp = mfma32(fr[f % RG], vf[producer ? f / 2 : 0], dp);
-      else st = mfma32(fr[f % RG], kf[producer ? f / 2 : 0], st);
+      if (f & 1) dp = mfma32(pfr[f % RG], vf[producer ? f / 2 : 0], f == 1 ? dpn : dp);
+      else st = mfma32(pfr[f % RG], kf[producer ? f / 2 : 0], f == 0 ? stn : st);
       __builtin_amdgcn_sched_barrier(0);
-      if (f + RG < NF) fread(f + RG);
+      if (f + RG < NFP) pfread(f + RG);
     }
     __builtin_amdgcn_sched_barrier(0);
     SPX_PRIO_VALU();
@@ -1988,13 +1996,15 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
   }
   uint32_t pref = entry(AH + 1);   // fetched one step before it joins the queue
   int sC = s_end;               // the consumers' tile: b - 1
+  if constexpr (!producer) {
 #pragma unroll
-  for (int i = 0; i < AH; ++i)
-    if (sq[i] < s_end) issue(sq[i], i, i);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    for (int i = 0; i < AH; ++i)
+      if (sq[i] < s_end) issue(sq[i], i, i);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
   __syncthreads();
   if constexpr (producer) {
-    if (sq[0] < s_end) score_mfma(0, 0);
+    if (sq[0] < s_end) { score_begin(0, 0); score_finish(); }
   }
   int rb = 0, kP = 0;           // ring buffer of tile b; b itself
   auto wrap = [](int x) { return x >= NS ? x - NS : x; };
@@ -2004,18 +2014,20 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
     // tile b + 1 has landed when at most the loads of tiles b + 2 .. b + kAhead - 1 are in flight
     static_assert(AH == 4, "the wait below counts two tiles");
 #ifdef SPX_WS_TIMING
-    const bool dbg = blockIdx.x == 0 && lane == 0 && (wave & 3) == SPX_WS_TIMING && kP < 128;
+#ifdef SPX_WS_TIMING_STEPS
+    const bool dbg = blockIdx.x == 0 && lane == 0 && (wave & 3) == SPX_WS_TIMING && kP < 127;
+#else
+    const bool dbg = false;
+#endif
     unsigned long long* const dbg_row = g_ws_dbg + kP * 16 + (producer ? 0 : 8);
     if (dbg) dbg_row[4] = __builtin_amdgcn_s_memtime();
 #endif
-    const int later = (sq[2] < s_end ? 1 : 0) + (sq[3] < s_end ? 1 : 0);
-#ifdef SPX_WS_WAITALL
-    if (later >= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    else
-#endif
-    if (later == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoads) : "memory");
-    else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (!producer) {
+      const int later = (sq[2] < s_end ? 1 : 0) + (sq[3] < s_end ? 1 : 0);
+      if (later == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoads) : "memory");
+      else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
 #ifdef SPX_WS_TIMING
     if (dbg) dbg_row[5] = __builtin_amdgcn_s_memtime();
 #endif
@@ -2023,18 +2035,14 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
 #ifdef SPX_WS_TIMING
     if (dbg) dbg_row[0] = __builtin_amdgcn_s_memtime();
 #endif
-    // tile b + kAhead into the buffer tile b - 2 left behind
-    if (sq[AH] < s_end) issue(sq[AH], wrap(rb + AH), (kP + AH) & (SM::kSets - 1));
-#ifdef SPX_WS_TIMING
-    if (dbg) dbg_row[3] = __builtin_amdgcn_s_memtime();
-#endif
     if constexpr (producer) {
       if (p_active) {
+        if (sq[1] < s_end) score_begin(wrap(rb + 1), (kP + 1) & (SM::kSets - 1));
         soft_valu(kP & (SM::kSets - 1), kP & 1, fq[0]);
 #ifdef SPX_WS_TIMING
         if (dbg) dbg_row[1] = __builtin_amdgcn_s_memtime();
 #endif
-        if (sq[1] < s_end) score_mfma(wrap(rb + 1), (kP + 1) & (SM::kSets - 1));
+        if (sq[1] < s_end) score_finish();
 #ifdef SPX_WS_TIMING
         if (dbg) dbg_row[2] = __builtin_amdgcn_s_memtime();
 #endif
@@ -2046,6 +2054,11 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
         if (dbg) dbg_row[1] = __builtin_amdgcn_s_memtime();
 #endif
       }
+      // tile b + kAhead into the buffer tile b - 2 left behind
+      if (sq[AH] < s_end) issue(sq[AH], wrap(rb + AH), (kP + AH) & (SM::kSets - 1));
+#ifdef SPX_WS_TIMING
+      if (dbg) dbg_row[3] = __builtin_amdgcn_s_memtime();
+#endif
     }
     // next step
     sC = sq[0];
@@ -2124,10 +2137,22 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkv_ws_kernel(
     }
     __syncthreads();
   }
+#ifdef SPX_WS_TIMING
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    g_ws_dbg[127 * 16 + 12] = __builtin_amdgcn_s_memtime();
+    g_ws_dbg[127 * 16 + 13] = __builtin_amdgcn_s_memrealtime();
+  }
+#endif
   if (threadIdx.x < 256)
     dkv_ws_role<D, true>(p, dO, NQp, neg, mrows, dKp, dVp);
   else
     dkv_ws_role<D, false>(p, dO, NQp, neg, mrows, dKp, dVp);
+#ifdef SPX_WS_TIMING
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    g_ws_dbg[127 * 16 + 14] = __builtin_amdgcn_s_memtime();
+    g_ws_dbg[127 * 16 + 15] = __builtin_amdgcn_s_memrealtime();
+  }
+#endif
 }
 
 // dK[kvh, c, :] = scaling * sum_{h in group} dKp[h, c, :],  dV likewise (no scaling); bf16 out

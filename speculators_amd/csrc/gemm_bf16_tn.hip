@@ -1,28 +1,25 @@
 // Weight-gradient GEMM for gfx950: C[M, N] (+)= A[T, M]^T * B[T, N], bf16 operands, fp32
-// accumulation, bf16 result (optionally added to what C holds: the gradient of a weight that
-// is applied once per TTT step accumulates in place).  Both operands are stored with the
-// contraction index T as the SLOW dimension (A = the output gradient dY [T, M], B = the layer
-// input X [T, N]), so an MFMA fragment -- 8 consecutive t for one m -- is a column of 8
-// rows in memory.  The tile is turned on its way into LDS:
-//   * every thread loads an 8 (t) x 8 (m) block with eight 16-byte row loads (a wave reads whole
-//     128-byte lines), transposes it in registers with sixteen-bit byte permutes (v_perm_b32, 32 per
-//     block) and writes eight 16-byte LDS rows [m][t0..t0+7];
-//   * LDS rows are 64 t-values + 16 bytes of padding (pitch 144): with it both the transposed
-//     writes (lanes = 8 t-chunks x 8 m-chunks) and the fragment reads (lanes = 32 rows) touch
-//     every bank the same number of times;
-// from there on it is the NT kernel: 256 x 256 tile, 4 waves x 128 x 128, slabs of 64 along
-// T in two LDS buffers, v_mfma_f32_32x32x16_bf16 with one LDS read issued per MFMA,
-// transposed accumulators and v_permlane32_swap for 16-byte stores.  The register transposes
-// ride between the MFMAs of the second half of a slab (the vector pipe is idle there).
-// Two sets of staging registers keep two slabs of loads in flight.
+// accumulation; the result is bf16 or fp32 and may be added to what C holds (the gradient of a
+// weight that is applied once per TTT step accumulates in place, in fp32 without any rounding
+// between the steps).  Both operands are stored with the contraction index T as the SLOW
+// dimension (A = the output gradient dY [T, M], B = the layer input X [T, N]), so an MFMA
+// fragment -- 8 consecutive t for one m -- is a column of 8 rows in memory.
 //
-// What bounds it: the LDS pipe.  A 16-byte LDS write from registers occupies the pipe twice as
-// long as a 16-byte read (counters: 8 against 4 index cycles), so the 16 writes per lane and
-// slab cost as much as the 32 fragment reads and the pipe is busy about 80 % of the kernel's
-// time, against 55 % in the NT kernel, whose tiles reach LDS without passing through registers.
-// Measured 0.95 - 1.05 PFLOP/s on the draft layers' weight-gradient shapes (T = 4096), the
-// vendor library's TN kernels 1.08 - 1.18: the host side of this package keeps the library
-// for the weight gradients and this kernel serves callers of the C interface.
+// The tiles are NOT transposed on their way in.  A slab of 64 t-rows x 256 columns of each
+// operand goes global -> LDS directly (buffer_load ... lds, whole 512-byte rows), exactly as it
+// lies in memory, and the fragments are taken with the transposing LDS read of gfx950
+// (ds_read_b64_tr_b16: inside every group of 16 lanes, lane 4u + w receives as element j element
+// w of the 8 bytes lane 4j + u points at).  Two such reads make one 32 x 16 operand fragment:
+// lane (G = lane / 16, s = lane % 16) points at row 8 (G / 2) + s / 4 (+ 4 for the second read) of
+// the 16-row K step and at bytes 32 (G % 2) + 8 (s % 4) of the fragment's 64-byte column block.
+// Bank conflicts: the rows of a slab are 512 bytes apart, so the 64-byte block b of row t sits at
+// block position b ^ (t % 4): the 4 + 4 rows one read touches then fall into four different
+// 64-byte bank groups, two rows each, which is the minimum for 512 bytes.
+//
+// From there on it is the NT kernel: 256 x 256 tile, 4 waves x 128 x 128 (one per SIMD), two
+// slab buffers, v_mfma_f32_32x32x16_bf16, the LDS reads of K step kk+1 and the global loads of
+// the next slab issued one at a time between the MFMAs of step kk, one barrier per slab,
+// accumulators kept transposed (lane = row of C).
 
 #include "spx_common.h"
 #include "../../include/spx.h"
@@ -35,43 +32,44 @@ constexpr int kNW = 4, kThreads = 256;
 constexpr int kTM = 256, kTN = 256, kTK = 64;
 constexpr int kWM = 2, kWN = 2;
 constexpr int kMI = kTM / kWM / 32, kNI = kTN / kWN / 32;  // 4 x 4 accumulators of 32 x 32 per wave
-constexpr int kPitch = kTK * 2 + 16;                        // 144 bytes per LDS row
-constexpr int kOpBytes = kTM * kPitch;                      // one operand of one slab: 36864
-constexpr int kBufBytes = 2 * kOpBytes;                     // A + B
-constexpr int kSmem = 2 * kBufBytes;                        // 147456
+constexpr int kRowBytes = kTM * 2;                          // 512: one t-row of a slab
+constexpr int kABytes = kTK * kRowBytes;                    // one slab of A: 32 KB
+constexpr int kBBytes = kABytes;
+constexpr int kBBase = 2 * kABytes;
+constexpr int kSmem = 2 * (kABytes + kBBytes);              // 128 KB
+constexpr int kLA = kTK / 2 / kNW;                          // wave-loads (2 rows each) of A per wave per slab
+constexpr int kLB = kLA;
+constexpr int kL = kLA + kLB;
 constexpr int kOob = 0x7ffffff0;
+static_assert(kTM == kTN, "both operands use one slab layout");
+static_assert(kABytes == 32768, "the buffer toggle flips bit 15");
 #ifndef SPX_GEMM_TN_GROUP_M
 #define SPX_GEMM_TN_GROUP_M 8
 #endif
 
-__device__ __forceinline__ bf16x8 as_frag(u32x4 v) {
-  union { u32x4 u; bf16x8 b; } c;
-  c.u = v;
-  return c.b;
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ i16x4 lds_read_tr16(const uint8_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) i16x4*)(uintptr_t)(uint32_t)(uintptr_t)(
+          (__attribute__((address_space(3))) const uint8_t*)p));
 }
 
-// output row i (0..7) of the transposed 8 x 8 block: element e of the result = in[e] element i
-__device__ __forceinline__ u32x4 transposed_row(const u32x4 (&in)[8], int i) {
-  const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
-  const int w = i >> 1;
-  u32x4 o;
-  o.x = __builtin_amdgcn_perm(in[1][w], in[0][w], sel);
-  o.y = __builtin_amdgcn_perm(in[3][w], in[2][w], sel);
-  o.z = __builtin_amdgcn_perm(in[5][w], in[4][w], sel);
-  o.w = __builtin_amdgcn_perm(in[7][w], in[6][w], sel);
-  return o;
-}
-
-template <bool ACC>
+// OUT: 0 = bf16 result, 1 = bf16 result added to C, 2 = fp32 result, 3 = fp32 result added to C
+template <int OUT>
 __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_bf16_tn_kernel(
     const uint16_t* __restrict__ A, int64_t lda, const uint16_t* __restrict__ B, int64_t ldb,
-    uint16_t* __restrict__ C, int64_t ldc, int M, int N, int T, int tiles_m, int tiles_n) {
+    void* __restrict__ Cv, int64_t ldc, int M, int N, int T, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
   // workgroup id -> tile: XCD-contiguous bands, then groups of GROUP_M tile rows
   const int n_wg = tiles_m * tiles_n;
-  int pid = blockIdx.x;
-  if (n_wg % 8 == 0) pid = (pid % 8) * (n_wg / 8) + pid / 8;
+  int pid;
+  {
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int base = n_wg >> 3, rem = n_wg & 7;
+    pid = xcd * base + min(xcd, rem) + local;
+  }
   constexpr int GROUP_M = SPX_GEMM_TN_GROUP_M;
   const int in_group = GROUP_M * tiles_n;
   const int first_m = (pid / in_group) * GROUP_M;
@@ -85,6 +83,7 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
   const int g = lane >> 5, col = lane & 31;
   const int wm = (wave / kWN) * (kTM / kWM), wn = (wave % kWN) * (kTN / kWN);
 
+  // acc[j][i]: registers = 32 columns of C at wn + 32 j, lane = row of C at wm + 32 i
   f32x16 acc[kNI][kMI];
 #pragma unroll
   for (int j = 0; j < kNI; ++j)
@@ -93,178 +92,220 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[j][i][r] = 0.f;
 
-  // ---- global side: this thread's 8 x 8 block of each operand: t rows tb*8 .. tb*8+7 of the slab,
-  // columns mc*8 .. mc*8+7 of the tile.  Rows past T (every row of a slab past the end) lie outside
-  // the buffer resource and read as zero: the whole offset is in the VGPR, which the range check sees.
-  const int tb = lane & 7, mc = (lane >> 3) + 8 * wave;
-  const __amdgpu_buffer_rsrc_t ares = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(A), 0, (int)((((int64_t)T - 1) * lda + M) * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t bres = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(B), 0, (int)((((int64_t)T - 1) * ldb + N) * 2), 0x00020000);
-  // A column chunk past the matrix edge may read the next row's valid memory instead of zeros: it
-  // only feeds rows / columns of C that are never stored.
+  // One buffer resource per operand, starting at the tile's first column.  The whole offset of a load,
+  // the slab's first row included, is in the vector register, which is what the range check sees: rows
+  // past T lie outside the resource and read as zero.  A 16-byte chunk past the last column would read
+  // the next row instead, so those lanes get an offset outside the resource.
+  const u32x4 ares = make_rsrc(A + m0, (uint32_t)((((int64_t)T - 1) * lda + min(M - m0, kTM)) * 2));
+  const u32x4 bres = make_rsrc(B + n0, (uint32_t)((((int64_t)T - 1) * ldb + min(N - n0, kTN)) * 2));
+
+  // global side: wave-load j of this wave covers slab rows 2 (wave * kLA + j) + lane / 32; the lane's LDS
+  // position is 16-byte chunk lane % 32 of the row, which holds the chunk of 64-byte block
+  // (position / 4) ^ (row % 4)
+  const int lrow = lane >> 5, lpos = lane & 31;
+  int aoff[kLA], boff[kLB];
+#pragma unroll
+  for (int j = 0; j < kLA; ++j) {
+    const int r = 2 * (wave * kLA + j) + lrow;
+    const int c8 = ((((lpos >> 2) ^ (r & 3)) << 2) | (lpos & 3)) * 8;  // first column of the chunk
+    aoff[j] = (m0 + c8 < M) ? (int)(((int64_t)r * lda + c8) * 2) : kOob;
+    boff[j] = (n0 + c8 < N) ? (int)(((int64_t)r * ldb + c8) * 2) : kOob;
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+  const uint32_t lds_a = lds0 + wave * kLA * 1024;
+  const uint32_t lds_b = lds0 + kBBase + wave * kLB * 1024;
+
+  uint32_t bufoff = 0;  // slab buffer the next loads go to
+  int ld_t0 = 0;        // first row of the slab being loaded
   const int a_row = (int)(lda * 2), b_row = (int)(ldb * 2);
-  const int a_v0 = tb * 8 * a_row + (m0 + mc * 8) * 2, b_v0 = tb * 8 * b_row + (n0 + mc * 8) * 2;
+  // load l (A loads first, then B) of the slab at ld_t0
+  auto issue_one = [&](int l) __attribute__((always_inline)) {
+    const bool isa = l < kLA;
+    const int j = isa ? l : l - kLA;
+    const uint32_t voff = (uint32_t)(isa ? aoff[j] : boff[j]) + (uint32_t)ld_t0 * (uint32_t)(isa ? a_row : b_row);
+    // (a lane that is out of range stays so: kOob plus the row offset lies past any resource size)
+    load_to_lds16<0>(isa ? ares : bres, (isa ? lds_a : lds_b) + bufoff + j * 1024, (int)voff, 0);
+  };
+  auto next_slab = [&]() __attribute__((always_inline)) { bufoff ^= kABytes; ld_t0 += kTK; };
 
-  // two register sets: set p holds the slabs of parity p between their loads and their staging
-  u32x4 ra[2][8], rb[2][8];
-  auto fetch_a = [&](int s, int p) __attribute__((always_inline)) {
-    const int base = a_v0 + s * (kTK * a_row);
+  // read side (see the head of the file)
+  const int tG = lane >> 4, ts = lane & 15;
+  const int trow = 8 * (tG >> 1) + (ts >> 2);
+  const int lane_off = trow * kRowBytes + ((ts >> 2) & 3) * 64 + 32 * (tG & 1) + 8 * (ts & 3);
+  uint32_t a_rd[kMI], b_rd[kNI];  // per fragment; bit 15 selects the slab buffer
 #pragma unroll
-    for (int j = 0; j < 8; ++j) ra[p][j] = __builtin_amdgcn_raw_buffer_load_b128(ares, base + j * a_row, 0, 0);
-  };
-  auto fetch_b = [&](int s, int p) __attribute__((always_inline)) {
-    const int base = b_v0 + s * (kTK * b_row);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) rb[p][j] = __builtin_amdgcn_raw_buffer_load_b128(bres, base + j * b_row, 0, 0);
-  };
-  // LDS side of the same block: rows mc*8 + i, 16-byte chunk tb
-  const int wr_off = (mc * 8) * kPitch + tb * 16;
-  // unit u (0..15): transposed row u % 8 of operand u / 8 (register set p), written to slab buffer `buf`
-  auto stage_unit = [&](int u, int buf, int p) __attribute__((always_inline)) {
-    const int i = u & 7;
-    const u32x4 o = (u < 8) ? transposed_row(ra[p], i) : transposed_row(rb[p], i);
-    *reinterpret_cast<u32x4*>(smem + buf * kBufBytes + (u < 8 ? 0 : kOpBytes) + wr_off + i * kPitch) = o;
-  };
+  for (int f = 0; f < kMI; ++f) {
+    a_rd[f] = lane_off ^ ((wm / 32 + f) * 64);
+    b_rd[f] = kBBase + (lane_off ^ ((wn / 32 + f) * 64));
+  }
 
-  // ---- read side: row = lane % 32 of a 32-row block, t chunk 2 kk + g
-  const int rd0 = col * kPitch + g * 16;
-  const int a_rd = (wm)*kPitch + rd0, b_rd = kOpBytes + wn * kPitch + rd0;
-  bf16x8 fa[2][kMI], fb[2][kNI];
-  auto read_one = [&](int set, int buf, int kk, int f) __attribute__((always_inline)) {
-    if (f < kMI)
-      fa[set][f] = as_frag(*reinterpret_cast<const u32x4*>(smem + buf * kBufBytes + a_rd + kk * 32 + f * 32 * kPitch));
-    else
-      fb[set][f - kMI] = as_frag(
-          *reinterpret_cast<const u32x4*>(smem + buf * kBufBytes + b_rd + kk * 32 + (f - kMI) * 32 * kPitch));
+  i16x4 fa[2][kMI][2], fb[2][kNI][2];
+  // operand fragment f (A fragments first, then B) of K step kk into register set `set`
+  auto read_one = [&](int set, int kk, int f) __attribute__((always_inline)) {
+    if (f < kMI) {
+      fa[set][f][0] = lds_read_tr16(smem + a_rd[f] + kk * 16 * kRowBytes);
+      fa[set][f][1] = lds_read_tr16(smem + a_rd[f] + kk * 16 * kRowBytes + 4 * kRowBytes);
+    } else {
+      fb[set][f - kMI][0] = lds_read_tr16(smem + b_rd[f - kMI] + kk * 16 * kRowBytes);
+      fb[set][f - kMI][1] = lds_read_tr16(smem + b_rd[f - kMI] + kk * 16 * kRowBytes + 4 * kRowBytes);
+    }
   };
-  // One step of 16 along T: the 16 MFMAs on register set `set`; between them, one at a time, the
-  // LDS reads that fill the other set with step rk of buffer rbuf.  `plan` says what else rides
-  // along: 1 = the staging units of A of the next slab (buffer wbuf), then the loads of A of
-  // slab nxt into the registers just freed; 2 = the same for B
-  auto step = [&](int set, int rbuf, int rk, int plan, int wbuf, int nxt) __attribute__((always_inline)) {
-    constexpr int kF = kMI + kNI;
-    int reads = 0;
+  auto frag = [&](const i16x4 (&h)[2]) __attribute__((always_inline)) {
+    const i16x8 v = __builtin_shufflevector(h[0], h[1], 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, v);
+  };
+  // One K step: the kNI x kMI MFMAs on register set `set`; between them, one at a time, the LDS
+  // reads that fill the other set with K step rk and the global loads [l0, l0 + nl).
+  auto step = [&](int set, int rk, int l0, int nl) __attribute__((always_inline)) {
+    constexpr int kN = kNI * kMI, kF = kMI + kNI;
+    int reads = 0, loads = 0;
 #pragma unroll
     for (int j = 0; j < kNI; ++j)
 #pragma unroll
       for (int i = 0; i < kMI; ++i) {
-        acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[set][j], fa[set][i], acc[j][i], 0, 0, 0);
+        acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(fb[set][j]), frag(fa[set][i]), acc[j][i], 0, 0, 0);
         const int idx = j * kMI + i;
         __builtin_amdgcn_sched_barrier(0);
         if (reads < kF) {
-          read_one(set ^ 1, rbuf, rk, reads++);
+          read_one(set ^ 1, rk, reads++);
           __builtin_amdgcn_sched_barrier(0);
         }
-        if (plan == 1 || plan == 2) {
-          if (idx & 1) stage_unit((plan == 2 ? 8 : 0) + (idx >> 1), wbuf, wbuf);
-          if (idx == 15) {
-            if (plan == 1) fetch_a(nxt, wbuf); else fetch_b(nxt, wbuf);
-          }
+        if (nl > 0 && (nl >= kN || idx % (kN / nl) == kN / nl - 1) && loads < nl) {
+          issue_one(l0 + loads++);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+  };
+
+  // the loads of a slab are spread over the step after the barrier (kLdT of them) and step 0 of the
+  // next slab (the rest); steps 1 and 2 give them time to land
+  constexpr int kLdT = kL / 2, kLd0 = kL - kLdT;
+  auto slab = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    step(0, 1, kLdT, kLd0);
+    next_slab();
+    step(1, 2, 0, 0);
+    step(0, 3, 0, 0);
+    // every read of this slab's buffer has returned once set 1 is complete; then the barrier says:
+    // slab s+1 has landed for everybody, this buffer is free
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int f = 0; f < kMI; ++f) { a_rd[f] ^= kABytes; b_rd[f] ^= kBBytes; }
+    // K step 3 of slab s, under it the reads of step 0 of slab s+1 and the first loads of slab s+2
+    step(1, 0, 0, kLdT);
   };
 
   const int nslab = (T + kTK - 1) / kTK;
-  // prologue: slab 0 through the registers into buffer 0, slabs 1 and 2 on their way
-  fetch_a(0, 0);
-  fetch_b(0, 0);
 #pragma unroll
-  for (int u = 0; u < 16; ++u) stage_unit(u, 0, 0);
-  __syncthreads();
-  fetch_a(1, 1);  // past the end: zeros
-  fetch_b(1, 1);
-  fetch_a(2, 0);
-  fetch_b(2, 0);
+  for (int l = 0; l < kL; ++l) issue_one(l);
+  next_slab();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  // (past the last slab every row is out of range: zeros go into the free buffer)
 #pragma unroll
-  for (int f = 0; f < kMI + kNI; ++f) read_one(0, 0, 0, f);
+  for (int l = 0; l < kLdT; ++l) issue_one(l);
+#pragma unroll
+  for (int f = 0; f < kMI + kNI; ++f) read_one(0, 0, f);
+  for (int s = 0; s < nslab; ++s) slab();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-  // one slab: on entry register set 0 holds (or is receiving) step 0 of slab s (buffer cur) and the
-  // staging registers of parity cur ^ 1 hold (or are receiving) slab s + 1, those of parity cur slab
-  // s + 2.  A register set is reloaded, with the slab two further on, as soon as it has been written to
-  // LDS: a load has more than a slab's worth of MFMAs to arrive.
-  auto slab = [&](int s, int cur) __attribute__((always_inline)) {
-    __builtin_amdgcn_sched_barrier(0);
-    step(0, cur, 1, 0, 0, 0);
-    step(1, cur, 2, 1, cur ^ 1, s + 3);
-    step(0, cur, 3, 2, cur ^ 1, s + 3);
-    // every read of this slab's buffer has returned once set 1 is complete; the barrier says: slab
-    // s + 1 is in LDS for everybody, this buffer is free
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    // step 3 of slab s, under it the reads of step 0 of slab s + 1
-    step(1, cur ^ 1, 0, 0, 0, 0);
-  };
-  int s = 0;
-  for (; s + 1 < nslab; s += 2) {
-    slab(s, 0);
-    slab(s + 1, 1);
-  }
-  if (s < nslab) slab(s, 0);
-
-  // epilogue: a lane holds row m of C and, per accumulator, columns 8 q + 4 g + {0..3}
-  // (q = 0..3).  Swapping the q-odd words of the lower half-wave with the q-even words of
-  // the upper half-wave leaves every lane with 8 consecutive columns: 16-byte stores.
-  const bool fast = (ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0) && (n0 + kTN <= N);
+  // epilogue: a lane holds row m of C and, per accumulator, columns 8 q + 4 g + {0..3} (q = 0..3)
+  if constexpr (OUT >= 2) {
+    float* const C = reinterpret_cast<float*>(Cv);
+    const bool fast = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0) && (n0 + kTN <= N);
 #pragma unroll
-  for (int i = 0; i < kMI; ++i) {
-    const int m = m0 + wm + i * 32 + col;
+    for (int i = 0; i < kMI; ++i) {
+      const int m = m0 + wm + i * 32 + col;
+      if (m >= M) continue;
 #pragma unroll
-    for (int j = 0; j < kNI; ++j) {
-      f32x16 a = acc[j][i];
-      if (ACC && fast) {
-        // swap the fp32 words, add what C holds (one 16-byte load per lane, the store's own layout)
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          float v[8];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(a[8 * h + e]),
-                                                            __float_as_uint(a[8 * h + 4 + e]), false, false);
-            v[e] = __uint_as_float(sw[0]);
-            v[4 + e] = __uint_as_float(sw[1]);
-          }
-          const int n = n0 + wn + j * 32 + 16 * h + 8 * g;
-          if (m < M) {
-            u32x4* cp = reinterpret_cast<u32x4*>(&C[(int64_t)m * ldc + n]);
-            const u32x4 old = *cp;
-            u32x4 o;
-            o.x = pack_bf16x2(v[0] + bf16_lo(old.x), v[1] + bf16_hi(old.x));
-            o.y = pack_bf16x2(v[2] + bf16_lo(old.y), v[3] + bf16_hi(old.y));
-            o.z = pack_bf16x2(v[4] + bf16_lo(old.z), v[5] + bf16_hi(old.z));
-            o.w = pack_bf16x2(v[6] + bf16_lo(old.w), v[7] + bf16_hi(old.w));
-            *cp = o;
-          }
-        }
-        continue;
-      }
-      if (ACC && m < M) {
-        // ragged edge: what C holds, read in the accumulator's own layout (4 consecutive columns per q)
+      for (int j = 0; j < kNI; ++j) {
+        const f32x16& a = acc[j][i];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int n = n0 + wn + j * 32 + 8 * q + 4 * g;
+          float* cp = C + (int64_t)m * ldc + n;
+          if (fast) {
+            f32x4 v = {a[4 * q + 0], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+            if (OUT == 3) {
+              const f32x4 old = *reinterpret_cast<const f32x4*>(cp);
+              v[0] += old[0]; v[1] += old[1]; v[2] += old[2]; v[3] += old[3];
+            }
+            *reinterpret_cast<f32x4*>(cp) = v;
+          } else {
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (n + e < N) a[4 * q + e] += bf16_bits_to_f32(C[(int64_t)m * ldc + n + e]);
+            for (int e = 0; e < 4; ++e)
+              if (n + e < N) cp[e] = (OUT == 3 ? cp[e] : 0.f) + a[4 * q + e];
+          }
         }
       }
+    }
+    return;
+  } else {
+    // Swapping the q-odd words of the lower half-wave with the q-even words of the upper half-wave
+    // leaves every lane with 8 consecutive columns: 16-byte stores.
+    uint16_t* const C = reinterpret_cast<uint16_t*>(Cv);
+    constexpr bool ACC = OUT == 1;
+    const bool fast = (ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0) && (n0 + kTN <= N);
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {  // q pair (2h, 2h+1)
-        const uint32_t e0 = pack_bf16x2(a[8 * h + 0], a[8 * h + 1]), e1 = pack_bf16x2(a[8 * h + 2], a[8 * h + 3]);
-        const uint32_t o0 = pack_bf16x2(a[8 * h + 4], a[8 * h + 5]), o1 = pack_bf16x2(a[8 * h + 6], a[8 * h + 7]);
-        const auto s0 = __builtin_amdgcn_permlane32_swap(e0, o0, false, false);
-        const auto s1 = __builtin_amdgcn_permlane32_swap(e1, o1, false, false);
-        u32x4 v;
-        v.x = s0[0]; v.y = s1[0]; v.z = s0[1]; v.w = s1[1];
-        const int n = n0 + wn + j * 32 + 16 * h + 8 * g;
-        if (fast) {
-          if (m < M) *reinterpret_cast<u32x4*>(&C[(int64_t)m * ldc + n]) = v;
-        } else if (m < M) {
-          const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    for (int i = 0; i < kMI; ++i) {
+      const int m = m0 + wm + i * 32 + col;
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (n + e < N) C[(int64_t)m * ldc + n + e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+      for (int j = 0; j < kNI; ++j) {
+        f32x16 a = acc[j][i];
+        if (ACC && fast) {
+          // swap the fp32 words, add what C holds (one 16-byte load per lane, the store's own layout)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(a[8 * h + e]),
+                                                              __float_as_uint(a[8 * h + 4 + e]), false, false);
+              v[e] = __uint_as_float(sw[0]);
+              v[4 + e] = __uint_as_float(sw[1]);
+            }
+            const int n = n0 + wn + j * 32 + 16 * h + 8 * g;
+            if (m < M) {
+              u32x4* cp = reinterpret_cast<u32x4*>(&C[(int64_t)m * ldc + n]);
+              const u32x4 old = *cp;
+              u32x4 o;
+              o.x = pack_bf16x2(v[0] + bf16_lo(old.x), v[1] + bf16_hi(old.x));
+              o.y = pack_bf16x2(v[2] + bf16_lo(old.y), v[3] + bf16_hi(old.y));
+              o.z = pack_bf16x2(v[4] + bf16_lo(old.z), v[5] + bf16_hi(old.z));
+              o.w = pack_bf16x2(v[6] + bf16_lo(old.w), v[7] + bf16_hi(old.w));
+              *cp = o;
+            }
+          }
+          continue;
+        }
+        if (ACC && m < M) {
+          // ragged edge: what C holds, read in the accumulator's own layout (4 consecutive columns per q)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int n = n0 + wn + j * 32 + 8 * q + 4 * g;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + e < N) a[4 * q + e] += bf16_bits_to_f32(C[(int64_t)m * ldc + n + e]);
+          }
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {  // q pair (2h, 2h+1)
+          const uint32_t e0 = pack_bf16x2(a[8 * h + 0], a[8 * h + 1]), e1 = pack_bf16x2(a[8 * h + 2], a[8 * h + 3]);
+          const uint32_t o0 = pack_bf16x2(a[8 * h + 4], a[8 * h + 5]), o1 = pack_bf16x2(a[8 * h + 6], a[8 * h + 7]);
+          const auto s0 = __builtin_amdgcn_permlane32_swap(e0, o0, false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(e1, o1, false, false);
+          u32x4 v;
+          v.x = s0[0]; v.y = s1[0]; v.z = s0[1]; v.w = s1[1];
+          const int n = n0 + wn + j * 32 + 16 * h + 8 * g;
+          if (fast) {
+            if (m < M) *reinterpret_cast<u32x4*>(&C[(int64_t)m * ldc + n]) = v;
+          } else if (m < M) {
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (n + e < N) C[(int64_t)m * ldc + n + e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+          }
         }
       }
     }
@@ -276,32 +317,50 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
 
 using namespace spx;
 
+#define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fname, what); } while (0)
+template <int OUT>
+static int launch_tn(const char* fname, const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                     int64_t ldc, int64_t M, int64_t N, int64_t T, void* stream) {
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  static std::atomic<uint64_t> lds_set;  // per kernel instantiation, one bit per device
+  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&tn::gemm_bf16_tn_kernel<OUT>), tn::kSmem,
+                                  lds_set, fname))
+    return rc;
+  const int tiles_m = (int)((M + tn::kTM - 1) / tn::kTM), tiles_n = (int)((N + tn::kTN - 1) / tn::kTN);
+  const dim3 grid((unsigned)(tiles_m * tiles_n)), block(tn::kThreads);
+  hipLaunchKernelGGL(tn::gemm_bf16_tn_kernel<OUT>, grid, block, tn::kSmem, st,
+                     reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb, c,
+                     ldc, (int)M, (int)N, (int)T, tiles_m, tiles_n);
+  return check_launch(fname);
+}
+
+static int gemm_tn_check(const char* fname, const void* a, int64_t lda, const void* b, int64_t ldb,
+                         const void* c, int64_t ldc, int64_t M, int64_t N, int64_t T) {
+  SPX_REQ_FN(M > 0 && N > 0 && T > 0, "M, N, T must be positive");
+  SPX_REQ_FN(M < (1ll << 31) && N < (1ll << 31) && T < (1ll << 31), "dimension too large");
+  SPX_REQ_FN(a && b && c, "null buffer");
+  SPX_REQ_FN(M % 8 == 0 && N % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0, "M, N, lda, ldb must be multiples of 8");
+  SPX_REQ_FN(lda >= M && ldb >= N && ldc >= N, "leading dimension too small");
+  SPX_REQ_FN(((uintptr_t)a | (uintptr_t)b) % 16 == 0, "a and b must be 16-byte aligned");
+  SPX_REQ_FN(((T + 4 * tn::kTK) * lda) * 2 < 0x7ffffff0ll && ((T + 4 * tn::kTK) * ldb) * 2 < 0x7ffffff0ll,
+             "each operand must span less than 2 GiB (32-bit buffer offsets)");
+  SPX_REQ_FN((int64_t)((M + tn::kTM - 1) / tn::kTM) * ((N + tn::kTN - 1) / tn::kTN) < (1ll << 31), "too many tiles");
+  return SPX_OK;
+}
+#undef SPX_REQ_FN
+
 extern "C" int spx_gemm_bf16_tn(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
                                 int64_t ldc, int64_t M, int64_t N, int64_t T, int accumulate,
                                 void* stream) {
-  SPX_REQUIRE(M > 0 && N > 0 && T > 0, "M, N, T must be positive");
-  SPX_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && T < (1ll << 31), "dimension too large");
-  SPX_REQUIRE(a && b && c, "null buffer");
-  SPX_REQUIRE(M % 8 == 0 && N % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0, "M, N, lda, ldb must be multiples of 8");
-  SPX_REQUIRE(lda >= M && ldb >= N && ldc >= N, "leading dimension too small");
-  SPX_REQUIRE(((uintptr_t)a | (uintptr_t)b) % 16 == 0, "a and b must be 16-byte aligned");
-  SPX_REQUIRE(((T + 4 * tn::kTK) * lda) * 2 < 0x7ffffff0ll && ((T + 4 * tn::kTK) * ldb) * 2 < 0x7ffffff0ll,
-              "each operand must span less than 2 GiB (32-bit buffer offsets)");
-  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  static std::atomic<uint64_t> lds_set[2];  // per kernel instantiation, one bit per device
-  const void* fn = accumulate ? reinterpret_cast<const void*>(&tn::gemm_bf16_tn_kernel<true>)
-                              : reinterpret_cast<const void*>(&tn::gemm_bf16_tn_kernel<false>);
-  if (int rc = ensure_dynamic_lds(fn, tn::kSmem, lds_set[accumulate ? 1 : 0], __func__)) return rc;
-  const int tiles_m = (int)((M + tn::kTM - 1) / tn::kTM), tiles_n = (int)((N + tn::kTN - 1) / tn::kTN);
-  const dim3 grid((unsigned)(tiles_m * tiles_n)), block(tn::kThreads);
-  auto ap = reinterpret_cast<const uint16_t*>(a);
-  auto bp = reinterpret_cast<const uint16_t*>(b);
-  auto cp = reinterpret_cast<uint16_t*>(c);
-  if (accumulate)
-    hipLaunchKernelGGL(tn::gemm_bf16_tn_kernel<true>, grid, block, tn::kSmem, st, ap, lda, bp, ldb, cp, ldc,
-                       (int)M, (int)N, (int)T, tiles_m, tiles_n);
-  else
-    hipLaunchKernelGGL(tn::gemm_bf16_tn_kernel<false>, grid, block, tn::kSmem, st, ap, lda, bp, ldb, cp, ldc,
-                       (int)M, (int)N, (int)T, tiles_m, tiles_n);
-  return check_launch(__func__);
+  if (int rc = gemm_tn_check(__func__, a, lda, b, ldb, c, ldc, M, N, T)) return rc;
+  return accumulate ? launch_tn<1>(__func__, a, lda, b, ldb, c, ldc, M, N, T, stream)
+                    : launch_tn<0>(__func__, a, lda, b, ldb, c, ldc, M, N, T, stream);
+}
+
+extern "C" int spx_gemm_bf16_tn_f32(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                                    int64_t ldc, int64_t M, int64_t N, int64_t T, int accumulate,
+                                    void* stream) {
+  if (int rc = gemm_tn_check(__func__, a, lda, b, ldb, c, ldc, M, N, T)) return rc;
+  return accumulate ? launch_tn<3>(__func__, a, lda, b, ldb, c, ldc, M, N, T, stream)
+                    : launch_tn<2>(__func__, a, lda, b, ldb, c, ldc, M, N, T, stream);
 }

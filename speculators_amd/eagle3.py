@@ -110,8 +110,9 @@ class Attention(nn.Module):
                                     pos.contiguous(), inv_freq, self.hq, self.hkv, self.d, pos_offset,
                                     kv_out=None if kvc is None else kvc.window(pos_offset))
             if kvc is not None:
-                out = A.ttt_attention_cached(q, k, v, kvc, mask, self.scaling)
-                return gemm.linear_staged(out.reshape(1, t, self.hq * self.d), W(self.o_proj.weight))
+                wo = W(self.o_proj.weight)
+                out = A.ttt_attention_cached(q, k, v, kvc, mask, self.scaling, out=wo.x_slot(t))
+                return gemm.linear_staged(out.reshape(1, t, self.hq * self.d), wo)
         else:
             q = gemm.linear_staged(x, W(self.q_proj.weight))
             k = gemm.linear_staged(x, W(self.k_proj.weight))
@@ -140,8 +141,10 @@ class MLP(nn.Module):
     def forward(self, x):
         W = self._stager.get
         # gate and up as one GEMM, SwiGLU on the two halves of its output
-        act = gemm.gate_up_swiglu(x, W(self.gate_proj.weight, self.up_proj.weight))
-        return gemm.linear_staged(act, W(self.down_proj.weight))
+        wd = W(self.down_proj.weight)
+        act = gemm.gate_up_swiglu(x, W(self.gate_proj.weight, self.up_proj.weight),
+                                  out=wd.x_slot(x.numel() // x.shape[-1]))
+        return gemm.linear_staged(act, wd)
 
 
 class _Prenormed(NamedTuple):
@@ -161,6 +164,7 @@ class DecoderLayer(nn.Module):
         super().__init__()
         self.first = layer_idx == 0
         self.cfg = cfg
+        self._stager = stager
         self.self_attn = Attention(cfg, (2 if self.first else 1) * cfg.hidden_size, stager)
         self.mlp = MLP(cfg, stager)
         self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps, stager)
@@ -184,8 +188,11 @@ class DecoderLayer(nn.Module):
             else:
                 residual = hidden
                 # both norms write straight into the halves of the 2H-wide projection input
+                att = self.self_attn
+                wqkv = self._stager.get(att.q_proj.weight, att.k_proj.weight, att.v_proj.weight)
                 xin = FO.pair_norm_cat(embeds, hidden, self.input_layernorm.gain,
-                                       self.hidden_norm.gain, eps)
+                                       self.hidden_norm.gain, eps,
+                                       out=None if att.qk_norm else wqkv.x_slot(hidden.shape[-2]))
             a = self.self_attn(xin, position_ids, pos_offset, inv_freq, cache, mask)
         else:
             if isinstance(x, _Prenormed):  # the previous layer already applied this layer's input norm
@@ -194,7 +201,8 @@ class DecoderLayer(nn.Module):
                 residual, xn = x, self.input_layernorm(x)
             a = self.self_attn(xn, position_ids, pos_offset, inv_freq, cache, mask)
         post = self.post_attention_layernorm
-        y, z = FO.add_rms_norm(residual, a, post.gain, post.eps)
+        wgu = self._stager.get(self.mlp.gate_proj.weight, self.mlp.up_proj.weight)
+        y, z = FO.add_rms_norm(residual, a, post.gain, post.eps, out=wgu.x_slot(a.shape[-2]))
         m = self.mlp(z)
         if next_norm is None:
             return y + m
@@ -293,7 +301,7 @@ class Eagle3DraftModel(nn.Module):
         cfg = self.config
         device = hidden_states.device
         t = hidden_states.shape[1]
-        self._stager.begin()
+        self._stager.begin(uses=ttt_steps)
         hidden_states = compute_input(hidden_states)
         if verifier_last_hidden_states is not None:
             verifier_last_hidden_states = compute_input(verifier_last_hidden_states)

@@ -67,7 +67,7 @@ class _AddRMSNorm(torch.autograd.Function):
     gradient that reaches ``s`` along the residual stream into the norm's input gradient."""
 
     @staticmethod
-    def forward(ctx, a, b, weight, eps):
+    def forward(ctx, a, b, weight, eps, out=None):
         _need_bf16(a, b, weight)
         h = a.shape[-1]
         a2, b2 = a.reshape(-1, h), b.reshape(-1, h)
@@ -77,7 +77,8 @@ class _AddRMSNorm(torch.autograd.Function):
             b2 = b2.contiguous()
         rows = a2.shape[0]
         s = torch.empty(rows, h, device=a.device, dtype=torch.bfloat16)
-        y = torch.empty(rows, h, device=a.device, dtype=torch.bfloat16)
+        y = out if out is not None and out.shape == (rows, h) and out.is_contiguous() else \
+            torch.empty(rows, h, device=a.device, dtype=torch.bfloat16)
         rstd = torch.empty(rows, device=a.device, dtype=torch.float32)
         w = weight.contiguous()
         _lib.call("spx_add_rmsnorm_fwd", _lib.ptr(a2), a2.stride(0), _lib.ptr(b2), b2.stride(0),
@@ -93,7 +94,7 @@ class _AddRMSNorm(torch.autograd.Function):
         s, w, rstd = ctx.saved_tensors
         rows, h = s.shape
         if dy is None:  # the normalised output was not used
-            return ds, ds, None, None
+            return ds, ds, None, None, None
         dy2 = dy.reshape(rows, h).to(torch.bfloat16)
         if dy2.stride(1) != 1:
             dy2 = dy2.contiguous()
@@ -110,12 +111,13 @@ class _AddRMSNorm(torch.autograd.Function):
                   _lib.ptr(ds2), ds2.stride(0) if ds2 is not None else 0, _lib.ptr(rstd), _lib.ptr(dx),
                   h, _lib.ptr(dw), _lib.ptr(scratch), rows, h, _lib.stream_ptr(s.device))
         dx = dx.view(ctx.shape)
-        return dx, dx, dw, None
+        return dx, dx, dw, None, None
 
 
-def add_rms_norm(a: torch.Tensor, b: torch.Tensor, weight: torch.Tensor, eps: float):
-    """``(a + b, rms_norm(a + b))``: the residual add in front of a norm, fused into it."""
-    return _AddRMSNorm.apply(a, b, weight, eps)
+def add_rms_norm(a: torch.Tensor, b: torch.Tensor, weight: torch.Tensor, eps: float, out=None):
+    """``(a + b, rms_norm(a + b))``: the residual add in front of a norm, fused into it.  ``out``:
+    a contiguous ``[rows, H]`` bf16 buffer for the normalised result."""
+    return _AddRMSNorm.apply(a, b, weight, eps, out)
 
 
 class _PairNormCat(torch.autograd.Function):
@@ -124,7 +126,7 @@ class _PairNormCat(torch.autograd.Function):
     models/eagle3/model_definitions.py:70-94)."""
 
     @staticmethod
-    def forward(ctx, a, b, wa, wb, eps):
+    def forward(ctx, a, b, wa, wb, eps, out=None):
         _need_bf16(a, b, wa, wb)
         h = a.shape[-1]
         a2, b2 = a.reshape(-1, h), b.reshape(-1, h)
@@ -133,7 +135,8 @@ class _PairNormCat(torch.autograd.Function):
         if b2.stride(1) != 1:
             b2 = b2.contiguous()
         rows = a2.shape[0]
-        out = torch.empty(rows, 2 * h, device=a.device, dtype=torch.bfloat16)
+        if out is None or out.shape != (rows, 2 * h) or not out.is_contiguous():
+            out = torch.empty(rows, 2 * h, device=a.device, dtype=torch.bfloat16)
         rstd = torch.empty(2, rows, device=a.device, dtype=torch.float32)
         wa, wb = wa.contiguous(), wb.contiguous()
         st = _lib.stream_ptr(a.device)
@@ -167,12 +170,12 @@ class _PairNormCat(torch.autograd.Function):
                           dy2.stride(0), _lib.ptr(rstd[i]), _lib.ptr(dx), h, _lib.ptr(dw),
                           _lib.ptr(scratch), rows, h, st)
             grads.append((dx.view(ctx.shapes[i]) if dx is not None else None, dw))
-        return grads[0][0], grads[1][0], grads[0][1], grads[1][1], None
+        return grads[0][0], grads[1][0], grads[0][1], grads[1][1], None, None
 
 
-def pair_norm_cat(a, b, weight_a, weight_b, eps: float) -> torch.Tensor:
-    """See ``_PairNormCat``."""
-    return _PairNormCat.apply(a, b, weight_a, weight_b, eps)
+def pair_norm_cat(a, b, weight_a, weight_b, eps: float, out=None) -> torch.Tensor:
+    """See ``_PairNormCat``.  ``out``: a contiguous ``[rows, 2H]`` bf16 buffer for the result."""
+    return _PairNormCat.apply(a, b, weight_a, weight_b, eps, out)
 
 
 class _RopeRelayout(torch.autograd.Function):

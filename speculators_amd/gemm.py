@@ -4,8 +4,8 @@
 (``x @ weight.T``) for bf16 tensors.  The backward computes the input gradient
 with the same NT kernel against a transposed copy of the weight
 (``weight_t``, ``[K, N]`` contiguous) -- kept by the caller for frozen weights
-such as ``lm_head`` (model.py:70-71) so it is made once -- and leaves the
-weight gradient (a TN product) to the rocBLAS/hipBLASLt matmul of PyTorch.
+such as ``lm_head`` (model.py:70-71) so it is made once.  The weight gradient is the
+transposed-operand product ``gemm_tn``.
 The models call the ``*_staged`` forms below with the compute weights of ``weights.WeightStager``.
 """
 
@@ -51,9 +51,10 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
 
 
 def gemm_tn(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
-            accumulate: bool = False) -> torch.Tensor:
-    """``a[T, M].T @ b[T, N] -> [M, N]`` (bf16, fp32 accumulation): the weight gradient
-    ``dY.T @ X`` of a Linear.  ``accumulate`` adds the product to ``out``."""
+            accumulate: bool = False, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """``a[T, M].T @ b[T, N] -> [M, N]`` (bf16 operands, fp32 accumulation): the weight gradient
+    ``dY.T @ X`` of a Linear.  ``accumulate`` adds the product to ``out``.  The result is bf16 or,
+    with ``out_dtype=torch.float32`` (or an fp32 ``out``), fp32."""
     if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
         raise _lib.SpxError("gemm_tn takes bf16 operands")
     if a.dim() != 2 or b.dim() != 2 or a.shape[0] != b.shape[0]:
@@ -67,16 +68,19 @@ def gemm_tn(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
     if out is None:
         if accumulate:
             raise ValueError("accumulate needs the tensor to add to")
-        out = torch.empty(m, n, device=a.device, dtype=torch.bfloat16)
-    elif out.shape != (m, n) or out.dtype != torch.bfloat16 or out.stride(1) != 1:
-        raise ValueError(f"out must be a bf16 [{m}, {n}] tensor with unit column stride")
+        if out_dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError("out_dtype must be bfloat16 or float32")
+        out = torch.empty(m, n, device=a.device, dtype=out_dtype)
+    elif out.shape != (m, n) or out.dtype not in (torch.bfloat16, torch.float32) or out.stride(1) != 1:
+        raise ValueError(f"out must be a bf16 or fp32 [{m}, {n}] tensor with unit column stride")
+    entry = "spx_gemm_bf16_tn_f32" if out.dtype == torch.float32 else "spx_gemm_bf16_tn"
     # 32-bit byte offsets inside the kernel: a contraction that spans 2 GiB or more of an
     # operand is fed in bands of rows, every band after the first added to the result
     rows = max(_MAX_SPAN // (2 * max(a.stride(0), b.stride(0))) - 256, 1)
     st = _lib.stream_ptr(a.device)
     for t0 in range(0, t, rows):
         at, bt = a[t0:t0 + rows], b[t0:t0 + rows]
-        _lib.call("spx_gemm_bf16_tn", _lib.ptr(at), at.stride(0), _lib.ptr(bt), bt.stride(0),
+        _lib.call(entry, _lib.ptr(at), at.stride(0), _lib.ptr(bt), bt.stride(0),
                   _lib.ptr(out), out.stride(0), m, n, at.shape[0], int(accumulate or t0 > 0), st)
     return out
 
@@ -99,7 +103,9 @@ class _Linear(torch.autograd.Function):
             wt = weight_t if weight_t is not None else weight.t().contiguous()
             dx = gemm_nt(dy2, wt).view(ctx.x_shape)
         if ctx.needs_input_grad[1]:
-            dw = torch.matmul(dy2.t(), x2)
+            from .weights import wgrad_product
+
+            dw = wgrad_product(dy2 if dy2.stride(1) == 1 else dy2.contiguous(), x2, None).to(weight.dtype)
         return dx, dw, None
 
 
@@ -111,9 +117,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor | None 
 
 class _StagedLinear(torch.autograd.Function):
     """``x @ w.T`` against a staged weight (``weights.Staged``): on the MFMA kernel of this library
-    (``hip``) or on PyTorch's hipBLASLt matmul.  The weight gradient is added into the staged
-    weight's fp32 accumulator inside the GEMM; the first such product of a backward returns the
-    accumulator to autograd, the others nothing (see ``weights``)."""
+    (``hip``) or on PyTorch's hipBLASLt matmul.  The weight gradient is left to the staged weight,
+    which computes it over all of its uses at once (``weights.Staged.defer``)."""
 
     @staticmethod
     def forward(ctx, x, _token, staged, hip: bool):
@@ -124,6 +129,7 @@ class _StagedLinear(torch.autograd.Function):
         y = gemm_nt(x2, w) if hip else torch.nn.functional.linear(x2, w)
         ctx.save_for_backward(x2, w)
         ctx.staged, ctx.hip, ctx.x_shape = staged, hip, x.shape
+        ctx.slot = staged.take(x2) if ctx.needs_input_grad[1] else -1
         return y.view(*x.shape[:-1], w.shape[0])
 
     @staticmethod
@@ -134,7 +140,7 @@ class _StagedLinear(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             dx = (gemm_nt(dy2, ctx.staged.wt) if ctx.hip else torch.matmul(dy2, w)).view(ctx.x_shape)
         if ctx.needs_input_grad[1]:
-            dw = ctx.staged.add_wgrad(dy2, x2)
+            dw = ctx.staged.defer(ctx.slot, dy2, x2)
         return dx, dw, None, None
 
 
@@ -151,8 +157,9 @@ class _QKVRope(torch.autograd.Function):
     """q/k/v projections of one input as ONE GEMM against the staged concatenation of the three
     weights, followed by the rotary embedding + head-major relayout of each part.  The backward
     undoes the relayout into the three column blocks of one ``[T, Nq + 2 Nkv]`` buffer, so the
-    input gradient is one GEMM (no per-projection partial results to add up) and the weight
-    gradient one GEMM that accumulates across TTT steps in fp32."""
+    input gradient is one GEMM (no per-projection partial results to add up); that buffer is the
+    step's slot of the staged weight's output-gradient buffer, from which the weight gradient of
+    all TTT steps comes as one product."""
 
     @staticmethod
     def forward(ctx, x, _token, staged, position_ids, inv_freq, hq, hkv, d, offset, kv_out=None):
@@ -180,6 +187,7 @@ class _QKVRope(torch.autograd.Function):
             col += heads * d
         ctx.save_for_backward(x2, wcat, position_ids, inv_freq)
         ctx.meta = (x.shape, hq, hkv, d, offset, n, staged)
+        ctx.slot = staged.take(x2) if ctx.needs_input_grad[1] else -1
         ctx.set_materialize_grads(False)
         return tuple(outs)
 
@@ -189,7 +197,9 @@ class _QKVRope(torch.autograd.Function):
         shape, hq, hkv, d, offset, n, staged = ctx.meta
         t = x2.shape[0]
         st = _lib.stream_ptr(x2.device)
-        dqkv = torch.empty(t, n, device=x2.device, dtype=torch.bfloat16)
+        dqkv = staged.dy_slot(ctx.slot, t) if ctx.needs_input_grad[1] else None
+        if dqkv is None:
+            dqkv = torch.empty(t, n, device=x2.device, dtype=torch.bfloat16)
         col = 0
         for g, heads, rotate in ((dq, hq, 1), (dk, hkv, 1), (dv, hkv, 0)):
             part = dqkv[:, col:]
@@ -208,7 +218,7 @@ class _QKVRope(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             dx = torch.matmul(dqkv, wcat).view(shape)
         if ctx.needs_input_grad[1]:
-            dw = staged.add_wgrad(dqkv, x2)
+            dw = staged.defer(ctx.slot, dqkv, x2)
         return (dx, dw) + (None,) * 8
 
 
@@ -223,11 +233,13 @@ def qkv_rope(x, staged, position_ids, inv_freq, hq: int, hkv: int, d: int, offse
 class _GateUpSwiGLU(torch.autograd.Function):
     """``silu(x @ Wg.T) * (x @ Wu.T)`` with the two projections as ONE GEMM against the staged
     concatenation of the two weights; the SwiGLU kernels read (and, in the backward, write) the two
-    column halves of the merged ``[T, 2F]`` buffer in place, so the input gradient is one GEMM and
-    the weight gradient one GEMM that accumulates across TTT steps in fp32."""
+    column halves of the merged ``[T, 2F]`` buffer in place, so the input gradient is one GEMM; the
+    backward's ``[T, 2F]`` buffer is the step's slot of the staged weight's output-gradient buffer,
+    from which the weight gradient of all TTT steps comes as one product.  ``out``: where the
+    result goes (the input slot of the down projection's staged weight)."""
 
     @staticmethod
-    def forward(ctx, x, _token, staged):
+    def forward(ctx, x, _token, staged, out=None):
         if x.dtype != torch.bfloat16:
             raise _lib.SpxError("the HIP layer kernels take bf16 tensors")
         wcat = staged.w
@@ -235,11 +247,13 @@ class _GateUpSwiGLU(torch.autograd.Function):
         f = wcat.shape[0] // 2
         gu = torch.nn.functional.linear(x2, wcat)  # [T, 2F]
         rows = x2.shape[0]
-        out = torch.empty(rows, f, device=x.device, dtype=torch.bfloat16)
+        if out is None or out.shape != (rows, f) or not out.is_contiguous():
+            out = torch.empty(rows, f, device=x.device, dtype=torch.bfloat16)
         _lib.call("spx_swiglu_rows_fwd", _lib.ptr(gu), 2 * f, _lib.ptr(gu[:, f:]), 2 * f, _lib.ptr(out), f,
                   rows, f, _lib.stream_ptr(x.device))
         ctx.save_for_backward(x2, gu, wcat)
         ctx.meta = (x.shape, f, staged)
+        ctx.slot = staged.take(x2) if ctx.needs_input_grad[1] else -1
         return out.view(*x.shape[:-1], f)
 
     @staticmethod
@@ -250,7 +264,9 @@ class _GateUpSwiGLU(torch.autograd.Function):
         d2 = dout.reshape(rows, f).to(torch.bfloat16)
         if d2.stride(1) != 1 or d2.stride(0) % 8:
             d2 = d2.contiguous()
-        dgu = torch.empty(rows, 2 * f, device=x2.device, dtype=torch.bfloat16)
+        dgu = staged.dy_slot(ctx.slot, rows) if ctx.needs_input_grad[1] else None
+        if dgu is None:
+            dgu = torch.empty(rows, 2 * f, device=x2.device, dtype=torch.bfloat16)
         _lib.call("spx_swiglu_rows_bwd", _lib.ptr(gu), 2 * f, _lib.ptr(gu[:, f:]), 2 * f, _lib.ptr(d2),
                   d2.stride(0), _lib.ptr(dgu), 2 * f, _lib.ptr(dgu[:, f:]), 2 * f, rows, f,
                   _lib.stream_ptr(x2.device))
@@ -258,11 +274,11 @@ class _GateUpSwiGLU(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             dx = torch.matmul(dgu, wcat).view(shape)
         if ctx.needs_input_grad[1]:
-            dw = staged.add_wgrad(dgu, x2)
-        return dx, dw, None
+            dw = staged.defer(ctx.slot, dgu, x2)
+        return dx, dw, None, None
 
 
-def gate_up_swiglu(x, staged):
+def gate_up_swiglu(x, staged, out=None):
     """See ``_GateUpSwiGLU``; ``staged`` holds the row-wise concatenation of the gate and up
     weights."""
-    return _GateUpSwiGLU.apply(x, staged.token, staged)
+    return _GateUpSwiGLU.apply(x, staged.token, staged, out)

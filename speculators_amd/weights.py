@@ -12,14 +12,19 @@ touches is *staged* once per forward:
     tensor hooks and post-accumulate-grad hooks see it like any other gradient, and it is cast to
     the parameter's dtype there (fp32 for master weights);
   * a weight that is applied several times in one forward (once per TTT step) does not hand
-    autograd one weight-sized gradient per use: the uses add their products into ONE fp32
-    accumulator inside the GEMM (``out_dtype=float32``, beta = 1), the use whose backward runs
-    first returns that accumulator to autograd and the others return nothing.  No rounding happens
-    between the uses.  Autograd casts a gradient to the dtype of the tensor it belongs to (and
-    would copy the accumulator, half filled, into bf16), so the accumulator does not travel as
-    the gradient of the bf16 weight: the staging node has a second, fp32 output of the weight's
-    shape that occupies no memory (``Staged.token``, one element expanded), the products take
-    it as their differentiable input and return the accumulator as ITS gradient;
+    autograd one weight-sized gradient per use, and its gradient is not summed over the uses in
+    memory either: the inputs ``X_j`` of its uses lie one after the other in ONE buffer
+    (``Staged.x_slot``: the kernel that produces an input writes it there) and so do the output
+    gradients ``dY_j`` of the backward, so that the weight gradient of all uses is ONE product
+    ``[dY_0; dY_1; ...]^T [X_0; X_1; ...]`` with the contraction running over ``uses * T`` rows
+    (``spx_gemm_bf16_tn_f32``): the sum over the uses happens in the MFMA accumulators, in fp32,
+    and the gradient is written once.  That product runs in the staging node's backward, which
+    autograd calls after every use has run its own.  The node has a second, fp32 output of the
+    weight's shape that occupies no memory (``Staged.token``, one element expanded); the
+    products take it as their differentiable input, and the first one to run its backward
+    returns an equally empty marker for it so that the node is reached.  A use whose input
+    is not in the buffer (nobody asked for the slot, or it was full) is added by a product of
+    its own (accumulating in fp32);
   * frozen weights (``lm_head``, ``verifier_lm_head``, ``embed_tokens``, ``verifier_norm``) are
     cast (and transposed where the backward needs it) once and kept until the parameter changes:
     the key is ``(data_ptr, _version, dtype)``; ``WeightStager.invalidate()`` drops every kept
@@ -73,19 +78,45 @@ def _cat_bf16(params) -> torch.Tensor:
     return out
 
 
+def _tn_ok(t: torch.Tensor) -> bool:
+    return (t.dtype == torch.bfloat16 and t.stride(1) == 1 and t.shape[1] % 8 == 0
+            and t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0)
+
+
+def wgrad_product(dy: torch.Tensor, x: torch.Tensor, acc: torch.Tensor | None) -> torch.Tensor:
+    """``acc (+)= dy.T @ x`` with an fp32 result: on the transposing MFMA kernel of this library
+    where its alignment rules hold, else on PyTorch's matmul."""
+    if _tn_ok(dy) and _tn_ok(x):
+        from .gemm import gemm_tn
+
+        if acc is None:
+            return gemm_tn(dy, x, out_dtype=torch.float32)
+        return gemm_tn(dy, x, acc, accumulate=True)
+    if acc is None:
+        return torch.mm(dy.t(), x, out_dtype=torch.float32)
+    return torch.addmm(acc, dy.t(), x, out_dtype=torch.float32, out=acc)
+
+
 class Staged:
     """One compute weight of this forward.  ``w``: bf16 ``[rows, cols]`` (or 1-D for a norm gain);
-    ``rows_of``: the row count of every parameter in it; ``acc``: the fp32 gradient accumulator of
-    the running backward (None outside one)."""
+    ``rows_of``: the row count of every parameter in it; ``uses``: how many products the forward
+    is expected to run against it (the size of the input / output-gradient buffers)."""
 
-    __slots__ = ("w", "token", "rows_of", "acc", "_wt")
+    __slots__ = ("w", "token", "rows_of", "uses", "_wt", "_xs", "_fill", "_dys", "_live", "_extras",
+                 "_marked")
 
-    def __init__(self, w, rows_of):
+    def __init__(self, w, rows_of, uses: int = 1):
         self.w = w
         self.token = None  # fp32 stand-in of w's shape that carries the gradient edge (trainable only)
         self.rows_of = rows_of
-        self.acc = None
+        self.uses = uses
         self._wt = None
+        self._xs = None    # [uses * T, cols]: the inputs of the uses, one after the other
+        self._fill = 0     # rows of _xs taken by products so far
+        self._dys = None   # [uses * T, rows]: the output gradients, same row positions (backward only)
+        self._live = []    # (first row, rows) of the uses whose backward has run
+        self._extras = []  # (dy, x) of uses outside the buffers
+        self._marked = False
 
     @property
     def trainable(self) -> bool:
@@ -98,20 +129,81 @@ class Staged:
             self._wt = self.w.detach().t().contiguous()
         return self._wt
 
-    def add_wgrad(self, dy2: torch.Tensor, x2: torch.Tensor):
-        """``acc += dy2.T @ x2`` in fp32 inside the GEMM.  Returns the accumulator if this call
-        created it (the caller returns it to autograd as the gradient of ``token``), else None."""
-        if self.acc is None:
-            self.acc = torch.mm(dy2.t(), x2, out_dtype=torch.float32)
-            return self.acc
-        torch.addmm(self.acc, dy2.t(), x2, out_dtype=torch.float32, out=self.acc)
-        return None
+    # ---- forward side
+    def x_slot(self, rows: int):
+        """Where the input ``[rows, cols]`` of the next product against this weight should be
+        written so that its weight gradient joins the one product over all uses; None when
+        there is nothing to gain (frozen weight, no graph, a single use) or no room."""
+        if self.token is None or self.uses <= 1 or not torch.is_grad_enabled():
+            return None
+        if self._xs is None:
+            self._xs = torch.empty(self.uses * rows, self.w.shape[1], device=self.w.device,
+                                   dtype=torch.bfloat16)
+        if self._fill + rows > self._xs.shape[0]:
+            return None
+        return self._xs[self._fill:self._fill + rows]
+
+    def take(self, x2: torch.Tensor) -> int:
+        """Called by a product's forward with its input: the first row of ``x2`` in the input
+        buffer if it is the slot ``x_slot`` handed out (the slot is then taken), else -1."""
+        xs = self._xs
+        if xs is None:
+            return -1
+        rows = x2.shape[0]
+        if (x2.data_ptr() == xs.data_ptr() + self._fill * xs.stride(0) * 2 and x2.is_contiguous()
+                and x2.shape[1] == xs.shape[1] and self._fill + rows <= xs.shape[0]):
+            self._fill += rows
+            return self._fill - rows
+        return -1
+
+    # ---- backward side
+    def dy_slot(self, r0: int, rows: int):
+        """Where the output gradient of the use at rows ``r0`` belongs (None for a use outside the
+        buffers): a backward that allocates its own result writes it here."""
+        if r0 < 0:
+            return None
+        if self._dys is None:
+            self._dys = torch.empty(self._xs.shape[0], self.w.shape[0], device=self.w.device,
+                                    dtype=torch.bfloat16)
+        return self._dys[r0:r0 + rows]
+
+    def defer(self, r0: int, dy2: torch.Tensor, x2: torch.Tensor):
+        """Record one use's ``(dy, x)`` for the weight-gradient product the staging node runs.
+        Returns what the calling backward returns as the gradient of ``token``."""
+        if r0 >= 0:
+            slot = self.dy_slot(r0, dy2.shape[0])
+            if dy2.data_ptr() != slot.data_ptr():
+                slot.copy_(dy2)
+            self._live.append((r0, dy2.shape[0]))
+        else:
+            self._extras.append((dy2, x2))
+        if self._marked:
+            return None
+        self._marked = True
+        return torch.zeros(1, device=self.w.device, dtype=torch.float32).expand(self.w.shape)
+
+    def finish(self):
+        """The fp32 weight gradient of every recorded use (None if there is none): one product
+        per run of adjacent uses in the buffers -- normally one -- plus one per outside use."""
+        acc = None
+        runs: list = []
+        for r0, n in sorted(self._live):
+            if runs and runs[-1][0] + runs[-1][1] == r0:
+                runs[-1][1] += n
+            else:
+                runs.append([r0, n])
+        for r0, n in runs:
+            acc = wgrad_product(self._dys[r0:r0 + n], self._xs[r0:r0 + n], acc)
+        for dy2, x2 in self._extras:
+            acc = wgrad_product(dy2, x2, acc)
+        self._dys, self._live, self._extras, self._marked = None, [], [], False
+        return acc
 
 
 class _Stage(torch.autograd.Function):
     """params -> (their bf16 row-wise concatenation, the fp32 token that carries its gradient);
-    backward: split the token's gradient, cast to each parameter's dtype.  That gradient is
-    normally the fp32 accumulator of ``Staged.add_wgrad``."""
+    backward: the weight-gradient product over all recorded uses (``Staged.finish``), split and
+    cast to each parameter's dtype."""
 
     @staticmethod
     def forward(ctx, staged: Staged, *params):
@@ -124,11 +216,16 @@ class _Stage(torch.autograd.Function):
             w = _cat_bf16(params)
         token = torch.zeros(1, device=w.device, dtype=torch.float32).expand(w.shape)
         ctx.mark_non_differentiable(w)
+        ctx.set_materialize_grads(False)
         return w, token
 
     @staticmethod
     def backward(ctx, _gw, g):
-        ctx.staged.acc = None  # consumed: a later backward through a retained graph starts afresh
+        # g is the marker of ``Staged.defer`` (no memory behind it): the gradient is computed here,
+        # now that every use has run its backward
+        acc = ctx.staged.finish()
+        if acc is not None:
+            g = acc
         if g is None:
             return (None,) * (1 + len(ctx.rows))
         parts = g.split(ctx.rows, dim=0) if len(ctx.rows) > 1 else (g,)
@@ -149,9 +246,13 @@ class WeightStager:
     def __init__(self):
         self._fwd: dict = {}
         self._frozen: dict = {}
+        self._uses = 1
 
-    def begin(self):
+    def begin(self, uses: int = 1):
+        """``uses``: how often the forward applies each trainable layer weight (the TTT / MTP
+        step count)."""
         self._fwd = {}
+        self._uses = max(int(uses), 1)
 
     def invalidate(self):
         """Forget every kept copy of a frozen weight (they are rebuilt on the next forward)."""
@@ -170,7 +271,7 @@ class WeightStager:
                 raise _lib.SpxError("libspx_hip works on HIP device tensors only (got a CPU parameter)")
         rows_of = [p.shape[0] for p in params]
         if torch.is_grad_enabled() and any(p.requires_grad for p in params):
-            st = Staged(None, rows_of)
+            st = Staged(None, rows_of, self._uses)
             st.w, st.token = _Stage.apply(st, *params)
         else:
             fkey = tuple((p.data_ptr(), p._version, p.dtype) for p in params)

@@ -100,6 +100,49 @@ def test_gemm_tn_matches_fp32_reference(t, m, n, accumulate):
     assert (got - ref).abs().max() <= 2 ** -8 * ref.abs().max() + 1e-3
 
 
+@pytest.mark.parametrize("t,m,n", [(72, 8, 8), (200, 264, 520), (129, 40, 1000), (4096, 512, 256), (257, 776, 392)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_gemm_tn_fp32_result(t, m, n, accumulate):
+    """The same product with an fp32 result: no rounding of the result at all, and accumulation
+    over calls adds in fp32 (the gradient of an fp32 master weight summed over the TTT steps)."""
+    from speculators_amd.gemm import gemm_tn
+
+    g = torch.Generator().manual_seed(3 * t + m + n)
+    a = torch.randn(t, m, generator=g).bfloat16()
+    b = torch.randn(t, n, generator=g).bfloat16()
+    ref = a.double().T @ b.double()
+    if accumulate:
+        c0 = torch.randn(m, n, generator=g) * 30
+        out_full = torch.full((m, n + 12), 7.0, device="cuda")
+        out = out_full[:, 4:4 + n]
+        out.copy_(c0)
+        got = gemm_tn(a.cuda(), b.cuda(), out, accumulate=True)
+        assert got.data_ptr() == out.data_ptr()
+        assert (out_full[:, :4] == 7).all() and (out_full[:, 4 + n:] == 7).all()
+        ref = ref + c0.double()
+    else:
+        got = gemm_tn(a.cuda(), b.cuda(), out_dtype=torch.float32)
+    assert got.dtype == torch.float32
+    # fp32 accumulation of t products of bf16 values
+    assert (got.double().cpu() - ref).abs().max() <= 2e-6 * t ** 0.5 * ref.abs().max() + 1e-5
+
+
+def test_gemm_tn_fp32_accumulates_like_one_fp32_sum():
+    """Seven calls into one fp32 accumulator (one per TTT step) equal the fp32 sum of the seven
+    products to fp32 rounding, where a bf16 accumulator would lose 2^-8 per call."""
+    from speculators_amd.gemm import gemm_tn
+
+    g = torch.Generator(device="cuda").manual_seed(2)
+    acc = torch.zeros(512, 768, device="cuda")
+    want = torch.zeros(512, 768, device="cuda", dtype=torch.float64)
+    for _ in range(7):
+        dy = torch.randn(1024, 512, device="cuda", generator=g).bfloat16()
+        x = torch.randn(1024, 768, device="cuda", generator=g).bfloat16()
+        gemm_tn(dy, x, acc, accumulate=True)
+        want += dy.double().t() @ x.double()
+    assert (acc.double() - want).abs().max() <= 1e-5 * want.abs().max()
+
+
 def test_gemm_tn_strided_operands_and_output():
     from speculators_amd.gemm import gemm_tn
 
