@@ -346,7 +346,11 @@ class Eagle3DraftModel(nn.Module):
             # looked up without a graph whatever embed_requires_grad says, as the reference does
             # (models/eagle3/core.py:270-271): the flag only marks the parameter as trainable
             with torch.no_grad():
-                embeds = F.embedding(input_ids, self.embed_tokens.weight)
+                # (the looked-up rows are cast to bf16 before the norm either way)
+                table = self.embed_tokens.weight
+                if not table.requires_grad:
+                    table = self._stager.get(table).w  # frozen: its bf16 copy is made once and kept
+                embeds = F.embedding(input_ids, table)
             y = (embeds.to(hidden.dtype), hidden)
             normed = None
             last = len(self.layers) - 1

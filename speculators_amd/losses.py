@@ -135,10 +135,13 @@ class _FusedLoss(torch.autograd.Function):
         lead = used.shape[:-1]
         am_d, am_t, lse_t = am_d.view(lead), am_t.view(lead), lse_t.view(lead)
         ctx.mark_non_differentiable(am_d, am_t, lse_t)
+        ctx.set_materialize_grads(False)  # no zero tensors for the outputs that carry no gradient
         return loss.view(lead), am_d, am_t, lse_t
 
     @staticmethod
     def backward(ctx, grad_rows, _gd, _gt, _gl):
+        if grad_rows is None:
+            return (None,) * 7
         x, y, lse_d, lse_t, extra, am_t = ctx.saved_tensors
         rows, vocab = x.shape
         full_rows = 1
@@ -200,11 +203,15 @@ class _HeadFusedLoss(torch.autograd.Function):
         ctx.save_for_backward(x, None if op == OP_CE else y, lse_d, lse_t, extra, am_t, weight_t)
         ctx.op, ctx.total_rows = op, logits.shape[0]
         ctx.mark_non_differentiable(am_d, am_t, lse_t, logits)
+        ctx.set_materialize_grads(False)  # no [T, Vd] zeros for the logits, which carry no gradient
         return loss, am_d, am_t, lse_t, logits
 
     @staticmethod
     def backward(ctx, grad_rows, _gd, _gt, _gl, _glogits):
         from .gemm import gemm_nt
+
+        if grad_rows is None:
+            return (None,) * 9
 
         x, y, lse_d, lse_t, extra, am_t, weight_t = ctx.saved_tensors
         rows, vocab = x.shape
@@ -407,11 +414,15 @@ class _HeadLabelCE(torch.autograd.Function):
         ctx.save_for_backward(logits, labels, out[1], weight_t)
         ctx.ignore_index = int(ignore_index)
         ctx.mark_non_differentiable(logits)
+        ctx.set_materialize_grads(False)  # no [rows, V] zeros for the logits, which carry no gradient
         return out[0], logits
 
     @staticmethod
     def backward(ctx, grad_rows, _grad_logits):
         from .gemm import gemm_nt
+
+        if grad_rows is None:
+            return (None,) * 5
 
         logits, labels, lse, weight_t = ctx.saved_tensors
         rows, vocab = logits.shape
