@@ -80,13 +80,15 @@ class MTPLayer(nn.Module):
     def forward(self, hidden, embeds, position_ids, inv_freq, mask):
         # both norms write into the halves of the 2H-wide projection input; each residual add is
         # fused into the norm that follows it
+        rows = hidden.shape[-2]
+        w_in = self._stager.get(self.input_proj.weight)
         x = gemm.linear_staged(
             FO.pair_norm_cat(embeds, hidden, self.token_layernorm.gain, self.hidden_layernorm.gain,
-                             self.token_layernorm.eps),
-            self._stager.get(self.input_proj.weight))
+                             self.token_layernorm.eps, out=w_in.x_slot(rows)), w_in)
         a = self.self_attn(self.input_layernorm(x), position_ids, 0, inv_freq, {}, mask)
         post, final = self.post_attention_layernorm, self.final_layernorm
-        y, z = FO.add_rms_norm(x, a, post.gain, post.eps)
+        w_gu = self._stager.get(self.mlp.gate_proj.weight, self.mlp.up_proj.weight)
+        y, z = FO.add_rms_norm(x, a, post.gain, post.eps, out=w_gu.x_slot(rows))
         _, out = FO.add_rms_norm(y, self.mlp(z), final.gain, final.eps)
         return out
 
@@ -134,7 +136,7 @@ class MTPDraftModel(nn.Module):
             raise NotImplementedError(
                 "the HIP MTP path takes packed rows without padding masks (attention_mask=None, "
                 "as the training collate produces them)")
-        self._stager.begin()
+        self._stager.begin(uses=cfg.num_speculative_steps)
         hidden_states = compute_input(hidden_states)
         input_ids = input_ids.long()
         device = input_ids.device

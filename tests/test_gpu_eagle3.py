@@ -285,6 +285,93 @@ def test_requires_bf16_and_hip_tensors():
         model(hs.cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.cuda(), ttt_steps=1)
 
 
+def test_weight_gradient_over_all_steps_in_one_product():
+    """The decoder projections' weight gradients come from one product over the stacked inputs and
+    output gradients of all TTT steps, run when autograd reaches the staging node.  That must be
+    invisible: ``torch.autograd.grad`` and ``backward()`` agree bit for bit, a retained graph can be
+    walked twice, a hook on the parameter sees the gradient, and the result equals the step-by-step
+    sum (the same model run with one use per weight expected, i.e. one product per step)."""
+    shape = _shape()
+    w = {k_: v.bfloat16() for k_, v in OE.random_weights(shape, seed=6, std=0.05).items()}
+    hs, ids, doc, mask, pos, vl = _batch(shape, 160, 3, [90, 60])
+    args = (hs.bfloat16().cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.bfloat16().cuda())
+    for dtype, auto in ((torch.bfloat16, False), (torch.float32, True)):
+        model = _make(shape, w, dtype)
+        names = [n for n, p in model.named_parameters() if p.requires_grad]
+        params = [p for _, p in model.named_parameters() if p.requires_grad]
+
+        def fwd():
+            with torch.autocast("cuda", dtype=torch.bfloat16, enabled=auto):
+                return model(*args, ttt_steps=3, ttt_step_loss_decay=0.8)[1]
+
+        seen = {}
+        layer = model.layers[0]
+        handle = layer.mlp.gate_proj.weight.register_hook(lambda g: seen.setdefault("gate", g.clone()))
+        loss = fwd()
+        loss.backward(retain_graph=True)
+        handle.remove()
+        g_bwd = [p.grad.clone() for p in params]
+        assert torch.equal(seen["gate"], layer.mlp.gate_proj.weight.grad)
+        assert all(g.dtype == dtype for g in g_bwd)
+        # the same graph again: the gradients double (to one more rounding of the sum)
+        loss.backward()
+        for n, p, g in zip(names, params, g_bwd, strict=True):
+            want = 2 * g.float()
+            assert (p.grad.float() - want).abs().max() <= 2 ** -7 * want.abs().max() + 1e-12, n
+        model.zero_grad(set_to_none=True)
+        g_fn = torch.autograd.grad(fwd(), params)
+        for n, a, b in zip(names, g_fn, g_bwd, strict=True):
+            assert torch.equal(a, b), n
+        # one product per step instead (no stacking): same sums up to fp32 summation order
+        ref = _make(shape, w, dtype)
+        begin = ref._stager.begin
+        ref._stager.begin = lambda uses=1: begin(1)
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=auto):
+            ref(*args, ttt_steps=3, ttt_step_loss_decay=0.8)[1].backward()
+        ref_grads = {n: p.grad for n, p in ref.named_parameters() if p.requires_grad}
+        for n, g in zip(names, g_bwd, strict=True):
+            r = ref_grads[n].float()
+            tol = (2 ** -7 if dtype == torch.bfloat16 else 1e-5) * r.abs().max() + 1e-12
+            assert (g.float() - r).abs().max() <= tol, n
+
+
+def test_backward_of_a_single_step_loss_reaches_only_the_steps_before_it():
+    """A loss that stops after the first TTT step of a three-step forward: the later steps never
+    run a backward, and the stacked weight-gradient product covers the first step's rows only.
+    The gradients equal those of a one-step forward."""
+    from speculators_amd import metrics as MT
+
+    shape = _shape()
+    w = {k_: v.bfloat16() for k_, v in OE.random_weights(shape, seed=8, std=0.05).items()}
+    hs, ids, doc, mask, pos, vl = _batch(shape, 128, 5, [70, 50])
+    args = (hs.bfloat16().cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.bfloat16().cuda())
+    model = _make(shape, w)
+    params = {n: p for n, p in model.named_parameters() if p.requires_grad}
+    step_losses = []
+    orig = MT.compute_metrics
+
+    def spy(*a, **k):
+        out = orig(*a, **k)
+        step_losses.append(out[0])
+        return out
+
+    MT.compute_metrics = spy
+    try:
+        model(*args, ttt_steps=3)
+    finally:
+        MT.compute_metrics = orig
+    assert len(step_losses) == 3
+    step_losses[0].backward()
+    got = {n: p.grad.clone() for n, p in params.items() if p.grad is not None}
+    model.zero_grad(set_to_none=True)
+    model(*args, ttt_steps=1)[1].backward()
+    for n, p in params.items():
+        if p.grad is None:
+            assert n not in got, n
+            continue
+        assert torch.equal(got[n], p.grad), n
+
+
 def test_gradient_accumulation_semantics_across_iterations():
     """The weight gradients are written into ``.grad`` by the GEMMs themselves (merged q/k/v
     buffer, beta = 1 accumulation over TTT steps): a second backward without ``zero_grad`` must
