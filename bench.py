@@ -223,7 +223,7 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
     from speculators_amd import _lib
     from speculators_amd import attention as A
     from speculators_amd import losses as L
-    from speculators_amd.gemm import gemm_nt
+    from speculators_amd.gemm import gemm_nt, gemm_tn
     from speculators_amd.data import plan_rows
 
     h, vd = cfg["hidden_size"], cfg["draft_vocab_size"]
@@ -389,6 +389,32 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
 
     ms_b = time_events(torch, attn_bwd, 10)
     mfma(f"attn_bwd[dq + dkv + diag kernels, TTT step {step}]", 10.0 * pairs * d * hq, ms_b, 1)
+    del q, kk, vv, o, go
+
+    # ... and at the first step (no diagonal keys)
+    mask0 = A.create_ttt_mask(torch.zeros(t, dtype=torch.long, device=device), t, None)
+    q = torch.randn(1, hq, t, d, device=device, generator=g).bfloat16().requires_grad_(True)
+    kk = torch.randn(1, hkv, t, d, device=device, generator=g).bfloat16().requires_grad_(True)
+    vv = torch.randn(1, hkv, t, d, device=device, generator=g).bfloat16().requires_grad_(True)
+    pairs0 = t * (t + 1) / 2
+    ms_f = time_events(torch, lambda: A.ttt_attention(q.detach(), kk.detach(), vv.detach(), mask0), 10)
+    mfma("attn_fwd_kernel[TTT step 0]", 4.0 * pairs0 * d * hq, ms_f, 1)
+    o = A.ttt_attention(q, kk, vv, mask0)
+    go = torch.randn_like(o)
+    ms_b = time_events(torch, lambda: torch.autograd.grad(o, (q, kk, vv), go, retain_graph=True), 10)
+    mfma("attn_bwd[dq + dkv kernels, TTT step 0]", 10.0 * pairs0 * d * hq, ms_b, 1)
+    del q, kk, vv, o, go
+
+    # weight gradient of the merged gate / up projection over all TTT steps in one product: the steps'
+    # output gradients [K T, 2F] and inputs [K T, H] lie one after the other, the contraction runs over
+    # K T rows, the fp32 result is written once
+    f2 = 2 * cfg["intermediate_size"]
+    dys = torch.randn(k_steps * t, f2, device=device, generator=g).bfloat16()
+    xs = torch.randn(k_steps * t, h, device=device, generator=g).bfloat16()
+    acc = torch.empty(f2, h, device=device, dtype=torch.float32)
+    ms = time_events(torch, lambda: gemm_tn(dys, xs, acc), 5)
+    mfma(f"gemm_bf16_tn_kernel[gate+up weight gradient, all {k_steps} steps: (K T x 2F)^T (K T x H) -> fp32]",
+         2.0 * k_steps * t * f2 * h, ms, 1)
     return out
 
 
