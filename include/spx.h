@@ -302,6 +302,28 @@ int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
                      void* dv, int64_t dv_head_stride, void* workspace,
                      int64_t workspace_bytes, void* stream);
 
+/* Attention with one interval of visible keys per query: out[i, h, :] = softmax over the keys
+ * row_lo[i] <= c < row_hi[i] (out of T; an empty interval gives a zero row).  This is the mask
+ * transformers' create_causal_mask builds from a 2-D padding mask -- key j visible to query i iff
+ * j <= i and attention_mask[j] -- when the non-padding positions of a row are contiguous, which is
+ * how the MTP forward is called with `attention_mask` (models/mtp/core.py:180-186, 119).  Layouts,
+ * lse, workspace sizes (spx_ttt_attn_workspace_bytes) and determinism as for spx_ttt_attn_fwd /
+ * spx_ttt_attn_bwd at ttt_step 0. */
+int spx_span_attn_fwd(const void* q, int64_t q_head_stride, const void* k,
+                      int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                      const int32_t* row_lo, const int32_t* row_hi, int64_t T,
+                      int32_t Hq, int32_t Hkv, int32_t D, float scaling,
+                      void* out, float* lse, void* workspace,
+                      int64_t workspace_bytes, void* stream);
+int spx_span_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
+                      int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                      const void* out, const void* dout, const float* lse,
+                      const int32_t* row_lo, const int32_t* row_hi, int64_t T,
+                      int32_t Hq, int32_t Hkv, int32_t D, float scaling, void* dq,
+                      int64_t dq_head_stride, void* dk, int64_t dk_head_stride,
+                      void* dv, int64_t dv_head_stride, void* workspace,
+                      int64_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------- DFlash attention
  * Per-row key intervals of the anchored-block mask, create_anchor_block_mask_mod
  * (models/dflash/attention.py:7-100), for run-contiguous document ids.  Row

@@ -12,7 +12,8 @@ Follows, in plain PyTorch on the CPU:
     ``find_packed_sequence_indices`` (called through ``create_causal_mask`` with
     ``attention_mask=None`` at models/mtp/core.py:180-186)
 
-Pinned by: the block-diagonal causal matrix of
+Pinned by: ``create_causal_mask`` of the library itself for the padding-mask form, the
+block-diagonal causal matrix of
 tests/unit/models/test_mtp_attention.py:17-55 (documents [1, 3, 2]), the loss
 properties of tests/unit/models/test_mtp_model.py (all-zero mask -> exactly 0,
 zero step weight -> that step's loss 0, short sequences give fewer steps), the
@@ -57,6 +58,17 @@ def packed_causal_mask(position_ids: torch.Tensor) -> torch.Tensor:
     return causal[None] & (seq[:, :, None] == seq[:, None, :])
 
 
+def padded_causal_mask(attention_mask: torch.Tensor) -> torch.Tensor:
+    """Dense bool ``[B, L, L]`` for a 2-D padding mask ``[B, L]``: query i sees key j iff j <= i
+    and ``attention_mask[b, j]`` is non-zero.  With a mask given, ``create_causal_mask`` does not
+    look for packed sequences in the positions (transformers ``masking_utils.py``: the detection
+    runs only for ``attention_mask is None``), so there is no same-sequence term."""
+    n = attention_mask.shape[1]
+    idx = torch.arange(n)
+    causal = idx[:, None] >= idx[None, :]
+    return causal[None] & (attention_mask != 0)[:, None, :]
+
+
 def _qwen3_layer(x, w, p, shape: DraftShape, cos, sin, mask, attn):
     """One row ``[1, L, H]`` through the Qwen3 decoder layer."""
     n = x.shape[1]
@@ -92,8 +104,9 @@ def mtp_layer(hidden, embeds, w, shape: DraftShape, cos, sin, mask, attn="dense"
 
 
 def mtp_forward(w, shape: DraftShape, input_ids, hidden_states, position_ids=None, loss_mask=None,
-                step_weights=None, num_steps: int = 3, attn: str = "dense"):
-    """``(logits_list, loss, metrics)`` of models/mtp/core.py:114-231."""
+                step_weights=None, num_steps: int = 3, attn: str = "dense", attention_mask=None):
+    """``(logits_list, loss, metrics)`` of models/mtp/core.py:114-231.  ``attention_mask``
+    (``[B, L]`` padding mask) replaces the packed-sequence mask as in core.py:180-186."""
     input_ids = input_ids.long()
     b, n = input_ids.shape
     if step_weights is not None and len(step_weights) != num_steps:
@@ -111,7 +124,8 @@ def mtp_forward(w, shape: DraftShape, input_ids, hidden_states, position_ids=Non
         metrics["loss_total"] = torch.tensor(1.0)
         return logits_list, total, metrics
     pos = position_ids[:, :valid]
-    masks = packed_causal_mask(pos)
+    masks = packed_causal_mask(pos) if attention_mask is None else \
+        padded_causal_mask(attention_mask[:, :valid])
     current = hidden_states
     for step in range(steps):
         hid = current[:, :valid]

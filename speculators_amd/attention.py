@@ -204,9 +204,100 @@ def ttt_attention(q, k, v, mask: TTTMask, scaling: float | None = None) -> torch
     return _TTTAttention.apply(q, k, v, mask, scaling)
 
 
+@dataclass
+class SpanMask:
+    """One interval ``[row_lo, row_hi)`` of visible keys per query (int32 ``[T]`` each) over the
+    ``T`` keys of a packed row: what ``transformers.masking_utils.create_causal_mask`` yields for a
+    2-D padding mask whose non-padding positions are contiguous in every batch row (the way the
+    MTP forward passes ``attention_mask``, models/mtp/core.py:180-186)."""
+
+    row_lo: torch.Tensor
+    row_hi: torch.Tensor
+    total_seq_len: int
+
+
+def create_padding_span_mask(attention_mask: torch.Tensor) -> SpanMask:
+    """``attention_mask [B, L]`` (non-zero = token, zero = padding) -> the ``SpanMask`` of the packed
+    row ``[1, B * L]``: query ``i`` of batch row ``b`` sees the keys ``j <= i`` of its own row with
+    ``attention_mask[b, j] != 0``.  Those must form one run per row (left or right padding); a row
+    with holes raises.  A query in front of its row's first token sees nothing and yields zeros."""
+    if attention_mask.dim() != 2:
+        raise ValueError(f"attention_mask must be [batch, seq_len], got {tuple(attention_mask.shape)}")
+    if not attention_mask.is_cuda:
+        raise _lib.SpxError("libspx_hip works on HIP device tensors only (got a CPU tensor)")
+    keep = attention_mask != 0
+    b, n = keep.shape
+    idx = torch.arange(n, device=keep.device, dtype=torch.int64)
+    count = keep.sum(-1)
+    first = torch.where(keep, idx, n).amin(-1)
+    last = torch.where(keep, idx, -1).amax(-1)
+    if bool(((last - first + 1 != count) & (count > 0)).any()):
+        raise ValueError("attention_mask must mark one contiguous run of tokens per row "
+                         "(left or right padding)")
+    first = torch.where(count > 0, first, torch.zeros_like(first))
+    end = torch.where(count > 0, last + 1, torch.zeros_like(last))
+    base = (torch.arange(b, device=keep.device, dtype=torch.int64) * n).unsqueeze(1)
+    lo = (base + first.unsqueeze(1)).expand(b, n)
+    hi = base + torch.minimum(idx.unsqueeze(0) + 1, end.unsqueeze(1))
+    hi = torch.maximum(hi, lo)  # empty, never negative
+    return SpanMask(lo.reshape(-1).to(torch.int32).contiguous(), hi.reshape(-1).to(torch.int32).contiguous(),
+                    b * n)
+
+
+class _SpanAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, mask: SpanMask, scaling: float):
+        if q.dim() != 4 or q.shape[0] != 1:
+            raise ValueError("the packed batch layout has batch size 1: q must be [1, Hq, T, D]")
+        if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
+            raise _lib.SpxError("the HIP attention kernels take bf16 q/k/v")
+        _, hq, t, d = q.shape
+        hkv = k.shape[1]
+        if t != mask.total_seq_len or k.shape[2] != t or v.shape != k.shape:
+            raise ValueError(f"q {tuple(q.shape)} / k {tuple(k.shape)} do not match a span mask over "
+                             f"{mask.total_seq_len} positions")
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        dev = q.device
+        out = torch.empty(1, t, hq, d, device=dev, dtype=torch.bfloat16)
+        lse = torch.empty(hq, t, device=dev, dtype=torch.float32)
+        ws = torch.empty(_workspace_bytes(t, hq, hkv, d, False), device=dev, dtype=torch.uint8)
+        _lib.call("spx_span_attn_fwd", _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1), _lib.ptr(v),
+                  v.stride(1), _lib.ptr(mask.row_lo), _lib.ptr(mask.row_hi), t, hq, hkv, d, float(scaling),
+                  _lib.ptr(out), _lib.ptr(lse), _lib.ptr(ws), ws.numel(), _lib.stream_ptr(dev))
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.mask, ctx.scaling = mask, float(scaling)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse = ctx.saved_tensors
+        mask = ctx.mask
+        _, hq, t, d = q.shape
+        hkv = k.shape[1]
+        dev = q.device
+        dout = dout.to(torch.bfloat16).contiguous()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        ws = torch.empty(_workspace_bytes(t, hq, hkv, d, True), device=dev, dtype=torch.uint8)
+        _lib.call("spx_span_attn_bwd", _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1), _lib.ptr(v),
+                  v.stride(1), _lib.ptr(out), _lib.ptr(dout), _lib.ptr(lse), _lib.ptr(mask.row_lo),
+                  _lib.ptr(mask.row_hi), t, hq, hkv, d, ctx.scaling, _lib.ptr(dq), dq.stride(1),
+                  _lib.ptr(dk), dk.stride(1), _lib.ptr(dv), dv.stride(1), _lib.ptr(ws), ws.numel(),
+                  _lib.stream_ptr(dev))
+        return dq, dk, dv, None, None
+
+
+def span_attention(q, k, v, mask: SpanMask, scaling: float | None = None) -> torch.Tensor:
+    """``[1, Hq, T, D]`` x ``[1, Hkv, T, D]`` -> ``[1, T, Hq, D]`` (bf16) under a ``SpanMask``."""
+    if scaling is None:
+        scaling = q.shape[-1] ** -0.5
+    return _SpanAttention.apply(q, k, v, mask, scaling)
+
+
 def ttt_hip_attention_forward(module, query, key, value, attention_mask, scaling=None, **_kwargs):
     """The attention-function signature of the reference registry
     (models/attention.py:20-66); ``attention_mask`` must be a ``TTTMask``."""
+    if isinstance(attention_mask, SpanMask):
+        return span_attention(query, key, value, attention_mask, scaling), None
     if not isinstance(attention_mask, TTTMask):
         raise TypeError(
             f"attention impl '{ATTN_IMPL_TTT}' needs a TTTMask descriptor as attention_mask, "

@@ -2593,6 +2593,74 @@ extern "C" int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void
                         workspace, st, __func__);
 }
 
+// ================================================================ span attention
+// Per query an interval [row_lo, row_hi) of visible keys out of T (no diagonal keys): the mask of a
+// padded batch row, where a query sees the non-padding keys up to itself.
+static AttnParams span_params(const void* q, int64_t q_hs, const void* k, int64_t k_hs, const void* v,
+                              int64_t v_hs, const int32_t* row_lo, const int32_t* row_hi, int64_t T,
+                              int32_t Hq, int32_t Hkv, float scaling) {
+  AttnParams p = ttt_params(q, q_hs, k, k_hs, v, v_hs, row_lo, T, 0, Hq, Hkv, scaling);
+  p.b1 = row_hi;
+  return p;
+}
+
+extern "C" int spx_span_attn_fwd(const void* q, int64_t q_head_stride, const void* k,
+                                 int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                                 const int32_t* row_lo, const int32_t* row_hi, int64_t T, int32_t Hq,
+                                 int32_t Hkv, int32_t D, float scaling, void* out, float* lse,
+                                 void* workspace, int64_t workspace_bytes, void* stream) {
+  if (int rc = shape_checks(__func__, T, T, Hq, Hkv, D)) return rc;
+  SPX_REQUIRE(q && k && v && row_lo && row_hi && out && lse && workspace, "null buffer");
+  SPX_REQUIRE(q_head_stride >= T * D && k_head_stride >= T * D && v_head_stride >= T * D,
+              "head stride smaller than T*D");
+  SPX_REQUIRE(q_head_stride % 8 == 0 && k_head_stride % 8 == 0 && v_head_stride % 8 == 0,
+              "head strides must be multiples of 8 elements");
+  SPX_REQUIRE(workspace_bytes >= fwd_workspace_bytes(T, Hkv, D), "workspace too small");
+  SPX_REQUIRE(all_aligned16({q, k, v, out, workspace}), "buffers must be 16-byte aligned");
+  AttnParams p = span_params(q, q_head_stride, k, k_head_stride, v, v_head_stride, row_lo, row_hi, T, Hq,
+                             Hkv, scaling);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (D == 256) return launch_fwd<256>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
+  if (D == 128) return launch_fwd<128>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
+  return launch_fwd<64>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
+}
+
+extern "C" int spx_span_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
+                                 int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                                 const void* out, const void* dout, const float* lse,
+                                 const int32_t* row_lo, const int32_t* row_hi, int64_t T, int32_t Hq,
+                                 int32_t Hkv, int32_t D, float scaling, void* dq,
+                                 int64_t dq_head_stride, void* dk, int64_t dk_head_stride, void* dv,
+                                 int64_t dv_head_stride, void* workspace, int64_t workspace_bytes,
+                                 void* stream) {
+  if (int rc = shape_checks(__func__, T, T, Hq, Hkv, D)) return rc;
+  SPX_REQUIRE(q && k && v && out && dout && lse && row_lo && row_hi && dq && dk && dv && workspace,
+              "null buffer");
+  SPX_REQUIRE(q_head_stride >= T * D && dq_head_stride >= T * D && k_head_stride >= T * D &&
+              v_head_stride >= T * D && dk_head_stride >= T * D && dv_head_stride >= T * D,
+              "head stride smaller than T*D");
+  SPX_REQUIRE((q_head_stride | k_head_stride | v_head_stride | dq_head_stride | dk_head_stride |
+               dv_head_stride) % 8 == 0, "head strides must be multiples of 8 elements");
+  SPX_REQUIRE(workspace_bytes >= bwd_workspace_bytes(T, T, Hq, Hkv, D), "workspace too small");
+  SPX_REQUIRE(all_aligned16({q, k, v, out, dout, dq, dk, dv, workspace}), "buffers must be 16-byte aligned");
+  AttnParams p = span_params(q, q_head_stride, k, k_head_stride, v, v_head_stride, row_lo, row_hi, T, Hq,
+                             Hkv, scaling);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  auto Op = reinterpret_cast<const uint16_t*>(out);
+  auto dOp = reinterpret_cast<const uint16_t*>(dout);
+  auto dQp = reinterpret_cast<uint16_t*>(dq);
+  auto dKp = reinterpret_cast<uint16_t*>(dk);
+  auto dVp = reinterpret_cast<uint16_t*>(dv);
+  if (D == 256)
+    return launch_bwd<256>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp, dv_head_stride,
+                           workspace, st, __func__);
+  if (D == 128)
+    return launch_bwd<128>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp,
+                           dv_head_stride, workspace, st, __func__);
+  return launch_bwd<64>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp, dv_head_stride,
+                        workspace, st, __func__);
+}
+
 // ---------------------------------------------------------------- allocation-free variant
 // The forward's only scratch is the key-contiguous copy V^T [Hkv, D, round_up(T, 128)].  Here it
 // lives in a file-scope device array instead of a caller-owned workspace.  Every GPU holds its

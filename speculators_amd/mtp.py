@@ -132,10 +132,6 @@ class MTPDraftModel(nn.Module):
     def forward(self, input_ids, hidden_states, attention_mask=None, position_ids=None,
                 loss_mask=None, step_weights=None, return_dict: bool = True, **_kwargs):
         cfg = self.config
-        if attention_mask is not None:
-            raise NotImplementedError(
-                "the HIP MTP path takes packed rows without padding masks (attention_mask=None, "
-                "as the training collate produces them)")
         self._stager.begin(uses=cfg.num_speculative_steps)
         hidden_states = compute_input(hidden_states)
         input_ids = input_ids.long()
@@ -160,11 +156,18 @@ class MTPDraftModel(nn.Module):
             return all_logits, total_loss, metrics
 
         pos = position_ids[:, :valid].to(torch.int64)
-        # sequence index inside each row (a new sequence wherever the position does not grow
-        # by one), made unique across rows: the packed row [1, B * valid] never mixes rows
-        diff = torch.diff(pos, prepend=pos[:, :1] - 1, dim=-1)
-        seq = (diff != 1).cumsum(-1) + torch.arange(b, device=device).unsqueeze(1) * (valid + 1)
-        mask = A.create_ttt_mask(seq.reshape(-1), b * valid, None)
+        if attention_mask is None:
+            # sequence index inside each row (a new sequence wherever the position does not grow
+            # by one), made unique across rows: the packed row [1, B * valid] never mixes rows
+            diff = torch.diff(pos, prepend=pos[:, :1] - 1, dim=-1)
+            seq = (diff != 1).cumsum(-1) + torch.arange(b, device=device).unsqueeze(1) * (valid + 1)
+            mask = A.create_ttt_mask(seq.reshape(-1), b * valid, None)
+        else:
+            # a padding mask switches the packed-sequence detection off (create_causal_mask only
+            # looks at position restarts when no mask is given): key j <= i with attention_mask[j]
+            if attention_mask.shape != (b, n):
+                raise ValueError(f"attention_mask must be {(b, n)}, got {tuple(attention_mask.shape)}")
+            mask = A.create_padding_span_mask(attention_mask[:, :valid].to(device))
         flat_pos = pos.reshape(-1).contiguous()
         inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device, cfg.rope_scaling)
         layer = self.mtp_layers[0]

@@ -122,6 +122,83 @@ def test_attention_head_dim_256(t, hq, hkv, docs):
         assert err <= 2e-2 * want.abs().max().item(), (name, err, want.abs().max().item())
 
 
+@pytest.mark.parametrize("d,hq,hkv", [(64, 4, 2), (128, 2, 1), (256, 2, 1)])
+def test_span_attention_under_a_padding_mask(d, hq, hkv):
+    """Attention with one key interval per query (right- and left-padded rows, an all-padding row):
+    forward and backward against the dense oracle under the padding-mask form of the causal mask."""
+    from speculators_amd.attention import create_padding_span_mask, span_attention
+
+    b, n = 4, 96
+    am = torch.ones(b, n, dtype=torch.long)
+    am[0, 70:] = 0   # right padding
+    am[1, :25] = 0   # left padding
+    am[3, :] = 0     # nothing but padding
+    t = b * n
+    g = torch.Generator().manual_seed(d)
+    q = torch.randn(1, hq, t, d, generator=g).bfloat16()
+    k = torch.randn(1, hkv, t, d, generator=g).bfloat16()
+    v = torch.randn(1, hkv, t, d, generator=g).bfloat16()
+    go = torch.randn(1, t, hq, d, generator=g).bfloat16()
+    mask = create_padding_span_mask(am.cuda())
+    # the packed row never mixes batch rows: block diagonal of the per-row masks
+    dense = torch.zeros(t, t, dtype=torch.bool)
+    per_row = OM.padded_causal_mask(am)
+    for r in range(b):
+        dense[r * n:(r + 1) * n, r * n:(r + 1) * n] = per_row[r]
+    lo, hi = mask.row_lo.cpu(), mask.row_hi.cpu()
+    idx = torch.arange(t)
+    assert torch.equal(dense, (idx[None, :] >= lo[:, None]) & (idx[None, :] < hi[:, None]))
+    qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    out = span_attention(qg, kg, vg, mask, d ** -0.5)
+    out.backward(go.cuda())
+    qr, kr, vr = (x.float().requires_grad_(True) for x in (q, k, v))
+    ref = dense_attention(qr, kr, vr, dense, d ** -0.5)
+    ref.backward(go.float())
+    assert (out.float().cpu() - ref).abs().max() <= 2e-2 * ref.abs().max()
+    assert not out[0, 3 * n:].any()  # queries that see nothing give zeros
+    for name, got, want in (("dq", qg.grad, qr.grad), ("dk", kg.grad, kr.grad), ("dv", vg.grad, vr.grad)):
+        err = (got.float().cpu() - want).abs().max().item()
+        assert err <= 2e-2 * want.abs().max().item(), (name, err, want.abs().max().item())
+    with pytest.raises(ValueError, match="contiguous run"):
+        create_padding_span_mask(torch.tensor([[1, 0, 1, 1]]).cuda())
+
+
+def test_model_with_a_padding_mask_matches_oracle():
+    """``attention_mask`` (models/mtp/core.py:119,180-186): right- and left-padded rows.  The padded
+    positions are kept out of the loss; logits are compared where the mask marks a token."""
+    shape = _shape()
+    steps = 2
+    w = {k: v.bfloat16() for k, v in OM.random_weights(shape, seed=4, std=0.05).items()}
+    g = torch.Generator().manual_seed(9)
+    b, n = 2, 150
+    ids = torch.randint(0, shape.vocab_size, (b, n), generator=g)
+    hs = torch.randn(b, n, shape.hidden_size, generator=g).bfloat16()
+    am = torch.ones(b, n, dtype=torch.long)
+    am[0, 110:] = 0
+    am[1, :30] = 0
+    lm = ((torch.rand(b, n, generator=g) < 0.7) & (am != 0)).float()
+    model = _make(shape, w, steps)
+    logits, loss, m = model(ids.cuda(), hs.cuda(), attention_mask=am.cuda(), loss_mask=lm.cuda())
+    loss.backward()
+    wf = {k: v.float().requires_grad_(True) for k, v in w.items()}
+    rl, rloss, rm = OM.mtp_forward(wf, shape, ids, hs.float(), loss_mask=lm, num_steps=steps,
+                                   attention_mask=am)
+    rloss.backward()
+    assert abs(loss.item() - rloss.item()) <= 1e-3 * abs(rloss.item())
+    valid = n - steps - 1
+    tok = am[:, :valid] != 0
+    for k in range(steps):
+        got, want = logits[k].float().cpu()[tok], rl[k][tok]
+        assert (got - want).abs().max() <= 2e-2 * want.abs().max(), k
+    for name, p in model.named_parameters():
+        if p.requires_grad:
+            want = wf[name].grad
+            assert (p.grad.float().cpu() - want).abs().max() <= 3e-2 * want.abs().max() + 1e-6, name
+    # without the mask the same call splits the rows at position restarts instead: a different result
+    with pytest.raises(ValueError, match="attention_mask must be"):
+        model(ids.cuda(), hs.cuda(), attention_mask=am[:, :10].cuda())
+
+
 def _shape(**kw):
     base = dict(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=64,
                 intermediate_size=512, vocab_size=1000, draft_vocab_size=1000, rms_norm_eps=1e-6,
@@ -213,8 +290,10 @@ def test_model_properties_of_the_reference_tests():
         assert len(short) == 1
         with pytest.raises(ValueError, match="expected exactly 3 weights"):
             model(ids, hs, step_weights=[1.0])
-        with pytest.raises(NotImplementedError):
-            model(ids, hs, attention_mask=torch.ones(1, 40, device="cuda"))
+        # an all-ones padding mask and a single packed sequence are the same mask
+        with_mask, _, _ = model(ids, hs, attention_mask=torch.ones_like(ids))
+        plain, _, _ = model(ids, hs)
+        assert all(torch.equal(a, b_) for a, b_ in zip(with_mask, plain, strict=True))
         with pytest.raises(RuntimeError, match="bf16"):
             model(ids, hs.float())
 

@@ -68,6 +68,28 @@ def test_mask_matches_transformers_create_causal_mask():
     assert torch.equal(allow, OM.packed_causal_mask(pos)[0])
 
 
+def test_padding_mask_matches_transformers_create_causal_mask():
+    """With a 2-D padding mask the library drops the packed-sequence detection (position restarts
+    no longer split the row) and masks the padded KEYS; fully masked query rows aside (the library
+    un-masks them for the sdpa kernel), the restated mask is the library's."""
+    from transformers import Qwen3Config
+    from transformers.masking_utils import create_causal_mask
+
+    cfg = Qwen3Config(hidden_size=32, num_attention_heads=4, num_key_value_heads=2, head_dim=8,
+                      intermediate_size=64, vocab_size=61, num_hidden_layers=1)
+    cfg._attn_implementation = "eager"
+    pos = torch.tensor([[0, 1, 2, 0, 1, 0, 1, 2, 3, 0], [0, 1, 2, 3, 4, 5, 6, 7, 8, 9]])
+    am = torch.tensor([[1, 1, 1, 1, 1, 1, 1, 0, 0, 0], [0, 0, 0, 1, 1, 1, 1, 1, 1, 1]])
+    m = create_causal_mask(config=cfg, inputs_embeds=torch.zeros(2, 10, 32), attention_mask=am,
+                           past_key_values=None, position_ids=pos)
+    allow = m[:, 0] if m.dtype == torch.bool else m[:, 0] == 0
+    want = OM.padded_causal_mask(am)
+    has_key = want.any(-1)
+    assert torch.equal(allow[has_key], want[has_key])
+    # row 0: the position restarts at 3 and 5 do not split the row any more
+    assert want[0, 6, 0] and not OM.packed_causal_mask(pos)[0, 6, 0]
+
+
 def test_layer_matches_transformers_qwen3_modules():
     """The restated layer against the library's Qwen3DecoderLayer wired like
     models/mtp/model_definitions.py:95-116."""
