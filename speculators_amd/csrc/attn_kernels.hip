@@ -1696,12 +1696,6 @@ __device__ __forceinline__ int64_t uni(int64_t v) {
   return (int64_t)(((uint64_t)hi << 32) | lo);
 }
 
-#ifdef SPX_WS_TIMING
-__device__ unsigned long long g_ws_dbg[128 * 16];
-extern "C" int spx_debug_ws_timing(unsigned long long* host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_ws_dbg), sizeof(g_ws_dbg));
-}
-#endif
 
 // Four 16-bit values per lane from LDS, transposed inside every group of 16 lanes: lane 4u + w of
 // a group receives, as element j, element w of the 8 bytes that lane 4j + u of the group points at.
@@ -2013,52 +2007,25 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
     if (!p_active && !c_active) break;
     // tile b + 1 has landed when at most the loads of tiles b + 2 .. b + kAhead - 1 are in flight
     static_assert(AH == 4, "the wait below counts two tiles");
-#ifdef SPX_WS_TIMING
-#ifdef SPX_WS_TIMING_STEPS
-    const bool dbg = blockIdx.x == 0 && lane == 0 && (wave & 3) == SPX_WS_TIMING && kP < 127;
-#else
-    const bool dbg = false;
-#endif
-    unsigned long long* const dbg_row = g_ws_dbg + kP * 16 + (producer ? 0 : 8);
-    if (dbg) dbg_row[4] = __builtin_amdgcn_s_memtime();
-#endif
     if constexpr (!producer) {
       const int later = (sq[2] < s_end ? 1 : 0) + (sq[3] < s_end ? 1 : 0);
       if (later == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoads) : "memory");
       else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads) : "memory");
       else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-#ifdef SPX_WS_TIMING
-    if (dbg) dbg_row[5] = __builtin_amdgcn_s_memtime();
-#endif
     __syncthreads();
-#ifdef SPX_WS_TIMING
-    if (dbg) dbg_row[0] = __builtin_amdgcn_s_memtime();
-#endif
     if constexpr (producer) {
       if (p_active) {
         if (sq[1] < s_end) score_begin(wrap(rb + 1), (kP + 1) & (SM::kSets - 1));
         soft_valu(kP & (SM::kSets - 1), kP & 1, fq[0]);
-#ifdef SPX_WS_TIMING
-        if (dbg) dbg_row[1] = __builtin_amdgcn_s_memtime();
-#endif
         if (sq[1] < s_end) score_finish();
-#ifdef SPX_WS_TIMING
-        if (dbg) dbg_row[2] = __builtin_amdgcn_s_memtime();
-#endif
       }
     } else {
       if (c_active) {
         consume(wrap(rb + NS - 1), (kP - 1) & 1);
-#ifdef SPX_WS_TIMING
-        if (dbg) dbg_row[1] = __builtin_amdgcn_s_memtime();
-#endif
       }
       // tile b + kAhead into the buffer tile b - 2 left behind
       if (sq[AH] < s_end) issue(sq[AH], wrap(rb + AH), (kP + AH) & (SM::kSets - 1));
-#ifdef SPX_WS_TIMING
-      if (dbg) dbg_row[3] = __builtin_amdgcn_s_memtime();
-#endif
     }
     // next step
     sC = sq[0];
@@ -2137,22 +2104,10 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkv_ws_kernel(
     }
     __syncthreads();
   }
-#ifdef SPX_WS_TIMING
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    g_ws_dbg[127 * 16 + 12] = __builtin_amdgcn_s_memtime();
-    g_ws_dbg[127 * 16 + 13] = __builtin_amdgcn_s_memrealtime();
-  }
-#endif
   if (threadIdx.x < 256)
     dkv_ws_role<D, true>(p, dO, NQp, neg, mrows, dKp, dVp);
   else
     dkv_ws_role<D, false>(p, dO, NQp, neg, mrows, dKp, dVp);
-#ifdef SPX_WS_TIMING
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    g_ws_dbg[127 * 16 + 14] = __builtin_amdgcn_s_memtime();
-    g_ws_dbg[127 * 16 + 15] = __builtin_amdgcn_s_memrealtime();
-  }
-#endif
 }
 
 // dK[kvh, c, :] = scaling * sum_{h in group} dKp[h, c, :],  dV likewise (no scaling); bf16 out
