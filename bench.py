@@ -35,10 +35,11 @@ TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "kernels_config1_hbm_traffic_pm
 TRAFFIC_ROWS = {
     "gemm_fwd": ("gemm_bf16_nt_kernel", 512000),
     "gemm_dx": ("gemm_bf16_nt_kernel", 65536),
-    "loss_fwd": ("loss_fwd_kernel<unsigned short, 0, true, false", None),
-    "loss_fwd_reuse": ("loss_fwd_kernel<unsigned short, 0, true, true", None),
-    "loss_bwd": ("loss_bwd_kernel<unsigned short, 0", None),
-    "attn_fwd": ("attn_fwd_kernel<128", None),
+    "loss_fwd": ("loss_fwd_kernel<unsigned short, 0, true, false, false", None),
+    "loss_fwd_reuse": ("loss_fwd_kernel<unsigned short, 0, true, true, false", None),
+    "gemm_tn": ("gemm_bf16_tn_kernel<2>", None),
+    # (the summary averages the attention kernels over TTT steps 0 and 6 and the loss backward over its
+    # full and packed launches: no per-launch figure for those)
 }
 
 
@@ -301,7 +302,7 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
                   _lib.ptr(rg), None, _lib.ptr(grad), vd, st)
 
     ms = time_events(torch, loss_bwd, 20)
-    hbm("loss_bwd_kernel[KL, T rows x Vd]", 3.0 * t * vd * 2, ms, 0, "loss_bwd")
+    hbm("loss_bwd_kernel[KL, T rows x Vd]", 3.0 * t * vd * 2, ms, 0)
 
     # what the model launches while lm_head is frozen: the same gradient with the live rows (loss
     # mask Bernoulli(0.7), as in the timed step) packed to the front; dead rows are neither read
@@ -380,7 +381,7 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
     vv = torch.randn(1, hkv, (step + 1) * t, d, device=device, generator=g).bfloat16().requires_grad_(True)
     pairs = t * (t + 1) / 2 + step * t
     ms_f = time_events(torch, lambda: A.ttt_attention(q.detach(), kk.detach(), vv.detach(), mask), 10)
-    mfma(f"attn_fwd_kernel[TTT step {step}]", 4.0 * pairs * d * hq, ms_f, 1, "attn_fwd")
+    mfma(f"attn_fwd_kernel[TTT step {step}]", 4.0 * pairs * d * hq, ms_f, 1)
     o = A.ttt_attention(q, kk, vv, mask)
     go = torch.randn_like(o)
 
@@ -414,7 +415,7 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
     acc = torch.empty(f2, h, device=device, dtype=torch.float32)
     ms = time_events(torch, lambda: gemm_tn(dys, xs, acc), 5)
     mfma(f"gemm_bf16_tn_kernel[gate+up weight gradient, all {k_steps} steps: (K T x 2F)^T (K T x H) -> fp32]",
-         2.0 * k_steps * t * f2 * h, ms, 1)
+         2.0 * k_steps * t * f2 * h, ms, 1, "gemm_tn")
     return out
 
 
