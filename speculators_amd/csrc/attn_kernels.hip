@@ -16,6 +16,8 @@
 // Key tiles that no row of a workgroup can see are skipped analytically; no
 // dense mask or BlockMask exists anywhere.
 
+#include <type_traits>
+
 #include "attn_common.h"
 #include "../../include/spx.h"
 
@@ -255,21 +257,36 @@ __device__ __forceinline__ void pin_block(f32x16& a) {
 }
 
 // ---------------------------------------------------------------- forward
-// One workgroup = 4 waves = 4 * 32 * NSB query rows of one head.  With NSB = 2 a
-// wave owns two 32-row sub-blocks, so every K / V^T fragment read from LDS
-// feeds two MFMAs (LDS bandwidth, not the matrix core, bounds NSB = 1).
-// wave priority around the MFMA clusters: with two waves on a SIMD the arbiter then prefers the
-// wave that is in its matrix phase and fills the gaps with the other wave's vector work
-#ifndef SPX_PRIO
-#define SPX_PRIO 1
+// One workgroup = 4 waves = 4 * 32 * NSB query rows of one head (NSB = 2: a wave owns two 32-row
+// sub-blocks and every K / V^T fragment read from LDS feeds two MFMAs; the kernels run NSB = 1).
+// Wave priorities (s_setprio) per phase, (matrix phase, vector phase) per kernel; equal values = no changes.
+// Forward: the wave that is in its soft-max gets the higher priority.  Its vector instructions are short and
+// slot in between the MFMAs of the other wave, which needs one issue slot per 32 cycles; the other way
+// round (matrix phase first) the vector wave waits behind MFMAs that are themselves waiting for the pipe
+// (measured at the Llama-3.1-8B shape: 825 TFLOP/s with the matrix phase first, 826 without priorities, 880
+// with the vector phase first).  The dQ and dK/dV kernels measure best with the matrix phase first.
+#ifndef SPX_FWD_PRIO
+#define SPX_FWD_PRIO 0, 3
 #endif
-#if SPX_PRIO
-#define SPX_PRIO_MFMA() __builtin_amdgcn_s_setprio(3)
-#define SPX_PRIO_VALU() __builtin_amdgcn_s_setprio(0)
-#else
-#define SPX_PRIO_MFMA()
-#define SPX_PRIO_VALU()
+#ifndef SPX_DQ_PRIO
+#define SPX_DQ_PRIO 3, 0
 #endif
+#ifndef SPX_DKV_PRIO
+#define SPX_DKV_PRIO 3, 0
+#endif
+constexpr int prio_first(int a, int) { return a; }
+constexpr int prio_second(int, int b) { return b; }
+template <int M, int V>
+struct PrioPair {
+  static __device__ __forceinline__ void matrix() { if constexpr (M != V) __builtin_amdgcn_s_setprio(M); }
+  static __device__ __forceinline__ void vector() { if constexpr (M != V) __builtin_amdgcn_s_setprio(V); }
+};
+#define SPX_FWD_PRIO_MFMA() PrioPair<prio_first(SPX_FWD_PRIO), prio_second(SPX_FWD_PRIO)>::matrix()
+#define SPX_FWD_PRIO_VALU() PrioPair<prio_first(SPX_FWD_PRIO), prio_second(SPX_FWD_PRIO)>::vector()
+#define SPX_DQ_PRIO_MFMA() PrioPair<prio_first(SPX_DQ_PRIO), prio_second(SPX_DQ_PRIO)>::matrix()
+#define SPX_DQ_PRIO_VALU() PrioPair<prio_first(SPX_DQ_PRIO), prio_second(SPX_DQ_PRIO)>::vector()
+#define SPX_DKV_PRIO_MFMA() PrioPair<prio_first(SPX_DKV_PRIO), prio_second(SPX_DKV_PRIO)>::matrix()
+#define SPX_DKV_PRIO_VALU() PrioPair<prio_first(SPX_DKV_PRIO), prio_second(SPX_DKV_PRIO)>::vector()
 #ifndef SPX_DKV_REMAT
 #define SPX_DKV_REMAT 1
 #endif
@@ -329,7 +346,8 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
   const int qb = n_qb - 1 - rest / group;  // late (heavy, under a causal mask) blocks first
   const int m0 = qb * BM;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: what derives from it is scalar too
   const int g = lane >> 5, col = lane & 31;
   int i[NSB], ic[NSB];
 #pragma unroll
@@ -444,9 +462,17 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
   auto issue = [&](int n0, int buf) __attribute__((always_inline)) {
     if constexpr (PF == 2) {
       const uint32_t kb = lds0 + buf * SM::kBuf + wave * LPK * 1024;
+      if (n0 + kBN <= p.NKV) {
+        // every row of the tile exists: the lane's offset inside a tile is loop invariant, the tile's
+        // first row goes into the scalar offset (no vector arithmetic per load)
 #pragma unroll
-      for (int j = 0; j < LPK; ++j)
-        load_to_lds16<0>(kres, kb + j * 1024, min(n0 + k_row[j], last_row) * RBK + k_col[j], 0);
+        for (int j = 0; j < LPK; ++j) load_to_lds16<0>(kres, kb + j * 1024, k_row[j] * RBK + k_col[j], n0 * RBK);
+      } else {
+        // the last, ragged tile: rows past the end repeat the last one (they are masked out)
+#pragma unroll
+        for (int j = 0; j < LPK; ++j)
+          load_to_lds16<0>(kres, kb + j * 1024, min(n0 + k_row[j], last_row) * RBK + k_col[j], 0);
+      }
       const uint32_t vb = lds0 + buf * SM::kBuf + SM::kTileK + wave * LPV * 1024;
 #pragma unroll
       for (int j = 0; j < LPV; ++j) load_to_lds16<0>(vres, vb + j * 1024, v_off[j], n0 * 2);
@@ -456,18 +482,20 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
   const int rdk = col * RBK + ((g ^ swz_k(col)) * 16);
   const int rdv = col * 128 + ((g ^ swz_v(col)) * 16);
 
-  // one pass over the key tiles of one interval class
+  // one pass over the key tiles of one interval class.  The tile loop is unrolled over the two tile
+  // buffers: the buffer is then a compile-time constant and the fragment reads address it through
+  // the immediate offset of ds_read (no vector add per read).
   auto run_pass = [&](const int (&aa)[NSB], const int (&bb)[NSB], int w_amin, int w_amax,
                       int w_bmin, int w_bmax, int blk_a, int blk_b) {
     if (blk_b <= blk_a) return;
     const int n_begin = (blk_a / kBN) * kBN;
     if (PF == 1) fetch(n_begin);
-    int buf = 0;
     if constexpr (PF == 2) {
       __syncthreads();  // a previous pass may still be reading either buffer
       issue(n_begin, 0);
     }
-    for (int n0 = n_begin; n0 < blk_b; n0 += kBN) {
+    auto tile = [&](int n0, auto buf_c) __attribute__((always_inline)) {
+      constexpr int buf = decltype(buf_c)::value;
       if constexpr (PF == 2) {
         // this wave's loads of tile n0 have landed; after the barrier everybody's have, and nobody
         // reads the other buffer any more: the next tile goes there
@@ -482,11 +510,10 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
       }
       const uint8_t* const tk = fwd_smem + buf * SM::kBuf;
       const uint8_t* const tv = tk + SM::kTileK;
-      buf ^= 1;
-      if (n0 >= w_bmax || n0 + kBN <= w_amin) continue;  // nothing visible for this wave
+      if (n0 >= w_bmax || n0 + kBN <= w_amin) return;  // nothing visible for this wave
 
       f32x16 st[NSB][2];
-      SPX_PRIO_MFMA();
+      SPX_FWD_PRIO_MFMA();
       // K fragments go through a ring of four registers: the read of fragment f + 4 is
       // issued right after the MFMA of fragment f, so no MFMA waits for LDS; the two
       // 32-key halves alternate so that consecutive MFMAs use different accumulators
@@ -515,7 +542,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-      SPX_PRIO_VALU();
+      SPX_FWD_PRIO_VALU();
       const bool need_mask = (n0 < w_amax) || (n0 + kBN > w_bmin);
       int m_lo[NSB], m_hi[NSB];
 #pragma unroll
@@ -576,7 +603,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         }
         l_run[sb] += rs0 + rs1;
       }
-      SPX_PRIO_MFMA();
+      SPX_FWD_PRIO_MFMA();
       {
         // V^T fragments through the same kind of ring; fragment f = (16-key step s, D block db)
         constexpr int NF = 4 * NDB;
@@ -608,7 +635,11 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-      SPX_PRIO_VALU();
+      SPX_FWD_PRIO_VALU();
+    };
+    for (int n0 = n_begin; n0 < blk_b; n0 += 2 * kBN) {
+      tile(n0, std::integral_constant<int, 0>{});
+      if (n0 + kBN < blk_b) tile(n0 + kBN, std::integral_constant<int, 1>{});
     }
   };
 
@@ -999,7 +1030,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
           f32x16 st, dp;
           // K and V fragments alternate through a ring of four registers (fragment 2 kk is
           // K, 2 kk + 1 is V): the read of fragment f + 4 follows the MFMA of fragment f
-          SPX_PRIO_MFMA();
+          SPX_DQ_PRIO_MFMA();
           {
             constexpr int NF = 2 * NKK;
             bf16x8 fr[4];
@@ -1025,7 +1056,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
             }
             __builtin_amdgcn_sched_barrier(0);
           }
-          SPX_PRIO_VALU();
+          SPX_DQ_PRIO_VALU();
 #pragma unroll
           for (int r = 0; r < 16; ++r) st[r] = fast_exp2(st[r]);
           if (need_mask) {
@@ -1041,7 +1072,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
           }
 #pragma unroll
           for (int r = 0; r < 16; ++r) dp[r] *= st[r];
-          SPX_PRIO_MFMA();
+          SPX_DQ_PRIO_MFMA();
           {
             // K^T fragments through the same kind of ring; fragment f = (16-key step s2, D block db)
             constexpr int NF = 2 * NDB;
@@ -1067,7 +1098,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
             }
             __builtin_amdgcn_sched_barrier(0);
           }
-          SPX_PRIO_VALU();
+          SPX_DQ_PRIO_VALU();
         }
       }
     }
@@ -1884,7 +1915,7 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
     __builtin_amdgcn_sched_barrier(0);
   };
   auto score_finish = [&]() __attribute__((always_inline)) {
-    SPX_PRIO_MFMA();
+    SPX_DKV_PRIO_MFMA();
 #pragma unroll
     for (int f = 0; f < NFP; ++f) {
       __builtin_amdgcn_sched_barrier(0);
@@ -1894,7 +1925,7 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
       if (f + RG < NFP) pfread(f + RG);
     }
     __builtin_amdgcn_sched_barrier(0);
-    SPX_PRIO_VALU();
+    SPX_DKV_PRIO_VALU();
   };
   auto soft_valu = [&](int set, int par, bool full) __attribute__((always_inline)) {
     const int* const a1_s = reinterpret_cast<const int*>(small0 + set * (SM::kSmall / 4) + 64);
@@ -1937,7 +1968,7 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
     pb[1] = *reinterpret_cast<const bf16x8*>(slot + 1 * 1024);
     sb[0] = *reinterpret_cast<const bf16x8*>(slot + 2 * 1024);
     sb[1] = *reinterpret_cast<const bf16x8*>(slot + 3 * 1024);
-    SPX_PRIO_MFMA();
+    SPX_DKV_PRIO_MFMA();
     constexpr int NF = 2 * 2 * NDB;
     i16x4 lo[RG], hi[RG];
     // fragment f: even = dO^T (for dV), odd = Q'^T (for dK); e = f / 2: k step s2 = e / NDB, row block db
@@ -1975,7 +2006,7 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
       if (f + RG < NF) fread(f + RG);
     }
     __builtin_amdgcn_sched_barrier(0);
-    SPX_PRIO_VALU();
+    SPX_DKV_PRIO_VALU();
   };
 
   // ---- prologue.  Tile k of the sequence of steps lives in ring buffer k % kStages, its per-row
