@@ -132,6 +132,130 @@ def test_layer_matches_transformers_qwen3_modules():
     assert torch.allclose(got, want, atol=2e-5, rtol=1e-4), (got - want).abs().max()
 
 
+
+def _hybrid_shape(**kw):
+    base = dict(hidden_size=32, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+                intermediate_size=48, vocab_size=61, draft_vocab_size=61, rms_norm_eps=1e-6,
+                rope_theta=10000.0)
+    base.update(kw)
+    return OM.HybridShape(**base)
+
+
+def _library_hybrid(model_type, shape, w):
+    """(decoder layer, norm class, rotary module) of the library for one hybrid flavour, the
+    layer at the last full-attention index as models/mtp/model_definitions.py:52-68 picks it,
+    loaded with the oracle's weights."""
+    common = dict(hidden_size=32, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+                  intermediate_size=48, vocab_size=61, num_hidden_layers=4, rms_norm_eps=1e-6,
+                  attention_bias=False, layer_types=["linear_attention", "full_attention"] * 2,
+                  rope_parameters={"rope_type": "default", "rope_theta": 10000.0,
+                                   "partial_rotary_factor": shape.partial_rotary_factor})
+    moe = dict(num_experts=shape.num_experts, num_experts_per_tok=shape.num_experts_per_tok,
+               moe_intermediate_size=shape.moe_intermediate_size,
+               shared_expert_intermediate_size=shape.shared_expert_intermediate_size)
+    if model_type == "qwen3_next":
+        from transformers import Qwen3NextConfig
+        from transformers.models.qwen3_next import modeling_qwen3_next as M
+        cfg = Qwen3NextConfig(**common, **moe, norm_topk_prob=shape.norm_topk_prob,
+                              decoder_sparse_step=1, mlp_only_layers=[])
+        classes = (M.Qwen3NextDecoderLayer, M.Qwen3NextRMSNorm, M.Qwen3NextRotaryEmbedding)
+    elif model_type == "qwen3_5_text":
+        from transformers.models.qwen3_5 import modeling_qwen3_5 as M
+        from transformers.models.qwen3_5.configuration_qwen3_5 import Qwen3_5TextConfig
+        cfg = Qwen3_5TextConfig(**common)
+        classes = (M.Qwen3_5DecoderLayer, M.Qwen3_5RMSNorm, M.Qwen3_5TextRotaryEmbedding)
+    else:
+        from transformers.models.qwen3_5_moe import modeling_qwen3_5_moe as M
+        from transformers.models.qwen3_5_moe.configuration_qwen3_5_moe import Qwen3_5MoeTextConfig
+        cfg = Qwen3_5MoeTextConfig(**common, **moe)
+        classes = (M.Qwen3_5MoeDecoderLayer, M.Qwen3_5MoeRMSNorm, M.Qwen3_5MoeTextRotaryEmbedding)
+    cfg._attn_implementation = "eager"
+    layer = classes[0](cfg, 3)
+    p = "mtp_layers.0."
+    own = dict(layer.named_parameters())
+    sd = {k[len(p):]: v for k, v in w.items() if k.startswith(p) and k[len(p):] in own}
+    assert set(sd) == set(own), set(own) ^ set(sd)
+    layer.load_state_dict(sd, strict=True)
+    return layer, classes[1], classes[2](cfg)
+
+
+@pytest.mark.parametrize("model_type,kw", [
+    ("qwen3_next", dict(num_experts=6, num_experts_per_tok=2, moe_intermediate_size=24,
+                        shared_expert_intermediate_size=40, norm_topk_prob=True)),
+    ("qwen3_next", dict(num_experts=5, num_experts_per_tok=3, moe_intermediate_size=16,
+                        shared_expert_intermediate_size=16, norm_topk_prob=False,
+                        partial_rotary_factor=0.5)),
+    ("qwen3_5_text", dict()),
+    ("qwen3_5_moe_text", dict(num_experts=6, num_experts_per_tok=2, moe_intermediate_size=24,
+                              shared_expert_intermediate_size=40)),
+])
+def test_hybrid_layer_matches_transformers_modules(model_type, kw):
+    """The restated hybrid layer (gain 1 + w norms, gated attention, partial rotary embedding,
+    sparse MoE with a shared expert) against the library's decoder layer of each flavour wired
+    like models/mtp/model_definitions.py:95-116, output and gradients."""
+    shape = _hybrid_shape(model_type=model_type, **kw)
+    w = {k: v.requires_grad_(True) for k, v in OM.random_weights(shape, 5, std=0.1).items()}
+    layer, norm_class, rot = _library_hybrid(model_type, shape, w)
+    p = "mtp_layers.0."
+    norms = {}
+    for name in ("hidden_layernorm", "token_layernorm", "final_layernorm"):
+        norms[name] = norm_class(32, eps=1e-6)
+        norms[name].weight.data.copy_(w[p + name + ".weight"])
+    g = torch.Generator().manual_seed(6)
+    n = 11
+    hidden = torch.randn(1, n, 32, generator=g)
+    embeds = torch.randn(1, n, 32, generator=g)
+    pos = torch.tensor([[0, 1, 2, 3, 0, 1, 2, 0, 1, 2, 3]])
+    mask = OM.packed_causal_mask(pos)
+    add = torch.zeros(1, 1, n, n).masked_fill(~mask[:, None], float("-inf"))
+    proj = F.linear(torch.cat([norms["token_layernorm"](embeds), norms["hidden_layernorm"](hidden)], -1),
+                    w[p + "input_proj.weight"].detach())
+    out = layer(hidden_states=proj, attention_mask=add, position_ids=pos,
+                position_embeddings=rot(proj, pos))
+    out = out[0] if isinstance(out, tuple) else out
+    want = norms["final_layernorm"](out)
+    cos, sin = OM.rope_tables(pos[0], OM.rotary_dim(shape), 10000.0, torch.float32)
+    assert cos.shape[-1] == int(16 * shape.partial_rotary_factor)
+    got = OM.mtp_layer(hidden, embeds, w, shape, cos, sin, mask[0])
+    assert torch.allclose(got, want, atol=2e-5, rtol=1e-4), (got - want).abs().max()
+    probe = torch.randn(want.shape, generator=g)
+    (want * probe).sum().backward()
+    (got * probe).sum().backward()
+    own = dict(layer.named_parameters())
+    for name, param in own.items():
+        assert torch.allclose(w[p + name].grad, param.grad, atol=2e-5, rtol=1e-3), name
+    assert torch.allclose(w[p + "final_layernorm.weight"].grad, norms["final_layernorm"].weight.grad,
+                          atol=2e-5, rtol=1e-3)
+
+
+def test_hybrid_routing_and_norm_against_closed_forms():
+    """What the mathematics fixes: zero weights make the norm a plain normalisation; routing scores
+    are the k largest soft-max probabilities, in descending order, summing to 1 when renormalised;
+    one expert with top-1 routing and a zero shared gate weight reduces the block to that expert's
+    SwiGLU MLP plus half the shared expert's."""
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(1, 7, 32, generator=g)
+    y = OM.zero_centered_rms_norm(x, torch.zeros(32), 1e-6)
+    assert torch.allclose(y.pow(2).mean(-1), torch.ones(1, 7), atol=1e-4)
+    wr = torch.randn(6, 32, generator=g)
+    scores, idx = OM.moe_routing(x[0], wr, 3, True)
+    probs = F.softmax(x[0] @ wr.t(), dim=-1)
+    assert torch.equal(idx, probs.argsort(dim=-1, descending=True)[:, :3])
+    assert torch.allclose(scores.sum(-1), torch.ones(7), atol=1e-6)
+    raw, _ = OM.moe_routing(x[0], wr, 3, False)
+    assert torch.allclose(raw, probs.gather(1, idx), atol=1e-7)
+    shape = _hybrid_shape(num_experts=1, num_experts_per_tok=1, moe_intermediate_size=24,
+                          shared_expert_intermediate_size=40)
+    w = OM.random_weights(shape, 2, std=0.1)
+    p = "mtp_layers.0.mlp."
+    w[p + "shared_expert_gate.weight"].zero_()
+    got = OM.sparse_moe(x, w, p, shape)
+    gu, dn = w[p + "experts.gate_up_proj"][0], w[p + "experts.down_proj"][0]
+    a, b = F.linear(x, gu).chunk(2, dim=-1)
+    want = F.linear(F.silu(a) * b, dn) + 0.5 * OM.swiglu_mlp(x, w, p + "shared_expert.")
+    assert torch.allclose(got, want, atol=1e-5)
+
+
 def _inputs(shape, b, n, seed):
     g = torch.Generator().manual_seed(seed)
     return (torch.randint(0, shape.vocab_size, (b, n), generator=g),
