@@ -420,6 +420,32 @@ int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* position_ids,
                       int32_t heads, int32_t D, int32_t rotate, int32_t inverse,
                       int64_t position_offset, void* stream);
 
+/* The same with the two things the hybrid MTP flavours need (their layers are the library's
+ * Qwen3NextDecoderLayer / Qwen3_5DecoderLayer / Qwen3_5MoeDecoderLayer, wrapped at
+ * models/mtp/model_definitions.py:159-205): the token-major side has a head stride of its own
+ * (x_head_stride elements; the widened q projection holds [query | gate] per head, 2 D apart), and
+ * only the first rotary_dim elements of every head are rotated (pairs i, i + rotary_dim / 2; the
+ * rest is copied), rotary_dim a multiple of 16, inv_freq f32 [rotary_dim / 2]. */
+int spx_rope_relayout_partial(const void* x, int64_t ld_x, int32_t x_head_stride,
+                              const int64_t* position_ids, const float* inv_freq, void* out,
+                              int64_t ld_out, int64_t T, int32_t heads, int32_t D,
+                              int32_t rotary_dim, int32_t rotate, int32_t inverse,
+                              int64_t position_offset, void* stream);
+
+/* Output gate of the gated attention (`attn_output * torch.sigmoid(gate)` of Qwen3NextAttention,
+ * reached through models/mtp/model_definitions.py:159-205): y = bf16(o * bf16(sigmoid(gate))) on
+ * [rows, heads, D] bf16 tensors; o, y, dy, d_o have contiguous heads and a row stride, the gate
+ * and its gradient a row stride and a head stride (they are the second halves of the 2 D columns
+ * per head of the q projection and of its output gradient).  Backward: d_o = dy * sig,
+ * dgate = dy * o * sig * (1 - sig). */
+int spx_sigmoid_gate_fwd(const void* o, int64_t ld_o, const void* gate, int64_t ld_gate,
+                         int32_t gate_head_stride, void* y, int64_t ld_y, int64_t rows,
+                         int32_t heads, int32_t D, void* stream);
+int spx_sigmoid_gate_bwd(const void* o, int64_t ld_o, const void* gate, int64_t ld_gate,
+                         int32_t gate_head_stride, const void* dy, int64_t ld_dy, void* d_o,
+                         int64_t ld_do, void* dgate, int64_t ld_dgate, int32_t dgate_head_stride,
+                         int64_t rows, int32_t heads, int32_t D, void* stream);
+
 /* out = bf16(silu(gate)) * up  (LlamaMLP / Qwen3MLP act_fn(gate_proj(x)) * up_proj(x)),
  * bf16; and its backward.  rows x F elements per tensor, each with its own row stride, so
  * that gate and up can be the two column halves of one merged gate/up projection. */
@@ -486,6 +512,50 @@ int spx_gemm_bf16_tn(const void* a, int64_t lda, const void* b, int64_t ldb,
 int spx_gemm_bf16_tn_f32(const void* a, int64_t lda, const void* b, int64_t ldb,
                          void* c, int64_t ldc, int64_t M, int64_t N, int64_t T,
                          int accumulate, void* stream);
+
+/* ---------------------------------------------------------------- sparse MoE block
+ * The expert products of the MoE MLP of the hybrid MTP flavours (Qwen3NextSparseMoeBlock /
+ * Qwen3NextExperts of the library, reached through models/mtp/model_definitions.py:159-205).
+ * The library loops over the experts that were hit, gathering each one's tokens; here the
+ * (token, slot) pairs are sorted by expert once and every product runs over all experts in one
+ * launch.  group_offsets: int32 [groups + 1] on the device, non-decreasing from 0 to at most
+ * `rows`; group e owns the sorted rows [group_offsets[e], group_offsets[e + 1]).  The host never
+ * reads the offsets.
+ *
+ * spx_gemm_bf16_nt_grouped: c[r, :] = a[r, :] * b_e^T for the rows r of group e, b_e = b +
+ * e * b_group_stride ([N, K], row stride ldb).  The workspace (spx_gemm_grouped_workspace_bytes,
+ * 4-byte aligned) holds the tile table the launch builds on the device.  Same operand rules as
+ * spx_gemm_bf16_nt.
+ * spx_gemm_bf16_tn_grouped: c_e[M, N] (+)= a[rows of e, :M]^T * b[rows of e, :N], c_e = c +
+ * e * c_group_stride elements; out_f32 selects an fp32 c; without `accumulate` an empty group
+ * gets zeros.  Same operand rules as spx_gemm_bf16_tn. */
+int64_t spx_gemm_grouped_workspace_bytes(int64_t rows, int64_t groups);
+int spx_gemm_bf16_nt_grouped(const void* a, int64_t lda, const void* b, int64_t ldb,
+                             int64_t b_group_stride, void* c, int64_t ldc, int64_t rows,
+                             int64_t N, int64_t K, const int32_t* group_offsets, int64_t groups,
+                             void* workspace, int64_t workspace_bytes, void* stream);
+int spx_gemm_bf16_tn_grouped(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                             int64_t ldc, int64_t c_group_stride, int64_t M, int64_t N,
+                             int64_t rows, const int32_t* group_offsets, int64_t groups,
+                             int out_f32, int accumulate, void* stream);
+
+/* Row movement between the token order [tokens, H] and the expert-sorted order [rows, H] (bf16;
+ * index_select / index_add_ of Qwen3NextExperts.forward and their backward):
+ *   spx_moe_gather_rows:  out[p] = scale[p] * x[src_row[p]]   (scale f32 [rows] or NULL; an index
+ *                         outside [0, src_rows) gives a zero row)
+ *   spx_moe_combine_rows: out[t] = sum_j weight[t, j] * sorted[pos[t, j]], j = 0 .. k-1 in that
+ *                         order in fp32, one rounding (weight f32 [tokens, k] or NULL = ones)
+ *   spx_moe_pair_dot:     out[t, j] = <a[t], sorted[pos[t, j]]> in fp32 (the gradient of the
+ *                         routing weights). */
+int spx_moe_gather_rows(const void* x, int64_t ld_x, int64_t src_rows, const int32_t* src_row,
+                        const float* scale, void* out, int64_t ld_out, int64_t rows, int64_t H,
+                        void* stream);
+int spx_moe_combine_rows(const void* sorted, int64_t ld_sorted, int64_t sorted_rows,
+                         const int32_t* pos, const float* weight, void* out, int64_t ld_out,
+                         int64_t tokens, int32_t k, int64_t H, void* stream);
+int spx_moe_pair_dot(const void* a, int64_t ld_a, const void* sorted, int64_t ld_sorted,
+                     int64_t sorted_rows, const int32_t* pos, float* out, int64_t tokens,
+                     int32_t k, int64_t H, void* stream);
 
 #ifdef __cplusplus
 }

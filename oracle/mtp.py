@@ -124,13 +124,29 @@ def moe_routing(x2, router_weight, top_k: int, renormalise: bool):
     return top.to(logits.dtype), idx
 
 
-def sparse_moe(x, w, prefix, shape: HybridShape):
+def sparse_moe(x, w, prefix, shape: HybridShape, routing: dict | None = None):
     """``Qwen3NextSparseMoeBlock`` on ``[1, L, H]``: every token's ``top_k`` experts (SwiGLU with
     the merged ``gate_up_proj [E, 2I, H]``, ``down_proj [E, H, I]``) weighted by the router scores,
-    plus the shared expert scaled by ``sigmoid(shared_expert_gate(x))``."""
+    plus the shared expert scaled by ``sigmoid(shared_expert_gate(x))``.
+
+    ``routing`` (tests of a bf16 implementation, whose top-k may differ from the fp32 one where two
+    probabilities nearly tie): ``routing["forced"]``, expert ids ``[L, k]`` to use instead of this
+    function's own top-k (the scores are still this function's probabilities at those experts);
+    the function's own choice, all probabilities and the router logits are left in
+    ``routing["own"]`` / ``routing["probs"]`` / ``routing["logits"]``."""
     x2 = x.reshape(-1, x.shape[-1])
     scores, idx = moe_routing(x2, w[prefix + "gate.weight"], shape.num_experts_per_tok,
                               shape.norm_topk_prob)
+    if routing is not None:
+        logits = F.linear(x2, w[prefix + "gate.weight"])
+        probs = F.softmax(logits, dtype=torch.float, dim=-1)
+        routing["own"], routing["probs"], routing["logits"] = idx, probs.detach(), logits.detach()
+        if routing.get("forced") is not None:
+            idx = routing["forced"]
+            scores = probs.gather(1, idx)
+            if shape.norm_topk_prob:
+                scores = scores / scores.sum(dim=-1, keepdim=True)
+            scores = scores.to(logits.dtype)
     out = torch.zeros_like(x2)
     gate_up, down = w[prefix + "experts.gate_up_proj"], w[prefix + "experts.down_proj"]
     for e in range(shape.num_experts):
@@ -145,7 +161,7 @@ def sparse_moe(x, w, prefix, shape: HybridShape):
     return (out + shared).reshape(x.shape)
 
 
-def _hybrid_layer(x, w, p, shape: HybridShape, cos, sin, mask, attn):
+def _hybrid_layer(x, w, p, shape: HybridShape, cos, sin, mask, attn, routing=None):
     """One row ``[1, L, H]`` through the full-attention decoder layer of the hybrid flavours."""
     n = x.shape[1]
     hq, hkv, d = shape.num_attention_heads, shape.num_key_value_heads, shape.head_dim
@@ -170,7 +186,7 @@ def _hybrid_layer(x, w, p, shape: HybridShape, cos, sin, mask, attn):
     x = x + F.linear(o, w[a + "o_proj.weight"])
     z = zero_centered_rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
     if shape.num_experts > 0:
-        return x + sparse_moe(z, w, p + "mlp.", shape)
+        return x + sparse_moe(z, w, p + "mlp.", shape, routing)
     return x + swiglu_mlp(z, w, p + "mlp.")
 
 
@@ -204,7 +220,7 @@ def _qwen3_layer(x, w, p, shape: DraftShape, cos, sin, mask, attn):
     return x + swiglu_mlp(z, w, p + "mlp.")
 
 
-def mtp_layer(hidden, embeds, w, shape: DraftShape, cos, sin, mask, attn="dense"):
+def mtp_layer(hidden, embeds, w, shape: DraftShape, cos, sin, mask, attn="dense", routing=None):
     """models/mtp/model_definitions.py:95-116 on one row."""
     p = "mtp_layers.0."
     hybrid = isinstance(shape, HybridShape)
@@ -212,14 +228,20 @@ def mtp_layer(hidden, embeds, w, shape: DraftShape, cos, sin, mask, attn="dense"
     hn = norm(hidden, w[p + "hidden_layernorm.weight"], shape.rms_norm_eps)
     en = norm(embeds, w[p + "token_layernorm.weight"], shape.rms_norm_eps)
     proj = F.linear(torch.cat([en, hn], dim=-1), w[p + "input_proj.weight"])
-    out = (_hybrid_layer if hybrid else _qwen3_layer)(proj, w, p, shape, cos, sin, mask, attn)
+    if hybrid:
+        out = _hybrid_layer(proj, w, p, shape, cos, sin, mask, attn, routing)
+    else:
+        out = _qwen3_layer(proj, w, p, shape, cos, sin, mask, attn)
     return norm(out, w[p + "final_layernorm.weight"], shape.rms_norm_eps)
 
 
 def mtp_forward(w, shape: DraftShape, input_ids, hidden_states, position_ids=None, loss_mask=None,
-                step_weights=None, num_steps: int = 3, attn: str = "dense", attention_mask=None):
+                step_weights=None, num_steps: int = 3, attn: str = "dense", attention_mask=None,
+                routing=None):
     """``(logits_list, loss, metrics)`` of models/mtp/core.py:114-231.  ``attention_mask``
-    (``[B, L]`` padding mask) replaces the packed-sequence mask as in core.py:180-186."""
+    (``[B, L]`` padding mask) replaces the packed-sequence mask as in core.py:180-186.
+    ``routing``: a list with one dict per (step, batch row), in that order, handed to
+    ``sparse_moe`` (see there)."""
     input_ids = input_ids.long()
     b, n = input_ids.shape
     if step_weights is not None and len(step_weights) != num_steps:
@@ -248,7 +270,7 @@ def mtp_forward(w, shape: DraftShape, input_ids, hidden_states, position_ids=Non
             cos, sin = rope_tables(pos[r], rotary_dim(shape), shape.rope_theta, hid.dtype,
                                    shape.rope_scaling)
             rows.append(mtp_layer(hid[r:r + 1], emb[r:r + 1].to(hid.dtype), w, shape, cos, sin,
-                                  masks[r], attn))
+                                  masks[r], attn, None if routing is None else routing[step * b + r]))
         out = torch.cat(rows, dim=0)
         logits = F.linear(out, w["lm_head.weight"])
         logits_list.append(logits)

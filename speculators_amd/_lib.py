@@ -75,7 +75,20 @@ SIGNATURES["spx_unpack_rows"] = [_P, _I64, _P, _I64, _I64, _I64, _P, _I64, _P]
 SIGNATURES["spx_gemm_bf16_nt_rows"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P, _P]
 SIGNATURES["spx_gemm_bf16_tn"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I, _P]
 SIGNATURES["spx_gemm_bf16_tn_f32"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I, _P]
-RESTYPES = {"spx_ttt_attn_workspace_bytes": c_int64, "spx_ttt_attn_fwd_static_max_bytes": c_int64, "spx_dflash_attn_workspace_bytes": c_int64,
+SIGNATURES["spx_rope_relayout_partial"] = [_P, _I64, _I32, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _I32,
+                                           _I64, _P]
+SIGNATURES["spx_sigmoid_gate_fwd"] = [_P, _I64, _P, _I64, _I32, _P, _I64, _I64, _I32, _I32, _P]
+SIGNATURES["spx_sigmoid_gate_bwd"] = [_P, _I64, _P, _I64, _I32, _P, _I64, _P, _I64, _P, _I64, _I32, _I64, _I32,
+                                      _I32, _P]
+SIGNATURES["spx_gemm_grouped_workspace_bytes"] = [_I64, _I64]
+SIGNATURES["spx_gemm_bf16_nt_grouped"] = [_P, _I64, _P, _I64, _I64, _P, _I64, _I64, _I64, _I64, _P, _I64, _P,
+                                          _I64, _P]
+SIGNATURES["spx_gemm_bf16_tn_grouped"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I64, _P, _I64, _I, _I,
+                                          _P]
+SIGNATURES["spx_moe_gather_rows"] = [_P, _I64, _I64, _P, _P, _P, _I64, _I64, _I64, _P]
+SIGNATURES["spx_moe_combine_rows"] = [_P, _I64, _I64, _P, _P, _P, _I64, _I64, _I32, _I64, _P]
+SIGNATURES["spx_moe_pair_dot"] = [_P, _I64, _P, _I64, _I64, _P, _P, _I64, _I32, _I64, _P]
+RESTYPES = {"spx_gemm_grouped_workspace_bytes": c_int64, "spx_ttt_attn_workspace_bytes": c_int64, "spx_ttt_attn_fwd_static_max_bytes": c_int64, "spx_dflash_attn_workspace_bytes": c_int64,
             "spx_rmsnorm_bwd_slots": c_int64}
 
 _lib = None

@@ -202,8 +202,10 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
                                                    const int64_t* __restrict__ pos,
                                                    const float* __restrict__ inv_freq,
                                                    uint16_t* __restrict__ out, int64_t ld_out, int T,
-                                                   int heads, int D, int rotate, int64_t pos_offset) {
-  // one thread: 8 consecutive d of the first half and the matching 8 of the second half
+                                                   int heads, int D, int rotate, int64_t pos_offset,
+                                                   int tok_head_stride, int rot) {
+  // one thread: 8 consecutive d of the first half of the rotated part and the matching 8 of its
+  // second half, or 16 consecutive d of the part that passes unrotated (rot < D: partial rotary)
   const int per_row = D / 16;
   const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t total = (int64_t)T * heads * per_row;
@@ -211,16 +213,18 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
   const int d0 = (int)(item % per_row) * 8;
   const int h = (int)((item / per_row) % heads);
   const int t = (int)(item / ((int64_t)per_row * heads));
-  const int half = D / 2;
+  const bool pass = d0 * 2 >= rot;  // items past the rotated part copy 16 contiguous elements
+  const int half = pass ? 8 : rot / 2;
+  const int dA = pass ? d0 * 2 : d0;
   // the head-major side is [heads][T][D] with a head stride of its own (0 = T * D, contiguous):
   // it may be a window of a longer key / value cache
   const int64_t hs = INVERSE ? (ld_x ? ld_x : (int64_t)T * D) : (ld_out ? ld_out : (int64_t)T * D);
-  const uint16_t* src = INVERSE ? x + (int64_t)h * hs + (int64_t)t * D : x + (int64_t)t * ld_x + h * D;
-  uint16_t* dst = INVERSE ? out + (int64_t)t * ld_out + h * D : out + (int64_t)h * hs + (int64_t)t * D;
+  const uint16_t* src = INVERSE ? x + (int64_t)h * hs + (int64_t)t * D : x + (int64_t)t * ld_x + h * tok_head_stride;
+  uint16_t* dst = INVERSE ? out + (int64_t)t * ld_out + h * tok_head_stride : out + (int64_t)h * hs + (int64_t)t * D;
   float a[8], b[8], oa[8], ob[8];
-  unpack8f(*reinterpret_cast<const u32x4*>(src + d0), a);
-  unpack8f(*reinterpret_cast<const u32x4*>(src + half + d0), b);
-  if (rotate) {
+  unpack8f(*reinterpret_cast<const u32x4*>(src + dA), a);
+  unpack8f(*reinterpret_cast<const u32x4*>(src + half + dA), b);
+  if (rotate && !pass) {
     const float p = (float)(pos[t] + pos_offset);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -236,8 +240,53 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
 #pragma unroll
     for (int e = 0; e < 8; ++e) { oa[e] = a[e]; ob[e] = b[e]; }
   }
-  *reinterpret_cast<u32x4*>(dst + d0) = pack8f(oa);
-  *reinterpret_cast<u32x4*>(dst + half + d0) = pack8f(ob);
+  *reinterpret_cast<u32x4*>(dst + dA) = pack8f(oa);
+  *reinterpret_cast<u32x4*>(dst + half + dA) = pack8f(ob);
+}
+
+// Output gate of the gated attention (Qwen3-Next): y = bf16(o * bf16(sigmoid(gate))), every tensor
+// [rows, heads, D] with a row stride and a head stride of its own (the gate is the second half of
+// every head's 2 D columns of the widened q projection).  One thread: 8 consecutive elements.
+__global__ __launch_bounds__(256) void sigmoid_gate_fwd_kernel(
+    const uint16_t* __restrict__ o, int64_t ld_o, const uint16_t* __restrict__ gate, int64_t ld_g, int hs_g,
+    uint16_t* __restrict__ y, int64_t ld_y, int64_t rows, int heads, int D) {
+  const int per_head = D / 8;
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (item >= rows * heads * per_head) return;
+  const int d0 = (int)(item % per_head) * 8;
+  const int h = (int)((item / per_head) % heads);
+  const int64_t r = item / ((int64_t)per_head * heads);
+  float a[8], g[8], out[8];
+  unpack8f(*reinterpret_cast<const u32x4*>(o + r * ld_o + h * D + d0), a);
+  unpack8f(*reinterpret_cast<const u32x4*>(gate + r * ld_g + (int64_t)h * hs_g + d0), g);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = a[e] * round_bf16(1.f / (1.f + __expf(-g[e])));
+  *reinterpret_cast<u32x4*>(y + r * ld_y + h * D + d0) = pack8f(out);
+}
+
+// do = bf16(dy * sig), dgate = bf16(dy * o * sig * (1 - sig)), sig = sigmoid(gate) in fp32
+__global__ __launch_bounds__(256) void sigmoid_gate_bwd_kernel(
+    const uint16_t* __restrict__ o, int64_t ld_o, const uint16_t* __restrict__ gate, int64_t ld_g, int hs_g,
+    const uint16_t* __restrict__ dy, int64_t ld_dy, uint16_t* __restrict__ d_o, int64_t ld_do,
+    uint16_t* __restrict__ dgate, int64_t ld_dg, int hs_dg, int64_t rows, int heads, int D) {
+  const int per_head = D / 8;
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (item >= rows * heads * per_head) return;
+  const int d0 = (int)(item % per_head) * 8;
+  const int h = (int)((item / per_head) % heads);
+  const int64_t r = item / ((int64_t)per_head * heads);
+  float a[8], g[8], d[8], oa[8], og[8];
+  unpack8f(*reinterpret_cast<const u32x4*>(o + r * ld_o + h * D + d0), a);
+  unpack8f(*reinterpret_cast<const u32x4*>(gate + r * ld_g + (int64_t)h * hs_g + d0), g);
+  unpack8f(*reinterpret_cast<const u32x4*>(dy + r * ld_dy + h * D + d0), d);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float sg = 1.f / (1.f + __expf(-g[e]));
+    oa[e] = d[e] * sg;
+    og[e] = d[e] * a[e] * sg * (1.f - sg);
+  }
+  *reinterpret_cast<u32x4*>(d_o + r * ld_do + h * D + d0) = pack8f(oa);
+  *reinterpret_cast<u32x4*>(dgate + r * ld_dg + (int64_t)h * hs_dg + d0) = pack8f(og);
 }
 
 // ---------------------------------------------------------------- SwiGLU
@@ -472,19 +521,87 @@ extern "C" int spx_add_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weig
                             dw_scratch, rows, H, stream);
 }
 
+static int rope_relayout_impl(const char* fn, const void* x, int64_t ld_x, const int64_t* position_ids,
+                              const float* inv_freq, void* out, int64_t ld_out, int64_t T, int32_t heads,
+                              int32_t D, int32_t rotate, int32_t inverse, int64_t position_offset,
+                              int32_t tok_head_stride, int32_t rot, void* stream);
+
 extern "C" int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* position_ids,
                                  const float* inv_freq, void* out, int64_t ld_out, int64_t T,
                                  int32_t heads, int32_t D, int32_t rotate, int32_t inverse,
                                  int64_t position_offset, void* stream) {
-  SPX_REQUIRE(T > 0 && heads > 0 && D > 0 && D % 16 == 0, "T, heads > 0 and D a multiple of 16");
-  SPX_REQUIRE(x && out && (!rotate || (position_ids && inv_freq)), "null buffer");
-  SPX_REQUIRE(al16(x) && al16(out), "buffers must be 16-byte aligned");
+  return rope_relayout_impl(__func__, x, ld_x, position_ids, inv_freq, out, ld_out, T, heads, D, rotate,
+                            inverse, position_offset, D, D, stream);
+}
+
+extern "C" int spx_rope_relayout_partial(const void* x, int64_t ld_x, int32_t x_head_stride,
+                                         const int64_t* position_ids, const float* inv_freq, void* out,
+                                         int64_t ld_out, int64_t T, int32_t heads, int32_t D,
+                                         int32_t rotary_dim, int32_t rotate, int32_t inverse,
+                                         int64_t position_offset, void* stream) {
+  return rope_relayout_impl(__func__, x, ld_x, position_ids, inv_freq, out, ld_out, T, heads, D, rotate,
+                            inverse, position_offset, x_head_stride, rotary_dim, stream);
+}
+
+#define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fn, what); } while (0)
+extern "C" int spx_sigmoid_gate_fwd(const void* o, int64_t ld_o, const void* gate, int64_t ld_gate,
+                                    int32_t gate_head_stride, void* y, int64_t ld_y, int64_t rows,
+                                    int32_t heads, int32_t D, void* stream) {
+  const char* fn = __func__;
+  SPX_REQ_FN(rows > 0 && heads > 0 && D > 0 && D % 8 == 0, "rows, heads > 0 and D a positive multiple of 8");
+  SPX_REQ_FN(o && gate && y && al16(o) && al16(gate) && al16(y), "null or unaligned buffer");
+  const int64_t hd = (int64_t)heads * D;
+  SPX_REQ_FN(ld_o % 8 == 0 && ld_y % 8 == 0 && ld_gate % 8 == 0 && gate_head_stride % 8 == 0, "strides must be multiples of 8");
+  SPX_REQ_FN(ld_o >= hd && ld_y >= hd && gate_head_stride >= D && ld_gate >= (int64_t)(heads - 1) * gate_head_stride + D,
+             "stride too small");
+  const int64_t items = rows * heads * (D / 8);
+  hipLaunchKernelGGL(sigmoid_gate_fwd_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const uint16_t*>(o), ld_o,
+                     reinterpret_cast<const uint16_t*>(gate), ld_gate, (int)gate_head_stride,
+                     reinterpret_cast<uint16_t*>(y), ld_y, rows, (int)heads, (int)D);
+  return check_launch(fn);
+}
+
+extern "C" int spx_sigmoid_gate_bwd(const void* o, int64_t ld_o, const void* gate, int64_t ld_gate,
+                                    int32_t gate_head_stride, const void* dy, int64_t ld_dy, void* d_o,
+                                    int64_t ld_do, void* dgate, int64_t ld_dgate,
+                                    int32_t dgate_head_stride, int64_t rows, int32_t heads, int32_t D,
+                                    void* stream) {
+  const char* fn = __func__;
+  SPX_REQ_FN(rows > 0 && heads > 0 && D > 0 && D % 8 == 0, "rows, heads > 0 and D a positive multiple of 8");
+  SPX_REQ_FN(o && gate && dy && d_o && dgate, "null buffer");
+  SPX_REQ_FN(al16(o) && al16(gate) && al16(dy) && al16(d_o) && al16(dgate), "buffers must be 16-byte aligned");
+  const int64_t hd = (int64_t)heads * D;
+  SPX_REQ_FN(ld_o % 8 == 0 && ld_dy % 8 == 0 && ld_do % 8 == 0 && ld_gate % 8 == 0 && ld_dgate % 8 == 0 &&
+                 gate_head_stride % 8 == 0 && dgate_head_stride % 8 == 0, "strides must be multiples of 8");
+  SPX_REQ_FN(ld_o >= hd && ld_dy >= hd && ld_do >= hd && gate_head_stride >= D && dgate_head_stride >= D &&
+                 ld_gate >= (int64_t)(heads - 1) * gate_head_stride + D &&
+                 ld_dgate >= (int64_t)(heads - 1) * dgate_head_stride + D, "stride too small");
+  const int64_t items = rows * heads * (D / 8);
+  hipLaunchKernelGGL(sigmoid_gate_bwd_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const uint16_t*>(o), ld_o,
+                     reinterpret_cast<const uint16_t*>(gate), ld_gate, (int)gate_head_stride,
+                     reinterpret_cast<const uint16_t*>(dy), ld_dy, reinterpret_cast<uint16_t*>(d_o), ld_do,
+                     reinterpret_cast<uint16_t*>(dgate), ld_dgate, (int)dgate_head_stride, rows, (int)heads, (int)D);
+  return check_launch(fn);
+}
+
+static int rope_relayout_impl(const char* fn, const void* x, int64_t ld_x, const int64_t* position_ids,
+                              const float* inv_freq, void* out, int64_t ld_out, int64_t T, int32_t heads,
+                              int32_t D, int32_t rotate, int32_t inverse, int64_t position_offset,
+                              int32_t tok_head_stride, int32_t rot, void* stream) {
+  SPX_REQ_FN(T > 0 && heads > 0 && D > 0 && D % 16 == 0, "T, heads > 0 and D a multiple of 16");
+  SPX_REQ_FN(rot > 0 && rot <= D && rot % 16 == 0, "the rotary dimension must be a multiple of 16 in 16 .. D");
+  SPX_REQ_FN(tok_head_stride >= D && tok_head_stride % 8 == 0, "bad head stride of the token-major side");
+  SPX_REQ_FN(x && out && (!rotate || (position_ids && inv_freq)), "null buffer");
+  SPX_REQ_FN(al16(x) && al16(out), "buffers must be 16-byte aligned");
+  const int64_t tok_row = (int64_t)(heads - 1) * tok_head_stride + D;
   if (inverse) {
-    SPX_REQUIRE(ld_out % 8 == 0 && ld_out >= (int64_t)heads * D, "bad output row stride");
-    SPX_REQUIRE(ld_x == 0 || (ld_x % 8 == 0 && ld_x >= T * D), "bad head stride of the head-major input");
+    SPX_REQ_FN(ld_out % 8 == 0 && ld_out >= tok_row, "bad output row stride");
+    SPX_REQ_FN(ld_x == 0 || (ld_x % 8 == 0 && ld_x >= T * D), "bad head stride of the head-major input");
   } else {
-    SPX_REQUIRE(ld_x % 8 == 0 && ld_x >= (int64_t)heads * D, "bad input row stride");
-    SPX_REQUIRE(ld_out == 0 || (ld_out % 8 == 0 && ld_out >= T * D), "bad head stride of the head-major output");
+    SPX_REQ_FN(ld_x % 8 == 0 && ld_x >= tok_row, "bad input row stride");
+    SPX_REQ_FN(ld_out == 0 || (ld_out % 8 == 0 && ld_out >= T * D), "bad head stride of the head-major output");
   }
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const int64_t total = T * heads * (D / 16);
@@ -493,12 +610,13 @@ extern "C" int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* pos
   auto op = reinterpret_cast<uint16_t*>(out);
   if (inverse)
     hipLaunchKernelGGL(rope_kernel<true>, dim3(grid), dim3(256), 0, st, xp, ld_x, position_ids, inv_freq, op,
-                       ld_out, (int)T, (int)heads, (int)D, (int)rotate, position_offset);
+                       ld_out, (int)T, (int)heads, (int)D, (int)rotate, position_offset, (int)tok_head_stride, (int)rot);
   else
     hipLaunchKernelGGL(rope_kernel<false>, dim3(grid), dim3(256), 0, st, xp, ld_x, position_ids, inv_freq, op,
-                       ld_out, (int)T, (int)heads, (int)D, (int)rotate, position_offset);
-  return check_launch(__func__);
+                       ld_out, (int)T, (int)heads, (int)D, (int)rotate, position_offset, (int)tok_head_stride, (int)rot);
+  return check_launch(fn);
 }
+#undef SPX_REQ_FN
 
 static unsigned swiglu_grid(int64_t n8) {
   return (unsigned)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536);

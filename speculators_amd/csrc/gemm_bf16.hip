@@ -76,7 +76,8 @@ __global__ __launch_bounds__(kGemmThreads, SPX_GEMM_MINW)
 __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf16_nt_kernel(
     const uint16_t* __restrict__ A, int64_t lda, const uint16_t* __restrict__ B, int64_t ldb,
     uint16_t* __restrict__ C, int64_t ldc, int M, int N, int K, int tiles_m, int tiles_n,
-    const int32_t* __restrict__ m_live) {
+    const int32_t* __restrict__ m_live, const int32_t* __restrict__ tile_tab,
+    const int32_t* __restrict__ group_off, int64_t b_group_stride) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   // the row count may live on the device (rows packed to the front by the producer of A): the tile
   // grid shrinks to the rows that count and the workgroups beyond it leave at once
@@ -84,6 +85,11 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
     M = min(M, max(*m_live, 0));
     tiles_m = (M + kTM - 1) / kTM;
   }
+  // grouped product: the rows of A are sorted by group, group e = rows [group_off[e], group_off[e+1])
+  // is multiplied by its own B (b_group_stride elements apart).  The tile rows come from a table on
+  // the device (tile_tab[0] = their number, then (group, first row) per tile row): no tile spans
+  // two groups, and the host never learns the group sizes
+  if (tile_tab) tiles_m = min(tile_tab[0], tiles_m);
 
   // workgroup id -> tile: XCD-contiguous bands, then groups of GROUP_M tile rows.  Workgroups go to
   // the eight XCDs round robin: XCD x gets the ids x, x + 8, ...; they are renumbered so that each XCD
@@ -103,7 +109,14 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   const int group_sz = min(tiles_m - first_m, GROUP_M);
   const int tile_m = first_m + (pid % in_group) % group_sz;
   const int tile_n = (pid % in_group) / group_sz;
-  const int m0 = tile_m * kTM, n0 = tile_n * kTN;
+  int m0 = tile_m * kTM;
+  const int n0 = tile_n * kTN;
+  if (tile_tab) {
+    const int grp = tile_tab[1 + 2 * tile_m];
+    m0 = tile_tab[2 + 2 * tile_m];
+    M = min(M, max(group_off[grp + 1], 0));  // rows from here on belong to the next group
+    B += (int64_t)grp * b_group_stride;
+  }
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -297,7 +310,9 @@ using namespace spx;
 
 #define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fname, what); } while (0)
 static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
-                        int64_t ldc, int64_t M, int64_t N, int64_t K, const int32_t* m_live, void* stream) {
+                        int64_t ldc, int64_t M, int64_t N, int64_t K, const int32_t* m_live, void* stream,
+                        const int32_t* tile_tab = nullptr, const int32_t* group_off = nullptr,
+                        int64_t b_group_stride = 0, int64_t groups = 0) {
   SPX_REQ_FN(M > 0 && N > 0 && K > 0, "M, N, K must be positive");
   SPX_REQ_FN(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "dimension too large");
   SPX_REQ_FN(a && b && c, "null buffer");
@@ -312,20 +327,84 @@ static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const voi
   const void* fn = imm ? reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<true>)
                        : reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<false>);
   if (int rc = ensure_dynamic_lds(fn, kGemmSmem, lds_set[imm], fname)) return rc;
-  const int tiles_m = (int)((M + kTM - 1) / kTM), tiles_n = (int)((N + kTN - 1) / kTN);
-  SPX_REQ_FN((int64_t)tiles_m * tiles_n < (1ll << 31), "too many tiles");
+  // grouped: every group may end in a partly filled tile row
+  const int64_t tiles_m64 = (M + kTM - 1) / kTM + (tile_tab ? groups : 0);
+  const int tiles_n = (int)((N + kTN - 1) / kTN);
+  SPX_REQ_FN(tiles_m64 * tiles_n < (1ll << 31), "too many tiles");
+  const int tiles_m = (int)tiles_m64;
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(kGemmThreads);
   if (imm)
     hipLaunchKernelGGL(gemm_bf16_nt_kernel<true>, grid, block, kGemmSmem, st,
                        reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,
-                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live);
+                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live,
+                       tile_tab, group_off, b_group_stride);
   else
     hipLaunchKernelGGL(gemm_bf16_nt_kernel<false>, grid, block, kGemmSmem, st,
                        reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,
-                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live);
+                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live,
+                       tile_tab, group_off, b_group_stride);
   return check_launch(fname);
 }
-#undef SPX_REQ_FN
+
+namespace spx {
+// tab[0] = number of tile rows, then (group, first row) of every tile row: group e contributes
+// ceil(rows_e / kTM) of them.  One workgroup; thread t owns a contiguous run of groups.
+__global__ __launch_bounds__(256) void gemm_group_tiles_kernel(const int32_t* __restrict__ group_off, int groups,
+                                                               int rows, int32_t* __restrict__ tab) {
+  __shared__ int sums[256];
+  const int t = threadIdx.x;
+  const int per = (groups + 255) / 256;
+  const int e0 = min(t * per, groups), e1 = min(e0 + per, groups);
+  int mine = 0;
+  // (offsets are clamped to [0, rows]: the table is sized for that many rows whatever they hold)
+  auto clamped = [&](int e) { return min(max(group_off[e], 0), rows); };
+  for (int e = e0; e < e1; ++e) mine += (max(clamped(e + 1) - clamped(e), 0) + kTM - 1) / kTM;
+  sums[t] = mine;
+  __syncthreads();
+  if (t == 0) {
+    int run = 0;
+    for (int i = 0; i < 256; ++i) {
+      const int v = sums[i];
+      sums[i] = run;
+      run += v;
+    }
+    tab[0] = run;
+  }
+  __syncthreads();
+  int at = sums[t];
+  for (int e = e0; e < e1; ++e) {
+    const int r0 = clamped(e), r1 = clamped(e + 1);
+    for (int r = r0; r < r1; r += kTM, ++at) {
+      tab[1 + 2 * at] = e;
+      tab[2 + 2 * at] = r;
+    }
+  }
+}
+}  // namespace spx
+
+extern "C" int64_t spx_gemm_grouped_workspace_bytes(int64_t rows, int64_t groups) {
+  if (rows < 0 || groups < 0) return 0;
+  return (int64_t)sizeof(int32_t) * (1 + 2 * ((rows + kTM - 1) / kTM + groups));
+}
+
+extern "C" int spx_gemm_bf16_nt_grouped(const void* a, int64_t lda, const void* b, int64_t ldb,
+                                        int64_t b_group_stride, void* c, int64_t ldc, int64_t rows,
+                                        int64_t N, int64_t K, const int32_t* group_offsets,
+                                        int64_t groups, void* workspace, int64_t workspace_bytes,
+                                        void* stream) {
+  const char* fname = __func__;
+  SPX_REQ_FN(groups > 0 && groups < (1 << 24), "groups must be positive");
+  SPX_REQ_FN(group_offsets && workspace, "null group offsets or workspace");
+  SPX_REQ_FN(workspace_bytes >= spx_gemm_grouped_workspace_bytes(rows, groups), "workspace too small");
+  SPX_REQ_FN(((uintptr_t)workspace) % 4 == 0 && b_group_stride % 8 == 0 && b_group_stride >= 0,
+             "unaligned workspace or group stride");
+  int32_t* tab = reinterpret_cast<int32_t*>(workspace);
+  hipLaunchKernelGGL(gemm_group_tiles_kernel, dim3(1), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     group_offsets, (int)groups, (int)rows, tab);
+  if (int rc = check_launch(fname)) return rc;
+  return gemm_nt_impl(fname, a, lda, b, ldb, c, ldc, rows, N, K, nullptr, stream, tab, group_offsets,
+                      b_group_stride, groups);
+}
 
 extern "C" int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
                                 int64_t ldc, int64_t M, int64_t N, int64_t K, void* stream) {
@@ -341,3 +420,4 @@ extern "C" int spx_gemm_bf16_nt_rows(const void* a, int64_t lda, const void* b, 
   }
   return gemm_nt_impl(__func__, a, lda, b, ldb, c, ldc, M, N, K, m_live, stream);
 }
+#undef SPX_REQ_FN

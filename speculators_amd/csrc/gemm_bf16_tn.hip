@@ -59,8 +59,21 @@ __device__ __forceinline__ i16x4 lds_read_tr16(const uint8_t* p) {
 template <int OUT>
 __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_bf16_tn_kernel(
     const uint16_t* __restrict__ A, int64_t lda, const uint16_t* __restrict__ B, int64_t ldb,
-    void* __restrict__ Cv, int64_t ldc, int M, int N, int T, int tiles_m, int tiles_n) {
+    void* __restrict__ Cv, int64_t ldc, int M, int N, int T, int tiles_m, int tiles_n,
+    const int32_t* __restrict__ group_off, int64_t c_group_stride) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  // grouped product (blockIdx.y = group): the contraction runs over the group's rows
+  // [group_off[e], group_off[e+1]) of both operands, and every group has a C of its own.  An empty
+  // group multiplies nothing: zeros are written (or C is left as it is when the result is added)
+  if (group_off) {
+    const int e = blockIdx.y;
+    const int t0 = min(max(group_off[e], 0), T), t1 = min(max(group_off[e + 1], t0), T);
+    A += (int64_t)t0 * lda;
+    B += (int64_t)t0 * ldb;
+    T = t1 - t0;
+    Cv = reinterpret_cast<uint8_t*>(Cv) + e * c_group_stride * (OUT >= 2 ? 4 : 2);
+    if ((OUT & 1) && T == 0) return;
+  }
 
   // workgroup id -> tile: XCD-contiguous bands, then groups of GROUP_M tile rows
   const int n_wg = tiles_m * tiles_n;
@@ -96,8 +109,8 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
   // the slab's first row included, is in the vector register, which is what the range check sees: rows
   // past T lie outside the resource and read as zero.  A 16-byte chunk past the last column would read
   // the next row instead, so those lanes get an offset outside the resource.
-  const u32x4 ares = make_rsrc(A + m0, (uint32_t)((((int64_t)T - 1) * lda + min(M - m0, kTM)) * 2));
-  const u32x4 bres = make_rsrc(B + n0, (uint32_t)((((int64_t)T - 1) * ldb + min(N - n0, kTN)) * 2));
+  const u32x4 ares = make_rsrc(A + m0, T > 0 ? (uint32_t)((((int64_t)T - 1) * lda + min(M - m0, kTM)) * 2) : 0u);
+  const u32x4 bres = make_rsrc(B + n0, T > 0 ? (uint32_t)((((int64_t)T - 1) * ldb + min(N - n0, kTN)) * 2) : 0u);
 
   // global side: wave-load j of this wave covers slab rows 2 (wave * kLA + j) + lane / 32; the lane's LDS
   // position is 16-byte chunk lane % 32 of the row, which holds the chunk of 64-byte block
@@ -320,17 +333,18 @@ using namespace spx;
 #define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fname, what); } while (0)
 template <int OUT>
 static int launch_tn(const char* fname, const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
-                     int64_t ldc, int64_t M, int64_t N, int64_t T, void* stream) {
+                     int64_t ldc, int64_t M, int64_t N, int64_t T, void* stream,
+                     const int32_t* group_off = nullptr, int64_t c_group_stride = 0, int64_t groups = 1) {
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   static std::atomic<uint64_t> lds_set;  // per kernel instantiation, one bit per device
   if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&tn::gemm_bf16_tn_kernel<OUT>), tn::kSmem,
                                   lds_set, fname))
     return rc;
   const int tiles_m = (int)((M + tn::kTM - 1) / tn::kTM), tiles_n = (int)((N + tn::kTN - 1) / tn::kTN);
-  const dim3 grid((unsigned)(tiles_m * tiles_n)), block(tn::kThreads);
+  const dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)groups), block(tn::kThreads);
   hipLaunchKernelGGL(tn::gemm_bf16_tn_kernel<OUT>, grid, block, tn::kSmem, st,
                      reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb, c,
-                     ldc, (int)M, (int)N, (int)T, tiles_m, tiles_n);
+                     ldc, (int)M, (int)N, (int)T, tiles_m, tiles_n, group_off, c_group_stride);
   return check_launch(fname);
 }
 
@@ -347,7 +361,6 @@ static int gemm_tn_check(const char* fname, const void* a, int64_t lda, const vo
   SPX_REQ_FN((int64_t)((M + tn::kTM - 1) / tn::kTM) * ((N + tn::kTN - 1) / tn::kTN) < (1ll << 31), "too many tiles");
   return SPX_OK;
 }
-#undef SPX_REQ_FN
 
 extern "C" int spx_gemm_bf16_tn(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
                                 int64_t ldc, int64_t M, int64_t N, int64_t T, int accumulate,
@@ -364,3 +377,20 @@ extern "C" int spx_gemm_bf16_tn_f32(const void* a, int64_t lda, const void* b, i
   return accumulate ? launch_tn<3>(__func__, a, lda, b, ldb, c, ldc, M, N, T, stream)
                     : launch_tn<2>(__func__, a, lda, b, ldb, c, ldc, M, N, T, stream);
 }
+
+extern "C" int spx_gemm_bf16_tn_grouped(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                                        int64_t ldc, int64_t c_group_stride, int64_t M, int64_t N,
+                                        int64_t rows, const int32_t* group_offsets, int64_t groups,
+                                        int out_f32, int accumulate, void* stream) {
+  const char* fname = __func__;
+  if (int rc = gemm_tn_check(fname, a, lda, b, ldb, c, ldc, M, N, rows)) return rc;
+  SPX_REQ_FN(group_offsets && groups > 0 && groups < 65536, "null group offsets or a group count outside 1 .. 65535");
+  SPX_REQ_FN(c_group_stride >= (M - 1) * ldc + N, "groups of c overlap");
+  SPX_REQ_FN(c_group_stride % (out_f32 ? 4 : 8) == 0, "the groups of c must be 16-byte aligned among each other");
+  if (out_f32)
+    return accumulate ? launch_tn<3>(fname, a, lda, b, ldb, c, ldc, M, N, rows, stream, group_offsets, c_group_stride, groups)
+                      : launch_tn<2>(fname, a, lda, b, ldb, c, ldc, M, N, rows, stream, group_offsets, c_group_stride, groups);
+  return accumulate ? launch_tn<1>(fname, a, lda, b, ldb, c, ldc, M, N, rows, stream, group_offsets, c_group_stride, groups)
+                    : launch_tn<0>(fname, a, lda, b, ldb, c, ldc, M, N, rows, stream, group_offsets, c_group_stride, groups);
+}
+#undef SPX_REQ_FN

@@ -187,24 +187,94 @@ class _RopeRelayout(torch.autograd.Function):
         x2 = x.reshape(t, heads * d)
         if x2.stride(1) != 1:
             x2 = x2.contiguous()
+        # the table covers the rotated part of a head: all of it, or its first elements only
+        rot = 2 * inv_freq.numel() if rotate else d
         out = torch.empty(1, heads, t, d, device=x.device, dtype=torch.bfloat16)
-        _lib.call("spx_rope_relayout", _lib.ptr(x2), x2.stride(0), _lib.ptr(position_ids),
-                  _lib.ptr(inv_freq), _lib.ptr(out), 0, t, heads, d, int(rotate), 0, int(offset),
+        _lib.call("spx_rope_relayout_partial", _lib.ptr(x2), x2.stride(0), d, _lib.ptr(position_ids),
+                  _lib.ptr(inv_freq), _lib.ptr(out), 0, t, heads, d, rot, int(rotate), 0, int(offset),
                   _lib.stream_ptr(x.device))
         ctx.save_for_backward(position_ids, inv_freq)
-        ctx.meta = (x.shape, heads, d, t, rotate, offset)
+        ctx.meta = (x.shape, heads, d, t, rotate, offset, rot)
         return out
 
     @staticmethod
     def backward(ctx, dout):
         position_ids, inv_freq = ctx.saved_tensors
-        shape, heads, d, t, rotate, offset = ctx.meta
+        shape, heads, d, t, rotate, offset, rot = ctx.meta
         dout = dout.to(torch.bfloat16).contiguous()
         dx = torch.empty(t, heads * d, device=dout.device, dtype=torch.bfloat16)
-        _lib.call("spx_rope_relayout", _lib.ptr(dout), 0, _lib.ptr(position_ids), _lib.ptr(inv_freq),
-                  _lib.ptr(dx), heads * d, t, heads, d, int(rotate), 1, int(offset),
+        _lib.call("spx_rope_relayout_partial", _lib.ptr(dout), 0, d, _lib.ptr(position_ids),
+                  _lib.ptr(inv_freq), _lib.ptr(dx), heads * d, t, heads, d, rot, int(rotate), 1, int(offset),
                   _lib.stream_ptr(dout.device))
         return dx.view(shape), None, None, None, None, None
+
+
+class _SplitQueryGate(torch.autograd.Function):
+    """``[T, heads * 2 D]`` (the widened q projection of the gated attention: per head the query,
+    then its output gate) -> the two ``[T, heads, D]`` halves as strided views; the backward writes
+    both gradients into one buffer of the input's layout."""
+
+    @staticmethod
+    def forward(ctx, y, heads):
+        t = y.shape[-2]
+        d = y.shape[-1] // (2 * heads)
+        y4 = y.reshape(t, heads, 2, d)
+        ctx.meta = (y.shape, t, heads, d)
+        return y4[:, :, 0], y4[:, :, 1]
+
+    @staticmethod
+    def backward(ctx, dq, dgate):
+        shape, t, heads, d = ctx.meta
+        dy = torch.empty(t, heads, 2, d, device=(dq if dq is not None else dgate).device, dtype=torch.bfloat16)
+        for half, g in ((0, dq), (1, dgate)):
+            if g is None:
+                dy[:, :, half].zero_()
+            else:
+                dy[:, :, half].copy_(g.reshape(t, heads, d))
+        return dy.view(shape), None
+
+
+def split_query_gate(y: torch.Tensor, heads: int):
+    return _SplitQueryGate.apply(y, heads)
+
+
+class _SigmoidGate(torch.autograd.Function):
+    """``o * sigmoid(gate)`` with the rounding points of the bf16 eager form; ``o [.., T, heads * D]``
+    contiguous rows, ``gate [T, heads, D]`` with any row and head stride."""
+
+    @staticmethod
+    def forward(ctx, o, gate):
+        _need_bf16(o, gate)
+        t, heads, d = gate.shape
+        o2 = o.reshape(t, heads * d)
+        if o2.stride(1) != 1:
+            o2 = o2.contiguous()
+        if gate.stride(2) != 1:
+            gate = gate.contiguous()
+        y = torch.empty(t, heads * d, device=o.device, dtype=torch.bfloat16)
+        _lib.call("spx_sigmoid_gate_fwd", _lib.ptr(o2), o2.stride(0), _lib.ptr(gate), gate.stride(0),
+                  gate.stride(1), _lib.ptr(y), heads * d, t, heads, d, _lib.stream_ptr(o.device))
+        ctx.save_for_backward(o2, gate)
+        ctx.o_shape = o.shape
+        return y.view(o.shape)
+
+    @staticmethod
+    def backward(ctx, dy):
+        o2, gate = ctx.saved_tensors
+        t, heads, d = gate.shape
+        dy2 = dy.reshape(t, heads * d).to(torch.bfloat16)
+        if dy2.stride(1) != 1:
+            dy2 = dy2.contiguous()
+        d_o = torch.empty(t, heads * d, device=dy.device, dtype=torch.bfloat16)
+        dgate = torch.empty(t, heads, d, device=dy.device, dtype=torch.bfloat16)
+        _lib.call("spx_sigmoid_gate_bwd", _lib.ptr(o2), o2.stride(0), _lib.ptr(gate), gate.stride(0),
+                  gate.stride(1), _lib.ptr(dy2), dy2.stride(0), _lib.ptr(d_o), heads * d, _lib.ptr(dgate),
+                  heads * d, d, t, heads, d, _lib.stream_ptr(dy.device))
+        return d_o.view(ctx.o_shape), dgate
+
+
+def sigmoid_gate(o: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    return _SigmoidGate.apply(o, gate)
 
 
 def rope_relayout(x, position_ids, inv_freq, heads: int, rotate: bool = True, offset: int = 0):
@@ -219,7 +289,9 @@ def rope_relayout(x, position_ids, inv_freq, heads: int, rotate: bool = True, of
 def rope_inv_freq(head_dim: int, theta: float, device, scaling: dict | None = None) -> torch.Tensor:
     """fp32 inverse frequencies, evaluated like the HF rotary initialisation the draft layer
     inherits from its verifier config: ``scaling`` is the HF rope-parameter dict
-    (``rope_type`` "default", "linear" or "llama3"; Llama-3.1 verifiers use "llama3")."""
+    (``rope_type`` "default", "linear" or "llama3"; Llama-3.1 verifiers use "llama3").
+    ``head_dim`` is the number of rotated elements per head (all of them, or the first
+    ``int(head_dim * partial_rotary_factor)`` for a partial rotary embedding)."""
     inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
     kind = "default"
     if scaling:

@@ -7,9 +7,12 @@ Keeps the call contract of ``MTPDraftModel.forward`` (models/mtp/core.py:114-231
 
 with the reference's metric keys (``loss_step_{k}``, ``loss_sum``, ``loss_total``) and
 state-dict names (``mtp_layers.0.*``, ``embed_tokens``, ``lm_head``).  The layer is
-the Qwen3 flavour of ``MTPLayerMixin`` (models/mtp/model_definitions.py:78-151):
-two RMSNorms, ``input_proj (2H -> H)``, a Qwen3 decoder layer with per-head q/k
-RMSNorm, a final RMSNorm.  Attention runs on the HIP interval-masked kernel (causal
+``MTPLayerMixin`` (models/mtp/model_definitions.py:78-151) around a decoder layer:
+two RMSNorms, ``input_proj (2H -> H)``, the layer, a final RMSNorm.  The layer is the
+Qwen3 one with per-head q/k RMSNorm (``qwen3``) or the full-attention layer of the hybrid
+flavours (``qwen3_next``, ``qwen3_5_text``, ``qwen3_5_moe_text``, models/mtp/model_definitions.py:
+159-205; ``hybrid.py``): gain ``1 + w`` norms, gated attention, partial rotary embedding,
+dense or sparse-MoE MLP.  Attention runs on the HIP interval-masked kernel (causal
 inside each packed sequence, sequences found from the position restarts as
 ``create_causal_mask`` does at models/mtp/core.py:180-186), ``lm_head`` on the MFMA
 GEMM, the loss on the label cross-entropy kernel.
@@ -32,6 +35,7 @@ from . import fused_ops as FO
 from . import gemm
 from . import losses as L
 from .eagle3 import MLP, Attention, RMSNorm
+from .hybrid import HybridMTPLayer
 from .weights import WeightStager, compute_input
 
 IGNORE_INDEX = -100
@@ -59,6 +63,67 @@ class MTPConfig:
     model_type: str = "qwen3"
     attn_implementation: str = A.ATTN_IMPL_TTT
     qk_norm: bool = True  # Qwen3 attention
+    # hybrid flavours (qwen3_next, qwen3_5_text, qwen3_5_moe_text)
+    partial_rotary_factor: float = 1.0
+    num_experts: int = 0  # 0: dense MLP of intermediate_size
+    num_experts_per_tok: int = 0
+    moe_intermediate_size: int = 0
+    shared_expert_intermediate_size: int = 0
+    norm_topk_prob: bool = True
+
+    @property
+    def rotary_dim(self) -> int:
+        return int(self.head_dim * self.partial_rotary_factor)
+
+    @classmethod
+    def from_transformer_config(cls, tc, num_speculative_steps: int = 3, **overrides) -> "MTPConfig":
+        """From the verifier's (text) layer config, as ``MTPDraftModel.__init__`` reads
+        ``config.transformer_layer_config`` (models/mtp/core.py:82-90).  The hybrid flavours take
+        the layer at the last ``full_attention`` index (models/mtp/model_definitions.py:52-68); a
+        ``qwen3_next`` layer there is sparse when the library's ``Qwen3NextDecoderLayer`` makes it
+        so (``mlp_only_layers`` / ``decoder_sparse_step``), a ``qwen3_5_moe_text`` layer always."""
+        model_type = resolve_model_type(tc.model_type)
+        rope = dict(getattr(tc, "rope_parameters", None) or getattr(tc, "rope_scaling", None) or {})
+        theta = rope.pop("rope_theta", None) or getattr(tc, "rope_theta", 10000.0)
+        factor = rope.pop("partial_rotary_factor", None) or getattr(tc, "partial_rotary_factor", 1.0)
+        rope.pop("mrope_section", None)
+        rope.pop("mrope_interleaved", None)
+        kind = rope.get("rope_type", rope.get("type", "default"))
+        head_dim = getattr(tc, "head_dim", None) or tc.hidden_size // tc.num_attention_heads
+        kw = dict(hidden_size=tc.hidden_size, num_attention_heads=tc.num_attention_heads,
+                  num_key_value_heads=tc.num_key_value_heads, head_dim=head_dim,
+                  intermediate_size=tc.intermediate_size, vocab_size=tc.vocab_size,
+                  num_speculative_steps=num_speculative_steps, rms_norm_eps=tc.rms_norm_eps,
+                  rope_theta=float(theta), rope_scaling=None if kind == "default" else rope,
+                  model_type=model_type)
+        if model_type != "qwen3":
+            kw["partial_rotary_factor"] = float(factor)
+            sparse = model_type == "qwen3_5_moe_text"
+            if model_type == "qwen3_next":
+                types = list(getattr(tc, "layer_types", None) or [])
+                idx = max((i for i, t in enumerate(types) if t == "full_attention"), default=0)
+                if types and "full_attention" not in types:
+                    raise ValueError("Hybrid MTP layer requires at least one 'full_attention' entry in "
+                                     f"config.layer_types, got: {types}")
+                sparse = (idx not in (getattr(tc, "mlp_only_layers", None) or [])
+                          and tc.num_experts > 0 and (idx + 1) % tc.decoder_sparse_step == 0)
+            if sparse:
+                kw.update(num_experts=tc.num_experts, num_experts_per_tok=tc.num_experts_per_tok,
+                          moe_intermediate_size=tc.moe_intermediate_size,
+                          shared_expert_intermediate_size=tc.shared_expert_intermediate_size,
+                          norm_topk_prob=getattr(tc, "norm_topk_prob", True))
+        kw.update(overrides)
+        return cls(**kw)
+
+
+MODEL_TYPES = ("qwen3", "qwen3_next", "qwen3_5_text", "qwen3_5_moe_text")
+
+
+def resolve_model_type(model_type: str) -> str:
+    """models/mtp/model_definitions.py:31-35."""
+    if model_type in MODEL_TYPES:
+        return model_type
+    raise ValueError(f"Unsupported MTP model type '{model_type}'. Supported types: {sorted(MODEL_TYPES)}")
 
 
 class MTPLayer(nn.Module):
@@ -96,13 +161,13 @@ class MTPLayer(nn.Module):
 class MTPDraftModel(nn.Module):
     def __init__(self, config: MTPConfig):
         super().__init__()
-        if config.model_type != "qwen3":
-            raise ValueError(f"Unsupported MTP model type '{config.model_type}'. Supported types: ['qwen3']")
+        resolve_model_type(config.model_type)
         self.config = config
         self._stager = WeightStager()
         self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size)
         self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
-        self.mtp_layers = nn.ModuleList([MTPLayer(config, self._stager)])
+        layer_class = MTPLayer if config.model_type == "qwen3" else HybridMTPLayer
+        self.mtp_layers = nn.ModuleList([layer_class(config, self._stager)])
         # the verifier's embedding and head are frozen (model.py:70-71)
         self.embed_tokens.weight.requires_grad_(False)
         self.lm_head.weight.requires_grad_(False)
@@ -169,7 +234,7 @@ class MTPDraftModel(nn.Module):
                 raise ValueError(f"attention_mask must be {(b, n)}, got {tuple(attention_mask.shape)}")
             mask = A.create_padding_span_mask(attention_mask[:, :valid].to(device))
         flat_pos = pos.reshape(-1).contiguous()
-        inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device, cfg.rope_scaling)
+        inv_freq = FO.rope_inv_freq(cfg.rotary_dim, cfg.rope_theta, device, cfg.rope_scaling)
         layer = self.mtp_layers[0]
 
         current = hidden_states

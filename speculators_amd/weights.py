@@ -103,7 +103,7 @@ class Staged:
     is expected to run against it (the size of the input / output-gradient buffers)."""
 
     __slots__ = ("w", "token", "rows_of", "uses", "_wt", "_xs", "_fill", "_dys", "_live", "_extras",
-                 "_marked")
+                 "_marked", "_acc")
 
     def __init__(self, w, rows_of, uses: int = 1):
         self.w = w
@@ -117,6 +117,7 @@ class Staged:
         self._live = []    # (first row, rows) of the uses whose backward has run
         self._extras = []  # (dy, x) of uses outside the buffers
         self._marked = False
+        self._acc = None   # fp32 gradient buffer of uses that add their gradient themselves
 
     @property
     def trainable(self) -> bool:
@@ -126,7 +127,8 @@ class Staged:
     def wt(self) -> torch.Tensor:
         """``w.T`` contiguous (made on first use, kept with the staged weight)."""
         if self._wt is None:
-            self._wt = self.w.detach().t().contiguous()
+            # (a stack of expert weights [E, N, K] is transposed expert by expert)
+            self._wt = self.w.detach().transpose(-1, -2).contiguous()
         return self._wt
 
     # ---- forward side
@@ -177,15 +179,29 @@ class Staged:
             self._live.append((r0, dy2.shape[0]))
         else:
             self._extras.append((dy2, x2))
+        return self.mark()
+
+    def mark(self):
+        """What a use's backward returns as the gradient of ``token``: the empty marker that makes
+        autograd reach the staging node, once per backward; None afterwards."""
         if self._marked:
             return None
         self._marked = True
         return torch.zeros(1, device=self.w.device, dtype=torch.float32).expand(self.w.shape)
 
+    def grad_buffer(self):
+        """``(buffer, holds)``: the fp32 buffer of ``w``'s shape that uses which compute their weight
+        gradient themselves (the grouped expert products) add it to, and whether an earlier use of
+        this backward has written it already (the first one overwrites)."""
+        holds = self._acc is not None
+        if not holds:
+            self._acc = torch.empty(self.w.shape, device=self.w.device, dtype=torch.float32)
+        return self._acc, holds
+
     def finish(self):
         """The fp32 weight gradient of every recorded use (None if there is none): one product
         per run of adjacent uses in the buffers -- normally one -- plus one per outside use."""
-        acc = None
+        acc = self._acc
         runs: list = []
         for r0, n in sorted(self._live):
             if runs and runs[-1][0] + runs[-1][1] == r0:
@@ -196,7 +212,7 @@ class Staged:
             acc = wgrad_product(self._dys[r0:r0 + n], self._xs[r0:r0 + n], acc)
         for dy2, x2 in self._extras:
             acc = wgrad_product(dy2, x2, acc)
-        self._dys, self._live, self._extras, self._marked = None, [], [], False
+        self._dys, self._live, self._extras, self._marked, self._acc = None, [], [], False, None
         return acc
 
 
@@ -286,14 +302,18 @@ class WeightStager:
         self._fwd[key] = st
         return st
 
-    def gain(self, p: torch.Tensor) -> torch.Tensor:
+    def gain(self, p: torch.Tensor, plus_one: bool = False) -> torch.Tensor:
         """A small 1-D weight (an RMSNorm gain) in bf16 for the running forward: the parameter
         itself, or an ordinary differentiable cast of an fp32 master (its per-use gradients are
-        tiny; autograd sums them and casts the sum back)."""
-        key = ("gain", id(p))
+        tiny; autograd sums them and casts the sum back).  ``plus_one``: the gain is ``1 + p``
+        (evaluated in fp32), the form of the Qwen3-Next norms."""
+        key = ("gain", id(p), plus_one)
         hit = self._fwd.get(key)
         if hit is None:
             _check_param_dtype(p)
-            hit = p if p.dtype == torch.bfloat16 else p.to(torch.bfloat16)
+            if plus_one:
+                hit = (1.0 + p.float()).to(torch.bfloat16)
+            else:
+                hit = p if p.dtype == torch.bfloat16 else p.to(torch.bfloat16)
             self._fwd[key] = hit
         return hit
