@@ -82,9 +82,12 @@ SEQ_LEN3, TTT_STEPS3 = 8192, 5
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", choices=["eagle3", "eagle3-70b", "mtp", "dflash"], default="eagle3",
+    ap.add_argument("--workload", choices=["eagle3", "eagle3-70b", "mtp", "mtp-next", "dflash"],
+                    default="eagle3",
                     help="eagle3 = configs[1], the headline; eagle3-70b = configs[3]; mtp = configs[4] (MTP "
-                         "head, full-vocab CE); dflash = configs[2] (anchored blocks, 5 layers)")
+                         "head, full-vocab CE); mtp-next = the same shape with the qwen3_next layer (gated "
+                         "attention, partial rotary, 512-expert MoE); dflash = configs[2] (anchored blocks, "
+                         "5 layers)")
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seq-len", type=int, default=SEQ_LEN)
@@ -529,6 +532,9 @@ def cpu_baseline(torch, device, cfg, t, k_steps):
 CONFIG4 = dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=2, head_dim=256,
                intermediate_size=6144, vocab_size=151936, rms_norm_eps=1e-6, rope_theta=1000000.0)
 MTP_SEQ_LEN, MTP_BATCH, MTP_STEPS = 16384, 2, 3
+# the hybrid flavour of the same shape: the MTP layer of Qwen3-Next-80B-A3B (its model card's sizes)
+NEXT_EXTRA = dict(model_type="qwen3_next", partial_rotary_factor=0.25, num_experts=512, num_experts_per_tok=10,
+                  moe_intermediate_size=512, shared_expert_intermediate_size=512, norm_topk_prob=True)
 
 
 def run_mtp(args):
@@ -546,13 +552,14 @@ def run_mtp(args):
     torch.cuda.set_device(device)
     n = args.seq_len if args.seq_len != SEQ_LEN else MTP_SEQ_LEN
     b, k_steps = MTP_BATCH, MTP_STEPS
-    cfg = MTPConfig(num_speculative_steps=k_steps, **CONFIG4)
+    hybrid = args.workload == "mtp-next"
+    cfg = MTPConfig(num_speculative_steps=k_steps, **CONFIG4, **(NEXT_EXTRA if hybrid else {}))
     torch.manual_seed(0)
     model = MTPDraftModel(cfg)
     with torch.no_grad():
         for name, p_ in model.named_parameters():
             if name.endswith("norm.weight"):
-                p_.fill_(1.0)
+                p_.fill_(0.0 if hybrid else 1.0)  # the hybrid flavour's gain is 1 + weight
             else:
                 p_.normal_(0.0, 0.02)
     model = model.to(torch.bfloat16).to(device)
@@ -643,6 +650,29 @@ def run_mtp(args):
 
     rec("attn_bwd[head_dim 256, causal per row]", "mfma", 10.0 * pairs * d * hq,
         time_events(torch, attn_bwd, 3), k_steps)
+    del q, kk, vv, o, gd
+    if hybrid:
+        from speculators_amd import moe
+
+        e, topk, inter = cfg.num_experts, cfg.num_experts_per_tok, cfg.moe_intermediate_size
+        tok = b * t_row
+        idx = torch.stack([torch.randperm(e, device=device)[:topk] for _ in range(64)]).repeat(tok // 64 + 1, 1)[:tok]
+        _, src_row, _, off = moe.sort_pairs(idx, e)
+        pairs_n = tok * topk
+        xs = torch.randn(pairs_n, h, device=device).bfloat16()
+        w_gu = (torch.randn(e, 2 * inter, h, device=device) * 0.02).bfloat16()
+        hid = moe.gemm_nt_grouped(xs, w_gu, off)
+        rec("gemm_bf16_nt_kernel[grouped: experts' gate+up, T*k rows x H x 2I, 512 groups]", "mfma",
+            2.0 * pairs_n * h * 2 * inter, time_events(torch, lambda: moe.gemm_nt_grouped(xs, w_gu, off, out=hid), 3),
+            k_steps)
+        dw = torch.empty(e, 2 * inter, h, device=device, dtype=torch.float32)
+        rec("gemm_bf16_tn_kernel[grouped: experts' gate+up weight gradient, fp32]", "mfma",
+            2.0 * pairs_n * h * 2 * inter, time_events(torch, lambda: moe.gemm_tn_grouped(hid, xs, off, dw), 3),
+            k_steps)
+        xt = torch.randn(tok, h, device=device).bfloat16()
+        rec("gather_rows_kernel[T*k rows of H]", "hbm", 2.0 * pairs_n * h * 2,
+            time_events(torch, lambda: moe.gather_rows(xt, src_row), 3), 2 * k_steps)
+        del xs, w_gu, hid, dw, xt
     dominant = max(kernels, key=lambda r: r["ms_per_launch"] * r["launches_per_step"])
 
     cpu = None
@@ -650,7 +680,10 @@ def run_mtp(args):
         from oracle import mtp as OM
         from oracle.eagle3 import DraftShape
 
-        shape = DraftShape(draft_vocab_size=CONFIG4["vocab_size"], qk_norm=True, **CONFIG4)
+        if hybrid:
+            shape = OM.HybridShape(draft_vocab_size=CONFIG4["vocab_size"], **CONFIG4, **NEXT_EXTRA)
+        else:
+            shape = DraftShape(draft_vocab_size=CONFIG4["vocab_size"], qk_norm=True, **CONFIG4)
         tn = args.cpu_seq_len
         torch.set_num_threads(os.cpu_count() or 1)
         wts = {k_: v_.requires_grad_(k_ not in ("embed_tokens.weight", "lm_head.weight"))
@@ -678,7 +711,11 @@ def run_mtp(args):
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": f"configs[4]: MTP head, one Qwen3 decoder layer, hidden 2048, 16 q / 2 kv heads, "
+        "config": {"workload": (f"configs[4] shape with the qwen3_next layer: gated attention, rotary on 64 of 256, "
+                                f"512 experts top-10 of width 512 + shared expert 512, hidden 2048, 16 q / 2 kv "
+                                f"heads, head_dim 256, vocab 151936, batch {b}, seq {n}, {k_steps} prediction "
+                                f"steps, label cross-entropy, loss_mask Bernoulli(0.7)") if hybrid else
+                               f"configs[4]: MTP head, one Qwen3 decoder layer, hidden 2048, 16 q / 2 kv heads, "
                                f"head_dim 256, FFN 6144 (assumed), vocab 151936, batch {b}, seq {n}, "
                                f"{k_steps} prediction steps, label cross-entropy, loss_mask Bernoulli(0.7)",
                    "seq_len": n, "batch": b, "steps": k_steps, "tokens_per_step": tokens,
@@ -853,7 +890,7 @@ def main():
         print(f"bench.py: this build runs on ONE GPU (no collectives are built); got --gpus {args.gpus}",
               file=sys.stderr)
         sys.exit(2)
-    if args.workload == "mtp":
+    if args.workload in ("mtp", "mtp-next"):
         run_mtp(args)
         return
     if args.workload == "dflash":

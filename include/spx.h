@@ -539,6 +539,15 @@ int spx_gemm_bf16_tn_grouped(const void* a, int64_t lda, const void* b, int64_t 
                              int64_t rows, const int32_t* group_offsets, int64_t groups,
                              int out_f32, int accumulate, void* stream);
 
+/* out[b][c][r] = in[b][r][c] for `batches` bf16 matrices of R x C (multiples of 8), row strides
+ * ld_in / ld_out and batch strides in elements: the transposed copies the input-gradient
+ * products need of a weight stack (a product against W needs W^T in this library's NT form; the
+ * reference's autograd gets it from the BLAS library's NN form).  No counterpart in the
+ * reference. */
+int spx_transpose_bf16(const void* in, int64_t ld_in, int64_t batch_stride_in, void* out,
+                       int64_t ld_out, int64_t batch_stride_out, int64_t R, int64_t C,
+                       int64_t batches, void* stream);
+
 /* Row movement between the token order [tokens, H] and the expert-sorted order [rows, H] (bf16;
  * index_select / index_add_ of Qwen3NextExperts.forward and their backward):
  *   spx_moe_gather_rows:  out[p] = scale[p] * x[src_row[p]]   (scale f32 [rows] or NULL; an index

@@ -244,6 +244,41 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
   *reinterpret_cast<u32x4*>(dst + half + dA) = pack8f(ob);
 }
 
+// out[b][c][r] = in[b][r][c] for a stack of bf16 matrices (the per-expert transposes the input
+// gradient products of a stack of expert weights need).  One wave = one 64 x 64 tile, one lane =
+// one 8 x 8 block transposed in registers: every load and store instruction moves whole 128-byte
+// row segments (8 lanes x 16 bytes) and no LDS is involved.
+__global__ __launch_bounds__(256) void transpose_stack_kernel(const uint16_t* __restrict__ in, int64_t ld_in,
+                                                              int64_t bs_in, uint16_t* __restrict__ out,
+                                                              int64_t ld_out, int64_t bs_out, int R, int C,
+                                                              int tiles_r, int tiles_c, int64_t n_tiles) {
+  const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tile >= n_tiles) return;
+  const int lane = threadIdx.x & 63;
+  const int tc = (int)(tile % tiles_c);
+  const int tr = (int)((tile / tiles_c) % tiles_r);
+  const int64_t b = tile / ((int64_t)tiles_c * tiles_r);
+  const int r0 = tr * 64 + (lane >> 3) * 8, c0 = tc * 64 + (lane & 7) * 8;
+  if (r0 >= R || c0 >= C) return;  // R and C are multiples of 8: a block is inside or outside
+  const uint16_t* src = in + b * bs_in + (int64_t)r0 * ld_in + c0;
+  uint16_t* dst = out + b * bs_out + (int64_t)c0 * ld_out + r0;
+  u32x4 v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)i * ld_in);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    uint32_t o[4];
+#pragma unroll
+    for (int ip = 0; ip < 4; ++ip) {
+      const uint32_t a = v[2 * ip][j >> 1], c = v[2 * ip + 1][j >> 1];
+      o[ip] = (j & 1) ? ((a >> 16) | (c & 0xffff0000u)) : ((a & 0xffffu) | (c << 16));
+    }
+    u32x4 w;
+    w.x = o[0]; w.y = o[1]; w.z = o[2]; w.w = o[3];
+    *reinterpret_cast<u32x4*>(dst + (int64_t)j * ld_out) = w;
+  }
+}
+
 // Output gate of the gated attention (Qwen3-Next): y = bf16(o * bf16(sigmoid(gate))), every tensor
 // [rows, heads, D] with a row stride and a head stride of its own (the gate is the second half of
 // every head's 2 D columns of the widened q projection).  One thread: 8 consecutive elements.
@@ -544,6 +579,26 @@ extern "C" int spx_rope_relayout_partial(const void* x, int64_t ld_x, int32_t x_
 }
 
 #define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fn, what); } while (0)
+extern "C" int spx_transpose_bf16(const void* in, int64_t ld_in, int64_t batch_stride_in, void* out,
+                                  int64_t ld_out, int64_t batch_stride_out, int64_t R, int64_t C,
+                                  int64_t batches, void* stream) {
+  const char* fn = __func__;
+  SPX_REQ_FN(R > 0 && C > 0 && batches > 0 && R % 8 == 0 && C % 8 == 0 && R < (1ll << 31) && C < (1ll << 31),
+             "R and C must be positive multiples of 8");
+  SPX_REQ_FN(in && out && in != out && al16(in) && al16(out), "null, aliased or unaligned buffer");
+  SPX_REQ_FN(ld_in % 8 == 0 && ld_out % 8 == 0 && ld_in >= C && ld_out >= R, "row strides must be multiples of 8, ld_in >= C, ld_out >= R");
+  SPX_REQ_FN(batch_stride_in % 8 == 0 && batch_stride_out % 8 == 0 && batch_stride_in >= 0 && batch_stride_out >= 0,
+             "batch strides must be multiples of 8");
+  const int tiles_r = (int)((R + 63) / 64), tiles_c = (int)((C + 63) / 64);
+  const int64_t n_tiles = (int64_t)tiles_r * tiles_c * batches;
+  SPX_REQ_FN((n_tiles + 3) / 4 < (1ll << 31), "too many tiles");
+  hipLaunchKernelGGL(transpose_stack_kernel, dim3((unsigned)((n_tiles + 3) / 4)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const uint16_t*>(in), ld_in,
+                     batch_stride_in, reinterpret_cast<uint16_t*>(out), ld_out, batch_stride_out, (int)R, (int)C,
+                     tiles_r, tiles_c, n_tiles);
+  return check_launch(fn);
+}
+
 extern "C" int spx_sigmoid_gate_fwd(const void* o, int64_t ld_o, const void* gate, int64_t ld_gate,
                                     int32_t gate_head_stride, void* y, int64_t ld_y, int64_t rows,
                                     int32_t heads, int32_t D, void* stream) {

@@ -78,6 +78,20 @@ def _cat_bf16(params) -> torch.Tensor:
     return out
 
 
+def transposed_copy(w: torch.Tensor) -> torch.Tensor:
+    """``w.transpose(-1, -2)`` as a new contiguous tensor; a stack ``[E, N, K]`` is transposed
+    matrix by matrix.  On the library's kernel where its alignment rules hold."""
+    if (w.dtype == torch.bfloat16 and w.is_cuda and w.dim() in (2, 3) and w.is_contiguous()
+            and w.shape[-1] % 8 == 0 and w.shape[-2] % 8 == 0 and w.data_ptr() % 16 == 0):
+        r, c = w.shape[-2], w.shape[-1]
+        batches = w.shape[0] if w.dim() == 3 else 1
+        out = torch.empty(*w.shape[:-2], c, r, device=w.device, dtype=w.dtype)
+        _lib.call("spx_transpose_bf16", _lib.ptr(w), c, r * c, _lib.ptr(out), r, r * c, r, c, batches,
+                  _lib.stream_ptr(w.device))
+        return out
+    return w.transpose(-1, -2).contiguous()
+
+
 def _tn_ok(t: torch.Tensor) -> bool:
     return (t.dtype == torch.bfloat16 and t.stride(1) == 1 and t.shape[1] % 8 == 0
             and t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0)
@@ -127,8 +141,7 @@ class Staged:
     def wt(self) -> torch.Tensor:
         """``w.T`` contiguous (made on first use, kept with the staged weight)."""
         if self._wt is None:
-            # (a stack of expert weights [E, N, K] is transposed expert by expert)
-            self._wt = self.w.detach().transpose(-1, -2).contiguous()
+            self._wt = transposed_copy(self.w.detach())
         return self._wt
 
     # ---- forward side

@@ -282,3 +282,14 @@ def test_pack_row_map_and_unpack_rows(rows, with_labels):
     ref = torch.zeros(total, cols, dtype=torch.bfloat16)
     ref[:rows][live] = packed.cpu()[want[live].long()]
     assert torch.equal(back[:, :cols].cpu(), ref) and (back[:, cols:] == 5).all()
+
+
+@pytest.mark.parametrize("shape", [(64, 64), (8, 8), (72, 200), (3, 136, 72), (5, 64, 1024), (2, 8, 264)])
+def test_transposed_copy_of_a_matrix_or_a_stack(shape):
+    """Bit-exact against ``transpose(-1, -2).contiguous()``: tiles at and across the 64 x 64 edge."""
+    from speculators_amd.weights import transposed_copy
+
+    g = torch.Generator().manual_seed(sum(shape))
+    w = torch.randn(*shape, generator=g).bfloat16().cuda()
+    got = transposed_copy(w)
+    assert got.is_contiguous() and torch.equal(got, w.transpose(-1, -2).contiguous())
