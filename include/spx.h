@@ -425,12 +425,14 @@ int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* position_ids,
  * models/mtp/model_definitions.py:159-205): the token-major side has a head stride of its own
  * (x_head_stride elements; the widened q projection holds [query | gate] per head, 2 D apart), and
  * only the first rotary_dim elements of every head are rotated (pairs i, i + rotary_dim / 2; the
- * rest is copied), rotary_dim a multiple of 16, inv_freq f32 [rotary_dim / 2]. */
+ * rest is copied), rotary_dim a multiple of 16, inv_freq f32 [rotary_dim / 2].  table_scale
+ * multiplies cos and sin before they are rounded: the attention factor of the yarn frequency
+ * scaling (`cos = emb.cos() * self.attention_scaling` in the library's rotary modules), 1 otherwise. */
 int spx_rope_relayout_partial(const void* x, int64_t ld_x, int32_t x_head_stride,
                               const int64_t* position_ids, const float* inv_freq, void* out,
                               int64_t ld_out, int64_t T, int32_t heads, int32_t D,
                               int32_t rotary_dim, int32_t rotate, int32_t inverse,
-                              int64_t position_offset, void* stream);
+                              int64_t position_offset, float table_scale, void* stream);
 
 /* Output gate of the gated attention (`attn_output * torch.sigmoid(gate)` of Qwen3NextAttention,
  * reached through models/mtp/model_definitions.py:159-205): y = bf16(o * bf16(sigmoid(gate))) on

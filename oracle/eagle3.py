@@ -66,6 +66,7 @@ def rope_inv_freq(head_dim, theta, scaling=None):
     parameters the draft inherits from its verifier (models/eagle3/core.py:105-112 keeps them
     in the layer config; Llama-3.1 ships ``rope_type = "llama3"``):
       linear: every frequency divided by ``factor``;
+      yarn:   see ``_yarn_inv_freq``; its table factor is ``rope_table_scale``;
       llama3: wavelengths above ``L / low_freq_factor`` (L = original_max_position_embeddings)
               are divided by ``factor``, those below ``L / high_freq_factor`` kept, and the band
               between is blended linearly in ``L / wavelength``.
@@ -77,6 +78,8 @@ def rope_inv_freq(head_dim, theta, scaling=None):
     factor = float(scaling["factor"])
     if kind == "linear":
         return inv / factor
+    if kind == "yarn":
+        return _yarn_inv_freq(inv, head_dim, theta, scaling)
     if kind != "llama3":
         raise NotImplementedError(f"rope_type '{kind}'")
     lo, hi = float(scaling["low_freq_factor"]), float(scaling["high_freq_factor"])
@@ -89,12 +92,56 @@ def rope_inv_freq(head_dim, theta, scaling=None):
     return torch.where(band, mid, out)
 
 
+def _yarn_inv_freq(inv, dim, theta, scaling):
+    """YaRN frequencies (transformers ``_compute_yarn_parameters``): a linear ramp over the
+    frequency index between the index whose wavelength fits the original context ``beta_fast``
+    times and the one that fits it ``beta_slow`` times; below the ramp the frequency is kept,
+    above it divided by ``factor``."""
+    factor = float(scaling["factor"])
+    ctx = float(scaling["original_max_position_embeddings"])
+    fast, slow = scaling.get("beta_fast") or 32, scaling.get("beta_slow") or 1
+
+    def index_of(rotations):
+        return dim * math.log(ctx / (rotations * 2 * math.pi)) / (2 * math.log(theta))
+
+    lo, hi = index_of(fast), index_of(slow)
+    if scaling.get("truncate", True):
+        lo, hi = math.floor(lo), math.ceil(hi)
+    lo, hi = max(lo, 0), min(hi, dim - 1)
+    if lo == hi:
+        hi += 0.001
+    ramp = torch.clamp((torch.arange(dim // 2, dtype=torch.float32) - lo) / (hi - lo), 0, 1)
+    keep = 1 - ramp
+    freqs = theta ** (torch.arange(0, dim, 2, dtype=torch.int64).float() / dim)
+    return (1.0 / (factor * freqs)) * (1 - keep) + (1.0 / freqs) * keep
+
+
+def rope_table_scale(scaling=None) -> float:
+    """The factor on both tables (``attention_scaling`` of the HF rotary modules): 1 except for
+    yarn, where it is ``attention_factor`` if given, else ``0.1 ln(factor) + 1`` (with ``mscale`` /
+    ``mscale_all_dim``: the ratio of the two such terms)."""
+    kind = (scaling or {}).get("rope_type", (scaling or {}).get("type", "default"))
+    if kind != "yarn":
+        return 1.0
+    if scaling.get("attention_factor") is not None:
+        return float(scaling["attention_factor"])
+    factor = float(scaling["factor"])
+
+    def term(m=1.0):
+        return 1.0 if factor <= 1 else 0.1 * m * math.log(factor) + 1.0
+
+    if scaling.get("mscale") and scaling.get("mscale_all_dim"):
+        return term(scaling["mscale"]) / term(scaling["mscale_all_dim"])
+    return term()
+
+
 def rope_tables(position_ids, head_dim, theta, dtype, scaling=None):
-    """cos/sin ``[1, T, D]``: fp32 outer product, duplicated halves, cast."""
+    """cos/sin ``[1, T, D]``: fp32 outer product, duplicated halves, table scale, cast."""
     inv = rope_inv_freq(head_dim, theta, scaling)
     ang = position_ids.reshape(1, -1, 1).float() * inv.reshape(1, 1, -1)
     ang = torch.cat([ang, ang], dim=-1)
-    return ang.cos().to(dtype), ang.sin().to(dtype)
+    scale = rope_table_scale(scaling)
+    return (ang.cos() * scale).to(dtype), (ang.sin() * scale).to(dtype)
 
 
 def rotate_half(x):

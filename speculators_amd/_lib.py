@@ -76,7 +76,7 @@ SIGNATURES["spx_gemm_bf16_nt_rows"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64,
 SIGNATURES["spx_gemm_bf16_tn"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I, _P]
 SIGNATURES["spx_gemm_bf16_tn_f32"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I, _P]
 SIGNATURES["spx_rope_relayout_partial"] = [_P, _I64, _I32, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _I32,
-                                           _I64, _P]
+                                           _I64, _F, _P]
 SIGNATURES["spx_sigmoid_gate_fwd"] = [_P, _I64, _P, _I64, _I32, _P, _I64, _I64, _I32, _I32, _P]
 SIGNATURES["spx_sigmoid_gate_bwd"] = [_P, _I64, _P, _I64, _I32, _P, _I64, _P, _I64, _P, _I64, _I32, _I64, _I32,
                                       _I32, _P]

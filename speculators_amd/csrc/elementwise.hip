@@ -203,7 +203,7 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
                                                    const float* __restrict__ inv_freq,
                                                    uint16_t* __restrict__ out, int64_t ld_out, int T,
                                                    int heads, int D, int rotate, int64_t pos_offset,
-                                                   int tok_head_stride, int rot) {
+                                                   int tok_head_stride, int rot, float table_scale) {
   // one thread: 8 consecutive d of the first half of the rotated part and the matching 8 of its
   // second half, or 16 consecutive d of the part that passes unrotated (rot < D: partial rotary)
   const int per_row = D / 16;
@@ -229,8 +229,9 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float ang = p * inv_freq[d0 + e];
-      const float c = round_bf16(cosf(ang));
-      float s = round_bf16(sinf(ang));
+      // (table_scale: the attention factor some frequency scalings put on both tables, 1 otherwise)
+      const float c = round_bf16(cosf(ang) * table_scale);
+      float s = round_bf16(sinf(ang) * table_scale);
       if (INVERSE) s = -s;
       // x*cos + rotate_half(x)*sin with each bf16 op rounded
       oa[e] = round_bf16(a[e] * c) + round_bf16(-b[e] * s);
@@ -559,23 +560,23 @@ extern "C" int spx_add_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weig
 static int rope_relayout_impl(const char* fn, const void* x, int64_t ld_x, const int64_t* position_ids,
                               const float* inv_freq, void* out, int64_t ld_out, int64_t T, int32_t heads,
                               int32_t D, int32_t rotate, int32_t inverse, int64_t position_offset,
-                              int32_t tok_head_stride, int32_t rot, void* stream);
+                              int32_t tok_head_stride, int32_t rot, float table_scale, void* stream);
 
 extern "C" int spx_rope_relayout(const void* x, int64_t ld_x, const int64_t* position_ids,
                                  const float* inv_freq, void* out, int64_t ld_out, int64_t T,
                                  int32_t heads, int32_t D, int32_t rotate, int32_t inverse,
                                  int64_t position_offset, void* stream) {
   return rope_relayout_impl(__func__, x, ld_x, position_ids, inv_freq, out, ld_out, T, heads, D, rotate,
-                            inverse, position_offset, D, D, stream);
+                            inverse, position_offset, D, D, 1.f, stream);
 }
 
 extern "C" int spx_rope_relayout_partial(const void* x, int64_t ld_x, int32_t x_head_stride,
                                          const int64_t* position_ids, const float* inv_freq, void* out,
                                          int64_t ld_out, int64_t T, int32_t heads, int32_t D,
                                          int32_t rotary_dim, int32_t rotate, int32_t inverse,
-                                         int64_t position_offset, void* stream) {
+                                         int64_t position_offset, float table_scale, void* stream) {
   return rope_relayout_impl(__func__, x, ld_x, position_ids, inv_freq, out, ld_out, T, heads, D, rotate,
-                            inverse, position_offset, x_head_stride, rotary_dim, stream);
+                            inverse, position_offset, x_head_stride, rotary_dim, table_scale, stream);
 }
 
 #define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fn, what); } while (0)
@@ -644,7 +645,8 @@ extern "C" int spx_sigmoid_gate_bwd(const void* o, int64_t ld_o, const void* gat
 static int rope_relayout_impl(const char* fn, const void* x, int64_t ld_x, const int64_t* position_ids,
                               const float* inv_freq, void* out, int64_t ld_out, int64_t T, int32_t heads,
                               int32_t D, int32_t rotate, int32_t inverse, int64_t position_offset,
-                              int32_t tok_head_stride, int32_t rot, void* stream) {
+                              int32_t tok_head_stride, int32_t rot, float table_scale, void* stream) {
+  SPX_REQ_FN(table_scale > 0.f && table_scale < 1e4f, "the table scale must be positive and finite");
   SPX_REQ_FN(T > 0 && heads > 0 && D > 0 && D % 16 == 0, "T, heads > 0 and D a multiple of 16");
   SPX_REQ_FN(rot > 0 && rot <= D && rot % 16 == 0, "the rotary dimension must be a multiple of 16 in 16 .. D");
   SPX_REQ_FN(tok_head_stride >= D && tok_head_stride % 8 == 0, "bad head stride of the token-major side");
@@ -665,10 +667,12 @@ static int rope_relayout_impl(const char* fn, const void* x, int64_t ld_x, const
   auto op = reinterpret_cast<uint16_t*>(out);
   if (inverse)
     hipLaunchKernelGGL(rope_kernel<true>, dim3(grid), dim3(256), 0, st, xp, ld_x, position_ids, inv_freq, op,
-                       ld_out, (int)T, (int)heads, (int)D, (int)rotate, position_offset, (int)tok_head_stride, (int)rot);
+                       ld_out, (int)T, (int)heads, (int)D, (int)rotate, position_offset, (int)tok_head_stride, (int)rot,
+                       table_scale);
   else
     hipLaunchKernelGGL(rope_kernel<false>, dim3(grid), dim3(256), 0, st, xp, ld_x, position_ids, inv_freq, op,
-                       ld_out, (int)T, (int)heads, (int)D, (int)rotate, position_offset, (int)tok_head_stride, (int)rot);
+                       ld_out, (int)T, (int)heads, (int)D, (int)rotate, position_offset, (int)tok_head_stride, (int)rot,
+                       table_scale);
   return check_launch(fn);
 }
 #undef SPX_REQ_FN

@@ -178,6 +178,21 @@ def pair_norm_cat(a, b, weight_a, weight_b, eps: float, out=None) -> torch.Tenso
     return _PairNormCat.apply(a, b, weight_a, weight_b, eps, out)
 
 
+def rope_call(x_ptr, ld_x, x_head_stride, position_ids, inv_freq, out_ptr, ld_out, t, heads, d, rotate,
+              inverse, offset, table_scale, stream):
+    """One launch of the rotary relayout kernel; the rotated part of a head is what the frequency
+    table covers (all of it, or its first ``2 * len(inv_freq)`` elements)."""
+    rot = 2 * inv_freq.numel() if rotate else d
+    _lib.call("spx_rope_relayout_partial", x_ptr, ld_x, x_head_stride, _lib.ptr(position_ids), _lib.ptr(inv_freq),
+              out_ptr, ld_out, t, heads, d, rot, int(rotate), int(inverse), int(offset), float(table_scale),
+              stream)
+
+
+def table_scale_of(inv_freq) -> float:
+    """The attention factor ``rope_inv_freq`` attached to the table (1 for most scalings)."""
+    return float(getattr(inv_freq, "attention_scaling", 1.0))
+
+
 class _RopeRelayout(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, position_ids, inv_freq, heads, rotate, offset):
@@ -187,25 +202,22 @@ class _RopeRelayout(torch.autograd.Function):
         x2 = x.reshape(t, heads * d)
         if x2.stride(1) != 1:
             x2 = x2.contiguous()
-        # the table covers the rotated part of a head: all of it, or its first elements only
-        rot = 2 * inv_freq.numel() if rotate else d
+        scale = table_scale_of(inv_freq)
         out = torch.empty(1, heads, t, d, device=x.device, dtype=torch.bfloat16)
-        _lib.call("spx_rope_relayout_partial", _lib.ptr(x2), x2.stride(0), d, _lib.ptr(position_ids),
-                  _lib.ptr(inv_freq), _lib.ptr(out), 0, t, heads, d, rot, int(rotate), 0, int(offset),
-                  _lib.stream_ptr(x.device))
+        rope_call(_lib.ptr(x2), x2.stride(0), d, position_ids, inv_freq, _lib.ptr(out), 0, t, heads, d, rotate,
+                  0, offset, scale, _lib.stream_ptr(x.device))
         ctx.save_for_backward(position_ids, inv_freq)
-        ctx.meta = (x.shape, heads, d, t, rotate, offset, rot)
+        ctx.meta = (x.shape, heads, d, t, rotate, offset, scale)
         return out
 
     @staticmethod
     def backward(ctx, dout):
         position_ids, inv_freq = ctx.saved_tensors
-        shape, heads, d, t, rotate, offset, rot = ctx.meta
+        shape, heads, d, t, rotate, offset, scale = ctx.meta
         dout = dout.to(torch.bfloat16).contiguous()
         dx = torch.empty(t, heads * d, device=dout.device, dtype=torch.bfloat16)
-        _lib.call("spx_rope_relayout_partial", _lib.ptr(dout), 0, d, _lib.ptr(position_ids),
-                  _lib.ptr(inv_freq), _lib.ptr(dx), heads * d, t, heads, d, rot, int(rotate), 1, int(offset),
-                  _lib.stream_ptr(dout.device))
+        rope_call(_lib.ptr(dout), 0, d, position_ids, inv_freq, _lib.ptr(dx), heads * d, t, heads, d, rotate, 1,
+                  offset, scale, _lib.stream_ptr(dout.device))
         return dx.view(shape), None, None, None, None, None
 
 
@@ -288,12 +300,16 @@ def rope_relayout(x, position_ids, inv_freq, heads: int, rotate: bool = True, of
 
 def rope_inv_freq(head_dim: int, theta: float, device, scaling: dict | None = None) -> torch.Tensor:
     """fp32 inverse frequencies, evaluated like the HF rotary initialisation the draft layer
-    inherits from its verifier config: ``scaling`` is the HF rope-parameter dict
-    (``rope_type`` "default", "linear" or "llama3"; Llama-3.1 verifiers use "llama3").
-    ``head_dim`` is the number of rotated elements per head (all of them, or the first
-    ``int(head_dim * partial_rotary_factor)`` for a partial rotary embedding)."""
+    inherits from its verifier config: ``scaling`` is the HF rope-parameter dict (``rope_type``
+    "default", "linear", "llama3" or "yarn"; Llama-3.1 verifiers use "llama3").  ``head_dim`` is the
+    number of rotated elements per head (all of them, or the first
+    ``int(head_dim * partial_rotary_factor)`` for a partial rotary embedding).  The factor yarn puts
+    on the cos / sin tables rides on the returned tensor as ``attention_scaling`` (read by the rotary
+    kernels' wrappers through ``table_scale_of``).  "dynamic" and "longrope" pick their frequencies
+    from the length of the running sequence and are not built."""
     inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
     kind = "default"
+    table_scale = 1.0
     if scaling:
         kind = scaling.get("rope_type", scaling.get("type", "default"))
     if kind == "linear":
@@ -309,10 +325,51 @@ def rope_inv_freq(head_dim: int, theta: float, device, scaling: dict | None = No
         blended = (1 - smooth) * scaled / factor + smooth * scaled
         medium = (wavelen >= old_len / high) & (wavelen <= old_len / low)
         inv = torch.where(medium, blended, scaled)
+    elif kind == "yarn":
+        inv, table_scale = _yarn(inv, head_dim, theta, scaling)
     elif kind != "default":
         raise NotImplementedError(
-            f"rope_type '{kind}' is not built on the HIP path (default, linear and llama3 are)")
-    return inv.to(device)
+            f"rope_type '{kind}' is not built on the HIP path (default, linear, llama3 and yarn are)")
+    inv = inv.to(device)
+    inv.attention_scaling = table_scale
+    return inv
+
+
+def _yarn(inv, dim: int, theta: float, scaling: dict):
+    """YaRN (``_compute_yarn_parameters`` of transformers' ``modeling_rope_utils.py``): frequencies
+    whose wavelength fits the original context ``beta_fast`` times or more are kept, those that fit
+    it ``beta_slow`` times or less are divided by ``factor``, a linear ramp over the frequency index
+    blends between; both tables are scaled by ``0.1 ln(factor) + 1`` unless the config says
+    otherwise."""
+    factor = float(scaling["factor"])
+    old_len = float(scaling["original_max_position_embeddings"])
+    mscale, mscale_all = scaling.get("mscale"), scaling.get("mscale_all_dim")
+
+    def get_mscale(scale, m=1.0):
+        return 1.0 if scale <= 1 else 0.1 * m * math.log(scale) + 1.0
+
+    table_scale = scaling.get("attention_factor")
+    if table_scale is None:
+        if mscale and mscale_all:
+            table_scale = get_mscale(factor, mscale) / get_mscale(factor, mscale_all)
+        else:
+            table_scale = get_mscale(factor)
+    beta_fast = scaling.get("beta_fast") or 32
+    beta_slow = scaling.get("beta_slow") or 1
+
+    def correction_dim(rotations):
+        return dim * math.log(old_len / (rotations * 2 * math.pi)) / (2 * math.log(theta))
+
+    low, high = correction_dim(beta_fast), correction_dim(beta_slow)
+    if scaling.get("truncate", True):
+        low, high = math.floor(low), math.ceil(high)
+    low, high = max(low, 0), min(high, dim - 1)
+    if low == high:
+        high += 0.001
+    ramp = torch.clamp((torch.arange(dim // 2, dtype=torch.float32) - low) / (high - low), 0, 1)
+    keep = 1 - ramp
+    freqs = theta ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim)
+    return (1.0 / (factor * freqs)) * (1 - keep) + (1.0 / freqs) * keep, float(table_scale)
 
 
 class _SwiGLU(torch.autograd.Function):

@@ -14,6 +14,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
+from . import fused_ops as FO
 
 _MAX_SPAN = 0x7ffffff0 - 64  # bytes an operand of the weight-gradient product (gemm_tn) may span per call
 
@@ -171,6 +172,7 @@ class _QKVRope(torch.autograd.Function):
         qkv = torch.nn.functional.linear(x2, wcat)
         n = qkv.shape[1]
         st = _lib.stream_ptr(x.device)
+        scale = FO.table_scale_of(inv_freq)
         outs, col = [], 0
         for idx, (heads, rotate) in enumerate(((hq, 1), (hkv, 1), (hkv, 0))):
             if idx and kv_out is not None:
@@ -181,12 +183,12 @@ class _QKVRope(torch.autograd.Function):
                 out = torch.empty(1, heads, t, d, device=x.device, dtype=torch.bfloat16)
                 head_stride = 0
             part = qkv[:, col:]
-            _lib.call("spx_rope_relayout", _lib.ptr(part), n, _lib.ptr(position_ids), _lib.ptr(inv_freq),
-                      _lib.ptr(out), head_stride, t, heads, d, rotate, 0, int(offset), st)
+            FO.rope_call(_lib.ptr(part), n, d, position_ids, inv_freq, _lib.ptr(out), head_stride, t, heads, d,
+                         rotate, 0, offset, scale, st)
             outs.append(out)
             col += heads * d
         ctx.save_for_backward(x2, wcat, position_ids, inv_freq)
-        ctx.meta = (x.shape, hq, hkv, d, offset, n, staged)
+        ctx.meta = (x.shape, hq, hkv, d, offset, n, staged, scale)
         ctx.slot = staged.take(x2) if ctx.needs_input_grad[1] else -1
         ctx.set_materialize_grads(False)
         return tuple(outs)
@@ -194,7 +196,7 @@ class _QKVRope(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dq, dk, dv):
         x2, wcat, position_ids, inv_freq = ctx.saved_tensors
-        shape, hq, hkv, d, offset, n, staged = ctx.meta
+        shape, hq, hkv, d, offset, n, staged, scale = ctx.meta
         t = x2.shape[0]
         st = _lib.stream_ptr(x2.device)
         dqkv = staged.dy_slot(ctx.slot, t) if ctx.needs_input_grad[1] else None
@@ -211,8 +213,8 @@ class _QKVRope(torch.autograd.Function):
                 if not (g.stride(3) == 1 and g.stride(2) == d and g.stride(1) % 8 == 0
                         and g.stride(1) >= t * d and g.data_ptr() % 16 == 0):
                     g = g.contiguous()
-                _lib.call("spx_rope_relayout", _lib.ptr(g), g.stride(1), _lib.ptr(position_ids),
-                          _lib.ptr(inv_freq), _lib.ptr(part), n, t, heads, d, rotate, 1, int(offset), st)
+                FO.rope_call(_lib.ptr(g), g.stride(1), d, position_ids, inv_freq, _lib.ptr(part), n, t, heads, d,
+                             rotate, 1, offset, scale, st)
             col += heads * d
         dx = dw = None
         if ctx.needs_input_grad[0]:

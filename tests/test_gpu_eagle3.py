@@ -56,6 +56,11 @@ VARIANTS = [
     dict(num_hidden_layers=2, rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
                                             "high_freq_factor": 4.0,
                                             "original_max_position_embeddings": 64}),
+    # YaRN: blended frequencies and the attention factor on both tables (q/k/v as one product, and
+    # with per-head q/k norms the stand-alone rotary kernel)
+    dict(rope_scaling={"rope_type": "yarn", "factor": 16.0, "original_max_position_embeddings": 32}),
+    dict(qk_norm=True, rope_scaling={"rope_type": "yarn", "factor": 4.0, "original_max_position_embeddings": 64,
+                                     "attention_factor": 1.3}),
     dict(embed_requires_grad=True),  # marks the parameter trainable; the lookup itself has no graph
 ]
 

@@ -162,8 +162,15 @@ _LLAMA31 = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_
             "original_max_position_embeddings": 8192}
 
 
+_YARN = {"rope_type": "yarn", "factor": 4.0, "original_max_position_embeddings": 32768}
+
+
 @pytest.mark.parametrize("scaling", [None, {"rope_type": "linear", "factor": 4.0}, _LLAMA31,
-                                     dict(_LLAMA31, factor=32.0, original_max_position_embeddings=64)])
+                                     dict(_LLAMA31, factor=32.0, original_max_position_embeddings=64),
+                                     _YARN, dict(_YARN, factor=40.0, beta_fast=16, beta_slow=2,
+                                                 original_max_position_embeddings=4096, mscale=1.0,
+                                                 mscale_all_dim=0.7),
+                                     dict(_YARN, attention_factor=1.25, truncate=False)])
 @pytest.mark.parametrize("head_dim,theta", [(128, 500000.0), (64, 10000.0)])
 def test_rope_inv_freq_matches_transformers(scaling, head_dim, theta):
     """The oracle's inverse frequencies == the HF rotary initialisation (library routine), and
@@ -186,9 +193,18 @@ def test_rope_inv_freq_matches_transformers(scaling, head_dim, theta):
         factor = 1.0
     else:
         want, factor = ROPE_INIT_FUNCTIONS[kind](cfg, "cpu")
-    assert factor == 1.0
+    assert (factor == 1.0) == (kind != "yarn")
+    assert E.rope_table_scale(scaling) == pytest.approx(factor, rel=1e-12)
     assert torch.equal(got, want)
-    assert torch.equal(rope_inv_freq(head_dim, theta, "cpu", scaling), got)
+    mine = rope_inv_freq(head_dim, theta, "cpu", scaling)
+    assert torch.equal(mine, got) and mine.attention_scaling == pytest.approx(factor, rel=1e-12)
+    if kind == "yarn":  # the tables of the library's rotary module, attention factor included
+        from transformers.models.llama.modeling_llama import LlamaRotaryEmbedding
+
+        pos = torch.tensor([[0, 1, 5, 1000, 40000]])
+        cos, sin = LlamaRotaryEmbedding(cfg)(torch.zeros(1, 5, 8), pos)
+        mc, ms = E.rope_tables(pos[0], head_dim, theta, torch.float32, scaling)
+        assert torch.allclose(mc, cos, atol=1e-6) and torch.allclose(ms, sin, atol=1e-6)
     if kind == "llama3":  # the scaling does something: low frequencies shrink by `factor`
         base = E.rope_inv_freq(head_dim, theta, None)
         assert torch.equal(got[0], base[0]) and torch.isclose(got[-1], base[-1] / scaling["factor"])
@@ -197,7 +213,8 @@ def test_rope_inv_freq_matches_transformers(scaling, head_dim, theta):
 def test_rope_scaling_rejects_unknown_types():
     from speculators_amd.fused_ops import rope_inv_freq
 
-    with pytest.raises(NotImplementedError):
-        rope_inv_freq(64, 10000.0, "cpu", {"rope_type": "yarn", "factor": 2.0})
-    with pytest.raises(NotImplementedError):
-        E.rope_inv_freq(64, 10000.0, {"rope_type": "yarn", "factor": 2.0})
+    for kind in ("dynamic", "longrope"):
+        with pytest.raises(NotImplementedError):
+            rope_inv_freq(64, 10000.0, "cpu", {"rope_type": kind, "factor": 2.0})
+        with pytest.raises(NotImplementedError):
+            E.rope_inv_freq(64, 10000.0, {"rope_type": kind, "factor": 2.0})
