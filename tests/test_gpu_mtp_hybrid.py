@@ -319,3 +319,85 @@ def test_hybrid_model_forward_backward_matches_oracle(model_type, kw, master):
         err = (prm.grad.float().cpu() - want).abs().max().item()
         floor = (wb[name].grad.float() - want).abs().max().item()
         assert err <= max(2e-2 * scale, 2 * floor) + 1e-6, (name, err, floor, scale)
+
+
+def test_moe_block_at_the_qwen3_next_sizes():
+    """512 experts, top-10, hidden 2048, expert width 512 (the Qwen3-Next-80B-A3B MTP layer) on 6000
+    tokens: sampled tokens against a per-token fp32 evaluation with the block's own expert choice,
+    equivariance under a permutation of the tokens, and a sampled expert's weight gradient against
+    the fp32 product over exactly the tokens routed to it."""
+    from types import SimpleNamespace
+
+    from speculators_amd.hybrid import SparseMoeBlock
+    from speculators_amd.weights import WeightStager
+
+    cfg = SimpleNamespace(hidden_size=2048, num_experts=512, num_experts_per_tok=10, moe_intermediate_size=512,
+                          shared_expert_intermediate_size=512, norm_topk_prob=True)
+    torch.manual_seed(0)
+    stager = WeightStager()
+    block = SparseMoeBlock(cfg, stager)
+    with torch.no_grad():
+        for name, prm in block.named_parameters():
+            prm.normal_(0.0, 0.3 if name == "gate.weight" else 0.03)
+        # expert 7 is a favourite (more than one 256-row tile of tokens), experts 500.. are avoided
+        block.gate.weight[7, 0] = 4.0
+        block.gate.weight[500:, 0] = -40.0
+    block = block.bfloat16().cuda()
+    block.routing_log = []
+    t = 6000
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn(1, t, 2048, device="cuda", generator=g)
+    x[..., 0] = x[..., 0].abs() + 0.5
+    x = x.bfloat16().requires_grad_(True)
+    go = torch.randn(1, t, 2048, device="cuda", generator=g).bfloat16()
+    stager.begin()
+    out = block(x)
+    out.backward(go)
+    idx = block.routing_log[0]
+    assert idx.shape == (t, 10) and (idx.sort(-1).values.diff(dim=-1) > 0).all()  # ten distinct experts
+    counts = torch.bincount(idx.reshape(-1), minlength=512)
+    assert counts.sum() == t * 10 and counts.max() > 256  # some expert spans more than one tile
+
+    w = {k: v.detach().float() for k, v in block.named_parameters()}
+    rows = torch.randint(0, t, (24,), device="cuda", generator=g)
+    xs = x.detach()[0, rows].float()
+    probs = F.softmax((x.detach()[0, rows] @ block.gate.weight.t()).float(), dim=-1)
+    sc = probs.gather(1, idx[rows])
+    sc = (sc / sc.sum(-1, keepdim=True)).bfloat16().float()
+    want = torch.zeros(24, 2048, device="cuda")
+    for i in range(24):
+        for j in range(10):
+            e = int(idx[rows[i], j])
+            a, b = (w["experts.gate_up_proj"][e] @ xs[i]).chunk(2)
+            want[i] += sc[i, j] * (w["experts.down_proj"][e] @ (F.silu(a) * b))
+        a, b = w["shared_expert.gate_proj.weight"] @ xs[i], w["shared_expert.up_proj.weight"] @ xs[i]
+        gate = torch.sigmoid(w["shared_expert_gate.weight"] @ xs[i])
+        want[i] += gate * (w["shared_expert.down_proj.weight"] @ (F.silu(a) * b))
+    err = (out[0, rows].float() - want).abs().max().item()
+    assert err <= 2e-2 * want.abs().max().item(), err
+
+    # a permutation of the tokens permutes the output rows (bit for bit: every row's arithmetic is its own)
+    perm = torch.randperm(t, device="cuda", generator=g)
+    stager.begin()
+    with torch.no_grad():
+        out_p = block(x.detach()[:, perm])
+    assert torch.equal(out_p, out.detach()[:, perm])
+
+    # weight gradient of the busiest expert: d(down_proj[e]) = sum over its (token, slot) pairs of
+    # score * go_t (outer) act_t
+    e = int(counts.argmax())
+    tok, slot = (idx == e).nonzero(as_tuple=True)
+    xe = x.detach()[0, tok].float()
+    a, b = (xe @ w["experts.gate_up_proj"][e].t()).chunk(2, dim=-1)
+    act = (F.silu(a) * b).bfloat16().float()
+    pe = F.softmax((x.detach()[0, tok] @ block.gate.weight.t()).float(), dim=-1)
+    se = pe.gather(1, idx[tok])
+    se = (se / se.sum(-1, keepdim=True)).bfloat16().float()[torch.arange(tok.numel()), slot]
+    want_dw = (go[0, tok].float() * se[:, None]).t() @ act
+    got_dw = block.experts.down_proj.grad[e].float()
+    assert (got_dw - want_dw).abs().max() <= 3e-2 * want_dw.abs().max()
+    # an expert nobody chose has a zero gradient
+    unused = (counts == 0).nonzero().flatten()
+    assert unused.numel() >= 12
+    assert (block.experts.down_proj.grad[unused] == 0).all()
+    assert (block.experts.gate_up_proj.grad[unused] == 0).all()
