@@ -686,8 +686,19 @@ def run_mtp(args):
             shape = DraftShape(draft_vocab_size=CONFIG4["vocab_size"], qk_norm=True, **CONFIG4)
         tn = args.cpu_seq_len
         torch.set_num_threads(os.cpu_count() or 1)
-        wts = {k_: v_.requires_grad_(k_ not in ("embed_tokens.weight", "lm_head.weight"))
-               for k_, v_ in OM.random_weights(shape, 0).items()}
+        if hybrid:
+            # 512 expert stacks in fp32 with their gradients: one short row pair bounds the time (the
+            # experts' weight-gradient stacks cost the same whatever the length); eight random experts
+            # tiled 64 times (the values do not matter for the time, drawing 1.6 G normals does)
+            tn = min(tn, 128)
+            few = OM.random_weights(OM.HybridShape(draft_vocab_size=CONFIG4["vocab_size"], **CONFIG4,
+                                                   **dict(NEXT_EXTRA, num_experts=8)), 0)
+            reps = NEXT_EXTRA["num_experts"] // 8
+            raw = {k_: (v_.repeat(reps, *([1] * (v_.dim() - 1))) if ".mlp.gate.weight" in k_ or ".experts." in k_
+                        else v_) for k_, v_ in few.items()}
+        else:
+            raw = OM.random_weights(shape, 0)
+        wts = {k_: v_.requires_grad_(k_ not in ("embed_tokens.weight", "lm_head.weight")) for k_, v_ in raw.items()}
         cg = torch.Generator().manual_seed(0)
         cids = torch.randint(0, shape.vocab_size, (b, tn), generator=cg)
         chs = torch.randn(b, tn, shape.hidden_size, generator=cg)
@@ -698,13 +709,16 @@ def run_mtp(args):
             _, l_, _ = OM.mtp_forward(wts, shape, cids, chs, step_weights=sw, num_steps=k_steps, attn="sdpa")
             l_.backward()
 
-        cpu_step()
+        if not hybrid:
+            cpu_step()
         c0 = time.perf_counter()
         cpu_step()
         cdt = time.perf_counter() - c0
         cpu = {"value": round(b * tn / cdt, 2), "unit": "tokens/s", "cores": torch.get_num_threads(),
                "kind": "port", "sample": f"oracle MTP forward+backward, configs[4] shape at batch {b} x seq {tn}, "
-                                         "fp32, 1 warm-up + 1 timed iteration"}
+                                         + ("fp32, qwen3_next layer with 512 experts (8 random ones tiled), one timed "
+                                            "iteration, no warm-up" if hybrid else
+                                            "fp32, 1 warm-up + 1 timed iteration")}
     print(json.dumps({
         "metric": "MTP train tokens/sec (fwd+bwd) @Qwen3-Next-like MTP head, full-vocab CE",
         "value": round(tokens / (ms_per_step * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,

@@ -148,7 +148,10 @@ def sparse_moe(x, w, prefix, shape: HybridShape, routing: dict | None = None):
                 scores = scores / scores.sum(dim=-1, keepdim=True)
             scores = scores.to(logits.dtype)
     out = torch.zeros_like(x2)
-    gate_up, down = w[prefix + "experts.gate_up_proj"], w[prefix + "experts.down_proj"]
+    # (one unbind per stack: its backward stacks the experts' gradients once, where indexing the
+    # stack per expert would materialise a stack-sized gradient for every expert)
+    gate_up = w[prefix + "experts.gate_up_proj"].unbind(0)
+    down = w[prefix + "experts.down_proj"].unbind(0)
     for e in range(shape.num_experts):
         rows, slot = torch.where(idx == e)
         if rows.numel() == 0:

@@ -1,4 +1,5 @@
-"""Host logic of the MTP model configuration (no GPU)."""
+"""Host logic of the MTP path that needs no GPU: the configuration derived from the library's
+configs, the router arithmetic and the expert sort."""
 
 import pytest
 
@@ -30,3 +31,32 @@ def test_config_from_the_library_configs():
     assert (c.model_type, c.rotary_dim, c.num_experts) == ("qwen3", 64, 0)
     with pytest.raises(ValueError, match="Unsupported MTP model type"):
         MTPConfig.from_transformer_config(type("C", (), {"model_type": "llama"})())
+
+
+def test_route_equals_the_oracle_router_and_sort_pairs_is_a_stable_expert_sort():
+    import torch
+
+    from oracle import mtp as OM
+    from speculators_amd import moe
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(50, 32, generator=g)
+    wr = torch.randn(12, 32, generator=g)
+    for renorm in (True, False):
+        scores, idx = moe.route(x @ wr.t(), 4, renorm)
+        want_s, want_i = OM.moe_routing(x, wr, 4, renorm)
+        assert torch.equal(idx, want_i) and torch.equal(scores, want_s)
+    order, src_row, pos, off = moe.sort_pairs(idx, 12)
+    flat = idx.reshape(-1)
+    # sorted by expert, token order kept inside an expert (what makes the weight gradients reproducible)
+    assert torch.equal(flat[order], flat.sort(stable=True).values)
+    keys = flat[order] * 1000 + order
+    assert (keys.diff() > 0).all()
+    assert torch.equal(src_row.long(), order // 4)
+    assert off[0] == 0 and off[-1] == 200 and torch.equal(off[1:].long(), torch.bincount(flat, minlength=12).cumsum(0))
+    assert torch.equal(order[pos.reshape(-1).long()], torch.arange(200))
+    # an expert nobody chose is an empty group
+    idx2 = idx.clone()
+    idx2[idx2 == 3] = 5
+    _, _, _, off2 = moe.sort_pairs(idx2, 12)
+    assert off2[4] == off2[3]
