@@ -51,6 +51,30 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
     return out
 
 
+_CUS = 256  # workgroups the chip runs at a time (one per compute unit for the GEMM kernels)
+
+
+def _split_bands(t: int, m: int, n: int) -> int:
+    """How many row bands the contraction of a ``[t, m]^T [t, n]`` product is cut into: enough to
+    give every compute unit a workgroup, every band at least 1024 rows long; 1 = no split."""
+    tiles = -(-m // 256) * -(-n // 256)
+    if tiles * 2 > _CUS or t < 2048:
+        return 1
+    return max(1, min(_CUS // tiles, t // 1024))
+
+
+_band_cache: dict = {}
+
+
+def _band_offsets(t: int, step: int, bands: int, device) -> torch.Tensor:
+    key = (t, step, bands, str(device))
+    off = _band_cache.get(key)
+    if off is None:
+        off = torch.tensor([min(i * step, t) for i in range(bands + 1)], dtype=torch.int32, device=device)
+        _band_cache[key] = off
+    return off
+
+
 def gemm_tn(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
             accumulate: bool = False, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """``a[T, M].T @ b[T, N] -> [M, N]`` (bf16 operands, fp32 accumulation): the weight gradient
@@ -74,6 +98,22 @@ def gemm_tn(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
         out = torch.empty(m, n, device=a.device, dtype=out_dtype)
     elif out.shape != (m, n) or out.dtype not in (torch.bfloat16, torch.float32) or out.stride(1) != 1:
         raise ValueError(f"out must be a bf16 or fp32 [{m}, {n}] tensor with unit column stride")
+    # A small result with a long contraction leaves most of the chip idle (one workgroup per
+    # 256 x 256 tile of the result): the contraction is then cut into row bands, every band's
+    # product goes to an fp32 partial of its own (the grouped kernel with the bands as groups) and
+    # the partials are summed in a fixed order
+    bands = _split_bands(t, m, n)
+    if bands > 1 and max(a.stride(0), b.stride(0)) * 2 * (t + 256) < _MAX_SPAN:
+        step = -(-t // bands)
+        off = _band_offsets(t, step, bands, a.device)
+        part = torch.empty(bands, m, n, device=a.device, dtype=torch.float32)
+        _lib.call("spx_gemm_bf16_tn_grouped", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0), _lib.ptr(part),
+                  n, m * n, m, n, t, _lib.ptr(off), bands, 1, 0, _lib.stream_ptr(a.device))
+        total = part.sum(0)
+        if accumulate:
+            total += out  # in fp32: what the result holds is added before the one rounding
+        out.copy_(total)
+        return out
     entry = "spx_gemm_bf16_tn_f32" if out.dtype == torch.float32 else "spx_gemm_bf16_tn"
     # 32-bit byte offsets inside the kernel: a contraction that spans 2 GiB or more of an
     # operand is fed in bands of rows, every band after the first added to the result

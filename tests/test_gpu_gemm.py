@@ -209,3 +209,26 @@ def test_gemm_nt_with_a_row_count_on_the_device(m, live):
     gemm_nt(a_dirty, b, out, m_live=count)
     assert torch.equal(out[:n_live], want[:n_live])
     assert (out[n_live:] == 7).all()
+
+
+@pytest.mark.parametrize("t,m,n", [(8192, 264, 136), (5000, 512, 512), (20000, 8, 1024)])
+@pytest.mark.parametrize("fp32", [False, True])
+def test_gemm_tn_small_result_long_contraction(t, m, n, fp32):
+    """A result of a few tiles over a long contraction runs as row bands with fp32 partials summed
+    in a fixed order: same answer as the fp32 product, repeatable bit for bit, and accumulation
+    adds once."""
+    from speculators_amd.gemm import _split_bands, gemm_tn
+
+    assert _split_bands(t, m, n) > 1
+    g = torch.Generator(device="cuda").manual_seed(t + m)
+    a = torch.randn(t, m, device="cuda", generator=g).bfloat16()
+    b = torch.randn(t, n, device="cuda", generator=g).bfloat16()
+    want = a.double().t() @ b.double()
+    dt = torch.float32 if fp32 else torch.bfloat16
+    got = gemm_tn(a, b, out_dtype=dt)
+    tol = 2e-6 * t ** 0.5 if fp32 else 2 ** -8
+    assert got.dtype == dt and (got.double() - want).abs().max() <= tol * want.abs().max() + 1e-4
+    assert torch.equal(got, gemm_tn(a, b, out_dtype=dt))
+    acc = got.clone()
+    gemm_tn(a, b, acc, accumulate=True)
+    assert (acc.double() - 2 * want).abs().max() <= 2.5 * tol * want.abs().max() * 2 + 1e-4
