@@ -540,6 +540,17 @@ int spx_gemm_bf16_tn_grouped(const void* a, int64_t lda, const void* b, int64_t 
                              int64_t ldc, int64_t c_group_stride, int64_t M, int64_t N,
                              int64_t rows, const int32_t* group_offsets, int64_t groups,
                              int out_f32, int accumulate, void* stream);
+/* The same over `segments` segments of `segment_rows` rows each, one below the other in a and b
+ * (the expert-sorted rows of the K prediction steps of an MTP forward, models/mtp/core.py:190-226
+ * applies the layer once per step): group_offsets is int32 [segments][groups + 1], each row
+ * relative to its segment, and c_e (+)= sum over the segments of the group's product.  The sum
+ * over the steps happens in the accumulators; c is written once.  A segment whose row of offsets
+ * is all zero contributes nothing. */
+int spx_gemm_bf16_tn_grouped_multi(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                                   int64_t ldc, int64_t c_group_stride, int64_t M, int64_t N,
+                                   int64_t segment_rows, int64_t segments,
+                                   const int32_t* group_offsets, int64_t groups, int out_f32,
+                                   int accumulate, void* stream);
 
 /* out[b][c][r] = in[b][r][c] for `batches` bf16 matrices of R x C (multiples of 8), row strides
  * ld_in / ld_out and batch strides in elements: the transposed copies the input-gradient

@@ -85,6 +85,8 @@ SIGNATURES["spx_gemm_bf16_nt_grouped"] = [_P, _I64, _P, _I64, _I64, _P, _I64, _I
                                           _I64, _P]
 SIGNATURES["spx_gemm_bf16_tn_grouped"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I64, _P, _I64, _I, _I,
                                           _P]
+SIGNATURES["spx_gemm_bf16_tn_grouped_multi"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I64, _I64, _P, _I64,
+                                                _I, _I, _P]
 SIGNATURES["spx_transpose_bf16"] = [_P, _I64, _I64, _P, _I64, _I64, _I64, _I64, _I64, _P]
 SIGNATURES["spx_moe_gather_rows"] = [_P, _I64, _I64, _P, _P, _P, _I64, _I64, _I64, _P]
 SIGNATURES["spx_moe_combine_rows"] = [_P, _I64, _I64, _P, _P, _P, _I64, _I64, _I32, _I64, _P]

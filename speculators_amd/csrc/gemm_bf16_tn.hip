@@ -56,23 +56,51 @@ __device__ __forceinline__ i16x4 lds_read_tr16(const uint8_t* p) {
 }
 
 // OUT: 0 = bf16 result, 1 = bf16 result added to C, 2 = fp32 result, 3 = fp32 result added to C
-template <int OUT>
+// MULTI: the operands are n_seg segments of T rows each, one below the other; group e owns the rows
+// [group_off[s][e], group_off[s][e+1]) of every segment s and its contraction runs over all of them
+// (the expert-sorted rows of several uses of one expert stack: one product, one write of C)
+template <int OUT, bool MULTI = false>
 __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_bf16_tn_kernel(
     const uint16_t* __restrict__ A, int64_t lda, const uint16_t* __restrict__ B, int64_t ldb,
     void* __restrict__ Cv, int64_t ldc, int M, int N, int T, int tiles_m, int tiles_n,
-    const int32_t* __restrict__ group_off, int64_t c_group_stride) {
+    const int32_t* __restrict__ group_off, int64_t c_group_stride, int n_seg = 1, int n_groups = 0) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   // grouped product (blockIdx.y = group): the contraction runs over the group's rows
   // [group_off[e], group_off[e+1]) of both operands, and every group has a C of its own.  An empty
   // group multiplies nothing: zeros are written (or C is left as it is when the result is added)
-  if (group_off) {
+  const uint16_t* const A0 = A;
+  const uint16_t* const B0 = B;
+  const int seg_rows = T;
+  int seg = 0;
+  // rows [first, last) of segment s that belong to this workgroup's group
+  auto seg_range = [&](int s, int& first, int& last) __attribute__((always_inline)) {
     const int e = blockIdx.y;
-    const int t0 = min(max(group_off[e], 0), T), t1 = min(max(group_off[e + 1], t0), T);
-    A += (int64_t)t0 * lda;
-    B += (int64_t)t0 * ldb;
+    const int32_t* o = group_off + (MULTI ? (int64_t)s * (n_groups + 1) : 0);
+    first = min(max(o[e], 0), seg_rows);
+    last = min(max(o[e + 1], first), seg_rows);
+  };
+  int total_slabs = 0;
+  if (group_off) {
+    int t0, t1;
+    if (MULTI) {
+      for (int s2 = 0; s2 < n_seg; ++s2) {
+        seg_range(s2, t0, t1);
+        total_slabs += (t1 - t0 + kTK - 1) / kTK;
+      }
+      // the first segment that has rows (n_seg if none has)
+      for (seg = 0; seg < n_seg; ++seg) {
+        seg_range(seg, t0, t1);
+        if (t1 > t0) break;
+      }
+      if (seg == n_seg) t0 = t1 = 0;
+    } else {
+      seg_range(0, t0, t1);
+    }
+    A += ((int64_t)seg * seg_rows + t0) * lda;
+    B += ((int64_t)seg * seg_rows + t0) * ldb;
     T = t1 - t0;
-    Cv = reinterpret_cast<uint8_t*>(Cv) + e * c_group_stride * (OUT >= 2 ? 4 : 2);
-    if ((OUT & 1) && T == 0) return;
+    Cv = reinterpret_cast<uint8_t*>(Cv) + blockIdx.y * c_group_stride * (OUT >= 2 ? 4 : 2);
+    if ((OUT & 1) && (MULTI ? total_slabs == 0 : T == 0)) return;
   }
 
   // workgroup id -> tile: XCD-contiguous bands, then groups of GROUP_M tile rows
@@ -109,8 +137,8 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
   // the slab's first row included, is in the vector register, which is what the range check sees: rows
   // past T lie outside the resource and read as zero.  A 16-byte chunk past the last column would read
   // the next row instead, so those lanes get an offset outside the resource.
-  const u32x4 ares = make_rsrc(A + m0, T > 0 ? (uint32_t)((((int64_t)T - 1) * lda + min(M - m0, kTM)) * 2) : 0u);
-  const u32x4 bres = make_rsrc(B + n0, T > 0 ? (uint32_t)((((int64_t)T - 1) * ldb + min(N - n0, kTN)) * 2) : 0u);
+  u32x4 ares = make_rsrc(A + m0, T > 0 ? (uint32_t)((((int64_t)T - 1) * lda + min(M - m0, kTM)) * 2) : 0u);
+  u32x4 bres = make_rsrc(B + n0, T > 0 ? (uint32_t)((((int64_t)T - 1) * ldb + min(N - n0, kTN)) * 2) : 0u);
 
   // global side: wave-load j of this wave covers slab rows 2 (wave * kLA + j) + lane / 32; the lane's LDS
   // position is 16-byte chunk lane % 32 of the row, which holds the chunk of 64-byte block
@@ -139,7 +167,26 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
     // (a lane that is out of range stays so: kOob plus the row offset lies past any resource size)
     load_to_lds16<0>(isa ? ares : bres, (isa ? lds_a : lds_b) + bufoff + j * 1024, (int)voff, 0);
   };
-  auto next_slab = [&]() __attribute__((always_inline)) { bufoff ^= kABytes; ld_t0 += kTK; };
+  auto next_slab = [&]() __attribute__((always_inline)) {
+    bufoff ^= kABytes;
+    ld_t0 += kTK;
+    if (MULTI && ld_t0 >= T && seg < n_seg) {
+      // this segment's rows are all requested: go on with the next segment that has rows (the
+      // resources are rebuilt around it, so rows past its end read as zero like before); when
+      // there is none left the resources are empty and every further load brings zeros
+      int t0 = 0, t1 = 0;
+      for (++seg; seg < n_seg; ++seg) {
+        seg_range(seg, t0, t1);
+        if (t1 > t0) break;
+      }
+      if (seg >= n_seg) t0 = t1 = 0;
+      T = t1 - t0;
+      ld_t0 = 0;
+      const int64_t row0 = (int64_t)min(seg, n_seg - 1) * seg_rows + t0;
+      ares = make_rsrc(A0 + row0 * lda + m0, T > 0 ? (uint32_t)((((int64_t)T - 1) * lda + min(M - m0, kTM)) * 2) : 0u);
+      bres = make_rsrc(B0 + row0 * ldb + n0, T > 0 ? (uint32_t)((((int64_t)T - 1) * ldb + min(N - n0, kTN)) * 2) : 0u);
+    }
+  };
 
   // read side (see the head of the file)
   const int tG = lane >> 4, ts = lane & 15;
@@ -209,7 +256,7 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
     step(1, 0, 0, kLdT);
   };
 
-  const int nslab = (T + kTK - 1) / kTK;
+  const int nslab = MULTI ? total_slabs : (T + kTK - 1) / kTK;
 #pragma unroll
   for (int l = 0; l < kL; ++l) issue_one(l);
   next_slab();
@@ -331,20 +378,22 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
 using namespace spx;
 
 #define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fname, what); } while (0)
-template <int OUT>
+template <int OUT, bool MULTI = false>
 static int launch_tn(const char* fname, const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
                      int64_t ldc, int64_t M, int64_t N, int64_t T, void* stream,
-                     const int32_t* group_off = nullptr, int64_t c_group_stride = 0, int64_t groups = 1) {
+                     const int32_t* group_off = nullptr, int64_t c_group_stride = 0, int64_t groups = 1,
+                     int64_t segments = 1) {
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   static std::atomic<uint64_t> lds_set;  // per kernel instantiation, one bit per device
-  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&tn::gemm_bf16_tn_kernel<OUT>), tn::kSmem,
+  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&tn::gemm_bf16_tn_kernel<OUT, MULTI>), tn::kSmem,
                                   lds_set, fname))
     return rc;
   const int tiles_m = (int)((M + tn::kTM - 1) / tn::kTM), tiles_n = (int)((N + tn::kTN - 1) / tn::kTN);
   const dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)groups), block(tn::kThreads);
-  hipLaunchKernelGGL(tn::gemm_bf16_tn_kernel<OUT>, grid, block, tn::kSmem, st,
+  hipLaunchKernelGGL((tn::gemm_bf16_tn_kernel<OUT, MULTI>), grid, block, tn::kSmem, st,
                      reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb, c,
-                     ldc, (int)M, (int)N, (int)T, tiles_m, tiles_n, group_off, c_group_stride);
+                     ldc, (int)M, (int)N, (int)T, tiles_m, tiles_n, group_off, c_group_stride, (int)segments,
+                     (int)groups);
   return check_launch(fname);
 }
 
@@ -392,5 +441,27 @@ extern "C" int spx_gemm_bf16_tn_grouped(const void* a, int64_t lda, const void* 
                       : launch_tn<2>(fname, a, lda, b, ldb, c, ldc, M, N, rows, stream, group_offsets, c_group_stride, groups);
   return accumulate ? launch_tn<1>(fname, a, lda, b, ldb, c, ldc, M, N, rows, stream, group_offsets, c_group_stride, groups)
                     : launch_tn<0>(fname, a, lda, b, ldb, c, ldc, M, N, rows, stream, group_offsets, c_group_stride, groups);
+}
+
+extern "C" int spx_gemm_bf16_tn_grouped_multi(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                                              int64_t ldc, int64_t c_group_stride, int64_t M, int64_t N,
+                                              int64_t segment_rows, int64_t segments,
+                                              const int32_t* group_offsets, int64_t groups, int out_f32,
+                                              int accumulate, void* stream) {
+  const char* fname = __func__;
+  if (int rc = gemm_tn_check(fname, a, lda, b, ldb, c, ldc, M, N, segment_rows)) return rc;
+  SPX_REQ_FN(group_offsets && groups > 0 && groups < 65536, "null group offsets or a group count outside 1 .. 65535");
+  SPX_REQ_FN(segments > 0 && segments <= 64, "1 .. 64 segments");
+  SPX_REQ_FN(c_group_stride >= (M - 1) * ldc + N, "groups of c overlap");
+  SPX_REQ_FN(c_group_stride % (out_f32 ? 4 : 8) == 0, "the groups of c must be 16-byte aligned among each other");
+  if (out_f32)
+    return accumulate ? launch_tn<3, true>(fname, a, lda, b, ldb, c, ldc, M, N, segment_rows, stream, group_offsets,
+                                           c_group_stride, groups, segments)
+                      : launch_tn<2, true>(fname, a, lda, b, ldb, c, ldc, M, N, segment_rows, stream, group_offsets,
+                                           c_group_stride, groups, segments);
+  return accumulate ? launch_tn<1, true>(fname, a, lda, b, ldb, c, ldc, M, N, segment_rows, stream, group_offsets,
+                                         c_group_stride, groups, segments)
+                    : launch_tn<0, true>(fname, a, lda, b, ldb, c, ldc, M, N, segment_rows, stream, group_offsets,
+                                         c_group_stride, groups, segments);
 }
 #undef SPX_REQ_FN

@@ -67,10 +67,90 @@ def gemm_tn_grouped(a: torch.Tensor, b: torch.Tensor, offsets: torch.Tensor, out
     return out
 
 
-def gather_rows(x2: torch.Tensor, src_row: torch.Tensor, scale: torch.Tensor | None = None) -> torch.Tensor:
+def gemm_tn_grouped_multi(a: torch.Tensor, b: torch.Tensor, offsets: torch.Tensor, out: torch.Tensor,
+                          accumulate: bool = False) -> torch.Tensor:
+    """The grouped weight gradient over several uses at once: ``a [S * rows, M]`` and
+    ``b [S * rows, N]`` are S segments of ``rows`` sorted rows each, ``offsets [S, groups + 1]``
+    holds every segment's group boundaries (a row of zeros: that segment has nothing), and
+    ``out[e] (+)= sum_s a[rows of e in s].T @ b[rows of e in s]``."""
+    segments, g1 = offsets.shape
+    rows = a.shape[0] // segments
+    m, n = a.shape[1], b.shape[1]
+    if (a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or a.shape[0] != segments * rows
+            or b.shape[0] != a.shape[0] or not a.is_contiguous() or not b.is_contiguous()):
+        raise ValueError("a and b must be contiguous bf16 stacks of equally long segments")
+    if out.shape != (g1 - 1, m, n) or not out.is_contiguous() or out.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError(f"out must be a contiguous bf16 or fp32 [{g1 - 1}, {m}, {n}] tensor")
+    if offsets.dtype != torch.int32 or not offsets.is_contiguous() or offsets.device != a.device:
+        raise ValueError("offsets must be a contiguous int32 tensor on the operands' device")
+    _lib.call("spx_gemm_bf16_tn_grouped_multi", _lib.ptr(a), m, _lib.ptr(b), n, _lib.ptr(out), n, m * n, m, n,
+              rows, segments, _lib.ptr(offsets), g1 - 1, int(out.dtype == torch.float32), int(accumulate),
+              _lib.stream_ptr(a.device))
+    return out
+
+
+class _ExpertStacks:
+    """Inputs, output gradients and group boundaries of all uses of one expert weight stack in one
+    forward / backward, one use below the other, so that the stack's weight gradient is ONE
+    multi-segment grouped product when autograd reaches its staging node (the sum over the uses
+    happens in the MFMA accumulators and the gradient is written once)."""
+
+    def __init__(self, staged: Staged, rows: int, x_cols: int, dy_cols: int):
+        w = staged.w
+        # (no reference back to `staged`: it owns this object and its hook, and the buffers go
+        # with it as soon as the graph is dropped)
+        self.w_shape, self.rows, self.dy_cols = w.shape, rows, dy_cols
+        self.x = torch.empty(staged.uses * rows, x_cols, device=w.device, dtype=torch.bfloat16)
+        self.dy = None
+        self.off = torch.zeros(staged.uses, w.shape[0] + 1, device=w.device, dtype=torch.int32)
+        self.fill = 0
+        self.live = False
+        staged._finishers.append(self.add_gradient)
+
+    @staticmethod
+    def use(staged: Staged, rows: int, x_cols: int, dy_cols: int):
+        """``(stacks, use index)`` for the next product against ``staged``, or ``(None, -1)`` when
+        there is nothing to gain (frozen, one use, no graph) or no room."""
+        if staged.token is None or staged.uses <= 1 or not torch.is_grad_enabled():
+            return None, -1
+        st = staged.aux
+        if st is None:
+            st = staged.aux = _ExpertStacks(staged, rows, x_cols, dy_cols)
+        if st.rows != rows or st.fill >= staged.uses:
+            return None, -1
+        st.fill += 1
+        return st, st.fill - 1
+
+    def x_slot(self, u: int) -> torch.Tensor:
+        return self.x[u * self.rows:(u + 1) * self.rows]
+
+    def dy_slot(self, u: int) -> torch.Tensor:
+        if self.dy is None:
+            self.dy = torch.empty(self.x.shape[0], self.dy_cols, device=self.x.device, dtype=torch.bfloat16)
+        return self.dy[u * self.rows:(u + 1) * self.rows]
+
+    def record(self, u: int, offsets: torch.Tensor):
+        self.off[u].copy_(offsets)
+        self.live = True
+
+    def add_gradient(self, acc):
+        if not self.live:
+            return acc
+        fresh = acc is None
+        if fresh:
+            acc = torch.empty(self.w_shape, device=self.x.device, dtype=torch.float32)
+        gemm_tn_grouped_multi(self.dy, self.x, self.off, acc, accumulate=not fresh)
+        self.off.zero_()  # uses whose backward does not run next time contribute nothing
+        self.live = False
+        return acc
+
+
+def gather_rows(x2: torch.Tensor, src_row: torch.Tensor, scale: torch.Tensor | None = None,
+                out: torch.Tensor | None = None) -> torch.Tensor:
     """``out[p] = scale[p] * x2[src_row[p]]`` (bf16 rows, ``src_row`` int32, ``scale`` fp32)."""
     rows, h = src_row.numel(), x2.shape[1]
-    out = torch.empty(rows, h, device=x2.device, dtype=torch.bfloat16)
+    if out is None:
+        out = torch.empty(rows, h, device=x2.device, dtype=torch.bfloat16)
     _lib.call("spx_moe_gather_rows", _lib.ptr(x2), x2.stride(0), x2.shape[0], _lib.ptr(src_row),
               _lib.ptr(scale), _lib.ptr(out), h, rows, h, _lib.stream_ptr(x2.device))
     return out
@@ -142,9 +222,14 @@ class _ExpertsMLP(torch.autograd.Function):
         order, src_row, pos, off = sort_pairs(idx, e)
         rows = src_row.numel()
         st = _lib.stream_ptr(x2.device)
-        xs = gather_rows(x2, src_row)
+        # with several uses per forward the inputs of the two products go straight into the stacks
+        # that the one weight-gradient product over all uses reads
+        stack_gu, use_gu = _ExpertStacks.use(st_gu, rows, h, i2)
+        stack_dn, use_dn = _ExpertStacks.use(st_dn, rows, inter, h)
+        xs = gather_rows(x2, src_row, out=None if stack_gu is None else stack_gu.x_slot(use_gu))
         hid = gemm_nt_grouped(xs, w_gu, off)
-        act = torch.empty(rows, inter, device=x2.device, dtype=torch.bfloat16)
+        act = (torch.empty(rows, inter, device=x2.device, dtype=torch.bfloat16) if stack_dn is None
+               else stack_dn.x_slot(use_dn))
         up = hid[:, inter:]
         _lib.call("spx_swiglu_rows_fwd", _lib.ptr(hid), i2, _lib.ptr(up), i2, _lib.ptr(act), inter, rows,
                   inter, st)
@@ -153,6 +238,7 @@ class _ExpertsMLP(torch.autograd.Function):
         out = combine_rows(ys, pos, wts)
         ctx.save_for_backward(xs, hid, act, ys, pos, src_row, off, order, wts)
         ctx.staged = (st_gu, st_dn)
+        ctx.stacks = ((stack_gu, use_gu), (stack_dn, use_dn))
         ctx.score_dtype = scores.dtype
         return out
 
@@ -167,22 +253,29 @@ class _ExpertsMLP(torch.autograd.Function):
         dscores = None
         if ctx.needs_input_grad[1]:
             dscores = pair_dot(dout, ys, pos).to(ctx.score_dtype)
-        dys = gather_rows(dout, src_row, wts.reshape(-1)[order].contiguous())
+        (stack_gu, use_gu), (stack_dn, use_dn) = ctx.stacks
+        want_gu, want_dn = ctx.needs_input_grad[3], ctx.needs_input_grad[4]
+        dys = gather_rows(dout, src_row, wts.reshape(-1)[order].contiguous(),
+                          out=stack_dn.dy_slot(use_dn) if stack_dn is not None and want_dn else None)
         dact = gemm_nt_grouped(dys, st_dn.wt, off)
-        dh = torch.empty(rows, i2, device=dout.device, dtype=torch.bfloat16)
+        dh = (stack_gu.dy_slot(use_gu) if stack_gu is not None and want_gu
+              else torch.empty(rows, i2, device=dout.device, dtype=torch.bfloat16))
         _lib.call("spx_swiglu_rows_bwd", _lib.ptr(hid), i2, _lib.ptr(hid[:, inter:]), i2, _lib.ptr(dact), inter,
                   _lib.ptr(dh), i2, _lib.ptr(dh[:, inter:]), i2, rows, inter, st)
         dx = None
         if ctx.needs_input_grad[0]:
             dx = combine_rows(gemm_nt_grouped(dh, st_gu.wt, off), pos, None)
         marks = []
-        for need, staged, dy2, x2 in ((ctx.needs_input_grad[3], st_gu, dh, xs),
-                                     (ctx.needs_input_grad[4], st_dn, dys, act)):
+        for need, staged, dy2, x2, stack, use in ((want_gu, st_gu, dh, xs, stack_gu, use_gu),
+                                                 (want_dn, st_dn, dys, act, stack_dn, use_dn)):
             if not need:
                 marks.append(None)
                 continue
-            buf, holds = staged.grad_buffer()
-            gemm_tn_grouped(dy2, x2, off, buf, accumulate=holds)
+            if stack is not None:
+                stack.record(use, off)  # the product runs once, over all uses, in the staging node
+            else:
+                buf, holds = staged.grad_buffer()
+                gemm_tn_grouped(dy2, x2, off, buf, accumulate=holds)
             marks.append(staged.mark())
         return dx, dscores, None, marks[0], marks[1], None, None
 

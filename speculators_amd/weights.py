@@ -117,7 +117,7 @@ class Staged:
     is expected to run against it (the size of the input / output-gradient buffers)."""
 
     __slots__ = ("w", "token", "rows_of", "uses", "_wt", "_xs", "_fill", "_dys", "_live", "_extras",
-                 "_marked", "_acc")
+                 "_marked", "_acc", "aux", "_finishers")
 
     def __init__(self, w, rows_of, uses: int = 1):
         self.w = w
@@ -132,6 +132,8 @@ class Staged:
         self._extras = []  # (dy, x) of uses outside the buffers
         self._marked = False
         self._acc = None   # fp32 gradient buffer of uses that add their gradient themselves
+        self.aux = None    # whatever a family of products keeps per staged weight (the expert stacks)
+        self._finishers = []  # callables acc -> acc that add deferred gradients when the node runs
 
     @property
     def trainable(self) -> bool:
@@ -225,6 +227,8 @@ class Staged:
             acc = wgrad_product(self._dys[r0:r0 + n], self._xs[r0:r0 + n], acc)
         for dy2, x2 in self._extras:
             acc = wgrad_product(dy2, x2, acc)
+        for add_deferred in self._finishers:
+            acc = add_deferred(acc)
         self._dys, self._live, self._extras, self._marked, self._acc = None, [], [], False, None
         return acc
 

@@ -72,6 +72,41 @@ def test_grouped_tn_product(sizes, m, n, fp32):
         assert err <= 2 ** -7 * want[e].abs().max().item() + 1e-3, (e, err)
 
 
+@pytest.mark.parametrize("fp32", [False, True])
+def test_grouped_tn_product_over_several_segments(fp32):
+    """One product over the sorted rows of several uses: segments with different group sizes, a
+    group that is empty in some segments or in all, a segment that contributes nothing (offsets
+    all zero), group sizes around the 64-row slab."""
+    from speculators_amd.moe import gemm_tn_grouped_multi
+
+    seg_sizes = [[5, 0, 130, 64, 1, 0, 56], [0, 0, 7, 200, 49, 0, 0], [0] * 7, [63, 0, 65, 0, 128, 0, 0]]
+    rows, m, n = 256, 264, 136
+    g = torch.Generator().manual_seed(11)
+    a = torch.randn(len(seg_sizes) * rows, m, generator=g).bfloat16()
+    b = torch.randn(len(seg_sizes) * rows, n, generator=g).bfloat16()
+    off = torch.stack([_groups(sz) for sz in seg_sizes])
+    off[2] = 0
+    want = torch.zeros(7, m, n, dtype=torch.float64)
+    for s_, sz in enumerate(seg_sizes):
+        if s_ == 2:
+            continue
+        r0 = s_ * rows
+        for e, c in enumerate(sz):
+            want[e] += a[r0:r0 + c].double().t() @ b[r0:r0 + c].double()
+            r0 += c
+    dt = torch.float32 if fp32 else torch.bfloat16
+    out = torch.full((7, m, n), 3.0, dtype=dt, device="cuda")
+    gemm_tn_grouped_multi(a.cuda(), b.cuda(), off.cuda(), out)
+    tol = 1e-5 if fp32 else 2 ** -8
+    for e in range(7):
+        err = (out[e].double().cpu() - want[e]).abs().max().item()
+        assert err <= tol * want[e].abs().max().item() + 1e-3, (e, err)
+    assert (out[1] == 0).all() and (out[5] == 0).all()  # empty everywhere: zeros written
+    first = out.clone()
+    gemm_tn_grouped_multi(a.cuda(), b.cuda(), off.cuda(), out, accumulate=True)
+    assert (out.double() - 2 * first.double()).abs().max() <= 2 ** -7 * want.abs().max() + 1e-3
+
+
 def test_row_movement_kernels():
     """gather / combine / pair dot against index arithmetic; bad indices give zero rows."""
     from speculators_amd import moe
