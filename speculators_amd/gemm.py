@@ -11,6 +11,8 @@ The models call the ``*_staged`` forms below with the compute weights of ``weigh
 
 from __future__ import annotations
 
+import os
+
 import torch
 
 from . import _lib
@@ -156,6 +158,26 @@ def linear(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor | None 
     return _Linear.apply(x, weight, weight_t)
 
 
+# Which GEMM runs the decoder-layer projections (q/k/v, o, gate/up, down and their input
+# gradients): "hipblaslt" = PyTorch's matmul (the library GEMM; measured a few percent faster on
+# these shapes), "spx" = this library's MFMA kernel (the input gradients then run against the
+# transposed copy of the staged weight).  The fc / lm_head / verifier-head products and every
+# weight gradient always run on this library's kernels.
+DECODER_GEMM = os.environ.get("SPX_DECODER_GEMM", "hipblaslt")
+if DECODER_GEMM not in ("hipblaslt", "spx"):
+    raise ValueError(f"SPX_DECODER_GEMM must be 'hipblaslt' or 'spx', got {DECODER_GEMM!r}")
+
+
+def _project(x2: torch.Tensor, staged) -> torch.Tensor:
+    """``x2 @ staged.w.T`` of a decoder-layer projection."""
+    return gemm_nt(x2, staged.w) if DECODER_GEMM == "spx" else torch.nn.functional.linear(x2, staged.w)
+
+
+def _project_back(dy2: torch.Tensor, staged) -> torch.Tensor:
+    """``dy2 @ staged.w``: the input gradient of a decoder-layer projection."""
+    return gemm_nt(dy2, staged.wt) if DECODER_GEMM == "spx" else torch.matmul(dy2, staged.w)
+
+
 class _StagedLinear(torch.autograd.Function):
     """``x @ w.T`` against a staged weight (``weights.Staged``): on the MFMA kernel of this library
     (``hip``) or on PyTorch's hipBLASLt matmul.  The weight gradient is left to the staged weight,
@@ -167,7 +189,7 @@ class _StagedLinear(torch.autograd.Function):
             raise _lib.SpxError("the HIP layer kernels take bf16 tensors")
         w = staged.w
         x2 = x.reshape(-1, x.shape[-1])
-        y = gemm_nt(x2, w) if hip else torch.nn.functional.linear(x2, w)
+        y = gemm_nt(x2, w) if hip else _project(x2, staged)
         ctx.save_for_backward(x2, w)
         ctx.staged, ctx.hip, ctx.x_shape = staged, hip, x.shape
         ctx.slot = staged.take(x2) if ctx.needs_input_grad[1] else -1
@@ -179,7 +201,7 @@ class _StagedLinear(torch.autograd.Function):
         dy2 = dy.reshape(-1, dy.shape[-1]).to(torch.bfloat16)
         dx = dw = None
         if ctx.needs_input_grad[0]:
-            dx = (gemm_nt(dy2, ctx.staged.wt) if ctx.hip else torch.matmul(dy2, w)).view(ctx.x_shape)
+            dx = (gemm_nt(dy2, ctx.staged.wt) if ctx.hip else _project_back(dy2, ctx.staged)).view(ctx.x_shape)
         if ctx.needs_input_grad[1]:
             dw = ctx.staged.defer(ctx.slot, dy2, x2)
         return dx, dw, None, None
@@ -189,7 +211,7 @@ def linear_staged(x: torch.Tensor, staged, hip: bool = False) -> torch.Tensor:
     """``x[..., K] @ staged.w[N, K].T``; see ``_StagedLinear``."""
     if not torch.is_grad_enabled() or not (x.requires_grad or staged.trainable):
         x2 = x.reshape(-1, x.shape[-1])
-        y = gemm_nt(x2, staged.w) if hip else torch.nn.functional.linear(x2, staged.w)
+        y = gemm_nt(x2, staged.w) if hip else _project(x2, staged)
         return y.view(*x.shape[:-1], staged.w.shape[0])
     return _StagedLinear.apply(x, staged.token, staged, hip)
 
@@ -209,7 +231,7 @@ class _QKVRope(torch.autograd.Function):
         wcat = staged.w
         t = x.shape[-2]
         x2 = x.reshape(t, x.shape[-1])
-        qkv = torch.nn.functional.linear(x2, wcat)
+        qkv = _project(x2, staged)
         n = qkv.shape[1]
         st = _lib.stream_ptr(x.device)
         scale = FO.table_scale_of(inv_freq)
@@ -258,7 +280,7 @@ class _QKVRope(torch.autograd.Function):
             col += heads * d
         dx = dw = None
         if ctx.needs_input_grad[0]:
-            dx = torch.matmul(dqkv, wcat).view(shape)
+            dx = _project_back(dqkv, staged).view(shape)
         if ctx.needs_input_grad[1]:
             dw = staged.defer(ctx.slot, dqkv, x2)
         return (dx, dw) + (None,) * 8
@@ -287,7 +309,7 @@ class _GateUpSwiGLU(torch.autograd.Function):
         wcat = staged.w
         x2 = x.reshape(-1, x.shape[-1])
         f = wcat.shape[0] // 2
-        gu = torch.nn.functional.linear(x2, wcat)  # [T, 2F]
+        gu = _project(x2, staged)  # [T, 2F]
         rows = x2.shape[0]
         if out is None or out.shape != (rows, f) or not out.is_contiguous():
             out = torch.empty(rows, f, device=x.device, dtype=torch.bfloat16)
@@ -314,7 +336,7 @@ class _GateUpSwiGLU(torch.autograd.Function):
                   _lib.stream_ptr(x2.device))
         dx = dw = None
         if ctx.needs_input_grad[0]:
-            dx = torch.matmul(dgu, wcat).view(shape)
+            dx = _project_back(dgu, staged).view(shape)
         if ctx.needs_input_grad[1]:
             dw = staged.defer(ctx.slot, dgu, x2)
         return dx, dw, None, None

@@ -471,3 +471,31 @@ def test_head_node_falls_back_for_compound_losses():
     assert torch.equal(got[0][0], got[1][0])
     for k in got[0][1]:
         assert torch.equal(got[0][1][k], got[1][1][k]), k
+
+
+def test_decoder_projections_on_the_library_gemm(monkeypatch):
+    """``SPX_DECODER_GEMM=spx``: the decoder-layer projections and their input gradients on this
+    library's MFMA kernel instead of the library GEMM behind ``torch.matmul``.  Same loss and
+    gradients up to the rounding of a bf16 product evaluated in another order."""
+    from speculators_amd import gemm
+
+    shape = _shape(num_hidden_layers=2)
+    w = {k_: v.bfloat16() for k_, v in OE.random_weights(shape, seed=8, std=0.05).items()}
+    hs, ids, doc, mask, pos, vl = _batch(shape, 200, 3, [120, 70])
+    args = (hs.bfloat16().cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.bfloat16().cuda())
+    results = {}
+    for kind in ("hipblaslt", "spx"):
+        monkeypatch.setattr(gemm, "DECODER_GEMM", kind)
+        model = _make(shape, w, torch.bfloat16)
+        _, loss, metrics = model(*args, ttt_steps=3, ttt_step_loss_decay=0.8)
+        loss.backward()
+        results[kind] = (loss.item(), {n: p.grad.float() for n, p in model.named_parameters() if p.grad is not None},
+                         metrics)
+    (la, ga, ma), (lb, gb, mb) = results["hipblaslt"], results["spx"]
+    assert abs(la - lb) <= 2e-3 * abs(la)
+    assert ga.keys() == gb.keys()
+    for n in ga:
+        assert (ga[n] - gb[n]).abs().max() <= 3e-2 * ga[n].abs().max() + 1e-6, n
+    for k_ in ma:
+        if k_.endswith("_total"):
+            assert torch.equal(ma[k_], mb[k_]), k_
