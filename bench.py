@@ -37,7 +37,7 @@ TRAFFIC_ROWS = {
     "gemm_dx": ("gemm_bf16_nt_kernel", 65536),
     "loss_fwd": ("loss_fwd_kernel<unsigned short, 0, true, false, false", None),
     "loss_fwd_reuse": ("loss_fwd_kernel<unsigned short, 0, true, true, false", None),
-    "gemm_tn": ("gemm_bf16_tn_kernel<2>", None),
+    "gemm_tn": ("gemm_bf16_tn_kernel<2, false>", None),
     # (the summary averages the attention kernels over TTT steps 0 and 6 and the loss backward over its
     # full and packed launches: no per-launch figure for those)
 }
