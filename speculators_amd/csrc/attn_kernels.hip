@@ -1214,7 +1214,7 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
 #define SPX_DKV_XCD 1
 #endif
 #ifndef SPX_DKV256_ONEPASS
-#define SPX_DKV256_ONEPASS 1
+#define SPX_DKV256_ONEPASS 2
 #endif
 #ifndef SPX_DKV256_PF1
 #define SPX_DKV256_PF1 2
@@ -1222,17 +1222,31 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
 #ifndef SPX_DKV256_PF2
 #define SPX_DKV256_PF2 1
 #endif
+// Four 16-bit values per lane from LDS, transposed inside every group of 16 lanes: lane 4u + w of
+// a group receives, as element j, element w of the 8 bytes that lane 4j + u of the group points at.
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ i16x4 lds_read_tr16(const uint8_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) i16x4*)(uintptr_t)(uint32_t)(uintptr_t)(
+          (__attribute__((address_space(3))) const uint8_t*)p));
+}
+
 // PF: how the query tiles reach LDS (see FwdSmem): 0 at the point of use, 1 through registers one
 // tile ahead, 2 global -> LDS into the other of two buffers, 3 the same with tiles of 32 instead of 64
 // query rows.  A buffer holds the tiles the pass multiplies with: Q always, dO and Q^T for dK, dO^T for
 // dV.  At head_dim 256 two buffers of 64-row tiles fit the 160 KB of LDS only for the dV pass; with
 // 32-row tiles all four fit, the register staging is gone and dK and dV come out of ONE pass.
-template <int D, int PASS, int QT = 64>
+// 4: like 2, but only the row-major Q and dO tiles are loaded: the A operands of the accumulating
+// products (Q^T, dO^T fragments) come out of them through the transposing LDS read of gfx950
+// (ds_read_b64_tr_b16), so two buffers of 64-row tiles fit at head_dim 256 as well, a step is 64
+// rows long and half as many loads are issued per row.
+template <int D, int PASS, int QT = 64, bool TR = false>
 struct DkvSmem {
   static constexpr bool kDoV = PASS != 2, kDoK = PASS != 1;
-  static constexpr int kTileR = QT * D * 2, kTileT = D * QT * 2;  // Q / dO and Q^T / dO^T tiles, unpadded
+  static constexpr int kTileR = QT * D * 2, kTileT = TR ? 0 : D * QT * 2;  // Q / dO and Q^T / dO^T tiles, unpadded
   static constexpr int kOffdO = kTileR;
-  static constexpr int kOffQt = (kDoK ? 2 : 1) * kTileR;
+  static constexpr int kOffQt = ((kDoK || TR) ? 2 : 1) * kTileR;
   static constexpr int kOffdOt = kOffQt + (kDoK ? kTileT : 0);
   static constexpr int kBuf = kOffdOt + (kDoV ? kTileT : 0);
   static constexpr int kSmall = 6 * 64 * 4;                     // lse, delta, a1, b1, a2, b2 of 64 rows
@@ -1265,9 +1279,11 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
   uint16_t* Qts = dOs + 64 * QS;       // [D][TS]
   uint16_t* dOts = Qts + D * TS;       // [D][TS]
   constexpr bool kDma = PF >= 2;
+  constexpr bool kTR = PF == 4;                  // transposed operands by transposing LDS reads
   constexpr int QT = PF == 3 ? 32 : 64;          // query rows per LDS tile
   constexpr int NQB = QT / 32, NSUB = 64 / QT;   // 32-row halves per tile, tiles per 64-row step
-  using SM = DkvSmem<D, PASS, QT>;
+  using SM = DkvSmem<D, PASS, QT, kTR>;
+  static_assert(!kTR || PASS == 0, "the transposing-read mode computes both gradients");
   static_assert(!kDma || SM::kBytesDma <= 160 * 1024, "two buffers of this pass's tiles do not fit in LDS");
   uint8_t* const sm8 = reinterpret_cast<uint8_t*>(smem);
   float* lse_s = reinterpret_cast<float*>(kDma ? sm8 + 2 * SM::kBuf : sm8 + (2 * 64 * QS + 2 * D * TS) * 2);  // [64]
@@ -1433,7 +1449,12 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
   constexpr int RBQ = D * 2, CKQ = RBQ / 16;   // bytes / 16-byte chunks per row of Q and dO
   constexpr int RBT = QT * 2, CKT = RBT / 16;  // ... of Q^T and dO^T
   constexpr int LPR = (QT * RBQ / 1024) / NW, LPT = (D * RBT / 1024) / NW;  // wave loads per wave and tile
-  auto swz_r = [](int r) { return CKQ == 8 ? (r >> 1) & 7 : r & 15; };
+  // (with transposing reads the rows of a 4 + 4 row group must also fall into different 64-byte bank
+  // groups: the row's two low bits go to the chunk index's bits 2 - 3)
+  auto swz_r = [](int r) {
+    if (kTR) return CKQ == 8 ? ((r & 4) | ((r >> 2) & 2) | ((r >> 1) & 1)) : ((r & 3) << 2) | ((r >> 2) & 3);
+    return CKQ == 8 ? (r >> 1) & 7 : r & 15;
+  };
   auto swz_t = [](int r) { return CKT == 8 ? (r >> 1) & 7 : (r >> 2) & 3; };
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)sm8;
   u32x4 qres, dres, qtres, dtres;
@@ -1456,11 +1477,11 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         const int cofs = ((lane_v % CKQ) ^ swz_r(r)) * 16;
         const int ir = min(mq + r, p.NQ - 1);
         load_to_lds16<0>(qres, rb + j * 1024, ir * RBQ + cofs, 0);
-        if (kDoK) load_to_lds16<0>(dres, rb + SM::kOffdO + j * 1024, ir * (p.Hq * RBQ) + cofs, 0);
+        if (kDoK || kTR) load_to_lds16<0>(dres, rb + SM::kOffdO + j * 1024, ir * (p.Hq * RBQ) + cofs, 0);
       }
       const uint32_t tb2 = lds0 + b * SM::kBuf + wave * LPT * 1024;
 #pragma unroll
-      for (int j = 0; j < LPT; ++j) {
+      for (int j = 0; j < (kTR ? 0 : LPT); ++j) {
         const int r = (wave * LPT + j) * (1024 / RBT) + lane_v / CKT;
         const int tofs = r * NQp * 2 + ((lane_v % CKT) ^ swz_t(r)) * 16;
         if (kDoK) load_to_lds16<0>(qtres, tb2 + SM::kOffQt + j * 1024, tofs, mq * 2);
@@ -1470,6 +1491,14 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
   };
   const int rdr = col * RBQ + ((g ^ swz_r(col)) * 16);
   const int rdt = col * RBT + ((g ^ swz_t(col)) * 16);
+  // transposing reads: lane s of 16-lane group G points at row 4 (G >> 1) + (s >> 2) (+ 8 for the
+  // second read) of a 16-row k step, bytes 8 (s & 3) of the 64-byte block 32 db + 16 (G & 1): the k
+  // index order of the P / dS operands (rows 4 g .. 4 g + 3, then 8 + 4 g .. 8 + 4 g + 3)
+  const int tG = lane >> 4, ts = lane & 15;
+  const int trow = 4 * (tG >> 1) + (ts >> 2);
+  const int tcl = 2 * (tG & 1) + ((ts & 3) >> 1);
+  const int rt0 = trow * RBQ + ((tcl ^ swz_r(trow)) * 16) + (ts & 1) * 8;
+  const int rt1 = (trow + 8) * RBQ + ((tcl ^ swz_r(trow + 8)) * 16) + (ts & 1) * 8;
   const float* const lse_s0 = lse_s;
   const uint8_t* tile = sm8;
   int buf = 0;
@@ -1522,7 +1551,8 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
 
     // the two 32-row halves of the query tile one after the other (keeps 32 score
     // registers live instead of 64)
-#pragma unroll
+    // (head_dim 256 has no registers to spare for two unrolled halves in flight: a real loop there)
+#pragma unroll(kTR ? 1 : NQB)
     for (int qbl = 0; qbl < NQB; ++qbl) {
       const int qb = sub_now * NQB + qbl;  // 32-row half inside the 64-row step (per-row scalars); qbl: inside the LDS tile
       // the scores start from -lse of their query row and dO V^T from -delta (LDS holds both
@@ -1609,7 +1639,12 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
         auto fread = [&](int f) {
           const int e = f / PER, s2 = e / NDB, db = e % NDB;
           const bool is_q = kDoK && (!kDoV || (f % PER) == 1);
-          if constexpr (kDma) {
+          if constexpr (kTR) {
+            const uint8_t* base = tile + (is_q ? 0 : SM::kOffdO) + (qbl * 32 + s2 * 16) * RBQ;
+            const i16x4 lo = lds_read_tr16(base + (rt0 ^ (db * 64)));
+            const i16x4 hi = lds_read_tr16(base + (rt1 ^ (db * 64)));
+            fr[f % RG] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+          } else if constexpr (kDma) {
             const uint8_t* base = tile + (is_q ? SM::kOffQt : SM::kOffdOt);
             fr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 base + db * 32 * RBT + (rdt ^ ((qbl * 2 + s2) * 32))));
@@ -1728,15 +1763,6 @@ __device__ __forceinline__ int64_t uni(int64_t v) {
 }
 
 
-// Four 16-bit values per lane from LDS, transposed inside every group of 16 lanes: lane 4u + w of
-// a group receives, as element j, element w of the 8 bytes that lane 4j + u of the group points at.
-typedef short i16x4 __attribute__((ext_vector_type(4)));
-typedef short i16x8 __attribute__((ext_vector_type(8)));
-__device__ __forceinline__ i16x4 lds_read_tr16(const uint8_t* p) {
-  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-      (__attribute__((address_space(3))) i16x4*)(uintptr_t)(uint32_t)(uintptr_t)(
-          (__attribute__((address_space(3))) const uint8_t*)p));
-}
 
 // One role of the kernel as a function of its own (not inlined): the register allocation of the
 // producers (K / V fragments, scores) and of the consumers (128 accumulator registers) then do not
@@ -2361,7 +2387,8 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   // (the wave-specialised dK/dV kernel transposes inside LDS and needs no Q^T / dO^T; it lists the query
   // tiles that see a key block in LDS, which bounds their number)
   const bool use_ws = D <= 128 && SPX_DKV_WS && (p.NQ + 63) / 64 <= DkvWsSmem<(D <= 128 ? D : 128)>::kListCap;
-  const bool kNeedT = !use_ws;
+  // (nor does the one-pass head_dim-256 kernel with transposing LDS reads)
+  const bool kNeedT = !use_ws && !(D > 128 && SPX_DKV256_ONEPASS == 2);
   hipLaunchKernelGGL(transpose_bf16_kernel<true>, qgrid, dim3(64), 0, st, p.Q, p.q_hs, (int64_t)D, p.NQ, D,
                      kNeedT ? qt : nullptr, (int64_t)D * NQp, (int64_t)NQp, p.scale_log2e, qs);
   if (kNeedT)
@@ -2418,6 +2445,15 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
     hipLaunchKernelGGL((attn_bwd_dkv_ws_kernel<D>), dim3((unsigned)(n_pair_ws * p.Hq)), dim3(512), smem, st, ps,
                        dOp, NQp, neg, mrows, tb, dkp, dvp);
    }
+  } else if constexpr (D > 128 && SPX_DKV256_ONEPASS == 2) {
+    // dK and dV in one pass over 64-row tiles of Q and dO alone (two buffers of two 32 KB tiles); the
+    // transposed operands come out of them through transposing LDS reads
+    constexpr size_t smem = DkvSmem<D, 0, 64, true>::kBytesDma;
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, 4, 0>),
+                                    (int)smem, dkv_lds_set[0], fn))
+      return rc;
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, 4, 0>), kgrid, kblock, smem, st, ps, dOp, qt, dot,
+                       NQp, lse, delta, tb, dkp, dvp);
   } else if constexpr (D > 128 && SPX_DKV256_ONEPASS) {
     // dK and dV in one pass over 32-row tiles (two buffers of four 16 KB tiles)
     constexpr size_t smem = DkvSmem<D, 0, 32>::kBytesDma;
