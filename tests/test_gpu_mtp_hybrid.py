@@ -436,3 +436,34 @@ def test_moe_block_at_the_qwen3_next_sizes():
     assert unused.numel() >= 12
     assert (block.experts.down_proj.grad[unused] == 0).all()
     assert (block.experts.gate_up_proj.grad[unused] == 0).all()
+
+
+def test_hybrid_model_with_a_padding_mask_matches_oracle():
+    """``attention_mask`` (models/mtp/core.py:119,180-186) through the gated-attention layer:
+    right- and left-padded rows, dense MLP flavour (no routing in the way)."""
+    shape = _hybrid_shape(model_type="qwen3_5_text")
+    steps = 2
+    w = {k: v.bfloat16() for k, v in OM.random_weights(shape, seed=4, std=0.05).items()}
+    g = torch.Generator().manual_seed(9)
+    b, n = 2, 150
+    ids = torch.randint(0, shape.vocab_size, (b, n), generator=g)
+    hs = torch.randn(b, n, shape.hidden_size, generator=g).bfloat16()
+    am = torch.ones(b, n, dtype=torch.long)
+    am[0, 110:] = 0
+    am[1, :30] = 0
+    lm = ((torch.rand(b, n, generator=g) < 0.7) & (am != 0)).float()
+    model = _make(shape, w, steps)
+    logits, loss, _ = model(ids.cuda(), hs.cuda(), attention_mask=am.cuda(), loss_mask=lm.cuda())
+    loss.backward()
+    wf = {k: v.float().requires_grad_(True) for k, v in w.items()}
+    rl, rloss, _ = OM.mtp_forward(wf, shape, ids, hs.float(), loss_mask=lm, num_steps=steps, attention_mask=am)
+    rloss.backward()
+    assert abs(loss.item() - rloss.item()) <= 1e-3 * abs(rloss.item())
+    tok = am[:, :n - steps - 1] != 0
+    for k in range(steps):
+        got, want = logits[k].float().cpu()[tok], rl[k][tok]
+        assert (got - want).abs().max() <= 2e-2 * want.abs().max(), k
+    for name, prm in model.named_parameters():
+        if prm.requires_grad:
+            want = wf[name].grad
+            assert (prm.grad.float().cpu() - want).abs().max() <= 3e-2 * want.abs().max() + 1e-6, name
