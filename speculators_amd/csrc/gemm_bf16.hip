@@ -350,7 +350,8 @@ namespace spx {
 // tab[0] = number of tile rows, then (group, first row) of every tile row: group e contributes
 // ceil(rows_e / kTM) of them.  One workgroup; thread t owns a contiguous run of groups.
 __global__ __launch_bounds__(256) void gemm_group_tiles_kernel(const int32_t* __restrict__ group_off, int groups,
-                                                               int rows, int32_t* __restrict__ tab) {
+                                                               int rows, int max_tiles,
+                                                               int32_t* __restrict__ tab) {
   __shared__ int sums[256];
   const int t = threadIdx.x;
   const int per = (groups + 255) / 256;
@@ -368,13 +369,14 @@ __global__ __launch_bounds__(256) void gemm_group_tiles_kernel(const int32_t* __
       sums[i] = run;
       run += v;
     }
-    tab[0] = run;
+    tab[0] = min(run, max_tiles);  // (offsets that do not ascend could ask for more than the table holds)
   }
   __syncthreads();
   int at = sums[t];
   for (int e = e0; e < e1; ++e) {
     const int r0 = clamped(e), r1 = clamped(e + 1);
     for (int r = r0; r < r1; r += kTM, ++at) {
+      if (at >= max_tiles) break;
       tab[1 + 2 * at] = e;
       tab[2 + 2 * at] = r;
     }
@@ -400,7 +402,7 @@ extern "C" int spx_gemm_bf16_nt_grouped(const void* a, int64_t lda, const void* 
              "unaligned workspace or group stride");
   int32_t* tab = reinterpret_cast<int32_t*>(workspace);
   hipLaunchKernelGGL(gemm_group_tiles_kernel, dim3(1), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
-                     group_offsets, (int)groups, (int)rows, tab);
+                     group_offsets, (int)groups, (int)rows, (int)((rows + kTM - 1) / kTM + groups), tab);
   if (int rc = check_launch(fname)) return rc;
   return gemm_nt_impl(fname, a, lda, b, ldb, c, ldc, rows, N, K, nullptr, stream, tab, group_offsets,
                       b_group_stride, groups);
