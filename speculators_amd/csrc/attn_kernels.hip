@@ -826,14 +826,26 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const uint16_t* __restr
 // PF: how a key tile reaches LDS: 0 through registers at the point of use, 1 through registers one tile
 // ahead, 3 global -> LDS directly into the other of two buffers, with tiles of 32 instead of 64 keys so
 // that two buffers of the three tiles (K, V, K^T) fit beside a second workgroup (see FwdSmem).
+// Four 16-bit values per lane from LDS, transposed inside every group of 16 lanes: lane 4u + w of
+// a group receives, as element j, element w of the 8 bytes that lane 4j + u of the group points at.
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ i16x4 lds_read_tr16(const uint8_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) i16x4*)(uintptr_t)(uint32_t)(uintptr_t)(
+          (__attribute__((address_space(3))) const uint8_t*)p));
+}
+
 template <int D, int NW, int PF>
 struct DqSmem {
-  static constexpr int TB = PF == 3 ? 32 : kBN;                      // keys per tile
+  // mode 4: only the row-major K and V tiles, 64 keys each; the K^T fragments of the dQ product come
+  // out of the K tile through transposing LDS reads
+  static constexpr int TB = PF == 3 ? 32 : (PF == 4 ? 64 : kBN);     // keys per tile
   static constexpr int KS = D + kKPad, VS = kBN + kVPad;
-  static constexpr int kTileK = TB * D * 2, kTileT = D * TB * 2;     // mode 3: unpadded, swizzled
+  static constexpr int kTileK = TB * D * 2, kTileT = PF == 4 ? 0 : D * TB * 2;  // modes 3, 4: unpadded, swizzled
   static constexpr int kBuf = 2 * kTileK + kTileT;
   static constexpr int kDiag = NW * 2 * 32 * D * 2;  // K and V rows of 32 queries per wave (TTT diagonal keys)
-  static constexpr int kTiles0 = PF == 3 ? 2 * kBuf : (2 * kBN * KS + D * VS) * 2;
+  static constexpr int kTiles0 = PF >= 3 ? 2 * kBuf : (2 * kBN * KS + D * VS) * 2;
   static constexpr int kTiles = kTiles0 > kDiag ? kTiles0 : kDiag;
   static constexpr int kBytes = kTiles + 4 * NW * (int)sizeof(int);
 };
@@ -844,7 +856,8 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
     const float* __restrict__ LSE, const float* __restrict__ Delta, uint16_t* __restrict__ dQ,
     int64_t dq_hs) {
   using SM = DqSmem<D, NW, PF>;
-  constexpr bool kDma = PF == 3;
+  constexpr bool kDma = PF >= 3;
+  constexpr bool kTR = PF == 4;
   constexpr int TB = SM::TB;
   constexpr int KS = SM::KS;
   constexpr int VS = SM::VS;
@@ -963,7 +976,11 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
   constexpr int RBK = D * 2, CKK = RBK / 16;   // bytes / 16-byte chunks per row of K and V
   constexpr int RBT = TB * 2, CKT = RBT / 16;  // ... of K^T
   constexpr int LPK = (TB * RBK / 1024) / NW, LPT = (D * RBT / 1024) / NW;
-  auto swz_k = [](int r) { return CKK == 8 ? (r >> 1) & 7 : r & 15; };
+  auto swz_k = [](int r) {
+    // (transposing reads touch 4 + 4 rows x 64 bytes: those rows must fall into different 64-byte bank groups)
+    if (kTR) return CKK == 8 ? ((r & 4) | ((r >> 2) & 2) | ((r >> 1) & 1)) : ((r & 3) << 2) | ((r >> 2) & 3);
+    return CKK == 8 ? (r >> 1) & 7 : r & 15;
+  };
   auto swz_t = [](int r) { return CKT == 8 ? (r >> 1) & 7 : (r >> 2) & 3; };
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)dq_smem;
   u32x4 kres, vres, tres;
@@ -987,7 +1004,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
       }
       const uint32_t tb0 = lds0 + b * SM::kBuf + 2 * SM::kTileK + wave * LPT * 1024;
 #pragma unroll
-      for (int j = 0; j < LPT; ++j) {
+      for (int j = 0; j < (kTR ? 0 : LPT); ++j) {
         const int r = (wave * LPT + j) * (1024 / RBT) + lane_v / CKT;
         load_to_lds16<0>(tres, tb0 + j * 1024, r * p.NKVp * 2 + ((lane_v % CKT) ^ swz_t(r)) * 16, n0 * 2);
       }
@@ -995,6 +1012,12 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
   };
   const int rdk = col * RBK + ((g ^ swz_k(col)) * 16);
   const int rdt = col * RBT + ((g ^ swz_t(col)) * 16);
+  // transposing reads (see the dK/dV kernel): rows 4 (G >> 1) + (s >> 2) (+ 8) of a 16-key step
+  const int tG = lane >> 4, ts = lane & 15;
+  const int trow = 4 * (tG >> 1) + (ts >> 2);
+  const int tcl = 2 * (tG & 1) + ((ts & 3) >> 1);
+  const int rt0 = trow * RBK + ((tcl ^ swz_k(trow)) * 16) + (ts & 1) * 8;
+  const int rt1 = (trow + 8) * RBK + ((tcl ^ swz_k(trow + 8)) * 16) + (ts & 1) * 8;
 
   auto run_pass = [&](const int (&aa)[NSB], const int (&bb)[NSB], int w_amin, int w_amax,
                       int w_bmin, int w_bmax, int blk_a, int blk_b) {
@@ -1025,7 +1048,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb) {
         // the 32-key halves of the tile one after the other: 32 score registers live
-#pragma unroll
+#pragma unroll(kTR && D > 128 ? 1 : TB / 32)
         for (int kb = 0; kb < TB / 32; ++kb) {
           f32x16 st, dp;
           // K and V fragments alternate through a ring of four registers (fragment 2 kk is
@@ -1078,7 +1101,12 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_DQ_MINB) void attn_bwd_d
             constexpr int NF = 2 * NDB;
             bf16x8 fr[4];
             auto fread = [&](int f) {
-              if constexpr (kDma)
+              if constexpr (kTR) {
+                const uint8_t* base = tile + (kb * 32 + (f / NDB) * 16) * RBK;
+                const i16x4 lo = lds_read_tr16(base + (rt0 ^ ((f % NDB) * 64)));
+                const i16x4 hi = lds_read_tr16(base + (rt1 ^ ((f % NDB) * 64)));
+                fr[f & 3] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+              } else if constexpr (kDma)
                 fr[f & 3] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                     tile + 2 * SM::kTileK + (f % NDB) * 32 * RBT + (rdt ^ ((kb * 2 + f / NDB) * 32))));
               else
@@ -1222,16 +1250,6 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
 #ifndef SPX_DKV256_PF2
 #define SPX_DKV256_PF2 1
 #endif
-// Four 16-bit values per lane from LDS, transposed inside every group of 16 lanes: lane 4u + w of
-// a group receives, as element j, element w of the 8 bytes that lane 4j + u of the group points at.
-typedef short i16x4 __attribute__((ext_vector_type(4)));
-typedef short i16x8 __attribute__((ext_vector_type(8)));
-__device__ __forceinline__ i16x4 lds_read_tr16(const uint8_t* p) {
-  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-      (__attribute__((address_space(3))) i16x4*)(uintptr_t)(uint32_t)(uintptr_t)(
-          (__attribute__((address_space(3))) const uint8_t*)p));
-}
-
 // PF: how the query tiles reach LDS (see FwdSmem): 0 at the point of use, 1 through registers one
 // tile ahead, 2 global -> LDS into the other of two buffers, 3 the same with tiles of 32 instead of 64
 // query rows.  A buffer holds the tiles the pass multiplies with: Q always, dO and Q^T for dK, dO^T for
@@ -2292,7 +2310,7 @@ static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 #define SPX_FWD_CFG 1, 4, 2
 #endif
 #ifndef SPX_DQ_CFG
-#define SPX_DQ_CFG 1, 4, 3
+#define SPX_DQ_CFG 1, 4, 4
 #endif
 // head_dim 256: the next tile is prefetched into registers as well; the few registers that
 // spill cost far less than exposing the global-load latency with one workgroup per CU
@@ -2300,7 +2318,7 @@ static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 #define SPX_FWD256_PF 2
 #endif
 #ifndef SPX_DQ256_PF
-#define SPX_DQ256_PF 3
+#define SPX_DQ256_PF 4
 #endif
 #ifndef SPX_DKV_CFG
 #define SPX_DKV_CFG 4, 2
@@ -2380,9 +2398,12 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   w += round_up(2 * (int64_t)p.Hq * NQp * 4, 256);
   int32_t* mrows = reinterpret_cast<int32_t*>(w); // [4][NQp]
 
+  // (the dQ kernel's transposing-read mode takes its K^T fragments from the row-major K tile)
+  constexpr bool kNeedKt = (D > 128 ? (int)SPX_DQ256_PF : kDqPF) != 4;
   dim3 tgrid((unsigned)(p.NKVp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hkv);
-  hipLaunchKernelGGL(transpose_bf16_kernel<false>, tgrid, dim3(64), 0, st, p.K, p.k_hs, (int64_t)D, p.NKV, D,
-                     kt, (int64_t)D * p.NKVp, (int64_t)p.NKVp, 1.f, nullptr);
+  if (kNeedKt)
+    hipLaunchKernelGGL(transpose_bf16_kernel<false>, tgrid, dim3(64), 0, st, p.K, p.k_hs, (int64_t)D, p.NKV, D,
+                       kt, (int64_t)D * p.NKVp, (int64_t)p.NKVp, 1.f, nullptr);
   dim3 qgrid((unsigned)(NQp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hq);
   // (the wave-specialised dK/dV kernel transposes inside LDS and needs no Q^T / dO^T; it lists the query
   // tiles that see a key block in LDS, which bounds their number)
@@ -2412,7 +2433,7 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   {
     constexpr int kDqPFd = D > 128 ? (int)SPX_DQ256_PF : kDqPF;
     constexpr int dq_smem = DqSmem<D, kDqNW, kDqPFd>::kBytes;
-    if (kDqPFd == 3 && ((int64_t)p.NKV * D * 2 >= (1ll << 31) || (int64_t)D * p.NKVp * 2 >= (1ll << 31))) {
+    if (kDqPFd >= 3 && ((int64_t)p.NKV * D * 2 >= (1ll << 31) || (int64_t)D * p.NKVp * 2 >= (1ll << 31))) {
       last_error() = std::string(fn) + ": keys of one head must span less than 2 GiB";
       return SPX_ERR_ARG;
     }
