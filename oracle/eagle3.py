@@ -61,25 +61,50 @@ def rms_norm(x, weight, eps):
     return weight * xf.to(x.dtype)
 
 
-def rope_inv_freq(head_dim, theta, scaling=None):
+def rope_kind(scaling=None) -> str:
+    return (scaling or {}).get("rope_type", (scaling or {}).get("type", "default"))
+
+
+def rope_inv_freq(head_dim, theta, scaling=None, seq_len=None):
     """fp32 inverse frequencies of the rotary embedding.  ``scaling`` follows the HF rope
     parameters the draft inherits from its verifier (models/eagle3/core.py:105-112 keeps them
     in the layer config; Llama-3.1 ships ``rope_type = "llama3"``):
-      linear: every frequency divided by ``factor``;
-      yarn:   see ``_yarn_inv_freq``; its table factor is ``rope_table_scale``;
-      llama3: wavelengths above ``L / low_freq_factor`` (L = original_max_position_embeddings)
-              are divided by ``factor``, those below ``L / high_freq_factor`` kept, and the band
-              between is blended linearly in ``L / wavelength``.
-    Pinned against ``transformers.modeling_rope_utils.ROPE_INIT_FUNCTIONS``."""
+      linear:   every frequency divided by ``factor``;
+      yarn:     see ``_yarn_inv_freq``; its table factor is ``rope_table_scale``;
+      llama3:   wavelengths above ``L / low_freq_factor`` (L = original_max_position_embeddings)
+                are divided by ``factor``, those below ``L / high_freq_factor`` kept, and the band
+                between is blended linearly in ``L / wavelength``;
+      dynamic:  the base grows with the running length ``seq_len`` once that passes
+                ``max_position_embeddings`` (a key of ``scaling`` here; the library keeps it on the
+                model config): ``theta * (factor * n / L - (factor - 1)) ** (d / (d - 2))``;
+      longrope: per-frequency divisors, ``long_factor`` when ``seq_len`` is beyond
+                ``original_max_position_embeddings``, ``short_factor`` otherwise; table factor
+                ``sqrt(1 + ln(factor) / ln(L_original))``.
+    ``seq_len`` only matters to the last two; which length a rotary module runs with from call to call
+    is ``RotaryState``.  Pinned against ``transformers.modeling_rope_utils.ROPE_INIT_FUNCTIONS``."""
     inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
-    kind = (scaling or {}).get("rope_type", (scaling or {}).get("type", "default"))
+    kind = rope_kind(scaling)
     if kind == "default":
         return inv
+    if kind == "longrope":
+        long = seq_len is not None and int(seq_len) > int(scaling["original_max_position_embeddings"])
+        ext = torch.tensor(scaling["long_factor" if long else "short_factor"], dtype=torch.float32)
+        shape = torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim
+        return 1.0 / (ext * theta ** shape)
     factor = float(scaling["factor"])
     if kind == "linear":
         return inv / factor
     if kind == "yarn":
         return _yarn_inv_freq(inv, head_dim, theta, scaling)
+    if kind == "dynamic":
+        ctx = int(scaling["max_position_embeddings"])
+        if seq_len is None:
+            base = theta * ((factor * ctx / ctx) - (factor - 1)) ** (head_dim / (head_dim - 2))
+        else:
+            # (the library's update hands the length over as an int64 tensor: the base is an fp32 value)
+            n = torch.maximum(torch.as_tensor(int(seq_len), dtype=torch.int64), torch.tensor(ctx, dtype=torch.int64))
+            base = theta * ((factor * n / ctx) - (factor - 1)) ** (head_dim / (head_dim - 2))
+        return 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
     if kind != "llama3":
         raise NotImplementedError(f"rope_type '{kind}'")
     lo, hi = float(scaling["low_freq_factor"]), float(scaling["high_freq_factor"])
@@ -119,8 +144,18 @@ def _yarn_inv_freq(inv, dim, theta, scaling):
 def rope_table_scale(scaling=None) -> float:
     """The factor on both tables (``attention_scaling`` of the HF rotary modules): 1 except for
     yarn, where it is ``attention_factor`` if given, else ``0.1 ln(factor) + 1`` (with ``mscale`` /
-    ``mscale_all_dim``: the ratio of the two such terms)."""
-    kind = (scaling or {}).get("rope_type", (scaling or {}).get("type", "default"))
+    ``mscale_all_dim``: the ratio of the two such terms), and longrope, where it is
+    ``attention_factor`` if given, else ``sqrt(1 + ln(factor) / ln(L_original))`` for a factor above 1
+    (``factor`` defaults to ``max_position_embeddings / L_original``)."""
+    kind = rope_kind(scaling)
+    if kind == "longrope":
+        if scaling.get("attention_factor") is not None:
+            return float(scaling["attention_factor"])
+        ctx0 = scaling["original_max_position_embeddings"]
+        factor = scaling.get("factor")
+        if factor is None:
+            factor = scaling["max_position_embeddings"] / ctx0
+        return 1.0 if factor <= 1.0 else math.sqrt(1 + math.log(factor) / math.log(ctx0))
     if kind != "yarn":
         return 1.0
     if scaling.get("attention_factor") is not None:
@@ -135,9 +170,52 @@ def rope_table_scale(scaling=None) -> float:
     return term()
 
 
-def rope_tables(position_ids, head_dim, theta, dtype, scaling=None):
-    """cos/sin ``[1, T, D]``: fp32 outer product, duplicated halves, table scale, cast."""
-    inv = rope_inv_freq(head_dim, theta, scaling)
+class RotaryState:
+    """The frequencies one rotary module runs with from call to call (``dynamic_rope_update`` of
+    transformers' ``modeling_rope_utils.py``, which wraps the forward of every HF rotary module).
+    With ``n = max(position_ids) + 1`` of the call:
+      longrope: the long divisors if ``n > original_max_position_embeddings``, else the short ones;
+      dynamic:  recomputed for ``n`` whenever ``n`` exceeds every length seen so far (starting from
+                ``max_position_embeddings``), kept otherwise -- until a call with
+                ``n < max_position_embeddings`` puts the original frequencies back;
+      every other type: fixed."""
+
+    def __init__(self, head_dim, theta, scaling=None):
+        self.head_dim, self.theta, self.scaling = head_dim, theta, scaling
+        self.kind = rope_kind(scaling)
+        self.original = rope_inv_freq(head_dim, theta, scaling)
+        self.current = self.original
+        if self.kind == "dynamic":
+            self.ctx = int(scaling["max_position_embeddings"])
+            self.seen = self.ctx
+
+    def inv_freq(self, position_ids):
+        if self.kind == "longrope":
+            n = int(position_ids.max()) + 1
+            if n > int(self.scaling["original_max_position_embeddings"]):
+                return rope_inv_freq(self.head_dim, self.theta, self.scaling,
+                                     int(self.scaling["original_max_position_embeddings"]) + 1)
+            return self.original
+        if self.kind == "dynamic":
+            n = int(position_ids.max()) + 1
+            if n > self.seen:
+                self.current = rope_inv_freq(self.head_dim, self.theta, self.scaling, n)
+                self.seen = n
+            if n < self.ctx and self.seen > self.ctx:
+                self.current, self.seen = self.original, self.ctx
+            return self.current
+        return self.original
+
+
+def rope_tables(position_ids, head_dim, theta, dtype, scaling=None, state=None, inv_freq=None):
+    """cos/sin ``[1, T, D]``: fp32 outer product, duplicated halves, table scale, cast.  ``state``: the
+    ``RotaryState`` of the module when several calls follow each other (a fresh one otherwise);
+    ``inv_freq``: the frequencies themselves, where the caller has asked the state already."""
+    if inv_freq is None:
+        if state is None:
+            state = RotaryState(head_dim, theta, scaling)
+        inv_freq = state.inv_freq(position_ids)
+    inv = inv_freq
     ang = position_ids.reshape(1, -1, 1).float() * inv.reshape(1, 1, -1)
     ang = torch.cat([ang, ang], dim=-1)
     scale = rope_table_scale(scaling)
@@ -215,7 +293,7 @@ def eagle3_forward(w, shape: DraftShape, hidden_states, input_ids, document_ids,
                    loss_mask=None, position_ids=None, verifier_last_hidden_states=None,
                    ttt_steps: int = 3, ttt_step_loss_decay: float = 1.0,
                    loss_config=None, attn: str = "dense", return_logits: bool = False,
-                   verifier_logits=None, d2t=None):
+                   verifier_logits=None, d2t=None, rotary_state=None):
     """-> (draft_tokens, loss, metrics[, logits per step]).
     models/eagle3/core.py:192-365.  ``verifier_logits`` (``[1, T, Vt]``, with the ``d2t`` offset
     table) stands in for ``verifier_last_hidden_states``: the targets are then those logits at
@@ -261,10 +339,14 @@ def eagle3_forward(w, shape: DraftShape, hidden_states, input_ids, document_ids,
 
     caches = [dict() for _ in range(shape.num_hidden_layers)]
     draft_tokens, all_logits = [], []
+    # one rotary module serves every step (and every later forward pass: hand the state in again)
+    if rotary_state is None:
+        rotary_state = RotaryState(shape.head_dim, shape.rope_theta, shape.rope_scaling)
     for step in range(ttt_steps):
         with torch.no_grad():
             embeds = F.embedding(input_ids, w["embed_tokens.weight"])
-        cos, sin = rope_tables(position_ids, shape.head_dim, shape.rope_theta, dtype, shape.rope_scaling)
+        cos, sin = rope_tables(position_ids, shape.head_dim, shape.rope_theta, dtype, shape.rope_scaling,
+                               rotary_state)
         y = first_layer(torch.cat([embeds, hidden], -1), w, shape, cos, sin,
                         caches[0], mask_for(0, step), attn)
         for li in range(1, shape.num_hidden_layers):

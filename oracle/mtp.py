@@ -39,7 +39,7 @@ import torch
 import torch.nn.functional as F
 
 from .attention import dense_attention
-from .eagle3 import DraftShape, apply_rope, rms_norm, rope_tables, swiglu_mlp
+from .eagle3 import DraftShape, RotaryState, apply_rope, rms_norm, rope_tables, swiglu_mlp
 
 IGNORE_INDEX = -100
 
@@ -265,13 +265,17 @@ def mtp_forward(w, shape: DraftShape, input_ids, hidden_states, position_ids=Non
     masks = packed_causal_mask(pos) if attention_mask is None else \
         padded_causal_mask(attention_mask[:, :valid])
     current = hidden_states
+    rotary = RotaryState(rotary_dim(shape), shape.rope_theta, shape.rope_scaling)
     for step in range(steps):
         hid = current[:, :valid]
         emb = F.embedding(input_ids[:, step + 1:step + 1 + valid], w["embed_tokens.weight"])
         rows = []
+        # the rotary module is called once per step with the positions of the whole batch
+        # (models/mtp/core.py:196): a length-dependent rope type sees their maximum
+        inv = rotary.inv_freq(pos)
         for r in range(b):
             cos, sin = rope_tables(pos[r], rotary_dim(shape), shape.rope_theta, hid.dtype,
-                                   shape.rope_scaling)
+                                   shape.rope_scaling, inv_freq=inv)
             rows.append(mtp_layer(hid[r:r + 1], emb[r:r + 1].to(hid.dtype), w, shape, cos, sin,
                                   masks[r], attn, None if routing is None else routing[step * b + r]))
         out = torch.cat(rows, dim=0)

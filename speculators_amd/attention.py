@@ -197,11 +197,31 @@ def ttt_attention_cached(q, k_new, v_new, cache: TTTKVCache, mask: TTTMask,
     return _TTTAttentionCached.apply(q, mask, scaling, cache, n, out, *cache.k_parts, *cache.v_parts)
 
 
+KERNEL_HEAD_DIMS = (64, 128, 256)
+
+
+def _at_kernel_head_dim(fn, q, k, v, mask, scaling):
+    """Run ``fn`` at a head size the kernels are built for.  Any other ``D <= 256`` (96 and 80 occur
+    among the verifiers the reference lists) is widened with zero columns to the next one: zero
+    columns of q / k add nothing to a score, zero columns of v give zero output columns, which are
+    cut off again; the soft-max scale stays that of the real ``D``.  The copies make this the slow
+    way round, and the result is exactly that of a kernel of the real width."""
+    d = q.shape[-1]
+    if scaling is None:
+        scaling = d ** -0.5
+    if d in KERNEL_HEAD_DIMS:
+        return fn(q, k, v, mask, scaling)
+    wide = next((s for s in KERNEL_HEAD_DIMS if s >= d), None)
+    if wide is None or k.shape[-1] != d or v.shape[-1] != d:
+        raise ValueError(f"head_dim {d}: q, k and v must share one head size of at most {KERNEL_HEAD_DIMS[-1]}")
+    pad = (0, wide - d)
+    F = torch.nn.functional
+    return fn(F.pad(q, pad), F.pad(k, pad), F.pad(v, pad), mask, scaling)[..., :d]
+
+
 def ttt_attention(q, k, v, mask: TTTMask, scaling: float | None = None) -> torch.Tensor:
     """``[1, Hq, T, D]`` x ``[1, Hkv, (step+1)*T, D]`` -> ``[1, T, Hq, D]`` (bf16)."""
-    if scaling is None:
-        scaling = q.shape[-1] ** -0.5
-    return _TTTAttention.apply(q, k, v, mask, scaling)
+    return _at_kernel_head_dim(_TTTAttention.apply, q, k, v, mask, scaling)
 
 
 @dataclass
@@ -288,9 +308,7 @@ class _SpanAttention(torch.autograd.Function):
 
 def span_attention(q, k, v, mask: SpanMask, scaling: float | None = None) -> torch.Tensor:
     """``[1, Hq, T, D]`` x ``[1, Hkv, T, D]`` -> ``[1, T, Hq, D]`` (bf16) under a ``SpanMask``."""
-    if scaling is None:
-        scaling = q.shape[-1] ** -0.5
-    return _SpanAttention.apply(q, k, v, mask, scaling)
+    return _at_kernel_head_dim(_SpanAttention.apply, q, k, v, mask, scaling)
 
 
 def ttt_hip_attention_forward(module, query, key, value, attention_mask, scaling=None, **_kwargs):
@@ -404,9 +422,7 @@ class _DFlashAttention(torch.autograd.Function):
 
 def dflash_attention(q, k, v, mask: DFlashMask, scaling: float | None = None) -> torch.Tensor:
     """``[1, Hq, NQ, D]`` x ``[1, Hkv, T + NQ, D]`` -> ``[1, NQ, Hq, D]`` (bf16)."""
-    if scaling is None:
-        scaling = q.shape[-1] ** -0.5
-    return _DFlashAttention.apply(q, k, v, mask, scaling)
+    return _at_kernel_head_dim(_DFlashAttention.apply, q, k, v, mask, scaling)
 
 
 def dflash_hip_attention_forward(module, query, key, value, attention_mask, scaling=None, **_kwargs):

@@ -43,7 +43,7 @@ class DFlashConfig:
     num_hidden_layers: int = 5
     rms_norm_eps: float = 1e-6
     rope_theta: float = 1000000.0
-    rope_scaling: dict | None = None  # HF rope parameters (rope_type default / linear / llama3)
+    rope_scaling: dict | None = None  # HF rope parameters (any rope_type of the library; see fused_ops.rope_inv_freq)
     block_size: int = 8
     mask_token_id: int | None = None
     sliding_window: int | None = None
@@ -146,6 +146,7 @@ class DFlashDraftModel(nn.Module):
         h = config.hidden_size
         self.block_size = config.block_size
         self._stager = st = WeightStager()
+        self._rotary = FO.RotaryFrequencies(config.head_dim, config.rope_theta, config.rope_scaling)
         self.draft_vocab_size = config.draft_vocab_size
         self.verifier_vocab_size = config.vocab_size
         self.use_draft_vocab = config.draft_vocab_size != config.vocab_size
@@ -231,7 +232,7 @@ class DFlashDraftModel(nn.Module):
         block_pos = get_base_indices_for_anchored_blocks(position_ids[0, anchor_pos], bs)
         kv_pos = torch.cat([position_ids.reshape(-1), block_pos]).to(torch.int64).contiguous()
         q_pos = block_pos.to(torch.int64).contiguous()
-        inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device, cfg.rope_scaling)
+        inv_freq = self._rotary.select(device, self._rotary.top(kv_pos))
         block_idx = get_base_indices_for_anchored_blocks(anchor_pos, bs)
         with torch.no_grad():
             idx = block_idx if cfg.sample_from_anchor else (block_idx - 1) % t

@@ -47,7 +47,7 @@ class Eagle3Config:
     num_hidden_layers: int = 1
     rms_norm_eps: float = 1e-5
     rope_theta: float = 500000.0
-    rope_scaling: dict | None = None  # HF rope parameters (rope_type default / linear / llama3)
+    rope_scaling: dict | None = None  # HF rope parameters (any rope_type of the library; see fused_ops.rope_inv_freq)
     norm_before_residual: bool = False
     norm_before_fc: bool = False
     fc_norm: bool = False
@@ -216,6 +216,7 @@ class Eagle3DraftModel(nn.Module):
         h = config.hidden_size
         self.hidden_size = h
         self._stager = st = WeightStager()
+        self._rotary = FO.RotaryFrequencies(config.head_dim, config.rope_theta, config.rope_scaling)
         self.draft_vocab_size = config.draft_vocab_size
         self.verifier_vocab_size = config.vocab_size
         self.use_draft_vocab = config.draft_vocab_size != config.vocab_size
@@ -338,8 +339,8 @@ class Eagle3DraftModel(nn.Module):
 
         caches = [{"steps": ttt_steps} for _ in self.layers]
         stats_cache: dict = {}
-        inv_freq = FO.rope_inv_freq(cfg.head_dim, cfg.rope_theta, device, cfg.rope_scaling)
         position_ids = position_ids.reshape(-1).to(torch.int64).contiguous()
+        rope_top = self._rotary.top(position_ids)
         draft_tokens = []
         self.last_logits = []
         for step in range(ttt_steps):
@@ -354,6 +355,8 @@ class Eagle3DraftModel(nn.Module):
             y = (embeds.to(hidden.dtype), hidden)
             normed = None
             last = len(self.layers) - 1
+            # (the positions of step j are position_ids + j; a length-dependent rope type looks at them)
+            inv_freq = self._rotary.select(device, rope_top, step)
             for li, layer in enumerate(self.layers):
                 mask = sw_mask if li in cfg.sliding_layers else full_mask
                 # the norm that reads this layer's output: the next layer's input norm, or the

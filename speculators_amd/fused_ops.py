@@ -298,20 +298,25 @@ def rope_relayout(x, position_ids, inv_freq, heads: int, rotate: bool = True, of
     return _RopeRelayout.apply(x, pos.contiguous(), inv_freq, heads, rotate, offset)
 
 
-def rope_inv_freq(head_dim: int, theta: float, device, scaling: dict | None = None) -> torch.Tensor:
+def _rope_kind(scaling) -> str:
+    return (scaling or {}).get("rope_type", (scaling or {}).get("type", "default"))
+
+
+def rope_inv_freq(head_dim: int, theta: float, device, scaling: dict | None = None,
+                  seq_len: int | None = None) -> torch.Tensor:
     """fp32 inverse frequencies, evaluated like the HF rotary initialisation the draft layer
     inherits from its verifier config: ``scaling`` is the HF rope-parameter dict (``rope_type``
-    "default", "linear", "llama3" or "yarn"; Llama-3.1 verifiers use "llama3").  ``head_dim`` is the
-    number of rotated elements per head (all of them, or the first
-    ``int(head_dim * partial_rotary_factor)`` for a partial rotary embedding).  The factor yarn puts
-    on the cos / sin tables rides on the returned tensor as ``attention_scaling`` (read by the rotary
-    kernels' wrappers through ``table_scale_of``).  "dynamic" and "longrope" pick their frequencies
-    from the length of the running sequence and are not built."""
-    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
-    kind = "default"
+    "default", "linear", "llama3", "yarn", "dynamic" or "longrope"; Llama-3.1 verifiers use
+    "llama3").  ``head_dim`` is the number of rotated elements per head (all of them, or the first
+    ``int(head_dim * partial_rotary_factor)`` for a partial rotary embedding).  The factor yarn and
+    longrope put on the cos / sin tables rides on the returned tensor as ``attention_scaling`` (read
+    by the rotary kernels' wrappers through ``table_scale_of``).  "dynamic" and "longrope" depend on
+    the length ``seq_len`` of the running sequence (``max_position_embeddings`` travels in
+    ``scaling`` for them); which length applies from call to call is ``RotaryFrequencies``."""
+    steps = torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim
+    inv = 1.0 / (theta ** steps)
+    kind = _rope_kind(scaling)
     table_scale = 1.0
-    if scaling:
-        kind = scaling.get("rope_type", scaling.get("type", "default"))
     if kind == "linear":
         inv = inv / float(scaling["factor"])
     elif kind == "llama3":
@@ -327,12 +332,81 @@ def rope_inv_freq(head_dim: int, theta: float, device, scaling: dict | None = No
         inv = torch.where(medium, blended, scaled)
     elif kind == "yarn":
         inv, table_scale = _yarn(inv, head_dim, theta, scaling)
+    elif kind == "dynamic":
+        # NTK-aware: the base grows once the sequence is longer than the trained context
+        # (_compute_dynamic_ntk_parameters of transformers' modeling_rope_utils.py, whose forward-time
+        # update passes the length as an int64 tensor: the new base is an fp32 value)
+        factor, ctx = float(scaling["factor"]), int(scaling["max_position_embeddings"])
+        if seq_len is None or int(seq_len) <= ctx:
+            grow = (factor * ctx / ctx) - (factor - 1) if seq_len is None else \
+                (factor * torch.tensor(ctx, dtype=torch.int64) / ctx) - (factor - 1)
+        else:
+            grow = (factor * torch.tensor(int(seq_len), dtype=torch.int64) / ctx) - (factor - 1)
+        base = theta * grow ** (head_dim / (head_dim - 2))
+        inv = 1.0 / (base ** steps)
+    elif kind == "longrope":
+        # per-frequency divisors (_compute_longrope_parameters): the long set beyond the original context
+        ctx0 = int(scaling["original_max_position_embeddings"])
+        long = seq_len is not None and int(seq_len) > ctx0
+        ext = torch.tensor(scaling["long_factor" if long else "short_factor"], dtype=torch.float32)
+        inv = 1.0 / (ext * theta ** steps)
+        table_scale = scaling.get("attention_factor")
+        if table_scale is None:
+            factor = scaling.get("factor")
+            if factor is None:
+                factor = int(scaling["max_position_embeddings"]) / ctx0
+            table_scale = 1.0 if factor <= 1.0 else math.sqrt(1 + math.log(factor) / math.log(ctx0))
     elif kind != "default":
-        raise NotImplementedError(
-            f"rope_type '{kind}' is not built on the HIP path (default, linear, llama3 and yarn are)")
+        raise NotImplementedError(f"rope_type '{kind}' is not one of default, linear, llama3, yarn, dynamic, longrope")
     inv = inv.to(device)
-    inv.attention_scaling = table_scale
+    inv.attention_scaling = float(table_scale)
     return inv
+
+
+class RotaryFrequencies:
+    """The inverse frequencies a model's rotary embedding runs with from call to call: fixed for most
+    types; "longrope" switches to its long divisors when the highest position of the call is beyond
+    the original context, "dynamic" recomputes them whenever a call is longer than every call before
+    it (and than ``max_position_embeddings``) and goes back to the original ones on a call shorter
+    than ``max_position_embeddings`` -- the behaviour of ``dynamic_rope_update``, which wraps the
+    forward of every HF rotary module (the reference builds the verifier's, models/eagle3/core.py:112).
+    Only those two types look at the positions (one device-to-host read per forward pass)."""
+
+    def __init__(self, head_dim: int, theta: float, scaling: dict | None = None):
+        self.head_dim, self.theta, self.scaling = head_dim, theta, scaling
+        self.kind = _rope_kind(scaling)
+        self.by_length = self.kind in ("dynamic", "longrope")
+        self._made: dict = {}
+        if self.kind == "dynamic":
+            self._ctx = int(scaling["max_position_embeddings"])
+            self._seen = self._ctx
+            self._length = None
+
+    def top(self, position_ids) -> int | None:
+        """Highest position of the call (``None`` where the frequencies do not depend on it)."""
+        return int(position_ids.max()) if self.by_length else None
+
+    def _get(self, device, length):
+        key = (str(device), length)
+        if key not in self._made:
+            self._made[key] = rope_inv_freq(self.head_dim, self.theta, device, self.scaling, length)
+        return self._made[key]
+
+    def select(self, device, top: int | None = None, offset: int = 0) -> torch.Tensor:
+        """Frequencies of a call whose highest position is ``top + offset``."""
+        if not self.by_length:
+            return self._get(device, None)
+        n = top + offset + 1
+        if self.kind == "longrope":
+            ctx0 = int(self.scaling["original_max_position_embeddings"])
+            return self._get(device, ctx0 + 1 if n > ctx0 else None)
+        if n > self._seen:
+            self._seen, self._length = n, n
+        if n < self._ctx and self._seen > self._ctx:
+            self._seen, self._length = self._ctx, None
+        if len(self._made) > 64:
+            self._made.clear()
+        return self._get(device, self._length)
 
 
 def _yarn(inv, dim: int, theta: float, scaling: dict):

@@ -59,7 +59,7 @@ class MTPConfig:
     num_speculative_steps: int = 3
     rms_norm_eps: float = 1e-6
     rope_theta: float = 1000000.0
-    rope_scaling: dict | None = None  # HF rope parameters (rope_type default / linear / llama3)
+    rope_scaling: dict | None = None  # HF rope parameters (any rope_type of the library; see fused_ops.rope_inv_freq)
     model_type: str = "qwen3"
     attn_implementation: str = A.ATTN_IMPL_TTT
     qk_norm: bool = True  # Qwen3 attention
@@ -89,6 +89,8 @@ class MTPConfig:
         rope.pop("mrope_section", None)
         rope.pop("mrope_interleaved", None)
         kind = rope.get("rope_type", rope.get("type", "default"))
+        if kind in ("dynamic", "longrope"):  # the trained context travels with the rope parameters here
+            rope.setdefault("max_position_embeddings", tc.max_position_embeddings)
         head_dim = getattr(tc, "head_dim", None) or tc.hidden_size // tc.num_attention_heads
         kw = dict(hidden_size=tc.hidden_size, num_attention_heads=tc.num_attention_heads,
                   num_key_value_heads=tc.num_key_value_heads, head_dim=head_dim,
@@ -164,6 +166,7 @@ class MTPDraftModel(nn.Module):
         resolve_model_type(config.model_type)
         self.config = config
         self._stager = WeightStager()
+        self._rotary = FO.RotaryFrequencies(config.rotary_dim, config.rope_theta, config.rope_scaling)
         self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size)
         self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
         layer_class = MTPLayer if config.model_type == "qwen3" else HybridMTPLayer
@@ -234,7 +237,7 @@ class MTPDraftModel(nn.Module):
                 raise ValueError(f"attention_mask must be {(b, n)}, got {tuple(attention_mask.shape)}")
             mask = A.create_padding_span_mask(attention_mask[:, :valid].to(device))
         flat_pos = pos.reshape(-1).contiguous()
-        inv_freq = FO.rope_inv_freq(cfg.rotary_dim, cfg.rope_theta, device, cfg.rope_scaling)
+        rope_top = self._rotary.top(flat_pos)
         layer = self.mtp_layers[0]
 
         current = hidden_states
@@ -243,6 +246,8 @@ class MTPDraftModel(nn.Module):
             with torch.no_grad():
                 emb = F.embedding(input_ids[:, step + 1:step + 1 + valid], self.embed_tokens.weight)
                 emb = emb.to(hidden_states.dtype).reshape(1, b * valid, cfg.hidden_size)
+            # (asked once per step, like the rotary module: models/mtp/core.py:196)
+            inv_freq = self._rotary.select(device, rope_top)
             out = layer(hid, emb, flat_pos, inv_freq, mask)
             targets = input_ids[:, step + 2:step + 2 + valid]
             if loss_mask is not None:

@@ -98,6 +98,38 @@ def test_backward_matches_dense_oracle_autograd(t, hq, hkv, d, docs, window, ste
         assert err <= 2e-2 * kr.grad[:, :, t:].abs().max().item() + 1e-5
 
 
+@pytest.mark.parametrize("d", [96, 80, 40, 192])
+def test_head_sizes_between_the_kernels(d):
+    """A head size the kernels are not built for runs through the next wider one (zero columns):
+    forward and all three gradients against the dense oracle at the real width."""
+    from speculators_amd.attention import create_ttt_mask, ttt_attention
+
+    t, hq, hkv, steps, window = 160, 4, 2, 2, None
+    g = torch.Generator().manual_seed(d)
+    doc = _docs(t, [90, 60])
+    mask = create_ttt_mask(doc.cuda(), t, window).extended()
+    q = torch.randn(1, hq, t, d, generator=g).bfloat16()
+    k = torch.randn(1, hkv, steps * t, d, generator=g).bfloat16()
+    v = torch.randn(1, hkv, steps * t, d, generator=g).bfloat16()
+    go = torch.randn(1, t, hq, d, generator=g).bfloat16()
+    qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    out = ttt_attention(qg, kg, vg, mask)  # default scale: that of the real head size
+    assert out.shape == (1, t, hq, d)
+    out.backward(go.cuda())
+    qr, kr, vr = (x.float().requires_grad_(True) for x in (q, k, v))
+    ref = dense_attention(qr, kr, vr, OM.ttt_mask_dense(doc, t, 1, window), d ** -0.5)
+    ref.backward(go.float())
+    assert (out.float().cpu() - ref).abs().max().item() <= 2e-2 * ref.abs().max().item()
+    for name, got, want in (("dq", qg.grad, qr.grad), ("dk", kg.grad, kr.grad), ("dv", vg.grad, vr.grad)):
+        assert got.shape == want.shape
+        err = (got.float().cpu() - want).abs().max().item()
+        assert err <= 2e-2 * want.abs().max().item() + 1e-5, (name, err)
+    with pytest.raises(ValueError):
+        ttt_attention(torch.zeros(1, hq, t, 320, device="cuda", dtype=torch.bfloat16),
+                      torch.zeros(1, hkv, 2 * t, 320, device="cuda", dtype=torch.bfloat16),
+                      torch.zeros(1, hkv, 2 * t, 320, device="cuda", dtype=torch.bfloat16), mask)
+
+
 def _random_cases(n, seed):
     """Seeded shapes that land on every edge of the tiling: sequences shorter than one key tile,
     one row past a tile, ragged document packs with and without padding, windows shorter and

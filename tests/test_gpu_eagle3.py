@@ -17,6 +17,9 @@ def _shape(**kw):
     return OE.DraftShape(**base)
 
 
+_HALF = 32  # frequencies per head at the head size of `_shape`
+
+
 def _batch(shape, t, seed, docs):
     g = torch.Generator().manual_seed(seed)
     hs = torch.randn(1, t, shape.num_aux * shape.hidden_size, generator=g)
@@ -62,6 +65,14 @@ VARIANTS = [
     dict(qk_norm=True, rope_scaling={"rope_type": "yarn", "factor": 4.0, "original_max_position_embeddings": 64,
                                      "attention_factor": 1.3}),
     dict(embed_requires_grad=True),  # marks the parameter trainable; the lookup itself has no graph
+    # length-dependent types (the batch's highest position is 170, + 1 per TTT step): longrope whose
+    # long divisors set in between step 0 and step 1, NTK-dynamic whose base grows at every step
+    dict(rope_scaling={"rope_type": "longrope", "original_max_position_embeddings": 171,
+                       "max_position_embeddings": 1368,
+                       "short_factor": [1.0 + 0.01 * i for i in range(_HALF)],
+                       "long_factor": [1.5 + 0.2 * i for i in range(_HALF)]}),
+    dict(num_hidden_layers=2, rope_scaling={"rope_type": "dynamic", "factor": 2.0,
+                                            "max_position_embeddings": 100}),
 ]
 
 

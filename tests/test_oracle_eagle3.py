@@ -213,8 +213,65 @@ def test_rope_inv_freq_matches_transformers(scaling, head_dim, theta):
 def test_rope_scaling_rejects_unknown_types():
     from speculators_amd.fused_ops import rope_inv_freq
 
-    for kind in ("dynamic", "longrope"):
-        with pytest.raises(NotImplementedError):
-            rope_inv_freq(64, 10000.0, "cpu", {"rope_type": kind, "factor": 2.0})
-        with pytest.raises(NotImplementedError):
-            E.rope_inv_freq(64, 10000.0, {"rope_type": kind, "factor": 2.0})
+    with pytest.raises(NotImplementedError):
+        rope_inv_freq(64, 10000.0, "cpu", {"rope_type": "no-such-type", "factor": 2.0})
+    with pytest.raises(NotImplementedError):
+        E.rope_inv_freq(64, 10000.0, {"rope_type": "no-such-type", "factor": 2.0})
+
+
+def _length_dependent_cases(head_dim):
+    g = torch.Generator().manual_seed(head_dim)
+    long = (1 + 3 * torch.rand(head_dim // 2, generator=g)).tolist()
+    short = (1 + 0.2 * torch.rand(head_dim // 2, generator=g)).tolist()
+    longrope = {"rope_type": "longrope", "long_factor": long, "short_factor": short,
+                "original_max_position_embeddings": 128}
+    return [({"rope_type": "dynamic", "factor": 2.0}, 256),
+            ({"rope_type": "dynamic", "factor": 4.0}, 64),
+            (longrope, 1024),                                    # factor = 1024 / 128
+            (dict(longrope, factor=8.0, attention_factor=1.3), 1024),
+            (dict(longrope, factor=1.0), 1024)]                  # no table factor
+
+
+@pytest.mark.parametrize("head_dim,theta", [(64, 10000.0), (128, 500000.0)])
+@pytest.mark.parametrize("case", range(5))
+def test_length_dependent_rope_follows_the_library_module_call_by_call(case, head_dim, theta):
+    """"dynamic" and "longrope": the frequencies the HF rotary module runs with over a sequence of
+    calls (growth, a shorter call that keeps the grown base, the reset below the trained context;
+    either side of the longrope threshold) == the oracle's ``RotaryState`` == the product's
+    ``RotaryFrequencies``, bit for bit, tables and table factor included."""
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaRotaryEmbedding
+
+    from speculators_amd.fused_ops import RotaryFrequencies
+
+    scaling, ctx = _length_dependent_cases(head_dim)[case]
+    params = {"rope_theta": theta}
+    params.update(scaling)
+    cfg = LlamaConfig(hidden_size=head_dim * 4, num_attention_heads=4, head_dim=head_dim,
+                      rope_parameters=params, max_position_embeddings=ctx)
+    module = LlamaRotaryEmbedding(cfg)
+    mine = dict(scaling, max_position_embeddings=ctx)
+    state = E.RotaryState(head_dim, theta, mine)
+    product = RotaryFrequencies(head_dim, theta, mine)
+    assert product.by_length and torch.equal(module.inv_freq, state.original)
+    assert E.rope_table_scale(mine) == pytest.approx(module.attention_scaling, rel=1e-12)
+    for top in (50, 300, 280, 1000, 400, 100, 260, 63, 64, 65, 127, 128, 129, 255, 256, 257):
+        pos = torch.arange(top - 20, top).unsqueeze(0)
+        cos, sin = module(torch.zeros(1, 20, 8), pos)
+        assert torch.equal(state.inv_freq(pos), module.inv_freq), top
+        mc, ms = E.rope_tables(pos[0], head_dim, theta, torch.float32, mine, inv_freq=module.inv_freq)
+        assert torch.equal(mc, cos) and torch.equal(ms, sin)
+        # the product is asked with the highest position split into base + offset (a TTT step)
+        got = product.select("cpu", product.top(pos) - 3, 3)
+        assert torch.equal(got, module.inv_freq), top
+        assert got.attention_scaling == pytest.approx(module.attention_scaling, rel=1e-12)
+
+
+def test_fixed_rope_types_never_read_the_positions():
+    from speculators_amd.fused_ops import RotaryFrequencies
+
+    for scaling in (None, _LLAMA31, _YARN, {"rope_type": "linear", "factor": 2.0}):
+        r = RotaryFrequencies(64, 10000.0, scaling)
+        assert not r.by_length and r.top(None) is None
+        assert r.select("cpu") is r.select("cpu", None, 5)
+        assert torch.equal(r.select("cpu"), E.rope_inv_freq(64, 10000.0, scaling))
