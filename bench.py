@@ -268,6 +268,10 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
     y = torch.empty(t, vd, device=device, dtype=torch.bfloat16)
     ms = time_events(torch, lambda: gemm_nt(x, w, y), 20)
     mfma("gemm_bf16_nt_kernel[lm_head fwd T x H x Vd]", 2.0 * t * h * vd, ms, k_steps + 1, "gemm_fwd")
+    # the vendor library on the same product: a yardstick beside the kernel above, not part of the step
+    ms = time_events(torch, lambda: torch.nn.functional.linear(x, w), 20)
+    mfma("hipBLASLt through torch.nn.functional.linear[lm_head fwd T x H x Vd, yardstick]",
+         2.0 * t * h * vd, ms, 0)
     wt = w.t().contiguous()
     dx = torch.empty(t, h, device=device, dtype=torch.bfloat16)
     ms = time_events(torch, lambda: gemm_nt(y, wt, dx), 20)

@@ -2,8 +2,11 @@
 // accumulate, bf16 out, for gfx950.
 //
 // One workgroup of 4 waves owns a 256 x 256 tile of C (each wave a 128 x 128
-// patch = 4 x 4 accumulators of v_mfma_f32_32x32x16_bf16, one wave per SIMD)
-// and walks K in slabs of 64.
+// patch = 8 x 8 accumulators of v_mfma_f32_16x16x32_bf16, one wave per SIMD)
+// and walks K in slabs of 64.  (The 16 x 16 x 32 form of the instruction reads and
+// writes its accumulator half as often per multiply-add as the 32 x 32 x 16 form:
+// a register-only loop of it holds 2.09 PFLOP/s at the power limit of the chip, the
+// 32 x 32 x 16 form 1.83.)
 //
 // Global -> LDS directly (buffer_load ... lds): no staging registers and no
 // LDS store instructions.  A wave-load fills 8 rows x 128 B of LDS linearly
@@ -14,12 +17,12 @@
 // multiplied.  They are issued one at a time between the MFMAs (a burst would
 // stall the wave at issue until the memory pipeline has room), and so are the
 // LDS reads: operand fragments are double buffered in registers, the reads of
-// K step kk+1 run under the MFMAs of step kk, and the last step of a slab is
-// multiplied after the barrier that opens the next slab, so no LDS latency is
-// exposed and there is one barrier per slab.
+// K step kk+1 (32 columns) run under the MFMAs of step kk, and the last step of a
+// slab is multiplied after the barrier that opens the next slab, so no LDS latency
+// is exposed and there is one barrier per slab.
 //
 // The accumulators are kept transposed (lane = row of C, registers = 4
-// consecutive columns); v_permlane32_swap pairs them into 8 consecutive
+// consecutive columns); v_permlane16_swap pairs them into 8 consecutive
 // columns for 16-byte stores.  Workgroup ids are remapped so that each XCD
 // (ids are dealt round-robin over the 8 XCDs) works on a compact band of
 // tiles and shares its A / B panels in that XCD's L2.
@@ -47,7 +50,8 @@ constexpr int kWM = SPX_GEMM_WM, kWN = SPX_GEMM_WN;  // waves along M / N of the
 constexpr int kNW = kWM * kWN;
 constexpr int kGemmThreads = 64 * kNW;
 constexpr int kTM = 256, kTN = 256, kTK = 64;
-constexpr int kMI = kTM / kWM / 32, kNI = kTN / kWN / 32;  // 32x32 accumulators per wave
+constexpr int kMI = kTM / kWM / 16, kNI = kTN / kWN / 16;  // 16x16 accumulators per wave
+constexpr int kKSteps = kTK / 32;                          // MFMA K steps per slab
 constexpr int kRowBytes = kTK * 2;                          // 128
 constexpr int kABytes = kTM * kRowBytes;                    // one slab of A: 32 KB
 constexpr int kBBytes = kTN * kRowBytes;
@@ -59,6 +63,18 @@ constexpr int kL = kLA + kLB;
 constexpr int kOob = 0x7ffffff0;
 static_assert(kABytes == 32768 && kBBytes == 32768, "the buffer toggle flips bit 15");
 static_assert(kLA % 4 == 0 && kLB % 4 == 0, "loads are grouped in fours (immediate offsets)");
+
+// acc += a * b with v_mfma_f32_16x16x32_bf16, the accumulator pinned to the accumulation registers
+// and written in place.  (With 64 accumulator tuples that fill that register file, the compiler's own
+// choice of destination leaves them permuted at the end of a loop body and moves them back through
+// vector registers on every trip.)  The compiler does not know what the statement is: whoever reads
+// an accumulator with a vector instruction afterwards waits for the matrix pipe first
+// (`mfma_results_ready`).
+__device__ __forceinline__ void mfma16(f32x4& acc, bf16x8 a, bf16x8 b) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+// more wait states than the longest matrix instruction needs before its result may be read
+__device__ __forceinline__ void mfma_results_ready() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 __device__ __forceinline__ bf16x8 as_frag(u32x4 v) {
   union { u32x4 u; bf16x8 b; } c;
@@ -120,17 +136,17 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int g = lane >> 5, col = lane & 31;
+  const int q = lane >> 4, r16 = lane & 15;
   const int wm = (wave / kWN) * (kTM / kWM), wn = (wave % kWN) * (kTN / kWN);
 
-  // acc[j][i]: registers = 32 columns of C at wn + 32 j, lane = row of C at wm + 32 i
-  f32x16 acc[kNI][kMI];
+  // acc[j][i]: lane = row wm + 16 i + lane % 16 of C, registers = columns wn + 16 j + 4 (lane / 16) + {0..3}
+  f32x4 acc[kNI][kMI];
 #pragma unroll
   for (int j = 0; j < kNI; ++j)
 #pragma unroll
     for (int i = 0; i < kMI; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[j][i][r] = 0.f;
+      for (int r = 0; r < 4; ++r) acc[j][i][r] = 0.f;
 
   // One buffer resource per operand; the K position goes into the scalar offset.  Rows
   // past the matrix edge get an offset outside the resource and read as zero, so no
@@ -186,23 +202,23 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   };
   auto next_slab = [&]() __attribute__((always_inline)) { bufoff ^= kABytes; ld_k0 += kTK; };
 
-  // read side: row = lane % 32 of a 32-row block, K chunk 2 kk + g in slot chunk ^ f(row)
-  const int fr = (col & 7) ^ ((col >> 3) & 1);
-  const int off0 = col * kRowBytes + ((g ^ fr) * 16);
-  uint32_t a_rd[4], b_rd[4];  // per K step of 16; bit 15 selects the slab buffer
+  // read side: row = lane % 16 of a 16-row block, K chunk 4 kk + lane / 16 in slot chunk ^ f(row)
+  const int fr = (r16 & 7) ^ (r16 >> 3);
+  const int off0 = r16 * kRowBytes + ((q ^ fr) * 16);
+  uint32_t a_rd[kKSteps], b_rd[kKSteps];  // per K step of 32; bit 15 selects the slab buffer
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) {
-    a_rd[kk] = wm * kRowBytes + (off0 ^ (kk * 32));
-    b_rd[kk] = kBBase + wn * kRowBytes + (off0 ^ (kk * 32));
+  for (int kk = 0; kk < kKSteps; ++kk) {
+    a_rd[kk] = wm * kRowBytes + (off0 ^ (kk * 64));
+    b_rd[kk] = kBBase + wn * kRowBytes + (off0 ^ (kk * 64));
   }
 
   bf16x8 fa[2][kMI], fb[2][kNI];
   // operand fragment f (A fragments first, then B) of K step kk into register set `set`
   auto read_one = [&](int set, int kk, int f) __attribute__((always_inline)) {
     if (f < kMI)
-      fa[set][f] = as_frag(*reinterpret_cast<const u32x4*>(smem + a_rd[kk] + f * 32 * kRowBytes));
+      fa[set][f] = as_frag(*reinterpret_cast<const u32x4*>(smem + a_rd[kk] + f * 16 * kRowBytes));
     else
-      fb[set][f - kMI] = as_frag(*reinterpret_cast<const u32x4*>(smem + b_rd[kk] + (f - kMI) * 32 * kRowBytes));
+      fb[set][f - kMI] = as_frag(*reinterpret_cast<const u32x4*>(smem + b_rd[kk] + (f - kMI) * 16 * kRowBytes));
   };
   // One K step: the kNI x kMI MFMAs on register set `set`; between them, one at a time,
   // the LDS reads that fill the other set with K step rk and the global loads
@@ -214,7 +230,7 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
     for (int j = 0; j < kNI; ++j)
 #pragma unroll
       for (int i = 0; i < kMI; ++i) {
-        acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[set][j], fa[set][i], acc[j][i], 0, 0, 0);
+        mfma16(acc[j][i], fb[set][j], fa[set][i]);
         const int idx = j * kMI + i;
         __builtin_amdgcn_sched_barrier(0);
         if (reads < kF) {
@@ -229,25 +245,23 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
       }
   };
 
-  // the loads of a slab are spread over the step after the barrier (kLdT of them) and
-  // step 0 of the next slab (the rest); steps 1 and 2 give them time to land
-  constexpr int kLdT = kL / 2, kLd0 = kL - kLdT;
-  // one slab: on entry set 0 holds (or is receiving) K step 0 of slab s and the first
-  // kLdT loads of slab s+1 are issued
+  // the loads of a slab are issued in the step after the barrier that frees its buffer, one per
+  // four MFMAs; the step after that gives them time to land
+  static_assert(kKSteps == 2, "a slab is two K steps: one before, one after the barrier");
+  constexpr int kLdT = kL;
+  // one slab: on entry set 0 holds (or is receiving) K step 0 of slab s and the loads of slab s+1
+  // are issued
   auto slab = [&](bool full) __attribute__((always_inline)) {
     __builtin_amdgcn_sched_barrier(0);
-    step(0, 1, kLdT, kLd0, full);
+    step(0, 1, 0, 0, full);
     next_slab();
-    step(1, 2, 0, 0, full);
-    step(0, 3, 0, 0, full);
     // every read of this slab's buffer has returned once set 1 is complete; then the
     // barrier says: slab s+1 has landed for everybody, this buffer is free
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) { a_rd[kk] ^= kABytes; b_rd[kk] ^= kBBytes; }
-    // K step 3 of slab s, under it the reads of step 0 of slab s+1 and the first loads
-    // of slab s+2
+    for (int kk = 0; kk < kKSteps; ++kk) { a_rd[kk] ^= kABytes; b_rd[kk] ^= kBBytes; }
+    // K step 1 of slab s, under it the reads of step 0 of slab s+1 and the loads of slab s+2
     step(1, 0, 0, kLdT, full);
   };
 
@@ -269,36 +283,35 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   for (; s < nslab; ++s) slab(false);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-  // epilogue: a lane holds row m of C and, per accumulator, columns 8 q + 4 g + {0..3}
-  // (q = 0..3).  Swapping the q-odd words of the lower half-wave with the q-even words of
-  // the upper half-wave leaves every lane with 8 consecutive columns: 16-byte stores.
+  mfma_results_ready();
+  // epilogue: a lane holds row m of C and, per accumulator, columns 4 q + {0..3} of a 16-column
+  // block (q = lane / 16).  Swapping the words of the q-odd lanes for block j with those of the
+  // q-even lanes for block j + 1 leaves every lane with 8 consecutive columns: 16-byte stores.
   const bool fast = (ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0) && (n0 + kTN <= N);
 #pragma unroll
   for (int i = 0; i < kMI; ++i) {
-    const int m = m0 + wm + i * 32 + col;
+    const int m = m0 + wm + i * 16 + r16;
 #pragma unroll
-    for (int j = 0; j < kNI; ++j) {
-      const f32x16& a = acc[j][i];
+    for (int j = 0; j < kNI; j += 2) {
+      const f32x4& a = acc[j][i];
+      const f32x4& b = acc[j + 1][i];
+      const uint32_t e0 = pack_bf16x2(a[0], a[1]), e1 = pack_bf16x2(a[2], a[3]);
+      const uint32_t o0 = pack_bf16x2(b[0], b[1]), o1 = pack_bf16x2(b[2], b[3]);
+      // odd rows of 16 lanes of the first operand <-> even rows of the second
+      const auto s0 = __builtin_amdgcn_permlane16_swap(e0, o0, false, false);
+      const auto s1 = __builtin_amdgcn_permlane16_swap(e1, o1, false, false);
+      // q even: (own, neighbour's) words of block j = its columns 4 q + 0..7;
+      // q odd: (neighbour's, own) words of block j + 1 = its columns 4 (q - 1) + 0..7
+      u32x4 v;
+      v.x = s0[0]; v.y = s1[0]; v.z = s0[1]; v.w = s1[1];
+      const int n = n0 + wn + (j + (q & 1)) * 16 + 4 * (q & 2);
+      if (fast) {
+        if (m < M) *reinterpret_cast<u32x4*>(&C[(int64_t)m * ldc + n]) = v;
+      } else if (m < M) {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {  // q pair (2h, 2h+1)
-        const uint32_t e0 = pack_bf16x2(a[8 * h + 0], a[8 * h + 1]), e1 = pack_bf16x2(a[8 * h + 2], a[8 * h + 3]);
-        const uint32_t o0 = pack_bf16x2(a[8 * h + 4], a[8 * h + 5]), o1 = pack_bf16x2(a[8 * h + 6], a[8 * h + 7]);
-        // lanes 32..63 of the first operand <-> lanes 0..31 of the second
-        const auto s0 = __builtin_amdgcn_permlane32_swap(e0, o0, false, false);
-        const auto s1 = __builtin_amdgcn_permlane32_swap(e1, o1, false, false);
-        // lower half: (own q-even, partner's q-even) = columns 16 h + 0..7;
-        // upper half: (partner's q-odd, own q-odd) = columns 16 h + 8..15
-        u32x4 v;
-        v.x = s0[0]; v.y = s1[0]; v.z = s0[1]; v.w = s1[1];
-        const int n = n0 + wn + j * 32 + 16 * h + 8 * g;
-        if (fast) {
-          if (m < M) *reinterpret_cast<u32x4*>(&C[(int64_t)m * ldc + n]) = v;
-        } else if (m < M) {
-          const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (n + e < N) C[(int64_t)m * ldc + n + e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
-        }
+        for (int e = 0; e < 8; ++e)
+          if (n + e < N) C[(int64_t)m * ldc + n + e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
       }
     }
   }
