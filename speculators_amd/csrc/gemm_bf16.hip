@@ -64,18 +64,6 @@ constexpr int kOob = 0x7ffffff0;
 static_assert(kABytes == 32768 && kBBytes == 32768, "the buffer toggle flips bit 15");
 static_assert(kLA % 4 == 0 && kLB % 4 == 0, "loads are grouped in fours (immediate offsets)");
 
-// acc += a * b with v_mfma_f32_16x16x32_bf16, the accumulator pinned to the accumulation registers
-// and written in place.  (With 64 accumulator tuples that fill that register file, the compiler's own
-// choice of destination leaves them permuted at the end of a loop body and moves them back through
-// vector registers on every trip.)  The compiler does not know what the statement is: whoever reads
-// an accumulator with a vector instruction afterwards waits for the matrix pipe first
-// (`mfma_results_ready`).
-__device__ __forceinline__ void mfma16(f32x4& acc, bf16x8 a, bf16x8 b) {
-  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-}
-// more wait states than the longest matrix instruction needs before its result may be read
-__device__ __forceinline__ void mfma_results_ready() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
-
 __device__ __forceinline__ bf16x8 as_frag(u32x4 v) {
   union { u32x4 u; bf16x8 b; } c;
   c.u = v;
