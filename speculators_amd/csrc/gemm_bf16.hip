@@ -43,6 +43,9 @@ namespace spx {
 #ifndef SPX_GEMM_MINW
 #define SPX_GEMM_MINW 1
 #endif
+#ifndef SPX_GEMM_READ_EVERY
+#define SPX_GEMM_READ_EVERY 2  // MFMAs per LDS fragment read
+#endif
 #ifndef SPX_GEMM_GROUP_M
 #define SPX_GEMM_GROUP_M 8
 #endif
@@ -210,7 +213,9 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   };
   // One K step: the kNI x kMI MFMAs on register set `set`; between them, one at a time,
   // the LDS reads that fill the other set with K step rk and the global loads
-  // [l0, l0 + nl).  Reads go first: their data is needed at the next step.
+  // [l0, l0 + nl).  A read after every second MFMA (a 16 x 16 x 32 MFMA occupies the pipe for 16
+  // cycles: a read and its address arithmetic behind each one leave the pipe waiting), in the first
+  // half of the step: their data is needed at the next step.
   auto step = [&](int set, int rk, int l0, int nl, bool full) __attribute__((always_inline)) {
     constexpr int kN = kNI * kMI, kF = kMI + kNI;
     int reads = 0, loads = 0;
@@ -221,9 +226,8 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
         mfma16(acc[j][i], fb[set][j], fa[set][i]);
         const int idx = j * kMI + i;
         __builtin_amdgcn_sched_barrier(0);
-        if (reads < kF) {
+        if (reads < kF && idx % SPX_GEMM_READ_EVERY == SPX_GEMM_READ_EVERY - 1) {
           read_one(set ^ 1, rk, reads++);
-          if (kF > kN && reads < kF) read_one(set ^ 1, rk, reads++);
           __builtin_amdgcn_sched_barrier(0);
         }
         if (nl > 0 && (nl >= kN || idx % (kN / nl) == kN / nl - 1) && loads < nl) {
