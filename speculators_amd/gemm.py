@@ -159,13 +159,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor | None 
 
 
 # Which GEMM runs the decoder-layer projections (q/k/v, o, gate/up, down and their input
-# gradients): "hipblaslt" = PyTorch's matmul (the library GEMM; measured a few percent faster on
-# these shapes), "spx" = this library's MFMA kernel (the input gradients then run against the
-# transposed copy of the staged weight).  The fc / lm_head / verifier-head products and every
-# weight gradient always run on this library's kernels.
-DECODER_GEMM = os.environ.get("SPX_DECODER_GEMM", "hipblaslt")
-if DECODER_GEMM not in ("hipblaslt", "spx"):
-    raise ValueError(f"SPX_DECODER_GEMM must be 'hipblaslt' or 'spx', got {DECODER_GEMM!r}")
+# gradients): "hipblaslt" = PyTorch's matmul (the library GEMM), "spx" = this library's MFMA kernel
+# (the input gradients then run against the transposed copy of the staged weight), "mixed" = each
+# where it is faster on these shapes: the forward products on hipBLASLt (3 - 8 % ahead there), the
+# input gradients on this library's kernel (8 - 20 % ahead of the library's NN product).  The fc /
+# lm_head / verifier-head products and every weight gradient always run on this library's kernels.
+DECODER_GEMM = os.environ.get("SPX_DECODER_GEMM", "mixed")
+if DECODER_GEMM not in ("hipblaslt", "spx", "mixed"):
+    raise ValueError(f"SPX_DECODER_GEMM must be 'hipblaslt', 'spx' or 'mixed', got {DECODER_GEMM!r}")
 
 
 def _project(x2: torch.Tensor, staged) -> torch.Tensor:
@@ -174,8 +175,13 @@ def _project(x2: torch.Tensor, staged) -> torch.Tensor:
 
 
 def _project_back(dy2: torch.Tensor, staged) -> torch.Tensor:
-    """``dy2 @ staged.w``: the input gradient of a decoder-layer projection."""
-    return gemm_nt(dy2, staged.wt) if DECODER_GEMM == "spx" else torch.matmul(dy2, staged.w)
+    """``dy2 @ staged.w``: the input gradient of a decoder-layer projection ("mixed": this one on the
+    library's kernel against the transposed copy, the forward product on hipBLASLt)."""
+    # (the kernel contracts in chunks of 8: a projection a few columns wide -- a gate of width 1 --
+    # stays with the library)
+    if DECODER_GEMM != "hipblaslt" and dy2.shape[1] % 8 == 0 and dy2.stride(0) % 8 == 0 and dy2.stride(1) == 1:
+        return gemm_nt(dy2, staged.wt)
+    return torch.matmul(dy2, staged.w)
 
 
 class _StagedLinear(torch.autograd.Function):

@@ -485,8 +485,9 @@ def test_head_node_falls_back_for_compound_losses():
 
 
 def test_decoder_projections_on_the_library_gemm(monkeypatch):
-    """``SPX_DECODER_GEMM=spx``: the decoder-layer projections and their input gradients on this
-    library's MFMA kernel instead of the library GEMM behind ``torch.matmul``.  Same loss and
+    """``SPX_DECODER_GEMM``: the decoder-layer projections and their input gradients on this
+    library's MFMA kernel (``spx``), on the library GEMM behind ``torch.matmul`` (``hipblaslt``), or
+    the forward products there and the input gradients here (``mixed``, the default).  Same loss and
     gradients up to the rounding of a bf16 product evaluated in another order."""
     from speculators_amd import gemm
 
@@ -495,18 +496,21 @@ def test_decoder_projections_on_the_library_gemm(monkeypatch):
     hs, ids, doc, mask, pos, vl = _batch(shape, 200, 3, [120, 70])
     args = (hs.bfloat16().cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.bfloat16().cuda())
     results = {}
-    for kind in ("hipblaslt", "spx"):
+    assert gemm.DECODER_GEMM in ("hipblaslt", "spx", "mixed")
+    for kind in ("hipblaslt", "spx", "mixed"):
         monkeypatch.setattr(gemm, "DECODER_GEMM", kind)
         model = _make(shape, w, torch.bfloat16)
         _, loss, metrics = model(*args, ttt_steps=3, ttt_step_loss_decay=0.8)
         loss.backward()
         results[kind] = (loss.item(), {n: p.grad.float() for n, p in model.named_parameters() if p.grad is not None},
                          metrics)
-    (la, ga, ma), (lb, gb, mb) = results["hipblaslt"], results["spx"]
-    assert abs(la - lb) <= 2e-3 * abs(la)
-    assert ga.keys() == gb.keys()
-    for n in ga:
-        assert (ga[n] - gb[n]).abs().max() <= 3e-2 * ga[n].abs().max() + 1e-6, n
-    for k_ in ma:
-        if k_.endswith("_total"):
-            assert torch.equal(ma[k_], mb[k_]), k_
+    la, ga, ma = results["hipblaslt"]
+    for other in ("spx", "mixed"):
+        lb, gb, mb = results[other]
+        assert abs(la - lb) <= 2e-3 * abs(la), other
+        assert ga.keys() == gb.keys()
+        for n in ga:
+            assert (ga[n] - gb[n]).abs().max() <= 3e-2 * ga[n].abs().max() + 1e-6, (other, n)
+        for k_ in ma:
+            if k_.endswith("_total"):
+                assert torch.equal(ma[k_], mb[k_]), (other, k_)
