@@ -878,6 +878,7 @@ def run_probes():
     lds = probe(1, 2)
     co = probe(2, 12)
     dma = probe(3, 2)
+    m16 = probe(4, 4)
     mixes = ["64 x v_exp_f32", "64 x v_fma_f32", "64 x (v_max_f32 + v_add_f32)"]
     out = {
         "mfma_32x32x16_bf16_registers_only": {
@@ -885,6 +886,11 @@ def run_probes():
                                 "frac_of_2500": round(m[0] / PEAK_BF16_TFLOPS, 3)},
             "zero_operands": {"tflops": round(m[2], 1), "shader_clock_ghz": round(m[3], 3)},
             "note": "one wave per SIMD, four independent accumulators; 32 cycles per instruction and SIMD"},
+        "mfma_16x16x32_bf16_registers_only": {
+            "random_operands": {"tflops": round(m16[0], 1), "shader_clock_ghz": round(m16[1], 3),
+                                "frac_of_2500": round(m16[0] / PEAK_BF16_TFLOPS, 3)},
+            "zero_operands": {"tflops": round(m16[2], 1), "shader_clock_ghz": round(m16[3], 3)},
+            "note": "one wave per SIMD, 64 independent accumulators; 16 cycles per instruction and SIMD"},
         "lds_read_b128": {"bytes_per_clock_per_cu": round(lds[0], 1), "bytes_per_ns_per_cu": round(lds[1], 1),
                           "note": "8 waves per CU, 16 conflict-free reads in flight per wave"},
         "vector_work_beside_a_busy_matrix_pipe": [

@@ -8,6 +8,8 @@
 //      pipe busy (two waves per SIMD, one role each)
 //   3  what a wave pays for issuing global -> LDS loads (buffer_load_dwordx4 ... lds) while the
 //      other waves of the CU read LDS and run MFMAs
+//   4  matrix pipe as in 0 with v_mfma_f32_16x16x32_bf16 (the same multiply-adds per cycle; the
+//      accumulator is read and written half as often per multiply-add)
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -47,6 +49,35 @@ __global__ __launch_bounds__(256, 1) void mfma_kernel(const float* seed, float* 
   const unsigned long long c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
   if (threadIdx.x == 0 && blockIdx.x == 0) { clk[0] = c1 - c0; clk[1] = r1 - r0; }
   out[blockIdx.x * 256 + threadIdx.x] = a0[lane & 15] + a1[1] + a2[2] + a3[3];
+}
+
+// ---- 4: matrix pipe, 16 x 16 x 32 --------------------------------------------------------------
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+__global__ __launch_bounds__(256, 1) void mfma16_kernel(const float* seed, float* out, unsigned long long* clk,
+                                                        int iters, int zero) {
+  bf16x8 x[4], y[4];
+#pragma unroll
+  for (int f = 0; f < 4; ++f)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      x[f][i] = (__bf16)(zero ? 0.f : seed[(threadIdx.x * 8 + i + 97 * f) & 4095]);
+      y[f][i] = (__bf16)(zero ? 0.f : seed[(threadIdx.x * 8 + i + 2048 + 131 * f) & 4095]);
+    }
+  f32x4 a[64];
+#pragma unroll
+  for (int q = 0; q < 64; ++q) a[q] = {};
+  const unsigned long long c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int q = 0; q < 64; ++q)
+      a[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x[q & 3], y[(q >> 2) & 3], a[q], 0, 0, 0);
+  }
+  const unsigned long long c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+  if (threadIdx.x == 0 && blockIdx.x == 0) { clk[0] = c1 - c0; clk[1] = r1 - r0; }
+  float r = 0.f;
+#pragma unroll
+  for (int q = 0; q < 64; ++q) r += a[q][1];
+  out[blockIdx.x * 256 + threadIdx.x] = r;
 }
 
 // ---- 1: LDS reads -----------------------------------------------------------------------------
@@ -211,6 +242,7 @@ int timed(F&& launch, float* ms) {
 //   2: for each of the three vector mixes {cycles per 32 MFMAs alone, cycles of the vector loop body alone,
 //      cycles per 32 MFMAs together, cycles of the vector loop body together}  (12 values)
 //   3: {cycles per 1 KB load with the other waves idle, with the other waves reading LDS and running MFMAs}
+//   4: as 0, with v_mfma_f32_16x16x32_bf16
 extern "C" int spx_probe(int which, double* out, int n) {
   Buffers b;
   hipDeviceProp_t prop;
@@ -237,6 +269,20 @@ extern "C" int spx_probe(int which, double* out, int n) {
       const double flop = (double)wgs * 4 * iters * 32 * 2.0 * 32 * 32 * 16;
       out[2 * zero] = flop / (ms * 1e-3) / 1e12;
       out[2 * zero + 1] = (double)clk[0] / ((double)clk[1] * 10.0);  // s_memrealtime counts at 100 MHz
+    }
+    return 4;
+  }
+  if (which == 4) {
+    if (n < 4) return -2;
+    const int iters = 2000, wgs = cus * 4;  // 64 MFMAs of 16 x 16 x 32 per iteration = 32 of 32 x 32 x 16
+    for (int zero = 0; zero < 2; ++zero) {
+      float ms;
+      if (timed([&] { hipLaunchKernelGGL(mfma16_kernel, dim3(wgs), dim3(256), 0, 0, b.seed, b.out, b.clk, iters, zero); }, &ms))
+        return -1;
+      PROBE_CHECK(hipMemcpy(clk, b.clk, 16, hipMemcpyDeviceToHost));
+      const double flop = (double)wgs * 4 * iters * 64 * 2.0 * 16 * 16 * 32;
+      out[2 * zero] = flop / (ms * 1e-3) / 1e12;
+      out[2 * zero + 1] = (double)clk[0] / ((double)clk[1] * 10.0);
     }
     return 4;
   }
