@@ -854,6 +854,13 @@ def run_dflash(args):
         "kernels": kernels, "cpu_baseline": None}))
 
 
+def _decoder_gemm_mode():
+    """Whose GEMM ran the decoder-layer projections (SPX_DECODER_GEMM, see speculators_amd/gemm.py)."""
+    from speculators_amd import gemm
+
+    return gemm.DECODER_GEMM
+
+
 def run_probes():
     """The hardware figures the kernel designs rest on, measured by speculators_amd/libspx_probes.so
     (csrc/probes/hw_probes.hip); one JSON object."""
@@ -1025,7 +1032,8 @@ def main():
                                + "full attention, "
                                f"targets from {'verifier hidden states through the frozen verifier head' if args.targets == 'hidden' else 'full-vocab verifier logits gathered through d2t'}",
                    "seq_len": t, "ttt_steps": k_steps, "tokens_per_step": tokens,
-                   "regime": args.regime, "final_loss": round(float(loss.detach()), 6)},
+                   "regime": args.regime, "final_loss": round(float(loss.detach()), 6),
+                   "decoder_gemm": _decoder_gemm_mode()},
         "other_regime": {"regime": "bf16" if autocast else "autocast", "ms_per_step": round(other_ms, 3),
                          "value": round(tokens / (other_ms * 1e-3), 1), "unit": "tokens/s",
                          "final_loss": round(other_loss, 6)},
