@@ -482,6 +482,23 @@ int spx_gemm_bf16_nt_rows(const void* a, int64_t lda, const void* b, int64_t ldb
                           void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
                           const int32_t* m_live, void* stream);
 
+/* spx_gemm_bf16_nt_rows with the contraction cut into up to max_parts (1 .. 8) parts when the tiles of
+ * the rows that count leave compute units idle: the product of 2860 live rows by a 4096-column weight is
+ * 192 tiles of 256 x 256 on 256 compute units, one round of a whole contraction; cut in four it is three
+ * rounds of a quarter.  The kernel chooses the number of parts from the row count it reads on the device
+ * (the count that needs the fewest rounds, if that saves a tenth or more; else one part and the direct
+ * bf16 store of spx_gemm_bf16_nt_rows); every part leaves an fp32 partial in `workspace`
+ * (spx_gemm_split_workspace_bytes(M, N, max_parts) = max_parts * M * N * 4 bytes, 16-byte aligned) and a
+ * second kernel adds the parts in their order, so the result does not depend on scheduling.  N and ldc
+ * multiples of 8, c 16-byte aligned; m_live may be NULL (all M rows count).  Used for the lm_head
+ * input-gradient product of the frozen head (model.py:66-69 is the Linear whose backward this is).
+ * No counterpart in the reference. */
+int64_t spx_gemm_split_workspace_bytes(int64_t M, int64_t N, int32_t max_parts);
+int spx_gemm_bf16_nt_rows_split(const void* a, int64_t lda, const void* b, int64_t ldb,
+                                void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                                const int32_t* m_live, int32_t max_parts, void* workspace,
+                                int64_t workspace_bytes, void* stream);
+
 /* The two ends of a packed-rows product (spx_*_bwd_packed -> spx_gemm_bf16_nt_rows).
  * spx_pack_row_map: row_map[r] = number of live rows before r if row r is live
  * (row_grad[r] != 0 and, when labels is not NULL, labels[r] != ignore_index), else -1;

@@ -73,6 +73,7 @@ SIGNATURES["spx_gemm_bf16_nt"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64
 SIGNATURES["spx_pack_row_map"] = [_P, _P, _I64, _I64, _P, _P, _P]
 SIGNATURES["spx_unpack_rows"] = [_P, _I64, _P, _I64, _I64, _I64, _P, _I64, _P]
 SIGNATURES["spx_gemm_bf16_nt_rows"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P, _P]
+SIGNATURES["spx_gemm_bf16_nt_rows_split"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P, _I32, _P, _I64, _P]
 SIGNATURES["spx_gemm_bf16_tn"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I, _P]
 SIGNATURES["spx_gemm_bf16_tn_f32"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I, _P]
 SIGNATURES["spx_rope_relayout_partial"] = [_P, _I64, _I32, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _I32,
@@ -81,6 +82,7 @@ SIGNATURES["spx_sigmoid_gate_fwd"] = [_P, _I64, _P, _I64, _I32, _P, _I64, _I64, 
 SIGNATURES["spx_sigmoid_gate_bwd"] = [_P, _I64, _P, _I64, _I32, _P, _I64, _P, _I64, _P, _I64, _I32, _I64, _I32,
                                       _I32, _P]
 SIGNATURES["spx_gemm_grouped_workspace_bytes"] = [_I64, _I64]
+SIGNATURES["spx_gemm_split_workspace_bytes"] = [_I64, _I64, _I32]
 SIGNATURES["spx_gemm_bf16_nt_grouped"] = [_P, _I64, _P, _I64, _I64, _P, _I64, _I64, _I64, _I64, _P, _I64, _P,
                                           _I64, _P]
 SIGNATURES["spx_gemm_bf16_tn_grouped"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I64, _P, _I64, _I, _I,
@@ -91,7 +93,7 @@ SIGNATURES["spx_transpose_bf16"] = [_P, _I64, _I64, _P, _I64, _I64, _I64, _I64, 
 SIGNATURES["spx_moe_gather_rows"] = [_P, _I64, _I64, _P, _P, _P, _I64, _I64, _I64, _P]
 SIGNATURES["spx_moe_combine_rows"] = [_P, _I64, _I64, _P, _P, _P, _I64, _I64, _I32, _I64, _P]
 SIGNATURES["spx_moe_pair_dot"] = [_P, _I64, _P, _I64, _I64, _P, _P, _I64, _I32, _I64, _P]
-RESTYPES = {"spx_gemm_grouped_workspace_bytes": c_int64, "spx_ttt_attn_workspace_bytes": c_int64, "spx_ttt_attn_fwd_static_max_bytes": c_int64, "spx_dflash_attn_workspace_bytes": c_int64,
+RESTYPES = {"spx_gemm_grouped_workspace_bytes": c_int64, "spx_gemm_split_workspace_bytes": c_int64, "spx_ttt_attn_workspace_bytes": c_int64, "spx_ttt_attn_fwd_static_max_bytes": c_int64, "spx_dflash_attn_workspace_bytes": c_int64,
             "spx_rmsnorm_bwd_slots": c_int64}
 
 _lib = None

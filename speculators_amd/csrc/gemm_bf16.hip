@@ -78,14 +78,34 @@ __device__ __forceinline__ bf16x8 as_frag(u32x4 v) {
 // instruction's immediate offset (which moves the LDS and the global address alike, so
 // the per-lane global offset is stored minus that immediate).  Needs every row offset to
 // be at least the immediate: lda, ldb >= 64.  Without it every load sets M0 itself.
+// Into how many parts the contraction of a product of n_tiles tiles is cut (each part a workgroup of
+// its own with an fp32 partial result): the number s <= max_parts for which the rounds the chip needs,
+// ceil(n_tiles s / cus) / s, are fewest -- if that saves a tenth or more and leaves every part at least
+// 16 slabs.  192 tiles on 256 compute units: 4 parts (3 rounds of a quarter instead of 1 round of a
+// whole); 128: 2; 256: 1.  Evaluated on the device by the product and by the kernel that adds the parts.
+__device__ __forceinline__ int choose_k_parts(int n_tiles, int max_parts, int cus, int nslab) {
+  if (n_tiles <= 0) return 1;
+  const int64_t r1 = (n_tiles + cus - 1) / cus;
+  int best = 1;
+  int64_t best_r = r1;
+  for (int s2 = 2; s2 <= max_parts; ++s2) {
+    if (nslab / s2 < 16) break;
+    const int64_t r = ((int64_t)n_tiles * s2 + cus - 1) / cus;
+    if (r * 10 <= 9 * r1 * s2 && r * best < best_r * s2) { best = s2; best_r = r; }
+  }
+  return best;
+}
+
 template <bool kImm>
 __global__ __launch_bounds__(kGemmThreads, SPX_GEMM_MINW)
 __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf16_nt_kernel(
     const uint16_t* __restrict__ A, int64_t lda, const uint16_t* __restrict__ B, int64_t ldb,
     uint16_t* __restrict__ C, int64_t ldc, int M, int N, int K, int tiles_m, int tiles_n,
     const int32_t* __restrict__ m_live, const int32_t* __restrict__ tile_tab,
-    const int32_t* __restrict__ group_off, int64_t b_group_stride) {
+    const int32_t* __restrict__ group_off, int64_t b_group_stride, float* __restrict__ part_ws,
+    int max_parts, int cus) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int M_host = M;
   // the row count may live on the device (rows packed to the front by the producer of A): the tile
   // grid shrinks to the rows that count and the workgroups beyond it leave at once
   if (m_live) {
@@ -101,13 +121,26 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   // workgroup id -> tile: XCD-contiguous bands, then groups of GROUP_M tile rows.  Workgroups go to
   // the eight XCDs round robin: XCD x gets the ids x, x + 8, ...; they are renumbered so that each XCD
   // works on one contiguous band of tiles (any grid size: the first n % 8 XCDs get one more)
-  const int n_wg = tiles_m * tiles_n;
+  // contraction in parts (part_ws): the workgroups of part p multiply columns [p, p + 1) * part length of
+  // K and leave an fp32 partial in part_ws[p]; gemm_splitk_reduce_kernel adds the parts in order
+  const int n_tiles = tiles_m * tiles_n;
+  const int parts = part_ws ? choose_k_parts(n_tiles, max_parts, cus, (K + kTK - 1) / kTK) : 1;
+  const int n_wg = n_tiles * parts;
   if ((int)blockIdx.x >= n_wg) return;
   int pid;
   {
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
     const int base = n_wg >> 3, rem = n_wg & 7;
     pid = xcd * base + min(xcd, rem) + local;
+  }
+  const int part = pid / n_tiles;
+  pid -= part * n_tiles;
+  if (parts > 1) {
+    const int slabs = ((K + kTK - 1) / kTK + parts - 1) / parts;
+    const int k_begin = part * slabs * kTK;
+    A += k_begin;
+    B += k_begin;
+    K = max(min(K - k_begin, slabs * kTK), 0);
   }
   constexpr int GROUP_M = SPX_GEMM_GROUP_M;
   const int in_group = GROUP_M * tiles_n;
@@ -276,6 +309,21 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   mfma_results_ready();
+  if (parts > 1) {
+    // this part's fp32 partial, in the accumulators' own layout: 16 bytes per lane and accumulator
+    float* const P = part_ws + (int64_t)part * M_host * N;
+#pragma unroll
+    for (int i = 0; i < kMI; ++i) {
+      const int m = m0 + wm + i * 16 + r16;
+      if (m >= M) continue;
+#pragma unroll
+      for (int j = 0; j < kNI; ++j) {
+        const int n = n0 + wn + j * 16 + 4 * q;
+        if (n < N) *reinterpret_cast<f32x4*>(P + (int64_t)m * N + n) = acc[j][i];  // (N is a multiple of 8 here)
+      }
+    }
+    return;
+  }
   // epilogue: a lane holds row m of C and, per accumulator, columns 4 q + {0..3} of a 16-column
   // block (q = lane / 16).  Swapping the words of the q-odd lanes for block j with those of the
   // q-even lanes for block j + 1 leaves every lane with 8 consecutive columns: 16-byte stores.
@@ -309,15 +357,56 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   }
 }
 
+// C[m, n .. n + 7] = the sum of the parts of a product whose contraction was cut (in the order of the
+// parts, fp32, one rounding).  Re-derives the number of parts like the product did; nothing to do for one.
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ part_ws,
+                                                                 uint16_t* __restrict__ C, int64_t ldc, int M_host,
+                                                                 int N, int K, int tiles_n,
+                                                                 const int32_t* __restrict__ m_live, int max_parts,
+                                                                 int cus) {
+  const int M = m_live ? min(M_host, max(*m_live, 0)) : M_host;
+  const int parts = choose_k_parts(((M + kTM - 1) / kTM) * tiles_n, max_parts, cus, (K + kTK - 1) / kTK);
+  if (parts <= 1) return;
+  const int n8 = N / 8;
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (item >= (int64_t)M * n8) return;
+  const int m = (int)(item / n8), n = (int)(item % n8) * 8;
+  f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+  for (int p = 0; p < parts; ++p) {
+    const float* src = part_ws + ((int64_t)p * M_host + m) * N + n;
+    const f32x4 a = *reinterpret_cast<const f32x4*>(src), b = *reinterpret_cast<const f32x4*>(src + 4);
+    lo[0] += a[0]; lo[1] += a[1]; lo[2] += a[2]; lo[3] += a[3];
+    hi[0] += b[0]; hi[1] += b[1]; hi[2] += b[2]; hi[3] += b[3];
+  }
+  u32x4 v;
+  v.x = pack_bf16x2(lo[0], lo[1]); v.y = pack_bf16x2(lo[2], lo[3]);
+  v.z = pack_bf16x2(hi[0], hi[1]); v.w = pack_bf16x2(hi[2], hi[3]);
+  *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+}
+
 }  // namespace spx
 
 using namespace spx;
+
+// compute units of the current device (looked up once per device)
+static int compute_units() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n <= 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
 
 #define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fname, what); } while (0)
 static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
                         int64_t ldc, int64_t M, int64_t N, int64_t K, const int32_t* m_live, void* stream,
                         const int32_t* tile_tab = nullptr, const int32_t* group_off = nullptr,
-                        int64_t b_group_stride = 0, int64_t groups = 0) {
+                        int64_t b_group_stride = 0, int64_t groups = 0, float* part_ws = nullptr,
+                        int max_parts = 1) {
   SPX_REQ_FN(M > 0 && N > 0 && K > 0, "M, N, K must be positive");
   SPX_REQ_FN(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "dimension too large");
   SPX_REQ_FN(a && b && c, "null buffer");
@@ -337,18 +426,28 @@ static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const voi
   const int tiles_n = (int)((N + kTN - 1) / kTN);
   SPX_REQ_FN(tiles_m64 * tiles_n < (1ll << 31), "too many tiles");
   const int tiles_m = (int)tiles_m64;
-  const dim3 grid((unsigned)(tiles_m * tiles_n)), block(kGemmThreads);
+  // (a contraction in parts: room for every part of every tile; the kernel decides how many it uses)
+  SPX_REQ_FN((int64_t)tiles_m * tiles_n * max_parts < (1ll << 31), "too many tiles");
+  const int cus = compute_units();
+  const dim3 grid((unsigned)(tiles_m * tiles_n * (part_ws ? max_parts : 1))), block(kGemmThreads);
   if (imm)
     hipLaunchKernelGGL(gemm_bf16_nt_kernel<true>, grid, block, kGemmSmem, st,
                        reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,
                        reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live,
-                       tile_tab, group_off, b_group_stride);
+                       tile_tab, group_off, b_group_stride, part_ws, max_parts, cus);
   else
     hipLaunchKernelGGL(gemm_bf16_nt_kernel<false>, grid, block, kGemmSmem, st,
                        reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,
                        reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live,
-                       tile_tab, group_off, b_group_stride);
-  return check_launch(fname);
+                       tile_tab, group_off, b_group_stride, part_ws, max_parts, cus);
+  if (int rc = check_launch(fname)) return rc;
+  if (part_ws) {
+    const int64_t items = M * (N / 8);
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, part_ws,
+                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_n, m_live, max_parts, cus);
+    return check_launch(fname);
+  }
+  return 0;
 }
 
 namespace spx {
@@ -416,6 +515,25 @@ extern "C" int spx_gemm_bf16_nt_grouped(const void* a, int64_t lda, const void* 
 extern "C" int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
                                 int64_t ldc, int64_t M, int64_t N, int64_t K, void* stream) {
   return gemm_nt_impl(__func__, a, lda, b, ldb, c, ldc, M, N, K, nullptr, stream);
+}
+
+extern "C" int64_t spx_gemm_split_workspace_bytes(int64_t M, int64_t N, int32_t max_parts) {
+  if (M <= 0 || N <= 0 || max_parts < 1) return 0;
+  return (int64_t)max_parts * M * N * (int64_t)sizeof(float);
+}
+
+extern "C" int spx_gemm_bf16_nt_rows_split(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                                           int64_t ldc, int64_t M, int64_t N, int64_t K, const int32_t* m_live,
+                                           int32_t max_parts, void* workspace, int64_t workspace_bytes,
+                                           void* stream) {
+  const char* fname = __func__;
+  SPX_REQ_FN(max_parts >= 1 && max_parts <= 8, "max_parts must be 1 .. 8");
+  SPX_REQ_FN(N % 8 == 0 && ldc % 8 == 0 && c && ((uintptr_t)c) % 16 == 0,
+             "N and ldc must be multiples of 8 and c 16-byte aligned");
+  SPX_REQ_FN(workspace && ((uintptr_t)workspace) % 16 == 0, "null or unaligned workspace");
+  SPX_REQ_FN(M > 0 && workspace_bytes >= spx_gemm_split_workspace_bytes(M, N, max_parts), "workspace too small");
+  return gemm_nt_impl(fname, a, lda, b, ldb, c, ldc, M, N, K, m_live, stream, nullptr, nullptr, 0, 0,
+                      reinterpret_cast<float*>(workspace), max_parts);
 }
 
 extern "C" int spx_gemm_bf16_nt_rows(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,

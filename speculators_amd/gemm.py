@@ -21,13 +21,22 @@ from . import fused_ops as FO
 _MAX_SPAN = 0x7ffffff0 - 64  # bytes an operand of the weight-gradient product (gemm_tn) may span per call
 
 
+# parts the contraction of a live-rows product may be cut into (gemm_nt(split=True)); 1 = never cut
+SPLIT_PARTS = int(os.environ.get("SPX_GEMM_SPLIT_PARTS", "4"))
+if not 1 <= SPLIT_PARTS <= 8:
+    raise ValueError(f"SPX_GEMM_SPLIT_PARTS must be 1 .. 8, got {SPLIT_PARTS}")
+
+
 def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
-            m_live: torch.Tensor | None = None) -> torch.Tensor:
+            m_live: torch.Tensor | None = None, split: bool = False) -> torch.Tensor:
     """``a[M, K] @ b[N, K].T -> [M, N]`` (bf16, fp32 accumulation).
 
     ``m_live`` (a one-element int32 device tensor) says how many leading rows of ``a`` count:
     the rows from there on are neither read nor written, and the host never learns the
-    number (no synchronisation)."""
+    number (no synchronisation).  ``split``: the kernel may cut the contraction into up to
+    ``SPLIT_PARTS`` parts when the tiles of the rows that count would leave compute units idle
+    (decided on the device from the row count; fp32 partials in a workspace, added in a fixed
+    order)."""
     if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
         raise _lib.SpxError("gemm_nt takes bf16 operands")
     if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
@@ -48,8 +57,16 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
     else:
         if m_live.dtype != torch.int32 or m_live.numel() != 1 or m_live.device != a.device:
             raise ValueError("m_live must be a one-element int32 tensor on the operands' device")
-        _lib.call("spx_gemm_bf16_nt_rows", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
-                  _lib.ptr(out), out.stride(0), m, n, k, _lib.ptr(m_live), st)
+        # (a product of many rounds of tiles has little to gain from cutting: at most 1 / rounds)
+        few_tiles = -(-m // 256) * -(-n // 256) <= 2 * 256
+        if split and SPLIT_PARTS > 1 and few_tiles and n % 8 == 0 and out.stride(0) % 8 == 0 and k >= 64 * 16 * 2:
+            ws = torch.empty(SPLIT_PARTS * m * n, device=a.device, dtype=torch.float32)
+            _lib.call("spx_gemm_bf16_nt_rows_split", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
+                      _lib.ptr(out), out.stride(0), m, n, k, _lib.ptr(m_live), SPLIT_PARTS, _lib.ptr(ws),
+                      ws.numel() * 4, st)
+        else:
+            _lib.call("spx_gemm_bf16_nt_rows", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
+                      _lib.ptr(out), out.stride(0), m, n, k, _lib.ptr(m_live), st)
     return out
 
 

@@ -224,7 +224,7 @@ class _HeadFusedLoss(torch.autograd.Function):
             _lib.ptr(lse_d), _lib.ptr(lse_t), _lib.ptr(extra), _lib.ptr(am_t), _lib.ptr(g), None,
             _lib.ptr(row_map), _lib.ptr(packed), packed.stride(0), _lib.stream_ptr(x.device),
         )
-        dx_packed = gemm_nt(packed, weight_t, m_live=count)
+        dx_packed = gemm_nt(packed, weight_t, m_live=count, split=True)
         return (_unpack_rows(dx_packed, row_map, ctx.total_rows), None, None, None, None, None,
                 None, None, None)
 
@@ -433,7 +433,7 @@ class _HeadLabelCE(torch.autograd.Function):
                   _lib.ptr(lse), _lib.ptr(g), rows, vocab, _lib.dtype_code(logits), ctx.ignore_index,
                   _lib.ptr(row_map), _lib.ptr(packed), packed.stride(0),
                   _lib.stream_ptr(logits.device))
-        dx_packed = gemm_nt(packed, weight_t, m_live=count)
+        dx_packed = gemm_nt(packed, weight_t, m_live=count, split=True)
         return _unpack_rows(dx_packed, row_map, rows), None, None, None, None
 
 

@@ -211,6 +211,76 @@ def test_gemm_nt_with_a_row_count_on_the_device(m, live):
     assert (out[n_live:] == 7).all()
 
 
+def _cu_rounds(tiles, parts, cus=256):
+    return -(-tiles * parts // cus) / parts
+
+
+@pytest.mark.parametrize("m,n,k,live,parts_expected", [
+    (4096, 4096, 4096, 2860, 4),     # 12 x 16 = 192 tiles: three rounds of a quarter instead of one whole
+    (4096, 4096, 4096, 2000, 2),     # 128 tiles: one round of a half
+    (4096, 4096, 4096, 4096, 1),     # 256 tiles: nothing to gain, the direct store
+    (4096, 4096, 4096, 0, 1),        # nothing counts, nothing is written
+    (1200, 520, 6000, 700, 4),       # ragged: 3 x 3 tiles, N not a tile multiple, last part shorter
+    (1200, 520, 1000, 700, 1),       # contraction too short to cut
+])
+def test_gemm_nt_rows_with_the_contraction_in_parts(m, n, k, live, parts_expected):
+    """``gemm_nt(split=True)``: the kernel cuts the contraction when the live rows' tiles leave compute
+    units idle (the count of parts follows from the row count on the device) and adds the fp32 partials
+    in order.  Same rows written as by the plain live-rows product, equal to it up to the rounding of
+    one bf16 value (and to the fp32 product), repeatable bit for bit; dead rows untouched."""
+    from speculators_amd import gemm as G
+
+    tiles = -(-min(live, m) // 256) * -(-n // 256)
+    best = min(range(1, G.SPLIT_PARTS + 1), key=lambda s_: (_cu_rounds(tiles, s_), s_)) if tiles else 1
+    if k // 64 // max(best, 1) < 16 or _cu_rounds(tiles, best) > 0.9 * _cu_rounds(tiles, 1):
+        best = 1
+    assert best == parts_expected  # (the rule the kernel applies, restated for the cases above)
+    g = torch.Generator(device="cuda").manual_seed(m + live)
+    a = torch.randn(m, k, device="cuda", generator=g).bfloat16()
+    b = (torch.randn(n, k, device="cuda", generator=g) * 0.05).bfloat16()
+    n_live = min(live, m)
+    a[n_live:] = float("nan")
+    count = torch.tensor([live], dtype=torch.int32, device="cuda")
+    plain = torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda")
+    G.gemm_nt(a, b, plain, m_live=count)
+    outs = []
+    for _ in range(2):
+        out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda")
+        G.gemm_nt(a, b, out, m_live=count, split=True)
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    assert (outs[0][n_live:] == 7).all()
+    if n_live:
+        ref = a[:n_live].float() @ b.float().t()
+        scale = ref.abs().max().item()
+        assert (outs[0][:n_live].float() - ref).abs().max().item() <= 1e-2 * scale
+        assert (outs[0][:n_live].float() - plain[:n_live].float()).abs().max().item() <= 1e-2 * scale
+        if parts_expected == 1:
+            assert torch.equal(outs[0][:n_live], plain[:n_live])
+
+
+def test_gemm_nt_rows_split_rejects_bad_arguments():
+    from speculators_amd import _lib
+
+    a = torch.zeros(256, 2048, dtype=torch.bfloat16, device="cuda")
+    b = torch.zeros(264, 2048, dtype=torch.bfloat16, device="cuda")
+    c = torch.zeros(256, 264, dtype=torch.bfloat16, device="cuda")
+    cnt = torch.tensor([256], dtype=torch.int32, device="cuda")
+    ws = torch.zeros(4 * 256 * 264, dtype=torch.float32, device="cuda")
+    st = _lib.stream_ptr(a.device)
+
+    def call(parts, ws_bytes, n=264, ldc=264):
+        _lib.call("spx_gemm_bf16_nt_rows_split", _lib.ptr(a), 2048, _lib.ptr(b), 2048, _lib.ptr(c), ldc, 256, n,
+                  2048, _lib.ptr(cnt), parts, _lib.ptr(ws), ws_bytes, st)
+
+    call(4, ws.numel() * 4)
+    assert _lib.load().spx_gemm_split_workspace_bytes(256, 264, 4) == 4 * 256 * 264 * 4
+    for bad in (dict(parts=0, ws_bytes=ws.numel() * 4), dict(parts=9, ws_bytes=ws.numel() * 4),
+                dict(parts=4, ws_bytes=ws.numel() * 4 - 1), dict(parts=4, ws_bytes=ws.numel() * 4, n=260)):
+        with pytest.raises(_lib.SpxError):
+            call(**bad)
+
+
 @pytest.mark.parametrize("t,m,n", [(8192, 264, 136), (5000, 512, 512), (20000, 8, 1024)])
 @pytest.mark.parametrize("fp32", [False, True])
 def test_gemm_tn_small_result_long_contraction(t, m, n, fp32):
