@@ -312,3 +312,41 @@ def test_reused_target_statistics_give_the_same_rows(op_name):
     go = torch.randn_like(fresh)
     (fresh * go).sum().backward(); (reused * go).sum().backward()
     torch.testing.assert_close(b.grad.float(), a.grad.float(), atol=1e-6, rtol=1e-3)
+
+
+@pytest.mark.parametrize("live_fraction", [0.15, 0.45, 1.0])
+def test_head_and_loss_node_with_the_input_gradient_in_parts(live_fraction, monkeypatch):
+    """The frozen head + loss node over a sparse loss mask: its input-gradient product runs over the
+    packed live rows and, when their tiles are few, with the contraction cut into parts
+    (``spx_gemm_bf16_nt_rows_split``).  Against the same node with the cut switched off (one rounding of
+    a bf16 value apart) and against autograd through the fp32 oracle loss; dead rows get exact zeros."""
+    from speculators_amd import gemm as G
+    from speculators_amd import losses as L
+
+    t, h, vd = 1024, 512, 4096
+    g = torch.Generator().manual_seed(int(live_fraction * 100))
+    x = (torch.randn(1, t, h, generator=g) * 0.5).bfloat16()
+    w = (torch.randn(vd, h, generator=g) * 0.05).bfloat16()
+    tg = (torch.randn(1, t, vd, generator=g) * 2).bfloat16()
+    mask = (torch.rand(1, t, generator=g) < live_fraction).float()
+    grads = {}
+    for parts in (4, 1):
+        monkeypatch.setattr(G, "SPLIT_PARTS", parts)
+        xg = x.cuda().requires_grad_(True)
+        wc = w.cuda()
+        loss = L.head_fused_rows(L.OP_KL, xg, wc, wc.t().contiguous(), tg.cuda())[0]
+        (loss * mask.cuda()).sum().backward()
+        grads[parts] = xg.grad.float().cpu()
+    xr = x.float().requires_grad_(True)
+    # (the oracle sees the logits the kernel sees: rounded to bf16, gradient straight through)
+    logits = xr @ w.float().t()
+    logits = logits + (logits.detach().bfloat16().float() - logits.detach())
+    ref = OL.kl_div(logits, tg.float())
+    (ref * mask).sum().backward()
+    want = xr.grad
+    scale = want.abs().max().item()
+    dead = mask[0] == 0
+    for parts in (4, 1):
+        assert (grads[parts][0][dead] == 0).all()
+        assert (grads[parts] - want).abs().max().item() <= 2e-2 * scale + 1e-6, parts
+    assert (grads[4] - grads[1]).abs().max().item() <= 1e-2 * scale + 1e-6
