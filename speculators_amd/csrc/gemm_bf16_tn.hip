@@ -9,17 +9,21 @@
 // operand goes global -> LDS directly (buffer_load ... lds, whole 512-byte rows), exactly as it
 // lies in memory, and the fragments are taken with the transposing LDS read of gfx950
 // (ds_read_b64_tr_b16: inside every group of 16 lanes, lane 4u + w receives as element j element
-// w of the 8 bytes lane 4j + u points at).  Two such reads make one 32 x 16 operand fragment:
-// lane (G = lane / 16, s = lane % 16) points at row 8 (G / 2) + s / 4 (+ 4 for the second read) of
-// the 16-row K step and at bytes 32 (G % 2) + 8 (s % 4) of the fragment's 64-byte column block.
-// Bank conflicts: the rows of a slab are 512 bytes apart, so the 64-byte block b of row t sits at
-// block position b ^ (t % 4): the 4 + 4 rows one read touches then fall into four different
-// 64-byte bank groups, two rows each, which is the minimum for 512 bytes.
+// w of the 8 bytes lane 4j + u points at).  Two such reads make one 16 x 32 operand fragment of
+// v_mfma_f32_16x16x32_bf16: lane (G = lane / 16, s = lane % 16) points at row 8 G + s / 4 (+ 4 for
+// the second read) of the 32-row K step and at bytes 8 (s % 4) of the fragment's 32-byte column
+// block, and ends up with rows 8 G .. 8 G + 7 of column s.
+// Bank conflicts: the rows of a slab are 512 bytes apart, so the 32-byte piece p of row t sits at
+// piece position p ^ h(t), h(t) = t % 4 + 4 (t / 8 % 2): the 8 rows that one half of the lanes of a
+// read touches then cover all 64 banks once.
 //
 // From there on it is the NT kernel: 256 x 256 tile, 4 waves x 128 x 128 (one per SIMD), two
-// slab buffers, v_mfma_f32_32x32x16_bf16, the LDS reads of K step kk+1 and the global loads of
-// the next slab issued one at a time between the MFMAs of step kk, one barrier per slab,
-// accumulators kept transposed (lane = row of C).
+// slab buffers, 8 x 8 accumulators of 16 x 16 per wave pinned to the accumulation registers, the LDS
+// reads of K step kk+1 and the global loads of the next slab issued one at a time between the MFMAs
+// of step kk, one barrier per slab, accumulators kept transposed (lane = row of C).  The slab loop is
+// written out for two slabs, so that the buffer a read goes to is a constant: a fragment read is an
+// address register per fragment plus an immediate, with no vector arithmetic between the MFMAs
+// (with 16-cycle MFMAs the kernel is bound by what a wave can issue, and every instruction counts).
 
 #include "spx_common.h"
 #include "../../include/spx.h"
@@ -31,7 +35,14 @@ namespace tn {
 constexpr int kNW = 4, kThreads = 256;
 constexpr int kTM = 256, kTN = 256, kTK = 64;
 constexpr int kWM = 2, kWN = 2;
-constexpr int kMI = kTM / kWM / 32, kNI = kTN / kWN / 32;  // 4 x 4 accumulators of 32 x 32 per wave
+constexpr int kMI = kTM / kWM / 16, kNI = kTN / kWN / 16;  // 8 x 8 accumulators of 16 x 16 per wave
+constexpr int kKSteps = kTK / 32;                          // MFMA K steps per slab
+#ifndef SPX_GEMM_TN_READ_EVERY
+#define SPX_GEMM_TN_READ_EVERY 2  // MFMAs per LDS fragment (two transposing reads) in the K step before the barrier
+#endif
+#ifndef SPX_GEMM_TN_READ_EVERY_B
+#define SPX_GEMM_TN_READ_EVERY_B 4  // the same in the K step after it, which also issues the global loads
+#endif
 constexpr int kRowBytes = kTM * 2;                          // 512: one t-row of a slab
 constexpr int kABytes = kTK * kRowBytes;                    // one slab of A: 32 KB
 constexpr int kBBytes = kABytes;
@@ -42,17 +53,18 @@ constexpr int kLB = kLA;
 constexpr int kL = kLA + kLB;
 constexpr int kOob = 0x7ffffff0;
 static_assert(kTM == kTN, "both operands use one slab layout");
-static_assert(kABytes == 32768, "the buffer toggle flips bit 15");
+static_assert(kABytes + (kKSteps - 1) * 32 * kRowBytes + 4 * kRowBytes < 65536,
+              "slab buffer, K step and row pair of a fragment read go into the 16-bit offset field");
 #ifndef SPX_GEMM_TN_GROUP_M
 #define SPX_GEMM_TN_GROUP_M 8
 #endif
 
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef short i16x8 __attribute__((ext_vector_type(8)));
-__device__ __forceinline__ i16x4 lds_read_tr16(const uint8_t* p) {
-  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-      (__attribute__((address_space(3))) i16x4*)(uintptr_t)(uint32_t)(uintptr_t)(
-          (__attribute__((address_space(3))) const uint8_t*)p));
+// transposing read at a 32-bit LDS address (base included): a constant added to it goes into the
+// offset field of the instruction
+__device__ __forceinline__ i16x4 lds_read_tr16_at(uint32_t addr) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(uintptr_t)addr);
 }
 
 // OUT: 0 = bf16 result, 1 = bf16 result added to C, 2 = fp32 result, 3 = fp32 result added to C
@@ -121,17 +133,17 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int g = lane >> 5, col = lane & 31;
+  const int q = lane >> 4, r16 = lane & 15;
   const int wm = (wave / kWN) * (kTM / kWM), wn = (wave % kWN) * (kTN / kWN);
 
-  // acc[j][i]: registers = 32 columns of C at wn + 32 j, lane = row of C at wm + 32 i
-  f32x16 acc[kNI][kMI];
+  // acc[j][i]: lane = row wm + 16 i + lane % 16 of C, registers = columns wn + 16 j + 4 (lane / 16) + {0..3}
+  f32x4 acc[kNI][kMI];
 #pragma unroll
   for (int j = 0; j < kNI; ++j)
 #pragma unroll
     for (int i = 0; i < kMI; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[j][i][r] = 0.f;
+      for (int r = 0; r < 4; ++r) acc[j][i][r] = 0.f;
 
   // One buffer resource per operand, starting at the tile's first column.  The whole offset of a load,
   // the slab's first row included, is in the vector register, which is what the range check sees: rows
@@ -141,14 +153,15 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
   u32x4 bres = make_rsrc(B + n0, T > 0 ? (uint32_t)((((int64_t)T - 1) * ldb + min(N - n0, kTN)) * 2) : 0u);
 
   // global side: wave-load j of this wave covers slab rows 2 (wave * kLA + j) + lane / 32; the lane's LDS
-  // position is 16-byte chunk lane % 32 of the row, which holds the chunk of 64-byte block
-  // (position / 4) ^ (row % 4)
+  // position is 16-byte chunk lane % 32 of the row, which holds a chunk of the 32-byte piece
+  // (position / 2) ^ h(row)
   const int lrow = lane >> 5, lpos = lane & 31;
   int aoff[kLA], boff[kLB];
 #pragma unroll
   for (int j = 0; j < kLA; ++j) {
     const int r = 2 * (wave * kLA + j) + lrow;
-    const int c8 = ((((lpos >> 2) ^ (r & 3)) << 2) | (lpos & 3)) * 8;  // first column of the chunk
+    const int hr = (r & 3) | (((r >> 3) & 1) << 2);
+    const int c8 = ((((lpos >> 1) ^ hr) << 1) | (lpos & 1)) * 8;  // first column of the chunk
     aoff[j] = (m0 + c8 < M) ? (int)(((int64_t)r * lda + c8) * 2) : kOob;
     boff[j] = (n0 + c8 < N) ? (int)(((int64_t)r * ldb + c8) * 2) : kOob;
   }
@@ -189,25 +202,29 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
   };
 
   // read side (see the head of the file)
-  const int tG = lane >> 4, ts = lane & 15;
-  const int trow = 8 * (tG >> 1) + (ts >> 2);
-  const int lane_off = trow * kRowBytes + ((ts >> 2) & 3) * 64 + 32 * (tG & 1) + 8 * (ts & 3);
-  uint32_t a_rd[kMI], b_rd[kNI];  // per fragment; bit 15 selects the slab buffer
+  const int trow = 8 * q + (r16 >> 2);
+  const int lane_off = trow * kRowBytes + (((r16 >> 2) | ((q & 1) << 2)) * 32) + 8 * (r16 & 3);
+  uint32_t a_rd[kMI], b_rd[kNI];  // per fragment: LDS address in slab buffer 0
 #pragma unroll
   for (int f = 0; f < kMI; ++f) {
-    a_rd[f] = lane_off ^ ((wm / 32 + f) * 64);
-    b_rd[f] = kBBase + (lane_off ^ ((wn / 32 + f) * 64));
+    a_rd[f] = lds0 + (lane_off ^ ((wm / 16 + f) * 32));
+    b_rd[f] = lds0 + kBBase + (lane_off ^ ((wn / 16 + f) * 32));
+    // (kept opaque: otherwise the B operand's 64 KB base is folded out of the register into the
+    // constant and no longer fits the offset field)
+    asm volatile("" : "+v"(a_rd[f]), "+v"(b_rd[f]));
   }
 
   i16x4 fa[2][kMI][2], fb[2][kNI][2];
-  // operand fragment f (A fragments first, then B) of K step kk into register set `set`
-  auto read_one = [&](int set, int kk, int f) __attribute__((always_inline)) {
+  // operand fragment f (A fragments first, then B) of K step kk of slab buffer buf into register
+  // set `set`; buf and kk are constants where this is called, so they end up in the offset field
+  auto read_one = [&](int set, int buf, int kk, int f) __attribute__((always_inline)) {
+    const uint32_t o = buf * kABytes + kk * 32 * kRowBytes;
     if (f < kMI) {
-      fa[set][f][0] = lds_read_tr16(smem + a_rd[f] + kk * 16 * kRowBytes);
-      fa[set][f][1] = lds_read_tr16(smem + a_rd[f] + kk * 16 * kRowBytes + 4 * kRowBytes);
+      fa[set][f][0] = lds_read_tr16_at(a_rd[f] + o);
+      fa[set][f][1] = lds_read_tr16_at(a_rd[f] + o + 4 * kRowBytes);
     } else {
-      fb[set][f - kMI][0] = lds_read_tr16(smem + b_rd[f - kMI] + kk * 16 * kRowBytes);
-      fb[set][f - kMI][1] = lds_read_tr16(smem + b_rd[f - kMI] + kk * 16 * kRowBytes + 4 * kRowBytes);
+      fb[set][f - kMI][0] = lds_read_tr16_at(b_rd[f - kMI] + o);
+      fb[set][f - kMI][1] = lds_read_tr16_at(b_rd[f - kMI] + o + 4 * kRowBytes);
     }
   };
   auto frag = [&](const i16x4 (&h)[2]) __attribute__((always_inline)) {
@@ -216,18 +233,18 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
   };
   // One K step: the kNI x kMI MFMAs on register set `set`; between them, one at a time, the LDS
   // reads that fill the other set with K step rk and the global loads [l0, l0 + nl).
-  auto step = [&](int set, int rk, int l0, int nl) __attribute__((always_inline)) {
+  auto step = [&](int set, int rbuf, int rk, int l0, int nl, int every) __attribute__((always_inline)) {
     constexpr int kN = kNI * kMI, kF = kMI + kNI;
     int reads = 0, loads = 0;
 #pragma unroll
     for (int j = 0; j < kNI; ++j)
 #pragma unroll
       for (int i = 0; i < kMI; ++i) {
-        acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(fb[set][j]), frag(fa[set][i]), acc[j][i], 0, 0, 0);
+        mfma16(acc[j][i], frag(fb[set][j]), frag(fa[set][i]));
         const int idx = j * kMI + i;
         __builtin_amdgcn_sched_barrier(0);
-        if (reads < kF) {
-          read_one(set ^ 1, rk, reads++);
+        if (reads < kF && idx % every == every - 1) {
+          read_one(set ^ 1, rbuf, rk, reads++);
           __builtin_amdgcn_sched_barrier(0);
         }
         if (nl > 0 && (nl >= kN || idx % (kN / nl) == kN / nl - 1) && loads < nl) {
@@ -237,23 +254,21 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
       }
   };
 
-  // the loads of a slab are spread over the step after the barrier (kLdT of them) and step 0 of the
-  // next slab (the rest); steps 1 and 2 give them time to land
-  constexpr int kLdT = kL / 2, kLd0 = kL - kLdT;
-  auto slab = [&]() __attribute__((always_inline)) {
+  // the loads of a slab are issued in the step after the barrier that frees its buffer, one per four
+  // MFMAs; the step after that gives them time to land
+  static_assert(kKSteps == 2, "a slab is two K steps: one before, one after the barrier");
+  constexpr int kLdT = kL;
+  // buf: the buffer slab s lies in, a constant in each of the two copies of the loop body
+  auto slab = [&](int buf) __attribute__((always_inline)) {
     __builtin_amdgcn_sched_barrier(0);
-    step(0, 1, kLdT, kLd0);
+    step(0, buf, 1, 0, 0, SPX_GEMM_TN_READ_EVERY);
     next_slab();
-    step(1, 2, 0, 0);
-    step(0, 3, 0, 0);
     // every read of this slab's buffer has returned once set 1 is complete; then the barrier says:
     // slab s+1 has landed for everybody, this buffer is free
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
-#pragma unroll
-    for (int f = 0; f < kMI; ++f) { a_rd[f] ^= kABytes; b_rd[f] ^= kBBytes; }
-    // K step 3 of slab s, under it the reads of step 0 of slab s+1 and the first loads of slab s+2
-    step(1, 0, 0, kLdT);
+    // K step 1 of slab s, under it the reads of step 0 of slab s+1 and the loads of slab s+2
+    step(1, buf ^ 1, 0, 0, kLdT, SPX_GEMM_TN_READ_EVERY_B);
   };
 
   const int nslab = MULTI ? total_slabs : (T + kTK - 1) / kTK;
@@ -266,106 +281,101 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
 #pragma unroll
   for (int l = 0; l < kLdT; ++l) issue_one(l);
 #pragma unroll
-  for (int f = 0; f < kMI + kNI; ++f) read_one(0, 0, f);
-  for (int s = 0; s < nslab; ++s) slab();
+  for (int f = 0; f < kMI + kNI; ++f) read_one(0, 0, 0, f);
+  int s = 0;
+  for (; s + 1 < nslab; s += 2) {
+    slab(0);
+    slab(1);
+  }
+  if (s < nslab) slab(0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-  // epilogue: a lane holds row m of C and, per accumulator, columns 8 q + 4 g + {0..3} (q = 0..3)
+  mfma_results_ready();
+  // epilogue: a lane holds row m of C and, per accumulator, columns 4 q + {0..3} of a 16-column block
   if constexpr (OUT >= 2) {
     float* const C = reinterpret_cast<float*>(Cv);
     const bool fast = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0) && (n0 + kTN <= N);
 #pragma unroll
     for (int i = 0; i < kMI; ++i) {
-      const int m = m0 + wm + i * 32 + col;
+      const int m = m0 + wm + i * 16 + r16;
       if (m >= M) continue;
 #pragma unroll
       for (int j = 0; j < kNI; ++j) {
-        const f32x16& a = acc[j][i];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = n0 + wn + j * 32 + 8 * q + 4 * g;
-          float* cp = C + (int64_t)m * ldc + n;
-          if (fast) {
-            f32x4 v = {a[4 * q + 0], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
-            if (OUT == 3) {
-              const f32x4 old = *reinterpret_cast<const f32x4*>(cp);
-              v[0] += old[0]; v[1] += old[1]; v[2] += old[2]; v[3] += old[3];
-            }
-            *reinterpret_cast<f32x4*>(cp) = v;
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (n + e < N) cp[e] = (OUT == 3 ? cp[e] : 0.f) + a[4 * q + e];
+        const f32x4& a = acc[j][i];
+        const int n = n0 + wn + j * 16 + 4 * q;
+        float* cp = C + (int64_t)m * ldc + n;
+        if (fast) {
+          f32x4 v = a;
+          if (OUT == 3) {
+            const f32x4 old = *reinterpret_cast<const f32x4*>(cp);
+            v[0] += old[0]; v[1] += old[1]; v[2] += old[2]; v[3] += old[3];
           }
+          *reinterpret_cast<f32x4*>(cp) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < N) cp[e] = (OUT == 3 ? cp[e] : 0.f) + a[e];
         }
       }
     }
     return;
   } else {
-    // Swapping the q-odd words of the lower half-wave with the q-even words of the upper half-wave
-    // leaves every lane with 8 consecutive columns: 16-byte stores.
+    // Swapping the words of the q-odd lanes for block j with those of the q-even lanes for block j + 1
+    // (v_permlane16_swap) leaves every lane with 8 consecutive columns: 16-byte stores.
     uint16_t* const C = reinterpret_cast<uint16_t*>(Cv);
     constexpr bool ACC = OUT == 1;
     const bool fast = (ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0) && (n0 + kTN <= N);
 #pragma unroll
     for (int i = 0; i < kMI; ++i) {
-      const int m = m0 + wm + i * 32 + col;
+      const int m = m0 + wm + i * 16 + r16;
 #pragma unroll
-      for (int j = 0; j < kNI; ++j) {
-        f32x16 a = acc[j][i];
+      for (int j = 0; j < kNI; j += 2) {
+        f32x4 a = acc[j][i], b = acc[j + 1][i];
+        // q even: columns 4 q + 0..7 of block j; q odd: columns 4 (q - 1) + 0..7 of block j + 1
+        const int n = n0 + wn + (j + (q & 1)) * 16 + 4 * (q & 2);
         if (ACC && fast) {
           // swap the fp32 words, add what C holds (one 16-byte load per lane, the store's own layout)
+          float v[8];
 #pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            float v[8];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(a[8 * h + e]),
-                                                              __float_as_uint(a[8 * h + 4 + e]), false, false);
-              v[e] = __uint_as_float(sw[0]);
-              v[4 + e] = __uint_as_float(sw[1]);
-            }
-            const int n = n0 + wn + j * 32 + 16 * h + 8 * g;
-            if (m < M) {
-              u32x4* cp = reinterpret_cast<u32x4*>(&C[(int64_t)m * ldc + n]);
-              const u32x4 old = *cp;
-              u32x4 o;
-              o.x = pack_bf16x2(v[0] + bf16_lo(old.x), v[1] + bf16_hi(old.x));
-              o.y = pack_bf16x2(v[2] + bf16_lo(old.y), v[3] + bf16_hi(old.y));
-              o.z = pack_bf16x2(v[4] + bf16_lo(old.z), v[5] + bf16_hi(old.z));
-              o.w = pack_bf16x2(v[6] + bf16_lo(old.w), v[7] + bf16_hi(old.w));
-              *cp = o;
-            }
+          for (int e = 0; e < 4; ++e) {
+            const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(a[e]), __float_as_uint(b[e]), false, false);
+            v[e] = __uint_as_float(sw[0]);
+            v[4 + e] = __uint_as_float(sw[1]);
+          }
+          if (m < M) {
+            u32x4* cp = reinterpret_cast<u32x4*>(&C[(int64_t)m * ldc + n]);
+            const u32x4 old = *cp;
+            u32x4 o;
+            o.x = pack_bf16x2(v[0] + bf16_lo(old.x), v[1] + bf16_hi(old.x));
+            o.y = pack_bf16x2(v[2] + bf16_lo(old.y), v[3] + bf16_hi(old.y));
+            o.z = pack_bf16x2(v[4] + bf16_lo(old.z), v[5] + bf16_hi(old.z));
+            o.w = pack_bf16x2(v[6] + bf16_lo(old.w), v[7] + bf16_hi(old.w));
+            *cp = o;
           }
           continue;
         }
         if (ACC && m < M) {
-          // ragged edge: what C holds, read in the accumulator's own layout (4 consecutive columns per q)
+          // ragged edge: what C holds, read in the accumulators' own layout (4 consecutive columns each)
+          const int na = n0 + wn + j * 16 + 4 * q;
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int n = n0 + wn + j * 32 + 8 * q + 4 * g;
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (n + e < N) a[4 * q + e] += bf16_bits_to_f32(C[(int64_t)m * ldc + n + e]);
+          for (int e = 0; e < 4; ++e) {
+            if (na + e < N) a[e] += bf16_bits_to_f32(C[(int64_t)m * ldc + na + e]);
+            if (na + 16 + e < N) b[e] += bf16_bits_to_f32(C[(int64_t)m * ldc + na + 16 + e]);
           }
         }
+        const uint32_t e0 = pack_bf16x2(a[0], a[1]), e1 = pack_bf16x2(a[2], a[3]);
+        const uint32_t o0 = pack_bf16x2(b[0], b[1]), o1 = pack_bf16x2(b[2], b[3]);
+        const auto s0 = __builtin_amdgcn_permlane16_swap(e0, o0, false, false);
+        const auto s1 = __builtin_amdgcn_permlane16_swap(e1, o1, false, false);
+        u32x4 v;
+        v.x = s0[0]; v.y = s1[0]; v.z = s0[1]; v.w = s1[1];
+        if (fast) {
+          if (m < M) *reinterpret_cast<u32x4*>(&C[(int64_t)m * ldc + n]) = v;
+        } else if (m < M) {
+          const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {  // q pair (2h, 2h+1)
-          const uint32_t e0 = pack_bf16x2(a[8 * h + 0], a[8 * h + 1]), e1 = pack_bf16x2(a[8 * h + 2], a[8 * h + 3]);
-          const uint32_t o0 = pack_bf16x2(a[8 * h + 4], a[8 * h + 5]), o1 = pack_bf16x2(a[8 * h + 6], a[8 * h + 7]);
-          const auto s0 = __builtin_amdgcn_permlane32_swap(e0, o0, false, false);
-          const auto s1 = __builtin_amdgcn_permlane32_swap(e1, o1, false, false);
-          u32x4 v;
-          v.x = s0[0]; v.y = s1[0]; v.z = s0[1]; v.w = s1[1];
-          const int n = n0 + wn + j * 32 + 16 * h + 8 * g;
-          if (fast) {
-            if (m < M) *reinterpret_cast<u32x4*>(&C[(int64_t)m * ldc + n]) = v;
-          } else if (m < M) {
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-              if (n + e < N) C[(int64_t)m * ldc + n + e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
-          }
+          for (int e = 0; e < 8; ++e)
+            if (n + e < N) C[(int64_t)m * ldc + n + e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
         }
       }
     }

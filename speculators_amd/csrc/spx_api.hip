@@ -41,6 +41,6 @@ int ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& don
 
 }  // namespace spx
 
-extern "C" int spx_version(void) { return 111; }
+extern "C" int spx_version(void) { return 112; }
 
 extern "C" const char* spx_last_error(void) { return spx::last_error().c_str(); }
