@@ -481,6 +481,21 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
   // fragment reads of mode 2: byte offsets of this lane's row and chunk (step 0) inside a tile
   const int rdk = col * RBK + ((g ^ swz_k(col)) * 16);
   const int rdv = col * 128 + ((g ^ swz_v(col)) * 16);
+  // The fragment reads as LDS addresses, one register per swizzle term, kept opaque to the
+  // compiler: what is added to them per read (buffer, key half, D block) is a constant and goes
+  // into the offset field.  Formed on the symbol of the dynamic array instead, every read costs a
+  // vector add of that link-time constant.
+  uint32_t krd[NKK], vrd[4];
+#pragma unroll
+  for (int j = 0; j < NKK; ++j) {
+    krd[j] = lds0 + (uint32_t)(rdk ^ (j * 32));
+    asm volatile("" : "+v"(krd[j]));
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    vrd[j] = lds0 + (uint32_t)(SM::kTileK + (rdv ^ (j * 32)));
+    asm volatile("" : "+v"(vrd[j]));
+  }
 
   // one pass over the key tiles of one interval class.  The tile loop is unrolled over the two tile
   // buffers: the buffer is then a compile-time constant and the fragment reads address it through
@@ -523,8 +538,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         bf16x8 kfr[RG];
         auto kread = [&](int f) {
           if constexpr (PF == 2)
-            kfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-                tk + (f & 1) * 32 * RBK + (rdk ^ ((f >> 1) * 32))));
+            kfr[f % RG] = as_bf16x8(lds_read128(krd[f >> 1] + buf * SM::kBuf + (f & 1) * 32 * RBK));
           else
             kfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 &Ks[((f & 1) * 32 + col) * KS + g * 8 + (f >> 1) * 16]));
@@ -611,8 +625,7 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         bf16x8 vfr[RG];
         auto vread = [&](int f) {
           if constexpr (PF == 2)
-            vfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
-                tv + (f % NDB) * 32 * 128 + (rdv ^ ((f / NDB) * 32))));
+            vfr[f % RG] = as_bf16x8(lds_read128(vrd[f / NDB] + buf * SM::kBuf + (f % NDB) * 32 * 128));
           else
             vfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 &Vs[((f % NDB) * 32 + col) * VS + (f / NDB) * 16 + 8 * g]));

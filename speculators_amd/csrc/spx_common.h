@@ -63,6 +63,12 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return c.u;
 }
 
+// 16-byte LDS read at a 32-bit LDS address; a constant added to the address goes into the offset
+// field of the instruction
+__device__ __forceinline__ u32x4 lds_read128(uint32_t addr) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>((uintptr_t)addr);
+}
+
 // acc += a * b with v_mfma_f32_16x16x32_bf16, the accumulator pinned to the accumulation registers
 // and written in place.  (With 64 accumulator tuples that fill that register file, the compiler's own
 // choice of destination leaves them permuted at the end of a loop body and moves them back through
