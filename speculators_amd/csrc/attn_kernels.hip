@@ -485,16 +485,21 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
   // compiler: what is added to them per read (buffer, key half, D block) is a constant and goes
   // into the offset field.  Formed on the symbol of the dynamic array instead, every read costs a
   // vector add of that link-time constant.
-  uint32_t krd[NKK], vrd[4];
+  // Only where both tile buffers lie inside the 64 KB an offset field reaches (head_dim <= 128); past
+  // that the constants need an add again and the registers are better left to the accumulators.
+  constexpr bool kAbsRd = PF == 2 && 2 * SM::kBuf <= 65536;
+  uint32_t krd[kAbsRd ? NKK : 1], vrd[kAbsRd ? 4 : 1];
+  if constexpr (kAbsRd) {
 #pragma unroll
-  for (int j = 0; j < NKK; ++j) {
-    krd[j] = lds0 + (uint32_t)(rdk ^ (j * 32));
-    asm volatile("" : "+v"(krd[j]));
-  }
+    for (int j = 0; j < NKK; ++j) {
+      krd[j] = lds0 + (uint32_t)(rdk ^ (j * 32));
+      asm volatile("" : "+v"(krd[j]));
+    }
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    vrd[j] = lds0 + (uint32_t)(SM::kTileK + (rdv ^ (j * 32)));
-    asm volatile("" : "+v"(vrd[j]));
+    for (int j = 0; j < 4; ++j) {
+      vrd[j] = lds0 + (uint32_t)(SM::kTileK + (rdv ^ (j * 32)));
+      asm volatile("" : "+v"(vrd[j]));
+    }
   }
 
   // one pass over the key tiles of one interval class.  The tile loop is unrolled over the two tile
@@ -537,8 +542,11 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         constexpr int RG = SPX_FWD_RING;
         bf16x8 kfr[RG];
         auto kread = [&](int f) {
-          if constexpr (PF == 2)
+          if constexpr (kAbsRd)
             kfr[f % RG] = as_bf16x8(lds_read128(krd[f >> 1] + buf * SM::kBuf + (f & 1) * 32 * RBK));
+          else if constexpr (PF == 2)
+            kfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                tk + (f & 1) * 32 * RBK + (rdk ^ ((f >> 1) * 32))));
           else
             kfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 &Ks[((f & 1) * 32 + col) * KS + g * 8 + (f >> 1) * 16]));
@@ -624,8 +632,11 @@ __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_
         constexpr int RG = SPX_FWD_RING;
         bf16x8 vfr[RG];
         auto vread = [&](int f) {
-          if constexpr (PF == 2)
+          if constexpr (kAbsRd)
             vfr[f % RG] = as_bf16x8(lds_read128(vrd[f / NDB] + buf * SM::kBuf + (f % NDB) * 32 * 128));
+          else if constexpr (PF == 2)
+            vfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
+                tv + (f % NDB) * 32 * 128 + (rdv ^ ((f / NDB) * 32))));
           else
             vfr[f % RG] = as_bf16x8(*reinterpret_cast<const u32x4*>(
                 &Vs[((f % NDB) * 32 + col) * VS + (f / NDB) * 16 + 8 * g]));
