@@ -7,9 +7,12 @@ mapping, with the first-layer changes of ``Eagle3FirstLayerMixin``
 Llama blocks it is built from (RMSNorm fp32-inside, half-split RoPE computed in
 fp32 and cast, SwiGLU MLP, K/V cache that grows by T keys per step).
 
-Pinned by: agreement with the HF ``LlamaDecoderLayer`` / ``LlamaRotaryEmbedding``
-library modules patched the way the reference patches them
-(tests/test_oracle_eagle3.py), agreement of the dense-mask attention with
+Pinned by (tests/test_oracle_eagle3.py): ``first_layer`` == the HF ``LlamaAttention`` /
+``LlamaMLP`` / ``LlamaRMSNorm`` / ``LlamaRotaryEmbedding`` modules patched the way the
+reference patches them, and with ``qk_norm`` == ``Qwen3Attention`` (q/k RMSNorm before the
+rotation) wired the same way; ``later_layer`` == the library's whole ``LlamaDecoderLayer`` /
+``Qwen3DecoderLayer`` over three TTT steps on one ``DynamicCache`` (output and every
+gradient); agreement of the dense-mask attention with
 ``F.scaled_dot_product_attention``, the reference's mask / loss / metric golden
 vectors through the modules it calls, and shift / alignment invariants
 (step-k rows only see targets k positions later).  The whole-model loss on

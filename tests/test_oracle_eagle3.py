@@ -275,3 +275,176 @@ def test_fixed_rope_types_never_read_the_positions():
         assert not r.by_length and r.top(None) is None
         assert r.select("cpu") is r.select("cpu", None, 5)
         assert torch.equal(r.select("cpu"), E.rope_inv_freq(64, 10000.0, scaling))
+
+
+# ---------------------------------------------------------------- layers after the first, q/k norm
+def _randomise_gains(w, seed):
+    g = torch.Generator().manual_seed(seed)
+    for name in list(w):
+        if name.endswith("norm.weight") or "layernorm" in name:
+            w[name] = 1 + 0.2 * torch.randn(w[name].shape, generator=g)
+    return w
+
+
+def _ttt_batch(t, docs, pad):
+    doc = torch.tensor(sum(([i] * n for i, n in enumerate(docs)), []) + [-1] * pad)
+    pos = torch.cat([1 + torch.arange(n) for n in docs] + [torch.zeros(pad, dtype=torch.long)]).unsqueeze(0)
+    assert doc.numel() == t
+    return doc, pos
+
+
+def _additive(mask):
+    return torch.zeros(1, 1, *mask.shape).masked_fill(~mask[None, None], float("-inf"))
+
+
+@pytest.mark.parametrize("family", ["llama", "qwen3"])
+def test_later_layer_equals_hf_decoder_layer(family):
+    """``later_layer`` (every EAGLE3 layer after the first: models/eagle3/core.py:286-300 runs the
+    unpatched ``decoder_layer_class`` of models/base_components.py:39-52) against the library's own
+    ``LlamaDecoderLayer`` / ``Qwen3DecoderLayer`` -- classes used whole, nothing wired here -- over
+    three TTT steps sharing one ``DynamicCache``, packed documents plus padding, a windowed mask,
+    random norm gains.  Output and the gradient of the input and of every parameter."""
+    from transformers import DynamicCache, LlamaConfig, Qwen3Config
+    from transformers.models.llama.modeling_llama import LlamaDecoderLayer, LlamaRotaryEmbedding
+    from transformers.models.qwen3.modeling_qwen3 import Qwen3DecoderLayer, Qwen3RotaryEmbedding
+
+    qk = family == "qwen3"
+    shape = _tiny_shape(num_hidden_layers=2, qk_norm=qk)
+    w = _randomise_gains(E.random_weights(shape, seed=11, std=0.2), 12)
+    common = dict(hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+                  intermediate_size=128, vocab_size=128, rms_norm_eps=1e-6, num_hidden_layers=2,
+                  attention_bias=False,
+                  rope_parameters={"rope_type": "default", "rope_theta": 10000.0})
+    if qk:
+        cfg = Qwen3Config(**common, layer_types=["full_attention"] * 2, sliding_window=None)
+        layer, rot = Qwen3DecoderLayer(cfg, 1), Qwen3RotaryEmbedding(cfg)
+    else:
+        cfg = LlamaConfig(**common)
+        layer, rot = LlamaDecoderLayer(cfg, 1), LlamaRotaryEmbedding(cfg)
+    cfg._attn_implementation = "eager"
+    layer.self_attn.config._attn_implementation = "eager"
+    p = "layers.1."
+    names = {n: prm for n, prm in layer.named_parameters()}
+    assert set(names) == {k[len(p):] for k in w if k.startswith(p)}
+    for n, prm in names.items():
+        prm.data.copy_(w[p + n])
+    wl = {k: v.clone().requires_grad_(True) for k, v in w.items() if k.startswith(p)}
+
+    t = 20
+    doc, pos = _ttt_batch(t, [8, 9], 3)
+    g = torch.Generator().manual_seed(13)
+    xs = [torch.randn(1, t, 64, generator=g) for _ in range(3)]
+    xs_hf = [x.clone().requires_grad_(True) for x in xs]
+    xs_or = [x.clone().requires_grad_(True) for x in xs]
+    cache_hf, cache_or = DynamicCache(), {}
+    probe = torch.randn(3, 1, t, 64, generator=g)
+    total_hf = total_or = 0.0
+    for step in range(3):
+        mask = M.ttt_mask_dense(doc, t, step, sliding_window=5)
+        cos, sin = rot(xs[step], pos + step)
+        ref = layer(xs_hf[step], attention_mask=_additive(mask), position_ids=pos + step,
+                    past_key_values=cache_hf, use_cache=True, position_embeddings=(cos, sin))
+        ref = ref[0] if isinstance(ref, tuple) else ref
+        c2, s2 = E.rope_tables(pos + step, 16, 10000.0, torch.float32)
+        got = E.later_layer(xs_or[step], wl, 1, shape, c2, s2, cache_or, mask)
+        assert torch.allclose(got, ref, atol=3e-5), (step, (got - ref).abs().max())
+        total_hf = total_hf + (ref * probe[step]).sum()
+        total_or = total_or + (got * probe[step]).sum()
+    total_hf.backward()
+    total_or.backward()
+    for a, b in zip(xs_or, xs_hf):   # step 0's input also reaches steps 1, 2 through the cache
+        assert torch.allclose(a.grad, b.grad, atol=1e-4, rtol=1e-4)
+    for n, prm in names.items():
+        assert torch.allclose(wl[p + n].grad, prm.grad, atol=2e-4, rtol=1e-4), n
+
+
+def test_later_layer_pin_notices_a_post_norm_or_a_dropped_residual():
+    """The comparison above has teeth: the plausible slips (normalising after the attention
+    instead of before it, a residual taken from the normalised input) move the output by far
+    more than its tolerance."""
+    shape = _tiny_shape(num_hidden_layers=2)
+    w = _randomise_gains(E.random_weights(shape, seed=11, std=0.2), 12)
+    t = 12
+    doc, pos = _ttt_batch(t, [7, 5], 0)
+    x = torch.randn(1, t, 64, generator=torch.Generator().manual_seed(1))
+    cos, sin = E.rope_tables(pos, 16, 10000.0, torch.float32)
+    mask = M.ttt_mask_dense(doc, t, 0)
+    good = E.later_layer(x, w, 1, shape, cos, sin, {}, mask)
+    p = "layers.1."
+    a = E._attention_block(x, w, p + "self_attn.", shape, cos, sin, {}, mask, "dense")
+    post = x + E.rms_norm(a, w[p + "input_layernorm.weight"], shape.rms_norm_eps)
+    post = post + E.swiglu_mlp(E.rms_norm(post, w[p + "post_attention_layernorm.weight"], 1e-6), w, p + "mlp.")
+    xn = E.rms_norm(x, w[p + "input_layernorm.weight"], shape.rms_norm_eps)
+    y = xn + E._attention_block(xn, w, p + "self_attn.", shape, cos, sin, {}, mask, "dense")
+    wrong_res = y + E.swiglu_mlp(E.rms_norm(y, w[p + "post_attention_layernorm.weight"], 1e-6), w, p + "mlp.")
+    assert (good - post).abs().max() > 1e-2 and (good - wrong_res).abs().max() > 1e-2
+
+
+def test_first_layer_with_qk_norm_equals_hf_qwen3_blocks():
+    """EAGLE3 on Qwen3 layers: ``Eagle3FirstLayerMixin`` (models/eagle3/model_definitions.py:14-110)
+    mixed into ``Qwen3DecoderLayer`` (models/base_components.py:46-51) swaps q/k/v for projections
+    of the 2H input and otherwise runs the library's ``Qwen3Attention.forward``: per-head RMSNorm
+    of q and k BEFORE the rotary embedding.  The oracle's first layer with ``qk_norm`` against the
+    library's ``Qwen3Attention`` / ``Qwen3MLP`` / ``Qwen3RMSNorm`` / ``Qwen3RotaryEmbedding``
+    composed that way, three TTT steps on one ``DynamicCache``, non-trivial q/k gains; a
+    norm-after-RoPE variant is noticed."""
+    from transformers import DynamicCache, Qwen3Config
+    from transformers.models.qwen3.modeling_qwen3 import (
+        Qwen3Attention, Qwen3MLP, Qwen3RMSNorm, Qwen3RotaryEmbedding)
+
+    shape = _tiny_shape(qk_norm=True, norm_before_residual=False)
+    w = _randomise_gains(E.random_weights(shape, seed=21, std=0.2), 22)
+    cfg = Qwen3Config(hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+                      intermediate_size=128, vocab_size=128, rms_norm_eps=1e-6, num_hidden_layers=1,
+                      attention_bias=False, layer_types=["full_attention"], sliding_window=None,
+                      rope_parameters={"rope_type": "default", "rope_theta": 10000.0})
+    cfg._attn_implementation = "eager"
+    attn = Qwen3Attention(cfg, 0)
+    attn.q_proj = torch.nn.Linear(128, 64, bias=False)
+    attn.k_proj = torch.nn.Linear(128, 32, bias=False)
+    attn.v_proj = torch.nn.Linear(128, 32, bias=False)
+    p = "layers.0."
+    for n in "qkvo":
+        getattr(attn, n + "_proj").weight.data.copy_(w[p + f"self_attn.{n}_proj.weight"])
+    attn.q_norm.weight.data.copy_(w[p + "self_attn.q_norm.weight"])
+    attn.k_norm.weight.data.copy_(w[p + "self_attn.k_norm.weight"])
+    mlp = Qwen3MLP(cfg)
+    for n in ("gate", "up", "down"):
+        getattr(mlp, n + "_proj").weight.data.copy_(w[p + f"mlp.{n}_proj.weight"])
+    norms = {}
+    for n in ("input_layernorm", "hidden_norm", "post_attention_layernorm"):
+        norms[n] = Qwen3RMSNorm(64, eps=1e-6)
+        norms[n].weight.data.copy_(w[p + n + ".weight"])
+    rot = Qwen3RotaryEmbedding(cfg)
+
+    t = 20
+    doc, pos = _ttt_batch(t, [8, 9], 3)
+    g = torch.Generator().manual_seed(23)
+    cache_hf, cache_or, cache_bad = DynamicCache(), {}, {}
+    with torch.no_grad():
+        for step in range(3):
+            x = torch.randn(1, t, 128, generator=g)
+            mask = M.ttt_mask_dense(doc, t, step)
+            cos, sin = rot(x, pos + step)
+            e, h = x.split(64, -1)
+            residual = h                                # norm_before_residual = False
+            e, h = norms["input_layernorm"](e), norms["hidden_norm"](h)
+            a, _ = attn(hidden_states=torch.cat([e, h], -1), attention_mask=_additive(mask),
+                        position_embeddings=(cos, sin), past_key_values=cache_hf)
+            y = residual + a
+            ref = y + mlp(norms["post_attention_layernorm"](y))
+            c2, s2 = E.rope_tables(pos + step, 16, 10000.0, torch.float32)
+            got = E.first_layer(x, w, shape, c2, s2, cache_or, mask)
+            assert torch.allclose(got, ref, atol=3e-5), (step, (got - ref).abs().max())
+            # the slip this pin is for: normalising after the rotation
+            xin = torch.cat([e, h], -1)
+            q = torch.nn.functional.linear(xin, w[p + "self_attn.q_proj.weight"]).view(1, t, 4, 16).transpose(1, 2)
+            k = torch.nn.functional.linear(xin, w[p + "self_attn.k_proj.weight"]).view(1, t, 2, 16).transpose(1, 2)
+            v = torch.nn.functional.linear(xin, w[p + "self_attn.v_proj.weight"]).view(1, t, 2, 16).transpose(1, 2)
+            q = E.rms_norm(E.apply_rope(q, c2, s2), w[p + "self_attn.q_norm.weight"], 1e-6)
+            k = E.rms_norm(E.apply_rope(k, c2, s2), w[p + "self_attn.k_norm.weight"], 1e-6)
+            cache_bad["k"] = k if "k" not in cache_bad else torch.cat([cache_bad["k"], k], 2)
+            cache_bad["v"] = v if "v" not in cache_bad else torch.cat([cache_bad["v"], v], 2)
+            o = dense_attention(q, cache_bad["k"], cache_bad["v"], mask, 16 ** -0.5)
+            bad = torch.nn.functional.linear(o.reshape(1, t, 64), w[p + "self_attn.o_proj.weight"])
+            assert (bad - a).abs().max() > 1e-2

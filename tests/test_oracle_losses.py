@@ -212,3 +212,39 @@ def test_dpace_equals_per_block_double_loop_on_random_masks():
     # no gradient reaches the row losses through the weight
     ce = torch.rand(1, 8, generator=g, requires_grad=True)
     assert not L.dpace_loss_decay(None, torch.ones(1, 8), 4, 0.5, ce).requires_grad
+
+
+def test_compound_loss_is_the_weighted_sum_and_reports_terms_only_when_several():
+    """losses/utils.py:233-266: total = sum_name weight * loss_function(name); the ``{name}_loss``
+    entries are the UNWEIGHTED, detached per-term values and exist only for more than one term.
+    Checked against the closed form built from the single-term reduction (itself pinned above),
+    with a mask, a decay and weights that do not sum to one."""
+    g = torch.Generator().manual_seed(7)
+    a = torch.randn(1, 12, 40, generator=g, requires_grad=True)
+    b = torch.randn(1, 12, 40, generator=g)
+    m = (torch.rand(1, 12, generator=g) < 0.6).float()
+    pos = torch.full((1, 12), 2)
+    d = partial(L.exp_loss_decay, gamma=0.8)
+    single = {n: L.loss_function(a, b, m, pos, L.LOSS_FNS[n], d) for n in ("ce", "tv", "kl_div")}
+
+    cfg = L.resolve_loss_config({"ce": 0.25, "tv": 0.75})
+    total, terms = L.compound_loss(a, b, m, pos, cfg, d)
+    assert torch.isclose(total, 0.25 * single["ce"] + 0.75 * single["tv"], rtol=1e-6)
+    assert set(terms) == {"ce_loss", "tv_loss"}
+    assert torch.equal(terms["ce_loss"], single["ce"].detach()) and not terms["ce_loss"].requires_grad
+    assert torch.equal(terms["tv_loss"], single["tv"].detach())
+    # the weights are applied as given: no renormalisation, order of the mapping irrelevant
+    cfg3 = L.resolve_loss_config({"tv": 2.0, "kl_div": 0.5, "ce": 1.5})
+    total3, terms3 = L.compound_loss(a, b, m, pos, cfg3, d)
+    assert torch.isclose(total3, 2.0 * single["tv"] + 0.5 * single["kl_div"] + 1.5 * single["ce"], rtol=1e-6)
+    assert set(terms3) == {"tv_loss", "kl_div_loss", "ce_loss"}
+    # the gradient is the weighted sum of the terms' gradients (the terms dict carries none)
+    gt, = torch.autograd.grad(total, a, retain_graph=True)
+    gc, = torch.autograd.grad(single["ce"], a, retain_graph=True)
+    gv, = torch.autograd.grad(single["tv"], a, retain_graph=True)
+    assert torch.allclose(gt, 0.25 * gc + 0.75 * gv, atol=1e-7)
+    # one term: the weight still applies, nothing is reported
+    one, none = L.compound_loss(a, b, m, pos, L.resolve_loss_config({"tv": 0.3}), d)
+    assert none == {} and torch.isclose(one, 0.3 * single["tv"], rtol=1e-6)
+    plain, none = L.compound_loss(a, b, m, pos, L.resolve_loss_config("kl_div"), d)
+    assert none == {} and torch.equal(plain, single["kl_div"])
