@@ -103,9 +103,6 @@ def parse_args():
     ap.add_argument("--cpu-baseline", choices=["sample", "off"], default="sample")
     ap.add_argument("--cpu-seq-len", type=int, default=1024)
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline timing")
-    ap.add_argument("--probes", action="store_true",
-                    help="run the hardware probes (matrix-pipe ceiling and clock under load, LDS bandwidth, "
-                         "vector work beside a busy matrix pipe, cost of issuing global->LDS loads) and print them")
     ap.add_argument("--only-kernels", action="store_true",
                     help="run only the per-kernel timing loops (for rocprofv3 counter runs)")
     return ap.parse_args()
@@ -861,62 +858,8 @@ def _decoder_gemm_mode():
     return gemm.DECODER_GEMM
 
 
-def run_probes():
-    """The hardware figures the kernel designs rest on, measured by speculators_amd/libspx_probes.so
-    (csrc/probes/hw_probes.hip); one JSON object."""
-    import ctypes
-
-    path = os.path.join(ROOT, "speculators_amd", "libspx_probes.so")
-    if not os.path.exists(path):
-        print(f"bench.py: {path} is missing (make -C speculators_amd/csrc)", file=sys.stderr)
-        sys.exit(2)
-    lib = ctypes.CDLL(path)
-    lib.spx_probe.restype = ctypes.c_int
-    lib.spx_probe.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.c_int]
-
-    def probe(which, n):
-        buf = (ctypes.c_double * n)()
-        got = lib.spx_probe(which, buf, n)
-        if got != n:
-            raise RuntimeError(f"probe {which} failed ({got})")
-        return [float(v) for v in buf]
-
-    m = probe(0, 4)
-    lds = probe(1, 2)
-    co = probe(2, 12)
-    dma = probe(3, 2)
-    m16 = probe(4, 4)
-    mixes = ["64 x v_exp_f32", "64 x v_fma_f32", "64 x (v_max_f32 + v_add_f32)"]
-    out = {
-        "mfma_32x32x16_bf16_registers_only": {
-            "random_operands": {"tflops": round(m[0], 1), "shader_clock_ghz": round(m[1], 3),
-                                "frac_of_2500": round(m[0] / PEAK_BF16_TFLOPS, 3)},
-            "zero_operands": {"tflops": round(m[2], 1), "shader_clock_ghz": round(m[3], 3)},
-            "note": "one wave per SIMD, four independent accumulators; 32 cycles per instruction and SIMD"},
-        "mfma_16x16x32_bf16_registers_only": {
-            "random_operands": {"tflops": round(m16[0], 1), "shader_clock_ghz": round(m16[1], 3),
-                                "frac_of_2500": round(m16[0] / PEAK_BF16_TFLOPS, 3)},
-            "zero_operands": {"tflops": round(m16[2], 1), "shader_clock_ghz": round(m16[3], 3)},
-            "note": "one wave per SIMD, 64 independent accumulators; 16 cycles per instruction and SIMD"},
-        "lds_read_b128": {"bytes_per_clock_per_cu": round(lds[0], 1), "bytes_per_ns_per_cu": round(lds[1], 1),
-                          "note": "8 waves per CU, 16 conflict-free reads in flight per wave"},
-        "vector_work_beside_a_busy_matrix_pipe": [
-            {"vector_loop_body": mixes[i],
-             "mfma_wave_cycles_per_32_mfma": {"alone": round(co[4 * i], 1), "together": round(co[4 * i + 2], 1)},
-             "vector_wave_cycles_per_body": {"alone": round(co[4 * i + 1], 1), "together": round(co[4 * i + 3], 1)}}
-            for i in range(3)],
-        "global_to_lds_load_issue_cycles_per_1kb_wave_load": {
-            "other_waves_idle": round(dma[0], 1), "other_waves_reading_lds_and_running_mfma": round(dma[1], 1),
-            "note": "four loads back to back per wave, four loading waves per CU, data resident in L2"},
-    }
-    print(json.dumps(out))
-
-
 def main():
     args = parse_args()
-    if args.probes:
-        run_probes()
-        return
     if args.gpus != 1:
         print(f"bench.py: this build runs on ONE GPU (no collectives are built); got --gpus {args.gpus}",
               file=sys.stderr)

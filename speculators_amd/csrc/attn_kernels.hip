@@ -1912,9 +1912,6 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
   }
   auto issue = [&](int s_, int buf, int set) __attribute__((always_inline)) {
     const int mq = s_ * 32;
-#ifdef SPX_WS_NODMA
-    if (p.NQ > 0) return;
-#endif
     const uint32_t rb = lds0 + buf * SM::kTile;
 #pragma unroll
     for (int j = 0; j < LPW; ++j)
@@ -2043,20 +2040,8 @@ __device__ __attribute__((noinline)) void dkv_ws_role(
     auto fread = [&](int f) {
       const int e = f / 2, s2 = e / NDB, db = e % NDB;
       const uint8_t* const base = tile + ((f & 1) ? 0 : 32 * RBQ) + s2 * 16 * RBQ;
-#ifdef SPX_WS_SLOWT
-      // element-wise gather of the same fragment (checking aid)
-      i16x4 l4, h4;
-      for (int j = 0; j < 8; ++j) {
-        const int qr = s2 * 16 + (j < 4 ? 4 * g + j : 8 + 4 * g + j - 4), dd = db * 32 + col;
-        const int pos = ((dd >> 3) ^ swz_r(qr)) * 16 + (dd & 7) * 2;
-        const short v = *reinterpret_cast<const short*>(tile + ((f & 1) ? 0 : 32 * RBQ) + qr * RBQ + pos);
-        if (j < 4) l4[j] = v; else h4[j - 4] = v;
-      }
-      lo[f % RG] = l4; hi[f % RG] = h4;
-#else
       lo[f % RG] = lds_read_tr16(base + (rt0 ^ (db * 64)));
       hi[f % RG] = lds_read_tr16(base + (rt1 ^ (db * 64)));
-#endif
     };
     auto frag = [&](int f) {
       const i16x8 v = __builtin_shufflevector(lo[f % RG], hi[f % RG], 0, 1, 2, 3, 4, 5, 6, 7);

@@ -75,11 +75,27 @@ __device__ __forceinline__ u32x4 lds_read128(uint32_t addr) {
 // vector registers on every trip.)  The compiler does not know what the statement is: whoever reads
 // an accumulator with a vector instruction afterwards waits for the matrix pipe first
 // (`mfma_results_ready`).
+//
+// Cross-check build: compiled with -DSPX_MFMA_BUILTIN=1 the same statement is the compiler's own
+// builtin, whose result hazards the compiler places itself (slower: the accumulators are copied
+// around, see above).  The GEMM tests must pass on both builds; running them once on that build
+// after an edit of a kernel that uses mfma16 shows whether a hand-placed wait has gone missing.
+#ifndef SPX_MFMA_BUILTIN
+#define SPX_MFMA_BUILTIN 0
+#endif
 __device__ __forceinline__ void mfma16(f32x4& acc, bf16x8 a, bf16x8 b) {
+#if SPX_MFMA_BUILTIN
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+#else
   asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+#endif
 }
 // more wait states than the longest matrix instruction needs before its result may be read
-__device__ __forceinline__ void mfma_results_ready() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+__device__ __forceinline__ void mfma_results_ready() {
+#if !SPX_MFMA_BUILTIN
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#endif
+}
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }

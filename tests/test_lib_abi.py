@@ -33,20 +33,6 @@ def test_library_exports_every_declared_symbol():
     assert set(_lib.SIGNATURES) | {"spx_version", "spx_last_error"} == set(_declared_symbols())
 
 
-def test_probe_library_is_built_and_separate_from_the_product():
-    """The hardware probes of ``bench.py --probes`` live in a library of their own: it exports its
-    one entry point, and the product library exports no probe."""
-    import ctypes
-
-    from speculators_amd import _lib
-
-    path = os.path.join(ROOT, "speculators_amd", "libspx_probes.so")
-    if not os.path.exists(path):
-        pytest.fail("libspx_probes.so is not built; run __graft_entry__.build()")
-    assert hasattr(ctypes.CDLL(path), "spx_probe")
-    assert not hasattr(_lib.load(), "spx_probe")
-
-
 def test_argument_errors_do_not_need_a_gpu():
     from speculators_amd import _lib
 
