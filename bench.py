@@ -100,6 +100,12 @@ def parse_args():
                     help="autocast: fp32 master weights, forward under torch.autocast(bf16), fp32 "
                          "gradients (the regime of the reference's Trainer, train/trainer.py:459-465); "
                          "bf16: the whole model cast to bf16 (the reference's integration tests)")
+    ap.add_argument("--window", type=int, default=0,
+                    help="sliding window of every draft layer for the HEADLINE figure (0 = full attention, what "
+                         "BASELINE's configs[1] names).  The reference's scripts/train.py makes every EAGLE3 draft "
+                         "layer sliding-window with W = 2048 unless --full-attention-indices is given "
+                         "(scripts/train.py:176-179,498-506; train/config/schema.py:172-183): the default run "
+                         "times that configuration as a second figure, `reference_default_config`")
     ap.add_argument("--cpu-baseline", choices=["sample", "off"], default="sample")
     ap.add_argument("--cpu-seq-len", type=int, default=1024)
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline timing")
@@ -218,9 +224,18 @@ class GemmProbe:
         return sum(a.elapsed_time(b) for a, b in self.pairs) / len(self.pairs)
 
 
-def kernel_rooflines(torch, cfg, t, k_steps, device):
+def windowed_pairs(t, window):
+    """Live (query, context key) pairs of one document of ``t`` rows under a causal mask with a
+    sliding window (``kv > q - window``); no window = all ``t (t + 1) / 2``."""
+    if not window or window >= t:
+        return t * (t + 1) / 2
+    return window * (window + 1) / 2 + (t - window) * window
+
+
+def kernel_rooflines(torch, cfg, t, k_steps, device, windows=(None,)):
     """Per-kernel average launch time (HIP events on the launch stream) against the
-    algorithmic flops / bytes of that launch."""
+    algorithmic flops / bytes of that launch.  ``windows``: the sliding windows (None = full
+    attention) the attention kernels are timed with."""
     from speculators_amd import _lib
     from speculators_amd import attention as A
     from speculators_amd import losses as L
@@ -375,40 +390,29 @@ def kernel_rooflines(torch, cfg, t, k_steps, device):
         2.0 * t * 4 * h * 2 + t * 7 * 8, ms, 0)
     del hs, p_aux, p_last
 
-    # TTT attention at the last step (k = K-1 diagonals): forward and backward
-    step = k_steps - 1
-    mask = A.create_ttt_mask(torch.zeros(t, dtype=torch.long, device=device), t, None)
-    for _ in range(step):
-        mask = mask.extended()
-    q = torch.randn(1, hq, t, d, device=device, generator=g).bfloat16().requires_grad_(True)
-    kk = torch.randn(1, hkv, (step + 1) * t, d, device=device, generator=g).bfloat16().requires_grad_(True)
-    vv = torch.randn(1, hkv, (step + 1) * t, d, device=device, generator=g).bfloat16().requires_grad_(True)
-    pairs = t * (t + 1) / 2 + step * t
-    ms_f = time_events(torch, lambda: A.ttt_attention(q.detach(), kk.detach(), vv.detach(), mask), 10)
-    mfma(f"attn_fwd_kernel[TTT step {step}]", 4.0 * pairs * d * hq, ms_f, 1)
-    o = A.ttt_attention(q, kk, vv, mask)
-    go = torch.randn_like(o)
+    # TTT attention, forward and backward, at the first step (no diagonal keys) and at the last one
+    # (K - 1 diagonal keys per row), full and -- where asked -- with every layer's sliding window
+    def attn_rows(step, window):
+        mask = A.create_ttt_mask(torch.zeros(t, dtype=torch.long, device=device), t, window)
+        for _ in range(step):
+            mask = mask.extended()
+        q = torch.randn(1, hq, t, d, device=device, generator=g).bfloat16().requires_grad_(True)
+        kk = torch.randn(1, hkv, (step + 1) * t, d, device=device, generator=g).bfloat16().requires_grad_(True)
+        vv = torch.randn(1, hkv, (step + 1) * t, d, device=device, generator=g).bfloat16().requires_grad_(True)
+        pairs = windowed_pairs(t, window) + step * t
+        tag = f"TTT step {step}" + (f", window {window}" if window else "")
+        key = f"attn_step{step}" + (f"_w{window}" if window else "")
+        ms_f = time_events(torch, lambda: A.ttt_attention(q.detach(), kk.detach(), vv.detach(), mask), 10)
+        mfma(f"attn_fwd_kernel[{tag}]", 4.0 * pairs * d * hq, ms_f, 1, key + "_fwd")
+        o = A.ttt_attention(q, kk, vv, mask)
+        go = torch.randn_like(o)
+        ms_b = time_events(torch, lambda: torch.autograd.grad(o, (q, kk, vv), go, retain_graph=True), 10)
+        names = "dq + dkv + diag kernels" if step else "dq + dkv kernels"
+        mfma(f"attn_bwd[{names}, {tag}]", 10.0 * pairs * d * hq, ms_b, 1, key + "_bwd")
 
-    def attn_bwd():
-        torch.autograd.grad(o, (q, kk, vv), go, retain_graph=True)
-
-    ms_b = time_events(torch, attn_bwd, 10)
-    mfma(f"attn_bwd[dq + dkv + diag kernels, TTT step {step}]", 10.0 * pairs * d * hq, ms_b, 1)
-    del q, kk, vv, o, go
-
-    # ... and at the first step (no diagonal keys)
-    mask0 = A.create_ttt_mask(torch.zeros(t, dtype=torch.long, device=device), t, None)
-    q = torch.randn(1, hq, t, d, device=device, generator=g).bfloat16().requires_grad_(True)
-    kk = torch.randn(1, hkv, t, d, device=device, generator=g).bfloat16().requires_grad_(True)
-    vv = torch.randn(1, hkv, t, d, device=device, generator=g).bfloat16().requires_grad_(True)
-    pairs0 = t * (t + 1) / 2
-    ms_f = time_events(torch, lambda: A.ttt_attention(q.detach(), kk.detach(), vv.detach(), mask0), 10)
-    mfma("attn_fwd_kernel[TTT step 0]", 4.0 * pairs0 * d * hq, ms_f, 1)
-    o = A.ttt_attention(q, kk, vv, mask0)
-    go = torch.randn_like(o)
-    ms_b = time_events(torch, lambda: torch.autograd.grad(o, (q, kk, vv), go, retain_graph=True), 10)
-    mfma("attn_bwd[dq + dkv kernels, TTT step 0]", 10.0 * pairs0 * d * hq, ms_b, 1)
-    del q, kk, vv, o, go
+    for window in windows:
+        attn_rows(k_steps - 1, window)
+        attn_rows(0, window)
 
     # weight gradient of the merged gate / up projection over all TTT steps in one product: the steps'
     # output gradients [K T, 2F] and inputs [K T, H] lie one after the other, the contraction runs over
@@ -886,15 +890,22 @@ def main():
     if big:
         t = SEQ_LEN3 if t == SEQ_LEN else t
         k_steps = TTT_STEPS3 if k_steps == TTT_STEPS else k_steps
+    REF_WINDOW = 2048  # noqa: N806 - the reference's default sliding window (train/config/schema.py:172-183)
+    head_window = args.window or None
+    # the attention kernels are timed with the headline's mask and with the reference default's
+    kernel_windows = (head_window,) if head_window else (None, REF_WINDOW)
     if args.only_kernels:
-        print(json.dumps({"kernels": kernel_rooflines(torch, CONFIG1, t, k_steps, device)}))
+        print(json.dumps({"kernels": kernel_rooflines(torch, CONFIG1, t, k_steps, device, kernel_windows)}))
         return
     batch, d2t, t2d = make_inputs(torch, CONFIG1, t, device, args.targets == "logits")
     loss_cfg = None  # kl_div, the reference default
     autocast = args.regime == "autocast"
 
-    def build(auto):
-        mdl = make_model(torch, CONFIG1, device, d2t, t2d, torch.float32 if auto else torch.bfloat16)
+    def build(auto, window=head_window):
+        cfg = dict(CONFIG1)
+        if window:  # every draft layer sliding-window, as scripts/train.py builds them by default
+            cfg.update(sliding_window=window, sliding_layers=(0,))
+        mdl = make_model(torch, cfg, device, d2t, t2d, torch.float32 if auto else torch.bfloat16)
 
         def one_step():
             mdl.zero_grad(set_to_none=True)
@@ -919,6 +930,28 @@ def main():
     del model, step, loss
     torch.cuda.empty_cache()
 
+    # the reference's default training configuration beside the headline: the same step with every
+    # draft layer sliding-window (W = 2048), same regime, same inputs
+    ref_default = None
+    if not head_window and t > REF_WINDOW:
+        model, step = build(autocast, REF_WINDOW)
+        for _ in range(args.warmup):
+            step()
+        with quiet_gc():
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                loss = step()
+            torch.cuda.synchronize()
+        w_ms = (time.perf_counter() - t0) / args.steps * 1e3
+        ref_default = {"sliding_window": REF_WINDOW, "sliding_layers": "all", "regime": args.regime,
+                       "ms_per_step": round(w_ms, 3), "value": round(t / (w_ms * 1e-3), 1), "unit": "tokens/s",
+                       "final_loss": round(float(loss.detach()), 6),
+                       "note": "what scripts/train.py trains by default (scripts/train.py:176-179,498-506); "
+                               "BASELINE's configs[1] names no window, so the headline above is full attention"}
+        del model, step, loss
+        torch.cuda.empty_cache()
+
     model, step = build(autocast)
     for _ in range(args.warmup):
         step()
@@ -936,7 +969,7 @@ def main():
     tokens = int((batch["document_ids"] != -1).sum().item())
     value = tokens / (ms_per_step * 1e-3)
 
-    kernels = [] if args.no_kernels else kernel_rooflines(torch, CONFIG1, t, k_steps, device)
+    kernels = [] if args.no_kernels else kernel_rooflines(torch, CONFIG1, t, k_steps, device, kernel_windows)
     in_step = probe.mean_ms()
     for rec in kernels:
         if rec["kernel"].startswith("gemm_bf16_nt_kernel[lm_head fwd") and in_step:
@@ -972,11 +1005,12 @@ def main():
                                + ("fp32 master weights under torch.autocast(bf16), fp32 gradients "
                                   "(the reference Trainer's regime), " if autocast else
                                   "bf16 weights and activations (whole model cast), ")
-                               + "full attention, "
-                               f"targets from {'verifier hidden states through the frozen verifier head' if args.targets == 'hidden' else 'full-vocab verifier logits gathered through d2t'}",
+                               + (f"sliding window {head_window} on every layer, " if head_window else "full attention, ")
+                               + f"targets from {'verifier hidden states through the frozen verifier head' if args.targets == 'hidden' else 'full-vocab verifier logits gathered through d2t'}",
                    "seq_len": t, "ttt_steps": k_steps, "tokens_per_step": tokens,
                    "regime": args.regime, "final_loss": round(float(loss.detach()), 6),
-                   "decoder_gemm": _decoder_gemm_mode()},
+                   "sliding_window": head_window, "decoder_gemm": _decoder_gemm_mode()},
+        "reference_default_config": ref_default,
         "other_regime": {"regime": "bf16" if autocast else "autocast", "ms_per_step": round(other_ms, 3),
                          "value": round(tokens / (other_ms * 1e-3), 1), "unit": "tokens/s",
                          "final_loss": round(other_loss, 6)},

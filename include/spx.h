@@ -279,7 +279,11 @@ int spx_ttt_attn_fwd(const void* q, int64_t q_head_stride, const void* k,
  * launches allocates or frees memory.  Results are bit-identical to spx_ttt_attn_fwd.  All calls
  * on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two
  * host threads) race on it; calls ordered on one stream do not.  Nothing has to be cleared
- * between calls: each call rewrites every byte of the array it later reads. */
+ * between calls: each call rewrites every byte of the array it later reads.
+ * The FIRST call on a device for a given head_dim does set-up work that is not allowed while a
+ * stream is being captured (it looks up the array's address, which may load the code object, and
+ * raises the kernel's dynamic-LDS limit): make one call per device and head_dim outside capture
+ * before capturing; every later call only launches kernels. */
 int64_t spx_ttt_attn_fwd_static_max_bytes(void);
 int spx_ttt_attn_fwd_static(const void* q, int64_t q_head_stride, const void* k,
                             int64_t k_head_stride, const void* v, int64_t v_head_stride,

@@ -27,6 +27,22 @@ if not 1 <= SPLIT_PARTS <= 8:
     raise ValueError(f"SPX_GEMM_SPLIT_PARTS must be 1 .. 8, got {SPLIT_PARTS}")
 
 
+_split_ws: dict = {}
+
+
+def _split_workspace(device, numel: int) -> torch.Tensor:
+    """The fp32 partials of a product cut along its contraction: one buffer per (device, stream), kept
+    and grown on demand, so a TTT loop does not allocate hundreds of MB per step for a workspace the
+    kernel leaves untouched whenever the device-side row count asks for one part.  Launches of one
+    stream are ordered, so consecutive products may share it."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _split_ws.get(key)
+    if ws is None or ws.numel() < numel:
+        ws = torch.empty(numel, device=device, dtype=torch.float32)
+        _split_ws[key] = ws
+    return ws
+
+
 def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
             m_live: torch.Tensor | None = None, split: bool = False) -> torch.Tensor:
     """``a[M, K] @ b[N, K].T -> [M, N]`` (bf16, fp32 accumulation).
@@ -60,10 +76,10 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
         # (a product of many rounds of tiles has little to gain from cutting: at most 1 / rounds)
         few_tiles = -(-m // 256) * -(-n // 256) <= 2 * 256
         if split and SPLIT_PARTS > 1 and few_tiles and n % 8 == 0 and out.stride(0) % 8 == 0 and k >= 64 * 16 * 2:
-            ws = torch.empty(SPLIT_PARTS * m * n, device=a.device, dtype=torch.float32)
+            ws = _split_workspace(a.device, SPLIT_PARTS * m * n)
             _lib.call("spx_gemm_bf16_nt_rows_split", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
                       _lib.ptr(out), out.stride(0), m, n, k, _lib.ptr(m_live), SPLIT_PARTS, _lib.ptr(ws),
-                      ws.numel() * 4, st)
+                      SPLIT_PARTS * m * n * 4, st)
         else:
             _lib.call("spx_gemm_bf16_nt_rows", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
                       _lib.ptr(out), out.stride(0), m, n, k, _lib.ptr(m_live), st)

@@ -302,3 +302,32 @@ def test_gemm_tn_small_result_long_contraction(t, m, n, fp32):
     acc = got.clone()
     gemm_tn(a, b, acc, accumulate=True)
     assert (acc.double() - 2 * want).abs().max() <= 2.5 * tol * want.abs().max() * 2 + 1e-4
+
+
+@pytest.mark.parametrize("m,n", [(20, 13), (9, 64), (64, 1)])
+def test_weight_gradient_of_unaligned_operands_takes_the_library_product(m, n):
+    """``weights.wgrad_product`` hands operands the transposing MFMA kernel cannot take (a width that
+    is no multiple of 8: a gate of width 1, an odd hidden size) to PyTorch's matmul: fp32 result,
+    with and without a gradient to add to, against the fp64 product; aligned operands of the same
+    size class take the kernel and agree with it."""
+    from speculators_amd import weights
+
+    g = torch.Generator().manual_seed(m * 100 + n)
+    t = 300
+    dy = torch.randn(t, m, generator=g).bfloat16().cuda()
+    x = torch.randn(t, n, generator=g).bfloat16().cuda()
+    assert not (weights._tn_ok(dy) and weights._tn_ok(x))
+    want = dy.double().t() @ x.double()
+    got = weights.wgrad_product(dy, x, None)
+    assert got.dtype == torch.float32 and got.shape == (m, n)
+    assert (got.double() - want).abs().max() <= 1e-5 * want.abs().max() + 1e-6
+    acc0 = torch.randn(m, n, generator=g).cuda()
+    acc = acc0.clone()
+    got2 = weights.wgrad_product(dy, x, acc)
+    assert got2 is acc
+    assert (acc.double() - (acc0.double() + want)).abs().max() <= 1e-5 * want.abs().max() + 1e-6
+    # the aligned neighbour runs on the kernel and gives the same kind of answer
+    dy8, x8 = torch.nn.functional.pad(dy, (0, -m % 8)), torch.nn.functional.pad(x, (0, -n % 8))
+    assert weights._tn_ok(dy8) and weights._tn_ok(x8)
+    got8 = weights.wgrad_product(dy8, x8, None)
+    assert (got8[:m, :n].double() - want).abs().max() <= 1e-5 * want.abs().max() + 1e-6

@@ -467,3 +467,46 @@ def test_hybrid_model_with_a_padding_mask_matches_oracle():
         if prm.requires_grad:
             want = wf[name].grad
             assert (prm.grad.float().cpu() - want).abs().max() <= 3e-2 * want.abs().max() + 1e-6, name
+
+
+def test_hybrid_projections_on_this_librarys_gemm_agree_with_the_default(monkeypatch):
+    """``SPX_DECODER_GEMM=spx`` on a hybrid MoE layer: every projection the kernel can take runs on
+    it, and the ones it cannot (the shared expert's gate of width 1: a contraction of one element
+    in its input gradient) stay with PyTorch's matmul inside the same mode.  Loss, logits and every
+    gradient against the default mode."""
+    from speculators_amd import gemm
+
+    shape = _hybrid_shape(model_type="qwen3_5_moe_text", **_MOE)
+    steps = 2
+    w = {k: v.bfloat16() for k, v in OM.random_weights(shape, seed=3, std=0.05).items()}
+    g = torch.Generator().manual_seed(6)
+    b, n = 2, 150
+    ids = torch.randint(0, shape.vocab_size, (b, n), generator=g).cuda()
+    hs = torch.randn(b, n, shape.hidden_size, generator=g).bfloat16().cuda()
+    lm = (torch.rand(b, n, generator=g) < 0.7).float().cuda()
+    sw = OM.compute_step_weights(0.6, steps)
+    seen = []
+    real_back = gemm._project_back
+
+    def spy(dy2, staged):
+        seen.append((gemm.DECODER_GEMM, dy2.shape[1]))
+        return real_back(dy2, staged)
+
+    monkeypatch.setattr(gemm, "_project_back", spy)
+    results = {}
+    for kind in ("mixed", "spx"):
+        monkeypatch.setattr(gemm, "DECODER_GEMM", kind)
+        model = _make(shape, w, steps)
+        logits, loss, _ = model(ids, hs, loss_mask=lm, step_weights=sw)
+        loss.backward()
+        results[kind] = (loss.item(), [l.float() for l in logits],
+                         {nm: p.grad.float() for nm, p in model.named_parameters() if p.grad is not None})
+    assert ("spx", 1) in seen, seen      # the width-1 gate went through the fall-back branch under spx
+    la, lga, ga = results["mixed"]
+    lb, lgb, gb = results["spx"]
+    assert abs(la - lb) <= 2e-3 * abs(la)
+    for a, b_ in zip(lga, lgb):
+        assert (a - b_).abs().max() <= 3e-2 * a.abs().max()
+    assert ga.keys() == gb.keys()
+    for nm in ga:
+        assert (ga[nm] - gb[nm]).abs().max() <= 3e-2 * ga[nm].abs().max() + 1e-6, nm

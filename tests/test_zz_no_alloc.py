@@ -49,6 +49,19 @@ def test_static_scratch_forward_equals_workspace_forward_twice_then_smaller():
         assert torch.isfinite(ref.float()).all()
         assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
         assert torch.equal(got_lse, ref_lse)
+        # a further call (the set-up of this device and head size is done) takes no memory from the
+        # device and none from torch's pool: free bytes and allocated bytes stand still across it
+        out = torch.empty(1, t, hq, d, device="cuda", dtype=torch.bfloat16)
+        lse = torch.empty(hq, t, device="cuda", dtype=torch.float32)
+        torch.cuda.synchronize()
+        free0, alloc0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+        _lib.call("spx_ttt_attn_fwd_static", _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1), _lib.ptr(v),
+                  v.stride(1), _lib.ptr(mask.row_lo), t, step, hq, hkv, d, float(d ** -0.5), _lib.ptr(out),
+                  _lib.ptr(lse), _lib.stream_ptr(q.device))
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free0
+        assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
 
 
 def test_static_scratch_rejects_shapes_above_its_limit():
