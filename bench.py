@@ -96,6 +96,9 @@ def parse_args():
                     help="hidden: verifier_last_hidden_states through the frozen verifier head "
                          "(the reference's forward contract); logits: full-vocab verifier "
                          "logits gathered through d2t")
+    ap.add_argument("--loss", default="kl_div",
+                    help="loss spec of the EAGLE3 workloads (losses/utils.py:184-230): kl_div (the reference "
+                         "default, the headline), ce, tv, ... or a JSON weighting such as '{\"ce\": 0.1, \"tv\": 0.9}'")
     ap.add_argument("--regime", choices=["autocast", "bf16"], default="autocast",
                     help="autocast: fp32 master weights, forward under torch.autocast(bf16), fp32 "
                          "gradients (the regime of the reference's Trainer, train/trainer.py:459-465); "
@@ -283,6 +286,16 @@ def kernel_rooflines(torch, cfg, t, k_steps, device, windows=(None,)):
     # the vendor library on the same product: a yardstick beside the kernel above, not part of the step
     ms = time_events(torch, lambda: torch.nn.functional.linear(x, w), 20)
     mfma("hipBLASLt through torch.nn.functional.linear[lm_head fwd T x H x Vd, yardstick]",
+         2.0 * t * h * vd, ms, 0)
+    # the same product with per-row soft-max statistics (log-sum-exp, first-index arg-max of the bf16 results)
+    # out of its epilogue: with the product stored (what a KL loss would still need of the verifier head) and
+    # without (all a cross-entropy loss needs: the verifier's logits never exist in memory)
+    from speculators_amd.gemm import gemm_nt_stats
+    ms = time_events(torch, lambda: gemm_nt_stats(x, w, store=True), 20)
+    mfma("gemm_bf16_nt_kernel<statistics epilogue> + reduce[verifier head T x H x Vd, product stored]",
+         2.0 * t * h * vd, ms, 0)
+    ms = time_events(torch, lambda: gemm_nt_stats(x, w, store=False), 20)
+    mfma("gemm_bf16_nt_kernel<statistics epilogue> + reduce[verifier head T x H x Vd, statistics only: ce targets]",
          2.0 * t * h * vd, ms, 0)
     wt = w.t().contiguous()
     dx = torch.empty(t, h, device=device, dtype=torch.bfloat16)
@@ -592,6 +605,26 @@ def run_mtp(args):
     ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
     tokens = b * n
     final_loss = float(loss.detach())
+    # the same iteration with the row log-sum-exp streamed by the label cross-entropy kernel instead of
+    # taken from the head product's epilogue (the default): what that fusion is worth on this workload
+    from speculators_amd import losses as losses_mod
+    epi_default = losses_mod.HEAD_CE_EPILOGUE_STATS
+    losses_mod.HEAD_CE_EPILOGUE_STATS = not epi_default
+    try:
+        for _ in range(2):
+            step()
+        with quiet_gc():
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                loss = step()
+            torch.cuda.synchronize()
+        other_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    finally:
+        losses_mod.HEAD_CE_EPILOGUE_STATS = epi_default
+    head_stats = {"epilogue_statistics" if epi_default else "streamed_statistics": round(ms_per_step, 3),
+                  "streamed_statistics" if epi_default else "epilogue_statistics": round(other_ms, 3),
+                  "unit": "ms_per_step", "default": "epilogue_statistics" if epi_default else "streamed_statistics"}
     del loss
     model.zero_grad(set_to_none=True)
     torch.cuda.empty_cache()
@@ -611,14 +644,30 @@ def run_mtp(args):
     w = model.lm_head.weight
     logits = gemm.gemm_nt(x, w)
     rec("gemm_bf16_nt_kernel[lm_head fwd rows x H x V]", "mfma", 2.0 * rows * h * v,
-        time_events(torch, lambda: gemm.gemm_nt(x, w, out=logits), 5), k_steps)
+        time_events(torch, lambda: gemm.gemm_nt(x, w, out=logits), 5), 0 if epi_default else k_steps)
     lab = torch.randint(0, v, (rows,), device=device)
     lab[torch.rand(rows, device=device) > 0.7] = -100
     live = int((lab != -100).sum())
     lg = logits.detach().requires_grad_(True)
     out = label_cross_entropy(lg, lab)
     rec("label_ce_fwd_kernel[rows x V, 70% live rows]", "hbm", live * v * 2.0,
-        time_events(torch, lambda: label_cross_entropy(logits, lab), 5), k_steps)
+        time_events(torch, lambda: label_cross_entropy(logits, lab), 5), 0 if epi_default else k_steps)
+    # the head product with every row's log-sum-exp out of its epilogue + one element per row for the loss:
+    # what replaces the two launches above in the model
+    lse_buf = torch.empty(rows, device=device)
+    st_ws = torch.empty(_lib.load().spx_gemm_stats_workspace_bytes(rows, v) // 4, device=device)
+    loss_buf = torch.empty(rows, device=device)
+    stp = _lib.stream_ptr(device)
+
+    def head_stats_ce():
+        _lib.call("spx_gemm_bf16_nt_stats", _lib.ptr(x), x.stride(0), _lib.ptr(w), w.stride(0), _lib.ptr(logits),
+                  logits.stride(0), rows, v, h, _lib.ptr(lse_buf), None, _lib.ptr(st_ws), st_ws.numel() * 4, stp)
+        _lib.call("spx_label_ce_from_lse", _lib.ptr(logits), logits.stride(0), _lib.ptr(lab), rows, v,
+                  _lib.dtype_code(logits), -100, _lib.ptr(lse_buf), _lib.ptr(loss_buf), stp)
+
+    rec("gemm_bf16_nt_kernel<statistics epilogue> + reduce + label_ce_pick[lm_head fwd + CE rows x H x V]", "mfma",
+        2.0 * rows * h * v, time_events(torch, head_stats_ce, 5), k_steps if epi_default else 0)
+    del st_ws
     go = torch.ones_like(out)
 
     def ce_bwd():
@@ -741,6 +790,7 @@ def run_mtp(args):
                    "final_loss": round(final_loss, 6)},
         "roofline": {k_: dominant[k_] for k_ in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
                     | {"kernel": dominant["kernel"]},
+        "head_cross_entropy_statistics": head_stats,
         "kernels": kernels, "cpu_baseline": cpu}))
 
 
@@ -898,7 +948,8 @@ def main():
         print(json.dumps({"kernels": kernel_rooflines(torch, CONFIG1, t, k_steps, device, kernel_windows)}))
         return
     batch, d2t, t2d = make_inputs(torch, CONFIG1, t, device, args.targets == "logits")
-    loss_cfg = None  # kl_div, the reference default
+    from speculators_amd import losses as losses_mod
+    loss_cfg = None if args.loss == "kl_div" else losses_mod.resolve_loss_config(args.loss)  # None = kl_div
     autocast = args.regime == "autocast"
 
     def build(auto, window=head_window):
@@ -1001,7 +1052,7 @@ def main():
                                 "configs[1]: EAGLE3 draft, Llama-3.1-8B shape, one draft layer, ")
                                +
                                f"batch 1, seq {t}, TTT {k_steps}, vocab 128256 -> draft 32000, "
-                               "kl_div loss, "
+                               f"{args.loss} loss, "
                                + ("fp32 master weights under torch.autocast(bf16), fp32 gradients "
                                   "(the reference Trainer's regime), " if autocast else
                                   "bf16 weights and activations (whole model cast), ")

@@ -71,7 +71,8 @@ int spx_vocab_gather(const void* full, int64_t ld_full, const int64_t* d2t,
  * and argmax_target are INPUTS holding the statistics of the same target rows
  * from an earlier call -- the verifier row is the same at every TTT step, only
  * shifted -- so the target max / sum / arg-max are not recomputed, and ce does
- * not read the target rows at all. */
+ * not read the target rows at all: `targets` may then be NULL (the arg-max can come
+ * from spx_gemm_bf16_nt_stats, and the verifier's logits never exist in memory). */
 int spx_fused_vocab_loss_fwd(int op, const void* logits, int64_t ld_logits,
                              const void* targets, int64_t ld_targets,
                              int64_t rows, int64_t vocab, int dtype,
@@ -147,6 +148,14 @@ int spx_fused_vocab_loss_bwd_packed(int op, const void* logits, int64_t ld_logit
 int spx_label_ce_fwd(const void* logits, int64_t ld_logits, const int64_t* labels,
                      int64_t rows, int64_t vocab, int dtype, int64_t ignore_index,
                      float* loss, float* lse, int32_t* argmax, void* stream);
+
+/* The label cross-entropy of rows whose log-sum-exp is known already (spx_gemm_bf16_nt_stats
+ * computes it in the head product's epilogue): loss[r] = lse[r] - logits[r, labels[r]], 0 for an
+ * ignored label, NaN for a label outside [0, vocab) -- the values spx_label_ce_fwd returns,
+ * with one element of every row read instead of the row (models/mtp/core.py:204-216). */
+int spx_label_ce_from_lse(const void* logits, int64_t ld_logits, const int64_t* labels,
+                          int64_t rows, int64_t vocab, int dtype, int64_t ignore_index,
+                          const float* lse, float* loss, void* stream);
 
 /* dlogits[r, j] = grad_rows[r] * (softmax(logits[r, :])[j] - [j == labels[r]]);
  * rows with grad_rows[r] == 0 or an ignored label are exact zeros and are not
@@ -476,6 +485,24 @@ int spx_swiglu_bwd(const void* gate, const void* up, const void* dout, void* dga
 int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb,
                      void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
                      void* stream);
+
+/* spx_gemm_bf16_nt whose epilogue also yields, per row m of c, the soft-max statistics of that
+ * row AS ROUNDED TO bf16: lse[m] = log sum_n exp(c[m, n]) (natural logarithm, fp32) and
+ * argmax[m] = the first n that attains max_n c[m, n] (-0 and +0 compare equal, as torch.argmax
+ * has it).  Either of lse and argmax may be null (not both): what is not asked for is not
+ * computed.  These are what the loss kernels otherwise compute by streaming c again:
+ * with them a cross-entropy against arg-max targets (losses/eager.py ce_loss; the eager
+ * reference takes argmax of the full target logits, models/eagle3/metrics.py:100-117) never
+ * needs the target logits in memory, and the full-vocabulary cross-entropy of MTP
+ * (models/mtp/core.py:190-226) needs lse[m] and one element of row m only.  This is the
+ * forward half of "lm_head + loss in one pass": c MAY BE NULL, then the product is reduced to
+ * its statistics and never written.  workspace: spx_gemm_stats_workspace_bytes(M, N) bytes
+ * (per-tile partial statistics, 12 bytes per row and 256 columns), 4-byte aligned, caller owned. */
+int64_t spx_gemm_stats_workspace_bytes(int64_t M, int64_t N);
+int spx_gemm_bf16_nt_stats(const void* a, int64_t lda, const void* b, int64_t ldb,
+                           void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                           float* lse, int32_t* argmax, void* workspace,
+                           int64_t workspace_bytes, void* stream);
 
 /* The same product with the number of rows of a (and c) that count read from device
  * memory at run time: rows >= min(M, *m_live) are neither read nor written.  For an

@@ -601,7 +601,10 @@ static int loss_fwd_impl(const char* fname, int op, const void* logits, int64_t 
   SPX_REQ_FN(dtype == SPX_DTYPE_BF16 || dtype == SPX_DTYPE_F32, "dtype must be bf16 or f32");
   SPX_REQ_FN(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "rows >= 0 and 0 < vocab < 2^31");
   const bool gather = sa.d2t != nullptr;
-  SPX_REQ_FN(ld_logits >= vocab && ld_targets >= (gather ? sa.vt : vocab), "row stride smaller than vocab");
+  // cross-entropy with the target rows' arg-max handed in reads no target element: the rows may be absent
+  const bool no_targets = !targets && reuse_target_stats && op == SPX_LOSS_CE && !gather;
+  SPX_REQ_FN(ld_logits >= vocab && (no_targets || ld_targets >= (gather ? sa.vt : vocab)),
+             "row stride smaller than vocab");
   SPX_REQ_FN(rows < (1ll << 31), "too many rows");
   if (gather) {
     SPX_REQ_FN(sa.vt > 0 && sa.vt < (1ll << 31), "0 < vt < 2^31");
@@ -614,7 +617,7 @@ static int loss_fwd_impl(const char* fname, int op, const void* logits, int64_t 
     SPX_REQ_FN(!sa.prev || kind_ok(sa.prev_kind), "unknown prev_correct element kind");
   }
   if (rows == 0) return SPX_OK;
-  SPX_REQ_FN(logits && targets && loss && lse_draft && lse_target && extra, "null buffer");
+  SPX_REQ_FN(logits && (targets || no_targets) && loss && lse_draft && lse_target && extra, "null buffer");
   // the second-pass reductions (rkl, jsd, tv) recompute from both rows anyway
   const bool known = reuse_target_stats && (op == SPX_LOSS_KL || op == SPX_LOSS_CE);
   if (known && op == SPX_LOSS_CE) SPX_REQ_FN(argmax_target, "ce with reused statistics needs argmax_target");
@@ -622,7 +625,7 @@ static int loss_fwd_impl(const char* fname, int op, const void* logits, int64_t 
   const int64_t per16 = dtype == SPX_DTYPE_BF16 ? 8 : 4;
   const bool vec = aligned16(logits) && ld_logits % per16 == 0 &&
                    (gather ? (!sa.gathered || (aligned16(sa.gathered) && sa.ld_gathered % per16 == 0))
-                           : (aligned16(targets) && ld_targets % per16 == 0));
+                           : (no_targets || (aligned16(targets) && ld_targets % per16 == 0)));
 #define SPX_GO(TT, VV, KK, GG)                                                                    \
   launch_fwd<TT, VV, KK, GG>(op, reinterpret_cast<const TT*>(logits), ld_logits,                  \
                              reinterpret_cast<const TT*>(targets), ld_targets, rows, vocab, loss, \

@@ -96,14 +96,20 @@ __device__ __forceinline__ int choose_k_parts(int n_tiles, int max_parts, int cu
   return best;
 }
 
-template <bool kImm>
+// kStats != 0: the epilogue also reduces every row of the tile to the soft-max statistics of its 256
+// bf16-rounded results -- the row maximum, with bit 0 of kStats sum_n 2^((c[m, n] - max) log2 e) and
+// with bit 1 the first column that holds the maximum -- and leaves them in stat_ws, laid out [3][tiles_n][M] (maxima as
+// float, sums as float, columns as int32); gemm_row_stats_reduce_kernel folds the tiles_n entries
+// of a row into log-sum-exp and arg-max.  C may then be null: the product itself is not stored
+// (a cross-entropy against arg-max targets needs nothing else of the target logits).
+template <bool kImm, int kStats = 0>
 __global__ __launch_bounds__(kGemmThreads, SPX_GEMM_MINW)
 __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf16_nt_kernel(
     const uint16_t* __restrict__ A, int64_t lda, const uint16_t* __restrict__ B, int64_t ldb,
     uint16_t* __restrict__ C, int64_t ldc, int M, int N, int K, int tiles_m, int tiles_n,
     const int32_t* __restrict__ m_live, const int32_t* __restrict__ tile_tab,
     const int32_t* __restrict__ group_off, int64_t b_group_stride, float* __restrict__ part_ws,
-    int max_parts, int cus) {
+    int max_parts, int cus, float* __restrict__ stat_ws = nullptr) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int M_host = M;
   // the row count may live on the device (rows packed to the front by the producer of A): the tile
@@ -328,15 +334,74 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   // block (q = lane / 16).  Swapping the words of the q-odd lanes for block j with those of the
   // q-even lanes for block j + 1 leaves every lane with 8 consecutive columns: 16-byte stores.
   const bool fast = (ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0) && (n0 + kTN <= N);
+  // kStats: (maximum, sum, first column) of this wave's 128 columns per row, lanes q == 0 -> LDS.
+  // The slab buffers are dead, but another wave's last (all-zero) global -> LDS loads may still be
+  // landing in them: everybody has waited for their own above, the barrier makes that mutual
+  float* const st_lds = reinterpret_cast<float*>(smem);  // [wave][3][128]
+  if constexpr (kStats != 0) __syncthreads();
+  const bool edge_n = n0 + kTN > N;
 #pragma unroll
   for (int i = 0; i < kMI; ++i) {
     const int m = m0 + wm + i * 16 + r16;
+    uint32_t pk[kNI][2];
+#pragma unroll
+    for (int j = 0; j < kNI; ++j) {
+      pk[j][0] = pack_bf16x2(acc[j][i][0], acc[j][i][1]);
+      pk[j][1] = pack_bf16x2(acc[j][i][2], acc[j][i][3]);
+    }
+    if constexpr (kStats != 0) {
+      // the 32 values of this lane, as the consumer of C reads them (rounded to bf16).  Every
+      // comparison below is a floating-point one: -0 and +0 are one value, as for torch.argmax
+      float v[kNI][4];
+#pragma unroll
+      for (int j = 0; j < kNI; ++j) {
+        v[j][0] = bf16_lo(pk[j][0]); v[j][1] = bf16_hi(pk[j][0]);
+        v[j][2] = bf16_lo(pk[j][1]); v[j][3] = bf16_hi(pk[j][1]);
+      }
+      const int nb = n0 + wn + 4 * q;  // column of v[j][r] = nb + 16 j + r
+      if (edge_n) {
+#pragma unroll
+        for (int j = 0; j < kNI; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[j][r] = (nb + 16 * j + r < N) ? v[j][r] : -INFINITY;
+      }
+      float mx = v[0][0];
+#pragma unroll
+      for (int j = 0; j < kNI; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mx = fmaxf(mx, v[j][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m2 = (mx == -INFINITY) ? 0.f : mx * kLog2e;  // (a half tile past the last column)
+      float z = 0.f;
+      int first = 0x7fffffff;
+      if constexpr ((kStats & 1) != 0) {
+#pragma unroll
+        for (int j = 0; j < kNI; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) z += fast_exp2(fmaf(v[j][r], kLog2e, -m2));
+        z += __shfl_xor(z, 16, 64);
+        z += __shfl_xor(z, 32, 64);
+      }
+      if constexpr ((kStats & 2) != 0) {
+        int loc = 128;  // column inside the lane's 128-column stripe (a constant per element); 128 = none
+#pragma unroll
+        for (int j = kNI - 1; j >= 0; --j)
+#pragma unroll
+          for (int r = 3; r >= 0; --r) loc = (v[j][r] == mx) ? 16 * j + r : loc;  // descending: the lowest stays
+        first = (loc < 128) ? nb + loc : 0x7fffffff;
+        first = min(first, __shfl_xor(first, 16, 64));
+        first = min(first, __shfl_xor(first, 32, 64));
+      }
+      if (q == 0) {
+        float* const d = st_lds + wave * 384 + i * 16 + r16;
+        d[0] = mx; d[128] = z; d[256] = __int_as_float(first);
+      }
+    }
+    if (kStats != 0 && C == nullptr) continue;
 #pragma unroll
     for (int j = 0; j < kNI; j += 2) {
-      const f32x4& a = acc[j][i];
-      const f32x4& b = acc[j + 1][i];
-      const uint32_t e0 = pack_bf16x2(a[0], a[1]), e1 = pack_bf16x2(a[2], a[3]);
-      const uint32_t o0 = pack_bf16x2(b[0], b[1]), o1 = pack_bf16x2(b[2], b[3]);
+      const uint32_t e0 = pk[j][0], e1 = pk[j][1], o0 = pk[j + 1][0], o1 = pk[j + 1][1];
       // odd rows of 16 lanes of the first operand <-> even rows of the second
       const auto s0 = __builtin_amdgcn_permlane16_swap(e0, o0, false, false);
       const auto s1 = __builtin_amdgcn_permlane16_swap(e1, o1, false, false);
@@ -355,6 +420,76 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
       }
     }
   }
+  if constexpr (kStats != 0) {
+    // the two waves that share a band of rows: the left one (lower columns) folds both halves
+    static_assert(kWN == 2 && kTM / kWM == 128, "two column halves per row band");
+    __syncthreads();
+    if (wn == 0) {
+      const float* const a = st_lds + wave * 384;
+      const float* const b = a + 384;  // wave + 1: the same rows, columns 128 .. 255
+#pragma unroll
+      for (int rr = lane; rr < 128; rr += 64) {
+        const int m = m0 + wm + rr;
+        if (m >= M) continue;
+        const float ma = a[rr], mb = b[rr];
+        const float mm = fmaxf(ma, mb);  // (ma is finite: the left half always has a column inside N)
+        const float z = a[128 + rr] * fast_exp2((ma - mm) * kLog2e) +
+                        ((mb == -INFINITY) ? 0.f : b[128 + rr] * fast_exp2((mb - mm) * kLog2e));
+        const int first = (mb > ma) ? __float_as_int(b[256 + rr]) : __float_as_int(a[256 + rr]);
+        const int64_t at = (int64_t)tile_n * M_host + m, plane = (int64_t)tiles_n * M_host;
+        stat_ws[at] = mm;
+        stat_ws[plane + at] = z;
+        reinterpret_cast<int32_t*>(stat_ws)[2 * plane + at] = first;
+      }
+    }
+  }
+}
+
+// Folds the per-tile statistics of gemm_bf16_nt_kernel<.., kStats> into one log-sum-exp (natural
+// logarithm) and one first-index arg-max per row: the tiles in ascending column order, a later
+// tile wins only with a strictly greater maximum.  A workgroup takes 32 rows; eight threads share a row,
+// each folds a contiguous eighth of the tiles (reads of one tile's entries are contiguous over the rows),
+// and the eight partial results are folded in their order through LDS.
+__global__ __launch_bounds__(256) void gemm_row_stats_reduce_kernel(const float* __restrict__ stat_ws, int M,
+                                                                    int tiles_n, float* __restrict__ lse,
+                                                                    int32_t* __restrict__ argmax) {
+  __shared__ float sm[8][32], sz[8][32];
+  __shared__ int si[8][32];
+  const int row = threadIdx.x & 31, part = threadIdx.x >> 5;
+  const int m = blockIdx.x * 32 + row;
+  const int64_t plane = (int64_t)tiles_n * M;
+  const int per = (tiles_n + 7) / 8;
+  const int t0 = part * per, t1 = min(t0 + per, tiles_n);
+  float mm = -INFINITY, z = 0.f;
+  int first = 0x7fffffff;
+  if (m < M) {
+    for (int t = t0; t < t1; ++t) {
+      const int64_t at = (int64_t)t * M + m;
+      const float pm = stat_ws[at], pz = stat_ws[plane + at];
+      if (pm > mm) {
+        z = z * fast_exp2((mm - pm) * kLog2e) + pz;  // (the first tile: 0 * 2^-inf)
+        mm = pm;
+        first = reinterpret_cast<const int32_t*>(stat_ws)[2 * plane + at];
+      } else {
+        z += pz * fast_exp2((pm - mm) * kLog2e);
+      }
+    }
+  }
+  sm[part][row] = mm; sz[part][row] = z; si[part][row] = first;
+  __syncthreads();
+  if (part != 0 || m >= M) return;
+  for (int p = 1; p < 8; ++p) {
+    const float pm = sm[p][row], pz = sz[p][row];
+    if (pm > mm) {
+      z = z * fast_exp2((mm - pm) * kLog2e) + pz;
+      mm = pm;
+      first = si[p][row];
+    } else if (pm != -INFINITY) {  // (a part with no tiles)
+      z += pz * fast_exp2((pm - mm) * kLog2e);
+    }
+  }
+  if (lse) lse[m] = (mm * kLog2e + fast_log2(z)) * kLn2;
+  if (argmax) argmax[m] = first;
 }
 
 // C[m, n .. n + 7] = the sum of the parts of a product whose contraction was cut (in the order of the
@@ -406,10 +541,10 @@ static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const voi
                         int64_t ldc, int64_t M, int64_t N, int64_t K, const int32_t* m_live, void* stream,
                         const int32_t* tile_tab = nullptr, const int32_t* group_off = nullptr,
                         int64_t b_group_stride = 0, int64_t groups = 0, float* part_ws = nullptr,
-                        int max_parts = 1) {
+                        int max_parts = 1, float* stat_ws = nullptr, int stats_mode = 0) {
   SPX_REQ_FN(M > 0 && N > 0 && K > 0, "M, N, K must be positive");
   SPX_REQ_FN(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "dimension too large");
-  SPX_REQ_FN(a && b && c, "null buffer");
+  SPX_REQ_FN(a && b && (c || stat_ws), "null buffer");
   SPX_REQ_FN(K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0, "K, lda, ldb must be multiples of 8");
   SPX_REQ_FN(lda >= K && ldb >= K && ldc >= N, "leading dimension too small");
   SPX_REQ_FN(((uintptr_t)a | (uintptr_t)b) % 16 == 0, "a and b must be 16-byte aligned");
@@ -417,10 +552,17 @@ static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const voi
              "256 rows of an operand must span less than 2 GiB (32-bit offsets inside a tile)");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool imm = lda >= kTK && ldb >= kTK;
-  static std::atomic<uint64_t> lds_set[2];  // per kernel instantiation, one bit per device
-  const void* fn = imm ? reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<true>)
-                       : reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<false>);
-  if (int rc = ensure_dynamic_lds(fn, kGemmSmem, lds_set[imm], fname)) return rc;
+  static std::atomic<uint64_t> lds_set[8];  // per kernel instantiation, one bit per device
+  const int which = (imm ? 1 : 0) + 2 * (stat_ws ? stats_mode : 0);
+  const void* const fns[8] = {reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<false, 0>),
+                              reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<true, 0>),
+                              reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<false, 1>),
+                              reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<true, 1>),
+                              reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<false, 2>),
+                              reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<true, 2>),
+                              reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<false, 3>),
+                              reinterpret_cast<const void*>(&gemm_bf16_nt_kernel<true, 3>)};
+  if (int rc = ensure_dynamic_lds(fns[which], kGemmSmem, lds_set[which], fname)) return rc;
   // grouped: every group may end in a partly filled tile row
   const int64_t tiles_m64 = (M + kTM - 1) / kTM + (tile_tab ? groups : 0);
   const int tiles_n = (int)((N + kTN - 1) / kTN);
@@ -430,16 +572,22 @@ static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const voi
   SPX_REQ_FN((int64_t)tiles_m * tiles_n * max_parts < (1ll << 31), "too many tiles");
   const int cus = compute_units();
   const dim3 grid((unsigned)(tiles_m * tiles_n * (part_ws ? max_parts : 1))), block(kGemmThreads);
-  if (imm)
-    hipLaunchKernelGGL(gemm_bf16_nt_kernel<true>, grid, block, kGemmSmem, st,
-                       reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,
-                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live,
-                       tile_tab, group_off, b_group_stride, part_ws, max_parts, cus);
-  else
-    hipLaunchKernelGGL(gemm_bf16_nt_kernel<false>, grid, block, kGemmSmem, st,
-                       reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,
-                       reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live,
-                       tile_tab, group_off, b_group_stride, part_ws, max_parts, cus);
+#define SPX_GEMM_LAUNCH(IMM, STATS)                                                                              \
+  hipLaunchKernelGGL((gemm_bf16_nt_kernel<IMM, STATS>), grid, block, kGemmSmem, st,                              \
+                     reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,       \
+                     reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live,      \
+                     tile_tab, group_off, b_group_stride, part_ws, max_parts, cus, stat_ws)
+  switch (which) {
+    case 0: SPX_GEMM_LAUNCH(false, 0); break;
+    case 1: SPX_GEMM_LAUNCH(true, 0); break;
+    case 2: SPX_GEMM_LAUNCH(false, 1); break;
+    case 3: SPX_GEMM_LAUNCH(true, 1); break;
+    case 4: SPX_GEMM_LAUNCH(false, 2); break;
+    case 5: SPX_GEMM_LAUNCH(true, 2); break;
+    case 6: SPX_GEMM_LAUNCH(false, 3); break;
+    default: SPX_GEMM_LAUNCH(true, 3); break;
+  }
+#undef SPX_GEMM_LAUNCH
   if (int rc = check_launch(fname)) return rc;
   if (part_ws) {
     const int64_t items = M * (N / 8);
@@ -515,6 +663,28 @@ extern "C" int spx_gemm_bf16_nt_grouped(const void* a, int64_t lda, const void* 
 extern "C" int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
                                 int64_t ldc, int64_t M, int64_t N, int64_t K, void* stream) {
   return gemm_nt_impl(__func__, a, lda, b, ldb, c, ldc, M, N, K, nullptr, stream);
+}
+
+extern "C" int64_t spx_gemm_stats_workspace_bytes(int64_t M, int64_t N) {
+  if (M <= 0 || N <= 0) return 0;
+  return 3 * ((N + kTN - 1) / kTN) * M * (int64_t)sizeof(float);
+}
+
+extern "C" int spx_gemm_bf16_nt_stats(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
+                                      int64_t ldc, int64_t M, int64_t N, int64_t K, float* lse,
+                                      int32_t* argmax, void* workspace, int64_t workspace_bytes,
+                                      void* stream) {
+  const char* fname = __func__;
+  SPX_REQ_FN(lse || argmax, "null lse and null argmax: nothing to compute");
+  SPX_REQ_FN(workspace && ((uintptr_t)workspace) % 4 == 0, "null or unaligned workspace");
+  SPX_REQ_FN(M > 0 && N > 0 && workspace_bytes >= spx_gemm_stats_workspace_bytes(M, N), "workspace too small");
+  if (int rc = gemm_nt_impl(fname, a, lda, b, ldb, c, c ? ldc : N, M, N, K, nullptr, stream, nullptr, nullptr, 0,
+                            0, nullptr, 1, reinterpret_cast<float*>(workspace), (lse ? 1 : 0) + (argmax ? 2 : 0)))
+    return rc;
+  hipLaunchKernelGGL(gemm_row_stats_reduce_kernel, dim3((unsigned)((M + 31) / 32)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const float*>(workspace), (int)M,
+                     (int)((N + kTN - 1) / kTN), lse, argmax);
+  return check_launch(fname);
 }
 
 extern "C" int64_t spx_gemm_split_workspace_bytes(int64_t M, int64_t N, int32_t max_parts) {

@@ -129,6 +129,25 @@ __global__ __launch_bounds__(kLossThreads) void label_ce_bwd_kernel(
   }
 }
 
+// loss[r] = lse[r] - x[r, label[r]] for rows whose log-sum-exp is already known (the statistics
+// epilogue of the head product, spx_gemm_bf16_nt_stats): one element of the row is read instead of
+// the row.  Ignored rows: loss 0; a label outside [0, vocab) that is not the ignore index: NaN,
+// as in label_ce_fwd_kernel.
+template <typename T>
+__global__ __launch_bounds__(256) void label_ce_pick_kernel(const T* __restrict__ logits, int64_t ld,
+                                                            const int64_t* __restrict__ labels, int64_t rows,
+                                                            int64_t vocab, int64_t ignore_index,
+                                                            const float* __restrict__ lse,
+                                                            float* __restrict__ loss) {
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= rows) return;
+  const int64_t label = labels[r];
+  float l = 0.f;
+  if (label != ignore_index)
+    l = (label >= 0 && label < vocab) ? lse[r] - load1(logits + r * ld + label) : __builtin_nanf("");
+  loss[r] = l;
+}
+
 }  // namespace spx
 
 using namespace spx;
@@ -159,6 +178,23 @@ extern "C" int spx_label_ce_fwd(const void* logits, int64_t ld_logits, const int
   if (dtype == SPX_DTYPE_BF16) { if (vec) SPX_LAUNCH(uint16_t, true); else SPX_LAUNCH(uint16_t, false); }
   else { if (vec) SPX_LAUNCH(float, true); else SPX_LAUNCH(float, false); }
 #undef SPX_LAUNCH
+  return check_launch(__func__);
+}
+
+extern "C" int spx_label_ce_from_lse(const void* logits, int64_t ld_logits, const int64_t* labels,
+                                     int64_t rows, int64_t vocab, int dtype, int64_t ignore_index,
+                                     const float* lse, float* loss, void* stream) {
+  if (int rc = label_ce_checks(__func__, logits, ld_logits, labels, rows, vocab, dtype)) return rc;
+  SPX_REQUIRE(loss && lse, "null buffer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)((rows + 255) / 256)), block(256);
+  if (dtype == SPX_DTYPE_BF16)
+    hipLaunchKernelGGL(label_ce_pick_kernel<uint16_t>, grid, block, 0, st,
+                       reinterpret_cast<const uint16_t*>(logits), ld_logits, labels, rows, vocab, ignore_index,
+                       lse, loss);
+  else
+    hipLaunchKernelGGL(label_ce_pick_kernel<float>, grid, block, 0, st, reinterpret_cast<const float*>(logits),
+                       ld_logits, labels, rows, vocab, ignore_index, lse, loss);
   return check_launch(__func__);
 }
 

@@ -330,8 +330,10 @@ class Eagle3DraftModel(nn.Module):
                     targets = (MT.TargetGather(compute_input(verifier_logits), self.d2t)
                                if self.use_draft_vocab else compute_input(verifier_logits))
                 else:
-                    targets = self._linear(self.verifier_norm(verifier_last_hidden_states),
-                                           self.verifier_lm_head.weight)
+                    # applied lazily: a cross-entropy loss takes the target rows' statistics from the
+                    # head product's epilogue and never sees the rows (metrics.VerifierHead)
+                    targets = MT.VerifierHead(self.verifier_norm(verifier_last_hidden_states),
+                                              self._stager.get(self.verifier_lm_head.weight).w)
             loss = torch.zeros((), device=device)
             prev_correct = (loss_mask.clone() if loss_mask is not None
                             else torch.ones(1, t, device=device, dtype=torch.bool))

@@ -86,6 +86,36 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
     return out
 
 
+def gemm_nt_stats(a: torch.Tensor, b: torch.Tensor, store: bool = True, want_argmax: bool = True,
+                  want_lse: bool = True):
+    """``gemm_nt(a, b)`` whose epilogue also reduces every row of the (bf16-rounded) product to its
+    soft-max statistics: returns ``(c [M, N] bf16 or None, lse [M] f32, argmax [M] i32 or None)``.
+    ``store=False``: the product is not written at all (``c`` is None) -- the statistics are all a
+    cross-entropy against arg-max targets needs of the verifier's logits."""
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
+        raise _lib.SpxError("gemm_nt_stats takes bf16 operands")
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise ValueError(f"shape mismatch: a {tuple(a.shape)} b {tuple(b.shape)}")
+    if a.stride(1) != 1:
+        a = a.contiguous()
+    if b.stride(1) != 1:
+        b = b.contiguous()
+    m, k = a.shape
+    n = b.shape[0]
+    dev = a.device
+    out = torch.empty(m, n, device=dev, dtype=torch.bfloat16) if store else None
+    if not (want_lse or want_argmax):
+        raise ValueError("gemm_nt_stats: ask for the log-sum-exp, the arg-max or both")
+    lse = torch.empty(m, device=dev, dtype=torch.float32) if want_lse else None
+    am = torch.empty(m, device=dev, dtype=torch.int32) if want_argmax else None
+    nbytes = _lib.load().spx_gemm_stats_workspace_bytes(m, n)
+    ws = torch.empty(nbytes // 4, device=dev, dtype=torch.float32)
+    _lib.call("spx_gemm_bf16_nt_stats", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
+              _lib.ptr(out), out.stride(0) if store else 0, m, n, k, _lib.ptr(lse), _lib.ptr(am), _lib.ptr(ws),
+              nbytes, _lib.stream_ptr(dev))
+    return out, lse, am
+
+
 _CUS = 256  # workgroups the chip runs at a time (one per compute unit for the GEMM kernels)
 
 

@@ -64,6 +64,11 @@ def fused_loss_forward(op: int, logits: torch.Tensor, targets: torch.Tensor, tar
     read the targets at all).  ``step``: see ``StepPass``; with ``step.d2t`` the returned
     ``targets2d`` are the gathered draft-vocabulary rows."""
     gather = step is not None and step.d2t is not None
+    if targets is None:
+        # cross-entropy against arg-max targets whose arg-max is known: no target row is read
+        if op != OP_CE or target_stats is None or gather:
+            raise ValueError("only ce with known target statistics runs without the target rows")
+        return _ce_without_targets(logits, target_stats, step)
     if not gather and logits.shape != targets.shape:
         raise ValueError(f"logits {tuple(logits.shape)} and targets {tuple(targets.shape)} differ")
     if gather and logits.shape[:-1] != targets.shape[:-1]:
@@ -114,6 +119,31 @@ def fused_loss_forward(op: int, logits: torch.Tensor, targets: torch.Tensor, tar
         _lib.stream_ptr(dev),
     )
     return stats[0], stats[1], lse_t, stats[3], arg[0], am_t, x, y
+
+
+def _ce_without_targets(logits, target_stats, step):
+    x = _rows_2d(logits)
+    rows, vocab = x.shape
+    dev = x.device
+    stats = torch.empty(4, rows, device=dev, dtype=torch.float32)
+    arg = torch.empty(1, rows, device=dev, dtype=torch.int32)
+    lse_t, am_t = target_stats[0].reshape(-1), target_stats[1].reshape(-1)
+    if lse_t.numel() != rows or am_t.numel() != rows or lse_t.stride(0) != 1 or am_t.stride(0) != 1:
+        raise ValueError("target_stats must be contiguous [rows] tensors")
+    if step is not None:
+        _lib.call(
+            "spx_vocab_loss_step_fwd", OP_CE, _lib.ptr(x), x.stride(0), None, 0, None, 0, None, 0, rows, vocab,
+            _lib.dtype_code(x), _lib.ptr(stats[0]), _lib.ptr(stats[1]), _lib.ptr(lse_t), _lib.ptr(stats[3]),
+            _lib.ptr(arg[0]), _lib.ptr(am_t), 1, _lib.ptr(step.mask),
+            _lib.kind_code(step.mask) if step.mask is not None else 0, _lib.ptr(step.prev),
+            _lib.kind_code(step.prev) if step.prev is not None else 0, _lib.ptr(step.counts),
+            _lib.stream_ptr(dev))
+    else:
+        _lib.call(
+            "spx_fused_vocab_loss_fwd", OP_CE, _lib.ptr(x), x.stride(0), None, 0, rows, vocab,
+            _lib.dtype_code(x), _lib.ptr(stats[0]), _lib.ptr(stats[1]), _lib.ptr(lse_t), _lib.ptr(stats[3]),
+            _lib.ptr(arg[0]), _lib.ptr(am_t), 1, _lib.stream_ptr(dev))
+    return stats[0], stats[1], lse_t, stats[3], arg[0], am_t, x, None
 
 
 class _FusedLoss(torch.autograd.Function):
@@ -240,8 +270,8 @@ def head_fused_rows(op: int, x, weight, weight_t, targets, target_stats=None, n_
         raise ValueError("x must be [1, T, H] (the packed batch layout)")
     t = x.shape[1]
     n = t if n_rows is None else int(n_rows)
-    y = _rows_2d(targets)
-    if y.shape[0] != n:
+    y = None if targets is None else _rows_2d(targets)
+    if y is not None and y.shape[0] != n:
         raise ValueError(f"targets have {y.shape[0]} rows, expected {n}")
     ks = (None, None) if target_stats is None else (target_stats[0], target_stats[1])
     loss, am_d, am_t, lse_t, logits = _HeadFusedLoss.apply(x[0], weight, weight_t, y, op, ks[0], ks[1], n,
@@ -402,15 +432,26 @@ class _HeadLabelCE(torch.autograd.Function):
     no gradient of their own."""
 
     @staticmethod
-    def forward(ctx, x2, weight, weight_t, labels, ignore_index):
-        from .gemm import gemm_nt
+    def forward(ctx, x2, weight, weight_t, labels, ignore_index, epilogue_stats=False):
+        from .gemm import gemm_nt, gemm_nt_stats
 
-        logits = gemm_nt(x2, weight)
-        rows, vocab = logits.shape
-        out = torch.empty(2, rows, device=logits.device, dtype=torch.float32)
-        _lib.call("spx_label_ce_fwd", _lib.ptr(logits), logits.stride(0), _lib.ptr(labels), rows,
-                  vocab, _lib.dtype_code(logits), int(ignore_index), _lib.ptr(out[0]),
-                  _lib.ptr(out[1]), None, _lib.stream_ptr(logits.device))
+        if epilogue_stats:
+            # the head product's epilogue leaves every row's log-sum-exp; the loss then reads one
+            # element of each row instead of streaming the [rows, V] logits a second time
+            logits, lse, _ = gemm_nt_stats(x2, weight, want_argmax=False)
+            rows, vocab = logits.shape
+            out = torch.empty(2, rows, device=logits.device, dtype=torch.float32)
+            out[1] = lse
+            _lib.call("spx_label_ce_from_lse", _lib.ptr(logits), logits.stride(0), _lib.ptr(labels), rows,
+                      vocab, _lib.dtype_code(logits), int(ignore_index), _lib.ptr(out[1]), _lib.ptr(out[0]),
+                      _lib.stream_ptr(logits.device))
+        else:
+            logits = gemm_nt(x2, weight)
+            rows, vocab = logits.shape
+            out = torch.empty(2, rows, device=logits.device, dtype=torch.float32)
+            _lib.call("spx_label_ce_fwd", _lib.ptr(logits), logits.stride(0), _lib.ptr(labels), rows,
+                      vocab, _lib.dtype_code(logits), int(ignore_index), _lib.ptr(out[0]),
+                      _lib.ptr(out[1]), None, _lib.stream_ptr(logits.device))
         ctx.save_for_backward(logits, labels, out[1], weight_t)
         ctx.ignore_index = int(ignore_index)
         ctx.mark_non_differentiable(logits)
@@ -422,7 +463,7 @@ class _HeadLabelCE(torch.autograd.Function):
         from .gemm import gemm_nt
 
         if grad_rows is None:
-            return (None,) * 5
+            return (None,) * 6
 
         logits, labels, lse, weight_t = ctx.saved_tensors
         rows, vocab = logits.shape
@@ -434,11 +475,22 @@ class _HeadLabelCE(torch.autograd.Function):
                   _lib.ptr(row_map), _lib.ptr(packed), packed.stride(0),
                   _lib.stream_ptr(logits.device))
         dx_packed = gemm_nt(packed, weight_t, m_live=count, split=True)
-        return _unpack_rows(dx_packed, row_map, rows), None, None, None, None
+        return _unpack_rows(dx_packed, row_map, rows), None, None, None, None, None
+
+
+# Whether the frozen-head cross-entropy takes its row statistics from the head product's epilogue
+# (spx_gemm_bf16_nt_stats, log-sum-exp only) instead of a streaming pass over the logits
+# (spx_label_ce_fwd).  Measured at the MTP head shape (32760 rows x 2048 -> 151936, 70 % live rows):
+# product + epilogue statistics + their reduction + one element per row 16.7 ms, product 15.9 ms +
+# streaming pass 1.25 ms = 17.2 ms; the iteration 199.1 against 200.4 ms.  (With the arg-max computed
+# too and a reduction of one thread per row the epilogue form LOST 1 ms per step: two compares per
+# element more on every row, with the matrix pipe idle, cost what the streaming pass costs.)
+HEAD_CE_EPILOGUE_STATS = True
 
 
 def head_label_cross_entropy(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor,
-                             labels: torch.Tensor, ignore_index: int = -100):
+                             labels: torch.Tensor, ignore_index: int = -100,
+                             epilogue_stats: bool | None = None):
     """``logits = x @ weight.T`` and ``F.cross_entropy(logits, labels, ignore_index=...,
     reduction="none")`` (models/mtp/core.py:190-216) for a FROZEN ``weight [V, H]`` whose
     transpose ``weight_t [H, V]`` the caller keeps: returns ``(loss [...] f32, logits [..., V])``.
@@ -453,7 +505,9 @@ def head_label_cross_entropy(x: torch.Tensor, weight: torch.Tensor, weight_t: to
         raise ValueError("weight_t must be the contiguous transpose of weight")
     x2 = x.reshape(-1, x.shape[-1])
     lab = labels.reshape(-1).to(torch.int64).contiguous()
-    loss, logits = _HeadLabelCE.apply(x2, weight, weight_t, lab, ignore_index)
+    if epilogue_stats is None:
+        epilogue_stats = HEAD_CE_EPILOGUE_STATS
+    loss, logits = _HeadLabelCE.apply(x2, weight, weight_t, lab, ignore_index, bool(epilogue_stats))
     return loss.view(labels.shape), logits.view(*labels.shape, weight.shape[0])
 
 

@@ -79,12 +79,42 @@ class TargetGather:
         return self.compact
 
 
+class VerifierHead:
+    """The frozen verifier head (``verifier_lm_head(verifier_norm(h))``, models/eagle3/core.py:250-253)
+    applied lazily, standing where ``compute_metrics`` takes the targets.  A cross-entropy loss needs
+    nothing of the target logits but their row arg-max (losses/eager.py ``ce_loss``), and the acceptance
+    metrics need the same: with that loss alone the head product is reduced to per-row statistics in its
+    own epilogue (``gemm.gemm_nt_stats(store=False)``) and the ``[T, Vd]`` target logits are never
+    written or read.  Any other loss gets them the ordinary way (``materialize``)."""
+
+    def __init__(self, x: torch.Tensor, weight: torch.Tensor):
+        if x.dim() != 3 or x.shape[0] != 1:
+            raise ValueError("verifier hidden states must be [1, T, H] (the packed batch layout)")
+        self.x, self.weight = x, weight
+        self.logits = None
+
+    def materialize(self) -> torch.Tensor:
+        from . import gemm
+
+        if self.logits is None:
+            self.logits = gemm.gemm_nt(self.x[0], self.weight).view(1, self.x.shape[1], self.weight.shape[0])
+        return self.logits
+
+    def stats(self):
+        """(lse [T] f32, argmax [T] i32) of the target rows; the rows themselves are not stored.  The
+        cross-entropy reads the arg-max only: the log-sum-exp is not computed (zeros stand in)."""
+        from . import gemm
+
+        _, _, am = gemm.gemm_nt_stats(self.x[0], self.weight, store=False, want_lse=False)
+        return torch.zeros(am.shape, device=am.device, dtype=torch.float32), am
+
+
 def _step_views(logits, targets, loss_mask, prev_correct, ttt_step):
     """align_for_step (models/eagle3/metrics.py:16-48): views only."""
     n = logits.shape[1] - ttt_step
     return (
         logits[:, :n],
-        targets[:, ttt_step:],
+        None if targets is None else targets[:, ttt_step:],
         None if loss_mask is None else loss_mask[:, ttt_step:],
         None if prev_correct is None else prev_correct[:, :n],
     )
@@ -145,6 +175,16 @@ def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
         if (targets.compact is None and ttt_step == 0 and name0 in L.PRIMITIVE_OP
                 and fn0 is L._HIP_LOSS_FN_MAP.get(name0)):
             gather, targets = targets, targets.full  # read through d2t inside the first loss pass
+        else:
+            targets = targets.materialize()
+    if isinstance(targets, VerifierHead):
+        (name0, (fn0, _w0)), = list(loss_config.items())[:1]
+        ce_only = (len(loss_config) == 1 and name0 == "ce" and fn0 is L._HIP_LOSS_FN_MAP.get("ce")
+                   and target_stats_cache is not None and targets.logits is None)
+        if ce_only:
+            if "ce" not in target_stats_cache:
+                target_stats_cache["ce"] = targets.stats()
+            targets = None  # every step reads the statistics; no target row exists
         else:
             targets = targets.materialize()
     s_logits, s_targets, s_mask, s_prev = _step_views(

@@ -514,3 +514,74 @@ def test_decoder_projections_on_the_library_gemm(monkeypatch):
         for k_ in ma:
             if k_.endswith("_total"):
                 assert torch.equal(ma[k_], mb[k_]), (other, k_)
+
+
+def test_cross_entropy_loss_never_materialises_the_verifier_logits(monkeypatch):
+    """With ``ce`` as the only loss the verifier head is reduced to per-row statistics in the
+    epilogue of its product (``metrics.VerifierHead`` -> ``spx_gemm_bf16_nt_stats`` with no output):
+    no ``[T, Vd]`` target tensor is made at any step.  Loss within 1e-3 of the fp32 oracle, the
+    ``_total`` counts exact, and against the same model with the target logits materialised: loss,
+    every metric, the draft tokens and every gradient bit for bit."""
+    from speculators_amd import losses as L
+    from speculators_amd import metrics as MT
+
+    shape = _shape(num_hidden_layers=2, norm_output=True)
+    w32 = OE.random_weights(shape, seed=4, std=0.05)
+    w = {k: v.bfloat16() for k, v in w32.items()}
+    t = 300
+    hs, ids, doc, mask, pos, vl = _batch(shape, t, 9, [150, 130])
+    args = (hs.bfloat16().cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.bfloat16().cuda())
+    cfg = L.resolve_loss_config("ce")
+
+    def run(model):
+        toks, loss, metrics = model(*args, ttt_steps=3, ttt_step_loss_decay=0.8, loss_config=cfg)
+        loss.backward()
+        return (loss.detach(), toks, metrics,
+                {k: p.grad.clone() for k, p in model.named_parameters() if p.grad is not None})
+
+    calls = {"materialize": 0, "stats": 0}
+    real_mat, real_stats = MT.VerifierHead.materialize, MT.VerifierHead.stats
+
+    def mat(self):
+        calls["materialize"] += 1
+        return real_mat(self)
+
+    def stats(self):
+        calls["stats"] += 1
+        return real_stats(self)
+
+    monkeypatch.setattr(MT.VerifierHead, "materialize", mat)
+    monkeypatch.setattr(MT.VerifierHead, "stats", stats)
+    got = run(_make(shape, w))
+    assert calls == {"materialize": 0, "stats": 1}
+
+    # the same with the target logits in memory (the statistics then come from the loss kernel's pass)
+    monkeypatch.setattr(MT.VerifierHead, "stats", lambda self: (_ for _ in ()).throw(AssertionError("unused")))
+    real_cm = MT.compute_metrics
+
+    def cm(logits, targets, *a, **kw):
+        if isinstance(targets, MT.VerifierHead):
+            targets = targets.materialize()
+        return real_cm(logits, targets, *a, **kw)
+
+    import speculators_amd.eagle3 as E3
+    monkeypatch.setattr(E3.MT, "compute_metrics", cm)
+    want = run(_make(shape, w))
+    assert calls["materialize"] == 3
+    assert torch.equal(got[0], want[0])
+    for a, b in zip(got[1], want[1]):
+        assert torch.equal(a, b)
+    assert got[2].keys() == want[2].keys()
+    for k in got[2]:
+        assert torch.equal(got[2][k], want[2][k]), k
+    assert got[3].keys() == want[3].keys() and len(got[3]) > 5
+    for k in got[3]:
+        assert torch.equal(got[3][k], want[3][k]), k
+
+    wf = {k: v.float() for k, v in w.items()}
+    _, rloss, rm = OE.eagle3_forward(wf, shape, hs.bfloat16().float(), ids, doc, mask, pos, vl.bfloat16().float(),
+                                     ttt_steps=3, ttt_step_loss_decay=0.8, loss_config=OL.resolve_loss_config("ce"))
+    assert abs(got[0].item() - rloss.item()) <= 1e-3 * abs(rloss.item())
+    for k in range(3):
+        assert got[2][f"full_acc_{k}_total"].item() == rm[f"full_acc_{k}_total"].item()
+        assert got[2][f"cond_acc_{k}_total"].item() == rm[f"cond_acc_{k}_total"].item()

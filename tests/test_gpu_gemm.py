@@ -331,3 +331,93 @@ def test_weight_gradient_of_unaligned_operands_takes_the_library_product(m, n):
     assert weights._tn_ok(dy8) and weights._tn_ok(x8)
     got8 = weights.wgrad_product(dy8, x8, None)
     assert (got8[:m, :n].double() - want).abs().max() <= 1e-5 * want.abs().max() + 1e-6
+
+
+def _stats_reference(c):
+    """(lse, first-index arg-max) of bf16 rows, the way the streaming loss kernels see them."""
+    cf = c.float()
+    return torch.logsumexp(cf.double(), -1), cf.argmax(-1)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (300, 1000, 136), (512, 32000, 256), (130, 2432, 512),
+                                   (700, 151936, 64)])
+def test_gemm_with_row_statistics_in_the_epilogue(m, n, k):
+    """``spx_gemm_bf16_nt_stats``: the product is the plain product bit for bit; per row the
+    log-sum-exp of the bf16-rounded results (1e-6 relative against float64 and against the
+    streaming label-CE kernel's) and their first-index arg-max (exact, ``torch.argmax`` and the
+    kernel's); with the product not stored the statistics are the same bits.  Shapes: one tile,
+    ragged edges in both directions, a last tile whose right half lies past the last column
+    (2432 = 9.5 tiles; 151936 = 593.5), the two vocabulary sizes."""
+    from speculators_amd import _lib
+    from speculators_amd.gemm import gemm_nt, gemm_nt_stats
+
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).bfloat16().cuda()
+    b = (torch.randn(n, k, generator=g) * (4.0 / k ** 0.5)).bfloat16().cuda()
+    plain = gemm_nt(a, b)
+    c, lse, am = gemm_nt_stats(a, b)
+    assert torch.equal(c.view(torch.int16), plain.view(torch.int16))
+    want_lse, want_am = _stats_reference(c)
+    assert torch.equal(am.long(), want_am)
+    assert ((lse.double() - want_lse).abs() <= 1e-6 * want_lse.abs() + 1e-6).all()
+    # the two-kernel path: the streaming kernel over the stored product
+    labels = torch.zeros(m, dtype=torch.int64, device="cuda")
+    out = torch.empty(2, m, device="cuda")
+    am2 = torch.empty(m, device="cuda", dtype=torch.int32)
+    _lib.call("spx_label_ce_fwd", _lib.ptr(c), c.stride(0), _lib.ptr(labels), m, n, _lib.dtype_code(c), -100,
+              _lib.ptr(out[0]), _lib.ptr(out[1]), _lib.ptr(am2), _lib.stream_ptr(c.device))
+    assert torch.equal(am, am2)
+    assert ((lse - out[1]).abs() <= 1e-6 * out[1].abs() + 1e-6).all()
+    none, lse3, am3 = gemm_nt_stats(a, b, store=False)
+    assert none is None and torch.equal(lse3, lse) and torch.equal(am3, am)
+    # only one of the two asked for: the same bits as when both are computed
+    _, lse4, no_am = gemm_nt_stats(a, b, want_argmax=False)
+    assert no_am is None and torch.equal(lse4, lse)
+    _, no_lse, am5 = gemm_nt_stats(a, b, store=False, want_lse=False)
+    assert no_lse is None and torch.equal(am5, am)
+
+
+def test_row_statistics_break_ties_towards_the_first_column():
+    """Equal maxima in one row -- inside a lane's columns, across the lanes of a wave, across the two
+    waves of a tile and across tiles -- resolve to the lowest column; -0 and +0 are one value."""
+    from speculators_amd.gemm import gemm_nt_stats
+
+    g = torch.Generator().manual_seed(5)
+    m, k, n = 64, 64, 1024
+    a = torch.randn(m, k, generator=g).bfloat16().cuda()
+    b = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    big = (torch.randn(k, generator=g) * 2).bfloat16()
+    # duplicates of one strong column at distances that cross each of the boundaries
+    for cols in ([5, 6], [40, 41 + 16], [100, 100 + 128], [200, 200 + 256, 900], [1023, 3]):
+        bb = b.clone()
+        bb[cols] = big
+        c, _, am = gemm_nt_stats(a, bb.cuda())
+        cf = c.float()
+        assert torch.equal(am.long(), cf.argmax(-1))
+        rows_won = (am.long() == min(cols)).sum().item()
+        assert rows_won > 0  # the duplicated column wins some rows, and then always at its first copy
+        assert not torch.isin(am.long(), torch.tensor(sorted(cols)[1:], device="cuda")).any()
+    # an all-zero product: every element ties (and a sign of zero must not matter)
+    c, lse, am = gemm_nt_stats(torch.zeros(m, k).bfloat16().cuda(), b.cuda())
+    assert (am == 0).all() and torch.allclose(lse, torch.full_like(lse, float(torch.log(torch.tensor(float(n))))))
+    neg = a.clone()
+    bz = torch.zeros(n, k).bfloat16()
+    bz[7, 0] = -0.0
+    c, _, am = gemm_nt_stats(neg, bz.cuda())
+    assert (am == 0).all()
+
+
+def test_gemm_stats_rejects_bad_arguments():
+    from speculators_amd import _lib
+
+    lib = _lib.load()
+    a = torch.zeros(256, 64, device="cuda", dtype=torch.bfloat16)
+    lse = torch.empty(256, device="cuda")
+    ws = torch.empty(16, device="cuda")
+    assert lib.spx_gemm_stats_workspace_bytes(256, 300) == 3 * 2 * 256 * 4
+    rc = lib.spx_gemm_bf16_nt_stats(_lib.ptr(a), 64, _lib.ptr(a), 64, None, 0, 256, 256, 64, _lib.ptr(lse), None,
+                                    _lib.ptr(ws), 64, None)
+    assert rc == 1 and b"workspace too small" in lib.spx_last_error()
+    rc = lib.spx_gemm_bf16_nt_stats(_lib.ptr(a), 64, _lib.ptr(a), 64, None, 0, 256, 256, 64, None, None,
+                                    _lib.ptr(ws), 1 << 20, None)
+    assert rc == 1 and b"null lse and null argmax" in lib.spx_last_error()

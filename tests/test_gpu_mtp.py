@@ -301,7 +301,9 @@ def test_model_properties_of_the_reference_tests():
 def test_head_and_loss_as_one_node_equals_the_two_node_path():
     """Frozen head + label cross-entropy as one autograd node (packed loss backward, row-counted
     input-gradient product) against linear + label_cross_entropy: same losses, same logits, and
-    the same input gradient bit for bit -- zero rows included."""
+    the same input gradient bit for bit -- zero rows included.  (With the row statistics taken from
+    the head product's epilogue the log-sum-exp is summed in another order: that form is compared in
+    test_head_cross_entropy_with_epilogue_statistics_equals_the_streaming_form.)"""
     from speculators_amd import gemm
     from speculators_amd import losses as L
 
@@ -318,7 +320,7 @@ def test_head_and_loss_as_one_node_equals_the_two_node_path():
     gw[1, 7] = 0.0                  # a live label with a zero incoming gradient
 
     x1 = x.clone().requires_grad_(True)
-    loss1, logits1 = L.head_label_cross_entropy(x1, w, wt, labels)
+    loss1, logits1 = L.head_label_cross_entropy(x1, w, wt, labels, epilogue_stats=False)
     (loss1 * gw).sum().backward()
     x2 = x.clone().requires_grad_(True)
     logits2 = gemm.linear(x2, w, wt)
@@ -351,10 +353,14 @@ def test_head_and_loss_node_with_no_or_all_rows_live(frac):
         assert torch.isfinite(x.grad.float()).all() and (x.grad != 0).any()
 
 
-def test_model_with_and_without_the_fused_head_node_agree():
+def test_model_with_and_without_the_fused_head_node_agree(monkeypatch):
     """The MTP model's loss, logits and parameter gradients do not depend on whether the head and
     the loss are one autograd node or two (bit for bit: the packed product computes the same
-    dot products in the same order)."""
+    dot products in the same order; the row statistics streamed in both, not taken from the head
+    product's epilogue, whose sum runs in another order)."""
+    from speculators_amd import losses as L
+
+    monkeypatch.setattr(L, "HEAD_CE_EPILOGUE_STATS", False)
     shape = _shape()
     steps = 2
     w = {k: v.bfloat16() for k, v in OM.random_weights(shape, seed=4, std=0.05).items()}
@@ -377,3 +383,39 @@ def test_model_with_and_without_the_fused_head_node_agree():
     assert got[0][2].keys() == got[1][2].keys() and len(got[0][2]) > 0
     for k in got[0][2]:
         assert torch.equal(got[0][2][k], got[1][2][k]), k
+
+
+@pytest.mark.parametrize("rows,hidden,vocab", [(300, 128, 5000), (520, 256, 151936)])
+def test_head_cross_entropy_with_epilogue_statistics_equals_the_streaming_form(rows, hidden, vocab):
+    """The frozen head + label cross-entropy node with the row log-sum-exp taken from the head
+    product's epilogue (``spx_gemm_bf16_nt_stats`` + ``spx_label_ce_from_lse``) against the form
+    that streams the logits again (``spx_label_ce_fwd``): same logits bit for bit, losses within
+    1e-6 relative (exact zeros at ignored labels, NaN at a bad label in both), input gradients within
+    the rounding of one bf16 step, and the loss against ``F.cross_entropy`` on the same logits."""
+    from speculators_amd import losses as L
+
+    g = torch.Generator().manual_seed(rows)
+    x = torch.randn(rows, hidden, generator=g).bfloat16().cuda()
+    w = (torch.randn(vocab, hidden, generator=g) * 0.05).bfloat16().cuda()
+    wt = w.t().contiguous()
+    labels = torch.randint(0, vocab, (rows,), generator=g)
+    labels[::7] = -100
+    labels = labels.cuda()
+    gr = torch.randn(rows, generator=g).cuda()
+    res = []
+    for epi in (True, False):
+        xi = x.clone().requires_grad_(True)
+        loss, logits = L.head_label_cross_entropy(xi, w, wt, labels, -100, epilogue_stats=epi)
+        (loss * gr).sum().backward()
+        res.append((loss.detach(), logits, xi.grad))
+    (la, ga, da), (lb, gb, db) = res
+    assert torch.equal(ga.view(torch.int16), gb.view(torch.int16))
+    assert (la[::7] == 0).all() and (lb[::7] == 0).all()
+    assert ((la - lb).abs() <= 1e-6 * lb.abs() + 1e-6).all()
+    ref = torch.nn.functional.cross_entropy(ga.float(), labels, ignore_index=-100, reduction="none")
+    assert ((la - ref).abs() <= 2e-6 * ref.abs() + 2e-6).all()
+    assert (da.float() - db.float()).abs().max() <= 1e-2 * db.float().abs().max()
+    bad = labels.clone()
+    bad[1] = vocab + 3
+    lo, _ = L.head_label_cross_entropy(x, w, wt, bad, -100, epilogue_stats=True)
+    assert torch.isnan(lo[1]) and torch.isfinite(lo[2])
