@@ -294,7 +294,7 @@ def kernel_rooflines(torch, cfg, t, k_steps, device, windows=(None,)):
     ms = time_events(torch, lambda: gemm_nt_stats(x, w, store=True), 20)
     mfma("gemm_bf16_nt_kernel<statistics epilogue> + reduce[verifier head T x H x Vd, product stored]",
          2.0 * t * h * vd, ms, 0)
-    ms = time_events(torch, lambda: gemm_nt_stats(x, w, store=False), 20)
+    ms = time_events(torch, lambda: gemm_nt_stats(x, w, store=False, want_lse=False), 20)
     mfma("gemm_bf16_nt_kernel<statistics epilogue> + reduce[verifier head T x H x Vd, statistics only: ce targets]",
          2.0 * t * h * vd, ms, 0)
     wt = w.t().contiguous()
