@@ -341,6 +341,259 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
   }
 }
 
+// ---- forward with the d2t gather, pipelined ------------------------------------------------------
+// The first step of a TTT loop whose targets arrive as full-vocabulary verifier logits: the same row pass
+// as loss_fwd_kernel<.., GATHER> (gather through d2t, both online soft-maxes, KL or CE, both arg-maxes,
+// the gathered row written out, the acceptance chain), arranged so that nothing waits for memory:
+//   * the draft ids are walked in tiles of 2048; the ascending span [lo, hi) of the full row that a tile
+//     maps to is known for every tile before the loop starts (a table in LDS, built from 2 table reads
+//     per tile), so the span of tile t + 2 and that tile's piece of the draft row are requested -- global
+//     -> LDS directly, no registers -- while tile t is reduced: a ring of three slots, one workgroup
+//     barrier per tile, a fixed number of loads per wave and tile so that one s_waitcnt constant tells
+//     when a slot has landed;
+//   * picking element i + d2t[i] out of the staged span is done with lane = id (consecutive lanes read
+//     LDS addresses a few bytes apart: about two lanes per bank) instead of lane = chunk of 8 ids (lanes
+//     64 bytes apart: 16 lanes per bank); each wave then turns its 512 picks into 8-id chunks through a
+//     1 KB LDS strip of its own, so the gathered row is written 16 bytes per lane;
+//   * a tile whose span does not fit a slot (a table that is not spread evenly) reads its elements
+//     from global memory directly, as the general kernel does.
+// bf16 rows, 16-byte aligned, KL or CE; everything else stays with loss_fwd_kernel<.., GATHER>.
+constexpr int kPipeTileIds = kLossThreads * 8;        // 2048 draft ids per tile
+constexpr int kPipeSpanLoads = 5;                     // 1 KB wave-loads per wave and span
+constexpr int kPipeCap = kPipeSpanLoads * kLossWaves * 512;  // 10240 elements of the full row per slot
+constexpr int kPipeSlotBytes = kPipeCap * 2 + kPipeTileIds * 2;  // span + the tile's draft-row piece
+constexpr int kPipeSlots = 3;
+constexpr int kPipeMaxTiles = 128;                    // draft vocabulary <= 262144
+constexpr int kPipeOffY = kPipeSlots * kPipeSlotBytes;  // byte offsets inside the dynamic LDS block
+constexpr int kPipeOffSpan = kPipeOffY + kPipeTileIds * 2;
+constexpr int kPipeSmem = kPipeOffSpan + kPipeMaxTiles * 2 * 4;
+static_assert(2 * kPipeSmem + 1024 <= 160 * 1024, "two workgroups per compute unit");
+
+template <int OP>
+__global__ __launch_bounds__(kLossThreads) void loss_fwd_gather_pipe_kernel(
+    const uint16_t* __restrict__ logits, int64_t ld_logits, const uint16_t* __restrict__ targets,
+    int64_t ld_targets, int64_t vocab, float* __restrict__ loss, float* __restrict__ lse_draft,
+    float* __restrict__ lse_target, float* __restrict__ extra, int32_t* __restrict__ argmax_draft,
+    int32_t* __restrict__ argmax_target, StepArgs sa) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t psm[];
+  uint16_t* const ybuf = reinterpret_cast<uint16_t*>(psm + kPipeOffY);  // [4 waves][512]
+  int* const span = reinterpret_cast<int*>(psm + kPipeOffSpan);         // [tiles][2]: lo, length (-1: direct)
+  const int64_t r = blockIdx.x;
+  const uint16_t* xrow = logits + r * ld_logits;
+  const uint16_t* yrow = targets + r * ld_targets;
+  uint16_t* grow = sa.gathered ? reinterpret_cast<uint16_t*>(sa.gathered) + r * sa.ld_gathered : nullptr;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ntiles = (int)((vocab + kPipeTileIds - 1) / kPipeTileIds);
+
+  for (int t = tid; t < ntiles; t += kLossThreads) {
+    const int64_t i0 = (int64_t)t * kPipeTileIds, i1 = min(vocab, i0 + kPipeTileIds) - 1;
+    int64_t lo = i0 + sa.d2t[i0], hi = i1 + sa.d2t[i1] + 1;
+    lo = max((int64_t)0, min(lo, sa.vt)) & ~(int64_t)7;
+    hi = max(lo, min(hi, sa.vt));
+    span[2 * t] = (int)lo;
+    span[2 * t + 1] = (hi - lo <= kPipeCap) ? (int)(hi - lo) : -1;
+  }
+  __syncthreads();
+
+  constexpr int kOob = 0x7ffffff0;  // an offset outside every resource: the lane writes zeros, nothing is fetched
+  const u32x4 yres = make_rsrc(yrow, (uint32_t)(sa.vt * 2));
+  const u32x4 xres = make_rsrc(xrow, (uint32_t)(vocab * 2));
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)psm;
+  // tile u into slot u % 3: kPipeSpanLoads wave-loads of the span (the four waves interleaved, lanes past
+  // the span's end switched off) and one of this wave's 512 ids of the draft row -- always six loads
+  // (a tile past the last one: six loads all the same, every lane switched off)
+  auto request = [&](int u) __attribute__((always_inline)) {
+    const bool live = u < ntiles;
+    const int lo = live ? span[2 * u] : 0, len = live ? span[2 * u + 1] : -1;
+    const uint32_t dst = lds0 + (u % kPipeSlots) * kPipeSlotBytes;
+#pragma unroll
+    for (int k = 0; k < kPipeSpanLoads; ++k) {
+      const int e = (k * kLossWaves + wave) * 512 + lane * 8;
+      load_to_lds16<0>(yres, dst + (k * kLossWaves + wave) * 1024, e < len ? (lo + e) * 2 : kOob, 0);
+    }
+    const int64_t xb = (int64_t)u * kPipeTileIds + wave * 512 + lane * 8;
+    load_to_lds16<0>(xres, dst + kPipeCap * 2 + wave * 1024, xb < vocab ? (int)(xb * 2) : kOob, 0);
+  };
+  // The table entries of this lane's 8 picks of tile u (lane = id inside the wave's 512 ids; the low
+  // words of the int64 offsets: |d2t| < 2^31).  The loads are statements the compiler does not look
+  // into, like the span requests: it would otherwise guard their first use with a wait that also
+  // covers every span request issued since (it does not count those), and the ring would run one
+  // tile deep.  Their registers must not be read before `landed` has named them.
+  auto load_offsets = [&](int u, int (&d)[8]) __attribute__((always_inline)) {
+    const int64_t wbase = (int64_t)u * kPipeTileIds + wave * 512;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int64_t id = min(wbase + lane + 64 * k, vocab - 1);
+      const int32_t* const ptr = reinterpret_cast<const int32_t*>(sa.d2t + id);
+      asm volatile("global_load_dword %0, %1, off" : "=v"(d[k]) : "v"(ptr) : "memory");
+    }
+  };
+  // all vector-memory operations but the newest six have completed; d is what the wait releases.
+  // (No branch may stand between a load_offsets and the `landed` that names its registers: a merge of
+  // two paths lets the compiler copy the registers, and a copy made before the wait copies stale data.)
+  auto landed = [&](int (&d)[8]) __attribute__((always_inline)) {
+    asm volatile("s_waitcnt vmcnt(6)"
+                 : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]), "+v"(d[4]), "+v"(d[5]), "+v"(d[6]), "+v"(d[7])
+                 :: "memory");
+  };
+
+  RowStats s;
+  s.md = kNegBig; s.zd = 0.f; s.mt = kNegBig; s.zt = 0.f; s.at = 0.f;
+  s.bd = -INFINITY; s.id = 0x7fffffff; s.bt = -INFINITY; s.it = 0x7fffffff; s.xt = 0.f;
+
+  // One tile.  Order of the vector-memory operations (they complete in order): offsets(0), slot(0),
+  // slot(1), and per tile t: offsets(t + 1), the gathered row's store of t, slot(t + 2) -- every tile,
+  // also those past the last one, whose loads fetch nothing.  At the top of tile t the six newest are
+  // slot(t + 1): waiting for all but six says offsets(t) and slot(t) are in
+  auto tile = [&](int t, int (&cur)[8], int (&nxt)[8]) __attribute__((always_inline)) {
+    landed(cur);
+    __syncthreads();  // every wave's part of slot(t) has landed, every wave is done with slot(t - 1)
+    load_offsets(t + 1, nxt);
+    const bool live = t < ntiles;
+    const int lo = live ? span[2 * t] : 0, len = live ? span[2 * t + 1] : -1;
+    const uint8_t* const slot = psm + (t % kPipeSlots) * kPipeSlotBytes;
+    const uint16_t* const buf = reinterpret_cast<const uint16_t*>(slot);
+    const int64_t wbase = (int64_t)t * kPipeTileIds + wave * 512;
+    uint16_t* const ystrip = ybuf + wave * 512;
+    // (32-bit arithmetic: ids and columns are below 2^30 here)
+    const int id0 = (int)wbase + lane, nvocab = (int)vocab, nvt = (int)sa.vt;
+    const unsigned ulen = len > 0 ? (unsigned)len : 0u;
+    const int slot_lo = -lo;
+    bool need = false;  // some pick of this lane is not in the staged span
+    int rel[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      rel[k] = id0 + 64 * k + cur[k] + slot_lo;  // column - lo
+      const bool staged = (unsigned)rel[k] < ulen;
+      need |= (id0 + 64 * k < nvocab) && !staged;
+      ystrip[lane + 64 * k] = buf[staged ? rel[k] : 0];
+    }
+    if (__any(need)) {  // (wave-uniform: the common case issues no global load here)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int j = rel[k] + lo;
+        if ((id0 + 64 * k < nvocab) && !((unsigned)rel[k] < ulen))  // -inf: a column outside the full row
+          ystrip[lane + 64 * k] = ((unsigned)j < (unsigned)nvt) ? yrow[j] : (uint16_t)0xff80;
+      }
+    }
+    // the strip is private to the wave: its own writes, in order, then its own reads
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int64_t base = wbase + lane * 8;
+    const u32x4 yraw = *reinterpret_cast<const u32x4*>(ystrip + lane * 8);
+    const u32x4 xraw = *reinterpret_cast<const u32x4*>(slot + kPipeCap * 2 + wave * 1024 + lane * 16);
+    if (grow && base + 8 <= vocab) st16(grow + base, yraw);
+    request(t + 2);
+    if (base < vocab) {
+      float x[8], y[8];
+      x[0] = bf16_lo(xraw.x); x[1] = bf16_hi(xraw.x); x[2] = bf16_lo(xraw.y); x[3] = bf16_hi(xraw.y);
+      x[4] = bf16_lo(xraw.z); x[5] = bf16_hi(xraw.z); x[6] = bf16_lo(xraw.w); x[7] = bf16_hi(xraw.w);
+      y[0] = bf16_lo(yraw.x); y[1] = bf16_hi(yraw.x); y[2] = bf16_lo(yraw.y); y[3] = bf16_hi(yraw.y);
+      y[4] = bf16_lo(yraw.z); y[5] = bf16_hi(yraw.z); y[6] = bf16_lo(yraw.w); y[7] = bf16_hi(yraw.w);
+      if (base + 8 > vocab) {  // the draft vocabulary ends inside this chunk (the last tile only)
+        const uint32_t yw[4] = {yraw.x, yraw.y, yraw.z, yraw.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if (base + i < vocab) {
+            if (grow) grow[base + i] = (uint16_t)(yw[i >> 1] >> (16 * (i & 1)));
+          } else {
+            x[i] = kNegBig; y[i] = kNegBig;  // tail padding, like load8_guard
+          }
+        }
+      }
+      float cx = x[0], cy = y[0];
+#pragma unroll
+      for (int i = 1; i < 8; ++i) { cx = fmaxf(cx, x[i]); cy = fmaxf(cy, y[i]); }
+      if (cx > s.bd) {  // strict: an earlier chunk of this thread keeps a tie
+        int k = 7;
+#pragma unroll
+        for (int i = 6; i >= 0; --i) k = (x[i] == cx) ? i : k;
+        s.bd = cx; s.id = (int)base + k;
+      }
+      if (cy > s.bt) {
+        int k = 7;
+        float xv = x[7];
+#pragma unroll
+        for (int i = 6; i >= 0; --i) {
+          const bool hit = y[i] == cy;
+          k = hit ? i : k;
+          xv = hit ? x[i] : xv;
+        }
+        s.bt = cy; s.it = (int)base + k; s.xt = xv;
+      }
+      {
+        const float cxs = cx * kLog2e;
+        float mn = s.md, z = s.zd;
+        if (cxs > mn) {
+          z *= fast_exp2(mn - cxs);
+          mn = cxs;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) z += fast_exp2(fmaf(x[i], kLog2e, -mn));
+        s.zd = z; s.md = mn;
+      }
+      if (OP != SPX_LOSS_CE) {
+        float mn = fmaxf(s.mt, cy * kLog2e);
+        float rs = fast_exp2(s.mt - mn);
+        float z = s.zt * rs, a = s.at * rs;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float e = fast_exp2(fmaf(y[i], kLog2e, -mn));
+          z += e;
+          a = fmaf(e, y[i] - x[i], a);
+        }
+        s.zt = z; s.at = a; s.mt = mn;
+      }
+    }
+  };
+
+  int off_a[8], off_b[8];
+  load_offsets(0, off_a);
+  request(0);
+  request(1);
+  // two tiles per trip: the two register sets swap roles, nothing is copied; an odd tile count runs one
+  // tile past the end (all of its work is switched off by its ids)
+  for (int t = 0; t < ntiles; t += 2) {
+    tile(t, off_a, off_b);
+    tile(t + 1, off_b, off_a);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the requests past the end still write LDS
+  __syncthreads();
+
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) merge(s, shuffle_xor(s, m));
+  __shared__ RowStats part[kLossWaves];
+  if (lane == 0) part[wave] = s;
+  __syncthreads();
+  s = part[0];
+#pragma unroll
+  for (int w = 1; w < kLossWaves; ++w) merge(s, part[w]);
+  const float lse_d = (s.md + fast_log2(s.zd)) * kLn2;
+  const float lse_t = (OP != SPX_LOSS_CE) ? (s.mt + fast_log2(s.zt)) * kLn2 : 0.f;
+  float row_loss;
+  if (OP == SPX_LOSS_KL) row_loss = s.at / s.zt - lse_t + lse_d;
+  else row_loss = lse_d - s.xt;
+  if (tid == 0) {
+    loss[r] = row_loss;
+    lse_draft[r] = lse_d;
+    extra[r] = (OP == SPX_LOSS_KL) ? row_loss : 0.f;
+    if (argmax_draft) argmax_draft[r] = s.id;
+    lse_target[r] = lse_t;
+    if (argmax_target) argmax_target[r] = s.it;
+    if (sa.counts) {
+      const bool m = sa.mask ? mask_value(sa.mask, sa.mask_kind, r) != 0.f : true;
+      const bool was = sa.prev ? mask_value(sa.prev, sa.prev_kind, r) != 0.f : true;
+      const bool now = was && (s.id == s.it);
+      if (m && now) atomicAdd(&sa.counts[0], 1);
+      if (m) atomicAdd(&sa.counts[1], 1);
+      if (was) atomicAdd(&sa.counts[2], 1);
+      if (sa.prev) store_flag(sa.prev, sa.prev_kind, r, now);
+    }
+  }
+}
+
 // ---- backward --------------------------------------------------------------
 template <typename T, int OP, bool VEC>
 __global__ __launch_bounds__(kLossThreads) void loss_bwd_kernel(
@@ -626,6 +879,26 @@ static int loss_fwd_impl(const char* fname, int op, const void* logits, int64_t 
   const bool vec = aligned16(logits) && ld_logits % per16 == 0 &&
                    (gather ? (!sa.gathered || (aligned16(sa.gathered) && sa.ld_gathered % per16 == 0))
                            : (no_targets || (aligned16(targets) && ld_targets % per16 == 0)));
+  // the first step of the verifier-logits entry in its common form: the pipelined kernel
+  if (gather && vec && dtype == SPX_DTYPE_BF16 && (op == SPX_LOSS_KL || op == SPX_LOSS_CE) &&
+      aligned16(targets) && ld_targets % 8 == 0 && vocab <= (int64_t)kPipeMaxTiles * kPipeTileIds &&
+      sa.vt < (1ll << 30)) {
+    static std::atomic<uint64_t> lds_set[2];  // per instantiation, one bit per device
+    const bool kl = op == SPX_LOSS_KL;
+    const void* fn = kl ? reinterpret_cast<const void*>(&loss_fwd_gather_pipe_kernel<SPX_LOSS_KL>)
+                        : reinterpret_cast<const void*>(&loss_fwd_gather_pipe_kernel<SPX_LOSS_CE>);
+    if (int rc = ensure_dynamic_lds(fn, kPipeSmem, lds_set[kl], fname)) return rc;
+    const dim3 grid((unsigned)rows), block(kLossThreads);
+    auto lg = reinterpret_cast<const uint16_t*>(logits);
+    auto tg = reinterpret_cast<const uint16_t*>(targets);
+    if (kl)
+      hipLaunchKernelGGL(loss_fwd_gather_pipe_kernel<SPX_LOSS_KL>, grid, block, kPipeSmem, st, lg, ld_logits, tg,
+                         ld_targets, vocab, loss, lse_draft, lse_target, extra, argmax_draft, argmax_target, sa);
+    else
+      hipLaunchKernelGGL(loss_fwd_gather_pipe_kernel<SPX_LOSS_CE>, grid, block, kPipeSmem, st, lg, ld_logits, tg,
+                         ld_targets, vocab, loss, lse_draft, lse_target, extra, argmax_draft, argmax_target, sa);
+    return check_launch(fname);
+  }
 #define SPX_GO(TT, VV, KK, GG)                                                                    \
   launch_fwd<TT, VV, KK, GG>(op, reinterpret_cast<const TT*>(logits), ld_logits,                  \
                              reinterpret_cast<const TT*>(targets), ld_targets, rows, vocab, loss, \

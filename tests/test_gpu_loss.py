@@ -350,3 +350,66 @@ def test_head_and_loss_node_with_the_input_gradient_in_parts(live_fraction, monk
         assert (grads[parts][0][dead] == 0).all()
         assert (grads[parts] - want).abs().max().item() <= 2e-2 * scale + 1e-6, parts
     assert (grads[4] - grads[1]).abs().max().item() <= 1e-2 * scale + 1e-6
+
+
+@pytest.mark.parametrize("op_name", ["kl_div", "ce"])
+@pytest.mark.parametrize("case", ["even", "skewed", "ragged", "one_tile", "clustered"])
+def test_pipelined_gather_pass_on_the_edges_of_its_tiling(op_name, case):
+    """The pipelined form of the one-pass kernel (bf16, 16-byte aligned rows, kl / ce: spans of the
+    full row staged two tiles deep, picks with lane = id) against the three-kernel form, bit for bit:
+    a table spread evenly; one that is dense at the low ids and sparse at the high ones, so that
+    the spans of the late tiles do not fit a buffer and are read directly; a draft vocabulary that
+    ends inside a chunk of 8 (rows kept aligned by their stride); one smaller than a tile; ids
+    clustered in two far-apart runs (a span boundary inside a tile)."""
+    from speculators_amd import _lib
+    from speculators_amd import losses as L
+
+    g = torch.Generator().manual_seed(len(case) * 7 + len(op_name))
+    rows = 21
+    if case == "even":
+        vt, vd = 40000, 9000
+        sel = torch.randperm(vt, generator=g)[:vd]
+    elif case == "skewed":
+        vt, vd = 200000, 6144
+        dense = torch.arange(4000)                                  # ids 0..3999 map to themselves
+        sparse = 4000 + torch.randperm(vt - 4000, generator=g)[:vd - 4000]  # 2144 ids over 196000 columns
+        sel = torch.cat([dense, sparse])
+    elif case == "ragged":
+        vt, vd = 30000, 4099
+        sel = torch.randperm(vt, generator=g)[:vd]
+    elif case == "one_tile":
+        vt, vd = 3000, 700
+        sel = torch.randperm(vt, generator=g)[:vd]
+    else:
+        vt, vd = 150000, 5000
+        sel = torch.cat([torch.arange(100, 2600), torch.arange(140000, 142500)])
+    d2t, _ = OV.build_vocab_mappings(sel.tolist(), vt)
+    vt_ld, vd_ld = -(-vt // 8) * 8, -(-vd // 8) * 8
+    full = (torch.randn(rows, vt_ld, generator=g) * 2).bfloat16().cuda()[:, :vt]
+    logits = (torch.randn(rows, vd_ld, generator=g) * 2).bfloat16().cuda()[:, :vd]
+    compact = L.vocab_gather(full.contiguous(), d2t.cuda())
+    assert torch.equal(compact.cpu(), OV.gather_targets(full.cpu(), d2t))
+    for i in range(0, rows, 3):
+        logits[i, compact[i].float().argmax()] = 30.0
+    mask = (torch.rand(rows, generator=g) < 0.7).float().cuda()
+    prev0 = (torch.rand(rows, generator=g) < 0.8).cuda()
+    op = L.PRIMITIVE_OP[op_name]
+    ref = L.fused_loss_forward(op, logits, compact)
+    out = torch.empty(6, device="cuda")
+    prev_ref = prev0.clone()
+    _lib.call("spx_ttt_step_reduce", _lib.ptr(ref[0]), _lib.ptr(ref[4]), _lib.ptr(ref[5]), _lib.ptr(mask),
+              _lib.kind_code(mask), _lib.ptr(prev_ref), _lib.kind_code(prev_ref), rows, 0.7,
+              _lib.ptr(out), None, _lib.stream_ptr(mask.device))
+    prev_got = prev0.clone()
+    step = L.StepPass(d2t=d2t.cuda(), mask=mask, prev=prev_got,
+                      counts=torch.zeros(3, dtype=torch.int32, device="cuda"))
+    assert full.stride(0) % 8 == 0 and logits.stride(0) % 8 == 0  # the pipelined kernel's precondition
+    got = L.fused_loss_forward(op, logits, full, step=step)
+    assert torch.equal(step.gathered, compact)
+    names = ("loss", "lse_draft", "lse_target", "extra", "argmax_draft", "argmax_target")
+    for name, a, b in zip(names, got[:6], ref[:6], strict=True):
+        if op_name == "ce" and name in ("lse_target", "extra"):
+            continue  # not defined for ce
+        assert torch.equal(a, b), name
+    assert torch.equal(prev_got, prev_ref)
+    assert step.counts.tolist() == [int(out[1]), int(out[2]), int(out[4])]
