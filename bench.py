@@ -1003,6 +1003,33 @@ def main():
         del model, step, loss
         torch.cuda.empty_cache()
 
+    # the other entry point beside the headline: targets handed over as full-vocabulary verifier logits, whose
+    # first TTT step gathers through d2t inside the loss pass (spx_vocab_loss_step_fwd)
+    other_entry = None
+    if not head_window:
+        alt = "hidden" if args.targets == "logits" else "logits"
+        saved = batch
+        batch, _d2t, _t2d = make_inputs(torch, CONFIG1, t, device, alt == "logits")
+        model, step = build(autocast)
+        for _ in range(args.warmup):
+            step()
+        with quiet_gc():
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                loss = step()
+            torch.cuda.synchronize()
+        a_ms = (time.perf_counter() - t0) / args.steps * 1e3
+        other_entry = {"targets": alt, "regime": args.regime, "ms_per_step": round(a_ms, 3),
+                       "value": round(t / (a_ms * 1e-3), 1), "unit": "tokens/s",
+                       "final_loss": round(float(loss.detach()), 6),
+                       "note": ("full-vocabulary verifier logits gathered through d2t in the first step's loss pass "
+                                "(no verifier-head product)" if alt == "logits" else
+                                "verifier hidden states through the frozen verifier head")}
+        del model, step, loss
+        batch = saved
+        torch.cuda.empty_cache()
+
     model, step = build(autocast)
     for _ in range(args.warmup):
         step()
@@ -1062,6 +1089,7 @@ def main():
                    "regime": args.regime, "final_loss": round(float(loss.detach()), 6),
                    "sliding_window": head_window, "decoder_gemm": _decoder_gemm_mode()},
         "reference_default_config": ref_default,
+        "other_targets_entry": other_entry,
         "other_regime": {"regime": "bf16" if autocast else "autocast", "ms_per_step": round(other_ms, 3),
                          "value": round(tokens / (other_ms * 1e-3), 1), "unit": "tokens/s",
                          "final_loss": round(other_loss, 6)},

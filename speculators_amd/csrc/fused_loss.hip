@@ -396,38 +396,46 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_gather_pipe_kernel(
   }
   __syncthreads();
 
-  constexpr int kOob = 0x7ffffff0;  // an offset outside every resource: the lane writes zeros, nothing is fetched
-  const u32x4 yres = make_rsrc(yrow, (uint32_t)(sa.vt * 2));
-  const u32x4 xres = make_rsrc(xrow, (uint32_t)(vocab * 2));
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)psm;
-  // tile u into slot u % 3: kPipeSpanLoads wave-loads of the span (the four waves interleaved, lanes past
-  // the span's end switched off) and one of this wave's 512 ids of the draft row -- always six loads
-  // (a tile past the last one: six loads all the same, every lane switched off)
+  // Per-lane byte offsets that never change: every tile moves the BASE of its buffer resources (scalar
+  // arithmetic) and sets their size to what the tile may touch, so lanes past a span's end, past the
+  // draft vocabulary or past the table fetch nothing and deliver zeros, without a vector instruction
+  int span_voff[kPipeSpanLoads];
+#pragma unroll
+  for (int k = 0; k < kPipeSpanLoads; ++k) span_voff[k] = ((k * kLossWaves + wave) * 512 + lane * 8) * 2;
+  const int x_voff = (wave * 512 + lane * 8) * 2;
+  const int off_voff = lane * 8;
+  // tile u into slot u % 3: kPipeSpanLoads wave-loads of the span (the four waves interleaved) and one of
+  // this wave's 512 ids of the draft row -- always six loads, also for a tile past the last one (resources
+  // of size zero)
   auto request = [&](int u) __attribute__((always_inline)) {
     const bool live = u < ntiles;
     const int lo = live ? span[2 * u] : 0, len = live ? span[2 * u + 1] : -1;
+    // (sizes in whole 16-byte pieces: a load that straddles the end of a resource delivers nothing at
+    // all, and the rows' pitch, a multiple of 8 elements, covers the rounding)
+    const u32x4 yres = make_rsrc(yrow + lo, len > 0 ? (uint32_t)((len + 7) & ~7) * 2u : 0u);
+    const int64_t x0 = (int64_t)u * kPipeTileIds;
+    const u32x4 xres = make_rsrc(xrow + x0,
+                                 live ? (uint32_t)((min((int64_t)kPipeTileIds, vocab - x0) + 7) & ~(int64_t)7) * 2u : 0u);
     const uint32_t dst = lds0 + (u % kPipeSlots) * kPipeSlotBytes;
 #pragma unroll
-    for (int k = 0; k < kPipeSpanLoads; ++k) {
-      const int e = (k * kLossWaves + wave) * 512 + lane * 8;
-      load_to_lds16<0>(yres, dst + (k * kLossWaves + wave) * 1024, e < len ? (lo + e) * 2 : kOob, 0);
-    }
-    const int64_t xb = (int64_t)u * kPipeTileIds + wave * 512 + lane * 8;
-    load_to_lds16<0>(xres, dst + kPipeCap * 2 + wave * 1024, xb < vocab ? (int)(xb * 2) : kOob, 0);
+    for (int k = 0; k < kPipeSpanLoads; ++k)
+      load_to_lds16<0>(yres, dst + (k * kLossWaves + wave) * 1024, span_voff[k], 0);
+    load_to_lds16<0>(xres, dst + kPipeCap * 2 + wave * 1024, x_voff, 0);
   };
   // The table entries of this lane's 8 picks of tile u (lane = id inside the wave's 512 ids; the low
-  // words of the int64 offsets: |d2t| < 2^31).  The loads are statements the compiler does not look
-  // into, like the span requests: it would otherwise guard their first use with a wait that also
-  // covers every span request issued since (it does not count those), and the ring would run one
-  // tile deep.  Their registers must not be read before `landed` has named them.
+  // words of the int64 offsets: |d2t| < 2^31; 0 past the vocabulary).  The loads are statements the
+  // compiler does not look into, like the span requests: it would otherwise guard their first use with a
+  // wait that also covers every span request issued since (it does not count those), and the ring would
+  // run one tile deep.  Their registers must not be read before `landed` has named them.
   auto load_offsets = [&](int u, int (&d)[8]) __attribute__((always_inline)) {
-    const int64_t wbase = (int64_t)u * kPipeTileIds + wave * 512;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const int64_t id = min(wbase + lane + 64 * k, vocab - 1);
-      const int32_t* const ptr = reinterpret_cast<const int32_t*>(sa.d2t + id);
-      asm volatile("global_load_dword %0, %1, off" : "=v"(d[k]) : "v"(ptr) : "memory");
-    }
+    const int64_t w0 = (int64_t)u * kPipeTileIds + wave * 512;
+    const u32x4 dres = make_rsrc(sa.d2t + min(w0, vocab), (uint32_t)max((int64_t)0, min((int64_t)512, vocab - w0)) * 8u);
+#define SPX_LOAD_OFF(K) \
+    asm volatile("buffer_load_dword %0, %1, %2, 0 offen offset:%3" : "=v"(d[K]) : "v"(off_voff), "s"(dres), "n"(K * 512) : "memory")
+    SPX_LOAD_OFF(0); SPX_LOAD_OFF(1); SPX_LOAD_OFF(2); SPX_LOAD_OFF(3);
+    SPX_LOAD_OFF(4); SPX_LOAD_OFF(5); SPX_LOAD_OFF(6); SPX_LOAD_OFF(7);
+#undef SPX_LOAD_OFF
   };
   // all vector-memory operations but the newest six have completed; d is what the wait releases.
   // (No branch may stand between a load_offsets and the `landed` that names its registers: a merge of
@@ -459,14 +467,14 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_gather_pipe_kernel(
     // (32-bit arithmetic: ids and columns are below 2^30 here)
     const int id0 = (int)wbase + lane, nvocab = (int)vocab, nvt = (int)sa.vt;
     const unsigned ulen = len > 0 ? (unsigned)len : 0u;
-    const int slot_lo = -lo;
+    const int delta = id0 - lo;
     bool need = false;  // some pick of this lane is not in the staged span
     int rel[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-      rel[k] = id0 + 64 * k + cur[k] + slot_lo;  // column - lo
+      rel[k] = cur[k] + delta + 64 * k;  // column - lo
       const bool staged = (unsigned)rel[k] < ulen;
-      need |= (id0 + 64 * k < nvocab) && !staged;
+      need |= !staged;
       ystrip[lane + 64 * k] = buf[staged ? rel[k] : 0];
     }
     if (__any(need)) {  // (wave-uniform: the common case issues no global load here)

@@ -30,7 +30,7 @@ def test_hand_issued_loads_are_not_read_before_their_wait(tmp_path):
         pending, loads, waits = set(), 0, 0
         for line in body:
             ins = line.strip()
-            m = re.match(r"global_load_dword (v\d+), v\[", ins)
+            m = re.match(r"buffer_load_dword (v\d+), v\d+, s\[", ins)
             if m:
                 pending.add(m.group(1))
                 loads += 1
