@@ -486,6 +486,21 @@ int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb,
                      void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
                      void* stream);
 
+/* spx_gemm_bf16_nt for products whose number of 256 x 256 output tiles leaves the last round of
+ * workgroups mostly empty (384 tiles on 256 compute units: the second round is half empty and
+ * takes as long as a full one).  The tiles of that last round -- when they are at most half a
+ * round -- are cut along the contraction into up to max_parts parts (fp32 partials in the
+ * workspace, added in a fixed order by a second small kernel: results do not depend on timing);
+ * every other tile is computed and stored exactly as by spx_gemm_bf16_nt, and so is every tile
+ * when the last round is more than half full.  workspace: spx_gemm_tail_workspace_bytes()
+ * bytes, 16-byte aligned, caller owned.  No counterpart in the reference (its Linears run on
+ * the vendor library, which picks another tile shape for such products). */
+int64_t spx_gemm_tail_workspace_bytes(void);
+int spx_gemm_bf16_nt_tail(const void* a, int64_t lda, const void* b, int64_t ldb,
+                          void* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                          int32_t max_parts, void* workspace, int64_t workspace_bytes,
+                          void* stream);
+
 /* spx_gemm_bf16_nt whose epilogue also yields, per row m of c, the soft-max statistics of that
  * row AS ROUNDED TO bf16: lse[m] = log sum_n exp(c[m, n]) (natural logarithm, fp32) and
  * argmax[m] = the first n that attains max_n c[m, n] (-0 and +0 compare equal, as torch.argmax

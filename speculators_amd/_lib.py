@@ -73,6 +73,8 @@ SIGNATURES["spx_pack_batch"] = [_P, _I, _I64, _I64, _I64, _P, _P, _I, _P, _P, _P
 SIGNATURES["spx_gemm_bf16_nt"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P]
 SIGNATURES["spx_pack_row_map"] = [_P, _P, _I64, _I64, _P, _P, _P]
 SIGNATURES["spx_unpack_rows"] = [_P, _I64, _P, _I64, _I64, _I64, _P, _I64, _P]
+SIGNATURES["spx_gemm_bf16_nt_tail"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I32, _P, _I64, _P]
+SIGNATURES["spx_gemm_tail_workspace_bytes"] = []
 SIGNATURES["spx_gemm_bf16_nt_stats"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P, _P, _P, _I64, _P]
 SIGNATURES["spx_gemm_stats_workspace_bytes"] = [_I64, _I64]
 SIGNATURES["spx_gemm_bf16_nt_rows"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P, _P]
@@ -96,7 +98,7 @@ SIGNATURES["spx_transpose_bf16"] = [_P, _I64, _I64, _P, _I64, _I64, _I64, _I64, 
 SIGNATURES["spx_moe_gather_rows"] = [_P, _I64, _I64, _P, _P, _P, _I64, _I64, _I64, _P]
 SIGNATURES["spx_moe_combine_rows"] = [_P, _I64, _I64, _P, _P, _P, _I64, _I64, _I32, _I64, _P]
 SIGNATURES["spx_moe_pair_dot"] = [_P, _I64, _P, _I64, _I64, _P, _P, _I64, _I32, _I64, _P]
-RESTYPES = {"spx_gemm_grouped_workspace_bytes": c_int64, "spx_gemm_stats_workspace_bytes": c_int64, "spx_gemm_split_workspace_bytes": c_int64, "spx_ttt_attn_workspace_bytes": c_int64, "spx_ttt_attn_fwd_static_max_bytes": c_int64, "spx_dflash_attn_workspace_bytes": c_int64,
+RESTYPES = {"spx_gemm_grouped_workspace_bytes": c_int64, "spx_gemm_tail_workspace_bytes": c_int64, "spx_gemm_stats_workspace_bytes": c_int64, "spx_gemm_split_workspace_bytes": c_int64, "spx_ttt_attn_workspace_bytes": c_int64, "spx_ttt_attn_fwd_static_max_bytes": c_int64, "spx_dflash_attn_workspace_bytes": c_int64,
             "spx_rmsnorm_bwd_slots": c_int64}
 
 _lib = None

@@ -102,6 +102,35 @@ __device__ __forceinline__ int choose_k_parts(int n_tiles, int max_parts, int cu
 // float, sums as float, columns as int32); gemm_row_stats_reduce_kernel folds the tiles_n entries
 // of a row into log-sum-exp and arg-max.  C may then be null: the product itself is not stored
 // (a cross-entropy against arg-max targets needs nothing else of the target logits).
+// The tiles of the last, partly filled round of a product (n_tiles % cus of them, when they are at most
+// half a round): each is cut along the contraction into as many parts as fill the idle compute units
+// (at most max_parts, every part at least 16 slabs), so that the round takes a part's time instead of a
+// tile's.  384 tiles on 256 compute units: 256 whole tiles, then 128 tiles x 2 halves -- 1.5 rounds of
+// work in 1.5 rounds of time instead of 2.  first = index of the first tile that is cut (n_tiles: none).
+__host__ __device__ __forceinline__ void tail_plan(int n_tiles, int cus, int nslab, int max_parts, int& first,
+                                                   int& parts) {
+  first = n_tiles;
+  parts = 1;
+  if (n_tiles <= 0 || cus <= 0) return;
+  const int rem = n_tiles % cus;
+  if (rem == 0 || rem * 2 > cus) return;
+  int tp = cus / rem;
+  if (tp > max_parts) tp = max_parts;
+  while (tp > 1 && nslab / tp < 16) --tp;
+  if (tp > 1) { first = n_tiles - rem; parts = tp; }
+}
+
+// tile index -> (tile row, tile column): groups of GROUP_M tile rows, columns inside a group first
+__device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+  constexpr int GROUP_M = SPX_GEMM_GROUP_M;
+  const int in_group = GROUP_M * tiles_n;
+  const int group_id = pid / in_group;
+  const int first_m = group_id * GROUP_M;
+  const int group_sz = min(tiles_m - first_m, GROUP_M);
+  tile_m = first_m + (pid % in_group) % group_sz;
+  tile_n = (pid % in_group) / group_sz;
+}
+
 template <bool kImm, int kStats = 0>
 __global__ __launch_bounds__(kGemmThreads, SPX_GEMM_MINW)
 __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf16_nt_kernel(
@@ -109,7 +138,7 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
     uint16_t* __restrict__ C, int64_t ldc, int M, int N, int K, int tiles_m, int tiles_n,
     const int32_t* __restrict__ m_live, const int32_t* __restrict__ tile_tab,
     const int32_t* __restrict__ group_off, int64_t b_group_stride, float* __restrict__ part_ws,
-    int max_parts, int cus, float* __restrict__ stat_ws = nullptr) {
+    int max_parts, int cus, float* __restrict__ stat_ws = nullptr, int tail_mode = 0) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int M_host = M;
   // the row count may live on the device (rows packed to the front by the producer of A): the tile
@@ -130,17 +159,42 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   // contraction in parts (part_ws): the workgroups of part p multiply columns [p, p + 1) * part length of
   // K and leave an fp32 partial in part_ws[p]; gemm_splitk_reduce_kernel adds the parts in order
   const int n_tiles = tiles_m * tiles_n;
-  const int parts = part_ws ? choose_k_parts(n_tiles, max_parts, cus, (K + kTK - 1) / kTK) : 1;
-  const int n_wg = n_tiles * parts;
+  // tail_mode: only the tiles of the last, partly filled round are cut (tail_plan); their partials go to
+  // part_ws as whole tiles, [part][tail tile][256][256] fp32, and gemm_tail_reduce_kernel adds them
+  int parts = 1, tail_first = n_tiles, tail_parts = 1;
+  if (tail_mode) tail_plan(n_tiles, cus, (K + kTK - 1) / kTK, max_parts, tail_first, tail_parts);
+  else if (part_ws) parts = choose_k_parts(n_tiles, max_parts, cus, (K + kTK - 1) / kTK);
+  const int n_tail = n_tiles - tail_first;
+  const int n_wg = tail_mode ? n_tiles + n_tail * (tail_parts - 1) : n_tiles * parts;
   if ((int)blockIdx.x >= n_wg) return;
   int pid;
   {
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int base = n_wg >> 3, rem = n_wg & 7;
-    pid = xcd * base + min(xcd, rem) + local;
+    if (tail_mode && tail_parts > 1 && (tail_first & 7) == 0) {
+      // every XCD first walks its band of the whole tiles, then its band of the cut ones: the workgroups
+      // are dispatched in the order of their ids, so the whole tiles fill the chip first and the parts of
+      // the last round follow everywhere at once
+      const int wb = tail_first >> 3, np = n_wg - tail_first;
+      if (local < wb) pid = xcd * wb + local;
+      else pid = tail_first + xcd * (np >> 3) + min(xcd, np & 7) + (local - wb);
+    } else {
+      const int base = n_wg >> 3, rem = n_wg & 7;
+      pid = xcd * base + min(xcd, rem) + local;
+    }
   }
-  const int part = pid / n_tiles;
-  pid -= part * n_tiles;
+  int part;
+  if (tail_mode) {
+    part = 0;
+    if (pid >= tail_first) {
+      const int qq = pid - tail_first;
+      part = qq / n_tail;
+      pid = tail_first + qq % n_tail;
+      parts = tail_parts;
+    }
+  } else {
+    part = pid / n_tiles;
+    pid -= part * n_tiles;
+  }
   if (parts > 1) {
     const int slabs = ((K + kTK - 1) / kTK + parts - 1) / parts;
     const int k_begin = part * slabs * kTK;
@@ -148,13 +202,8 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
     B += k_begin;
     K = max(min(K - k_begin, slabs * kTK), 0);
   }
-  constexpr int GROUP_M = SPX_GEMM_GROUP_M;
-  const int in_group = GROUP_M * tiles_n;
-  const int group_id = pid / in_group;
-  const int first_m = group_id * GROUP_M;
-  const int group_sz = min(tiles_m - first_m, GROUP_M);
-  const int tile_m = first_m + (pid % in_group) % group_sz;
-  const int tile_n = (pid % in_group) / group_sz;
+  int tile_m, tile_n;
+  tile_coords(pid, tiles_m, tiles_n, tile_m, tile_n);
   int m0 = tile_m * kTM;
   const int n0 = tile_n * kTN;
   if (tile_tab) {
@@ -315,6 +364,17 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   mfma_results_ready();
+  if (parts > 1 && tail_mode) {
+    // this part's fp32 partial of a tile of the last round: a 256 x 256 tile of its own
+    float* const P = part_ws + ((int64_t)(part * n_tail + (pid - tail_first)) << 16);
+#pragma unroll
+    for (int i = 0; i < kMI; ++i) {
+      const int rr = wm + i * 16 + r16;
+#pragma unroll
+      for (int j = 0; j < kNI; ++j) *reinterpret_cast<f32x4*>(P + rr * kTN + wn + j * 16 + 4 * q) = acc[j][i];
+    }
+    return;
+  }
   if (parts > 1) {
     // this part's fp32 partial, in the accumulators' own layout: 16 bytes per lane and accumulator
     float* const P = part_ws + (int64_t)part * M_host * N;
@@ -492,6 +552,44 @@ __global__ __launch_bounds__(256) void gemm_row_stats_reduce_kernel(const float*
   if (argmax) argmax[m] = first;
 }
 
+// The tiles of the last round of a product cut by tail_plan: C[tile] = the sum of its parts, in their
+// order, fp32, one rounding.  blockIdx.x = tail tile, 256 threads x 32 passes of 8 columns.
+__global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const float* __restrict__ part_ws,
+                                                               uint16_t* __restrict__ C, int64_t ldc, int M, int N,
+                                                               int K, int tiles_m, int tiles_n, int max_parts,
+                                                               int cus) {
+  int tail_first, tail_parts;
+  tail_plan(tiles_m * tiles_n, cus, (K + kTK - 1) / kTK, max_parts, tail_first, tail_parts);
+  const int n_tail = tiles_m * tiles_n - tail_first;
+  if (tail_parts <= 1 || (int)blockIdx.x >= n_tail) return;
+  int tile_m, tile_n;
+  tile_coords(tail_first + blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * kTM, n0 = tile_n * kTN;
+  const bool fast = (ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
+  for (int it = threadIdx.x; it < kTM * (kTN / 8); it += 256) {
+    const int rr = it / (kTN / 8), cc = (it % (kTN / 8)) * 8;
+    const int m = m0 + rr, n = n0 + cc;
+    if (m >= M || n >= N) continue;
+    f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+    for (int p = 0; p < tail_parts; ++p) {
+      const float* src = part_ws + ((int64_t)(p * n_tail + blockIdx.x) << 16) + rr * kTN + cc;
+      const f32x4 a = *reinterpret_cast<const f32x4*>(src), b = *reinterpret_cast<const f32x4*>(src + 4);
+      lo[0] += a[0]; lo[1] += a[1]; lo[2] += a[2]; lo[3] += a[3];
+      hi[0] += b[0]; hi[1] += b[1]; hi[2] += b[2]; hi[3] += b[3];
+    }
+    u32x4 v;
+    v.x = pack_bf16x2(lo[0], lo[1]); v.y = pack_bf16x2(lo[2], lo[3]);
+    v.z = pack_bf16x2(hi[0], hi[1]); v.w = pack_bf16x2(hi[2], hi[3]);
+    if (fast && n + 8 <= N) {
+      *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+    } else {
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      for (int e = 0; e < 8; ++e)
+        if (n + e < N) C[(int64_t)m * ldc + n + e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+    }
+  }
+}
+
 // C[m, n .. n + 7] = the sum of the parts of a product whose contraction was cut (in the order of the
 // parts, fp32, one rounding).  Re-derives the number of parts like the product did; nothing to do for one.
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ part_ws,
@@ -536,12 +634,15 @@ static int compute_units() {
   return n;
 }
 
+// an upper bound of compute_units() over the devices this library runs on (MI355X: 256)
+static int compute_units_max() { return 512; }
+
 #define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fname, what); } while (0)
 static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
                         int64_t ldc, int64_t M, int64_t N, int64_t K, const int32_t* m_live, void* stream,
                         const int32_t* tile_tab = nullptr, const int32_t* group_off = nullptr,
                         int64_t b_group_stride = 0, int64_t groups = 0, float* part_ws = nullptr,
-                        int max_parts = 1, float* stat_ws = nullptr, int stats_mode = 0) {
+                        int max_parts = 1, float* stat_ws = nullptr, int stats_mode = 0, int tail_mode = 0) {
   SPX_REQ_FN(M > 0 && N > 0 && K > 0, "M, N, K must be positive");
   SPX_REQ_FN(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "dimension too large");
   SPX_REQ_FN(a && b && (c || stat_ws), "null buffer");
@@ -571,12 +672,18 @@ static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const voi
   // (a contraction in parts: room for every part of every tile; the kernel decides how many it uses)
   SPX_REQ_FN((int64_t)tiles_m * tiles_n * max_parts < (1ll << 31), "too many tiles");
   const int cus = compute_units();
-  const dim3 grid((unsigned)(tiles_m * tiles_n * (part_ws ? max_parts : 1))), block(kGemmThreads);
+  int64_t n_grid = (int64_t)tiles_m * tiles_n * (part_ws ? max_parts : 1);
+  int tail_first = tiles_m * tiles_n, tail_parts = 1;
+  if (tail_mode) {
+    tail_plan(tiles_m * tiles_n, cus, (int)((K + kTK - 1) / kTK), max_parts, tail_first, tail_parts);
+    n_grid = (int64_t)tiles_m * tiles_n + (int64_t)(tiles_m * tiles_n - tail_first) * (tail_parts - 1);
+  }
+  const dim3 grid((unsigned)n_grid), block(kGemmThreads);
 #define SPX_GEMM_LAUNCH(IMM, STATS)                                                                              \
   hipLaunchKernelGGL((gemm_bf16_nt_kernel<IMM, STATS>), grid, block, kGemmSmem, st,                              \
                      reinterpret_cast<const uint16_t*>(a), lda, reinterpret_cast<const uint16_t*>(b), ldb,       \
                      reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n, m_live,      \
-                     tile_tab, group_off, b_group_stride, part_ws, max_parts, cus, stat_ws)
+                     tile_tab, group_off, b_group_stride, part_ws, max_parts, cus, stat_ws, tail_mode)
   switch (which) {
     case 0: SPX_GEMM_LAUNCH(false, 0); break;
     case 1: SPX_GEMM_LAUNCH(true, 0); break;
@@ -589,6 +696,15 @@ static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const voi
   }
 #undef SPX_GEMM_LAUNCH
   if (int rc = check_launch(fname)) return rc;
+  if (tail_mode) {
+    if (tail_parts > 1) {
+      hipLaunchKernelGGL(gemm_tail_reduce_kernel, dim3((unsigned)(tiles_m * tiles_n - tail_first)), dim3(256), 0, st,
+                         part_ws, reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n,
+                         max_parts, cus);
+      return check_launch(fname);
+    }
+    return 0;
+  }
   if (part_ws) {
     const int64_t items = M * (N / 8);
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, part_ws,
@@ -663,6 +779,22 @@ extern "C" int spx_gemm_bf16_nt_grouped(const void* a, int64_t lda, const void* 
 extern "C" int spx_gemm_bf16_nt(const void* a, int64_t lda, const void* b, int64_t ldb, void* c,
                                 int64_t ldc, int64_t M, int64_t N, int64_t K, void* stream) {
   return gemm_nt_impl(__func__, a, lda, b, ldb, c, ldc, M, N, K, nullptr, stream);
+}
+
+extern "C" int64_t spx_gemm_tail_workspace_bytes(void) {
+  // (tiles of the last round) x (parts) never exceeds the compute units; one fp32 tile each
+  return (int64_t)compute_units_max() * kTM * kTN * (int64_t)sizeof(float);
+}
+
+extern "C" int spx_gemm_bf16_nt_tail(const void* a, int64_t lda, const void* b, int64_t ldb, void* c, int64_t ldc,
+                                     int64_t M, int64_t N, int64_t K, int32_t max_parts, void* workspace,
+                                     int64_t workspace_bytes, void* stream) {
+  const char* fname = __func__;
+  SPX_REQ_FN(max_parts >= 1 && max_parts <= 8, "max_parts must be 1 .. 8");
+  SPX_REQ_FN(workspace && ((uintptr_t)workspace) % 16 == 0, "null or unaligned workspace");
+  SPX_REQ_FN(workspace_bytes >= spx_gemm_tail_workspace_bytes(), "workspace too small");
+  return gemm_nt_impl(fname, a, lda, b, ldb, c, ldc, M, N, K, nullptr, stream, nullptr, nullptr, 0, 0,
+                      reinterpret_cast<float*>(workspace), max_parts, nullptr, 0, 1);
 }
 
 extern "C" int64_t spx_gemm_stats_workspace_bytes(int64_t M, int64_t N) {

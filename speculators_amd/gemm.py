@@ -21,11 +21,18 @@ from . import fused_ops as FO
 _MAX_SPAN = 0x7ffffff0 - 64  # bytes an operand of the weight-gradient product (gemm_tn) may span per call
 
 
+_CUS = 256  # workgroups the chip runs at a time (one per compute unit for the GEMM kernels)
+
 # parts the contraction of a live-rows product may be cut into (gemm_nt(split=True)); 1 = never cut
 SPLIT_PARTS = int(os.environ.get("SPX_GEMM_SPLIT_PARTS", "4"))
 if not 1 <= SPLIT_PARTS <= 8:
     raise ValueError(f"SPX_GEMM_SPLIT_PARTS must be 1 .. 8, got {SPLIT_PARTS}")
 
+
+# parts the tiles of a mostly empty last round of a product may be cut into (spx_gemm_bf16_nt_tail); 1 = never
+TAIL_PARTS = int(os.environ.get("SPX_GEMM_TAIL_PARTS", "4"))
+if not 1 <= TAIL_PARTS <= 8:
+    raise ValueError(f"SPX_GEMM_TAIL_PARTS must be 1 .. 8, got {TAIL_PARTS}")
 
 _split_ws: dict = {}
 
@@ -68,6 +75,15 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None,
     # (operands of any size go in one launch: the kernel's 32-bit offsets are relative to a tile)
     st = _lib.stream_ptr(a.device)
     if m_live is None:
+        # a last round of tiles that fills at most half the chip is cut along the contraction
+        # (the kernel decides from the same numbers; here only whether the workspace is handed over)
+        rem = (-(-m // 256) * -(-n // 256)) % _CUS
+        if TAIL_PARTS > 1 and 0 < rem <= _CUS // 2 and k >= 64 * 16 * 2 and a.is_cuda:
+            nbytes = _lib.load().spx_gemm_tail_workspace_bytes()
+            ws = _split_workspace(a.device, nbytes // 4)
+            _lib.call("spx_gemm_bf16_nt_tail", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
+                      _lib.ptr(out), out.stride(0), m, n, k, TAIL_PARTS, _lib.ptr(ws), nbytes, st)
+            return out
         _lib.call("spx_gemm_bf16_nt", _lib.ptr(a), a.stride(0), _lib.ptr(b), b.stride(0),
                   _lib.ptr(out), out.stride(0), m, n, k, st)
     else:
@@ -116,7 +132,6 @@ def gemm_nt_stats(a: torch.Tensor, b: torch.Tensor, store: bool = True, want_arg
     return out, lse, am
 
 
-_CUS = 256  # workgroups the chip runs at a time (one per compute unit for the GEMM kernels)
 
 
 def _split_bands(t: int, m: int, n: int) -> int:
@@ -224,17 +239,33 @@ def linear(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor | None 
 # Which GEMM runs the decoder-layer projections (q/k/v, o, gate/up, down and their input
 # gradients): "hipblaslt" = PyTorch's matmul (the library GEMM), "spx" = this library's MFMA kernel
 # (the input gradients then run against the transposed copy of the staged weight), "mixed" = each
-# where it is faster on these shapes: the forward products on hipBLASLt (3 - 8 % ahead there), the
-# input gradients on this library's kernel (8 - 20 % ahead of the library's NN product).  The fc /
+# where it is faster on these shapes: the forward products on hipBLASLt (6 - 12 % ahead there) except
+# those whose tile count leaves the last round of workgroups mostly idle, which this library's kernel
+# cuts along the contraction (the merged q/k/v projection: 10 % ahead of the library), the input
+# gradients on this library's kernel (8 - 20 % ahead of the library's NN product).  The fc /
 # lm_head / verifier-head products and every weight gradient always run on this library's kernels.
 DECODER_GEMM = os.environ.get("SPX_DECODER_GEMM", "mixed")
 if DECODER_GEMM not in ("hipblaslt", "spx", "mixed"):
     raise ValueError(f"SPX_DECODER_GEMM must be 'hipblaslt', 'spx' or 'mixed', got {DECODER_GEMM!r}")
 
 
+def _tail_cut_applies(m: int, n: int, k: int) -> bool:
+    """Whether ``gemm_nt`` cuts the last round of tiles of an ``[m, k] x [n, k]^T`` product (the rule of
+    ``spx_gemm_bf16_nt_tail``): the shapes on which a 256 x 256 tiling loses most to tile quantisation
+    and the cut wins it back (the merged q/k/v projection of the 8B shape: 384 tiles)."""
+    rem = (-(-m // 256) * -(-n // 256)) % _CUS
+    return TAIL_PARTS > 1 and 0 < rem <= _CUS // 2 and k >= 64 * 16 * 2 and (-(-m // 256) * -(-n // 256)) < 2 * _CUS
+
+
 def _project(x2: torch.Tensor, staged) -> torch.Tensor:
     """``x2 @ staged.w.T`` of a decoder-layer projection."""
-    return gemm_nt(x2, staged.w) if DECODER_GEMM == "spx" else torch.nn.functional.linear(x2, staged.w)
+    if DECODER_GEMM == "spx":
+        return gemm_nt(x2, staged.w)
+    if (DECODER_GEMM == "mixed" and x2.dtype == torch.bfloat16
+            and _tail_cut_applies(x2.shape[0], staged.w.shape[0], x2.shape[1])):
+        # (measured at [4096, 8192] x [6144, 8192]^T: 322 us here, 357 us on the library)
+        return gemm_nt(x2, staged.w)
+    return torch.nn.functional.linear(x2, staged.w)
 
 
 def _project_back(dy2: torch.Tensor, staged) -> torch.Tensor:

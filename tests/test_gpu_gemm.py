@@ -421,3 +421,38 @@ def test_gemm_stats_rejects_bad_arguments():
     rc = lib.spx_gemm_bf16_nt_stats(_lib.ptr(a), 64, _lib.ptr(a), 64, None, 0, 256, 256, 64, None, None,
                                     _lib.ptr(ws), 1 << 20, None)
     assert rc == 1 and b"null lse and null argmax" in lib.spx_last_error()
+
+
+@pytest.mark.parametrize("m,n,k,parts", [(512, 768, 4096, 4), (300, 1000, 8192, 4), (4096, 6144, 2048, 2),
+                                         (512, 768, 1024, 1), (4096, 4096, 4096, 1), (1024, 1800, 2048 + 64, 2)])
+def test_gemm_nt_with_the_last_round_of_tiles_cut_along_the_contraction(m, n, k, parts):
+    """``spx_gemm_bf16_nt_tail``: a last round of tiles that leaves at least half of the 256 compute
+    units idle is cut along the contraction (6 tiles -> 4 parts each; 384 tiles -> the last 128 in 2),
+    every other tile -- and every tile when nothing is cut (short contraction, full rounds) -- is the plain
+    kernel's bit for bit.  Ragged edges in both directions; against the float64 product."""
+    from speculators_amd import _lib
+    from speculators_amd import gemm
+
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).bfloat16().cuda()
+    b = (torch.randn(n, k, generator=g) / k ** 0.5).bfloat16().cuda()
+    plain = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+    _lib.call("spx_gemm_bf16_nt", _lib.ptr(a), k, _lib.ptr(b), k, _lib.ptr(plain), n, m, n, k,
+              _lib.stream_ptr(a.device))
+    got = gemm.gemm_nt(a, b)     # takes the tail entry point whenever the tile count asks for it
+    tiles = -(-m // 256) * -(-n // 256)
+    rem = tiles % 256
+    assert (0 < rem <= 128) or parts == 1
+    if parts == 1:
+        assert torch.equal(got.view(torch.int16), plain.view(torch.int16))
+    else:
+        assert not torch.equal(got.view(torch.int16), plain.view(torch.int16))  # another summation order
+        # the tiles of the full rounds are untouched: tile index -> (row group of 8, column, row)
+        if tiles > 256:
+            assert torch.equal(got[:256, :256].view(torch.int16), plain[:256, :256].view(torch.int16))
+    want = a.double() @ b.double().t()
+    err = (got.double() - want).abs().max().item()
+    assert err <= 1e-2 * want.abs().max().item(), err
+    # run to run identical (fixed order of the parts)
+    again = gemm.gemm_nt(a, b)
+    assert torch.equal(again.view(torch.int16), got.view(torch.int16))
