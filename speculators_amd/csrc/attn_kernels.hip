@@ -265,15 +265,9 @@ __device__ __forceinline__ void pin_block(f32x16& a) {
 // round (matrix phase first) the vector wave waits behind MFMAs that are themselves waiting for the pipe
 // (measured at the Llama-3.1-8B shape: 825 TFLOP/s with the matrix phase first, 826 without priorities, 880
 // with the vector phase first).  The dQ and dK/dV kernels measure best with the matrix phase first.
-#ifndef SPX_FWD_PRIO
 #define SPX_FWD_PRIO 0, 3
-#endif
-#ifndef SPX_DQ_PRIO
 #define SPX_DQ_PRIO 3, 0
-#endif
-#ifndef SPX_DKV_PRIO
 #define SPX_DKV_PRIO 3, 0
-#endif
 constexpr int prio_first(int a, int) { return a; }
 constexpr int prio_second(int, int b) { return b; }
 template <int M, int V>
@@ -287,18 +281,10 @@ struct PrioPair {
 #define SPX_DQ_PRIO_VALU() PrioPair<prio_first(SPX_DQ_PRIO), prio_second(SPX_DQ_PRIO)>::vector()
 #define SPX_DKV_PRIO_MFMA() PrioPair<prio_first(SPX_DKV_PRIO), prio_second(SPX_DKV_PRIO)>::matrix()
 #define SPX_DKV_PRIO_VALU() PrioPair<prio_first(SPX_DKV_PRIO), prio_second(SPX_DKV_PRIO)>::vector()
-#ifndef SPX_DKV_REMAT
 #define SPX_DKV_REMAT 1
-#endif
-#ifndef SPX_FWD_MINB
 #define SPX_FWD_MINB 2
-#endif
-#ifndef SPX_DQ_MINB
 #define SPX_DQ_MINB 2
-#endif
-#ifndef SPX_DKV_MINB
 #define SPX_DKV_MINB 1
-#endif
 // How the forward kernel brings a key tile into LDS: through registers at the point of use (0),
 // through registers one tile ahead (1), or with global -> LDS loads into the other of two tile
 // buffers (2).  A 16-byte LDS write from registers holds the LDS pipe twice as long as a 16-byte
@@ -314,9 +300,7 @@ struct FwdSmem {
 
 // operand fragments in flight per product (registers: 4 per fragment): the LDS pipe delivers
 // well over 150 B/clk per CU, what a wave waits for is the latency of its own reads
-#ifndef SPX_FWD_RING
 #define SPX_FWD_RING 8
-#endif
 template <int D, int NSB, int NW, int PF>
 __global__ __launch_bounds__(64 * NW, D > 128 ? 1 : SPX_FWD_MINB) void attn_fwd_kernel(AttnParams p,
                                                                 const uint16_t* __restrict__ Vt,
@@ -1262,18 +1246,7 @@ __global__ __launch_bounds__(64) void attn_tile_bounds_kernel(AttnParams p, int3
 // PASS 0 computes dK and dV together; PASS 1 only dV, PASS 2 only dK (head_dim 256: the two
 // accumulator sets and both operand fragments do not fit the register file together, so
 // the kernel is launched once per pass and the scores are recomputed).
-#ifndef SPX_DKV_XCD
 #define SPX_DKV_XCD 1
-#endif
-#ifndef SPX_DKV256_ONEPASS
-#define SPX_DKV256_ONEPASS 2
-#endif
-#ifndef SPX_DKV256_PF1
-#define SPX_DKV256_PF1 2
-#endif
-#ifndef SPX_DKV256_PF2
-#define SPX_DKV256_PF2 1
-#endif
 // PF: how the query tiles reach LDS (see FwdSmem): 0 at the point of use, 1 through registers one
 // tile ahead, 2 global -> LDS into the other of two buffers, 3 the same with tiles of 32 instead of 64
 // query rows.  A buffer holds the tiles the pass multiplies with: Q always, dO and Q^T for dK, dO^T for
@@ -1298,9 +1271,7 @@ struct DkvSmem {
 
 // operand fragments in flight per product in the dK/dV kernel (one wave per SIMD: nothing else
 // hides the latency of its LDS reads)
-#ifndef SPX_DKV_RING
 #define SPX_DKV_RING 8
-#endif
 template <int D, int NW, int PF, int PASS>
 __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
     AttnParams p, const uint16_t* __restrict__ dO, const uint16_t* __restrict__ Qt,
@@ -1750,9 +1721,6 @@ __global__ __launch_bounds__(64 * NW, SPX_DKV_MINB) void attn_bwd_dkv_kernel(
   }
 }
 
-#ifndef SPX_DKV_WS
-#define SPX_DKV_WS 1
-#endif
 // ---------------------------------------------------------------- dK / dV, wave-specialised
 // The work of attn_bwd_dkv_kernel for head_dim <= 128 (both gradients in one pass), split over
 // TWO waves per SIMD that run different halves of it, so that each SIMD has a wave for the matrix
@@ -2315,23 +2283,13 @@ __global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
 // ---------------------------------------------------------------- launchers
 static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 
-#ifndef SPX_FWD_CFG
 #define SPX_FWD_CFG 1, 4, 2
-#endif
-#ifndef SPX_DQ_CFG
 #define SPX_DQ_CFG 1, 4, 4
-#endif
 // head_dim 256: the next tile is prefetched into registers as well; the few registers that
 // spill cost far less than exposing the global-load latency with one workgroup per CU
-#ifndef SPX_FWD256_PF
 #define SPX_FWD256_PF 2
-#endif
-#ifndef SPX_DQ256_PF
 #define SPX_DQ256_PF 4
-#endif
-#ifndef SPX_DKV_CFG
 #define SPX_DKV_CFG 4, 2
-#endif
 // (sub-blocks per wave, waves per workgroup, register prefetch) of the forward / dQ kernels,
 // (waves per workgroup, register prefetch) of the dK/dV kernel
 constexpr int cfg_nsb(int nsb, int, int) { return nsb; }
@@ -2390,8 +2348,7 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   const int NQp = (int)round_up(p.NQ, 128);
   char* w = reinterpret_cast<char*>(workspace);
   uint16_t* kt = reinterpret_cast<uint16_t*>(w);
-  uint16_t* qt = kt + (int64_t)p.Hkv * D * p.NKVp;
-  uint16_t* dot = qt + (int64_t)p.Hq * D * NQp;
+  // (the room behind K^T once held Q^T and dO^T; the layout of the workspace has not moved)
   w += round_up(((int64_t)p.Hkv * D * p.NKVp + 2 * (int64_t)p.Hq * D * NQp) * 2, 256);
   float* delta = reinterpret_cast<float*>(w);
   w += round_up((int64_t)p.Hq * p.NQ * 4, 256);
@@ -2414,16 +2371,16 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
     hipLaunchKernelGGL(transpose_bf16_kernel<false>, tgrid, dim3(64), 0, st, p.K, p.k_hs, (int64_t)D, p.NKV, D,
                        kt, (int64_t)D * p.NKVp, (int64_t)p.NKVp, 1.f, nullptr);
   dim3 qgrid((unsigned)(NQp / 64), (unsigned)((D + 63) / 64), (unsigned)p.Hq);
-  // (the wave-specialised dK/dV kernel transposes inside LDS and needs no Q^T / dO^T; it lists the query
-  // tiles that see a key block in LDS, which bounds their number)
-  const bool use_ws = D <= 128 && SPX_DKV_WS && (p.NQ + 63) / 64 <= DkvWsSmem<(D <= 128 ? D : 128)>::kListCap;
-  // (nor does the one-pass head_dim-256 kernel with transposing LDS reads)
-  const bool kNeedT = !use_ws && !(D > 128 && SPX_DKV256_ONEPASS == 2);
+  // (neither dK/dV kernel needs Q^T / dO^T: both transpose inside LDS.  The wave-specialised one lists the
+  // query tiles that see a key block in LDS, which bounds their number)
+  if (D <= 128 && (p.NQ + 63) / 64 > DkvWsSmem<(D <= 128 ? D : 128)>::kListCap) {
+    last_error() = std::string(fn) + ": more than " +
+                   std::to_string(64 * DkvWsSmem<(D <= 128 ? D : 128)>::kListCap) +
+                   " query rows in one call at head_dim <= 128";
+    return SPX_ERR_ARG;
+  }
   hipLaunchKernelGGL(transpose_bf16_kernel<true>, qgrid, dim3(64), 0, st, p.Q, p.q_hs, (int64_t)D, p.NQ, D,
-                     kNeedT ? qt : nullptr, (int64_t)D * NQp, (int64_t)NQp, p.scale_log2e, qs);
-  if (kNeedT)
-    hipLaunchKernelGGL(transpose_bf16_kernel<false>, qgrid, dim3(64), 0, st, dOp, (int64_t)D,
-                       (int64_t)p.Hq * D, p.NQ, D, dot, (int64_t)D * NQp, (int64_t)NQp, 1.f, nullptr);
+                     (uint16_t*)nullptr, (int64_t)D * NQp, (int64_t)NQp, p.scale_log2e, qs);
   // the dK/dV and diagonal-key kernels read the scaled queries: their scores are q' . k with no
   // factor of their own, and what they accumulate against q' carries scale * log2(e) once too
   // often: dK = ln 2 * sum dS q'
@@ -2455,64 +2412,31 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
                        dim3(64 * kDqNW), dq_smem, st, p, dOp, kt, lse, delta, dQp, dq_hs);
   }
 
-  constexpr int kPF = D > 128 ? 1 : kDkvPF;
-  constexpr int kPF1 = SPX_DKV256_PF1, kPF2 = SPX_DKV256_PF2;
-  if ((kPF == 2 || D > 128) && (int64_t)p.NQ * p.Hq * D * 2 >= (1ll << 31)) {
+  if (D > 128 && (int64_t)p.NQ * p.Hq * D * 2 >= (1ll << 31)) {
     last_error() = std::string(fn) + ": queries must span less than 2 GiB";
     return SPX_ERR_ARG;
   }
-  const int n_kb = (p.NKV + 32 * kDkvNW - 1) / (32 * kDkvNW);
-  const dim3 kgrid((unsigned)(n_kb * p.Hq)), kblock(64 * kDkvNW);
-  static std::atomic<uint64_t> dkv_lds_set[2];  // per head_dim instantiation, one bit per device
-  if (use_ws) {
-   if constexpr (D <= 128 && SPX_DKV_WS) {
+  static std::atomic<uint64_t> dkv_lds_set;  // per head_dim instantiation, one bit per device
+  if constexpr (D <= 128) {
     // producer / consumer waves, two per SIMD (see attn_bwd_dkv_ws_kernel)
     constexpr int smem = DkvWsSmem<D>::kBytes;
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_ws_kernel<D>), smem,
-                                    dkv_lds_set[0], fn))
+                                    dkv_lds_set, fn))
       return rc;
     const int n_pair_ws = ((p.NKV + 127) / 128 + 1) / 2;  // a workgroup takes two key blocks
     hipLaunchKernelGGL((attn_bwd_dkv_ws_kernel<D>), dim3((unsigned)(n_pair_ws * p.Hq)), dim3(512), smem, st, ps,
                        dOp, NQp, neg, mrows, tb, dkp, dvp);
-   }
-  } else if constexpr (D > 128 && SPX_DKV256_ONEPASS == 2) {
+  } else {
     // dK and dV in one pass over 64-row tiles of Q and dO alone (two buffers of two 32 KB tiles); the
     // transposed operands come out of them through transposing LDS reads
+    const int n_kb = (p.NKV + 32 * kDkvNW - 1) / (32 * kDkvNW);
+    const dim3 kgrid((unsigned)(n_kb * p.Hq)), kblock(64 * kDkvNW);
     constexpr size_t smem = DkvSmem<D, 0, 64, true>::kBytesDma;
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, 4, 0>),
-                                    (int)smem, dkv_lds_set[0], fn))
+                                    (int)smem, dkv_lds_set, fn))
       return rc;
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, 4, 0>), kgrid, kblock, smem, st, ps, dOp, qt, dot,
-                       NQp, lse, delta, tb, dkp, dvp);
-  } else if constexpr (D > 128 && SPX_DKV256_ONEPASS) {
-    // dK and dV in one pass over 32-row tiles (two buffers of four 16 KB tiles)
-    constexpr size_t smem = DkvSmem<D, 0, 32>::kBytesDma;
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, 3, 0>),
-                                    (int)smem, dkv_lds_set[0], fn))
-      return rc;
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, 3, 0>), kgrid, kblock, smem, st, ps, dOp, qt, dot,
-                       NQp, lse, delta, tb, dkp, dvp);
-  } else if constexpr (D > 128) {
-    // one launch per gradient (each loads only the tiles it multiplies with)
-    constexpr size_t smem1 = kPF1 == 2 ? DkvSmem<D, 1>::kBytesDma : DkvSmem<D, 1>::kBytes;
-    constexpr size_t smem2 = kPF2 == 2 ? DkvSmem<D, 2>::kBytesDma : DkvSmem<D, 2>::kBytes;
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF1, 1>),
-                                    (int)smem1, dkv_lds_set[0], fn))
-      return rc;
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF2, 2>),
-                                    (int)smem2, dkv_lds_set[1], fn))
-      return rc;
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF1, 1>), kgrid, kblock, smem1, st, ps, dOp, qt,
-                       dot, NQp, lse, delta, tb, dkp, dvp);
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF2, 2>), kgrid, kblock, smem2, st, ps, dOp, qt,
-                       dot, NQp, lse, delta, tb, dkp, dvp);
-  } else {
-    constexpr size_t smem = kPF == 2 ? DkvSmem<D, 0>::kBytesDma : DkvSmem<D, 0>::kBytes;
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkv_kernel<D, kDkvNW, kPF, 0>),
-                                    (int)smem, dkv_lds_set[0], fn))
-      return rc;
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, kPF, 0>), kgrid, kblock, smem, st, ps, dOp, qt, dot,
-                       NQp, lse, delta, tb, dkp, dvp);
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D, kDkvNW, 4, 0>), kgrid, kblock, smem, st, ps, dOp,
+                       (const uint16_t*)nullptr, (const uint16_t*)nullptr, NQp, lse, delta, tb, dkp, dvp);
   }
   const int64_t items = (int64_t)p.NKV * D / 4 * p.Hkv;
   hipLaunchKernelGGL(attn_dkv_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, dkp,

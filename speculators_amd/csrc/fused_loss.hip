@@ -637,9 +637,7 @@ __global__ __launch_bounds__(kLossThreads) void loss_bwd_kernel(
   const int label = (OP == SPX_LOSS_CE) ? argmax_target[r] : -1;
   const float cd = -lse_d * kLog2e, ct = -lse_t * kLog2e;
 
-#ifndef SPX_LOSS_BWD_UNROLL
 #define SPX_LOSS_BWD_UNROLL 1
-#endif
   constexpr int UNR = SPX_LOSS_BWD_UNROLL;
   for (int64_t c0 = tid; c0 < nchunks; c0 += kLossThreads * UNR) {
     float xs[UNR][8], ys[UNR][8];

@@ -34,21 +34,11 @@
 
 namespace spx {
 
-#ifndef SPX_GEMM_WM
 #define SPX_GEMM_WM 2
-#endif
-#ifndef SPX_GEMM_WN
 #define SPX_GEMM_WN 2
-#endif
-#ifndef SPX_GEMM_MINW
 #define SPX_GEMM_MINW 1
-#endif
-#ifndef SPX_GEMM_READ_EVERY
 #define SPX_GEMM_READ_EVERY 2  // MFMAs per LDS fragment read
-#endif
-#ifndef SPX_GEMM_GROUP_M
 #define SPX_GEMM_GROUP_M 8
-#endif
 constexpr int kWM = SPX_GEMM_WM, kWN = SPX_GEMM_WN;  // waves along M / N of the tile
 constexpr int kNW = kWM * kWN;
 constexpr int kGemmThreads = 64 * kNW;

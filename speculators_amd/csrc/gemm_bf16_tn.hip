@@ -37,12 +37,8 @@ constexpr int kTM = 256, kTN = 256, kTK = 64;
 constexpr int kWM = 2, kWN = 2;
 constexpr int kMI = kTM / kWM / 16, kNI = kTN / kWN / 16;  // 8 x 8 accumulators of 16 x 16 per wave
 constexpr int kKSteps = kTK / 32;                          // MFMA K steps per slab
-#ifndef SPX_GEMM_TN_READ_EVERY
 #define SPX_GEMM_TN_READ_EVERY 2  // MFMAs per LDS fragment (two transposing reads) in the K step before the barrier
-#endif
-#ifndef SPX_GEMM_TN_READ_EVERY_B
 #define SPX_GEMM_TN_READ_EVERY_B 4  // the same in the K step after it, which also issues the global loads
-#endif
 constexpr int kRowBytes = kTM * 2;                          // 512: one t-row of a slab
 constexpr int kABytes = kTK * kRowBytes;                    // one slab of A: 32 KB
 constexpr int kBBytes = kABytes;
@@ -55,9 +51,7 @@ constexpr int kOob = 0x7ffffff0;
 static_assert(kTM == kTN, "both operands use one slab layout");
 static_assert(kABytes + (kKSteps - 1) * 32 * kRowBytes + 4 * kRowBytes < 65536,
               "slab buffer, K step and row pair of a fragment read go into the 16-bit offset field");
-#ifndef SPX_GEMM_TN_GROUP_M
 #define SPX_GEMM_TN_GROUP_M 8
-#endif
 
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef short i16x8 __attribute__((ext_vector_type(8)));

@@ -16,9 +16,7 @@ __device__ __forceinline__ void load8_vec(const T* p, float v[8]);
 
 // streaming accesses bypass the cache hierarchy's allocate-on-access policy: every row is
 // read (and every gradient row written) exactly once per launch
-#ifndef SPX_LOSS_NT
 #define SPX_LOSS_NT 1
-#endif
 __device__ __forceinline__ u32x4 ld16(const void* p) {
 #if SPX_LOSS_NT
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));

@@ -130,6 +130,25 @@ def test_head_sizes_between_the_kernels(d):
                       torch.zeros(1, hkv, 2 * t, 320, device="cuda", dtype=torch.bfloat16), mask)
 
 
+def test_backward_refuses_more_rows_than_its_tile_list_holds():
+    """The dK/dV kernel at head_dim <= 128 lists the query tiles that see a key block in LDS: a call
+    with more rows than that list holds is refused before anything is launched (there is no
+    second kernel behind it), and the forward of the same call still runs."""
+    from speculators_amd._lib import SpxError
+    from speculators_amd.attention import create_ttt_mask, ttt_attention
+
+    t = 131072 + 64
+    doc = torch.zeros(1, t, dtype=torch.long, device="cuda")
+    mask = create_ttt_mask(doc, t, 256)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    q, k, v = (torch.randn(1, 1, t, 64, device="cuda", generator=g).bfloat16().requires_grad_(True)
+               for _ in range(3))
+    out = ttt_attention(q, k, v, mask)
+    assert torch.isfinite(out.float()).all()
+    with pytest.raises(SpxError, match="query rows in one call"):
+        out.backward(torch.ones_like(out))
+
+
 def _random_cases(n, seed):
     """Seeded shapes that land on every edge of the tiling: sequences shorter than one key tile,
     one row past a tile, ragged document packs with and without padding, windows shorter and
