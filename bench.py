@@ -351,6 +351,13 @@ def kernel_rooflines(torch, cfg, t, k_steps, device, windows=(None,)):
 
     ms = time_events(torch, loss_bwd_packed, 20)
     hbm(f"loss_bwd_kernel[KL, packed: {n_live} live of T rows x Vd]", 3.0 * n_live * vd * 2, ms, k_steps)
+    # the yardstick of that launch's size: a plain copy of n_live rows (one read + one write per element;
+    # the kernel above reads two rows for every row it writes)
+    src = lg[:n_live]
+    dst = torch.empty_like(src)
+    ms = time_events(torch, lambda: dst.copy_(src), 20)
+    hbm(f"reference copy[{n_live} x Vd bf16, torch copy_]", 2.0 * n_live * vd * 2, ms, 0)
+    del src, dst
 
     # the first step of the verifier-logits entry point: target rows read THROUGH d2t from the
     # full-vocabulary logits, draft-vocabulary rows written out for the later steps, acceptance

@@ -186,13 +186,13 @@ class DecoderLayer(nn.Module):
                 residual = hidden
                 xin = torch.cat([embeds, hidden], dim=-1)
             else:
-                residual = hidden
-                # both norms write straight into the halves of the 2H-wide projection input
+                # both norms write straight into the halves of the 2H-wide projection input; the
+                # residual goes through the same node (its gradient is folded into the norm's)
                 att = self.self_attn
                 wqkv = self._stager.get(att.q_proj.weight, att.k_proj.weight, att.v_proj.weight)
-                xin = FO.pair_norm_cat(embeds, hidden, self.input_layernorm.gain,
-                                       self.hidden_norm.gain, eps,
-                                       out=None if att.qk_norm else wqkv.x_slot(hidden.shape[-2]))
+                xin, residual = FO.pair_norm_cat(
+                    embeds, hidden, self.input_layernorm.gain, self.hidden_norm.gain, eps,
+                    out=None if att.qk_norm else wqkv.x_slot(hidden.shape[-2]), residual=True)
             a = self.self_attn(xin, position_ids, pos_offset, inv_freq, cache, mask)
         else:
             if isinstance(x, _Prenormed):  # the previous layer already applied this layer's input norm

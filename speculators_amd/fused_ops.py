@@ -86,6 +86,9 @@ class _AddRMSNorm(torch.autograd.Function):
                   _lib.stream_ptr(a.device))
         ctx.save_for_backward(s, w, rstd)
         ctx.shape = a.shape
+        # (a product of gemm.linear_staged says where its output gradient belongs; the sum's gradient
+        # IS that gradient)
+        ctx.grad_slot = getattr(b, "spx_grad_slot", None)
         ctx.set_materialize_grads(False)  # an unused output arrives as None, not as zeros
         return s.view(a.shape), y.view(a.shape)
 
@@ -103,7 +106,15 @@ class _AddRMSNorm(torch.autograd.Function):
             ds2 = ds.reshape(rows, h).to(torch.bfloat16)
             if ds2.stride(1) != 1:
                 ds2 = ds2.contiguous()
-        dx = torch.empty(rows, h, device=s.device, dtype=torch.bfloat16)
+        dx = None
+        if ctx.grad_slot is not None and ctx.needs_input_grad[1]:
+            staged, r0, n = ctx.grad_slot
+            if n == rows:
+                dx = staged.dy_slot(r0, rows)
+                if dx.shape != (rows, h) or not dx.is_contiguous():
+                    dx = None
+        if dx is None:
+            dx = torch.empty(rows, h, device=s.device, dtype=torch.bfloat16)
         scratch = dw = None
         if ctx.needs_input_grad[2]:
             scratch, dw = _dw_buffers(rows, h, s.device)
@@ -123,10 +134,12 @@ def add_rms_norm(a: torch.Tensor, b: torch.Tensor, weight: torch.Tensor, eps: fl
 class _PairNormCat(torch.autograd.Function):
     """``cat([rms_norm(a, wa), rms_norm(b, wb)], -1)`` written straight into the halves of one
     ``[rows, 2H]`` buffer (the input of the first EAGLE3 layer's q/k/v projections,
-    models/eagle3/model_definitions.py:70-94)."""
+    models/eagle3/model_definitions.py:70-94).  With ``residual`` the node also hands ``b`` through
+    as a second output -- the layer's residual stream -- so that the gradient arriving along it is
+    folded into the norm's input gradient by the same kernel instead of being added afterwards."""
 
     @staticmethod
-    def forward(ctx, a, b, wa, wb, eps, out=None):
+    def forward(ctx, a, b, wa, wb, eps, out=None, residual=False):
         _need_bf16(a, b, wa, wb)
         h = a.shape[-1]
         a2, b2 = a.reshape(-1, h), b.reshape(-1, h)
@@ -146,15 +159,25 @@ class _PairNormCat(torch.autograd.Function):
                   _lib.ptr(rstd[1]), rows, h, float(eps), st)
         ctx.save_for_backward(a2, b2, wa, wb, rstd)
         ctx.shapes = (a.shape, b.shape)
-        return out.view(*a.shape[:-1], 2 * h)
+        cat = out.view(*a.shape[:-1], 2 * h)
+        if not residual:
+            return cat
+        ctx.set_materialize_grads(False)  # an unused output arrives as None, not as zeros
+        return cat, b.view_as(b)
 
     @staticmethod
-    def backward(ctx, dy):
+    def backward(ctx, dy, dres=None):
         a2, b2, wa, wb, rstd = ctx.saved_tensors
         rows, h = a2.shape
+        if dy is None:  # only the handed-through residual was used
+            return None, dres, None, None, None, None, None
         dy2 = dy.reshape(rows, 2 * h).to(torch.bfloat16)
         if dy2.stride(1) != 1:
             dy2 = dy2.contiguous()
+        if dres is not None:
+            dres = dres.reshape(rows, h).to(torch.bfloat16)
+            if dres.stride(1) != 1:
+                dres = dres.contiguous()
         st = _lib.stream_ptr(a2.device)
         grads = []
         for i, (x, w) in enumerate(((a2, wa), (b2, wb))):
@@ -164,18 +187,24 @@ class _PairNormCat(torch.autograd.Function):
                 dx = torch.empty(rows, h, device=x.device, dtype=torch.bfloat16)
             if need_dw:
                 scratch, dw = _dw_buffers(rows, h, x.device)
-            if need_dx or need_dw:
-                half = dy2[:, i * h:]
+            half = dy2[:, i * h:]
+            if i == 1 and dres is not None and need_dx:
+                # the residual's gradient rides along: dx = rms_norm_bwd(half) + dres
+                _lib.call("spx_add_rmsnorm_bwd", _lib.ptr(x), x.stride(0), _lib.ptr(w), _lib.ptr(half),
+                          dy2.stride(0), _lib.ptr(dres), dres.stride(0), _lib.ptr(rstd[i]), _lib.ptr(dx),
+                          h, _lib.ptr(dw), _lib.ptr(scratch), rows, h, st)
+            elif need_dx or need_dw:
                 _lib.call("spx_rmsnorm_bwd", _lib.ptr(x), x.stride(0), _lib.ptr(w), _lib.ptr(half),
                           dy2.stride(0), _lib.ptr(rstd[i]), _lib.ptr(dx), h, _lib.ptr(dw),
                           _lib.ptr(scratch), rows, h, st)
             grads.append((dx.view(ctx.shapes[i]) if dx is not None else None, dw))
-        return grads[0][0], grads[1][0], grads[0][1], grads[1][1], None, None
+        return grads[0][0], grads[1][0], grads[0][1], grads[1][1], None, None, None
 
 
-def pair_norm_cat(a, b, weight_a, weight_b, eps: float, out=None) -> torch.Tensor:
-    """See ``_PairNormCat``.  ``out``: a contiguous ``[rows, 2H]`` bf16 buffer for the result."""
-    return _PairNormCat.apply(a, b, weight_a, weight_b, eps, out)
+def pair_norm_cat(a, b, weight_a, weight_b, eps: float, out=None, residual: bool = False):
+    """See ``_PairNormCat``.  ``out``: a contiguous ``[rows, 2H]`` bf16 buffer for the result;
+    ``residual``: return ``(cat, b)`` with ``b`` handed through the node."""
+    return _PairNormCat.apply(a, b, weight_a, weight_b, eps, out, residual)
 
 
 def rope_call(x_ptr, ld_x, x_head_stride, position_ids, inv_freq, out_ptr, ld_out, t, heads, d, rotate,

@@ -293,6 +293,7 @@ class _StagedLinear(torch.autograd.Function):
         ctx.save_for_backward(x2, w)
         ctx.staged, ctx.hip, ctx.x_shape = staged, hip, x.shape
         ctx.slot = staged.take(x2) if ctx.needs_input_grad[1] else -1
+        ctx.rows = x2.shape[0]
         return y.view(*x.shape[:-1], w.shape[0])
 
     @staticmethod
@@ -313,7 +314,13 @@ def linear_staged(x: torch.Tensor, staged, hip: bool = False) -> torch.Tensor:
         x2 = x.reshape(-1, x.shape[-1])
         y = gemm_nt(x2, staged.w) if hip else _project(x2, staged)
         return y.view(*x.shape[:-1], staged.w.shape[0])
-    return _StagedLinear.apply(x, staged.token, staged, hip)
+    y = _StagedLinear.apply(x, staged.token, staged, hip)
+    node = y.grad_fn
+    if node is not None and getattr(node, "slot", -1) >= 0:
+        # where the gradient of `y` belongs, for the backward that produces it (fused_ops._AddRMSNorm):
+        # written there, it is not copied into the weight's output-gradient buffer afterwards
+        y.spx_grad_slot = (staged, node.slot, node.rows)
+    return y
 
 
 class _QKVRope(torch.autograd.Function):

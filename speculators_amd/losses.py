@@ -274,8 +274,9 @@ def head_fused_rows(op: int, x, weight, weight_t, targets, target_stats=None, n_
     if y is not None and y.shape[0] != n:
         raise ValueError(f"targets have {y.shape[0]} rows, expected {n}")
     ks = (None, None) if target_stats is None else (target_stats[0], target_stats[1])
-    loss, am_d, am_t, lse_t, logits = _HeadFusedLoss.apply(x[0], weight, weight_t, y, op, ks[0], ks[1], n,
-                                                           step)
+    # (a view, not x[0]: the backward of a select writes the gradient into a zero-filled copy)
+    loss, am_d, am_t, lse_t, logits = _HeadFusedLoss.apply(x.reshape(t, x.shape[2]), weight, weight_t, y, op,
+                                                           ks[0], ks[1], n, step)
     lead = (1, n)
     return (loss.view(lead), am_d.view(lead), am_t.view(lead), lse_t.view(lead),
             logits.view(1, t, weight.shape[0]))
