@@ -315,6 +315,22 @@ int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
                      void* dv, int64_t dv_head_stride, void* workspace,
                      int64_t workspace_bytes, void* stream);
 
+/* The same, ADDING to what dk and dv hold (dq is written): dk = bf16(float(dk) + this call's
+ * gradient), one rounding per call.  The K / V rows of one TTT step are keys of every later step
+ * (DynamicCache.update, models/eagle3/core.py:283-300), so their gradient is a sum over the steps'
+ * backwards, which the reference's autograd forms with one add per tensor and step.  A caller that
+ * owns one [Hkv, steps*T, D] gradient buffer per layer runs the last step's backward with
+ * spx_ttt_attn_bwd (every row of its (ttt_step+1)*T written) and the earlier steps' with this
+ * entry point, in descending step order on one stream. */
+int spx_ttt_attn_bwd_accumulate(const void* q, int64_t q_head_stride, const void* k,
+                                int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                                const void* out, const void* dout, const float* lse,
+                                const int32_t* row_lo, int64_t T, int32_t ttt_step,
+                                int32_t Hq, int32_t Hkv, int32_t D, float scaling, void* dq,
+                                int64_t dq_head_stride, void* dk, int64_t dk_head_stride,
+                                void* dv, int64_t dv_head_stride, void* workspace,
+                                int64_t workspace_bytes, void* stream);
+
 /* Attention with one interval of visible keys per query: out[i, h, :] = softmax over the keys
  * row_lo[i] <= c < row_hi[i] (out of T; an empty interval gives a zero row).  This is the mask
  * transformers' create_causal_mask builds from a 2-D padding mask -- key j visible to query i iff

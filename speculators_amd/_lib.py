@@ -37,6 +37,7 @@ SIGNATURES: dict[str, list] = {
     "spx_ttt_attn_bwd": [_P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32,
                          _F, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P],
 }
+SIGNATURES["spx_ttt_attn_bwd_accumulate"] = SIGNATURES["spx_ttt_attn_bwd"]
 SIGNATURES["spx_vocab_loss_step_fwd"] = [_I, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I, _P, _P, _P,
                                          _P, _P, _P, _I, _P, _I, _P, _I, _P, _P]
 SIGNATURES["spx_ttt_step_mean"] = [_P, _P, _I, _I64, _F, _P, _P, _P, _P]

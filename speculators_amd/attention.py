@@ -125,16 +125,31 @@ class TTTKVCache:
         self.v = torch.empty(1, hkv, steps * t, d, device=device, dtype=torch.bfloat16)
         self.k_parts: list = []
         self.v_parts: list = []
+        self.grads = _CacheGrads()
 
     def window(self, j: int):
         lo = j * self.t
         return self.k[:, :, lo:lo + self.t], self.v[:, :, lo:lo + self.t]
 
 
+class _CacheGrads:
+    """dK / dV of one layer's cache during ONE backward pass: a ``[1, Hkv, n * T, D]`` buffer each,
+    allocated by the first attention node the pass reaches (the latest step in it, ``n`` steps of
+    keys), added to by the nodes of the earlier steps.  Holds no tensor of the graph."""
+
+    def __init__(self):
+        self.task, self.dk, self.dv, self.low = -1, None, None, 0
+
+
 class _TTTAttentionCached(torch.autograd.Function):
     """TTT attention over a ``TTTKVCache``: the per-step key / value tensors (windows of the
-    cache, already written) are the differentiable inputs, the kernels read the cache in place and
-    the backward hands every step the matching window of the full dK / dV."""
+    cache, already written) are the differentiable inputs, the kernels read the cache in place.
+    The keys of step j are seen by every step from j on, so their gradient is a sum over those steps'
+    backwards.  Autograd would form it with one add per tensor and step; here the nodes of one
+    backward pass share one dK / dV buffer per layer (``_CacheGrads``): the node of the latest step
+    writes it, every earlier one adds to it inside its kernels, and a node returns the gradient of
+    its OWN step's keys only -- complete by then, because the nodes of all later steps depend on
+    this node's output and have run."""
 
     @staticmethod
     def forward(ctx, q, mask: TTTMask, scaling: float, cache: TTTKVCache, n_parts: int, out, *parts):
@@ -157,6 +172,7 @@ class _TTTAttentionCached(torch.autograd.Function):
         ctx.save_for_backward(q, out, lse)
         ctx.kv = (k, v)  # windows of the cache: later steps only write rows beyond them
         ctx.mask, ctx.scaling, ctx.n_parts = mask, float(scaling), n_parts
+        ctx.grads = cache.grads  # (not the cache: its per-step tensors belong to the graph)
         return out
 
     @staticmethod
@@ -169,16 +185,37 @@ class _TTTAttentionCached(torch.autograd.Function):
         dev = q.device
         dout = dout.to(torch.bfloat16).contiguous()
         dq = torch.empty_like(q)
-        dk = torch.empty(1, hkv, n * t, d, device=dev, dtype=torch.bfloat16)
-        dv = torch.empty(1, hkv, n * t, d, device=dev, dtype=torch.bfloat16)
+        g = ctx.grads
+        task = torch._C._current_graph_task_id()
+        shared = task >= 0
+        if shared and g.task == task:
+            if n > g.low:
+                raise RuntimeError("the attention node of a later TTT step ran after an earlier step's "
+                                   "in one backward pass")
+            entry = "spx_ttt_attn_bwd_accumulate"
+            dk, dv = g.dk[:, :, :n * t], g.dv[:, :, :n * t]
+        else:
+            entry = "spx_ttt_attn_bwd"
+            dk = torch.empty(1, hkv, n * t, d, device=dev, dtype=torch.bfloat16)
+            dv = torch.empty(1, hkv, n * t, d, device=dev, dtype=torch.bfloat16)
+            if shared:
+                g.task, g.dk, g.dv = task, dk, dv
         ws = torch.empty(_workspace_bytes(t, hq, hkv, d, True), device=dev, dtype=torch.uint8)
-        _lib.call("spx_ttt_attn_bwd", _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1),
+        _lib.call(entry, _lib.ptr(q), q.stride(1), _lib.ptr(k), k.stride(1),
                   _lib.ptr(v), v.stride(1), _lib.ptr(out), _lib.ptr(dout), _lib.ptr(lse),
                   _lib.ptr(mask.row_lo), t, mask.ttt_step, hq, hkv, d, ctx.scaling,
                   _lib.ptr(dq), dq.stride(1), _lib.ptr(dk), dk.stride(1), _lib.ptr(dv),
                   dv.stride(1), _lib.ptr(ws), ws.numel(), _lib.stream_ptr(dev))
-        dks = [dk[:, :, i * t:(i + 1) * t] for i in range(n)]
-        dvs = [dv[:, :, i * t:(i + 1) * t] for i in range(n)]
+        if not shared:  # outside a backward pass of the engine: every step's window, to be summed by the caller
+            dks = [dk[:, :, i * t:(i + 1) * t] for i in range(n)]
+            dvs = [dv[:, :, i * t:(i + 1) * t] for i in range(n)]
+            return (dq, None, None, None, None, None, *dks, *dvs)
+        g.low = n
+        own = slice((n - 1) * t, n * t)
+        dks, dvs = [None] * n, [None] * n
+        dks[-1], dvs[-1] = dk[:, :, own], dv[:, :, own]
+        if n == 1:  # the first step's node is the last to run: the pass is done with the buffers
+            g.task, g.dk, g.dv = -1, None, None
         return (dq, None, None, None, None, None, *dks, *dvs)
 
 

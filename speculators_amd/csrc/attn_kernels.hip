@@ -2162,10 +2162,12 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkv_ws_kernel(
     dkv_ws_role<D, false>(p, dO, NQp, neg, mrows, dKp, dVp);
 }
 
-// dK[kvh, c, :] = scaling * sum_{h in group} dKp[h, c, :],  dV likewise (no scaling); bf16 out
+// dK[kvh, c, :] = scaling * sum_{h in group} dKp[h, c, :],  dV likewise (no scaling); bf16 out.
+// `accumulate`: what dK / dV hold is added (in fp32, one rounding).
 __global__ __launch_bounds__(256) void attn_dkv_reduce_kernel(
     const float* __restrict__ dKp, const float* __restrict__ dVp, int NKV, int D, int Hq, int Hkv,
-    float scaling, uint16_t* __restrict__ dK, int64_t dk_hs, uint16_t* __restrict__ dV, int64_t dv_hs) {
+    float scaling, uint16_t* __restrict__ dK, int64_t dk_hs, uint16_t* __restrict__ dV, int64_t dv_hs,
+    int accumulate) {
   const int64_t per_head = (int64_t)NKV * D / 4;  // float4 items
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= per_head * Hkv) return;
@@ -2178,8 +2180,15 @@ __global__ __launch_bounds__(256) void attn_dkv_reduce_kernel(
     sk += *reinterpret_cast<const f32x4*>(dKp + base);
     sv += *reinterpret_cast<const f32x4*>(dVp + base);
   }
+  sk *= scaling;
   u32x2 wk, wv;
-  wk.x = pack_bf16x2(sk.x * scaling, sk.y * scaling); wk.y = pack_bf16x2(sk.z * scaling, sk.w * scaling);
+  if (accumulate) {
+    wk = *reinterpret_cast<const u32x2*>(dK + (int64_t)kvh * dk_hs + off);
+    wv = *reinterpret_cast<const u32x2*>(dV + (int64_t)kvh * dv_hs + off);
+    sk.x += bf16_lo(wk.x); sk.y += bf16_hi(wk.x); sk.z += bf16_lo(wk.y); sk.w += bf16_hi(wk.y);
+    sv.x += bf16_lo(wv.x); sv.y += bf16_hi(wv.x); sv.z += bf16_lo(wv.y); sv.w += bf16_hi(wv.y);
+  }
+  wk.x = pack_bf16x2(sk.x, sk.y); wk.y = pack_bf16x2(sk.z, sk.w);
   wv.x = pack_bf16x2(sv.x, sv.y); wv.y = pack_bf16x2(sv.z, sv.w);
   *reinterpret_cast<u32x2*>(dK + (int64_t)kvh * dk_hs + off) = wk;
   *reinterpret_cast<u32x2*>(dV + (int64_t)kvh * dv_hs + off) = wv;
@@ -2199,7 +2208,7 @@ __global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
     const uint16_t* __restrict__ V, int64_t v_hs, const uint16_t* __restrict__ dO,
     const float* __restrict__ LSE, const float* __restrict__ Delta, int T, int n_extra, int Hq,
     int Hkv, float scale_log2e, float scaling, uint16_t* dK, int64_t dk_hs, uint16_t* dV,
-    int64_t dv_hs) {
+    int64_t dv_hs, int accumulate) {
   constexpr int EPL = D / 16;
   // item = kvh * T + i: neighbouring 16-lane rows take neighbouring positions of one K/V head, so
   // their key / value / gradient rows are contiguous in memory.  The tail clamps (no early
@@ -2243,6 +2252,10 @@ __global__ __launch_bounds__(256) void ttt_attn_bwd_diag_kernel(
       vv[e] = vn[e];
       gk[e] = 0.f;
       gv[e] = 0.f;
+    }
+    if (accumulate) {  // what the gradient rows hold is the starting value
+      ld_bf16s<EPL>(dK + gko, gk);
+      ld_bf16s<EPL>(dV + gvo, gv);
     }
     if (j < n_extra) {
       const int64_t rn = ((int64_t)(j + 1) * T + i) * D + d0;
@@ -2344,7 +2357,7 @@ static int launch_fwd(AttnParams p, void* workspace, uint16_t* O, float* lse, hi
 template <int D>
 static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, const float* lse,
                       uint16_t* dQp, int64_t dq_hs, uint16_t* dKp, int64_t dk_hs, uint16_t* dVp,
-                      int64_t dv_hs, void* workspace, hipStream_t st, const char* fn) {
+                      int64_t dv_hs, void* workspace, hipStream_t st, const char* fn, int accumulate = 0) {
   const int NQp = (int)round_up(p.NQ, 128);
   char* w = reinterpret_cast<char*>(workspace);
   uint16_t* kt = reinterpret_cast<uint16_t*>(w);
@@ -2440,18 +2453,18 @@ static int launch_bwd(AttnParams p, const uint16_t* Op, const uint16_t* dOp, con
   }
   const int64_t items = (int64_t)p.NKV * D / 4 * p.Hkv;
   hipLaunchKernelGGL(attn_dkv_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, dkp,
-                     dvp, p.NKV, D, p.Hq, p.Hkv, kLn2, dKp, dk_hs, dVp, dv_hs);
+                     dvp, p.NKV, D, p.Hq, p.Hkv, kLn2, dKp, dk_hs, dVp, dv_hs, accumulate);
   if (p.n_extra > 0) {
     const dim3 dgrid((unsigned)(((int64_t)p.T * p.Hkv + 15) / 16));
     // eight heads per K/V head in registers where they fit (head_dim <= 128), else four
     if (D <= 128 && p.Hq / p.Hkv > 4)
       hipLaunchKernelGGL((ttt_attn_bwd_diag_kernel<D, (D <= 128 ? 8 : 4)>), dgrid, dim3(256), 0, st, ps.Q,
                          ps.q_hs, p.K, p.k_hs, p.V, p.v_hs, dOp, lse, delta, p.T, p.n_extra, p.Hq, p.Hkv,
-                         1.f, kLn2, dKp, dk_hs, dVp, dv_hs);
+                         1.f, kLn2, dKp, dk_hs, dVp, dv_hs, accumulate);
     else
       hipLaunchKernelGGL((ttt_attn_bwd_diag_kernel<D, 4>), dgrid, dim3(256), 0, st, ps.Q, ps.q_hs, p.K,
                          p.k_hs, p.V, p.v_hs, dOp, lse, delta, p.T, p.n_extra, p.Hq, p.Hkv,
-                         1.f, kLn2, dKp, dk_hs, dVp, dv_hs);
+                         1.f, kLn2, dKp, dk_hs, dVp, dv_hs, accumulate);
   }
   return check_launch(fn);
 }
@@ -2532,25 +2545,25 @@ extern "C" int spx_ttt_attn_fwd(const void* q, int64_t q_head_stride, const void
   return launch_fwd<64>(p, workspace, reinterpret_cast<uint16_t*>(out), lse, st, __func__);
 }
 
-extern "C" int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
-                                int64_t k_head_stride, const void* v, int64_t v_head_stride,
-                                const void* out, const void* dout, const float* lse,
-                                const int32_t* row_lo, int64_t T, int32_t ttt_step, int32_t Hq,
-                                int32_t Hkv, int32_t D, float scaling, void* dq,
-                                int64_t dq_head_stride, void* dk, int64_t dk_head_stride, void* dv,
-                                int64_t dv_head_stride, void* workspace, int64_t workspace_bytes,
-                                void* stream) {
-  if (int rc = shape_checks(__func__, T, T, Hq, Hkv, D)) return rc;
-  SPX_REQUIRE(ttt_step >= 0 && ttt_step < 64, "0 <= ttt_step < 64");
-  SPX_REQUIRE(q && k && v && out && dout && lse && row_lo && dq && dk && dv && workspace, "null buffer");
+#define SPX_REQ_FN(cond, what) do { if (!(cond)) return spx::fail_arg(fname, what); } while (0)
+static int ttt_attn_bwd_impl(const char* fname, int accumulate, const void* q, int64_t q_head_stride,
+                             const void* k, int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                             const void* out, const void* dout, const float* lse, const int32_t* row_lo,
+                             int64_t T, int32_t ttt_step, int32_t Hq, int32_t Hkv, int32_t D, float scaling,
+                             void* dq, int64_t dq_head_stride, void* dk, int64_t dk_head_stride, void* dv,
+                             int64_t dv_head_stride, void* workspace, int64_t workspace_bytes,
+                             void* stream) {
+  if (int rc = shape_checks(fname, T, T, Hq, Hkv, D)) return rc;
+  SPX_REQ_FN(ttt_step >= 0 && ttt_step < 64, "0 <= ttt_step < 64");
+  SPX_REQ_FN(q && k && v && out && dout && lse && row_lo && dq && dk && dv && workspace, "null buffer");
   const int64_t kv_rows = (int64_t)(ttt_step + 1) * T * D;
-  SPX_REQUIRE(q_head_stride >= T * D && dq_head_stride >= T * D, "q / dq head stride smaller than T*D");
-  SPX_REQUIRE(k_head_stride >= kv_rows && v_head_stride >= kv_rows && dk_head_stride >= kv_rows &&
+  SPX_REQ_FN(q_head_stride >= T * D && dq_head_stride >= T * D, "q / dq head stride smaller than T*D");
+  SPX_REQ_FN(k_head_stride >= kv_rows && v_head_stride >= kv_rows && dk_head_stride >= kv_rows &&
               dv_head_stride >= kv_rows, "k/v/dk/dv head stride smaller than (ttt_step+1)*T*D");
-  SPX_REQUIRE((q_head_stride | k_head_stride | v_head_stride | dq_head_stride | dk_head_stride |
+  SPX_REQ_FN((q_head_stride | k_head_stride | v_head_stride | dq_head_stride | dk_head_stride |
                dv_head_stride) % 8 == 0, "head strides must be multiples of 8 elements");
-  SPX_REQUIRE(workspace_bytes >= bwd_workspace_bytes(T, T, Hq, Hkv, D), "workspace too small");
-  SPX_REQUIRE(all_aligned16({q, k, v, out, dout, dq, dk, dv, workspace}), "buffers must be 16-byte aligned");
+  SPX_REQ_FN(workspace_bytes >= bwd_workspace_bytes(T, T, Hq, Hkv, D), "workspace too small");
+  SPX_REQ_FN(all_aligned16({q, k, v, out, dout, dq, dk, dv, workspace}), "buffers must be 16-byte aligned");
   AttnParams p = ttt_params(q, q_head_stride, k, k_head_stride, v, v_head_stride, row_lo, T, ttt_step,
                             Hq, Hkv, scaling);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -2561,12 +2574,38 @@ extern "C" int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void
   auto dVp = reinterpret_cast<uint16_t*>(dv);
   if (D == 256)
     return launch_bwd<256>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp, dv_head_stride,
-                           workspace, st, __func__);
+                           workspace, st, fname, accumulate);
   if (D == 128)
     return launch_bwd<128>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp,
-                           dv_head_stride, workspace, st, __func__);
+                           dv_head_stride, workspace, st, fname, accumulate);
   return launch_bwd<64>(p, Op, dOp, lse, dQp, dq_head_stride, dKp, dk_head_stride, dVp, dv_head_stride,
-                        workspace, st, __func__);
+                        workspace, st, fname, accumulate);
+}
+
+extern "C" int spx_ttt_attn_bwd(const void* q, int64_t q_head_stride, const void* k,
+                                int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                                const void* out, const void* dout, const float* lse,
+                                const int32_t* row_lo, int64_t T, int32_t ttt_step, int32_t Hq,
+                                int32_t Hkv, int32_t D, float scaling, void* dq,
+                                int64_t dq_head_stride, void* dk, int64_t dk_head_stride, void* dv,
+                                int64_t dv_head_stride, void* workspace, int64_t workspace_bytes,
+                                void* stream) {
+  return ttt_attn_bwd_impl(__func__, 0, q, q_head_stride, k, k_head_stride, v, v_head_stride, out, dout, lse,
+                           row_lo, T, ttt_step, Hq, Hkv, D, scaling, dq, dq_head_stride, dk, dk_head_stride,
+                           dv, dv_head_stride, workspace, workspace_bytes, stream);
+}
+
+extern "C" int spx_ttt_attn_bwd_accumulate(const void* q, int64_t q_head_stride, const void* k,
+                                           int64_t k_head_stride, const void* v, int64_t v_head_stride,
+                                           const void* out, const void* dout, const float* lse,
+                                           const int32_t* row_lo, int64_t T, int32_t ttt_step, int32_t Hq,
+                                           int32_t Hkv, int32_t D, float scaling, void* dq,
+                                           int64_t dq_head_stride, void* dk, int64_t dk_head_stride,
+                                           void* dv, int64_t dv_head_stride, void* workspace,
+                                           int64_t workspace_bytes, void* stream) {
+  return ttt_attn_bwd_impl(__func__, 1, q, q_head_stride, k, k_head_stride, v, v_head_stride, out, dout, lse,
+                           row_lo, T, ttt_step, Hq, Hkv, D, scaling, dq, dq_head_stride, dk, dk_head_stride,
+                           dv, dv_head_stride, workspace, workspace_bytes, stream);
 }
 
 // ================================================================ span attention

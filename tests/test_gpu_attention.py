@@ -130,6 +130,74 @@ def test_head_sizes_between_the_kernels(d):
                       torch.zeros(1, hkv, 2 * t, 320, device="cuda", dtype=torch.bfloat16), mask)
 
 
+class _Into(torch.autograd.Function):
+    """Writes ``x`` into a window of the K / V cache and returns the window (what the q/k/v
+    projection node of the models does with its ``kv_out``)."""
+
+    @staticmethod
+    def forward(ctx, x, window):
+        # (through an alias with a version counter of its own: the models' kernels write the window
+        # through its address, which autograd does not see either)
+        torch.from_dlpack(window[0].detach()).copy_(x)
+        return window[0]
+
+    @staticmethod
+    def backward(ctx, g):
+        return g, None
+
+
+@pytest.mark.parametrize("window", [None, 48])
+def test_cache_gradients_shared_by_a_backward_pass_equal_autograds_sum(window):
+    """Three chained TTT steps over one K / V cache: the attention nodes of a backward pass add
+    their dK / dV into one buffer per layer and return their own step's rows only.  Against the
+    same chain on concatenated tensors, where every node returns every step's rows and autograd
+    adds them (itself checked against the dense oracle above).  Twice: the second pass must
+    start from a fresh buffer."""
+    from speculators_amd.attention import TTTKVCache, create_ttt_mask, ttt_attention, ttt_attention_cached
+
+    t, hq, hkv, d, steps = 192, 4, 2, 64, 3
+    g = torch.Generator().manual_seed(7)
+    doc = _docs(t, [100, 92]).cuda()
+    xs = [torch.randn(1, t, hq * d, generator=g).bfloat16().cuda() for _ in range(steps)]
+    go = torch.randn(1, t, hq, d, generator=g).bfloat16().cuda()
+
+    def heads(x, n):  # [1, T, n*D] -> [1, n, T, D]
+        return x.view(1, t, n, d).transpose(1, 2).contiguous()
+
+    def chain(cached):
+        leaves = [x.clone().requires_grad_(True) for x in xs]
+        mask = create_ttt_mask(doc, t, window)
+        cache = TTTKVCache(hkv, t, d, steps, "cuda")
+        ks, vs, h, total = [], [], None, 0
+        for j in range(steps):
+            h = leaves[j] if h is None else (leaves[j] + 0.5 * h)
+            q = heads(h, hq)
+            k_new, v_new = heads(h[..., :hkv * d], hkv), heads(h[..., hkv * d:2 * hkv * d] * 0.5, hkv)
+            if cached:
+                kw, vw = cache.window(j)
+                out = ttt_attention_cached(q, _Into.apply(k_new, (kw,)), _Into.apply(v_new, (vw,)), cache, mask)
+            else:
+                ks.append(k_new)
+                vs.append(v_new)
+                out = ttt_attention(q, torch.cat(ks, 2), torch.cat(vs, 2), mask)
+            total = total + (out.float() * go.float()).sum() * (j + 1)
+            h = out.reshape(1, t, hq * d)
+            mask = mask.extended()
+        return leaves, total
+
+    want_leaves, want = chain(False)
+    want.backward()
+    leaves, got = chain(True)
+    assert (got - want).abs().item() <= 1e-3 * want.abs().item() + 1e-3
+    for rep in range(2):
+        for x in leaves:
+            x.grad = None
+        got.backward(retain_graph=rep == 0)
+        for j, (a, b) in enumerate(zip(leaves, want_leaves)):
+            err = (a.grad.float() - b.grad.float()).abs().max().item()
+            assert err <= 2 ** -6 * b.grad.float().abs().max().item(), (rep, j, err)
+
+
 def test_backward_refuses_more_rows_than_its_tile_list_holds():
     """The dK/dV kernel at head_dim <= 128 lists the query tiles that see a key block in LDS: a call
     with more rows than that list holds is refused before anything is launched (there is no
