@@ -33,14 +33,17 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "kernels_config1_hbm_traffic_pmc.txt")
 # bench key -> (substring of the kernel name, launch grid in threads or None = any)
 TRAFFIC_ROWS = {
-    "gemm_fwd": ("gemm_bf16_nt_kernel", 512000),
-    "gemm_dx": ("gemm_bf16_nt_kernel", 65536),
+    "gemm_fwd": ("gemm_bf16_nt_kernel<true, 0>", 512000),
+    "gemm_dx": ("gemm_bf16_nt_kernel<true, 0>", 65536),
     "loss_fwd": ("loss_fwd_kernel<unsigned short, 0, true, false, false", None),
     "loss_fwd_reuse": ("loss_fwd_kernel<unsigned short, 0, true, true, false", None),
     "gemm_tn": ("gemm_bf16_tn_kernel<2, false>", None),
-    # (the summary averages the attention kernels over TTT steps 0 and 6 and the loss backward over its
-    # full and packed launches: no per-launch figure for those)
+    # (the summary averages the loss backward over its full and packed launches: no per-launch figure)
 }
+# The attention kernels are listed per timed call in lines that start with "[attn_step<k>]" or
+# "[attn_step<k>_w<window>]": a forward call is the V^T transpose + attn_fwd_kernel, a backward call every
+# other kernel of the section (one launch of each per call); their sums are the keys "<section>_fwd|_bwd"
+ATTN_FWD_KERNELS = ("attn_fwd_kernel", "transpose_bf16_kernel<false>")
 
 
 def load_measured_traffic(path=TRAFFIC_SUMMARY):
@@ -53,11 +56,21 @@ def load_measured_traffic(path=TRAFFIC_SUMMARY):
     m = re.search(r"FETCH_SIZE under-reads by\s+a factor ([0-9.]+)", text.replace("\n#", " "))
     fetch_scale = float(m.group(1)) if m else 1.0
     rows = []
+    out = {}
+    calls = {}
     for line in text.splitlines():
         m = re.match(r"^(?!#)(.*?) grid=(\d+)\s+n=\s*\d+\s+FETCH_KiB avg\s+([0-9.]+)\s+WRITE_KiB avg\s+([0-9.]+)", line)
-        if m:
-            rows.append((m.group(1), int(m.group(2)), float(m.group(3)), float(m.group(4))))
-    out = {}
+        if not m:
+            continue
+        name, kib = m.group(1), fetch_scale * float(m.group(3)) + float(m.group(4))
+        sec = re.match(r"^\[(attn_step\w+)\] (.*)$", name)
+        if sec:
+            side = "_fwd" if any(k in sec.group(2) for k in ATTN_FWD_KERNELS) else "_bwd"
+            calls[sec.group(1) + side] = calls.get(sec.group(1) + side, 0.0) + kib
+        else:
+            rows.append((name, int(m.group(2)), float(m.group(3)), float(m.group(4))))
+    for key, kib in calls.items():
+        out[key] = int(kib * 1024)
     for key, (name, grid) in TRAFFIC_ROWS.items():
         hit = [r for r in rows if name in r[0] and (grid is None or r[1] == grid)]
         if len(hit) == 1:
