@@ -394,7 +394,7 @@ def kernel_rooflines(torch, cfg, t, k_steps, device, windows=(None,)):
                   _lib.ptr(counts), st)
 
     ms = time_events(torch, loss_step_gather, 20)
-    hbm("loss_fwd_kernel[KL + d2t gather from T x Vt + acceptance chain, step 0 of --targets logits]",
+    hbm("loss_fwd_gather_pipe_kernel[KL + d2t gather from T x Vt + acceptance chain, step 0 of --targets logits]",
         float(t) * (vd * 2 + touched + vd * 2), ms, 0)
     del tg, lg, grad, y, full, gathered
 

@@ -433,6 +433,18 @@ int spx_add_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weight, const v
                         int64_t ld_dy, const void* dres, int64_t ld_dres, const float* rstd,
                         void* dx, int64_t ld_dx, void* dweight, float* dw_scratch,
                         int64_t rows, int64_t H, void* stream);
+/* The backward of either norm for a gain that is applied several times in one forward (once per
+ * TTT step: models/eagle3/core.py:286-306): dx as above (dres may be NULL), while the gain's
+ * gradient stays as partial sums in dw_scratch (spx_rmsnorm_bwd_slots(rows, H) * H floats) --
+ * written when accumulate == 0, added to when != 0 (every use with the same rows and H) -- until
+ * spx_rmsnorm_dweight reduces them once, in a fixed order, to dweight (bf16 [H]).  The sum over the
+ * uses is then formed in fp32 with one rounding, where autograd adds rounded per-use gradients. */
+int spx_rmsnorm_bwd_partial(const void* x, int64_t ld_x, const void* weight, const void* dy,
+                            int64_t ld_dy, const void* dres, int64_t ld_dres,
+                            const float* rstd, void* dx, int64_t ld_dx, float* dw_scratch,
+                            int32_t accumulate, int64_t rows, int64_t H, void* stream);
+int spx_rmsnorm_dweight(const float* dw_scratch, int64_t slots, int64_t H, void* dweight,
+                        void* stream);
 
 /* Rotary embedding fused with the head-major relayout that precedes attention
  * (apply_rotary_pos_emb + the view/transpose of LlamaAttention.forward; for

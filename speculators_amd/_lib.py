@@ -60,6 +60,8 @@ SIGNATURES["spx_rmsnorm_bwd_slots"] = [_I64, _I64]
 SIGNATURES["spx_rmsnorm_bwd"] = [_P, _I64, _P, _P, _I64, _P, _P, _I64, _P, _P, _I64, _I64, _P]
 SIGNATURES["spx_add_rmsnorm_fwd"] = [_P, _I64, _P, _I64, _P, _I64, _P, _P, _I64, _P, _I64, _I64, _F, _P]
 SIGNATURES["spx_add_rmsnorm_bwd"] = [_P, _I64, _P, _P, _I64, _P, _I64, _P, _P, _I64, _P, _P, _I64, _I64, _P]
+SIGNATURES["spx_rmsnorm_bwd_partial"] = [_P, _I64, _P, _P, _I64, _P, _I64, _P, _P, _I64, _P, _I32, _I64, _I64, _P]
+SIGNATURES["spx_rmsnorm_dweight"] = [_P, _I64, _I64, _P, _P]
 SIGNATURES["spx_rope_relayout"] = [_P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _I64, _P]
 SIGNATURES["spx_swiglu_rows_fwd"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _P]
 SIGNATURES["spx_swiglu_rows_bwd"] = [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _P]

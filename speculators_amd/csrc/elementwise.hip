@@ -89,13 +89,14 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(
 // dx = rstd * (g - xhat * mean(g * xhat)), g = dy * w, xhat = x * rstd;
 // dw partial sums: block b accumulates the rows b, b + gridDim.x, ... per column.
 // dres (may be null): gradient that reaches x along the residual stream, added before the
-// one rounding of dx.  dx may be null (only dw wanted).
+// one rounding of dx.  dx may be null (only dw wanted).  accumulate: the partial sums start from
+// what dw_part holds (a gain that is applied several times per forward: one buffer, one final sum).
 template <int MAXC, bool WAVE_ROWS>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(
     const uint16_t* __restrict__ x, int64_t ld_x, const uint16_t* __restrict__ w,
     const uint16_t* __restrict__ dy, int64_t ld_dy, const float* __restrict__ rstd,
     uint16_t* __restrict__ dx, int64_t ld_dx, float* __restrict__ dw_part, int64_t rows, int H,
-    const uint16_t* __restrict__ dres = nullptr, int64_t ld_dres = 0) {
+    const uint16_t* __restrict__ dres = nullptr, int64_t ld_dres = 0, int accumulate = 0) {
   __shared__ float red[4];
   const int nthr = WAVE_ROWS ? 64 : 256;
   const int t = WAVE_ROWS ? (threadIdx.x & 63) : threadIdx.x;
@@ -108,6 +109,13 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(
     if (ch < nch) unpack8f(*reinterpret_cast<const u32x4*>(w + ch * 8), wv[c]);
 #pragma unroll
     for (int e = 0; e < 8; ++e) dwacc[c][e] = 0.f;
+    if (accumulate && dw_part && ch < nch) {
+      const int64_t slot0 = WAVE_ROWS ? (int64_t)blockIdx.x * 4 + wave : blockIdx.x;
+      const float* o = dw_part + slot0 * H + ch * 8;
+      const f32x4 a = *reinterpret_cast<const f32x4*>(o), b = *reinterpret_cast<const f32x4*>(o + 4);
+      dwacc[c][0] = a.x; dwacc[c][1] = a.y; dwacc[c][2] = a.z; dwacc[c][3] = a.w;
+      dwacc[c][4] = b.x; dwacc[c][5] = b.y; dwacc[c][6] = b.z; dwacc[c][7] = b.w;
+    }
   }
   const int64_t first = WAVE_ROWS ? (int64_t)blockIdx.x * 4 + wave : blockIdx.x;
   const int64_t stride = WAVE_ROWS ? (int64_t)gridDim.x * 4 : gridDim.x;
@@ -507,13 +515,14 @@ extern "C" int spx_add_rmsnorm_fwd(const void* a, int64_t ld_a, const void* b, i
 static int rmsnorm_bwd_launch(const char* fn, const void* x, int64_t ld_x, const void* weight, const void* dy,
                               int64_t ld_dy, const void* dres, int64_t ld_dres, const float* rstd, void* dx,
                               int64_t ld_dx, void* dweight, float* dw_scratch, int64_t rows, int64_t H,
-                              void* stream) {
+                              void* stream, bool partial_only = false, int accumulate = 0) {
   if (!(rows > 0 && H > 0)) return fail_arg(fn, "bad sizes");
   if (!(H % 8 == 0 && ld_x % 8 == 0 && ld_dy % 8 == 0 && ld_dx % 8 == 0 && ld_dres % 8 == 0))
     return fail_arg(fn, "H and the row strides must be multiples of 8");
   if (H > 16384) return fail_arg(fn, "H must be at most 16384");
   if (!(x && weight && dy && rstd)) return fail_arg(fn, "null buffer");
-  if (!(dx || dweight)) return fail_arg(fn, "neither dx nor dweight requested");
+  if (!(dx || dweight || partial_only)) return fail_arg(fn, "neither dx nor dweight requested");
+  if (partial_only && !dw_scratch) return fail_arg(fn, "null dw_scratch");
   if (dres && !dx) return fail_arg(fn, "a residual gradient needs dx");
   if (dweight && !dw_scratch)
     return fail_arg(fn, "dweight needs dw_scratch (spx_rmsnorm_bwd_slots(rows, H) * H floats)");
@@ -525,17 +534,17 @@ static int rmsnorm_bwd_launch(const char* fn, const void* x, int64_t ld_x, const
   auto dyp = reinterpret_cast<const uint16_t*>(dy);
   auto drp = reinterpret_cast<const uint16_t*>(dres);
   auto dxp = reinterpret_cast<uint16_t*>(dx);
-  float* part = dweight ? dw_scratch : nullptr;
+  float* part = (dweight || partial_only) ? dw_scratch : nullptr;
   const int64_t slots = spx_rmsnorm_bwd_slots(rows, H);
   if (H <= 512)
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<1, true>), dim3((unsigned)(slots / 4)), dim3(256), 0, st, xp, ld_x,
-                       wp, dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H, drp, ld_dres);
+                       wp, dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H, drp, ld_dres, accumulate);
   else if (H <= 4096)
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<2, false>), dim3((unsigned)slots), dim3(256), 0, st, xp, ld_x, wp,
-                       dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H, drp, ld_dres);
+                       dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H, drp, ld_dres, accumulate);
   else
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<8, false>), dim3((unsigned)slots), dim3(256), 0, st, xp, ld_x, wp,
-                       dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H, drp, ld_dres);
+                       dyp, ld_dy, rstd, dxp, ld_dx, part, rows, (int)H, drp, ld_dres, accumulate);
   if (dweight)
     hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((H + 31) / 32)), dim3(256), 0, st, part, slots, (int)H,
                        reinterpret_cast<uint16_t*>(dweight));
@@ -555,6 +564,25 @@ extern "C" int spx_add_rmsnorm_bwd(const void* x, int64_t ld_x, const void* weig
                                    int64_t H, void* stream) {
   return rmsnorm_bwd_launch(__func__, x, ld_x, weight, dy, ld_dy, dres, ld_dres, rstd, dx, ld_dx, dweight,
                             dw_scratch, rows, H, stream);
+}
+
+extern "C" int spx_rmsnorm_bwd_partial(const void* x, int64_t ld_x, const void* weight, const void* dy,
+                                       int64_t ld_dy, const void* dres, int64_t ld_dres, const float* rstd,
+                                       void* dx, int64_t ld_dx, float* dw_scratch, int32_t accumulate,
+                                       int64_t rows, int64_t H, void* stream) {
+  return rmsnorm_bwd_launch(__func__, x, ld_x, weight, dy, ld_dy, dres, ld_dres, rstd, dx, ld_dx, nullptr,
+                            dw_scratch, rows, H, stream, true, accumulate != 0);
+}
+
+extern "C" int spx_rmsnorm_dweight(const float* dw_scratch, int64_t slots, int64_t H, void* dweight,
+                                   void* stream) {
+  const char* fn = __func__;
+  if (!(slots > 0 && H > 0 && H % 8 == 0 && H <= 16384)) return fail_arg(fn, "bad sizes");
+  if (!(dw_scratch && dweight && al16(dw_scratch))) return fail_arg(fn, "null or unaligned buffer");
+  hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((H + 31) / 32)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), dw_scratch, slots, (int)H,
+                     reinterpret_cast<uint16_t*>(dweight));
+  return check_launch(fn);
 }
 
 static int rope_relayout_impl(const char* fn, const void* x, int64_t ld_x, const int64_t* position_ids,

@@ -33,6 +33,7 @@ class _RMSNorm(torch.autograd.Function):
                   _lib.ptr(rstd), rows, h, float(eps), _lib.stream_ptr(x.device))
         ctx.save_for_backward(x2, w, rstd)
         ctx.shape = x.shape
+        ctx.gain_grads = getattr(weight, "spx_gain_grads", None)
         return y.view(x.shape)
 
     @staticmethod
@@ -43,12 +44,7 @@ class _RMSNorm(torch.autograd.Function):
         if dy2.stride(1) != 1:
             dy2 = dy2.contiguous()
         dx = torch.empty(rows, h, device=x2.device, dtype=torch.bfloat16)
-        dw = scratch = None
-        if ctx.needs_input_grad[1]:
-            scratch, dw = _dw_buffers(rows, h, x2.device)
-        _lib.call("spx_rmsnorm_bwd", _lib.ptr(x2), x2.stride(0), _lib.ptr(w), _lib.ptr(dy2),
-                  dy2.stride(0), _lib.ptr(rstd), _lib.ptr(dx), h, _lib.ptr(dw), _lib.ptr(scratch),
-                  rows, h, _lib.stream_ptr(x2.device))
+        dw = _norm_backward(ctx.gain_grads, ctx.needs_input_grad[1], x2, w, dy2, None, rstd, dx, rows, h)
         return dx.view(ctx.shape), dw, None
 
 
@@ -60,6 +56,73 @@ def _dw_buffers(rows: int, h: int, device):
     slots = int(_lib.load().spx_rmsnorm_bwd_slots(rows, h))
     return (torch.empty(slots * h, device=device, dtype=torch.float32),
             torch.empty(h, device=device, dtype=torch.bfloat16))
+
+
+class GainGrads:
+    """The gradient of one RMSNorm gain over ALL of its uses in one backward pass (a draft layer's
+    norms run once per TTT step): the uses leave their partial column sums in one fp32 buffer --
+    the first writes it, the others add to it inside their kernels -- and the node that staged
+    the gain (``weights._StageGain``), which autograd runs after every use, reduces it once.
+    A staged gain carries its ``GainGrads`` as the attribute ``spx_gain_grads``."""
+
+    def __init__(self):
+        self.scratch, self.slots, self.h, self.marked = None, 0, 0, False
+
+    def target(self, rows: int, h: int, device):
+        """``(scratch, accumulate)`` for a use over ``rows`` rows, None if it cannot share the buffer
+        (another row count lays the partial sums out differently): it then returns a gradient of
+        its own, which autograd adds."""
+        slots = int(_lib.load().spx_rmsnorm_bwd_slots(rows, h))
+        if self.scratch is None:
+            self.scratch = torch.empty(slots * h, device=device, dtype=torch.float32)
+            self.slots, self.h = slots, h
+            return self.scratch, 0
+        if (slots, h) != (self.slots, self.h) or self.scratch.device != device:
+            return None
+        return self.scratch, 1
+
+    def mark(self, device):
+        """What a use returns as the gain's gradient: an empty marker that makes autograd reach the
+        staging node, once per backward pass; None afterwards."""
+        if self.marked:
+            return None
+        self.marked = True
+        return torch.zeros(1, device=device, dtype=torch.bfloat16).expand(self.h)
+
+    def finish(self):
+        """The summed gradient (bf16 ``[H]``) of the uses recorded since the last call, or None."""
+        scratch, self.scratch, self.marked = self.scratch, None, False
+        if scratch is None:
+            return None
+        dw = torch.empty(self.h, device=scratch.device, dtype=torch.bfloat16)
+        _lib.call("spx_rmsnorm_dweight", _lib.ptr(scratch), self.slots, self.h, _lib.ptr(dw),
+                  _lib.stream_ptr(scratch.device))
+        return dw
+
+
+def _norm_backward(grads, need_dw, x, w, dy, dres, rstd, dx, rows, h):
+    """One launch of the norm's backward; returns the gradient to hand autograd for the gain."""
+    dev = x.device
+    st = _lib.stream_ptr(dev)
+    ld_dres = dres.stride(0) if dres is not None else 0
+    if need_dw and grads is not None:
+        tgt = grads.target(rows, h, dev)
+        if tgt is not None:
+            _lib.call("spx_rmsnorm_bwd_partial", _lib.ptr(x), x.stride(0), _lib.ptr(w), _lib.ptr(dy),
+                      dy.stride(0), _lib.ptr(dres), ld_dres, _lib.ptr(rstd), _lib.ptr(dx), h,
+                      _lib.ptr(tgt[0]), tgt[1], rows, h, st)
+            return grads.mark(dev)
+    scratch = dw = None
+    if need_dw:
+        scratch, dw = _dw_buffers(rows, h, dev)
+    if dres is not None:
+        _lib.call("spx_add_rmsnorm_bwd", _lib.ptr(x), x.stride(0), _lib.ptr(w), _lib.ptr(dy), dy.stride(0),
+                  _lib.ptr(dres), ld_dres, _lib.ptr(rstd), _lib.ptr(dx), h, _lib.ptr(dw), _lib.ptr(scratch),
+                  rows, h, st)
+    else:
+        _lib.call("spx_rmsnorm_bwd", _lib.ptr(x), x.stride(0), _lib.ptr(w), _lib.ptr(dy), dy.stride(0),
+                  _lib.ptr(rstd), _lib.ptr(dx), h, _lib.ptr(dw), _lib.ptr(scratch), rows, h, st)
+    return dw
 
 
 class _AddRMSNorm(torch.autograd.Function):
@@ -89,6 +152,7 @@ class _AddRMSNorm(torch.autograd.Function):
         # (a product of gemm.linear_staged says where its output gradient belongs; the sum's gradient
         # IS that gradient)
         ctx.grad_slot = getattr(b, "spx_grad_slot", None)
+        ctx.gain_grads = getattr(weight, "spx_gain_grads", None)
         ctx.set_materialize_grads(False)  # an unused output arrives as None, not as zeros
         return s.view(a.shape), y.view(a.shape)
 
@@ -115,12 +179,7 @@ class _AddRMSNorm(torch.autograd.Function):
                     dx = None
         if dx is None:
             dx = torch.empty(rows, h, device=s.device, dtype=torch.bfloat16)
-        scratch = dw = None
-        if ctx.needs_input_grad[2]:
-            scratch, dw = _dw_buffers(rows, h, s.device)
-        _lib.call("spx_add_rmsnorm_bwd", _lib.ptr(s), h, _lib.ptr(w), _lib.ptr(dy2), dy2.stride(0),
-                  _lib.ptr(ds2), ds2.stride(0) if ds2 is not None else 0, _lib.ptr(rstd), _lib.ptr(dx),
-                  h, _lib.ptr(dw), _lib.ptr(scratch), rows, h, _lib.stream_ptr(s.device))
+        dw = _norm_backward(ctx.gain_grads, ctx.needs_input_grad[2], s, w, dy2, ds2, rstd, dx, rows, h)
         dx = dx.view(ctx.shape)
         return dx, dx, dw, None, None
 
@@ -151,6 +210,7 @@ class _PairNormCat(torch.autograd.Function):
         if out is None or out.shape != (rows, 2 * h) or not out.is_contiguous():
             out = torch.empty(rows, 2 * h, device=a.device, dtype=torch.bfloat16)
         rstd = torch.empty(2, rows, device=a.device, dtype=torch.float32)
+        ctx.gain_grads = (getattr(wa, "spx_gain_grads", None), getattr(wb, "spx_gain_grads", None))
         wa, wb = wa.contiguous(), wb.contiguous()
         st = _lib.stream_ptr(a.device)
         _lib.call("spx_rmsnorm_fwd", _lib.ptr(a2), a2.stride(0), _lib.ptr(wa), _lib.ptr(out), 2 * h,
@@ -178,26 +238,19 @@ class _PairNormCat(torch.autograd.Function):
             dres = dres.reshape(rows, h).to(torch.bfloat16)
             if dres.stride(1) != 1:
                 dres = dres.contiguous()
-        st = _lib.stream_ptr(a2.device)
         grads = []
         for i, (x, w) in enumerate(((a2, wa), (b2, wb))):
             need_dx, need_dw = ctx.needs_input_grad[i], ctx.needs_input_grad[2 + i]
-            dx = dw = scratch = None
+            dx = dw = None
             if need_dx:
                 dx = torch.empty(rows, h, device=x.device, dtype=torch.bfloat16)
-            if need_dw:
-                scratch, dw = _dw_buffers(rows, h, x.device)
-            half = dy2[:, i * h:]
-            if i == 1 and dres is not None and need_dx:
-                # the residual's gradient rides along: dx = rms_norm_bwd(half) + dres
-                _lib.call("spx_add_rmsnorm_bwd", _lib.ptr(x), x.stride(0), _lib.ptr(w), _lib.ptr(half),
-                          dy2.stride(0), _lib.ptr(dres), dres.stride(0), _lib.ptr(rstd[i]), _lib.ptr(dx),
-                          h, _lib.ptr(dw), _lib.ptr(scratch), rows, h, st)
-            elif need_dx or need_dw:
-                _lib.call("spx_rmsnorm_bwd", _lib.ptr(x), x.stride(0), _lib.ptr(w), _lib.ptr(half),
-                          dy2.stride(0), _lib.ptr(rstd[i]), _lib.ptr(dx), h, _lib.ptr(dw),
-                          _lib.ptr(scratch), rows, h, st)
+            if need_dx or need_dw:
+                # (the residual's gradient rides along with b's: dx = rms_norm_bwd(half) + dres)
+                dw = _norm_backward(ctx.gain_grads[i], need_dw, x, w, dy2[:, i * h:],
+                                    dres if i == 1 and need_dx else None, rstd[i], dx, rows, h)
             grads.append((dx.view(ctx.shapes[i]) if dx is not None else None, dw))
+        if dres is not None and not ctx.needs_input_grad[1]:
+            raise RuntimeError("the handed-through residual received a gradient but b needs none")
         return grads[0][0], grads[1][0], grads[0][1], grads[1][1], None, None, None
 
 

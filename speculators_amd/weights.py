@@ -273,6 +273,30 @@ class _Stage(torch.autograd.Function):
         return (None, *grads)
 
 
+class _StageGain(torch.autograd.Function):
+    """bf16 compute copy of an RMSNorm gain (``1 + p`` for the zero-centred form).  Its backward
+    adds what the uses left in the gain's ``GainGrads`` (reduced here, once) to whatever gradient
+    arrives the ordinary way, and casts to the parameter's dtype."""
+
+    @staticmethod
+    def forward(ctx, p, plus_one, grads):
+        ctx.grads, ctx.dtype = grads, p.dtype
+        if plus_one:
+            return (1.0 + p.detach().float()).to(torch.bfloat16)
+        return p.detach().to(torch.bfloat16) if p.dtype != torch.bfloat16 else p.detach().clone()
+
+    @staticmethod
+    def backward(ctx, g):
+        total = ctx.grads.finish()
+        if total is None:
+            out = g
+        elif g is None or g.stride(0) == 0:  # nothing but the empty marker arrived
+            out = total
+        else:
+            out = (total.float() + g.float())
+        return (out.to(ctx.dtype) if out is not None else None), None, None
+
+
 class WeightStager:
     """Hands out the ``Staged`` compute weights of one model.  ``begin()`` starts a forward."""
 
@@ -320,15 +344,22 @@ class WeightStager:
         return st
 
     def gain(self, p: torch.Tensor, plus_one: bool = False) -> torch.Tensor:
-        """A small 1-D weight (an RMSNorm gain) in bf16 for the running forward: the parameter
-        itself, or an ordinary differentiable cast of an fp32 master (its per-use gradients are
-        tiny; autograd sums them and casts the sum back).  ``plus_one``: the gain is ``1 + p``
-        (evaluated in fp32), the form of the Qwen3-Next norms."""
+        """A small 1-D weight (an RMSNorm gain) in bf16 for the running forward.  ``plus_one``: the
+        gain is ``1 + p`` (evaluated in fp32), the form of the Qwen3-Next norms.  A trainable gain
+        goes through one autograd node (``_StageGain``) and carries a ``fused_ops.GainGrads``: the
+        norm kernels of all its uses leave their partial sums there, and the node reduces them
+        once, after the last use's backward."""
         key = ("gain", id(p), plus_one)
         hit = self._fwd.get(key)
         if hit is None:
             _check_param_dtype(p)
-            if plus_one:
+            if p.requires_grad and torch.is_grad_enabled():
+                from .fused_ops import GainGrads
+
+                grads = GainGrads()
+                hit = _StageGain.apply(p, plus_one, grads)
+                hit.spx_gain_grads = grads
+            elif plus_one:
                 hit = (1.0 + p.float()).to(torch.bfloat16)
             else:
                 hit = p if p.dtype == torch.bfloat16 else p.to(torch.bfloat16)

@@ -251,6 +251,60 @@ def test_stager_refuses_fp32_outside_autocast_and_keeps_frozen_copies():
         assert compute_input(torch.ones(2, 2, device="cuda")).dtype == torch.bfloat16
 
 
+@pytest.mark.parametrize("master", [False, True])
+def test_gain_gradient_over_several_uses_is_reduced_once(master):
+    """A gain read through the weight stager and applied four times in one forward -- by all three
+    norm nodes, three times over the same number of rows and once over another -- gets the sum of
+    the per-use gradients: the uses with equal rows leave partial sums in one buffer that the
+    staging node reduces, the odd one hands autograd a gradient of its own.  Against fp32 autograd
+    of the same expression; a second backward over the retained graph gives the same result."""
+    from speculators_amd import fused_ops as FO
+    from speculators_amd.weights import WeightStager
+
+    h, rows = 512, 300
+    g = torch.Generator().manual_seed(3)
+    p = (1 + 0.2 * torch.randn(h, generator=g))
+    xs = [(torch.randn(1, r, h, generator=g) * 2).bfloat16() for r in (rows, rows, rows, 77)]
+    gos = [torch.randn(1, r, h, generator=g).bfloat16() for r in (rows, rows, rows, 77)]
+    extra = torch.randn(1, rows, h, generator=g).bfloat16()
+
+    def expression(norm, add_norm, pair, gain, x):
+        y0 = norm(x[0], gain)
+        _, y1 = add_norm(x[1], extra_d, gain)
+        y2 = pair(x[2], x[0], gain, gain)  # both halves of the pair use the gain
+        y3 = norm(x[3], gain)
+        return y0, y1, y2, y3
+
+    param = p.cuda().to(torch.float32 if master else torch.bfloat16).requires_grad_(True)
+    extra_d = extra.cuda()
+    stager = WeightStager()
+    stager.begin()
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=master):
+        gain = stager.gain(param)
+        assert stager.gain(param) is gain and gain.dtype == torch.bfloat16
+        outs = expression(lambda x, w: FO.rms_norm(x, w, 1e-5),
+                          lambda a, b, w: FO.add_rms_norm(a, b, w, 1e-5),
+                          lambda a, b, wa, wb: FO.pair_norm_cat(a, b, wa, wb, 1e-5),
+                          gain, [x.cuda() for x in xs])
+    go2 = torch.cat([gos[2], gos[0]], -1)
+    total = sum((o.float() * w.cuda().float()).sum() for o, w in zip(outs, (gos[0], gos[1], go2, gos[3])))
+    total.backward(retain_graph=True)
+    first = param.grad.clone()
+    assert first.dtype == param.dtype
+    param.grad = None
+    total.backward()
+    assert torch.equal(param.grad, first)
+
+    pr = p.bfloat16().float().requires_grad_(True)
+    extra_d = extra.float()
+    ref = expression(lambda x, w: OE.rms_norm(x, w, 1e-5),
+                     lambda a, b, w: (None, OE.rms_norm(a + b, w, 1e-5)),
+                     lambda a, b, wa, wb: torch.cat([OE.rms_norm(a, wa, 1e-5), OE.rms_norm(b, wb, 1e-5)], -1),
+                     pr, [x.float() for x in xs])
+    sum((o * w.float()).sum() for o, w in zip(ref, (gos[0], gos[1], go2, gos[3]))).backward()
+    _close(first, pr.grad, rel=1e-2)
+
+
 @pytest.mark.parametrize("rows", [1, 63, 64, 1024, 1025, 5000])
 @pytest.mark.parametrize("with_labels", [False, True])
 def test_pack_row_map_and_unpack_rows(rows, with_labels):
