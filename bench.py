@@ -333,11 +333,13 @@ def kernel_rooflines(torch, cfg, t, k_steps, device, windows=(None,)):
                   _lib.ptr(stats[0]), _lib.ptr(stats[1]), _lib.ptr(stats[2]), _lib.ptr(stats[3]),
                   _lib.ptr(arg[0]), _lib.ptr(arg[1]), 1, st)
 
+    # (what the timed step launches is the one-pass form further down; these two are the streaming forward of
+    # the validation pass and of every configuration the one-pass form does not cover)
     ms = time_events(torch, loss_fwd, 20)
-    hbm("loss_fwd_kernel[KL, T rows x Vd, step 0]", 2.0 * t * vd * 2, ms, 1, "loss_fwd")
+    hbm("loss_fwd_kernel[KL, T rows x Vd, step 0]", 2.0 * t * vd * 2, ms, 0, "loss_fwd")
     ms = time_events(torch, loss_fwd_reuse, 20)
     hbm("loss_fwd_kernel[KL, T rows x Vd, steps >= 1 (target statistics reused)]", 2.0 * t * vd * 2,
-        ms, k_steps - 1, "loss_fwd_reuse")
+        ms, 0, "loss_fwd_reuse")
     rg = torch.full((t,), 1.0 / t, device=device)
     grad = torch.empty(t, vd, device=device, dtype=torch.bfloat16)
 
@@ -363,7 +365,23 @@ def kernel_rooflines(torch, cfg, t, k_steps, device, windows=(None,)):
                   _lib.ptr(rg_live), None, _lib.ptr(row_map), _lib.ptr(grad), vd, st)
 
     ms = time_events(torch, loss_bwd_packed, 20)
-    hbm(f"loss_bwd_kernel[KL, packed: {n_live} live of T rows x Vd]", 3.0 * n_live * vd * 2, ms, k_steps)
+    hbm(f"loss_bwd_kernel[KL, packed: {n_live} live of T rows x Vd]", 3.0 * n_live * vd * 2, ms, 0)
+    # what the timed step launches while lm_head is frozen: loss, statistics, acceptance chain AND the
+    # unit-weight logits gradient of the live rows in one read of the row pair.  Step 0 reads every target row
+    # (their statistics are made there), the later steps only those of the live rows.
+    mask_f = live_mask.float()
+    prev_fg = live_mask.clone()
+    cnt_fg = torch.zeros(3, device=device, dtype=torch.int32)
+    step_fg = L.StepPass(mask=mask_f, prev=prev_fg, counts=cnt_fg, grad_in_pass=True)
+    fg0 = L._loss_forward_with_grad(L.OP_KL, lg, tg, None, step_fg)
+    known_fg = (fg0[1].clone(), fg0[3].clone())
+    ms = time_events(torch, lambda: L._loss_forward_with_grad(L.OP_KL, lg, tg, None, step_fg), 20)
+    hbm(f"loss_fwd_grad_kernel[KL forward + logits gradient of {n_live} live rows, step 0, + row map]",
+        (2.0 * t + n_live) * vd * 2, ms, 1)
+    ms = time_events(torch, lambda: L._loss_forward_with_grad(L.OP_KL, lg, tg, known_fg, step_fg), 20)
+    hbm(f"loss_fwd_grad_kernel[KL forward + logits gradient of {n_live} live rows, steps >= 1, + row map]",
+        (1.0 * t + 2.0 * n_live) * vd * 2, ms, k_steps - 1)
+    del fg0
     # the yardstick of that launch's size: a plain copy of n_live rows (one read + one write per element;
     # the kernel above reads two rows for every row it writes)
     src = lg[:n_live]

@@ -111,6 +111,28 @@ int spx_vocab_loss_step_fwd(int op, const void* logits, int64_t ld_logits,
                             const void* mask, int mask_kind, void* prev_correct,
                             int prev_kind, int32_t* counts, void* stream);
 
+/* The row pass of a TTT step that also leaves the gradient of the logits behind (kl and ce, bf16,
+ * vocab a multiple of 8 and at most 32768, 16-byte aligned rows): a workgroup holds the whole row
+ * pair in registers, so logits and targets are read ONCE for loss_forward_kernel and
+ * loss_backward_kernel together (losses/fused.py:91-235) -- three row transfers per live row
+ * instead of five.  Outputs and the acceptance chain as for spx_vocab_loss_step_fwd (no d2t
+ * form); additionally, for every row r with row_map[r] >= 0 (spx_pack_row_map of the loss mask),
+ *   grad_logits[row_map[r], :] = softmax(logits[r]) - softmax(targets[r])          (kl)
+ *                                softmax(logits[r]) - onehot(argmax targets[r])     (ce)
+ * i.e. the gradient for a row weight of ONE: what follows is linear in the rows, so the weight
+ * the reduction behind the loss gives row r is applied to the result of the input-gradient
+ * product (spx_unpack_rows_scaled).  Rows mapped to -1 get no gradient row; with
+ * reuse_target_stats their target row is not read and their loss is written as 0 (a masked
+ * row's loss enters no sum), their arg-max outputs and chain update are as for any row. */
+int spx_vocab_loss_step_fwd_grad(int op, const void* logits, int64_t ld_logits,
+                                 const void* targets, int64_t ld_targets, int64_t rows,
+                                 int64_t vocab, float* loss, float* lse_draft,
+                                 float* lse_target, float* extra, int32_t* argmax_draft,
+                                 int32_t* argmax_target, int reuse_target_stats,
+                                 const void* mask, int mask_kind, void* prev_correct,
+                                 int prev_kind, int32_t* counts, const int32_t* row_map,
+                                 void* grad_logits, int64_t ld_grad, void* stream);
+
 /* grad_logits[r, :] = g_r * dL_r/dlogits, g_r = row_grad[r] * (*scale)
  * (scale may be NULL = 1).  Rows with g_r == 0 are written as exact zeros
  * without reading the inputs.  Closed forms of losses/fused.py:11-18; replaces
@@ -584,6 +606,12 @@ int spx_pack_row_map(const float* row_grad, const int64_t* labels, int64_t ignor
 int spx_unpack_rows(const void* packed, int64_t ld_packed, const int32_t* row_map,
                     int64_t rows, int64_t total_rows, int64_t cols, void* out,
                     int64_t ld_out, void* stream);
+/* The same with every live row multiplied by row_scale[r] (f32 [rows]) on its way: the row
+ * weights of a product whose packed operand was made for unit weights
+ * (spx_vocab_loss_step_fwd_grad). */
+int spx_unpack_rows_scaled(const void* packed, int64_t ld_packed, const int32_t* row_map,
+                           const float* row_scale, int64_t rows, int64_t total_rows,
+                           int64_t cols, void* out, int64_t ld_out, void* stream);
 
 /* c[M, N] (+)= a[T, M]^T * b[T, N], bf16 inputs, fp32 accumulation, bf16 output:
  * the weight-gradient product of the backward of torch.nn.Linear (dW = dY^T X)

@@ -76,6 +76,9 @@ SIGNATURES["spx_pack_batch"] = [_P, _I, _I64, _I64, _I64, _P, _P, _I, _P, _P, _P
 SIGNATURES["spx_gemm_bf16_nt"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P]
 SIGNATURES["spx_pack_row_map"] = [_P, _P, _I64, _I64, _P, _P, _P]
 SIGNATURES["spx_unpack_rows"] = [_P, _I64, _P, _I64, _I64, _I64, _P, _I64, _P]
+SIGNATURES["spx_unpack_rows_scaled"] = [_P, _I64, _P, _P, _I64, _I64, _I64, _P, _I64, _P]
+SIGNATURES["spx_vocab_loss_step_fwd_grad"] = [_I, _P, _I64, _P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _I,
+                                              _P, _I, _P, _I, _P, _P, _P, _I64, _P]
 SIGNATURES["spx_gemm_bf16_nt_tail"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I32, _P, _I64, _P]
 SIGNATURES["spx_gemm_tail_workspace_bytes"] = []
 SIGNATURES["spx_gemm_bf16_nt_stats"] = [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _P, _P, _P, _I64, _P]

@@ -416,11 +416,13 @@ __global__ __launch_bounds__(1024) void pack_row_map_kernel(const float* __restr
   if (tid == 0) *count = base_s;
 }
 
-// out[r, :] = row_map[r] >= 0 ? packed[row_map[r], :] : 0 for r < rows, 0 for rows <= r < total_rows
+// out[r, :] = row_map[r] >= 0 ? packed[row_map[r], :] : 0 for r < rows, 0 for rows <= r < total_rows;
+// with row_scale every live row is multiplied by row_scale[r] on its way (fp32, one rounding)
 __global__ __launch_bounds__(256) void unpack_rows_kernel(const uint16_t* __restrict__ packed, int64_t ld,
                                                           const int32_t* __restrict__ row_map, int rows,
                                                           int cols8, uint16_t* __restrict__ out,
-                                                          int64_t ld_out) {
+                                                          int64_t ld_out,
+                                                          const float* __restrict__ row_scale = nullptr) {
   const int r = blockIdx.x;
   const int src = r < rows ? row_map[r] : -1;
   u32x4* o = reinterpret_cast<u32x4*>(out + (int64_t)r * ld_out);
@@ -430,7 +432,20 @@ __global__ __launch_bounds__(256) void unpack_rows_kernel(const uint16_t* __rest
     return;
   }
   const u32x4* in = reinterpret_cast<const u32x4*>(packed + (int64_t)src * ld);
-  for (int c = threadIdx.x; c < cols8; c += 256) o[c] = in[c];
+  if (!row_scale) {
+    for (int c = threadIdx.x; c < cols8; c += 256) o[c] = in[c];
+    return;
+  }
+  const float f = row_scale[r];
+  for (int c = threadIdx.x; c < cols8; c += 256) {
+    const u32x4 v = in[c];
+    u32x4 w;
+    w.x = pack_bf16x2(bf16_lo(v.x) * f, bf16_hi(v.x) * f);
+    w.y = pack_bf16x2(bf16_lo(v.y) * f, bf16_hi(v.y) * f);
+    w.z = pack_bf16x2(bf16_lo(v.z) * f, bf16_hi(v.z) * f);
+    w.w = pack_bf16x2(bf16_lo(v.w) * f, bf16_hi(v.w) * f);
+    o[c] = w;
+  }
 }
 
 }  // namespace spx
@@ -456,6 +471,20 @@ extern "C" int spx_unpack_rows(const void* packed, int64_t ld_packed, const int3
   hipLaunchKernelGGL(unpack_rows_kernel, dim3((unsigned)total_rows), dim3(256), 0,
                      reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const uint16_t*>(packed), ld_packed,
                      row_map, (int)rows, (int)(cols / 8), reinterpret_cast<uint16_t*>(out), ld_out);
+  return check_launch(__func__);
+}
+
+extern "C" int spx_unpack_rows_scaled(const void* packed, int64_t ld_packed, const int32_t* row_map,
+                                      const float* row_scale, int64_t rows, int64_t total_rows, int64_t cols,
+                                      void* out, int64_t ld_out, void* stream) {
+  SPX_REQUIRE(rows > 0 && total_rows >= rows && total_rows < (1ll << 31), "rows out of range");
+  SPX_REQUIRE(cols > 0 && cols % 8 == 0 && ld_packed % 8 == 0 && ld_out % 8 == 0 && ld_packed >= cols && ld_out >= cols,
+              "cols and the row strides must be multiples of 8 (bf16), strides at least cols");
+  SPX_REQUIRE(packed && row_map && row_scale && out, "null buffer");
+  SPX_REQUIRE(al16(packed) && al16(out), "buffers must be 16-byte aligned");
+  hipLaunchKernelGGL(unpack_rows_kernel, dim3((unsigned)total_rows), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const uint16_t*>(packed), ld_packed,
+                     row_map, (int)rows, (int)(cols / 8), reinterpret_cast<uint16_t*>(out), ld_out, row_scale);
   return check_launch(__func__);
 }
 

@@ -341,6 +341,183 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
   }
 }
 
+// ---- forward and logits gradient in one pass -------------------------------------------------------
+// The head of a TTT step is frozen while the draft layers train, and which rows carry a gradient is
+// known before the loss is (the loss mask): the row pass can then leave the gradient of the logits
+// behind as well, and the row pair is read ONCE instead of once by the forward and once more by the
+// backward.  One workgroup of 512 threads holds a whole row pair in registers (eight 16-byte chunks of
+// each row per thread as they come from memory, requested before anything is computed: vocab <= 32768,
+// bf16), reduces it to the row statistics exactly like loss_fwd_kernel, and, for a row that row_map
+// sends to a slot >= 0, goes over its registers a second time and writes
+//   grad[slot, :] = softmax(x) - softmax(y)   (kl)      softmax(x) - onehot(argmax y)   (ce)
+// -- the gradient for a row weight of ONE; the caller applies the weight the reduction behind the loss
+// gives the row to the input-gradient product's result (which is linear in it).  Rows mapped to -1 get
+// no gradient row, and with the target statistics handed in (KNOWN) their target row is not read at
+// all and their loss is written as zero: a masked row's loss enters no sum.
+constexpr int kFgThreads = 512, kFgWaves = kFgThreads / 64, kFgChunks = 8;
+template <int OP, bool KNOWN>
+__global__ __launch_bounds__(kFgThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void loss_fwd_grad_kernel(
+    const uint16_t* __restrict__ logits, int64_t ld_logits, const uint16_t* __restrict__ targets,
+    int64_t ld_targets, int64_t vocab, float* __restrict__ loss, float* __restrict__ lse_draft,
+    float* __restrict__ lse_target, float* __restrict__ extra, int32_t* __restrict__ argmax_draft,
+    int32_t* __restrict__ argmax_target, StepArgs sa, const int32_t* __restrict__ row_map,
+    uint16_t* __restrict__ grad, int64_t ld_grad) {
+  const int64_t r = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int nchunks = (int)(vocab >> 3);  // vocab is a multiple of 8 here
+  const int slot = row_map[r];
+  const bool live = slot >= 0;
+  const uint16_t* xrow = logits + r * ld_logits;
+  const uint16_t* yrow = targets ? targets + r * ld_targets : nullptr;
+  const bool read_y = !(KNOWN && (OP == SPX_LOSS_CE || !live));
+  u32x4 xr[kFgChunks], yr[kFgChunks];
+#pragma unroll
+  for (int k = 0; k < kFgChunks; ++k) {
+    const int c = tid + k * kFgThreads;
+    if (c < nchunks) {
+      xr[k] = ld16(xrow + ((int64_t)c << 3));
+      if (read_y) yr[k] = ld16(yrow + ((int64_t)c << 3));
+    }
+  }
+  const float lt2_known = KNOWN ? lse_target[r] * kLog2e : 0.f;  // base-2 target lse
+  RowStats s;
+  s.md = kNegBig; s.zd = 0.f; s.mt = kNegBig; s.zt = 0.f; s.at = 0.f;
+  s.bd = -INFINITY; s.id = 0x7fffffff; s.bt = -INFINITY; s.it = 0x7fffffff; s.xt = 0.f;
+  auto unpack = [](u32x4 raw, float v[8]) {
+    v[0] = bf16_lo(raw.x); v[1] = bf16_hi(raw.x); v[2] = bf16_lo(raw.y); v[3] = bf16_hi(raw.y);
+    v[4] = bf16_lo(raw.z); v[5] = bf16_hi(raw.z); v[6] = bf16_lo(raw.w); v[7] = bf16_hi(raw.w);
+  };
+#pragma unroll
+  for (int k = 0; k < kFgChunks; ++k) {
+    const int c = tid + k * kFgThreads;
+    if (c >= nchunks) continue;
+    const int base = c << 3;
+    float x[8], y[8];
+    unpack(xr[k], x);
+    if (read_y) unpack(yr[k], y);
+    float cx = x[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) cx = fmaxf(cx, x[i]);
+    if (cx > s.bd) {  // strict: an earlier chunk of this thread keeps a tie
+      int kk = 7;
+#pragma unroll
+      for (int i = 6; i >= 0; --i) kk = (x[i] == cx) ? i : kk;
+      s.bd = cx; s.id = base + kk;
+    }
+    {
+      const float cxs = cx * kLog2e;
+      float mn = s.md, z = s.zd;
+      if (cxs > mn) {
+        z *= fast_exp2(mn - cxs);
+        mn = cxs;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) z += fast_exp2(fmaf(x[i], kLog2e, -mn));
+      s.zd = z; s.md = mn;
+    }
+    if (!KNOWN) {
+      float cy = y[0];
+#pragma unroll
+      for (int i = 1; i < 8; ++i) cy = fmaxf(cy, y[i]);
+      if (cy > s.bt) {
+        int kk = 7;
+        float xv = x[7];
+#pragma unroll
+        for (int i = 6; i >= 0; --i) {
+          const bool hit = y[i] == cy;
+          kk = hit ? i : kk;
+          xv = hit ? x[i] : xv;
+        }
+        s.bt = cy; s.it = base + kk; s.xt = xv;
+      }
+      if (OP != SPX_LOSS_CE) {
+        float mn = fmaxf(s.mt, cy * kLog2e);
+        float rs = fast_exp2(s.mt - mn);
+        float z = s.zt * rs, a = s.at * rs;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float e = fast_exp2(fmaf(y[i], kLog2e, -mn));
+          z += e;
+          a = fmaf(e, y[i] - x[i], a);
+        }
+        s.zt = z; s.at = a; s.mt = mn;
+      }
+    } else if (OP != SPX_LOSS_CE && live) {
+      float a = s.at;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float pr = fast_exp2(fmaf(y[i], kLog2e, -lt2_known));  // the target probability
+        a = fmaf(pr, y[i] - x[i], a);
+      }
+      s.at = a;
+    }
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) merge(s, shuffle_xor(s, m));
+  __shared__ RowStats part[kFgWaves];
+  if ((tid & 63) == 0) part[tid >> 6] = s;
+  __syncthreads();
+  s = part[0];
+#pragma unroll
+  for (int w = 1; w < kFgWaves; ++w) merge(s, part[w]);
+
+  const float lse_d = (s.md + fast_log2(s.zd)) * kLn2;
+  const float lse_t = KNOWN ? lse_target[r]
+                            : ((OP != SPX_LOSS_CE) ? (s.mt + fast_log2(s.zt)) * kLn2 : 0.f);
+  if (KNOWN) {
+    s.it = argmax_target[r];
+    if (OP == SPX_LOSS_CE) s.xt = (s.it >= 0 && s.it < vocab) ? load1(xrow + s.it) : 0.f;
+  }
+  if (tid == 0) {
+    float row_loss;
+    if (OP == SPX_LOSS_KL) row_loss = (KNOWN && !live) ? 0.f : (KNOWN ? s.at : s.at / s.zt) - lse_t + lse_d;
+    else row_loss = lse_d - s.xt;
+    loss[r] = row_loss;
+    lse_draft[r] = lse_d;
+    extra[r] = OP == SPX_LOSS_KL ? row_loss : 0.f;
+    if (argmax_draft) argmax_draft[r] = s.id;
+    if (!KNOWN) {
+      lse_target[r] = lse_t;
+      if (argmax_target) argmax_target[r] = s.it;
+    }
+    if (sa.counts) {
+      const bool m = sa.mask ? mask_value(sa.mask, sa.mask_kind, r) != 0.f : true;
+      const bool was = sa.prev ? mask_value(sa.prev, sa.prev_kind, r) != 0.f : true;
+      const bool now = was && (s.id == s.it);
+      if (m && now) atomicAdd(&sa.counts[0], 1);
+      if (m) atomicAdd(&sa.counts[1], 1);
+      if (was) atomicAdd(&sa.counts[2], 1);
+      if (sa.prev) store_flag(sa.prev, sa.prev_kind, r, now);
+    }
+  }
+  if (!live) return;
+  uint16_t* grow = grad + (int64_t)slot * ld_grad;
+  const float cd = -lse_d * kLog2e, ct = -lse_t * kLog2e;
+  const int label = s.it;
+  // (the packed chunks are what stays in registers between the passes, not their 64 + 64 unpacked values)
+#pragma unroll
+  for (int k = 0; k < kFgChunks; ++k) {
+    asm volatile("" : "+v"(xr[k].x), "+v"(xr[k].y), "+v"(xr[k].z), "+v"(xr[k].w));
+    if (OP != SPX_LOSS_CE) asm volatile("" : "+v"(yr[k].x), "+v"(yr[k].y), "+v"(yr[k].z), "+v"(yr[k].w));
+  }
+#pragma unroll
+  for (int k = 0; k < kFgChunks; ++k) {
+    const int c = tid + k * kFgThreads;
+    if (c >= nchunks) continue;
+    const int base = c << 3;
+    float x[8], y[8], o[8];
+    unpack(xr[k], x);
+    if (OP != SPX_LOSS_CE) unpack(yr[k], y);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float dp = fast_exp2(fmaf(x[i], kLog2e, cd));
+      if (OP == SPX_LOSS_CE) o[i] = dp - ((base + i) == label ? 1.f : 0.f);
+      else o[i] = dp - fast_exp2(fmaf(y[i], kLog2e, ct));
+    }
+    store8_vec<uint16_t>(grow + ((int64_t)c << 3), o);
+  }
+}
+
 // ---- forward with the d2t gather, pipelined ------------------------------------------------------
 // The first step of a TTT loop whose targets arrive as full-vocabulary verifier logits: the same row pass
 // as loss_fwd_kernel<.., GATHER> (gather through d2t, both online soft-maxes, KL or CE, both arg-maxes,
@@ -946,6 +1123,50 @@ extern "C" int spx_vocab_loss_step_fwd(int op, const void* logits, int64_t ld_lo
   return loss_fwd_impl(__func__, op, logits, ld_logits, targets, ld_targets, rows, vocab, dtype, loss,
                        lse_draft, lse_target, extra, argmax_draft, argmax_target, reuse_target_stats,
                        sa, stream);
+}
+
+extern "C" int spx_vocab_loss_step_fwd_grad(int op, const void* logits, int64_t ld_logits,
+                                            const void* targets, int64_t ld_targets, int64_t rows,
+                                            int64_t vocab, float* loss, float* lse_draft,
+                                            float* lse_target, float* extra, int32_t* argmax_draft,
+                                            int32_t* argmax_target, int reuse_target_stats,
+                                            const void* mask, int mask_kind, void* prev_correct,
+                                            int prev_kind, int32_t* counts, const int32_t* row_map,
+                                            void* grad_logits, int64_t ld_grad, void* stream) {
+  const char* fname = __func__;
+  SPX_REQ_FN(op == SPX_LOSS_KL || op == SPX_LOSS_CE, "the one-pass form is built for kl and ce");
+  SPX_REQ_FN(rows >= 0 && rows < (1ll << 31), "bad row count");
+  SPX_REQ_FN(vocab > 0 && vocab % 8 == 0 && vocab <= (int64_t)kFgThreads * kFgChunks * 8,
+             "vocab must be a multiple of 8, at most 32768");
+  const bool known = reuse_target_stats != 0;
+  const bool no_targets = known && op == SPX_LOSS_CE;
+  SPX_REQ_FN(ld_logits >= vocab && ld_grad >= vocab && (no_targets || ld_targets >= vocab),
+             "row stride smaller than vocab");
+  SPX_REQ_FN(ld_logits % 8 == 0 && ld_grad % 8 == 0 && (no_targets || ld_targets % 8 == 0),
+             "row strides must be multiples of 8 elements");
+  if (counts) {
+    SPX_REQ_FN(!mask || kind_ok(mask_kind), "unknown mask element kind");
+    SPX_REQ_FN(!prev_correct || kind_ok(prev_kind), "unknown prev_correct element kind");
+  }
+  if (rows == 0) return SPX_OK;
+  SPX_REQ_FN(logits && (targets || no_targets) && loss && lse_draft && lse_target && extra && argmax_target &&
+                 row_map && grad_logits, "null buffer");
+  SPX_REQ_FN(!counts || argmax_draft, "the acceptance chain needs both arg-max outputs");
+  SPX_REQ_FN(aligned16(logits) && aligned16(grad_logits) && (no_targets || aligned16(targets)),
+             "rows must be 16-byte aligned");
+  const StepArgs sa = {nullptr, 0, nullptr, 0, mask, mask_kind, prev_correct, prev_kind, counts};
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)rows), block(kFgThreads);
+  auto lg = reinterpret_cast<const uint16_t*>(logits);
+  auto tg = reinterpret_cast<const uint16_t*>(targets);
+  auto gr = reinterpret_cast<uint16_t*>(grad_logits);
+#define SPX_FG(OPV, KN)                                                                                     \
+  hipLaunchKernelGGL((loss_fwd_grad_kernel<OPV, KN>), grid, block, 0, st, lg, ld_logits, tg, ld_targets, vocab, \
+                     loss, lse_draft, lse_target, extra, argmax_draft, argmax_target, sa, row_map, gr, ld_grad)
+  if (op == SPX_LOSS_KL) { if (known) SPX_FG(SPX_LOSS_KL, true); else SPX_FG(SPX_LOSS_KL, false); }
+  else { if (known) SPX_FG(SPX_LOSS_CE, true); else SPX_FG(SPX_LOSS_CE, false); }
+#undef SPX_FG
+  return check_launch(fname);
 }
 
 static int loss_bwd_impl(const char* fname, int op, const void* logits, int64_t ld_logits,

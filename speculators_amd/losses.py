@@ -45,13 +45,19 @@ class StepPass:
     is read at column ``i + d2t[i]`` while streaming; the draft-vocabulary rows come back in
     ``gathered`` (``[rows, Vd]``) for the later steps and the backward.
     ``counts`` (int32 ``[3]``, zeroed): the acceptance chain is done row by row in the same pass
-    (``mask`` / ``prev`` are the step's 1-D views, ``prev`` is updated in place)."""
+    (``mask`` / ``prev`` are the step's 1-D views, ``prev`` is updated in place).
+    ``grad_in_pass``: a promise of the caller that the reduction behind the row losses gives a row
+    whose ``mask`` entry is zero the weight zero (the masked mean of ``compute_metrics`` does).  The
+    head + loss node may then leave the gradient of the logits behind in the same row pass
+    (``spx_vocab_loss_step_fwd_grad``) instead of reading both rows again in its backward; masked
+    rows get no gradient whatever arrives for them."""
 
     d2t: torch.Tensor | None = None
     gathered: torch.Tensor | None = None
     mask: torch.Tensor | None = None
     prev: torch.Tensor | None = None
     counts: torch.Tensor | None = None
+    grad_in_pass: bool = False
 
 
 def fused_loss_forward(op: int, logits: torch.Tensor, targets: torch.Tensor, target_stats=None,
@@ -201,6 +207,57 @@ def _packed_row_map(row_grad: torch.Tensor, labels: torch.Tensor | None = None, 
     return out[:rows], out[rows:]
 
 
+def _unpack_rows_scaled(packed: torch.Tensor, row_map: torch.Tensor, row_scale: torch.Tensor, total_rows: int):
+    """``_unpack_rows`` with live row r multiplied by ``row_scale[r]`` (fp32) on its way."""
+    out = torch.empty(total_rows, packed.shape[1], device=packed.device, dtype=packed.dtype)
+    _lib.call("spx_unpack_rows_scaled", _lib.ptr(packed), packed.stride(0), _lib.ptr(row_map), _lib.ptr(row_scale),
+              row_map.numel(), total_rows, packed.shape[1], _lib.ptr(out), out.stride(0),
+              _lib.stream_ptr(packed.device))
+    return out
+
+
+# The head + loss node writes the logits gradient in its forward row pass where it can (see StepPass)
+HEAD_LOSS_ONE_PASS = True
+
+
+def _one_pass_ok(op, x, y, step) -> bool:
+    if not (HEAD_LOSS_ONE_PASS and step is not None and step.grad_in_pass and step.d2t is None
+            and step.mask is not None and op in (OP_KL, OP_CE) and x.dtype == torch.bfloat16):
+        return False
+    rows, vocab = x.shape
+    if rows == 0 or vocab % 8 or vocab > 32768 or x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+        return False
+    if step.mask.numel() != rows or (y is None and op != OP_CE):
+        return False
+    return y is None or (y.dtype == torch.bfloat16 and y.stride(1) == 1 and y.stride(0) % 8 == 0
+                         and y.data_ptr() % 16 == 0)
+
+
+def _loss_forward_with_grad(op, x, y, known, step):
+    """The row pass that also writes the unit-weight logits gradient of the unmasked rows, packed to
+    the front.  Returns ``(loss, lse_t, am_d, am_t, packed, row_map, count)``."""
+    rows, vocab = x.shape
+    dev = x.device
+    mask_f = step.mask if step.mask.dtype == torch.float32 else step.mask.to(torch.float32)
+    row_map, count = _packed_row_map(mask_f.contiguous())
+    packed = torch.empty(rows, vocab, device=dev, dtype=torch.bfloat16)
+    stats = torch.empty(4, rows, device=dev, dtype=torch.float32)
+    arg = torch.empty(2, rows, device=dev, dtype=torch.int32)
+    lse_t, am_t = stats[2], arg[1]
+    if known is not None:
+        lse_t, am_t = known[0].reshape(-1), known[1].reshape(-1)
+        if lse_t.numel() != rows or am_t.numel() != rows or lse_t.stride(0) != 1 or am_t.stride(0) != 1:
+            raise ValueError("target_stats must be contiguous [rows] tensors")
+    _lib.call(
+        "spx_vocab_loss_step_fwd_grad", op, _lib.ptr(x), x.stride(0), _lib.ptr(y),
+        y.stride(0) if y is not None else 0, rows, vocab, _lib.ptr(stats[0]), _lib.ptr(stats[1]),
+        _lib.ptr(lse_t), _lib.ptr(stats[3]), _lib.ptr(arg[0]), _lib.ptr(am_t), int(known is not None),
+        _lib.ptr(step.mask), _lib.kind_code(step.mask), _lib.ptr(step.prev),
+        _lib.kind_code(step.prev) if step.prev is not None else 0, _lib.ptr(step.counts),
+        _lib.ptr(row_map), _lib.ptr(packed), packed.stride(0), _lib.stream_ptr(dev))
+    return stats[0], lse_t, arg[0], am_t, packed, row_map, count
+
+
 def _unpack_rows(packed: torch.Tensor, row_map: torch.Tensor, total_rows: int):
     """One row per position again: live rows from their packed slot, the others (and the rows past
     the map, up to ``total_rows``) zero.  Slots past the count are never read."""
@@ -228,10 +285,17 @@ class _HeadFusedLoss(torch.autograd.Function):
 
         logits = gemm_nt(x2, weight)
         known = (known_lse_t, known_am_t) if known_lse_t is not None else None
-        loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, logits[:n_rows], targets, known,
-                                                                         step)
-        ctx.save_for_backward(x, None if op == OP_CE else y, lse_d, lse_t, extra, am_t, weight_t)
         ctx.op, ctx.total_rows = op, logits.shape[0]
+        xs = logits[:n_rows]
+        ys = None if targets is None else _rows_2d(targets)
+        ctx.one_pass = (known is not None or ys is not None) and _one_pass_ok(op, xs, ys, step)
+        if ctx.one_pass:
+            # the rows are read once: loss, statistics, chain and the (unit-weight) logits gradient
+            loss, lse_t, am_d, am_t, packed, row_map, count = _loss_forward_with_grad(op, xs, ys, known, step)
+            ctx.save_for_backward(packed, row_map, count, weight_t)
+        else:
+            loss, lse_d, lse_t, extra, am_d, am_t, x, y = fused_loss_forward(op, xs, targets, known, step)
+            ctx.save_for_backward(x, None if op == OP_CE else y, lse_d, lse_t, extra, am_t, weight_t)
         ctx.mark_non_differentiable(am_d, am_t, lse_t, logits)
         ctx.set_materialize_grads(False)  # no [T, Vd] zeros for the logits, which carry no gradient
         return loss, am_d, am_t, lse_t, logits
@@ -242,6 +306,12 @@ class _HeadFusedLoss(torch.autograd.Function):
 
         if grad_rows is None:
             return (None,) * 9
+        if ctx.one_pass:
+            packed, row_map, count, weight_t = ctx.saved_tensors
+            g = grad_rows.reshape(-1).to(torch.float32).contiguous()
+            dx_packed = gemm_nt(packed, weight_t, m_live=count, split=True)
+            return (_unpack_rows_scaled(dx_packed, row_map, g, ctx.total_rows), None, None, None, None, None,
+                    None, None, None)
 
         x, y, lse_d, lse_t, extra, am_t, weight_t = ctx.saved_tensors
         rows, vocab = x.shape

@@ -214,8 +214,10 @@ def compute_metrics(logits, targets, loss_mask, prev_correct, ttt_step: int,
             # the first term's row pass also gathers the targets (first step of a TargetGather)
             # and advances the acceptance chain
             counts = torch.zeros(3, device=dev, dtype=torch.int32)
+            # (a row the mask removes has weight zero in the masked mean below: the head + loss node may
+            # write the logits gradient of the other rows in the same pass)
             step = L.StepPass(d2t=gather.d2t if gather is not None else None, mask=mask1, prev=prev1,
-                              counts=counts)
+                              counts=counts, grad_in_pass=head is not None and mask1 is not None)
         elif gather is not None:
             s_targets = gather.compact
         if fn is L._HIP_LOSS_FN_MAP.get(name) and op is not None:

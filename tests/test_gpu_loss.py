@@ -156,6 +156,73 @@ def test_step_pass_gathers_and_counts_in_the_row_pass(op_name, dtype, vt, vd):
     assert torch.equal(out2, out)
 
 
+@pytest.mark.parametrize("op_name", ["kl_div", "ce"])
+@pytest.mark.parametrize("known", [False, True])
+@pytest.mark.parametrize("vocab", [32000, 32768, 8, 1000])
+def test_row_pass_that_also_writes_the_logits_gradient(op_name, known, vocab):
+    """``spx_vocab_loss_step_fwd_grad`` (a workgroup keeps the row pair in registers: loss, statistics,
+    acceptance chain and the unit-weight logits gradient of the unmasked rows in ONE read of the rows)
+    against the streaming kernels: arg-maxes, counts and ``prev_correct`` identical, row losses and
+    log-sum-exps within 1e-5 (another summation order), masked rows with known statistics report a
+    zero loss; the packed gradient rows against ``softmax(x) - softmax(y)`` / ``softmax(x) - onehot``
+    in fp32 (one bf16 rounding), rows past the live count untouched; the scaled unpack."""
+    from speculators_amd import _lib
+    from speculators_amd import losses as L
+
+    g = torch.Generator().manual_seed(vocab + 7 * known)
+    rows = 41
+    logits = (torch.randn(rows, vocab, generator=g) * 2).bfloat16().cuda()
+    targets = (torch.randn(rows, vocab, generator=g) * 2).bfloat16().cuda()
+    for i in range(0, rows, 3):
+        logits[i, targets[i].float().argmax()] = 30.0
+    targets[5, 1] = targets[5].float().max()  # a tie inside the target row: the first index wins
+    targets[5, 0] = targets[5, 1]
+    mask = (torch.rand(rows, generator=g) < 0.7).float().cuda()
+    mask[0], mask[1] = 0.0, 1.0
+    prev0 = (torch.rand(rows, generator=g) < 0.8).cuda()
+    op = L.PRIMITIVE_OP[op_name]
+
+    base = L.fused_loss_forward(op, logits, targets)  # the statistics of step 0
+    stats = (base[2].clone(), base[5].clone()) if known else None
+    prev_ref = prev0.clone()
+    step_ref = L.StepPass(mask=mask, prev=prev_ref, counts=torch.zeros(3, dtype=torch.int32, device="cuda"))
+    ref = L.fused_loss_forward(op, logits, targets, stats, step=step_ref)
+
+    prev_got = prev0.clone()
+    step = L.StepPass(mask=mask, prev=prev_got, counts=torch.zeros(3, dtype=torch.int32, device="cuda"),
+                      grad_in_pass=True)
+    assert L._one_pass_ok(op, logits, targets, step)
+    loss, lse_t, am_d, am_t, packed, row_map, count = L._loss_forward_with_grad(
+        op, logits, None if (known and op_name == "ce") else targets, stats, step)
+    live = mask.bool()
+    n_live = int(live.sum())
+    assert int(count) == n_live
+    assert torch.equal(am_d, ref[4]) and torch.equal(am_t, ref[5])
+    assert torch.equal(prev_got, prev_ref) and step.counts.tolist() == step_ref.counts.tolist()
+    want_loss = ref[0] if not known else torch.where(live, ref[0], torch.zeros_like(ref[0]))
+    if op_name == "ce":
+        want_loss = ref[0]  # the draft row alone gives it: also for a masked row
+    assert (loss - want_loss).abs().max().item() <= 1e-5 * max(1.0, want_loss.abs().max().item())
+    assert (lse_t - ref[2]).abs().max().item() <= 1e-5 * max(1.0, ref[2].abs().max().item())
+
+    p = torch.softmax(logits.float(), -1)
+    if op_name == "ce":
+        q = torch.nn.functional.one_hot(ref[5].long(), vocab).float()
+    else:
+        q = torch.softmax(targets.float(), -1)
+    want = (p - q)[live]
+    got = packed[:n_live].float()
+    assert (got - want).abs().max().item() <= 2 ** -8 * want.abs().max().item() + 1e-6
+    assert torch.equal(row_map[live].long().cpu(), torch.arange(n_live)) and (row_map[~live] == -1).all()
+
+    scale = torch.randn(rows, generator=g).cuda()
+    cols = packed[:, :8].contiguous()
+    out = L._unpack_rows_scaled(cols, row_map, scale, rows + 3)
+    want_out = torch.zeros(rows + 3, 8, device="cuda")
+    want_out[:rows][live] = cols[:n_live].float() * scale[live, None]
+    assert torch.equal(out, want_out.bfloat16())
+
+
 def test_compute_metrics_with_target_gather_equals_materialised_targets():
     """compute_metrics over three TTT steps with the targets given as full-vocabulary logits +
     d2t (first step reads through the table and leaves the draft-vocabulary rows behind) against
