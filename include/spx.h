@@ -122,8 +122,9 @@ int spx_vocab_loss_step_fwd(int op, const void* logits, int64_t ld_logits,
  * i.e. the gradient for a row weight of ONE: what follows is linear in the rows, so the weight
  * the reduction behind the loss gives row r is applied to the result of the input-gradient
  * product (spx_unpack_rows_scaled).  Rows mapped to -1 get no gradient row; with
- * reuse_target_stats their target row is not read and their loss is written as 0 (a masked
- * row's loss enters no sum), their arg-max outputs and chain update are as for any row. */
+ * reuse_target_stats their target row is not read and their loss and lse_draft are written as 0
+ * (a masked row's loss enters no sum), their arg-max outputs and chain update are as for any
+ * row. */
 int spx_vocab_loss_step_fwd_grad(int op, const void* logits, int64_t ld_logits,
                                  const void* targets, int64_t ld_targets, int64_t rows,
                                  int64_t vocab, float* loss, float* lse_draft,

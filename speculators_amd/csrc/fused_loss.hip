@@ -353,7 +353,8 @@ __global__ __launch_bounds__(kLossThreads) void loss_fwd_kernel(
 // -- the gradient for a row weight of ONE; the caller applies the weight the reduction behind the loss
 // gives the row to the input-gradient product's result (which is linear in it).  Rows mapped to -1 get
 // no gradient row, and with the target statistics handed in (KNOWN) their target row is not read at
-// all and their loss is written as zero: a masked row's loss enters no sum.
+// all, no soft-max of their draft row is formed and their loss is written as zero: a masked row's loss enters
+// no sum.  (Their arg-max outputs and their part of the acceptance chain are those of any row.)
 constexpr int kFgThreads = 512, kFgWaves = kFgThreads / 64, kFgChunks = 8;
 template <int OP, bool KNOWN>
 __global__ __launch_bounds__(kFgThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void loss_fwd_grad_kernel(
@@ -380,6 +381,8 @@ __global__ __launch_bounds__(kFgThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     }
   }
   const float lt2_known = KNOWN ? lse_target[r] * kLog2e : 0.f;  // base-2 target lse
+  // a masked row whose target statistics are known needs nothing but the draft row's arg-max
+  const bool soft_x = live || !KNOWN;
   RowStats s;
   s.md = kNegBig; s.zd = 0.f; s.mt = kNegBig; s.zt = 0.f; s.at = 0.f;
   s.bd = -INFINITY; s.id = 0x7fffffff; s.bt = -INFINITY; s.it = 0x7fffffff; s.xt = 0.f;
@@ -404,7 +407,7 @@ __global__ __launch_bounds__(kFgThreads) __attribute__((amdgpu_waves_per_eu(4, 4
       for (int i = 6; i >= 0; --i) kk = (x[i] == cx) ? i : kk;
       s.bd = cx; s.id = base + kk;
     }
-    {
+    if (soft_x) {
       const float cxs = cx * kLog2e;
       float mn = s.md, z = s.zd;
       if (cxs > mn) {
@@ -461,7 +464,7 @@ __global__ __launch_bounds__(kFgThreads) __attribute__((amdgpu_waves_per_eu(4, 4
 #pragma unroll
   for (int w = 1; w < kFgWaves; ++w) merge(s, part[w]);
 
-  const float lse_d = (s.md + fast_log2(s.zd)) * kLn2;
+  const float lse_d = soft_x ? (s.md + fast_log2(s.zd)) * kLn2 : 0.f;
   const float lse_t = KNOWN ? lse_target[r]
                             : ((OP != SPX_LOSS_CE) ? (s.mt + fast_log2(s.zt)) * kLn2 : 0.f);
   if (KNOWN) {
@@ -470,7 +473,8 @@ __global__ __launch_bounds__(kFgThreads) __attribute__((amdgpu_waves_per_eu(4, 4
   }
   if (tid == 0) {
     float row_loss;
-    if (OP == SPX_LOSS_KL) row_loss = (KNOWN && !live) ? 0.f : (KNOWN ? s.at : s.at / s.zt) - lse_t + lse_d;
+    if (!soft_x) row_loss = 0.f;
+    else if (OP == SPX_LOSS_KL) row_loss = (KNOWN ? s.at : s.at / s.zt) - lse_t + lse_d;
     else row_loss = lse_d - s.xt;
     loss[r] = row_loss;
     lse_draft[r] = lse_d;
