@@ -543,7 +543,9 @@ __global__ __launch_bounds__(256) void gemm_row_stats_reduce_kernel(const float*
 }
 
 // The tiles of the last round of a product cut by tail_plan: C[tile] = the sum of its parts, in their
-// order, fp32, one rounding.  blockIdx.x = tail tile, 256 threads x 32 passes of 8 columns.
+// order, fp32, one rounding.  blockIdx.x = (tail tile, one of kTailSlices bands of 32 rows): 256 threads x 4
+// passes of 8 columns, enough workgroups to fill the chip for the 128 tiles of half a round.
+constexpr int kTailSlices = 8;
 __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const float* __restrict__ part_ws,
                                                                uint16_t* __restrict__ C, int64_t ldc, int M, int N,
                                                                int K, int tiles_m, int tiles_n, int max_parts,
@@ -551,18 +553,20 @@ __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const float* __re
   int tail_first, tail_parts;
   tail_plan(tiles_m * tiles_n, cus, (K + kTK - 1) / kTK, max_parts, tail_first, tail_parts);
   const int n_tail = tiles_m * tiles_n - tail_first;
-  if (tail_parts <= 1 || (int)blockIdx.x >= n_tail) return;
+  const int tail_idx = (int)blockIdx.x / kTailSlices, slice = (int)blockIdx.x % kTailSlices;
+  if (tail_parts <= 1 || tail_idx >= n_tail) return;
   int tile_m, tile_n;
-  tile_coords(tail_first + blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+  tile_coords(tail_first + tail_idx, tiles_m, tiles_n, tile_m, tile_n);
   const int m0 = tile_m * kTM, n0 = tile_n * kTN;
   const bool fast = (ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
-  for (int it = threadIdx.x; it < kTM * (kTN / 8); it += 256) {
+  constexpr int kItems = kTM * (kTN / 8) / kTailSlices;
+  for (int it = slice * kItems + threadIdx.x; it < (slice + 1) * kItems; it += 256) {
     const int rr = it / (kTN / 8), cc = (it % (kTN / 8)) * 8;
     const int m = m0 + rr, n = n0 + cc;
     if (m >= M || n >= N) continue;
     f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
     for (int p = 0; p < tail_parts; ++p) {
-      const float* src = part_ws + ((int64_t)(p * n_tail + blockIdx.x) << 16) + rr * kTN + cc;
+      const float* src = part_ws + ((int64_t)(p * n_tail + tail_idx) << 16) + rr * kTN + cc;
       const f32x4 a = *reinterpret_cast<const f32x4*>(src), b = *reinterpret_cast<const f32x4*>(src + 4);
       lo[0] += a[0]; lo[1] += a[1]; lo[2] += a[2]; lo[3] += a[3];
       hi[0] += b[0]; hi[1] += b[1]; hi[2] += b[2]; hi[3] += b[3];
@@ -688,7 +692,8 @@ static int gemm_nt_impl(const char* fname, const void* a, int64_t lda, const voi
   if (int rc = check_launch(fname)) return rc;
   if (tail_mode) {
     if (tail_parts > 1) {
-      hipLaunchKernelGGL(gemm_tail_reduce_kernel, dim3((unsigned)(tiles_m * tiles_n - tail_first)), dim3(256), 0, st,
+      hipLaunchKernelGGL(gemm_tail_reduce_kernel,
+                         dim3((unsigned)((tiles_m * tiles_n - tail_first) * kTailSlices)), dim3(256), 0, st,
                          part_ws, reinterpret_cast<uint16_t*>(c), ldc, (int)M, (int)N, (int)K, tiles_m, tiles_n,
                          max_parts, cus);
       return check_launch(fname);
