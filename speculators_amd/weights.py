@@ -213,9 +213,11 @@ class Staged:
             self._acc = torch.empty(self.w.shape, device=self.w.device, dtype=torch.float32)
         return self._acc, holds
 
-    def finish(self):
+    def finish(self, bf16_ok: bool = False):
         """The fp32 weight gradient of every recorded use (None if there is none): one product
-        per run of adjacent uses in the buffers -- normally one -- plus one per outside use."""
+        per run of adjacent uses in the buffers -- normally one -- plus one per outside use.
+        ``bf16_ok``: the parameters are bf16, so when ONE product is all there is, it writes bf16
+        itself (the same fp32 accumulation and the same one rounding as a cast of its fp32 result)."""
         acc = self._acc
         runs: list = []
         for r0, n in sorted(self._live):
@@ -223,6 +225,14 @@ class Staged:
                 runs[-1][1] += n
             else:
                 runs.append([r0, n])
+        if bf16_ok and acc is None and len(runs) == 1 and not self._extras and not self._finishers:
+            r0, n = runs[0]
+            dy, x = self._dys[r0:r0 + n], self._xs[r0:r0 + n]
+            if _tn_ok(dy) and _tn_ok(x):
+                from .gemm import gemm_tn
+
+                self._dys, self._live, self._marked = None, [], False
+                return gemm_tn(dy, x, out_dtype=torch.bfloat16)
         for r0, n in runs:
             acc = wgrad_product(self._dys[r0:r0 + n], self._xs[r0:r0 + n], acc)
         for dy2, x2 in self._extras:
@@ -256,7 +266,7 @@ class _Stage(torch.autograd.Function):
     def backward(ctx, _gw, g):
         # g is the marker of ``Staged.defer`` (no memory behind it): the gradient is computed here,
         # now that every use has run its backward
-        acc = ctx.staged.finish()
+        acc = ctx.staged.finish(bf16_ok=all(dt == torch.bfloat16 for dt in ctx.dtypes))
         if acc is not None:
             g = acc
         if g is None:
