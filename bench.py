@@ -38,6 +38,8 @@ TRAFFIC_ROWS = {
     "loss_fwd": ("loss_fwd_kernel<unsigned short, 0, true, false, false", None),
     "loss_fwd_reuse": ("loss_fwd_kernel<unsigned short, 0, true, true, false", None),
     "gemm_tn": ("gemm_bf16_tn_kernel<2, false>", None),
+    "loss_fwd_grad_step0": ("loss_fwd_grad_kernel<0, false>", None),
+    "loss_fwd_grad": ("loss_fwd_grad_kernel<0, true>", None),
     # (the summary averages the loss backward over its full and packed launches: no per-launch figure)
 }
 # The attention kernels are listed per timed call in lines that start with "[attn_step<k>]" or
@@ -377,10 +379,10 @@ def kernel_rooflines(torch, cfg, t, k_steps, device, windows=(None,)):
     known_fg = (fg0[1].clone(), fg0[3].clone())
     ms = time_events(torch, lambda: L._loss_forward_with_grad(L.OP_KL, lg, tg, None, step_fg), 20)
     hbm(f"loss_fwd_grad_kernel[KL forward + logits gradient of {n_live} live rows, step 0, + row map]",
-        (2.0 * t + n_live) * vd * 2, ms, 1)
+        (2.0 * t + n_live) * vd * 2, ms, 1, "loss_fwd_grad_step0")
     ms = time_events(torch, lambda: L._loss_forward_with_grad(L.OP_KL, lg, tg, known_fg, step_fg), 20)
     hbm(f"loss_fwd_grad_kernel[KL forward + logits gradient of {n_live} live rows, steps >= 1, + row map]",
-        (1.0 * t + 2.0 * n_live) * vd * 2, ms, k_steps - 1)
+        (1.0 * t + 2.0 * n_live) * vd * 2, ms, k_steps - 1, "loss_fwd_grad")
     del fg0
     # the yardstick of that launch's size: a plain copy of n_live rows (one read + one write per element;
     # the kernel above reads two rows for every row it writes)
