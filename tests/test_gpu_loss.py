@@ -357,6 +357,55 @@ def test_full_size_rows_properties():
     torch.testing.assert_close(rows[:, idx].detach().cpu(), ref, **LOSS_TOL)
 
 
+def test_full_size_row_pass_with_gradient_properties():
+    """The one-read row pass at the config[1] row shape (4096 x 32000 bf16, 70 % of the rows live, target
+    statistics of an earlier step handed in): against the streaming kernels on the same rows -- arg-maxes,
+    counts and chain identical, row losses within 1e-5 -- and through what needs no oracle at size: KL rows
+    >= 0, every gradient row sums to ~0 (two soft-maxes), the gradient of a row paired with itself is zero,
+    rows past the live count are untouched, two runs agree bit for bit."""
+    from speculators_amd import losses as L
+
+    g = torch.Generator(device="cuda").manual_seed(9)
+    t, v = 4096, 32000
+    x = (torch.randn(t, v, device="cuda", generator=g) * 2).bfloat16()
+    y = (torch.randn(t, v, device="cuda", generator=g) * 2).bfloat16()
+    y[7] = x[7]  # a row paired with itself
+    mask = (torch.rand(t, device="cuda", generator=g) < 0.7).float()
+    mask[7] = 1.0
+    base = L.fused_loss_forward(L.OP_KL, x, y)
+    known = (base[2].clone(), base[5].clone())
+    prev0 = torch.rand(t, device="cuda", generator=g) < 0.8
+
+    def run(one_pass):
+        prev = prev0.clone()
+        step = L.StepPass(mask=mask, prev=prev, counts=torch.zeros(3, dtype=torch.int32, device="cuda"),
+                          grad_in_pass=one_pass)
+        if one_pass:
+            out = L._loss_forward_with_grad(L.OP_KL, x, y, known, step)
+            return out, prev, step.counts
+        return L.fused_loss_forward(L.OP_KL, x, y, known, step=step), prev, step.counts
+
+    (loss, _lse_t, am_d, am_t, packed, row_map, count), prev_a, counts_a = run(True)
+    ref, prev_b, counts_b = run(False)
+    live = mask.bool()
+    n_live = int(live.sum())
+    assert int(count) == n_live and counts_a.tolist() == counts_b.tolist() and torch.equal(prev_a, prev_b)
+    assert torch.equal(am_d, ref[4]) and torch.equal(am_t, ref[5])
+    assert (loss[live] - ref[0][live]).abs().max().item() <= 1e-5 * ref[0].abs().max().item()
+    assert (loss[~live] == 0).all() and (loss >= -1e-5).all()
+    grad = packed[:n_live].float()
+    assert grad.sum(-1).abs().max().item() < 2e-2
+    assert grad[int(row_map[7])].abs().max().item() == 0.0
+    packed2 = L._loss_forward_with_grad(L.OP_KL, x, y, known, L.StepPass(
+        mask=mask, prev=prev0.clone(), counts=torch.zeros(3, dtype=torch.int32, device="cuda"), grad_in_pass=True))[4]
+    assert torch.equal(packed2[:n_live], packed[:n_live])
+    # a 32-row sample against the closed form in fp32
+    idx = torch.nonzero(live).flatten()[::97][:32]
+    want = torch.softmax(x[idx].float(), -1) - torch.softmax(y[idx].float(), -1)
+    got = packed[row_map[idx].long()].float()
+    assert (got - want).abs().max().item() <= 2 ** -8 * want.abs().max().item() + 1e-7
+
+
 @pytest.mark.parametrize("op_name", ["kl_div", "ce"])
 def test_reused_target_statistics_give_the_same_rows(op_name):
     """Steps >= 1 reuse the verifier rows' lse / arg-max from step 0: same loss, arg-maxes
