@@ -165,7 +165,7 @@ def test_row_pass_that_also_writes_the_logits_gradient(op_name, known, vocab):
     against the streaming kernels: arg-maxes, counts and ``prev_correct`` identical, row losses and
     log-sum-exps within 1e-5 (another summation order), masked rows with known statistics report a
     zero loss; the packed gradient rows against ``softmax(x) - softmax(y)`` / ``softmax(x) - onehot``
-    in fp32 (one bf16 rounding), rows past the live count untouched; the scaled unpack."""
+    in fp32 (one bf16 rounding); the scaled unpack."""
     from speculators_amd import _lib
     from speculators_amd import losses as L
 
@@ -362,7 +362,7 @@ def test_full_size_row_pass_with_gradient_properties():
     statistics of an earlier step handed in): against the streaming kernels on the same rows -- arg-maxes,
     counts and chain identical, row losses within 1e-5 -- and through what needs no oracle at size: KL rows
     >= 0, every gradient row sums to ~0 (two soft-maxes), the gradient of a row paired with itself is zero,
-    rows past the live count are untouched, two runs agree bit for bit."""
+    two runs agree bit for bit."""
     from speculators_amd import losses as L
 
     g = torch.Generator(device="cuda").manual_seed(9)
