@@ -66,12 +66,15 @@ class GainGrads:
     A staged gain carries its ``GainGrads`` as the attribute ``spx_gain_grads``."""
 
     def __init__(self):
-        self.scratch, self.slots, self.h, self.marked = None, 0, 0, False
+        self.scratch, self.slots, self.h, self.marked, self.task = None, 0, 0, False, None
 
     def target(self, rows: int, h: int, device):
         """``(scratch, accumulate)`` for a use over ``rows`` rows, None if it cannot share the buffer
         (another row count lays the partial sums out differently): it then returns a gradient of
         its own, which autograd adds."""
+        task = torch._C._current_graph_task_id()
+        if task != self.task:  # a pass that never reached the staging node leaves nothing behind
+            self.scratch, self.marked, self.task = None, False, task
         slots = int(_lib.load().spx_rmsnorm_bwd_slots(rows, h))
         if self.scratch is None:
             self.scratch = torch.empty(slots * h, device=device, dtype=torch.float32)

@@ -117,7 +117,7 @@ class Staged:
     is expected to run against it (the size of the input / output-gradient buffers)."""
 
     __slots__ = ("w", "token", "rows_of", "uses", "_wt", "_xs", "_fill", "_dys", "_live", "_extras",
-                 "_marked", "_acc", "aux", "_finishers")
+                 "_marked", "_acc", "aux", "_finishers", "_task")
 
     def __init__(self, w, rows_of, uses: int = 1):
         self.w = w
@@ -134,6 +134,7 @@ class Staged:
         self._acc = None   # fp32 gradient buffer of uses that add their gradient themselves
         self.aux = None    # whatever a family of products keeps per staged weight (the expert stacks)
         self._finishers = []  # callables acc -> acc that add deferred gradients when the node runs
+        self._task = None     # the backward pass (autograd graph task) the recorded uses belong to
 
     @property
     def trainable(self) -> bool:
@@ -174,11 +175,21 @@ class Staged:
         return -1
 
     # ---- backward side
+    def _enter_pass(self):
+        """What the uses record belongs to ONE backward pass, which ends in ``finish`` when autograd
+        reaches the staging node.  A pass that never got there (``autograd.grad`` for other inputs
+        over a retained graph) must not leak its records into the next one."""
+        task = torch._C._current_graph_task_id()
+        if task != self._task:
+            self._dys, self._live, self._extras, self._marked, self._acc = None, [], [], False, None
+            self._task = task
+
     def dy_slot(self, r0: int, rows: int):
         """Where the output gradient of the use at rows ``r0`` belongs (None for a use outside the
         buffers): a backward that allocates its own result writes it here."""
         if r0 < 0:
             return None
+        self._enter_pass()
         if self._dys is None:
             self._dys = torch.empty(self._xs.shape[0], self.w.shape[0], device=self.w.device,
                                     dtype=torch.bfloat16)
@@ -187,6 +198,7 @@ class Staged:
     def defer(self, r0: int, dy2: torch.Tensor, x2: torch.Tensor):
         """Record one use's ``(dy, x)`` for the weight-gradient product the staging node runs.
         Returns what the calling backward returns as the gradient of ``token``."""
+        self._enter_pass()
         if r0 >= 0:
             slot = self.dy_slot(r0, dy2.shape[0])
             if dy2.data_ptr() != slot.data_ptr():
@@ -199,6 +211,7 @@ class Staged:
     def mark(self):
         """What a use's backward returns as the gradient of ``token``: the empty marker that makes
         autograd reach the staging node, once per backward; None afterwards."""
+        self._enter_pass()
         if self._marked:
             return None
         self._marked = True
@@ -208,6 +221,7 @@ class Staged:
         """``(buffer, holds)``: the fp32 buffer of ``w``'s shape that uses which compute their weight
         gradient themselves (the grouped expert products) add it to, and whether an earlier use of
         this backward has written it already (the first one overwrites)."""
+        self._enter_pass()
         holds = self._acc is not None
         if not holds:
             self._acc = torch.empty(self.w.shape, device=self.w.device, dtype=torch.float32)

@@ -518,6 +518,31 @@ def test_logits_gradient_written_in_the_forward_row_pass(loss_fn, master, monkey
         assert (a - b).abs().max().item() <= 2 ** -6 * b.abs().max().item() + 1e-12, k
 
 
+def test_a_backward_pass_for_some_inputs_leaves_nothing_behind():
+    """``autograd.grad`` for ONE parameter over a retained graph runs the uses' backwards but never
+    reaches the staging nodes of the other weights and gains: what those uses recorded (output
+    gradients of the one-product weight gradient, partial sums of the gain gradients, the shared dK / dV
+    buffer) belongs to that pass and must not enter the full ``backward()`` that follows."""
+    shape = _shape(num_hidden_layers=2)
+    w = {k: v.bfloat16() for k, v in OE.random_weights(shape, seed=1, std=0.05).items()}
+    t = 200
+    hs, ids, doc, mask, pos, vl = _batch(shape, t, 3, [90, 100])
+    args = (hs.bfloat16().cuda(), ids.cuda(), doc.cuda(), mask.cuda(), pos.cuda(), vl.bfloat16().cuda())
+    grads = []
+    for partial_first in (False, True):
+        model = _make(shape, w)
+        _, loss, _ = model(*args, ttt_steps=3, ttt_step_loss_decay=0.8)
+        if partial_first:
+            (one,) = torch.autograd.grad(loss, [model.fc.weight], retain_graph=True)
+        loss.backward()
+        grads.append({k: p.grad.clone() for k, p in model.named_parameters() if p.grad is not None})
+        if partial_first:
+            assert torch.equal(one, grads[-1]["fc.weight"])
+    assert grads[0].keys() == grads[1].keys() and len(grads[0]) > 5
+    for k in grads[0]:
+        assert torch.equal(grads[0][k], grads[1][k]), k
+
+
 def test_head_node_falls_back_for_compound_losses():
     """A weighted sum of losses keeps the two-node form (the logits feed several reductions)."""
     from speculators_amd import losses as L
