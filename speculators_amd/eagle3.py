@@ -103,7 +103,10 @@ class Attention(nn.Module):
             if pos.dtype != torch.int64:
                 pos = pos.to(torch.int64)
             kvc = cache.get("kv")
-            if kvc is None and cache.get("steps") and self.attn_fn is A.ttt_hip_attention_forward:
+            # (a head size the kernels are not built for goes the general way below: the attention
+            # function widens it with zero columns)
+            if (kvc is None and cache.get("steps") and self.attn_fn is A.ttt_hip_attention_forward
+                    and self.d in A.KERNEL_HEAD_DIMS):
                 # all TTT steps' keys / values of this layer in one buffer, written in place
                 kvc = cache["kv"] = A.TTTKVCache(self.hkv, t, self.d, cache["steps"], x.device)
             q, k, v = gemm.qkv_rope(x, W(self.q_proj.weight, self.k_proj.weight, self.v_proj.weight),

@@ -108,12 +108,13 @@ def test_random_shapes(t, hq, hkv, d, docs, anchors, bs, window, ncf):
     test_forward_backward_match_dense_oracle(t, hq, hkv, d, docs, anchors, bs, window, ncf)
 
 
-@pytest.mark.parametrize("weighting,sliding", [("fixed-exp-decay", False), ("dpace", True)])
-def test_model_forward_backward_matches_oracle(weighting, sliding):
+@pytest.mark.parametrize("weighting,sliding,head_dim", [("fixed-exp-decay", False, 64), ("dpace", True, 64),
+                                                        ("fixed-exp-decay", True, 96)])
+def test_model_forward_backward_matches_oracle(weighting, sliding, head_dim):
     from speculators_amd import losses as L
     from speculators_amd.dflash import DFlashConfig, DFlashDraftModel
 
-    kw = dict(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=64,
+    kw = dict(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=head_dim,
               intermediate_size=512, vocab_size=2000, draft_vocab_size=704, num_aux=2,
               num_hidden_layers=2, rms_norm_eps=1e-6, rope_theta=10000.0)
     sl = dict(sliding_window=40, sliding_layers=(1,)) if sliding else {}

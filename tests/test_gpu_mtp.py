@@ -227,7 +227,8 @@ def _make(shape, w, steps):
 
 
 @pytest.mark.parametrize("variant", [dict(), dict(head_dim=128, num_attention_heads=2, num_key_value_heads=1),
-                                     dict(head_dim=256, num_attention_heads=2, num_key_value_heads=1)])
+                                     dict(head_dim=256, num_attention_heads=2, num_key_value_heads=1),
+                                     dict(head_dim=96, num_attention_heads=2, num_key_value_heads=1)])
 def test_model_forward_backward_matches_oracle(variant):
     shape = _shape(**variant)
     steps = 3
