@@ -38,7 +38,6 @@ namespace spx {
 #define SPX_GEMM_WN 2
 #define SPX_GEMM_MINW 1
 #define SPX_GEMM_READ_EVERY 2  // MFMAs per LDS fragment read
-#define SPX_GEMM_GROUP_M 8
 constexpr int kWM = SPX_GEMM_WM, kWN = SPX_GEMM_WN;  // waves along M / N of the tile
 constexpr int kNW = kWM * kWN;
 constexpr int kGemmThreads = 64 * kNW;
@@ -110,15 +109,24 @@ __host__ __device__ __forceinline__ void tail_plan(int n_tiles, int cus, int nsl
   if (tp > 1) { first = n_tiles - rem; parts = tp; }
 }
 
-// tile index -> (tile row, tile column): groups of GROUP_M tile rows, columns inside a group first
+// tile index -> (tile row, tile column).  256 consecutive indices (what the chip runs at a time) are a block of
+// 16 x 16 tiles, so that a 256-row band of either operand is used by 16 of the tiles in flight, and the blocks walk
+// along the longer side of the tile grid; 32 consecutive indices (what one XCD runs: see the kernel) are 8 tiles
+// along the longer side x 4 along the shorter, 12 operand bands through that XCD's L2.  In detail: panels of 16
+// along the shorter side; inside a panel groups of 8 along the longer side; inside a group the longer side first.
 __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
-  constexpr int GROUP_M = SPX_GEMM_GROUP_M;
-  const int in_group = GROUP_M * tiles_n;
-  const int group_id = pid / in_group;
-  const int first_m = group_id * GROUP_M;
-  const int group_sz = min(tiles_m - first_m, GROUP_M);
-  tile_m = first_m + (pid % in_group) % group_sz;
-  tile_n = (pid % in_group) / group_sz;
+  constexpr int kPanel = 16, kGroup = 8;
+  const bool m_long = tiles_m >= tiles_n;
+  const int tl = m_long ? tiles_m : tiles_n, ts = m_long ? tiles_n : tiles_m;
+  const int panel = pid / (tl * kPanel);
+  const int ps = min(ts - panel * kPanel, kPanel);
+  const int p = pid - panel * tl * kPanel;
+  const int g = p / (kGroup * ps);
+  const int gsz = min(tl - g * kGroup, kGroup);
+  const int r = p - g * kGroup * ps;
+  const int l = g * kGroup + r % gsz, sh = panel * kPanel + r / gsz;
+  tile_m = m_long ? l : sh;
+  tile_n = m_long ? sh : l;
 }
 
 template <bool kImm, int kStats = 0>
@@ -143,9 +151,10 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   // two groups, and the host never learns the group sizes
   if (tile_tab) tiles_m = min(tile_tab[0], tiles_m);
 
-  // workgroup id -> tile: XCD-contiguous bands, then groups of GROUP_M tile rows.  Workgroups go to
-  // the eight XCDs round robin: XCD x gets the ids x, x + 8, ...; they are renumbered so that each XCD
-  // works on one contiguous band of tiles (any grid size: the first n % 8 XCDs get one more)
+  // workgroup id -> tile index (tile_coords turns that into a tile).  Workgroups go to the eight XCDs round
+  // robin, XCD x gets the ids x, x + 8, ...: they are renumbered so that in every round of 256 workgroups each
+  // XCD has 32 consecutive tile indices, and in what is left after the last whole round one contiguous piece
+  // (the first n % 8 XCDs one more).
   // contraction in parts (part_ws): the workgroups of part p multiply columns [p, p + 1) * part length of
   // K and leave an fp32 partial in part_ws[p]; gemm_splitk_reduce_kernel adds the parts in order
   const int n_tiles = tiles_m * tiles_n;
@@ -159,17 +168,17 @@ __attribute__((amdgpu_waves_per_eu(SPX_GEMM_MINW, SPX_GEMM_MINW))) void gemm_bf1
   if ((int)blockIdx.x >= n_wg) return;
   int pid;
   {
+    constexpr int kRound = 256, kPer = kRound / 8;
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    if (tail_mode && tail_parts > 1 && (tail_first & 7) == 0) {
-      // every XCD first walks its band of the whole tiles, then its band of the cut ones: the workgroups
-      // are dispatched in the order of their ids, so the whole tiles fill the chip first and the parts of
-      // the last round follow everywhere at once
-      const int wb = tail_first >> 3, np = n_wg - tail_first;
-      if (local < wb) pid = xcd * wb + local;
-      else pid = tail_first + xcd * (np >> 3) + min(xcd, np & 7) + (local - wb);
+    // tail_mode with a cut last round: the whole tiles are whole rounds, the parts of the cut tiles are "what
+    // is left" -- dispatched after them (workgroups start in the order of their ids) and everywhere at once
+    const int whole = (tail_mode && tail_parts > 1) ? tail_first : n_wg;
+    const int full = whole / kRound * kRound;
+    if ((int)blockIdx.x < full) {
+      pid = (local / kPer) * kRound + xcd * kPer + local % kPer;
     } else {
-      const int base = n_wg >> 3, rem = n_wg & 7;
-      pid = xcd * base + min(xcd, rem) + local;
+      const int nr = n_wg - full;
+      pid = full + xcd * (nr >> 3) + min(xcd, nr & 7) + (local - full / 8);
     }
   }
   int part;

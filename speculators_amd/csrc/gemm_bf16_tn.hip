@@ -51,7 +51,6 @@ constexpr int kOob = 0x7ffffff0;
 static_assert(kTM == kTN, "both operands use one slab layout");
 static_assert(kABytes + (kKSteps - 1) * 32 * kRowBytes + 4 * kRowBytes < 65536,
               "slab buffer, K step and row pair of a fragment read go into the 16-bit offset field");
-#define SPX_GEMM_TN_GROUP_M 8
 
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef short i16x8 __attribute__((ext_vector_type(8)));
@@ -109,20 +108,43 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(1, 
     if ((OUT & 1) && (MULTI ? total_slabs == 0 : T == 0)) return;
   }
 
-  // workgroup id -> tile: XCD-contiguous bands, then groups of GROUP_M tile rows
+  // workgroup id -> tile.  The operands of a weight gradient are GBs (the contraction runs over the rows of
+  // several steps): what a tile order can save is memory traffic behind the L2s.  The 256 tiles that run at a
+  // time (a round) form a block of 16 x 16 tiles, so every 256-column band of either operand that the round
+  // touches is used by 16 of its tiles, and the rounds walk along the longer side of the tile grid: a band of
+  // the operand on that side is read in one round only, the other operand again every round.  Inside a round
+  // each XCD (workgroups go to them round robin) has 32 neighbouring tiles, 8 along the longer side x 4: 12
+  // bands through its L2, and a band of the longer side's operand is shared by four XCDs at the same time.
   const int n_wg = tiles_m * tiles_n;
   int pid;
   {
+    constexpr int kRound = 256, kPer = kRound / 8;
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int base = n_wg >> 3, rem = n_wg & 7;
-    pid = xcd * base + min(xcd, rem) + local;
+    const int full = n_wg / kRound * kRound;
+    if ((int)blockIdx.x < full) {
+      pid = (local / kPer) * kRound + xcd * kPer + local % kPer;
+    } else {  // the last, partial round: one contiguous piece per XCD (the first n % 8 get one tile more)
+      const int nr = n_wg - full, base = nr >> 3, rem = nr & 7;
+      pid = full + xcd * base + min(xcd, rem) + (local - full / 8);
+    }
   }
-  constexpr int GROUP_M = SPX_GEMM_TN_GROUP_M;
-  const int in_group = GROUP_M * tiles_n;
-  const int first_m = (pid / in_group) * GROUP_M;
-  const int group_sz = min(tiles_m - first_m, GROUP_M);
-  const int tile_m = first_m + (pid % in_group) % group_sz;
-  const int tile_n = (pid % in_group) / group_sz;
+  int tile_m, tile_n;
+  {
+    // tiles in the order of pid: panels of kPanel along the shorter side; inside a panel groups of kGroup along
+    // the longer side; inside a group the longer side first (the NT kernel's tile_coords: same order)
+    constexpr int kPanel = 16, kGroup = 8;
+    const bool m_long = tiles_m >= tiles_n;
+    const int tl = m_long ? tiles_m : tiles_n, ts = m_long ? tiles_n : tiles_m;
+    const int panel = pid / (tl * kPanel);
+    const int ps = min(ts - panel * kPanel, kPanel);
+    const int p = pid - panel * tl * kPanel;
+    const int g = p / (kGroup * ps);
+    const int gsz = min(tl - g * kGroup, kGroup);
+    const int r = p - g * kGroup * ps;
+    const int l = g * kGroup + r % gsz, sh = panel * kPanel + r / gsz;
+    tile_m = m_long ? l : sh;
+    tile_n = m_long ? sh : l;
+  }
   const int m0 = tile_m * kTM, n0 = tile_n * kTN;
 
   const int tid = threadIdx.x, lane = tid & 63;
