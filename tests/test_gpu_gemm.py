@@ -456,3 +456,28 @@ def test_gemm_nt_with_the_last_round_of_tiles_cut_along_the_contraction(m, n, k,
     # run to run identical (fixed order of the parts)
     again = gemm.gemm_nt(a, b)
     assert torch.equal(again.view(torch.int16), got.view(torch.int16))
+
+
+@pytest.mark.parametrize("tiles", [(17, 20), (20, 17), (35, 3), (3, 35), (40, 33)])
+def test_every_tile_of_a_ragged_tile_grid_is_computed_once(tiles):
+    """Tile grids that are no multiple of the tile order's panels (16), groups (8) or rounds (256 tiles), in
+    both orientations, with partial edge tiles: every element of the result of both GEMM kernels against an
+    fp32 product (a tile left out or written twice by a wrong workgroup -> tile map shows up as a whole
+    256 x 256 block of garbage)."""
+    from speculators_amd.gemm import gemm_nt, gemm_tn
+
+    tm, tn = tiles
+    m, n, k = tm * 256 - 8, tn * 256 - 248, 64
+    g = torch.Generator(device="cuda").manual_seed(tm * 100 + tn)
+    a = torch.randn(m, k, generator=g, device="cuda").bfloat16()
+    b = torch.randn(n, k, generator=g, device="cuda").bfloat16()
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    gemm_nt(a, b, out=out)
+    ref = a.float() @ b.float().T
+    torch.testing.assert_close(out.float(), ref, rtol=1e-2, atol=0.1)
+    # the weight-gradient orientation: a^T b over 64 rows, fp32 result
+    at = torch.randn(k, m, generator=g, device="cuda").bfloat16()
+    bt = torch.randn(k, n, generator=g, device="cuda").bfloat16()
+    out32 = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+    gemm_tn(at, bt, out=out32)
+    torch.testing.assert_close(out32, at.float().T @ bt.float(), rtol=1e-4, atol=1e-3)
